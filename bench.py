@@ -1,0 +1,398 @@
+#!/usr/bin/env python3
+"""Benchmark of the per-partition array execution path on one MI355X.
+
+Headline (one JSON line on stdout): dense conjugate gradient at n = 16384 in fp64, iterations per
+second, with the roofline of its dominant kernel (the tiled matvec, HBM-bound) and a CPU baseline
+(the oracle's restatement of the reference CPU path) timed on the host cores of the same box.
+A "step" is one CG iteration: one matvec over the 2x2 tile grid, two dots, two scalar ops and three
+fused vector updates. Inputs are generated on the device before the timed region starts.
+
+The other workloads (fused elementwise 2^24, Jacobi 2-D 8192^2, Jacobi 3-D 512^3, LSTM step) are
+measured the same way and reported under "also" in the same line.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+FP64_MFMA_PEAK_TFLOPS = 78.6
+
+
+def _dev():
+    from charmnumeric_amd import _lib as L
+
+    L.check(L.lib.cnh_init(0))
+    return L
+
+
+class Buf:
+    def __init__(self, L, nbytes, zero=False):
+        p = C.c_void_p()
+        L.check(L.lib.cnh_alloc(int(nbytes), 1 if zero else 0, C.byref(p)))
+        self.ptr = p.value
+        self.L = L
+        self.nbytes = int(nbytes)
+
+    def get(self, dtype=np.float64, count=None):
+        n = self.nbytes // np.dtype(dtype).itemsize if count is None else count
+        out = np.empty(n, dtype=dtype)
+        self.L.check(self.L.lib.cnh_d2h(out.ctypes.data, self.ptr, out.nbytes, None))
+        return out
+
+    def free(self):
+        if self.ptr:
+            self.L.lib.cnh_free(self.ptr)
+            self.ptr = None
+
+
+class Events:
+    """Pairs of HIP events on one stream; elapsed times read after a sync."""
+
+    def __init__(self, L, n):
+        self.L = L
+        self.a = [C.c_void_p() for _ in range(n)]
+        self.b = [C.c_void_p() for _ in range(n)]
+        for e in self.a + self.b:
+            L.check(L.lib.cnh_event_create(C.byref(e)))
+
+    def times_ms(self, used):
+        out = []
+        ms = C.c_float()
+        for i in range(used):
+            self.L.check(self.L.lib.cnh_event_elapsed_ms(self.a[i], self.b[i], C.byref(ms)))
+            out.append(ms.value)
+        return out
+
+    def free(self):
+        for e in self.a + self.b:
+            self.L.lib.cnh_event_destroy(e)
+
+
+def _compile(L, ast, dtype, nd):
+    k = C.c_void_p()
+    L.check(L.lib.cnh_compile_group(C.byref(ast), dtype, nd, 0, C.byref(k)))
+    return k
+
+
+def _launch1(L, k, nd, ins, scalars, outs, stream=None):
+    """One partition, broadcast scalars resident on the device."""
+    n_in, n_out = len(ins), len(outs)
+    ia = (L.Memref * max(1, n_in))(*ins)
+    oa = (L.Memref * max(1, n_out))(*outs)
+    sp = (C.c_void_p * max(1, len(scalars)))(*[C.c_void_p(s) for s in scalars])
+    L.check(L.lib.cnh_launch_group(k, nd, n_in, ia, len(scalars), sp, 1, n_out, oa, stream))
+
+
+# -------------------------------------------------------------------------------------------------
+# C2: dense CG, n = 16384
+# -------------------------------------------------------------------------------------------------
+def cg_asts(L):
+    from charmnumeric_amd.astbuild import AstBuilder
+
+    def scalar_div():
+        b = AstBuilder(L.F64, 1)
+        b.binary(L.OP_DIV, 3, b.broadcast(1), b.broadcast(2), is_temp=False)
+        return b.finish()
+
+    def axpy(op):
+        # out = u (op) s * v
+        b = AstBuilder(L.F64, 1)
+        u, v = b.leaf(1), b.leaf(2)
+        t = b.binary(L.OP_MUL, 100, b.broadcast(3), v)
+        b.binary(op, 4, u, t, is_temp=False)
+        return b.finish()
+
+    return scalar_div(), axpy(L.OP_ADD), axpy(L.OP_SUB)
+
+
+def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True):
+    tile = tile_rule_tile or cg_tile(n)
+    g = (n + tile - 1) // tile
+    t0 = time.time()
+    tiles = []
+    for i in range(g):
+        for j in range(g):
+            nr, nc = min(tile, n - i * tile), min(tile, n - j * tile)
+            b = Buf(L, nr * nc * 8)
+            L.check(L.lib.cnh_fill_cg_matrix(b.ptr, n, i * tile, nr, j * tile, nc, nc, seed, None))
+            tiles.append(b)
+    tptr = L.vparr([t.ptr for t in tiles])
+    vec = lambda: Buf(L, n * 8, zero=True)
+    bvec, x, r, p, Ap = vec(), vec(), vec(), vec(), vec()
+    x2, r2, p2 = vec(), vec(), vec()
+    L.check(L.lib.cnh_fill_uniform(bvec.ptr, n, seed, 1, 0, -1.0, 1.0, None))
+    sc = Buf(L, 8 * 8, zero=True)  # rtr, pAp, alpha, rtr_new, beta
+    S = lambda i: sc.ptr + 8 * i
+    ast_div, ast_add, ast_sub = cg_asts(L)
+    k_div, k_add, k_sub = (_compile(L, a, L.F64, 1) for a in (ast_div, ast_add, ast_sub))
+    mr = lambda b_, cnt=n: L.Memref.dense(b_.ptr, (cnt,))
+    smr = lambda i: L.Memref.dense(S(i), (1,))
+
+    def reset():
+        L.check(L.lib.cnh_memset0(x.ptr, n * 8, None))
+        L.check(L.lib.cnh_d2d(r.ptr, bvec.ptr, n * 8, None))
+        L.check(L.lib.cnh_d2d(p.ptr, bvec.ptr, n * 8, None))
+        L.check(L.lib.cnh_dot_partial(L.F64, n, r.ptr, r.ptr, S(0), None))
+
+    state = {"x": x, "r": r, "p": p, "x2": x2, "r2": r2, "p2": p2, "rtr": 0, "rtr_new": 3}
+
+    def iteration(ev=None, i=0):
+        st = state
+        if ev is not None:
+            L.check(L.lib.cnh_event_record(ev.a[i], None))
+        L.check(L.lib.cnh_gemv_tiles(L.F64, n, n, tile, tptr, st["p"].ptr, Ap.ptr, None))
+        if ev is not None:
+            L.check(L.lib.cnh_event_record(ev.b[i], None))
+        L.check(L.lib.cnh_dot_partial(L.F64, n, st["p"].ptr, Ap.ptr, S(1), None))
+        _launch1(L, k_div, 1, [], [S(st["rtr"]), S(1)], [smr(2)])                       # alpha
+        _launch1(L, k_add, 1, [mr(st["x"]), mr(st["p"])], [S(2)], [mr(st["x2"])])      # x + alpha p
+        _launch1(L, k_sub, 1, [mr(st["r"]), mr(Ap)], [S(2)], [mr(st["r2"])])           # r - alpha Ap
+        L.check(L.lib.cnh_dot_partial(L.F64, n, st["r2"].ptr, st["r2"].ptr, S(st["rtr_new"]), None))
+        _launch1(L, k_div, 1, [], [S(st["rtr_new"]), S(st["rtr"])], [smr(4)])           # beta
+        _launch1(L, k_add, 1, [mr(st["r2"]), mr(st["p"])], [S(4)], [mr(st["p2"])])     # r + beta p
+        st["x"], st["x2"] = st["x2"], st["x"]
+        st["r"], st["r2"] = st["r2"], st["r"]
+        st["p"], st["p2"] = st["p2"], st["p"]
+        st["rtr"], st["rtr_new"] = st["rtr_new"], st["rtr"]
+
+    reset()
+    for _ in range(warmup):
+        iteration()
+    L.check(L.lib.cnh_device_sync())
+    setup_s = time.time() - t0
+
+    reset()
+    ev = Events(L, steps)
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    L.check(L.lib.cnh_event_create(C.byref(e0)))
+    L.check(L.lib.cnh_event_create(C.byref(e1)))
+    L.check(L.lib.cnh_device_sync())
+    w0 = time.perf_counter()
+    L.check(L.lib.cnh_event_record(e0, None))
+    for i in range(steps):
+        iteration(ev, i)
+    L.check(L.lib.cnh_event_record(e1, None))
+    L.check(L.lib.cnh_device_sync())
+    wall = time.perf_counter() - w0
+    ms = C.c_float()
+    L.check(L.lib.cnh_event_elapsed_ms(e0, e1, C.byref(ms)))
+    gemv_ms = ev.times_ms(steps)
+    res = {
+        "n": n, "tile": tile, "steps": steps, "wall_s": wall, "gpu_ms": ms.value,
+        "ms_per_step": wall * 1e3 / steps, "iters_per_s": steps / wall,
+        "gemv_avg_us": 1e3 * float(np.mean(gemv_ms)), "gemv_min_us": 1e3 * float(np.min(gemv_ms)),
+        "setup_s": setup_s,
+        "rtr_final": float(sc.get(np.float64)[state["rtr"]]),
+        "x": state["x"].get() if check else None,
+    }
+    ev.free()
+    for b_ in tiles + [bvec, x, r, p, Ap, x2, r2, p2, sc]:
+        b_.free()
+    return res
+
+
+def cg_tile(n, odf=4, pes=1, min_tile=512):
+    """Tile edge of a 2-D array under the reference rule (decomposition_solver.hpp:100-122)."""
+    tile = min_tile
+    while ((n + tile - 1) // tile) ** 2 > odf * pes:
+        tile *= 2
+    return tile
+
+
+def cpu_cg_setup(n, seed=2):
+    from oracle import cn_oracle as O
+
+    orc = O.Oracle()
+    tile = cg_tile(n)
+    g = (n + tile - 1) // tile
+    tiles = [[orc.cg_matrix(n, i * tile, min(tile, n - i * tile), j * tile, min(tile, n - j * tile),
+                            seed) for j in range(g)] for i in range(g)]
+    b = orc.uniform(n, seed, 1, -1.0, 1.0)
+    return orc, tile, g, tiles, b
+
+
+def cpu_cg(setup, n, iters, threads):
+    """CG with the oracle's kernels in the reference's order of operations; returns (it/s, x, rtr)."""
+    from oracle import cn_oracle as O
+
+    orc, tile, g, tiles, b = setup
+    lib = orc.lib
+    x = np.zeros(n)
+    r = b.copy()
+    p = b.copy()
+    rtr = orc.dot(r, r)
+    Ap = np.zeros(n)
+    part = np.zeros(tile)
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        # tile GEMV + partial accumulate on the 1-D owner, column tiles in order
+        for i in range(g):
+            rows = tiles[i][0].shape[0]
+            seg = Ap[i * tile:i * tile + rows]
+            for j in range(g):
+                t = tiles[i][j]
+                xs = p[j * tile:j * tile + t.shape[1]]
+                lib.orc_gemv_sub_mt(O.F64, O.ptr(t), t.shape[1], 0, 0, t.shape[0], t.shape[1],
+                                    O.ptr(xs), O.ptr(part), threads)
+                if j == 0:
+                    seg[:] = part[:rows]
+                else:
+                    lib.orc_axpy1(O.F64, rows, O.ptr(part), O.ptr(seg))
+        pAp = orc.dot(p, Ap)
+        alpha = rtr / pAp
+        x = x + alpha * p
+        r = r - alpha * Ap
+        rtr_new = orc.dot(r, r)
+        beta = rtr_new / rtr
+        p = r + beta * p
+        rtr = rtr_new
+    dt = time.perf_counter() - t0
+    return iters / dt, x, rtr
+
+
+# -------------------------------------------------------------------------------------------------
+# C1: fused elementwise 2^24 + sum + dot
+# -------------------------------------------------------------------------------------------------
+def c1_ast(L):
+    from charmnumeric_amd.astbuild import AstBuilder
+
+    b = AstBuilder(L.F64, 1)
+    x, y = b.leaf(0), b.leaf(1)
+    t1 = b.binary(L.OP_MUL, 100, b.scalar(2.5), x)
+    t2 = b.binary(L.OP_MUL, 101, b.scalar(0.5), y)
+    t3 = b.binary(L.OP_SUB, 102, t1, t2)
+    t4 = b.binary(L.OP_MUL, 103, x, y)
+    b.binary(L.OP_ADD, 10, t3, t4, is_temp=False)
+    return b.finish()
+
+
+def run_c1(L, n=1 << 24, parts=4, reps=20):
+    per = n // parts
+    xs, ys, zs = [], [], []
+    for q in range(parts):
+        xb, yb, zb = Buf(L, per * 8), Buf(L, per * 8), Buf(L, per * 8)
+        L.check(L.lib.cnh_fill_uniform(xb.ptr, per, 0, 0, q * per, -1.0, 1.0, None))
+        L.check(L.lib.cnh_fill_uniform(yb.ptr, per, 0, 1, q * per, -1.0, 1.0, None))
+        xs.append(xb); ys.append(yb); zs.append(zb)
+    k = _compile(L, c1_ast(L), L.F64, 1)
+    ins = (L.Memref * (4 * parts))()
+    outs = (L.Memref * parts)()
+    for q in range(parts):
+        mx, my = L.Memref.dense(xs[q].ptr, (per,)), L.Memref.dense(ys[q].ptr, (per,))
+        ins[4 * q], ins[4 * q + 1], ins[4 * q + 2], ins[4 * q + 3] = mx, my, mx, my
+        outs[q] = L.Memref.dense(zs[q].ptr, (per,))
+    ones = Buf(L, 8)
+    res = Buf(L, 16, zero=True)
+    zp = L.vparr([z.ptr for z in zs])
+    lens = L.i64arr([per] * parts)
+
+    def ew():
+        L.check(L.lib.cnh_launch_group_batched(k, 1, parts, 4, ins, 0, None, 0, 1, outs, None))
+
+    def sm():
+        L.check(L.lib.cnh_sum_tiles(L.F64, parts, zp, lens, res.ptr, None))
+
+    def dt():
+        L.check(L.lib.cnh_dot_tiles(L.F64, parts, zp, zp, lens, res.ptr + 8, None))
+
+    out = {}
+    for name, fn, nbytes in (("elementwise", ew, 24 * n), ("sum", sm, 8 * n), ("dot_zz", dt, 8 * n)):
+        for _ in range(3):
+            fn()
+        ev = Events(L, reps)
+        L.check(L.lib.cnh_device_sync())
+        for i in range(reps):
+            L.check(L.lib.cnh_event_record(ev.a[i], None))
+            fn()
+            L.check(L.lib.cnh_event_record(ev.b[i], None))
+        L.check(L.lib.cnh_device_sync())
+        t = ev.times_ms(reps)
+        ev.free()
+        us = 1e3 * float(np.median(t))
+        out[name] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
+                     "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+    for b_ in xs + ys + zs + [ones, res]:
+        b_.free()
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--n", type=int, default=16384, help="order of the CG system")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-also", action="store_true", help="skip the secondary workloads")
+    ap.add_argument("--cpu-iters", type=int, default=10)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: every partition of the path lives on a single MI355X; "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    L = _dev()
+    name = C.create_string_buffer(256)
+    L.check(L.lib.cnh_device_name(name, 256))
+    n = args.n
+    cg = run_cg(L, n, args.steps, args.warmup)
+    gemv_bytes = 8.0 * n * n + 2 * 8.0 * n
+    achieved = gemv_bytes / (cg["gemv_avg_us"] * 1e-6) / 1e9
+    line = {
+        "metric": "cg_iterations_per_second_n16384_fp64",
+        "value": round(cg["iters_per_s"], 2),
+        "unit": "iterations/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(cg["ms_per_step"], 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f64",
+        "data": "synthetic",
+        "config": {"workload": f"dense CG, n={n}, A in {cg['tile']}^2 row-major tiles, one CG "
+                               "iteration per step (matvec, 2 dots, 2 scalar ops, 3 fused updates)",
+                   "device": name.value.decode()},
+        "roofline": {"bound": "hbm", "kernel": "gemv_rows<double>", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": None, "avg_us": round(cg["gemv_avg_us"], 2),
+                     "bytes_per_launch": gemv_bytes},
+        "gemv_roofline_iters_per_s": round(HBM_PEAK_GBS * 1e9 / gemv_bytes, 1),
+        "rtr_final": cg["rtr_final"],
+    }
+    if not args.no_also:
+        also = {}
+        try:
+            also["c1_fused_elementwise_2p24"] = run_c1(L)
+        except Exception as exc:  # report, do not hide
+            also["c1_error"] = str(exc)
+        line["also"] = also
+    if not args.no_cpu:
+        cores = os.cpu_count() or 1
+        threads = min(cores, 16)
+        setup = cpu_cg_setup(n)
+        ips1, xc, rtr_c = cpu_cg(setup, n, max(2, args.cpu_iters // 2), 1)
+        ipsN, _, _ = cpu_cg(setup, n, args.cpu_iters, threads)
+        line["cpu_baseline"] = {
+            "value": round(ipsN, 3), "unit": "iterations/s", "cores": threads, "kind": "port",
+            "sample": f"same system (n={n}, {cg['tile']}^2 tiles), {args.cpu_iters} CG iterations, "
+                      f"oracle kernels, tile matvec split over {threads} threads",
+            "one_core": round(ips1, 3),
+        }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,579 @@
+// AST -> HIP source for one fused group (host-only).
+#include "codegen.h"
+
+#include <cmath>
+#include <cstring>
+#include <map>
+#include <sstream>
+
+namespace cnh {
+
+const char* dtype_ctype(int dtype) {
+    switch (dtype) {
+    case CNH_F32: return "float";
+    case CNH_F64: return "double";
+    case CNH_I32: return "int";
+    case CNH_I64: return "long long";
+    }
+    return "void";
+}
+
+namespace {
+
+bool is_int(int dt) { return dt == CNH_I32 || dt == CNH_I64; }
+
+std::string fmt(const char* f, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, f);
+    vsnprintf(buf, sizeof buf, f, ap);
+    va_end(ap);
+    return buf;
+}
+
+// Literal of a scalar leaf in the group's element type. Integers are cast through int64,
+// floats through double (src/jit.cpp:108-116 upstream).
+std::string literal(int dtype, double c) {
+    if (is_int(dtype)) {
+        long long v = 0;
+        if (std::isfinite(c) && c > -9.2233720368547758e18 && c < 9.2233720368547758e18)
+            v = (long long)c;
+        if (dtype == CNH_I32)
+            v = (long long)(int32_t)(uint32_t)(uint64_t)v;
+        if (v == (-9223372036854775807LL - 1))
+            return "((T)(-9223372036854775807LL - 1))";
+        return fmt("((T)(%lldLL))", v);
+    }
+    if (dtype == CNH_F32) {
+        float f = (float)c;
+        if (std::isnan(f))
+            return "((T)__builtin_nanf(\"\"))";
+        if (std::isinf(f))
+            return f > 0 ? "((T)__builtin_inff())" : "((T)(-__builtin_inff()))";
+        return fmt("((T)(%af))", (double)f);
+    }
+    if (std::isnan(c))
+        return "((T)__builtin_nan(\"\"))";
+    if (std::isinf(c))
+        return c > 0 ? "((T)__builtin_inf())" : "((T)(-__builtin_inf()))";
+    return fmt("((T)(%a))", c);
+}
+
+struct Value {
+    std::string expr;
+    bool scalar = false;
+    bool valid = false;
+};
+
+std::string leaf_key(const cnh_ast_node& root, int oi, const cnh_ast_node& op) {
+    // Same identity rule as the upstream leafUseKey (src/jit.cpp:265-284): name, rank, region.
+    std::string key = fmt("%d|%d", op.result_name, op.ndims);
+    if (!root.has_operand_region[oi])
+        return key + "|null";
+    const cnh_region& r = root.operand_regions[oi];
+    if (r.is_global)
+        return key + "|global";
+    for (int d = 0; d < op.ndims && d < CNH_MAX_ND; ++d)
+        key += fmt("|%d:%d:%d", r.start[d], r.stop[d], r.step[d]);
+    return key;
+}
+
+std::string binop(int dtype, int opc, const std::string& a, const std::string& b) {
+    if (is_int(dtype)) {
+        switch (opc) {
+        case CNH_OP_ADD: return "(T)((UT)" + a + " + (UT)" + b + ")";
+        case CNH_OP_SUB: return "(T)((UT)" + a + " - (UT)" + b + ")";
+        case CNH_OP_MUL: return "(T)((UT)" + a + " * (UT)" + b + ")";
+        default: return "cn_idiv(" + a + ", " + b + ")";
+        }
+    }
+    const char* sym = opc == CNH_OP_ADD ? "+" : opc == CNH_OP_SUB ? "-" : opc == CNH_OP_MUL ? "*" : "/";
+    return a + " " + sym + " " + b;
+}
+
+} // namespace
+
+int build_group_program(const cnh_ast* ast, int dtype, int ndims, GroupProgram& p,
+                        std::string& err) {
+    if (!ast || !ast->nodes || !ast->roots || ast->n_roots <= 0) {
+        err = "empty AST";
+        return -2;
+    }
+    if (ndims < 1 || ndims > CNH_MAX_ND) {
+        err = fmt("ndims %d not in 1..3", ndims);
+        return -2;
+    }
+    if (dtype < 0 || dtype > 3) {
+        err = fmt("unknown dtype %d", dtype);
+        return -2;
+    }
+    for (int r = 0; r < ast->n_roots; ++r)
+        if (ast->roots[r] < 0 || ast->roots[r] >= ast->n_nodes) {
+            err = "root index out of range";
+            return -2;
+        }
+    p = GroupProgram();
+    p.dtype = dtype;
+    p.ndims = ndims;
+
+    std::map<int, int> internal;
+    for (int r = 0; r < ast->n_roots; ++r)
+        internal[ast->nodes[ast->roots[r]].result_name] = 1;
+
+    std::map<std::string, int> load_by_key;
+    std::map<int, int> bcast_by_name;
+    std::map<int, Value> values; // result_name -> expression
+
+    for (int r = 0; r < ast->n_roots; ++r) {
+        const cnh_ast_node& root = ast->nodes[ast->roots[r]];
+        if (root.n_operands < 0 || root.n_operands > 2) {
+            err = "operand count out of range";
+            return -2;
+        }
+        for (int oi = 0; oi < root.n_operands; ++oi) {
+            int on = root.operands[oi];
+            if (on < 0)
+                continue;
+            if (on >= ast->n_nodes) {
+                err = "operand index out of range";
+                return -2;
+            }
+            const cnh_ast_node& op = ast->nodes[on];
+            if (internal.count(op.result_name))
+                continue;
+            if (root.opcode == CNH_OP_SET_REGION && oi == 0)
+                continue;
+            if (op.opcode != CNH_OP_NOOP && op.opcode != CNH_OP_CREATE)
+                continue;
+            if (op.is_scalar) {
+                Value v;
+                v.expr = literal(dtype, op.scalar);
+                v.scalar = true;
+                v.valid = true;
+                values[op.result_name] = v;
+            } else if (op.is_broadcast) {
+                if (!bcast_by_name.count(op.result_name)) {
+                    bcast_by_name[op.result_name] = (int)p.bcast_nodes.size();
+                    p.bcast_nodes.push_back(on);
+                }
+                Value v;
+                v.expr = fmt("s[%d]", bcast_by_name[op.result_name]);
+                v.scalar = true;
+                v.valid = true;
+                values[op.result_name] = v;
+            } else {
+                std::string key = leaf_key(root, oi, op);
+                LeafUse u;
+                u.node = on;
+                u.root = r;
+                u.operand = oi;
+                u.name = op.result_name;
+                u.has_region = root.has_operand_region[oi] && !root.operand_regions[oi].is_global;
+                u.region = root.operand_regions[oi];
+                auto it = load_by_key.find(key);
+                if (it == load_by_key.end()) {
+                    u.load = (int)p.load_leaf.size();
+                    load_by_key[key] = u.load;
+                    p.load_leaf.push_back((int)p.leaves.size());
+                } else {
+                    u.load = it->second;
+                    p.load_leaf[u.load] = (int)p.leaves.size(); // the later argument wins
+                }
+                p.leaves.push_back(u);
+            }
+        }
+    }
+
+    auto lookup = [&](const cnh_ast_node& root, int oi) -> Value {
+        Value none;
+        if (oi >= root.n_operands || root.operands[oi] < 0)
+            return none;
+        const cnh_ast_node& op = ast->nodes[root.operands[oi]];
+        std::string key = leaf_key(root, oi, op);
+        if (root.has_operand_region[oi]) {
+            auto it = load_by_key.find(key);
+            if (it != load_by_key.end()) {
+                Value v;
+                v.expr = fmt("l[%d]", it->second);
+                v.valid = true;
+                return v;
+            }
+        }
+        auto it = values.find(op.result_name);
+        if (it != values.end())
+            return it->second;
+        auto it2 = load_by_key.find(key);
+        if (it2 != load_by_key.end()) {
+            Value v;
+            v.expr = fmt("l[%d]", it2->second);
+            v.valid = true;
+            return v;
+        }
+        return none;
+    };
+
+    int n_tmp = 0;
+    std::ostringstream body;
+    for (int r = 0; r < ast->n_roots; ++r) {
+        const cnh_ast_node& root = ast->nodes[ast->roots[r]];
+        int opc = root.opcode;
+        if (opc == CNH_OP_NOOP || opc == CNH_OP_CREATE)
+            continue;
+        Value res;
+        if (opc == CNH_OP_SET_REGION) {
+            res = lookup(root, 1);
+            if (!res.valid) {
+                err = "SET_REGION without a usable right-hand side";
+                return -10;
+            }
+        } else if (opc >= CNH_OP_ADD && opc <= CNH_OP_DIV) {
+            Value a = lookup(root, 0), b = lookup(root, 1);
+            if (!a.valid || !b.valid) {
+                err = "binary op with an unresolved operand";
+                return -11;
+            }
+            std::string name = fmt("t%d", n_tmp++);
+            body << "    const T " << name << " = " << binop(dtype, opc, a.expr, b.expr) << ";\n";
+            res.expr = name;
+            res.scalar = a.scalar && b.scalar;
+            res.valid = true;
+        } else if (opc == CNH_OP_TANH || opc == CNH_OP_EXP) {
+            if (is_int(dtype)) {
+                err = "tanh/exp have no integer form";
+                return -21;
+            }
+            Value a = lookup(root, 0);
+            if (!a.valid || a.scalar) {
+                err = "unary op needs an array operand";
+                return -12;
+            }
+            std::string name = fmt("t%d", n_tmp++);
+            const char* fn = opc == CNH_OP_TANH ? "cn_tanh" : "cn_exp";
+            body << "    const T " << name << " = " << fn << "(" << a.expr << ");\n";
+            res.expr = name;
+            res.valid = true;
+            p.uses_transcendental = true;
+        } else {
+            err = fmt("opcode %d cannot be part of a fused group", opc);
+            return -13;
+        }
+        values[root.result_name] = res;
+    }
+
+    for (int r = 0; r < ast->n_roots; ++r) {
+        const cnh_ast_node& root = ast->nodes[ast->roots[r]];
+        if (root.opcode == CNH_OP_NOOP || root.opcode == CNH_OP_CREATE || root.is_temp)
+            continue;
+        auto it = values.find(root.result_name);
+        if (it == values.end() || !it->second.valid) {
+            err = "output root without a value";
+            return -15;
+        }
+        p.out_roots.push_back(r);
+        bool sr = root.opcode == CNH_OP_SET_REGION;
+        p.out_is_set_region.push_back(sr ? 1 : 0);
+        int target = root.result_name;
+        if (sr && root.n_operands > 0 && root.operands[0] >= 0)
+            target = ast->nodes[root.operands[0]].result_name;
+        p.out_target.push_back(target);
+        p.out_region.push_back(root.region);
+        p.out_expr.push_back(it->second.expr);
+    }
+    for (size_t j = 0; j < p.out_expr.size(); ++j)
+        body << "    o[" << j << "] = " << p.out_expr[j] << ";\n";
+    p.body = body.str();
+    return 0;
+}
+
+namespace {
+
+// Text shared by every variant: element type, scalar block, helpers and the group body.
+std::string prelude(const GroupProgram& p) {
+    int NL = (int)p.load_leaf.size(), NS = (int)p.bcast_nodes.size(), NO = (int)p.out_roots.size();
+    std::ostringstream s;
+    s << "// generated by libcnhip for one fused group; dtype " << dtype_ctype(p.dtype) << ", rank "
+      << p.ndims << "\n";
+    s << "typedef " << dtype_ctype(p.dtype) << " T;\n";
+    s << "typedef unsigned " << (p.dtype == CNH_I64 ? "long long" : "int") << " UT;\n";
+    s << "typedef long long i64;\n";
+    s << "#define NL " << NL << "\n#define NS " << NS << "\n#define NO " << NO << "\n";
+    s << "#define NLA " << (NL > 0 ? NL : 1) << "\n#define NSA " << (NS > 0 ? NS : 1)
+      << "\n#define NOA " << (NO > 0 ? NO : 1) << "\n";
+    s << "struct Scal { const T* p[NSA]; T v[NSA]; };\n";
+    if (is_int(p.dtype)) {
+        // Truncating signed division; x/0 -> 0 and MIN/-1 -> MIN are fixed here because the
+        // upstream operation (arith.divsi) leaves both undefined.
+        s << "__device__ __forceinline__ T cn_idiv(T a, T b) {\n"
+             "    if (b == 0) return 0;\n"
+             "    if (b == -1) return (T)((UT)0 - (UT)a);\n"
+             "    return a / b;\n}\n";
+    } else if (p.dtype == CNH_F64) {
+        s << "__device__ __forceinline__ T cn_exp(T x) { return exp(x); }\n"
+             "__device__ __forceinline__ T cn_tanh(T x) { return tanh(x); }\n";
+    } else {
+        s << "__device__ __forceinline__ T cn_exp(T x) { return expf(x); }\n"
+             "__device__ __forceinline__ T cn_tanh(T x) { return tanhf(x); }\n";
+    }
+    s << "__device__ __forceinline__ void load_scalars(const Scal& sc, T* s) {\n"
+         "#pragma unroll\n"
+         "    for (int i = 0; i < NS; ++i) s[i] = sc.p[i] ? *sc.p[i] : sc.v[i];\n}\n";
+    s << "__device__ __forceinline__ void group_eval(const T* l, const T* s, T* o) {\n"
+      << "    (void)l; (void)s;\n"
+      << p.body << "}\n";
+    s << "template <typename S> __device__ __forceinline__ int find_seg(const S* segs, int n, i64 "
+         "blk) {\n"
+         "    int lo = 0, hi = n - 1;\n"
+         "    while (lo < hi) { int mid = (lo + hi + 1) >> 1; if (segs[mid].blk0 <= blk) lo = mid; "
+         "else hi = mid - 1; }\n"
+         "    return lo;\n}\n";
+    return s.str();
+}
+
+std::string flat_source(const GroupProgram& p) {
+    int vec = 16 / dtype_size(p.dtype);
+    int unr = 4;
+    std::ostringstream s;
+    s << prelude(p);
+    s << "#define VECW " << vec << "\n#define UNR " << unr << "\n";
+    s << R"(
+// Contiguous segments: every memref of a partition is dense and has the same element count.
+struct Seg { i64 n; i64 blk0; const T* in[NLA]; T* out[NOA]; };
+template <int VEC> struct alignas(VEC * sizeof(T)) Pack { T x[VEC]; };
+
+template <int VEC, int U>
+__device__ __forceinline__ void flat_run(const Seg& sg, i64 blk, const T* s) {
+    typedef Pack<VEC> P;
+    const i64 per_block = 256LL * VEC * U;
+    const i64 base = blk * per_block;
+    const i64 n = sg.n;
+    if (base + per_block <= n) {
+        P lv[NLA][U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const i64 i = base + ((i64)u * 256 + threadIdx.x) * VEC;
+#pragma unroll
+            for (int k = 0; k < NL; ++k) lv[k][u] = *reinterpret_cast<const P*>(sg.in[k] + i);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const i64 i = base + ((i64)u * 256 + threadIdx.x) * VEC;
+            P ov[NOA];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                T l[NLA], o[NOA];
+#pragma unroll
+                for (int k = 0; k < NL; ++k) l[k] = lv[k][u].x[e];
+                group_eval(l, s, o);
+#pragma unroll
+                for (int j = 0; j < NO; ++j) ov[j].x[e] = o[j];
+            }
+#pragma unroll
+            for (int j = 0; j < NO; ++j) *reinterpret_cast<P*>(sg.out[j] + i) = ov[j];
+        }
+    } else {
+#pragma unroll
+        for (int u = 0; u < U * VEC; ++u) {
+            const i64 i = base + (i64)u * 256 + threadIdx.x;
+            if (i < n) {
+                T l[NLA], o[NOA];
+#pragma unroll
+                for (int k = 0; k < NL; ++k) l[k] = sg.in[k][i];
+                group_eval(l, s, o);
+#pragma unroll
+                for (int j = 0; j < NO; ++j) sg.out[j][i] = o[j];
+            }
+        }
+    }
+}
+
+extern "C" __global__ __launch_bounds__(256) void grp_flat_v(const Seg* segs, int nseg, Scal sc) {
+    T s[NSA]; load_scalars(sc, s);
+    const int k = find_seg(segs, nseg, (i64)blockIdx.x);
+    flat_run<VECW, UNR>(segs[k], (i64)blockIdx.x - segs[k].blk0, s);
+}
+extern "C" __global__ __launch_bounds__(256) void grp_flat_s(const Seg* segs, int nseg, Scal sc) {
+    T s[NSA]; load_scalars(sc, s);
+    const int k = find_seg(segs, nseg, (i64)blockIdx.x);
+    flat_run<1, UNR * VECW>(segs[k], (i64)blockIdx.x - segs[k].blk0, s);
+}
+extern "C" __global__ __launch_bounds__(256) void grp_flat1_v(Seg seg, Scal sc) {
+    T s[NSA]; load_scalars(sc, s);
+    flat_run<VECW, UNR>(seg, (i64)blockIdx.x, s);
+}
+extern "C" __global__ __launch_bounds__(256) void grp_flat1_s(Seg seg, Scal sc) {
+    T s[NSA]; load_scalars(sc, s);
+    flat_run<1, UNR * VECW>(seg, (i64)blockIdx.x, s);
+}
+)";
+    return s.str();
+}
+
+std::string nd_source(const GroupProgram& p) {
+    std::ostringstream s;
+    s << prelude(p);
+    s << R"(
+// Strided cells: arbitrary memref descriptors (offset folded into the pointer), rank padded to 3.
+struct Cell {
+    i64 sizes[3]; i64 blk0; i64 nchunks;
+    const T* in[NLA]; i64 istr[NLA][3];
+    T* out[NOA]; i64 ostr[NOA][3];
+};
+#define ND_PER_THREAD 4
+
+__device__ __forceinline__ void nd_run(const Cell& c, i64 blk, const T* s) {
+    const i64 outer = blk / c.nchunks;
+    const i64 chunk = blk - outer * c.nchunks;
+    const i64 i1 = outer % c.sizes[1];
+    const i64 i0 = outer / c.sizes[1];
+    const i64 x0 = chunk * (256 * ND_PER_THREAD) + threadIdx.x;
+    T lv[NLA][ND_PER_THREAD];
+#pragma unroll
+    for (int u = 0; u < ND_PER_THREAD; ++u) {
+        const i64 x = x0 + (i64)u * 256;
+        if (x < c.sizes[2]) {
+#pragma unroll
+            for (int k = 0; k < NL; ++k)
+                lv[k][u] = c.in[k][i0 * c.istr[k][0] + i1 * c.istr[k][1] + x * c.istr[k][2]];
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < ND_PER_THREAD; ++u) {
+        const i64 x = x0 + (i64)u * 256;
+        if (x < c.sizes[2]) {
+            T l[NLA], o[NOA];
+#pragma unroll
+            for (int k = 0; k < NL; ++k) l[k] = lv[k][u];
+            group_eval(l, s, o);
+#pragma unroll
+            for (int j = 0; j < NO; ++j)
+                c.out[j][i0 * c.ostr[j][0] + i1 * c.ostr[j][1] + x * c.ostr[j][2]] = o[j];
+        }
+    }
+}
+
+extern "C" __global__ __launch_bounds__(256) void grp_nd(const Cell* cells, int ncell, Scal sc) {
+    T s[NSA]; load_scalars(sc, s);
+    const int k = find_seg(cells, ncell, (i64)blockIdx.x);
+    nd_run(cells[k], (i64)blockIdx.x - cells[k].blk0, s);
+}
+extern "C" __global__ __launch_bounds__(256) void grp_nd1(Cell cell, Scal sc) {
+    T s[NSA]; load_scalars(sc, s);
+    nd_run(cell, (i64)blockIdx.x, s);
+}
+)";
+    return s.str();
+}
+
+std::string tiles_source(const GroupProgram& p) {
+    std::ostringstream s;
+    s << prelude(p);
+    s << R"(
+// Gather over tiled arrays resident on this device: every element of every destination tile is
+// produced by one thread, which resolves each shifted/strided input coordinate to its owning
+// tile (tile edge is a power of two) and reads it there. Rank padded to 3.
+struct Tiled {
+    int shift; int tile; int off[3]; int shape[3]; int glo[3]; int grid[3];
+    const T* const* tiles;
+};
+struct DTile { i64 blk0; int cs[3]; int w[3]; int nchunks; int pad; T* dst; const T* cur; };
+struct LeafReg { int arr; int start[3]; int step[3]; };
+struct TilesArgs {
+    int out_off[3];
+    int rs[3], re[3], rst[3];   // assigned region in the target's own coordinates
+    LeafReg leaf[NLA];
+};
+#define TL_PER_THREAD 4
+
+__device__ __forceinline__ T tiled_read(const Tiled& a, int g0, int g1, int g2) {
+    const int t0 = g0 >> a.shift, t1 = g1 >> a.shift, t2 = g2 >> a.shift;
+    const int lo0 = max(t0 << a.shift, a.off[0]);
+    const int lo1 = max(t1 << a.shift, a.off[1]);
+    const int lo2 = max(t2 << a.shift, a.off[2]);
+    const int w1 = min((t1 + 1) << a.shift, a.off[1] + a.shape[1]) - lo1;
+    const int w2 = min((t2 + 1) << a.shift, a.off[2] + a.shape[2]) - lo2;
+    const int ti = ((t0 - a.glo[0]) * a.grid[1] + (t1 - a.glo[1])) * a.grid[2] + (t2 - a.glo[2]);
+    const T* base = a.tiles[ti];
+    return base[((i64)(g0 - lo0) * w1 + (g1 - lo1)) * w2 + (g2 - lo2)];
+}
+
+extern "C" __global__ __launch_bounds__(256) void grp_tiles(const Tiled* arrs, const DTile* dts,
+                                                            int ndt, TilesArgs ta, Scal sc) {
+    T s[NSA]; load_scalars(sc, s);
+    const int k = find_seg(dts, ndt, (i64)blockIdx.x);
+    const DTile& dt = dts[k];
+    const i64 blk = (i64)blockIdx.x - dt.blk0;
+    const i64 outer = blk / dt.nchunks;
+    const int chunk = (int)(blk - outer * dt.nchunks);
+    const int l1 = (int)(outer % dt.w[1]);
+    const int l0 = (int)(outer / dt.w[1]);
+    const int a0 = dt.cs[0] + l0 - ta.out_off[0];
+    const int a1 = dt.cs[1] + l1 - ta.out_off[1];
+    const bool in01 = a0 >= ta.rs[0] && a0 < ta.re[0] && (a0 - ta.rs[0]) % ta.rst[0] == 0 &&
+                      a1 >= ta.rs[1] && a1 < ta.re[1] && (a1 - ta.rs[1]) % ta.rst[1] == 0;
+    const int k0 = (a0 - ta.rs[0]) / ta.rst[0];
+    const int k1 = (a1 - ta.rs[1]) / ta.rst[1];
+#pragma unroll
+    for (int u = 0; u < TL_PER_THREAD; ++u) {
+        const int l2 = chunk * (256 * TL_PER_THREAD) + u * 256 + (int)threadIdx.x;
+        if (l2 >= dt.w[2]) continue;
+        const i64 di = ((i64)l0 * dt.w[1] + l1) * dt.w[2] + l2;
+        const int a2 = dt.cs[2] + l2 - ta.out_off[2];
+        const bool inside = in01 && a2 >= ta.rs[2] && a2 < ta.re[2] &&
+                            (a2 - ta.rs[2]) % ta.rst[2] == 0;
+        if (inside) {
+            const int k2 = (a2 - ta.rs[2]) / ta.rst[2];
+            T l[NLA], o[NOA];
+#pragma unroll
+            for (int q = 0; q < NL; ++q) {
+                const LeafReg& lr = ta.leaf[q];
+                const Tiled& a = arrs[lr.arr];
+                l[q] = tiled_read(a, lr.start[0] + k0 * lr.step[0] + a.off[0],
+                                  lr.start[1] + k1 * lr.step[1] + a.off[1],
+                                  lr.start[2] + k2 * lr.step[2] + a.off[2]);
+            }
+            group_eval(l, s, o);
+            dt.dst[di] = o[0];
+        } else if (dt.cur != nullptr && dt.cur != dt.dst) {
+            dt.dst[di] = dt.cur[di];
+        }
+    }
+}
+)";
+    return s.str();
+}
+
+} // namespace
+
+std::string slide_source(const GroupProgram& p, std::string& err); // codegen_slide.cpp
+
+int emit_variant_source(const GroupProgram& p, const std::string& variant, std::string& src,
+                        std::string& err) {
+    if (p.out_roots.empty()) {
+        err = "group has no output root";
+        return -16;
+    }
+    if (variant == "flat") {
+        src = flat_source(p);
+        return 0;
+    }
+    if (variant == "nd") {
+        src = nd_source(p);
+        return 0;
+    }
+    if (variant == "tiles") {
+        if (p.out_roots.size() != 1) {
+            err = "the tiled variant needs exactly one output root";
+            return -17;
+        }
+        src = tiles_source(p);
+        return 0;
+    }
+    if (variant == "slide") {
+        src = slide_source(p, err);
+        return src.empty() ? -18 : 0;
+    }
+    err = "unknown kernel variant '" + variant + "'";
+    return -2;
+}
+
+} // namespace cnh

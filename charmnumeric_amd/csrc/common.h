@@ -1,0 +1,56 @@
+// Shared internals of libcnhip (not part of the C ABI).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+
+#include "../../include/cnhip.h"
+
+namespace cnh {
+
+// Thread-local error text behind cnh_last_error().
+int set_error(int code, const char* fmt, ...);
+std::string& error_slot();
+
+#define CNH_HIP(expr)                                                                            \
+    do {                                                                                         \
+        hipError_t _e = (expr);                                                                  \
+        if (_e != hipSuccess)                                                                    \
+            return cnh::set_error(-100, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e),   \
+                                  __FILE__, __LINE__);                                           \
+    } while (0)
+
+#define CNH_CHECK(cond, code, ...)                                                               \
+    do {                                                                                         \
+        if (!(cond))                                                                             \
+            return cnh::set_error(code, __VA_ARGS__);                                            \
+    } while (0)
+
+inline int dtype_size(int dt) {
+    switch (dt) {
+    case CNH_F32:
+    case CNH_I32: return 4;
+    case CNH_F64:
+    case CNH_I64: return 8;
+    }
+    return 0;
+}
+
+inline hipStream_t as_stream(cnh_stream s) { return reinterpret_cast<hipStream_t>(s); }
+
+// Lazily selects the device on first use of any entry point.
+int ensure_init();
+
+// Device scratch for reduction partials, one region per stream handle so that calls on
+// different streams never share slots. Returns a device pointer to `bytes` bytes.
+int reduce_workspace(hipStream_t s, size_t bytes, void** out);
+
+// Descriptor tables (per-partition pointers/shapes) live on the device. Identical tables are
+// uploaded once and found again by content hash, so steady-state launches issue no copy.
+int desc_upload(const void* host, size_t bytes, hipStream_t s, const void** dev_out);
+
+} // namespace cnh

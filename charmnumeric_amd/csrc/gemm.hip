@@ -1,0 +1,216 @@
+// C += A * B for row-major panels with row strides.
+// Upstream: Eigen `C.noalias() += A*B` / KokkosBlas::gemm on strided sub-block views, one call per
+// arriving panel pair (src/backend_internal.hpp:113-133, src/executor_incremental.cpp:97-132).
+// fp64 is the one dense contraction of the path, so it runs on the matrix cores
+// (v_mfma_f64_16x16x4_f64): 64x64 workgroup tiles, four wavefronts of 32x32, K in steps of 16
+// staged through double-buffered LDS. Other element types use a plain LDS-tiled kernel.
+#include "common.h"
+
+using namespace cnh;
+
+namespace {
+
+typedef double v4d __attribute__((ext_vector_type(4)));
+
+constexpr int BM = 64, BN = 64, BK = 16, PAD = 16;
+
+// Workgroup ids are dealt round-robin to the 8 XCDs; give every XCD a contiguous run of logical
+// tiles so that the workgroups sharing a B column panel also share one L2.
+__device__ __forceinline__ int xcd_remap(int b, int nblocks) {
+    if (nblocks % 8 != 0)
+        return b;
+    return (b % 8) * (nblocks / 8) + b / 8;
+}
+
+template <bool FULL>
+__global__ __launch_bounds__(256) void gemm_f64_mfma(int M, int N, int K,
+                                                     const double* __restrict__ A, int64_t lda,
+                                                     const double* __restrict__ B, int64_t ldb,
+                                                     double* __restrict__ C, int64_t ldc) {
+    __shared__ double As[2][BK][BM + PAD];
+    __shared__ double Bs[2][BK][BN + PAD];
+    const int nbm = (M + BM - 1) / BM, nbn = (N + BN - 1) / BN;
+    const int logical = xcd_remap(blockIdx.x, nbm * nbn);
+    const int bn = logical / nbm, bm = logical - bn * nbm;
+    const int m0 = bm * BM, n0 = bn * BN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    // staging assignment: A tile 64 rows x 16 k, B tile 16 k x 64 n; 4 doubles per lane each
+    const int a_row = tid >> 2, a_k = (tid & 3) * 4;
+    const int b_k = tid >> 4, b_n = (tid & 15) * 4;
+
+    double ra[4], rb[4];
+    auto fetch = [&](int k0) {
+        const int gr = m0 + a_row;
+        const int gk = k0 + a_k;
+        if (FULL) {
+            const double2 v0 = *reinterpret_cast<const double2*>(A + (int64_t)gr * lda + gk);
+            const double2 v1 = *reinterpret_cast<const double2*>(A + (int64_t)gr * lda + gk + 2);
+            ra[0] = v0.x; ra[1] = v0.y; ra[2] = v1.x; ra[3] = v1.y;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                ra[j] = (gr < M && gk + j < K) ? A[(int64_t)gr * lda + gk + j] : 0.0;
+        }
+        const int bk = k0 + b_k;
+        const int gn = n0 + b_n;
+        if (FULL) {
+            const double2 v0 = *reinterpret_cast<const double2*>(B + (int64_t)bk * ldb + gn);
+            const double2 v1 = *reinterpret_cast<const double2*>(B + (int64_t)bk * ldb + gn + 2);
+            rb[0] = v0.x; rb[1] = v0.y; rb[2] = v1.x; rb[3] = v1.y;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                rb[j] = (bk < K && gn + j < N) ? B[(int64_t)bk * ldb + gn + j] : 0.0;
+        }
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            As[buf][a_k + j][a_row] = ra[j];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            Bs[buf][b_k][b_n + j] = rb[j];
+    };
+
+    v4d acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+            acc[i][j] = (v4d){0.0, 0.0, 0.0, 0.0};
+
+    const int nk = (K + BK - 1) / BK;
+    fetch(0);
+    stage(0);
+    __syncthreads();
+    const int lr = lane & 15, lk = lane >> 4;
+    for (int t = 0; t < nk; ++t) {
+        const int buf = t & 1;
+        if (t + 1 < nk)
+            fetch((t + 1) * BK);
+#pragma unroll
+        for (int ks = 0; ks < BK / 4; ++ks) {
+            const int kk = ks * 4 + lk;
+            double a[2], b[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+                a[i] = As[buf][kk][wm * 32 + i * 16 + lr];
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                b[j] = Bs[buf][kk][wn * 32 + j * 16 + lr];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+        if (t + 1 < nk) {
+            stage(buf ^ 1);
+            __syncthreads();
+        }
+    }
+    // D layout of the 16x16x4 f64 instruction: lane holds column (lane % 16) of rows
+    // 4*(lane / 16) + {0,1,2,3}.
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int col = n0 + wn * 32 + j * 16 + lr;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int row = m0 + wm * 32 + i * 16 + lk * 4 + r;
+                if (FULL || (row < M && col < N)) {
+                    double* c = C + (int64_t)row * ldc + col;
+                    *c = *c + acc[i][j][r];
+                }
+            }
+        }
+}
+
+template <typename T>
+struct Acc {
+    typedef T type;
+};
+template <>
+struct Acc<int32_t> {
+    typedef uint32_t type;
+};
+template <>
+struct Acc<int64_t> {
+    typedef uint64_t type;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_tiled_generic(int M, int N, int K,
+                                                          const T* __restrict__ A, int64_t lda,
+                                                          const T* __restrict__ B, int64_t ldb,
+                                                          T* __restrict__ C, int64_t ldc) {
+    typedef typename Acc<T>::type U;
+    __shared__ T As[16][17];
+    __shared__ T Bs[16][17];
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const int row = blockIdx.y * 16 + ty, col = blockIdx.x * 16 + tx;
+    U acc = 0;
+    for (int k0 = 0; k0 < K; k0 += 16) {
+        As[ty][tx] = (row < M && k0 + tx < K) ? A[(int64_t)row * lda + k0 + tx] : (T)0;
+        Bs[ty][tx] = (k0 + ty < K && col < N) ? B[(int64_t)(k0 + ty) * ldb + col] : (T)0;
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 16; ++k)
+            acc += (U)As[ty][k] * (U)Bs[k][tx];
+        __syncthreads();
+    }
+    if (row < M && col < N)
+        C[(int64_t)row * ldc + col] = (T)((U)C[(int64_t)row * ldc + col] + acc);
+}
+
+template <typename T>
+int run_generic(int M, int N, int K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C,
+                int64_t ldc, hipStream_t st) {
+    dim3 grid((N + 15) / 16, (M + 15) / 16);
+    CNH_CHECK(grid.y <= 65535, -3, "cnh_gemm_acc: M too large for this element type");
+    hipLaunchKernelGGL(gemm_tiled_generic<T>, grid, dim3(256), 0, st, M, N, K, (const T*)A, lda,
+                       (const T*)B, ldb, (T*)C, ldc);
+    CNH_HIP(hipGetLastError());
+    return 0;
+}
+
+} // namespace
+
+extern "C" int cnh_gemm_acc(int dtype, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda,
+                            const void* B, int64_t ldb, void* C, int64_t ldc, cnh_stream s) {
+    if (int rc = ensure_init())
+        return rc;
+    CNH_CHECK(M >= 0 && N >= 0 && K >= 0, -2, "cnh_gemm_acc: negative extent");
+    CNH_CHECK(M < (1ll << 30) && N < (1ll << 30) && K < (1ll << 30), -3,
+              "cnh_gemm_acc: extent too large");
+    if (M == 0 || N == 0 || K == 0)
+        return 0;
+    CNH_CHECK(A && B && C, -2, "cnh_gemm_acc: null pointer");
+    CNH_CHECK(lda >= K && ldb >= N && ldc >= N, -2, "cnh_gemm_acc: row stride shorter than the row");
+    hipStream_t st = as_stream(s);
+    switch (dtype) {
+    case CNH_F64: {
+        const int64_t blocks = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+        CNH_CHECK(blocks < (1ll << 31), -3, "cnh_gemm_acc: too many tiles");
+        const bool full = (M % BM == 0) && (N % BN == 0) && (K % BK == 0) && (lda % 2 == 0) &&
+                          (ldb % 2 == 0) && (((uintptr_t)A & 15) == 0) && (((uintptr_t)B & 15) == 0);
+        if (full)
+            hipLaunchKernelGGL(gemm_f64_mfma<true>, dim3((unsigned)blocks), dim3(256), 0, st, (int)M,
+                               (int)N, (int)K, (const double*)A, lda, (const double*)B, ldb,
+                               (double*)C, ldc);
+        else
+            hipLaunchKernelGGL(gemm_f64_mfma<false>, dim3((unsigned)blocks), dim3(256), 0, st,
+                               (int)M, (int)N, (int)K, (const double*)A, lda, (const double*)B, ldb,
+                               (double*)C, ldc);
+        CNH_HIP(hipGetLastError());
+        return 0;
+    }
+    case CNH_F32: return run_generic<float>((int)M, (int)N, (int)K, A, lda, B, ldb, C, ldc, st);
+    case CNH_I32: return run_generic<int32_t>((int)M, (int)N, (int)K, A, lda, B, ldb, C, ldc, st);
+    case CNH_I64: return run_generic<int64_t>((int)M, (int)N, (int)K, A, lda, B, ldb, C, ldc, st);
+    }
+    return set_error(-2, "unknown dtype %d", dtype);
+}

@@ -1,0 +1,247 @@
+// Bandwidth-bound matvec over row-major tiles, and the 1-D partial accumulate.
+// Upstream: every 2-D tile chare runs an Eigen GEMV on its sub-matrix and ships the partial rows
+// to the 1-D owner, which adds them in arrival order (src/backend_internal.hpp:28-41,
+// src/execute_node.cpp:116-273,489-583). Here one launch covers the whole tile grid: one
+// wavefront per matrix row walks the column tiles in index order with 128-bit loads, so the
+// matrix is read from HBM exactly once and the per-row sum has a fixed order.
+#include "common.h"
+
+#include <vector>
+
+using namespace cnh;
+
+namespace {
+
+struct ColTile {
+    const void* base; // first element of tile (ti, tj)
+    int64_t ld;       // row stride of that tile in elements
+    int64_t ncols;    // columns held by that tile
+    int64_t xoff;     // offset of its first column in x
+};
+
+template <typename T>
+struct Acc {
+    typedef T type;
+};
+template <>
+struct Acc<int32_t> {
+    typedef uint32_t type;
+};
+template <>
+struct Acc<int64_t> {
+    typedef uint64_t type;
+};
+
+template <typename A>
+__device__ __forceinline__ A wave_sum(A v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        if (sizeof(A) == 8) {
+            unsigned long long u;
+            __builtin_memcpy(&u, &v, 8);
+            unsigned lo = (unsigned)u, hi = (unsigned)(u >> 32);
+            lo = __shfl_down(lo, off, 64);
+            hi = __shfl_down(hi, off, 64);
+            u = ((unsigned long long)hi << 32) | lo;
+            A o;
+            __builtin_memcpy(&o, &u, 8);
+            v = v + o;
+        } else {
+            unsigned u;
+            __builtin_memcpy(&u, &v, 4);
+            u = __shfl_down(u, off, 64);
+            A o;
+            __builtin_memcpy(&o, &u, 4);
+            v = v + o;
+        }
+    }
+    return v;
+}
+
+constexpr int kWavesPerBlock = 4;
+constexpr int kUnroll = 8;
+
+// tiles[ti * ncol_tiles + tj]; row r belongs to tile row r / tile_rows.
+template <typename T, bool VEC16>
+__global__ __launch_bounds__(kWavesPerBlock * 64) void gemv_rows(const ColTile* __restrict__ tiles,
+                                                                 int ncol_tiles, int64_t tile_rows,
+                                                                 int64_t rows,
+                                                                 const T* __restrict__ x,
+                                                                 T* __restrict__ y, int beta) {
+    typedef typename Acc<T>::type A;
+    constexpr int VEC = 16 / sizeof(T);
+    struct alignas(16) P {
+        T v[VEC];
+    };
+    const int lane = threadIdx.x & 63;
+    const int64_t r = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    if (r >= rows)
+        return;
+    const int64_t ti = r / tile_rows;
+    const int64_t lr = r - ti * tile_rows;
+    A total = 0;
+    for (int tj = 0; tj < ncol_tiles; ++tj) {
+        const ColTile ct = tiles[ti * ncol_tiles + tj];
+        const T* row = (const T*)ct.base + lr * ct.ld;
+        const T* xv = x + ct.xoff;
+        A acc[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+            acc[u] = 0;
+        int64_t c = 0;
+        if (VEC16) {
+            const int64_t step = 64 * VEC;
+            for (; c + kUnroll * step <= ct.ncols; c += kUnroll * step) {
+                P av[kUnroll], xs[kUnroll];
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u)
+                    av[u] = *reinterpret_cast<const P*>(row + c + u * step + lane * VEC);
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u)
+                    xs[u] = *reinterpret_cast<const P*>(xv + c + u * step + lane * VEC);
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e)
+                        acc[u] += (A)av[u].v[e] * (A)xs[u].v[e];
+            }
+            for (; c + step <= ct.ncols; c += step) {
+                P av = *reinterpret_cast<const P*>(row + c + lane * VEC);
+                P xs = *reinterpret_cast<const P*>(xv + c + lane * VEC);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e)
+                    acc[0] += (A)av.v[e] * (A)xs.v[e];
+            }
+        }
+        for (int64_t j = c + lane; j < ct.ncols; j += 64)
+            acc[1] += (A)row[j] * (A)xv[j];
+        A part = 0;
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+            part += acc[u];
+        part = wave_sum<A>(part);
+        total = tj == 0 ? part : total + part; // column tiles added in index order
+    }
+    if (lane == 0)
+        y[r] = beta ? (T)((A)y[r] + total) : (T)total;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void axpy1_kernel(int64_t n, const T* __restrict__ p,
+                                                    T* __restrict__ y) {
+    typedef typename Acc<T>::type A;
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n)
+        y[i] = (T)((A)y[i] + (A)p[i]);
+}
+
+template <typename T>
+int run_gemv(const std::vector<ColTile>& tiles, int ncol_tiles, int64_t tile_rows, int64_t rows,
+             const void* x, void* y, int beta, hipStream_t st) {
+    bool vec = ((uintptr_t)x & 15) == 0;
+    constexpr int VEC = 16 / sizeof(T);
+    for (const ColTile& t : tiles) {
+        if (((uintptr_t)t.base & 15) || (t.ld % VEC) || (t.xoff % VEC))
+            vec = false;
+    }
+    const void* dtiles = nullptr;
+    if (int rc = desc_upload(tiles.data(), tiles.size() * sizeof(ColTile), st, &dtiles))
+        return rc;
+    int64_t blocks = (rows + kWavesPerBlock - 1) / kWavesPerBlock;
+    CNH_CHECK(blocks < (1ll << 31), -3, "matvec with %lld rows is too large for one launch",
+              (long long)rows);
+    if (vec)
+        hipLaunchKernelGGL((gemv_rows<T, true>), dim3((unsigned)blocks), dim3(kWavesPerBlock * 64),
+                           0, st, (const ColTile*)dtiles, ncol_tiles, tile_rows, rows, (const T*)x,
+                           (T*)y, beta);
+    else
+        hipLaunchKernelGGL((gemv_rows<T, false>), dim3((unsigned)blocks), dim3(kWavesPerBlock * 64),
+                           0, st, (const ColTile*)dtiles, ncol_tiles, tile_rows, rows, (const T*)x,
+                           (T*)y, beta);
+    CNH_HIP(hipGetLastError());
+    return 0;
+}
+
+int dispatch_gemv(int dtype, const std::vector<ColTile>& tiles, int ncol_tiles, int64_t tile_rows,
+                  int64_t rows, const void* x, void* y, int beta, hipStream_t st) {
+    switch (dtype) {
+    case CNH_F32: return run_gemv<float>(tiles, ncol_tiles, tile_rows, rows, x, y, beta, st);
+    case CNH_F64: return run_gemv<double>(tiles, ncol_tiles, tile_rows, rows, x, y, beta, st);
+    case CNH_I32: return run_gemv<int32_t>(tiles, ncol_tiles, tile_rows, rows, x, y, beta, st);
+    case CNH_I64: return run_gemv<int64_t>(tiles, ncol_tiles, tile_rows, rows, x, y, beta, st);
+    }
+    return set_error(-2, "unknown dtype %d", dtype);
+}
+
+} // namespace
+
+extern "C" {
+
+int cnh_gemv(int dtype, int64_t rows, int64_t cols, const void* A, int64_t lda, const void* x,
+             void* y, int beta, cnh_stream s) {
+    if (int rc = ensure_init())
+        return rc;
+    CNH_CHECK(rows >= 0 && cols >= 0 && lda >= cols, -2, "cnh_gemv: bad shape %lld x %lld, lda %lld",
+              (long long)rows, (long long)cols, (long long)lda);
+    CNH_CHECK(beta == 0 || beta == 1, -2, "cnh_gemv: beta must be 0 or 1");
+    if (rows == 0)
+        return 0;
+    CNH_CHECK(y != nullptr && (cols == 0 || (A != nullptr && x != nullptr)), -2,
+              "cnh_gemv: null pointer");
+    std::vector<ColTile> tiles(1);
+    tiles[0] = {A, lda, cols, 0};
+    return dispatch_gemv(dtype, tiles, 1, rows, rows, x, y, beta, as_stream(s));
+}
+
+int cnh_gemv_tiles(int dtype, int64_t rows, int64_t cols, int32_t tile, const void* const* tptr,
+                   const void* x, void* y, cnh_stream s) {
+    if (int rc = ensure_init())
+        return rc;
+    CNH_CHECK(rows > 0 && cols > 0 && tile > 0, -2, "cnh_gemv_tiles: bad shape");
+    CNH_CHECK(tptr && x && y, -2, "cnh_gemv_tiles: null pointer");
+    int64_t gr = (rows + tile - 1) / tile, gc = (cols + tile - 1) / tile;
+    std::vector<ColTile> tiles((size_t)(gr * gc));
+    for (int64_t i = 0; i < gr; ++i)
+        for (int64_t j = 0; j < gc; ++j) {
+            const void* p = tptr[i * gc + j];
+            CNH_CHECK(p != nullptr, -2, "cnh_gemv_tiles: tile (%lld,%lld) is null", (long long)i,
+                      (long long)j);
+            int64_t nc = std::min<int64_t>(tile, cols - j * tile);
+            tiles[(size_t)(i * gc + j)] = {p, nc, nc, j * tile};
+        }
+    return dispatch_gemv(dtype, tiles, (int)gc, tile, rows, x, y, 0, as_stream(s));
+}
+
+int cnh_axpy1(int dtype, int64_t n, const void* partial, void* y, cnh_stream s) {
+    if (int rc = ensure_init())
+        return rc;
+    CNH_CHECK(n >= 0, -2, "cnh_axpy1: negative length");
+    if (n == 0)
+        return 0;
+    CNH_CHECK(partial && y, -2, "cnh_axpy1: null pointer");
+    unsigned blocks = (unsigned)((n + 255) / 256);
+    hipStream_t st = as_stream(s);
+    switch (dtype) {
+    case CNH_F32:
+        hipLaunchKernelGGL(axpy1_kernel<float>, dim3(blocks), dim3(256), 0, st, n,
+                           (const float*)partial, (float*)y);
+        break;
+    case CNH_F64:
+        hipLaunchKernelGGL(axpy1_kernel<double>, dim3(blocks), dim3(256), 0, st, n,
+                           (const double*)partial, (double*)y);
+        break;
+    case CNH_I32:
+        hipLaunchKernelGGL(axpy1_kernel<int32_t>, dim3(blocks), dim3(256), 0, st, n,
+                           (const int32_t*)partial, (int32_t*)y);
+        break;
+    case CNH_I64:
+        hipLaunchKernelGGL(axpy1_kernel<int64_t>, dim3(blocks), dim3(256), 0, st, n,
+                           (const int64_t*)partial, (int64_t*)y);
+        break;
+    default: return set_error(-2, "unknown dtype %d", dtype);
+    }
+    CNH_HIP(hipGetLastError());
+    return 0;
+}
+
+} // extern "C"

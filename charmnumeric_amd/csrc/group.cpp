@@ -1,0 +1,598 @@
+// Fused-group kernels: hipRTC build, cache and launch.
+// Stands in for ArrayDAGGroup::compile_node (src/dag_group_compile.cpp:6-56 upstream) and
+// dispatch_kernel<N,T> (src/dispatch.hpp:137-265): same argument order (memref per leaf use,
+// scalar per broadcast leaf, memref per non-temp root), but all partitions of a node go into
+// one launch and broadcast scalars may stay on the device.
+#include "codegen.h"
+
+#include <hip/hiprtc.h>
+
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <vector>
+
+using namespace cnh;
+
+struct KernelVariant {
+    std::string src;
+    std::vector<char> code;
+    hipModule_t mod = nullptr;
+    std::map<std::string, hipFunction_t> fns;
+};
+
+struct cnh_kernel {
+    GroupProgram prog;
+    uint64_t key = 0;
+    int refs = 1;
+    std::map<std::string, KernelVariant> variants;
+};
+
+namespace {
+
+std::mutex g_kmu;
+std::map<uint64_t, cnh_kernel*> g_kernels; // key -> kernel (key 0 = not cached)
+
+int build_variant(cnh_kernel* k, const std::string& variant, KernelVariant** out) {
+    auto it = k->variants.find(variant);
+    if (it != k->variants.end() && !it->second.code.empty()) {
+        *out = &it->second;
+        return 0;
+    }
+    KernelVariant& v = k->variants[variant];
+    if (v.src.empty()) {
+        std::string err;
+        int rc = emit_variant_source(k->prog, variant, v.src, err);
+        if (rc) {
+            k->variants.erase(variant);
+            return set_error(rc, "codegen(%s): %s", variant.c_str(), err.c_str());
+        }
+    }
+    hiprtcProgram prog;
+    hiprtcResult r = hiprtcCreateProgram(&prog, v.src.c_str(), "cnh_group.hip", 0, nullptr, nullptr);
+    if (r != HIPRTC_SUCCESS)
+        return set_error(-110, "hiprtcCreateProgram: %s", hiprtcGetErrorString(r));
+    // No FMA contraction: the upstream group is a chain of separately rounded IEEE operations.
+    const char* opts[] = {"--offload-arch=gfx950", "-O3",     "-ffp-contract=off",
+                          "-Xclang",               "-target-feature", "-Xclang",
+                          "-packed-fp32-ops",      "-std=c++17"};
+    r = hiprtcCompileProgram(prog, (int)(sizeof opts / sizeof opts[0]), opts);
+    if (r != HIPRTC_SUCCESS) {
+        size_t n = 0;
+        hiprtcGetProgramLogSize(prog, &n);
+        std::string log(n, '\0');
+        if (n)
+            hiprtcGetProgramLog(prog, &log[0]);
+        hiprtcDestroyProgram(&prog);
+        return set_error(-111, "hiprtc compile failed (%s):\n%s", hiprtcGetErrorString(r),
+                         log.c_str());
+    }
+    size_t cs = 0;
+    hiprtcGetCodeSize(prog, &cs);
+    v.code.resize(cs);
+    hiprtcGetCode(prog, v.code.data());
+    hiprtcDestroyProgram(&prog);
+    *out = &v;
+    return 0;
+}
+
+int get_function(cnh_kernel* k, const std::string& variant, const char* name, hipFunction_t* fn) {
+    KernelVariant* v = nullptr;
+    if (int rc = build_variant(k, variant, &v))
+        return rc;
+    if (!v->mod)
+        CNH_HIP(hipModuleLoadData(&v->mod, v->code.data()));
+    auto it = v->fns.find(name);
+    if (it == v->fns.end()) {
+        hipFunction_t f;
+        CNH_HIP(hipModuleGetFunction(&f, v->mod, name));
+        it = v->fns.emplace(name, f).first;
+    }
+    *fn = it->second;
+    return 0;
+}
+
+// Scal { const T* p[NSA]; T v[NSA]; } as the generated code lays it out.
+int pack_scalars(const GroupProgram& p, int n_scalar, const void* const* scalars, int on_device,
+                 std::vector<unsigned char>& buf) {
+    int ns = (int)p.bcast_nodes.size();
+    CNH_CHECK(n_scalar == ns, -4, "group expects %d broadcast scalars, got %d", ns, n_scalar);
+    int nsa = ns > 0 ? ns : 1;
+    int esz = dtype_size(p.dtype);
+    size_t bytes = (size_t)nsa * 8 + (size_t)nsa * esz;
+    bytes = (bytes + 7) & ~size_t(7);
+    buf.assign(bytes, 0);
+    for (int i = 0; i < ns; ++i) {
+        CNH_CHECK(scalars && scalars[i], -4, "broadcast scalar %d is null", i);
+        if (on_device) {
+            const void* ptr = scalars[i];
+            std::memcpy(&buf[(size_t)i * 8], &ptr, 8);
+        } else {
+            std::memcpy(&buf[(size_t)nsa * 8 + (size_t)i * esz], scalars[i], esz);
+        }
+    }
+    return 0;
+}
+
+bool dense_memref(int nd, const cnh_memref& m) {
+    int64_t expect = 1;
+    for (int d = nd - 1; d >= 0; --d) {
+        if (m.sizes[d] != 1 && m.strides[d] != expect)
+            return false;
+        expect *= m.sizes[d];
+    }
+    return true;
+}
+
+int launch(hipFunction_t fn, int64_t blocks, void** params, hipStream_t st) {
+    CNH_CHECK(blocks > 0 && blocks < (1ll << 31), -3, "launch of %lld workgroups is out of range",
+              (long long)blocks);
+    CNH_HIP(hipModuleLaunchKernel(fn, (unsigned)blocks, 1, 1, 256, 1, 1, 0, st, params, nullptr));
+    return 0;
+}
+
+} // namespace
+
+extern "C" {
+
+int cnh_compile_group(const cnh_ast* ast, int dtype, int ndims, uint64_t key, cnh_kernel** out) {
+    CNH_CHECK(out != nullptr, -2, "cnh_compile_group: null output");
+    std::lock_guard<std::mutex> lk(g_kmu);
+    if (key != 0) {
+        auto it = g_kernels.find(key);
+        if (it != g_kernels.end()) {
+            it->second->refs++;
+            *out = it->second;
+            return 0;
+        }
+    }
+    cnh_kernel* k = new cnh_kernel;
+    std::string err;
+    int rc = build_group_program(ast, dtype, ndims, k->prog, err);
+    if (rc) {
+        delete k;
+        return set_error(rc, "cnh_compile_group: %s", err.c_str());
+    }
+    k->key = key;
+    if (key != 0) {
+        g_kernels[key] = k;
+        k->refs++; // the cache holds one reference
+    }
+    *out = k;
+    return 0;
+}
+
+int cnh_kernel_release(cnh_kernel* k) {
+    if (!k)
+        return 0;
+    std::lock_guard<std::mutex> lk(g_kmu);
+    if (--k->refs > 0)
+        return 0;
+    for (auto& kv : k->variants)
+        if (kv.second.mod)
+            (void)hipModuleUnload(kv.second.mod);
+    if (k->key != 0)
+        g_kernels.erase(k->key);
+    delete k;
+    return 0;
+}
+
+int cnh_kernel_signature(const cnh_kernel* k, int* n_in, int* n_scalar, int* n_out) {
+    CNH_CHECK(k != nullptr, -2, "null kernel");
+    if (n_in)
+        *n_in = (int)k->prog.leaves.size();
+    if (n_scalar)
+        *n_scalar = (int)k->prog.bcast_nodes.size();
+    if (n_out)
+        *n_out = (int)k->prog.out_roots.size();
+    return 0;
+}
+
+int64_t cnh_kernel_source(cnh_kernel* k, const char* variant, char* buf, size_t cap) {
+    CNH_CHECK(k != nullptr && variant != nullptr, -2, "null argument");
+    KernelVariant& v = k->variants[variant];
+    if (v.src.empty()) {
+        std::string err;
+        int rc = emit_variant_source(k->prog, variant, v.src, err);
+        if (rc) {
+            k->variants.erase(variant);
+            return set_error(rc, "codegen(%s): %s", variant, err.c_str());
+        }
+    }
+    if (buf && cap > 0) {
+        size_t n = v.src.size() < cap - 1 ? v.src.size() : cap - 1;
+        std::memcpy(buf, v.src.data(), n);
+        buf[n] = '\0';
+    }
+    return (int64_t)v.src.size() + 1;
+}
+
+int cnh_kernel_build(cnh_kernel* k, const char* variant) {
+    CNH_CHECK(k != nullptr && variant != nullptr, -2, "null argument");
+    KernelVariant* v = nullptr;
+    return build_variant(k, variant, &v);
+}
+
+int cnh_launch_group_batched(cnh_kernel* k, int ndims, int n_parts, int n_in, const cnh_memref* in,
+                             int n_scalar, const void* const* scalars, int scalars_on_device,
+                             int n_out, const cnh_memref* out, cnh_stream s) {
+    if (int rc = ensure_init())
+        return rc;
+    CNH_CHECK(k != nullptr, -2, "null kernel");
+    const GroupProgram& p = k->prog;
+    CNH_CHECK(ndims == p.ndims, -4, "kernel was compiled for rank %d, launched with %d", p.ndims,
+              ndims);
+    CNH_CHECK(n_in == (int)p.leaves.size(), -4, "group expects %d input memrefs, got %d",
+              (int)p.leaves.size(), n_in);
+    CNH_CHECK(n_out == (int)p.out_roots.size(), -4, "group expects %d output memrefs, got %d",
+              (int)p.out_roots.size(), n_out);
+    CNH_CHECK(n_parts >= 0, -2, "negative partition count");
+    CNH_CHECK(n_out >= 1 && out != nullptr, -2, "a group needs at least one output memref");
+    CNH_CHECK(n_in == 0 || in != nullptr, -2, "null input memrefs");
+    std::vector<unsigned char> scal;
+    if (int rc = pack_scalars(p, n_scalar, scalars, scalars_on_device, scal))
+        return rc;
+
+    const int NL = (int)p.load_leaf.size();
+    const int NLA = NL > 0 ? NL : 1, NOA = n_out;
+    const int esz = dtype_size(p.dtype);
+    const int vec = 16 / esz, unr = 4;
+
+    // Shapes must agree across all memrefs of a partition (identity indexing maps upstream).
+    bool all_dense = true, all_aligned = true;
+    std::vector<int> live;
+    for (int q = 0; q < n_parts; ++q) {
+        const cnh_memref* pi = in + (size_t)q * n_in;
+        const cnh_memref* po = out + (size_t)q * n_out;
+        int64_t total = 1;
+        for (int d = 0; d < ndims; ++d) {
+            CNH_CHECK(po[0].sizes[d] >= 0, -4, "negative extent");
+            total *= po[0].sizes[d];
+        }
+        if (total == 0)
+            continue;
+        live.push_back(q);
+        for (int i = 0; i < n_in + n_out; ++i) {
+            const cnh_memref& m = i < n_in ? pi[i] : po[i - n_in];
+            CNH_CHECK(m.aligned != nullptr, -4, "partition %d: memref %d has a null pointer", q, i);
+            for (int d = 0; d < ndims; ++d)
+                CNH_CHECK(m.sizes[d] == po[0].sizes[d], -4,
+                          "partition %d: memref %d extent %lld differs from the output's %lld in "
+                          "dim %d",
+                          q, i, (long long)m.sizes[d], (long long)po[0].sizes[d], d);
+            if (!dense_memref(ndims, m))
+                all_dense = false;
+            uintptr_t addr = (uintptr_t)m.aligned + (uintptr_t)(m.offset * esz);
+            if (addr & 15)
+                all_aligned = false;
+        }
+    }
+    if (live.empty())
+        return 0;
+    hipStream_t st = as_stream(s);
+    auto base_ptr = [&](const cnh_memref& m) -> uint64_t {
+        return (uint64_t)((uintptr_t)m.aligned + (uintptr_t)(m.offset * esz));
+    };
+
+    if (all_dense) {
+        const int per_block = 256 * vec * unr;
+        const size_t seg_words = 2 + NLA + NOA;
+        std::vector<uint64_t> segs(seg_words * live.size(), 0);
+        int64_t blocks = 0;
+        for (size_t j = 0; j < live.size(); ++j) {
+            int q = live[j];
+            const cnh_memref* pi = in + (size_t)q * n_in;
+            const cnh_memref* po = out + (size_t)q * n_out;
+            int64_t n = 1;
+            for (int d = 0; d < ndims; ++d)
+                n *= po[0].sizes[d];
+            uint64_t* sg = &segs[j * seg_words];
+            sg[0] = (uint64_t)n;
+            sg[1] = (uint64_t)blocks;
+            for (int l = 0; l < NL; ++l)
+                sg[2 + l] = base_ptr(pi[p.load_leaf[l]]);
+            for (int o = 0; o < n_out; ++o)
+                sg[2 + NLA + o] = base_ptr(po[o]);
+            blocks += (n + per_block - 1) / per_block;
+        }
+        hipFunction_t fn;
+        if (live.size() == 1) {
+            if (int rc = get_function(k, "flat", all_aligned ? "grp_flat1_v" : "grp_flat1_s", &fn))
+                return rc;
+            void* params[] = {segs.data(), scal.data()};
+            return launch(fn, blocks, params, st);
+        }
+        if (int rc = get_function(k, "flat", all_aligned ? "grp_flat_v" : "grp_flat_s", &fn))
+            return rc;
+        const void* dsegs = nullptr;
+        if (int rc = desc_upload(segs.data(), segs.size() * 8, st, &dsegs))
+            return rc;
+        int nseg = (int)live.size();
+        void* params[] = {&dsegs, &nseg, scal.data()};
+        return launch(fn, blocks, params, st);
+    }
+
+    // Strided cells.
+    const size_t cell_words = 5 + NLA + 3 * NLA + NOA + 3 * NOA;
+    std::vector<int64_t> cells(cell_words * live.size(), 0);
+    int64_t blocks = 0;
+    const int pad = CNH_MAX_ND - ndims;
+    for (size_t j = 0; j < live.size(); ++j) {
+        int q = live[j];
+        const cnh_memref* pi = in + (size_t)q * n_in;
+        const cnh_memref* po = out + (size_t)q * n_out;
+        int64_t* c = &cells[j * cell_words];
+        int64_t sz[3] = {1, 1, 1};
+        for (int d = 0; d < ndims; ++d)
+            sz[pad + d] = po[0].sizes[d];
+        int64_t nchunks = (sz[2] + 1023) / 1024;
+        c[0] = sz[0];
+        c[1] = sz[1];
+        c[2] = sz[2];
+        c[3] = blocks;
+        c[4] = nchunks;
+        int64_t* cin = c + 5;
+        int64_t* cistr = cin + NLA;
+        int64_t* cout = cistr + 3 * NLA;
+        int64_t* costr = cout + NOA;
+        for (int l = 0; l < NL; ++l) {
+            const cnh_memref& m = pi[p.load_leaf[l]];
+            cin[l] = (int64_t)base_ptr(m);
+            for (int d = 0; d < ndims; ++d)
+                cistr[l * 3 + pad + d] = m.strides[d];
+        }
+        for (int o = 0; o < n_out; ++o) {
+            cout[o] = (int64_t)base_ptr(po[o]);
+            for (int d = 0; d < ndims; ++d)
+                costr[o * 3 + pad + d] = po[o].strides[d];
+        }
+        blocks += sz[0] * sz[1] * nchunks;
+    }
+    hipFunction_t fn;
+    if (live.size() == 1) {
+        if (int rc = get_function(k, "nd", "grp_nd1", &fn))
+            return rc;
+        void* params[] = {cells.data(), scal.data()};
+        return launch(fn, blocks, params, st);
+    }
+    if (int rc = get_function(k, "nd", "grp_nd", &fn))
+        return rc;
+    const void* dcells = nullptr;
+    if (int rc = desc_upload(cells.data(), cells.size() * 8, st, &dcells))
+        return rc;
+    int ncell = (int)live.size();
+    void* params[] = {&dcells, &ncell, scal.data()};
+    return launch(fn, blocks, params, st);
+}
+
+int cnh_launch_group(cnh_kernel* k, int ndims, int n_in, const cnh_memref* in, int n_scalar,
+                     const void* const* scalars, int scalars_on_device, int n_out,
+                     const cnh_memref* out, cnh_stream s) {
+    return cnh_launch_group_batched(k, ndims, 1, n_in, in, n_scalar, scalars, scalars_on_device,
+                                    n_out, out, s);
+}
+
+} // extern "C"
+
+// ---------------------------------------------------------------------------------------------
+// Tiled launch: all tiles of the target in one launch, neighbour tiles read in place.
+// ---------------------------------------------------------------------------------------------
+namespace {
+
+struct TiledDev {
+    int32_t shift, tile, off[3], shape[3], glo[3], grid[3];
+    const void* tiles;
+};
+static_assert(sizeof(TiledDev) == 64, "TiledDev layout must match the generated struct");
+
+struct DTileDev {
+    int64_t blk0;
+    int32_t cs[3], w[3], nchunks, pad;
+    void* dst;
+    const void* cur;
+};
+static_assert(sizeof(DTileDev) == 56, "DTileDev layout must match the generated struct");
+
+int check_tiled(const cnh_tiled* t, int nd, const char* what) {
+    CNH_CHECK(t != nullptr, -2, "%s: null descriptor", what);
+    CNH_CHECK(t->ndims == nd, -4, "%s: rank %d, expected %d", what, t->ndims, nd);
+    CNH_CHECK(t->tile > 0 && (t->tile & (t->tile - 1)) == 0, -4,
+              "%s: tile edge %d is not a power of two", what, t->tile);
+    CNH_CHECK(t->tiles != nullptr, -4, "%s: null tile table", what);
+    int64_t count = 1;
+    for (int d = 0; d < nd; ++d) {
+        CNH_CHECK(t->shape[d] > 0 && t->offset[d] >= 0, -4, "%s: bad shape/offset in dim %d", what, d);
+        int glo = t->offset[d] / t->tile;
+        int ghi = (t->offset[d] + t->shape[d] + t->tile - 1) / t->tile;
+        CNH_CHECK(t->grid_lo[d] == glo && t->grid[d] == ghi - glo, -4,
+                  "%s: tile grid in dim %d is [%d,+%d), decomposition implies [%d,+%d)", what, d,
+                  t->grid_lo[d], t->grid[d], glo, ghi - glo);
+        count *= t->grid[d];
+    }
+    for (int64_t i = 0; i < count; ++i)
+        CNH_CHECK(t->tiles[i] != nullptr, -4, "%s: tile %lld has a null pointer", what, (long long)i);
+    return 0;
+}
+
+int make_tiled_dev(const cnh_tiled* t, hipStream_t st, TiledDev& d) {
+    int nd = t->ndims, pad = CNH_MAX_ND - nd;
+    std::memset(&d, 0, sizeof d);
+    d.tile = t->tile;
+    d.shift = 0;
+    while ((1 << d.shift) < t->tile)
+        d.shift++;
+    int64_t count = 1;
+    for (int i = 0; i < 3; ++i) {
+        d.off[i] = 0;
+        d.shape[i] = 1;
+        d.glo[i] = 0;
+        d.grid[i] = 1;
+    }
+    for (int i = 0; i < nd; ++i) {
+        d.off[pad + i] = t->offset[i];
+        d.shape[pad + i] = t->shape[i];
+        d.glo[pad + i] = t->grid_lo[i];
+        d.grid[pad + i] = t->grid[i];
+        count *= t->grid[i];
+    }
+    const void* table = nullptr;
+    if (int rc = desc_upload(t->tiles, (size_t)count * sizeof(void*), st, &table))
+        return rc;
+    d.tiles = table;
+    return 0;
+}
+
+} // namespace
+
+extern "C" int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* in, int n_scalar,
+                                      const void* const* scalars, int scalars_on_device,
+                                      const cnh_tiled* cur, const cnh_tiled* dst, cnh_stream s) {
+    if (int rc = ensure_init())
+        return rc;
+    CNH_CHECK(k != nullptr, -2, "null kernel");
+    const GroupProgram& p = k->prog;
+    const int nd = p.ndims;
+    CNH_CHECK(p.out_roots.size() == 1, -17, "the tiled launch needs exactly one output root");
+    CNH_CHECK(n_in == (int)p.leaves.size(), -4, "group expects %d tiled inputs, got %d",
+              (int)p.leaves.size(), n_in);
+    if (int rc = check_tiled(dst, nd, "dst"))
+        return rc;
+    if (cur) {
+        if (int rc = check_tiled(cur, nd, "cur"))
+            return rc;
+        CNH_CHECK(cur->tile == dst->tile, -4, "cur and dst differ in tile edge");
+        for (int d = 0; d < nd; ++d)
+            CNH_CHECK(cur->offset[d] == dst->offset[d] && cur->shape[d] == dst->shape[d], -4,
+                      "cur and dst differ in decomposition");
+    }
+    for (int i = 0; i < n_in; ++i)
+        if (int rc = check_tiled(&in[i], nd, "input"))
+            return rc;
+    std::vector<unsigned char> scal;
+    if (int rc = pack_scalars(p, n_scalar, scalars, scalars_on_device, scal))
+        return rc;
+    hipStream_t st = as_stream(s);
+    const int pad = CNH_MAX_ND - nd;
+
+    // Assigned region (target coordinates) and the input region of every distinct load.
+    int rs[3] = {0, 0, 0}, re[3] = {1, 1, 1}, rst[3] = {1, 1, 1};
+    const bool set_region = p.out_is_set_region[0] && !p.out_region[0].is_global;
+    for (int d = 0; d < nd; ++d) {
+        if (set_region) {
+            rs[pad + d] = p.out_region[0].start[d];
+            re[pad + d] = p.out_region[0].stop[d];
+            rst[pad + d] = p.out_region[0].step[d];
+        } else {
+            rs[pad + d] = 0;
+            re[pad + d] = dst->shape[d];
+            rst[pad + d] = 1;
+        }
+        CNH_CHECK(rst[pad + d] >= 1 && rs[pad + d] >= 0 && re[pad + d] <= dst->shape[d], -4,
+                  "assigned region [%d:%d:%d] does not fit the target extent %d in dim %d",
+                  rs[pad + d], re[pad + d], rst[pad + d], dst->shape[d], d);
+    }
+    const int NL = (int)p.load_leaf.size();
+    const int NLA = NL > 0 ? NL : 1;
+    std::vector<const cnh_tiled*> arrays;
+    std::vector<int32_t> targs(12 + 7 * NLA, 0);
+    for (int d = 0; d < 3; ++d) {
+        targs[d] = d >= pad ? dst->offset[d - pad] : 0;
+        targs[3 + d] = rs[d];
+        targs[6 + d] = re[d];
+        targs[9 + d] = rst[d];
+    }
+    for (int l = 0; l < NL; ++l) {
+        const LeafUse& u = p.leaves[p.load_leaf[l]];
+        const cnh_tiled* arr = &in[p.load_leaf[l]];
+        int ai = -1;
+        for (size_t a = 0; a < arrays.size(); ++a)
+            if (arrays[a]->tiles[0] == arr->tiles[0] && arrays[a]->tile == arr->tile &&
+                std::memcmp(arrays[a]->offset, arr->offset, sizeof arr->offset) == 0 &&
+                std::memcmp(arrays[a]->shape, arr->shape, sizeof arr->shape) == 0)
+                ai = (int)a;
+        if (ai < 0) {
+            ai = (int)arrays.size();
+            arrays.push_back(arr);
+        }
+        int32_t* lr = &targs[12 + 7 * l];
+        lr[0] = ai;
+        for (int d = 0; d < 3; ++d) {
+            lr[1 + d] = 0;
+            lr[4 + d] = 1;
+        }
+        for (int d = 0; d < nd; ++d) {
+            int start = u.has_region ? u.region.start[d] : 0;
+            int stop = u.has_region ? u.region.stop[d] : arr->shape[d];
+            int step = u.has_region ? u.region.step[d] : 1;
+            CNH_CHECK(step >= 1, -4, "input %d: step %d in dim %d", l, step, d);
+            int count = (stop - start + step - 1) / step;
+            int ocount = (re[pad + d] - rs[pad + d] + rst[pad + d] - 1) / rst[pad + d];
+            CNH_CHECK(count == ocount, -4,
+                      "input %d has %d elements in dim %d, the assigned region has %d", l, count, d,
+                      ocount);
+            CNH_CHECK(start >= 0 && start + (count - 1) * step < arr->shape[d], -4,
+                      "input %d: region [%d:%d:%d] leaves the array extent %d in dim %d", l, start,
+                      stop, step, arr->shape[d], d);
+            lr[1 + pad + d] = start;
+            lr[4 + pad + d] = step;
+        }
+    }
+
+    // Destination tiles.
+    int64_t ntiles = 1;
+    for (int d = 0; d < nd; ++d)
+        ntiles *= dst->grid[d];
+    std::vector<DTileDev> dts;
+    int64_t blocks = 0;
+    for (int64_t t = 0; t < ntiles; ++t) {
+        int ti[3] = {0, 0, 0};
+        int64_t rem = t;
+        for (int d = nd - 1; d >= 0; --d) {
+            ti[d] = (int)(rem % dst->grid[d]);
+            rem /= dst->grid[d];
+        }
+        DTileDev dt;
+        std::memset(&dt, 0, sizeof dt);
+        for (int d = 0; d < 3; ++d) {
+            dt.cs[d] = 0;
+            dt.w[d] = 1;
+        }
+        bool empty = false;
+        for (int d = 0; d < nd; ++d) {
+            int g = dst->grid_lo[d] + ti[d];
+            int lo = std::max(g * dst->tile, dst->offset[d]);
+            int hi = std::min((g + 1) * dst->tile, dst->offset[d] + dst->shape[d]);
+            if (hi <= lo)
+                empty = true;
+            dt.cs[pad + d] = lo;
+            dt.w[pad + d] = hi - lo;
+        }
+        if (empty)
+            continue;
+        dt.nchunks = (dt.w[2] + 1023) / 1024;
+        dt.blk0 = blocks;
+        dt.dst = dst->tiles[t];
+        dt.cur = cur ? cur->tiles[t] : nullptr;
+        blocks += (int64_t)dt.w[0] * dt.w[1] * dt.nchunks;
+        dts.push_back(dt);
+    }
+    if (dts.empty())
+        return 0;
+
+    std::vector<TiledDev> adev(arrays.size() ? arrays.size() : 1);
+    for (size_t a = 0; a < arrays.size(); ++a)
+        if (int rc = make_tiled_dev(arrays[a], st, adev[a]))
+            return rc;
+    const void* d_arrs = nullptr;
+    const void* d_dts = nullptr;
+    if (int rc = desc_upload(adev.data(), adev.size() * sizeof(TiledDev), st, &d_arrs))
+        return rc;
+    if (int rc = desc_upload(dts.data(), dts.size() * sizeof(DTileDev), st, &d_dts))
+        return rc;
+    hipFunction_t fn;
+    if (int rc = get_function(k, "tiles", "grp_tiles", &fn))
+        return rc;
+    int ndt = (int)dts.size();
+    void* params[] = {&d_arrs, &d_dts, &ndt, targs.data(), scal.data()};
+    return launch(fn, blocks, params, st);
+}

@@ -1,0 +1,367 @@
+// Deterministic reductions: dot, sum, sum of squared differences, max |a-b|.
+// Upstream REDUCE is a per-tile Eigen/KokkosBlas dot followed by a Charm++ reduction that adds
+// the contributions one after the other (src/executor_reduce.cpp:8-119,
+// src/executor_reducer.cpp:11-57). Here: stage 1 — every workgroup reduces a fixed slice with
+// 128-bit loads, a wavefront shuffle tree and an LDS tree; stage 2 — one workgroup folds the
+// slices of each tile in a fixed tree and then adds the tiles in index order. The workgroup
+// count depends only on the element counts, so results never depend on scheduling.
+#include "common.h"
+
+#include <vector>
+
+using namespace cnh;
+
+namespace {
+
+enum Mode { M_DOT = 0, M_SUM = 1, M_SUMSQ_DIFF = 2, M_MAXABS_DIFF = 3 };
+
+struct Chunk {
+    const void* a;
+    const void* b;
+    int64_t n;
+    int64_t per_block; // elements per workgroup (multiple of 512)
+    int32_t blk0;      // first stage-1 workgroup / first partial slot
+    int32_t nblk;
+};
+
+constexpr int kThreads = 256;
+constexpr int kMaxBlocksPerChunk = 1024;
+
+template <typename T>
+struct Acc {
+    typedef T type;
+};
+template <>
+struct Acc<int32_t> {
+    typedef uint32_t type;
+};
+template <>
+struct Acc<int64_t> {
+    typedef uint64_t type;
+};
+
+template <typename A, int MODE>
+__device__ __forceinline__ A combine(A x, A y) {
+    if (MODE == M_MAXABS_DIFF)
+        return x > y ? x : y;
+    return x + y;
+}
+
+template <typename T, typename A, int MODE>
+__device__ __forceinline__ A term(T a, T b) {
+    if (MODE == M_DOT)
+        return (A)a * (A)b;
+    if (MODE == M_SUM)
+        return (A)a;
+    if (MODE == M_SUMSQ_DIFF) {
+        A d = (A)a - (A)b;
+        return d * d;
+    }
+    A d = (A)a - (A)b;
+    return d < (A)0 ? (A)0 - d : d;
+}
+
+template <typename A>
+__device__ __forceinline__ A shfl_down_any(A v, int off) {
+    if (sizeof(A) == 8) {
+        unsigned long long u;
+        __builtin_memcpy(&u, &v, 8);
+        unsigned lo = (unsigned)u, hi = (unsigned)(u >> 32);
+        lo = __shfl_down(lo, off, 64);
+        hi = __shfl_down(hi, off, 64);
+        u = ((unsigned long long)hi << 32) | lo;
+        A r;
+        __builtin_memcpy(&r, &u, 8);
+        return r;
+    } else {
+        unsigned u;
+        __builtin_memcpy(&u, &v, 4);
+        u = __shfl_down(u, off, 64);
+        A r;
+        __builtin_memcpy(&r, &u, 4);
+        return r;
+    }
+}
+
+// Wavefront shuffle tree, then an LDS tree over the wavefronts of the workgroup.
+template <typename A, int MODE, int THREADS>
+__device__ __forceinline__ A block_reduce(A v, A* lds) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1)
+        v = combine<A, MODE>(v, shfl_down_any<A>(v, off));
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0)
+        lds[wave] = v;
+    __syncthreads();
+    constexpr int NW = THREADS / 64;
+    if (threadIdx.x == 0) {
+        A r = lds[0];
+#pragma unroll
+        for (int w = 1; w < NW; ++w)
+            r = combine<A, MODE>(r, lds[w]);
+        v = r;
+    }
+    __syncthreads();
+    return v;
+}
+
+template <typename T, int MODE, int THREADS>
+__device__ __forceinline__ typename Acc<T>::type slice_reduce(const T* a, const T* b, int64_t lo,
+                                                               int64_t hi) {
+    typedef typename Acc<T>::type A;
+    constexpr int VEC = 16 / sizeof(T);
+    struct alignas(16) P {
+        T x[VEC];
+    };
+    A acc0 = 0, acc1 = 0;
+    const bool two = MODE != M_SUM;
+    const bool aligned = (((uintptr_t)(a + lo)) & 15) == 0 &&
+                         (!two || (((uintptr_t)(b + lo)) & 15) == 0);
+    int64_t i = lo + (int64_t)threadIdx.x * VEC;
+    if (aligned) {
+        const int64_t stride = (int64_t)THREADS * VEC;
+        for (; i + stride + VEC <= hi; i += 2 * stride) {
+            P a0 = *reinterpret_cast<const P*>(a + i);
+            P a1 = *reinterpret_cast<const P*>(a + i + stride);
+            P b0 = a0, b1 = a1;
+            if (two) {
+                b0 = *reinterpret_cast<const P*>(b + i);
+                b1 = *reinterpret_cast<const P*>(b + i + stride);
+            }
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                acc0 = combine<A, MODE>(acc0, term<T, A, MODE>(a0.x[e], b0.x[e]));
+                acc1 = combine<A, MODE>(acc1, term<T, A, MODE>(a1.x[e], b1.x[e]));
+            }
+        }
+        for (; i + VEC <= hi; i += stride) {
+            P a0 = *reinterpret_cast<const P*>(a + i);
+            P b0 = a0;
+            if (two)
+                b0 = *reinterpret_cast<const P*>(b + i);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e)
+                acc0 = combine<A, MODE>(acc0, term<T, A, MODE>(a0.x[e], b0.x[e]));
+        }
+        // ragged end of the slice: fewer than VEC elements
+        if (i < hi) {
+            for (int64_t j = i; j < hi; ++j)
+                acc0 = combine<A, MODE>(acc0, term<T, A, MODE>(a[j], two ? b[j] : a[j]));
+        }
+    } else {
+        for (int64_t j = lo + threadIdx.x; j < hi; j += THREADS)
+            acc0 = combine<A, MODE>(acc0, term<T, A, MODE>(a[j], two ? b[j] : a[j]));
+    }
+    return combine<A, MODE>(acc0, acc1);
+}
+
+template <typename T, int MODE>
+__global__ __launch_bounds__(kThreads) void reduce_stage1(const Chunk* __restrict__ chunks,
+                                                          int nchunk,
+                                                          typename Acc<T>::type* __restrict__ partials) {
+    typedef typename Acc<T>::type A;
+    __shared__ A lds[kThreads / 64];
+    int lo = 0, hi = nchunk - 1;
+    const int blk = blockIdx.x;
+    while (lo < hi) {
+        int mid = (lo + hi + 1) >> 1;
+        if (chunks[mid].blk0 <= blk)
+            lo = mid;
+        else
+            hi = mid - 1;
+    }
+    const Chunk c = chunks[lo];
+    const int64_t b0 = (int64_t)(blk - c.blk0) * c.per_block;
+    const int64_t b1 = b0 + c.per_block < c.n ? b0 + c.per_block : c.n;
+    A v = slice_reduce<T, MODE, kThreads>((const T*)c.a, (const T*)c.b, b0, b1);
+    v = block_reduce<A, MODE, kThreads>(v, lds);
+    if (threadIdx.x == 0)
+        partials[blk] = v;
+}
+
+// One workgroup: per chunk a fixed tree over its slots, then chunks added in index order.
+template <typename T, int MODE>
+__global__ __launch_bounds__(kThreads) void reduce_stage2(const Chunk* __restrict__ chunks,
+                                                          int nchunk,
+                                                          const typename Acc<T>::type* __restrict__ partials,
+                                                          T* __restrict__ out) {
+    typedef typename Acc<T>::type A;
+    __shared__ A lds[kThreads / 64];
+    A total = 0;
+    for (int c = 0; c < nchunk; ++c) {
+        const int b0 = chunks[c].blk0, nb = chunks[c].nblk;
+        A v = 0;
+        for (int i = threadIdx.x; i < nb; i += kThreads)
+            v = combine<A, MODE>(v, partials[b0 + i]);
+        v = block_reduce<A, MODE, kThreads>(v, lds);
+        if (threadIdx.x == 0)
+            total = c == 0 ? v : combine<A, MODE>(total, v);
+    }
+    if (threadIdx.x == 0)
+        *out = (T)total;
+}
+
+// Short single tile: one workgroup of 1024 lanes does everything in one launch.
+template <typename T, int MODE>
+__global__ __launch_bounds__(1024) void reduce_single(const T* __restrict__ a,
+                                                      const T* __restrict__ b, int64_t n,
+                                                      T* __restrict__ out) {
+    typedef typename Acc<T>::type A;
+    __shared__ A lds[1024 / 64];
+    A v = slice_reduce<T, MODE, 1024>(a, b, 0, n);
+    v = block_reduce<A, MODE, 1024>(v, lds);
+    if (threadIdx.x == 0)
+        *out = (T)v;
+}
+
+// Sequential sum of per-tile partials in index order (the upstream reducer's a += b loop).
+template <typename T>
+__global__ void reduce_final_seq(const T* __restrict__ partials, int n, T* __restrict__ out) {
+    typedef typename Acc<T>::type A;
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        A acc = (A)partials[0];
+        for (int i = 1; i < n; ++i)
+            acc += (A)partials[i];
+        *out = (T)acc;
+    }
+}
+
+constexpr int64_t kSingleMax = 1 << 16;
+
+template <typename T, int MODE>
+int run_tiles(int n_tiles, const void* const* a, const void* const* b, const int64_t* n, void* out,
+              hipStream_t st) {
+    CNH_CHECK(n_tiles >= 1, -2, "reduction over %d tiles", n_tiles);
+    CNH_CHECK(out != nullptr && a != nullptr && n != nullptr, -2, "null argument");
+    const bool two = MODE != M_SUM;
+    CNH_CHECK(!two || b != nullptr, -2, "null second operand");
+    for (int t = 0; t < n_tiles; ++t) {
+        CNH_CHECK(n[t] >= 0, -2, "tile %d has negative length", t);
+        CNH_CHECK(n[t] == 0 || (a[t] != nullptr && (!two || b[t] != nullptr)), -2,
+                  "tile %d has a null pointer", t);
+    }
+    if (n_tiles == 1 && n[0] <= kSingleMax) {
+        hipLaunchKernelGGL((reduce_single<T, MODE>), dim3(1), dim3(1024), 0, st, (const T*)a[0],
+                           (const T*)(two ? b[0] : a[0]), n[0], (T*)out);
+        CNH_HIP(hipGetLastError());
+        return 0;
+    }
+    std::vector<Chunk> chunks(n_tiles);
+    int blocks = 0;
+    for (int t = 0; t < n_tiles; ++t) {
+        Chunk& c = chunks[t];
+        c.a = a[t];
+        c.b = two ? b[t] : a[t];
+        c.n = n[t];
+        int64_t nb = (n[t] + 8191) / 8192;
+        if (nb < 1)
+            nb = 1;
+        if (nb > kMaxBlocksPerChunk)
+            nb = kMaxBlocksPerChunk;
+        int64_t per = (n[t] + nb - 1) / nb;
+        per = (per + 511) / 512 * 512;
+        if (per < 512)
+            per = 512;
+        nb = n[t] > 0 ? (n[t] + per - 1) / per : 1;
+        c.per_block = per;
+        c.blk0 = blocks;
+        c.nblk = (int)nb;
+        blocks += (int)nb;
+    }
+    typedef typename Acc<T>::type A;
+    void* ws = nullptr;
+    if (int rc = reduce_workspace(st, (size_t)blocks * sizeof(A), &ws))
+        return rc;
+    const void* dchunks = nullptr;
+    if (int rc = desc_upload(chunks.data(), chunks.size() * sizeof(Chunk), st, &dchunks))
+        return rc;
+    hipLaunchKernelGGL((reduce_stage1<T, MODE>), dim3(blocks), dim3(kThreads), 0, st,
+                       (const Chunk*)dchunks, n_tiles, (A*)ws);
+    CNH_HIP(hipGetLastError());
+    hipLaunchKernelGGL((reduce_stage2<T, MODE>), dim3(1), dim3(kThreads), 0, st,
+                       (const Chunk*)dchunks, n_tiles, (const A*)ws, (T*)out);
+    CNH_HIP(hipGetLastError());
+    return 0;
+}
+
+template <int MODE>
+int dispatch_tiles(int dtype, int n_tiles, const void* const* a, const void* const* b,
+                   const int64_t* n, void* out, hipStream_t st) {
+    switch (dtype) {
+    case CNH_F32: return run_tiles<float, MODE>(n_tiles, a, b, n, out, st);
+    case CNH_F64: return run_tiles<double, MODE>(n_tiles, a, b, n, out, st);
+    case CNH_I32: return run_tiles<int32_t, MODE>(n_tiles, a, b, n, out, st);
+    case CNH_I64: return run_tiles<int64_t, MODE>(n_tiles, a, b, n, out, st);
+    }
+    return set_error(-2, "unknown dtype %d", dtype);
+}
+
+} // namespace
+
+extern "C" {
+
+int cnh_dot_tiles(int dtype, int n_tiles, const void* const* a, const void* const* b,
+                  const int64_t* n, void* out, cnh_stream s) {
+    if (int rc = ensure_init())
+        return rc;
+    return dispatch_tiles<M_DOT>(dtype, n_tiles, a, b, n, out, as_stream(s));
+}
+
+int cnh_dot_partial(int dtype, int64_t n, const void* a, const void* b, void* partial_slot,
+                    cnh_stream s) {
+    const void* aa[1] = {a};
+    const void* bb[1] = {b};
+    int64_t nn[1] = {n};
+    return cnh_dot_tiles(dtype, 1, aa, bb, nn, partial_slot, s);
+}
+
+int cnh_reduce_final(int dtype, int n_partials, const void* partials, void* out, cnh_stream s) {
+    if (int rc = ensure_init())
+        return rc;
+    CNH_CHECK(n_partials >= 1 && partials && out, -2, "cnh_reduce_final: bad arguments");
+    hipStream_t st = as_stream(s);
+    switch (dtype) {
+    case CNH_F32:
+        hipLaunchKernelGGL(reduce_final_seq<float>, dim3(1), dim3(64), 0, st, (const float*)partials,
+                           n_partials, (float*)out);
+        break;
+    case CNH_F64:
+        hipLaunchKernelGGL(reduce_final_seq<double>, dim3(1), dim3(64), 0, st,
+                           (const double*)partials, n_partials, (double*)out);
+        break;
+    case CNH_I32:
+        hipLaunchKernelGGL(reduce_final_seq<int32_t>, dim3(1), dim3(64), 0, st,
+                           (const int32_t*)partials, n_partials, (int32_t*)out);
+        break;
+    case CNH_I64:
+        hipLaunchKernelGGL(reduce_final_seq<int64_t>, dim3(1), dim3(64), 0, st,
+                           (const int64_t*)partials, n_partials, (int64_t*)out);
+        break;
+    default: return set_error(-2, "unknown dtype %d", dtype);
+    }
+    CNH_HIP(hipGetLastError());
+    return 0;
+}
+
+int cnh_sum_tiles(int dtype, int n_tiles, const void* const* a, const int64_t* n, void* out,
+                  cnh_stream s) {
+    if (int rc = ensure_init())
+        return rc;
+    return dispatch_tiles<M_SUM>(dtype, n_tiles, a, nullptr, n, out, as_stream(s));
+}
+
+int cnh_sumsq_diff_tiles(int n_tiles, const void* const* a, const void* const* b, const int64_t* n,
+                         void* out, cnh_stream s) {
+    if (int rc = ensure_init())
+        return rc;
+    return run_tiles<double, M_SUMSQ_DIFF>(n_tiles, a, b, n, out, as_stream(s));
+}
+
+int cnh_maxabs_diff_tiles(int n_tiles, const void* const* a, const void* const* b,
+                          const int64_t* n, void* out, cnh_stream s) {
+    if (int rc = ensure_init())
+        return rc;
+    return run_tiles<double, M_MAXABS_DIFF>(n_tiles, a, b, n, out, as_stream(s));
+}
+
+} // extern "C"

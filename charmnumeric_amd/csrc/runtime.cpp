@@ -1,0 +1,348 @@
+// libcnhip runtime: device selection, storage, copies, streams/events, descriptor cache.
+// Stands in for Array<N,T> storage (src/backend.hpp:112-200 upstream), the row-wise gather of
+// src/partition_get.cpp:42-65 and the fence/callback completion of src/dispatch.hpp:40-53.
+#include "common.h"
+
+#include <cstring>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+namespace cnh {
+
+std::string& error_slot() {
+    static thread_local std::string msg;
+    return msg;
+}
+
+int set_error(int code, const char* fmt, ...) {
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    error_slot() = buf;
+    return code;
+}
+
+namespace {
+std::mutex g_mu;
+bool g_inited = false;
+int g_device = 0;
+hipStream_t g_upload_stream = nullptr;
+
+struct Workspace {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+};
+std::unordered_map<hipStream_t, Workspace> g_ws;
+
+// Descriptor slab: device memory + pinned host mirror, bump-allocated.
+const size_t kSlabBytes = 16u << 20;
+char* g_slab_dev = nullptr;
+char* g_slab_host = nullptr;
+size_t g_slab_used = 0;
+struct DescEntry {
+    size_t off, bytes;
+};
+std::unordered_map<uint64_t, std::vector<DescEntry>> g_desc;
+
+uint64_t fnv1a(const void* p, size_t n) {
+    const unsigned char* b = static_cast<const unsigned char*>(p);
+    uint64_t h = 1469598103934665603ull;
+    for (size_t i = 0; i < n; ++i) {
+        h ^= b[i];
+        h *= 1099511628211ull;
+    }
+    return h;
+}
+} // namespace
+
+int ensure_init() {
+    if (g_inited)
+        return 0;
+    return cnh_init(0);
+}
+
+int reduce_workspace(hipStream_t s, size_t bytes, void** out) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    Workspace& w = g_ws[s];
+    if (w.bytes < bytes) {
+        // The old block may still be read by kernels in flight on `s`; it is parked, not freed.
+        size_t want = bytes < (1u << 20) ? (1u << 20) : bytes;
+        void* p = nullptr;
+        CNH_HIP(hipMalloc(&p, want));
+        w.ptr = p;
+        w.bytes = want;
+    }
+    *out = w.ptr;
+    return 0;
+}
+
+int desc_upload(const void* host, size_t bytes, hipStream_t, const void** dev_out) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (!g_slab_dev) {
+        CNH_HIP(hipMalloc((void**)&g_slab_dev, kSlabBytes));
+        CNH_HIP(hipHostMalloc((void**)&g_slab_host, kSlabBytes, hipHostMallocDefault));
+        CNH_HIP(hipStreamCreateWithFlags(&g_upload_stream, hipStreamNonBlocking));
+    }
+    CNH_CHECK(bytes <= kSlabBytes / 4, -3, "descriptor table of %zu bytes is too large", bytes);
+    uint64_t h = fnv1a(host, bytes);
+    auto it = g_desc.find(h);
+    if (it != g_desc.end())
+        for (const DescEntry& e : it->second)
+            if (e.bytes == bytes && std::memcmp(g_slab_host + e.off, host, bytes) == 0) {
+                *dev_out = g_slab_dev + e.off;
+                return 0;
+            }
+    size_t need = (bytes + 255) & ~size_t(255);
+    if (g_slab_used + need > kSlabBytes) {
+        // Tables handed out earlier may still be in use by queued kernels: drain, then recycle.
+        CNH_HIP(hipDeviceSynchronize());
+        g_desc.clear();
+        g_slab_used = 0;
+    }
+    size_t off = g_slab_used;
+    g_slab_used += need;
+    std::memcpy(g_slab_host + off, host, bytes);
+    CNH_HIP(hipMemcpyAsync(g_slab_dev + off, g_slab_host + off, bytes, hipMemcpyHostToDevice,
+                           g_upload_stream));
+    CNH_HIP(hipStreamSynchronize(g_upload_stream));
+    g_desc[h].push_back({off, bytes});
+    *dev_out = g_slab_dev + off;
+    return 0;
+}
+
+} // namespace cnh
+
+using namespace cnh;
+
+extern "C" {
+
+int cnh_version(void) { return 100; }
+
+const char* cnh_last_error(void) { return error_slot().c_str(); }
+
+int cnh_init(int device) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (g_inited && device == g_device)
+        return 0;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0)
+        return set_error(-101, "no HIP device available (%s)",
+                         e == hipSuccess ? "device count is 0" : hipGetErrorString(e));
+    CNH_CHECK(device >= 0 && device < count, -2, "device %d out of range (have %d)", device, count);
+    CNH_HIP(hipSetDevice(device));
+    g_device = device;
+    g_inited = true;
+    return 0;
+}
+
+int cnh_device_name(char* buf, size_t cap) {
+    if (int rc = ensure_init())
+        return rc;
+    hipDeviceProp_t prop;
+    CNH_HIP(hipGetDeviceProperties(&prop, g_device));
+    snprintf(buf, cap, "%s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
+    return 0;
+}
+
+int cnh_alloc(size_t bytes, int zero, void** dptr) {
+    if (int rc = ensure_init())
+        return rc;
+    CNH_CHECK(dptr != nullptr, -2, "cnh_alloc: null output pointer");
+    void* p = nullptr;
+    CNH_HIP(hipMalloc(&p, bytes ? bytes : 1));
+    if (zero && bytes)
+        CNH_HIP(hipMemset(p, 0, bytes));
+    *dptr = p;
+    return 0;
+}
+
+int cnh_free(void* dptr) {
+    if (!dptr)
+        return 0;
+    CNH_HIP(hipFree(dptr));
+    return 0;
+}
+
+int cnh_h2d(void* dst, const void* src, size_t bytes, cnh_stream s) {
+    if (int rc = ensure_init())
+        return rc;
+    if (bytes == 0)
+        return 0;
+    CNH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, as_stream(s)));
+    CNH_HIP(hipStreamSynchronize(as_stream(s)));
+    return 0;
+}
+
+int cnh_d2h(void* dst, const void* src, size_t bytes, cnh_stream s) {
+    if (int rc = ensure_init())
+        return rc;
+    if (bytes == 0)
+        return 0;
+    CNH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, as_stream(s)));
+    CNH_HIP(hipStreamSynchronize(as_stream(s)));
+    return 0;
+}
+
+int cnh_d2d(void* dst, const void* src, size_t bytes, cnh_stream s) {
+    if (int rc = ensure_init())
+        return rc;
+    if (bytes == 0)
+        return 0;
+    CNH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, as_stream(s)));
+    return 0;
+}
+
+int cnh_d2h_region(int nd, int esz, void* dst_host, const int64_t* dst_strides,
+                   const int64_t* dst_start, const void* src_dev, const int64_t* src_strides,
+                   const int64_t* src_start, const int64_t* counts, cnh_stream s) {
+    if (int rc = ensure_init())
+        return rc;
+    CNH_CHECK(nd >= 1 && nd <= CNH_MAX_ND, -2, "cnh_d2h_region: ndims %d not in 1..3", nd);
+    CNH_CHECK(esz == 4 || esz == 8, -2, "cnh_d2h_region: element size %d not in {4,8}", esz);
+    CNH_CHECK(dst_strides[nd - 1] == 1 && src_strides[nd - 1] == 1, -2,
+              "cnh_d2h_region: innermost stride must be 1");
+    for (int d = 0; d < nd; ++d)
+        if (counts[d] <= 0)
+            return 0;
+    int64_t doff = 0, soff = 0;
+    for (int d = 0; d < nd; ++d) {
+        doff += dst_start[d] * dst_strides[d];
+        soff += src_start[d] * src_strides[d];
+    }
+    char* dbase = static_cast<char*>(dst_host) + doff * esz;
+    const char* sbase = static_cast<const char*>(src_dev) + soff * esz;
+    hipStream_t st = as_stream(s);
+    if (nd == 1) {
+        CNH_HIP(hipMemcpyAsync(dbase, sbase, (size_t)counts[0] * esz, hipMemcpyDeviceToHost, st));
+    } else {
+        // One 2-D copy per outermost index (a single one for ndims == 2).
+        int64_t planes = nd == 3 ? counts[0] : 1;
+        int rd = nd - 2; // row dimension
+        for (int64_t p = 0; p < planes; ++p) {
+            char* dp = dbase + (nd == 3 ? p * dst_strides[0] * esz : 0);
+            const char* sp = sbase + (nd == 3 ? p * src_strides[0] * esz : 0);
+            CNH_HIP(hipMemcpy2DAsync(dp, (size_t)dst_strides[rd] * esz, sp,
+                                     (size_t)src_strides[rd] * esz, (size_t)counts[nd - 1] * esz,
+                                     (size_t)counts[rd], hipMemcpyDeviceToHost, st));
+        }
+    }
+    CNH_HIP(hipStreamSynchronize(st));
+    return 0;
+}
+
+int cnh_stream_create(cnh_stream* out) {
+    if (int rc = ensure_init())
+        return rc;
+    hipStream_t st;
+    CNH_HIP(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
+    *out = st;
+    return 0;
+}
+
+int cnh_stream_destroy(cnh_stream s) {
+    if (!s)
+        return 0;
+    CNH_HIP(hipStreamDestroy(as_stream(s)));
+    return 0;
+}
+
+int cnh_stream_sync(cnh_stream s) {
+    if (int rc = ensure_init())
+        return rc;
+    CNH_HIP(hipStreamSynchronize(as_stream(s)));
+    return 0;
+}
+
+namespace {
+struct HostCb {
+    void (*fn)(void*);
+    void* arg;
+};
+void host_cb_trampoline(void* p) {
+    HostCb* cb = static_cast<HostCb*>(p);
+    cb->fn(cb->arg);
+    delete cb;
+}
+} // namespace
+
+int cnh_stream_callback(cnh_stream s, void (*fn)(void*), void* arg) {
+    if (int rc = ensure_init())
+        return rc;
+    CNH_CHECK(fn != nullptr, -2, "cnh_stream_callback: null function");
+    HostCb* cb = new HostCb{fn, arg};
+    hipError_t e = hipLaunchHostFunc(as_stream(s), host_cb_trampoline, cb);
+    if (e != hipSuccess) {
+        delete cb;
+        return set_error(-100, "hipLaunchHostFunc failed: %s", hipGetErrorString(e));
+    }
+    return 0;
+}
+
+int cnh_device_sync(void) {
+    if (int rc = ensure_init())
+        return rc;
+    CNH_HIP(hipDeviceSynchronize());
+    return 0;
+}
+
+int cnh_event_create(cnh_event* out) {
+    if (int rc = ensure_init())
+        return rc;
+    hipEvent_t e;
+    CNH_HIP(hipEventCreate(&e));
+    *out = e;
+    return 0;
+}
+
+int cnh_event_destroy(cnh_event e) {
+    if (!e)
+        return 0;
+    CNH_HIP(hipEventDestroy(reinterpret_cast<hipEvent_t>(e)));
+    return 0;
+}
+
+int cnh_event_record(cnh_event e, cnh_stream s) {
+    CNH_HIP(hipEventRecord(reinterpret_cast<hipEvent_t>(e), as_stream(s)));
+    return 0;
+}
+
+int cnh_event_sync(cnh_event e) {
+    CNH_HIP(hipEventSynchronize(reinterpret_cast<hipEvent_t>(e)));
+    return 0;
+}
+
+int cnh_event_elapsed_ms(cnh_event a, cnh_event b, float* ms) {
+    CNH_HIP(hipEventElapsedTime(ms, reinterpret_cast<hipEvent_t>(a), reinterpret_cast<hipEvent_t>(b)));
+    return 0;
+}
+
+int cnh_scalar_to_dtype(int dtype, double s, void* out8) {
+    std::memset(out8, 0, 8);
+    switch (dtype) {
+    case CNH_F32: {
+        float v = (float)s;
+        std::memcpy(out8, &v, 4);
+        return 0;
+    }
+    case CNH_F64:
+        std::memcpy(out8, &s, 8);
+        return 0;
+    case CNH_I32: {
+        int32_t v = (int32_t)s;
+        std::memcpy(out8, &v, 4);
+        return 0;
+    }
+    case CNH_I64: {
+        int64_t v = (int64_t)s;
+        std::memcpy(out8, &v, 8);
+        return 0;
+    }
+    }
+    return set_error(-2, "cnh_scalar_to_dtype: unknown dtype %d", dtype);
+}
+
+} // extern "C"

@@ -1,0 +1,238 @@
+/*
+ * cnhip.h — C ABI of libcnhip: the MI355X (gfx950) executor back end for charmnumeric's
+ * per-partition array execution path.
+ *
+ * Each entry point replaces one seam of the upstream C++ backend; the comment on every
+ * declaration names the upstream function (file:line in the charmnumeric tree) it stands in for.
+ *
+ * Conventions
+ *   - return 0 on success, < 0 on error; cnh_last_error() returns the message of the last error
+ *     raised on the calling thread. Nothing throws or aborts across this boundary.
+ *   - the library never frees caller memory and never keeps a host pointer past return.
+ *   - sizes, strides and offsets are in ELEMENTS (int64), as in the upstream MemRef descriptor.
+ *   - dtype codes are the wire values F32=0, F64=1, I32=2, I64=3 (charmnumeric.py:34-40).
+ *   - a cnh_stream of NULL is the device's default stream. Work on one stream is ordered.
+ *   - one thread per handle at a time (the upstream scheduler runs entry methods to completion).
+ */
+#ifndef CNHIP_H
+#define CNHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CNH_MAX_ND 3
+
+/* Opcode numbering: src/opcodes.hpp:3-20. */
+enum {
+    CNH_OP_COPY = -5, CNH_OP_SET_REGION = -4, CNH_OP_GET_REGION = -3, CNH_OP_CREATE = -2,
+    CNH_OP_NOOP = -1, CNH_OP_ADD = 0, CNH_OP_SUB = 1, CNH_OP_MUL = 2, CNH_OP_DIV = 3,
+    CNH_OP_MATMUL = 4, CNH_OP_TANH = 5, CNH_OP_EXP = 6, CNH_OP_TILE = 7, CNH_OP_REDUCE = 8,
+    CNH_OP_MATMATMUL = 9, CNH_OP_DIAG = 10
+};
+enum { CNH_F32 = 0, CNH_F64 = 1, CNH_I32 = 2, CNH_I64 = 3 };
+
+typedef void* cnh_stream;
+typedef void* cnh_event;
+
+/* ArrayRegion<N> (src/array_region.hpp:21-33); N <= 3 carried at run time. */
+typedef struct cnh_region {
+    int32_t is_global;
+    int32_t ndims;
+    int32_t start[CNH_MAX_ND];
+    int32_t stop[CNH_MAX_ND];
+    int32_t step[CNH_MAX_ND];
+} cnh_region;
+
+/* One AST node, with the fields the upstream backend reads from charmtyles' ASTNode
+ * (src/jit.cpp:223-385, src/execute_node_regions.cpp:56-107, tests/test_jit.cpp:35-46).
+ * operands[] index into the flat node array; leaves are NOOP/CREATE nodes. */
+typedef struct cnh_ast_node {
+    int32_t result_name;
+    int32_t opcode;
+    int32_t is_temp;
+    int32_t is_scalar;
+    int32_t is_broadcast;
+    int32_t ndims;
+    int32_t dtype;
+    int32_t n_operands;
+    int32_t operands[2];
+    int32_t has_operand_region[2];
+    double scalar;
+    cnh_region operand_regions[2];
+    cnh_region region;
+} cnh_ast_node;
+
+/* AST{roots[]}: flat, temporaries first (src/jit.cpp:120-122). */
+typedef struct cnh_ast {
+    int32_t n_nodes;
+    int32_t n_roots;
+    const cnh_ast_node* nodes;
+    const int32_t* roots;
+} cnh_ast;
+
+/* MemRef<N,T> {allocated, aligned, offset, sizes[N], strides[N]} (src/array_region.hpp:404-415). */
+typedef struct cnh_memref {
+    void* allocated;
+    void* aligned;
+    int64_t offset;
+    int64_t sizes[CNH_MAX_ND];
+    int64_t strides[CNH_MAX_ND];
+} cnh_memref;
+
+/* ---- library state ---- */
+int cnh_init(int device);               /* selects the device; idempotent */
+const char* cnh_last_error(void);
+int cnh_device_name(char* buf, size_t cap);
+int cnh_version(void);
+
+/* ---- storage: Array<N,T> ctor zero-fill / data_ptr / copyToHost / copyToDevice / dtor
+ *      (src/backend.hpp:112-200) ---- */
+int cnh_alloc(size_t bytes, int zero, void** dptr);
+int cnh_free(void* dptr);
+int cnh_memset0(void* dptr, size_t bytes, cnh_stream s);
+int cnh_h2d(void* dst_dev, const void* src_host, size_t bytes, cnh_stream s); /* returns after the copy */
+int cnh_d2h(void* dst_host, const void* src_dev, size_t bytes, cnh_stream s); /* returns after the copy */
+int cnh_d2d(void* dst_dev, const void* src_dev, size_t bytes, cnh_stream s);  /* asynchronous */
+/* Strided device -> host gather of one tile into a global row-major host buffer; replaces the
+ * one-message-per-innermost-row gather of src/partition_get.cpp:42-65 +
+ * src/dag_group_runtime.cpp:99-118. counts/strides/starts in elements. */
+int cnh_d2h_region(int ndims, int esz, void* dst_host, const int64_t* dst_strides,
+                   const int64_t* dst_start, const void* src_dev, const int64_t* src_strides,
+                   const int64_t* src_start, const int64_t* counts, cnh_stream s);
+
+/* ---- completion: CT_KOKKOS_FENCE / hapiAddCallback (src/executor_core.cpp:618-627,761-774,
+ *      src/dispatch.hpp:40-53) ---- */
+int cnh_stream_create(cnh_stream* out);
+int cnh_stream_destroy(cnh_stream s);
+int cnh_stream_sync(cnh_stream s);
+int cnh_stream_callback(cnh_stream s, void (*fn)(void*), void* arg);
+int cnh_device_sync(void);
+int cnh_event_create(cnh_event* out);
+int cnh_event_destroy(cnh_event e);
+int cnh_event_record(cnh_event e, cnh_stream s);
+int cnh_event_sync(cnh_event e);
+int cnh_event_elapsed_ms(cnh_event start, cnh_event stop, float* ms);
+
+/* ---- SET_REGION scalar fill and strided copy; halo pack/unpack
+ *      (src/executor_ast_visitor.cpp:112-313, src/executor_core.cpp:8-143,
+ *       src/execute_node.cpp:1001-1181). Element i of dim d is at
+ *      (start[d] + i*step[d]) * strides[d]. Byte-wise, bit-exact; esz in {4, 8}. ---- */
+int cnh_fill_region(int ndims, int esz, void* dst, const int64_t* dst_strides,
+                    const int64_t* dst_start, const int64_t* dst_step, const int64_t* counts,
+                    const void* scalar8, cnh_stream s);
+int cnh_copy_region(int ndims, int esz, void* dst, const int64_t* dst_strides,
+                    const int64_t* dst_start, const int64_t* dst_step, const void* src,
+                    const int64_t* src_strides, const int64_t* src_start, const int64_t* src_step,
+                    const int64_t* counts, cnh_stream s);
+/* Scalar -> dtype conversion used by the fill ((T)double, src/executor_ast_visitor.cpp:112-147). */
+int cnh_scalar_to_dtype(int dtype, double s, void* out8);
+
+/* ---- fused groups: ArrayDAGGroup::compile_node (src/dag_group_compile.cpp:6-56) and
+ *      dispatch_kernel<N,T> (src/dispatch.hpp:137-265) ---- */
+typedef struct cnh_kernel cnh_kernel;
+/* Generates HIP source for the group and registers it under `key` (the upstream cache key is
+ * node->identifier). Non-zero return = "could not compile": the caller falls back, as upstream
+ * does on a null compile result (src/execute_node.cpp:102-112). Code objects are built with
+ * hipRTC on first launch of each kernel variant. */
+int cnh_compile_group(const cnh_ast* ast, int dtype, int ndims, uint64_t key, cnh_kernel** out);
+int cnh_kernel_release(cnh_kernel* k);
+/* Argument counts in the upstream order: memref per leaf use, scalar per unique broadcast leaf,
+ * memref per non-temp root (src/jit.cpp:78-87). */
+int cnh_kernel_signature(const cnh_kernel* k, int* n_in, int* n_scalar, int* n_out);
+/* Generated source of one variant ("flat", "nd", "tiles"), NUL-terminated; returns needed size. */
+int64_t cnh_kernel_source(cnh_kernel* k, const char* variant, char* buf, size_t cap);
+/* Builds the code object of one variant for gfx950 without loading it (works without a GPU). */
+int cnh_kernel_build(cnh_kernel* k, const char* variant);
+/* One fragment / one tile. scalars[i] points at one element of the group dtype; with
+ * scalars_on_device != 0 they are device pointers and are read by the kernel itself (no host
+ * round trip for dot results feeding later groups). */
+int cnh_launch_group(cnh_kernel* k, int ndims, int n_in, const cnh_memref* in, int n_scalar,
+                     const void* const* scalars, int scalars_on_device, int n_out,
+                     const cnh_memref* out, cnh_stream s);
+/* All partitions (or all aligned cells) of a node in ONE launch: in[p*n_in + i], out[p*n_out + o]. */
+int cnh_launch_group_batched(cnh_kernel* k, int ndims, int n_parts, int n_in, const cnh_memref* in,
+                             int n_scalar, const void* const* scalars, int scalars_on_device,
+                             int n_out, const cnh_memref* out, cnh_stream s);
+
+/* Shifted-slice groups over tiles that all live on this device: replaces send_remote_input +
+ * receive_data + align_fragments + M kernel calls + the SET_REGION copy
+ * (src/executor_core.cpp:8-143,684-747, src/partition_comm.cpp:26-61,
+ *  src/execute_node.cpp:1338-1585, src/executor_ast_visitor.cpp:268-311) by one launch that
+ * reads neighbour tiles directly and writes every tile of the target.
+ * A tiled array is described by its decomposition (tile edge, per-dim offset and shape,
+ * src/array_region.hpp:293-387) and a table of tile base pointers in row-major tile-grid order;
+ * every tile is row-major contiguous over its own local extent (src/backend.hpp:112-200). */
+typedef struct cnh_tiled {
+    int32_t ndims;
+    int32_t tile;
+    int32_t offset[CNH_MAX_ND];
+    int32_t shape[CNH_MAX_ND];
+    int32_t grid_lo[CNH_MAX_ND];   /* first tile index per dim: offset / tile */
+    int32_t grid[CNH_MAX_ND];      /* tiles per dim */
+    void* const* tiles;            /* host array of device pointers, prod(grid) entries */
+} cnh_tiled;
+/* in[i] describes the array behind leaf use i (regions come from the AST); dst is where the
+ * SET_REGION target's new contents are written (all elements of every tile: computed inside the
+ * assigned region, copied from `cur` outside it); cur is the target's current contents. dst may
+ * equal cur only when no input aliases the target with a different region. */
+int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* in, int n_scalar,
+                           const void* const* scalars, int scalars_on_device,
+                           const cnh_tiled* cur, const cnh_tiled* dst, cnh_stream s);
+
+/* ---- REDUCE: eigen_dot + contribute + reduce_dot_sum + reduce_result
+ *      (src/backend_internal.hpp:88-93, src/executor_reduce.cpp:8-119,
+ *       src/executor_reducer.cpp:11-57, src/partition_comm.cpp:69-111) ---- */
+/* dot of one 1-D tile -> *partial_slot (device). Fixed grid and fixed-order tree: the result
+ * depends only on (n, data), never on scheduling. */
+int cnh_dot_partial(int dtype, int64_t n, const void* a, const void* b, void* partial_slot,
+                    cnh_stream s);
+/* Sequential sum of the per-tile partials in index order -> *out (device). */
+int cnh_reduce_final(int dtype, int n_partials, const void* partials, void* out, cnh_stream s);
+/* All tiles in one launch + the final pass: out = sum_t dot(a[t], b[t]), tiles in index order. */
+int cnh_dot_tiles(int dtype, int n_tiles, const void* const* a, const void* const* b,
+                  const int64_t* n, void* out, cnh_stream s);
+/* Extensions with no upstream counterpart (upstream REDUCE is 1-D dot only,
+ * src/executor_reduce.cpp:9-12): sum of elements, sum of squared differences, max |a-b|,
+ * over lists of contiguous chunks. fp64 only for the last two. */
+int cnh_sum_tiles(int dtype, int n_tiles, const void* const* a, const int64_t* n, void* out,
+                  cnh_stream s);
+int cnh_sumsq_diff_tiles(int n_tiles, const void* const* a, const void* const* b, const int64_t* n,
+                         void* out, cnh_stream s);
+int cnh_maxabs_diff_tiles(int n_tiles, const void* const* a, const void* const* b,
+                          const int64_t* n, void* out, cnh_stream s);
+
+/* ---- MATMUL (matvec): eigen_gemv_sub + 1-D partial accumulate
+ *      (src/backend_internal.hpp:28-41, src/execute_node.cpp:226-229,563-577) ---- */
+/* y[i] = beta*y[i] + sum_j A[i*lda + j] * x[j], beta in {0,1}; row-major. */
+int cnh_gemv(int dtype, int64_t rows, int64_t cols, const void* A, int64_t lda, const void* x,
+             void* y, int beta, cnh_stream s);
+/* y += partial (src/execute_node.cpp:572-576). */
+int cnh_axpy1(int dtype, int64_t n, const void* partial, void* y, cnh_stream s);
+/* The whole tiled matvec in one launch: A is a grid_r x grid_c grid of row-major tiles
+ * (tile (i,j) holds rows [i*tile, ..) x cols [j*tile, ..) of a rows x cols matrix, row stride =
+ * its own column count); y[r] = sum over column tiles j = 0,1,.. in that order. */
+int cnh_gemv_tiles(int dtype, int64_t rows, int64_t cols, int32_t tile, const void* const* tiles,
+                   const void* x, void* y, cnh_stream s);
+
+/* ---- MATMATMUL: C += A_panel * B_panel, row-major with row strides
+ *      (src/backend_internal.hpp:113-133, src/executor_incremental.cpp:97-132) ---- */
+int cnh_gemm_acc(int dtype, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda,
+                 const void* B, int64_t ldb, void* C, int64_t ldc, cnh_stream s);
+
+/* ---- synthetic inputs generated on the device (no upstream counterpart: upstream has no RNG,
+ *      charmnumeric/random.py:4-5, and no bulk upload, charmnumeric.py:863-878) ---- */
+/* out[k] = lo + (hi-lo)*u01(seed, stream_id, first+k); counter-based SplitMix64, fp64. */
+int cnh_fill_uniform(double* out, int64_t n, uint64_t seed, uint64_t stream_id, uint64_t first,
+                     double lo, double hi, cnh_stream s);
+/* Block of the dense CG test matrix of order n (symmetric, diagonal 2.0). */
+int cnh_fill_cg_matrix(double* out, int64_t n, int64_t row0, int64_t nrows, int64_t col0,
+                       int64_t ncols, int64_t ld, uint64_t seed, cnh_stream s);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

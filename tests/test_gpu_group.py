@@ -1,0 +1,223 @@
+"""GPU parity: fused groups through the C ABI vs the CPU oracle (bit-exact for + - * /)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from charmnumeric_amd import _lib as L
+from charmnumeric_amd.astbuild import AstBuilder
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def _run_c1(dev, orc, n, parts, dtype=L.F64, misalign=0):
+    npdt = H.NP[dtype]
+    if dtype in (L.F64, L.F32):
+        x = orc.uniform(n, 0, 0, -1.0, 1.0).astype(npdt)
+        y = orc.uniform(n, 0, 1, -1.0, 1.0).astype(npdt)
+    else:
+        rng = np.random.default_rng(3)
+        x = rng.integers(-1000, 1000, n).astype(npdt)
+        y = rng.integers(-1000, 1000, n).astype(npdt)
+    ast = H.ast_c1(dtype)
+    k = H.compile_group(ast, dtype, 1)
+    bounds = np.linspace(0, n, parts + 1).astype(np.int64)
+    ins, outs, zbufs = [], [], []
+    for p in range(parts):
+        lo, hi = int(bounds[p]), int(bounds[p + 1])
+        pad = misalign
+        xb = dev.array(np.concatenate([np.zeros(pad, npdt), x[lo:hi]]))
+        yb = dev.array(np.concatenate([np.zeros(pad, npdt), y[lo:hi]]))
+        zb = dev.empty((hi - lo + pad,), npdt)
+        mx = L.Memref.dense(xb.ptr, (hi - lo,), offset=pad)
+        my = L.Memref.dense(yb.ptr, (hi - lo,), offset=pad)
+        mz = L.Memref.dense(zb.ptr, (hi - lo,), offset=pad)
+        ins.append([mx, my, mx, my])  # one memref per leaf use: x, y, x, y
+        outs.append([mz])
+        zbufs.append((zb, pad))
+    H.launch_batched(k, 1, ins, [], outs)
+    dev.sync()
+    got = np.concatenate([zb.get()[pad:] for zb, pad in zbufs])
+    want = np.empty(n, npdt)
+    assert orc.eval_group(ast, dtype, 1, [x, y, x, y], [], [want]) == 0
+    L.check(L.lib.cnh_kernel_release(k))
+    dev.free_all()
+    return got, want, x, y
+
+
+@pytest.mark.parametrize("n,parts", [(1 << 20, 4), (1000003, 3), (17, 1), (2048, 1), (5000, 7)])
+def test_c1_fused_elementwise_bit_exact(dev, orc, n, parts):
+    got, want, x, y = _run_c1(dev, orc, n, parts)
+    assert np.array_equal(got.view(np.int64), want.view(np.int64))
+    # closed form in NumPy, same operand order
+    ref = ((2.5 * x) - (0.5 * y)) + (x * y)
+    assert np.array_equal(got.view(np.int64), ref.view(np.int64))
+
+
+def test_c1_misaligned_pointers_use_scalar_path(dev, orc):
+    got, want, _, _ = _run_c1(dev, orc, 100001, 2, misalign=1)
+    assert np.array_equal(got.view(np.int64), want.view(np.int64))
+
+
+@pytest.mark.parametrize("dtype", [L.F32, L.I32, L.I64])
+def test_c1_other_dtypes_bit_exact(dev, orc, dtype):
+    got, want, _, _ = _run_c1(dev, orc, 70001, 2, dtype=dtype)
+    assert got.tobytes() == want.tobytes()
+
+
+def test_c1_full_size_properties(dev, orc):
+    """2^24 elements in 4 partitions: bit-exact vs NumPy and linear in the partition split."""
+    got, want, x, y = _run_c1(dev, orc, 1 << 24, 4)
+    ref = ((2.5 * x) - (0.5 * y)) + (x * y)
+    assert np.array_equal(got.view(np.int64), ref.view(np.int64))
+    got1, _, _, _ = _run_c1(dev, orc, 1 << 24, 1)
+    assert np.array_equal(got.view(np.int64), got1.view(np.int64))
+
+
+def test_reference_elementwise_known_answer(dev, orc):
+    """2*(a+b+3) with a=1.5, b=-0.5 in f32 is 8.0 everywhere (upstream integration test)."""
+    b = AstBuilder(L.F32, 1)
+    a_, b_ = b.leaf(0), b.leaf(1)
+    t1 = b.binary(L.OP_ADD, 100, a_, b_)
+    t2 = b.binary(L.OP_ADD, 101, t1, b.scalar(3.0))
+    b.binary(L.OP_MUL, 2, b.scalar(2.0), t2, is_temp=False)
+    ast = b.finish()
+    k = H.compile_group(ast, L.F32, 1)
+    av = dev.array(np.full(32, 1.5, np.float32))
+    bv = dev.array(np.full(32, -0.5, np.float32))
+    out = dev.empty((32,), np.float32)
+    H.launch_batched(k, 1, [[av.memref(), bv.memref()]], [], [[out.memref()]])
+    assert np.array_equal(out.get(), np.full(32, 8.0, np.float32))
+    dev.free_all()
+
+
+def test_strided_cells_2d_3d(dev, orc):
+    """Strided views (the fragment path's aligned cells) go through the 'nd' variant."""
+    rng = np.random.default_rng(5)
+    for nd, shape, sl in [
+        (2, (37, 53), (slice(3, 30), slice(5, 50, 2))),
+        (3, (9, 14, 40), (slice(1, 8), slice(2, 13, 3), slice(0, 39))),
+        (1, (1000,), (slice(10, 900, 7),)),
+    ]:
+        a = rng.standard_normal(shape)
+        bq = rng.standard_normal(shape)
+        bld = AstBuilder(L.F64, nd)
+        la, lb = bld.leaf(0), bld.leaf(1)
+        t = bld.binary(L.OP_DIV, 100, la, lb)
+        bld.binary(L.OP_SUB, 2, t, bld.scalar(0.1), is_temp=False)
+        ast = bld.finish()
+        k = H.compile_group(ast, L.F64, nd)
+        va, vb = a[sl], bq[sl]
+        da, db = dev.array(a), dev.array(bq)
+        out = dev.array(np.zeros(shape))
+
+        def view_mr(buf, host, view):
+            off = (view.__array_interface__["data"][0] - host.__array_interface__["data"][0]) // 8
+            return L.Memref.strided(buf.ptr, view.shape, [s // 8 for s in view.strides], off)
+
+        oh = np.zeros(shape)
+        ov = oh[sl]
+        H.launch_batched(k, nd, [[view_mr(da, a, va), view_mr(db, bq, vb)]], [],
+                         [[view_mr(out, oh, ov)]])
+        got = out.get()
+        want = np.zeros(shape)
+        assert orc.eval_group(ast, L.F64, nd, [va, vb], [], [want[sl]]) == 0
+        assert np.array_equal(got.view(np.int64), want.view(np.int64))
+        assert np.array_equal(want[sl], (va / vb) - 0.1)
+        dev.free_all()
+
+
+def test_broadcast_scalars_device_and_host(dev, orc):
+    """x + alpha*p with alpha a size-1 device array (the CG update); scalar/scalar op alpha=a/b."""
+    n = 4099
+    x = orc.uniform(n, 7, 0, -1, 1)
+    p = orc.uniform(n, 7, 1, -1, 1)
+    b = AstBuilder(L.F64, 1)
+    lx, lp = b.leaf(0), b.leaf(1)
+    al = b.broadcast(5)
+    t = b.binary(L.OP_MUL, 100, al, lp)
+    b.binary(L.OP_ADD, 2, lx, t, is_temp=False)
+    ast = b.finish()
+    k = H.compile_group(ast, L.F64, 1)
+    dx, dp = dev.array(x), dev.array(p)
+    alpha = np.array([0.37], np.float64)
+    dal = dev.array(alpha)
+    out = dev.empty((n,), np.float64)
+    H.launch_batched(k, 1, [[dx.memref(), dp.memref()]], [dal.ptr], [[out.memref()]],
+                     scalars_on_device=True)
+    got_dev = out.get()
+    out2 = dev.empty((n,), np.float64)
+    H.launch_batched(k, 1, [[dx.memref(), dp.memref()]], [alpha.ctypes.data], [[out2.memref()]],
+                     scalars_on_device=False)
+    got_host = out2.get()
+    want = np.empty(n)
+    assert orc.eval_group(ast, L.F64, 1, [x, p], [0.37], [want]) == 0
+    assert np.array_equal(got_dev, want) and np.array_equal(got_host, want)
+    assert np.array_equal(want, x + 0.37 * p)
+
+    # scalar / scalar -> one element
+    b2 = AstBuilder(L.F64, 1)
+    s1, s2 = b2.broadcast(6), b2.broadcast(7)
+    b2.binary(L.OP_DIV, 8, s1, s2, is_temp=False)
+    ast2 = b2.finish()
+    k2 = H.compile_group(ast2, L.F64, 1)
+    num, den = dev.array(np.array([3.0])), dev.array(np.array([7.0]))
+    res = dev.empty((1,), np.float64)
+    H.launch_batched(k2, 1, [[]], [num.ptr, den.ptr], [[res.memref()]], scalars_on_device=True)
+    assert res.get()[0] == 3.0 / 7.0
+    dev.free_all()
+
+
+def test_exp_tanh_within_one_ulp_of_host_libm(dev, orc):
+    """sigmoid = 1/(1+exp(x*-1)) and tanh against the oracle's host libm: <= 1 ulp."""
+    xs = np.concatenate([
+        np.linspace(-40, 40, 200001),
+        orc.uniform(200000, 9, 0, -8.0, 8.0),
+        np.array([0.0, -0.0, 1e-300, -1e-300, 1e-8, -1e-8, 0.5, -0.5, 20.0, -20.0, 700.0, -700.0]),
+    ])
+    for which in ("sigmoid", "tanh", "exp"):
+        b = AstBuilder(L.F64, 1)
+        lx = b.leaf(0)
+        if which == "sigmoid":
+            t0 = b.binary(L.OP_MUL, 100, lx, b.scalar(-1))
+            t1 = b.unary(L.OP_EXP, 101, t0)
+            t2 = b.binary(L.OP_ADD, 102, b.scalar(1.0), t1)
+            b.binary(L.OP_DIV, 2, b.scalar(1.0), t2, is_temp=False)
+        elif which == "tanh":
+            b.unary(L.OP_TANH, 2, lx, is_temp=False)
+        else:
+            b.unary(L.OP_EXP, 2, lx, is_temp=False)
+        ast = b.finish()
+        k = H.compile_group(ast, L.F64, 1)
+        dx = dev.array(xs)
+        out = dev.empty(xs.shape, np.float64)
+        H.launch_batched(k, 1, [[dx.memref()]], [], [[out.memref()]])
+        got = out.get()
+        want = np.empty_like(xs)
+        assert orc.eval_group(ast, L.F64, 1, [xs], [], [want]) == 0
+        d = H.ulp_distance(got, want)
+        assert d <= 1, f"{which}: {d} ulp"
+        dev.free_all()
+
+
+def test_error_paths(dev):
+    ast = H.ast_c1(L.F64)
+    k = H.compile_group(ast, L.F64, 1)
+    a = dev.empty((16,), np.float64)
+    m = a.memref()
+    ins = (L.Memref * 4)(m, m, m, m)
+    outs = (L.Memref * 1)(m)
+    # wrong input count
+    rc = L.lib.cnh_launch_group(k, 1, 3, ins, 0, None, 0, 1, outs, None)
+    assert rc < 0 and b"expects 4" in L.lib.cnh_last_error()
+    # wrong rank
+    rc = L.lib.cnh_launch_group(k, 2, 4, ins, 0, None, 0, 1, outs, None)
+    assert rc < 0
+    # tanh on integers cannot be compiled (no integer body upstream either)
+    b = AstBuilder(L.I32, 1)
+    b.unary(L.OP_TANH, 2, b.leaf(0), is_temp=False)
+    kk = C.c_void_p()
+    rc = L.lib.cnh_compile_group(C.byref(b.finish()), L.I32, 1, 0, C.byref(kk))
+    assert rc < 0
+    dev.free_all()

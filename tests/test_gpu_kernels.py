@@ -1,0 +1,327 @@
+"""GPU parity for the non-JIT seams: fill/copy, reductions, matvec, matmatmul, generators."""
+import ctypes as C
+import math
+
+import numpy as np
+import pytest
+
+from charmnumeric_amd import _lib as L
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+REL = 1e-12  # reductions, matvec and matmatmul: |got - ref| <= 1e-12 * sum |terms|
+
+
+def test_generators_match_oracle_and_numpy(dev, orc):
+    n = 100003
+    d = dev.empty((n,), np.float64)
+    L.check(L.lib.cnh_fill_uniform(d.ptr, n, 0, 1, 5, -1.0, 1.0, None))
+    got = d.get()
+    want = orc.uniform(n, 0, 1, -1.0, 1.0, first=5)
+    assert np.array_equal(got, want)
+    assert np.array_equal(got, H.np_uniform(n, 0, 1, -1.0, 1.0, first=5))
+    m = dev.empty((96, 160), np.float64)
+    L.check(L.lib.cnh_fill_cg_matrix(m.ptr, 512, 64, 96, 32, 160, 160, 2, None))
+    got = m.get()
+    want = orc.cg_matrix(512, 64, 96, 32, 160, 2)
+    assert np.array_equal(got, want)
+    full = orc.cg_matrix(512, 0, 512, 0, 512, 2)
+    assert np.array_equal(full, full.T) and np.all(np.diag(full) == 2.0)
+    dev.free_all()
+
+
+@pytest.mark.parametrize("esz,npdt", [(8, np.float64), (4, np.int32)])
+def test_fill_and_copy_region_bit_exact(dev, esz, npdt):
+    rng = np.random.default_rng(1)
+    # strided 17 -> 9 assignment held by the upstream tests: coarse[1:-1,1:-1] = fine[2:-2:2,2:-2:2]
+    n, cn = 17, 9
+    fine = rng.integers(-99, 99, (n, n)).astype(npdt)
+    coarse = np.zeros((cn, cn), npdt)
+    dfine, dcoarse = dev.array(fine), dev.array(coarse)
+    L.check(L.lib.cnh_copy_region(2, esz, dcoarse.ptr, H.L.i64arr([cn, 1]), H.L.i64arr([1, 1]),
+                                  H.L.i64arr([1, 1]), dfine.ptr, H.L.i64arr([n, 1]),
+                                  H.L.i64arr([2, 2]), H.L.i64arr([2, 2]), H.L.i64arr([7, 7]), None))
+    want = coarse.copy()
+    want[1:-1, 1:-1] = fine[2:-2:2, 2:-2:2]
+    assert np.array_equal(dcoarse.get(), want)
+    # 3-D fill of a strided box
+    a = rng.integers(-9, 9, (6, 7, 300)).astype(npdt)
+    da = dev.array(a)
+    val = np.array([5], dtype=npdt)
+    buf8 = np.zeros(8, np.uint8)
+    buf8[:esz] = val.view(np.uint8)
+    L.check(L.lib.cnh_fill_region(3, esz, da.ptr, H.L.i64arr([2100, 300, 1]), H.L.i64arr([1, 0, 3]),
+                                  H.L.i64arr([2, 3, 1]), H.L.i64arr([3, 3, 290]),
+                                  buf8.ctypes.data, None))
+    want = a.copy()
+    want[1:6:2, 0:7:3, 3:293] = 5
+    assert np.array_equal(da.get(), want)
+    # 1-D halo-style pack
+    v = rng.integers(-9, 9, 5000).astype(npdt)
+    dv = dev.array(v)
+    pk = dev.empty((1200,), npdt)
+    L.check(L.lib.cnh_copy_region(1, esz, pk.ptr, H.L.i64arr([1]), H.L.i64arr([0]),
+                                  H.L.i64arr([1]), dv.ptr, H.L.i64arr([1]), H.L.i64arr([100]),
+                                  H.L.i64arr([4]), H.L.i64arr([1200]), None))
+    assert np.array_equal(pk.get(), v[100:4900:4])
+    # empty region is a no-op
+    L.check(L.lib.cnh_copy_region(1, esz, pk.ptr, H.L.i64arr([1]), H.L.i64arr([0]),
+                                  H.L.i64arr([1]), dv.ptr, H.L.i64arr([1]), H.L.i64arr([0]),
+                                  H.L.i64arr([1]), H.L.i64arr([0]), None))
+    dev.free_all()
+
+
+def test_d2h_region_gathers_tiles(dev):
+    g = np.arange(40 * 56, dtype=np.float64).reshape(40, 56)
+    out = np.zeros_like(g)
+    for i in range(0, 40, 16):
+        for j in range(0, 56, 16):
+            t = np.ascontiguousarray(g[i:i + 16, j:j + 16])
+            dt = dev.array(t)
+            L.check(L.lib.cnh_d2h_region(2, 8, out.ctypes.data, H.L.i64arr([56, 1]),
+                                         H.L.i64arr([i, j]), dt.ptr, H.L.i64arr([t.shape[1], 1]),
+                                         H.L.i64arr([0, 0]), H.L.i64arr(list(t.shape)), None))
+    assert np.array_equal(out, g)
+    dev.free_all()
+
+
+def _tiles(dev, arr, parts):
+    bounds = np.linspace(0, arr.size, parts + 1).astype(np.int64)
+    bufs = [dev.array(arr[bounds[i]:bounds[i + 1]]) for i in range(parts)]
+    return bufs, [int(bounds[i + 1] - bounds[i]) for i in range(parts)]
+
+
+@pytest.mark.parametrize("n,parts", [(1 << 22, 4), (16384, 1), (100003, 3), (5, 1), (70000, 1)])
+def test_dot_and_sum_fp64(dev, orc, n, parts):
+    a = orc.uniform(n, 0, 0, -1, 1)
+    b = orc.uniform(n, 0, 1, -1, 1)
+    ab, lens = _tiles(dev, a, parts)
+    bb, _ = _tiles(dev, b, parts)
+    out = dev.empty((1,), np.float64)
+    L.check(L.lib.cnh_dot_tiles(L.F64, parts, L.vparr([x.ptr for x in ab]),
+                                L.vparr([x.ptr for x in bb]), L.i64arr(lens), out.ptr, None))
+    got = out.get()[0]
+    ref = math.fsum((a * b).tolist())
+    denom = math.fsum(np.abs(a * b).tolist())
+    assert abs(got - ref) <= REL * denom
+    assert abs(orc.dot(a, b) - ref) <= REL * denom
+    # determinism: same launch twice gives the same bits
+    out2 = dev.empty((1,), np.float64)
+    L.check(L.lib.cnh_dot_tiles(L.F64, parts, L.vparr([x.ptr for x in ab]),
+                                L.vparr([x.ptr for x in bb]), L.i64arr(lens), out2.ptr, None))
+    assert out2.get()[0].tobytes() == np.float64(got).tobytes()
+    L.check(L.lib.cnh_sum_tiles(L.F64, parts, L.vparr([x.ptr for x in ab]), L.i64arr(lens),
+                                out.ptr, None))
+    got = out.get()[0]
+    assert abs(got - math.fsum(a.tolist())) <= REL * math.fsum(np.abs(a).tolist())
+    dev.free_all()
+
+
+def test_dot_closed_forms_and_ints(dev):
+    # ones . ones = N (upstream examples/reduction.py)
+    for n in (64, 1 << 20):
+        o = dev.array(np.ones(n, np.float32))
+        out = dev.empty((1,), np.float32)
+        L.check(L.lib.cnh_dot_partial(L.F32, n, o.ptr, o.ptr, out.ptr, None))
+        assert out.get()[0] == np.float32(n)
+    # integer dot wraps modulo 2^32 / 2^64: bit-exact whatever the order
+    rng = np.random.default_rng(0)
+    for dt, npdt in ((L.I32, np.int32), (L.I64, np.int64)):
+        a = rng.integers(-2**30, 2**30, 300001).astype(npdt)
+        b = rng.integers(-2**30, 2**30, 300001).astype(npdt)
+        da, db = dev.array(a), dev.array(b)
+        out = dev.empty((1,), npdt)
+        L.check(L.lib.cnh_dot_partial(dt, a.size, da.ptr, db.ptr, out.ptr, None))
+        with np.errstate(over="ignore"):
+            want = np.sum(a * b, dtype=npdt)
+        assert out.get()[0] == want
+    # arange sum
+    n = 100000
+    ar = dev.array(np.arange(n, dtype=np.float64))
+    out = dev.empty((1,), np.float64)
+    L.check(L.lib.cnh_sum_tiles(L.F64, 1, L.vparr([ar.ptr]), L.i64arr([n]), out.ptr, None))
+    assert out.get()[0] == n * (n - 1) / 2
+    dev.free_all()
+
+
+def test_reduce_final_sequential(dev, orc):
+    p = np.array([1e16, 1.0, -1e16, 3.0])
+    dp = dev.array(p)
+    out = dev.empty((1,), np.float64)
+    L.check(L.lib.cnh_reduce_final(L.F64, 4, dp.ptr, out.ptr, None))
+    assert out.get()[0] == ((1e16 + 1.0) + -1e16) + 3.0  # left-to-right, like the upstream reducer
+
+
+def test_sumsq_and_maxabs_diff(dev, orc):
+    n = 300007
+    a = orc.uniform(n, 4, 0, 0, 1)
+    b = orc.uniform(n, 4, 1, 0, 1)
+    ab, lens = _tiles(dev, a, 3)
+    bb, _ = _tiles(dev, b, 3)
+    out = dev.empty((1,), np.float64)
+    L.check(L.lib.cnh_sumsq_diff_tiles(3, L.vparr([x.ptr for x in ab]),
+                                       L.vparr([x.ptr for x in bb]), L.i64arr(lens), out.ptr, None))
+    ref = math.fsum(((a - b) ** 2).tolist())
+    assert abs(out.get()[0] - ref) <= REL * ref
+    L.check(L.lib.cnh_maxabs_diff_tiles(3, L.vparr([x.ptr for x in ab]),
+                                        L.vparr([x.ptr for x in bb]), L.i64arr(lens), out.ptr, None))
+    assert out.get()[0] == np.max(np.abs(a - b))  # exact, order-independent
+    dev.free_all()
+
+
+def _check_matvec(got, A, x):
+    ref = np.array([math.fsum((A[i] * x).tolist()) for i in range(A.shape[0])])
+    denom = np.abs(A) @ np.abs(x)
+    assert np.all(np.abs(got - ref) <= REL * denom + 1e-300)
+
+
+def test_gemv_closed_forms(dev):
+    # A[i,j] = i + j, x = 1  =>  y_i = N*i + N(N-1)/2 exactly (upstream examples/matvec.py)
+    n = 512
+    A = np.add.outer(np.arange(n, dtype=np.float64), np.arange(n, dtype=np.float64))
+    dA, dx, dy = dev.array(A), dev.array(np.ones(n)), dev.empty((n,), np.float64)
+    L.check(L.lib.cnh_gemv(L.F64, n, n, dA.ptr, n, dx.ptr, dy.ptr, 0, None))
+    assert np.array_equal(dy.get(), n * np.arange(n) + n * (n - 1) / 2)
+    # ones(M,N) @ arange(1..N) = N(N+1)/2 (upstream examples/matvec_slice.py)
+    M, N = 96, 1000
+    dA = dev.array(np.ones((M, N)))
+    dx = dev.array(np.arange(1, N + 1, dtype=np.float64))
+    dy = dev.empty((M,), np.float64)
+    L.check(L.lib.cnh_gemv(L.F64, M, N, dA.ptr, N, dx.ptr, dy.ptr, 0, None))
+    assert np.array_equal(dy.get(), np.full(M, N * (N + 1) / 2))
+    dev.free_all()
+
+
+@pytest.mark.parametrize("rows,cols,lda", [(300, 257, 257), (128, 4096, 4100), (1000, 33, 40)])
+def test_gemv_sub_matrix_views(dev, orc, rows, cols, lda):
+    rng = np.random.default_rng(2)
+    full = rng.standard_normal((rows, lda))
+    x = rng.standard_normal(cols)
+    y0 = rng.standard_normal(rows)
+    dA, dx, dy = dev.array(full), dev.array(x), dev.array(y0)
+    L.check(L.lib.cnh_gemv(L.F64, rows, cols, dA.ptr, lda, dx.ptr, dy.ptr, 0, None))
+    _check_matvec(dy.get(), full[:, :cols], x)
+    # beta = 1 accumulates on top of y, then axpy1 adds a partial
+    dy.put(y0)
+    L.check(L.lib.cnh_gemv(L.F64, rows, cols, dA.ptr, lda, dx.ptr, dy.ptr, 1, None))
+    got = dy.get()
+    ref = y0 + full[:, :cols] @ x
+    assert np.allclose(got, ref, rtol=1e-12, atol=1e-12)
+    part = dev.array(y0)
+    L.check(L.lib.cnh_axpy1(L.F64, rows, part.ptr, dy.ptr, None))
+    assert np.array_equal(dy.get(), got + y0)
+    dev.free_all()
+
+
+def test_gemv_tiles_matches_oracle_tiling(dev, orc):
+    """2x2 (ragged) tile grid; partials added in column-tile order like the 1-D accumulate."""
+    rows, cols, tile = 700, 900, 512
+    A = orc.cg_matrix(1024, 0, rows, 0, cols, 2)
+    x = orc.uniform(cols, 2, 1, -1, 1)
+    gr, gc = 2, 2
+    bufs = []
+    for i in range(gr):
+        for j in range(gc):
+            bufs.append(dev.array(np.ascontiguousarray(A[i * tile:(i + 1) * tile,
+                                                         j * tile:(j + 1) * tile])))
+    dx, dy = dev.array(x), dev.empty((rows,), np.float64)
+    L.check(L.lib.cnh_gemv_tiles(L.F64, rows, cols, tile, L.vparr([b.ptr for b in bufs]), dx.ptr,
+                                 dy.ptr, None))
+    got = dy.get()
+    _check_matvec(got, A, x)
+    # oracle: per-tile gemv then sequential accumulate of the partials
+    want = np.zeros(rows)
+    for i in range(gr):
+        acc = None
+        for j in range(gc):
+            t = np.ascontiguousarray(A[i * tile:(i + 1) * tile, j * tile:(j + 1) * tile])
+            part = orc.gemv(t, np.ascontiguousarray(x[j * tile:(j + 1) * tile]))
+            acc = part if acc is None else acc + part
+        want[i * tile:i * tile + acc.size] = acc
+    denom = np.abs(A) @ np.abs(x)
+    assert np.all(np.abs(got - want) <= REL * denom)
+    dev.free_all()
+
+
+@pytest.mark.parametrize("M,N,K", [(64, 64, 16), (128, 192, 64), (70, 50, 33), (256, 512, 256),
+                                   (1, 1, 1), (17, 130, 5)])
+def test_gemm_acc_fp64_mfma(dev, orc, M, N, K):
+    rng = np.random.default_rng(M * 1000 + N + K)
+    A = rng.standard_normal((M, K))
+    B = rng.standard_normal((K, N))
+    C0 = rng.standard_normal((M, N))
+    dA, dB, dC = dev.array(A), dev.array(B), dev.array(C0)
+    L.check(L.lib.cnh_gemm_acc(L.F64, M, N, K, dA.ptr, K, dB.ptr, N, dC.ptr, N, None))
+    got = dC.get()
+    want = orc.gemm_acc(A, B, C0.copy())
+    denom = np.abs(A) @ np.abs(B) + np.abs(C0)
+    assert np.all(np.abs(got - want) <= REL * denom)
+    # independent pin: long double accumulation
+    ref = (A.astype(np.longdouble) @ B.astype(np.longdouble) + C0).astype(np.float64)
+    assert np.all(np.abs(got - ref) <= REL * denom)
+    dev.free_all()
+
+
+def test_gemm_ones_closed_form_and_strided_panels(dev, orc):
+    # ones(M,K) @ ones(K,N) = K exactly (upstream examples/matmatmul.py), C zeroed first
+    M, N, K = 96, 160, 200
+    dA, dB = dev.array(np.ones((M, K))), dev.array(np.ones((K, N)))
+    dC = dev.array(np.zeros((M, N)))
+    L.check(L.lib.cnh_gemm_acc(L.F64, M, N, K, dA.ptr, K, dB.ptr, N, dC.ptr, N, None))
+    assert np.array_equal(dC.get(), np.full((M, N), float(K)))
+    # panels inside larger buffers (row strides > extents), accumulated twice
+    rng = np.random.default_rng(11)
+    Af, Bf, Cf = rng.standard_normal((64, 100)), rng.standard_normal((48, 90)), np.zeros((64, 80))
+    dA, dB, dC = dev.array(Af), dev.array(Bf), dev.array(Cf)
+    for _ in range(2):
+        L.check(L.lib.cnh_gemm_acc(L.F64, 64, 70, 48, dA.ptr + 8 * 4, 100, dB.ptr + 8 * 6, 90,
+                                   dC.ptr + 8 * 2, 80, None))
+    want = Cf.copy()
+    want[:, 2:72] = 2 * (Af[:, 4:52] @ Bf[:, 6:76])
+    assert np.allclose(dC.get(), want, rtol=1e-12, atol=1e-12)
+    dev.free_all()
+
+
+@pytest.mark.parametrize("dt,npdt", [(L.F32, np.float32), (L.I32, np.int32), (L.I64, np.int64)])
+def test_gemm_other_dtypes(dev, orc, dt, npdt):
+    rng = np.random.default_rng(4)
+    M, N, K = 37, 45, 29
+    if npdt == np.float32:
+        A, B = rng.standard_normal((M, K)).astype(npdt), rng.standard_normal((K, N)).astype(npdt)
+    else:
+        A = rng.integers(-50, 50, (M, K)).astype(npdt)
+        B = rng.integers(-50, 50, (K, N)).astype(npdt)
+    C0 = np.zeros((M, N), npdt)
+    dA, dB, dC = dev.array(A), dev.array(B), dev.array(C0)
+    L.check(L.lib.cnh_gemm_acc(dt, M, N, K, dA.ptr, K, dB.ptr, N, dC.ptr, N, None))
+    want = orc.gemm_acc(A, B, C0.copy())
+    if npdt == np.float32:
+        assert np.allclose(dC.get(), want, rtol=1e-5, atol=1e-5)
+    else:
+        assert np.array_equal(dC.get(), want)
+    dev.free_all()
+
+
+def test_stream_event_and_callback(dev):
+    s = C.c_void_p()
+    L.check(L.lib.cnh_stream_create(C.byref(s)))
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    L.check(L.lib.cnh_event_create(C.byref(e0)))
+    L.check(L.lib.cnh_event_create(C.byref(e1)))
+    d = dev.empty((1 << 20,), np.float64)
+    L.check(L.lib.cnh_event_record(e0, s))
+    L.check(L.lib.cnh_fill_uniform(d.ptr, 1 << 20, 1, 2, 0, 0.0, 1.0, s))
+    L.check(L.lib.cnh_event_record(e1, s))
+    hit = []
+    CB = C.CFUNCTYPE(None, C.c_void_p)
+    cb = CB(lambda _: hit.append(1))
+    L.check(L.lib.cnh_stream_callback(s, C.cast(cb, C.c_void_p), None))
+    L.check(L.lib.cnh_stream_sync(s))
+    ms = C.c_float()
+    L.check(L.lib.cnh_event_elapsed_ms(e0, e1, C.byref(ms)))
+    assert ms.value >= 0 and hit == [1]
+    L.check(L.lib.cnh_event_destroy(e0))
+    L.check(L.lib.cnh_event_destroy(e1))
+    L.check(L.lib.cnh_stream_destroy(s))
+    dev.free_all()

@@ -1,0 +1,120 @@
+"""GPU parity: shifted-slice groups over tiles resident on one device (stencils, slice copies)."""
+import numpy as np
+import pytest
+
+from charmnumeric_amd import _lib as L
+from charmnumeric_amd.astbuild import AstBuilder
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def _sweeps(dev, u0, tile, ast, nd, nsweeps, np_step):
+    k = H.compile_group(ast, L.F64, nd)
+    a = H.TiledArray(dev, u0, tile)
+    b = H.TiledArray(dev, np.zeros_like(u0), tile)
+    ref = u0.copy()
+    for _ in range(nsweeps):
+        H.launch_tiles(k, [a] * 2 * nd, [], a, b)
+        a, b = b, a
+        ref = np_step(ref)
+    dev.sync()
+    got = a.gather()
+    dev.free_all()
+    return got, ref
+
+
+@pytest.mark.parametrize("n,tile", [(64, 16), (70, 32), (33, 64)])
+def test_jacobi2d_tiles_bit_exact(dev, n, tile):
+    u0 = np.zeros((n, n))
+    u0[0, :] = 1.0
+    got, ref = _sweeps(dev, u0, tile, H.ast_jacobi2d(n), 2, 7, H.np_jacobi2d)
+    assert np.array_equal(got.view(np.int64), ref.view(np.int64))
+    # hot top row: after k sweeps only rows <= k are non-zero; row 1 interior after sweep 1 = 0.25
+    assert np.all(got[8:, :] == 0.0)
+    one = H.np_jacobi2d(u0)
+    assert np.all(one[1, 1:-1] == 0.25)
+
+
+@pytest.mark.parametrize("n,tile", [(32, 16), (20, 8)])
+def test_jacobi3d_tiles_bit_exact(dev, orc, n, tile):
+    u0 = orc.uniform(n ** 3, 1, 0, 0.0, 1.0).reshape(n, n, n)
+    u0[0], u0[-1], u0[:, 0], u0[:, -1], u0[:, :, 0], u0[:, :, -1] = 0, 0, 0, 0, 0, 0
+    got, ref = _sweeps(dev, u0, tile, H.ast_jacobi3d(n), 3, 4, H.np_jacobi3d)
+    assert np.array_equal(got.view(np.int64), ref.view(np.int64))
+
+
+def test_reference_jacobi3d_known_answer(dev):
+    """4^3 grid, faces 1.0: every interior point becomes (1/6)*3 = 0.5 (upstream test)."""
+    u0 = np.zeros((4, 4, 4))
+    u0[0], u0[-1], u0[:, 0], u0[:, -1], u0[:, :, 0], u0[:, :, -1] = 1, 1, 1, 1, 1, 1
+    got, _ = _sweeps(dev, u0, 2, H.ast_jacobi3d(4, coef=1.0 / 6.0), 3, 1,
+                     lambda u: H.np_jacobi3d(u, 1.0 / 6.0))
+    assert np.allclose(got[1:-1, 1:-1, 1:-1], 0.5, rtol=0, atol=1e-15)
+    assert np.all(got[0] == 1.0)
+
+
+def test_shifted_slice_sum_with_offset_decomposition(dev):
+    """src[100:300] + src[150:350] on arange(512): the result lives in a decomposition whose
+    offset (150) lines its tiles up with the second operand (upstream solver test vector)."""
+    src = np.arange(512, dtype=np.float64)
+    b = AstBuilder(L.F64, 1)
+    s = b.leaf(0)
+    b.binary(L.OP_ADD, 2, s, s, ((100,), (300,), (1,)), ((150,), (350,), (1,)), is_temp=False)
+    k = H.compile_group(b.finish(), L.F64, 1)
+    a = H.TiledArray(dev, src, 64)
+    out = H.TiledArray(dev, np.zeros(200), 64, offset=(150,))
+    H.launch_tiles(k, [a, a], [], None, out)
+    assert np.array_equal(out.gather(), src[100:300] + src[150:350])
+    dev.free_all()
+
+
+def test_strided_slice_assignment_between_arrays(dev):
+    """coarse[1:-1,1:-1] = fine[2:-2:2,2:-2:2] for n=17 (upstream integration test)."""
+    n, cn = 17, 9
+    fine = np.arange(n * n, dtype=np.float64).reshape(n, n)
+    coarse = np.full((cn, cn), -1.0)
+    b = AstBuilder(L.F64, 2)
+    tgt, src = b.leaf(0), b.leaf(1)
+    b.set_region(5, tgt, src, ((1, 1), (cn - 1, cn - 1), (1, 1)),
+                 rhs_region=((2, 2), (n - 2, n - 2), (2, 2)))
+    k = H.compile_group(b.finish(), L.F64, 2)
+    f = H.TiledArray(dev, fine, 8)
+    c = H.TiledArray(dev, coarse, 4)
+    H.launch_tiles(k, [f], [], c, c)  # in place: the target is not an input
+    want = coarse.copy()
+    want[1:-1, 1:-1] = fine[2:-2:2, 2:-2:2]
+    assert np.array_equal(c.gather(), want)
+    dev.free_all()
+
+
+def test_strided_target_region(dev):
+    """fine[2:-2:2] = 3*coarse[1:-1] leaves the odd points untouched."""
+    n, cn = 33, 17
+    fine = np.arange(n, dtype=np.float64)
+    coarse = np.arange(cn, dtype=np.float64) * 10
+    b = AstBuilder(L.F64, 1)
+    tgt, src = b.leaf(0), b.leaf(1)
+    t = b.binary(L.OP_MUL, 100, b.scalar(3.0), src, None, ((1,), (cn - 1,), (1,)))
+    b.set_region(5, tgt, t, ((2,), (n - 2,), (2,)))
+    k = H.compile_group(b.finish(), L.F64, 1)
+    f = H.TiledArray(dev, fine, 8)
+    f2 = H.TiledArray(dev, np.zeros(n), 8)
+    c = H.TiledArray(dev, coarse, 8)
+    H.launch_tiles(k, [c], [], f, f2)
+    want = fine.copy()
+    want[2:-2:2] = 3.0 * coarse[1:-1]
+    assert np.array_equal(f2.gather(), want)
+    dev.free_all()
+
+
+def test_tiles_rejects_bad_descriptors(dev):
+    n = 64
+    k = H.compile_group(H.ast_jacobi2d(n), L.F64, 2)
+    a = H.TiledArray(dev, np.zeros((n, n)), 16)
+    small = H.TiledArray(dev, np.zeros((32, 32)), 16)
+    with pytest.raises(L.CnhError):
+        H.launch_tiles(k, [small] * 4, [], a, a)      # input regions leave the 32x32 array
+    with pytest.raises(L.CnhError):
+        H.launch_tiles(k, [a] * 3, [], a, a)          # wrong number of inputs
+    dev.free_all()
