@@ -106,7 +106,7 @@ def cg_asts(L):
         return b.finish()
 
     def axpy(op):
-        # out = u (op) s * v
+        # out = u (op) s * v; leaf uses are collected root by root, so the memref order is (v, u)
         b = AstBuilder(L.F64, 1)
         u, v = b.leaf(1), b.leaf(2)
         t = b.binary(L.OP_MUL, 100, b.broadcast(3), v)
@@ -156,11 +156,11 @@ def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True):
             L.check(L.lib.cnh_event_record(ev.b[i], None))
         L.check(L.lib.cnh_dot_partial(L.F64, n, st["p"].ptr, Ap.ptr, S(1), None))
         _launch1(L, k_div, 1, [], [S(st["rtr"]), S(1)], [smr(2)])                       # alpha
-        _launch1(L, k_add, 1, [mr(st["x"]), mr(st["p"])], [S(2)], [mr(st["x2"])])      # x + alpha p
-        _launch1(L, k_sub, 1, [mr(st["r"]), mr(Ap)], [S(2)], [mr(st["r2"])])           # r - alpha Ap
+        _launch1(L, k_add, 1, [mr(st["p"]), mr(st["x"])], [S(2)], [mr(st["x2"])])      # x + alpha p
+        _launch1(L, k_sub, 1, [mr(Ap), mr(st["r"])], [S(2)], [mr(st["r2"])])           # r - alpha Ap
         L.check(L.lib.cnh_dot_partial(L.F64, n, st["r2"].ptr, st["r2"].ptr, S(st["rtr_new"]), None))
         _launch1(L, k_div, 1, [], [S(st["rtr_new"]), S(st["rtr"])], [smr(4)])           # beta
-        _launch1(L, k_add, 1, [mr(st["r2"]), mr(st["p"])], [S(4)], [mr(st["p2"])])     # r + beta p
+        _launch1(L, k_add, 1, [mr(st["p"]), mr(st["r2"])], [S(4)], [mr(st["p2"])])     # r + beta p
         st["x"], st["x2"] = st["x2"], st["x"]
         st["r"], st["r2"] = st["r2"], st["r"]
         st["p"], st["p2"] = st["p2"], st["p"]

@@ -177,6 +177,11 @@ _PROTOS = {
     "cnh_kernel_release": (C.c_int, [C.c_void_p]),
     "cnh_kernel_signature": (C.c_int, [C.c_void_p, C.POINTER(C.c_int), C.POINTER(C.c_int),
                                        C.POINTER(C.c_int)]),
+    "cnh_kernel_input": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int),
+                                   C.POINTER(Region)]),
+    "cnh_kernel_scalar": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_int)]),
+    "cnh_kernel_output": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int),
+                                    C.POINTER(C.c_int), C.POINTER(Region)]),
     "cnh_kernel_source": (C.c_int64, [C.c_void_p, C.c_char_p, C.c_char_p, C.c_size_t]),
     "cnh_kernel_build": (C.c_int, [C.c_void_p, C.c_char_p]),
     "cnh_launch_group": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.POINTER(Memref), C.c_int, _vpp,

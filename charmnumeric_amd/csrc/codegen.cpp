@@ -155,6 +155,7 @@ int build_group_program(const cnh_ast* ast, int dtype, int ndims, GroupProgram& 
                 if (!bcast_by_name.count(op.result_name)) {
                     bcast_by_name[op.result_name] = (int)p.bcast_nodes.size();
                     p.bcast_nodes.push_back(on);
+                    p.bcast_names.push_back(op.result_name);
                 }
                 Value v;
                 v.expr = fmt("s[%d]", bcast_by_name[op.result_name]);
@@ -270,6 +271,7 @@ int build_group_program(const cnh_ast* ast, int dtype, int ndims, GroupProgram& 
             return -15;
         }
         p.out_roots.push_back(r);
+        p.out_names.push_back(root.result_name);
         bool sr = root.opcode == CNH_OP_SET_REGION;
         p.out_is_set_region.push_back(sr ? 1 : 0);
         int target = root.result_name;

@@ -27,6 +27,8 @@ struct GroupProgram {
     std::vector<LeafUse> leaves;  // argument order: one memref per leaf use
     std::vector<int> load_leaf;   // distinct load -> the leaf use that supplies its memref
     std::vector<int> bcast_nodes; // one run-time scalar per unique broadcast leaf
+    std::vector<int> bcast_names; // array name of each broadcast leaf
+    std::vector<int> out_names;   // result name of each output root
     std::vector<int> out_roots;   // root positions of the non-temp roots
     std::vector<int> out_is_set_region;
     std::vector<int> out_target;  // SET_REGION target array name (or result name)

@@ -188,6 +188,42 @@ int cnh_kernel_signature(const cnh_kernel* k, int* n_in, int* n_scalar, int* n_o
     return 0;
 }
 
+int cnh_kernel_input(const cnh_kernel* k, int i, int* name, int* has_region, cnh_region* region) {
+    CNH_CHECK(k != nullptr, -2, "null kernel");
+    CNH_CHECK(i >= 0 && i < (int)k->prog.leaves.size(), -2, "input index %d out of range", i);
+    const LeafUse& u = k->prog.leaves[i];
+    if (name)
+        *name = u.name;
+    if (has_region)
+        *has_region = u.has_region ? 1 : 0;
+    if (region)
+        *region = u.region;
+    return 0;
+}
+
+int cnh_kernel_scalar(const cnh_kernel* k, int i, int* name) {
+    CNH_CHECK(k != nullptr, -2, "null kernel");
+    CNH_CHECK(i >= 0 && i < (int)k->prog.bcast_names.size(), -2, "scalar index %d out of range", i);
+    if (name)
+        *name = k->prog.bcast_names[i];
+    return 0;
+}
+
+int cnh_kernel_output(const cnh_kernel* k, int i, int* result_name, int* target_name,
+                      int* is_set_region, cnh_region* region) {
+    CNH_CHECK(k != nullptr, -2, "null kernel");
+    CNH_CHECK(i >= 0 && i < (int)k->prog.out_roots.size(), -2, "output index %d out of range", i);
+    if (result_name)
+        *result_name = k->prog.out_names[i];
+    if (target_name)
+        *target_name = k->prog.out_target[i];
+    if (is_set_region)
+        *is_set_region = k->prog.out_is_set_region[i];
+    if (region)
+        *region = k->prog.out_region[i];
+    return 0;
+}
+
 int64_t cnh_kernel_source(cnh_kernel* k, const char* variant, char* buf, size_t cap) {
     CNH_CHECK(k != nullptr && variant != nullptr, -2, "null argument");
     KernelVariant& v = k->variants[variant];

@@ -143,6 +143,14 @@ int cnh_kernel_release(cnh_kernel* k);
 /* Argument counts in the upstream order: memref per leaf use, scalar per unique broadcast leaf,
  * memref per non-temp root (src/jit.cpp:78-87). */
 int cnh_kernel_signature(const cnh_kernel* k, int* n_in, int* n_scalar, int* n_out);
+/* Which array each argument stands for, so a caller can bind buffers by name: input i is leaf
+ * use i (array name + the region attached to that use, has_region = 0 when it is the whole
+ * array); scalar i is the size-1 array `name`; output i is root `result_name`, which for a
+ * SET_REGION root assigns `region` of array `target_name`. */
+int cnh_kernel_input(const cnh_kernel* k, int i, int* name, int* has_region, cnh_region* region);
+int cnh_kernel_scalar(const cnh_kernel* k, int i, int* name);
+int cnh_kernel_output(const cnh_kernel* k, int i, int* result_name, int* target_name,
+                      int* is_set_region, cnh_region* region);
 /* Generated source of one variant ("flat", "nd", "tiles"), NUL-terminated; returns needed size. */
 int64_t cnh_kernel_source(cnh_kernel* k, const char* variant, char* buf, size_t cap);
 /* Builds the code object of one variant for gfx950 without loading it (works without a GPU). */
