@@ -327,6 +327,148 @@ def run_c1(L, n=1 << 24, parts=4, reps=20):
     return out
 
 
+# -------------------------------------------------------------------------------------------------
+# C3 / C4: Jacobi sweeps over tiles resident on the device
+# -------------------------------------------------------------------------------------------------
+def jacobi_ast(L, nd, n):
+    from charmnumeric_amd.astbuild import AstBuilder
+
+    b = AstBuilder(L.F64, nd)
+    u = b.leaf(0)
+
+    def reg(shift):
+        return (tuple(shift), tuple(s + n - 2 for s in shift), (1,) * nd)
+
+    shifts = []
+    for d in range(nd):
+        lo, hi = [1] * nd, [1] * nd
+        lo[d], hi[d] = 0, 2
+        shifts += [reg(lo), reg(hi)]
+    t = b.binary(L.OP_ADD, 100, u, u, shifts[0], shifts[1])
+    for i, r in enumerate(shifts[2:]):
+        t = b.binary(L.OP_ADD, 101 + i, t, u, None, r)
+    coef = 0.25 if nd == 2 else 0.16666666666666666
+    t = b.binary(L.OP_MUL, 120, b.scalar(coef), t)
+    b.set_region(121, u, t, reg([1] * nd))
+    return b.finish()
+
+
+class TiledDev:
+    """n^nd fp64 array in row-major tiles of edge `tile`, one device buffer per tile."""
+
+    def __init__(self, L, nd, n, tile):
+        self.L, self.nd, self.n, self.tile = L, nd, n, tile
+        self.g = (n + tile - 1) // tile
+        self.bufs = []
+        for idx in np.ndindex(*([self.g] * nd)):
+            ext = [min(tile, n - i * tile) for i in idx]
+            self.bufs.append((idx, ext, Buf(L, int(np.prod(ext)) * 8, zero=True)))
+        self.ptrs = (C.c_void_p * len(self.bufs))(*[C.c_void_p(b.ptr) for _, _, b in self.bufs])
+        d = L.Tiled()
+        d.ndims, d.tile = nd, tile
+        for i in range(nd):
+            d.offset[i], d.shape[i], d.grid_lo[i], d.grid[i] = 0, n, 0, self.g
+        d.tiles = C.cast(self.ptrs, C.POINTER(C.c_void_p))
+        self.desc = d
+
+    def free(self):
+        for _, _, b in self.bufs:
+            b.free()
+
+
+def run_jacobi(L, nd, n, tile, sweeps, reduce_every=10, reps_note=""):
+    a, b = TiledDev(L, nd, n, tile), TiledDev(L, nd, n, tile)
+    # initial state: 2-D hot top row; 3-D uniform[0,1) interior with zero faces
+    for (idx, ext, buf), (_, _, buf2) in zip(a.bufs, b.bufs):
+        if nd == 2:
+            if idx[0] == 0:
+                one = np.array([1.0]).view(np.uint8)
+                L.check(L.lib.cnh_fill_region(2, 8, buf.ptr, L.i64arr([ext[1], 1]), L.i64arr([0, 0]),
+                                              L.i64arr([1, 1]), L.i64arr([1, ext[1]]),
+                                              one.ctypes.data, None))
+    if nd == 3:
+        _fill_3d(L, a, n)
+    k = _compile(L, jacobi_ast(L, nd, n), L.F64, nd)
+    nleaf = 2 * nd
+    res = Buf(L, 8, zero=True)
+    ntile = len(a.bufs)
+    lens = L.i64arr([int(np.prod(e)) for _, e, _ in a.bufs])
+
+    def sweep(src, dst):
+        descs = (L.Tiled * nleaf)(*([src.desc] * nleaf))
+        L.check(L.lib.cnh_launch_group_tiles(k, nleaf, descs, 0, None, 0, C.byref(src.desc),
+                                             C.byref(dst.desc), None))
+
+    def residual(src, dst):
+        fn = L.lib.cnh_sumsq_diff_tiles if nd == 2 else L.lib.cnh_maxabs_diff_tiles
+        L.check(fn(ntile, dst.ptrs, src.ptrs, lens, res.ptr, None))
+
+    for _ in range(3):
+        sweep(a, b)
+        sweep(b, a)
+    L.check(L.lib.cnh_device_sync())
+    ev = Events(L, sweeps)
+    evr = Events(L, max(1, sweeps // reduce_every))
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    L.check(L.lib.cnh_event_create(C.byref(e0)))
+    L.check(L.lib.cnh_event_create(C.byref(e1)))
+    L.check(L.lib.cnh_event_record(e0, None))
+    cur, nxt = a, b
+    nres = 0
+    for i in range(sweeps):
+        L.check(L.lib.cnh_event_record(ev.a[i], None))
+        sweep(cur, nxt)
+        L.check(L.lib.cnh_event_record(ev.b[i], None))
+        if (i + 1) % reduce_every == 0:
+            L.check(L.lib.cnh_event_record(evr.a[nres], None))
+            residual(cur, nxt)
+            L.check(L.lib.cnh_event_record(evr.b[nres], None))
+            nres += 1
+        cur, nxt = nxt, cur
+    L.check(L.lib.cnh_event_record(e1, None))
+    L.check(L.lib.cnh_device_sync())
+    ms = C.c_float()
+    L.check(L.lib.cnh_event_elapsed_ms(e0, e1, C.byref(ms)))
+    t = ev.times_ms(sweeps)
+    tr = evr.times_ms(nres) if nres else [0.0]
+    us = 1e3 * float(np.median(t))
+    interior = (n - 2) ** nd
+    nbytes = 8.0 * ((n ** nd - (4 if nd == 2 else 0)) + interior) if nd == 2 else 8.0 * (n ** 3 + interior)
+    out = {"sweeps": sweeps, "us_per_sweep": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
+           "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+           "bytes_per_sweep": nbytes, "total_ms_with_reductions": round(ms.value, 3),
+           "reduction_us": round(1e3 * float(np.median(tr)), 2),
+           "last_reduction": float(res.get(np.float64)[0]), "partitions": ntile, "tile": tile}
+    ev.free()
+    evr.free()
+    a.free()
+    b.free()
+    res.free()
+    return out
+
+
+def _fill_3d(L, arr, n):
+    """Interior uniform[0,1) (seed 1, element index = row-major flat index), faces 0."""
+    t = arr.tile
+    for idx, ext, buf in arr.bufs:
+        L.check(L.lib.cnh_fill_uniform_tile(buf.ptr, 3, L.i64arr(ext), L.i64arr([i * t for i in idx]),
+                                            L.i64arr([n, n, n]), 1, 0, 0.0, 1.0, None))
+    # zero the six faces
+    zero = np.zeros(1).view(np.uint8)
+    for idx, ext, buf in arr.bufs:
+        st = L.i64arr([ext[1] * ext[2], ext[2], 1])
+        for d in range(3):
+            for side in (0, 1):
+                if (side == 0 and idx[d] != 0) or (side == 1 and idx[d] != arr.g - 1):
+                    continue
+                start = [0, 0, 0]
+                cnt = list(ext)
+                start[d] = 0 if side == 0 else ext[d] - 1
+                cnt[d] = 1
+                L.check(L.lib.cnh_fill_region(3, 8, buf.ptr, st, L.i64arr(start), L.i64arr([1, 1, 1]),
+                                              L.i64arr(cnt), zero.ctypes.data, None))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -343,6 +485,8 @@ def main():
         sys.exit(2)
 
     L = _dev()
+    if os.environ.get("CNH_BENCH_MARCH2D"):
+        L.check(L.lib.cnh_set_option(b"slide2d_march", 1))
     name = C.create_string_buffer(256)
     L.check(L.lib.cnh_device_name(name, 256))
     n = args.n
@@ -378,6 +522,14 @@ def main():
             also["c1_fused_elementwise_2p24"] = run_c1(L)
         except Exception as exc:  # report, do not hide
             also["c1_error"] = str(exc)
+        try:
+            also["c3_jacobi2d_8192"] = run_jacobi(L, 2, 8192, 2048, 200)
+        except Exception as exc:
+            also["c3_error"] = str(exc)
+        try:
+            also["c4_jacobi3d_512"] = run_jacobi(L, 3, 512, 128, 100)
+        except Exception as exc:
+            also["c4_error"] = str(exc)
         line["also"] = also
     if not args.no_cpu:
         cores = os.cpu_count() or 1

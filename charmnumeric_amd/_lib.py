@@ -150,6 +150,7 @@ _PROTOS = {
     "cnh_last_error": (C.c_char_p, []),
     "cnh_device_name": (C.c_int, [C.c_char_p, C.c_size_t]),
     "cnh_version": (C.c_int, []),
+    "cnh_set_option": (C.c_int, [C.c_char_p, C.c_int]),
     "cnh_alloc": (C.c_int, [C.c_size_t, C.c_int, _vpp]),
     "cnh_free": (C.c_int, [C.c_void_p]),
     "cnh_memset0": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p]),
@@ -207,6 +208,8 @@ _PROTOS = {
                                C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p]),
     "cnh_fill_uniform": (C.c_int, [C.c_void_p, C.c_int64, C.c_uint64, C.c_uint64, C.c_uint64,
                                    C.c_double, C.c_double, C.c_void_p]),
+    "cnh_fill_uniform_tile": (C.c_int, [C.c_void_p, C.c_int, _i64p, _i64p, _i64p, C.c_uint64,
+                                        C.c_uint64, C.c_double, C.c_double, C.c_void_p]),
     "cnh_fill_cg_matrix": (C.c_int, [C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int64,
                                      C.c_int64, C.c_int64, C.c_uint64, C.c_void_p]),
 }

@@ -333,79 +333,88 @@ std::string prelude(const GroupProgram& p) {
 
 std::string flat_source(const GroupProgram& p) {
     int vec = 16 / dtype_size(p.dtype);
-    int unr = 4;
     std::ostringstream s;
     s << prelude(p);
-    s << "#define VECW " << vec << "\n#define UNR " << unr << "\n";
+    s << "#define VECW " << vec << "\n";
     s << R"(
 // Contiguous segments: every memref of a partition is dense and has the same element count.
+// One 128-bit vector per lane and a grid that covers the data once: on this part the plain form
+// streams faster than unrolled or persistent ones. NT selects non-temporal loads and stores for
+// launches whose traffic exceeds what the last-level cache could keep anyway.
 struct Seg { i64 n; i64 blk0; const T* in[NLA]; T* out[NOA]; };
-template <int VEC> struct alignas(VEC * sizeof(T)) Pack { T x[VEC]; };
+typedef T TV __attribute__((ext_vector_type(VECW)));
 
-template <int VEC, int U>
-__device__ __forceinline__ void flat_run(const Seg& sg, i64 blk, const T* s) {
-    typedef Pack<VEC> P;
-    const i64 per_block = 256LL * VEC * U;
-    const i64 base = blk * per_block;
+template <bool NT>
+__device__ __forceinline__ void flat_vec(const Seg& sg, i64 blk, const T* s) {
+    const i64 i = (blk * 256 + threadIdx.x) * VECW;
     const i64 n = sg.n;
-    if (base + per_block <= n) {
-        P lv[NLA][U];
+    if (i + VECW <= n) {
+        TV lv[NLA];
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const i64 i = base + ((i64)u * 256 + threadIdx.x) * VEC;
+        for (int k = 0; k < NL; ++k) {
+            const TV* src = reinterpret_cast<const TV*>(sg.in[k] + i);
+            lv[k] = NT ? __builtin_nontemporal_load(src) : *src;
+        }
+        TV ov[NOA];
 #pragma unroll
-            for (int k = 0; k < NL; ++k) lv[k][u] = *reinterpret_cast<const P*>(sg.in[k] + i);
+        for (int e = 0; e < VECW; ++e) {
+            T l[NLA], o[NOA];
+#pragma unroll
+            for (int k = 0; k < NL; ++k) l[k] = lv[k][e];
+            group_eval(l, s, o);
+#pragma unroll
+            for (int j = 0; j < NO; ++j) ov[j][e] = o[j];
         }
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const i64 i = base + ((i64)u * 256 + threadIdx.x) * VEC;
-            P ov[NOA];
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) {
-                T l[NLA], o[NOA];
-#pragma unroll
-                for (int k = 0; k < NL; ++k) l[k] = lv[k][u].x[e];
-                group_eval(l, s, o);
-#pragma unroll
-                for (int j = 0; j < NO; ++j) ov[j].x[e] = o[j];
-            }
-#pragma unroll
-            for (int j = 0; j < NO; ++j) *reinterpret_cast<P*>(sg.out[j] + i) = ov[j];
+        for (int j = 0; j < NO; ++j) {
+            TV* dst = reinterpret_cast<TV*>(sg.out[j] + i);
+            if (NT) __builtin_nontemporal_store(ov[j], dst); else *dst = ov[j];
         }
     } else {
+        for (i64 x = i; x < n; ++x) {
+            T l[NLA], o[NOA];
 #pragma unroll
-        for (int u = 0; u < U * VEC; ++u) {
-            const i64 i = base + (i64)u * 256 + threadIdx.x;
-            if (i < n) {
-                T l[NLA], o[NOA];
+            for (int k = 0; k < NL; ++k) l[k] = sg.in[k][x];
+            group_eval(l, s, o);
 #pragma unroll
-                for (int k = 0; k < NL; ++k) l[k] = sg.in[k][i];
-                group_eval(l, s, o);
-#pragma unroll
-                for (int j = 0; j < NO; ++j) sg.out[j][i] = o[j];
-            }
+            for (int j = 0; j < NO; ++j) sg.out[j][x] = o[j];
         }
     }
 }
 
-extern "C" __global__ __launch_bounds__(256) void grp_flat_v(const Seg* segs, int nseg, Scal sc) {
-    T s[NSA]; load_scalars(sc, s);
-    const int k = find_seg(segs, nseg, (i64)blockIdx.x);
-    flat_run<VECW, UNR>(segs[k], (i64)blockIdx.x - segs[k].blk0, s);
+// Pointers that are not 16-byte aligned: one element per lane.
+__device__ __forceinline__ void flat_scalar(const Seg& sg, i64 blk, const T* s) {
+#pragma unroll
+    for (int u = 0; u < VECW; ++u) {
+        const i64 i = (blk * VECW + u) * 256 + threadIdx.x;
+        if (i < sg.n) {
+            T l[NLA], o[NOA];
+#pragma unroll
+            for (int k = 0; k < NL; ++k) l[k] = sg.in[k][i];
+            group_eval(l, s, o);
+#pragma unroll
+            for (int j = 0; j < NO; ++j) sg.out[j][i] = o[j];
+        }
+    }
 }
-extern "C" __global__ __launch_bounds__(256) void grp_flat_s(const Seg* segs, int nseg, Scal sc) {
-    T s[NSA]; load_scalars(sc, s);
-    const int k = find_seg(segs, nseg, (i64)blockIdx.x);
-    flat_run<1, UNR * VECW>(segs[k], (i64)blockIdx.x - segs[k].blk0, s);
+
+#define FLAT_ENTRY(NAME, CALL)                                                                   \
+extern "C" __global__ __launch_bounds__(256) void grp_flat_##NAME(const Seg* segs, int nseg,    \
+                                                                  Scal sc) {                     \
+    T s[NSA]; load_scalars(sc, s);                                                               \
+    const int k = find_seg(segs, nseg, (i64)blockIdx.x);                                         \
+    const Seg& sg = segs[k];                                                                     \
+    const i64 blk = (i64)blockIdx.x - sg.blk0;                                                   \
+    CALL;                                                                                        \
+}                                                                                                \
+extern "C" __global__ __launch_bounds__(256) void grp_flat1_##NAME(Seg sg, Scal sc) {           \
+    T s[NSA]; load_scalars(sc, s);                                                               \
+    const i64 blk = (i64)blockIdx.x;                                                             \
+    CALL;                                                                                        \
 }
-extern "C" __global__ __launch_bounds__(256) void grp_flat1_v(Seg seg, Scal sc) {
-    T s[NSA]; load_scalars(sc, s);
-    flat_run<VECW, UNR>(seg, (i64)blockIdx.x, s);
-}
-extern "C" __global__ __launch_bounds__(256) void grp_flat1_s(Seg seg, Scal sc) {
-    T s[NSA]; load_scalars(sc, s);
-    flat_run<1, UNR * VECW>(seg, (i64)blockIdx.x, s);
-}
+FLAT_ENTRY(v, flat_vec<false>(sg, blk, s))
+FLAT_ENTRY(vn, flat_vec<true>(sg, blk, s))
+FLAT_ENTRY(s, flat_scalar(sg, blk, s))
 )";
     return s.str();
 }
@@ -546,13 +555,46 @@ extern "C" __global__ __launch_bounds__(256) void grp_tiles(const Tiled* arrs, c
 
 } // namespace
 
-std::string slide_source(const GroupProgram& p, std::string& err); // codegen_slide.cpp
+std::string slide_source(const GroupProgram& p, const SlideConfig& cfg, std::string& err); // codegen_slide.cpp
+
+std::string direct_source(const GroupProgram& p, const DirectConfig& cfg, std::string& err); // codegen_direct.cpp
+
+std::string DirectConfig::variant() const {
+    char buf[64];
+    snprintf(buf, sizeof buf, "direct@%d,%d,%d", tx, ry, rz);
+    return buf;
+}
+
+bool DirectConfig::parse(const std::string& variant, DirectConfig& out) {
+    out = DirectConfig();
+    if (variant == "direct")
+        return true;
+    return sscanf(variant.c_str(), "direct@%d,%d,%d", &out.tx, &out.ry, &out.rz) == 3;
+}
+
+std::string SlideConfig::variant() const {
+    char buf[96];
+    snprintf(buf, sizeof buf, "slide@%d,%d,%d,%d,%d", march2d, bx, ry, zc, pd);
+    return buf;
+}
+
+bool SlideConfig::parse(const std::string& variant, SlideConfig& out) {
+    out = SlideConfig();
+    if (variant == "slide")
+        return true;
+    return sscanf(variant.c_str(), "slide@%d,%d,%d,%d,%d", &out.march2d, &out.bx, &out.ry, &out.zc,
+                  &out.pd) == 5;
+}
 
 int emit_variant_source(const GroupProgram& p, const std::string& variant, std::string& src,
                         std::string& err) {
     if (p.out_roots.empty()) {
         err = "group has no output root";
         return -16;
+    }
+    if (variant == "prelude") {
+        src = prelude(p);
+        return 0;
     }
     if (variant == "flat") {
         src = flat_source(p);
@@ -570,8 +612,22 @@ int emit_variant_source(const GroupProgram& p, const std::string& variant, std::
         src = tiles_source(p);
         return 0;
     }
-    if (variant == "slide") {
-        src = slide_source(p, err);
+    if (variant.compare(0, 6, "direct") == 0) {
+        DirectConfig cfg;
+        if (!DirectConfig::parse(variant, cfg)) {
+            err = "malformed register-window variant '" + variant + "'";
+            return -2;
+        }
+        src = direct_source(p, cfg, err);
+        return src.empty() ? -18 : 0;
+    }
+    if (variant.compare(0, 5, "slide") == 0) {
+        SlideConfig cfg;
+        if (!SlideConfig::parse(variant, cfg)) {
+            err = "malformed sliding-window variant '" + variant + "'";
+            return -2;
+        }
+        src = slide_source(p, cfg, err);
         return src.empty() ? -18 : 0;
     }
     err = "unknown kernel variant '" + variant + "'";

@@ -4,6 +4,7 @@
 // scalar leaves are constants cast to that type, size-1 arrays are run-time scalars.
 #pragma once
 
+#include <array>
 #include <string>
 #include <vector>
 
@@ -42,6 +43,43 @@ struct GroupProgram {
 // compile either (tanh/exp on integers, a unary op on a scalar, unknown opcodes).
 int build_group_program(const cnh_ast* ast, int dtype, int ndims, GroupProgram& out,
                         std::string& err);
+
+// Launch geometry of the sliding-window variant. Kernel dimensions are (march, row, column).
+// A rank-3 array maps to them one to one. A rank-2 array maps to (-, dim0, dim1) — one patch per
+// workgroup, nothing to march — or, with march2d, to (dim0, -, dim1): a row strip marched down.
+// Overrides of the built-in geometry (0 = keep the default); the variant name carries them.
+struct SlideConfig {
+    int march2d = 1, bx = 0, ry = 0, zc = 0, pd = 0;
+    std::string variant() const;                      // "slide" or "slide@m,bx,ry,zc,pd"
+    static bool parse(const std::string& variant, SlideConfig& out);
+};
+struct SlideShape {
+    bool march2d = false;
+    int halo[3] = {0, 0, 0};
+    int bx = 0, ty = 0, ry = 0, zc = 0, pd = 1;       // patch width, lane rows, rows per lane,
+                                                       // march chunk, planes in flight
+    std::vector<std::array<int, 3>> shifts; // per distinct load, in kernel dimensions
+    int kdim(int ndims, int d) const {
+        if (ndims == 3)
+            return d;
+        return march2d ? (d == 0 ? 0 : 2) : d + 1;
+    }
+};
+// 0 when the group is a same-array unit-step stencil the sliding-window variant can run.
+int slide_shape(const GroupProgram& p, const SlideConfig& cfg, SlideShape& sh, std::string& err);
+
+// Register-window stencil variant (no LDS): lane grid tx x (256/tx), ry rows and rz planes per lane.
+struct DirectConfig {
+    int tx = 0, ry = 0, rz = 0;                       // 0 = built-in default
+    std::string variant() const;                      // "direct" or "direct@tx,ry,rz"
+    static bool parse(const std::string& variant, DirectConfig& out);
+};
+struct DirectShape {
+    int halo[3] = {0, 0, 0};
+    int tx = 0, ty = 0, ry = 0, rz = 0;
+    std::vector<std::array<int, 3>> shifts; // per distinct load, dims padded to (z, y, x)
+};
+int direct_shape(const GroupProgram& p, const DirectConfig& cfg, DirectShape& sh, std::string& err);
 
 // Source text of a kernel variant. `variant` is one of "flat", "nd", "tiles", "slide".
 int emit_variant_source(const GroupProgram& p, const std::string& variant, std::string& src,

@@ -70,9 +70,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void gemv_rows(const ColTile* 
                                                                  T* __restrict__ y, int beta) {
     typedef typename Acc<T>::type A;
     constexpr int VEC = 16 / sizeof(T);
-    struct alignas(16) P {
-        T v[VEC];
-    };
+    typedef T P __attribute__((ext_vector_type(VEC)));
     const int lane = threadIdx.x & 63;
     const int64_t r = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
     if (r >= rows)
@@ -95,7 +93,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void gemv_rows(const ColTile* 
                 P av[kUnroll], xs[kUnroll];
 #pragma unroll
                 for (int u = 0; u < kUnroll; ++u)
-                    av[u] = *reinterpret_cast<const P*>(row + c + u * step + lane * VEC);
+                    av[u] = __builtin_nontemporal_load(reinterpret_cast<const P*>(row + c + u * step + lane * VEC));
 #pragma unroll
                 for (int u = 0; u < kUnroll; ++u)
                     xs[u] = *reinterpret_cast<const P*>(xv + c + u * step + lane * VEC);
@@ -103,14 +101,14 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void gemv_rows(const ColTile* 
                 for (int u = 0; u < kUnroll; ++u)
 #pragma unroll
                     for (int e = 0; e < VEC; ++e)
-                        acc[u] += (A)av[u].v[e] * (A)xs[u].v[e];
+                        acc[u] += (A)av[u][e] * (A)xs[u][e];
             }
             for (; c + step <= ct.ncols; c += step) {
                 P av = *reinterpret_cast<const P*>(row + c + lane * VEC);
                 P xs = *reinterpret_cast<const P*>(xv + c + lane * VEC);
 #pragma unroll
                 for (int e = 0; e < VEC; ++e)
-                    acc[0] += (A)av.v[e] * (A)xs.v[e];
+                    acc[0] += (A)av[e] * (A)xs[e];
             }
         }
         for (int64_t j = c + lane; j < ct.ncols; j += 64)

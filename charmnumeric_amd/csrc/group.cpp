@@ -272,7 +272,7 @@ int cnh_launch_group_batched(cnh_kernel* k, int ndims, int n_parts, int n_in, co
     const int NL = (int)p.load_leaf.size();
     const int NLA = NL > 0 ? NL : 1, NOA = n_out;
     const int esz = dtype_size(p.dtype);
-    const int vec = 16 / esz, unr = 4;
+    const int vec = 16 / esz;
 
     // Shapes must agree across all memrefs of a partition (identity indexing maps upstream).
     bool all_dense = true, all_aligned = true;
@@ -311,10 +311,10 @@ int cnh_launch_group_batched(cnh_kernel* k, int ndims, int n_parts, int n_in, co
     };
 
     if (all_dense) {
-        const int per_block = 256 * vec * unr;
+        const int per_block = 256 * vec;
         const size_t seg_words = 2 + NLA + NOA;
         std::vector<uint64_t> segs(seg_words * live.size(), 0);
-        int64_t blocks = 0;
+        int64_t blocks = 0, total = 0;
         for (size_t j = 0; j < live.size(); ++j) {
             int q = live[j];
             const cnh_memref* pi = in + (size_t)q * n_in;
@@ -330,16 +330,19 @@ int cnh_launch_group_batched(cnh_kernel* k, int ndims, int n_parts, int n_in, co
             for (int o = 0; o < n_out; ++o)
                 sg[2 + NLA + o] = base_ptr(po[o]);
             blocks += (n + per_block - 1) / per_block;
+            total += n;
         }
+        // Streams larger than the last-level cache bypass it; small operands (CG vectors) stay.
+        const bool nontemporal = total * (int64_t)(NL + n_out) * esz >= (128ll << 20);
+        const char* suffix = !all_aligned ? "s" : nontemporal ? "vn" : "v";
+        std::string name = std::string(live.size() == 1 ? "grp_flat1_" : "grp_flat_") + suffix;
         hipFunction_t fn;
+        if (int rc = get_function(k, "flat", name.c_str(), &fn))
+            return rc;
         if (live.size() == 1) {
-            if (int rc = get_function(k, "flat", all_aligned ? "grp_flat1_v" : "grp_flat1_s", &fn))
-                return rc;
             void* params[] = {segs.data(), scal.data()};
             return launch(fn, blocks, params, st);
         }
-        if (int rc = get_function(k, "flat", all_aligned ? "grp_flat_v" : "grp_flat_s", &fn))
-            return rc;
         const void* dsegs = nullptr;
         if (int rc = desc_upload(segs.data(), segs.size() * 8, st, &dsegs))
             return rc;
@@ -480,6 +483,244 @@ int make_tiled_dev(const cnh_tiled* t, hipStream_t st, TiledDev& d) {
 
 } // namespace
 
+namespace {
+
+struct SlideArgsDev {
+    const void* cur;
+    void* dst;
+    int32_t shift, shape[3], grid[3], rs[3], re[3], nbx, nby, nzc, nblocks;
+};
+static_assert(sizeof(SlideArgsDev) == 88, "SlideArgsDev layout must match the generated struct");
+
+bool g_slide_enabled = false;
+SlideConfig g_slide_cfg;
+bool slide_disabled() { return !g_slide_enabled; }
+
+// Launches the sliding-window variant when the group is a unit-step stencil on the assigned
+// array itself, the decomposition has no offset and the new contents go to a second buffer.
+int try_launch_slide(cnh_kernel* k, const std::vector<const cnh_tiled*>& arrays,
+                     const cnh_tiled* cur, const cnh_tiled* dst,
+                     const std::vector<unsigned char>& scal, hipStream_t st, bool* handled) {
+    *handled = false;
+    const GroupProgram& p = k->prog;
+    SlideShape sh;
+    std::string why;
+    if (slide_disabled() || slide_shape(p, g_slide_cfg, sh, why) != 0)
+        return 0;
+    if (!cur || arrays.size() != 1 || cur->tile < 2)
+        return 0;
+    const int nd = p.ndims;
+    int64_t ntiles = 1;
+    for (int d = 0; d < nd; ++d) {
+        if (cur->offset[d] != 0 || dst->offset[d] != 0 || arrays[0]->offset[d] != 0 ||
+            arrays[0]->shape[d] != cur->shape[d])
+            return 0;
+        ntiles *= cur->grid[d];
+    }
+    if (arrays[0]->tile != cur->tile || arrays[0]->tiles[0] != cur->tiles[0])
+        return 0;
+    {
+        int64_t vol = 1; // in-tile offsets are 32-bit in the kernel
+        for (int d = 0; d < nd; ++d)
+            vol *= std::min(cur->tile, cur->shape[d]);
+        if (vol >= (1ll << 31))
+            return 0;
+    }
+    for (int64_t t = 0; t < ntiles; ++t)
+        if (cur->tiles[t] == dst->tiles[t])
+            return 0; // in place: a sweep would read values it has already written
+
+    SlideArgsDev a;
+    std::memset(&a, 0, sizeof a);
+    a.shift = 0;
+    while ((1 << a.shift) < cur->tile)
+        a.shift++;
+    for (int d = 0; d < 3; ++d) {
+        a.shape[d] = 1;
+        a.grid[d] = 1;
+        a.rs[d] = 0;
+        a.re[d] = 1;
+    }
+    bool vec = (cur->tile % 2) == 0;
+    for (int d = 0; d < nd; ++d) {
+        const int kd = sh.kdim(nd, d);
+        a.shape[kd] = cur->shape[d];
+        a.grid[kd] = cur->grid[d];
+        a.rs[kd] = p.out_region[0].start[d];
+        a.re[kd] = p.out_region[0].stop[d];
+    }
+    if (a.shape[2] % 2 != 0)
+        vec = false;
+    for (int64_t t = 0; t < ntiles; ++t)
+        if (((uintptr_t)cur->tiles[t] & 15) || ((uintptr_t)dst->tiles[t] & 15))
+            vec = false;
+    a.nbx = (a.shape[2] + sh.bx - 1) / sh.bx;
+    a.nby = (a.shape[1] + sh.ty * sh.ry - 1) / (sh.ty * sh.ry);
+    a.nzc = (a.shape[0] + sh.zc - 1) / sh.zc;
+    const int64_t blocks = (int64_t)a.nbx * a.nby * a.nzc;
+    CNH_CHECK(blocks > 0 && blocks < (1ll << 31), -3, "stencil launch of %lld workgroups",
+              (long long)blocks);
+    a.nblocks = (int)blocks;
+    const void* dcur = nullptr;
+    const void* ddst = nullptr;
+    if (int rc = desc_upload(cur->tiles, (size_t)ntiles * sizeof(void*), st, &dcur))
+        return rc;
+    if (int rc = desc_upload(dst->tiles, (size_t)ntiles * sizeof(void*), st, &ddst))
+        return rc;
+    a.cur = dcur;
+    a.dst = const_cast<void*>(ddst);
+    hipFunction_t fn;
+    int64_t volume = 1;
+    for (int d = 0; d < nd; ++d)
+        volume *= cur->shape[d];
+    const bool nontemporal = volume * 16 >= (128ll << 20); // read + write stream past the cache
+    if (int rc = get_function(k, g_slide_cfg.variant(),
+                              !vec ? "grp_slide_s" : nontemporal ? "grp_slide_vn" : "grp_slide_v", &fn))
+        return rc;
+    void* params[] = {&a, const_cast<unsigned char*>(scal.data())};
+    if (int rc = launch(fn, blocks, params, st))
+        return rc;
+    *handled = true;
+    return 0;
+}
+
+struct DirectArgsDev {
+    const void* cur;
+    void* dst;
+    int32_t tile, shape[3], grid[3], rs[3], re[3], tb[3], nblocks;
+};
+static_assert(sizeof(DirectArgsDev) == 88, "DirectArgsDev layout must match the generated struct");
+
+int g_stencil_mode = 2; // 0 = general gather, 1 = LDS sliding window, 2 = register window
+DirectConfig g_direct_cfg;
+
+// Launches the register-window variant under the same conditions as the sliding window, plus:
+// every tile extent along the fastest dimension is even (128-bit accesses never straddle tiles).
+int try_launch_direct(cnh_kernel* k, const std::vector<const cnh_tiled*>& arrays,
+                      const cnh_tiled* cur, const cnh_tiled* dst,
+                      const std::vector<unsigned char>& scal, hipStream_t st, bool* handled) {
+    *handled = false;
+    const GroupProgram& p = k->prog;
+    DirectShape sh;
+    std::string why;
+    if (g_stencil_mode != 2 || direct_shape(p, g_direct_cfg, sh, why) != 0)
+        return 0;
+    if (!cur || arrays.size() != 1 || cur->tile < 2 || (cur->tile % 2) != 0)
+        return 0;
+    // a lane's own rows and planes must not straddle tiles: the tile edge (a power of two) has
+    // to be a multiple of what one lane owns
+    if (cur->tile % sh.ry != 0 || cur->tile % sh.rz != 0)
+        return 0;
+    const int nd = p.ndims, pad = CNH_MAX_ND - nd;
+    int64_t ntiles = 1, vol = 1, volume = 1;
+    for (int d = 0; d < nd; ++d) {
+        if (cur->offset[d] != 0 || dst->offset[d] != 0 || arrays[0]->offset[d] != 0 ||
+            arrays[0]->shape[d] != cur->shape[d])
+            return 0;
+        ntiles *= cur->grid[d];
+        vol *= std::min(cur->tile, cur->shape[d]);
+        volume *= cur->shape[d];
+    }
+    if (arrays[0]->tile != cur->tile || arrays[0]->tiles[0] != cur->tiles[0] || vol >= (1ll << 31))
+        return 0;
+    if (cur->shape[nd - 1] % 2 != 0)
+        return 0;
+    for (int64_t t = 0; t < ntiles; ++t) {
+        if (cur->tiles[t] == dst->tiles[t])
+            return 0; // in place: a sweep would read values it has already written
+        if (((uintptr_t)cur->tiles[t] & 15) || ((uintptr_t)dst->tiles[t] & 15))
+            return 0;
+    }
+    DirectArgsDev a;
+    std::memset(&a, 0, sizeof a);
+    a.tile = cur->tile;
+    for (int d = 0; d < 3; ++d) {
+        a.shape[d] = 1;
+        a.grid[d] = 1;
+        a.rs[d] = 0;
+        a.re[d] = 1;
+    }
+    for (int d = 0; d < nd; ++d) {
+        a.shape[pad + d] = cur->shape[d];
+        a.grid[pad + d] = cur->grid[d];
+        a.rs[pad + d] = p.out_region[0].start[d];
+        a.re[pad + d] = p.out_region[0].stop[d];
+    }
+    const int ext[3] = {sh.rz, sh.ty * sh.ry, sh.tx * 2};
+    int64_t per_tile = 1;
+    for (int d = 0; d < 3; ++d) {
+        const int edge = std::min(a.tile, a.shape[d]);
+        a.tb[d] = (edge + ext[d] - 1) / ext[d];
+        per_tile *= a.tb[d];
+    }
+    const int64_t blocks = per_tile * ntiles;
+    CNH_CHECK(blocks > 0 && blocks < (1ll << 31), -3, "stencil launch of %lld workgroups",
+              (long long)blocks);
+    a.nblocks = (int)blocks;
+    const void* dcur = nullptr;
+    const void* ddst = nullptr;
+    if (int rc = desc_upload(cur->tiles, (size_t)ntiles * sizeof(void*), st, &dcur))
+        return rc;
+    if (int rc = desc_upload(dst->tiles, (size_t)ntiles * sizeof(void*), st, &ddst))
+        return rc;
+    a.cur = dcur;
+    a.dst = const_cast<void*>(ddst);
+    const bool nt_stores = volume * 16 >= (128ll << 20); // the written stream is not read back soon
+    hipFunction_t fn;
+    if (int rc = get_function(k, g_direct_cfg.variant(), nt_stores ? "grp_direct_nts" : "grp_direct", &fn))
+        return rc;
+    void* params[] = {&a, const_cast<unsigned char*>(scal.data())};
+    if (int rc = launch(fn, blocks, params, st))
+        return rc;
+    *handled = true;
+    return 0;
+}
+
+} // namespace
+
+extern "C" int cnh_set_option(const char* name, int value) {
+    CNH_CHECK(name != nullptr, -2, "null option name");
+    if (std::strcmp(name, "stencil_mode") == 0) {
+        CNH_CHECK(value >= 0 && value <= 2, -2, "stencil_mode must be 0, 1 or 2");
+        g_stencil_mode = value;
+        g_slide_enabled = value == 1;
+        return 0;
+    }
+    if (std::strcmp(name, "direct_tx") == 0) {
+        g_direct_cfg.tx = value;
+        return 0;
+    }
+    if (std::strcmp(name, "direct_ry") == 0) {
+        g_direct_cfg.ry = value;
+        return 0;
+    }
+    if (std::strcmp(name, "direct_rz") == 0) {
+        g_direct_cfg.rz = value;
+        return 0;
+    }
+    if (std::strcmp(name, "slide2d_march") == 0) {
+        g_slide_cfg.march2d = value != 0;
+        return 0;
+    }
+    if (std::strcmp(name, "slide_bx") == 0) {
+        g_slide_cfg.bx = value;
+        return 0;
+    }
+    if (std::strcmp(name, "slide_ry") == 0) {
+        g_slide_cfg.ry = value;
+        return 0;
+    }
+    if (std::strcmp(name, "slide_zc") == 0) {
+        g_slide_cfg.zc = value;
+        return 0;
+    }
+    if (std::strcmp(name, "slide_pd") == 0) {
+        g_slide_cfg.pd = value;
+        return 0;
+    }
+    return set_error(-2, "unknown option '%s'", name);
+}
+
 extern "C" int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* in, int n_scalar,
                                       const void* const* scalars, int scalars_on_device,
                                       const cnh_tiled* cur, const cnh_tiled* dst, cnh_stream s) {
@@ -572,6 +813,19 @@ extern "C" int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* 
             lr[1 + pad + d] = start;
             lr[4 + pad + d] = step;
         }
+    }
+
+    // Same-array unit-step stencil with ping-pong buffers: register-window or LDS sliding window.
+    {
+        bool handled = false;
+        if (int rc = try_launch_direct(k, arrays, cur, dst, scal, st, &handled))
+            return rc;
+        if (handled)
+            return 0;
+        if (int rc = try_launch_slide(k, arrays, cur, dst, scal, st, &handled))
+            return rc;
+        if (handled)
+            return 0;
     }
 
     // Destination tiles.

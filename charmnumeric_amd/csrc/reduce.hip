@@ -25,7 +25,7 @@ struct Chunk {
 };
 
 constexpr int kThreads = 256;
-constexpr int kMaxBlocksPerChunk = 1024;
+constexpr int kMaxBlocksPerChunk = 65536;
 
 template <typename T>
 struct Acc {
@@ -110,38 +110,43 @@ __device__ __forceinline__ typename Acc<T>::type slice_reduce(const T* a, const 
                                                                int64_t hi) {
     typedef typename Acc<T>::type A;
     constexpr int VEC = 16 / sizeof(T);
-    struct alignas(16) P {
-        T x[VEC];
-    };
+    typedef T P __attribute__((ext_vector_type(VEC)));
+    constexpr int U = 4; // independent 128-bit loads in flight per operand
     A acc0 = 0, acc1 = 0;
     const bool two = MODE != M_SUM;
+    const bool same = !two || a == b;
     const bool aligned = (((uintptr_t)(a + lo)) & 15) == 0 &&
                          (!two || (((uintptr_t)(b + lo)) & 15) == 0);
     int64_t i = lo + (int64_t)threadIdx.x * VEC;
     if (aligned) {
         const int64_t stride = (int64_t)THREADS * VEC;
-        for (; i + stride + VEC <= hi; i += 2 * stride) {
-            P a0 = *reinterpret_cast<const P*>(a + i);
-            P a1 = *reinterpret_cast<const P*>(a + i + stride);
-            P b0 = a0, b1 = a1;
-            if (two) {
-                b0 = *reinterpret_cast<const P*>(b + i);
-                b1 = *reinterpret_cast<const P*>(b + i + stride);
-            }
+        for (; i + (U - 1) * stride + VEC <= hi; i += U * stride) {
+            P av[U], bv[U];
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) {
-                acc0 = combine<A, MODE>(acc0, term<T, A, MODE>(a0.x[e], b0.x[e]));
-                acc1 = combine<A, MODE>(acc1, term<T, A, MODE>(a1.x[e], b1.x[e]));
-            }
+            for (int u = 0; u < U; ++u)
+                av[u] = __builtin_nontemporal_load(reinterpret_cast<const P*>(a + i + u * stride));
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                bv[u] = same ? av[u]
+                             : __builtin_nontemporal_load(reinterpret_cast<const P*>(b + i + u * stride));
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    if (u & 1)
+                        acc1 = combine<A, MODE>(acc1, term<T, A, MODE>(av[u][e], bv[u][e]));
+                    else
+                        acc0 = combine<A, MODE>(acc0, term<T, A, MODE>(av[u][e], bv[u][e]));
+                }
         }
         for (; i + VEC <= hi; i += stride) {
             P a0 = *reinterpret_cast<const P*>(a + i);
             P b0 = a0;
-            if (two)
+            if (!same)
                 b0 = *reinterpret_cast<const P*>(b + i);
 #pragma unroll
             for (int e = 0; e < VEC; ++e)
-                acc0 = combine<A, MODE>(acc0, term<T, A, MODE>(a0.x[e], b0.x[e]));
+                acc0 = combine<A, MODE>(acc0, term<T, A, MODE>(a0[e], b0[e]));
         }
         // ragged end of the slice: fewer than VEC elements
         if (i < hi) {

@@ -57,9 +57,66 @@ __global__ __launch_bounds__(256) void fill_cg_kernel(double* __restrict__ out, 
     out[i * ld + j] = v;
 }
 
+struct TileFill {
+    int64_t ext[3], origin[3], gshape[3];
+};
+
+// One tile of a row-major global array: the counter of an element is its global flat index.
+__global__ __launch_bounds__(256) void fill_tile_kernel(double* __restrict__ out, TileFill t,
+                                                        unsigned long long seed,
+                                                        unsigned long long stream, double lo,
+                                                        double w) {
+    const int64_t total = t.ext[0] * t.ext[1] * t.ext[2];
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    for (; i < total; i += stride) {
+        const int64_t l2 = i % t.ext[2];
+        const int64_t l1 = (i / t.ext[2]) % t.ext[1];
+        const int64_t l0 = i / (t.ext[2] * t.ext[1]);
+        const int64_t g = ((t.origin[0] + l0) * t.gshape[1] + (t.origin[1] + l1)) * t.gshape[2] +
+                          (t.origin[2] + l2);
+        double prod = __dmul_rn(w, u01(seed, stream, (unsigned long long)g));
+        out[i] = __dadd_rn(lo, prod);
+    }
+}
+
 } // namespace
 
 extern "C" {
+
+int cnh_fill_uniform_tile(double* out, int ndims, const int64_t* ext, const int64_t* origin,
+                          const int64_t* global_shape, uint64_t seed, uint64_t stream_id, double lo,
+                          double hi, cnh_stream s) {
+    if (int rc = ensure_init())
+        return rc;
+    CNH_CHECK(ndims >= 1 && ndims <= CNH_MAX_ND, -2, "cnh_fill_uniform_tile: ndims %d", ndims);
+    CNH_CHECK(out && ext && origin && global_shape, -2, "cnh_fill_uniform_tile: null pointer");
+    TileFill t;
+    const int pad = CNH_MAX_ND - ndims;
+    for (int d = 0; d < 3; ++d) {
+        t.ext[d] = 1;
+        t.origin[d] = 0;
+        t.gshape[d] = 1;
+    }
+    int64_t total = 1;
+    for (int d = 0; d < ndims; ++d) {
+        CNH_CHECK(ext[d] >= 0 && origin[d] >= 0 && origin[d] + ext[d] <= global_shape[d], -2,
+                  "cnh_fill_uniform_tile: tile leaves the array in dim %d", d);
+        t.ext[pad + d] = ext[d];
+        t.origin[pad + d] = origin[d];
+        t.gshape[pad + d] = global_shape[d];
+        total *= ext[d];
+    }
+    if (total == 0)
+        return 0;
+    int64_t want = (total + 255) / 256;
+    unsigned blocks = (unsigned)(want > 65536 ? 65536 : want);
+    hipLaunchKernelGGL(fill_tile_kernel, dim3(blocks), dim3(256), 0, as_stream(s), out, t,
+                       (unsigned long long)seed, (unsigned long long)stream_id, lo, hi - lo);
+    CNH_HIP(hipGetLastError());
+    return 0;
+}
+
 
 int cnh_fill_uniform(double* out, int64_t n, uint64_t seed, uint64_t stream_id, uint64_t first,
                      double lo, double hi, cnh_stream s) {

@@ -88,6 +88,10 @@ int cnh_init(int device);               /* selects the device; idempotent */
 const char* cnh_last_error(void);
 int cnh_device_name(char* buf, size_t cap);
 int cnh_version(void);
+/* Tuning switches. "stencil_mode" picks the kernel cnh_launch_group_tiles uses for same-array
+ * unit-step stencils: 2 (default) register window, 1 LDS sliding window, 0 general gather.
+ * "direct_tx/ry/rz" and "slide_bx/ry/zc/pd", "slide2d_march" override the kernel geometry. */
+int cnh_set_option(const char* name, int value);
 
 /* ---- storage: Array<N,T> ctor zero-fill / data_ptr / copyToHost / copyToDevice / dtor
  *      (src/backend.hpp:112-200) ---- */
@@ -236,6 +240,11 @@ int cnh_gemm_acc(int dtype, int64_t M, int64_t N, int64_t K, const void* A, int6
 /* out[k] = lo + (hi-lo)*u01(seed, stream_id, first+k); counter-based SplitMix64, fp64. */
 int cnh_fill_uniform(double* out, int64_t n, uint64_t seed, uint64_t stream_id, uint64_t first,
                      double lo, double hi, cnh_stream s);
+/* One tile of a row-major global array: the counter of an element is its global flat index, so
+ * the tiles of an array together hold exactly what one global fill would produce. */
+int cnh_fill_uniform_tile(double* out, int ndims, const int64_t* ext, const int64_t* origin,
+                          const int64_t* global_shape, uint64_t seed, uint64_t stream_id, double lo,
+                          double hi, cnh_stream s);
 /* Block of the dense CG test matrix of order n (symmetric, diagonal 2.0). */
 int cnh_fill_cg_matrix(double* out, int64_t n, int64_t row0, int64_t nrows, int64_t col0,
                        int64_t ncols, int64_t ld, uint64_t seed, cnh_stream s);

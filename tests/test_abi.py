@@ -41,11 +41,11 @@ def test_scalar_conversion():
     assert buf.view(np.float32)[0] == np.float32(0.1)
 
 
-@pytest.mark.parametrize("variant", ["flat", "nd", "tiles"])
+@pytest.mark.parametrize("variant", ["flat", "nd", "tiles", "slide", "direct"])
 def test_generated_source_builds_for_gfx950(variant):
     """hipRTC cross-compiles the generated source without a GPU."""
-    ast = H.ast_jacobi2d(64) if variant == "tiles" else H.ast_c1(L.F64)
-    nd = 2 if variant == "tiles" else 1
+    ast = H.ast_jacobi2d(64) if variant in ("tiles", "slide", "direct") else H.ast_c1(L.F64)
+    nd = 2 if variant in ("tiles", "slide", "direct") else 1
     k = H.compile_group(ast, L.F64, nd)
     src = H.kernel_source(k, variant)
     assert "group_eval" in src and "fma" not in src
@@ -93,3 +93,13 @@ def test_uncompilable_groups_report_an_error():
     n = b._new(5, L.OP_MATMUL)
     b._roots.append(n)
     assert L.lib.cnh_compile_group(C.byref(b.finish()), L.F64, 1, 0, C.byref(k)) < 0
+
+
+def test_slide_variant_builds_for_3d_and_is_refused_for_other_groups():
+    k = H.compile_group(H.ast_jacobi3d(32), L.F64, 3)
+    L.check(L.lib.cnh_kernel_build(k, b"slide"))
+    L.check(L.lib.cnh_kernel_build(k, b"direct"))
+    src = H.kernel_source(k, "slide")
+    assert "SL_SHIFT[NLA][3] = {{-1, 0, 0}, {1, 0, 0}, {0, -1, 0}, {0, 1, 0}, {0, 0, -1}, {0, 0, 1}}" in src
+    k1 = H.compile_group(H.ast_c1(L.F64), L.F64, 1)
+    assert L.lib.cnh_kernel_build(k1, b"slide") < 0

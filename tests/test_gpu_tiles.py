@@ -9,6 +9,18 @@ from tests import helpers as H
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(params=["direct", "slide", "slide-march2d", "gather"])
+def stencil_path(request):
+    """Run the stencil tests through the register-window kernel, the LDS sliding-window kernel
+    (both rank-2 mappings) and the general gather kernel."""
+    mode = {"gather": 0, "slide": 1, "slide-march2d": 1, "direct": 2}[request.param]
+    L.check(L.lib.cnh_set_option(b"stencil_mode", mode))
+    L.check(L.lib.cnh_set_option(b"slide2d_march", 1 if request.param == "slide-march2d" else 0))
+    yield request.param
+    L.check(L.lib.cnh_set_option(b"stencil_mode", 2))
+    L.check(L.lib.cnh_set_option(b"slide2d_march", 1))
+
+
 def _sweeps(dev, u0, tile, ast, nd, nsweeps, np_step):
     k = H.compile_group(ast, L.F64, nd)
     a = H.TiledArray(dev, u0, tile)
@@ -24,8 +36,8 @@ def _sweeps(dev, u0, tile, ast, nd, nsweeps, np_step):
     return got, ref
 
 
-@pytest.mark.parametrize("n,tile", [(64, 16), (70, 32), (33, 64)])
-def test_jacobi2d_tiles_bit_exact(dev, n, tile):
+@pytest.mark.parametrize("n,tile", [(64, 16), (70, 32), (33, 64), (1030, 256), (300, 4)])
+def test_jacobi2d_tiles_bit_exact(dev, stencil_path, n, tile):
     u0 = np.zeros((n, n))
     u0[0, :] = 1.0
     got, ref = _sweeps(dev, u0, tile, H.ast_jacobi2d(n), 2, 7, H.np_jacobi2d)
@@ -36,15 +48,15 @@ def test_jacobi2d_tiles_bit_exact(dev, n, tile):
     assert np.all(one[1, 1:-1] == 0.25)
 
 
-@pytest.mark.parametrize("n,tile", [(32, 16), (20, 8)])
-def test_jacobi3d_tiles_bit_exact(dev, orc, n, tile):
+@pytest.mark.parametrize("n,tile", [(32, 16), (20, 8), (70, 32), (37, 16)])
+def test_jacobi3d_tiles_bit_exact(dev, orc, stencil_path, n, tile):
     u0 = orc.uniform(n ** 3, 1, 0, 0.0, 1.0).reshape(n, n, n)
     u0[0], u0[-1], u0[:, 0], u0[:, -1], u0[:, :, 0], u0[:, :, -1] = 0, 0, 0, 0, 0, 0
     got, ref = _sweeps(dev, u0, tile, H.ast_jacobi3d(n), 3, 4, H.np_jacobi3d)
     assert np.array_equal(got.view(np.int64), ref.view(np.int64))
 
 
-def test_reference_jacobi3d_known_answer(dev):
+def test_reference_jacobi3d_known_answer(dev, stencil_path):
     """4^3 grid, faces 1.0: every interior point becomes (1/6)*3 = 0.5 (upstream test)."""
     u0 = np.zeros((4, 4, 4))
     u0[0], u0[-1], u0[:, 0], u0[:, -1], u0[:, :, 0], u0[:, :, -1] = 1, 1, 1, 1, 1, 1
