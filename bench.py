@@ -469,6 +469,138 @@ def _fill_3d(L, arr, n):
                                               L.i64arr(cnt), zero.ctypes.data, None))
 
 
+# -------------------------------------------------------------------------------------------------
+# C5: LSTM forward (gate matmatmul on the fp64 matrix cores + fused gate groups)
+# -------------------------------------------------------------------------------------------------
+def lstm_asts(L, d):
+    """The per-step statements of examples/lstm_forward.py:40-49 as SET_REGION groups on 2-D views
+    (batch x columns) of the step's slice."""
+    from charmnumeric_amd.astbuild import AstBuilder
+
+    def sigmoid():        # IFOGf[:, :3d] = 1.0 / (1.0 + exp(IFOG[:, :3d] * -1))
+        b = AstBuilder(L.F64, 2)
+        x = b.leaf(1)
+        t0 = b.binary(L.OP_MUL, 100, x, b.scalar(-1))
+        t1 = b.unary(L.OP_EXP, 101, t0)
+        t2 = b.binary(L.OP_ADD, 102, b.scalar(1.0), t1)
+        b.binary(L.OP_DIV, 2, b.scalar(1.0), t2, is_temp=False)
+        return b.finish()
+
+    def tanh():           # out = tanh(in)
+        b = AstBuilder(L.F64, 2)
+        b.unary(L.OP_TANH, 2, b.leaf(1), is_temp=False)
+        return b.finish()
+
+    def mul():            # out = a * b
+        b = AstBuilder(L.F64, 2)
+        b.binary(L.OP_MUL, 3, b.leaf(1), b.leaf(2), is_temp=False)
+        return b.finish()
+
+    def muladd():         # out = c + f * cprev   (C[t] += f * C[t-1])
+        b = AstBuilder(L.F64, 2)
+        t = b.binary(L.OP_MUL, 100, b.leaf(2), b.leaf(3))
+        b.binary(L.OP_ADD, 4, b.leaf(1), t, is_temp=False)
+        return b.finish()
+
+    return sigmoid(), tanh(), mul(), muladd()
+
+
+def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=False):
+    k_in = nin + d
+    X = Buf(L, steps * batch * nin * 8)
+    W = Buf(L, k_in * 4 * d * 8)
+    L.check(L.lib.cnh_fill_uniform(X.ptr, steps * batch * nin, seed, 0, 0, -1.0, 1.0, None))
+    # W = [W_ih^T ; W_hh^T] (k_in x 4d): streams 1 and 2 hold W_ih, W_hh as (4d x nin), (4d x d);
+    # the transpose is laid out directly by generating row r of W from column r of the stream.
+    bound = 1.0 / 32.0
+    Wih = Buf(L, 4 * d * nin * 8)
+    Whh = Buf(L, 4 * d * d * 8)
+    L.check(L.lib.cnh_fill_uniform(Wih.ptr, 4 * d * nin, seed, 1, 0, -bound, bound, None))
+    L.check(L.lib.cnh_fill_uniform(Whh.ptr, 4 * d * d, seed, 2, 0, -bound, bound, None))
+    i64 = L.i64arr
+    one = i64([1, 1])
+    zero2 = i64([0, 0])
+    # W[r, c] = Wih[c, r] for r < nin: a strided copy with swapped strides
+    L.check(L.lib.cnh_copy_region(2, 8, W.ptr, i64([4 * d, 1]), zero2, one, Wih.ptr, i64([1, nin]),
+                                  zero2, one, i64([nin, 4 * d]), None))
+    L.check(L.lib.cnh_copy_region(2, 8, W.ptr + nin * 4 * d * 8, i64([4 * d, 1]), zero2, one, Whh.ptr,
+                                  i64([1, d]), zero2, one, i64([d, 4 * d]), None))
+    Wih.free()
+    Whh.free()
+    Hin = Buf(L, steps * batch * k_in * 8, zero=True)
+    IFOG = Buf(L, steps * batch * 4 * d * 8, zero=True)
+    IFOGf = Buf(L, steps * batch * 4 * d * 8, zero=True)
+    Cc = Buf(L, steps * batch * d * 8, zero=True)
+    Ct = Buf(L, steps * batch * d * 8, zero=True)
+    Hout = Buf(L, steps * batch * d * 8, zero=True)
+    a_sig, a_tanh, a_mul, a_muladd = lstm_asts(L, d)
+    k_sig, k_tanh, k_mul, k_muladd = (_compile(L, a, L.F64, 2) for a in (a_sig, a_tanh, a_mul, a_muladd))
+
+    def view(buf, t, row_len, c0, ncols):
+        base = buf.ptr + (t * batch * row_len + c0) * 8
+        return L.Memref.strided(base, (batch, ncols), (row_len, 1))
+
+    ev = Events(L, steps)
+    evs = Events(L, steps)
+
+    def step(t, record):
+        if record:
+            L.check(L.lib.cnh_event_record(evs.a[t], None))
+        # Hin[t, :, :nin] = X[t]; Hin[t, :, nin:] = Hout[t-1] (h0 = 0 at t = 0)
+        L.check(L.lib.cnh_copy_region(2, 8, Hin.ptr + t * batch * k_in * 8, i64([k_in, 1]), zero2, one,
+                                      X.ptr + t * batch * nin * 8, i64([nin, 1]), zero2, one,
+                                      i64([batch, nin]), None))
+        if t > 0:
+            L.check(L.lib.cnh_copy_region(2, 8, Hin.ptr + (t * batch * k_in + nin) * 8, i64([k_in, 1]),
+                                          zero2, one, Hout.ptr + (t - 1) * batch * d * 8, i64([d, 1]),
+                                          zero2, one, i64([batch, d]), None))
+        if record:
+            L.check(L.lib.cnh_event_record(ev.a[t], None))
+        L.check(L.lib.cnh_gemm_acc(L.F64, batch, 4 * d, k_in, Hin.ptr + t * batch * k_in * 8, k_in,
+                                   W.ptr, 4 * d, IFOG.ptr + t * batch * 4 * d * 8, 4 * d, None))
+        if record:
+            L.check(L.lib.cnh_event_record(ev.b[t], None))
+        _launch1(L, k_sig, 2, [view(IFOG, t, 4 * d, 0, 3 * d)], [], [view(IFOGf, t, 4 * d, 0, 3 * d)])
+        _launch1(L, k_tanh, 2, [view(IFOG, t, 4 * d, 3 * d, d)], [], [view(IFOGf, t, 4 * d, 3 * d, d)])
+        _launch1(L, k_mul, 2, [view(IFOGf, t, 4 * d, 0, d), view(IFOGf, t, 4 * d, 3 * d, d)], [],
+                 [view(Cc, t, d, 0, d)])
+        if t > 0:
+            # leaf uses are collected root by root: (f, C[t-1]) of the product, then C[t]
+            _launch1(L, k_muladd, 2, [view(IFOGf, t, 4 * d, d, d), view(Cc, t - 1, d, 0, d),
+                                      view(Cc, t, d, 0, d)], [], [view(Cc, t, d, 0, d)])
+        _launch1(L, k_tanh, 2, [view(Cc, t, d, 0, d)], [], [view(Ct, t, d, 0, d)])
+        _launch1(L, k_mul, 2, [view(IFOGf, t, 4 * d, 2 * d, d), view(Ct, t, d, 0, d)], [],
+                 [view(Hout, t, d, 0, d)])
+        if record:
+            L.check(L.lib.cnh_event_record(evs.b[t], None))
+
+    out = {}
+    if timed:
+        for t in range(min(steps, 3)):   # warm-up (builds the kernels); IFOG must start from zero again
+            step(t, False)
+        L.check(L.lib.cnh_memset0(IFOG.ptr, IFOG.nbytes, None))
+        L.check(L.lib.cnh_device_sync())
+    for t in range(steps):
+        step(t, True)
+    L.check(L.lib.cnh_device_sync())
+    g = ev.times_ms(steps)
+    st = evs.times_ms(steps)
+    flop = 2.0 * batch * k_in * 4 * d
+    gus = 1e3 * float(np.median(g))
+    out = {"steps": steps, "gemm_us": round(gus, 2), "gemm_tflops": round(flop / gus / 1e6, 2),
+           "mfma_frac": round(flop / gus / 1e6 / FP64_MFMA_PEAK_TFLOPS, 4),
+           "step_us": round(1e3 * float(np.median(st)), 2), "flop_per_step": flop}
+    if keep:
+        out["Hout"] = Hout.get().reshape(steps, batch, d)
+        out["C"] = Cc.get().reshape(steps, batch, d)
+        out["IFOG"] = IFOG.get().reshape(steps, batch, 4 * d)
+    ev.free()
+    evs.free()
+    for b_ in (X, W, Hin, IFOG, IFOGf, Cc, Ct, Hout):
+        b_.free()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -530,6 +662,10 @@ def main():
             also["c4_jacobi3d_512"] = run_jacobi(L, 3, 512, 128, 100)
         except Exception as exc:
             also["c4_error"] = str(exc)
+        try:
+            also["c5_lstm_forward"] = run_lstm(L)
+        except Exception as exc:
+            also["c5_error"] = str(exc)
         line["also"] = also
     if not args.no_cpu:
         cores = os.cpu_count() or 1

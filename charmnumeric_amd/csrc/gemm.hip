@@ -11,8 +11,9 @@ using namespace cnh;
 namespace {
 
 typedef double v4d __attribute__((ext_vector_type(4)));
+typedef double v2d __attribute__((ext_vector_type(2)));
 
-constexpr int BM = 64, BN = 64, BK = 16, PAD = 16;
+constexpr int BK = 16, PAD = 16;
 
 // Workgroup ids are dealt round-robin to the 8 XCDs; give every XCD a contiguous run of logical
 // tiles so that the workgroups sharing a B column panel also share one L2.
@@ -22,11 +23,18 @@ __device__ __forceinline__ int xcd_remap(int b, int nblocks) {
     return (b % 8) * (nblocks / 8) + b / 8;
 }
 
-template <bool FULL>
-__global__ __launch_bounds__(256) void gemm_f64_mfma(int M, int N, int K,
-                                                     const double* __restrict__ A, int64_t lda,
-                                                     const double* __restrict__ B, int64_t ldb,
-                                                     double* __restrict__ C, int64_t ldc) {
+// WM x WN wavefronts per workgroup, each owning TM x TN tiles of 16x16. The fp64 matrix pipe
+// needs two or more wavefronts per SIMD to stay busy (one wavefront issues at ~70% of the rate
+// eight reach), hence the 8-wavefront shape for grids that give each CU a single workgroup.
+template <int WM, int WN, int TM, int TN, bool FULL>
+__global__ __launch_bounds__(WM * WN * 64) void gemm_f64_mfma(int M, int N, int K,
+                                                              const double* __restrict__ A, int64_t lda,
+                                                              const double* __restrict__ B, int64_t ldb,
+                                                              double* __restrict__ C, int64_t ldc) {
+    constexpr int NT = WM * WN * 64;
+    constexpr int BM = WM * TM * 16, BN = WN * TN * 16;
+    constexpr int APT = BM * BK / NT, BPT = BN * BK / NT;   // doubles staged per lane
+    static_assert(APT >= 2 && BPT >= 2 && APT % 2 == 0 && BPT % 2 == 0, "staging uses 128-bit loads");
     __shared__ double As[2][BK][BM + PAD];
     __shared__ double Bs[2][BK][BN + PAD];
     const int nbm = (M + BM - 1) / BM, nbn = (N + BN - 1) / BN;
@@ -34,51 +42,57 @@ __global__ __launch_bounds__(256) void gemm_f64_mfma(int M, int N, int K,
     const int bn = logical / nbm, bm = logical - bn * nbm;
     const int m0 = bm * BM, n0 = bn * BN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WN, wn = wave % WN;
 
-    // staging assignment: A tile 64 rows x 16 k, B tile 16 k x 64 n; 4 doubles per lane each
-    const int a_row = tid >> 2, a_k = (tid & 3) * 4;
-    const int b_k = tid >> 4, b_n = (tid & 15) * 4;
+    // staging assignment: A tile BM rows x 16 k (APT along k), B tile 16 k x BN (BPT along n)
+    const int a_row = tid / (BK / APT), a_k = (tid % (BK / APT)) * APT;
+    const int b_k = tid / (BN / BPT), b_n = (tid % (BN / BPT)) * BPT;
 
-    double ra[4], rb[4];
+    double ra[APT], rb[BPT];
     auto fetch = [&](int k0) {
         const int gr = m0 + a_row;
         const int gk = k0 + a_k;
         if (FULL) {
-            const double2 v0 = *reinterpret_cast<const double2*>(A + (int64_t)gr * lda + gk);
-            const double2 v1 = *reinterpret_cast<const double2*>(A + (int64_t)gr * lda + gk + 2);
-            ra[0] = v0.x; ra[1] = v0.y; ra[2] = v1.x; ra[3] = v1.y;
+#pragma unroll
+            for (int j = 0; j < APT; j += 2) {
+                const v2d v = *reinterpret_cast<const v2d*>(A + (int64_t)gr * lda + gk + j);
+                ra[j] = v[0];
+                ra[j + 1] = v[1];
+            }
         } else {
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < APT; ++j)
                 ra[j] = (gr < M && gk + j < K) ? A[(int64_t)gr * lda + gk + j] : 0.0;
         }
         const int bk = k0 + b_k;
         const int gn = n0 + b_n;
         if (FULL) {
-            const double2 v0 = *reinterpret_cast<const double2*>(B + (int64_t)bk * ldb + gn);
-            const double2 v1 = *reinterpret_cast<const double2*>(B + (int64_t)bk * ldb + gn + 2);
-            rb[0] = v0.x; rb[1] = v0.y; rb[2] = v1.x; rb[3] = v1.y;
+#pragma unroll
+            for (int j = 0; j < BPT; j += 2) {
+                const v2d v = *reinterpret_cast<const v2d*>(B + (int64_t)bk * ldb + gn + j);
+                rb[j] = v[0];
+                rb[j + 1] = v[1];
+            }
         } else {
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < BPT; ++j)
                 rb[j] = (bk < K && gn + j < N) ? B[(int64_t)bk * ldb + gn + j] : 0.0;
         }
     };
     auto stage = [&](int buf) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < APT; ++j)
             As[buf][a_k + j][a_row] = ra[j];
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < BPT; ++j)
             Bs[buf][b_k][b_n + j] = rb[j];
     };
 
-    v4d acc[2][2];
+    v4d acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TN; ++j)
             acc[i][j] = (v4d){0.0, 0.0, 0.0, 0.0};
 
     const int nk = (K + BK - 1) / BK;
@@ -93,17 +107,17 @@ __global__ __launch_bounds__(256) void gemm_f64_mfma(int M, int N, int K,
 #pragma unroll
         for (int ks = 0; ks < BK / 4; ++ks) {
             const int kk = ks * 4 + lk;
-            double a[2], b[2];
+            double a[TM], b[TN];
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
-                a[i] = As[buf][kk][wm * 32 + i * 16 + lr];
+            for (int i = 0; i < TM; ++i)
+                a[i] = As[buf][kk][(wm * TM + i) * 16 + lr];
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-                b[j] = Bs[buf][kk][wn * 32 + j * 16 + lr];
+            for (int j = 0; j < TN; ++j)
+                b[j] = Bs[buf][kk][(wn * TN + j) * 16 + lr];
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                for (int j = 0; j < TN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[i], b[j], acc[i][j], 0, 0, 0);
         }
         if (t + 1 < nk) {
@@ -114,13 +128,13 @@ __global__ __launch_bounds__(256) void gemm_f64_mfma(int M, int N, int K,
     // D layout of the 16x16x4 f64 instruction (measured on gfx950): register r of a lane holds
     // row 4*r + lane/16, column lane % 16.
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int col = n0 + wn * 32 + j * 16 + lr;
+        for (int j = 0; j < TN; ++j) {
+            const int col = n0 + (wn * TN + j) * 16 + lr;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int row = m0 + wm * 32 + i * 16 + r * 4 + lk;
+                const int row = m0 + (wm * TM + i) * 16 + r * 4 + lk;
                 if (FULL || (row < M && col < N)) {
                     double* c = C + (int64_t)row * ldc + col;
                     *c = *c + acc[i][j][r];
@@ -193,18 +207,34 @@ extern "C" int cnh_gemm_acc(int dtype, int64_t M, int64_t N, int64_t K, const vo
     hipStream_t st = as_stream(s);
     switch (dtype) {
     case CNH_F64: {
+        constexpr int BM = 64, BN = 64;
         const int64_t blocks = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
         CNH_CHECK(blocks < (1ll << 31), -3, "cnh_gemm_acc: too many tiles");
         const bool full = (M % BM == 0) && (N % BN == 0) && (K % BK == 0) && (lda % 2 == 0) &&
                           (ldb % 2 == 0) && (((uintptr_t)A & 15) == 0) && (((uintptr_t)B & 15) == 0);
-        if (full)
-            hipLaunchKernelGGL(gemm_f64_mfma<true>, dim3((unsigned)blocks), dim3(256), 0, st, (int)M,
-                               (int)N, (int)K, (const double*)A, lda, (const double*)B, ldb,
-                               (double*)C, ldc);
-        else
-            hipLaunchKernelGGL(gemm_f64_mfma<false>, dim3((unsigned)blocks), dim3(256), 0, st,
-                               (int)M, (int)N, (int)K, (const double*)A, lda, (const double*)B, ldb,
-                               (double*)C, ldc);
+        // 64x64 tiles either way; 8 wavefronts per workgroup unless the grid already gives
+        // every CU several workgroups.
+        const bool many = blocks >= 1024;
+        const dim3 grid((unsigned)blocks);
+        if (many) {
+            if (full)
+                hipLaunchKernelGGL((gemm_f64_mfma<2, 2, 2, 2, true>), grid, dim3(256), 0, st, (int)M,
+                                   (int)N, (int)K, (const double*)A, lda, (const double*)B, ldb,
+                                   (double*)C, ldc);
+            else
+                hipLaunchKernelGGL((gemm_f64_mfma<2, 2, 2, 2, false>), grid, dim3(256), 0, st, (int)M,
+                                   (int)N, (int)K, (const double*)A, lda, (const double*)B, ldb,
+                                   (double*)C, ldc);
+        } else {
+            if (full)
+                hipLaunchKernelGGL((gemm_f64_mfma<2, 4, 2, 1, true>), grid, dim3(512), 0, st, (int)M,
+                                   (int)N, (int)K, (const double*)A, lda, (const double*)B, ldb,
+                                   (double*)C, ldc);
+            else
+                hipLaunchKernelGGL((gemm_f64_mfma<2, 4, 2, 1, false>), grid, dim3(512), 0, st, (int)M,
+                                   (int)N, (int)K, (const double*)A, lda, (const double*)B, ldb,
+                                   (double*)C, ldc);
+        }
         CNH_HIP(hipGetLastError());
         return 0;
     }
