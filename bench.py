@@ -27,6 +27,10 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 FP64_MFMA_PEAK_TFLOPS = 78.6
+# HBM bytes per launch of the tiled matvec at n = 16384, from rocprofv3 FETCH_SIZE (x 2.0, the
+# factor a plain streaming kernel of known size gives on gfx950) + WRITE_SIZE (x 1.0):
+# (2 098 220 + 128.3) KiB, see profiles/bench_hbm_traffic_pmc.txt.
+GEMV_N16384_TRAFFIC_BYTES = 2148708659
 
 
 def _dev():
@@ -609,7 +613,7 @@ def main():
     ap.add_argument("--n", type=int, default=16384, help="order of the CG system")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-also", action="store_true", help="skip the secondary workloads")
-    ap.add_argument("--cpu-iters", type=int, default=10)
+    ap.add_argument("--cpu-iters", type=int, default=50)
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: every partition of the path lives on a single MI355X; "
@@ -643,7 +647,8 @@ def main():
                    "device": name.value.decode()},
         "roofline": {"bound": "hbm", "kernel": "gemv_rows<double>", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": None, "avg_us": round(cg["gemv_avg_us"], 2),
+                     "traffic": GEMV_N16384_TRAFFIC_BYTES if n == 16384 else None,
+                     "avg_us": round(cg["gemv_avg_us"], 2),
                      "bytes_per_launch": gemv_bytes},
         "gemv_roofline_iters_per_s": round(HBM_PEAK_GBS * 1e9 / gemv_bytes, 1),
         "rtr_final": cg["rtr_final"],
@@ -671,7 +676,7 @@ def main():
         cores = os.cpu_count() or 1
         threads = min(cores, 16)
         setup = cpu_cg_setup(n)
-        ips1, xc, rtr_c = cpu_cg(setup, n, max(2, args.cpu_iters // 2), 1)
+        ips1, xc, rtr_c = cpu_cg(setup, n, args.cpu_iters, 1)
         ipsN, _, _ = cpu_cg(setup, n, args.cpu_iters, threads)
         line["cpu_baseline"] = {
             "value": round(ipsN, 3), "unit": "iterations/s", "cores": threads, "kind": "port",
@@ -679,6 +684,9 @@ def main():
                       f"oracle kernels, tile matvec split over {threads} threads",
             "one_core": round(ips1, 3),
         }
+        if args.cpu_iters == args.steps and cg.get("x") is not None:
+            # same system, same number of iterations: the two solutions must agree
+            line["cg_parity_max_rel_diff"] = float(np.max(np.abs(cg["x"] - xc)) / np.max(np.abs(xc)))
     print(json.dumps(line))
 
 
