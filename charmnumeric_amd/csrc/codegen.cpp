@@ -310,8 +310,12 @@ std::string prelude(const GroupProgram& p) {
              "    if (b == -1) return (T)((UT)0 - (UT)a);\n"
              "    return a / b;\n}\n";
     } else if (p.dtype == CNH_F64) {
-        s << "__device__ __forceinline__ T cn_exp(T x) { return exp(x); }\n"
-             "__device__ __forceinline__ T cn_tanh(T x) { return tanh(x); }\n";
+        // exp/tanh must give what the host C library gives (upstream lowers math.exp/tanh to
+        // libm calls), so the group carries its own restatement instead of the device library's.
+        if (p.body.find("cn_exp(") != std::string::npos || p.body.find("cn_tanh(") != std::string::npos)
+            s << libm_f64_text()
+              << "__device__ __forceinline__ T cn_exp(T x) { return cn_exp_f64(x); }\n"
+                 "__device__ __forceinline__ T cn_tanh(T x) { return cn_tanh_f64(x); }\n";
     } else {
         s << "__device__ __forceinline__ T cn_exp(T x) { return expf(x); }\n"
              "__device__ __forceinline__ T cn_tanh(T x) { return tanhf(x); }\n";

@@ -87,4 +87,7 @@ int emit_variant_source(const GroupProgram& p, const std::string& variant, std::
 
 const char* dtype_ctype(int dtype);
 
+// fp64 exp/tanh restated to agree bit for bit with the host C library (codegen_libm.cpp).
+std::string libm_f64_text();
+
 } // namespace cnh

@@ -262,3 +262,26 @@ def launch_tiles(k, inputs, scalars, cur, dst, scalars_on_device=False):
     L.check(L.lib.cnh_launch_group_tiles(k, len(inputs), descs, len(scalars), sp,
                                          1 if scalars_on_device else 0,
                                          C.byref(cd) if cd is not None else None, C.byref(dd), None))
+
+
+def host_libm_is_the_restated_one():
+    """True where the host's exp/tanh are the algorithms the device code restates: x86-64 glibc
+    2.28..2.38 (table-driven exp with its FMA build selected at load time, fdlibm tanh/expm1)."""
+    import platform
+    if platform.machine() != "x86_64":
+        return False
+    lib, ver = platform.libc_ver()
+    if lib != "glibc":
+        return False
+    try:
+        major, minor = (int(t) for t in ver.split(".")[:2])
+    except ValueError:
+        return False
+    if (major, minor) < (2, 28) or (major, minor) > (2, 38):
+        return False
+    try:
+        with open("/proc/cpuinfo") as f:
+            flags = next((ln for ln in f if ln.startswith("flags")), "")
+    except OSError:
+        return False
+    return " fma " in flags + " " and " avx2 " in flags + " "

@@ -1,0 +1,104 @@
+"""The fp64 exp/tanh text that generated kernels carry, compiled for the host and compared with the
+host C library (what upstream's JIT calls, src/jit.cpp:399,445-459), plus an offline gfx950 build
+of a group that uses both."""
+import os
+import subprocess
+import sys
+
+import pytest
+
+from tests import helpers as H
+from charmnumeric_amd import _lib as L
+from charmnumeric_amd.astbuild import AstBuilder
+
+CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "charmnumeric_amd", "csrc")
+
+DRIVER = r"""
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+static const unsigned long long CN_EXP_TAB[256] = {
+#include "exp_table.inc"
+};
+#define CN_DEV static inline
+#include "libm_body.inc"
+static uint64_t sm(uint64_t* s) {
+    uint64_t z = (*s += 0x9E3779B97F4A7C15ull);
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull; z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+static long ulps(double a, double b) {
+    if (std::isnan(a) && std::isnan(b)) return 0;
+    int64_t x, y; memcpy(&x, &a, 8); memcpy(&y, &b, 8);
+    if (x < 0) x = INT64_MIN - x; if (y < 0) y = INT64_MIN - y;
+    return (long)(x > y ? x - y : y - x);
+}
+int main() {
+    uint64_t s = 7; long worst_e = 0, worst_t = 0, bad_e = 0, bad_t = 0;
+    const double rg[][2] = {{-746, -700}, {700, 710}, {-1, 1}, {-30, 30}, {-745, 710}, {-1e-3, 1e-3}};
+    for (auto& r : rg)
+        for (long i = 0; i < 400000; ++i) {
+            double x = r[0] + (r[1] - r[0]) * ((sm(&s) >> 11) * 0x1p-53);
+            long de = ulps(exp(x), cn_exp_f64(x)), dt = ulps(tanh(x), cn_tanh_f64(x));
+            if (de) { ++bad_e; if (de > worst_e) worst_e = de; }
+            if (dt) { ++bad_t; if (dt > worst_t) worst_t = dt; }
+        }
+    const double sp[] = {0.0, -0.0, INFINITY, -INFINITY, NAN, 709.78, 709.79, -745.1, -745.2, -708.4,
+                         1e-300, -1e-300, 22.0, -22.0, 21.999, 1.0, -1.0, 0x1p-55, 0x1p-54, 5e-324};
+    for (double x : sp) {
+        if (ulps(exp(x), cn_exp_f64(x))) { ++bad_e; worst_e = 99; }
+        if (ulps(tanh(x), cn_tanh_f64(x))) { ++bad_t; worst_t = 99; }
+    }
+    printf("%ld %ld %ld %ld\n", bad_e, worst_e, bad_t, worst_t);
+    return 0;
+}
+"""
+
+
+def test_device_exp_tanh_text_matches_host_libm(tmp_path):
+    body = open(os.path.join(CSRC, "libm_f64.inc")).read().splitlines()
+    assert body[0].startswith('R"CNLIBM(') and body[-1].startswith(')CNLIBM"')
+    (tmp_path / "libm_body.inc").write_text("\n".join(body[1:-1]) + "\n")
+    (tmp_path / "driver.cpp").write_text(DRIVER)
+    exe = tmp_path / "driver"
+    subprocess.check_call(["g++", "-O2", "-std=c++17", "-ffp-contract=off", "-mfma", "-I", CSRC,
+                           "-I", str(tmp_path), str(tmp_path / "driver.cpp"), "-o", str(exe)])
+    bad_e, worst_e, bad_t, worst_t = (int(t) for t in subprocess.check_output([str(exe)]).split())
+    print(f"exp: {bad_e} differing (worst {worst_e} ulp); tanh: {bad_t} differing (worst {worst_t} ulp)")
+    assert worst_e <= 1 and worst_t <= 1
+    if H.host_libm_is_the_restated_one():
+        assert bad_e == 0 and bad_t == 0
+
+
+def test_exp_table_is_what_its_definition_gives():
+    mp = pytest.importorskip("mpmath")
+    import struct
+    mp.mp.prec = 240
+    words = []
+    for ln in open(os.path.join(CSRC, "exp_table.inc")):
+        words += [int(t.strip().rstrip("ul"), 16) for t in ln.split(",") if t.strip().startswith("0x")]
+    assert len(words) == 256
+    for k in range(128):
+        v = mp.power(2, mp.mpf(k) / 128)
+        h = struct.unpack("<d", struct.pack("<Q", (words[2 * k + 1] + (k << 45)) & (2**64 - 1)))[0]
+        t = struct.unpack("<d", struct.pack("<Q", words[2 * k]))[0]
+        assert h == float(v)
+        assert abs(mp.mpf(h) * (1 + mp.mpf(t)) / v - 1) < mp.mpf(2) ** -105
+
+
+@pytest.mark.parametrize("variant", ["flat", "nd", "tiles"])
+def test_group_with_exp_and_tanh_builds_for_gfx950(variant):
+    b = AstBuilder(1, L.F64)
+    lx = b.leaf(1)
+    t0 = b.binary(L.OP_MUL, 100, lx, b.scalar(-1))
+    t1 = b.unary(L.OP_EXP, 101, t0)
+    t2 = b.binary(L.OP_ADD, 102, b.scalar(1.0), t1)
+    t3 = b.binary(L.OP_DIV, 103, b.scalar(1.0), t2)
+    b.unary(L.OP_TANH, 2, t3, is_temp=False)
+    k = H.compile_group(b.finish(), L.F64, 1)
+    src = H.kernel_source(k, variant)
+    assert "cn_exp_f64" in src and "CN_EXP_TAB" in src
+    L.check(L.lib.cnh_kernel_build(k, variant.encode()))
+    # groups without exp/tanh do not carry the text
+    assert "cn_exp_f64" not in H.kernel_source(H.compile_group(H.ast_c1(L.F64), L.F64, 1), variant)
