@@ -214,6 +214,25 @@ _PROTOS = {
                                      C.c_int64, C.c_int64, C.c_uint64, C.c_void_p]),
 }
 
+# Host executor (include/cnexec.h).
+_i32p = C.POINTER(C.c_int32)
+_PROTOS.update({
+    "cnx_create": (C.c_int, [C.c_int, C.c_int, C.c_int, _vpp]),
+    "cnx_destroy": (C.c_int, [C.c_void_p]),
+    "cnx_set_min_tile": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
+    "cnx_receive_dag": (C.c_int, [C.c_void_p, C.c_int, C.c_int64, C.c_char_p]),
+    "cnx_get": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int, C.c_void_p]),
+    "cnx_put": (C.c_int, [C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_void_p]),
+    "cnx_fill_uniform": (C.c_int, [C.c_void_p, C.c_int, C.c_uint64, C.c_uint64, C.c_double, C.c_double]),
+    "cnx_fill_cg_matrix": (C.c_int, [C.c_void_p, C.c_int, C.c_uint64]),
+    "cnx_sync": (C.c_int, [C.c_void_p]),
+    "cnx_array_info": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int),
+                                 C.POINTER(C.c_int), _i32p, _i32p]),
+    "cnx_stats": (C.c_int, [C.c_void_p, _i64p]),
+    "cnx_set_trace": (C.c_int, [C.c_void_p, C.c_int]),
+    "cnx_trace": (C.c_int64, [C.c_void_p, C.c_char_p, C.c_size_t]),
+})
+
 EXPORTS = tuple(_PROTOS)
 
 for _name, (_res, _args) in _PROTOS.items():

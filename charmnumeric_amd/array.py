@@ -1,0 +1,620 @@
+"""Array and ArrayView: the NumPy-like lazy frontend objects.
+
+API contract of upstream's frontend (charmnumeric/charmnumeric.py upstream): operators and their
+reflected forms (:394-482), slicing rules (:272-343: integers keep their dimension as extent 1,
+negative steps and newaxis are refused), dtype rules (:369-373: scalars never promote), matmul routing
+(:485-533), creation routines (:860-1062) and `.get(interface)` (:683-688). Everything is recorded
+through `lazy` and runs when something calls `execute` or `.get`.
+"""
+from __future__ import annotations
+
+import numbers
+
+import numpy as np
+
+from . import _lib as L
+from . import lazy
+
+_DEFAULT_DTYPE = np.dtype("float64")
+_SUPPORTED = (np.dtype("float32"), np.dtype("float64"), np.dtype("int32"), np.dtype("int64"))
+
+
+class DType:
+    """Element type numbers shared with the executor (charmnumeric.py:34-40 upstream)."""
+
+    FLOAT32, FLOAT64, INT32, INT64 = 0, 1, 2, 3
+
+    @staticmethod
+    def from_numpy(np_dtype):
+        return lazy.wire_dtype(_normalize_dtype(np_dtype))
+
+    @staticmethod
+    def to_numpy(wire):
+        try:
+            return _SUPPORTED[(0, 1, 2, 3).index(wire)]
+        except ValueError:
+            raise TypeError(f"Unsupported wire dtype {wire!r}") from None
+
+    @staticmethod
+    def promote(a, b):
+        return DType.from_numpy(np.result_type(DType.to_numpy(a), DType.to_numpy(b)))
+
+
+class _CallableInt(int):
+    """`a.size` that may also be called as `a.size()` (both spellings occur upstream)."""
+
+    def __call__(self):
+        return int(self)
+
+
+def _normalize_dtype(dtype, allow_none=False):
+    if dtype is None:
+        return None if allow_none else _DEFAULT_DTYPE
+    dt = np.dtype(dtype)
+    if dt not in _SUPPORTED:
+        raise TypeError(f"charmnumeric only supports float32, float64, int32, and int64; got {dt}")
+    return dt
+
+
+def _normalize_shape(shape):
+    out = (int(shape),) if isinstance(shape, numbers.Integral) else tuple(int(s) for s in shape)
+    if any(s < 0 for s in out):
+        raise ValueError(f"negative dimensions are not allowed: {out}")
+    if not 1 <= len(out) <= 3:
+        raise NotImplementedError(f"arrays of rank {len(out)} are not supported (1 to 3)")
+    if any(s == 0 for s in out):
+        raise NotImplementedError("zero-sized arrays are not supported")
+    return out
+
+
+def _is_scalar_like(v):
+    if isinstance(v, np.ndarray):
+        return v.ndim == 0
+    return isinstance(v, (bool, numbers.Real, np.generic))
+
+
+def _coerce_scalar(v):
+    if isinstance(v, (np.ndarray, np.generic)):
+        v = v.item()
+    if isinstance(v, bool):
+        return int(v)
+    if isinstance(v, numbers.Integral):
+        return int(v)
+    return float(v)
+
+
+def _size(shape):
+    n = 1
+    for s in shape:
+        n *= int(s)
+    return n
+
+
+# ---------------------------------------------------------------------------------------------
+# regions
+
+
+def _expand_key(key, ndims):
+    if not isinstance(key, tuple):
+        key = (key,)
+    if sum(1 for k in key if k is Ellipsis) > 1:
+        raise IndexError("an index can only have a single ellipsis")
+    if any(k is None for k in key):
+        raise NotImplementedError("np.newaxis is not supported yet")
+    explicit = sum(1 for k in key if k is not Ellipsis)
+    if explicit > ndims:
+        raise IndexError(f"too many indices for array: array is {ndims}-dimensional, "
+                         f"but {explicit} were indexed")
+    out = []
+    for k in key:
+        if k is Ellipsis:
+            out.extend([slice(None)] * (ndims - explicit))
+        else:
+            out.append(k)
+    out.extend([slice(None)] * (ndims - len(out)))
+    return out
+
+
+def parse_key(key, shape):
+    """Index expression -> (start, stop, step) per dimension, relative to an object of `shape`."""
+    ndims = len(shape)
+    start, stop, step = [0] * ndims, [0] * ndims, [1] * ndims
+    for d, item in enumerate(_expand_key(key, ndims)):
+        if isinstance(item, slice):
+            st = 1 if item.step is None else int(item.step)
+            if st == 0:
+                raise ValueError("slice step cannot be zero")
+            if st < 0:
+                raise NotImplementedError("negative slicing is not supported yet")
+            start[d], stop[d], step[d] = item.indices(shape[d])
+        elif isinstance(item, numbers.Integral):
+            i = int(item)
+            if i < 0:
+                i += shape[d]
+            if not 0 <= i < shape[d]:
+                raise IndexError(f"index {item} is out of bounds for axis {d} with size {shape[d]}")
+            start[d], stop[d], step[d] = i, i + 1, 1
+        else:
+            raise TypeError("only integers, slices, and ellipsis are valid charmnumeric indices")
+    return tuple(start), tuple(stop), tuple(step)
+
+
+def region_shape(region):
+    start, stop, step = region
+    return tuple(max(0, (stop[d] - start[d] + step[d] - 1) // step[d]) for d in range(len(start)))
+
+
+def compose(outer, inner):
+    """Region `inner` (relative to the view `outer`) expressed relative to outer's base array."""
+    if outer is None:
+        return inner
+    ostart, _, ostep = outer
+    istart, istop, istep = inner
+    nd = len(istart)
+    return (tuple(ostart[d] + istart[d] * ostep[d] for d in range(nd)),
+            tuple(ostart[d] + istop[d] * ostep[d] for d in range(nd)),
+            tuple(ostep[d] * istep[d] for d in range(nd)))
+
+
+def _is_whole(region, shape):
+    return region is None or all(region[0][d] == 0 and region[1][d] == shape[d] and region[2][d] == 1
+                                 for d in range(len(shape)))
+
+
+# ---------------------------------------------------------------------------------------------
+# the objects
+
+
+class _ArrayLike:
+    __array_priority__ = 1000
+
+    # -- basic properties --
+    @property
+    def ndim(self):
+        return self.ndims
+
+    @property
+    def size(self):
+        return _CallableInt(_size(self.shape))
+
+    @property
+    def itemsize(self):
+        return self.dtype.itemsize
+
+    @property
+    def nbytes(self):
+        return int(self.size) * self.itemsize
+
+    def wire_dtype(self):
+        return lazy.wire_dtype(self.dtype)
+
+    def __len__(self):
+        return self.shape[0]
+
+    def __bool__(self):
+        raise ValueError("The truth value of a charmnumeric array is ambiguous. "
+                         "Use .get(interface) to materialize it first.")
+
+    def __array__(self, dtype=None, copy=None):
+        raise TypeError("charmnumeric arrays are lazy frontend objects. "
+                        "Call .get(interface) before converting to numpy.")
+
+    # -- operand form --
+    def _ref(self, broadcast=False):
+        raise NotImplementedError
+
+    def _base(self):
+        raise NotImplementedError
+
+    # -- slicing --
+    def __getitem__(self, key):
+        inner = parse_key(key, self.shape)
+        return ArrayView(self._base(), compose(self._region(), inner))
+
+    def __setitem__(self, key, rhs):
+        inner = parse_key(key, self.shape)
+        region = compose(self._region(), inner)
+        shape = region_shape(inner)
+        base = self._base()
+        value = _coerce_assignment_operand(rhs, shape, self.dtype)
+        if isinstance(value, _ArrayLike):
+            if value.dtype != self.dtype:
+                raise NotImplementedError("assignment across dtypes is not implemented")
+            if tuple(value.shape) != tuple(shape):
+                raise ValueError(f"could not broadcast input from shape {value.shape} into shape {shape}")
+            operand = value._ref()
+        else:
+            operand = value
+        whole = lazy.ArrayRef(base.name, None, base.shape, base.ndims, base.wire_dtype())
+        lazy.record(lazy.Instr("set", name=base.name, operands=[operand], shape=shape,
+                               dtype=base.wire_dtype(), region=region, payload=whole))
+
+    # -- arithmetic --
+    def __add__(self, o):
+        return _binary(L.OP_ADD, self, o)
+
+    def __radd__(self, o):
+        return _binary(L.OP_ADD, o, self)
+
+    def __sub__(self, o):
+        return _binary(L.OP_SUB, self, o)
+
+    def __rsub__(self, o):
+        return _binary(L.OP_SUB, o, self)
+
+    def __mul__(self, o):
+        return _binary(L.OP_MUL, self, o)
+
+    def __rmul__(self, o):
+        return _binary(L.OP_MUL, o, self)
+
+    def __truediv__(self, o):
+        return _binary(L.OP_DIV, self, o)
+
+    def __rtruediv__(self, o):
+        return _binary(L.OP_DIV, o, self)
+
+    def __neg__(self):
+        # upstream spells negation as multiplication by -1 (charmnumeric.py:427-434)
+        return _binary(L.OP_MUL, self, -1)
+
+    def __matmul__(self, o):
+        return _matmul(self, o)
+
+    def dot(self, o):
+        return _matmul(self, o)
+
+    def matvec(self, vec):
+        return _matvec(self, vec)
+
+    def copy(self):
+        out = empty(self.shape, dtype=self.dtype)
+        out[...] = self
+        return out
+
+    def fill(self, value):
+        self[...] = value
+
+    def astype(self, dtype, copy=True):
+        if _normalize_dtype(dtype) != self.dtype:
+            raise NotImplementedError(
+                "dtype conversion for existing charmnumeric arrays is not implemented yet")
+        return self.copy() if copy else self
+
+
+class Array(_ArrayLike):
+    """A whole distributed array, existing or about to be computed."""
+
+    def __init__(self, shape, dtype, name=None):
+        self.shape = tuple(shape)
+        self.ndims = len(self.shape)
+        self.dtype = np.dtype(dtype)
+        self.name = lazy.new_name() if name is None else name
+
+    def __del__(self):
+        lazy.record_delete(self.name)
+
+    def __repr__(self):
+        return f"Array(shape={self.shape}, dtype={self.dtype.name}, name={self.name})"
+
+    def _base(self):
+        return self
+
+    def _region(self):
+        return None
+
+    def _ref(self, broadcast=False):
+        return lazy.ArrayRef(self.name, None, self.shape, self.ndims, self.wire_dtype(), broadcast)
+
+    def get(self, interface):
+        lazy.execute(interface)
+        data = interface.get(self.ndims, self.name, int(self.size), dtype=self.dtype)
+        return data.reshape(self.shape) if self.ndims > 1 else data
+
+
+class ArrayView(_ArrayLike):
+    """A rectangular, possibly strided, slice of an Array. Keeps its base alive."""
+
+    def __init__(self, base, region):
+        self.base = base
+        self.region = region
+        self.shape = region_shape(region)
+        self.ndims = base.ndims
+        self.dtype = base.dtype
+        if any(s == 0 for s in self.shape):
+            raise NotImplementedError("zero-sized slices are not supported")
+
+    @property
+    def name(self):
+        return self.base.name
+
+    def __repr__(self):
+        return f"ArrayView(shape={self.shape}, dtype={self.dtype.name}, name={self.name})"
+
+    def _base(self):
+        return self.base
+
+    def _region(self):
+        return self.region
+
+    def _ref(self, broadcast=False):
+        region = None if _is_whole(self.region, self.base.shape) else self.region
+        return lazy.ArrayRef(self.base.name, region, self.shape, self.base.ndims, self.wire_dtype(),
+                             broadcast)
+
+    def get(self, interface):
+        out = empty(self.shape, dtype=self.dtype)
+        out[...] = self
+        return out.get(interface)
+
+
+# ---------------------------------------------------------------------------------------------
+# operations
+
+
+def _as_operand(v):
+    if isinstance(v, _ArrayLike):
+        return v
+    if _is_scalar_like(v):
+        return _coerce_scalar(v)
+    host = np.asarray(v)
+    if host.ndim == 0:
+        return _coerce_scalar(host.item())
+    return asarray(host)
+
+
+def _binary(opcode, lhs, rhs):
+    lhs, rhs = _as_operand(lhs), _as_operand(rhs)
+    arrays = [x for x in (lhs, rhs) if isinstance(x, _ArrayLike)]
+    dtype = arrays[0].dtype
+    for a in arrays[1:]:
+        if a.dtype != dtype:
+            raise NotImplementedError(
+                f"elementwise operations across dtypes ({dtype} and {a.dtype}) are not implemented")
+    big = [a.shape for a in arrays if _size(a.shape) > 1]
+    shape = tuple(big[0]) if big else tuple(arrays[0].shape)
+    for other in big[1:]:
+        if tuple(other) != shape:
+            raise ValueError(f"operands could not be broadcast together with shapes "
+                             f"{arrays[0].shape} and {arrays[1].shape}")
+    operands = []
+    for x in (lhs, rhs):
+        if isinstance(x, _ArrayLike):
+            bc = _size(x.shape) == 1 and _size(shape) > 1
+            if bc and not _is_whole(x._region(), x._base().shape):
+                raise NotImplementedError("a one-element slice cannot be used as a scalar operand")
+            operands.append(x._ref(broadcast=bc))
+        else:
+            operands.append(x)
+    out = Array(shape, dtype)
+    lazy.record(lazy.Instr("op", name=out.name, opcode=opcode, operands=operands, shape=shape,
+                           dtype=out.wire_dtype()))
+    return out
+
+
+def unary(opcode, x):
+    x = asarray(x)
+    if x.dtype.kind != "f":
+        raise TypeError("tanh/exp need a floating-point array")
+    out = Array(x.shape, x.dtype)
+    lazy.record(lazy.Instr("op", name=out.name, opcode=opcode, operands=[x._ref()], shape=x.shape,
+                           dtype=out.wire_dtype()))
+    return out
+
+
+def _whole(x):
+    """An operand of a non-fusible operation must be a whole array: slices are copied out first."""
+    if isinstance(x, ArrayView) and not _is_whole(x.region, x.base.shape):
+        return x.copy()
+    return x
+
+
+def nonfusible(opcode, operands, shape, dtype):
+    operands = [_whole(o) for o in operands]
+    out = Array(shape, dtype)
+    lazy.record(lazy.Instr("nonfusible", name=out.name, opcode=opcode, operands=[o._ref() for o in operands],
+                           shape=shape, dtype=out.wire_dtype()))
+    return out
+
+
+def _same_dtype(a, b, what):
+    if a.dtype != b.dtype:
+        raise NotImplementedError(f"{what} across dtypes ({a.dtype} and {b.dtype}) is not implemented")
+    return a.dtype
+
+
+def _matmul(lhs, rhs):
+    rhs = _as_operand(rhs)
+    if not isinstance(rhs, _ArrayLike):
+        raise ValueError("matmul does not support scalar operands")
+    if lhs.ndims == 1 and rhs.ndims == 1:
+        if lhs.shape[0] != rhs.shape[0]:
+            raise ValueError(f"Shape mismatch for dot product: ({lhs.shape[0]},) @ ({rhs.shape[0]},)")
+        return nonfusible(L.OP_REDUCE, [lhs, rhs], (1,), _same_dtype(lhs, rhs, "dot"))
+    if lhs.ndims == 3:
+        raise NotImplementedError("matmul on a 3-D operand with a dropped dimension is not implemented")
+    if lhs.ndims != 2:
+        raise ValueError(f"matmul requires a 2D matrix, got {lhs.ndims}D")
+    if rhs.ndims == 1:
+        return _matvec(lhs, rhs)
+    if rhs.ndims == 2 and rhs.shape[1] == 1:
+        raise NotImplementedError("matmul with an (N, 1) column operand is not implemented")
+    if rhs.ndims == 2:
+        if lhs.shape[1] != rhs.shape[0]:
+            raise ValueError(f"Shape mismatch: ({lhs.shape[0]},{lhs.shape[1]}) @ "
+                             f"({rhs.shape[0]},{rhs.shape[1]})")
+        return nonfusible(L.OP_MATMATMUL, [lhs, rhs], (lhs.shape[0], rhs.shape[1]),
+                          _same_dtype(lhs, rhs, "matmul"))
+    raise NotImplementedError("matmul with a 3-D right operand is not implemented")
+
+
+def _matvec(mat, vec):
+    if not isinstance(vec, _ArrayLike):
+        raise ValueError("matvec requires an Array vector")
+    if mat.ndims != 2:
+        raise NotImplementedError(f"matvec on a {mat.ndims}D operand is not implemented")
+    if vec.ndims != 1:
+        raise ValueError("matvec requires a 1D vector (N,)")
+    if mat.shape[1] != vec.shape[0]:
+        raise ValueError(f"Shape mismatch: matrix cols {mat.shape[1]} != vector size {vec.shape[0]}")
+    return nonfusible(L.OP_MATMUL, [mat, vec], (mat.shape[0],), _same_dtype(mat, vec, "matvec"))
+
+
+# ---------------------------------------------------------------------------------------------
+# creation
+
+
+def create_array(shape, dtype=_DEFAULT_DTYPE):
+    shape = _normalize_shape(shape)
+    dtype = _normalize_dtype(dtype)
+    out = Array(shape, dtype)
+    lazy.record(lazy.Instr("create", name=out.name, shape=shape, dtype=out.wire_dtype()))
+    return out
+
+
+def empty(shape, dtype=_DEFAULT_DTYPE):
+    return create_array(shape, dtype=dtype)
+
+
+def zeros(shape, dtype=_DEFAULT_DTYPE):
+    return create_array(shape, dtype=dtype)       # new arrays are zero-filled by the executor
+
+
+def _assign_host_data(target, values):
+    """Whole-array load from host data. A constant array becomes one fill; anything else one bulk
+    upload (upstream assigns element by element here, charmnumeric.py:863-878)."""
+    host = np.ascontiguousarray(values, dtype=target.dtype)
+    if host.shape != tuple(target.shape):
+        raise ValueError(f"cannot assign data with shape {host.shape} into shape {target.shape}")
+    first = host.reshape(-1)[0]
+    if host.size == 1 or np.all(host == first):
+        target[...] = _coerce_scalar(first)
+        return target
+    lazy.record(lazy.Instr("call", name=target.name, opcode="put", shape=target.shape,
+                           dtype=target.wire_dtype(), payload=host.copy()))
+    return target
+
+
+def _from_host(values, dtype=None, copy=True, ndmin=0):
+    host = np.array(values, dtype=_normalize_dtype(dtype, allow_none=True), copy=copy)
+    while host.ndim < ndmin:
+        host = host[None]
+    if host.ndim == 0:
+        raise NotImplementedError("0D charmnumeric arrays are not supported yet")
+    out = create_array(host.shape, dtype=_normalize_dtype(host.dtype))
+    return _assign_host_data(out, host)
+
+
+def _coerce_assignment_operand(rhs, shape, dtype):
+    if isinstance(rhs, _ArrayLike):
+        return rhs
+    if _is_scalar_like(rhs):
+        return _coerce_scalar(rhs)
+    host = np.asarray(rhs, dtype=dtype)
+    if host.ndim == 0:
+        return _coerce_scalar(host.item())
+    try:
+        host = np.broadcast_to(host, shape)
+    except ValueError as exc:
+        raise ValueError(f"could not broadcast input from shape {host.shape} into shape {shape}") from exc
+    return _from_host(host, dtype=host.dtype)
+
+
+def full(shape, fill_value, dtype=None):
+    shape = _normalize_shape(shape)
+    if _is_scalar_like(fill_value):
+        dt = _normalize_dtype(dtype, allow_none=True)
+        if dt is None:
+            dt = _normalize_dtype(np.asarray(fill_value).dtype)
+        out = empty(shape, dtype=dt)
+        out[...] = _coerce_scalar(fill_value)
+        return out
+    host = np.asarray(fill_value, dtype=_normalize_dtype(dtype, allow_none=True))
+    try:
+        host = np.broadcast_to(host, shape)
+    except ValueError as exc:
+        raise ValueError(f"could not broadcast fill_value from shape {host.shape} into shape {shape}") from exc
+    return _from_host(host, dtype=host.dtype)
+
+
+def ones(shape, dtype=_DEFAULT_DTYPE):
+    return full(shape, 1, dtype=dtype)
+
+
+def _like(a, dtype, shape):
+    if isinstance(a, _ArrayLike):
+        s, d = a.shape, a.dtype
+    else:
+        host = np.asarray(a)
+        if host.ndim == 0:
+            raise NotImplementedError("0D charmnumeric arrays are not supported yet")
+        s, d = host.shape, _normalize_dtype(host.dtype)
+    return (s if shape is None else _normalize_shape(shape)), (d if dtype is None else _normalize_dtype(dtype))
+
+
+def empty_like(a, dtype=None, shape=None):
+    s, d = _like(a, dtype, shape)
+    return empty(s, dtype=d)
+
+
+def zeros_like(a, dtype=None, shape=None):
+    s, d = _like(a, dtype, shape)
+    return zeros(s, dtype=d)
+
+
+def ones_like(a, dtype=None, shape=None):
+    s, d = _like(a, dtype, shape)
+    return ones(s, dtype=d)
+
+
+def full_like(a, fill_value, dtype=None, shape=None):
+    s, d = _like(a, dtype, shape)
+    return full(s, fill_value, dtype=d)
+
+
+def asarray(a, dtype=None):
+    want = _normalize_dtype(dtype, allow_none=True)
+    if isinstance(a, _ArrayLike):
+        if want is None or want == a.dtype:
+            return a
+        raise NotImplementedError(
+            "dtype conversion for existing charmnumeric arrays is not implemented yet")
+    return _from_host(a, dtype=want, copy=False)
+
+
+def array(a, dtype=None, copy=True, ndmin=0):
+    want = _normalize_dtype(dtype, allow_none=True)
+    if isinstance(a, _ArrayLike):
+        if want is not None and want != a.dtype:
+            raise NotImplementedError(
+                "dtype conversion for existing charmnumeric arrays is not implemented yet")
+        if len(a.shape) < ndmin:
+            raise NotImplementedError("ndmin on an existing charmnumeric array is not implemented")
+        return a.copy() if copy else a
+    return _from_host(a, dtype=want, copy=copy, ndmin=ndmin)
+
+
+def copy(a, order="K"):
+    return array(a, copy=True)
+
+
+def copyto(dst, src):
+    if not isinstance(dst, _ArrayLike):
+        raise TypeError("copyto destination must be a charmnumeric Array or ArrayView")
+    dst[...] = src
+    return dst
+
+
+def arange(start, stop=None, step=1, dtype=None):
+    host = np.arange(start, stop, step, dtype=_normalize_dtype(dtype, allow_none=True))
+    return _from_host(host, dtype=host.dtype, copy=False)
+
+
+def eye(N, M=None, k=0, dtype=_DEFAULT_DTYPE):
+    rows = int(N)
+    cols = rows if M is None else int(M)
+    return _from_host(np.eye(rows, cols, int(k), dtype=_normalize_dtype(dtype)))
+
+
+def identity(n, dtype=_DEFAULT_DTYPE):
+    return eye(n, dtype=dtype)

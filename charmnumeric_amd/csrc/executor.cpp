@@ -1,0 +1,1118 @@
+// Host executor: one object that plays upstream's ArrayDAGGroup (shape pass, decomposition, compile
+// cache: src/dag_group_receive.cpp:190-575, src/dag_group_compile.cpp:6-56) and the per-partition
+// executors (routing per node: src/executor_core.cpp:195-775) for every partition of every array,
+// all resident on one device. Halo messages do not exist here: kernels read neighbour tiles.
+#include "../../include/cnexec.h"
+#include "common.h"
+
+#include <algorithm>
+#include <array>
+#include <cstring>
+#include <map>
+#include <memory>
+#include <sstream>
+#include <unordered_map>
+#include <vector>
+
+using namespace cnh;
+
+namespace {
+
+constexpr int kOpDelete = CNX_OP_DELETE, kOpSum = CNX_OP_SUM, kOpSumsqDiff = CNX_OP_SUMSQ_DIFF,
+              kOpMaxabsDiff = CNX_OP_MAXABS_DIFF;
+
+struct Reader {
+    const char* p;
+    const char* end;
+    bool ok = true;
+    template <typename T> T get() {
+        T v{};
+        if (!ok || (size_t)(end - p) < sizeof(T)) {
+            ok = false;
+            return v;
+        }
+        std::memcpy(&v, p, sizeof(T));
+        p += sizeof(T);
+        return v;
+    }
+};
+
+// Region in upstream's wire form (charmnumeric.py:194-207).
+bool read_region(Reader& r, cnh_region& out) {
+    std::memset(&out, 0, sizeof out);
+    out.is_global = r.get<int32_t>();
+    if (!r.ok)
+        return false;
+    if (out.is_global) {
+        out.is_global = 1;
+        return true;
+    }
+    out.ndims = r.get<int32_t>();
+    if (!r.ok || out.ndims < 1 || out.ndims > CNH_MAX_ND)
+        return r.ok = false;
+    for (int d = 0; d < out.ndims; ++d) {
+        out.start[d] = r.get<int32_t>();
+        out.stop[d] = r.get<int32_t>();
+        out.step[d] = r.get<int32_t>();
+    }
+    return r.ok;
+}
+
+int region_count(const cnh_region& r, int d) {
+    if (r.step[d] <= 0 || r.stop[d] <= r.start[d])
+        return 0;
+    return (r.stop[d] - r.start[d] + r.step[d] - 1) / r.step[d];
+}
+
+struct DagNode {
+    int id = 0;
+    int fusible = 0;
+    std::vector<cnh_ast_node> nodes;
+    std::vector<int32_t> roots;
+};
+
+// One distributed array: ArrayMetadata (src/backend.hpp:285-288) + the per-chare Array<N,T> buffers
+// (src/backend.hpp:112-200). All tiles of an array are carved from one device allocation, tile t
+// row-major over its own extent; a 1-D array is therefore contiguous as a whole.
+struct XArray {
+    int name = 0, ndims = 1, dtype = CNH_F64, tile = 1;
+    int32_t shape[3] = {1, 1, 1}, offset[3] = {0, 0, 0}, grid[3] = {1, 1, 1};
+    int64_t ntiles = 1, elems = 1;
+    size_t bytes = 0;
+    void* slab = nullptr;
+    void* alt = nullptr; // second buffer set for sweeps that read what they assign
+    std::vector<int64_t> tile_off, tile_elems;
+    std::vector<void*> tiles, alt_tiles;
+
+    void tile_extent(int64_t t, int32_t lo[3], int32_t ext[3]) const {
+        int64_t rem = t;
+        for (int d = 0; d < 3; ++d) {
+            lo[d] = 0;
+            ext[d] = 1;
+        }
+        for (int d = ndims - 1; d >= 0; --d) {
+            int ti = (int)(rem % grid[d]);
+            rem /= grid[d];
+            lo[d] = ti * tile;
+            ext[d] = std::min((ti + 1) * tile, (int)shape[d]) - lo[d];
+        }
+    }
+    cnh_tiled tiled(bool use_alt = false) const {
+        cnh_tiled t;
+        std::memset(&t, 0, sizeof t);
+        t.ndims = ndims;
+        t.tile = tile;
+        for (int d = 0; d < ndims; ++d) {
+            t.offset[d] = offset[d];
+            t.shape[d] = shape[d];
+            t.grid_lo[d] = 0;
+            t.grid[d] = grid[d];
+        }
+        t.tiles = use_alt ? alt_tiles.data() : tiles.data();
+        return t;
+    }
+};
+
+} // namespace
+
+struct cnx_executor {
+    bool dry = false; // no device: every decision is taken and traced, nothing is launched
+    int num_pes = 1, odf = 4;
+    int min_tile[4] = {0, 262144, 512, 64}; // CT_MIN_TILE_1D/2D/3D, src/backend.hpp:10-18
+    cnh_stream stream = nullptr;
+    std::map<int, XArray> arrays;
+    std::unordered_map<uint64_t, cnh_kernel*> kernels; // compile_cache, src/dag_group_compile.cpp:43-56
+    std::map<size_t, std::vector<void*>> free_list;    // src/backend.hpp:366-545
+    int64_t stats[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    bool trace_on = false;
+    std::string trace;
+    uintptr_t fake_ptr = 0x1000;
+
+    void log(const std::string& s) {
+        if (trace_on) {
+            trace += s;
+            trace += '\n';
+        }
+    }
+};
+
+namespace {
+
+using Ex = cnx_executor;
+
+std::string shape_str(const int32_t* s, int nd) {
+    std::ostringstream o;
+    o << "(";
+    for (int d = 0; d < nd; ++d)
+        o << (d ? "," : "") << s[d];
+    o << ")";
+    return o.str();
+}
+
+int slab_alloc(Ex* ex, size_t bytes, bool zero, void** out) {
+    auto it = ex->free_list.find(bytes);
+    if (it != ex->free_list.end() && !it->second.empty()) {
+        *out = it->second.back();
+        it->second.pop_back();
+        ex->stats[4]++;
+        // Reused buffers are cleared like new ones (src/backend.hpp:490-497).
+        if (zero && !ex->dry)
+            if (int rc = cnh_memset0(*out, bytes, ex->stream))
+                return rc;
+        return 0;
+    }
+    ex->stats[3]++;
+    ex->stats[7] += (int64_t)bytes;
+    if (ex->dry) {
+        *out = reinterpret_cast<void*>(ex->fake_ptr);
+        ex->fake_ptr += (bytes + 255) & ~(size_t)255;
+        return 0;
+    }
+    return cnh_alloc(bytes, zero ? 1 : 0, out);
+}
+
+void slab_release(Ex* ex, size_t bytes, void* p) {
+    if (p)
+        ex->free_list[bytes].push_back(p);
+}
+
+// Tile edge: the minimum tile of the rank, doubled until the array has at most odf*PEs tiles
+// (src/decomposition_solver.hpp:100-122). Offsets are 0 for every array created here.
+int tile_rule(const Ex* ex, int ndims, const int32_t* shape) {
+    int64_t max_tiles = (int64_t)std::max(1, ex->odf) * std::max(1, ex->num_pes);
+    int64_t tile = 1;
+    while (tile < ex->min_tile[ndims])
+        tile *= 2;
+    tile = std::max<int64_t>(tile, ex->min_tile[ndims]);
+    for (;;) {
+        int64_t count = 1;
+        for (int d = 0; d < ndims; ++d)
+            count *= (shape[d] + tile - 1) / tile;
+        if (count <= max_tiles || tile > (1 << 30))
+            break;
+        tile *= 2;
+    }
+    return (int)tile;
+}
+
+int make_array(Ex* ex, int name, int ndims, int dtype, const int32_t* shape, bool zero, XArray** out) {
+    CNH_CHECK(ndims >= 1 && ndims <= 3, -20, "array %d: unsupported rank %d", name, ndims);
+    CNH_CHECK(dtype_size(dtype) != 0, -20, "array %d: unknown dtype %d", name, dtype);
+    CNH_CHECK(ex->arrays.find(name) == ex->arrays.end(), -21, "array %d already exists", name);
+    XArray a;
+    a.name = name;
+    a.ndims = ndims;
+    a.dtype = dtype;
+    a.elems = 1;
+    for (int d = 0; d < ndims; ++d) {
+        CNH_CHECK(shape[d] >= 1, -20, "array %d: extent %d in dim %d", name, shape[d], d);
+        a.shape[d] = shape[d];
+        a.elems *= shape[d];
+    }
+    a.tile = tile_rule(ex, ndims, shape);
+    a.ntiles = 1;
+    for (int d = 0; d < ndims; ++d) {
+        a.grid[d] = (a.shape[d] + a.tile - 1) / a.tile;
+        a.ntiles *= a.grid[d];
+    }
+    const int esz = dtype_size(dtype);
+    int64_t off = 0;
+    for (int64_t t = 0; t < a.ntiles; ++t) {
+        int32_t lo[3], ext[3];
+        a.tile_extent(t, lo, ext);
+        int64_t n = (int64_t)ext[0] * ext[1] * ext[2];
+        a.tile_off.push_back(off);
+        a.tile_elems.push_back(n);
+        off += n * esz;
+        if (ndims > 1)
+            off = (off + 255) & ~(int64_t)255;
+    }
+    a.bytes = (size_t)std::max<int64_t>((off + 255) & ~(int64_t)255, 256);
+    if (int rc = slab_alloc(ex, a.bytes, zero, &a.slab))
+        return rc;
+    for (int64_t t = 0; t < a.ntiles; ++t)
+        a.tiles.push_back(static_cast<char*>(a.slab) + a.tile_off[t]);
+    ex->log("create " + std::to_string(name) + " shape=" + shape_str(a.shape, ndims) + " dtype=" +
+            std::to_string(dtype) + " tile=" + std::to_string(a.tile) + " tiles=" +
+            std::to_string(a.ntiles));
+    auto ins = ex->arrays.emplace(name, std::move(a));
+    ex->stats[6] = (int64_t)ex->arrays.size();
+    if (out)
+        *out = &ins.first->second;
+    return 0;
+}
+
+int ensure_alt(Ex* ex, XArray& a) {
+    if (a.alt)
+        return 0;
+    if (int rc = slab_alloc(ex, a.bytes, false, &a.alt))
+        return rc;
+    a.alt_tiles.clear();
+    for (int64_t t = 0; t < a.ntiles; ++t)
+        a.alt_tiles.push_back(static_cast<char*>(a.alt) + a.tile_off[t]);
+    return 0;
+}
+
+void drop_array(Ex* ex, int name) {
+    auto it = ex->arrays.find(name);
+    if (it == ex->arrays.end())
+        return;
+    slab_release(ex, it->second.bytes, it->second.slab);
+    slab_release(ex, it->second.bytes, it->second.alt);
+    ex->arrays.erase(it);
+    ex->stats[6] = (int64_t)ex->arrays.size();
+    ex->log("delete " + std::to_string(name));
+}
+
+int find_array(Ex* ex, int name, XArray** out, const char* what) {
+    auto it = ex->arrays.find(name);
+    CNH_CHECK(it != ex->arrays.end(), -22, "%s: array %d does not exist", what, name);
+    *out = &it->second;
+    return 0;
+}
+
+bool same_decomposition(const XArray& a, const XArray& b) {
+    if (a.ndims != b.ndims || a.tile != b.tile)
+        return false;
+    for (int d = 0; d < a.ndims; ++d)
+        if (a.shape[d] != b.shape[d] || a.offset[d] != b.offset[d])
+            return false;
+    return true;
+}
+
+bool region_is_whole(const cnh_region& r, const XArray& a) {
+    if (r.is_global)
+        return true;
+    if (r.ndims != a.ndims)
+        return false;
+    for (int d = 0; d < a.ndims; ++d)
+        if (r.start[d] != 0 || r.stop[d] != a.shape[d] || r.step[d] != 1)
+            return false;
+    return true;
+}
+
+bool same_region(const cnh_region& a, const cnh_region& b) {
+    if (a.is_global != b.is_global)
+        return false;
+    if (a.is_global)
+        return true;
+    if (a.ndims != b.ndims)
+        return false;
+    for (int d = 0; d < a.ndims; ++d)
+        if (a.start[d] != b.start[d] || a.stop[d] != b.stop[d] || a.step[d] != b.step[d])
+            return false;
+    return true;
+}
+
+uint64_t fnv(const void* data, size_t n, uint64_t h = 1469598103934665603ull) {
+    const unsigned char* p = static_cast<const unsigned char*>(data);
+    for (size_t i = 0; i < n; ++i) {
+        h ^= p[i];
+        h *= 1099511628211ull;
+    }
+    return h;
+}
+
+// ---- node kinds ----
+
+int exec_create(Ex* ex, const cnh_ast_node& n) {
+    CNH_CHECK(!n.region.is_global && n.region.ndims == n.ndims, -23,
+              "CREATE %d carries no shape", n.result_name);
+    int32_t shape[3] = {1, 1, 1};
+    for (int d = 0; d < n.ndims; ++d)
+        shape[d] = region_count(n.region, d);
+    return make_array(ex, n.result_name, n.ndims, n.dtype, shape, true, nullptr);
+}
+
+// SET_REGION with a scalar value: one strided fill per tile the region touches
+// (src/executor_ast_visitor.cpp:112-147).
+int exec_fill(Ex* ex, XArray& a, const cnh_region& reg, double value) {
+    cnh_region r = reg;
+    if (r.is_global) {
+        r.ndims = a.ndims;
+        for (int d = 0; d < a.ndims; ++d) {
+            r.start[d] = 0;
+            r.stop[d] = a.shape[d];
+            r.step[d] = 1;
+        }
+    }
+    CNH_CHECK(r.ndims == a.ndims, -24, "fill of array %d: region rank %d, array rank %d", a.name,
+              r.ndims, a.ndims);
+    for (int d = 0; d < a.ndims; ++d)
+        CNH_CHECK(r.step[d] >= 1 && r.start[d] >= 0 && r.stop[d] <= a.shape[d], -24,
+                  "fill of array %d: region [%d:%d:%d] leaves extent %d in dim %d", a.name,
+                  r.start[d], r.stop[d], r.step[d], a.shape[d], d);
+    unsigned char s8[8];
+    if (int rc = cnh_scalar_to_dtype(a.dtype, value, s8))
+        return rc;
+    const int esz = dtype_size(a.dtype);
+    int launches = 0;
+    for (int64_t t = 0; t < a.ntiles; ++t) {
+        int32_t lo[3], ext[3];
+        a.tile_extent(t, lo, ext);
+        int64_t start[3], step[3], counts[3], strides[3];
+        bool empty = false;
+        int64_t stride = 1;
+        for (int d = a.ndims - 1; d >= 0; --d) {
+            strides[d] = stride;
+            stride *= ext[d];
+        }
+        for (int d = 0; d < a.ndims; ++d) {
+            int64_t first = r.start[d];
+            if (first < lo[d])
+                first += ((lo[d] - first + r.step[d] - 1) / r.step[d]) * (int64_t)r.step[d];
+            int64_t last_excl = std::min<int64_t>(r.stop[d], lo[d] + ext[d]);
+            if (first >= last_excl) {
+                empty = true;
+                break;
+            }
+            start[d] = first - lo[d];
+            step[d] = r.step[d];
+            counts[d] = (last_excl - first + r.step[d] - 1) / r.step[d];
+        }
+        if (empty)
+            continue;
+        ++launches;
+        if (!ex->dry)
+            if (int rc = cnh_fill_region(a.ndims, esz, a.tiles[t], strides, start, step, counts, s8,
+                                         ex->stream))
+                return rc;
+    }
+    ex->log("fill " + std::to_string(a.name) + " tiles_touched=" + std::to_string(launches));
+    return 0;
+}
+
+struct Group {
+    std::vector<cnh_ast_node> nodes; // canonical names
+    std::vector<int32_t> roots;
+    std::map<int, int> canon_to_actual;
+    int dtype = CNH_F64;
+    int ndims = 1;
+    uint64_t key = 0;
+};
+
+// Renames arrays, temporaries and literals by first appearance so that structurally identical
+// groups (every CG iteration, every sweep) share one compiled kernel whatever their array names.
+void canonicalise(const DagNode& n, Group& g) {
+    g.nodes = n.nodes;
+    g.roots = n.roots;
+    std::map<int, int> to_canon;
+    int next = 1;
+    for (auto& a : g.nodes) {
+        auto it = to_canon.find(a.result_name);
+        if (it == to_canon.end()) {
+            it = to_canon.emplace(a.result_name, next++).first;
+            g.canon_to_actual[it->second] = a.result_name;
+        }
+        a.result_name = a.is_scalar ? -it->second : it->second;
+    }
+    // Element type of the kernel: the first root that is not F32 decides (src/jit.cpp:50-69).
+    g.dtype = CNH_F32;
+    for (int32_t r : g.roots)
+        if (g.nodes[r].dtype != CNH_F32) {
+            g.dtype = g.nodes[r].dtype;
+            break;
+        }
+    g.ndims = g.nodes[g.roots.back()].ndims;
+    uint64_t h = fnv(&g.dtype, sizeof g.dtype);
+    h = fnv(&g.ndims, sizeof g.ndims, h);
+    for (auto& a : g.nodes) {
+        // hash field by field: the struct has padding
+        int32_t head[10] = {a.result_name, a.opcode, a.is_temp, a.is_scalar, a.is_broadcast,
+                            a.ndims, a.dtype, a.n_operands, a.operands[0], a.operands[1]};
+        h = fnv(head, sizeof head, h);
+        h = fnv(&a.scalar, sizeof a.scalar, h);
+        h = fnv(a.has_operand_region, sizeof a.has_operand_region, h);
+        h = fnv(&a.operand_regions[0], sizeof(cnh_region), h);
+        h = fnv(&a.operand_regions[1], sizeof(cnh_region), h);
+        h = fnv(&a.region, sizeof(cnh_region), h);
+    }
+    h = fnv(g.roots.data(), g.roots.size() * sizeof(int32_t), h);
+    g.key = h;
+}
+
+int compile_cached(Ex* ex, Group& g, cnh_kernel** out) {
+    auto it = ex->kernels.find(g.key);
+    if (it != ex->kernels.end()) {
+        ex->stats[1]++;
+        *out = it->second;
+        return 0;
+    }
+    cnh_ast ast{(int32_t)g.nodes.size(), (int32_t)g.roots.size(), g.nodes.data(), g.roots.data()};
+    cnh_kernel* k = nullptr;
+    if (int rc = cnh_compile_group(&ast, g.dtype, g.ndims, g.key, &k))
+        return rc;
+    ex->stats[0]++;
+    ex->kernels[g.key] = k;
+    *out = k;
+    return 0;
+}
+
+// Shape of a new elementwise result: the root's own region when the message carries one, else the
+// shape of an operand region, else the shape of a non-broadcast operand array
+// (src/dag_group_receive.cpp:65-106).
+int result_shape(Ex* ex, const DagNode& n, const cnh_ast_node& root, int32_t shape[3]) {
+    shape[0] = shape[1] = shape[2] = 1;
+    if (!root.region.is_global && root.region.ndims == root.ndims) {
+        for (int d = 0; d < root.ndims; ++d)
+            shape[d] = region_count(root.region, d);
+        return 0;
+    }
+    bool found = false;
+    for (const auto& a : n.nodes) {
+        if (a.is_scalar || a.opcode == CNH_OP_NOOP)
+            continue;
+        for (int i = 0; i < a.n_operands; ++i) {
+            const cnh_ast_node& op = n.nodes[a.operands[i]];
+            if (op.is_scalar || op.opcode != CNH_OP_NOOP)
+                continue;
+            if (a.has_operand_region[i] && !a.operand_regions[i].is_global) {
+                for (int d = 0; d < op.ndims; ++d)
+                    shape[d] = region_count(a.operand_regions[i], d);
+                return 0;
+            }
+            auto it = ex->arrays.find(op.result_name);
+            if (it == ex->arrays.end())
+                continue;
+            if (!found || !op.is_broadcast) {
+                for (int d = 0; d < 3; ++d)
+                    shape[d] = d < it->second.ndims ? it->second.shape[d] : 1;
+                found = true;
+                if (!op.is_broadcast)
+                    return 0;
+            }
+        }
+    }
+    CNH_CHECK(found, -25, "cannot infer the shape of result %d", root.result_name);
+    return 0;
+}
+
+int exec_group(Ex* ex, const DagNode& n) {
+    const cnh_ast_node& root = n.nodes[n.roots.back()];
+    for (size_t i = 0; i + 1 < n.roots.size(); ++i)
+        CNH_CHECK(n.nodes[n.roots[i]].is_temp, -26,
+                  "node %d: only the last root of a group may be a result", n.id);
+
+    // SET_REGION with a literal: fill.
+    if (root.opcode == CNH_OP_SET_REGION && root.n_operands == 2 &&
+        n.nodes[root.operands[1]].is_scalar) {
+        XArray* target;
+        if (int rc = find_array(ex, n.nodes[root.operands[0]].result_name, &target, "SET_REGION"))
+            return rc;
+        return exec_fill(ex, *target, root.region, n.nodes[root.operands[1]].scalar);
+    }
+
+    Group g;
+    canonicalise(n, g);
+    cnh_kernel* k = nullptr;
+    if (int rc = compile_cached(ex, g, &k))
+        return rc;
+    int n_in = 0, n_scalar = 0, n_out = 0;
+    if (int rc = cnh_kernel_signature(k, &n_in, &n_scalar, &n_out))
+        return rc;
+    CNH_CHECK(n_out == 1, -26, "node %d: %d outputs (one expected)", n.id, n_out);
+
+    // Bind arguments by name.
+    std::vector<XArray*> in_arr(n_in);
+    std::vector<cnh_region> in_reg(n_in);
+    std::vector<int> in_has_reg(n_in);
+    for (int i = 0; i < n_in; ++i) {
+        int cname = 0;
+        if (int rc = cnh_kernel_input(k, i, &cname, &in_has_reg[i], &in_reg[i]))
+            return rc;
+        if (int rc = find_array(ex, g.canon_to_actual[cname], &in_arr[i], "group input"))
+            return rc;
+        CNH_CHECK(in_arr[i]->dtype == g.dtype, -27,
+                  "node %d: input array %d has dtype %d, the group computes in dtype %d", n.id,
+                  in_arr[i]->name, in_arr[i]->dtype, g.dtype);
+    }
+    std::vector<const void*> scalars(n_scalar ? n_scalar : 1, nullptr);
+    for (int i = 0; i < n_scalar; ++i) {
+        int cname = 0;
+        if (int rc = cnh_kernel_scalar(k, i, &cname))
+            return rc;
+        XArray* s;
+        if (int rc = find_array(ex, g.canon_to_actual[cname], &s, "broadcast scalar"))
+            return rc;
+        CNH_CHECK(s->elems == 1, -27, "node %d: broadcast operand %d has %lld elements", n.id,
+                  s->name, (long long)s->elems);
+        CNH_CHECK(s->dtype == g.dtype, -27, "node %d: broadcast operand %d has dtype %d, group %d",
+                  n.id, s->name, s->dtype, g.dtype);
+        scalars[i] = s->tiles[0];
+    }
+
+    const bool is_set = root.opcode == CNH_OP_SET_REGION;
+    XArray* target = nullptr;
+    if (is_set) {
+        if (int rc = find_array(ex, n.nodes[root.operands[0]].result_name, &target, "SET_REGION"))
+            return rc;
+        CNH_CHECK(target->dtype == g.dtype, -27, "node %d: target dtype %d, group dtype %d", n.id,
+                  target->dtype, g.dtype);
+    } else {
+        int32_t shape[3];
+        if (int rc = result_shape(ex, n, root, shape))
+            return rc;
+        if (int rc = make_array(ex, root.result_name, root.ndims, g.dtype, shape, false, &target))
+            return rc;
+        // make_array may rehash nothing (std::map), input pointers stay valid.
+    }
+
+    // Dense path: no shifted or strided operand, everything on one decomposition
+    // (the no-region fast path, src/execute_node.cpp:1263-1336).
+    bool dense = !is_set || region_is_whole(root.region, *target);
+    for (int i = 0; i < n_in && dense; ++i) {
+        if (in_has_reg[i] && !region_is_whole(in_reg[i], *in_arr[i]))
+            dense = false;
+        if (!same_decomposition(*in_arr[i], *target))
+            dense = false;
+    }
+    ex->stats[5]++;
+    if (dense) {
+        const int nd = target->ndims;
+        const int64_t parts = target->ntiles;
+        std::vector<cnh_memref> in(std::max<size_t>(1, (size_t)parts * n_in)), out((size_t)parts);
+        for (int64_t t = 0; t < parts; ++t) {
+            int32_t lo[3], ext[3];
+            target->tile_extent(t, lo, ext);
+            auto fill = [&](cnh_memref& m, void* ptr) {
+                std::memset(&m, 0, sizeof m);
+                m.allocated = m.aligned = ptr;
+                int64_t stride = 1;
+                for (int d = nd - 1; d >= 0; --d) {
+                    m.sizes[d] = ext[d];
+                    m.strides[d] = stride;
+                    stride *= ext[d];
+                }
+            };
+            for (int i = 0; i < n_in; ++i)
+                fill(in[(size_t)t * n_in + i], in_arr[i]->tiles[t]);
+            fill(out[(size_t)t], target->tiles[t]);
+        }
+        ex->log("group node=" + std::to_string(n.id) + " path=dense parts=" + std::to_string(parts) +
+                " inputs=" + std::to_string(n_in) + " scalars=" + std::to_string(n_scalar) +
+                " out=" + std::to_string(target->name));
+        if (ex->dry)
+            return 0;
+        return cnh_launch_group_batched(k, nd, (int)parts, n_in, in.data(), n_scalar, scalars.data(),
+                                        1, 1, out.data(), ex->stream);
+    }
+
+    // Shifted / strided operands or mixed decompositions: one launch over the target's tiles that
+    // reads whatever tiles the operand regions fall into (replaces the fragment path and its halo
+    // messages, src/execute_node.cpp:1338-1585, src/executor_core.cpp:8-143).
+    bool aliased = false;
+    if (is_set)
+        for (int i = 0; i < n_in; ++i)
+            if (in_arr[i] == target) {
+                cnh_region whole;
+                std::memset(&whole, 0, sizeof whole);
+                whole.is_global = 1;
+                const cnh_region& ir = in_has_reg[i] ? in_reg[i] : whole;
+                bool same = same_region(ir, root.region) ||
+                            (region_is_whole(ir, *target) && region_is_whole(root.region, *target));
+                if (!same)
+                    aliased = true;
+            }
+    if (aliased)
+        if (int rc = ensure_alt(ex, *target))
+            return rc;
+    std::vector<cnh_tiled> tin(std::max(1, n_in));
+    for (int i = 0; i < n_in; ++i)
+        tin[i] = in_arr[i]->tiled();
+    cnh_tiled cur = target->tiled(false);
+    cnh_tiled dst = aliased ? target->tiled(true) : cur;
+    ex->log("group node=" + std::to_string(n.id) + " path=tiles inputs=" + std::to_string(n_in) +
+            " scalars=" + std::to_string(n_scalar) + " out=" + std::to_string(target->name) +
+            (aliased ? " pingpong" : " inplace"));
+    if (!ex->dry)
+        if (int rc = cnh_launch_group_tiles(k, n_in, tin.data(), n_scalar, scalars.data(), 1,
+                                            is_set ? &cur : nullptr, &dst, ex->stream))
+            return rc;
+    if (aliased) {
+        std::swap(target->slab, target->alt);
+        std::swap(target->tiles, target->alt_tiles);
+    }
+    return 0;
+}
+
+int leaf_array(Ex* ex, const DagNode& n, const cnh_ast_node& root, int i, XArray** out,
+               const char* what) {
+    CNH_CHECK(root.n_operands > i, -28, "%s: operand %d missing", what, i);
+    const cnh_ast_node& op = n.nodes[root.operands[i]];
+    CNH_CHECK(!op.is_scalar && op.opcode == CNH_OP_NOOP, -28, "%s: operand %d is not an array", what, i);
+    if (int rc = find_array(ex, op.result_name, out, what))
+        return rc;
+    CNH_CHECK(!root.has_operand_region[i] || region_is_whole(root.operand_regions[i], **out), -29,
+              "%s on a slice of array %d is not supported", what, op.result_name);
+    return 0;
+}
+
+int new_scalar_array(Ex* ex, int name, int dtype, XArray** out) {
+    int32_t one[3] = {1, 1, 1};
+    return make_array(ex, name, 1, dtype, one, false, out);
+}
+
+// REDUCE: per-tile dots and their in-order sum, result = size-1 array
+// (src/executor_reduce.cpp:8-119, src/executor_reducer.cpp:11-57, src/partition_comm.cpp:69-111).
+int exec_reduce(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
+    XArray *a, *b;
+    if (int rc = leaf_array(ex, n, root, 0, &a, "REDUCE"))
+        return rc;
+    if (int rc = leaf_array(ex, n, root, 1, &b, "REDUCE"))
+        return rc;
+    CNH_CHECK(a->ndims == 1 && b->ndims == 1, -30, "REDUCE needs 1-D operands");
+    CNH_CHECK(a->shape[0] == b->shape[0], -30, "REDUCE: lengths %d and %d", a->shape[0], b->shape[0]);
+    CNH_CHECK(a->dtype == b->dtype, -27, "REDUCE: operand dtypes %d and %d", a->dtype, b->dtype);
+    XArray* out;
+    if (int rc = new_scalar_array(ex, root.result_name, a->dtype, &out))
+        return rc;
+    // make_array inserted into the map: re-find the operands (std::map keeps references valid).
+    ex->log("reduce " + std::to_string(a->name) + "." + std::to_string(b->name) + " tiles=" +
+            std::to_string(a->ntiles) + " out=" + std::to_string(out->name));
+    if (ex->dry)
+        return 0;
+    std::vector<const void*> pa(a->tiles.begin(), a->tiles.end()), pb(b->tiles.begin(), b->tiles.end());
+    return cnh_dot_tiles(a->dtype, (int)a->ntiles, pa.data(), pb.data(), a->tile_elems.data(),
+                         out->tiles[0], ex->stream);
+}
+
+int exec_reduce_ext(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
+    XArray *a, *b = nullptr;
+    if (int rc = leaf_array(ex, n, root, 0, &a, "reduction"))
+        return rc;
+    if (root.opcode != kOpSum) {
+        if (int rc = leaf_array(ex, n, root, 1, &b, "reduction"))
+            return rc;
+        CNH_CHECK(same_decomposition(*a, *b), -30, "reduction: operands differ in shape");
+        CNH_CHECK(a->dtype == CNH_F64 && b->dtype == CNH_F64, -27, "reduction: fp64 operands needed");
+    }
+    XArray* out;
+    if (int rc = new_scalar_array(ex, root.result_name, a->dtype, &out))
+        return rc;
+    ex->log("reduce_ext op=" + std::to_string(root.opcode) + " tiles=" + std::to_string(a->ntiles) +
+            " out=" + std::to_string(out->name));
+    if (ex->dry)
+        return 0;
+    std::vector<const void*> pa(a->tiles.begin(), a->tiles.end()), pb;
+    if (b)
+        pb.assign(b->tiles.begin(), b->tiles.end());
+    if (root.opcode == kOpSum)
+        return cnh_sum_tiles(a->dtype, (int)a->ntiles, pa.data(), a->tile_elems.data(), out->tiles[0],
+                             ex->stream);
+    if (root.opcode == kOpSumsqDiff)
+        return cnh_sumsq_diff_tiles((int)a->ntiles, pa.data(), pb.data(), a->tile_elems.data(),
+                                    out->tiles[0], ex->stream);
+    return cnh_maxabs_diff_tiles((int)a->ntiles, pa.data(), pb.data(), a->tile_elems.data(),
+                                 out->tiles[0], ex->stream);
+}
+
+// MATMUL: tile GEMVs, column tiles summed in index order (src/executor_matmul.cpp:150-498,
+// src/execute_node.cpp:116-273,489-583).
+int exec_matmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
+    XArray *A, *x;
+    if (int rc = leaf_array(ex, n, root, 0, &A, "MATMUL"))
+        return rc;
+    if (int rc = leaf_array(ex, n, root, 1, &x, "MATMUL"))
+        return rc;
+    CNH_CHECK(A->ndims == 2 && x->ndims == 1, -31, "MATMUL needs a 2-D and a 1-D operand");
+    CNH_CHECK(A->shape[1] == x->shape[0], -31, "MATMUL: %d columns, vector of %d", A->shape[1],
+              x->shape[0]);
+    CNH_CHECK(A->dtype == x->dtype, -27, "MATMUL: operand dtypes %d and %d", A->dtype, x->dtype);
+    int32_t shape[3] = {A->shape[0], 1, 1};
+    XArray* y;
+    if (int rc = make_array(ex, root.result_name, 1, A->dtype, shape, false, &y))
+        return rc;
+    ex->log("matmul A=" + std::to_string(A->name) + " tiles=" + std::to_string(A->ntiles) + " x=" +
+            std::to_string(x->name) + " out=" + std::to_string(y->name));
+    if (ex->dry)
+        return 0;
+    std::vector<const void*> pt(A->tiles.begin(), A->tiles.end());
+    // 1-D arrays are contiguous: tile 0 is the whole vector.
+    return cnh_gemv_tiles(A->dtype, A->shape[0], A->shape[1], A->tile, pt.data(), x->tiles[0],
+                          y->tiles[0], ex->stream);
+}
+
+// MATMATMUL: C (zeroed) += A_panel * B_panel for every k-overlapping pair of tiles, k ascending
+// (src/executor_matmatmul.cpp:105-484, src/executor_incremental.cpp:97-132).
+int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
+    XArray *A, *B;
+    if (int rc = leaf_array(ex, n, root, 0, &A, "MATMATMUL"))
+        return rc;
+    if (int rc = leaf_array(ex, n, root, 1, &B, "MATMATMUL"))
+        return rc;
+    CNH_CHECK(A->ndims == 2 && B->ndims == 2, -32, "MATMATMUL needs 2-D operands");
+    CNH_CHECK(A->shape[1] == B->shape[0], -32, "MATMATMUL: (%d,%d) @ (%d,%d)", A->shape[0],
+              A->shape[1], B->shape[0], B->shape[1]);
+    CNH_CHECK(A->dtype == B->dtype, -27, "MATMATMUL: operand dtypes %d and %d", A->dtype, B->dtype);
+    int32_t shape[3] = {A->shape[0], B->shape[1], 1};
+    XArray* Cc;
+    if (int rc = make_array(ex, root.result_name, 2, A->dtype, shape, true, &Cc))
+        return rc;
+    const int esz = dtype_size(A->dtype);
+    int calls = 0;
+    for (int ci = 0; ci < Cc->grid[0]; ++ci)
+        for (int cj = 0; cj < Cc->grid[1]; ++cj) {
+            int32_t clo[3], cext[3];
+            Cc->tile_extent((int64_t)ci * Cc->grid[1] + cj, clo, cext);
+            // rows of this C tile fall into A row tiles, its columns into B column tiles
+            for (int ai = clo[0] / A->tile; ai <= (clo[0] + cext[0] - 1) / A->tile; ++ai)
+                for (int bj = clo[1] / B->tile; bj <= (clo[1] + cext[1] - 1) / B->tile; ++bj) {
+                    int r0 = std::max(clo[0], ai * A->tile);
+                    int r1 = std::min(clo[0] + cext[0], std::min((ai + 1) * A->tile, (int)A->shape[0]));
+                    int c0 = std::max(clo[1], bj * B->tile);
+                    int c1 = std::min(clo[1] + cext[1], std::min((bj + 1) * B->tile, (int)B->shape[1]));
+                    // k pieces: common refinement of A's column tiles and B's row tiles
+                    int k0 = 0;
+                    const int K = A->shape[1];
+                    while (k0 < K) {
+                        int ak = k0 / A->tile, bk = k0 / B->tile;
+                        int k1 = std::min(K, std::min((ak + 1) * A->tile, (bk + 1) * B->tile));
+                        int32_t alo[3], aext[3], blo[3], bext[3];
+                        A->tile_extent((int64_t)ai * A->grid[1] + ak, alo, aext);
+                        B->tile_extent((int64_t)bk * B->grid[1] + bj, blo, bext);
+                        const char* ap = static_cast<const char*>(A->tiles[(size_t)ai * A->grid[1] + ak]) +
+                                         ((int64_t)(r0 - alo[0]) * aext[1] + (k0 - alo[1])) * esz;
+                        const char* bp = static_cast<const char*>(B->tiles[(size_t)bk * B->grid[1] + bj]) +
+                                         ((int64_t)(k0 - blo[0]) * bext[1] + (c0 - blo[1])) * esz;
+                        char* cp = static_cast<char*>(Cc->tiles[(size_t)ci * Cc->grid[1] + cj]) +
+                                   ((int64_t)(r0 - clo[0]) * cext[1] + (c0 - clo[1])) * esz;
+                        ++calls;
+                        if (!ex->dry)
+                            if (int rc = cnh_gemm_acc(A->dtype, r1 - r0, c1 - c0, k1 - k0, ap, aext[1],
+                                                      bp, bext[1], cp, cext[1], ex->stream))
+                                return rc;
+                        k0 = k1;
+                    }
+                }
+        }
+    ex->log("matmatmul A=" + std::to_string(A->name) + " B=" + std::to_string(B->name) + " out=" +
+            std::to_string(Cc->name) + " panel_products=" + std::to_string(calls));
+    return 0;
+}
+
+int exec_node(Ex* ex, const DagNode& n) {
+    CNH_CHECK(!n.roots.empty(), -33, "DAG node %d has no roots", n.id);
+    const cnh_ast_node& root = n.nodes[n.roots.back()];
+    ex->stats[2]++;
+    switch (root.opcode) {
+    case CNH_OP_CREATE: return exec_create(ex, root);
+    case kOpDelete: drop_array(ex, root.result_name); return 0;
+    case CNH_OP_REDUCE: return exec_reduce(ex, n, root);
+    case kOpSum:
+    case kOpSumsqDiff:
+    case kOpMaxabsDiff: return exec_reduce_ext(ex, n, root);
+    case CNH_OP_MATMUL: return exec_matmul(ex, n, root);
+    case CNH_OP_MATMATMUL: return exec_matmatmul(ex, n, root);
+    case CNH_OP_ADD:
+    case CNH_OP_SUB:
+    case CNH_OP_MUL:
+    case CNH_OP_DIV:
+    case CNH_OP_TANH:
+    case CNH_OP_EXP:
+    case CNH_OP_COPY:
+    case CNH_OP_SET_REGION: return exec_group(ex, n);
+    case CNH_OP_NOOP: return 0;
+    default:
+        return set_error(-34, "DAG node %d: opcode %d is not supported by this executor", n.id,
+                         root.opcode);
+    }
+}
+
+int parse_dag(const char* msg, int64_t size, std::vector<DagNode>& out) {
+    Reader r{msg, msg + size};
+    int32_t magic = r.get<int32_t>(), version = r.get<int32_t>(), count = r.get<int32_t>();
+    CNH_CHECK(r.ok && magic == CNX_DAG_MAGIC, -40, "not a DAG message (bad magic)");
+    CNH_CHECK(version == 1, -40, "DAG message version %d (1 expected)", version);
+    CNH_CHECK(count >= 0 && count <= (1 << 24), -40, "DAG message: %d nodes", count);
+    out.resize((size_t)count);
+    for (auto& n : out) {
+        n.id = r.get<int32_t>();
+        n.fusible = r.get<int32_t>();
+        int32_t na = r.get<int32_t>(), nr = r.get<int32_t>();
+        CNH_CHECK(r.ok && na >= 1 && na <= (1 << 20) && nr >= 1 && nr <= na, -41,
+                  "DAG node %d: %d AST nodes, %d roots", n.id, na, nr);
+        n.nodes.resize((size_t)na);
+        for (int i = 0; i < na; ++i) {
+            cnh_ast_node& a = n.nodes[i];
+            std::memset(&a, 0, sizeof a);
+            a.result_name = r.get<int32_t>();
+            a.opcode = r.get<int32_t>();
+            a.is_temp = r.get<int32_t>();
+            a.is_scalar = r.get<int32_t>();
+            a.is_broadcast = r.get<int32_t>();
+            a.ndims = r.get<int32_t>();
+            a.dtype = r.get<int32_t>();
+            a.n_operands = r.get<int32_t>();
+            CNH_CHECK(r.ok && a.n_operands >= 0 && a.n_operands <= 2, -41,
+                      "DAG node %d: AST node %d has %d operands", n.id, i, a.n_operands);
+            for (int j = 0; j < a.n_operands; ++j) {
+                a.operands[j] = r.get<int32_t>();
+                CNH_CHECK(r.ok && a.operands[j] >= 0 && a.operands[j] < i, -41,
+                          "DAG node %d: AST node %d refers to node %d", n.id, i, a.operands[j]);
+            }
+            a.scalar = r.get<double>();
+            for (int j = 0; j < a.n_operands; ++j) {
+                CNH_CHECK(read_region(r, a.operand_regions[j]), -41, "DAG node %d: bad region", n.id);
+                a.has_operand_region[j] = a.operand_regions[j].is_global ? 0 : 1;
+            }
+            CNH_CHECK(read_region(r, a.region), -41, "DAG node %d: bad region", n.id);
+            CNH_CHECK(a.ndims >= 0 && a.ndims <= 3, -41, "DAG node %d: rank %d", n.id, a.ndims);
+        }
+        n.roots.resize((size_t)nr);
+        for (auto& x : n.roots) {
+            x = r.get<int32_t>();
+            CNH_CHECK(r.ok && x >= 0 && x < na, -41, "DAG node %d: root index out of range", n.id);
+        }
+    }
+    CNH_CHECK(r.ok, -42, "DAG message truncated");
+    CNH_CHECK(r.p == r.end, -42, "DAG message has %lld trailing bytes", (long long)(r.end - r.p));
+    return 0;
+}
+
+} // namespace
+
+extern "C" {
+
+int cnx_create(int device, int num_pes, int odf, cnx_executor** out) {
+    CNH_CHECK(out != nullptr, -2, "null argument");
+    CNH_CHECK(num_pes >= 1 && odf >= 1, -2, "num_pes and odf must be positive");
+    auto ex = std::make_unique<cnx_executor>();
+    ex->dry = device < 0;
+    ex->num_pes = num_pes;
+    ex->odf = odf;
+    if (!ex->dry) {
+        if (int rc = cnh_init(device))
+            return rc;
+        if (int rc = cnh_stream_create(&ex->stream))
+            return rc;
+    }
+    *out = ex.release();
+    return 0;
+}
+
+int cnx_destroy(cnx_executor* ex) {
+    if (!ex)
+        return 0;
+    if (!ex->dry) {
+        cnh_stream_sync(ex->stream);
+        for (auto& kv : ex->arrays) {
+            cnh_free(kv.second.slab);
+            if (kv.second.alt)
+                cnh_free(kv.second.alt);
+        }
+        for (auto& kv : ex->free_list)
+            for (void* p : kv.second)
+                cnh_free(p);
+        cnh_stream_destroy(ex->stream);
+    }
+    // Kernels stay in the library-wide cache (keyed by content), as upstream's compile_cache does
+    // for the life of the process.
+    delete ex;
+    return 0;
+}
+
+int cnx_set_min_tile(cnx_executor* ex, int ndims, int min_tile) {
+    CNH_CHECK(ex != nullptr, -2, "null executor");
+    CNH_CHECK(ndims >= 1 && ndims <= 3 && min_tile >= 1, -2, "bad minimum tile %d for rank %d",
+              min_tile, ndims);
+    ex->min_tile[ndims] = min_tile;
+    return 0;
+}
+
+int cnx_set_trace(cnx_executor* ex, int on) {
+    CNH_CHECK(ex != nullptr, -2, "null executor");
+    ex->trace_on = on != 0;
+    return 0;
+}
+
+int64_t cnx_trace(cnx_executor* ex, char* buf, size_t cap) {
+    CNH_CHECK(ex != nullptr, -2, "null executor");
+    int64_t need = (int64_t)ex->trace.size() + 1;
+    if (buf && cap >= (size_t)need) {
+        std::memcpy(buf, ex->trace.c_str(), (size_t)need);
+        ex->trace.clear();
+    }
+    return need;
+}
+
+int cnx_receive_dag(cnx_executor* ex, int epoch, int64_t size, const char* msg) {
+    (void)epoch;
+    CNH_CHECK(ex != nullptr && msg != nullptr && size >= 12, -2, "bad DAG message");
+    std::vector<DagNode> dag;
+    if (int rc = parse_dag(msg, size, dag))
+        return rc;
+    for (const DagNode& n : dag)
+        if (int rc = exec_node(ex, n))
+            return rc;
+    return 0;
+}
+
+int cnx_get(cnx_executor* ex, int ndims, int epoch, int name, int64_t size, int dtype, void* host_out) {
+    (void)epoch;
+    CNH_CHECK(ex != nullptr && host_out != nullptr, -2, "null argument");
+    XArray* a;
+    if (int rc = find_array(ex, name, &a, "get"))
+        return rc;
+    CNH_CHECK(a->ndims == ndims && a->dtype == dtype && a->elems == size, -50,
+              "get of array %d: asked for rank %d dtype %d size %lld, array has rank %d dtype %d size %lld",
+              name, ndims, dtype, (long long)size, a->ndims, a->dtype, (long long)a->elems);
+    ex->log("get " + std::to_string(name) + " tiles=" + std::to_string(a->ntiles));
+    if (ex->dry) {
+        std::memset(host_out, 0, (size_t)size * dtype_size(dtype));
+        return 0;
+    }
+    const int esz = dtype_size(dtype);
+    int64_t gstr[3] = {1, 1, 1};
+    {
+        int64_t s = 1;
+        for (int d = ndims - 1; d >= 0; --d) {
+            gstr[d] = s;
+            s *= a->shape[d];
+        }
+    }
+    for (int64_t t = 0; t < a->ntiles; ++t) {
+        int32_t lo[3], ext[3];
+        a->tile_extent(t, lo, ext);
+        int64_t dstart[3], sstart[3] = {0, 0, 0}, counts[3], sstr[3];
+        int64_t s = 1;
+        for (int d = ndims - 1; d >= 0; --d) {
+            sstr[d] = s;
+            s *= ext[d];
+        }
+        for (int d = 0; d < ndims; ++d) {
+            dstart[d] = lo[d];
+            counts[d] = ext[d];
+        }
+        if (int rc = cnh_d2h_region(ndims, esz, host_out, gstr, dstart, a->tiles[t], sstr, sstart, counts,
+                                    ex->stream))
+            return rc;
+    }
+    return cnh_stream_sync(ex->stream);
+}
+
+int cnx_put(cnx_executor* ex, int name, int64_t size, int dtype, const void* host_in) {
+    CNH_CHECK(ex != nullptr && host_in != nullptr, -2, "null argument");
+    XArray* a;
+    if (int rc = find_array(ex, name, &a, "put"))
+        return rc;
+    CNH_CHECK(a->dtype == dtype && a->elems == size, -50,
+              "put into array %d: %lld elements of dtype %d offered, array has %lld of dtype %d", name,
+              (long long)size, dtype, (long long)a->elems, a->dtype);
+    ex->log("put " + std::to_string(name));
+    if (ex->dry)
+        return 0;
+    const int esz = dtype_size(dtype);
+    const int nd = a->ndims;
+    std::vector<char> stage;
+    for (int64_t t = 0; t < a->ntiles; ++t) {
+        int32_t lo[3], ext[3];
+        a->tile_extent(t, lo, ext);
+        const char* src = static_cast<const char*>(host_in);
+        if (a->ntiles == 1) {
+            if (int rc = cnh_h2d(a->tiles[0], src, (size_t)a->elems * esz, ex->stream))
+                return rc;
+            break;
+        }
+        stage.resize((size_t)a->tile_elems[t] * esz);
+        // rows of the innermost dimension are contiguous on both sides
+        int32_t e0 = nd >= 3 ? ext[0] : 1, e1 = nd >= 2 ? ext[nd - 2] : 1, e2 = ext[nd - 1];
+        int64_t g2 = 1, g1 = a->shape[nd - 1], g0 = nd >= 2 ? (int64_t)a->shape[nd - 1] * a->shape[nd - 2] : 0;
+        int32_t l0 = nd >= 3 ? lo[0] : 0, l1 = nd >= 2 ? lo[nd - 2] : 0, l2 = lo[nd - 1];
+        (void)g2;
+        size_t w = 0;
+        for (int i = 0; i < e0; ++i)
+            for (int j = 0; j < e1; ++j) {
+                const char* row = src + ((int64_t)(l0 + i) * g0 + (int64_t)(l1 + j) * g1 + l2) * esz;
+                std::memcpy(stage.data() + w, row, (size_t)e2 * esz);
+                w += (size_t)e2 * esz;
+            }
+        if (int rc = cnh_h2d(a->tiles[t], stage.data(), stage.size(), ex->stream))
+            return rc;
+    }
+    return 0;
+}
+
+int cnx_fill_uniform(cnx_executor* ex, int name, uint64_t seed, uint64_t stream_id, double lo, double hi) {
+    CNH_CHECK(ex != nullptr, -2, "null executor");
+    XArray* a;
+    if (int rc = find_array(ex, name, &a, "fill_uniform"))
+        return rc;
+    CNH_CHECK(a->dtype == CNH_F64, -27, "fill_uniform needs an fp64 array");
+    ex->log("fill_uniform " + std::to_string(name));
+    if (ex->dry)
+        return 0;
+    int64_t gshape[3];
+    for (int d = 0; d < 3; ++d)
+        gshape[d] = a->shape[d];
+    for (int64_t t = 0; t < a->ntiles; ++t) {
+        int32_t lo3[3], ext[3];
+        a->tile_extent(t, lo3, ext);
+        int64_t e[3], o[3];
+        for (int d = 0; d < 3; ++d) {
+            e[d] = ext[d];
+            o[d] = lo3[d];
+        }
+        if (int rc = cnh_fill_uniform_tile(static_cast<double*>(a->tiles[t]), a->ndims, e, o, gshape, seed,
+                                           stream_id, lo, hi, ex->stream))
+            return rc;
+    }
+    return 0;
+}
+
+int cnx_fill_cg_matrix(cnx_executor* ex, int name, uint64_t seed) {
+    CNH_CHECK(ex != nullptr, -2, "null executor");
+    XArray* a;
+    if (int rc = find_array(ex, name, &a, "fill_cg_matrix"))
+        return rc;
+    CNH_CHECK(a->dtype == CNH_F64 && a->ndims == 2 && a->shape[0] == a->shape[1], -27,
+              "fill_cg_matrix needs a square fp64 array");
+    ex->log("fill_cg_matrix " + std::to_string(name));
+    if (ex->dry)
+        return 0;
+    for (int64_t t = 0; t < a->ntiles; ++t) {
+        int32_t lo[3], ext[3];
+        a->tile_extent(t, lo, ext);
+        if (int rc = cnh_fill_cg_matrix(static_cast<double*>(a->tiles[t]), a->shape[0], lo[0], ext[0], lo[1],
+                                        ext[1], ext[1], seed, ex->stream))
+            return rc;
+    }
+    return 0;
+}
+
+int cnx_sync(cnx_executor* ex) {
+    CNH_CHECK(ex != nullptr, -2, "null executor");
+    if (ex->dry)
+        return 0;
+    return cnh_stream_sync(ex->stream);
+}
+
+int cnx_array_info(cnx_executor* ex, int name, int* ndims, int* dtype, int* tile, int32_t* shape3,
+                   int32_t* offset3) {
+    CNH_CHECK(ex != nullptr, -2, "null executor");
+    XArray* a;
+    if (int rc = find_array(ex, name, &a, "array_info"))
+        return rc;
+    if (ndims)
+        *ndims = a->ndims;
+    if (dtype)
+        *dtype = a->dtype;
+    if (tile)
+        *tile = a->tile;
+    for (int d = 0; d < 3; ++d) {
+        if (shape3)
+            shape3[d] = a->shape[d];
+        if (offset3)
+            offset3[d] = a->offset[d];
+    }
+    return 0;
+}
+
+int cnx_stats(cnx_executor* ex, int64_t out[8]) {
+    CNH_CHECK(ex != nullptr && out != nullptr, -2, "null argument");
+    ex->stats[6] = (int64_t)ex->arrays.size();
+    for (int i = 0; i < 8; ++i)
+        out[i] = ex->stats[i];
+    return 0;
+}
+
+} // extern "C"

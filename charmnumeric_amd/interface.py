@@ -1,0 +1,122 @@
+"""The interface object: where upstream's frontend talks to a Charm++ server over a CCS socket
+(charmnumeric/interface.py upstream), this one drives the in-process executor of libcnhip through
+its C ABI (include/cnexec.h). `connect` keeps upstream's signature; address and port are ignored."""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import _lib as L
+from . import lazy
+
+
+class CharmNumericInterface:
+    def __init__(self, device=0, max_pes=1):
+        """device < 0 selects the executor's dry mode: every decision is taken and logged, nothing
+        is allocated or launched (used by tests on machines without a GPU)."""
+        self.device = int(device)
+        self.max_pes = int(max_pes)
+        self.odf = None
+        self._ex = None
+        self._min_tiles = {}
+
+    # -- connection --------------------------------------------------------------------------
+    def connect(self, server_ip=None, server_port=None, odf=4):
+        if self._ex is not None:
+            raise RuntimeError("already connected")
+        ex = C.c_void_p()
+        L.check(L.lib.cnx_create(self.device, self.max_pes, int(odf), C.byref(ex)))
+        self._ex = ex
+        self.odf = int(odf)
+        for nd, t in self._min_tiles.items():
+            L.check(L.lib.cnx_set_min_tile(self._ex, nd, t))
+        return self
+
+    def set_min_tile(self, ndims, min_tile):
+        """Minimum tile edge per rank (CT_MIN_TILE_1D/2D/3D upstream, src/backend.hpp:10-18)."""
+        self._min_tiles[int(ndims)] = int(min_tile)
+        if self._ex is not None:
+            L.check(L.lib.cnx_set_min_tile(self._ex, int(ndims), int(min_tile)))
+
+    def close(self):
+        if self._ex is not None:
+            # instructions still pending refer to arrays of this executor: drop them
+            lazy.execute(self)
+            L.check(L.lib.cnx_destroy(self._ex))
+            self._ex = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        self.close()
+
+    def _handle(self):
+        if self._ex is None:
+            raise RuntimeError("interface is not connected")
+        return self._ex
+
+    # -- what the lazy core calls ------------------------------------------------------------------
+    def send_dag(self, epoch, message):
+        L.check(L.lib.cnx_receive_dag(self._handle(), int(epoch), len(message), message))
+
+    def direct_call(self, instr):
+        ex = self._handle()
+        if instr.opcode == "put":
+            host = instr.payload
+            L.check(L.lib.cnx_put(ex, instr.name, host.size, instr.dtype, host.ctypes.data_as(C.c_void_p)))
+        elif instr.opcode == "fill_uniform":
+            seed, stream, lo, hi = instr.payload
+            L.check(L.lib.cnx_fill_uniform(ex, instr.name, seed, stream, lo, hi))
+        elif instr.opcode == "fill_cg_matrix":
+            L.check(L.lib.cnx_fill_cg_matrix(ex, instr.name, instr.payload[0]))
+        else:
+            raise AssertionError(instr.opcode)
+
+    # -- data out ----------------------------------------------------------------------------
+    def get(self, ndims, name, size, dtype=np.float64):
+        """Array `name` as a flat NumPy array (upstream: interface.get(ndims, name, size, dtype=),
+        charmnumeric.py:683-688)."""
+        out = np.empty(int(size), dtype=np.dtype(dtype))
+        L.check(L.lib.cnx_get(self._handle(), int(ndims), 0, int(name), int(size), lazy.wire_dtype(dtype),
+                              out.ctypes.data_as(C.c_void_p)))
+        return out
+
+    def sync(self):
+        L.check(L.lib.cnx_sync(self._handle()))
+
+    # -- introspection -----------------------------------------------------------------------
+    def array_info(self, name):
+        nd, dt, tile = C.c_int(), C.c_int(), C.c_int()
+        shape, off = (C.c_int32 * 3)(), (C.c_int32 * 3)()
+        L.check(L.lib.cnx_array_info(self._handle(), int(name), C.byref(nd), C.byref(dt), C.byref(tile),
+                                     shape, off))
+        return {"ndims": nd.value, "dtype": dt.value, "tile": tile.value,
+                "shape": tuple(shape[:nd.value]), "offset": tuple(off[:nd.value])}
+
+    def stats(self):
+        out = (C.c_int64 * 8)()
+        L.check(L.lib.cnx_stats(self._handle(), out))
+        keys = ("compiled", "cache_hits", "nodes", "allocations", "reuses", "group_launches",
+                "live_arrays", "bytes_held")
+        return dict(zip(keys, out))
+
+    def set_trace(self, on=True):
+        L.check(L.lib.cnx_set_trace(self._handle(), 1 if on else 0))
+
+    def trace(self):
+        need = L.lib.cnx_trace(self._handle(), None, 0)
+        buf = C.create_string_buffer(int(need))
+        L.lib.cnx_trace(self._handle(), buf, need)
+        return buf.value.decode().splitlines()
+
+
+class LocalCluster(CharmNumericInterface):
+    """Context manager that starts an executor and connects to it; upstream's LocalCluster launches
+    `charmrun +p<max_pes> server` and connects with `odf` (charmnumeric/interface.py:25-129
+    upstream)."""
+
+    def __init__(self, server_binary=None, *, odf=4, max_pes=1, device=0, **_ignored):
+        super().__init__(device=device, max_pes=max_pes)
+        self.connect(odf=odf)

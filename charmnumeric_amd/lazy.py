@@ -1,0 +1,408 @@
+"""Lazy recording core of the frontend: every array operation is recorded in program order and
+shipped to the executor as a DAG of fused groups when something forces a flush.
+
+Upstream delegates this layer to charmtyles (``fusible_op`` / ``nonfusible_op`` / ``create_object``
+/ ``execute`` / ``set_auto_flush``, imported at charmnumeric/charmnumeric.py:5-16 and used by
+examples/jacobi2d.py:2-6 upstream); charmtyles is not part of the charmnumeric tree, so the grouping
+rule and the byte format here are this package's own. What is kept: the AST node fields and opcode /
+dtype numbers the backend consumes, and the observable semantics (program order, lazy execution,
+results identical to evaluating statement by statement).
+
+Grouping rule: consecutive elementwise operations of one result shape form a group; a group ends at
+the first result that must exist as an array afterwards (its handle is still alive, or something
+outside the group reads it), at an assignment ``target[region] = value`` that consumes the group's
+last result (which becomes the group's SET_REGION root), and before any other kind of instruction.
+Results that die inside their group are temporaries and never touch memory.
+"""
+from __future__ import annotations
+
+import struct
+
+import numpy as np
+
+from . import _lib as L
+
+# Extension opcodes of include/cnexec.h
+OP_DELETE, OP_SUM, OP_SUMSQ_DIFF, OP_MAXABS_DIFF = 100, 101, 102, 103
+DAG_MAGIC = 0x47444E43
+
+_ELEMENTWISE = {L.OP_ADD, L.OP_SUB, L.OP_MUL, L.OP_DIV, L.OP_TANH, L.OP_EXP}
+
+
+class ArrayRef:
+    """One use of an array (or of a slice of it) as an operand."""
+
+    __slots__ = ("name", "region", "shape", "base_ndims", "dtype", "broadcast")
+
+    def __init__(self, name, region, shape, base_ndims, dtype, broadcast=False):
+        self.name = name
+        self.region = region          # (start, stop, step) tuples relative to the base array, or None
+        self.shape = tuple(shape)
+        self.base_ndims = base_ndims
+        self.dtype = dtype            # wire dtype
+        self.broadcast = broadcast
+
+
+class Instr:
+    __slots__ = ("kind", "name", "opcode", "operands", "shape", "dtype", "region", "payload")
+
+    def __init__(self, kind, name=None, opcode=None, operands=(), shape=(), dtype=L.F64, region=None,
+                 payload=None):
+        self.kind = kind              # create | op | set | nonfusible | delete | call
+        self.name = name
+        self.opcode = opcode
+        self.operands = list(operands)  # ArrayRef or python scalars
+        self.shape = tuple(shape)
+        self.dtype = dtype
+        self.region = region
+        self.payload = payload
+
+
+class _State:
+    def __init__(self):
+        self.pending = []
+        self.next_name = 1
+        self.auto_flush = None        # (interface, threshold)
+        self.epoch = 0
+        self.flushing = False
+
+
+_state = _State()
+
+
+def new_name():
+    n = _state.next_name
+    _state.next_name += 1
+    return n
+
+
+def record(instr):
+    _state.pending.append(instr)
+    af = _state.auto_flush
+    if af is not None and not _state.flushing and len(_state.pending) >= af[1]:
+        execute(af[0])
+
+
+def record_delete(name):
+    # Called from handle finalisers; never flushes (it may run at any point, even at shutdown).
+    try:
+        _state.pending.append(Instr("delete", name=name))
+    except Exception:  # interpreter teardown
+        pass
+
+
+def set_auto_flush(interface, threshold):
+    """Flush to `interface` whenever `threshold` instructions are pending (examples/jacobi2d.py:6
+    upstream)."""
+    _state.auto_flush = (interface, int(threshold))
+
+
+def reset():
+    """Forget everything recorded and restart naming (what upstream's test fixture
+    reset_frontend_state does, tests/conftest.py:128-141 upstream)."""
+    _state.pending.clear()
+    _state.next_name = 1
+    _state.auto_flush = None
+    _state.epoch = 0
+
+
+def pending_count():
+    return len(_state.pending)
+
+
+# ---------------------------------------------------------------------------------------------
+# grouping
+
+
+class _Group:
+    __slots__ = ("ops", "set_idx", "shape", "dtype", "names")
+
+    def __init__(self, shape, dtype):
+        self.ops = []
+        self.set_idx = None
+        self.shape = shape
+        self.dtype = dtype
+        self.names = set()
+
+
+def _uses_of(batch):
+    """name -> indices of the instructions that read it; a negative index -(i+1) marks instruction
+    i writing into it (assignment target), which always counts as a use from outside any group."""
+    uses = {}
+    for i, ins in enumerate(batch):
+        if ins.kind in ("op", "set", "nonfusible", "call"):
+            for o in ins.operands:
+                if isinstance(o, ArrayRef):
+                    uses.setdefault(o.name, []).append(i)
+        if ins.kind in ("set", "call") and ins.name is not None:
+            uses.setdefault(ins.name, []).append(-(i + 1))
+    return uses
+
+
+def _plan(batch):
+    """Returns the list of work items in execution order:
+    ("group", _Group) | ("instr", index) | ("delete", name)."""
+    producer = {ins.name: i for i, ins in enumerate(batch) if ins.kind == "op"}
+    deleted = {ins.name for ins in batch if ins.kind == "delete"}
+    dropped = set()                     # dead code: op indices never emitted
+    forced = set()                      # op results that must be materialised
+
+    while True:
+        uses = _uses_of([ins if i not in dropped else Instr("nop") for i, ins in enumerate(batch)])
+        items, group_of = [], {}
+        cur = None
+        deferred = []
+
+        def close():
+            nonlocal cur
+            if cur is not None and cur.ops:
+                items.append(("group", cur))
+            cur = None
+            for name in deferred:
+                items.append(("delete", name))
+            deferred.clear()
+
+        for i, ins in enumerate(batch):
+            if i in dropped or ins.kind == "nop":
+                continue
+            if ins.kind == "op":
+                reads_slice_of_own = cur is not None and any(
+                    isinstance(o, ArrayRef) and o.region is not None and o.name in cur.names
+                    for o in ins.operands)
+                if cur is None or cur.shape != ins.shape or cur.dtype != ins.dtype or reads_slice_of_own:
+                    close()
+                    cur = _Group(ins.shape, ins.dtype)
+                cur.ops.append(i)
+                cur.names.add(ins.name)
+                group_of[i] = cur
+                if ins.name in forced:
+                    close()
+            elif ins.kind == "delete":
+                if ins.name in producer and producer[ins.name] in dropped:
+                    continue
+                deferred.append(ins.name)
+                if cur is None:
+                    close()
+            elif ins.kind == "set":
+                v = ins.operands[0]
+                fuse = (cur is not None and isinstance(v, ArrayRef) and v.region is None
+                        and batch[cur.ops[-1]].name == v.name and v.name not in forced
+                        and not v.broadcast)
+                if fuse:
+                    cur.set_idx = i
+                    group_of[i] = cur
+                    close()
+                else:
+                    close()
+                    items.append(("instr", i))
+            else:
+                close()
+                items.append(("instr", i))
+        close()
+
+        changed = False
+        for i, ins in enumerate(batch):
+            if ins.kind != "op" or i in dropped:
+                continue
+            g = group_of[i]
+            use_idx = uses.get(ins.name, [])
+            dead = ins.name in deleted
+            if dead and not use_idx:
+                dropped.add(i)          # computed, never read, handle gone
+                changed = True
+                continue
+            inside = all(u >= 0 and group_of.get(u) is g for u in use_idx)
+            is_last = g.ops[-1] == i
+            temp_ok = dead and inside and (not is_last or g.set_idx is not None)
+            if not temp_ok and ins.name not in forced:
+                # must exist as an array: its group has to end here
+                if not (is_last and g.set_idx is None):
+                    forced.add(ins.name)
+                    changed = True
+        if not changed:
+            return items, forced, deleted, producer, dropped
+
+
+# ---------------------------------------------------------------------------------------------
+# serialisation (format: include/cnexec.h)
+
+
+def _region_bytes(region):
+    if region is None:
+        return struct.pack("<i", 1)
+    start, stop, step = region
+    out = [struct.pack("<ii", 0, len(start))]
+    for d in range(len(start)):
+        out.append(struct.pack("<iii", int(start[d]), int(stop[d]), int(step[d])))
+    return b"".join(out)
+
+
+def _full_region(shape):
+    return (tuple(0 for _ in shape), tuple(int(s) for s in shape), tuple(1 for _ in shape))
+
+
+class _NodeWriter:
+    """Collects the AST nodes of one DAG node."""
+
+    def __init__(self):
+        self.nodes = []
+        self.roots = []
+        self._leaf = {}
+        self._next_scalar = -1
+
+    def _add(self, name, opcode, is_temp, is_scalar, is_broadcast, ndims, dtype, operands, scalar,
+             operand_regions, region):
+        self.nodes.append((name, opcode, is_temp, is_scalar, is_broadcast, ndims, dtype, operands, scalar,
+                           operand_regions, region))
+        return len(self.nodes) - 1
+
+    def leaf(self, ref):
+        key = (ref.name, bool(ref.broadcast))
+        if key not in self._leaf:
+            self._leaf[key] = self._add(ref.name, L.OP_NOOP, 0, 0, 1 if ref.broadcast else 0,
+                                        ref.base_ndims, ref.dtype, (), 0.0, (), None)
+        return self._leaf[key]
+
+    def scalar(self, value, ndims, dtype):
+        idx = self._add(self._next_scalar, L.OP_NOOP, 0, 1, 0, ndims, dtype, (), float(value), (), None)
+        self._next_scalar -= 1
+        return idx
+
+    def op(self, name, opcode, is_temp, ndims, dtype, operands, operand_regions, region=None, root=True):
+        idx = self._add(name, opcode, 1 if is_temp else 0, 0, 0, ndims, dtype, tuple(operands), 0.0,
+                        tuple(operand_regions), region)
+        if root:
+            self.roots.append(idx)
+        return idx
+
+    def to_bytes(self, node_id, fusible):
+        out = [struct.pack("<iiii", node_id, 1 if fusible else 0, len(self.nodes), len(self.roots))]
+        for (name, opcode, is_temp, is_scalar, is_bc, ndims, dtype, operands, scalar, oregs, region) in self.nodes:
+            out.append(struct.pack("<iiiiiiii", name, opcode, is_temp, is_scalar, is_bc, ndims, dtype,
+                                   len(operands)))
+            for o in operands:
+                out.append(struct.pack("<i", o))
+            out.append(struct.pack("<d", scalar))
+            for r in oregs:
+                out.append(_region_bytes(r))
+            out.append(_region_bytes(region))
+        out.append(struct.pack("<%di" % len(self.roots), *self.roots))
+        return b"".join(out)
+
+
+def _emit_group(batch, g, forced, deleted, node_id):
+    w = _NodeWriter()
+    index_of = {}                      # op result name -> AST node index inside this group
+    ndims = len(g.shape)
+    last = g.ops[-1]
+    for i in g.ops:
+        ins = batch[i]
+        opnds, oregs = [], []
+        for o in ins.operands:
+            if isinstance(o, ArrayRef):
+                if o.name in index_of and o.region is None:
+                    opnds.append(index_of[o.name])
+                    oregs.append(None)
+                else:
+                    opnds.append(w.leaf(o))
+                    oregs.append(o.region)
+            else:
+                opnds.append(w.scalar(o, ndims, ins.dtype))
+                oregs.append(None)
+        is_root_result = (i == last and g.set_idx is None)
+        region = _full_region(ins.shape) if is_root_result else None
+        index_of[ins.name] = w.op(ins.name, ins.opcode, not is_root_result, ndims, ins.dtype, opnds, oregs,
+                                  region)
+    if g.set_idx is not None:
+        s = batch[g.set_idx]
+        target = w.leaf(s.payload)      # ArrayRef of the whole target
+        w.op(new_name(), L.OP_SET_REGION, False, s.payload.base_ndims, s.dtype,
+             [target, index_of[batch[last].name]], [None, None], s.region)
+    return w.to_bytes(node_id, True)
+
+
+def _emit_instr(ins, node_id):
+    w = _NodeWriter()
+    if ins.kind == "create":
+        w.op(ins.name, L.OP_CREATE, False, len(ins.shape), ins.dtype, [], [], _full_region(ins.shape))
+        return w.to_bytes(node_id, False)
+    if ins.kind == "set":
+        v = ins.operands[0]
+        target = w.leaf(ins.payload)
+        if isinstance(v, ArrayRef):
+            value, vreg = w.leaf(v), v.region
+        else:
+            value, vreg = w.scalar(v, ins.payload.base_ndims, ins.dtype), None
+        w.op(new_name(), L.OP_SET_REGION, False, ins.payload.base_ndims, ins.dtype, [target, value],
+             [None, vreg], ins.region)
+        return w.to_bytes(node_id, isinstance(v, ArrayRef))
+    if ins.kind == "nonfusible":
+        opnds = [w.leaf(o) for o in ins.operands]
+        w.op(ins.name, ins.opcode, False, len(ins.shape), ins.dtype, opnds, [o.region for o in ins.operands],
+             _full_region(ins.shape))
+        return w.to_bytes(node_id, False)
+    raise AssertionError(ins.kind)
+
+
+def _emit_delete(name, node_id):
+    w = _NodeWriter()
+    w.op(name, OP_DELETE, False, 1, L.F64, [], [], None)
+    return w.to_bytes(node_id, False)
+
+
+def build_messages(batch):
+    """Turns a batch of instructions into a list of work for an interface:
+    ("dag", bytes) and ("call", Instr) in execution order."""
+    items, forced, deleted, producer, dropped = _plan(batch)
+    out, nodes = [], []
+    node_id = 0
+
+    def flush_nodes():
+        if nodes:
+            out.append(("dag", struct.pack("<iii", DAG_MAGIC, 1, len(nodes)) + b"".join(nodes)))
+            nodes.clear()
+
+    materialised = set()
+    for kind, what in items:
+        if kind == "group":
+            nodes.append(_emit_group(batch, what, forced, deleted, node_id))
+            if what.set_idx is None:
+                materialised.add(batch[what.ops[-1]].name)
+        elif kind == "delete":
+            if what in producer and what not in materialised:
+                continue                # a temporary: it never became an array
+            nodes.append(_emit_delete(what, node_id))
+        else:
+            ins = batch[what]
+            if ins.kind == "call":
+                flush_nodes()
+                out.append(("call", ins))
+                continue
+            nodes.append(_emit_instr(ins, node_id))
+        node_id += 1
+    flush_nodes()
+    return out
+
+
+def execute(interface):
+    """Ships everything recorded so far to the executor behind `interface`
+    (charmtyles.core.execute upstream: examples/jacobi3d.py:2,18)."""
+    if _state.flushing or not _state.pending:
+        return
+    _state.flushing = True
+    try:
+        batch = _state.pending
+        _state.pending = []
+        for kind, what in build_messages(batch):
+            if kind == "dag":
+                interface.send_dag(_state.epoch, what)
+                _state.epoch += 1
+            else:
+                interface.direct_call(what)
+    finally:
+        _state.flushing = False
+
+
+def wire_dtype(np_dtype):
+    return {np.dtype("float32"): L.F32, np.dtype("float64"): L.F64, np.dtype("int32"): L.I32,
+            np.dtype("int64"): L.I64}[np.dtype(np_dtype)]

@@ -1,0 +1,24 @@
+"""Seeded synthetic inputs generated on the device (upstream has no generator:
+charmnumeric/random.py:4-5 upstream only raises)."""
+from __future__ import annotations
+
+from . import lazy
+from .array import create_array
+
+
+def uniform(shape, seed, stream=0, low=0.0, high=1.0):
+    """fp64 array with element i (row-major) = low + (high-low)*u01(seed, stream, i), from the
+    counter-based SplitMix64 generator the tests restate in NumPy."""
+    out = create_array(shape, dtype="float64")
+    lazy.record(lazy.Instr("call", name=out.name, opcode="fill_uniform", shape=out.shape,
+                           dtype=out.wire_dtype(), payload=(int(seed), int(stream), float(low), float(high))))
+    return out
+
+
+def cg_matrix(n, seed):
+    """The dense symmetric test matrix of the CG workload: diagonal 2.0, off-diagonal
+    (u01(seed,0,i*n+j) + u01(seed,0,j*n+i)) / (2n)."""
+    out = create_array((int(n), int(n)), dtype="float64")
+    lazy.record(lazy.Instr("call", name=out.name, opcode="fill_cg_matrix", shape=out.shape,
+                           dtype=out.wire_dtype(), payload=(int(seed),)))
+    return out

@@ -1,0 +1,115 @@
+/*
+ * cnexec.h — the host executor of libcnhip: plays upstream's ArrayDAGGroup + PartitionImpl for all
+ * partitions of every array on one device, without Charm++.
+ *
+ * The entry points mirror the entry methods of src/backend.ci:10-18 (what the CCS handlers of the
+ * server call): a serialized DAG comes in through cnx_receive_dag, array contents leave through
+ * cnx_get. Everything between (shape pass, tile rule, array creation, kernel compilation and cache,
+ * per-node routing) happens inside, on top of the cnh_* calls of cnhip.h.
+ *
+ * Conventions as in cnhip.h: 0 on success, < 0 on error with cnh_last_error(); one thread per
+ * executor at a time.
+ *
+ * ---- DAG message (little endian) ----
+ * The upstream byte format is defined by charmtyles (DAG::deserialize, called from
+ * src/dag_group_receive.cpp:191-192) and is not part of the charmnumeric tree; this format carries
+ * the same information: the fields of DAGNode/ASTNode the backend reads
+ * (src/dag_group_compile.cpp:45-51, src/jit.cpp:223-385, src/execute_node_regions.cpp:56-107) and
+ * regions in upstream's own region encoding (charmnumeric.py:194-207).
+ *
+ *   message  := int32 magic (CNX_DAG_MAGIC), int32 version (1), int32 n_dag_nodes, dag_node*
+ *   dag_node := int32 id, int32 fusible, int32 n_ast_nodes, int32 n_roots, ast_node*, int32 roots[n_roots]
+ *   ast_node := int32 result_name, int32 opcode, int32 is_temp, int32 is_scalar, int32 is_broadcast,
+ *               int32 ndims, int32 dtype, int32 n_operands (<= 2), int32 operands[n_operands],
+ *               float64 scalar, region operand_regions[n_operands], region node_region
+ *   region   := int32 is_global, then if not global: int32 ndims, (int32 start, stop, step)[ndims]
+ *
+ * DAG nodes are listed in execution (program) order. operands[] index the ast_node list of the same
+ * DAG node. Opcodes are upstream's (src/opcodes.hpp:3-20) plus the extension opcodes below.
+ * Leaves are NOOP nodes naming an existing array (is_broadcast = 1 for a size-1 array used as a
+ * scalar), or is_scalar nodes carrying a literal.
+ *
+ * Root kinds and what they do:
+ *   CREATE      node_region = [0:shape) of a new zero-filled array `result_name`
+ *               (src/dag_group_receive.cpp:227-250, src/partition_lifecycle.cpp:43-88)
+ *   elementwise group of ADD/SUB/MUL/DIV/TANH/EXP temporaries ending in one non-temp root, or in a
+ *               SET_REGION root (operands: target leaf, value) — src/execute_node.cpp:1195-1585
+ *   SET_REGION  with a scalar value: fill (src/executor_ast_visitor.cpp:112-147)
+ *   REDUCE      dot of two 1-D arrays -> size-1 array (src/executor_reduce.cpp:8-119)
+ *   MATMUL      2-D array times 1-D array -> 1-D array (src/executor_matmul.cpp:150-498)
+ *   MATMATMUL   2-D times 2-D -> 2-D (src/executor_matmatmul.cpp:105-484)
+ *   CNX_OP_DELETE  drop array `result_name`; its buffer goes to the free list
+ *               (src/backend.hpp:366-545)
+ */
+#ifndef CNEXEC_H
+#define CNEXEC_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CNX_DAG_MAGIC 0x47444e43 /* "CNDG" */
+
+/* Extension opcodes (no upstream counterpart; upstream has no N-D reduction, no random numbers and
+ * no bulk upload: src/executor_reduce.cpp:9-12, charmnumeric/random.py:4-5, charmnumeric.py:863-878).
+ * Operand layout: SUM(a); SUMSQ_DIFF(a, b); MAXABS_DIFF(a, b) -> size-1 fp64 array `result_name`,
+ * over whole arrays of any rank; DELETE names the array in result_name. */
+enum {
+    CNX_OP_DELETE = 100,
+    CNX_OP_SUM = 101,
+    CNX_OP_SUMSQ_DIFF = 102,
+    CNX_OP_MAXABS_DIFF = 103
+};
+
+typedef struct cnx_executor cnx_executor;
+
+/* Start-up: what `charmrun +p<num_pes> server` plus the client's connect(ip, port, odf) fix
+ * (charmnumeric/interface.py:70-92): odf * num_pes caps the number of tiles per array
+ * (src/decomposition_solver.hpp:107-111). device is passed to cnh_init. */
+int cnx_create(int device, int num_pes, int odf, cnx_executor** out);
+int cnx_destroy(cnx_executor* ex);
+/* Overrides CT_MIN_TILE_1D/2D/3D (src/backend.hpp:10-18; the upstream tests build with 64). */
+int cnx_set_min_tile(cnx_executor* ex, int ndims, int min_tile);
+
+/* ArrayDAGGroup::receive_dag(int epoch, int size, char msg[size]) (src/backend.ci:15,
+ * src/dag_group_receive.cpp:190-575) followed by the partitions' run(): executes every node of the
+ * DAG in order. Returns when all work is queued on the executor's stream (not when it finished). */
+int cnx_receive_dag(cnx_executor* ex, int epoch, int64_t size, const char* msg);
+
+/* receive_get_request(int ndims, int epoch, int name, int size, int dtype) + gather + reply
+ * (src/backend.ci:16-17, src/partition_get.cpp:4-67, src/dag_group_runtime.cpp:55-118): copies
+ * array `name` into host_out as one global row-major array of `size` elements. Blocks. */
+int cnx_get(cnx_executor* ex, int ndims, int epoch, int name, int64_t size, int dtype, void* host_out);
+
+/* Extensions without upstream counterpart. */
+/* Bulk upload of a whole row-major host array into existing array `name`. Blocks. */
+int cnx_put(cnx_executor* ex, int name, int64_t size, int dtype, const void* host_in);
+/* array[i] = lo + (hi-lo)*u01(seed, stream_id, i), i = global row-major index; fp64 arrays. */
+int cnx_fill_uniform(cnx_executor* ex, int name, uint64_t seed, uint64_t stream_id, double lo, double hi);
+/* The dense CG test matrix (symmetric, diagonal 2.0) into the square fp64 array `name`. */
+int cnx_fill_cg_matrix(cnx_executor* ex, int name, uint64_t seed);
+/* Waits for everything queued so far. */
+int cnx_sync(cnx_executor* ex);
+
+/* Introspection (tests, logs). */
+/* ndims, dtype, tile edge, shape[3], offset[3] of array `name`; < 0 if unknown. */
+int cnx_array_info(cnx_executor* ex, int name, int* ndims, int* dtype, int* tile, int32_t* shape3,
+                   int32_t* offset3);
+/* Counters since creation: [0] kernels compiled (upstream num_compile, src/backend.hpp:241),
+ * [1] compile-cache hits, [2] DAG nodes executed, [3] device allocations, [4] free-list reuses,
+ * [5] fused-group launches, [6] live arrays, [7] bytes held (live + free list). */
+int cnx_stats(cnx_executor* ex, int64_t out[8]);
+/* Decision log: one text line per array creation, launch choice (dense / tiles, ping-pong or in
+ * place), reduction, product. cnx_trace copies the NUL-terminated log into buf when it fits, clears
+ * it, and returns the size needed. With device < 0 in cnx_create the executor takes every decision
+ * and logs it but allocates and launches nothing (host-logic tests on machines without a GPU). */
+int cnx_set_trace(cnx_executor* ex, int on);
+int64_t cnx_trace(cnx_executor* ex, char* buf, size_t cap);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

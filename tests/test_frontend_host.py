@@ -1,0 +1,252 @@
+"""Host logic of the frontend and the executor, exercised without a GPU: the executor's dry mode
+takes every decision (shapes, tiles, kernel compilation and cache, launch path) and logs it."""
+import struct
+
+import numpy as np
+import pytest
+
+import charmnumeric_amd as cnp
+from charmnumeric_amd import _lib as L
+from charmnumeric_amd import lazy
+from charmnumeric_amd.array import parse_key, compose, region_shape
+
+
+@pytest.fixture
+def itf():
+    cnp.reset()
+    it = cnp.CharmNumericInterface(device=-1)
+    it.connect(odf=4)
+    it.set_trace()
+    yield it
+    cnp.reset()
+    it.close()
+
+
+def lines(itf, prefix):
+    """Log lines starting with `prefix`; reading the log clears it."""
+    return [ln for ln in itf.trace() if ln.startswith(prefix)]
+
+
+# ---- slicing rules (charmnumeric.py:272-343 upstream) ----
+
+def test_parse_key_follows_numpy_for_slices_and_keeps_integer_dims():
+    shape = (10, 7, 5)
+    assert parse_key((slice(1, -1), 3), shape) == ((1, 3, 0), (9, 4, 5), (1, 1, 1))
+    assert parse_key(Ellipsis, shape) == ((0, 0, 0), (10, 7, 5), (1, 1, 1))
+    assert parse_key((Ellipsis, -1), shape) == ((0, 0, 4), (10, 7, 5), (1, 1, 1))
+    assert parse_key((slice(2, -2, 2),), (17,)) == ((2,), (15,), (2,))
+    assert region_shape(((2,), (15,), (2,))) == (7,)
+    with pytest.raises(NotImplementedError):
+        parse_key(slice(None, None, -1), (4,))
+    with pytest.raises(ValueError):
+        parse_key(slice(None, None, 0), (4,))
+    with pytest.raises(IndexError):
+        parse_key(10, (4,))
+    with pytest.raises(IndexError):
+        parse_key((0, 0), (4,))
+    with pytest.raises(NotImplementedError):
+        parse_key((None, 0), (4,))
+    with pytest.raises(TypeError):
+        parse_key("a", (4,))
+
+
+def test_view_of_view_composes_like_numpy():
+    base = np.arange(200)
+    outer = parse_key(slice(10, 190, 3), base.shape)
+    inner = parse_key(slice(2, 50, 4), region_shape(outer))
+    r = compose(outer, inner)
+    want = base[10:190:3][2:50:4]
+    got = base[r[0][0]:r[1][0]:r[2][0]]
+    assert np.array_equal(got, want)
+
+
+def test_dtype_and_shape_rules(itf):
+    a = cnp.zeros((8,), dtype=cnp.float32)
+    assert (a + 1.5).dtype == np.float32          # scalars never promote (charmnumeric.py:369-373)
+    assert (2 * a).shape == (8,)
+    i = cnp.zeros((8,), dtype=cnp.int32)
+    assert (i / 2).dtype == np.int32
+    with pytest.raises(NotImplementedError):
+        a + i
+    with pytest.raises(ValueError):
+        a + cnp.zeros((9,), dtype=cnp.float32)
+    with pytest.raises(TypeError):
+        cnp.zeros((4,), dtype=np.float16)
+    with pytest.raises(ValueError):
+        bool(a)
+    with pytest.raises(TypeError):
+        np.asarray(a)
+    with pytest.raises(ValueError):
+        a @ cnp.zeros((9,), dtype=cnp.float32)
+    with pytest.raises(ValueError):
+        cnp.zeros((4, 5)) @ cnp.zeros((4,))
+    with pytest.raises(ValueError):
+        cnp.zeros((4, 5)) @ cnp.zeros((4, 5))
+    assert a.size == 8 and a.size() == 8 and a.nbytes == 32 and len(a) == 8 and a.ndim == 1
+    assert a[2:6].shape == (4,) and cnp.zeros((4, 6))[1].shape == (1, 6)
+
+
+# ---- grouping ----
+
+def test_statement_with_dead_temporaries_is_one_group(itf):
+    a = cnp.zeros((128,), dtype=cnp.float32)
+    b = cnp.zeros((128,), dtype=cnp.float32)
+    x = 2 * (a + b + 3)
+    cnp.execute(itf)
+    g = lines(itf, "group")
+    assert len(g) == 1 and "path=dense" in g[0] and "inputs=2" in g[0]
+    assert itf.stats()["live_arrays"] == 3       # a, b, x: the two temporaries never became arrays
+    assert itf.array_info(x.name)["shape"] == (128,)
+
+
+def test_live_intermediate_is_materialised_and_splits_the_group(itf):
+    a = cnp.zeros((64,))
+    t = a + 1.0
+    u = t * 2.0
+    cnp.execute(itf)
+    g = lines(itf, "group")
+    assert len(g) == 2
+    assert itf.array_info(t.name)["shape"] == (64,) and itf.array_info(u.name)["shape"] == (64,)
+
+
+def test_unused_results_are_dropped(itf):
+    a = cnp.zeros((64,))
+    a + 1.0                                      # result dropped immediately
+    cnp.execute(itf)
+    assert lines(itf, "group") == []
+
+
+def test_stencil_statement_fuses_into_set_region_with_pingpong(itf):
+    u = cnp.zeros((64, 64))
+    u[0, :] = 1.0
+    u[1:-1, 1:-1] = 0.25 * (u[:-2, 1:-1] + u[2:, 1:-1] + u[1:-1, :-2] + u[1:-1, 2:])
+    cnp.execute(itf)
+    tr = itf.trace()
+    assert sum(ln.startswith("fill") for ln in tr) == 1
+    g = [ln for ln in tr if ln.startswith("group")]
+    assert len(g) == 1 and "path=tiles" in g[0] and "pingpong" in g[0] and "inputs=4" in g[0]
+
+
+def test_assignment_from_a_live_array_is_a_copy_group(itf):
+    a = cnp.zeros((17, 17))
+    c = cnp.zeros((9, 9))
+    c[1:-1, 1:-1] = a[2:-2:2, 2:-2:2]
+    cnp.execute(itf)
+    g = lines(itf, "group")
+    assert len(g) == 1 and "path=tiles" in g[0] and "inplace" in g[0]
+
+
+def test_pending_reader_runs_before_a_later_assignment(itf):
+    """t = u + 1 recorded before u[...] = 5 must see the old u: the assignment closes t's group."""
+    u = cnp.zeros((32,))
+    t = u + 1.0
+    u[...] = 5.0
+    cnp.execute(itf)
+    tr = itf.trace()
+    assert [ln.split()[0] for ln in tr if ln.split()[0] in ("group", "fill")] == ["group", "fill"]
+    assert t.shape == (32,)
+
+
+def test_cg_iteration_compiles_once_and_reuses_buffers(itf):
+    n = 256
+    A = cnp.zeros((n, n))
+    b = cnp.ones((n,))
+    x = cnp.zeros((n,))
+    r = b.copy()
+    p = b.copy()
+    rtr = r @ r
+    cnp.execute(itf)
+    compiled = []
+    for k in range(4):
+        Ap = A @ p
+        pAp = p @ Ap
+        alpha = rtr / pAp
+        x = x + alpha * p
+        r = r - alpha * Ap
+        rtr_new = r @ r
+        beta = rtr_new / rtr
+        p = r + beta * p
+        rtr = rtr_new
+        cnp.execute(itf)
+        compiled.append(itf.stats()["compiled"])
+    assert compiled[1] == compiled[0] == compiled[-1]         # every later iteration hits the cache
+    st = itf.stats()
+    assert st["reuses"] > 0 and st["live_arrays"] <= 12
+    tr = itf.trace()
+    assert sum(ln.startswith("matmul") for ln in tr) == 4
+    assert sum(ln.startswith("reduce") for ln in tr) == 1 + 2 * 4
+    scal = [ln for ln in tr if ln.startswith("group") and "scalars=1" in ln]
+    assert len(scal) == 3 * 4                                 # x, r, p updates take alpha/beta from the device
+
+
+def test_tile_rule_and_minimum_tile_override(itf):
+    """Tile = minimum tile of the rank doubled until the array has at most odf*PEs tiles
+    (src/decomposition_solver.hpp:100-122 upstream); the upstream tests build with minimum 64."""
+    a = cnp.zeros((1 << 24,))
+    m = cnp.zeros((16384, 16384))
+    u2 = cnp.zeros((8192, 8192))
+    cnp.execute(itf)
+    assert itf.array_info(a.name)["tile"] == 4194304
+    assert itf.array_info(m.name)["tile"] == 8192
+    assert itf.array_info(u2.name)["tile"] == 4096           # odf 4, one PE: 2x2 tiles
+    itf.set_min_tile(1, 64)
+    v = cnp.zeros((200,))
+    w = cnp.zeros((100,))
+    cnp.execute(itf)
+    assert itf.array_info(v.name)["tile"] == 64 and itf.array_info(w.name)["tile"] == 64
+    it16 = cnp.CharmNumericInterface(device=-1)
+    it16.connect(odf=16)
+    u3 = cnp.zeros((8192, 8192))
+    u4 = cnp.zeros((512, 512, 512))
+    cnp.execute(it16)
+    assert it16.array_info(u3.name)["tile"] == 2048
+    assert it16.array_info(u4.name)["tile"] == 256           # 16 tiles allowed: 128 would need 64
+    del u3, u4
+    it16.close()
+
+
+def test_matmatmul_panel_products_follow_the_tile_grids(itf):
+    itf.set_min_tile(2, 64)
+    A = cnp.zeros((128, 192))
+    B = cnp.zeros((192, 64))
+    Cm = A @ B
+    cnp.execute(itf)
+    # A: tile 128 (2 tiles allowed after doubling), B, C per the same rule; every product is logged
+    ln = lines(itf, "matmatmul")
+    assert len(ln) == 1 and "panel_products=" in ln[0]
+    assert itf.array_info(Cm.name)["shape"] == (128, 64)
+
+
+def test_malformed_messages_are_refused(itf):
+    with pytest.raises(RuntimeError, match="bad magic"):
+        itf.send_dag(0, struct.pack("<iii", 1, 1, 0))
+    good = struct.pack("<iii", lazy.DAG_MAGIC, 1, 1)
+    with pytest.raises(RuntimeError, match="truncated|AST nodes"):
+        itf.send_dag(0, good + struct.pack("<ii", 0, 0))
+    with pytest.raises(RuntimeError, match="version"):
+        itf.send_dag(0, struct.pack("<iii", lazy.DAG_MAGIC, 7, 0))
+    # a group that reads an array the executor has never seen
+    a = cnp.Array((8,), np.float64)
+    b = a + 1.0
+    with pytest.raises(RuntimeError, match="does not exist"):
+        cnp.execute(itf)
+    del b
+
+
+def test_get_checks_rank_size_and_dtype(itf):
+    a = cnp.zeros((8, 4))
+    cnp.execute(itf)
+    with pytest.raises(RuntimeError, match="asked for"):
+        itf.get(1, a.name, 32, dtype=np.float64)
+    with pytest.raises(RuntimeError, match="asked for"):
+        itf.get(2, a.name, 32, dtype=np.float32)
+    assert itf.get(2, a.name, 32, dtype=np.float64).shape == (32,)
+
+
+def test_auto_flush_threshold(itf):
+    cnp.set_auto_flush(itf, 5)
+    a = cnp.zeros((16,))
+    for _ in range(6):
+        a[...] = a + 1.0
+    assert lazy.pending_count() < 5
+    assert len(lines(itf, "group")) >= 1

@@ -1,0 +1,285 @@
+"""Programs written against the NumPy-like frontend, run through the DAG message, the host executor
+and the HIP kernels, and compared with NumPy evaluating the same statements in the same order.
+The first block restates the cases of upstream's integration tests
+(tests/test_backend_integration.py upstream) and of its self-checking example scripts."""
+import numpy as np
+import pytest
+
+import charmnumeric_amd as cnp
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture
+def itf():
+    cnp.reset()
+    it = cnp.CharmNumericInterface(device=0)
+    it.connect(odf=4)
+    yield it
+    cnp.reset()
+    it.close()
+
+
+@pytest.fixture
+def small_tiles(itf):
+    """Minimum tiles as in upstream's own test builds (64), so small arrays span several tiles."""
+    itf.set_min_tile(1, 64)
+    itf.set_min_tile(2, 16)
+    itf.set_min_tile(3, 8)
+    return itf
+
+
+# ---- upstream's integration cases ----
+
+def test_elementwise_expression_known_answer(itf):
+    a = cnp.create_array((32,), dtype=np.float32)
+    b = cnp.create_array((32,), dtype=np.float32)
+    a[:] = 1.5
+    b[:] = -0.5
+    got = (2.0 * (a + b + 3.0)).get(itf)
+    assert got.dtype == np.float32 and np.array_equal(got, np.full(32, 8.0, np.float32))
+
+
+@pytest.mark.parametrize("shape", [(8,), (4, 4), (4, 4, 4)])
+def test_add_on_every_rank(itf, shape):
+    lhs = cnp.create_array(shape, dtype=np.float32)
+    rhs = cnp.create_array(shape, dtype=np.float32)
+    lhs[...] = 1.0
+    rhs[...] = 1.0
+    got = (lhs + rhs).get(itf)
+    assert got.shape == shape and np.array_equal(got, np.full(shape, 2.0, np.float32))
+
+
+def test_shifted_slices_of_arange(small_tiles):
+    src = cnp.arange(512, dtype=np.float32)
+    got = (src[100:300] + src[150:350]).get(small_tiles)
+    host = np.arange(512, dtype=np.float32)
+    assert np.array_equal(got, host[100:300] + host[150:350])
+
+
+def test_strided_slice_assignment_17_to_9(small_tiles):
+    n, cn = 17, 9
+    coarse = cnp.create_array((cn, cn), dtype=np.float64)
+    fine = cnp.create_array((n, n), dtype=np.float64)
+    coarse[:, :] = 0.0
+    fine[:, :] = 1.0
+    coarse[1:-1, 1:-1] = fine[2:-2:2, 2:-2:2]
+    want = np.zeros((cn, cn))
+    want[1:-1, 1:-1] = np.ones((n, n))[2:-2:2, 2:-2:2]
+    assert np.array_equal(coarse.get(small_tiles), want)
+
+
+def _faces(u, v):
+    u[0, :, :] = v
+    u[-1, :, :] = v
+    u[:, 0, :] = v
+    u[:, -1, :] = v
+    u[:, :, 0] = v
+    u[:, :, -1] = v
+
+
+def test_jacobi3d_single_step_on_4_cubed(itf):
+    u = cnp.create_array((4, 4, 4), dtype=np.float32)
+    _faces(u, 1.0)
+    u[1:-1, 1:-1, 1:-1] = (1.0 / 6.0) * (u[:-2, 1:-1, 1:-1] + u[2:, 1:-1, 1:-1] + u[1:-1, :-2, 1:-1]
+                                          + u[1:-1, 2:, 1:-1] + u[1:-1, 1:-1, :-2] + u[1:-1, 1:-1, 2:])
+    w = np.zeros((4, 4, 4), np.float32)
+    _faces(w, 1.0)
+    c = np.float32(1.0 / 6.0)
+    w[1:-1, 1:-1, 1:-1] = c * (w[:-2, 1:-1, 1:-1] + w[2:, 1:-1, 1:-1] + w[1:-1, :-2, 1:-1]
+                               + w[1:-1, 2:, 1:-1] + w[1:-1, 1:-1, :-2] + w[1:-1, 1:-1, 2:])
+    got = u.get(itf)
+    assert np.array_equal(got, w)
+    assert np.allclose(got[1:-1, 1:-1, 1:-1], 0.5)
+
+
+# ---- upstream's example scripts ----
+
+def test_simple_example_with_overlapping_self_assignment(small_tiles):
+    """x = 2*(a+b+3); x[:50] = x[70:120] + 1 (examples/simple.py upstream)."""
+    a = cnp.zeros((128,), dtype=cnp.float32)
+    b = cnp.zeros((128,), dtype=cnp.float32)
+    x = 2 * (a + b + 3)
+    x[:50] = x[70:120] + 1
+    want = np.full(128, 6.0, np.float32)
+    want[:50] = want[70:120] + 1
+    assert np.array_equal(x.get(small_tiles), want)
+
+
+def test_reduction_example(itf):
+    """res = x @ x; x = x / res (examples/reduction.py upstream): ones(64) -> 1/64 everywhere."""
+    x = cnp.ones((64,), dtype=cnp.float32)
+    res = x @ x
+    x = x / res
+    assert np.array_equal(x.get(itf), np.full(64, 1.0 / 64.0, np.float32))
+    assert res.get(itf).item() == 64.0
+
+
+def test_matvec_closed_form(small_tiles):
+    """A[i,j] = i + j, x = 1: y_i = N*i + N(N-1)/2, exact in fp64 (examples/matvec.py upstream)."""
+    n = 96
+    host = np.add.outer(np.arange(n), np.arange(n)).astype(np.float64)
+    A = cnp.array(host)
+    x = cnp.ones((n,))
+    y = (A @ x).get(small_tiles)
+    assert np.array_equal(y, n * np.arange(n) + n * (n - 1) / 2)
+
+
+def test_matmatmul_of_ones_and_against_numpy(small_tiles):
+    A = cnp.ones((48, 80))
+    B = cnp.ones((80, 40))
+    assert np.array_equal((A @ B).get(small_tiles), np.full((48, 40), 80.0))
+    rng = np.random.default_rng(3)
+    ha, hb = rng.standard_normal((50, 70)), rng.standard_normal((70, 33))
+    got = (cnp.array(ha) @ cnp.array(hb)).get(small_tiles)
+    bound = 1e-12 * (np.abs(ha) @ np.abs(hb))
+    assert np.all(np.abs(got - ha @ hb) <= bound)
+
+
+def test_cg_example_against_the_closed_form(small_tiles):
+    """A = N*I + 1 1^T, b = 1..N: x = (b - sum(b)/(2N))/N; CG reaches it in two iterations
+    (examples/cg.py upstream)."""
+    itf = small_tiles
+    n = 128
+    A = cnp.ones((n, n), dtype=cnp.float64)
+    for i in range(n):
+        A[i, i] = n + 1.0
+    b = cnp.arange(1, n + 1, dtype=cnp.float64)
+    x = cnp.zeros((n,), dtype=cnp.float64)
+    r = b.copy()
+    p = b.copy()
+    rtr = r @ r
+    history = []
+    for k in range(3):
+        Ap = A @ p
+        pAp = p @ Ap
+        alpha = rtr / pAp
+        x = x + alpha * p
+        r = r - alpha * Ap
+        rtr_new = r @ r
+        beta = rtr_new / rtr
+        p = r + beta * p
+        rtr = rtr_new
+        history.append(rtr.get(itf).item())
+    bn = np.arange(1, n + 1, dtype=np.float64)
+    want = (bn - bn.sum() / (2 * n)) / n
+    got = x.get(itf)
+    assert np.allclose(got, want, rtol=1e-11, atol=0)
+    assert history[0] > history[1] and history[1] < 1e-12 * history[0]
+    st = itf.stats()
+    assert st["reuses"] > 0
+
+
+# ---- sweeps, multi-tile, ragged ----
+
+def test_jacobi2d_sweeps_match_numpy_bit_for_bit(small_tiles):
+    n = 70                                        # ragged against the tile edge
+    u = cnp.zeros((n, n), dtype=cnp.float64)
+    u[0, :] = 1.0
+    u[:, -1] = 0.5
+    w = np.zeros((n, n))
+    w[0, :] = 1.0
+    w[:, -1] = 0.5
+    for _ in range(7):
+        u[1:-1, 1:-1] = 0.25 * (u[:-2, 1:-1] + u[2:, 1:-1] + u[1:-1, :-2] + u[1:-1, 2:])
+        w[1:-1, 1:-1] = 0.25 * (w[:-2, 1:-1] + w[2:, 1:-1] + w[1:-1, :-2] + w[1:-1, 2:])
+    got = u.get(small_tiles)
+    assert np.array_equal(got, w)
+    assert small_tiles.array_info(u.name)["tile"] < n
+    st = small_tiles.stats()
+    assert st["compiled"] <= 4 and st["cache_hits"] >= 6
+
+
+def test_jacobi3d_sweeps_with_residual(small_tiles):
+    n = 20
+    u = cnp.random.uniform((n, n, n), seed=1, stream=0, low=0.0, high=1.0)
+    _faces(u, 0.0)
+    w = H.np_uniform(n * n * n, 1, 0, 0.0, 1.0).reshape(n, n, n)
+    _faces(w, 0.0)
+    c = 0.16666666666666666
+    for it in range(4):
+        old = u.copy()
+        u[1:-1, 1:-1, 1:-1] = c * (u[:-2, 1:-1, 1:-1] + u[2:, 1:-1, 1:-1] + u[1:-1, :-2, 1:-1]
+                                   + u[1:-1, 2:, 1:-1] + u[1:-1, 1:-1, :-2] + u[1:-1, 1:-1, 2:])
+        wold = w.copy()
+        w[1:-1, 1:-1, 1:-1] = c * (w[:-2, 1:-1, 1:-1] + w[2:, 1:-1, 1:-1] + w[1:-1, :-2, 1:-1]
+                                   + w[1:-1, 2:, 1:-1] + w[1:-1, 1:-1, :-2] + w[1:-1, 1:-1, 2:])
+        d = cnp.maxabs_diff(u, old).get(small_tiles).item()
+        assert d == np.max(np.abs(w - wold))
+        s = cnp.sumsq_diff(u, old).get(small_tiles).item()
+        ref = np.sum((w - wold) ** 2)
+        assert abs(s - ref) <= 1e-12 * ref
+    assert np.array_equal(u.get(small_tiles), w)
+
+
+def test_c1_statement_and_reductions(itf):
+    n = 1 << 20
+    x = cnp.random.uniform((n,), seed=0, stream=0, low=-1.0, high=1.0)
+    y = cnp.random.uniform((n,), seed=0, stream=1, low=-1.0, high=1.0)
+    z = ((2.5 * x) - (0.5 * y)) + (x * y)
+    hx, hy = H.np_uniform(n, 0, 0, -1.0, 1.0), H.np_uniform(n, 0, 1, -1.0, 1.0)
+    hz = ((2.5 * hx) - (0.5 * hy)) + (hx * hy)
+    assert np.array_equal(z.get(itf), hz)
+    s = cnp.sum(z).get(itf).item()
+    zz = (z @ z).get(itf).item()
+    import math
+    assert abs(s - math.fsum(hz)) <= 1e-12 * np.sum(np.abs(hz))
+    assert abs(zz - math.fsum(hz * hz)) <= 1e-12 * np.sum(hz * hz)
+
+
+def test_put_get_roundtrip_on_ragged_tiles(small_tiles):
+    rng = np.random.default_rng(11)
+    for shape, dt in [((200,), np.float64), ((37, 53), np.float32), ((9, 14, 21), np.int64),
+                      ((70, 70), np.int32)]:
+        host = (rng.standard_normal(shape) * 100).astype(dt)
+        a = cnp.array(host)
+        got = a.get(small_tiles)
+        assert got.dtype == dt and np.array_equal(got, host)
+        # and a strided view of it, copied out
+        key = tuple(slice(1, None, 2) for _ in shape)
+        assert np.array_equal(a[key].get(small_tiles), host[key])
+
+
+def test_integer_arithmetic_wraps_and_truncates(small_tiles):
+    host = np.array([7, -7, 2**31 - 1, -2**31, 5, -5, 0, 1] * 20, dtype=np.int32)
+    a = cnp.array(host)
+    with np.errstate(over="ignore"):
+        want = (host * np.int32(3) + np.int32(11))
+    assert np.array_equal((a * 3 + 11).get(small_tiles), want)
+    q = (a / 2).get(small_tiles)
+    assert np.array_equal(q, np.trunc(host / 2).astype(np.int32))
+
+
+def test_sigmoid_and_tanh_statement(itf):
+    n = 4096
+    hx = H.np_uniform(n, 9, 0, -8.0, 8.0)
+    x = cnp.array(hx)
+    s = 1.0 / (1.0 + cnp.exp(-x))
+    t = cnp.tanh(x)
+    import math
+    ws = np.array([1.0 / (1.0 + math.exp(v * -1)) for v in hx])
+    wt = np.array([math.tanh(v) for v in hx])
+    ds, dt = H.ulp_distance(s.get(itf), ws), H.ulp_distance(t.get(itf), wt)
+    lim = 0 if H.host_libm_is_the_restated_one() else 4
+    assert ds <= lim and dt <= min(lim, 1)
+
+
+def test_pending_reader_sees_the_old_contents(itf):
+    u = cnp.full((32,), 2.0)
+    t = u + 1.0
+    u[...] = 5.0
+    v = u + 1.0
+    assert np.array_equal(t.get(itf), np.full(32, 3.0))
+    assert np.array_equal(v.get(itf), np.full(32, 6.0))
+
+
+def test_view_of_view_assignment_and_inplace_update(small_tiles):
+    host = np.arange(400, dtype=np.float64).reshape(20, 20)
+    a = cnp.array(host)
+    v = a[2:18, 1:19][::2, 3:15:3]
+    v[1:, :] = 7.0
+    host[2:18, 1:19][::2, 3:15:3][1:, :] = 7.0
+    a[5, :] += a[6, :] * 2.0
+    host[5, :] += host[6, :] * 2.0
+    assert np.array_equal(a.get(small_tiles), host)

@@ -89,7 +89,7 @@ def test_exp_table_is_what_its_definition_gives():
 
 @pytest.mark.parametrize("variant", ["flat", "nd", "tiles"])
 def test_group_with_exp_and_tanh_builds_for_gfx950(variant):
-    b = AstBuilder(1, L.F64)
+    b = AstBuilder(L.F64, 1)
     lx = b.leaf(1)
     t0 = b.binary(L.OP_MUL, 100, lx, b.scalar(-1))
     t1 = b.unary(L.OP_EXP, 101, t0)
