@@ -605,6 +605,84 @@ def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=
     return out
 
 
+def run_frontend(n, steps, warmup):
+    """The same CG iteration and Jacobi sweeps written against the NumPy-like frontend: statements
+    -> DAG message -> host executor -> the same kernels. Shows what the whole stack costs on top of
+    the direct C ABI calls timed above (wall clock, flush + sync included)."""
+    import charmnumeric_amd as cnp
+    out = {}
+    cnp.reset()
+    itf = cnp.CharmNumericInterface(device=0)
+    itf.connect(odf=4)
+    try:
+        cnp.set_auto_flush(itf, 48)      # keep the device busy while later statements are recorded
+        A = cnp.random.cg_matrix(n, 2)
+        b = cnp.random.uniform((n,), seed=2, stream=1, low=-1.0, high=1.0)
+        x = cnp.zeros((n,))
+        r = b.copy()
+        p = b.copy()
+        rtr = r @ r
+
+        def iterate(k):
+            nonlocal x, r, p, rtr
+            for _ in range(k):
+                Ap = A @ p
+                pAp = p @ Ap
+                alpha = rtr / pAp
+                x = x + alpha * p
+                r = r - alpha * Ap
+                rtr_new = r @ r
+                beta = rtr_new / rtr
+                p = r + beta * p
+                rtr = rtr_new
+            cnp.execute(itf)
+            itf.sync()
+
+        iterate(warmup)
+        t0 = time.perf_counter()
+        iterate(steps)
+        dt = time.perf_counter() - t0
+        out["cg_iterations_per_s"] = round(steps / dt, 1)
+        out["cg_us_per_iteration"] = round(dt / steps * 1e6, 1)
+        out["cg_rtr_final"] = rtr.get(itf).item()
+        del A, b, x, r, p, rtr
+
+        for key, shape, sweeps in (("jacobi2d_8192", (8192, 8192), 100), ("jacobi3d_512", (512, 512, 512), 50)):
+            it16 = cnp.CharmNumericInterface(device=0)
+            it16.connect(odf=16 if len(shape) == 2 else 64)
+            cnp.set_auto_flush(it16, 48)
+            u = cnp.zeros(shape)
+            if len(shape) == 2:
+                u[0, :] = 1.0
+            else:
+                u[0, :, :] = 1.0
+
+            def sweep(k):
+                for _ in range(k):
+                    if len(shape) == 2:
+                        u[1:-1, 1:-1] = 0.25 * (u[:-2, 1:-1] + u[2:, 1:-1] + u[1:-1, :-2] + u[1:-1, 2:])
+                    else:
+                        u[1:-1, 1:-1, 1:-1] = 0.16666666666666666 * (
+                            u[:-2, 1:-1, 1:-1] + u[2:, 1:-1, 1:-1] + u[1:-1, :-2, 1:-1]
+                            + u[1:-1, 2:, 1:-1] + u[1:-1, 1:-1, :-2] + u[1:-1, 1:-1, 2:])
+                cnp.execute(it16)
+                it16.sync()
+
+            sweep(5)
+            t0 = time.perf_counter()
+            sweep(sweeps)
+            dt = time.perf_counter() - t0
+            out[key + "_us_per_sweep"] = round(dt / sweeps * 1e6, 1)
+            out[key + "_tile"] = it16.array_info(u.name)["tile"]
+            del u
+            cnp.execute(it16)
+            it16.close()
+    finally:
+        cnp.reset()
+        itf.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -671,6 +749,10 @@ def main():
             also["c5_lstm_forward"] = run_lstm(L)
         except Exception as exc:
             also["c5_error"] = str(exc)
+        try:
+            also["through_frontend"] = run_frontend(n, args.steps, args.warmup)
+        except Exception as exc:
+            also["frontend_error"] = str(exc)
         line["also"] = also
     if not args.no_cpu:
         cores = os.cpu_count() or 1

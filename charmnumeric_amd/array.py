@@ -175,7 +175,7 @@ class _ArrayLike:
 
     @property
     def size(self):
-        return _CallableInt(_size(self.shape))
+        return _CallableInt(self._n)
 
     @property
     def itemsize(self):
@@ -186,7 +186,7 @@ class _ArrayLike:
         return int(self.size) * self.itemsize
 
     def wire_dtype(self):
-        return lazy.wire_dtype(self.dtype)
+        return self._wire
 
     def __len__(self):
         return self.shape[0]
@@ -289,6 +289,8 @@ class Array(_ArrayLike):
         self.shape = tuple(shape)
         self.ndims = len(self.shape)
         self.dtype = np.dtype(dtype)
+        self._wire = lazy.wire_dtype(self.dtype)
+        self._n = _size(self.shape)
         self.name = lazy.new_name() if name is None else name
 
     def __del__(self):
@@ -304,7 +306,7 @@ class Array(_ArrayLike):
         return None
 
     def _ref(self, broadcast=False):
-        return lazy.ArrayRef(self.name, None, self.shape, self.ndims, self.wire_dtype(), broadcast)
+        return lazy.ArrayRef(self.name, None, self.shape, self.ndims, self._wire, broadcast)
 
     def get(self, interface):
         lazy.execute(interface)
@@ -321,6 +323,8 @@ class ArrayView(_ArrayLike):
         self.shape = region_shape(region)
         self.ndims = base.ndims
         self.dtype = base.dtype
+        self._wire = base._wire
+        self._n = _size(self.shape)
         if any(s == 0 for s in self.shape):
             raise NotImplementedError("zero-sized slices are not supported")
 
@@ -371,7 +375,7 @@ def _binary(opcode, lhs, rhs):
         if a.dtype != dtype:
             raise NotImplementedError(
                 f"elementwise operations across dtypes ({dtype} and {a.dtype}) are not implemented")
-    big = [a.shape for a in arrays if _size(a.shape) > 1]
+    big = [a.shape for a in arrays if a._n > 1]
     shape = tuple(big[0]) if big else tuple(arrays[0].shape)
     for other in big[1:]:
         if tuple(other) != shape:
@@ -380,7 +384,7 @@ def _binary(opcode, lhs, rhs):
     operands = []
     for x in (lhs, rhs):
         if isinstance(x, _ArrayLike):
-            bc = _size(x.shape) == 1 and _size(shape) > 1
+            bc = x._n == 1 and bool(big)
             if bc and not _is_whole(x._region(), x._base().shape):
                 raise NotImplementedError("a one-element slice cannot be used as a scalar operand")
             operands.append(x._ref(broadcast=bc))

@@ -76,11 +76,26 @@ def new_name():
     return n
 
 
+def _between_statements():
+    """True when what was recorded last is a complete statement: an assignment, a creation or a
+    non-elementwise operation, followed only by deletions. While an expression is being built the
+    last non-deletion is one of its elementwise operations, whose handle is alive only until the
+    expression is finished; flushing then would turn every such intermediate into a real array."""
+    p = _state.pending
+    i = len(p) - 1
+    while i >= 0 and p[i].kind == "delete":
+        i -= 1
+    return i >= 0 and p[i].kind != "op"
+
+
 def record(instr):
-    _state.pending.append(instr)
     af = _state.auto_flush
     if af is not None and not _state.flushing and len(_state.pending) >= af[1]:
-        execute(af[0])
+        # a program made of elementwise statements only has no such point: flush it anyway once
+        # the backlog is large
+        if _between_statements() or len(_state.pending) >= 16 * af[1]:
+            execute(af[0])
+    _state.pending.append(instr)
 
 
 def record_delete(name):
@@ -125,11 +140,13 @@ class _Group:
         self.names = set()
 
 
-def _uses_of(batch):
+def _uses_of(batch, dropped=()):
     """name -> indices of the instructions that read it; a negative index -(i+1) marks instruction
     i writing into it (assignment target), which always counts as a use from outside any group."""
     uses = {}
     for i, ins in enumerate(batch):
+        if i in dropped:
+            continue
         if ins.kind in ("op", "set", "nonfusible", "call"):
             for o in ins.operands:
                 if isinstance(o, ArrayRef):
@@ -148,7 +165,7 @@ def _plan(batch):
     forced = set()                      # op results that must be materialised
 
     while True:
-        uses = _uses_of([ins if i not in dropped else Instr("nop") for i, ins in enumerate(batch)])
+        uses = _uses_of(batch, dropped)
         items, group_of = [], {}
         cur = None
         deferred = []
@@ -163,7 +180,7 @@ def _plan(batch):
             deferred.clear()
 
         for i, ins in enumerate(batch):
-            if i in dropped or ins.kind == "nop":
+            if i in dropped:
                 continue
             if ins.kind == "op":
                 reads_slice_of_own = cur is not None and any(
@@ -227,18 +244,33 @@ def _plan(batch):
 # serialisation (format: include/cnexec.h)
 
 
+_GLOBAL_REGION = struct.pack("<i", 1)
+_region_cache = {}
+
+
 def _region_bytes(region):
     if region is None:
-        return struct.pack("<i", 1)
-    start, stop, step = region
-    out = [struct.pack("<ii", 0, len(start))]
-    for d in range(len(start)):
-        out.append(struct.pack("<iii", int(start[d]), int(stop[d]), int(step[d])))
-    return b"".join(out)
+        return _GLOBAL_REGION
+    out = _region_cache.get(region)
+    if out is None:
+        start, stop, step = region
+        flat = [0, len(start)]
+        for d in range(len(start)):
+            flat += [int(start[d]), int(stop[d]), int(step[d])]
+        out = struct.pack("<%di" % len(flat), *flat)
+        if len(_region_cache) < 4096:
+            _region_cache[region] = out
+    return out
 
 
 def _full_region(shape):
     return (tuple(0 for _ in shape), tuple(int(s) for s in shape), tuple(1 for _ in shape))
+
+
+_NODE_HEAD = [struct.Struct("<8i%dd" % 1 if k == 0 else "<8i%did" % k) for k in range(3)]
+# one DAG node holding a single operand-less AST node (id, fusible, 1 node, 1 root | node | global
+# region | root 0)
+_LONE_NODE = struct.Struct("<4i8idii")
 
 
 class _NodeWriter:
@@ -278,11 +310,8 @@ class _NodeWriter:
     def to_bytes(self, node_id, fusible):
         out = [struct.pack("<iiii", node_id, 1 if fusible else 0, len(self.nodes), len(self.roots))]
         for (name, opcode, is_temp, is_scalar, is_bc, ndims, dtype, operands, scalar, oregs, region) in self.nodes:
-            out.append(struct.pack("<iiiiiiii", name, opcode, is_temp, is_scalar, is_bc, ndims, dtype,
-                                   len(operands)))
-            for o in operands:
-                out.append(struct.pack("<i", o))
-            out.append(struct.pack("<d", scalar))
+            out.append(_NODE_HEAD[len(operands)].pack(name, opcode, is_temp, is_scalar, is_bc, ndims, dtype,
+                                                      len(operands), *operands, scalar))
             for r in oregs:
                 out.append(_region_bytes(r))
             out.append(_region_bytes(region))
@@ -345,9 +374,7 @@ def _emit_instr(ins, node_id):
 
 
 def _emit_delete(name, node_id):
-    w = _NodeWriter()
-    w.op(name, OP_DELETE, False, 1, L.F64, [], [], None)
-    return w.to_bytes(node_id, False)
+    return _LONE_NODE.pack(node_id, 0, 1, 1, name, OP_DELETE, 0, 0, 0, 1, L.F64, 0, 0.0, 1, 0)
 
 
 def build_messages(batch):
@@ -403,6 +430,9 @@ def execute(interface):
         _state.flushing = False
 
 
+_WIRE = {np.dtype("float32"): L.F32, np.dtype("float64"): L.F64, np.dtype("int32"): L.I32,
+         np.dtype("int64"): L.I64}
+
+
 def wire_dtype(np_dtype):
-    return {np.dtype("float32"): L.F32, np.dtype("float64"): L.F64, np.dtype("int32"): L.I32,
-            np.dtype("int64"): L.I64}[np.dtype(np_dtype)]
+    return _WIRE[np.dtype(np_dtype)]

@@ -243,10 +243,27 @@ def test_get_checks_rank_size_and_dtype(itf):
     assert itf.get(2, a.name, 32, dtype=np.float64).shape == (32,)
 
 
-def test_auto_flush_threshold(itf):
+def test_auto_flush_happens_between_statements(itf):
     cnp.set_auto_flush(itf, 5)
     a = cnp.zeros((16,))
     for _ in range(6):
-        a[...] = a + 1.0
-    assert lazy.pending_count() < 5
-    assert len(lines(itf, "group")) >= 1
+        a[...] = (a + 1.0) * 2.0
+    assert lazy.pending_count() < 5 + 4                      # threshold + one statement
+    tr = itf.trace()
+    groups = [ln for ln in tr if ln.startswith("group")]
+    assert len(groups) >= 3
+    # a flush in the middle of an expression would have turned its temporaries into arrays
+    assert all("path=" in ln for ln in groups) and itf.stats()["live_arrays"] == 1
+
+
+def test_auto_flush_never_splits_a_stencil_statement(itf):
+    cnp.set_auto_flush(itf, 3)
+    u = cnp.zeros((64, 64))
+    u[0, :] = 1.0
+    for _ in range(10):
+        u[1:-1, 1:-1] = 0.25 * (u[:-2, 1:-1] + u[2:, 1:-1] + u[1:-1, :-2] + u[1:-1, 2:])
+    cnp.execute(itf)
+    groups = [ln for ln in itf.trace() if ln.startswith("group")]
+    assert len(groups) == 10 and all("pingpong" in g and "inputs=4" in g for g in groups)
+    st = itf.stats()
+    assert st["live_arrays"] == 1 and st["compiled"] == 1 and st["cache_hits"] == 9
