@@ -68,9 +68,9 @@ int direct_shape(const GroupProgram& p, const DirectConfig& cfg, DirectShape& sh
             err = "halo wider than 2";
             return -18;
         }
-    // measured on MI355X: 8 rows per lane for rank 2; 2 rows x 4 planes per lane for rank 3
+    // measured on MI355X: 2 rows per lane for rank 2; 2 rows x 4 planes per lane for rank 3
     sh.tx = 64;
-    sh.ry = nd == 3 ? 2 : 8;
+    sh.ry = 2;
     sh.rz = nd == 3 ? 4 : 1;
     if (cfg.tx > 0)
         sh.tx = cfg.tx;
@@ -138,6 +138,11 @@ std::string direct_source(const GroupProgram& p, const DirectConfig& cfg, std::s
     }
     s << "};\n";
     s << R"(
+// n / d for 0 <= n < 2^31 as a multiply and a shift; the host fills m and s.
+struct FDiv { unsigned d, m, s; };
+__device__ __forceinline__ int fdiv(int n, const FDiv& f) {
+    return (int)(((unsigned long long)(unsigned)n * f.m) >> f.s);
+}
 struct DirectArgs {
     const T* const* cur;   // tile table of the current contents (row-major tile grid)
     T* const* dst;         // tile table of the new contents
@@ -146,34 +151,205 @@ struct DirectArgs {
     int grid[3];           // tiles per dimension
     int rs[3], re[3];      // assigned region
     int tb[3];             // workgroups per tile along z, y, x
+    int sg[3];             // tiles per ordering group along z, y, x
     int nblocks;
+    int nblocks8;          // nblocks / 8 when that is exact, else 0
+    int stagger;           // rotation of the order inside group g by (g % 8) * stagger workgroups
+    FDiv per_group;        // workgroups per ordering group
+    FDiv ggrid1, ggrid2;   // ordering groups along y and x
+    FDiv grow, gcol;       // workgroups per group along x and y
+    FDiv tbz, tby, tbx;    // = tb[0], tb[1], tb[2]
 };
 typedef T P2 __attribute__((ext_vector_type(2)));
+typedef int I2 __attribute__((ext_vector_type(2)));
 
-__device__ __forceinline__ int xcd_remap(int b, int n) {
-    return (n % 8 == 0) ? (b % 8) * (n / 8) + b / 8 : b;
-}
 __device__ __forceinline__ int floordiv2(int v) { return v >= 0 ? v / 2 : -((-v + 1) / 2); }
 
+// A build that runs the lanes of a wavefront as coroutines on a host (bounds checking of this
+// source) supplies its own lane exchange and readfirstlane.
+#ifndef DR_HOST_BUILD
+// Value of the same register in the previous / next lane of the wavefront (whole-wave shift by
+// one lane; the first / last lane keeps its own value and is patched by the caller).
+__device__ __forceinline__ T from_prev_lane(T v) {
+    I2 a = __builtin_bit_cast(I2, v), r;
+    r[0] = __builtin_amdgcn_update_dpp(a[0], a[0], 0x138, 0xf, 0xf, false);
+    r[1] = __builtin_amdgcn_update_dpp(a[1], a[1], 0x138, 0xf, 0xf, false);
+    return __builtin_bit_cast(T, r);
+}
+__device__ __forceinline__ T from_next_lane(T v) {
+    I2 a = __builtin_bit_cast(I2, v), r;
+    r[0] = __builtin_amdgcn_update_dpp(a[0], a[0], 0x130, 0xf, 0xf, false);
+    r[1] = __builtin_amdgcn_update_dpp(a[1], a[1], 0x130, 0xf, 0xf, false);
+    return __builtin_bit_cast(T, r);
+}
+__device__ __forceinline__ int wave_uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+#endif
+
+// Where a workgroup works: tile, tile extents, origin, and the patch inside the tile.
+struct Place {
+    int t, t0, t1, t2;           // tile index and coordinates
+    int bx, by, bz;              // workgroup inside the tile
+    int tz0, ty0, tx0;           // tile origin
+    int w0, w1, w2;              // tile extents
+};
+// Consecutive workgroup ids go round the 8 XCDs; give every XCD one contiguous run instead.
+__device__ __forceinline__ int xcd_order(const DirectArgs& a, int b) {
+    return a.nblocks8 ? (b & 7) * a.nblocks8 + (b >> 3) : b;
+}
+__device__ __forceinline__ Place locate(const DirectArgs& a, int blk) {
+    // Workgroups are ordered group by group (a group is sg^3 neighbouring tiles, so that what
+    // the tiles of a group re-read from each other stays in one L2), and inside a group x
+    // fastest, then y, then z across the whole group.
+    const int g = fdiv(blk, a.per_group);
+    // Groups that run at the same time start at different places of their tiles, so that they do
+    // not walk through the same address offsets in step.
+    int w = blk - g * (int)a.per_group.d + (g & 7) * a.stagger;
+    if (w >= (int)a.per_group.d) w -= (int)a.per_group.d;
+    const int gq = fdiv(g, a.ggrid2), g2 = g - gq * (int)a.ggrid2.d;
+    const int g0 = fdiv(gq, a.ggrid1), g1 = gq - g0 * (int)a.ggrid1.d;
+    const int wq = fdiv(w, a.grow), bxx = w - wq * (int)a.grow.d;
+    const int bzz = fdiv(wq, a.gcol), byy = wq - bzz * (int)a.gcol.d;
+    const int ix = fdiv(bxx, a.tbx), iy = fdiv(byy, a.tby), iz = fdiv(bzz, a.tbz);
+    Place p;
+    p.bx = bxx - ix * a.tb[2]; p.by = byy - iy * a.tb[1]; p.bz = bzz - iz * a.tb[0];
+    p.t0 = g0 * a.sg[0] + iz; p.t1 = g1 * a.sg[1] + iy; p.t2 = g2 * a.sg[2] + ix;
+    p.t = (p.t0 * a.grid[1] + p.t1) * a.grid[2] + p.t2;
+    p.tz0 = p.t0 * a.tile; p.ty0 = p.t1 * a.tile; p.tx0 = p.t2 * a.tile;
+    p.w0 = min(a.tile, a.shape[0] - p.tz0); p.w1 = min(a.tile, a.shape[1] - p.ty0);
+    p.w2 = min(a.tile, a.shape[2] - p.tx0);
+    return p;
+}
+
+// A wavefront takes the fast path when it is one run of 64 column pairs of one row group, its
+// rows and planes plus halo lie inside the tile, and all its rows and planes are assigned. Only
+// the x direction then needs care: the pairs to the left and right of a lane are its neighbour
+// lanes' centre pairs, and the two end lanes read theirs from the tile or its x neighbour.
+#define DR_WAVE_ROWS (DR_TX % 64 == 0)
+__device__ __forceinline__ bool wave_is_fast(const DirectArgs& a, const Place& p, int lz0, int ly0,
+                                             int x0) {
+    return DR_WAVE_ROWS && DR_HK == 1 && x0 + 128 <= p.w2 &&
+           ly0 - DR_H1 >= 0 && ly0 + DR_RY + DR_H1 <= p.w1 &&
+           lz0 - DR_H0 >= 0 && lz0 + DR_RZ + DR_H0 <= p.w0 &&
+           p.ty0 + ly0 >= a.rs[1] && p.ty0 + ly0 + DR_RY <= a.re[1] &&
+           p.tz0 + lz0 >= a.rs[0] && p.tz0 + lz0 + DR_RZ <= a.re[0];
+}
+
 template <bool NTS>
-__device__ __forceinline__ void direct_run(const DirectArgs& a, const T* s) {
-    // ---- which tile, which patch of it (all workgroup-uniform) ----
-    const int per_tile = a.tb[0] * a.tb[1] * a.tb[2];
-    const int blk = xcd_remap((int)blockIdx.x, a.nblocks);
-    const int t = blk / per_tile, w = blk - t * per_tile;
-    const int t2 = t % a.grid[2], t1 = (t / a.grid[2]) % a.grid[1], t0 = t / (a.grid[2] * a.grid[1]);
-    const int bx = w % a.tb[2], by = (w / a.tb[2]) % a.tb[1], bz = w / (a.tb[2] * a.tb[1]);
-    const int tz0 = t0 * a.tile, ty0 = t1 * a.tile, tx0 = t2 * a.tile;   // tile origin
-    const int w0 = min(a.tile, a.shape[0] - tz0), w1 = min(a.tile, a.shape[1] - ty0),
-              w2 = min(a.tile, a.shape[2] - tx0);                         // tile extents
+__device__ __forceinline__ void direct_fast(const DirectArgs& a, const T* s) {
+    const Place p = locate(a, xcd_order(a, (int)blockIdx.x));
+    const int tid = (int)threadIdx.x;
+    const int wv = wave_uniform(tid >> 6);              // wavefront inside the workgroup
+    const int lane = tid & 63;
+    const int lz0 = p.bz * DR_RZ;
+    const int ly0 = (p.by * DR_TY + (wv * 64) / DR_TX) * DR_RY;
+    const int x0 = (p.bx * DR_TX + (wv * 64) % DR_TX) * 2;   // first column of the wavefront
+    if (lz0 >= p.w0 || ly0 >= p.w1 || x0 >= p.w2) return;
+    if (!wave_is_fast(a, p, lz0, ly0, x0)) return;
+    const int w1 = p.w1, w2 = p.w2;
+    const int lx = x0 + 2 * lane;
+    const T* const own = a.cur[p.t];
+    const int origin = ((lz0 - DR_H0) * w1 + (ly0 - DR_H1)) * w2;   // window origin, column 0
+    const T* const pc = own + origin + lx;
+    // where the end lanes find the pair before column x0 and the pair after column x0+127
+    const T* lp = own + origin + x0;      // fallback: an address that exists (value unused)
+    int ls = w2;
+    if (x0 >= 2) lp = own + origin + (x0 - 2);
+    else if (p.t2 > 0) { ls = a.tile; lp = a.cur[p.t - 1] + ((lz0 - DR_H0) * w1 + (ly0 - DR_H1)) * ls + (a.tile - 2); }
+    const T* rp = own + origin + (x0 + 126);
+    int rstr = w2;
+    if (x0 + 130 <= w2) rp = own + origin + (x0 + 128);
+    else if (p.t2 + 1 < a.grid[2]) {
+        rstr = min(a.tile, a.shape[2] - p.tx0 - a.tile);
+        rp = a.cur[p.t + 1] + ((lz0 - DR_H0) * w1 + (ly0 - DR_H1)) * rstr;
+    }
+    const bool first = lane == 0, last = lane == 63;
+
+    // All loads first, none under a branch: the two end lanes of the wavefront fetch the pair
+    // beyond their end, every other lane re-reads its own centre pair (a cache hit), so each row
+    // costs one more full-wave load and the wavefront waits for memory once.
+    P2 win[DR_WZ][DR_WY][DR_WK];
+    P2 beyond[DR_WZ][DR_WY];
+#pragma unroll
+    for (int i = 0; i < DR_WZ; ++i)
+#pragma unroll
+        for (int j = 0; j < DR_WY; ++j)
+            if (DR_NEED[i][j][0] || DR_NEED[i][j][DR_HK] || DR_NEED[i][j][DR_WK - 1])
+                win[i][j][DR_HK] = *reinterpret_cast<const P2*>(pc + (i * w1 + j) * w2);
+#pragma unroll
+    for (int i = 0; i < DR_WZ; ++i)
+#pragma unroll
+        for (int j = 0; j < DR_WY; ++j)
+            if (DR_NEED[i][j][0] || DR_NEED[i][j][DR_WK - 1]) {
+                const T* src = pc + (i * w1 + j) * w2;
+                src = first ? lp + (i * w1 + j) * ls : src;
+                src = last ? rp + (i * w1 + j) * rstr : src;
+                beyond[i][j] = *reinterpret_cast<const P2*>(src);
+            }
+#pragma unroll
+    for (int i = 0; i < DR_WZ; ++i)
+#pragma unroll
+        for (int j = 0; j < DR_WY; ++j) {
+            if (DR_NEED[i][j][0]) {
+                P2 sh;
+                sh[0] = from_prev_lane(win[i][j][DR_HK][0]);
+                sh[1] = from_prev_lane(win[i][j][DR_HK][1]);
+                win[i][j][0] = first ? beyond[i][j] : sh;
+            }
+            if (DR_NEED[i][j][DR_WK - 1]) {
+                P2 sh;
+                sh[0] = from_next_lane(win[i][j][DR_HK][0]);
+                sh[1] = from_next_lane(win[i][j][DR_HK][1]);
+                win[i][j][DR_WK - 1] = last ? beyond[i][j] : sh;
+            }
+        }
+    T* const out_tile = a.dst[p.t];
+#pragma unroll
+    for (int rz = 0; rz < DR_RZ; ++rz)
+#pragma unroll
+        for (int ry = 0; ry < DR_RY; ++ry) {
+            P2 res;
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                T l[NLA], o[NOA];
+#pragma unroll
+                for (int q = 0; q < NL; ++q) {
+                    const int xx = e + DR_SHIFT[q][2];
+                    l[q] = win[rz + DR_H0 + DR_SHIFT[q][0]][ry + DR_H1 + DR_SHIFT[q][1]]
+                              [DR_HK + floordiv2(xx)][xx & 1];
+                }
+                group_eval(l, s, o);
+                const int gx = p.tx0 + lx + e;
+                res[e] = (gx >= a.rs[2] && gx < a.re[2]) ? o[0] : win[rz + DR_H0][ry + DR_H1][DR_HK][e];
+            }
+            P2* out = reinterpret_cast<P2*>(out_tile + (((lz0 + rz) * w1 + (ly0 + ry)) * w2 + lx));
+            if (NTS) __builtin_nontemporal_store(res, out); else *out = res;
+        }
+}
+
+// Everything the fast path leaves (or, with skip_fast = 0, everything): windows that touch
+// neighbour tiles in y or z, partial tiles, rows and planes outside the assigned region,
+// workgroups narrower than a wavefront. With a list, workgroup i does position list[i] of the
+// order (the host lists the workgroups on the y and z faces of the tiles); without, all of them.
+template <bool NTS>
+__device__ __forceinline__ void direct_rest(const DirectArgs& a, const T* s, int skip_fast,
+                                            const int* list) {
+    const Place p = locate(a, list ? list[blockIdx.x] : xcd_order(a, (int)blockIdx.x));
+    const int t = p.t, t0 = p.t0, t1 = p.t1, t2 = p.t2;
+    const int tz0 = p.tz0, ty0 = p.ty0, tx0 = p.tx0, w0 = p.w0, w1 = p.w1, w2 = p.w2;
     // extents of the next tiles (the previous ones are always full)
     const int w0n = min(a.tile, a.shape[0] - tz0 - a.tile), w1n = min(a.tile, a.shape[1] - ty0 - a.tile),
               w2n = min(a.tile, a.shape[2] - tx0 - a.tile);
-    const int lz0 = bz * DR_RZ;
+    const int lz0 = p.bz * DR_RZ;
     if (lz0 >= w0) return;
     const int tid = (int)threadIdx.x;
-    const int lx = (bx * DR_TX + tid % DR_TX) * 2;
-    const int ly0 = (by * DR_TY + tid / DR_TX) * DR_RY;
+    if (skip_fast && DR_WAVE_ROWS) {
+        const int wv = wave_uniform(tid >> 6);
+        const int wy0 = (p.by * DR_TY + (wv * 64) / DR_TX) * DR_RY;
+        const int wx0 = (p.bx * DR_TX + (wv * 64) % DR_TX) * 2;
+        if (wy0 < w1 && wx0 < w2 && wave_is_fast(a, p, lz0, wy0, wx0)) return;
+    }
+    const int lx = (p.bx * DR_TX + tid % DR_TX) * 2;
+    const int ly0 = (p.by * DR_TY + tid / DR_TX) * DR_RY;
     if (lx >= w2 || ly0 >= w1) return;
 
     // ---- the 27 tile pointers around this tile (uniform); missing neighbours fall back to own ----
@@ -280,19 +456,19 @@ __device__ __forceinline__ void direct_run(const DirectArgs& a, const T* s) {
 #pragma unroll
                     for (int e = 0; e < 2; ++e) {
                         const int gx = tx0 + lx + e;
-                        if (yin && gx >= a.rs[2] && gx < a.re[2]) {
-                            T l[NLA], o[NOA];
+                        // evaluated for every element and selected afterwards: window entries an
+                        // unassigned element would read exist (clamped), and straight-line code
+                        // keeps all loads ahead of the arithmetic
+                        const bool in_region = yin && gx >= a.rs[2] && gx < a.re[2];
+                        T l[NLA], o[NOA];
 #pragma unroll
-                            for (int q = 0; q < NL; ++q) {
-                                const int xx = e + DR_SHIFT[q][2];
-                                l[q] = win[rz + DR_H0 + DR_SHIFT[q][0]][ry + DR_H1 + DR_SHIFT[q][1]]
-                                          [DR_HK + floordiv2(xx)][xx & 1];
-                            }
-                            group_eval(l, s, o);
-                            res[e] = o[0];
-                        } else {
-                            res[e] = win[rz + DR_H0][ry + DR_H1][DR_HK][e];
+                        for (int q = 0; q < NL; ++q) {
+                            const int xx = e + DR_SHIFT[q][2];
+                            l[q] = win[rz + DR_H0 + DR_SHIFT[q][0]][ry + DR_H1 + DR_SHIFT[q][1]]
+                                      [DR_HK + floordiv2(xx)][xx & 1];
                         }
+                        group_eval(l, s, o);
+                        res[e] = in_region ? o[0] : win[rz + DR_H0][ry + DR_H1][DR_HK][e];
                     }
                     P2* out = reinterpret_cast<P2*>(out_tile + ((lz * w1 + ly) * w2 + lx));
                     if (NTS) __builtin_nontemporal_store(res, out); else *out = res;
@@ -302,13 +478,24 @@ __device__ __forceinline__ void direct_run(const DirectArgs& a, const T* s) {
     }
 }
 
-extern "C" __global__ __launch_bounds__(256) void grp_direct(DirectArgs a, Scal sc) {
+// nts: the written stream is not read back soon, store it non-temporally.
+extern "C" __global__ __launch_bounds__(256) void grp_direct_fast(DirectArgs a, Scal sc) {
     T s[NSA]; load_scalars(sc, s);
-    direct_run<false>(a, s);
+    direct_fast<false>(a, s);
 }
-extern "C" __global__ __launch_bounds__(256) void grp_direct_nts(DirectArgs a, Scal sc) {
+extern "C" __global__ __launch_bounds__(256) void grp_direct_fast_nts(DirectArgs a, Scal sc) {
     T s[NSA]; load_scalars(sc, s);
-    direct_run<true>(a, s);
+    direct_fast<true>(a, s);
+}
+extern "C" __global__ __launch_bounds__(256) void grp_direct_rest(DirectArgs a, Scal sc, int skip_fast,
+                                                                  const int* list) {
+    T s[NSA]; load_scalars(sc, s);
+    direct_rest<false>(a, s, skip_fast, list);
+}
+extern "C" __global__ __launch_bounds__(256) void grp_direct_rest_nts(DirectArgs a, Scal sc, int skip_fast,
+                                                                      const int* list) {
+    T s[NSA]; load_scalars(sc, s);
+    direct_rest<true>(a, s, skip_fast, list);
 }
 )";
     return s.str();

@@ -584,14 +584,34 @@ int try_launch_slide(cnh_kernel* k, const std::vector<const cnh_tiled*>& arrays,
     return 0;
 }
 
+struct FDivDev {
+    uint32_t d, m, s;
+};
+// n / d == (n * m) >> s for 0 <= n < 2^31: s = 31 + ceil(log2 d), m = ceil(2^s / d) < 2^32.
+FDivDev fdiv_make(uint32_t d) {
+    if (d == 0)
+        d = 1;
+    uint32_t L = 0;
+    while ((1ull << L) < d)
+        ++L;
+    FDivDev f;
+    f.d = d;
+    f.s = 31 + L;
+    f.m = (uint32_t)(((1ull << f.s) + d - 1) / d);
+    return f;
+}
 struct DirectArgsDev {
     const void* cur;
     void* dst;
-    int32_t tile, shape[3], grid[3], rs[3], re[3], tb[3], nblocks;
+    int32_t tile, shape[3], grid[3], rs[3], re[3], tb[3], sg[3], nblocks, nblocks8, stagger;
+    FDivDev per_group, ggrid1, ggrid2, grow, gcol, tbz, tby, tbx;
 };
-static_assert(sizeof(DirectArgsDev) == 88, "DirectArgsDev layout must match the generated struct");
+static_assert(sizeof(DirectArgsDev) == 16 + 4 * 22 + 12 * 8, "DirectArgsDev layout must match the generated struct");
 
 int g_stencil_mode = 2; // 0 = general gather, 1 = LDS sliding window, 2 = register window
+int g_direct_group = 0; // order workgroups by groups of neighbouring tiles (rank 3)
+int g_direct_lean = -1;   // wavefront-level lean kernel: 1 on, 0 off, -1 by rank
+int g_direct_stagger = 0; // concurrent groups start at different offsets of their tiles
 DirectConfig g_direct_cfg;
 
 // Launches the register-window variant under the same conditions as the sliding window, plus:
@@ -657,6 +677,30 @@ int try_launch_direct(cnh_kernel* k, const std::vector<const cnh_tiled*>& arrays
     CNH_CHECK(blocks > 0 && blocks < (1ll << 31), -3, "stencil launch of %lld workgroups",
               (long long)blocks);
     a.nblocks = (int)blocks;
+    a.nblocks8 = blocks % 8 == 0 ? (int)(blocks / 8) : 0;
+    // Ordering groups: G^3 neighbouring full tiles whose joint z-slab still fits an L2 (edge of a
+    // group at most 256 elements), G as large as the grid allows. Rank 3 only.
+    int G = 1;
+    if (nd == 3 && g_direct_group) {
+        for (int cand = 2; cand <= 4; cand *= 2) {
+            bool ok = (int64_t)cand * a.tile <= 256;
+            for (int d = 0; d < 3 && ok; ++d)
+                ok = a.grid[d] % cand == 0 && a.shape[d] == a.grid[d] * a.tile;
+            if (ok)
+                G = cand;
+        }
+    }
+    for (int d = 0; d < 3; ++d)
+        a.sg[d] = (d >= pad) ? G : 1;
+    a.per_group = fdiv_make((uint32_t)(per_tile * a.sg[0] * a.sg[1] * a.sg[2]));
+    a.ggrid1 = fdiv_make((uint32_t)(a.grid[1] / a.sg[1]));
+    a.ggrid2 = fdiv_make((uint32_t)(a.grid[2] / a.sg[2]));
+    a.grow = fdiv_make((uint32_t)(a.tb[2] * a.sg[2]));
+    a.gcol = fdiv_make((uint32_t)(a.tb[1] * a.sg[1]));
+    a.tbz = fdiv_make((uint32_t)a.tb[0]);
+    a.tby = fdiv_make((uint32_t)a.tb[1]);
+    a.tbx = fdiv_make((uint32_t)a.tb[2]);
+    a.stagger = g_direct_stagger ? (int)(a.per_group.d / 8) : 0;
     const void* dcur = nullptr;
     const void* ddst = nullptr;
     if (int rc = desc_upload(cur->tiles, (size_t)ntiles * sizeof(void*), st, &dcur))
@@ -666,12 +710,77 @@ int try_launch_direct(cnh_kernel* k, const std::vector<const cnh_tiled*>& arrays
     a.cur = dcur;
     a.dst = const_cast<void*>(ddst);
     const bool nt_stores = volume * 16 >= (128ll << 20); // the written stream is not read back soon
+    // Two launches over the same grid: wavefronts that lie inside their tile in y and z take the
+    // lean kernel, the other kernel does what is left (all of it when the lean one does not apply).
+    // measured on MI355X: the lean kernel pays off for rank 2 (tiles much wider than a wavefront
+    // run); with 128-wide tiles of rank 3 every wavefront reads both x neighbours and it does not
+    const bool want_lean = g_direct_lean < 0 ? nd == 2 : g_direct_lean != 0;
+    const bool lean = want_lean && sh.tx % 64 == 0 && sh.halo[2] >= 1;
+    int skip_fast = lean ? 1 : 0;
     hipFunction_t fn;
-    if (int rc = get_function(k, g_direct_cfg.variant(), nt_stores ? "grp_direct_nts" : "grp_direct", &fn))
+    if (lean) {
+        if (int rc = get_function(k, g_direct_cfg.variant(),
+                                  nt_stores ? "grp_direct_fast_nts" : "grp_direct_fast", &fn))
+            return rc;
+        void* params[] = {&a, const_cast<unsigned char*>(scal.data())};
+        if (int rc = launch(fn, blocks, params, st))
+            return rc;
+    }
+    if (int rc = get_function(k, g_direct_cfg.variant(),
+                              nt_stores ? "grp_direct_rest_nts" : "grp_direct_rest", &fn))
         return rc;
-    void* params[] = {&a, const_cast<unsigned char*>(scal.data())};
-    if (int rc = launch(fn, blocks, params, st))
-        return rc;
+    // When every workgroup away from the y and z faces of its tile consists of wavefronts the
+    // lean kernel takes, the second launch covers the face workgroups only.
+    const void* dlist = nullptr;
+    int64_t rest_blocks = blocks;
+    bool faces_only = lean && a.shape[2] % 128 == 0;
+    for (int d = 0; d < 2 && faces_only; ++d) {
+        // a partial last tile ends before its last workgroup row: its end is not on the list
+        if (a.grid[d] > 1 && a.shape[d] != a.grid[d] * a.tile)
+            faces_only = false;
+        else if (sh.halo[d] > 0)
+            faces_only = a.rs[d] <= ext[d] && a.re[d] >= a.shape[d] - ext[d];
+        else
+            faces_only = a.rs[d] == 0 && a.re[d] == a.shape[d];
+    }
+    std::vector<int32_t> list;
+    if (faces_only) {
+        // positions in the order locate() decodes: group by group, x fastest inside a group
+        const int gx = a.tb[2] * a.sg[2], gy = a.tb[1] * a.sg[1], gz = a.tb[0] * a.sg[0];
+        const int64_t per_group = (int64_t)gx * gy * gz;
+        const int64_t ngroups = blocks / per_group;
+        for (int64_t g = 0; g < ngroups; ++g)
+            for (int z = 0; z < gz; ++z) {
+                const int bz = z % a.tb[0];
+                const bool zf = sh.halo[0] > 0 && (bz == 0 || bz == a.tb[0] - 1);
+                for (int y = 0; y < gy; ++y) {
+                    const int by = y % a.tb[1];
+                    const bool yf = sh.halo[1] > 0 && (by == 0 || by == a.tb[1] - 1);
+                    if (!zf && !yf)
+                        continue;
+                    for (int x = 0; x < gx; ++x) {
+                        // undo the stagger: position w' = w + (g & 7) * stagger (mod per_group)
+                        int64_t w = ((int64_t)z * gy + y) * gx + x;
+                        int64_t pos = w - (int64_t)(g & 7) * a.stagger;
+                        if (pos < 0)
+                            pos += per_group;
+                        list.push_back((int32_t)(g * per_group + pos));
+                    }
+                }
+            }
+        if (list.empty())
+            rest_blocks = 0;
+        else {
+            if (int rc = desc_upload(list.data(), list.size() * sizeof(int32_t), st, &dlist))
+                return rc;
+            rest_blocks = (int64_t)list.size();
+        }
+    }
+    if (rest_blocks > 0) {
+        void* params[] = {&a, const_cast<unsigned char*>(scal.data()), &skip_fast, &dlist};
+        if (int rc = launch(fn, rest_blocks, params, st))
+            return rc;
+    }
     *handled = true;
     return 0;
 }
@@ -684,6 +793,18 @@ extern "C" int cnh_set_option(const char* name, int value) {
         CNH_CHECK(value >= 0 && value <= 2, -2, "stencil_mode must be 0, 1 or 2");
         g_stencil_mode = value;
         g_slide_enabled = value == 1;
+        return 0;
+    }
+    if (std::strcmp(name, "direct_lean") == 0) {
+        g_direct_lean = value;
+        return 0;
+    }
+    if (std::strcmp(name, "direct_stagger") == 0) {
+        g_direct_stagger = value != 0;
+        return 0;
+    }
+    if (std::strcmp(name, "direct_group") == 0) {
+        g_direct_group = value != 0;
         return 0;
     }
     if (std::strcmp(name, "direct_tx") == 0) {
