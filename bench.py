@@ -605,6 +605,35 @@ def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=
     return out
 
 
+def cpu_jacobi(nd, n, tile, sweeps, threads):
+    """The same sweep on the host through the oracle's chare-by-chare restatement of the reference
+    path (halo pack + delivery, aligned cells, one interpreted kernel per cell, SET_REGION copy),
+    `threads` chares side by side. A bounded sample: `sweeps` sweeps of the full-size array."""
+    from charmnumeric_amd import _lib as L
+    from oracle import cn_oracle as O
+
+    orc = O.Oracle()
+    ast = jacobi_ast(L, nd, n)
+    g = (n + tile - 1) // tile
+    tiles = []
+    for idx in np.ndindex(*([g] * nd)):
+        ext = [min(tile, n - i * tile) for i in idx]
+        t = np.zeros(ext)
+        if idx[0] == 0:
+            t[0] = 1.0
+        tiles.append(t)
+    t0 = time.perf_counter()
+    for _ in range(sweeps):
+        rc, st = orc.world_group(ast, L.F64, (n,) * nd, tile, tiles, threads)
+        if rc:
+            raise RuntimeError(f"oracle world sweep failed: {rc}")
+    dt = time.perf_counter() - t0
+    return {"us_per_sweep": round(dt / sweeps * 1e6, 1), "threads": threads, "sweeps": sweeps,
+            "messages_per_sweep": st["messages"], "halo_bytes_per_sweep": st["bytes"],
+            "kernel_calls_per_sweep": st["kernels"],
+            "what": "oracle restatement of the reference's fragment path, one thread per chare"}
+
+
 def run_frontend(n, steps, warmup):
     """The same CG iteration and Jacobi sweeps written against the NumPy-like frontend: statements
     -> DAG message -> host executor -> the same kernels. Shows what the whole stack costs on top of
@@ -766,6 +795,12 @@ def main():
                       f"oracle kernels, tile matvec split over {threads} threads",
             "one_core": round(ips1, 3),
         }
+        if not args.no_also and "also" in line:
+            try:
+                line["also"]["c3_jacobi2d_8192"]["cpu_port"] = cpu_jacobi(2, 8192, 2048, 3, threads)
+                line["also"]["c4_jacobi3d_512"]["cpu_port"] = cpu_jacobi(3, 512, 128, 2, threads)
+            except Exception as exc:
+                line["also"]["cpu_port_error"] = str(exc)
         if args.cpu_iters == args.steps and cg.get("x") is not None:
             # same system, same number of iterations: the two solutions must agree
             line["cg_parity_max_rel_diff"] = float(np.max(np.abs(cg["x"] - xc)) / np.max(np.abs(xc)))

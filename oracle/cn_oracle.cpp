@@ -1337,3 +1337,282 @@ void orc_fill_cg_matrix(double* out, int64_t n, int64_t row0, int64_t nrows, int
 }
 
 } // extern "C"
+
+// ---------------------------------------------------------------------------------------------
+// One fused SET_REGION group over one tiled array, carried out chare by chare the way the
+// reference does it: every chare packs the pieces of its tile that other chares' shifted
+// operands need (send_remote_inputs + send_remote_input, src/executor_core.cpp:8-143,684-690),
+// the receiving chare lists its local fragment and the received buffers per operand, refines them
+// into aligned cells, runs the group once per cell into a packed result buffer
+// (src/execute_node.cpp:1376-1585) and finally copies the buffer into its tile
+// (SET_REGION, src/executor_ast_visitor.cpp:268-311). Offsets 0, every leaf is the assigned array.
+// ---------------------------------------------------------------------------------------------
+namespace {
+
+struct RemoteBuffer {
+    int input_index;
+    orc_region region;
+    std::vector<char> data;
+};
+
+int tile_count(const orc_decomp& dc, int d) { return orc_decomp_num_chares(&dc, d); }
+
+} // namespace
+
+extern "C" int orc_world_group(const orc_ast* ast, int dtype, int nd, const int32_t* shape, int tile,
+                               void* const* tiles, int threads, int64_t* stats) {
+    if (nd < 1 || nd > ORC_MAX_ND || dtype < 0 || dtype > 3)
+        return -2;
+    const int esz = (dtype == ORC_F32 || dtype == ORC_I32) ? 4 : 8;
+    Program p = build_program(ast);
+    if (p.err)
+        return p.err;
+    if (p.out_roots.size() != 1)
+        return -3;
+    const orc_ast_node& root = ast->nodes[ast->roots[p.out_roots[0]]];
+    if (root.opcode != ORC_OP_SET_REGION || root.region.is_global || !p.bcast_nodes.empty())
+        return -3;
+    const int target = ast->nodes[root.operands[0]].result_name;
+    const orc_region r_out = root.region;
+    const int K = (int)p.leaves.size();
+    std::vector<orc_region> inputs(K);
+    for (int k = 0; k < K; ++k) {
+        const orc_ast_node& leaf = ast->nodes[p.leaves[k].node];
+        const orc_ast_node& user = ast->nodes[ast->roots[p.leaves[k].root]];
+        if (leaf.result_name != target || !user.has_operand_region[p.leaves[k].operand])
+            return -3;
+        inputs[k] = user.operand_regions[p.leaves[k].operand];
+    }
+    orc_decomp dc;
+    std::memset(&dc, 0, sizeof dc);
+    dc.ndims = nd;
+    dc.tile = tile;
+    int grid[ORC_MAX_ND] = {1, 1, 1};
+    int64_t nchares = 1;
+    for (int d = 0; d < nd; ++d) {
+        dc.global_shape[d] = shape[d];
+        grid[d] = tile_count(dc, d);
+        nchares *= grid[d];
+    }
+    std::vector<orc_decomp> in_dc(K, dc);
+    auto chare_index = [&](int64_t c, int32_t* idx) {
+        for (int d = nd - 1; d >= 0; --d) {
+            idx[d] = (int32_t)(c % grid[d]);
+            c /= grid[d];
+        }
+    };
+    auto chare_flat = [&](const int32_t* idx) {
+        int64_t c = 0;
+        for (int d = 0; d < nd; ++d)
+            c = c * grid[d] + idx[d];
+        return c;
+    };
+    auto tile_strides = [&](const orc_region& chare, int64_t* st) {
+        int64_t sdim = 1;
+        for (int d = nd - 1; d >= 0; --d) {
+            st[d] = sdim;
+            sdim *= rsize(chare, d);
+        }
+    };
+    int64_t n_msgs = 0, n_bytes = 0, n_kernels = 0, n_cells_max = 0;
+
+    // ---- phase 1: every chare packs and "sends" what others need from its tile ----
+    std::vector<std::vector<RemoteBuffer>> inbox((size_t)nchares);
+    for (int64_t c = 0; c < nchares; ++c) {
+        int32_t idx[ORC_MAX_ND] = {0, 0, 0};
+        chare_index(c, idx);
+        orc_region chare;
+        orc_decomp_chare_region_global(&dc, idx, &chare);
+        int64_t cst[ORC_MAX_ND];
+        tile_strides(chare, cst);
+        const int cap = 4096;
+        std::vector<int32_t> targets((size_t)cap * nd), which(cap);
+        std::vector<orc_region> regs(cap);
+        int ns = orc_send_remote_inputs(&r_out, K, inputs.data(), idx, &dc, in_dc.data(), cap,
+                                        targets.data(), regs.data(), which.data());
+        if (ns < 0)
+            return -4;
+        for (int m = 0; m < ns; ++m) {
+            RemoteBuffer rb;
+            rb.input_index = which[m];
+            rb.region = regs[m];
+            int64_t counts[ORC_MAX_ND], sstart[ORC_MAX_ND], sstep[ORC_MAX_ND], dstart[ORC_MAX_ND],
+                dstep[ORC_MAX_ND], dstr[ORC_MAX_ND];
+            int64_t total = 1;
+            for (int d = 0; d < nd; ++d) {
+                counts[d] = rsize(regs[m], d);
+                total *= counts[d];
+            }
+            int64_t sdim = 1;
+            for (int d = nd - 1; d >= 0; --d) {
+                dstr[d] = sdim;
+                sdim *= counts[d];
+                sstart[d] = regs[m].start[d] - chare.start[d];
+                sstep[d] = regs[m].step[d];
+                dstart[d] = 0;
+                dstep[d] = 1;
+            }
+            rb.data.resize((size_t)total * esz);
+            orc_copy_region(nd, esz, rb.data.data(), dstr, dstart, dstep, tiles[c], cst, sstart, sstep,
+                            counts);
+            n_msgs++;
+            n_bytes += total * esz;
+            inbox[(size_t)chare_flat(&targets[(size_t)m * nd])].push_back(std::move(rb));
+        }
+    }
+
+    // ---- phases 2 and 3 per chare: fragments -> aligned cells -> kernels -> SET_REGION copy ----
+    std::vector<int> rc_of((size_t)nchares, 0);
+    std::vector<int64_t> kern_of((size_t)nchares, 0), cells_of((size_t)nchares, 0);
+    std::vector<std::vector<char>> results((size_t)nchares);
+    std::vector<orc_region> myouts((size_t)nchares);
+    std::vector<char> has_out((size_t)nchares, 0);
+    run_blocks(nchares, threads, [&](int64_t c0, int64_t c1) {
+        for (int64_t c = c0; c < c1; ++c) {
+            int32_t idx[ORC_MAX_ND] = {0, 0, 0};
+            chare_index(c, idx);
+            orc_region chare, myout;
+            orc_decomp_chare_region_global(&dc, idx, &chare);
+            if (!orc_region_intersect(&r_out, &chare, &myout))
+                continue;
+            has_out[(size_t)c] = 1;
+            myouts[(size_t)c] = myout;
+            std::vector<orc_region> my_inputs(K);
+            int expected = 0;
+            if (orc_local_inputs(&r_out, K, inputs.data(), idx, &dc, in_dc.data(), my_inputs.data(),
+                                 &expected) < 0) {
+                rc_of[(size_t)c] = -5;
+                continue;
+            }
+            if (expected != (int)inbox[(size_t)c].size()) {
+                rc_of[(size_t)c] = -6; // planner inconsistency: sends do not match expectations
+                continue;
+            }
+            int64_t cst[ORC_MAX_ND];
+            tile_strides(chare, cst);
+            std::vector<orc_fragment> frags;
+            std::vector<const char*> bases;
+            std::vector<int32_t> begin(K + 1, 0);
+            for (int k = 0; k < K; ++k) {
+                begin[k] = (int32_t)frags.size();
+                orc_region local;
+                if (orc_region_intersect(&my_inputs[k], &chare, &local)) {
+                    orc_fragment f;
+                    std::memset(&f, 0, sizeof f);
+                    f.region = local;
+                    int64_t off = 0;
+                    for (int d = 0; d < nd; ++d) {
+                        f.src_strides[d] = cst[d];
+                        off += (int64_t)(local.start[d] - chare.start[d]) * cst[d];
+                    }
+                    frags.push_back(f);
+                    bases.push_back(static_cast<const char*>(tiles[c]) + off * esz);
+                }
+                for (const RemoteBuffer& rb : inbox[(size_t)c])
+                    if (rb.input_index == k) {
+                        orc_fragment f;
+                        std::memset(&f, 0, sizeof f);
+                        f.region = rb.region; // packed: strides all 0
+                        frags.push_back(f);
+                        bases.push_back(rb.data.data());
+                    }
+            }
+            begin[K] = (int32_t)frags.size();
+            const int cap = 1024;
+            std::vector<int32_t> of((size_t)cap * K);
+            std::vector<int64_t> oo((size_t)cap * K), osz((size_t)cap * K * ORC_MAX_ND),
+                ost((size_t)cap * K * ORC_MAX_ND);
+            std::vector<orc_region> cells((size_t)cap * K);
+            int M = orc_align_fragments(nd, K, begin.data(), frags.data(), my_inputs.data(), cap,
+                                        of.data(), oo.data(), osz.data(), ost.data(), cells.data());
+            if (M < 0) {
+                rc_of[(size_t)c] = -7;
+                continue;
+            }
+            cells_of[(size_t)c] = M;
+            // packed result buffer of this chare's part of the assigned region
+            int64_t rsz[ORC_MAX_ND], rst[ORC_MAX_ND], total = 1;
+            for (int d = 0; d < nd; ++d)
+                rsz[d] = rsize(myout, d);
+            for (int d = nd - 1; d >= 0; --d) {
+                rst[d] = total;
+                total *= rsz[d];
+            }
+            results[(size_t)c].assign((size_t)total * esz, 0);
+            for (int m = 0; m < M; ++m) {
+                std::vector<orc_memref> in(K);
+                for (int k = 0; k < K; ++k) {
+                    const size_t at = (size_t)k * M + m;
+                    orc_memref& mr = in[k];
+                    std::memset(&mr, 0, sizeof mr);
+                    char* ptr = const_cast<char*>(bases[of[at]]) + oo[at] * esz;
+                    mr.allocated = mr.aligned = ptr;
+                    for (int d = 0; d < nd; ++d) {
+                        mr.sizes[d] = osz[at * ORC_MAX_ND + d];
+                        mr.strides[d] = ost[at * ORC_MAX_ND + d];
+                    }
+                }
+                // where the cell lands in the result buffer: its corner mapped from operand 0's
+                // index space to the assigned region (src/execute_node.cpp:1492-1506)
+                orc_region corner;
+                orc_region_map(&cells[(size_t)0 * M + m], &my_inputs[0], &myout, &corner);
+                int64_t off = 0;
+                for (int d = 0; d < nd; ++d)
+                    off += ((int64_t)(corner.start[d] - myout.start[d]) / myout.step[d]) * rst[d];
+                orc_memref out;
+                std::memset(&out, 0, sizeof out);
+                out.allocated = out.aligned = results[(size_t)c].data() + off * esz;
+                for (int d = 0; d < nd; ++d) {
+                    out.sizes[d] = in[0].sizes[d];
+                    out.strides[d] = rst[d];
+                }
+                int rc = orc_eval_group(ast, dtype, nd, K, in.data(), 0, nullptr, 1, &out);
+                if (rc) {
+                    rc_of[(size_t)c] = rc;
+                    break;
+                }
+                kern_of[(size_t)c]++;
+            }
+        }
+    });
+    for (int64_t c = 0; c < nchares; ++c) {
+        if (rc_of[(size_t)c])
+            return rc_of[(size_t)c];
+        n_kernels += kern_of[(size_t)c];
+        n_cells_max = std::max(n_cells_max, cells_of[(size_t)c]);
+    }
+    // SET_REGION: packed result buffer -> strided part of the tile, one element at a time
+    run_blocks(nchares, threads, [&](int64_t c0, int64_t c1) {
+        for (int64_t c = c0; c < c1; ++c) {
+            if (!has_out[(size_t)c])
+                continue;
+            int32_t idx[ORC_MAX_ND] = {0, 0, 0};
+            chare_index(c, idx);
+            orc_region chare;
+            orc_decomp_chare_region_global(&dc, idx, &chare);
+            const orc_region& myout = myouts[(size_t)c];
+            int64_t cst[ORC_MAX_ND], counts[ORC_MAX_ND], sstr[ORC_MAX_ND], sstart[ORC_MAX_ND],
+                sstep[ORC_MAX_ND], dstart[ORC_MAX_ND], dstep[ORC_MAX_ND];
+            tile_strides(chare, cst);
+            int64_t sdim = 1;
+            for (int d = nd - 1; d >= 0; --d) {
+                counts[d] = rsize(myout, d);
+                sstr[d] = sdim;
+                sdim *= counts[d];
+                sstart[d] = 0;
+                sstep[d] = 1;
+                dstart[d] = myout.start[d] - chare.start[d];
+                dstep[d] = myout.step[d];
+            }
+            orc_copy_region(nd, esz, tiles[c], cst, dstart, dstep, results[(size_t)c].data(), sstr,
+                            sstart, sstep, counts);
+        }
+    });
+    if (stats) {
+        stats[0] = n_msgs;
+        stats[1] = n_bytes;
+        stats[2] = n_kernels;
+        stats[3] = n_cells_max;
+    }
+    return 0;
+}

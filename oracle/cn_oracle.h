@@ -151,6 +151,17 @@ int orc_group_dtype(const orc_ast* ast);
 int orc_eval_group(const orc_ast* ast, int dtype, int ndims, int n_in, const orc_memref* in,
                    int n_scalar, const void* const* scalars, int n_out, const orc_memref* out);
 
+/* One fused SET_REGION group over one tiled array (offset 0, `tile` edge, tiles in row-major grid
+ * order, each row-major over its own extent), executed chare by chare as the reference's fragment
+ * path does: halo pack + message per remote fragment, local + received fragments per operand,
+ * align_fragments, one kernel per aligned cell into a packed result buffer, SET_REGION copy
+ * (src/executor_core.cpp:8-143,684-747, src/execute_node.cpp:1376-1585,
+ * src/executor_ast_visitor.cpp:268-311). Every leaf must be the assigned array. `threads` chares
+ * run side by side in the compute phase. stats: [0] messages, [1] bytes packed, [2] kernel calls,
+ * [3] largest cell count of a chare. */
+int orc_world_group(const orc_ast* ast, int dtype, int ndims, const int32_t* shape, int tile,
+                    void* const* tiles, int threads, int64_t* stats);
+
 /* ---- SET_REGION fill / strided copy (src/executor_ast_visitor.cpp:112-313) ---- */
 /* Element i along dim d sits at (start[d] + i*step[d]) * strides[d]; byte-wise, bit-exact. */
 int orc_fill_region(int ndims, int esz, void* dst, const int64_t* dst_strides,

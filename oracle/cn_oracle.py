@@ -53,6 +53,7 @@ def load():
         "orc_group_signature": (i32, [vp, i32, vp, vp, vp, vp, vp, vp, vp, vp]),
         "orc_group_dtype": (i32, [vp]),
         "orc_eval_group": (i32, [vp, i32, i32, i32, vp, i32, vp, i32, vp]),
+        "orc_world_group": (i32, [vp, i32, i32, vp, i32, vp, i32, vp]),
         "orc_fill_region": (i32, [i32, i32, vp, vp, vp, vp, vp, vp]),
         "orc_copy_region": (i32, [i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp]),
         "orc_scalar_to_dtype": (i32, [i32, dbl, vp]),
@@ -134,6 +135,35 @@ class Oracle:
                                      C.addressof(in_arr), len(svals), C.addressof(sptr),
                                      len(outs), C.addressof(out_arr))
         return rc
+
+    # One SET_REGION group over a tiled array, chare by chare as the reference's fragment path
+    # runs it. `tiles` are the row-major tiles (row-major grid order), updated in place.
+    def world_group(self, ast, dtype, shape, tile, tiles, threads=1):
+        nd = len(shape)
+        shp = (C.c_int32 * 3)(*list(shape) + [1] * (3 - nd))
+        tp = (C.c_void_p * len(tiles))(*[C.c_void_p(ptr(t)) for t in tiles])
+        stats = (C.c_int64 * 4)()
+        rc = self.lib.orc_world_group(C.addressof(ast), dtype, nd, shp, int(tile), tp, int(threads), stats)
+        return rc, {"messages": stats[0], "bytes": stats[1], "kernels": stats[2], "max_cells": stats[3]}
+
+    @staticmethod
+    def split_tiles(arr, tile):
+        """Row-major tiles of a global array in row-major grid order (copies)."""
+        grid = [(n + tile - 1) // tile for n in arr.shape]
+        out = []
+        for idx in np.ndindex(*grid):
+            sl = tuple(slice(i * tile, min((i + 1) * tile, n)) for i, n in zip(idx, arr.shape))
+            out.append(np.array(arr[sl], order="C", copy=True))
+        return out
+
+    @staticmethod
+    def join_tiles(tiles, shape, tile):
+        grid = [(n + tile - 1) // tile for n in shape]
+        out = np.empty(shape, dtype=tiles[0].dtype)
+        for t, idx in zip(tiles, np.ndindex(*grid)):
+            sl = tuple(slice(i * tile, min((i + 1) * tile, n)) for i, n in zip(idx, shape))
+            out[sl] = t
+        return out
 
     def dot(self, a, b):
         dt = DTYPE_OF[a.dtype]
