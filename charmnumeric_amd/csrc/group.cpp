@@ -680,8 +680,8 @@ int try_launch_direct(cnh_kernel* k, const std::vector<const cnh_tiled*>& arrays
     a.nblocks8 = blocks % 8 == 0 ? (int)(blocks / 8) : 0;
     // Ordering groups: G^3 neighbouring full tiles whose joint z-slab still fits an L2 (edge of a
     // group at most 256 elements), G as large as the grid allows. Rank 3 only.
-    int G = 1;
-    if (nd == 3 && g_direct_group) {
+    int G = 1, Gx = 1;
+    if (nd == 3 && g_direct_group == 1) {
         for (int cand = 2; cand <= 4; cand *= 2) {
             bool ok = (int64_t)cand * a.tile <= 256;
             for (int d = 0; d < 3 && ok; ++d)
@@ -690,8 +690,15 @@ int try_launch_direct(cnh_kernel* k, const std::vector<const cnh_tiled*>& arrays
                 G = cand;
         }
     }
+    // Mode 2: the tiles of one row of the tile grid along x form a group, so that the column
+    // pairs a workgroup reads from its x neighbours are lines those neighbours load just then.
+    if (nd == 3 && g_direct_group == 2 && a.grid[2] > 1 && a.grid[2] <= 8 &&
+        a.shape[2] == a.grid[2] * a.tile)
+        Gx = a.grid[2];
     for (int d = 0; d < 3; ++d)
         a.sg[d] = (d >= pad) ? G : 1;
+    if (Gx > 1)
+        a.sg[2] = Gx;
     a.per_group = fdiv_make((uint32_t)(per_tile * a.sg[0] * a.sg[1] * a.sg[2]));
     a.ggrid1 = fdiv_make((uint32_t)(a.grid[1] / a.sg[1]));
     a.ggrid2 = fdiv_make((uint32_t)(a.grid[2] / a.sg[2]));
@@ -804,7 +811,7 @@ extern "C" int cnh_set_option(const char* name, int value) {
         return 0;
     }
     if (std::strcmp(name, "direct_group") == 0) {
-        g_direct_group = value != 0;
+        g_direct_group = value;
         return 0;
     }
     if (std::strcmp(name, "direct_tx") == 0) {
