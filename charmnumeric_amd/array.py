@@ -221,7 +221,13 @@ class _ArrayLike:
             if value.dtype != self.dtype:
                 raise NotImplementedError("assignment across dtypes is not implemented")
             if tuple(value.shape) != tuple(shape):
-                raise ValueError(f"could not broadcast input from shape {value.shape} into shape {shape}")
+                # a lower-rank value fits a region whose extra dimensions have extent 1
+                # (IFOG[t] = M with M 2-D)
+                squeeze = lambda sh: tuple(x for x in sh if x != 1)
+                if not (value.ndims < len(shape) and squeeze(value.shape) == squeeze(shape)
+                        and _is_whole(value._region(), value._base().shape)):
+                    raise ValueError(
+                        f"could not broadcast input from shape {value.shape} into shape {shape}")
             operand = value._ref()
         else:
             operand = value
@@ -292,9 +298,10 @@ class Array(_ArrayLike):
         self._wire = lazy.wire_dtype(self.dtype)
         self._n = _size(self.shape)
         self.name = lazy.new_name() if name is None else name
+        self._gen = lazy.generation()
 
     def __del__(self):
-        lazy.record_delete(self.name)
+        lazy.record_delete(self.name, self._gen)
 
     def __repr__(self):
         return f"Array(shape={self.shape}, dtype={self.dtype.name}, name={self.name})"
@@ -421,6 +428,21 @@ def nonfusible(opcode, operands, shape, dtype):
     return out
 
 
+def tile(x, reps):
+    """numpy.tile for arrays (charmnumeric/operations.py:52-72 upstream): the operand's shape is
+    left-padded with ones to the rank of `reps` and repeated."""
+    x = asarray(x)
+    reps = (int(reps),) if isinstance(reps, numbers.Integral) else tuple(int(r) for r in reps)
+    rank = max(x.ndims, len(reps))
+    if rank > 3:
+        raise NotImplementedError("arrays of rank above 3 are not supported")
+    shape = (1,) * (rank - x.ndims) + tuple(x.shape)
+    reps = (1,) * (rank - len(reps)) + reps
+    if any(r < 1 for r in reps):
+        raise NotImplementedError("zero-sized arrays are not supported")
+    return nonfusible(L.OP_TILE, [x], tuple(s * r for s, r in zip(shape, reps)), x.dtype)
+
+
 def _same_dtype(a, b, what):
     if a.dtype != b.dtype:
         raise NotImplementedError(f"{what} across dtypes ({a.dtype} and {b.dtype}) is not implemented")
@@ -435,21 +457,33 @@ def _matmul(lhs, rhs):
         if lhs.shape[0] != rhs.shape[0]:
             raise ValueError(f"Shape mismatch for dot product: ({lhs.shape[0]},) @ ({rhs.shape[0]},)")
         return nonfusible(L.OP_REDUCE, [lhs, rhs], (1,), _same_dtype(lhs, rhs, "dot"))
-    if lhs.ndims == 3:
-        raise NotImplementedError("matmul on a 3-D operand with a dropped dimension is not implemented")
-    if lhs.ndims != 2:
+    if lhs.ndims == 3 and rhs.ndims == 1:
+        raise NotImplementedError("matvec on a 3-D operand with a dropped dimension is not implemented")
+    if lhs.ndims not in (2, 3):
         raise ValueError(f"matmul requires a 2D matrix, got {lhs.ndims}D")
     if rhs.ndims == 1:
         return _matvec(lhs, rhs)
     if rhs.ndims == 2 and rhs.shape[1] == 1:
         raise NotImplementedError("matmul with an (N, 1) column operand is not implemented")
-    if rhs.ndims == 2:
-        if lhs.shape[1] != rhs.shape[0]:
-            raise ValueError(f"Shape mismatch: ({lhs.shape[0]},{lhs.shape[1]}) @ "
-                             f"({rhs.shape[0]},{rhs.shape[1]})")
-        return nonfusible(L.OP_MATMATMUL, [lhs, rhs], (lhs.shape[0], rhs.shape[1]),
-                          _same_dtype(lhs, rhs, "matmul"))
-    raise NotImplementedError("matmul with a 3-D right operand is not implemented")
+    lr, lc = _matrix_shape(lhs)
+    rr, rc = _matrix_shape(rhs)
+    if lc != rr:
+        raise ValueError(f"Shape mismatch: ({lr},{lc}) @ ({rr},{rc})")
+    return nonfusible(L.OP_MATMATMUL, [lhs, rhs], (lr, rc), _same_dtype(lhs, rhs, "matmul"))
+
+
+def _matrix_shape(x):
+    """(rows, cols) of a matmul operand: a 2-D array, or a 3-D one with exactly one extent of 1,
+    which is dropped (charmnumeric.py:579-592 upstream)."""
+    if x.ndims == 2:
+        return x.shape[0], x.shape[1]
+    if x.ndims == 3:
+        ones = [d for d in range(3) if x.shape[d] == 1]
+        if len(ones) != 1:
+            raise ValueError(f"3D matmatmul requires exactly one singleton dim, got shape {x.shape}")
+        rest = [d for d in range(3) if d != ones[0]]
+        return x.shape[rest[0]], x.shape[rest[1]]
+    raise ValueError(f"matmatmul requires 2D or 3D operand, got {x.ndims}D")
 
 
 def _matvec(mat, vec):

@@ -490,7 +490,9 @@ struct Tiled {
     int shift; int tile; int off[3]; int shape[3]; int glo[3]; int grid[3];
     const T* const* tiles;
 };
-struct DTile { i64 blk0; int cs[3]; int w[3]; int nchunks; int pad; T* dst; const T* cur; };
+// cs, w: origin and extents of the tile; bs, bw: the box of it this launch visits (the whole
+// tile, or just the part the assigned region touches when the launch works in place).
+struct DTile { i64 blk0; int cs[3]; int w[3]; int nchunks; int pad; int bs[3]; int bw[3]; T* dst; const T* cur; };
 struct LeafReg { int arr; int start[3]; int step[3]; };
 struct TilesArgs {
     int out_off[3];
@@ -519,8 +521,8 @@ extern "C" __global__ __launch_bounds__(256) void grp_tiles(const Tiled* arrs, c
     const i64 blk = (i64)blockIdx.x - dt.blk0;
     const i64 outer = blk / dt.nchunks;
     const int chunk = (int)(blk - outer * dt.nchunks);
-    const int l1 = (int)(outer % dt.w[1]);
-    const int l0 = (int)(outer / dt.w[1]);
+    const int l1 = dt.bs[1] + (int)(outer % dt.bw[1]);
+    const int l0 = dt.bs[0] + (int)(outer / dt.bw[1]);
     const int a0 = dt.cs[0] + l0 - ta.out_off[0];
     const int a1 = dt.cs[1] + l1 - ta.out_off[1];
     const bool in01 = a0 >= ta.rs[0] && a0 < ta.re[0] && (a0 - ta.rs[0]) % ta.rst[0] == 0 &&
@@ -529,8 +531,9 @@ extern "C" __global__ __launch_bounds__(256) void grp_tiles(const Tiled* arrs, c
     const int k1 = (a1 - ta.rs[1]) / ta.rst[1];
 #pragma unroll
     for (int u = 0; u < TL_PER_THREAD; ++u) {
-        const int l2 = chunk * (256 * TL_PER_THREAD) + u * 256 + (int)threadIdx.x;
-        if (l2 >= dt.w[2]) continue;
+        const int i2 = chunk * (256 * TL_PER_THREAD) + u * 256 + (int)threadIdx.x;
+        if (i2 >= dt.bw[2]) continue;
+        const int l2 = dt.bs[2] + i2;
         const i64 di = ((i64)l0 * dt.w[1] + l1) * dt.w[2] + l2;
         const int a2 = dt.cs[2] + l2 - ta.out_off[2];
         const bool inside = in01 && a2 >= ta.rs[2] && a2 < ta.re[2] &&

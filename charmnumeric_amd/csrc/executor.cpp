@@ -606,6 +606,8 @@ int exec_group(Ex* ex, const DagNode& n) {
     // Shifted / strided operands or mixed decompositions: one launch over the target's tiles that
     // reads whatever tiles the operand regions fall into (replaces the fragment path and its halo
     // messages, src/execute_node.cpp:1338-1585, src/executor_core.cpp:8-143).
+    // Reading the target through another region is a hazard only where that region can meet the
+    // assigned one: disjoint bounding boxes (C[t] = f(C[t-1])) are safe in place.
     bool aliased = false;
     if (is_set)
         for (int i = 0; i < n_in; ++i)
@@ -616,15 +618,59 @@ int exec_group(Ex* ex, const DagNode& n) {
                 const cnh_region& ir = in_has_reg[i] ? in_reg[i] : whole;
                 bool same = same_region(ir, root.region) ||
                             (region_is_whole(ir, *target) && region_is_whole(root.region, *target));
-                if (!same)
+                if (same)
+                    continue;
+                bool disjoint = false;
+                if (!ir.is_global && !root.region.is_global)
+                    for (int d = 0; d < target->ndims; ++d)
+                        if (ir.stop[d] <= root.region.start[d] || root.region.stop[d] <= ir.start[d])
+                            disjoint = true;
+                if (!disjoint)
                     aliased = true;
             }
     if (aliased)
         if (int rc = ensure_alt(ex, *target))
             return rc;
     std::vector<cnh_tiled> tin(std::max(1, n_in));
-    for (int i = 0; i < n_in; ++i)
+    for (int i = 0; i < n_in; ++i) {
         tin[i] = in_arr[i]->tiled();
+        if (in_arr[i]->ndims < target->ndims) {
+            // A lower-rank operand assigned into a higher-rank region (IFOG[t] = M with M 2-D):
+            // present it with extent-1 dimensions inserted where the assigned region has them.
+            // A row-major tile (e0, e1) is the same memory as (1, e0, e1) or (e0, 1, e1).
+            CNH_CHECK(is_set && !root.region.is_global && !in_has_reg[i], -35,
+                      "node %d: operand %d has rank %d in a rank-%d group", n.id, in_arr[i]->name,
+                      in_arr[i]->ndims, target->ndims);
+            const XArray& a = *in_arr[i];
+            cnh_tiled t;
+            std::memset(&t, 0, sizeof t);
+            t.ndims = target->ndims;
+            t.tile = a.tile;
+            t.tiles = a.tiles.data();
+            int j = 0;
+            for (int d = 0; d < target->ndims; ++d) {
+                const int cnt = region_count(root.region, d);
+                const int left_t = target->ndims - d, left_a = a.ndims - j;
+                if (j < a.ndims && a.shape[j] == cnt && !(cnt == 1 && left_t > left_a)) {
+                    t.shape[d] = a.shape[j];
+                    t.grid[d] = a.grid[j];
+                    ++j;
+                } else {
+                    CNH_CHECK(cnt == 1, -35, "node %d: operand %d of shape rank %d does not fit the "
+                              "assigned region", n.id, a.name, a.ndims);
+                    t.shape[d] = 1;
+                    t.grid[d] = 1;
+                }
+            }
+            CNH_CHECK(j == a.ndims, -35, "node %d: operand %d does not fit the assigned region", n.id,
+                      a.name);
+            tin[i] = t;
+        } else {
+            CNH_CHECK(in_arr[i]->ndims == target->ndims, -35,
+                      "node %d: operand %d has rank %d in a rank-%d group", n.id, in_arr[i]->name,
+                      in_arr[i]->ndims, target->ndims);
+        }
+    }
     cnh_tiled cur = target->tiled(false);
     cnh_tiled dst = aliased ? target->tiled(true) : cur;
     ex->log("group node=" + std::to_string(n.id) + " path=tiles inputs=" + std::to_string(n_in) +
@@ -738,61 +784,214 @@ int exec_matmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
                           y->tiles[0], ex->stream);
 }
 
+// A 2-D array, or a 3-D array with exactly one extent-1 dimension, seen as a matrix
+// (the dimension-dropped operands of charmnumeric.py:510-519, src/executor_matmatmul.cpp:485-813).
+struct MatView {
+    const XArray* a = nullptr;
+    int rd = 0, cd = 1; // which array dimensions are rows and columns
+    int rows = 0, cols = 0;
+    int tile_index(int tr, int tc) const {
+        int idx[3] = {0, 0, 0};
+        idx[rd] = tr;
+        idx[cd] = tc;
+        int64_t t = 0;
+        for (int d = 0; d < a->ndims; ++d)
+            t = t * a->grid[d] + idx[d];
+        return (int)t;
+    }
+    // extents of tile (tr, tc): rows, columns (= leading dimension: the dropped extent is 1)
+    void extent(int tr, int tc, int* lo_r, int* lo_c, int* er, int* ec) const {
+        int32_t lo[3], ext[3];
+        a->tile_extent(tile_index(tr, tc), lo, ext);
+        *lo_r = lo[rd];
+        *lo_c = lo[cd];
+        *er = ext[rd];
+        *ec = ext[cd];
+    }
+};
+
+int as_matrix(const XArray& a, MatView* m, const char* what) {
+    m->a = &a;
+    if (a.ndims == 2) {
+        m->rd = 0;
+        m->cd = 1;
+    } else {
+        CNH_CHECK(a.ndims == 3, -32, "%s needs 2-D operands (or 3-D with one extent of 1)", what);
+        int dropped = -1, ones = 0;
+        for (int d = 0; d < 3; ++d)
+            if (a.shape[d] == 1) {
+                ++ones;
+                if (dropped < 0)
+                    dropped = d;
+            }
+        CNH_CHECK(ones >= 1, -32, "%s: 3-D operand %d has no extent of 1", what, a.name);
+        m->rd = dropped == 0 ? 1 : 0;
+        m->cd = dropped == 2 ? 1 : 2;
+    }
+    m->rows = a.shape[m->rd];
+    m->cols = a.shape[m->cd];
+    return 0;
+}
+
 // MATMATMUL: C (zeroed) += A_panel * B_panel for every k-overlapping pair of tiles, k ascending
 // (src/executor_matmatmul.cpp:105-484, src/executor_incremental.cpp:97-132).
 int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
-    XArray *A, *B;
-    if (int rc = leaf_array(ex, n, root, 0, &A, "MATMATMUL"))
+    XArray *Aa, *Ba;
+    if (int rc = leaf_array(ex, n, root, 0, &Aa, "MATMATMUL"))
         return rc;
-    if (int rc = leaf_array(ex, n, root, 1, &B, "MATMATMUL"))
+    if (int rc = leaf_array(ex, n, root, 1, &Ba, "MATMATMUL"))
         return rc;
-    CNH_CHECK(A->ndims == 2 && B->ndims == 2, -32, "MATMATMUL needs 2-D operands");
-    CNH_CHECK(A->shape[1] == B->shape[0], -32, "MATMATMUL: (%d,%d) @ (%d,%d)", A->shape[0],
-              A->shape[1], B->shape[0], B->shape[1]);
-    CNH_CHECK(A->dtype == B->dtype, -27, "MATMATMUL: operand dtypes %d and %d", A->dtype, B->dtype);
-    int32_t shape[3] = {A->shape[0], B->shape[1], 1};
+    MatView A, B;
+    if (int rc = as_matrix(*Aa, &A, "MATMATMUL"))
+        return rc;
+    if (int rc = as_matrix(*Ba, &B, "MATMATMUL"))
+        return rc;
+    CNH_CHECK(A.cols == B.rows, -32, "MATMATMUL: (%d,%d) @ (%d,%d)", A.rows, A.cols, B.rows, B.cols);
+    CNH_CHECK(Aa->dtype == Ba->dtype, -27, "MATMATMUL: operand dtypes %d and %d", Aa->dtype, Ba->dtype);
+    int32_t shape[3] = {A.rows, B.cols, 1};
     XArray* Cc;
-    if (int rc = make_array(ex, root.result_name, 2, A->dtype, shape, true, &Cc))
+    if (int rc = make_array(ex, root.result_name, 2, Aa->dtype, shape, true, &Cc))
         return rc;
-    const int esz = dtype_size(A->dtype);
+    const int esz = dtype_size(Aa->dtype);
+    const int TA = Aa->tile, TB = Ba->tile;
     int calls = 0;
     for (int ci = 0; ci < Cc->grid[0]; ++ci)
         for (int cj = 0; cj < Cc->grid[1]; ++cj) {
             int32_t clo[3], cext[3];
             Cc->tile_extent((int64_t)ci * Cc->grid[1] + cj, clo, cext);
             // rows of this C tile fall into A row tiles, its columns into B column tiles
-            for (int ai = clo[0] / A->tile; ai <= (clo[0] + cext[0] - 1) / A->tile; ++ai)
-                for (int bj = clo[1] / B->tile; bj <= (clo[1] + cext[1] - 1) / B->tile; ++bj) {
-                    int r0 = std::max(clo[0], ai * A->tile);
-                    int r1 = std::min(clo[0] + cext[0], std::min((ai + 1) * A->tile, (int)A->shape[0]));
-                    int c0 = std::max(clo[1], bj * B->tile);
-                    int c1 = std::min(clo[1] + cext[1], std::min((bj + 1) * B->tile, (int)B->shape[1]));
+            for (int ai = clo[0] / TA; ai <= (clo[0] + cext[0] - 1) / TA; ++ai)
+                for (int bj = clo[1] / TB; bj <= (clo[1] + cext[1] - 1) / TB; ++bj) {
+                    int r0 = std::max(clo[0], ai * TA);
+                    int r1 = std::min(clo[0] + cext[0], std::min((ai + 1) * TA, A.rows));
+                    int c0 = std::max(clo[1], bj * TB);
+                    int c1 = std::min(clo[1] + cext[1], std::min((bj + 1) * TB, B.cols));
                     // k pieces: common refinement of A's column tiles and B's row tiles
                     int k0 = 0;
-                    const int K = A->shape[1];
+                    const int K = A.cols;
                     while (k0 < K) {
-                        int ak = k0 / A->tile, bk = k0 / B->tile;
-                        int k1 = std::min(K, std::min((ak + 1) * A->tile, (bk + 1) * B->tile));
-                        int32_t alo[3], aext[3], blo[3], bext[3];
-                        A->tile_extent((int64_t)ai * A->grid[1] + ak, alo, aext);
-                        B->tile_extent((int64_t)bk * B->grid[1] + bj, blo, bext);
-                        const char* ap = static_cast<const char*>(A->tiles[(size_t)ai * A->grid[1] + ak]) +
-                                         ((int64_t)(r0 - alo[0]) * aext[1] + (k0 - alo[1])) * esz;
-                        const char* bp = static_cast<const char*>(B->tiles[(size_t)bk * B->grid[1] + bj]) +
-                                         ((int64_t)(k0 - blo[0]) * bext[1] + (c0 - blo[1])) * esz;
+                        int ak = k0 / TA, bk = k0 / TB;
+                        int k1 = std::min(K, std::min((ak + 1) * TA, (bk + 1) * TB));
+                        int alr, alc, aer, aec, blr, blc, ber, bec;
+                        A.extent(ai, ak, &alr, &alc, &aer, &aec);
+                        B.extent(bk, bj, &blr, &blc, &ber, &bec);
+                        const char* ap = static_cast<const char*>(Aa->tiles[(size_t)A.tile_index(ai, ak)]) +
+                                         ((int64_t)(r0 - alr) * aec + (k0 - alc)) * esz;
+                        const char* bp = static_cast<const char*>(Ba->tiles[(size_t)B.tile_index(bk, bj)]) +
+                                         ((int64_t)(k0 - blr) * bec + (c0 - blc)) * esz;
                         char* cp = static_cast<char*>(Cc->tiles[(size_t)ci * Cc->grid[1] + cj]) +
                                    ((int64_t)(r0 - clo[0]) * cext[1] + (c0 - clo[1])) * esz;
                         ++calls;
                         if (!ex->dry)
-                            if (int rc = cnh_gemm_acc(A->dtype, r1 - r0, c1 - c0, k1 - k0, ap, aext[1],
-                                                      bp, bext[1], cp, cext[1], ex->stream))
+                            if (int rc = cnh_gemm_acc(Aa->dtype, r1 - r0, c1 - c0, k1 - k0, ap, aec, bp, bec,
+                                                      cp, cext[1], ex->stream))
                                 return rc;
                         k0 = k1;
                     }
                 }
         }
-    ex->log("matmatmul A=" + std::to_string(A->name) + " B=" + std::to_string(B->name) + " out=" +
+    ex->log("matmatmul A=" + std::to_string(Aa->name) + " B=" + std::to_string(Ba->name) + " out=" +
             std::to_string(Cc->name) + " panel_products=" + std::to_string(calls));
+    return 0;
+}
+
+// TILE: out[i0, i1, ..] = in[i0 % s0, i1 % s1, ..] with the input's shape left-padded with ones
+// to the output's rank (charmnumeric/operations.py:52-72, src/dag_group_receive.cpp:353-375).
+// One strided copy per (output tile, input tile, repetition) that meet; a repeated extent-1
+// dimension is a copy with source step 0.
+int exec_tile(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
+    CNH_CHECK(root.n_operands >= 1, -36, "TILE: no operand");
+    const cnh_ast_node& op = n.nodes[root.operands[0]];
+    XArray* in;
+    if (int rc = find_array(ex, op.result_name, &in, "TILE"))
+        return rc;
+    CNH_CHECK(!root.region.is_global && root.region.ndims == root.ndims, -36,
+              "TILE %d carries no result shape", root.result_name);
+    const int nd = root.ndims, delta = nd - in->ndims;
+    CNH_CHECK(delta >= 0 && nd <= 3, -36, "TILE: result rank %d below operand rank %d", nd, in->ndims);
+    int32_t oshape[3] = {1, 1, 1}, ishape[3] = {1, 1, 1};
+    for (int d = 0; d < nd; ++d) {
+        oshape[d] = region_count(root.region, d);
+        ishape[d] = d < delta ? 1 : in->shape[d - delta];
+        CNH_CHECK(oshape[d] % ishape[d] == 0, -36, "TILE: extent %d is not a multiple of %d", oshape[d],
+                  ishape[d]);
+    }
+    XArray* out;
+    if (int rc = make_array(ex, root.result_name, nd, in->dtype, oshape, false, &out))
+        return rc;
+    const int esz = dtype_size(in->dtype);
+    int copies = 0;
+    for (int64_t ot = 0; ot < out->ntiles; ++ot) {
+        int32_t olo[3], oext[3];
+        out->tile_extent(ot, olo, oext);
+        for (int64_t it = 0; it < in->ntiles; ++it) {
+            int32_t ilo_a[3], iext_a[3], ilo[3] = {0, 0, 0}, iext[3] = {1, 1, 1};
+            in->tile_extent(it, ilo_a, iext_a);
+            for (int d = 0; d < in->ndims; ++d) {
+                ilo[d + delta] = ilo_a[d];
+                iext[d + delta] = iext_a[d];
+            }
+            // per dimension: repetitions r with [r*s + ilo, r*s + ilo + iext) meeting the output tile
+            int rlo[3], rhi[3];
+            bool none = false;
+            for (int d = 0; d < nd; ++d) {
+                const int sdim = ishape[d];
+                rlo[d] = std::max(0, (olo[d] - ilo[d] - iext[d] + sdim) / sdim);
+                rhi[d] = std::min(oshape[d] / sdim - 1, (olo[d] + oext[d] - 1 - ilo[d]) / sdim);
+                if (ishape[d] == 1) { // extent-1 source: one copy with step 0 covers all repetitions
+                    rlo[d] = 0;
+                    rhi[d] = 0;
+                }
+                if (rhi[d] < rlo[d])
+                    none = true;
+            }
+            if (none)
+                continue;
+            int r[3] = {0, 0, 0};
+            for (r[0] = rlo[0]; r[0] <= (nd > 0 ? rhi[0] : 0); ++r[0])
+                for (r[1] = nd > 1 ? rlo[1] : 0; r[1] <= (nd > 1 ? rhi[1] : 0); ++r[1])
+                    for (r[2] = nd > 2 ? rlo[2] : 0; r[2] <= (nd > 2 ? rhi[2] : 0); ++r[2]) {
+                        int64_t dstart[3], dstep[3], sstart[3], sstep[3], counts[3], dstr[3], sstr[3];
+                        bool empty = false;
+                        int64_t ds = 1, ss = 1;
+                        for (int d = nd - 1; d >= 0; --d) {
+                            dstr[d] = ds;
+                            ds *= oext[d];
+                            sstr[d] = ss;
+                            ss *= iext[d];
+                        }
+                        for (int d = 0; d < nd; ++d) {
+                            if (ishape[d] == 1) {
+                                dstart[d] = 0;
+                                counts[d] = oext[d];
+                                sstart[d] = 0;
+                                sstep[d] = 0;
+                            } else {
+                                const int g0 = r[d] * ishape[d] + ilo[d]; // where this piece lands
+                                const int lo = std::max(g0, (int)olo[d]);
+                                const int hi = std::min(g0 + iext[d], olo[d] + oext[d]);
+                                if (hi <= lo)
+                                    empty = true;
+                                dstart[d] = lo - olo[d];
+                                counts[d] = hi - lo;
+                                sstart[d] = lo - g0;
+                                sstep[d] = 1;
+                            }
+                            dstep[d] = 1;
+                        }
+                        if (empty)
+                            continue;
+                        ++copies;
+                        if (!ex->dry)
+                            if (int rc = cnh_copy_region(nd, esz, out->tiles[ot], dstr, dstart, dstep,
+                                                         in->tiles[it], sstr, sstart, sstep, counts,
+                                                         ex->stream))
+                                return rc;
+                    }
+        }
+    }
+    ex->log("tile in=" + std::to_string(in->name) + " out=" + std::to_string(out->name) + " shape=" +
+            shape_str(out->shape, nd) + " copies=" + std::to_string(copies));
     return 0;
 }
 
@@ -809,6 +1008,7 @@ int exec_node(Ex* ex, const DagNode& n) {
     case kOpMaxabsDiff: return exec_reduce_ext(ex, n, root);
     case CNH_OP_MATMUL: return exec_matmul(ex, n, root);
     case CNH_OP_MATMATMUL: return exec_matmatmul(ex, n, root);
+    case CNH_OP_TILE: return exec_tile(ex, n, root);
     case CNH_OP_ADD:
     case CNH_OP_SUB:
     case CNH_OP_MUL:

@@ -427,10 +427,11 @@ static_assert(sizeof(TiledDev) == 64, "TiledDev layout must match the generated 
 struct DTileDev {
     int64_t blk0;
     int32_t cs[3], w[3], nchunks, pad;
+    int32_t bs[3], bw[3];
     void* dst;
     const void* cur;
 };
-static_assert(sizeof(DTileDev) == 56, "DTileDev layout must match the generated struct");
+static_assert(sizeof(DTileDev) == 80, "DTileDev layout must match the generated struct");
 
 int check_tiled(const cnh_tiled* t, int nd, const char* what) {
     CNH_CHECK(t != nullptr, -2, "%s: null descriptor", what);
@@ -987,11 +988,29 @@ extern "C" int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* 
         }
         if (empty)
             continue;
-        dt.nchunks = (dt.w[2] + 1023) / 1024;
-        dt.blk0 = blocks;
         dt.dst = dst->tiles[t];
         dt.cur = cur ? cur->tiles[t] : nullptr;
-        blocks += (int64_t)dt.w[0] * dt.w[1] * dt.nchunks;
+        // In place (or with nothing to copy from), elements outside the assigned region keep
+        // their values without being touched: visit only the part of the tile inside the
+        // region's bounding box, and skip tiles it misses.
+        const bool in_place = dt.cur == nullptr || dt.cur == dt.dst;
+        for (int d = 0; d < 3; ++d) {
+            dt.bs[d] = 0;
+            dt.bw[d] = dt.w[d];
+            if (in_place && d >= pad) {
+                const int lo = std::max(dt.cs[d], rs[d] + dst->offset[d - pad]);
+                const int hi = std::min(dt.cs[d] + dt.w[d], re[d] + dst->offset[d - pad]);
+                if (hi <= lo)
+                    empty = true;
+                dt.bs[d] = lo - dt.cs[d];
+                dt.bw[d] = hi - lo;
+            }
+        }
+        if (empty)
+            continue;
+        dt.nchunks = (dt.bw[2] + 1023) / 1024;
+        dt.blk0 = blocks;
+        blocks += (int64_t)dt.bw[0] * dt.bw[1] * dt.nchunks;
         dts.push_back(dt);
     }
     if (dts.empty())

@@ -148,7 +148,8 @@ int cnh_copy_region(int nd, int esz, void* dst, const int64_t* dst_strides,
     CNH_CHECK(esz == 4 || esz == 8, -2, "cnh_copy_region: element size %d not in {4,8}", esz);
     CNH_CHECK(dst && src, -2, "cnh_copy_region: null pointer");
     for (int d = 0; d < nd; ++d) {
-        CNH_CHECK(dst_step[d] >= 1 && src_step[d] >= 1, -2, "cnh_copy_region: step must be >= 1");
+        CNH_CHECK(dst_step[d] >= 1 && src_step[d] >= 0, -2,
+                  "cnh_copy_region: destination steps must be >= 1, source steps >= 0");
         if (counts[d] <= 0)
             return 0;
     }

@@ -65,6 +65,7 @@ class _State:
         self.auto_flush = None        # (interface, threshold)
         self.epoch = 0
         self.flushing = False
+        self.generation = 0           # bumped by reset(): handles of older generations are inert
 
 
 _state = _State()
@@ -98,9 +99,16 @@ def record(instr):
     _state.pending.append(instr)
 
 
-def record_delete(name):
+def generation():
+    return _state.generation
+
+
+def record_delete(name, gen):
     # Called from handle finalisers; never flushes (it may run at any point, even at shutdown).
+    # A handle created before the last reset() names nothing any more: names restart there.
     try:
+        if gen != _state.generation:
+            return
         _state.pending.append(Instr("delete", name=name))
     except Exception:  # interpreter teardown
         pass
@@ -119,6 +127,7 @@ def reset():
     _state.next_name = 1
     _state.auto_flush = None
     _state.epoch = 0
+    _state.generation += 1
 
 
 def pending_count():
@@ -204,7 +213,8 @@ def _plan(batch):
                 v = ins.operands[0]
                 fuse = (cur is not None and isinstance(v, ArrayRef) and v.region is None
                         and batch[cur.ops[-1]].name == v.name and v.name not in forced
-                        and not v.broadcast)
+                        and not v.broadcast and len(cur.shape) == ins.payload.base_ndims
+                        and cur.dtype == ins.dtype)
                 if fuse:
                     cur.set_idx = i
                     group_of[i] = cur

@@ -8,6 +8,7 @@ import numpy as np
 from . import _lib as L
 from . import lazy
 from .array import (_ArrayLike, _as_operand, _coerce_scalar, _is_scalar_like, asarray, nonfusible, unary)
+from .array import tile as _tile_array
 
 
 def tanh(x):
@@ -74,7 +75,9 @@ def norm2(x):
 
 
 def tile(x, reps):
-    raise NotImplementedError("tile is not implemented by this backend")
+    if _is_scalar_like(x):
+        return asarray(np.tile(_coerce_scalar(x), reps))
+    return _tile_array(x, reps)
 
 
 def diag(v, k=0):

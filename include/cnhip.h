@@ -124,7 +124,8 @@ int cnh_event_elapsed_ms(cnh_event start, cnh_event stop, float* ms);
 /* ---- SET_REGION scalar fill and strided copy; halo pack/unpack
  *      (src/executor_ast_visitor.cpp:112-313, src/executor_core.cpp:8-143,
  *       src/execute_node.cpp:1001-1181). Element i of dim d is at
- *      (start[d] + i*step[d]) * strides[d]. Byte-wise, bit-exact; esz in {4, 8}. ---- */
+ *      (start[d] + i*step[d]) * strides[d]. Byte-wise, bit-exact; esz in {4, 8}. A source step of
+ *      0 repeats the source along that dimension (TILE of an extent-1 dimension). ---- */
 int cnh_fill_region(int ndims, int esz, void* dst, const int64_t* dst_strides,
                     const int64_t* dst_start, const int64_t* dst_step, const int64_t* counts,
                     const void* scalar8, cnh_stream s);

@@ -283,3 +283,96 @@ def test_view_of_view_assignment_and_inplace_update(small_tiles):
     a[5, :] += a[6, :] * 2.0
     host[5, :] += host[6, :] * 2.0
     assert np.array_equal(a.get(small_tiles), host)
+
+
+# ---- the LSTM forward pass of upstream's example, statement for statement ----
+
+def _lstm_numpy(X, h0, W, n, b, d, word):
+    import math
+    sig = np.vectorize(lambda v: 1.0 / (1.0 + math.exp(v * -1)))
+    tanh = np.vectorize(math.tanh)
+    Hin = np.zeros((n, b, word + d))
+    Hout = np.zeros((n, b, d))
+    IFOG = np.zeros((n, b, 4 * d))
+    IFOGf = np.zeros((n, b, 4 * d))
+    Cc = np.zeros((n, b, d))
+    Ct = np.zeros((n, b, d))
+    for t in range(n):
+        prev = np.tile(h0, (b, 1)) if t == 0 else Hout[t - 1]
+        Hin[t, :, :word] = X[t]
+        Hin[t, :, word:] = prev
+        IFOG[t] = Hin[t].dot(W)
+        IFOGf[t, :, :3 * d] = sig(IFOG[t, :, :3 * d])
+        IFOGf[t, :, 3 * d:] = tanh(IFOG[t, :, 3 * d:])
+        Cc[t] = IFOGf[t, :, :d] * IFOGf[t, :, 3 * d:]
+        if t > 0:
+            Cc[t] += IFOGf[t, :, d:2 * d] * Cc[t - 1]
+        Ct[t] = tanh(Cc[t])
+        Hout[t] = IFOGf[t, :, 2 * d:3 * d] * Ct[t]
+    return Hout, Cc, IFOG
+
+
+@pytest.mark.parametrize("n,b,d,word,small", [(4, 32, 10, 10, False), (3, 48, 40, 24, True)])
+def test_lstm_forward_example(itf, n, b, d, word, small):
+    """examples/lstm_forward.py upstream: 3-D state arrays, one time step per leading index, a
+    dimension-dropped matmul per step, tile() for the first hidden state, in-place cell update."""
+    if small:
+        itf.set_min_tile(2, 16)
+        itf.set_min_tile(3, 8)
+    rng = np.random.default_rng(5)
+    hX = rng.uniform(-1, 1, (n, b, word))
+    hh0 = rng.uniform(-1, 1, (1, d))
+    hW = rng.uniform(-1, 1, (word + d, 4 * d)) / np.sqrt(word + d)
+    X, h0, WLSTM = cnp.array(hX), cnp.array(hh0), cnp.array(hW)
+    xphpb = word + d
+    Hin = cnp.zeros((n, b, xphpb))
+    Hout = cnp.zeros((n, b, d))
+    IFOG = cnp.zeros((n, b, d * 4))
+    IFOGf = cnp.zeros((n, b, d * 4))
+    Cs = cnp.zeros((n, b, d))
+    Ct = cnp.zeros((n, b, d))
+    for t in range(n):
+        prev = cnp.tile(h0, (b, 1)) if t == 0 else Hout[t - 1]
+        Hin[t, :, :word] = X[t]
+        Hin[t, :, word:] = prev
+        IFOG[t] = Hin[t].dot(WLSTM)
+        IFOGf[t, :, : 3 * d] = 1.0 / (1.0 + cnp.exp(-IFOG[t, :, : 3 * d]))
+        IFOGf[t, :, 3 * d:] = cnp.tanh(IFOG[t, :, 3 * d:])
+        Cs[t] = IFOGf[t, :, :d] * IFOGf[t, :, 3 * d:]
+        if t > 0:
+            Cs[t] += IFOGf[t, :, d: 2 * d] * Cs[t - 1]
+        Ct[t] = cnp.tanh(Cs[t])
+        Hout[t] = IFOGf[t, :, 2 * d: 3 * d] * Ct[t]
+    wH, wC, wI = _lstm_numpy(hX, hh0, hW, n, b, d, word)
+    gI = IFOG.get(itf)
+    bound = 1e-12 * (np.abs(np.concatenate([hX[0], np.tile(hh0, (b, 1))], axis=1)) @ np.abs(hW))
+    assert np.all(np.abs(gI[0] - wI[0]) <= bound)
+    assert np.allclose(Cs.get(itf), wC, rtol=1e-11, atol=1e-13)
+    assert np.allclose(Hout.get(itf), wH, rtol=1e-11, atol=1e-13)
+
+
+def test_tile_matches_numpy(small_tiles):
+    host = np.arange(12, dtype=np.float64).reshape(3, 4)
+    a = cnp.array(host)
+    for reps in [(2, 3), (1, 1), 2, (2, 1, 2), (5, 1)]:
+        assert np.array_equal(cnp.tile(a, reps).get(small_tiles), np.tile(host, reps))
+    row = cnp.array(np.arange(7, dtype=np.float64).reshape(1, 7))
+    assert np.array_equal(cnp.tile(row, (40, 1)).get(small_tiles), np.tile(np.arange(7.0).reshape(1, 7), (40, 1)))
+    v = cnp.arange(5, dtype=np.float64)
+    assert np.array_equal(cnp.tile(v, (3, 2)).get(small_tiles), np.tile(np.arange(5.0), (3, 2)))
+
+
+def test_disjoint_self_reference_updates_in_place(itf):
+    """C[t] = f(C[t-1]) reads and writes disjoint slabs of one array: no second buffer is needed,
+    and the values are those of the sequential program."""
+    n, b, d = 5, 8, 16
+    host = np.random.default_rng(1).standard_normal((n, b, d))
+    Cs = cnp.array(host)
+    itf.set_trace()
+    for t in range(1, n):
+        Cs[t] = Cs[t] * 0.5 + Cs[t - 1]
+        host[t] = host[t] * 0.5 + host[t - 1]
+    got = Cs.get(itf)
+    assert np.array_equal(got, host)
+    groups = [ln for ln in itf.trace() if ln.startswith("group")]
+    assert len(groups) == n - 1 and all("inplace" in g for g in groups)
