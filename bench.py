@@ -726,6 +726,46 @@ def run_frontend(n, steps, warmup):
             del u
             cnp.execute(it16)
             it16.close()
+        # configuration 5 written as upstream's example writes it (examples/lstm_forward.py upstream)
+        n, b, word, d = 64, 256, 1024, 1024
+        itl = cnp.CharmNumericInterface(device=0)
+        itl.connect(odf=4)
+        cnp.set_auto_flush(itl, 48)
+        X = cnp.random.uniform((n, b, word), seed=5, stream=0, low=-1.0, high=1.0)
+        W = cnp.random.uniform((word + d, 4 * d), seed=5, stream=1, low=-1.0 / 32, high=1.0 / 32)
+        h0 = cnp.zeros((1, d))
+        Hin = cnp.zeros((n, b, word + d))
+        Hout = cnp.zeros((n, b, d))
+        IFOG = cnp.zeros((n, b, 4 * d))
+        IFOGf = cnp.zeros((n, b, 4 * d))
+        Cs = cnp.zeros((n, b, d))
+        Ct = cnp.zeros((n, b, d))
+
+        def lstm_steps(t0, t1):
+            for t in range(t0, t1):
+                prev = cnp.tile(h0, (b, 1)) if t == 0 else Hout[t - 1]
+                Hin[t, :, :word] = X[t]
+                Hin[t, :, word:] = prev
+                IFOG[t] = Hin[t].dot(W)
+                IFOGf[t, :, : 3 * d] = 1.0 / (1.0 + cnp.exp(-IFOG[t, :, : 3 * d]))
+                IFOGf[t, :, 3 * d:] = cnp.tanh(IFOG[t, :, 3 * d:])
+                Cs[t] = IFOGf[t, :, :d] * IFOGf[t, :, 3 * d:]
+                if t > 0:
+                    Cs[t] += IFOGf[t, :, d: 2 * d] * Cs[t - 1]
+                Ct[t] = cnp.tanh(Cs[t])
+                Hout[t] = IFOGf[t, :, 2 * d: 3 * d] * Ct[t]
+            cnp.execute(itl)
+            itl.sync()
+
+        lstm_steps(0, 4)
+        t0 = time.perf_counter()
+        lstm_steps(4, n)
+        dt = time.perf_counter() - t0
+        out["lstm_us_per_step"] = round(dt / (n - 4) * 1e6, 1)
+        out["lstm_h_last_abs_mean"] = float(np.mean(np.abs(Hout[n - 1].get(itl))))
+        del X, W, h0, Hin, Hout, IFOG, IFOGf, Cs, Ct
+        cnp.execute(itl)
+        itl.close()
     finally:
         cnp.reset()
         itf.close()

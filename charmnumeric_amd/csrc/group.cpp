@@ -9,16 +9,25 @@
 
 #include <cstring>
 #include <map>
+#include <memory>
 #include <mutex>
 #include <vector>
 
 using namespace cnh;
 
-struct KernelVariant {
+// Code object of one generated source text. Kernels whose variants generate the same text (the
+// same group at another place of an array: regions travel as launch arguments) share it, so a
+// time loop over slabs compiles once. Code objects live as long as the library.
+struct CodeObject {
     std::string src;
     std::vector<char> code;
     hipModule_t mod = nullptr;
     std::map<std::string, hipFunction_t> fns;
+};
+
+struct KernelVariant {
+    std::string src;
+    std::shared_ptr<CodeObject> obj;
 };
 
 struct cnh_kernel {
@@ -32,10 +41,21 @@ namespace {
 
 std::mutex g_kmu;
 std::map<uint64_t, cnh_kernel*> g_kernels; // key -> kernel (key 0 = not cached)
+std::multimap<uint64_t, std::shared_ptr<CodeObject>> g_code; // hash of the source text -> code object
+std::mutex g_cmu;                                             // guards g_code
+
+uint64_t text_hash(const std::string& t) {
+    uint64_t h = 1469598103934665603ull;
+    for (unsigned char c : t) {
+        h ^= c;
+        h *= 1099511628211ull;
+    }
+    return h;
+}
 
 int build_variant(cnh_kernel* k, const std::string& variant, KernelVariant** out) {
     auto it = k->variants.find(variant);
-    if (it != k->variants.end() && !it->second.code.empty()) {
+    if (it != k->variants.end() && it->second.obj) {
         *out = &it->second;
         return 0;
     }
@@ -47,6 +67,17 @@ int build_variant(cnh_kernel* k, const std::string& variant, KernelVariant** out
             k->variants.erase(variant);
             return set_error(rc, "codegen(%s): %s", variant.c_str(), err.c_str());
         }
+    }
+    const uint64_t h = text_hash(v.src);
+    std::lock_guard<std::mutex> code_lock(g_cmu);
+    {
+        auto range = g_code.equal_range(h);
+        for (auto c = range.first; c != range.second; ++c)
+            if (c->second->src == v.src) {
+                v.obj = c->second;
+                *out = &v;
+                return 0;
+            }
     }
     hiprtcProgram prog;
     hiprtcResult r = hiprtcCreateProgram(&prog, v.src.c_str(), "cnh_group.hip", 0, nullptr, nullptr);
@@ -69,9 +100,13 @@ int build_variant(cnh_kernel* k, const std::string& variant, KernelVariant** out
     }
     size_t cs = 0;
     hiprtcGetCodeSize(prog, &cs);
-    v.code.resize(cs);
-    hiprtcGetCode(prog, v.code.data());
+    auto obj = std::make_shared<CodeObject>();
+    obj->src = v.src;
+    obj->code.resize(cs);
+    hiprtcGetCode(prog, obj->code.data());
     hiprtcDestroyProgram(&prog);
+    g_code.emplace(h, obj);
+    v.obj = obj;
     *out = &v;
     return 0;
 }
@@ -80,13 +115,14 @@ int get_function(cnh_kernel* k, const std::string& variant, const char* name, hi
     KernelVariant* v = nullptr;
     if (int rc = build_variant(k, variant, &v))
         return rc;
-    if (!v->mod)
-        CNH_HIP(hipModuleLoadData(&v->mod, v->code.data()));
-    auto it = v->fns.find(name);
-    if (it == v->fns.end()) {
+    CodeObject* c = v->obj.get();
+    if (!c->mod)
+        CNH_HIP(hipModuleLoadData(&c->mod, c->code.data()));
+    auto it = c->fns.find(name);
+    if (it == c->fns.end()) {
         hipFunction_t f;
-        CNH_HIP(hipModuleGetFunction(&f, v->mod, name));
-        it = v->fns.emplace(name, f).first;
+        CNH_HIP(hipModuleGetFunction(&f, c->mod, name));
+        it = c->fns.emplace(name, f).first;
     }
     *fn = it->second;
     return 0;
@@ -168,9 +204,6 @@ int cnh_kernel_release(cnh_kernel* k) {
     std::lock_guard<std::mutex> lk(g_kmu);
     if (--k->refs > 0)
         return 0;
-    for (auto& kv : k->variants)
-        if (kv.second.mod)
-            (void)hipModuleUnload(kv.second.mod);
     if (k->key != 0)
         g_kernels.erase(k->key);
     delete k;
