@@ -121,7 +121,12 @@ struct cnx_executor {
     int min_tile[4] = {0, 262144, 512, 64}; // CT_MIN_TILE_1D/2D/3D, src/backend.hpp:10-18
     cnh_stream stream = nullptr;
     std::map<int, XArray> arrays;
-    std::unordered_map<uint64_t, cnh_kernel*> kernels; // compile_cache, src/dag_group_compile.cpp:43-56
+    // compile_cache (src/dag_group_compile.cpp:43-56), bounded: a time loop over slabs makes a new
+    // group (same code, other regions) per step, and the oldest ones are let go
+    std::unordered_map<uint64_t, cnh_kernel*> kernels;
+    std::vector<uint64_t> kernel_order;
+    size_t kernel_next_evict = 0;
+    size_t max_kernels = 4096;
     std::map<size_t, std::vector<void*>> free_list;    // src/backend.hpp:366-545
     int64_t stats[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     bool trace_on = false;
@@ -449,6 +454,18 @@ int compile_cached(Ex* ex, Group& g, cnh_kernel** out) {
     if (int rc = cnh_compile_group(&ast, g.dtype, g.ndims, g.key, &k))
         return rc;
     ex->stats[0]++;
+    if (ex->kernel_order.size() < ex->max_kernels) {
+        ex->kernel_order.push_back(g.key);
+    } else { // ring: replace the oldest entry
+        const uint64_t old = ex->kernel_order[ex->kernel_next_evict];
+        auto victim = ex->kernels.find(old);
+        if (victim != ex->kernels.end()) {
+            cnh_kernel_release(victim->second);
+            ex->kernels.erase(victim);
+        }
+        ex->kernel_order[ex->kernel_next_evict] = g.key;
+        ex->kernel_next_evict = (ex->kernel_next_evict + 1) % ex->max_kernels;
+    }
     ex->kernels[g.key] = k;
     *out = k;
     return 0;
@@ -1111,8 +1128,8 @@ int cnx_destroy(cnx_executor* ex) {
                 cnh_free(p);
         cnh_stream_destroy(ex->stream);
     }
-    // Kernels stay in the library-wide cache (keyed by content), as upstream's compile_cache does
-    // for the life of the process.
+    for (auto& kv : ex->kernels)
+        cnh_kernel_release(kv.second);
     delete ex;
     return 0;
 }

@@ -190,10 +190,8 @@ int cnh_compile_group(const cnh_ast* ast, int dtype, int ndims, uint64_t key, cn
         return set_error(rc, "cnh_compile_group: %s", err.c_str());
     }
     k->key = key;
-    if (key != 0) {
-        g_kernels[key] = k;
-        k->refs++; // the cache holds one reference
-    }
+    if (key != 0)
+        g_kernels[key] = k; // found again by key while somebody holds it; gone with its last user
     *out = k;
     return 0;
 }

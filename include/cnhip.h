@@ -144,6 +144,9 @@ typedef struct cnh_kernel cnh_kernel;
  * does on a null compile result (src/execute_node.cpp:102-112). Code objects are built with
  * hipRTC on first launch of each kernel variant. */
 int cnh_compile_group(const cnh_ast* ast, int dtype, int ndims, uint64_t key, cnh_kernel** out);
+/* Drops one reference; the kernel object goes with its last holder (a later compile with the same
+ * key builds it again). Code objects are shared between kernels with identical generated text
+ * and stay loaded. */
 int cnh_kernel_release(cnh_kernel* k);
 /* Argument counts in the upstream order: memref per leaf use, scalar per unique broadcast leaf,
  * memref per non-temp root (src/jit.cpp:78-87). */

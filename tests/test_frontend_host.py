@@ -267,3 +267,19 @@ def test_auto_flush_never_splits_a_stencil_statement(itf):
     assert len(groups) == 10 and all("pingpong" in g and "inputs=4" in g for g in groups)
     st = itf.stats()
     assert st["live_arrays"] == 1 and st["compiled"] == 1 and st["cache_hits"] == 9
+
+
+def test_kernel_cache_is_bounded_over_a_long_slab_loop(itf):
+    """Each step assigns another slab: another group (same code, other regions). The executor keeps
+    a bounded number of them and lets the oldest go."""
+    n = 4500
+    a = cnp.zeros((n, 8))
+    for t in range(1, n):
+        a[t] = a[t - 1] * 0.5
+    cnp.execute(itf)
+    st = itf.stats()
+    assert st["compiled"] == n - 1 and st["group_launches"] == n - 1
+    # the first slabs were evicted: assigning them again compiles again instead of hitting the cache
+    a[1] = a[0] * 0.5
+    cnp.execute(itf)
+    assert itf.stats()["compiled"] == n
