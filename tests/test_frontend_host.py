@@ -283,3 +283,86 @@ def test_kernel_cache_is_bounded_over_a_long_slab_loop(itf):
     a[1] = a[0] * 0.5
     cnp.execute(itf)
     assert itf.stats()["compiled"] == n
+
+
+# ---- error behaviour of the executor (messages built by hand where the frontend would refuse) ----
+
+def _message(nodes_bytes):
+    return struct.pack("<iii", lazy.DAG_MAGIC, 1, len(nodes_bytes)) + b"".join(nodes_bytes)
+
+
+def _create(name, shape, dtype, node_id=0):
+    w = lazy._NodeWriter()
+    w.op(name, L.OP_CREATE, False, len(shape), dtype, [], [], lazy._full_region(shape))
+    return w.to_bytes(node_id, False)
+
+
+def test_executor_refuses_what_it_cannot_do(itf):
+    itf.send_dag(0, _message([_create(1, (8, 8), L.F64), _create(2, (8,), L.F64), _create(3, (8,), L.F32),
+                              _create(4, (9,), L.F64)]))
+    ref = lambda name, nd, dt=L.F64: lazy.ArrayRef(name, None, (8,) * nd, nd, dt)
+
+    def nonfusible(opcode, operands, shape, dtype=L.F64, name=50):
+        w = lazy._NodeWriter()
+        w.op(name, opcode, False, len(shape), dtype, [w.leaf(o) for o in operands], [None] * len(operands),
+             lazy._full_region(shape))
+        return _message([w.to_bytes(9, False)])
+
+    with pytest.raises(RuntimeError, match="not supported"):
+        itf.send_dag(1, nonfusible(L.OP_DIAG, [ref(2, 1)], (8, 8)))
+    with pytest.raises(RuntimeError, match="1-D operands"):
+        itf.send_dag(1, nonfusible(L.OP_REDUCE, [ref(1, 2), ref(1, 2)], (1,)))
+    with pytest.raises(RuntimeError, match="dtypes"):
+        itf.send_dag(1, nonfusible(L.OP_REDUCE, [ref(2, 1), ref(3, 1, L.F32)], (1,)))
+    with pytest.raises(RuntimeError, match="lengths"):
+        itf.send_dag(1, nonfusible(L.OP_REDUCE, [ref(2, 1), ref(4, 1)], (1,)))
+    with pytest.raises(RuntimeError, match="columns"):
+        itf.send_dag(1, nonfusible(L.OP_MATMUL, [ref(1, 2), ref(4, 1)], (8,)))
+    with pytest.raises(RuntimeError, match="does not exist"):
+        itf.send_dag(1, nonfusible(L.OP_REDUCE, [ref(77, 1), ref(2, 1)], (1,)))
+    with pytest.raises(RuntimeError, match="already exists"):
+        itf.send_dag(1, _message([_create(2, (8,), L.F64)]))
+    # a fill whose region leaves the array
+    w = lazy._NodeWriter()
+    t = w.leaf(ref(2, 1))
+    v = w.scalar(1.0, 1, L.F64)
+    w.op(60, L.OP_SET_REGION, False, 1, L.F64, [t, v], [None, None], ((0,), (12,), (1,)))
+    with pytest.raises(RuntimeError, match="leaves extent"):
+        itf.send_dag(1, _message([w.to_bytes(3, False)]))
+    # a group over arrays of another dtype than it computes in
+    w = lazy._NodeWriter()
+    a32 = w.leaf(ref(3, 1, L.F32))
+    w.op(61, L.OP_ADD, False, 1, L.F64, [a32, w.scalar(1.0, 1, L.F64)], [None, None], lazy._full_region((8,)))
+    with pytest.raises(RuntimeError, match="dtype"):
+        itf.send_dag(1, _message([w.to_bytes(4, True)]))
+    # nothing of the above left a half-made result behind that blocks later work
+    a = cnp.Array((8,), np.float64, name=2)
+    a._gen = -1                                   # a borrowed name: never deleted by this handle
+    assert itf.get(1, 2, 8).shape == (8,)
+
+
+def test_frontend_refuses_like_upstream():
+    cnp.reset()
+    a = cnp.zeros((4, 5))
+    with pytest.raises(NotImplementedError):
+        cnp.diag(cnp.zeros((4,)))
+    with pytest.raises(NotImplementedError):
+        a[::-1]
+    with pytest.raises(NotImplementedError):
+        a.astype(np.float32)
+    with pytest.raises(ValueError):
+        a[0:2, 0:2] = cnp.zeros((3, 3))
+    with pytest.raises(ValueError):
+        cnp.zeros((2, 3, 4)) @ cnp.zeros((4, 2))      # no extent of 1 to drop
+    with pytest.raises(ValueError):
+        cnp.matmul(2.0, a)
+    with pytest.raises(NotImplementedError):
+        cnp.zeros((0, 3))
+    with pytest.raises(NotImplementedError):
+        cnp.zeros((2, 2, 2, 2))
+    assert cnp.add(2, 3) == 5 and cnp.dot(2.0, 4.0) == 8.0
+    assert cnp.tanh(0.0) == 0.0 and cnp.exp(0) == 1.0
+    assert cnp.full((3,), 7).dtype == np.int64 and cnp.ones((2, 2)).dtype == np.float64
+    assert cnp.arange(5).shape == (5,) and cnp.eye(3).shape == (3, 3)
+    assert cnp.zeros_like(a).shape == (4, 5) and cnp.empty_like(a, dtype=np.int32).dtype == np.int32
+    cnp.reset()
