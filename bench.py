@@ -380,6 +380,8 @@ class TiledDev:
             # measured on MI355X: 64 tiles of 128^3 (16 MiB each) back to back 462 us per sweep,
             # 2 MiB + 256 B apart 424 us; tiles of 2048^2 are best back to back
             skew = (2 << 20) + 256 if nd == 3 else 0
+            if os.environ.get("CNH_BENCH_SKEW"):
+                skew = int(os.environ["CNH_BENCH_SKEW"])
         exts = [[min(tile, n - i * tile) for i in idx] for idx in np.ndindex(*([self.g] * nd))]
         offs, off = [], 0
         for ext in exts:

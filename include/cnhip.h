@@ -88,9 +88,15 @@ int cnh_init(int device);               /* selects the device; idempotent */
 const char* cnh_last_error(void);
 int cnh_device_name(char* buf, size_t cap);
 int cnh_version(void);
-/* Tuning switches. "stencil_mode" picks the kernel cnh_launch_group_tiles uses for same-array
- * unit-step stencils: 2 (default) register window, 1 LDS sliding window, 0 general gather.
- * "direct_tx/ry/rz" and "slide_bx/ry/zc/pd", "slide2d_march" override the kernel geometry. */
+/* Tuning switches (defaults are what measured best on MI355X; 0 restores a default geometry).
+ *   "stencil_mode"   kernel cnh_launch_group_tiles uses for same-array unit-step stencils:
+ *                    2 (default) register window, 1 LDS sliding window, 0 general gather
+ *   "direct_tx/ry/rz"  register window: lanes along x per workgroup row, rows and planes per lane
+ *   "direct_lean"    wavefront-level lean kernel with lane exchange: 1 on, 0 off, -1 (default) rank 2 only
+ *   "direct_group"   workgroup order for rank 3: 0 (default) tile by tile, 1 groups of G^3 tiles,
+ *                    2 rows of tiles along x
+ *   "direct_stagger" concurrent groups start at different places of their tiles (default 0)
+ *   "slide_bx/ry/zc/pd", "slide2d_march"  geometry of the sliding-window kernel */
 int cnh_set_option(const char* name, int value);
 
 /* ---- storage: Array<N,T> ctor zero-fill / data_ptr / copyToHost / copyToDevice / dtor
