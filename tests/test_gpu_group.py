@@ -221,6 +221,31 @@ def test_exp_tanh_within_one_ulp_of_host_libm(dev, orc):
     assert np.all(np.diff(em) >= 0)  # monotone
 
 
+def test_exp_tanh_fp32_against_host_libm(dev, orc):
+    """fp32 groups call the device library's expf/tanhf (no configuration uses fp32
+    transcendentals); this records how far they are from the host's expf/tanhf, which the oracle
+    calls, and holds them to 2 ulp."""
+    xs = np.concatenate([np.linspace(-30, 30, 100001), np.array([0.0, -0.0, 1e-20, 80.0, -100.0])]
+                        ).astype(np.float32)
+    for which, opc in (("tanhf", L.OP_TANH), ("expf", L.OP_EXP)):
+        b = AstBuilder(L.F32, 1)
+        b.unary(opc, 2, b.leaf(0), is_temp=False)
+        ast = b.finish()
+        k = H.compile_group(ast, L.F32, 1)
+        dx = dev.array(xs)
+        out = dev.empty(xs.shape, np.float32)
+        H.launch_batched(k, 1, [[dx.memref()]], [], [[out.memref()]])
+        got = out.get()
+        dev.free_all()
+        want = np.empty_like(xs)
+        assert orc.eval_group(ast, L.F32, 1, [xs], [], [want]) == 0
+        finite = np.isfinite(want) & np.isfinite(got)
+        assert np.array_equal(np.isfinite(want), np.isfinite(got))
+        d = H.ulp_distance(got[finite], want[finite])
+        print(f"{which}: max {d} ulp vs host libm")
+        assert d <= 2, f"{which}: {d} ulp"
+
+
 def test_sigmoid_chain(dev, orc):
     """1.0/(1.0+exp(x*-1)): the + - * / around exp are exact given the device's own exp; against
     the host-libm chain the result is identical where the host's exp is the one the device code
