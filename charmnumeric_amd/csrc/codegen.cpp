@@ -317,8 +317,10 @@ std::string prelude(const GroupProgram& p) {
               << "__device__ __forceinline__ T cn_exp(T x) { return cn_exp_f64(x); }\n"
                  "__device__ __forceinline__ T cn_tanh(T x) { return cn_tanh_f64(x); }\n";
     } else {
-        s << "__device__ __forceinline__ T cn_exp(T x) { return expf(x); }\n"
-             "__device__ __forceinline__ T cn_tanh(T x) { return tanhf(x); }\n";
+        if (p.body.find("cn_exp(") != std::string::npos || p.body.find("cn_tanh(") != std::string::npos)
+            s << libm_f32_text()
+              << "__device__ __forceinline__ T cn_exp(T x) { return cn_exp_f32(x); }\n"
+                 "__device__ __forceinline__ T cn_tanh(T x) { return cn_tanh_f32(x); }\n";
     }
     s << "__device__ __forceinline__ void load_scalars(const Scal& sc, T* s) {\n"
          "#pragma unroll\n"

@@ -89,5 +89,6 @@ const char* dtype_ctype(int dtype);
 
 // fp64 exp/tanh restated to agree bit for bit with the host C library (codegen_libm.cpp).
 std::string libm_f64_text();
+std::string libm_f32_text();
 
 } // namespace cnh

@@ -222,9 +222,9 @@ def test_exp_tanh_within_one_ulp_of_host_libm(dev, orc):
 
 
 def test_exp_tanh_fp32_against_host_libm(dev, orc):
-    """fp32 groups call the device library's expf/tanhf (no configuration uses fp32
-    transcendentals); this records how far they are from the host's expf/tanhf, which the oracle
-    calls, and holds them to 2 ulp."""
+    """fp32 groups carry a restatement of the host's expf/tanhf, which the oracle calls: tanhf is
+    identical, expf identical but for about one input in a billion that lands on the
+    neighbouring float."""
     xs = np.concatenate([np.linspace(-30, 30, 100001), np.array([0.0, -0.0, 1e-20, 80.0, -100.0])]
                         ).astype(np.float32)
     for which, opc in (("tanhf", L.OP_TANH), ("expf", L.OP_EXP)):
@@ -243,7 +243,9 @@ def test_exp_tanh_fp32_against_host_libm(dev, orc):
         assert np.array_equal(np.isfinite(want), np.isfinite(got))
         d = H.ulp_distance(got[finite], want[finite])
         print(f"{which}: max {d} ulp vs host libm")
-        assert d <= 2, f"{which}: {d} ulp"
+        assert d <= 1, f"{which}: {d} ulp"
+        if H.host_libm_is_the_restated_one():
+            assert np.array_equal(got[finite].view(np.uint32), want[finite].view(np.uint32)), which
 
 
 def test_sigmoid_chain(dev, orc):

@@ -71,6 +71,73 @@ def test_device_exp_tanh_text_matches_host_libm(tmp_path):
         assert bad_e == 0 and bad_t == 0
 
 
+DRIVER_F32 = r"""
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+static const unsigned long long CN_EXP2F_TAB[32] = {
+#include "exp2f_table.inc"
+};
+#define CN_DEV static inline
+#include "libm_body_f32.inc"
+static long ulps(float a, float b) {
+    if (std::isnan(a) && std::isnan(b)) return 0;
+    int32_t x, y; memcpy(&x, &a, 4); memcpy(&y, &b, 4);
+    if (x < 0) x = INT32_MIN - x; if (y < 0) y = INT32_MIN - y;
+    return (long)(x > y ? (int64_t)x - y : (int64_t)y - x);
+}
+int main() {
+    // every 37th float bit pattern (116 million values of each sign and magnitude), plus the
+    // neighbourhoods of every threshold either function branches on
+    long worst_e = 0, worst_t = 0, bad_e = 0, bad_t = 0;
+    auto one = [&](uint32_t u) {
+        float x; memcpy(&x, &u, 4);
+        long de = ulps(expf(x), cn_exp_f32(x)), dt = ulps(tanhf(x), cn_tanh_f32(x));
+        if (de) { ++bad_e; if (de > worst_e) worst_e = de; }
+        if (dt) { ++bad_t; if (dt > worst_t) worst_t = dt; }
+    };
+    for (uint64_t u = 0; u < (1ull << 32); u += 37) one((uint32_t)u);
+    const uint32_t edges[] = {0x42b00000u, 0x42b17218u, 0x42cff1b4u, 0x4195b844u, 0x3eb17218u, 0x3f851592u,
+                              0x33000000u, 0x41b00000u, 0x24000000u, 0x3f800000u, 0x7f800000u, 0u};
+    for (uint32_t e : edges)
+        for (int d = -2000; d <= 2000; ++d) { one(e + d); one((e + d) ^ 0x80000000u); }
+    printf("%ld %ld %ld %ld\n", bad_e, worst_e, bad_t, worst_t);
+    return 0;
+}
+"""
+
+
+def test_device_exp_tanh_fp32_text_matches_host_libm(tmp_path):
+    """tanhf must agree everywhere; expf everywhere but a few inputs in a billion (one known:
+    x = -0x1.f8cbb2p+5, where the host returns the neighbouring float)."""
+    body = open(os.path.join(CSRC, "libm_f32.inc")).read().splitlines()
+    assert body[0].startswith('R"CNLIBM(') and body[-1].startswith(')CNLIBM"')
+    (tmp_path / "libm_body_f32.inc").write_text("\n".join(body[1:-1]) + "\n")
+    (tmp_path / "driver.cpp").write_text(DRIVER_F32)
+    exe = tmp_path / "driver"
+    subprocess.check_call(["g++", "-O2", "-std=c++17", "-ffp-contract=off", "-mfma", "-I", CSRC,
+                           "-I", str(tmp_path), str(tmp_path / "driver.cpp"), "-o", str(exe)])
+    bad_e, worst_e, bad_t, worst_t = (int(t) for t in subprocess.check_output([str(exe)]).split())
+    print(f"expf: {bad_e} differing (worst {worst_e} ulp); tanhf: {bad_t} differing (worst {worst_t} ulp)")
+    assert worst_e <= 1 and worst_t <= 1
+    if H.host_libm_is_the_restated_one():
+        assert bad_e <= 2 and bad_t == 0
+
+
+def test_exp2f_table_is_what_its_definition_gives():
+    mp = pytest.importorskip("mpmath")
+    import struct
+    mp.mp.prec = 200
+    words = []
+    for ln in open(os.path.join(CSRC, "exp2f_table.inc")):
+        words += [int(t.strip().rstrip("ul"), 16) for t in ln.split(",") if t.strip().startswith("0x")]
+    assert len(words) == 32
+    for k in range(32):
+        h = struct.unpack("<d", struct.pack("<Q", (words[k] + (k << 47)) & (2**64 - 1)))[0]
+        assert h == float(mp.power(2, mp.mpf(k) / 32))
+
+
 def test_exp_table_is_what_its_definition_gives():
     mp = pytest.importorskip("mpmath")
     import struct
@@ -102,3 +169,13 @@ def test_group_with_exp_and_tanh_builds_for_gfx950(variant):
     L.check(L.lib.cnh_kernel_build(k, variant.encode()))
     # groups without exp/tanh do not carry the text
     assert "cn_exp_f64" not in H.kernel_source(H.compile_group(H.ast_c1(L.F64), L.F64, 1), variant)
+
+
+def test_fp32_group_with_exp_and_tanh_builds_for_gfx950():
+    b = AstBuilder(L.F32, 1)
+    t1 = b.unary(L.OP_EXP, 101, b.leaf(1))
+    b.unary(L.OP_TANH, 2, t1, is_temp=False)
+    k = H.compile_group(b.finish(), L.F32, 1)
+    src = H.kernel_source(k, "flat")
+    assert "cn_exp_f32" in src and "CN_EXP2F_TAB" in src and "cn_exp_f64" not in src
+    L.check(L.lib.cnh_kernel_build(k, b"flat"))
