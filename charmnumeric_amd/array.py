@@ -421,9 +421,10 @@ def _whole(x):
 
 
 def nonfusible(opcode, operands, shape, dtype):
-    operands = [_whole(o) for o in operands]
+    operands = [_whole(o) if isinstance(o, _ArrayLike) else o for o in operands]
     out = Array(shape, dtype)
-    lazy.record(lazy.Instr("nonfusible", name=out.name, opcode=opcode, operands=[o._ref() for o in operands],
+    lazy.record(lazy.Instr("nonfusible", name=out.name, opcode=opcode,
+                           operands=[o._ref() if isinstance(o, _ArrayLike) else o for o in operands],
                            shape=shape, dtype=out.wire_dtype()))
     return out
 
@@ -457,8 +458,6 @@ def _matmul(lhs, rhs):
         if lhs.shape[0] != rhs.shape[0]:
             raise ValueError(f"Shape mismatch for dot product: ({lhs.shape[0]},) @ ({rhs.shape[0]},)")
         return nonfusible(L.OP_REDUCE, [lhs, rhs], (1,), _same_dtype(lhs, rhs, "dot"))
-    if lhs.ndims == 3 and rhs.ndims == 1:
-        raise NotImplementedError("matvec on a 3-D operand with a dropped dimension is not implemented")
     if lhs.ndims not in (2, 3):
         raise ValueError(f"matmul requires a 2D matrix, got {lhs.ndims}D")
     if rhs.ndims == 1:
@@ -489,13 +488,22 @@ def _matrix_shape(x):
 def _matvec(mat, vec):
     if not isinstance(vec, _ArrayLike):
         raise ValueError("matvec requires an Array vector")
-    if mat.ndims != 2:
-        raise NotImplementedError(f"matvec on a {mat.ndims}D operand is not implemented")
+    if vec.ndims == 2 and vec.shape[1] == 1:
+        raise NotImplementedError("matvec with an (N, 1) column operand is not implemented")
     if vec.ndims != 1:
-        raise ValueError("matvec requires a 1D vector (N,)")
-    if mat.shape[1] != vec.shape[0]:
-        raise ValueError(f"Shape mismatch: matrix cols {mat.shape[1]} != vector size {vec.shape[0]}")
-    return nonfusible(L.OP_MATMUL, [mat, vec], (mat.shape[0],), _same_dtype(mat, vec, "matvec"))
+        raise ValueError("matvec requires a 1D vector (N,) or 2D column vector (N, 1)")
+    if mat.ndims == 2:
+        rows, cols = mat.shape
+    elif mat.ndims == 3:
+        ones = [d for d in range(3) if mat.shape[d] == 1]
+        if len(ones) != 1:
+            raise ValueError(f"3D matvec requires exactly one singleton dimension, got shape {mat.shape}")
+        rows, cols = (mat.shape[d] for d in range(3) if d != ones[0])
+    else:
+        raise ValueError(f"matvec requires a 2D or 3D matrix, got {mat.ndims}D")
+    if cols != vec.shape[0]:
+        raise ValueError(f"Shape mismatch: matrix cols {cols} != vector size {vec.shape[0]}")
+    return nonfusible(L.OP_MATMUL, [mat, vec], (rows,), _same_dtype(mat, vec, "matvec"))
 
 
 # ---------------------------------------------------------------------------------------------

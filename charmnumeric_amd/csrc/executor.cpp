@@ -775,32 +775,6 @@ int exec_reduce_ext(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
                                  out->tiles[0], ex->stream);
 }
 
-// MATMUL: tile GEMVs, column tiles summed in index order (src/executor_matmul.cpp:150-498,
-// src/execute_node.cpp:116-273,489-583).
-int exec_matmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
-    XArray *A, *x;
-    if (int rc = leaf_array(ex, n, root, 0, &A, "MATMUL"))
-        return rc;
-    if (int rc = leaf_array(ex, n, root, 1, &x, "MATMUL"))
-        return rc;
-    CNH_CHECK(A->ndims == 2 && x->ndims == 1, -31, "MATMUL needs a 2-D and a 1-D operand");
-    CNH_CHECK(A->shape[1] == x->shape[0], -31, "MATMUL: %d columns, vector of %d", A->shape[1],
-              x->shape[0]);
-    CNH_CHECK(A->dtype == x->dtype, -27, "MATMUL: operand dtypes %d and %d", A->dtype, x->dtype);
-    int32_t shape[3] = {A->shape[0], 1, 1};
-    XArray* y;
-    if (int rc = make_array(ex, root.result_name, 1, A->dtype, shape, false, &y))
-        return rc;
-    ex->log("matmul A=" + std::to_string(A->name) + " tiles=" + std::to_string(A->ntiles) + " x=" +
-            std::to_string(x->name) + " out=" + std::to_string(y->name));
-    if (ex->dry)
-        return 0;
-    std::vector<const void*> pt(A->tiles.begin(), A->tiles.end());
-    // 1-D arrays are contiguous: tile 0 is the whole vector.
-    return cnh_gemv_tiles(A->dtype, A->shape[0], A->shape[1], A->tile, pt.data(), x->tiles[0],
-                          y->tiles[0], ex->stream);
-}
-
 // A 2-D array, or a 3-D array with exactly one extent-1 dimension, seen as a matrix
 // (the dimension-dropped operands of charmnumeric.py:510-519, src/executor_matmatmul.cpp:485-813).
 struct MatView {
@@ -848,6 +822,40 @@ int as_matrix(const XArray& a, MatView* m, const char* what) {
     m->rows = a.shape[m->rd];
     m->cols = a.shape[m->cd];
     return 0;
+}
+
+// MATMUL: tile GEMVs, column tiles summed in index order (src/executor_matmul.cpp:150-498,
+// src/execute_node.cpp:116-273,489-583).
+int exec_matmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
+    XArray *Aa, *x;
+    if (int rc = leaf_array(ex, n, root, 0, &Aa, "MATMUL"))
+        return rc;
+    if (int rc = leaf_array(ex, n, root, 1, &x, "MATMUL"))
+        return rc;
+    // a 3-D matrix operand with one extent of 1 is the plane that remains
+    // (charmnumeric.py:552-563, the K14 case of src/executor_matmul.cpp upstream)
+    MatView A;
+    if (int rc = as_matrix(*Aa, &A, "MATMUL"))
+        return rc;
+    CNH_CHECK(x->ndims == 1, -31, "MATMUL needs a 1-D vector operand");
+    CNH_CHECK(A.cols == x->shape[0], -31, "MATMUL: %d columns, vector of %d", A.cols, x->shape[0]);
+    CNH_CHECK(Aa->dtype == x->dtype, -27, "MATMUL: operand dtypes %d and %d", Aa->dtype, x->dtype);
+    int32_t shape[3] = {A.rows, 1, 1};
+    XArray* y;
+    if (int rc = make_array(ex, root.result_name, 1, Aa->dtype, shape, false, &y))
+        return rc;
+    ex->log("matmul A=" + std::to_string(Aa->name) + " tiles=" + std::to_string(Aa->ntiles) + " x=" +
+            std::to_string(x->name) + " out=" + std::to_string(y->name));
+    if (ex->dry)
+        return 0;
+    const int gr = Aa->grid[A.rd], gc = Aa->grid[A.cd];
+    std::vector<const void*> pt((size_t)gr * gc);
+    for (int tr = 0; tr < gr; ++tr)
+        for (int tc = 0; tc < gc; ++tc)
+            pt[(size_t)tr * gc + tc] = Aa->tiles[(size_t)A.tile_index(tr, tc)];
+    // 1-D arrays are contiguous: tile 0 is the whole vector.
+    return cnh_gemv_tiles(Aa->dtype, A.rows, A.cols, Aa->tile, pt.data(), x->tiles[0], y->tiles[0],
+                          ex->stream);
 }
 
 // MATMATMUL: C (zeroed) += A_panel * B_panel for every k-overlapping pair of tiles, k ascending
@@ -1012,6 +1020,70 @@ int exec_tile(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
     return 0;
 }
 
+// DIAG with numpy.diag's meaning (charmnumeric/operations.py:125-148, src/dag_group_receive.cpp:330-347,
+// src/executor_transfer.cpp:180-358, src/execute_node.cpp:600-720): a vector becomes the k-th
+// diagonal of a zeroed square matrix, a matrix gives up its k-th diagonal. Vector index i pairs with
+// matrix element (i + max(0,-k), i + max(0,k)). One strided copy per matrix tile the diagonal crosses:
+// inside a row-major tile of width w the diagonal is a run with stride w + 1.
+int exec_diag(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
+    XArray* in;
+    if (int rc = leaf_array(ex, n, root, 0, &in, "DIAG"))
+        return rc;
+    int k = 0;
+    if (root.n_operands >= 2) {
+        const cnh_ast_node& kn = n.nodes[root.operands[1]];
+        CNH_CHECK(kn.is_scalar, -37, "DIAG: the offset must be a scalar operand");
+        k = (int)kn.scalar;
+    }
+    CNH_CHECK(in->ndims == 1 || in->ndims == 2, -37, "DIAG needs a 1-D or 2-D operand, got %d-D", in->ndims);
+    const int r_off = std::max(0, -k), c_off = std::max(0, k);
+    XArray *mat, *vec, *out;
+    int len;
+    if (in->ndims == 1) {
+        len = in->shape[0];
+        const int64_t side = (int64_t)len + std::abs(k);
+        CNH_CHECK(side <= INT32_MAX, -37, "DIAG: result side %lld too large", (long long)side);
+        int32_t shape[3] = {(int32_t)side, (int32_t)side, 1};
+        if (int rc = make_array(ex, root.result_name, 2, in->dtype, shape, true, &out))
+            return rc;
+        mat = out;
+        vec = in;
+    } else {
+        len = k >= 0 ? std::min(in->shape[0], in->shape[1] - k) : std::min(in->shape[0] + k, in->shape[1]);
+        CNH_CHECK(len > 0, -37, "DIAG: k=%d is out of range for shape (%d, %d)", k, in->shape[0], in->shape[1]);
+        int32_t shape[3] = {len, 1, 1};
+        if (int rc = make_array(ex, root.result_name, 1, in->dtype, shape, false, &out))
+            return rc;
+        mat = in;
+        vec = out;
+    }
+    const int esz = dtype_size(in->dtype);
+    int copies = 0;
+    for (int64_t t = 0; t < mat->ntiles; ++t) {
+        int32_t lo[3], ext[3];
+        mat->tile_extent(t, lo, ext);
+        const int i0 = std::max(0, std::max(lo[0] - r_off, lo[1] - c_off));
+        const int i1 = std::min(len, std::min(lo[0] + ext[0] - r_off, lo[1] + ext[1] - c_off));
+        if (i1 <= i0)
+            continue;
+        ++copies;
+        if (ex->dry)
+            continue;
+        const int64_t first = (int64_t)(i0 + r_off - lo[0]) * ext[1] + (i0 + c_off - lo[1]);
+        char* mp = static_cast<char*>(mat->tiles[(size_t)t]) + first * esz;
+        char* vp = static_cast<char*>(vec->tiles[0]) + (int64_t)i0 * esz; // 1-D arrays are contiguous
+        const int64_t mstr[1] = {ext[1] + 1}, vstr[1] = {1}, zero[1] = {0}, one[1] = {1}, cnt[1] = {i1 - i0};
+        const int rc = in->ndims == 1
+                           ? cnh_copy_region(1, esz, mp, mstr, zero, one, vp, vstr, zero, one, cnt, ex->stream)
+                           : cnh_copy_region(1, esz, vp, vstr, zero, one, mp, mstr, zero, one, cnt, ex->stream);
+        if (rc)
+            return rc;
+    }
+    ex->log("diag in=" + std::to_string(in->name) + " out=" + std::to_string(out->name) + " k=" +
+            std::to_string(k) + " copies=" + std::to_string(copies));
+    return 0;
+}
+
 int exec_node(Ex* ex, const DagNode& n) {
     CNH_CHECK(!n.roots.empty(), -33, "DAG node %d has no roots", n.id);
     const cnh_ast_node& root = n.nodes[n.roots.back()];
@@ -1026,6 +1098,7 @@ int exec_node(Ex* ex, const DagNode& n) {
     case CNH_OP_MATMUL: return exec_matmul(ex, n, root);
     case CNH_OP_MATMATMUL: return exec_matmatmul(ex, n, root);
     case CNH_OP_TILE: return exec_tile(ex, n, root);
+    case CNH_OP_DIAG: return exec_diag(ex, n, root);
     case CNH_OP_ADD:
     case CNH_OP_SUB:
     case CNH_OP_MUL:

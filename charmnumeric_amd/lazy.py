@@ -376,9 +376,10 @@ def _emit_instr(ins, node_id):
              [None, vreg], ins.region)
         return w.to_bytes(node_id, isinstance(v, ArrayRef))
     if ins.kind == "nonfusible":
-        opnds = [w.leaf(o) for o in ins.operands]
-        w.op(ins.name, ins.opcode, False, len(ins.shape), ins.dtype, opnds, [o.region for o in ins.operands],
-             _full_region(ins.shape))
+        opnds = [w.leaf(o) if isinstance(o, ArrayRef) else w.scalar(o, len(ins.shape), ins.dtype)
+                 for o in ins.operands]
+        w.op(ins.name, ins.opcode, False, len(ins.shape), ins.dtype, opnds,
+             [o.region if isinstance(o, ArrayRef) else None for o in ins.operands], _full_region(ins.shape))
         return w.to_bytes(node_id, False)
     raise AssertionError(ins.kind)
 

@@ -81,7 +81,20 @@ def tile(x, reps):
 
 
 def diag(v, k=0):
-    raise NotImplementedError("diag is not implemented by this backend")
+    """numpy.diag: a 1-D array becomes the k-th diagonal of a square matrix of zeros, a 2-D array
+    gives its k-th diagonal (charmnumeric/operations.py:125-148 upstream)."""
+    v = asarray(v)
+    k = int(k)
+    if v.ndims == 1:
+        n = v.shape[0] + abs(k)
+        return nonfusible(L.OP_DIAG, [v, k], (n, n), v.dtype)
+    if v.ndims == 2:
+        rows, cols = v.shape
+        length = max(0, min(rows, cols - k)) if k >= 0 else max(0, min(rows + k, cols))
+        if length == 0:
+            raise ValueError(f"k={k} is out of range for shape ({rows}, {cols})")
+        return nonfusible(L.OP_DIAG, [v, k], (length,), v.dtype)
+    raise ValueError(f"diag requires a 1D or 2D array, got {v.ndims}D")
 
 
 # ---- reductions without upstream counterpart: results are size-1 fp64 arrays on the device ----

@@ -217,6 +217,29 @@ def test_matmatmul_panel_products_follow_the_tile_grids(itf):
     assert itf.array_info(Cm.name)["shape"] == (128, 64)
 
 
+def test_diag_copies_once_per_tile_the_diagonal_crosses(itf):
+    itf.set_min_tile(1, 64)
+    itf.set_min_tile(2, 16)
+    v = cnp.ones((100,))
+    D = cnp.diag(v, 1)                  # 101 x 101 in 64-tiles: the super-diagonal meets 3 of 4
+    d = cnp.diag(D, -40)                # rows 40..100, columns 0..60: tiles (0,0) and (1,0)
+    e = cnp.diag(cnp.ones((64, 128)))
+    cnp.execute(itf)
+    log = [ln for ln in itf.trace() if ln.startswith("diag")]
+    assert log[0].endswith("k=1 copies=3") and log[1].endswith("k=-40 copies=2")
+    assert D.shape == (101, 101) and d.shape == (61,) and e.shape == (64,)
+
+
+def test_matvec_of_a_plane_keeps_the_tile_grid_of_the_rank3_array(itf):
+    itf.set_min_tile(3, 8)
+    A3 = cnp.ones((2, 40, 24))
+    y = A3[1, :, :].matvec(cnp.ones((24,)))
+    z = cnp.ones((40, 1, 24)).matvec(cnp.ones((24,)))
+    cnp.execute(itf)
+    assert y.shape == (40,) and z.shape == (40,)
+    assert sum(ln.startswith("matmul") for ln in itf.trace()) == 2
+
+
 def test_malformed_messages_are_refused(itf):
     with pytest.raises(RuntimeError, match="bad magic"):
         itf.send_dag(0, struct.pack("<iii", 1, 1, 0))
@@ -309,7 +332,10 @@ def test_executor_refuses_what_it_cannot_do(itf):
         return _message([w.to_bytes(9, False)])
 
     with pytest.raises(RuntimeError, match="not supported"):
-        itf.send_dag(1, nonfusible(L.OP_DIAG, [ref(2, 1)], (8, 8)))
+        itf.send_dag(1, nonfusible(55, [ref(2, 1)], (8, 8)))
+    itf.send_dag(0, _message([_create(5, (2, 2, 2), L.F64)]))
+    with pytest.raises(RuntimeError, match="1-D or 2-D"):
+        itf.send_dag(1, nonfusible(L.OP_DIAG, [lazy.ArrayRef(5, None, (2, 2, 2), 3, L.F64)], (2,)))
     with pytest.raises(RuntimeError, match="1-D operands"):
         itf.send_dag(1, nonfusible(L.OP_REDUCE, [ref(1, 2), ref(1, 2)], (1,)))
     with pytest.raises(RuntimeError, match="dtypes"):
@@ -344,8 +370,12 @@ def test_executor_refuses_what_it_cannot_do(itf):
 def test_frontend_refuses_like_upstream():
     cnp.reset()
     a = cnp.zeros((4, 5))
-    with pytest.raises(NotImplementedError):
-        cnp.diag(cnp.zeros((4,)))
+    with pytest.raises(ValueError):
+        cnp.diag(a, 5)                                # diagonal out of range
+    with pytest.raises(ValueError):
+        cnp.diag(cnp.zeros((2, 2, 2)))
+    with pytest.raises(ValueError):
+        cnp.zeros((2, 3, 4)).matvec(cnp.zeros((4,)))  # no extent of 1 to drop
     with pytest.raises(NotImplementedError):
         a[::-1]
     with pytest.raises(NotImplementedError):

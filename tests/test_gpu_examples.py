@@ -1,0 +1,266 @@
+"""The programs of upstream's self-checking example scripts that the other frontend tests do not
+already hold, written against this frontend and compared with NumPy running the same statements:
+red-black Gauss-Seidel by strided slices (examples/gauss_seidel.py), matvec and matmatmul on sliced
+and dimension-dropped operands (examples/matvec_slice.py, examples/matmatmul.py), the pieces and a
+whole V-cycle of the 2-D multigrid solver (examples/multigrid2d.py) and weighted Jacobi with a
+residual (examples/jacobi_iteration.py). Element-wise statements must match NumPy bit for bit;
+products are held to 1e-12 of the sum of absolute products."""
+import numpy as np
+import pytest
+
+import charmnumeric_amd as cnp
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture
+def itf():
+    cnp.reset()
+    it = cnp.CharmNumericInterface(device=0)
+    it.connect(odf=4)
+    it.set_min_tile(1, 64)
+    it.set_min_tile(2, 16)
+    it.set_min_tile(3, 8)
+    yield it
+    cnp.reset()
+    it.close()
+
+
+# ---- red-black Gauss-Seidel ----
+
+def _red_black_sweep(phi, f, h2):
+    for r0, c0 in ((1, 1), (2, 2), (1, 2), (2, 1)):          # red, red, black, black
+        rows, cols = slice(r0, -1, 2), slice(c0, -1, 2)
+        up, down = slice(r0 - 1, -2, 2), slice(r0 + 1, None, 2)
+        left, right = slice(c0 - 1, -2, 2), slice(c0 + 1, None, 2)
+        phi[rows, cols] = 0.25 * (phi[up, cols] + phi[down, cols] + phi[rows, left] + phi[rows, right]
+                                  - h2 * f[rows, cols])
+
+
+@pytest.mark.parametrize("n", [33, 64])
+def test_red_black_gauss_seidel(itf, n):
+    h2 = (1.0 / (n - 1)) ** 2
+    rng = np.random.default_rng(n)
+    f_host = rng.standard_normal((n, n))
+    phi_host = np.zeros((n, n))
+    phi, f = cnp.zeros((n, n)), cnp.array(f_host)
+    for _ in range(5):
+        _red_black_sweep(phi, f, h2)
+        _red_black_sweep(phi_host, f_host, h2)
+    got = phi.get(itf)
+    assert np.array_equal(got, phi_host)
+    assert np.abs(got).max() > 0
+
+
+# ---- products on slices ----
+
+def _close_product(got, a, b):
+    want = a @ b
+    assert got.shape == want.shape
+    assert np.all(np.abs(got - want) <= 1e-12 * (np.abs(a) @ np.abs(b)))
+
+
+@pytest.mark.parametrize("rows,cols", [
+    (slice(None), slice(None)), (slice(0, 32), slice(None)), (slice(None), slice(16, 48)),
+    (slice(8, 40), slice(10, 50)), (slice(3, 37), slice(5, 47))])
+def test_matvec_on_slices(itf, rows, cols):
+    rng = np.random.default_rng(5)
+    a_host, x_host = rng.standard_normal((128, 128)), np.arange(1.0, 129.0)
+    A, x = cnp.array(a_host), cnp.arange(1, 129, dtype=np.float64)
+    y = A[rows, cols].matvec(x[cols])
+    cnp.execute(itf)
+    _close_product(y.get(itf).reshape(-1), a_host[rows, cols], x_host[cols])
+
+
+def test_matvec_on_a_plane_of_a_rank3_array(itf):
+    rng = np.random.default_rng(6)
+    a_host, x_host = rng.standard_normal((2, 96, 128)), rng.standard_normal(128)
+    A3, x = cnp.array(a_host), cnp.array(x_host)
+    for plane in (0, 1):
+        y = A3[plane, :, :].matvec(x)
+        _close_product(y.get(itf).reshape(-1), a_host[plane], x_host)
+
+
+@pytest.mark.parametrize("ra,ca,cb", [
+    (slice(None), slice(None), slice(None)), (slice(0, 32), slice(None), slice(None)),
+    (slice(None), slice(None), slice(16, 48)), (slice(8, 40), slice(10, 50), slice(5, 45)),
+    (slice(3, 37), slice(5, 47), slice(7, 39))])
+def test_matmatmul_on_slices(itf, ra, ca, cb):
+    rng = np.random.default_rng(7)
+    a_host, b_host = rng.standard_normal((128, 128)), rng.standard_normal((128, 128))
+    A, B = cnp.array(a_host), cnp.array(b_host)
+    C = A[ra, ca] @ B[ca, cb]
+    cnp.execute(itf)
+    _close_product(C.get(itf), a_host[ra, ca], b_host[ca, cb])
+
+
+def test_matmatmul_shapes_chain_and_dropped_dimension(itf):
+    rng = np.random.default_rng(8)
+    a_host, b_host = rng.standard_normal((128, 64)), rng.standard_normal((64, 256))
+    _close_product((cnp.array(a_host) @ cnp.array(b_host)).get(itf), a_host, b_host)
+    # (A @ B) @ x
+    sq_a, sq_b, x_host = rng.standard_normal((96, 96)), rng.standard_normal((96, 96)), rng.standard_normal(96)
+    y = (cnp.array(sq_a) @ cnp.array(sq_b)).matvec(cnp.array(x_host))
+    want = (sq_a @ sq_b) @ x_host
+    got = y.get(itf).reshape(-1)
+    assert np.all(np.abs(got - want) <= 1e-11 * (np.abs(sq_a) @ np.abs(sq_b) @ np.abs(x_host)))
+    # A3[0] @ B
+    a3_host = rng.standard_normal((2, 96, 64))
+    C = cnp.array(a3_host)[0, :, :] @ cnp.array(b_host)
+    _close_product(C.get(itf), a3_host[0], b_host)
+
+
+# ---- diag ----
+
+@pytest.mark.parametrize("k", [0, 1, -1, 37, -70])
+@pytest.mark.parametrize("dtype", [np.float64, np.int32])
+def test_diag_builds_and_extracts(itf, k, dtype):
+    """numpy.diag both ways (examples/diag.py upstream), on tiles the diagonal enters off-corner."""
+    v_host = (np.arange(100) * 3 - 50).astype(dtype)
+    m_host = np.arange(96 * 150).reshape(96, 150).astype(dtype)
+    D = cnp.diag(cnp.array(v_host), k=k)
+    got = D.get(itf)
+    assert got.dtype == dtype and np.array_equal(got, np.diag(v_host, k=k))
+    assert np.array_equal(cnp.diag(D, k).get(itf), v_host)
+    assert np.array_equal(cnp.diag(cnp.array(m_host), k).get(itf), np.diag(m_host, k))
+    assert np.array_equal(cnp.diag(cnp.array(m_host.T.copy()), k).get(itf), np.diag(m_host.T, k))
+    assert np.array_equal(cnp.diag(cnp.array(m_host)[3:80, 5:121], k).get(itf), np.diag(m_host[3:80, 5:121], k))
+
+
+# ---- multigrid pieces ----
+
+def _pattern(n):
+    """Fills that cross tile boundaries and both parities: whole, interior, the four parity classes,
+    a block, two strided boxes, a small centre box."""
+    q, tq, e, te, se, mid = n // 4, 3 * n // 4 + 1, n // 8, 3 * n // 8, 7 * n // 8 + 1, n // 2
+    s = slice
+    return [((s(None), s(None)), 0.0), ((s(1, n - 1), s(1, n - 1)), 1.0),
+            ((s(1, n - 1, 2), s(1, n - 1, 2)), 2.0), ((s(2, n - 2, 2), s(1, n - 1, 2)), -1.0),
+            ((s(1, n - 1, 2), s(2, n - 2, 2)), 0.5), ((s(2, n - 2, 2), s(2, n - 2, 2)), -0.25),
+            ((s(q, tq), s(q, tq)), 3.0), ((s(te, se, 2), s(e, 5 * n // 8 + 1, 2)), -2.0),
+            ((s(e, se, 4), s(5 * n // 16, 15 * n // 16, 2)), 0.75),
+            ((s(mid - 2, mid + 3), s(mid - 2, mid + 3)), -4.0)]
+
+
+def _fill_pattern(arr):
+    for key, value in _pattern(arr.shape[0]):
+        arr[key] = float(value)
+
+
+def _smooth(u, f, h2, sweeps, omega=2.0 / 3.0):
+    for _ in range(sweeps):
+        upd = 0.25 * (u[:-2, 1:-1] + u[2:, 1:-1] + u[1:-1, :-2] + u[1:-1, 2:] + h2 * f[1:-1, 1:-1])
+        u[1:-1, 1:-1] = (1.0 - omega) * u[1:-1, 1:-1] + omega * upd
+
+
+def _residual(xp, u, f, h2):
+    r = xp.zeros(u.shape, dtype=np.float64)
+    r[1:-1, 1:-1] = f[1:-1, 1:-1] - (1.0 / h2) * (4.0 * u[1:-1, 1:-1] - u[:-2, 1:-1] - u[2:, 1:-1]
+                                                   - u[1:-1, :-2] - u[1:-1, 2:])
+    return r
+
+
+def _restrict(fine, coarse):
+    c, lo, hi = slice(2, -2, 2), slice(1, -3, 2), slice(3, -1, 2)
+    coarse[:, :] = 0.0
+    coarse[1:-1, 1:-1] = (0.25 * fine[c, c]
+                          + 0.125 * (fine[lo, c] + fine[hi, c] + fine[c, lo] + fine[c, hi])
+                          + 0.0625 * (fine[lo, lo] + fine[lo, hi] + fine[hi, lo] + fine[hi, hi]))
+
+
+def _prolong_and_correct(xp, e_coarse, u_fine):
+    n = u_fine.shape[0]
+    e = xp.zeros((n, n), dtype=np.float64)
+    e[2:-2:2, 2:-2:2] = e_coarse[1:-1, 1:-1]
+    e[1:-1:2, 2:-2:2] = 0.5 * (e_coarse[:-1, 1:-1] + e_coarse[1:, 1:-1])
+    e[2:-2:2, 1:-1:2] = 0.5 * (e_coarse[1:-1, :-1] + e_coarse[1:-1, 1:])
+    e[1:-1:2, 1:-1:2] = 0.25 * (e_coarse[:-1, :-1] + e_coarse[1:, :-1] + e_coarse[:-1, 1:] + e_coarse[1:, 1:])
+    u_fine[1:-1, 1:-1] = u_fine[1:-1, 1:-1] + e[1:-1, 1:-1]
+
+
+def _vcycle(xp, u, f, h, pre, post, coarse_sweeps):
+    n, h2 = u.shape[0], h * h
+    if n <= 5:
+        _smooth(u, f, h2, coarse_sweeps)
+        return
+    _smooth(u, f, h2, pre)
+    r = _residual(xp, u, f, h2)
+    nc = (n - 1) // 2 + 1
+    rc = xp.zeros((nc, nc), dtype=np.float64)
+    _restrict(r, rc)
+    ec = xp.zeros((nc, nc), dtype=np.float64)
+    _vcycle(xp, ec, rc, 2.0 * h, pre, post, coarse_sweeps)
+    _prolong_and_correct(xp, ec, u)
+    _smooth(u, f, h2, post)
+
+
+@pytest.mark.parametrize("n", [33, 65])
+def test_strided_fill_pattern(itf, n):
+    host = np.zeros((n, n))
+    dev = cnp.zeros((n, n))
+    _fill_pattern(host)
+    _fill_pattern(dev)
+    assert np.array_equal(dev.get(itf), host)
+
+
+@pytest.mark.parametrize("n", [33, 65])
+def test_full_weighting_restriction(itf, n):
+    nc = (n - 1) // 2 + 1
+    fine_host, coarse_host = np.zeros((n, n)), np.full((nc, nc), 9.0)
+    fine, coarse = cnp.zeros((n, n)), cnp.full((nc, nc), 9.0)
+    _fill_pattern(fine_host)
+    _fill_pattern(fine)
+    _restrict(fine_host, coarse_host)
+    _restrict(fine, coarse)
+    assert np.array_equal(coarse.get(itf), coarse_host)
+
+
+@pytest.mark.parametrize("n", [33, 65])
+def test_bilinear_prolongation(itf, n):
+    nc = (n - 1) // 2 + 1
+    ec_host, u_host = np.zeros((nc, nc)), np.zeros((n, n))
+    ec, u = cnp.zeros((nc, nc)), cnp.zeros((n, n))
+    _fill_pattern(ec_host)
+    _fill_pattern(ec)
+    _prolong_and_correct(np, ec_host, u_host)
+    _prolong_and_correct(cnp, ec, u)
+    assert np.array_equal(u.get(itf), u_host)
+
+
+def test_weighted_jacobi_and_residual(itf):
+    n = 65
+    h2 = (1.0 / (n - 1)) ** 2
+    u_host, f_host = np.zeros((n, n)), np.zeros((n, n))
+    u, f = cnp.zeros((n, n)), cnp.zeros((n, n))
+    for arr in (u_host, f_host, u, f):
+        _fill_pattern(arr)
+    _smooth(u_host, f_host, h2, 3)
+    _smooth(u, f, h2, 3)
+    assert np.array_equal(u.get(itf), u_host)
+    assert np.array_equal(_residual(cnp, u, f, h2).get(itf), _residual(np, u_host, f_host, h2))
+
+
+@pytest.mark.parametrize("auto_flush", [0, 24])
+def test_multigrid_v_cycles(itf, auto_flush):
+    """Two V-cycles from 65x65 down to 5x5 for -lap(u) = 2 pi^2 sin(pi x) sin(pi y): every level's
+    arrays, strided transfers between levels and temporaries, bit for bit against NumPy; and the
+    error against the continuous solution drops."""
+    n, h = 65, 1.0 / 64
+    xs = np.linspace(0.0, 1.0, n)
+    exact = np.outer(np.sin(np.pi * xs), np.sin(np.pi * xs))
+    f_host = 2.0 * np.pi ** 2 * exact
+    u_host = np.zeros((n, n))
+    if auto_flush:
+        cnp.set_auto_flush(itf, auto_flush)
+    try:
+        u, f = cnp.zeros((n, n)), cnp.array(f_host)
+        errs = []
+        for _ in range(2):
+            _vcycle(np, u_host, f_host, h, 2, 2, 40)
+            _vcycle(cnp, u, f, h, 2, 2, 40)
+            got = u.get(itf)
+            assert np.array_equal(got, u_host)
+            errs.append(np.abs(got - exact).max())
+    finally:
+        cnp.reset()
+    assert errs[1] < 0.2 * errs[0] < 0.1
