@@ -13,7 +13,7 @@ namespace {
 typedef double v4d __attribute__((ext_vector_type(4)));
 typedef double v2d __attribute__((ext_vector_type(2)));
 
-constexpr int BK = 16, PAD = 16;
+constexpr int PAD = 16;
 
 // Workgroup ids are dealt round-robin to the 8 XCDs; give every XCD a contiguous run of logical
 // tiles so that the workgroups sharing a B column panel also share one L2.
@@ -23,20 +23,27 @@ __device__ __forceinline__ int xcd_remap(int b, int nblocks) {
     return (b % 8) * (nblocks / 8) + b / 8;
 }
 
-// WM x WN wavefronts per workgroup, each owning TM x TN tiles of 16x16. The fp64 matrix pipe
-// needs two or more wavefronts per SIMD to stay busy (one wavefront issues at ~70% of the rate
-// eight reach), hence the 8-wavefront shape for grids that give each CU a single workgroup.
-template <int WM, int WN, int TM, int TN, bool FULL>
+// WM x WN wavefronts per workgroup, each owning TM x TN tiles of 16x16; K advances BKT at a time.
+// The fp64 matrix pipe needs two or more wavefronts per SIMD to stay busy (one wavefront issues at
+// ~70% of the rate eight reach), hence the 8-wavefront shape for grids that give each CU a single
+// workgroup. Global loads run two K steps ahead of the arithmetic (two register sets, one LDS
+// buffer being filled while the other is read): one K step of matrix instructions is shorter than
+// a trip to memory.
+template <int WM, int WN, int TM, int TN, int BKT, bool FULL>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_f64_mfma(int M, int N, int K,
                                                               const double* __restrict__ A, int64_t lda,
                                                               const double* __restrict__ B, int64_t ldb,
                                                               double* __restrict__ C, int64_t ldc) {
     constexpr int NT = WM * WN * 64;
     constexpr int BM = WM * TM * 16, BN = WN * TN * 16;
-    constexpr int APT = BM * BK / NT, BPT = BN * BK / NT;   // doubles staged per lane
+    constexpr int APT = BM * BKT / NT, BPT = BN * BKT / NT;   // doubles staged per lane
     static_assert(APT >= 2 && BPT >= 2 && APT % 2 == 0 && BPT % 2 == 0, "staging uses 128-bit loads");
-    __shared__ double As[2][BK][BM + PAD];
-    __shared__ double Bs[2][BK][BN + PAD];
+    static_assert(BKT % APT == 0 && BN % BPT == 0, "a lane's run stays inside one row");
+    // A stays row-major in LDS with rows of BKT + 1 doubles: the operand read of 16 consecutive
+    // rows at one k then touches 16 different bank pairs. B is k-major with rows of BN + 16.
+    constexpr int AP = BKT + 1;
+    __shared__ double As[2][BM][AP];
+    __shared__ __attribute__((aligned(16))) double Bs[2][BKT][BN + PAD];
     const int nbm = (M + BM - 1) / BM, nbn = (N + BN - 1) / BN;
     const int logical = xcd_remap(blockIdx.x, nbm * nbn);
     const int bn = logical / nbm, bm = logical - bn * nbm;
@@ -44,12 +51,11 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_f64_mfma(int M, int N, int 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
 
-    // staging assignment: A tile BM rows x 16 k (APT along k), B tile 16 k x BN (BPT along n)
-    const int a_row = tid / (BK / APT), a_k = (tid % (BK / APT)) * APT;
+    // staging assignment: A tile BM rows x BKT k (APT along k), B tile BKT k x BN (BPT along n)
+    const int a_row = tid / (BKT / APT), a_k = (tid % (BKT / APT)) * APT;
     const int b_k = tid / (BN / BPT), b_n = (tid % (BN / BPT)) * BPT;
 
-    double ra[APT], rb[BPT];
-    auto fetch = [&](int k0) {
+    auto fetch = [&](int k0, double (&ra)[APT], double (&rb)[BPT]) {
         const int gr = m0 + a_row;
         const int gk = k0 + a_k;
         if (FULL) {
@@ -79,13 +85,13 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_f64_mfma(int M, int N, int 
                 rb[j] = (bk < K && gn + j < N) ? B[(int64_t)bk * ldb + gn + j] : 0.0;
         }
     };
-    auto stage = [&](int buf) {
+    auto stage = [&](int buf, const double (&ra)[APT], const double (&rb)[BPT]) {
 #pragma unroll
         for (int j = 0; j < APT; ++j)
-            As[buf][a_k + j][a_row] = ra[j];
+            As[buf][a_row][a_k + j] = ra[j];
 #pragma unroll
-        for (int j = 0; j < BPT; ++j)
-            Bs[buf][b_k][b_n + j] = rb[j];
+        for (int j = 0; j < BPT; j += 2)
+            *reinterpret_cast<v2d*>(&Bs[buf][b_k][b_n + j]) = (v2d){rb[j], rb[j + 1]};
     };
 
     v4d acc[TM][TN];
@@ -95,22 +101,15 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_f64_mfma(int M, int N, int 
         for (int j = 0; j < TN; ++j)
             acc[i][j] = (v4d){0.0, 0.0, 0.0, 0.0};
 
-    const int nk = (K + BK - 1) / BK;
-    fetch(0);
-    stage(0);
-    __syncthreads();
     const int lr = lane & 15, lk = lane >> 4;
-    for (int t = 0; t < nk; ++t) {
-        const int buf = t & 1;
-        if (t + 1 < nk)
-            fetch((t + 1) * BK);
+    auto multiply = [&](int buf) {
 #pragma unroll
-        for (int ks = 0; ks < BK / 4; ++ks) {
+        for (int ks = 0; ks < BKT / 4; ++ks) {
             const int kk = ks * 4 + lk;
             double a[TM], b[TN];
 #pragma unroll
             for (int i = 0; i < TM; ++i)
-                a[i] = As[buf][kk][(wm * TM + i) * 16 + lr];
+                a[i] = As[buf][(wm * TM + i) * 16 + lr][kk];
 #pragma unroll
             for (int j = 0; j < TN; ++j)
                 b[j] = Bs[buf][kk][(wn * TN + j) * 16 + lr];
@@ -120,9 +119,42 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_f64_mfma(int M, int N, int 
                 for (int j = 0; j < TN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[i], b[j], acc[i][j], 0, 0, 0);
         }
-        if (t + 1 < nk) {
-            stage(buf ^ 1);
+    };
+
+    // Step t multiplies LDS buffer t&1, which holds K slice t. Register set t&1 receives slice
+    // t+2 while that runs; the other set (slice t+1, requested a step earlier) goes to LDS after it.
+    const int nk = (K + BKT - 1) / BKT;
+    double ra0[APT], rb0[BPT], ra1[APT], rb1[BPT];
+    fetch(0, ra0, rb0);
+    if (nk > 1)
+        fetch(BKT, ra1, rb1);
+    stage(0, ra0, rb0);
+    __syncthreads();
+    // At the top of every round LDS buffer 0 holds slice t and register set 1 slice t + 1.
+    // The steady-state rounds carry no conditions, so that the compiler's wait counts leave the
+    // younger pair of loads in flight while the older pair is stored.
+    int t = 0;
+    for (; t + 3 < nk; t += 2) {
+        fetch((t + 2) * BKT, ra0, rb0);
+        multiply(0);
+        stage(1, ra1, rb1);
+        __syncthreads();
+        fetch((t + 3) * BKT, ra1, rb1);
+        multiply(1);
+        stage(0, ra0, rb0);
+        __syncthreads();
+    }
+    if (t + 2 < nk)
+        fetch((t + 2) * BKT, ra0, rb0);
+    multiply(0);
+    if (t + 1 < nk) {
+        stage(1, ra1, rb1);
+        __syncthreads();
+        multiply(1);
+        if (t + 2 < nk) {
+            stage(0, ra0, rb0);
             __syncthreads();
+            multiply(0);
         }
     }
     // D layout of the 16x16x4 f64 instruction (measured on gfx950): register r of a lane holds
@@ -193,6 +225,34 @@ int run_generic(int M, int N, int K, const void* A, int64_t lda, const void* B, 
 
 } // namespace
 
+namespace {
+struct GemmArgs {
+    int M, N, K;
+    const double* A;
+    int64_t lda;
+    const double* B;
+    int64_t ldb;
+    double* C;
+    int64_t ldc;
+};
+
+template <int WM, int WN, int TM, int TN, int BKT>
+int launch_mfma(const GemmArgs& g, bool aligned, hipStream_t st) {
+    constexpr int BM = WM * TM * 16, BN = WN * TN * 16;
+    const int64_t blocks = (((int64_t)g.M + BM - 1) / BM) * (((int64_t)g.N + BN - 1) / BN);
+    CNH_CHECK(blocks < (1ll << 31), -3, "cnh_gemm_acc: too many tiles");
+    const bool full = aligned && g.M % BM == 0 && g.N % BN == 0 && g.K % BKT == 0;
+    if (full)
+        hipLaunchKernelGGL((gemm_f64_mfma<WM, WN, TM, TN, BKT, true>), dim3((unsigned)blocks),
+                           dim3(WM * WN * 64), 0, st, g.M, g.N, g.K, g.A, g.lda, g.B, g.ldb, g.C, g.ldc);
+    else
+        hipLaunchKernelGGL((gemm_f64_mfma<WM, WN, TM, TN, BKT, false>), dim3((unsigned)blocks),
+                           dim3(WM * WN * 64), 0, st, g.M, g.N, g.K, g.A, g.lda, g.B, g.ldb, g.C, g.ldc);
+    CNH_HIP(hipGetLastError());
+    return 0;
+}
+} // namespace
+
 extern "C" int cnh_gemm_acc(int dtype, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda,
                             const void* B, int64_t ldb, void* C, int64_t ldc, cnh_stream s) {
     if (int rc = ensure_init())
@@ -207,36 +267,16 @@ extern "C" int cnh_gemm_acc(int dtype, int64_t M, int64_t N, int64_t K, const vo
     hipStream_t st = as_stream(s);
     switch (dtype) {
     case CNH_F64: {
-        constexpr int BM = 64, BN = 64;
-        const int64_t blocks = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-        CNH_CHECK(blocks < (1ll << 31), -3, "cnh_gemm_acc: too many tiles");
-        const bool full = (M % BM == 0) && (N % BN == 0) && (K % BK == 0) && (lda % 2 == 0) &&
-                          (ldb % 2 == 0) && (((uintptr_t)A & 15) == 0) && (((uintptr_t)B & 15) == 0);
-        // 64x64 tiles either way; 8 wavefronts per workgroup unless the grid already gives
-        // every CU several workgroups.
-        const bool many = blocks >= 1024;
-        const dim3 grid((unsigned)blocks);
-        if (many) {
-            if (full)
-                hipLaunchKernelGGL((gemm_f64_mfma<2, 2, 2, 2, true>), grid, dim3(256), 0, st, (int)M,
-                                   (int)N, (int)K, (const double*)A, lda, (const double*)B, ldb,
-                                   (double*)C, ldc);
-            else
-                hipLaunchKernelGGL((gemm_f64_mfma<2, 2, 2, 2, false>), grid, dim3(256), 0, st, (int)M,
-                                   (int)N, (int)K, (const double*)A, lda, (const double*)B, ldb,
-                                   (double*)C, ldc);
-        } else {
-            if (full)
-                hipLaunchKernelGGL((gemm_f64_mfma<2, 4, 2, 1, true>), grid, dim3(512), 0, st, (int)M,
-                                   (int)N, (int)K, (const double*)A, lda, (const double*)B, ldb,
-                                   (double*)C, ldc);
-            else
-                hipLaunchKernelGGL((gemm_f64_mfma<2, 4, 2, 1, false>), grid, dim3(512), 0, st, (int)M,
-                                   (int)N, (int)K, (const double*)A, lda, (const double*)B, ldb,
-                                   (double*)C, ldc);
-        }
-        CNH_HIP(hipGetLastError());
-        return 0;
+        const bool aligned = (lda % 2 == 0) && (ldb % 2 == 0) && (((uintptr_t)A & 15) == 0) &&
+                             (((uintptr_t)B & 15) == 0);
+        const GemmArgs ga{(int)M, (int)N, (int)K, (const double*)A, lda, (const double*)B, ldb, (double*)C, ldc};
+        // 64x64 tiles of four wavefronts when that gives every CU several workgroups; smaller
+        // grids take 8 wavefronts per workgroup so that a CU with one workgroup still has two
+        // wavefronts per SIMD.
+        const int64_t blocks64 = ((M + 63) / 64) * ((N + 63) / 64);
+        if (blocks64 >= 1024)
+            return launch_mfma<2, 2, 2, 2, 16>(ga, aligned, st);
+        return launch_mfma<2, 4, 2, 1, 16>(ga, aligned, st);
     }
     case CNH_F32: return run_generic<float>((int)M, (int)N, (int)K, A, lda, B, ldb, C, ldc, st);
     case CNH_I32: return run_generic<int32_t>((int)M, (int)N, (int)K, A, lda, B, ldb, C, ldc, st);
