@@ -77,6 +77,12 @@ class Ast(C.Structure):
     ]
 
 
+class GemmJob(C.Structure):
+    """cnh_gemm_job: one C += A * B panel product of a batch."""
+    _fields_ = [("M", C.c_int64), ("N", C.c_int64), ("K", C.c_int64), ("A", C.c_void_p), ("lda", C.c_int64),
+                ("B", C.c_void_p), ("ldb", C.c_int64), ("C", C.c_void_p), ("ldc", C.c_int64)]
+
+
 class Memref(C.Structure):
     _fields_ = [
         ("allocated", C.c_void_p),
@@ -206,6 +212,7 @@ _PROTOS = {
                                  C.c_void_p, C.c_void_p]),
     "cnh_gemm_acc": (C.c_int, [C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_int64,
                                C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p]),
+    "cnh_gemm_acc_batch": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmJob), C.c_void_p]),
     "cnh_fill_uniform": (C.c_int, [C.c_void_p, C.c_int64, C.c_uint64, C.c_uint64, C.c_uint64,
                                    C.c_double, C.c_double, C.c_void_p]),
     "cnh_fill_uniform_tile": (C.c_int, [C.c_void_p, C.c_int, _i64p, _i64p, _i64p, C.c_uint64,

@@ -880,6 +880,7 @@ int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
     const int esz = dtype_size(Aa->dtype);
     const int TA = Aa->tile, TB = Ba->tile;
     int calls = 0;
+    std::vector<cnh_gemm_job> jobs;   // all panel products of the node go out as one launch
     for (int ci = 0; ci < Cc->grid[0]; ++ci)
         for (int cj = 0; cj < Cc->grid[1]; ++cj) {
             int32_t clo[3], cext[3];
@@ -907,14 +908,14 @@ int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
                         char* cp = static_cast<char*>(Cc->tiles[(size_t)ci * Cc->grid[1] + cj]) +
                                    ((int64_t)(r0 - clo[0]) * cext[1] + (c0 - clo[1])) * esz;
                         ++calls;
-                        if (!ex->dry)
-                            if (int rc = cnh_gemm_acc(Aa->dtype, r1 - r0, c1 - c0, k1 - k0, ap, aec, bp, bec,
-                                                      cp, cext[1], ex->stream))
-                                return rc;
+                        jobs.push_back(cnh_gemm_job{r1 - r0, c1 - c0, k1 - k0, ap, aec, bp, bec, cp, cext[1]});
                         k0 = k1;
                     }
                 }
         }
+    if (!ex->dry)
+        if (int rc = cnh_gemm_acc_batch(Aa->dtype, (int)jobs.size(), jobs.data(), ex->stream))
+            return rc;
     ex->log("matmatmul A=" + std::to_string(Aa->name) + " B=" + std::to_string(Ba->name) + " out=" +
             std::to_string(Cc->name) + " panel_products=" + std::to_string(calls));
     return 0;

@@ -6,6 +6,9 @@
 // staged through double-buffered LDS. Other element types use a plain LDS-tiled kernel.
 #include "common.h"
 
+#include <cstring>
+#include <vector>
+
 using namespace cnh;
 
 namespace {
@@ -23,17 +26,37 @@ __device__ __forceinline__ int xcd_remap(int b, int nblocks) {
     return (b % 8) * (nblocks / 8) + b / 8;
 }
 
+// One C block and the panel products that accumulate into it, in order; a launch covers a list
+// of such chains (a single product is a chain of one segment).
+struct GemmSeg {
+    const double* A;
+    int64_t lda;
+    const double* B;
+    int64_t ldb;
+    int32_t K, pad;
+};
+struct GemmChain {
+    double* C;
+    int64_t ldc;
+    int32_t M, N;
+    int32_t seg0, nseg; // segments [seg0, seg0 + nseg)
+    int32_t blk0, nbm;  // first workgroup of the chain, tiles along M
+};
+static_assert(sizeof(GemmSeg) == 40 && sizeof(GemmChain) == 40, "descriptor tables are uploaded as bytes");
+
 // WM x WN wavefronts per workgroup, each owning TM x TN tiles of 16x16; K advances BKT at a time.
 // The fp64 matrix pipe needs two or more wavefronts per SIMD to stay busy (one wavefront issues at
 // ~70% of the rate eight reach), hence the 8-wavefront shape for grids that give each CU a single
 // workgroup. Global loads run two K steps ahead of the arithmetic (two register sets, one LDS
 // buffer being filled while the other is read): one K step of matrix instructions is shorter than
-// a trip to memory.
+// a trip to memory. A workgroup keeps its accumulators across the segments of its chain, so the
+// panel products of one C block cost one pass over C however many K pieces they come in.
 template <int WM, int WN, int TM, int TN, int BKT, bool FULL>
-__global__ __launch_bounds__(WM * WN * 64) void gemm_f64_mfma(int M, int N, int K,
-                                                              const double* __restrict__ A, int64_t lda,
-                                                              const double* __restrict__ B, int64_t ldb,
-                                                              double* __restrict__ C, int64_t ldc) {
+__global__ __launch_bounds__(WM * WN * 64) void gemm_f64_mfma(const GemmChain* __restrict__ chains,
+                                                              int nchains,
+                                                              const GemmSeg* __restrict__ segs,
+                                                              int nblocks, GemmChain only_chain,
+                                                              GemmSeg only_seg) {
     constexpr int NT = WM * WN * 64;
     constexpr int BM = WM * TM * 16, BN = WN * TN * 16;
     constexpr int APT = BM * BKT / NT, BPT = BN * BKT / NT;   // doubles staged per lane
@@ -44,9 +67,16 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_f64_mfma(int M, int N, int 
     constexpr int AP = BKT + 1;
     __shared__ double As[2][BM][AP];
     __shared__ __attribute__((aligned(16))) double Bs[2][BKT][BN + PAD];
-    const int nbm = (M + BM - 1) / BM, nbn = (N + BN - 1) / BN;
-    const int logical = xcd_remap(blockIdx.x, nbm * nbn);
-    const int bn = logical / nbm, bm = logical - bn * nbm;
+    const int logical = xcd_remap(blockIdx.x, nblocks);
+    // a lone product travels in the kernel arguments (chains == nullptr), lists in a table
+    int ci = 0;
+    if (chains != nullptr)
+        while (ci + 1 < nchains && chains[ci + 1].blk0 <= logical)
+            ++ci;
+    const GemmChain ch = chains != nullptr ? chains[ci] : only_chain;
+    const int M = ch.M, N = ch.N;
+    const int local = logical - ch.blk0;
+    const int bn = local / ch.nbm, bm = local - bn * ch.nbm;
     const int m0 = bm * BM, n0 = bn * BN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
@@ -54,45 +84,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_f64_mfma(int M, int N, int 
     // staging assignment: A tile BM rows x BKT k (APT along k), B tile BKT k x BN (BPT along n)
     const int a_row = tid / (BKT / APT), a_k = (tid % (BKT / APT)) * APT;
     const int b_k = tid / (BN / BPT), b_n = (tid % (BN / BPT)) * BPT;
-
-    auto fetch = [&](int k0, double (&ra)[APT], double (&rb)[BPT]) {
-        const int gr = m0 + a_row;
-        const int gk = k0 + a_k;
-        if (FULL) {
-#pragma unroll
-            for (int j = 0; j < APT; j += 2) {
-                const v2d v = *reinterpret_cast<const v2d*>(A + (int64_t)gr * lda + gk + j);
-                ra[j] = v[0];
-                ra[j + 1] = v[1];
-            }
-        } else {
-#pragma unroll
-            for (int j = 0; j < APT; ++j)
-                ra[j] = (gr < M && gk + j < K) ? A[(int64_t)gr * lda + gk + j] : 0.0;
-        }
-        const int bk = k0 + b_k;
-        const int gn = n0 + b_n;
-        if (FULL) {
-#pragma unroll
-            for (int j = 0; j < BPT; j += 2) {
-                const v2d v = *reinterpret_cast<const v2d*>(B + (int64_t)bk * ldb + gn + j);
-                rb[j] = v[0];
-                rb[j + 1] = v[1];
-            }
-        } else {
-#pragma unroll
-            for (int j = 0; j < BPT; ++j)
-                rb[j] = (bk < K && gn + j < N) ? B[(int64_t)bk * ldb + gn + j] : 0.0;
-        }
-    };
-    auto stage = [&](int buf, const double (&ra)[APT], const double (&rb)[BPT]) {
-#pragma unroll
-        for (int j = 0; j < APT; ++j)
-            As[buf][a_row][a_k + j] = ra[j];
-#pragma unroll
-        for (int j = 0; j < BPT; j += 2)
-            *reinterpret_cast<v2d*>(&Bs[buf][b_k][b_n + j]) = (v2d){rb[j], rb[j + 1]};
-    };
+    const int lr = lane & 15, lk = lane >> 4;
 
     v4d acc[TM][TN];
 #pragma unroll
@@ -101,60 +93,108 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_f64_mfma(int M, int N, int 
         for (int j = 0; j < TN; ++j)
             acc[i][j] = (v4d){0.0, 0.0, 0.0, 0.0};
 
-    const int lr = lane & 15, lk = lane >> 4;
-    auto multiply = [&](int buf) {
+    for (int si = 0; si < ch.nseg; ++si) {
+        const GemmSeg sg = chains != nullptr ? segs[ch.seg0 + si] : only_seg;
+        const double* __restrict__ A = sg.A;
+        const double* __restrict__ B = sg.B;
+        const int64_t lda = sg.lda, ldb = sg.ldb;
+        const int K = sg.K;
+        if (si > 0)
+            __syncthreads();   // the previous segment's last reads of LDS are done
+
+        auto fetch = [&](int k0, double (&ra)[APT], double (&rb)[BPT]) {
+            const int gr = m0 + a_row;
+            const int gk = k0 + a_k;
+            if (FULL) {
 #pragma unroll
-        for (int ks = 0; ks < BKT / 4; ++ks) {
-            const int kk = ks * 4 + lk;
-            double a[TM], b[TN];
+                for (int j = 0; j < APT; j += 2) {
+                    const v2d v = *reinterpret_cast<const v2d*>(A + (int64_t)gr * lda + gk + j);
+                    ra[j] = v[0];
+                    ra[j + 1] = v[1];
+                }
+            } else {
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
-                a[i] = As[buf][(wm * TM + i) * 16 + lr][kk];
+                for (int j = 0; j < APT; ++j)
+                    ra[j] = (gr < M && gk + j < K) ? A[(int64_t)gr * lda + gk + j] : 0.0;
+            }
+            const int bk = k0 + b_k;
+            const int gn = n0 + b_n;
+            if (FULL) {
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
-                b[j] = Bs[buf][kk][(wn * TN + j) * 16 + lr];
+                for (int j = 0; j < BPT; j += 2) {
+                    const v2d v = *reinterpret_cast<const v2d*>(B + (int64_t)bk * ldb + gn + j);
+                    rb[j] = v[0];
+                    rb[j + 1] = v[1];
+                }
+            } else {
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+                for (int j = 0; j < BPT; ++j)
+                    rb[j] = (bk < K && gn + j < N) ? B[(int64_t)bk * ldb + gn + j] : 0.0;
+            }
+        };
+        auto stage = [&](int buf, const double (&ra)[APT], const double (&rb)[BPT]) {
+#pragma unroll
+            for (int j = 0; j < APT; ++j)
+                As[buf][a_row][a_k + j] = ra[j];
+#pragma unroll
+            for (int j = 0; j < BPT; j += 2)
+                *reinterpret_cast<v2d*>(&Bs[buf][b_k][b_n + j]) = (v2d){rb[j], rb[j + 1]};
+        };
+        auto multiply = [&](int buf) {
+#pragma unroll
+            for (int ks = 0; ks < BKT / 4; ++ks) {
+                const int kk = ks * 4 + lk;
+                double a[TM], b[TN];
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+                    a[i] = As[buf][(wm * TM + i) * 16 + lr][kk];
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[i], b[j], acc[i][j], 0, 0, 0);
-        }
-    };
+                    b[j] = Bs[buf][kk][(wn * TN + j) * 16 + lr];
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[i], b[j], acc[i][j], 0, 0, 0);
+            }
+        };
 
-    // Step t multiplies LDS buffer t&1, which holds K slice t. Register set t&1 receives slice
-    // t+2 while that runs; the other set (slice t+1, requested a step earlier) goes to LDS after it.
-    const int nk = (K + BKT - 1) / BKT;
-    double ra0[APT], rb0[BPT], ra1[APT], rb1[BPT];
-    fetch(0, ra0, rb0);
-    if (nk > 1)
-        fetch(BKT, ra1, rb1);
-    stage(0, ra0, rb0);
-    __syncthreads();
-    // At the top of every round LDS buffer 0 holds slice t and register set 1 slice t + 1.
-    // The steady-state rounds carry no conditions, so that the compiler's wait counts leave the
-    // younger pair of loads in flight while the older pair is stored.
-    int t = 0;
-    for (; t + 3 < nk; t += 2) {
-        fetch((t + 2) * BKT, ra0, rb0);
-        multiply(0);
-        stage(1, ra1, rb1);
-        __syncthreads();
-        fetch((t + 3) * BKT, ra1, rb1);
-        multiply(1);
+        // Step t multiplies LDS buffer t&1, which holds K slice t. Register set t&1 receives
+        // slice t+2 while that runs; the other set (slice t+1, requested a step earlier) goes to
+        // LDS after it.
+        const int nk = (K + BKT - 1) / BKT;
+        double ra0[APT], rb0[BPT], ra1[APT], rb1[BPT];
+        fetch(0, ra0, rb0);
+        if (nk > 1)
+            fetch(BKT, ra1, rb1);
         stage(0, ra0, rb0);
         __syncthreads();
-    }
-    if (t + 2 < nk)
-        fetch((t + 2) * BKT, ra0, rb0);
-    multiply(0);
-    if (t + 1 < nk) {
-        stage(1, ra1, rb1);
-        __syncthreads();
-        multiply(1);
-        if (t + 2 < nk) {
+        // At the top of every round LDS buffer 0 holds slice t and register set 1 slice t + 1.
+        // The steady-state rounds carry no conditions, so that the compiler's wait counts leave
+        // the younger pair of loads in flight while the older pair is stored.
+        int t = 0;
+        for (; t + 3 < nk; t += 2) {
+            fetch((t + 2) * BKT, ra0, rb0);
+            multiply(0);
+            stage(1, ra1, rb1);
+            __syncthreads();
+            fetch((t + 3) * BKT, ra1, rb1);
+            multiply(1);
             stage(0, ra0, rb0);
             __syncthreads();
-            multiply(0);
+        }
+        if (t + 2 < nk)
+            fetch((t + 2) * BKT, ra0, rb0);
+        multiply(0);
+        if (t + 1 < nk) {
+            stage(1, ra1, rb1);
+            __syncthreads();
+            multiply(1);
+            if (t + 2 < nk) {
+                stage(0, ra0, rb0);
+                __syncthreads();
+                multiply(0);
+            }
         }
     }
     // D layout of the 16x16x4 f64 instruction (measured on gfx950): register r of a lane holds
@@ -168,7 +208,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_f64_mfma(int M, int N, int 
             for (int r = 0; r < 4; ++r) {
                 const int row = m0 + (wm * TM + i) * 16 + r * 4 + lk;
                 if (FULL || (row < M && col < N)) {
-                    double* c = C + (int64_t)row * ldc + col;
+                    double* c = ch.C + (int64_t)row * ch.ldc + col;
                     *c = *c + acc[i][j][r];
                 }
             }
@@ -226,61 +266,122 @@ int run_generic(int M, int N, int K, const void* A, int64_t lda, const void* B, 
 } // namespace
 
 namespace {
-struct GemmArgs {
-    int M, N, K;
-    const double* A;
-    int64_t lda;
-    const double* B;
-    int64_t ldb;
-    double* C;
-    int64_t ldc;
-};
+
+int check_job(const cnh_gemm_job& j) {
+    CNH_CHECK(j.M >= 0 && j.N >= 0 && j.K >= 0, -2, "cnh_gemm_acc: negative extent");
+    CNH_CHECK(j.M < (1ll << 30) && j.N < (1ll << 30) && j.K < (1ll << 30), -3,
+              "cnh_gemm_acc: extent too large");
+    if (j.M == 0 || j.N == 0 || j.K == 0)
+        return 0;
+    CNH_CHECK(j.A && j.B && j.C, -2, "cnh_gemm_acc: null pointer");
+    CNH_CHECK(j.lda >= j.K && j.ldb >= j.N && j.ldc >= j.N, -2,
+              "cnh_gemm_acc: row stride shorter than the row");
+    return 0;
+}
 
 template <int WM, int WN, int TM, int TN, int BKT>
-int launch_mfma(const GemmArgs& g, bool aligned, hipStream_t st) {
+int launch_chains(std::vector<GemmChain>& chains, const std::vector<GemmSeg>& segs, bool full,
+                  hipStream_t st) {
     constexpr int BM = WM * TM * 16, BN = WN * TN * 16;
-    const int64_t blocks = (((int64_t)g.M + BM - 1) / BM) * (((int64_t)g.N + BN - 1) / BN);
-    CNH_CHECK(blocks < (1ll << 31), -3, "cnh_gemm_acc: too many tiles");
-    const bool full = aligned && g.M % BM == 0 && g.N % BN == 0 && g.K % BKT == 0;
+    int64_t blocks = 0;
+    for (GemmChain& c : chains) {
+        c.nbm = (c.M + BM - 1) / BM;
+        c.blk0 = (int32_t)blocks;
+        blocks += (int64_t)c.nbm * ((c.N + BN - 1) / BN);
+        CNH_CHECK(blocks < (1ll << 31), -3, "cnh_gemm_acc: too many tiles");
+    }
+    const GemmChain* dch = nullptr;
+    const GemmSeg* dsg = nullptr;
+    if (chains.size() > 1 || segs.size() > 1) {
+        // one table: chains, then segments
+        std::vector<unsigned char> table(chains.size() * sizeof(GemmChain) + segs.size() * sizeof(GemmSeg));
+        std::memcpy(table.data(), chains.data(), chains.size() * sizeof(GemmChain));
+        std::memcpy(table.data() + chains.size() * sizeof(GemmChain), segs.data(),
+                    segs.size() * sizeof(GemmSeg));
+        const void* dev = nullptr;
+        if (int rc = desc_upload(table.data(), table.size(), st, &dev))
+            return rc;
+        dch = static_cast<const GemmChain*>(dev);
+        dsg = reinterpret_cast<const GemmSeg*>(static_cast<const unsigned char*>(dev) +
+                                               chains.size() * sizeof(GemmChain));
+    }
+    const int nch = (int)chains.size(), nb = (int)blocks;
     if (full)
         hipLaunchKernelGGL((gemm_f64_mfma<WM, WN, TM, TN, BKT, true>), dim3((unsigned)blocks),
-                           dim3(WM * WN * 64), 0, st, g.M, g.N, g.K, g.A, g.lda, g.B, g.ldb, g.C, g.ldc);
+                           dim3(WM * WN * 64), 0, st, dch, nch, dsg, nb, chains[0], segs[0]);
     else
         hipLaunchKernelGGL((gemm_f64_mfma<WM, WN, TM, TN, BKT, false>), dim3((unsigned)blocks),
-                           dim3(WM * WN * 64), 0, st, g.M, g.N, g.K, g.A, g.lda, g.B, g.ldb, g.C, g.ldc);
+                           dim3(WM * WN * 64), 0, st, dch, nch, dsg, nb, chains[0], segs[0]);
     CNH_HIP(hipGetLastError());
     return 0;
 }
+
+int run_f64_batch(int njobs, const cnh_gemm_job* jobs, hipStream_t st) {
+    std::vector<GemmChain> chains;
+    std::vector<std::vector<GemmSeg>> per_chain;
+    bool full = true;
+    for (int i = 0; i < njobs; ++i) {
+        const cnh_gemm_job& j = jobs[i];
+        if (j.M == 0 || j.N == 0 || j.K == 0)
+            continue;
+        size_t c = 0;
+        for (; c < chains.size(); ++c)
+            if (chains[c].C == j.C && chains[c].M == j.M && chains[c].N == j.N && chains[c].ldc == j.ldc)
+                break;
+        if (c == chains.size()) {
+            chains.push_back(GemmChain{(double*)j.C, j.ldc, (int32_t)j.M, (int32_t)j.N, 0, 0, 0, 0});
+            per_chain.emplace_back();
+        }
+        per_chain[c].push_back(GemmSeg{(const double*)j.A, j.lda, (const double*)j.B, j.ldb, (int32_t)j.K, 0});
+        full = full && (j.M % 64 == 0) && (j.N % 64 == 0) && (j.K % 16 == 0) && (j.lda % 2 == 0) &&
+               (j.ldb % 2 == 0) && (((uintptr_t)j.A & 15) == 0) && (((uintptr_t)j.B & 15) == 0);
+    }
+    if (chains.empty())
+        return 0;
+    std::vector<GemmSeg> segs;
+    int64_t blocks64 = 0;
+    for (size_t c = 0; c < chains.size(); ++c) {
+        chains[c].seg0 = (int32_t)segs.size();
+        chains[c].nseg = (int32_t)per_chain[c].size();
+        segs.insert(segs.end(), per_chain[c].begin(), per_chain[c].end());
+        blocks64 += (int64_t)((chains[c].M + 63) / 64) * ((chains[c].N + 63) / 64);
+    }
+    // 64x64 tiles of four wavefronts when that gives every CU several workgroups; smaller grids
+    // take 8 wavefronts per workgroup so that a CU with one workgroup still has two per SIMD.
+    if (blocks64 >= 1024)
+        return launch_chains<2, 2, 2, 2, 16>(chains, segs, full, st);
+    return launch_chains<2, 4, 2, 1, 16>(chains, segs, full, st);
+}
+
 } // namespace
+
+extern "C" int cnh_gemm_acc_batch(int dtype, int njobs, const cnh_gemm_job* jobs, cnh_stream s) {
+    CNH_CHECK(njobs >= 0 && (njobs == 0 || jobs != nullptr), -2, "cnh_gemm_acc_batch: bad job list");
+    for (int i = 0; i < njobs; ++i)
+        if (int rc = check_job(jobs[i]))
+            return rc;
+    hipStream_t st = as_stream(s);
+    if (dtype == CNH_F64)
+        return run_f64_batch(njobs, jobs, st);
+    for (int i = 0; i < njobs; ++i) {
+        const cnh_gemm_job& j = jobs[i];
+        if (j.M == 0 || j.N == 0 || j.K == 0)
+            continue;
+        int rc;
+        switch (dtype) {
+        case CNH_F32: rc = run_generic<float>((int)j.M, (int)j.N, (int)j.K, j.A, j.lda, j.B, j.ldb, j.C, j.ldc, st); break;
+        case CNH_I32: rc = run_generic<int32_t>((int)j.M, (int)j.N, (int)j.K, j.A, j.lda, j.B, j.ldb, j.C, j.ldc, st); break;
+        case CNH_I64: rc = run_generic<int64_t>((int)j.M, (int)j.N, (int)j.K, j.A, j.lda, j.B, j.ldb, j.C, j.ldc, st); break;
+        default: return set_error(-2, "unknown dtype %d", dtype);
+        }
+        if (rc)
+            return rc;
+    }
+    return 0;
+}
 
 extern "C" int cnh_gemm_acc(int dtype, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda,
                             const void* B, int64_t ldb, void* C, int64_t ldc, cnh_stream s) {
-    if (int rc = ensure_init())
-        return rc;
-    CNH_CHECK(M >= 0 && N >= 0 && K >= 0, -2, "cnh_gemm_acc: negative extent");
-    CNH_CHECK(M < (1ll << 30) && N < (1ll << 30) && K < (1ll << 30), -3,
-              "cnh_gemm_acc: extent too large");
-    if (M == 0 || N == 0 || K == 0)
-        return 0;
-    CNH_CHECK(A && B && C, -2, "cnh_gemm_acc: null pointer");
-    CNH_CHECK(lda >= K && ldb >= N && ldc >= N, -2, "cnh_gemm_acc: row stride shorter than the row");
-    hipStream_t st = as_stream(s);
-    switch (dtype) {
-    case CNH_F64: {
-        const bool aligned = (lda % 2 == 0) && (ldb % 2 == 0) && (((uintptr_t)A & 15) == 0) &&
-                             (((uintptr_t)B & 15) == 0);
-        const GemmArgs ga{(int)M, (int)N, (int)K, (const double*)A, lda, (const double*)B, ldb, (double*)C, ldc};
-        // 64x64 tiles of four wavefronts when that gives every CU several workgroups; smaller
-        // grids take 8 wavefronts per workgroup so that a CU with one workgroup still has two
-        // wavefronts per SIMD.
-        const int64_t blocks64 = ((M + 63) / 64) * ((N + 63) / 64);
-        if (blocks64 >= 1024)
-            return launch_mfma<2, 2, 2, 2, 16>(ga, aligned, st);
-        return launch_mfma<2, 4, 2, 1, 16>(ga, aligned, st);
-    }
-    case CNH_F32: return run_generic<float>((int)M, (int)N, (int)K, A, lda, B, ldb, C, ldc, st);
-    case CNH_I32: return run_generic<int32_t>((int)M, (int)N, (int)K, A, lda, B, ldb, C, ldc, st);
-    case CNH_I64: return run_generic<int64_t>((int)M, (int)N, (int)K, A, lda, B, ldb, C, ldc, st);
-    }
-    return set_error(-2, "unknown dtype %d", dtype);
+    const cnh_gemm_job job{M, N, K, A, lda, B, ldb, C, ldc};
+    return cnh_gemm_acc_batch(dtype, 1, &job, s);
 }

@@ -29,7 +29,6 @@ namespace {
 std::mutex g_mu;
 bool g_inited = false;
 int g_device = 0;
-hipStream_t g_upload_stream = nullptr;
 
 struct Workspace {
     void* ptr = nullptr;
@@ -44,6 +43,8 @@ char* g_slab_host = nullptr;
 size_t g_slab_used = 0;
 struct DescEntry {
     size_t off, bytes;
+    hipStream_t stream; // where the copy was queued
+    bool visible;       // known complete for every stream
 };
 std::unordered_map<uint64_t, std::vector<DescEntry>> g_desc;
 
@@ -79,19 +80,27 @@ int reduce_workspace(hipStream_t s, size_t bytes, void** out) {
     return 0;
 }
 
-int desc_upload(const void* host, size_t bytes, hipStream_t, const void** dev_out) {
+// Descriptor tables are content-addressed: a table seen before is reused. A new one is written to
+// the pinned mirror of the slab and copied on the consumer's own stream, ahead of the kernel that
+// reads it, so the host does not wait for the copy. A slot of the mirror is written once per pass
+// over the slab, and the slab is recycled only after the device has drained.
+int desc_upload(const void* host, size_t bytes, hipStream_t st, const void** dev_out) {
     std::lock_guard<std::mutex> lk(g_mu);
     if (!g_slab_dev) {
         CNH_HIP(hipMalloc((void**)&g_slab_dev, kSlabBytes));
         CNH_HIP(hipHostMalloc((void**)&g_slab_host, kSlabBytes, hipHostMallocDefault));
-        CNH_HIP(hipStreamCreateWithFlags(&g_upload_stream, hipStreamNonBlocking));
     }
     CNH_CHECK(bytes <= kSlabBytes / 4, -3, "descriptor table of %zu bytes is too large", bytes);
     uint64_t h = fnv1a(host, bytes);
     auto it = g_desc.find(h);
     if (it != g_desc.end())
-        for (const DescEntry& e : it->second)
+        for (DescEntry& e : it->second)
             if (e.bytes == bytes && std::memcmp(g_slab_host + e.off, host, bytes) == 0) {
+                if (!e.visible && e.stream != st) {
+                    // uploaded on another stream: its copy must have landed before this one reads
+                    CNH_HIP(hipStreamSynchronize(e.stream));
+                    e.visible = true;
+                }
                 *dev_out = g_slab_dev + e.off;
                 return 0;
             }
@@ -105,10 +114,8 @@ int desc_upload(const void* host, size_t bytes, hipStream_t, const void** dev_ou
     size_t off = g_slab_used;
     g_slab_used += need;
     std::memcpy(g_slab_host + off, host, bytes);
-    CNH_HIP(hipMemcpyAsync(g_slab_dev + off, g_slab_host + off, bytes, hipMemcpyHostToDevice,
-                           g_upload_stream));
-    CNH_HIP(hipStreamSynchronize(g_upload_stream));
-    g_desc[h].push_back({off, bytes});
+    CNH_HIP(hipMemcpyAsync(g_slab_dev + off, g_slab_host + off, bytes, hipMemcpyHostToDevice, st));
+    g_desc[h].push_back({off, bytes, st, false});
     *dev_out = g_slab_dev + off;
     return 0;
 }
@@ -246,6 +253,16 @@ int cnh_stream_create(cnh_stream* out) {
 int cnh_stream_destroy(cnh_stream s) {
     if (!s)
         return 0;
+    {
+        // Descriptor tables whose copies were queued on this stream outlive it in the cache: let
+        // the copies land and mark them complete, so that no later call waits on a dead handle.
+        std::lock_guard<std::mutex> lk(g_mu);
+        CNH_HIP(hipStreamSynchronize(as_stream(s)));
+        for (auto& kv : g_desc)
+            for (DescEntry& e : kv.second)
+                if (e.stream == as_stream(s))
+                    e.visible = true;
+    }
     CNH_HIP(hipStreamDestroy(as_stream(s)));
     return 0;
 }

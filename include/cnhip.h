@@ -244,6 +244,20 @@ int cnh_gemv_tiles(int dtype, int64_t rows, int64_t cols, int32_t tile, const vo
  *      (src/backend_internal.hpp:113-133, src/executor_incremental.cpp:97-132) ---- */
 int cnh_gemm_acc(int dtype, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda,
                  const void* B, int64_t ldb, void* C, int64_t ldc, cnh_stream s);
+/* A list of such products in one launch, with the result of calling cnh_gemm_acc on each job in
+ * list order: jobs naming the same C block (same C, M, N, ldc) accumulate into it in that order
+ * (the panel pairs of one C partition, src/executor_matmatmul.cpp:105-484); C blocks of
+ * different chains must not overlap. */
+typedef struct cnh_gemm_job {
+    int64_t M, N, K;
+    const void* A;
+    int64_t lda;
+    const void* B;
+    int64_t ldb;
+    void* C;
+    int64_t ldc;
+} cnh_gemm_job;
+int cnh_gemm_acc_batch(int dtype, int njobs, const cnh_gemm_job* jobs, cnh_stream s);
 
 /* ---- synthetic inputs generated on the device (no upstream counterpart: upstream has no RNG,
  *      charmnumeric/random.py:4-5, and no bulk upload, charmnumeric.py:863-878) ---- */

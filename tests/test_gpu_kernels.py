@@ -283,6 +283,78 @@ def test_gemm_ones_closed_form_and_strided_panels(dev, orc):
     dev.free_all()
 
 
+@pytest.mark.parametrize("dt,npdt", [(L.F64, np.float64), (L.I64, np.int64)])
+@pytest.mark.parametrize("aligned", [True, False])
+def test_gemm_batch_is_the_jobs_one_after_another(dev, orc, dt, npdt, aligned):
+    """A matmatmul cut into tiles: several C blocks, each fed by several K pieces from panels inside
+    larger buffers. One batched launch must give what the same jobs give one call at a time: exactly
+    for integers; within the 1e-12 bar for fp64, where a workgroup adds the pieces of its block in
+    list order either way, but carries one running sum across them instead of adding per-piece sums."""
+    rng = np.random.default_rng(21)
+    M, N, K = (128, 192, 160) if aligned else (100, 150, 77)
+    kcuts = [0, 64, 96, K] if aligned else [0, 30, 31, K]
+    ncuts = [0, 128, N] if aligned else [0, 70, N]
+    mcuts = [0, 64, M] if aligned else [0, 33, M]
+    if npdt == np.float64:
+        A, B = rng.standard_normal((M, K)), rng.standard_normal((K, N))
+    else:
+        A, B = rng.integers(-9, 9, (M, K)).astype(npdt), rng.integers(-9, 9, (K, N)).astype(npdt)
+    C0 = np.zeros((M, N), npdt)
+    dA, dB, dC, dC1 = dev.array(A), dev.array(B), dev.array(C0), dev.array(C0)
+    esz = A.itemsize
+    jobs = []
+    for mi in range(len(mcuts) - 1):
+        for ni in range(len(ncuts) - 1):
+            for ki in range(len(kcuts) - 1):
+                m0, m1, n0, n1, k0, k1 = mcuts[mi], mcuts[mi + 1], ncuts[ni], ncuts[ni + 1], kcuts[ki], kcuts[ki + 1]
+                jobs.append((m1 - m0, n1 - n0, k1 - k0, (m0 * K + k0) * esz, (k0 * N + n0) * esz, (m0 * N + n0) * esz))
+    jobs.append((0, 5, 5, 0, 0, 0))                  # an empty job is skipped
+    arr = (L.GemmJob * len(jobs))()
+    for j, (m, n, k, oa, ob, oc) in zip(arr, jobs):
+        j.M, j.N, j.K, j.A, j.lda, j.B, j.ldb, j.C, j.ldc = m, n, k, dA.ptr + oa, K, dB.ptr + ob, N, dC.ptr + oc, N
+    L.check(L.lib.cnh_gemm_acc_batch(dt, len(jobs), arr, None))
+    for (m, n, k, oa, ob, oc) in jobs:
+        L.check(L.lib.cnh_gemm_acc(dt, m, n, k, dA.ptr + oa, K, dB.ptr + ob, N, dC1.ptr + oc, N, None))
+    got, one_by_one = dC.get(), dC1.get()
+    if npdt == np.float64:
+        bound = REL * (np.abs(A) @ np.abs(B))
+        assert np.all(np.abs(got - one_by_one) <= bound)
+        assert np.all(np.abs(got - (A.astype(np.longdouble) @ B.astype(np.longdouble)).astype(np.float64)) <= bound)
+    else:
+        assert np.array_equal(got, one_by_one) and np.array_equal(got, A @ B)
+    dev.free_all()
+
+
+def test_descriptor_table_outlives_the_stream_it_was_uploaded_on(dev):
+    """The same job list (hence the same descriptor table) on a stream, then on a second stream after
+    the first was destroyed: the cached table must be usable without touching the dead stream."""
+    rng = np.random.default_rng(31)
+    A, B = rng.standard_normal((64, 48)), rng.standard_normal((48, 64))
+    dA, dB, dC = dev.array(A), dev.array(B), dev.array(np.zeros((64, 64)))
+    arr = (L.GemmJob * 2)()
+    for j, (k0, k1) in zip(arr, ((0, 16), (16, 48))):
+        j.M, j.N, j.K, j.A, j.lda, j.B, j.ldb, j.C, j.ldc = 64, 64, k1 - k0, dA.ptr + k0 * 8, 48, dB.ptr + k0 * 64 * 8, 64, dC.ptr, 64
+    for _ in range(2):
+        st = C.c_void_p()
+        L.check(L.lib.cnh_stream_create(C.byref(st)))
+        L.check(L.lib.cnh_gemm_acc_batch(L.F64, 2, arr, st))
+        L.check(L.lib.cnh_stream_sync(st))
+        L.check(L.lib.cnh_stream_destroy(st))
+    L.check(L.lib.cnh_gemm_acc_batch(L.F64, 2, arr, None))
+    L.check(L.lib.cnh_device_sync())
+    assert np.all(np.abs(dC.get() - 3 * (A @ B)) <= 3 * REL * (np.abs(A) @ np.abs(B)))
+    dev.free_all()
+
+
+def test_gemm_batch_refuses_bad_jobs(dev):
+    arr = (L.GemmJob * 1)()
+    arr[0].M, arr[0].N, arr[0].K, arr[0].lda, arr[0].ldb, arr[0].ldc = 4, 4, 4, 2, 4, 4
+    arr[0].A = arr[0].B = arr[0].C = 256
+    assert L.lib.cnh_gemm_acc_batch(L.F64, 1, arr, None) != 0      # row stride shorter than the row
+    assert L.lib.cnh_gemm_acc_batch(L.F64, -1, arr, None) != 0
+    assert L.lib.cnh_gemm_acc_batch(L.F64, 0, None, None) == 0
+
+
 @pytest.mark.parametrize("dt,npdt", [(L.F32, np.float32), (L.I32, np.int32), (L.I64, np.int64)])
 def test_gemm_other_dtypes(dev, orc, dt, npdt):
     rng = np.random.default_rng(4)
