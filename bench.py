@@ -665,6 +665,8 @@ def run_frontend(n, steps, warmup):
     cnp.reset()
     itf = cnp.CharmNumericInterface(device=0)
     itf.connect(odf=4)
+    itf.set_pipeline(True)               # the executor works on its own thread while Python records
+    out["pipelined"] = True
     try:
         cnp.set_auto_flush(itf, 48)      # keep the device busy while later statements are recorded
         A = cnp.random.cg_matrix(n, 2)
@@ -701,6 +703,7 @@ def run_frontend(n, steps, warmup):
         for key, shape, sweeps in (("jacobi2d_8192", (8192, 8192), 100), ("jacobi3d_512", (512, 512, 512), 50)):
             it16 = cnp.CharmNumericInterface(device=0)
             it16.connect(odf=16 if len(shape) == 2 else 64)
+            it16.set_pipeline(True)
             cnp.set_auto_flush(it16, 48)
             u = cnp.zeros(shape)
             if len(shape) == 2:
@@ -732,6 +735,7 @@ def run_frontend(n, steps, warmup):
         n, b, word, d = 64, 256, 1024, 1024
         itl = cnp.CharmNumericInterface(device=0)
         itl.connect(odf=4)
+        itl.set_pipeline(True)
         cnp.set_auto_flush(itl, 48)
         X = cnp.random.uniform((n, b, word), seed=5, stream=0, low=-1.0, high=1.0)
         W = cnp.random.uniform((word + d, 4 * d), seed=5, stream=1, low=-1.0 / 32, high=1.0 / 32)

@@ -228,6 +228,7 @@ _PROTOS.update({
     "cnx_destroy": (C.c_int, [C.c_void_p]),
     "cnx_set_min_tile": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
     "cnx_receive_dag": (C.c_int, [C.c_void_p, C.c_int, C.c_int64, C.c_char_p]),
+    "cnx_set_async": (C.c_int, [C.c_void_p, C.c_int]),
     "cnx_get": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int, C.c_void_p]),
     "cnx_put": (C.c_int, [C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_void_p]),
     "cnx_fill_uniform": (C.c_int, [C.c_void_p, C.c_int, C.c_uint64, C.c_uint64, C.c_double, C.c_double]),

@@ -7,10 +7,15 @@
 
 #include <algorithm>
 #include <array>
+#include <condition_variable>
 #include <cstring>
+#include <deque>
 #include <map>
 #include <memory>
+#include <mutex>
 #include <sstream>
+#include <string>
+#include <thread>
 #include <unordered_map>
 #include <vector>
 
@@ -132,6 +137,17 @@ struct cnx_executor {
     bool trace_on = false;
     std::string trace;
     uintptr_t fake_ptr = 0x1000;
+    // Asynchronous mode: DAG messages queue up for a thread of the executor's own, as upstream's
+    // frontend hands them to a server and goes on recording. Every other entry point waits for
+    // the queue first; an error of a queued message is reported by the next call on the executor.
+    int device = 0;
+    bool async_on = false, busy = false, stop = false;
+    std::thread worker;
+    std::mutex qmu;
+    std::condition_variable qcv, idle_cv;
+    std::deque<std::vector<char>> queue;
+    int deferred_rc = 0;
+    std::string deferred_msg;
 
     void log(const std::string& s) {
         if (trace_on) {
@@ -1168,6 +1184,77 @@ int parse_dag(const char* msg, int64_t size, std::vector<DagNode>& out) {
 
 } // namespace
 
+namespace {
+
+int run_message(Ex* ex, const char* msg, int64_t size) {
+    std::vector<DagNode> dag;
+    if (int rc = parse_dag(msg, size, dag))
+        return rc;
+    for (const DagNode& n : dag)
+        if (int rc = exec_node(ex, n))
+            return rc;
+    return 0;
+}
+
+void worker_loop(Ex* ex) {
+    if (!ex->dry)
+        (void)hipSetDevice(ex->device);   // the current device is a per-thread setting
+    std::unique_lock<std::mutex> lk(ex->qmu);
+    for (;;) {
+        ex->qcv.wait(lk, [&] { return ex->stop || !ex->queue.empty(); });
+        if (ex->queue.empty())
+            return;   // stop requested and nothing left
+        std::vector<char> msg = std::move(ex->queue.front());
+        ex->queue.pop_front();
+        if (ex->deferred_rc != 0) {   // work behind a failed message is dropped
+            if (ex->queue.empty())
+                ex->idle_cv.notify_all();
+            continue;
+        }
+        ex->busy = true;
+        lk.unlock();
+        const int rc = run_message(ex, msg.data(), (int64_t)msg.size());
+        std::string text = rc ? cnh_last_error() : "";
+        lk.lock();
+        ex->busy = false;
+        if (rc) {
+            ex->deferred_rc = rc;
+            ex->deferred_msg = std::move(text);
+        }
+        if (ex->queue.empty())
+            ex->idle_cv.notify_all();
+    }
+}
+
+// Waits for queued messages and hands over the error one of them may have left.
+int drain(Ex* ex) {
+    if (!ex->async_on)
+        return 0;
+    std::unique_lock<std::mutex> lk(ex->qmu);
+    ex->idle_cv.wait(lk, [&] { return ex->queue.empty() && !ex->busy; });
+    if (ex->deferred_rc == 0)
+        return 0;
+    const int rc = ex->deferred_rc;
+    const std::string text = std::move(ex->deferred_msg);
+    ex->deferred_rc = 0;
+    ex->deferred_msg.clear();
+    lk.unlock();
+    return set_error(rc, "%s", text.c_str());
+}
+
+void stop_worker(Ex* ex) {
+    {
+        std::unique_lock<std::mutex> lk(ex->qmu);
+        ex->stop = true;
+        ex->qcv.notify_all();
+    }
+    if (ex->worker.joinable())
+        ex->worker.join();
+    ex->async_on = false;
+}
+
+} // namespace
+
 extern "C" {
 
 int cnx_create(int device, int num_pes, int odf, cnx_executor** out) {
@@ -1177,6 +1264,7 @@ int cnx_create(int device, int num_pes, int odf, cnx_executor** out) {
     ex->dry = device < 0;
     ex->num_pes = num_pes;
     ex->odf = odf;
+    ex->device = device;
     if (!ex->dry) {
         if (int rc = cnh_init(device))
             return rc;
@@ -1190,6 +1278,10 @@ int cnx_create(int device, int num_pes, int odf, cnx_executor** out) {
 int cnx_destroy(cnx_executor* ex) {
     if (!ex)
         return 0;
+    if (ex->async_on) {
+        (void)drain(ex);
+        stop_worker(ex);
+    }
     if (!ex->dry) {
         cnh_stream_sync(ex->stream);
         for (auto& kv : ex->arrays) {
@@ -1210,6 +1302,8 @@ int cnx_destroy(cnx_executor* ex) {
 
 int cnx_set_min_tile(cnx_executor* ex, int ndims, int min_tile) {
     CNH_CHECK(ex != nullptr, -2, "null executor");
+    if (int rc = drain(ex))
+        return rc;
     CNH_CHECK(ndims >= 1 && ndims <= 3 && min_tile >= 1, -2, "bad minimum tile %d for rank %d",
               min_tile, ndims);
     ex->min_tile[ndims] = min_tile;
@@ -1218,12 +1312,16 @@ int cnx_set_min_tile(cnx_executor* ex, int ndims, int min_tile) {
 
 int cnx_set_trace(cnx_executor* ex, int on) {
     CNH_CHECK(ex != nullptr, -2, "null executor");
+    if (int rc = drain(ex))
+        return rc;
     ex->trace_on = on != 0;
     return 0;
 }
 
 int64_t cnx_trace(cnx_executor* ex, char* buf, size_t cap) {
     CNH_CHECK(ex != nullptr, -2, "null executor");
+    if (int rc = drain(ex))
+        return rc;
     int64_t need = (int64_t)ex->trace.size() + 1;
     if (buf && cap >= (size_t)need) {
         std::memcpy(buf, ex->trace.c_str(), (size_t)need);
@@ -1235,18 +1333,37 @@ int64_t cnx_trace(cnx_executor* ex, char* buf, size_t cap) {
 int cnx_receive_dag(cnx_executor* ex, int epoch, int64_t size, const char* msg) {
     (void)epoch;
     CNH_CHECK(ex != nullptr && msg != nullptr && size >= 12, -2, "bad DAG message");
-    std::vector<DagNode> dag;
-    if (int rc = parse_dag(msg, size, dag))
-        return rc;
-    for (const DagNode& n : dag)
-        if (int rc = exec_node(ex, n))
-            return rc;
-    return 0;
+    if (!ex->async_on)
+        return run_message(ex, msg, size);
+    {
+        std::unique_lock<std::mutex> lk(ex->qmu);
+        if (ex->deferred_rc == 0) {
+            ex->queue.emplace_back(msg, msg + size);
+            ex->qcv.notify_one();
+            return 0;
+        }
+    }
+    return drain(ex);   // an earlier message failed: report that instead of queueing more
+}
+
+int cnx_set_async(cnx_executor* ex, int on) {
+    CNH_CHECK(ex != nullptr, -2, "null executor");
+    const int rc = drain(ex);
+    if (on && !ex->async_on) {
+        ex->stop = false;
+        ex->async_on = true;
+        ex->worker = std::thread(worker_loop, ex);
+    } else if (!on && ex->async_on) {
+        stop_worker(ex);
+    }
+    return rc;
 }
 
 int cnx_get(cnx_executor* ex, int ndims, int epoch, int name, int64_t size, int dtype, void* host_out) {
     (void)epoch;
     CNH_CHECK(ex != nullptr && host_out != nullptr, -2, "null argument");
+    if (int rc = drain(ex))
+        return rc;
     XArray* a;
     if (int rc = find_array(ex, name, &a, "get"))
         return rc;
@@ -1289,6 +1406,8 @@ int cnx_get(cnx_executor* ex, int ndims, int epoch, int name, int64_t size, int 
 
 int cnx_put(cnx_executor* ex, int name, int64_t size, int dtype, const void* host_in) {
     CNH_CHECK(ex != nullptr && host_in != nullptr, -2, "null argument");
+    if (int rc = drain(ex))
+        return rc;
     XArray* a;
     if (int rc = find_array(ex, name, &a, "put"))
         return rc;
@@ -1331,6 +1450,8 @@ int cnx_put(cnx_executor* ex, int name, int64_t size, int dtype, const void* hos
 
 int cnx_fill_uniform(cnx_executor* ex, int name, uint64_t seed, uint64_t stream_id, double lo, double hi) {
     CNH_CHECK(ex != nullptr, -2, "null executor");
+    if (int rc = drain(ex))
+        return rc;
     XArray* a;
     if (int rc = find_array(ex, name, &a, "fill_uniform"))
         return rc;
@@ -1358,6 +1479,8 @@ int cnx_fill_uniform(cnx_executor* ex, int name, uint64_t seed, uint64_t stream_
 
 int cnx_fill_cg_matrix(cnx_executor* ex, int name, uint64_t seed) {
     CNH_CHECK(ex != nullptr, -2, "null executor");
+    if (int rc = drain(ex))
+        return rc;
     XArray* a;
     if (int rc = find_array(ex, name, &a, "fill_cg_matrix"))
         return rc;
@@ -1378,6 +1501,8 @@ int cnx_fill_cg_matrix(cnx_executor* ex, int name, uint64_t seed) {
 
 int cnx_sync(cnx_executor* ex) {
     CNH_CHECK(ex != nullptr, -2, "null executor");
+    if (int rc = drain(ex))
+        return rc;
     if (ex->dry)
         return 0;
     return cnh_stream_sync(ex->stream);
@@ -1386,6 +1511,8 @@ int cnx_sync(cnx_executor* ex) {
 int cnx_array_info(cnx_executor* ex, int name, int* ndims, int* dtype, int* tile, int32_t* shape3,
                    int32_t* offset3) {
     CNH_CHECK(ex != nullptr, -2, "null executor");
+    if (int rc = drain(ex))
+        return rc;
     XArray* a;
     if (int rc = find_array(ex, name, &a, "array_info"))
         return rc;
@@ -1406,6 +1533,8 @@ int cnx_array_info(cnx_executor* ex, int name, int* ndims, int* dtype, int* tile
 
 int cnx_stats(cnx_executor* ex, int64_t out[8]) {
     CNH_CHECK(ex != nullptr && out != nullptr, -2, "null argument");
+    if (int rc = drain(ex))
+        return rc;
     ex->stats[6] = (int64_t)ex->arrays.size();
     for (int i = 0; i < 8; ++i)
         out[i] = ex->stats[i];

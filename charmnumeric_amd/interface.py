@@ -20,6 +20,20 @@ class CharmNumericInterface:
         self.odf = None
         self._ex = None
         self._min_tiles = {}
+        self._pipeline = False
+
+    # -- pipelining --------------------------------------------------------------------------
+    def set_pipeline(self, on=True):
+        """Upstream's frontend hands DAG messages to a server and goes on recording; with
+        pipelining on, the executor does the same with a thread of its own: send_dag returns once
+        the message is queued, and the executor works through the queue while Python records the
+        next statements. Whatever reads state back (get, sync, array_info, stats, trace, close)
+        waits for the queue first. An error of the executor then surfaces at the next call on the
+        interface, not at the send that caused it; work queued behind a failed message is
+        dropped."""
+        self._pipeline = bool(on)
+        if self._ex is not None:
+            L.check(L.lib.cnx_set_async(self._ex, 1 if on else 0))
 
     # -- connection --------------------------------------------------------------------------
     def connect(self, server_ip=None, server_port=None, odf=4):
@@ -31,6 +45,8 @@ class CharmNumericInterface:
         self.odf = int(odf)
         for nd, t in self._min_tiles.items():
             L.check(L.lib.cnx_set_min_tile(self._ex, nd, t))
+        if self._pipeline:
+            L.check(L.lib.cnx_set_async(self._ex, 1))
         return self
 
     def set_min_tile(self, ndims, min_tile):
@@ -42,9 +58,11 @@ class CharmNumericInterface:
     def close(self):
         if self._ex is not None:
             # instructions still pending refer to arrays of this executor: drop them
-            lazy.execute(self)
-            L.check(L.lib.cnx_destroy(self._ex))
-            self._ex = None
+            try:
+                lazy.execute(self)
+            finally:
+                ex, self._ex = self._ex, None
+                L.check(L.lib.cnx_destroy(ex))
 
     def __enter__(self):
         return self
@@ -107,6 +125,7 @@ class CharmNumericInterface:
 
     def trace(self):
         need = L.lib.cnx_trace(self._handle(), None, 0)
+        L.check(need)
         buf = C.create_string_buffer(int(need))
         L.lib.cnx_trace(self._handle(), buf, need)
         return buf.value.decode().splitlines()

@@ -78,6 +78,13 @@ int cnx_set_min_tile(cnx_executor* ex, int ndims, int min_tile);
  * src/dag_group_receive.cpp:190-575) followed by the partitions' run(): executes every node of the
  * DAG in order. Returns when all work is queued on the executor's stream (not when it finished). */
 int cnx_receive_dag(cnx_executor* ex, int epoch, int64_t size, const char* msg);
+/* Asynchronous mode (off by default). When on, cnx_receive_dag copies the message, queues it for a
+ * thread that belongs to the executor and returns; the messages run in the order received, as
+ * upstream's frontend hands messages to its server and goes on recording
+ * (charmnumeric/interface.py upstream). Every other call on the executor first waits for the
+ * queue. A queued message that fails makes the executor drop what is queued behind it, and its
+ * error code and text are returned by the next call on the executor, whichever it is. */
+int cnx_set_async(cnx_executor* ex, int on);
 
 /* receive_get_request(int ndims, int epoch, int name, int size, int dtype) + gather + reply
  * (src/backend.ci:16-17, src/partition_get.cpp:4-67, src/dag_group_runtime.cpp:55-118): copies

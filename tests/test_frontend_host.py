@@ -240,6 +240,35 @@ def test_matvec_of_a_plane_keeps_the_tile_grid_of_the_rank3_array(itf):
     assert sum(ln.startswith("matmul") for ln in itf.trace()) == 2
 
 
+def test_pipelined_interface_does_the_same_work_and_defers_errors(itf):
+    def program():
+        a = cnp.ones((300,))
+        b = cnp.arange(300, dtype=np.float64)
+        for _ in range(5):
+            b[1:-1] = 0.5 * (b[:-2] + b[2:]) + a[1:-1]
+            cnp.execute(itf)
+        s = b.dot(a)
+        cnp.execute(itf)
+        return s
+
+    kinds = lambda log: [ln.split()[0] for ln in log]
+    program()
+    cnp.execute(itf)
+    plain = kinds(itf.trace())
+    itf.set_pipeline(True)
+    program()
+    cnp.execute(itf)
+    assert kinds(itf.trace()) == plain          # reading the log waits for the queue
+    # an executor error surfaces at the next call that reads state back, and the queue keeps working
+    itf.send_dag(7, b"not a dag message")
+    with pytest.raises(RuntimeError):
+        itf.sync()
+    itf.sync()
+    itf.set_pipeline(False)
+    with pytest.raises(RuntimeError):
+        itf.send_dag(8, b"not a dag message")
+
+
 def test_malformed_messages_are_refused(itf):
     with pytest.raises(RuntimeError, match="bad magic"):
         itf.send_dag(0, struct.pack("<iii", 1, 1, 0))

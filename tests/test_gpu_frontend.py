@@ -351,6 +351,36 @@ def test_lstm_forward_example(itf, n, b, d, word, small):
     assert np.allclose(Hout.get(itf), wH, rtol=1e-11, atol=1e-13)
 
 
+def test_pipelined_executor_gives_the_same_results(small_tiles):
+    """Asynchronous mode: messages queue up for the executor's own thread while Python records;
+    reads wait for the queue. Same statements, same bits."""
+    itf = small_tiles
+    itf.set_pipeline(True)
+    cnp.set_auto_flush(itf, 8)
+    n = 70
+    rng = np.random.default_rng(12)
+    host = rng.standard_normal((n, n))
+    u = cnp.array(host)
+    w = cnp.array(rng.standard_normal((n,)))
+    x = cnp.ones((n,))
+    for _ in range(12):
+        u[1:-1, 1:-1] = 0.25 * (u[:-2, 1:-1] + u[2:, 1:-1] + u[1:-1, :-2] + u[1:-1, 2:])
+        host[1:-1, 1:-1] = 0.25 * (host[:-2, 1:-1] + host[2:, 1:-1] + host[1:-1, :-2] + host[1:-1, 2:])
+        x = x + 0.5 * w
+    assert np.array_equal(u.get(itf), host)
+    y = (u @ x).get(itf)
+    hx = np.ones(n)
+    for _ in range(12):
+        hx = hx + 0.5 * w.get(itf)
+    assert np.array_equal(x.get(itf), hx)
+    assert np.all(np.abs(y - host @ hx) <= 1e-12 * (np.abs(host) @ np.abs(hx)))
+    # an executor error is reported by the next call, and the interface works afterwards
+    itf.send_dag(99, b"not a dag message")
+    with pytest.raises(RuntimeError):
+        itf.sync()
+    assert np.array_equal(x.get(itf), hx)
+
+
 def test_tile_matches_numpy(small_tiles):
     host = np.arange(12, dtype=np.float64).reshape(3, 4)
     a = cnp.array(host)
