@@ -499,6 +499,7 @@ struct LeafReg { int arr; int start[3]; int step[3]; };
 struct TilesArgs {
     int out_off[3];
     int rs[3], re[3], rst[3];   // assigned region in the target's own coordinates
+    int lattice;                // 1: a DTile's bs/bw count points of the region's lattice (in place)
     LeafReg leaf[NLA];
 };
 #define TL_PER_THREAD 4
@@ -523,25 +524,30 @@ extern "C" __global__ __launch_bounds__(256) void grp_tiles(const Tiled* arrs, c
     const i64 blk = (i64)blockIdx.x - dt.blk0;
     const i64 outer = blk / dt.nchunks;
     const int chunk = (int)(blk - outer * dt.nchunks);
-    const int l1 = dt.bs[1] + (int)(outer % dt.bw[1]);
-    const int l0 = dt.bs[0] + (int)(outer / dt.bw[1]);
-    const int a0 = dt.cs[0] + l0 - ta.out_off[0];
-    const int a1 = dt.cs[1] + l1 - ta.out_off[1];
-    const bool in01 = a0 >= ta.rs[0] && a0 < ta.re[0] && (a0 - ta.rs[0]) % ta.rst[0] == 0 &&
-                      a1 >= ta.rs[1] && a1 < ta.re[1] && (a1 - ta.rs[1]) % ta.rst[1] == 0;
-    const int k0 = (a0 - ta.rs[0]) / ta.rst[0];
-    const int k1 = (a1 - ta.rs[1]) / ta.rst[1];
+    const int i1 = dt.bs[1] + (int)(outer % dt.bw[1]);
+    const int i0 = dt.bs[0] + (int)(outer / dt.bw[1]);
+    // in place: (i0, i1, i2) are indices into the region's lattice; otherwise tile coordinates
+    const int a0 = ta.lattice ? ta.rs[0] + i0 * ta.rst[0] : dt.cs[0] + i0 - ta.out_off[0];
+    const int a1 = ta.lattice ? ta.rs[1] + i1 * ta.rst[1] : dt.cs[1] + i1 - ta.out_off[1];
+    const int l0 = a0 + ta.out_off[0] - dt.cs[0];
+    const int l1 = a1 + ta.out_off[1] - dt.cs[1];
+    const bool in01 = ta.lattice ||
+                      (a0 >= ta.rs[0] && a0 < ta.re[0] && (a0 - ta.rs[0]) % ta.rst[0] == 0 &&
+                       a1 >= ta.rs[1] && a1 < ta.re[1] && (a1 - ta.rs[1]) % ta.rst[1] == 0);
+    const int k0 = ta.lattice ? i0 : (a0 - ta.rs[0]) / ta.rst[0];
+    const int k1 = ta.lattice ? i1 : (a1 - ta.rs[1]) / ta.rst[1];
 #pragma unroll
     for (int u = 0; u < TL_PER_THREAD; ++u) {
-        const int i2 = chunk * (256 * TL_PER_THREAD) + u * 256 + (int)threadIdx.x;
-        if (i2 >= dt.bw[2]) continue;
-        const int l2 = dt.bs[2] + i2;
+        const int j2 = chunk * (256 * TL_PER_THREAD) + u * 256 + (int)threadIdx.x;
+        if (j2 >= dt.bw[2]) continue;
+        const int i2 = dt.bs[2] + j2;
+        const int a2 = ta.lattice ? ta.rs[2] + i2 * ta.rst[2] : dt.cs[2] + i2 - ta.out_off[2];
+        const int l2 = a2 + ta.out_off[2] - dt.cs[2];
         const i64 di = ((i64)l0 * dt.w[1] + l1) * dt.w[2] + l2;
-        const int a2 = dt.cs[2] + l2 - ta.out_off[2];
-        const bool inside = in01 && a2 >= ta.rs[2] && a2 < ta.re[2] &&
-                            (a2 - ta.rs[2]) % ta.rst[2] == 0;
+        const bool inside = in01 && (ta.lattice || (a2 >= ta.rs[2] && a2 < ta.re[2] &&
+                                                    (a2 - ta.rs[2]) % ta.rst[2] == 0));
         if (inside) {
-            const int k2 = (a2 - ta.rs[2]) / ta.rst[2];
+            const int k2 = ta.lattice ? i2 : (a2 - ta.rs[2]) / ta.rst[2];
             T l[NLA], o[NOA];
 #pragma unroll
             for (int q = 0; q < NL; ++q) {

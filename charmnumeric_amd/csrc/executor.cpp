@@ -526,6 +526,40 @@ int result_shape(Ex* ex, const DagNode& n, const cnh_ast_node& root, int32_t sha
     return 0;
 }
 
+// True when {s0 + i*t0 < e0} and {s1 + j*t1 < e1} have no common element.
+bool progressions_disjoint(int64_t s0, int64_t e0, int64_t t0, int64_t s1, int64_t e1, int64_t t1) {
+    if (t0 < 1)
+        t0 = 1;
+    if (t1 < 1)
+        t1 = 1;
+    if (s0 >= e0 || s1 >= e1)
+        return true;
+    const int64_t last0 = s0 + (e0 - 1 - s0) / t0 * t0, last1 = s1 + (e1 - 1 - s1) / t1 * t1;
+    if (last0 < s1 || last1 < s0)
+        return true;
+    int64_t g = t0, h = t1;
+    while (h) {
+        const int64_t r = g % h;
+        g = h;
+        h = r;
+    }
+    if ((s1 - s0) % g != 0)
+        return true;
+    // a common element exists modulo lcm; walk the progression that starts later, at most
+    // t_other / g steps, and see whether one falls inside both ranges
+    const int64_t hi = std::min(last0, last1);
+    int64_t x = std::max(s0, s1), tx, so, to;
+    if (s0 >= s1) {
+        tx = t0, so = s1, to = t1;
+    } else {
+        tx = t1, so = s0, to = t0;
+    }
+    for (int64_t n = 0; n <= to / g && x <= hi; ++n, x += tx)
+        if ((x - so) % to == 0)
+            return false;
+    return true;
+}
+
 int exec_group(Ex* ex, const DagNode& n) {
     const cnh_ast_node& root = n.nodes[n.roots.back()];
     for (size_t i = 0; i + 1 < n.roots.size(); ++i)
@@ -640,7 +674,9 @@ int exec_group(Ex* ex, const DagNode& n) {
     // reads whatever tiles the operand regions fall into (replaces the fragment path and its halo
     // messages, src/execute_node.cpp:1338-1585, src/executor_core.cpp:8-143).
     // Reading the target through another region is a hazard only where that region can meet the
-    // assigned one: disjoint bounding boxes (C[t] = f(C[t-1])) are safe in place.
+    // assigned one. Two regions share no point when their index progressions miss each other in
+    // some dimension: other slabs (C[t] = f(C[t-1])), or the other colour of a red-black update
+    // (phi[1:-1:2, ...] = f(phi[0:-2:2, ...])). Those run in place.
     bool aliased = false;
     if (is_set)
         for (int i = 0; i < n_in; ++i)
@@ -656,7 +692,8 @@ int exec_group(Ex* ex, const DagNode& n) {
                 bool disjoint = false;
                 if (!ir.is_global && !root.region.is_global)
                     for (int d = 0; d < target->ndims; ++d)
-                        if (ir.stop[d] <= root.region.start[d] || root.region.stop[d] <= ir.start[d])
+                        if (progressions_disjoint(ir.start[d], ir.stop[d], ir.step[d], root.region.start[d],
+                                                  root.region.stop[d], root.region.step[d]))
                             disjoint = true;
                 if (!disjoint)
                     aliased = true;

@@ -931,7 +931,7 @@ extern "C" int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* 
     const int NL = (int)p.load_leaf.size();
     const int NLA = NL > 0 ? NL : 1;
     std::vector<const cnh_tiled*> arrays;
-    std::vector<int32_t> targs(12 + 7 * NLA, 0);
+    std::vector<int32_t> targs(13 + 7 * NLA, 0);   // TilesArgs of the generated kernel
     for (int d = 0; d < 3; ++d) {
         targs[d] = d >= pad ? dst->offset[d - pad] : 0;
         targs[3 + d] = rs[d];
@@ -951,7 +951,7 @@ extern "C" int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* 
             ai = (int)arrays.size();
             arrays.push_back(arr);
         }
-        int32_t* lr = &targs[12 + 7 * l];
+        int32_t* lr = &targs[13 + 7 * l];
         lr[0] = ai;
         for (int d = 0; d < 3; ++d) {
             lr[1 + d] = 0;
@@ -994,6 +994,7 @@ extern "C" int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* 
         ntiles *= dst->grid[d];
     std::vector<DTileDev> dts;
     int64_t blocks = 0;
+    bool lattice = false;
     for (int64_t t = 0; t < ntiles; ++t) {
         int ti[3] = {0, 0, 0};
         int64_t rem = t;
@@ -1022,19 +1023,29 @@ extern "C" int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* 
         dt.dst = dst->tiles[t];
         dt.cur = cur ? cur->tiles[t] : nullptr;
         // In place (or with nothing to copy from), elements outside the assigned region keep
-        // their values without being touched: visit only the part of the tile inside the
-        // region's bounding box, and skip tiles it misses.
+        // their values without being touched: the launch walks the points of the region's index
+        // lattice that fall into the tile (bs = index of the first one along each dimension,
+        // bw = how many), and skips tiles the region misses. A ping-pong launch writes every
+        // element of the new buffer and walks the whole tile.
         const bool in_place = dt.cur == nullptr || dt.cur == dt.dst;
+        lattice = in_place;
         for (int d = 0; d < 3; ++d) {
             dt.bs[d] = 0;
             dt.bw[d] = dt.w[d];
             if (in_place && d >= pad) {
-                const int lo = std::max(dt.cs[d], rs[d] + dst->offset[d - pad]);
-                const int hi = std::min(dt.cs[d] + dt.w[d], re[d] + dst->offset[d - pad]);
-                if (hi <= lo)
+                const int off = dst->offset[d - pad];
+                const int lo = std::max(dt.cs[d], rs[d] + off) - off;           // array coordinates
+                const int hi = std::min(dt.cs[d] + dt.w[d], re[d] + off) - off;
+                if (hi <= lo) {
                     empty = true;
-                dt.bs[d] = lo - dt.cs[d];
-                dt.bw[d] = hi - lo;
+                    continue;
+                }
+                const int kfirst = (lo - rs[d] + rst[d] - 1) / rst[d];          // first index with point >= lo
+                const int klast = (hi - 1 - rs[d]) / rst[d];                    // last index with point < hi
+                if (klast < kfirst)
+                    empty = true;
+                dt.bs[d] = kfirst;
+                dt.bw[d] = klast - kfirst + 1;
             }
         }
         if (empty)
@@ -1046,6 +1057,7 @@ extern "C" int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* 
     }
     if (dts.empty())
         return 0;
+    targs[12] = lattice ? 1 : 0;
 
     std::vector<TiledDev> adev(arrays.size() ? arrays.size() : 1);
     for (size_t a = 0; a < arrays.size(); ++a)

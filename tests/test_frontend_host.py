@@ -269,6 +269,45 @@ def test_pipelined_interface_does_the_same_work_and_defers_errors(itf):
         itf.send_dag(8, b"not a dag message")
 
 
+def test_in_place_when_read_and_written_lattices_miss_each_other(itf):
+    """An operand that reads the target array forces ping-pong buffers only if its index lattice can
+    meet the assigned one; red-black colours, other slabs and interleaved strides run in place."""
+    itf.set_min_tile(1, 64)
+    itf.set_min_tile(2, 16)
+    b = cnp.arange(200, dtype=np.float64)
+    phi = cnp.zeros((40, 40))
+    cnp.execute(itf)
+    itf.trace()
+
+    def how(stmt):
+        stmt()
+        cnp.execute(itf)
+        (line,) = lines(itf, "group")
+        return line.split()[-1]
+
+    def assign(dst, src):
+        def stmt():
+            b[dst] = b[src] * 2.0
+        return stmt
+
+    assert how(assign(slice(1, -1), slice(0, -2))) == "pingpong"             # shifted overlap
+    assert how(assign(slice(1, -1, 2), slice(0, -2, 2))) == "inplace"        # odd <- even
+    assert how(assign(slice(0, 10, 3), slice(1, 11, 3))) == "inplace"        # {0,3,6,9} <- {1,4,7,10}
+    assert how(assign(slice(0, 10, 2), slice(4, 14, 2))) == "pingpong"       # share 4, 6, 8
+    assert how(assign(slice(0, 9, 2), slice(3, 18, 3))) == "pingpong"        # share 6
+    assert how(assign(slice(0, 5, 2), slice(3, 12, 3))) == "inplace"         # {0,2,4} vs {3,6,9}
+    assert how(assign(slice(100, 150), slice(0, 50))) == "inplace"           # apart
+
+    def red():
+        phi[1:-1:2, 1:-1:2] = 0.25 * (phi[0:-2:2, 1:-1:2] + phi[2::2, 1:-1:2] + phi[1:-1:2, 0:-2:2]
+                                      + phi[1:-1:2, 2::2])
+    assert how(red) == "inplace"
+
+    def jacobi():
+        phi[1:-1, 1:-1] = 0.25 * (phi[:-2, 1:-1] + phi[2:, 1:-1] + phi[1:-1, :-2] + phi[1:-1, 2:])
+    assert how(jacobi) == "pingpong"
+
+
 def test_malformed_messages_are_refused(itf):
     with pytest.raises(RuntimeError, match="bad magic"):
         itf.send_dag(0, struct.pack("<iii", 1, 1, 0))
