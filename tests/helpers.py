@@ -2,6 +2,7 @@
 from __future__ import annotations
 
 import ctypes as C
+import os
 
 import numpy as np
 
@@ -262,6 +263,13 @@ def launch_tiles(k, inputs, scalars, cur, dst, scalars_on_device=False):
     L.check(L.lib.cnh_launch_group_tiles(k, len(inputs), descs, len(scalars), sp,
                                          1 if scalars_on_device else 0,
                                          C.byref(cd) if cd is not None else None, C.byref(dd), None))
+
+
+def golden():
+    """The known-answer vectors of upstream's tests, kept as data under tests/golden."""
+    import json
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "upstream_known_answers.json")) as f:
+        return json.load(f)
 
 
 def host_libm_is_the_restated_one():

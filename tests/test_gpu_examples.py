@@ -2,9 +2,10 @@
 already hold, written against this frontend and compared with NumPy running the same statements:
 red-black Gauss-Seidel by strided slices (examples/gauss_seidel.py), matvec and matmatmul on sliced
 and dimension-dropped operands (examples/matvec_slice.py, examples/matmatmul.py), the pieces and a
-whole V-cycle of the 2-D multigrid solver (examples/multigrid2d.py) and weighted Jacobi with a
-residual (examples/jacobi_iteration.py). Element-wise statements must match NumPy bit for bit;
-products are held to 1e-12 of the sum of absolute products."""
+whole V-cycle of the 2-D multigrid solver (examples/multigrid2d.py, with its weighted Jacobi smoother
+and residual), numpy.diag both ways (examples/diag.py) and the Jacobi iteration x += D^-1 (b - A x)
+built from diag and matvec (examples/jacobi_iteration.py). Element-wise statements must match NumPy
+bit for bit; products are held to 1e-12 of the sum of absolute products."""
 import numpy as np
 import pytest
 
@@ -125,6 +126,25 @@ def test_diag_builds_and_extracts(itf, k, dtype):
     assert np.array_equal(cnp.diag(cnp.array(m_host), k).get(itf), np.diag(m_host, k))
     assert np.array_equal(cnp.diag(cnp.array(m_host.T.copy()), k).get(itf), np.diag(m_host.T, k))
     assert np.array_equal(cnp.diag(cnp.array(m_host)[3:80, 5:121], k).get(itf), np.diag(m_host[3:80, 5:121], k))
+
+
+def test_jacobi_iteration_with_diag_and_matvec(itf):
+    """A = ones + 2N I assembled with diag, its diagonal read back with diag, 50 steps of
+    x += D^-1 (b - A x): converges to the direct solution (upstream checks atol 1e-6)."""
+    n = 128
+    A = cnp.ones((n, n)) + cnp.diag(cnp.full((n,), 2.0 * n))
+    d = cnp.diag(A).get(itf)
+    assert np.array_equal(d, np.full(n, 2.0 * n + 1.0))
+    b, x = cnp.ones((n,)), cnp.zeros((n,))
+    d_inv = cnp.full((n,), 1.0 / (2.0 * n + 1.0))
+    a_host = np.ones((n, n)) + 2.0 * n * np.eye(n)
+    x_host = np.zeros(n)
+    for _ in range(50):
+        x = x + d_inv * (b - A @ x)
+        x_host = x_host + (1.0 / (2.0 * n + 1.0)) * (1.0 - a_host @ x_host)
+    got = x.get(itf)
+    assert np.allclose(got, np.linalg.solve(a_host, np.ones(n)), atol=1e-6)
+    assert np.allclose(got, x_host, rtol=1e-12, atol=0)
 
 
 # ---- multigrid pieces ----

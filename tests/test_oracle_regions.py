@@ -12,6 +12,7 @@ import numpy as np
 import pytest
 
 from charmnumeric_amd._lib import Region  # struct layout only
+from tests import helpers as H
 
 
 def R(start, stop, step=None):
@@ -62,12 +63,11 @@ def rmap(lib, r, p1, p2):
 def test_reference_map_vectors(orc):
     """tests/test_jit.cpp:303-326: [64:127:2] in [2:127:2] -> [1:64] is [32:64], and back."""
     lib = orc.lib
-    m = rmap(lib, R(64, 127, 2), R(2, 127, 2), R(1, 64, 1))
-    assert m.as_tuple() == ((32,), (64,), (1,))
-    assert lib.orc_region_size_dim(C.addressof(m), 0) == 32
-    back = rmap(lib, R(32, 64, 1), R(1, 64, 1), R(2, 127, 2))
-    assert back.as_tuple() == ((64,), (128,), (2,))
-    assert lib.orc_region_size_dim(C.addressof(back), 0) == 32
+    for case in H.golden()["region_map"]["cases"]:
+        m = rmap(lib, R(*case["region"]), R(*case["from_parent"]), R(*case["to_parent"]))
+        a, b, c = case["expect"]
+        assert m.as_tuple() == ((a,), (b,), (c,))
+        assert lib.orc_region_size_dim(C.addressof(m), 0) == case["expect_size"]
 
 
 def test_reference_subtract_and_decompose_regressions(orc):
@@ -124,17 +124,19 @@ def _align(lib, nd, inputs, parents, cap=64):
 def test_reference_align_fragments_vectors(orc):
     """tests/test_jit.cpp:244-300: stepped parent [0:64:2], halves [0:32:2] and [32:64:2]."""
     lib = orc.lib
-    parent, left, right = R(0, 64, 2), R(0, 32, 2), R(32, 64, 2)
+    g = H.golden()["align_fragments"]
+    parent, left, right = R(*g["parent"]), R(*g["halves"][0]), R(*g["halves"][1])
     res = _align(lib, 1, [[(parent, None)], [(left, None), (right, None)]], [parent, parent])
     assert len(res[0]) == 2 and len(res[1]) == 2
-    assert [c["size"] for c in res[0]] == [16, 16]
-    assert [c["stride"] for c in res[0]] == [1, 1]           # packed fragments keep dense strides
-    assert [c["off"] for c in res[0]] == [0, 16]             # base, base + 16
-    assert [(c["frag"], c["off"]) for c in res[1]] == [(1, 0), (2, 0)]
+    assert [c["size"] for c in res[0]] == g["packed_parent"]["sizes"]
+    assert [c["stride"] for c in res[0]] == g["packed_parent"]["strides"]    # packed fragments keep dense strides
+    assert [c["off"] for c in res[0]] == g["packed_parent"]["offsets"]       # base, base + 16
+    assert [[c["frag"], c["off"]] for c in res[1]] == g["halves_cells"]
     # a local dense buffer with explicit stride 1 is addressed with stride 2 and offset 32
-    res = _align(lib, 1, [[(parent, (1,))], [(left, None), (right, None)]], [parent, parent])
-    assert [c["stride"] for c in res[0]] == [2, 2]
-    assert [c["off"] for c in res[0]] == [0, 32]
+    dl = g["dense_local_parent"]
+    res = _align(lib, 1, [[(parent, (dl["src_stride"],))], [(left, None), (right, None)]], [parent, parent])
+    assert [c["stride"] for c in res[0]] == dl["strides"]
+    assert [c["off"] for c in res[0]] == dl["offsets"]
 
 
 def test_reference_tile_rule_vectors(orc):
@@ -146,8 +148,12 @@ def test_reference_tile_rule_vectors(orc):
         return lib.orc_tile_rule(len(shape), (C.c_int32 * 3)(*shape), odf, pes, mint)
 
     # upstream vectors: B (200 elements) and TMP (200), B (100) all come out with tile 64
-    assert tile((200,), 4, 1, 64) == 64
-    assert tile((100,), 4, 1, 64) == 64
+    for case in H.golden()["tile_rule"]["cases"]:
+        assert tile(tuple(case["shape"]), case["odf"], case["pes"], case["min_tile"]) == case["tile"]
+    # the tiles upstream's solver cases end with are what the rule gives before offsets are chosen
+    for case in H.golden()["decomposition_offsets"]["cases"]:
+        if "shape" in case:
+            assert tile(tuple(s - 2 for s in case["shape"]), 4, 1, 64) == case["expect"]["tile"]
     # consequences of the doubling rule (tile count must not exceed odf * PEs)
     assert tile((512,), 4, 1, 64) == 128          # 8 tiles of 64 > 4 -> 128
     assert tile((129, 129), 4, 1, 64) == 128      # 3 x 3 tiles of 64 > 4 -> 2 x 2 of 128
