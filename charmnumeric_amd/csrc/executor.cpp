@@ -189,7 +189,10 @@ int slab_alloc(Ex* ex, size_t bytes, bool zero, void** out) {
         ex->fake_ptr += (bytes + 255) & ~(size_t)255;
         return 0;
     }
-    return cnh_alloc(bytes, zero ? 1 : 0, out);
+    // cleared on the executor's own stream, in order with whatever writes the array next
+    if (int rc = cnh_alloc(bytes, 0, out))
+        return rc;
+    return zero ? cnh_memset0(*out, bytes, ex->stream) : 0;
 }
 
 void slab_release(Ex* ex, size_t bytes, void* p) {

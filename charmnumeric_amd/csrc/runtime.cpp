@@ -3,6 +3,7 @@
 // src/partition_get.cpp:42-65 and the fence/callback completion of src/dispatch.hpp:40-53.
 #include "common.h"
 
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <unordered_map>
@@ -161,8 +162,12 @@ int cnh_alloc(size_t bytes, int zero, void** dptr) {
     CNH_CHECK(dptr != nullptr, -2, "cnh_alloc: null output pointer");
     void* p = nullptr;
     CNH_HIP(hipMalloc(&p, bytes ? bytes : 1));
-    if (zero && bytes)
-        CNH_HIP(hipMemset(p, 0, bytes));
+    if (zero && bytes) {
+        // The fill runs on the null stream, which streams made by cnh_stream_create do not wait
+        // for: without the wait a first write queued on such a stream can be overtaken by it.
+        CNH_HIP(hipMemsetAsync(p, 0, bytes, nullptr));
+        CNH_HIP(hipStreamSynchronize(nullptr));
+    }
     *dptr = p;
     return 0;
 }
