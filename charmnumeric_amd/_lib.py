@@ -191,6 +191,7 @@ _PROTOS = {
                                     C.POINTER(C.c_int), C.POINTER(Region)]),
     "cnh_kernel_source": (C.c_int64, [C.c_void_p, C.c_char_p, C.c_char_p, C.c_size_t]),
     "cnh_kernel_build": (C.c_int, [C.c_void_p, C.c_char_p]),
+    "cnh_kernel_variants_loaded": (C.c_int, [C.c_void_p, C.c_char_p]),
     "cnh_launch_group": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.POINTER(Memref), C.c_int, _vpp,
                                    C.c_int, C.c_int, C.POINTER(Memref), C.c_void_p]),
     "cnh_launch_group_batched": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int,

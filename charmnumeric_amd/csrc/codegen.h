@@ -78,7 +78,12 @@ struct DirectShape {
     int halo[3] = {0, 0, 0};
     int tx = 0, ty = 0, ry = 0, rz = 0;
     std::vector<std::array<int, 3>> shifts; // per distinct load, dims padded to (z, y, x)
+    // per distinct load: -1 = the assigned array itself (read through the window), else which of
+    // the other arrays it reads at the element's own position (source terms, weights)
+    std::vector<int> other;
+    std::vector<int> other_names; // array names in the order the indices above number them
 };
+constexpr int kDirectMaxOther = 4;
 int direct_shape(const GroupProgram& p, const DirectConfig& cfg, DirectShape& sh, std::string& err);
 
 // Source text of a kernel variant. `variant` is one of "flat", "nd", "tiles", "slide".

@@ -1,4 +1,5 @@
-// Register-window source for same-array unit-step stencils (the Jacobi-style SET_REGION groups).
+// Register-window source for same-array unit-step stencils (the Jacobi-style SET_REGION groups),
+// optionally with operands of other arrays read at the element's own position (source terms).
 //
 // Every lane owns RZ x RY output rows of one 16-byte column pair inside ONE tile. It first issues
 // all the 128-bit loads of its window (the rows and planes its shifted operands touch, aligned
@@ -42,16 +43,36 @@ int direct_shape(const GroupProgram& p, const DirectConfig& cfg, DirectShape& sh
         return -18;
     }
     sh.shifts.assign(p.load_leaf.size(), {0, 0, 0});
+    sh.other.assign(p.load_leaf.size(), -1);
+    bool reads_target = false;
     for (size_t l = 0; l < p.load_leaf.size(); ++l) {
         const LeafUse& u = p.leaves[p.load_leaf[l]];
-        if (u.name != p.out_target[0]) {
-            err = "operand is not the assigned array";
-            return -18;
-        }
         if (!u.has_region) {
             err = "operand without a region";
             return -18;
         }
+        if (u.name != p.out_target[0]) {
+            // another array (a source term, a weight): only at the element's own position
+            for (int d = 0; d < nd; ++d)
+                if (u.region.step[d] != 1 || u.region.start[d] != ro.start[d] ||
+                    u.region.stop[d] != ro.stop[d]) {
+                    err = "operand of another array is shifted";
+                    return -18;
+                }
+            size_t j = 0;
+            while (j < sh.other_names.size() && sh.other_names[j] != u.name)
+                ++j;
+            if (j == sh.other_names.size()) {
+                if ((int)j == kDirectMaxOther) {
+                    err = "too many arrays";
+                    return -18;
+                }
+                sh.other_names.push_back(u.name);
+            }
+            sh.other[l] = (int)j;
+            continue;
+        }
+        reads_target = true;
         for (int d = 0; d < nd; ++d) {
             if (u.region.step[d] != 1 ||
                 u.region.stop[d] - u.region.start[d] != ro.stop[d] - ro.start[d]) {
@@ -62,6 +83,10 @@ int direct_shape(const GroupProgram& p, const DirectConfig& cfg, DirectShape& sh
             sh.shifts[l][pad + d] = s;
             sh.halo[pad + d] = std::max(sh.halo[pad + d], std::abs(s));
         }
+    }
+    if (!reads_target) {
+        err = "the assigned array is not read";
+        return -18;
     }
     for (int d = 0; d < 3; ++d)
         if (sh.halo[d] > 2) {
@@ -125,6 +150,12 @@ std::string direct_source(const GroupProgram& p, const DirectConfig& cfg, std::s
         s << (l ? ", " : "") << "{" << sh.shifts[l][0] << ", " << sh.shifts[l][1] << ", "
           << sh.shifts[l][2] << "}";
     s << "};\n";
+    const int NOTH = (int)sh.other_names.size();
+    s << "#define DR_NOTH " << NOTH << "\n#define DR_NOTHA " << (NOTH > 0 ? NOTH : 1) << "\n";
+    s << "__device__ constexpr int DR_OTHER[NLA] = {";
+    for (size_t l = 0; l < sh.other.size(); ++l)
+        s << (l ? ", " : "") << sh.other[l];
+    s << "};\n";
     s << "__device__ constexpr bool DR_NEED[DR_WZ][DR_WY][DR_WK] = {";
     for (int z = 0; z < WZ; ++z) {
         s << (z ? ", " : "") << "{";
@@ -159,6 +190,7 @@ struct DirectArgs {
     FDiv ggrid1, ggrid2;   // ordering groups along y and x
     FDiv grow, gcol;       // workgroups per group along x and y
     FDiv tbz, tby, tbx;    // = tb[0], tb[1], tb[2]
+    const T* const* oth[4]; // tile tables of the other arrays read at the element's own position
 };
 typedef T P2 __attribute__((ext_vector_type(2)));
 typedef int I2 __attribute__((ext_vector_type(2)));
@@ -285,6 +317,16 @@ __device__ __forceinline__ void direct_fast(const DirectArgs& a, const T* s) {
                 src = last ? rp + (i * w1 + j) * rstr : src;
                 beyond[i][j] = *reinterpret_cast<const P2*>(src);
             }
+    P2 ov[DR_NOTHA][DR_RZ][DR_RY];
+#pragma unroll
+    for (int j = 0; j < DR_NOTH; ++j) {
+        const T* const ot = a.oth[j][p.t] + ((lz0 * w1 + ly0) * w2 + lx);
+#pragma unroll
+        for (int rz = 0; rz < DR_RZ; ++rz)
+#pragma unroll
+            for (int ry = 0; ry < DR_RY; ++ry)
+                ov[j][rz][ry] = *reinterpret_cast<const P2*>(ot + (rz * w1 + ry) * w2);
+    }
 #pragma unroll
     for (int i = 0; i < DR_WZ; ++i)
 #pragma unroll
@@ -314,8 +356,10 @@ __device__ __forceinline__ void direct_fast(const DirectArgs& a, const T* s) {
 #pragma unroll
                 for (int q = 0; q < NL; ++q) {
                     const int xx = e + DR_SHIFT[q][2];
-                    l[q] = win[rz + DR_H0 + DR_SHIFT[q][0]][ry + DR_H1 + DR_SHIFT[q][1]]
-                              [DR_HK + floordiv2(xx)][xx & 1];
+                    l[q] = DR_OTHER[q] >= 0
+                               ? ov[DR_OTHER[q] >= 0 ? DR_OTHER[q] : 0][rz][ry][e]
+                               : win[rz + DR_H0 + DR_SHIFT[q][0]][ry + DR_H1 + DR_SHIFT[q][1]]
+                                    [DR_HK + floordiv2(xx)][xx & 1];
                 }
                 group_eval(l, s, o);
                 const int gx = p.tx0 + lx + e;
@@ -439,6 +483,20 @@ __device__ __forceinline__ void direct_rest(const DirectArgs& a, const T* s, int
         }
     }
 
+    // ---- the other arrays, at the lane's own rows and planes (clamped into the tile: what a
+    // row or plane beyond the tile would read is never used) ----
+    P2 ov[DR_NOTHA][DR_RZ][DR_RY];
+#pragma unroll
+    for (int j = 0; j < DR_NOTH; ++j) {
+        const T* const ot = a.oth[j][t];
+#pragma unroll
+        for (int rz = 0; rz < DR_RZ; ++rz)
+#pragma unroll
+            for (int ry = 0; ry < DR_RY; ++ry)
+                ov[j][rz][ry] = *reinterpret_cast<const P2*>(
+                    ot + ((min(lz0 + rz, w0 - 1) * w1 + min(ly0 + ry, w1 - 1)) * w2 + lx));
+    }
+
     // ---- evaluate and store ----
 #pragma unroll
     for (int rz = 0; rz < DR_RZ; ++rz) {
@@ -464,8 +522,10 @@ __device__ __forceinline__ void direct_rest(const DirectArgs& a, const T* s, int
 #pragma unroll
                         for (int q = 0; q < NL; ++q) {
                             const int xx = e + DR_SHIFT[q][2];
-                            l[q] = win[rz + DR_H0 + DR_SHIFT[q][0]][ry + DR_H1 + DR_SHIFT[q][1]]
-                                      [DR_HK + floordiv2(xx)][xx & 1];
+                            l[q] = DR_OTHER[q] >= 0
+                                       ? ov[DR_OTHER[q] >= 0 ? DR_OTHER[q] : 0][rz][ry][e]
+                                       : win[rz + DR_H0 + DR_SHIFT[q][0]][ry + DR_H1 + DR_SHIFT[q][1]]
+                                            [DR_HK + floordiv2(xx)][xx & 1];
                         }
                         group_eval(l, s, o);
                         res[e] = in_region ? o[0] : win[rz + DR_H0][ry + DR_H1][DR_HK][e];

@@ -274,6 +274,15 @@ int64_t cnh_kernel_source(cnh_kernel* k, const char* variant, char* buf, size_t 
     return (int64_t)v.src.size() + 1;
 }
 
+int cnh_kernel_variants_loaded(const cnh_kernel* k, const char* prefix) {
+    CNH_CHECK(k != nullptr && prefix != nullptr, -2, "null argument");
+    int n = 0;
+    for (const auto& kv : k->variants)
+        if (kv.second.obj && kv.first.compare(0, std::strlen(prefix), prefix) == 0)
+            ++n;
+    return n;
+}
+
 int cnh_kernel_build(cnh_kernel* k, const char* variant) {
     CNH_CHECK(k != nullptr && variant != nullptr, -2, "null argument");
     KernelVariant* v = nullptr;
@@ -637,8 +646,10 @@ struct DirectArgsDev {
     void* dst;
     int32_t tile, shape[3], grid[3], rs[3], re[3], tb[3], sg[3], nblocks, nblocks8, stagger;
     FDivDev per_group, ggrid1, ggrid2, grow, gcol, tbz, tby, tbx;
+    const void* oth[kDirectMaxOther];
 };
-static_assert(sizeof(DirectArgsDev) == 16 + 4 * 22 + 12 * 8, "DirectArgsDev layout must match the generated struct");
+static_assert(sizeof(DirectArgsDev) == 16 + 4 * 22 + 12 * 8 + 8 * kDirectMaxOther,
+              "DirectArgsDev layout must match the generated struct");
 
 int g_stencil_mode = 2; // 0 = general gather, 1 = LDS sliding window, 2 = register window
 int g_direct_group = 0; // order workgroups by groups of neighbouring tiles (rank 3)
@@ -648,8 +659,13 @@ DirectConfig g_direct_cfg;
 
 // Launches the register-window variant under the same conditions as the sliding window, plus:
 // every tile extent along the fastest dimension is even (128-bit accesses never straddle tiles).
+int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const cnh_tiled*>& arrays,
+                  const cnh_tiled* const* others, int n_other, const cnh_tiled* cur,
+                  const cnh_tiled* dst, const std::vector<unsigned char>& scal, hipStream_t st,
+                  bool* handled);
+
 int try_launch_direct(cnh_kernel* k, const std::vector<const cnh_tiled*>& arrays,
-                      const cnh_tiled* cur, const cnh_tiled* dst,
+                      const std::vector<int>& leaf_array, const cnh_tiled* cur, const cnh_tiled* dst,
                       const std::vector<unsigned char>& scal, hipStream_t st, bool* handled) {
     *handled = false;
     const GroupProgram& p = k->prog;
@@ -657,8 +673,40 @@ int try_launch_direct(cnh_kernel* k, const std::vector<const cnh_tiled*>& arrays
     std::string why;
     if (g_stencil_mode != 2 || direct_shape(p, g_direct_cfg, sh, why) != 0)
         return 0;
-    if (!cur || arrays.size() != 1 || cur->tile < 2 || (cur->tile % 2) != 0)
+    if (!cur || arrays.empty() || cur->tile < 2 || (cur->tile % 2) != 0)
         return 0;
+    // Which operand array is the assigned one (read through the window), which are the others:
+    // the generated code numbers the others by name, the launch must hand it the same arrays.
+    int self = -1;
+    const cnh_tiled* others[kDirectMaxOther] = {nullptr, nullptr, nullptr, nullptr};
+    if (leaf_array.size() != sh.other.size())
+        return 0;
+    for (size_t l = 0; l < sh.other.size(); ++l) {
+        const int ai = leaf_array[l];
+        if (ai < 0 || ai >= (int)arrays.size())
+            return 0;
+        if (sh.other[l] < 0) {
+            if (self >= 0 && self != ai)
+                return 0;
+            self = ai;
+        } else {
+            const cnh_tiled*& slot = others[sh.other[l]];
+            if (slot != nullptr && slot != arrays[(size_t)ai])
+                return 0;
+            slot = arrays[(size_t)ai];
+        }
+    }
+    if (self < 0)
+        return 0;
+    const std::vector<const cnh_tiled*> own(1, arrays[(size_t)self]);
+    return launch_direct(k, sh, own, others, (int)sh.other_names.size(), cur, dst, scal, st, handled);
+}
+
+int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const cnh_tiled*>& arrays,
+                  const cnh_tiled* const* others, int n_other, const cnh_tiled* cur,
+                  const cnh_tiled* dst, const std::vector<unsigned char>& scal, hipStream_t st,
+                  bool* handled) {
+    const GroupProgram& p = k->prog;
     // a lane's own rows and planes must not straddle tiles: the tile edge (a power of two) has
     // to be a multiple of what one lane owns
     if (cur->tile % sh.ry != 0 || cur->tile % sh.rz != 0)
@@ -682,6 +730,19 @@ int try_launch_direct(cnh_kernel* k, const std::vector<const cnh_tiled*>& arrays
             return 0; // in place: a sweep would read values it has already written
         if (((uintptr_t)cur->tiles[t] & 15) || ((uintptr_t)dst->tiles[t] & 15))
             return 0;
+    }
+    // the other arrays are read at the element's own position: same decomposition, other memory
+    for (int j = 0; j < n_other; ++j) {
+        const cnh_tiled* o = others[j];
+        if (o == nullptr || o->ndims != cur->ndims || o->tile != cur->tile)
+            return 0;
+        for (int d = 0; d < nd; ++d)
+            if (o->offset[d] != 0 || o->shape[d] != cur->shape[d] || o->grid[d] != cur->grid[d] ||
+                o->grid_lo[d] != cur->grid_lo[d])
+                return 0;
+        for (int64_t t = 0; t < ntiles; ++t)
+            if (((uintptr_t)o->tiles[t] & 15) || o->tiles[t] == dst->tiles[t])
+                return 0;
     }
     DirectArgsDev a;
     std::memset(&a, 0, sizeof a);
@@ -748,6 +809,9 @@ int try_launch_direct(cnh_kernel* k, const std::vector<const cnh_tiled*>& arrays
         return rc;
     a.cur = dcur;
     a.dst = const_cast<void*>(ddst);
+    for (int j = 0; j < n_other; ++j)
+        if (int rc = desc_upload(others[j]->tiles, (size_t)ntiles * sizeof(void*), st, &a.oth[j]))
+            return rc;
     const bool nt_stores = volume * 16 >= (128ll << 20); // the written stream is not read back soon
     // Two launches over the same grid: wavefronts that lie inside their tile in y and z take the
     // lean kernel, the other kernel does what is left (all of it when the lean one does not apply).
@@ -931,6 +995,7 @@ extern "C" int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* 
     const int NL = (int)p.load_leaf.size();
     const int NLA = NL > 0 ? NL : 1;
     std::vector<const cnh_tiled*> arrays;
+    std::vector<int> leaf_array;   // per distinct load: index into `arrays`
     std::vector<int32_t> targs(13 + 7 * NLA, 0);   // TilesArgs of the generated kernel
     for (int d = 0; d < 3; ++d) {
         targs[d] = d >= pad ? dst->offset[d - pad] : 0;
@@ -953,6 +1018,7 @@ extern "C" int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* 
         }
         int32_t* lr = &targs[13 + 7 * l];
         lr[0] = ai;
+        leaf_array.push_back(ai);
         for (int d = 0; d < 3; ++d) {
             lr[1 + d] = 0;
             lr[4 + d] = 1;
@@ -978,7 +1044,7 @@ extern "C" int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* 
     // Same-array unit-step stencil with ping-pong buffers: register-window or LDS sliding window.
     {
         bool handled = false;
-        if (int rc = try_launch_direct(k, arrays, cur, dst, scal, st, &handled))
+        if (int rc = try_launch_direct(k, arrays, leaf_array, cur, dst, scal, st, &handled))
             return rc;
         if (handled)
             return 0;

@@ -169,6 +169,9 @@ int cnh_kernel_output(const cnh_kernel* k, int i, int* result_name, int* target_
 int64_t cnh_kernel_source(cnh_kernel* k, const char* variant, char* buf, size_t cap);
 /* Builds the code object of one variant for gfx950 without loading it (works without a GPU). */
 int cnh_kernel_build(cnh_kernel* k, const char* variant);
+/* How many variants whose name starts with `prefix` ("flat", "nd", "tiles", "slide", "direct")
+ * have a code object, i.e. were built or launched: tells a test which kernel a launch took. */
+int cnh_kernel_variants_loaded(const cnh_kernel* k, const char* prefix);
 /* One fragment / one tile. scalars[i] points at one element of the group dtype; with
  * scalars_on_device != 0 they are device pointers and are read by the kernel itself (no host
  * round trip for dot results feeding later groups). */

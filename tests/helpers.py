@@ -193,6 +193,50 @@ def ast_jacobi3d(n, dtype=L.F64, name=0, coef=0.16666666666666666):
     return b.finish()
 
 
+def ast_poisson2d(n, dtype=L.F64, u_name=0, f_name=1, coef=0.25):
+    """u[1:-1,1:-1] = coef*((((up+down)+left)+right)+f[1:-1,1:-1]): a Jacobi sweep with a source
+    term held in a second array."""
+    b = AstBuilder(dtype, 2)
+    u, f = b.leaf(u_name), b.leaf(f_name)
+    mid = ((1, 1), (n - 1, n - 1), (1, 1))
+    t1 = b.binary(L.OP_ADD, 100, u, u, ((0, 1), (n - 2, n - 1), (1, 1)), ((2, 1), (n, n - 1), (1, 1)))
+    t2 = b.binary(L.OP_ADD, 101, t1, u, None, ((1, 0), (n - 1, n - 2), (1, 1)))
+    t3 = b.binary(L.OP_ADD, 102, t2, u, None, ((1, 2), (n - 1, n), (1, 1)))
+    t4 = b.binary(L.OP_ADD, 103, t3, f, None, mid)
+    t5 = b.binary(L.OP_MUL, 104, b.scalar(coef), t4)
+    b.set_region(105, u, t5, mid)
+    return b.finish()
+
+
+def ast_poisson3d(n, dtype=L.F64, u_name=0, f_name=1, coef=0.16666666666666666):
+    """The 7-point sweep with a source term: u[1:-1,..] = coef*((sum of six neighbours)+f[1:-1,..])."""
+    b = AstBuilder(dtype, 3)
+    u, f = b.leaf(u_name), b.leaf(f_name)
+
+    def reg(s0, s1, s2):
+        return ((s0, s1, s2), (s0 + n - 2, s1 + n - 2, s2 + n - 2), (1, 1, 1))
+
+    shifts = [reg(0, 1, 1), reg(2, 1, 1), reg(1, 0, 1), reg(1, 2, 1), reg(1, 1, 0), reg(1, 1, 2)]
+    t = b.binary(L.OP_ADD, 100, u, u, shifts[0], shifts[1])
+    for i, r in enumerate(shifts[2:]):
+        t = b.binary(L.OP_ADD, 101 + i, t, u, None, r)
+    t = b.binary(L.OP_ADD, 109, t, f, None, reg(1, 1, 1))
+    t = b.binary(L.OP_MUL, 110, b.scalar(coef), t)
+    b.set_region(111, u, t, reg(1, 1, 1))
+    return b.finish()
+
+
+def np_poisson(u, f, coef):
+    v = u.copy()
+    if u.ndim == 2:
+        v[1:-1, 1:-1] = coef * ((((u[:-2, 1:-1] + u[2:, 1:-1]) + u[1:-1, :-2]) + u[1:-1, 2:]) + f[1:-1, 1:-1])
+    else:
+        v[1:-1, 1:-1, 1:-1] = coef * (((((((u[:-2, 1:-1, 1:-1] + u[2:, 1:-1, 1:-1]) + u[1:-1, :-2, 1:-1])
+                                          + u[1:-1, 2:, 1:-1]) + u[1:-1, 1:-1, :-2]) + u[1:-1, 1:-1, 2:]))
+                                      + f[1:-1, 1:-1, 1:-1])
+    return v
+
+
 def np_jacobi2d(u, coef=0.25):
     v = u.copy()
     v[1:-1, 1:-1] = coef * (((u[:-2, 1:-1] + u[2:, 1:-1]) + u[1:-1, :-2]) + u[1:-1, 2:])

@@ -56,6 +56,56 @@ def test_jacobi3d_tiles_bit_exact(dev, orc, stencil_path, n, tile):
     assert np.array_equal(got.view(np.int64), ref.view(np.int64))
 
 
+@pytest.mark.parametrize("nd,n,tile", [(2, 64, 16), (2, 70, 32), (2, 1030, 256), (2, 512, 256), (3, 20, 8),
+                                       (3, 36, 16), (3, 128, 128)])
+def test_sweep_with_source_term_in_a_second_array(dev, orc, stencil_path, nd, n, tile):
+    """u[1:-1,..] = c*((neighbours)+f[1:-1,..]): the register-window kernel reads the second array
+    at the element's own position; the other stencil modes take the general gather. Bit for bit
+    against NumPy on every path."""
+    shape = (n,) * nd
+    u0 = orc.uniform(n ** nd, 3, 0, -1.0, 1.0).reshape(shape)
+    f0 = orc.uniform(n ** nd, 4, 0, -1.0, 1.0).reshape(shape)
+    coef = 0.25 if nd == 2 else 1.0 / 6.0
+    ast = H.ast_poisson2d(n, coef=coef) if nd == 2 else H.ast_poisson3d(n, coef=coef)
+    k = H.compile_group(ast, L.F64, nd)
+    a, b = H.TiledArray(dev, u0, tile), H.TiledArray(dev, np.zeros_like(u0), tile)
+    f = H.TiledArray(dev, f0, tile)
+    ref = u0.copy()
+    for _ in range(3):
+        H.launch_tiles(k, [a] * (2 * nd) + [f], [], a, b)
+        a, b = b, a
+        ref = H.np_poisson(ref, f0, coef)
+    dev.sync()
+    got = a.gather()
+    took_direct = L.lib.cnh_kernel_variants_loaded(k, b"direct") > 0
+    dev.free_all()
+    assert np.array_equal(got.view(np.int64), ref.view(np.int64))
+    assert took_direct == (stencil_path == "direct")
+
+
+def test_source_term_at_a_shifted_position_takes_the_general_gather(dev):
+    """f read one column off the element's position is not something the register window holds."""
+    n, tile = 64, 16
+    rng = np.random.default_rng(2)
+    u0, f0 = rng.standard_normal((n, n)), rng.standard_normal((n, n))
+    b = AstBuilder(L.F64, 2)
+    u, f = b.leaf(0), b.leaf(1)
+    mid = ((1, 1), (n - 1, n - 1), (1, 1))
+    t1 = b.binary(L.OP_ADD, 100, u, u, ((0, 1), (n - 2, n - 1), (1, 1)), ((2, 1), (n, n - 1), (1, 1)))
+    t2 = b.binary(L.OP_ADD, 101, t1, f, None, ((1, 0), (n - 1, n - 2), (1, 1)))
+    b.set_region(102, u, t2, mid)
+    k = H.compile_group(b.finish(), L.F64, 2)
+    a, c, ft = H.TiledArray(dev, u0, tile), H.TiledArray(dev, np.zeros_like(u0), tile), H.TiledArray(dev, f0, tile)
+    H.launch_tiles(k, [a, a, ft], [], a, c)
+    dev.sync()
+    got = c.gather()
+    took_direct = L.lib.cnh_kernel_variants_loaded(k, b"direct") > 0
+    dev.free_all()
+    want = u0.copy()
+    want[1:-1, 1:-1] = (u0[:-2, 1:-1] + u0[2:, 1:-1]) + f0[1:-1, :-2]
+    assert np.array_equal(got, want) and not took_direct
+
+
 def test_reference_jacobi3d_known_answer(dev, stencil_path):
     """4^3 grid, faces 1.0: every interior point becomes (1/6)*3 = 0.5 (upstream test)."""
     u0 = np.zeros((4, 4, 4))
