@@ -746,13 +746,18 @@ int exec_group(Ex* ex, const DagNode& n) {
     }
     cnh_tiled cur = target->tiled(false);
     cnh_tiled dst = aliased ? target->tiled(true) : cur;
-    ex->log("group node=" + std::to_string(n.id) + " path=tiles inputs=" + std::to_string(n_in) +
-            " scalars=" + std::to_string(n_scalar) + " out=" + std::to_string(target->name) +
-            (aliased ? " pingpong" : " inplace"));
     if (!ex->dry)
         if (int rc = cnh_launch_group_tiles(k, n_in, tin.data(), n_scalar, scalars.data(), 1,
                                             is_set ? &cur : nullptr, &dst, ex->stream))
             return rc;
+    // which kernels this group has used so far: the register-window or sliding-window stencil
+    // kernels, or the general gather
+    const char* used = ex->dry ? "" : cnh_kernel_variants_loaded(k, "direct") > 0 ? " kernel=direct"
+                                  : cnh_kernel_variants_loaded(k, "slide") > 0  ? " kernel=slide"
+                                                                                : " kernel=gather";
+    ex->log("group node=" + std::to_string(n.id) + " path=tiles inputs=" + std::to_string(n_in) +
+            " scalars=" + std::to_string(n_scalar) + " out=" + std::to_string(target->name) +
+            (aliased ? " pingpong" : " inplace") + used);
     if (aliased) {
         std::swap(target->slab, target->alt);
         std::swap(target->tiles, target->alt_tiles);

@@ -95,7 +95,7 @@ def record(instr):
         # a program made of elementwise statements only has no such point: flush it anyway once
         # the backlog is large
         if _between_statements() or len(_state.pending) >= 16 * af[1]:
-            execute(af[0])
+            execute(af[0], hold_back=True)
     _state.pending.append(instr)
 
 
@@ -165,11 +165,12 @@ def _uses_of(batch, dropped=()):
     return uses
 
 
-def _plan(batch):
+def _plan(batch, dead_later=()):
     """Returns the list of work items in execution order:
-    ("group", _Group) | ("instr", index) | ("delete", name)."""
+    ("group", _Group) | ("instr", index) | ("delete", name).
+    `dead_later`: results whose handle is known to be dropped, unread, right after this batch."""
     producer = {ins.name: i for i, ins in enumerate(batch) if ins.kind == "op"}
-    deleted = {ins.name for ins in batch if ins.kind == "delete"}
+    deleted = {ins.name for ins in batch if ins.kind == "delete"} | set(dead_later)
     dropped = set()                     # dead code: op indices never emitted
     forced = set()                      # op results that must be materialised
 
@@ -388,10 +389,11 @@ def _emit_delete(name, node_id):
     return _LONE_NODE.pack(node_id, 0, 1, 1, name, OP_DELETE, 0, 0, 0, 1, L.F64, 0, 0.0, 1, 0)
 
 
-def build_messages(batch):
+def build_messages(batch, dead_later=(), fused_away=None):
     """Turns a batch of instructions into a list of work for an interface:
-    ("dag", bytes) and ("call", Instr) in execution order."""
-    items, forced, deleted, producer, dropped = _plan(batch)
+    ("dag", bytes) and ("call", Instr) in execution order. Names of `dead_later` that did not
+    become arrays are added to `fused_away`."""
+    items, forced, deleted, producer, dropped = _plan(batch, dead_later)
     out, nodes = [], []
     node_id = 0
 
@@ -419,24 +421,80 @@ def build_messages(batch):
             nodes.append(_emit_instr(ins, node_id))
         node_id += 1
     flush_nodes()
+    if fused_away is not None:
+        fused_away.update(n for n in dead_later if n in producer and n not in materialised)
     return out
 
 
-def execute(interface):
+def _hold_back_cut(batch, window):
+    """Where an automatic flush stops. A loop of the form
+
+        upd = f(u[...], ...)            # a result with a Python name
+        u[...] = g(u[...], upd)         # consumed by the next statement
+
+    leaves `upd` alive at every statement boundary: its handle goes only when the name is bound
+    again, one iteration later. Flushing right there would turn it into a real array and split
+    the statement in two. So the statements from the one that produced such a recent, still
+    undeleted result onwards stay pending; by the next flush their deletions have arrived, and
+    what is flushed now is planned knowing which of its results die, unread, in the part held
+    back. Returns the number of instructions to send."""
+    n = len(batch)
+    deleted = {ins.name for ins in batch if ins.kind == "delete"}
+    first_live = None
+    for i in range(max(0, n - window), n):
+        ins = batch[i]
+        if ins.kind == "op" and ins.name not in deleted:
+            first_live = i
+            break
+    if first_live is None:
+        return n
+    # the last statement boundary at or before that producer: a position whose predecessor
+    # (deletions aside) is not an elementwise operation
+    cut = first_live
+    while cut > 0:
+        j = cut - 1
+        while j >= 0 and batch[j].kind == "delete":
+            j -= 1
+        if j < 0 or batch[j].kind != "op":
+            break
+        cut -= 1
+    return cut if cut > 0 else n
+
+
+def execute(interface, hold_back=False):
     """Ships everything recorded so far to the executor behind `interface`
-    (charmtyles.core.execute upstream: examples/jacobi3d.py:2,18)."""
+    (charmtyles.core.execute upstream: examples/jacobi3d.py:2,18). An automatic flush
+    (`hold_back`) may keep the most recent statements pending, see _hold_back_cut."""
     if _state.flushing or not _state.pending:
         return
     _state.flushing = True
     try:
         batch = _state.pending
         _state.pending = []
-        for kind, what in build_messages(batch):
+        dead_later, fused_away = (), None
+        if hold_back and _state.auto_flush is not None:
+            cut = _hold_back_cut(batch, _state.auto_flush[1])
+            if cut < len(batch):
+                tail = batch[cut:]
+                batch = batch[:cut]
+                read_in_tail = {o.name for ins in tail if ins.kind != "delete"
+                                for o in ins.operands if isinstance(o, ArrayRef)}
+                read_in_tail |= {ins.name for ins in tail if ins.kind in ("set", "call") and ins.name is not None}
+                produced = {ins.name for ins in batch if ins.kind == "op"}
+                dead_later = {ins.name for ins in tail if ins.kind == "delete" and ins.name in produced
+                              and ins.name not in read_in_tail}
+                fused_away = set()
+                _state.pending = tail
+        for kind, what in build_messages(batch, dead_later, fused_away):
             if kind == "dag":
                 interface.send_dag(_state.epoch, what)
                 _state.epoch += 1
             else:
                 interface.direct_call(what)
+        if fused_away:
+            # their deletions wait in the part held back and have nothing to delete
+            _state.pending = [ins for ins in _state.pending
+                              if not (ins.kind == "delete" and ins.name in fused_away)]
     finally:
         _state.flushing = False
 

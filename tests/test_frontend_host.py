@@ -360,6 +360,29 @@ def test_auto_flush_never_splits_a_stencil_statement(itf):
     assert st["live_arrays"] == 1 and st["compiled"] == 1 and st["cache_hits"] == 9
 
 
+def test_auto_flush_keeps_a_named_intermediate_fused(itf):
+    """upd = f(u); u[...] = g(u, upd) in a loop: `upd` is alive at every statement boundary (its
+    handle goes when the name is bound again). An automatic flush holds the newest statements back
+    instead of turning `upd` into an array; only the explicit flush at the end has to."""
+    n = 96
+    u, f = cnp.zeros((n, n)), cnp.ones((n, n))
+    cnp.execute(itf)
+    itf.trace()
+    cnp.set_auto_flush(itf, 24)
+    for _ in range(20):
+        upd = 0.25 * (u[:-2, 1:-1] + u[2:, 1:-1] + u[1:-1, :-2] + u[1:-1, 2:] + 0.1 * f[1:-1, 1:-1])
+        u[1:-1, 1:-1] = (1.0 / 3.0) * u[1:-1, 1:-1] + (2.0 / 3.0) * upd
+    cnp.execute(itf)
+    log = itf.trace()
+    groups = [ln for ln in log if ln.startswith("group")]
+    assert len(groups) == 21 and sum("inputs=6" in ln for ln in groups) == 19
+    assert sum(ln.startswith("create") for ln in log) == 1      # the last upd only
+    assert not any(ln.startswith("delete") for ln in log)
+    del upd
+    cnp.execute(itf)
+    assert sum(ln.startswith("delete") for ln in itf.trace()) == 1
+
+
 def test_kernel_cache_is_bounded_over_a_long_slab_loop(itf):
     """Each step assigns another slab: another group (same code, other regions). The executor keeps
     a bounded number of them and lets the oldest go."""
