@@ -613,8 +613,12 @@ def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=
     st = evs.times_ms(steps)
     flop = 2.0 * batch * k_in * 4 * d
     gus = 1e3 * float(np.median(g))
+    ceiling = C.c_double()
+    L.check(L.lib.cnh_probe_mfma_f64(8192, C.byref(ceiling)))   # ~1 ms of back-to-back matrix instructions
     out = {"steps": steps, "gemm_us": round(gus, 2), "gemm_tflops": round(flop / gus / 1e6, 2),
            "mfma_frac": round(flop / gus / 1e6 / FP64_MFMA_PEAK_TFLOPS, 4),
+           "mfma_measured_ceiling_tflops": round(ceiling.value, 1),
+           "mfma_frac_of_measured_ceiling": round(flop / gus / 1e6 / ceiling.value, 4) if ceiling.value else None,
            "step_us": round(1e3 * float(np.median(st)), 2), "flop_per_step": flop}
     if keep:
         out["Hout"] = Hout.get().reshape(steps, batch, d)

@@ -355,6 +355,55 @@ int run_f64_batch(int njobs, const cnh_gemm_job* jobs, hipStream_t st) {
 
 } // namespace
 
+namespace {
+// Issue rate of the fp64 matrix instruction with nothing else in the way: 8 wavefronts per CU,
+// four independent accumulators each, operands in registers.
+__global__ __launch_bounds__(512) void mfma_f64_probe(double* out, int iters, double a0, double b0) {
+    v4d acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        acc[i] = (v4d){0.0, 0.0, 0.0, 0.0};
+    const double a = a0 + threadIdx.x, b = b0 - threadIdx.x;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            acc[i] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, acc[i], 0, 0, 0);
+    }
+    double s = 0.0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+    out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+} // namespace
+
+extern "C" int cnh_probe_mfma_f64(int iters, double* tflops) {
+    CNH_CHECK(iters >= 1 && iters <= (1 << 20) && tflops != nullptr, -2, "cnh_probe_mfma_f64: bad argument");
+    int dev = 0;
+    hipDeviceProp_t prop;
+    CNH_HIP(hipGetDevice(&dev));
+    CNH_HIP(hipGetDeviceProperties(&prop, dev));
+    const int blocks = prop.multiProcessorCount, threads = 512;
+    double* out = nullptr;
+    CNH_HIP(hipMalloc((void**)&out, (size_t)blocks * threads * sizeof(double)));
+    hipEvent_t e0, e1;
+    CNH_HIP(hipEventCreate(&e0));
+    CNH_HIP(hipEventCreate(&e1));
+    hipLaunchKernelGGL(mfma_f64_probe, dim3(blocks), dim3(threads), 0, nullptr, out, 64, 1.0, 2.0);   // warm-up
+    CNH_HIP(hipEventRecord(e0, nullptr));
+    hipLaunchKernelGGL(mfma_f64_probe, dim3(blocks), dim3(threads), 0, nullptr, out, iters, 1.0, 2.0);
+    CNH_HIP(hipEventRecord(e1, nullptr));
+    CNH_HIP(hipEventSynchronize(e1));
+    float ms = 0.0f;
+    CNH_HIP(hipEventElapsedTime(&ms, e0, e1));
+    CNH_HIP(hipEventDestroy(e0));
+    CNH_HIP(hipEventDestroy(e1));
+    CNH_HIP(hipFree(out));
+    const double flop = 2048.0 * 4.0 * iters * (double)blocks * (threads / 64);
+    *tflops = ms > 0.0f ? flop / ((double)ms * 1e9) : 0.0;
+    return 0;
+}
+
 extern "C" int cnh_gemm_acc_batch(int dtype, int njobs, const cnh_gemm_job* jobs, cnh_stream s) {
     CNH_CHECK(njobs >= 0 && (njobs == 0 || jobs != nullptr), -2, "cnh_gemm_acc_batch: bad job list");
     for (int i = 0; i < njobs; ++i)

@@ -261,6 +261,10 @@ typedef struct cnh_gemm_job {
     int64_t ldc;
 } cnh_gemm_job;
 int cnh_gemm_acc_batch(int dtype, int njobs, const cnh_gemm_job* jobs, cnh_stream s);
+/* Measurement aid without a counterpart upstream: the rate at which this device issues the fp64
+ * matrix instruction (v_mfma_f64_16x16x4) from registers, 8 wavefronts per CU with four
+ * accumulators each, `iters` rounds; the ceiling the matmatmul figure is set beside. Synchronous. */
+int cnh_probe_mfma_f64(int iters, double* tflops);
 
 /* ---- synthetic inputs generated on the device (no upstream counterpart: upstream has no RNG,
  *      charmnumeric/random.py:4-5, and no bulk upload, charmnumeric.py:863-878) ---- */
