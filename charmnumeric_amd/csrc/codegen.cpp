@@ -492,8 +492,10 @@ struct Tiled {
     int shift; int tile; int off[3]; int shape[3]; int glo[3]; int grid[3];
     const T* const* tiles;
 };
-// cs, w: origin and extents of the tile; bs, bw: the box of it this launch visits (the whole
-// tile, or just the part the assigned region touches when the launch works in place).
+// cs, w: origin and extents of the tile; bs, bw: what of it this launch visits. A ping-pong
+// launch walks the whole tile (bs = 0, bw = w, in elements). An in-place launch (TilesArgs.lattice)
+// walks the points of the assigned region's lattice that fall into the tile: bs = index of the
+// first such point along each dimension, bw = how many.
 struct DTile { i64 blk0; int cs[3]; int w[3]; int nchunks; int pad; int bs[3]; int bw[3]; T* dst; const T* cur; };
 struct LeafReg { int arr; int start[3]; int step[3]; };
 struct TilesArgs {
