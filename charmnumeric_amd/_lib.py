@@ -126,6 +126,7 @@ class Tiled(C.Structure):
         ("grid_lo", C.c_int32 * MAX_ND),
         ("grid", C.c_int32 * MAX_ND),
         ("tiles", C.POINTER(C.c_void_p)),
+        ("pitch", C.c_int64 * MAX_ND),
     ]
 
 

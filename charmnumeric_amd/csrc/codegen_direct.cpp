@@ -191,6 +191,9 @@ struct DirectArgs {
     FDiv grow, gcol;       // workgroups per group along x and y
     FDiv tbz, tby, tbx;    // = tb[0], tb[1], tb[2]
     const T* const* oth[4]; // tile tables of the other arrays read at the element's own position
+    int py, pz;            // elements between rows and between planes inside every tile when the
+                           // tiles are views into one larger row-major block; 0: a tile is
+                           // contiguous over its own extents
 };
 typedef T P2 __attribute__((ext_vector_type(2)));
 typedef int I2 __attribute__((ext_vector_type(2)));
@@ -280,19 +283,27 @@ __device__ __forceinline__ void direct_fast(const DirectArgs& a, const T* s) {
     const int w1 = p.w1, w2 = p.w2;
     const int lx = x0 + 2 * lane;
     const T* const own = a.cur[p.t];
-    const int origin = ((lz0 - DR_H0) * w1 + (ly0 - DR_H1)) * w2;   // window origin, column 0
+    // row and plane strides of this tile and of its x neighbours (their rows are as long as
+    // they are wide unless all tiles are views with common pitches)
+    const int PY = a.py ? a.py : w2, PZ = a.py ? a.pz : w1 * w2;
+    const int oz = lz0 - DR_H0, oy = ly0 - DR_H1;                    // window origin (plane, row)
+    const int origin = oz * PZ + oy * PY;
     const T* const pc = own + origin + lx;
     // where the end lanes find the pair before column x0 and the pair after column x0+127
     const T* lp = own + origin + x0;      // fallback: an address that exists (value unused)
-    int ls = w2;
+    int lpy = PY, lpz = PZ;
     if (x0 >= 2) lp = own + origin + (x0 - 2);
-    else if (p.t2 > 0) { ls = a.tile; lp = a.cur[p.t - 1] + ((lz0 - DR_H0) * w1 + (ly0 - DR_H1)) * ls + (a.tile - 2); }
+    else if (p.t2 > 0) {
+        lpy = a.py ? a.py : a.tile; lpz = a.py ? a.pz : w1 * a.tile;
+        lp = a.cur[p.t - 1] + oz * lpz + oy * lpy + (a.tile - 2);
+    }
     const T* rp = own + origin + (x0 + 126);
-    int rstr = w2;
+    int rpy = PY, rpz = PZ;
     if (x0 + 130 <= w2) rp = own + origin + (x0 + 128);
     else if (p.t2 + 1 < a.grid[2]) {
-        rstr = min(a.tile, a.shape[2] - p.tx0 - a.tile);
-        rp = a.cur[p.t + 1] + ((lz0 - DR_H0) * w1 + (ly0 - DR_H1)) * rstr;
+        const int rw = min(a.tile, a.shape[2] - p.tx0 - a.tile);
+        rpy = a.py ? a.py : rw; rpz = a.py ? a.pz : w1 * rw;
+        rp = a.cur[p.t + 1] + oz * rpz + oy * rpy;
     }
     const bool first = lane == 0, last = lane == 63;
 
@@ -306,26 +317,26 @@ __device__ __forceinline__ void direct_fast(const DirectArgs& a, const T* s) {
 #pragma unroll
         for (int j = 0; j < DR_WY; ++j)
             if (DR_NEED[i][j][0] || DR_NEED[i][j][DR_HK] || DR_NEED[i][j][DR_WK - 1])
-                win[i][j][DR_HK] = *reinterpret_cast<const P2*>(pc + (i * w1 + j) * w2);
+                win[i][j][DR_HK] = *reinterpret_cast<const P2*>(pc + i * PZ + j * PY);
 #pragma unroll
     for (int i = 0; i < DR_WZ; ++i)
 #pragma unroll
         for (int j = 0; j < DR_WY; ++j)
             if (DR_NEED[i][j][0] || DR_NEED[i][j][DR_WK - 1]) {
-                const T* src = pc + (i * w1 + j) * w2;
-                src = first ? lp + (i * w1 + j) * ls : src;
-                src = last ? rp + (i * w1 + j) * rstr : src;
+                const T* src = pc + i * PZ + j * PY;
+                src = first ? lp + i * lpz + j * lpy : src;
+                src = last ? rp + i * rpz + j * rpy : src;
                 beyond[i][j] = *reinterpret_cast<const P2*>(src);
             }
     P2 ov[DR_NOTHA][DR_RZ][DR_RY];
 #pragma unroll
     for (int j = 0; j < DR_NOTH; ++j) {
-        const T* const ot = a.oth[j][p.t] + ((lz0 * w1 + ly0) * w2 + lx);
+        const T* const ot = a.oth[j][p.t] + (lz0 * PZ + ly0 * PY + lx);
 #pragma unroll
         for (int rz = 0; rz < DR_RZ; ++rz)
 #pragma unroll
             for (int ry = 0; ry < DR_RY; ++ry)
-                ov[j][rz][ry] = *reinterpret_cast<const P2*>(ot + (rz * w1 + ry) * w2);
+                ov[j][rz][ry] = *reinterpret_cast<const P2*>(ot + rz * PZ + ry * PY);
     }
 #pragma unroll
     for (int i = 0; i < DR_WZ; ++i)
@@ -365,7 +376,7 @@ __device__ __forceinline__ void direct_fast(const DirectArgs& a, const T* s) {
                 const int gx = p.tx0 + lx + e;
                 res[e] = (gx >= a.rs[2] && gx < a.re[2]) ? o[0] : win[rz + DR_H0][ry + DR_H1][DR_HK][e];
             }
-            P2* out = reinterpret_cast<P2*>(out_tile + (((lz0 + rz) * w1 + (ly0 + ry)) * w2 + lx));
+            P2* out = reinterpret_cast<P2*>(out_tile + ((lz0 + rz) * PZ + (ly0 + ry) * PY + lx));
             if (NTS) __builtin_nontemporal_store(res, out); else *out = res;
         }
 }
@@ -477,7 +488,10 @@ __device__ __forceinline__ void direct_rest(const DirectArgs& a, const T* s, int
                     const T* r0 = xc[k] ? q01 : q00;
                     const T* r1 = xc[k] ? q11 : q10;
                     const T* base = yc[j] ? r1 : r0;
-                    const int off = (cz * yh[j] + yl[j]) * xw[k] + xl[k];
+                    // row and plane strides of the tile read: its own extents, or the common pitches
+                    const int rowlen = a.py ? a.py : xw[k];
+                    const int planelen = a.py ? a.pz : yh[j] * xw[k];
+                    const int off = cz * planelen + yl[j] * rowlen + xl[k];
                     win[i][j][k] = *reinterpret_cast<const P2*>(base + off);
                 }
         }
@@ -485,6 +499,7 @@ __device__ __forceinline__ void direct_rest(const DirectArgs& a, const T* s, int
 
     // ---- the other arrays, at the lane's own rows and planes (clamped into the tile: what a
     // row or plane beyond the tile would read is never used) ----
+    const int OPY = a.py ? a.py : w2, OPZ = a.py ? a.pz : w1 * w2;   // strides of this tile
     P2 ov[DR_NOTHA][DR_RZ][DR_RY];
 #pragma unroll
     for (int j = 0; j < DR_NOTH; ++j) {
@@ -494,7 +509,7 @@ __device__ __forceinline__ void direct_rest(const DirectArgs& a, const T* s, int
 #pragma unroll
             for (int ry = 0; ry < DR_RY; ++ry)
                 ov[j][rz][ry] = *reinterpret_cast<const P2*>(
-                    ot + ((min(lz0 + rz, w0 - 1) * w1 + min(ly0 + ry, w1 - 1)) * w2 + lx));
+                    ot + (min(lz0 + rz, w0 - 1) * OPZ + min(ly0 + ry, w1 - 1) * OPY + lx));
     }
 
     // ---- evaluate and store ----
@@ -530,7 +545,7 @@ __device__ __forceinline__ void direct_rest(const DirectArgs& a, const T* s, int
                         group_eval(l, s, o);
                         res[e] = in_region ? o[0] : win[rz + DR_H0][ry + DR_H1][DR_HK][e];
                     }
-                    P2* out = reinterpret_cast<P2*>(out_tile + ((lz * w1 + ly) * w2 + lx));
+                    P2* out = reinterpret_cast<P2*>(out_tile + (lz * OPZ + ly * OPY + lx));
                     if (NTS) __builtin_nontemporal_store(res, out); else *out = res;
                 }
             }

@@ -491,7 +491,25 @@ int check_tiled(const cnh_tiled* t, int nd, const char* what) {
     }
     for (int64_t i = 0; i < count; ++i)
         CNH_CHECK(t->tiles[i] != nullptr, -4, "%s: tile %lld has a null pointer", what, (long long)i);
+    bool any = false, all = true;
+    for (int d = 0; d < nd; ++d) {
+        any = any || t->pitch[d] != 0;
+        all = all && t->pitch[d] > 0;
+    }
+    CNH_CHECK(!any || (all && t->pitch[nd - 1] == 1), -4,
+              "%s: pitches must be all zero, or positive with 1 along the last dimension", what);
+    for (int d = 0; any && d + 1 < nd; ++d)
+        CNH_CHECK(t->pitch[d] >= t->pitch[d + 1] * std::min(t->tile, t->shape[d + 1]), -4,
+                  "%s: pitch %lld of dim %d is shorter than a tile's extent below it", what,
+                  (long long)t->pitch[d], d);
     return 0;
+}
+
+bool is_pitched(const cnh_tiled* t) {
+    for (int d = 0; d < t->ndims; ++d)
+        if (t->pitch[d] != 0)
+            return true;
+    return false;
 }
 
 int make_tiled_dev(const cnh_tiled* t, hipStream_t st, TiledDev& d) {
@@ -647,8 +665,9 @@ struct DirectArgsDev {
     int32_t tile, shape[3], grid[3], rs[3], re[3], tb[3], sg[3], nblocks, nblocks8, stagger;
     FDivDev per_group, ggrid1, ggrid2, grow, gcol, tbz, tby, tbx;
     const void* oth[kDirectMaxOther];
+    int32_t py, pz;
 };
-static_assert(sizeof(DirectArgsDev) == 16 + 4 * 22 + 12 * 8 + 8 * kDirectMaxOther,
+static_assert(sizeof(DirectArgsDev) == 16 + 4 * 22 + 12 * 8 + 8 * kDirectMaxOther + 8,
               "DirectArgsDev layout must match the generated struct");
 
 int g_stencil_mode = 2; // 0 = general gather, 1 = LDS sliding window, 2 = register window
@@ -731,10 +750,34 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
         if (((uintptr_t)cur->tiles[t] & 15) || ((uintptr_t)dst->tiles[t] & 15))
             return 0;
     }
+    // Pitched tiles (views into one row-major block): every array of the launch has to use the
+    // same pitches, even along the rows, and a pitch of 1 along them.
+    int64_t pitch[3] = {0, 0, 0};
+    bool pitched = false;
+    for (int d = 0; d < nd; ++d)
+        if (cur->pitch[d] != 0)
+            pitched = true;
+    if (pitched) {
+        for (int d = 0; d < nd; ++d) {
+            if (cur->pitch[d] <= 0 || cur->pitch[d] >= (1ll << 31))
+                return 0;
+            pitch[pad + d] = cur->pitch[d];
+        }
+        if (pitch[2] != 1 || pitch[1] % 2 != 0 || (nd == 3 && pitch[0] % 2 != 0))
+            return 0;
+    }
+    auto same_pitch = [&](const cnh_tiled* t) {
+        for (int d = 0; d < nd; ++d)
+            if (t->pitch[d] != cur->pitch[d])
+                return false;
+        return true;
+    };
+    if (!same_pitch(dst) || !same_pitch(arrays[0]))
+        return 0;
     // the other arrays are read at the element's own position: same decomposition, other memory
     for (int j = 0; j < n_other; ++j) {
         const cnh_tiled* o = others[j];
-        if (o == nullptr || o->ndims != cur->ndims || o->tile != cur->tile)
+        if (o == nullptr || o->ndims != cur->ndims || o->tile != cur->tile || !same_pitch(o))
             return 0;
         for (int d = 0; d < nd; ++d)
             if (o->offset[d] != 0 || o->shape[d] != cur->shape[d] || o->grid[d] != cur->grid[d] ||
@@ -812,6 +855,8 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
     for (int j = 0; j < n_other; ++j)
         if (int rc = desc_upload(others[j]->tiles, (size_t)ntiles * sizeof(void*), st, &a.oth[j]))
             return rc;
+    a.py = (int32_t)pitch[1];
+    a.pz = (int32_t)pitch[0];
     const bool nt_stores = volume * 16 >= (128ll << 20); // the written stream is not read back soon
     // Two launches over the same grid: wavefronts that lie inside their tile in y and z take the
     // lean kernel, the other kernel does what is left (all of it when the lean one does not apply).
@@ -1048,6 +1093,12 @@ extern "C" int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* 
             return rc;
         if (handled)
             return 0;
+        // the other kernels address a tile through its own extents
+        bool pitched = is_pitched(dst) || (cur && is_pitched(cur));
+        for (const cnh_tiled* a : arrays)
+            pitched = pitched || is_pitched(a);
+        CNH_CHECK(!pitched, -4, "tiles given as pitched views are taken by the register-window stencil "
+                  "kernels only, and this group or its arrays do not qualify for them");
         if (int rc = try_launch_slide(k, arrays, cur, dst, scal, st, &handled))
             return rc;
         if (handled)

@@ -190,7 +190,8 @@ int cnh_launch_group_batched(cnh_kernel* k, int ndims, int n_parts, int n_in, co
  * reads neighbour tiles directly and writes every tile of the target.
  * A tiled array is described by its decomposition (tile edge, per-dim offset and shape,
  * src/array_region.hpp:293-387) and a table of tile base pointers in row-major tile-grid order;
- * every tile is row-major contiguous over its own local extent (src/backend.hpp:112-200). */
+ * every tile is row-major over its own local extent (src/backend.hpp:112-200), contiguous unless
+ * pitches are given. */
 typedef struct cnh_tiled {
     int32_t ndims;
     int32_t tile;
@@ -199,6 +200,12 @@ typedef struct cnh_tiled {
     int32_t grid_lo[CNH_MAX_ND];   /* first tile index per dim: offset / tile */
     int32_t grid[CNH_MAX_ND];      /* tiles per dim */
     void* const* tiles;            /* host array of device pointers, prod(grid) entries */
+    /* Elements between consecutive indices of each dimension inside a tile. All zero: every tile
+     * is contiguous over its own extents (what a partition's buffer is upstream). Non-zero: the
+     * tiles are views into one larger row-major block and share these pitches (pitch of the last
+     * dimension 1); an executor that holds every partition of an array on one device may store
+     * it that way. */
+    int64_t pitch[CNH_MAX_ND];
 } cnh_tiled;
 /* in[i] describes the array behind leaf use i (regions come from the AST); dst is where the
  * SET_REGION target's new contents are written (all elements of every tile: computed inside the

@@ -33,7 +33,7 @@ def test_struct_layouts_match_header():
     assert L.AstNode.operand_regions.offset == 56
     assert L.AstNode.region.offset == 144
     assert C.sizeof(L.Memref) == 72
-    assert C.sizeof(L.Tiled) == 64
+    assert C.sizeof(L.Tiled) == 88 and L.Tiled.pitch.offset == 64
 
 
 def test_scalar_conversion():

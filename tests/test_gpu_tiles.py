@@ -106,6 +106,66 @@ def test_source_term_at_a_shifted_position_takes_the_general_gather(dev):
     assert np.array_equal(got, want) and not took_direct
 
 
+def _pitched_views(dev, host, tile):
+    """One row-major block on the device and a descriptor whose tiles are views into it."""
+    import ctypes as C
+    nd, n = host.ndim, host.shape[0]
+    block = dev.array(host)
+    g = (n + tile - 1) // tile
+    ptrs = (C.c_void_p * (g ** nd))()
+    for i, idx in enumerate(np.ndindex(*([g] * nd))):
+        off = 0
+        for d in range(nd):
+            off = off * n + idx[d] * tile
+        ptrs[i] = block.ptr + off * 8
+    d = L.Tiled()
+    d.ndims, d.tile = nd, tile
+    for k in range(nd):
+        d.offset[k], d.shape[k], d.grid_lo[k], d.grid[k] = 0, n, 0, g
+        d.pitch[k] = n ** (nd - 1 - k)
+    d.tiles = C.cast(ptrs, C.POINTER(C.c_void_p))
+    return block, ptrs, d
+
+
+@pytest.mark.parametrize("nd,n,tile,source", [(2, 70, 32, False), (2, 256, 128, True), (3, 36, 16, False),
+                                               (3, 64, 32, True)])
+def test_tiles_as_pitched_views_into_one_block(dev, nd, n, tile, source):
+    """The register-window kernels take tiles that are views into one row-major block (common row
+    and plane pitches): an array stored whole, addressed through the same tile grid. Bit for bit
+    against NumPy; other kernels refuse such descriptors."""
+    import ctypes as C
+    rng = np.random.default_rng(n + nd)
+    u0, f0 = rng.standard_normal((n,) * nd), rng.standard_normal((n,) * nd)
+    coef = 0.25 if nd == 2 else 1.0 / 6.0
+    if source:
+        ast = H.ast_poisson2d(n, coef=coef) if nd == 2 else H.ast_poisson3d(n, coef=coef)
+    else:
+        ast = H.ast_jacobi2d(n, coef=coef) if nd == 2 else H.ast_jacobi3d(n, coef=coef)
+    k = H.compile_group(ast, L.F64, nd)
+    ba, _pa, da = _pitched_views(dev, u0, tile)
+    bb, _pb, db = _pitched_views(dev, np.zeros_like(u0), tile)
+    bf, _pf, df = _pitched_views(dev, f0, tile)
+    nleaf = 2 * nd + (1 if source else 0)
+    ref = u0.copy()
+    for _ in range(3):
+        descs = (L.Tiled * nleaf)(*([da] * (2 * nd) + ([df] if source else [])))
+        L.check(L.lib.cnh_launch_group_tiles(k, nleaf, descs, 0, None, 0, C.byref(da), C.byref(db), None))
+        da, db, ba, bb = db, da, bb, ba
+        ref = H.np_poisson(ref, f0, coef) if source else (H.np_jacobi2d(ref, coef) if nd == 2 else H.np_jacobi3d(ref, coef))
+    dev.sync()
+    got = ba.get().reshape(u0.shape)
+    assert np.array_equal(got, ref)
+    assert L.lib.cnh_kernel_variants_loaded(k, b"direct") == 1
+    # the general gather addresses tiles through their own extents: pitched views are refused
+    L.check(L.lib.cnh_set_option(b"stencil_mode", 0))
+    try:
+        descs = (L.Tiled * nleaf)(*([da] * (2 * nd) + ([df] if source else [])))
+        assert L.lib.cnh_launch_group_tiles(k, nleaf, descs, 0, None, 0, C.byref(da), C.byref(db), None) != 0
+    finally:
+        L.check(L.lib.cnh_set_option(b"stencil_mode", 2))
+    dev.free_all()
+
+
 def test_reference_jacobi3d_known_answer(dev, stencil_path):
     """4^3 grid, faces 1.0: every interior point becomes (1/6)*3 = 0.5 (upstream test)."""
     u0 = np.zeros((4, 4, 4))
