@@ -27,10 +27,8 @@ int direct_shape(const GroupProgram& p, const DirectConfig& cfg, DirectShape& sh
         err = "register-window stencil needs a single SET_REGION root";
         return -18;
     }
-    if (p.dtype != CNH_F64 && p.dtype != CNH_I64) {
-        err = "register-window stencil is built for 8-byte elements";
-        return -18;
-    }
+    // A lane works on pairs of elements: 16-byte accesses for 8-byte types, 8-byte accesses for
+    // 4-byte types (half the width per access, still one coalesced run per wavefront).
     const cnh_region& ro = p.out_region[0];
     const int nd = p.ndims, pad = CNH_MAX_ND - nd;
     for (int d = 0; d < nd; ++d)
@@ -205,18 +203,20 @@ __device__ __forceinline__ int floordiv2(int v) { return v >= 0 ? v / 2 : -((-v 
 #ifndef DR_HOST_BUILD
 // Value of the same register in the previous / next lane of the wavefront (whole-wave shift by
 // one lane; the first / last lane keeps its own value and is patched by the caller).
-__device__ __forceinline__ T from_prev_lane(T v) {
-    I2 a = __builtin_bit_cast(I2, v), r;
-    r[0] = __builtin_amdgcn_update_dpp(a[0], a[0], 0x138, 0xf, 0xf, false);
-    r[1] = __builtin_amdgcn_update_dpp(a[1], a[1], 0x138, 0xf, 0xf, false);
-    return __builtin_bit_cast(T, r);
+template <int CTRL, typename V>
+__device__ __forceinline__ V lane_shift(V v) {
+    if constexpr (sizeof(V) == 8) {
+        I2 a = __builtin_bit_cast(I2, v), r;
+        r[0] = __builtin_amdgcn_update_dpp(a[0], a[0], CTRL, 0xf, 0xf, false);
+        r[1] = __builtin_amdgcn_update_dpp(a[1], a[1], CTRL, 0xf, 0xf, false);
+        return __builtin_bit_cast(V, r);
+    } else {
+        const int a = __builtin_bit_cast(int, v);
+        return __builtin_bit_cast(V, __builtin_amdgcn_update_dpp(a, a, CTRL, 0xf, 0xf, false));
+    }
 }
-__device__ __forceinline__ T from_next_lane(T v) {
-    I2 a = __builtin_bit_cast(I2, v), r;
-    r[0] = __builtin_amdgcn_update_dpp(a[0], a[0], 0x130, 0xf, 0xf, false);
-    r[1] = __builtin_amdgcn_update_dpp(a[1], a[1], 0x130, 0xf, 0xf, false);
-    return __builtin_bit_cast(T, r);
-}
+__device__ __forceinline__ T from_prev_lane(T v) { return lane_shift<0x138>(v); }
+__device__ __forceinline__ T from_next_lane(T v) { return lane_shift<0x130>(v); }
 __device__ __forceinline__ int wave_uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 #endif
 

@@ -857,7 +857,7 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
             return rc;
     a.py = (int32_t)pitch[1];
     a.pz = (int32_t)pitch[0];
-    const bool nt_stores = volume * 16 >= (128ll << 20); // the written stream is not read back soon
+    const bool nt_stores = volume * 2 * dtype_size(p.dtype) >= (128ll << 20); // the written stream is not read back soon
     // Two launches over the same grid: wavefronts that lie inside their tile in y and z take the
     // lean kernel, the other kernel does what is left (all of it when the lean one does not apply).
     // measured on MI355X: the lean kernel pays off for rank 2 (tiles much wider than a wavefront

@@ -20,3 +20,11 @@ def test_stencil_variants_build(make, nd, variant):
     src = H.kernel_source(k, variant)
     if variant == "direct":
         assert ("#define DR_NOTH 1" in src) == two_arrays
+
+
+@pytest.mark.parametrize("dt", [L.F32, L.I32, L.I64])
+def test_register_window_kernel_builds_for_other_element_types(dt):
+    k = H.compile_group(H.ast_jacobi2d(64, dtype=dt, coef=2.0), dt, 2)
+    L.check(L.lib.cnh_kernel_build(k, b"direct"))
+    k3 = H.compile_group(H.ast_jacobi3d(32, dtype=dt, coef=2.0), dt, 3)
+    L.check(L.lib.cnh_kernel_build(k3, b"direct"))

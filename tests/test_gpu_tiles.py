@@ -166,6 +166,35 @@ def test_tiles_as_pitched_views_into_one_block(dev, nd, n, tile, source):
     dev.free_all()
 
 
+@pytest.mark.parametrize("nd,n,tile", [(2, 64, 16), (2, 70, 32), (2, 2048 // 8, 128), (3, 36, 16), (3, 128, 128)])
+@pytest.mark.parametrize("dt,npdt", [(L.F32, np.float32), (L.I32, np.int32)])
+def test_four_byte_elements_on_every_stencil_path(dev, stencil_path, nd, n, tile, dt, npdt):
+    """upstream's jacobi2d example is a float32 grid: the register-window kernel works on pairs of
+    4-byte elements as well (8-byte accesses). Bit for bit against NumPy in the same type."""
+    rng = np.random.default_rng(n * nd)
+    if npdt == np.float32:
+        u0 = rng.standard_normal((n,) * nd).astype(npdt)
+        coef = npdt(0.25 if nd == 2 else 1.0 / 6.0)
+    else:
+        u0 = rng.integers(-1000, 1000, (n,) * nd).astype(npdt)
+        coef = npdt(3)
+    ast = H.ast_jacobi2d(n, dtype=dt, coef=float(coef)) if nd == 2 else H.ast_jacobi3d(n, dtype=dt, coef=float(coef))
+    k = H.compile_group(ast, dt, nd)
+    a, b = H.TiledArray(dev, u0, tile), H.TiledArray(dev, np.zeros_like(u0), tile)
+    ref = u0.copy()
+    for _ in range(3):
+        H.launch_tiles(k, [a] * (2 * nd), [], a, b)
+        a, b = b, a
+        with np.errstate(over="ignore"):
+            ref = (H.np_jacobi2d(ref, coef) if nd == 2 else H.np_jacobi3d(ref, coef)).astype(npdt)
+    dev.sync()
+    got = a.gather()
+    took_direct = L.lib.cnh_kernel_variants_loaded(k, b"direct") > 0
+    dev.free_all()
+    assert got.dtype == npdt and np.array_equal(got, ref)
+    assert took_direct == (stencil_path == "direct")
+
+
 def test_reference_jacobi3d_known_answer(dev, stencil_path):
     """4^3 grid, faces 1.0: every interior point becomes (1/6)*3 = 0.5 (upstream test)."""
     u0 = np.zeros((4, 4, 4))
