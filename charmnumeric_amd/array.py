@@ -119,6 +119,20 @@ def parse_key(key, shape):
     """Index expression -> (start, stop, step) per dimension, relative to an object of `shape`."""
     ndims = len(shape)
     start, stop, step = [0] * ndims, [0] * ndims, [1] * ndims
+    if type(key) is tuple and len(key) == ndims:
+        # the common form, one plain slice or integer per dimension: no ellipsis to expand
+        for d in range(ndims):
+            item = key[d]
+            if type(item) is slice and (item.step is None or (type(item.step) is int and item.step > 0)):
+                start[d], stop[d], step[d] = item.indices(shape[d])
+            elif type(item) is int and -shape[d] <= item < shape[d]:
+                i = item + shape[d] if item < 0 else item
+                start[d], stop[d] = i, i + 1
+            else:
+                break
+        else:
+            return tuple(start), tuple(stop), tuple(step)
+        start, stop, step = [0] * ndims, [0] * ndims, [1] * ndims
     for d, item in enumerate(_expand_key(key, ndims)):
         if isinstance(item, slice):
             st = 1 if item.step is None else int(item.step)
