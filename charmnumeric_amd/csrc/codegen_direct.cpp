@@ -387,8 +387,9 @@ __device__ __forceinline__ void direct_fast(const DirectArgs& a, const T* s) {
 // order (the host lists the workgroups on the y and z faces of the tiles); without, all of them.
 template <bool NTS>
 __device__ __forceinline__ void direct_rest(const DirectArgs& a, const T* s, int skip_fast,
-                                            const int* list) {
-    const Place p = locate(a, list ? list[blockIdx.x] : xcd_order(a, (int)blockIdx.x));
+                                            const int* list, int first_block) {
+    const int me = (int)blockIdx.x - first_block;   // this workgroup's number among those doing the rest
+    const Place p = locate(a, list ? list[me] : xcd_order(a, me));
     const int t = p.t, t0 = p.t0, t1 = p.t1, t2 = p.t2;
     const int tz0 = p.tz0, ty0 = p.ty0, tx0 = p.tx0, w0 = p.w0, w1 = p.w1, w2 = p.w2;
     // extents of the next tiles (the previous ones are always full)
@@ -565,12 +566,25 @@ extern "C" __global__ __launch_bounds__(256) void grp_direct_fast_nts(DirectArgs
 extern "C" __global__ __launch_bounds__(256) void grp_direct_rest(DirectArgs a, Scal sc, int skip_fast,
                                                                   const int* list) {
     T s[NSA]; load_scalars(sc, s);
-    direct_rest<false>(a, s, skip_fast, list);
+    direct_rest<false>(a, s, skip_fast, list, 0);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_direct_rest_nts(DirectArgs a, Scal sc, int skip_fast,
                                                                       const int* list) {
     T s[NSA]; load_scalars(sc, s);
-    direct_rest<true>(a, s, skip_fast, list);
+    direct_rest<true>(a, s, skip_fast, list, 0);
+}
+// Both in one launch: the first a.nblocks workgroups do the lean part, the ones after them what
+// the lean part leaves (those on `list`, or all positions again when there is no list). One
+// launch and no gap between the two, and the second part fills the tail of the first.
+extern "C" __global__ __launch_bounds__(256) void grp_direct_both(DirectArgs a, Scal sc, const int* list) {
+    T s[NSA]; load_scalars(sc, s);
+    if ((int)blockIdx.x < a.nblocks) direct_fast<false>(a, s);
+    else direct_rest<false>(a, s, 1, list, a.nblocks);
+}
+extern "C" __global__ __launch_bounds__(256) void grp_direct_both_nts(DirectArgs a, Scal sc, const int* list) {
+    T s[NSA]; load_scalars(sc, s);
+    if ((int)blockIdx.x < a.nblocks) direct_fast<true>(a, s);
+    else direct_rest<true>(a, s, 1, list, a.nblocks);
 }
 )";
     return s.str();

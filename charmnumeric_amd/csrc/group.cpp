@@ -674,6 +674,7 @@ int g_stencil_mode = 2; // 0 = general gather, 1 = LDS sliding window, 2 = regis
 int g_direct_group = 0; // order workgroups by groups of neighbouring tiles (rank 3)
 int g_direct_lean = -1;   // wavefront-level lean kernel: 1 on, 0 off, -1 by rank
 int g_direct_stagger = 0; // concurrent groups start at different offsets of their tiles
+int g_direct_merge = 1;   // lean part and the rest in one launch instead of two
 DirectConfig g_direct_cfg;
 
 // Launches the register-window variant under the same conditions as the sliding window, plus:
@@ -866,17 +867,6 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
     const bool lean = want_lean && sh.tx % 64 == 0 && sh.halo[2] >= 1;
     int skip_fast = lean ? 1 : 0;
     hipFunction_t fn;
-    if (lean) {
-        if (int rc = get_function(k, g_direct_cfg.variant(),
-                                  nt_stores ? "grp_direct_fast_nts" : "grp_direct_fast", &fn))
-            return rc;
-        void* params[] = {&a, const_cast<unsigned char*>(scal.data())};
-        if (int rc = launch(fn, blocks, params, st))
-            return rc;
-    }
-    if (int rc = get_function(k, g_direct_cfg.variant(),
-                              nt_stores ? "grp_direct_rest_nts" : "grp_direct_rest", &fn))
-        return rc;
     // When every workgroup away from the y and z faces of its tile consists of wavefronts the
     // lean kernel takes, the second launch covers the face workgroups only.
     const void* dlist = nullptr;
@@ -924,7 +914,29 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
             rest_blocks = (int64_t)list.size();
         }
     }
+    if (lean && g_direct_merge) {
+        // lean part and the rest in one launch
+        if (int rc = get_function(k, g_direct_cfg.variant(),
+                                  nt_stores ? "grp_direct_both_nts" : "grp_direct_both", &fn))
+            return rc;
+        void* params[] = {&a, const_cast<unsigned char*>(scal.data()), &dlist};
+        if (int rc = launch(fn, blocks + rest_blocks, params, st))
+            return rc;
+        *handled = true;
+        return 0;
+    }
+    if (lean) {
+        if (int rc = get_function(k, g_direct_cfg.variant(),
+                                  nt_stores ? "grp_direct_fast_nts" : "grp_direct_fast", &fn))
+            return rc;
+        void* params[] = {&a, const_cast<unsigned char*>(scal.data())};
+        if (int rc = launch(fn, blocks, params, st))
+            return rc;
+    }
     if (rest_blocks > 0) {
+        if (int rc = get_function(k, g_direct_cfg.variant(),
+                                  nt_stores ? "grp_direct_rest_nts" : "grp_direct_rest", &fn))
+            return rc;
         void* params[] = {&a, const_cast<unsigned char*>(scal.data()), &skip_fast, &dlist};
         if (int rc = launch(fn, rest_blocks, params, st))
             return rc;
@@ -945,6 +957,10 @@ extern "C" int cnh_set_option(const char* name, int value) {
     }
     if (std::strcmp(name, "direct_lean") == 0) {
         g_direct_lean = value;
+        return 0;
+    }
+    if (std::strcmp(name, "direct_merge") == 0) {
+        g_direct_merge = value != 0;
         return 0;
     }
     if (std::strcmp(name, "direct_stagger") == 0) {
