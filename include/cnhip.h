@@ -96,6 +96,7 @@ int cnh_version(void);
  *   "direct_group"   workgroup order for rank 3: 0 (default) tile by tile, 1 groups of G^3 tiles,
  *                    2 rows of tiles along x
  *   "direct_stagger" concurrent groups start at different places of their tiles (default 0)
+ *   "direct_merge"   lean part and the rest in one launch (default 1) or two
  *   "slide_bx/ry/zc/pd", "slide2d_march"  geometry of the sliding-window kernel */
 int cnh_set_option(const char* name, int value);
 
