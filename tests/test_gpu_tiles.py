@@ -195,6 +195,30 @@ def test_four_byte_elements_on_every_stencil_path(dev, stencil_path, nd, n, tile
     assert took_direct == (stencil_path == "direct")
 
 
+def test_bad_pitches_are_refused(dev):
+    import ctypes as C
+    n, tile = 64, 32
+    u0 = np.zeros((n, n))
+    k = H.compile_group(H.ast_jacobi2d(n), L.F64, 2)
+    ba, _pa, da = _pitched_views(dev, u0, tile)
+    bb, _pb, db = _pitched_views(dev, u0, tile)
+
+    def launch(src, dst):
+        descs = (L.Tiled * 4)(*([src] * 4))
+        return L.lib.cnh_launch_group_tiles(k, 4, descs, 0, None, 0, C.byref(src), C.byref(dst), None)
+
+    assert launch(da, db) == 0
+    for bad in ((0, 1), (n, 2), (tile - 2, 1), (-n, 1)):     # one missing, step along rows, too short, negative
+        da.pitch[0], da.pitch[1] = bad
+        assert launch(da, db) != 0, bad
+        assert b"pitch" in L.lib.cnh_last_error()
+    da.pitch[0], da.pitch[1] = n, 1
+    db.pitch[0], db.pitch[1] = 0, 0                          # source pitched, destination not
+    assert launch(da, db) != 0
+    dev.sync()
+    dev.free_all()
+
+
 def test_reference_jacobi3d_known_answer(dev, stencil_path):
     """4^3 grid, faces 1.0: every interior point becomes (1/6)*3 = 0.5 (upstream test)."""
     u0 = np.zeros((4, 4, 4))
