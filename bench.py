@@ -704,6 +704,30 @@ def run_frontend(n, steps, warmup):
         out["cg_rtr_final"] = rtr.get(itf).item()
         del A, b, x, r, p, rtr
 
+        # configuration 1 as examples/simple.py upstream writes it: one fused statement, sum, norm
+        m = 1 << 24
+        xs = cnp.random.uniform((m,), seed=0, stream=0, low=-1.0, high=1.0)
+        ys = cnp.random.uniform((m,), seed=0, stream=1, low=-1.0, high=1.0)
+        ones = cnp.ones((m,))
+
+        def c1(k):
+            for _ in range(k):
+                z = 2.5 * xs - 0.5 * ys + xs * ys
+                s_ = z @ ones
+                nrm2 = z @ z
+            cnp.execute(itf)
+            itf.sync()
+            return s_, nrm2
+
+        c1(3)
+        t0 = time.perf_counter()
+        s_, nrm2 = c1(20)
+        dt = time.perf_counter() - t0
+        out["c1_us_per_pass"] = round(dt / 20 * 1e6, 1)          # elementwise + two reductions
+        out["c1_sum"] = s_.get(itf).item()
+        out["c1_norm"] = float(np.sqrt(nrm2.get(itf).item()))
+        del xs, ys, ones, s_, nrm2
+
         for key, shape, sweeps in (("jacobi2d_8192", (8192, 8192), 100), ("jacobi3d_512", (512, 512, 512), 50)):
             it16 = cnp.CharmNumericInterface(device=0)
             it16.connect(odf=16 if len(shape) == 2 else 64)
