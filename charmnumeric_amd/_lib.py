@@ -117,6 +117,18 @@ class Memref(C.Structure):
         return m
 
 
+class Decomp(C.Structure):
+    """cnx_decomp: ArrayMetadata as the decomposition solver reads and writes it."""
+    _fields_ = [
+        ("name", C.c_int32),
+        ("ndims", C.c_int32),
+        ("shape", C.c_int32 * 3),
+        ("offset", C.c_int32 * 3),
+        ("tile", C.c_int32),
+        ("final", C.c_int32),
+    ]
+
+
 class Tiled(C.Structure):
     _fields_ = [
         ("ndims", C.c_int32),
@@ -240,7 +252,10 @@ _PROTOS.update({
     "cnx_array_info": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int),
                                  C.POINTER(C.c_int), _i32p, _i32p]),
     "cnx_stats": (C.c_int, [C.c_void_p, _i64p]),
+    "cnx_solve_decompositions": (C.c_int, [C.c_int, C.c_int, _i32p, C.c_int, C.POINTER(Decomp),
+                                           C.c_int64, C.c_char_p]),
     "cnx_set_trace": (C.c_int, [C.c_void_p, C.c_int]),
+    "cnx_set_solver": (C.c_int, [C.c_void_p, C.c_int]),
     "cnx_trace": (C.c_int64, [C.c_void_p, C.c_char_p, C.c_size_t]),
 })
 

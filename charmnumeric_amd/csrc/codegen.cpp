@@ -227,6 +227,12 @@ int build_group_program(const cnh_ast* ast, int dtype, int ndims, GroupProgram& 
                 err = "SET_REGION without a usable right-hand side";
                 return -10;
             }
+        } else if (opc == CNH_OP_COPY) {
+            res = lookup(root, 0);
+            if (!res.valid || res.scalar) {
+                err = "COPY needs an array operand";
+                return -12;
+            }
         } else if (opc >= CNH_OP_ADD && opc <= CNH_OP_DIV) {
             Value a = lookup(root, 0), b = lookup(root, 1);
             if (!a.valid || !b.valid) {

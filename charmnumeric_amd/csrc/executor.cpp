@@ -4,6 +4,7 @@
 // all resident on one device. Halo messages do not exist here: kernels read neighbour tiles.
 #include "../../include/cnexec.h"
 #include "common.h"
+#include "decomp.h"
 
 #include <algorithm>
 #include <array>
@@ -69,13 +70,6 @@ int region_count(const cnh_region& r, int d) {
     return (r.stop[d] - r.start[d] + r.step[d] - 1) / r.step[d];
 }
 
-struct DagNode {
-    int id = 0;
-    int fusible = 0;
-    std::vector<cnh_ast_node> nodes;
-    std::vector<int32_t> roots;
-};
-
 // One distributed array: ArrayMetadata (src/backend.hpp:285-288) + the per-chare Array<N,T> buffers
 // (src/backend.hpp:112-200). All tiles of an array are carved from one device allocation, tile t
 // row-major over its own extent; a 1-D array is therefore contiguous as a whole.
@@ -95,12 +89,20 @@ struct XArray {
             lo[d] = 0;
             ext[d] = 1;
         }
+        // tile g of the grid holds the elements i with (i + offset) / tile == g
+        // (src/array_region.hpp:293-387)
         for (int d = ndims - 1; d >= 0; --d) {
-            int ti = (int)(rem % grid[d]);
+            int g = offset[d] / tile + (int)(rem % grid[d]);
             rem /= grid[d];
-            lo[d] = ti * tile;
-            ext[d] = std::min((ti + 1) * tile, (int)shape[d]) - lo[d];
+            lo[d] = std::max(g * tile, (int)offset[d]) - offset[d];
+            ext[d] = std::min((g + 1) * tile, (int)(offset[d] + shape[d])) - offset[d] - lo[d];
         }
+    }
+    bool phased() const {
+        for (int d = 0; d < ndims; ++d)
+            if (offset[d] % tile != 0)
+                return true;
+        return false;
     }
     cnh_tiled tiled(bool use_alt = false) const {
         cnh_tiled t;
@@ -110,7 +112,7 @@ struct XArray {
         for (int d = 0; d < ndims; ++d) {
             t.offset[d] = offset[d];
             t.shape[d] = shape[d];
-            t.grid_lo[d] = 0;
+            t.grid_lo[d] = offset[d] / tile;
             t.grid[d] = grid[d];
         }
         t.tiles = use_alt ? alt_tiles.data() : tiles.data();
@@ -136,6 +138,16 @@ struct cnx_executor {
     int64_t stats[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     bool trace_on = false;
     std::string trace;
+    // Decomposition planning (off: tile rule and offset 0 for every array). When on, every DAG
+    // message is planned as a whole before its first node runs and new arrays are laid out with
+    // the tile and offset the plan gives them.
+    bool solver_on = false;
+    struct Planned {
+        int ndims = 0, tile = 0;
+        int32_t shape[3] = {1, 1, 1}, offset[3] = {0, 0, 0};
+    };
+    std::map<int, Planned> planned;
+    int next_tmp = -(1 << 30); // names of relayout copies
     uintptr_t fake_ptr = 0x1000;
     // Asynchronous mode: DAG messages queue up for a thread of the executor's own, as upstream's
     // frontend hands them to a server and goes on recording. Every other entry point waits for
@@ -234,9 +246,24 @@ int make_array(Ex* ex, int name, int ndims, int dtype, const int32_t* shape, boo
         a.elems *= shape[d];
     }
     a.tile = tile_rule(ex, ndims, shape);
+    auto plan = ex->planned.find(name);
+    if (plan != ex->planned.end()) {
+        const auto& p = plan->second;
+        bool fits = p.ndims == ndims && p.tile > 0 && (p.tile & (p.tile - 1)) == 0;
+        for (int d = 0; d < ndims && fits; ++d)
+            fits = p.shape[d] == shape[d] && p.offset[d] >= 0;
+        if (fits) {
+            a.tile = p.tile;
+            for (int d = 0; d < ndims; ++d)
+                a.offset[d] = p.offset[d];
+        } else {
+            ex->log("plan for " + std::to_string(name) + " does not fit the array; tile rule used");
+        }
+        ex->planned.erase(plan);
+    }
     a.ntiles = 1;
     for (int d = 0; d < ndims; ++d) {
-        a.grid[d] = (a.shape[d] + a.tile - 1) / a.tile;
+        a.grid[d] = (a.offset[d] + a.shape[d] + a.tile - 1) / a.tile - a.offset[d] / a.tile;
         a.ntiles *= a.grid[d];
     }
     const int esz = dtype_size(dtype);
@@ -264,7 +291,9 @@ int make_array(Ex* ex, int name, int ndims, int dtype, const int32_t* shape, boo
         a.tiles.push_back(static_cast<char*>(a.slab) + a.tile_off[t]);
     ex->log("create " + std::to_string(name) + " shape=" + shape_str(a.shape, ndims) + " dtype=" +
             std::to_string(dtype) + " tile=" + std::to_string(a.tile) + " tiles=" +
-            std::to_string(a.ntiles));
+            std::to_string(a.ntiles) + (a.phased() || a.offset[0] || a.offset[1] || a.offset[2]
+                                            ? " offset=" + shape_str(a.offset, ndims)
+                                            : std::string()));
     auto ins = ex->arrays.emplace(name, std::move(a));
     ex->stats[6] = (int64_t)ex->arrays.size();
     if (out)
@@ -304,8 +333,9 @@ int find_array(Ex* ex, int name, XArray** out, const char* what) {
 bool same_decomposition(const XArray& a, const XArray& b) {
     if (a.ndims != b.ndims || a.tile != b.tile)
         return false;
+    // equal extents, tile edges and phases give the same tiles, wherever the grids start
     for (int d = 0; d < a.ndims; ++d)
-        if (a.shape[d] != b.shape[d] || a.offset[d] != b.offset[d])
+        if (a.shape[d] != b.shape[d] || a.offset[d] % a.tile != b.offset[d] % b.tile)
             return false;
     return true;
 }
@@ -727,6 +757,8 @@ int exec_group(Ex* ex, const DagNode& n) {
                 if (j < a.ndims && a.shape[j] == cnt && !(cnt == 1 && left_t > left_a)) {
                     t.shape[d] = a.shape[j];
                     t.grid[d] = a.grid[j];
+                    t.offset[d] = a.offset[j];
+                    t.grid_lo[d] = a.offset[j] / a.tile;
                     ++j;
                 } else {
                     CNH_CHECK(cnt == 1, -35, "node %d: operand %d of shape rank %d does not fit the "
@@ -777,6 +809,50 @@ int leaf_array(Ex* ex, const DagNode& n, const cnh_ast_node& root, int i, XArray
     return 0;
 }
 
+// A copy of `src` laid out with another tile edge and offset, under a name of the executor's
+// own. Products and paired reductions want their operands on matching tile grids; upstream
+// redistributes them by messages (src/executor_matmul.cpp:150-498, src/executor_transfer.cpp),
+// here one gather launch does it. The caller drops the copy when it is done.
+int relayout(Ex* ex, XArray* src, int tile, const int32_t* offset, XArray** out) {
+    const int name = ex->next_tmp--;
+    Ex::Planned p;
+    p.ndims = src->ndims;
+    p.tile = tile;
+    for (int d = 0; d < src->ndims; ++d) {
+        p.shape[d] = src->shape[d];
+        p.offset[d] = offset ? offset[d] : 0;
+    }
+    ex->planned[name] = p;
+    DagNode dn;
+    dn.id = -1;
+    dn.nodes.resize(2);
+    for (auto& a : dn.nodes) {
+        std::memset(&a, 0, sizeof a);
+        a.ndims = src->ndims;
+        a.dtype = src->dtype;
+        a.region.is_global = 1;
+        a.operand_regions[0].is_global = a.operand_regions[1].is_global = 1;
+    }
+    dn.nodes[0].result_name = src->name;
+    dn.nodes[0].opcode = CNH_OP_NOOP;
+    dn.nodes[1].result_name = name;
+    dn.nodes[1].opcode = CNH_OP_COPY;
+    dn.nodes[1].n_operands = 1;
+    dn.roots = {1};
+    ex->log("relayout " + std::to_string(src->name) + " tile=" + std::to_string(tile) + " offset=" +
+            shape_str(p.offset, src->ndims));
+    if (int rc = exec_group(ex, dn))
+        return rc;
+    return find_array(ex, name, out, "relayout");
+}
+
+// The operand itself when its tile grid starts at element 0, else a copy that does.
+int unphased(Ex* ex, XArray* a, XArray** out, bool* is_copy) {
+    *is_copy = a->phased();
+    *out = a;
+    return *is_copy ? relayout(ex, a, a->tile, nullptr, out) : 0;
+}
+
 int new_scalar_array(Ex* ex, int name, int dtype, XArray** out) {
     int32_t one[3] = {1, 1, 1};
     return make_array(ex, name, 1, dtype, one, false, out);
@@ -801,39 +877,56 @@ int exec_reduce(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
             std::to_string(a->ntiles) + " out=" + std::to_string(out->name));
     if (ex->dry)
         return 0;
-    std::vector<const void*> pa(a->tiles.begin(), a->tiles.end()), pb(b->tiles.begin(), b->tiles.end());
+    // 1-D arrays are contiguous as a whole: b is cut where a's tiles end, whatever its own tiles are
+    std::vector<const void*> pa(a->tiles.begin(), a->tiles.end()), pb((size_t)a->ntiles);
+    for (int64_t t = 0; t < a->ntiles; ++t)
+        pb[(size_t)t] = static_cast<const char*>(b->tiles[0]) + a->tile_off[(size_t)t];
     return cnh_dot_tiles(a->dtype, (int)a->ntiles, pa.data(), pb.data(), a->tile_elems.data(),
                          out->tiles[0], ex->stream);
 }
 
 int exec_reduce_ext(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
     XArray *a, *b = nullptr;
+    int b_copy = 0;
     if (int rc = leaf_array(ex, n, root, 0, &a, "reduction"))
         return rc;
     if (root.opcode != kOpSum) {
         if (int rc = leaf_array(ex, n, root, 1, &b, "reduction"))
             return rc;
-        CNH_CHECK(same_decomposition(*a, *b), -30, "reduction: operands differ in shape");
+        bool same_shape = a->ndims == b->ndims;
+        for (int d = 0; d < a->ndims && same_shape; ++d)
+            same_shape = a->shape[d] == b->shape[d];
+        CNH_CHECK(same_shape, -30, "reduction: operands differ in shape");
         CNH_CHECK(a->dtype == CNH_F64 && b->dtype == CNH_F64, -27, "reduction: fp64 operands needed");
+        if (!same_decomposition(*a, *b)) {
+            if (int rc = relayout(ex, b, a->tile, a->offset, &b))
+                return rc;
+            b_copy = b->name;
+        }
     }
     XArray* out;
     if (int rc = new_scalar_array(ex, root.result_name, a->dtype, &out))
         return rc;
     ex->log("reduce_ext op=" + std::to_string(root.opcode) + " tiles=" + std::to_string(a->ntiles) +
             " out=" + std::to_string(out->name));
-    if (ex->dry)
-        return 0;
-    std::vector<const void*> pa(a->tiles.begin(), a->tiles.end()), pb;
-    if (b)
-        pb.assign(b->tiles.begin(), b->tiles.end());
-    if (root.opcode == kOpSum)
-        return cnh_sum_tiles(a->dtype, (int)a->ntiles, pa.data(), a->tile_elems.data(), out->tiles[0],
-                             ex->stream);
-    if (root.opcode == kOpSumsqDiff)
-        return cnh_sumsq_diff_tiles((int)a->ntiles, pa.data(), pb.data(), a->tile_elems.data(),
-                                    out->tiles[0], ex->stream);
-    return cnh_maxabs_diff_tiles((int)a->ntiles, pa.data(), pb.data(), a->tile_elems.data(),
-                                 out->tiles[0], ex->stream);
+    int rc = 0;
+    if (!ex->dry) {
+        std::vector<const void*> pa(a->tiles.begin(), a->tiles.end()), pb;
+        if (b)
+            pb.assign(b->tiles.begin(), b->tiles.end());
+        if (root.opcode == kOpSum)
+            rc = cnh_sum_tiles(a->dtype, (int)a->ntiles, pa.data(), a->tile_elems.data(), out->tiles[0],
+                               ex->stream);
+        else if (root.opcode == kOpSumsqDiff)
+            rc = cnh_sumsq_diff_tiles((int)a->ntiles, pa.data(), pb.data(), a->tile_elems.data(),
+                                      out->tiles[0], ex->stream);
+        else
+            rc = cnh_maxabs_diff_tiles((int)a->ntiles, pa.data(), pb.data(), a->tile_elems.data(),
+                                       out->tiles[0], ex->stream);
+    }
+    if (b_copy)
+        drop_array(ex, b_copy);
+    return rc;
 }
 
 // A 2-D array, or a 3-D array with exactly one extent-1 dimension, seen as a matrix
@@ -893,6 +986,9 @@ int exec_matmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
         return rc;
     if (int rc = leaf_array(ex, n, root, 1, &x, "MATMUL"))
         return rc;
+    bool a_copy = false;
+    if (int rc = unphased(ex, Aa, &Aa, &a_copy))
+        return rc;
     // a 3-D matrix operand with one extent of 1 is the plane that remains
     // (charmnumeric.py:552-563, the K14 case of src/executor_matmul.cpp upstream)
     MatView A;
@@ -907,16 +1003,20 @@ int exec_matmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
         return rc;
     ex->log("matmul A=" + std::to_string(Aa->name) + " tiles=" + std::to_string(Aa->ntiles) + " x=" +
             std::to_string(x->name) + " out=" + std::to_string(y->name));
-    if (ex->dry)
-        return 0;
-    const int gr = Aa->grid[A.rd], gc = Aa->grid[A.cd];
-    std::vector<const void*> pt((size_t)gr * gc);
-    for (int tr = 0; tr < gr; ++tr)
-        for (int tc = 0; tc < gc; ++tc)
-            pt[(size_t)tr * gc + tc] = Aa->tiles[(size_t)A.tile_index(tr, tc)];
-    // 1-D arrays are contiguous: tile 0 is the whole vector.
-    return cnh_gemv_tiles(Aa->dtype, A.rows, A.cols, Aa->tile, pt.data(), x->tiles[0], y->tiles[0],
-                          ex->stream);
+    int rc = 0;
+    if (!ex->dry) {
+        const int gr = Aa->grid[A.rd], gc = Aa->grid[A.cd];
+        std::vector<const void*> pt((size_t)gr * gc);
+        for (int tr = 0; tr < gr; ++tr)
+            for (int tc = 0; tc < gc; ++tc)
+                pt[(size_t)tr * gc + tc] = Aa->tiles[(size_t)A.tile_index(tr, tc)];
+        // 1-D arrays are contiguous: tile 0 is the whole vector.
+        rc = cnh_gemv_tiles(Aa->dtype, A.rows, A.cols, Aa->tile, pt.data(), x->tiles[0], y->tiles[0],
+                            ex->stream);
+    }
+    if (a_copy)
+        drop_array(ex, Aa->name);
+    return rc;
 }
 
 // MATMATMUL: C (zeroed) += A_panel * B_panel for every k-overlapping pair of tiles, k ascending
@@ -926,6 +1026,11 @@ int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
     if (int rc = leaf_array(ex, n, root, 0, &Aa, "MATMATMUL"))
         return rc;
     if (int rc = leaf_array(ex, n, root, 1, &Ba, "MATMATMUL"))
+        return rc;
+    bool a_copy = false, b_copy = false;
+    if (int rc = unphased(ex, Aa, &Aa, &a_copy))
+        return rc;
+    if (int rc = unphased(ex, Ba, &Ba, &b_copy))
         return rc;
     MatView A, B;
     if (int rc = as_matrix(*Aa, &A, "MATMATMUL"))
@@ -979,6 +1084,10 @@ int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
             return rc;
     ex->log("matmatmul A=" + std::to_string(Aa->name) + " B=" + std::to_string(Ba->name) + " out=" +
             std::to_string(Cc->name) + " panel_products=" + std::to_string(calls));
+    if (a_copy)
+        drop_array(ex, Aa->name);
+    if (b_copy)
+        drop_array(ex, Ba->name);
     return 0;
 }
 
@@ -1231,14 +1340,202 @@ int parse_dag(const char* msg, int64_t size, std::vector<DagNode>& out) {
 
 namespace {
 
+// The metadata pass and the solver call of src/dag_group_receive.cpp:222-399: the shape of every
+// array the message will produce, then tile and offset for all of them at once. A result whose
+// shape cannot be told in advance is left to the tile rule when it is created.
+void plan_message(Ex* ex, const std::vector<DagNode>& dag) {
+    std::map<int, DecompMeta> meta;
+    auto existing = [&](int name) {
+        if (meta.count(name))
+            return;
+        auto it = ex->arrays.find(name);
+        if (it == ex->arrays.end())
+            return;
+        DecompMeta m;
+        m.ndims = it->second.ndims;
+        m.tile = it->second.tile;
+        m.final = true;
+        for (int d = 0; d < m.ndims; ++d) {
+            m.shape[d] = it->second.shape[d];
+            m.offset[d] = it->second.offset[d];
+        }
+        meta[name] = m;
+    };
+    auto known = [&](const DagNode& n, const cnh_ast_node& root, int i) -> const DecompMeta* {
+        if (i >= root.n_operands)
+            return nullptr;
+        const cnh_ast_node& op = n.nodes[root.operands[i]];
+        if (op.is_scalar || op.opcode != CNH_OP_NOOP)
+            return nullptr;
+        auto it = meta.find(op.result_name);
+        return it == meta.end() ? nullptr : &it->second;
+    };
+    // rows and columns of a 2-D array or of the plane a 3-D array with an extent of 1 leaves
+    auto matrix_dims = [](const DecompMeta& m, int* rows, int* cols) {
+        if (m.ndims == 2) {
+            *rows = m.shape[0];
+            *cols = m.shape[1];
+            return true;
+        }
+        if (m.ndims != 3)
+            return false;
+        int dropped = -1;
+        for (int d = 0; d < 3 && dropped < 0; ++d)
+            if (m.shape[d] == 1)
+                dropped = d;
+        if (dropped < 0)
+            return false;
+        *rows = m.shape[dropped == 0 ? 1 : 0];
+        *cols = m.shape[dropped == 2 ? 1 : 2];
+        return true;
+    };
+    std::vector<int> fresh;
+    auto result = [&](int name, int nd, const int32_t* shape) {
+        if (nd < 1 || nd > 3 || meta.count(name) || ex->arrays.count(name))
+            return;
+        DecompMeta m;
+        m.ndims = nd;
+        for (int d = 0; d < nd; ++d) {
+            if (shape[d] < 1)
+                return;
+            m.shape[d] = shape[d];
+        }
+        meta[name] = m;
+        fresh.push_back(name);
+    };
+    for (const DagNode& n : dag) {
+        if (n.roots.empty())
+            continue;
+        for (const cnh_ast_node& a : n.nodes)
+            if (!a.is_scalar && a.opcode == CNH_OP_NOOP)
+                existing(a.result_name);
+        const cnh_ast_node& root = n.nodes[n.roots.back()];
+        int32_t shape[3] = {1, 1, 1};
+        switch (root.opcode) {
+        case CNH_OP_CREATE:
+        case CNH_OP_TILE:
+            if (!root.region.is_global && root.region.ndims == root.ndims) {
+                for (int d = 0; d < root.ndims; ++d)
+                    shape[d] = region_count(root.region, d);
+                result(root.result_name, root.ndims, shape);
+            }
+            break;
+        case CNH_OP_REDUCE:
+        case kOpSum:
+        case kOpSumsqDiff:
+        case kOpMaxabsDiff: result(root.result_name, 1, shape); break;
+        case CNH_OP_MATMUL: {
+            int rows, cols;
+            const DecompMeta* A = known(n, root, 0);
+            if (A && matrix_dims(*A, &rows, &cols)) {
+                shape[0] = rows;
+                result(root.result_name, 1, shape);
+            }
+            break;
+        }
+        case CNH_OP_MATMATMUL: {
+            int ar, ac, br, bc;
+            const DecompMeta *A = known(n, root, 0), *B = known(n, root, 1);
+            if (A && B && matrix_dims(*A, &ar, &ac) && matrix_dims(*B, &br, &bc)) {
+                shape[0] = ar;
+                shape[1] = bc;
+                result(root.result_name, 2, shape);
+            }
+            break;
+        }
+        case CNH_OP_DIAG: {
+            const DecompMeta* in = known(n, root, 0);
+            int k = root.n_operands >= 2 && n.nodes[root.operands[1]].is_scalar
+                        ? (int)n.nodes[root.operands[1]].scalar
+                        : 0;
+            if (in && in->ndims == 1) {
+                shape[0] = shape[1] = in->shape[0] + std::abs(k);
+                result(root.result_name, 2, shape);
+            } else if (in && in->ndims == 2) {
+                shape[0] = k >= 0 ? std::min(in->shape[0], in->shape[1] - k)
+                                  : std::min(in->shape[0] + k, in->shape[1]);
+                result(root.result_name, 1, shape);
+            }
+            break;
+        }
+        case CNH_OP_ADD:
+        case CNH_OP_SUB:
+        case CNH_OP_MUL:
+        case CNH_OP_DIV:
+        case CNH_OP_TANH:
+        case CNH_OP_EXP:
+        case CNH_OP_COPY: {
+            // as result_shape(): the root's own region, else the first region an array is read
+            // through, else the shape of an operand array
+            bool found = false;
+            if (!root.region.is_global && root.region.ndims == root.ndims) {
+                for (int d = 0; d < root.ndims; ++d)
+                    shape[d] = region_count(root.region, d);
+                found = true;
+            }
+            for (size_t ai = 0; ai < n.nodes.size() && !found; ++ai) {
+                const cnh_ast_node& a = n.nodes[ai];
+                if (a.is_scalar || a.opcode == CNH_OP_NOOP)
+                    continue;
+                bool settled = false;
+                for (int i = 0; i < a.n_operands && !settled; ++i) {
+                    const cnh_ast_node& op = n.nodes[a.operands[i]];
+                    if (op.is_scalar || op.opcode != CNH_OP_NOOP)
+                        continue;
+                    if (a.has_operand_region[i] && !a.operand_regions[i].is_global) {
+                        for (int d = 0; d < op.ndims && d < 3; ++d)
+                            shape[d] = region_count(a.operand_regions[i], d);
+                        found = settled = true;
+                        break;
+                    }
+                    auto it = meta.find(op.result_name);
+                    if (it == meta.end())
+                        continue;
+                    for (int d = 0; d < 3; ++d)
+                        shape[d] = d < it->second.ndims ? it->second.shape[d] : 1;
+                    found = true;
+                    settled = !op.is_broadcast;
+                }
+                if (settled)
+                    break;
+            }
+            if (found)
+                result(root.result_name, root.ndims, shape);
+            break;
+        }
+        default: break;
+        }
+    }
+    if (fresh.empty())
+        return;
+    solve_decompositions(meta, dag, ex->odf, ex->num_pes, ex->min_tile);
+    for (int name : fresh) {
+        const DecompMeta& m = meta[name];
+        Ex::Planned p;
+        p.ndims = m.ndims;
+        p.tile = m.tile;
+        for (int d = 0; d < m.ndims; ++d) {
+            p.shape[d] = m.shape[d];
+            p.offset[d] = m.offset[d];
+        }
+        ex->planned[name] = p;
+        ex->log("plan " + std::to_string(name) + " tile=" + std::to_string(p.tile) + " offset=" +
+                shape_str(p.offset, p.ndims));
+    }
+}
+
 int run_message(Ex* ex, const char* msg, int64_t size) {
     std::vector<DagNode> dag;
     if (int rc = parse_dag(msg, size, dag))
         return rc;
+    if (ex->solver_on)
+        plan_message(ex, dag);
+    int rc = 0;
     for (const DagNode& n : dag)
-        if (int rc = exec_node(ex, n))
-            return rc;
-    return 0;
+        if ((rc = exec_node(ex, n)) != 0)
+            break;
+    ex->planned.clear();
+    return rc;
 }
 
 void worker_loop(Ex* ex) {
@@ -1352,6 +1649,14 @@ int cnx_set_min_tile(cnx_executor* ex, int ndims, int min_tile) {
     CNH_CHECK(ndims >= 1 && ndims <= 3 && min_tile >= 1, -2, "bad minimum tile %d for rank %d",
               min_tile, ndims);
     ex->min_tile[ndims] = min_tile;
+    return 0;
+}
+
+int cnx_set_solver(cnx_executor* ex, int on) {
+    CNH_CHECK(ex != nullptr, -2, "null executor");
+    if (int rc = drain(ex))
+        return rc;
+    ex->solver_on = on != 0;
     return 0;
 }
 
@@ -1583,6 +1888,47 @@ int cnx_stats(cnx_executor* ex, int64_t out[8]) {
     ex->stats[6] = (int64_t)ex->arrays.size();
     for (int i = 0; i < 8; ++i)
         out[i] = ex->stats[i];
+    return 0;
+}
+
+int cnx_solve_decompositions(int odf, int num_pes, const int32_t min_tile[3], int n_arrays,
+                             cnx_decomp* arrays, int64_t size, const char* msg) {
+    CNH_CHECK(min_tile != nullptr && n_arrays >= 0 && (n_arrays == 0 || arrays != nullptr), -2,
+              "null argument");
+    CNH_CHECK(size == 0 || msg != nullptr, -2, "null DAG message");
+    std::vector<DagNode> dag;
+    if (size > 0)
+        if (int rc = parse_dag(msg, size, dag))
+            return rc;
+    std::map<int, DecompMeta> meta;
+    for (int i = 0; i < n_arrays; ++i) {
+        const cnx_decomp& a = arrays[i];
+        CNH_CHECK(a.ndims >= 1 && a.ndims <= 3 && a.tile >= 0, -20, "array %d: rank %d, tile %d", a.name,
+                  a.ndims, a.tile);
+        CNH_CHECK(meta.find(a.name) == meta.end(), -21, "array %d listed twice", a.name);
+        DecompMeta m;
+        m.ndims = a.ndims;
+        m.tile = a.tile;
+        m.final = a.final != 0;
+        for (int d = 0; d < 3; ++d) {
+            CNH_CHECK(d >= a.ndims || a.shape[d] >= 1, -20, "array %d: extent %d in dim %d", a.name,
+                      a.shape[d], d);
+            m.shape[d] = d < a.ndims ? a.shape[d] : 0;
+            m.offset[d] = d < a.ndims ? a.offset[d] : 0;
+        }
+        meta[a.name] = m;
+    }
+    const int mt[4] = {1, min_tile[0], min_tile[1], min_tile[2]};
+    for (int r = 1; r <= 3; ++r)
+        CNH_CHECK(mt[r] >= 1 && mt[r] <= (1 << 30), -20, "minimum tile %d for rank %d", mt[r], r);
+    solve_decompositions(meta, dag, odf, num_pes, mt);
+    for (int i = 0; i < n_arrays; ++i) {
+        const DecompMeta& m = meta[arrays[i].name];
+        arrays[i].tile = m.tile;
+        arrays[i].final = 1;
+        for (int d = 0; d < 3; ++d)
+            arrays[i].offset[d] = m.offset[d];
+    }
     return 0;
 }
 

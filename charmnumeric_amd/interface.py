@@ -4,6 +4,7 @@ its C ABI (include/cnexec.h). `connect` keeps upstream's signature; address and 
 from __future__ import annotations
 
 import ctypes as C
+import os
 
 import numpy as np
 
@@ -21,6 +22,18 @@ class CharmNumericInterface:
         self._ex = None
         self._min_tiles = {}
         self._pipeline = False
+        self._solver = os.environ.get("CHARMNUMERIC_SOLVER", "0") not in ("", "0")
+
+    # -- decomposition planning ----------------------------------------------------------------
+    def set_solver(self, on=True):
+        """Plan tile edges and offsets of new arrays per DAG message the way upstream's server
+        does (src/decomposition_solver.hpp upstream) instead of the tile rule with offset 0.
+        Values never depend on it. Off by default (environment variable CHARMNUMERIC_SOLVER=1
+        turns it on for every interface): with all tiles on one device, lined-up tiles save no
+        traffic."""
+        self._solver = bool(on)
+        if self._ex is not None:
+            L.check(L.lib.cnx_set_solver(self._ex, 1 if on else 0))
 
     # -- pipelining --------------------------------------------------------------------------
     def set_pipeline(self, on=True):
@@ -45,6 +58,8 @@ class CharmNumericInterface:
         self.odf = int(odf)
         for nd, t in self._min_tiles.items():
             L.check(L.lib.cnx_set_min_tile(self._ex, nd, t))
+        if self._solver:
+            L.check(L.lib.cnx_set_solver(self._ex, 1))
         if self._pipeline:
             L.check(L.lib.cnx_set_async(self._ex, 1))
         return self

@@ -74,6 +74,16 @@ int cnx_destroy(cnx_executor* ex);
 /* Overrides CT_MIN_TILE_1D/2D/3D (src/backend.hpp:10-18; the upstream tests build with 64). */
 int cnx_set_min_tile(cnx_executor* ex, int ndims, int min_tile);
 
+/* Decomposition planning, off by default. Off: every array gets the tile rule and offset 0 (on
+ * one device kernels read neighbouring tiles in place, so lining tiles up saves no traffic).
+ * On: each DAG message is planned as a whole before it runs, as upstream does
+ * (src/dag_group_receive.cpp:222-399 -> cnx_solve_decompositions below), and the arrays it
+ * produces are laid out with the planned tile edge and offset; values do not depend on it.
+ * Statements over arrays whose tiles line up run per tile; all others go through the general
+ * gather; a product or paired reduction whose operand's tile grid does not start at element 0
+ * works on a copy that does. */
+int cnx_set_solver(cnx_executor* ex, int on);
+
 /* ArrayDAGGroup::receive_dag(int epoch, int size, char msg[size]) (src/backend.ci:15,
  * src/dag_group_receive.cpp:190-575) followed by the partitions' run(): executes every node of the
  * DAG in order. Returns when all work is queued on the executor's stream (not when it finished). */
@@ -115,6 +125,27 @@ int cnx_stats(cnx_executor* ex, int64_t out[8]);
  * and logs it but allocates and launches nothing (host-logic tests on machines without a GPU). */
 int cnx_set_trace(cnx_executor* ex, int on);
 int64_t cnx_trace(cnx_executor* ex, char* buf, size_t cap);
+
+/* ArrayDAGGroup::compute_decompositions (src/dag_group_runtime.cpp:42-44 over
+ * src/decomposition_solver.hpp:94-1714): tile edge and offset of every array a DAG message
+ * produces. arrays[] is ArrayMetadata (src/backend.hpp:264-288) for the arrays the message names:
+ * existing ones with final = 1 (their tile and offset are kept), results with final = 0 and their
+ * shape filled in (tile 0 = the rank's minimum). On return every entry carries its tile and
+ * absolute offset and final = 1. min_tile = CT_MIN_TILE_1D/2D/3D. msg is a DAG message as above
+ * (size 0: tile rule only); a leaf may name a temporary root of the same DAG node
+ * (is_temp = 1), which stands for that root's expression. Pure host code: no device is touched.
+ * Upstream iterates hash maps; where its answer depends on their order (which of several
+ * already-placed arrays a component is rooted at) this function takes ascending array names. */
+typedef struct cnx_decomp {
+    int32_t name;
+    int32_t ndims;
+    int32_t shape[3];
+    int32_t offset[3];
+    int32_t tile;
+    int32_t final;
+} cnx_decomp;
+int cnx_solve_decompositions(int odf, int num_pes, const int32_t min_tile[3], int n_arrays,
+                             cnx_decomp* arrays, int64_t size, const char* msg);
 
 #ifdef __cplusplus
 }
