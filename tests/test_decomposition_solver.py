@@ -276,3 +276,79 @@ def test_tree_phases_minimise_the_weighted_misalignment():
     got = total[out[B][1][0] % T, out[Cc][1][0] % T, out[D][1][0] % T]
     assert got == total.min(), (out, int(got), int(total.min()))
     assert all(out[n] == (T, (fixed[n],)) for n in fixed)
+
+
+# ---- the executor under the solver (dry mode: decisions only) ----
+
+@pytest.fixture
+def planned_itf():
+    import charmnumeric_amd as cnp
+    cnp.reset()
+    it = cnp.CharmNumericInterface(device=-1)
+    it.connect(odf=4)
+    for nd in (1, 2, 3):
+        it.set_min_tile(nd, 64)
+    it.set_solver(True)
+    it.set_trace()
+    yield it
+    cnp.reset()
+    it.close()
+
+
+def test_executor_lays_results_out_as_planned(planned_itf):
+    import charmnumeric_amd as cnp
+    it = planned_itf
+    a = cnp.zeros(512)
+    b = a[150:350] + 1.0
+    c = b + b
+    d = a[2:202:2] * 2.0
+    lazy.execute(it)
+    log = it.trace()
+    assert it.array_info(a.name)["offset"] == (0,)
+    assert it.array_info(b.name) == {"ndims": 1, "dtype": L.F64, "tile": 64, "shape": (200,),
+                                     "offset": (150,)}
+    assert it.array_info(c.name)["offset"] == (150,)
+    assert it.array_info(d.name)["tile"] == 64 and it.array_info(d.name)["offset"] == (1,)
+    assert any(ln.startswith(f"plan {b.name} tile=64 offset=(150)") for ln in log)
+    # b and c are cut alike: per-tile launch; b against a needs the gather
+    kinds = {ln.split("out=")[1].split()[0]: ln for ln in log if ln.startswith("group")}
+    assert "path=dense" in kinds[str(c.name)]
+    assert "path=tiles" in kinds[str(b.name)]
+
+
+def test_executor_without_the_solver_keeps_offset_zero(planned_itf):
+    import charmnumeric_amd as cnp
+    it = planned_itf
+    it.set_solver(False)
+    a = cnp.zeros(512)
+    b = a[150:350] + 1.0
+    lazy.execute(it)
+    assert it.array_info(b.name)["offset"] == (0,)
+    assert not any(ln.startswith("plan") for ln in it.trace())
+
+
+def test_products_of_offset_operands_are_copied_first(planned_itf):
+    import charmnumeric_amd as cnp
+    it = planned_itf
+    A = cnp.zeros((200, 180))
+    v = cnp.zeros(400)
+    B = A[3:163, 5:165] * 1.0
+    x = v[11:171] * 1.0
+    lazy.execute(it)                       # B and x are placed before any product names them
+    assert it.array_info(B.name)["offset"] == (3, 5)
+    assert it.array_info(x.name)["offset"] == (11,)
+    it.trace()
+    y = B @ x
+    C2 = B @ B
+    lazy.execute(it)
+    log = it.trace()
+    assert sum(ln.startswith("relayout") for ln in log) == 3
+    assert it.array_info(y.name)["offset"] == (0,) and it.array_info(C2.name)["offset"] == (0, 0)
+    # the copies are gone again
+    assert it.stats()["live_arrays"] == 6
+    # within one message the solver keeps product operands at 0 itself (no copy needed)
+    B2 = A[3:163, 5:165] * 2.0
+    y2 = B2 @ x
+    lazy.execute(it)
+    assert it.array_info(B2.name)["offset"] == (0, 0)
+    assert sum(ln.startswith("relayout") for ln in it.trace()) == 0
