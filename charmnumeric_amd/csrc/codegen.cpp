@@ -502,7 +502,9 @@ struct Tiled {
 // launch walks the whole tile (bs = 0, bw = w, in elements). An in-place launch (TilesArgs.lattice)
 // walks the points of the assigned region's lattice that fall into the tile: bs = index of the
 // first such point along each dimension, bw = how many.
-struct DTile { i64 blk0; int cs[3]; int w[3]; int nchunks; int pad; int bs[3]; int bw[3]; T* dst; const T* cur; };
+// rsh: a workgroup covers 2^rsh consecutive rows with 256 >> rsh lanes each (short rows, e.g. the
+// 128-wide tiles of rank-3 arrays, would otherwise leave most lanes idle); 0 = one row.
+struct DTile { i64 blk0; int cs[3]; int w[3]; int nchunks; int rsh; int bs[3]; int bw[3]; T* dst; const T* cur; };
 struct LeafReg { int arr; int start[3]; int step[3]; };
 struct TilesArgs {
     int out_off[3];
@@ -524,16 +526,28 @@ __device__ __forceinline__ T tiled_read(const Tiled& a, int g0, int g1, int g2) 
     return base[((i64)(g0 - lo0) * w1 + (g1 - lo1)) * w2 + (g2 - lo2)];
 }
 
-extern "C" __global__ __launch_bounds__(256) void grp_tiles(const Tiled* arrs, const DTile* dts,
-                                                            int ndt, TilesArgs ta, Scal sc) {
-    T s[NSA]; load_scalars(sc, s);
+template <bool ROWS>
+__device__ __forceinline__ void tiles_run(const Tiled* arrs, const DTile* dts, int ndt,
+                                          const TilesArgs& ta, const T* s) {
     const int k = find_seg(dts, ndt, (i64)blockIdx.x);
     const DTile& dt = dts[k];
     const i64 blk = (i64)blockIdx.x - dt.blk0;
-    const i64 outer = blk / dt.nchunks;
-    const int chunk = (int)(blk - outer * dt.nchunks);
-    const int i1 = dt.bs[1] + (int)(outer % dt.bw[1]);
-    const int i0 = dt.bs[0] + (int)(outer / dt.bw[1]);
+    const i64 group = blk / dt.nchunks;
+    const int chunk = (int)(blk - group * dt.nchunks);
+    int lanes = 256, lx = (int)threadIdx.x, i0, i1;
+    if (ROWS) {
+        // rows differ between the lanes of a workgroup: 32-bit arithmetic per lane
+        lanes = 256 >> dt.rsh;
+        lx = (int)threadIdx.x & (lanes - 1);
+        const unsigned row = ((unsigned)group << dt.rsh) + ((unsigned)threadIdx.x >> (8 - dt.rsh));
+        if (row >= (unsigned)dt.bw[0] * (unsigned)dt.bw[1]) return;
+        const unsigned q = row / (unsigned)dt.bw[1];
+        i0 = dt.bs[0] + (int)q;
+        i1 = dt.bs[1] + (int)(row - q * (unsigned)dt.bw[1]);
+    } else {
+        i1 = dt.bs[1] + (int)(group % dt.bw[1]);
+        i0 = dt.bs[0] + (int)(group / dt.bw[1]);
+    }
     // in place: (i0, i1, i2) are indices into the region's lattice; otherwise tile coordinates
     const int a0 = ta.lattice ? ta.rs[0] + i0 * ta.rst[0] : dt.cs[0] + i0 - ta.out_off[0];
     const int a1 = ta.lattice ? ta.rs[1] + i1 * ta.rst[1] : dt.cs[1] + i1 - ta.out_off[1];
@@ -546,7 +560,7 @@ extern "C" __global__ __launch_bounds__(256) void grp_tiles(const Tiled* arrs, c
     const int k1 = ta.lattice ? i1 : (a1 - ta.rs[1]) / ta.rst[1];
 #pragma unroll
     for (int u = 0; u < TL_PER_THREAD; ++u) {
-        const int j2 = chunk * (256 * TL_PER_THREAD) + u * 256 + (int)threadIdx.x;
+        const int j2 = chunk * (lanes * TL_PER_THREAD) + u * lanes + lx;
         if (j2 >= dt.bw[2]) continue;
         const int i2 = dt.bs[2] + j2;
         const int a2 = ta.lattice ? ta.rs[2] + i2 * ta.rst[2] : dt.cs[2] + i2 - ta.out_off[2];
@@ -571,6 +585,17 @@ extern "C" __global__ __launch_bounds__(256) void grp_tiles(const Tiled* arrs, c
             dt.dst[di] = dt.cur[di];
         }
     }
+}
+
+extern "C" __global__ __launch_bounds__(256) void grp_tiles(const Tiled* arrs, const DTile* dts,
+                                                            int ndt, TilesArgs ta, Scal sc) {
+    T s[NSA]; load_scalars(sc, s);
+    tiles_run<false>(arrs, dts, ndt, ta, s);
+}
+extern "C" __global__ __launch_bounds__(256) void grp_tiles_rows(const Tiled* arrs, const DTile* dts,
+                                                                 int ndt, TilesArgs ta, Scal sc) {
+    T s[NSA]; load_scalars(sc, s);
+    tiles_run<true>(arrs, dts, ndt, ta, s);
 }
 )";
     return s.str();

@@ -466,7 +466,7 @@ static_assert(sizeof(TiledDev) == 64, "TiledDev layout must match the generated 
 
 struct DTileDev {
     int64_t blk0;
-    int32_t cs[3], w[3], nchunks, pad;
+    int32_t cs[3], w[3], nchunks, rsh;
     int32_t bs[3], bw[3];
     void* dst;
     const void* cur;
@@ -673,6 +673,7 @@ static_assert(sizeof(DirectArgsDev) == 16 + 4 * 22 + 12 * 8 + 8 * kDirectMaxOthe
 int g_stencil_mode = 2; // 0 = general gather, 1 = LDS sliding window, 2 = register window
 int g_direct_group = 0; // order workgroups by groups of neighbouring tiles (rank 3)
 int g_direct_lean = -1;   // wavefront-level lean kernel: 1 on, 0 off, -1 by rank
+int g_tiles_rows = 1;     // general gather: short rows share a workgroup
 int g_direct_stagger = 0; // concurrent groups start at different offsets of their tiles
 int g_direct_merge = 1;   // lean part and the rest in one launch instead of two
 DirectConfig g_direct_cfg;
@@ -959,6 +960,10 @@ extern "C" int cnh_set_option(const char* name, int value) {
         g_direct_lean = value;
         return 0;
     }
+    if (std::strcmp(name, "tiles_rows") == 0) {
+        g_tiles_rows = value != 0;
+        return 0;
+    }
     if (std::strcmp(name, "direct_merge") == 0) {
         g_direct_merge = value != 0;
         return 0;
@@ -1127,7 +1132,7 @@ extern "C" int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* 
         ntiles *= dst->grid[d];
     std::vector<DTileDev> dts;
     int64_t blocks = 0;
-    bool lattice = false;
+    bool lattice = false, any_rows = false;
     for (int64_t t = 0; t < ntiles; ++t) {
         int ti[3] = {0, 0, 0};
         int64_t rem = t;
@@ -1183,9 +1188,20 @@ extern "C" int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* 
         }
         if (empty)
             continue;
-        dt.nchunks = (dt.bw[2] + 1023) / 1024;
+        // Four elements per lane along the last dimension. A row shorter than 1024 elements
+        // shares its workgroup with the rows after it: 2^rsh rows of 256 >> rsh lanes each.
+        const int64_t rows = (int64_t)dt.bw[0] * dt.bw[1];
+        int lanes = 16;
+        while (lanes < 256 && lanes * 4 < dt.bw[2])
+            lanes *= 2;
+        dt.rsh = 0;
+        while (g_tiles_rows && (256 >> dt.rsh) > lanes && (1 << dt.rsh) < rows)
+            dt.rsh++;
+        lanes = 256 >> dt.rsh;
+        dt.nchunks = (dt.bw[2] + lanes * 4 - 1) / (lanes * 4);
         dt.blk0 = blocks;
-        blocks += (int64_t)dt.bw[0] * dt.bw[1] * dt.nchunks;
+        blocks += ((rows + (1 << dt.rsh) - 1) >> dt.rsh) * dt.nchunks;
+        any_rows = any_rows || dt.rsh > 0;
         dts.push_back(dt);
     }
     if (dts.empty())
@@ -1203,7 +1219,7 @@ extern "C" int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* 
     if (int rc = desc_upload(dts.data(), dts.size() * sizeof(DTileDev), st, &d_dts))
         return rc;
     hipFunction_t fn;
-    if (int rc = get_function(k, "tiles", "grp_tiles", &fn))
+    if (int rc = get_function(k, "tiles", any_rows ? "grp_tiles_rows" : "grp_tiles", &fn))
         return rc;
     int ndt = (int)dts.size();
     void* params[] = {&d_arrs, &d_dts, &ndt, targs.data(), scal.data()};

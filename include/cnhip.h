@@ -97,6 +97,7 @@ int cnh_version(void);
  *                    2 rows of tiles along x
  *   "direct_stagger" concurrent groups start at different places of their tiles (default 0)
  *   "direct_merge"   lean part and the rest in one launch (default 1) or two
+ *   "tiles_rows"     general gather: rows shorter than 1024 elements share a workgroup (default 1)
  *   "slide_bx/ry/zc/pd", "slide2d_march"  geometry of the sliding-window kernel */
 int cnh_set_option(const char* name, int value);
 
