@@ -227,6 +227,7 @@ _PROTOS = {
     "cnh_gemm_acc": (C.c_int, [C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_int64,
                                C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p]),
     "cnh_gemm_acc_batch": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmJob), C.c_void_p]),
+    "cnh_gemm_batch": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmJob), C.c_int, C.c_void_p]),
     "cnh_probe_mfma_f64": (C.c_int, [C.c_int, C.POINTER(C.c_double)]),
     "cnh_fill_uniform": (C.c_int, [C.c_void_p, C.c_int64, C.c_uint64, C.c_uint64, C.c_uint64,
                                    C.c_double, C.c_double, C.c_void_p]),

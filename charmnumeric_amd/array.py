@@ -288,8 +288,11 @@ class _ArrayLike:
         return _matvec(self, vec)
 
     def copy(self):
-        out = empty(self.shape, dtype=self.dtype)
-        out[...] = self
+        """A new array holding these values: one COPY node (upstream's opcode -5), which fuses like
+        any element-wise operation, instead of a zero-filled array assigned afterwards."""
+        out = Array(self.shape, self.dtype)
+        lazy.record(lazy.Instr("op", name=out.name, opcode=L.OP_COPY, operands=[self._ref()],
+                               shape=self.shape, dtype=out.wire_dtype()))
         return out
 
     def fill(self, value):

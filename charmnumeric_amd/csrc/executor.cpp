@@ -1040,8 +1040,11 @@ int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
     CNH_CHECK(A.cols == B.rows, -32, "MATMATMUL: (%d,%d) @ (%d,%d)", A.rows, A.cols, B.rows, B.cols);
     CNH_CHECK(Aa->dtype == Ba->dtype, -27, "MATMATMUL: operand dtypes %d and %d", Aa->dtype, Ba->dtype);
     int32_t shape[3] = {A.rows, B.cols, 1};
+    // fp64 products overwrite their result (every C element belongs to exactly one chain), so the
+    // new array needs no zero-fill; the other types accumulate into zeros as upstream does
+    const bool f64 = Aa->dtype == CNH_F64;
     XArray* Cc;
-    if (int rc = make_array(ex, root.result_name, 2, Aa->dtype, shape, true, &Cc))
+    if (int rc = make_array(ex, root.result_name, 2, Aa->dtype, shape, !f64, &Cc))
         return rc;
     const int esz = dtype_size(Aa->dtype);
     const int TA = Aa->tile, TB = Ba->tile;
@@ -1079,9 +1082,10 @@ int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
                     }
                 }
         }
-    if (!ex->dry)
-        if (int rc = cnh_gemm_acc_batch(Aa->dtype, (int)jobs.size(), jobs.data(), ex->stream))
+    if (!ex->dry) {
+        if (int rc = cnh_gemm_batch(Aa->dtype, (int)jobs.size(), jobs.data(), f64 ? 1 : 0, ex->stream))
             return rc;
+    }
     ex->log("matmatmul A=" + std::to_string(Aa->name) + " B=" + std::to_string(Ba->name) + " out=" +
             std::to_string(Cc->name) + " panel_products=" + std::to_string(calls));
     if (a_copy)

@@ -56,7 +56,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_f64_mfma(const GemmChain* _
                                                               int nchains,
                                                               const GemmSeg* __restrict__ segs,
                                                               int nblocks, GemmChain only_chain,
-                                                              GemmSeg only_seg) {
+                                                              GemmSeg only_seg, int overwrite) {
     constexpr int NT = WM * WN * 64;
     constexpr int BM = WM * TM * 16, BN = WN * TN * 16;
     constexpr int APT = BM * BKT / NT, BPT = BN * BKT / NT;   // doubles staged per lane
@@ -209,7 +209,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_f64_mfma(const GemmChain* _
                 const int row = m0 + (wm * TM + i) * 16 + r * 4 + lk;
                 if (FULL || (row < M && col < N)) {
                     double* c = ch.C + (int64_t)row * ch.ldc + col;
-                    *c = *c + acc[i][j][r];
+                    *c = overwrite ? acc[i][j][r] : *c + acc[i][j][r];
                 }
             }
         }
@@ -281,7 +281,7 @@ int check_job(const cnh_gemm_job& j) {
 
 template <int WM, int WN, int TM, int TN, int BKT>
 int launch_chains(std::vector<GemmChain>& chains, const std::vector<GemmSeg>& segs, bool full,
-                  hipStream_t st) {
+                  int overwrite, hipStream_t st) {
     constexpr int BM = WM * TM * 16, BN = WN * TN * 16;
     int64_t blocks = 0;
     for (GemmChain& c : chains) {
@@ -308,15 +308,15 @@ int launch_chains(std::vector<GemmChain>& chains, const std::vector<GemmSeg>& se
     const int nch = (int)chains.size(), nb = (int)blocks;
     if (full)
         hipLaunchKernelGGL((gemm_f64_mfma<WM, WN, TM, TN, BKT, true>), dim3((unsigned)blocks),
-                           dim3(WM * WN * 64), 0, st, dch, nch, dsg, nb, chains[0], segs[0]);
+                           dim3(WM * WN * 64), 0, st, dch, nch, dsg, nb, chains[0], segs[0], overwrite);
     else
         hipLaunchKernelGGL((gemm_f64_mfma<WM, WN, TM, TN, BKT, false>), dim3((unsigned)blocks),
-                           dim3(WM * WN * 64), 0, st, dch, nch, dsg, nb, chains[0], segs[0]);
+                           dim3(WM * WN * 64), 0, st, dch, nch, dsg, nb, chains[0], segs[0], overwrite);
     CNH_HIP(hipGetLastError());
     return 0;
 }
 
-int run_f64_batch(int njobs, const cnh_gemm_job* jobs, hipStream_t st) {
+int run_f64_batch(int njobs, const cnh_gemm_job* jobs, int overwrite, hipStream_t st) {
     std::vector<GemmChain> chains;
     std::vector<std::vector<GemmSeg>> per_chain;
     bool full = true;
@@ -349,8 +349,8 @@ int run_f64_batch(int njobs, const cnh_gemm_job* jobs, hipStream_t st) {
     // 64x64 tiles of four wavefronts when that gives every CU several workgroups; smaller grids
     // take 8 wavefronts per workgroup so that a CU with one workgroup still has two per SIMD.
     if (blocks64 >= 1024)
-        return launch_chains<2, 2, 2, 2, 16>(chains, segs, full, st);
-    return launch_chains<2, 4, 2, 1, 16>(chains, segs, full, st);
+        return launch_chains<2, 2, 2, 2, 16>(chains, segs, full, overwrite, st);
+    return launch_chains<2, 4, 2, 1, 16>(chains, segs, full, overwrite, st);
 }
 
 } // namespace
@@ -404,14 +404,15 @@ extern "C" int cnh_probe_mfma_f64(int iters, double* tflops) {
     return 0;
 }
 
-extern "C" int cnh_gemm_acc_batch(int dtype, int njobs, const cnh_gemm_job* jobs, cnh_stream s) {
-    CNH_CHECK(njobs >= 0 && (njobs == 0 || jobs != nullptr), -2, "cnh_gemm_acc_batch: bad job list");
+extern "C" int cnh_gemm_batch(int dtype, int njobs, const cnh_gemm_job* jobs, int overwrite, cnh_stream s) {
+    CNH_CHECK(njobs >= 0 && (njobs == 0 || jobs != nullptr), -2, "cnh_gemm_batch: bad job list");
+    CNH_CHECK(!overwrite || dtype == CNH_F64, -3, "cnh_gemm_batch: overwriting products are fp64 only");
     for (int i = 0; i < njobs; ++i)
         if (int rc = check_job(jobs[i]))
             return rc;
     hipStream_t st = as_stream(s);
     if (dtype == CNH_F64)
-        return run_f64_batch(njobs, jobs, st);
+        return run_f64_batch(njobs, jobs, overwrite ? 1 : 0, st);
     for (int i = 0; i < njobs; ++i) {
         const cnh_gemm_job& j = jobs[i];
         if (j.M == 0 || j.N == 0 || j.K == 0)
@@ -427,6 +428,10 @@ extern "C" int cnh_gemm_acc_batch(int dtype, int njobs, const cnh_gemm_job* jobs
             return rc;
     }
     return 0;
+}
+
+extern "C" int cnh_gemm_acc_batch(int dtype, int njobs, const cnh_gemm_job* jobs, cnh_stream s) {
+    return cnh_gemm_batch(dtype, njobs, jobs, 0, s);
 }
 
 extern "C" int cnh_gemm_acc(int dtype, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda,

@@ -26,7 +26,7 @@ from . import _lib as L
 OP_DELETE, OP_SUM, OP_SUMSQ_DIFF, OP_MAXABS_DIFF = 100, 101, 102, 103
 DAG_MAGIC = 0x47444E43
 
-_ELEMENTWISE = {L.OP_ADD, L.OP_SUB, L.OP_MUL, L.OP_DIV, L.OP_TANH, L.OP_EXP}
+_ELEMENTWISE = {L.OP_ADD, L.OP_SUB, L.OP_MUL, L.OP_DIV, L.OP_TANH, L.OP_EXP, L.OP_COPY}
 
 
 class ArrayRef:

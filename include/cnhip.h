@@ -270,6 +270,11 @@ typedef struct cnh_gemm_job {
     int64_t ldc;
 } cnh_gemm_job;
 int cnh_gemm_acc_batch(int dtype, int njobs, const cnh_gemm_job* jobs, cnh_stream s);
+/* The same with a choice of what happens to C. overwrite = 0: C += the products of its chain
+ * (cnh_gemm_acc_batch). overwrite = 1 (fp64 only): C = the products of its chain; what C held is
+ * neither read nor kept, so a freshly allocated result needs no zero-fill
+ * (upstream zero-fills result_data and accumulates, src/executor_matmatmul.cpp:105-160). */
+int cnh_gemm_batch(int dtype, int njobs, const cnh_gemm_job* jobs, int overwrite, cnh_stream s);
 /* Measurement aid without a counterpart upstream: the rate at which this device issues the fp64
  * matrix instruction (v_mfma_f64_16x16x4) from registers, 8 wavefronts per CU with four
  * accumulators each, `iters` rounds; the ceiling the matmatmul figure is set beside. Synchronous. */

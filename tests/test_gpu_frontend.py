@@ -137,6 +137,21 @@ def test_matmatmul_of_ones_and_against_numpy(small_tiles):
     assert np.all(np.abs(got - ha @ hb) <= bound)
 
 
+def test_matmatmul_result_is_not_zero_filled_first(itf):
+    """fp64 products overwrite their result: a buffer taken back from the free list with other
+    contents must not leak into it."""
+    rng = np.random.default_rng(8)
+    ha, hb = rng.standard_normal((96, 200)), rng.standard_normal((200, 80))
+    A, B = cnp.array(ha), cnp.array(hb)
+    junk = cnp.array(np.full((96, 80), np.nan))
+    junk.get(itf)
+    del junk                               # its buffer (same size as the product's) is free again
+    got = (A @ B).get(itf)
+    want = (ha.astype(np.longdouble) @ hb.astype(np.longdouble)).astype(np.float64)
+    assert np.all(np.abs(got - want) <= 1e-12 * (np.abs(ha) @ np.abs(hb)))
+    assert itf.stats()["reuses"] >= 1
+
+
 def test_cg_example_against_the_closed_form(small_tiles):
     """A = N*I + 1 1^T, b = 1..N: x = (b - sum(b)/(2N))/N; CG reaches it in two iterations
     (examples/cg.py upstream)."""

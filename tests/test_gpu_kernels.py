@@ -325,6 +325,28 @@ def test_gemm_batch_is_the_jobs_one_after_another(dev, orc, dt, npdt, aligned):
     dev.free_all()
 
 
+@pytest.mark.parametrize("M,N,K", [(128, 192, 160), (100, 150, 77)])
+def test_gemm_batch_overwrites_without_reading(dev, M, N, K):
+    """overwrite = 1: C becomes the product whatever it held (NaNs included), two K pieces per block."""
+    rng = np.random.default_rng(M + K)
+    A, B = rng.standard_normal((M, K)), rng.standard_normal((K, N))
+    C0 = np.full((M, N), np.nan)
+    dA, dB, dC = dev.array(A), dev.array(B), dev.array(C0)
+    kc = K // 2
+    arr = (L.GemmJob * 2)()
+    for j, (k0, k1) in zip(arr, ((0, kc), (kc, K))):
+        j.M, j.N, j.K, j.A, j.lda, j.B, j.ldb, j.C, j.ldc = M, N, k1 - k0, dA.ptr + 8 * k0, K, dB.ptr + 8 * k0 * N, N, dC.ptr, N
+    L.check(L.lib.cnh_gemm_batch(L.F64, 2, arr, 1, None))
+    got = dC.get()
+    bound = REL * (np.abs(A) @ np.abs(B))
+    assert np.all(np.abs(got - (A.astype(np.longdouble) @ B.astype(np.longdouble)).astype(np.float64)) <= bound)
+    # accumulate on top of it
+    L.check(L.lib.cnh_gemm_batch(L.F64, 2, arr, 0, None))
+    assert np.all(np.abs(dC.get() - 2 * got) <= 2 * bound)
+    assert L.lib.cnh_gemm_batch(L.I64, 2, arr, 1, None) != 0          # overwriting is fp64 only
+    dev.free_all()
+
+
 def test_descriptor_table_outlives_the_stream_it_was_uploaded_on(dev):
     """The same job list (hence the same descriptor table) on a stream, then on a second stream after
     the first was destroyed: the cached table must be usable without touching the dead stream."""
