@@ -352,3 +352,49 @@ def test_products_of_offset_operands_are_copied_first(planned_itf):
     lazy.execute(it)
     assert it.array_info(B2.name)["offset"] == (0, 0)
     assert sum(ln.startswith("relayout") for ln in it.trace()) == 0
+
+
+# ---- assignments across ranks (src/decomposition_solver.hpp:333-353,728-786) ----
+
+def test_plane_assigned_into_a_slab_lines_up_with_it():
+    """X[3, 10:110, 20:120] = Y with Y a fresh 2-D array: Y's rows meet X's dimension 1 and its
+    columns dimension 2, so Y wants offset (10, 20); the lower-rank array also takes the tile of
+    the higher-rank one."""
+    X, Y, SET = 1, 2, 9
+    w = lazy._NodeWriter()
+    w.op(SET, L.OP_SET_REGION, False, 3, L.F64, [w.leaf(Ref(X, 3)), w.leaf(Ref(Y, 2))], [None, None],
+         region=reg([3, 10, 20], [4, 110, 120]))
+    out = solve({X: ((8, 200, 200), (0, 0, 0), 64, True), Y: ((100, 100), (0, 0), 128, False)},
+                message(w), odf=64)
+    assert out[Y] == (64, (10, 20))
+    assert out[X] == (64, (0, 0, 0))
+
+
+def test_slab_read_into_a_plane_lines_up_with_it():
+    """The other way round: P[5:105, 7:107] = Z with Z a fresh (1, 100, 100) array read whole:
+    Z's dimensions 1 and 2 meet P's 0 and 1; dimension 0 (extent 1) meets nothing and stays 0."""
+    P, Z, SET = 1, 2, 9
+    w = lazy._NodeWriter()
+    w.op(SET, L.OP_SET_REGION, False, 2, L.F64, [w.leaf(Ref(P, 2)), w.leaf(Ref(Z, 3))], [None, None],
+         region=reg([5, 7], [105, 107]))
+    out = solve({P: ((300, 300), (0, 0), 64, True), Z: ((1, 100, 100), (0, 0, 0), 0, False)},
+                message(w), odf=64)
+    assert out[Z][0] == 64
+    assert out[Z][1] == (0, 5, 7)
+
+
+def test_cycle_with_conflicting_wishes_follows_the_heavier_one():
+    """t reads a[8:108] and b[40:140]; b[8:108] = t closes a cycle through t, so t is settled from
+    the wishes of its producers and its consumer one by one, weighted by volume: phase 8 is asked
+    for by a (256 elements) and by the assignment (t's own 100), phase 40 by b (256 or 4096)."""
+    a, b, t = 1, 2, 3
+    for nb, want in ((256, 8), (4096, 40)):
+        w = lazy._NodeWriter()
+        w.op(t, L.OP_ADD, False, 1, L.F64, [w.leaf(Ref(a, 1)), w.leaf(Ref(b, 1))],
+             [reg([8], [108]), reg([40], [140])])
+        w2 = lazy._NodeWriter()
+        w2.op(20, L.OP_SET_REGION, False, 1, L.F64, [w2.leaf(Ref(b, 1)), w2.leaf(Ref(t, 1))], [None, None],
+              region=reg([8], [108]))
+        out = solve({a: ((256,), (0,), 64, True), b: ((nb,), (0,), 64, True), t: ((100,), (0,), 0, False)},
+                    message(w, w2), odf=64)
+        assert out[t][0] == 64 and out[t][1][0] % 64 == want, (nb, out[t])
