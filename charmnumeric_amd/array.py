@@ -225,6 +225,21 @@ class _ArrayLike:
         inner = parse_key(key, self.shape)
         return ArrayView(self._base(), compose(self._region(), inner))
 
+    def get_region(self, region, **kwargs):
+        """The view of `region` = (start, stop, step) per dimension, in this object's own
+        coordinates, or any object with those three attributes (upstream's ArrayRegion,
+        charmnumeric.py:690-695,789-794 upstream; its keyword arguments are derived here)."""
+        if not isinstance(region, tuple):
+            region = (region.start, region.stop, region.step)
+        start, stop, step = (tuple(int(v) for v in part) for part in region)
+        if not len(start) == len(stop) == len(step) == self.ndims:
+            raise IndexError(f"region of rank {len(start)} on an array of rank {self.ndims}")
+        for d in range(self.ndims):
+            if step[d] < 1 or start[d] < 0 or stop[d] > self.shape[d] or stop[d] <= start[d]:
+                raise IndexError(f"region [{start[d]}:{stop[d]}:{step[d]}] does not fit extent "
+                                 f"{self.shape[d]} in dimension {d}")
+        return ArrayView(self._base(), compose(self._region(), (start, stop, step)))
+
     def __setitem__(self, key, rhs):
         inner = parse_key(key, self.shape)
         region = compose(self._region(), inner)

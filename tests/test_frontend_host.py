@@ -487,3 +487,20 @@ def test_frontend_refuses_like_upstream():
     assert cnp.arange(5).shape == (5,) and cnp.eye(3).shape == (3, 3)
     assert cnp.zeros_like(a).shape == (4, 5) and cnp.empty_like(a, dtype=np.int32).dtype == np.int32
     cnp.reset()
+
+
+def test_get_region_is_the_slice_of_the_same_bounds(itf):
+    a = cnp.zeros((40, 30))
+    v = a.get_region(((2, 5), (38, 29), (3, 2)))
+    w = a[2:38:3, 5:29:2]
+    assert v.shape == w.shape == (12, 12) and v.region == w.region
+    inner = v.get_region(((1, 0), (5, 12), (2, 1)))             # a view of a view composes
+    assert inner.region == w[1:5:2, :].region
+
+    class R:
+        start, stop, step = (0, 0), (40, 30), (1, 1)
+    assert a.get_region(R()).shape == (40, 30)
+    for bad in (((0,), (40,), (1,)), ((0, 0), (41, 30), (1, 1)), ((0, 0), (40, 30), (0, 1)),
+                ((5, 0), (5, 30), (1, 1))):
+        with pytest.raises(IndexError):
+            a.get_region(bad)
