@@ -284,3 +284,22 @@ def test_multigrid_v_cycles(itf, auto_flush):
     finally:
         cnp.reset()
     assert errs[1] < 0.2 * errs[0] < 0.1
+
+
+# ---- 1-D Jacobi through a named temporary (examples/jacobi.py upstream) ----
+
+@pytest.mark.parametrize("n,dtype", [(128, np.float32), (1000, np.float64)])
+def test_jacobi_1d_with_a_temporary(itf, n, dtype):
+    u = cnp.zeros((n,), dtype=dtype)
+    hu = np.zeros((n,), dtype=dtype)
+    u[0] = 1.0
+    u[-1] = 1.0
+    hu[0] = hu[-1] = 1.0
+    for _ in range(3):
+        t = 0.5 * (u[:-2] + u[2:])
+        u[1:-1] = t
+        ht = 0.5 * (hu[:-2] + hu[2:])
+        hu[1:-1] = ht
+    got = u.get(itf)
+    assert got.dtype == dtype and np.array_equal(got, hu)
+    assert got[1] == 0.625 and got[2] == 0.25 and got[3] == 0.125   # three sweeps from the ends
