@@ -1,9 +1,15 @@
-"""Seeded synthetic inputs generated on the device (upstream has no generator:
-charmnumeric/random.py:4-5 upstream only raises)."""
+"""Seeded synthetic inputs generated on the device. Upstream has no generator: its `randn`
+(charmnumeric/random.py:4-5 upstream) returns a new float32 array of the asked shape, which the
+server zero-fills; that function is kept with that behaviour."""
 from __future__ import annotations
 
 from . import lazy
 from .array import create_array
+
+
+def randn(*args):
+    """As upstream's: a new float32 array of shape `args` (zero-filled, no random numbers)."""
+    return create_array(tuple(args), dtype="float32")
 
 
 def uniform(shape, seed, stream=0, low=0.0, high=1.0):

@@ -504,3 +504,8 @@ def test_get_region_is_the_slice_of_the_same_bounds(itf):
                 ((5, 0), (5, 30), (1, 1))):
         with pytest.raises(IndexError):
             a.get_region(bad)
+
+
+def test_randn_is_upstreams_placeholder(itf):
+    r = cnp.random.randn(3, 5)
+    assert r.shape == (3, 5) and r.dtype == np.float32
