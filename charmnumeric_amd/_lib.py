@@ -117,6 +117,10 @@ class Memref(C.Structure):
         return m
 
 
+class GemvPanel(C.Structure):
+    _fields_ = [("base", C.c_void_p), ("ld", C.c_int64), ("ncols", C.c_int64), ("xoff", C.c_int64)]
+
+
 class Decomp(C.Structure):
     """cnx_decomp: ArrayMetadata as the decomposition solver reads and writes it."""
     _fields_ = [
@@ -227,6 +231,8 @@ _PROTOS = {
     "cnh_gemm_acc": (C.c_int, [C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_int64,
                                C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p]),
     "cnh_gemm_acc_batch": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmJob), C.c_void_p]),
+    "cnh_gemv_panels": (C.c_int, [C.c_int, C.c_int64, C.c_int32, C.c_int64, C.c_int64, C.c_int64,
+                                  C.POINTER(GemvPanel), C.c_void_p, C.c_void_p, C.c_void_p]),
     "cnh_gemm_batch": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmJob), C.c_int, C.c_void_p]),
     "cnh_probe_mfma_f64": (C.c_int, [C.c_int, C.POINTER(C.c_double)]),
     "cnh_fill_uniform": (C.c_int, [C.c_void_p, C.c_int64, C.c_uint64, C.c_uint64, C.c_uint64,

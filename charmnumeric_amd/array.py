@@ -452,8 +452,26 @@ def _whole(x):
     return x
 
 
+def _window_ok(x):
+    """Products and dots read unit-step slices in place (upstream sends the view's region with the
+    node, charmnumeric.py:595-616 upstream); anything else is copied out first. A 3-D operand
+    gives up its first extent-1 dimension, and the rows of what remains must be contiguous."""
+    if not isinstance(x, ArrayView) or _is_whole(x.region, x.base.shape):
+        return True
+    if any(st != 1 for st in x.region[2]):
+        return False
+    if x.ndims == 3:
+        ones = [d for d in range(3) if x.shape[d] == 1]
+        return bool(ones) and (ones[0] != 2 or x.base.shape[2] == 1)
+    return True
+
+
+_WINDOWED = (L.OP_REDUCE, L.OP_MATMUL, L.OP_MATMATMUL)
+
+
 def nonfusible(opcode, operands, shape, dtype):
-    operands = [_whole(o) if isinstance(o, _ArrayLike) else o for o in operands]
+    operands = [_whole(o) if isinstance(o, _ArrayLike) and not (opcode in _WINDOWED and _window_ok(o))
+                else o for o in operands]
     out = Array(shape, dtype)
     lazy.record(lazy.Instr("nonfusible", name=out.name, opcode=opcode,
                            operands=[o._ref() if isinstance(o, _ArrayLike) else o for o in operands],

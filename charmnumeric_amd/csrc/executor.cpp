@@ -809,6 +809,35 @@ int leaf_array(Ex* ex, const DagNode& n, const cnh_ast_node& root, int i, XArray
     return 0;
 }
 
+// Operand i of a product or dot with the window it is read through (the whole array when the node
+// carries no region): unit steps only, inside the array.
+int leaf_window(Ex* ex, const DagNode& n, const cnh_ast_node& root, int i, XArray** out,
+                cnh_region* win, const char* what) {
+    CNH_CHECK(root.n_operands > i, -28, "%s: operand %d missing", what, i);
+    const cnh_ast_node& op = n.nodes[root.operands[i]];
+    CNH_CHECK(!op.is_scalar && op.opcode == CNH_OP_NOOP, -28, "%s: operand %d is not an array", what, i);
+    if (int rc = find_array(ex, op.result_name, out, what))
+        return rc;
+    const XArray& a = **out;
+    std::memset(win, 0, sizeof *win);
+    win->ndims = a.ndims;
+    const bool whole = !root.has_operand_region[i] || root.operand_regions[i].is_global;
+    CNH_CHECK(whole || root.operand_regions[i].ndims == a.ndims, -29,
+              "%s: region of rank %d on array %d of rank %d", what, root.operand_regions[i].ndims,
+              a.name, a.ndims);
+    for (int d = 0; d < a.ndims; ++d) {
+        win->start[d] = whole ? 0 : root.operand_regions[i].start[d];
+        win->stop[d] = whole ? a.shape[d] : root.operand_regions[i].stop[d];
+        win->step[d] = whole ? 1 : root.operand_regions[i].step[d];
+        CNH_CHECK(win->step[d] == 1, -29, "%s on a strided slice of array %d is not supported", what,
+                  a.name);
+        CNH_CHECK(win->start[d] >= 0 && win->stop[d] > win->start[d] && win->stop[d] <= a.shape[d], -29,
+                  "%s: window [%d:%d] leaves extent %d of array %d in dim %d", what, win->start[d],
+                  win->stop[d], a.shape[d], a.name, d);
+    }
+    return 0;
+}
+
 // A copy of `src` laid out with another tile edge and offset, under a name of the executor's
 // own. Products and paired reductions want their operands on matching tile grids; upstream
 // redistributes them by messages (src/executor_matmul.cpp:150-498, src/executor_transfer.cpp),
@@ -862,27 +891,41 @@ int new_scalar_array(Ex* ex, int name, int dtype, XArray** out) {
 // (src/executor_reduce.cpp:8-119, src/executor_reducer.cpp:11-57, src/partition_comm.cpp:69-111).
 int exec_reduce(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
     XArray *a, *b;
-    if (int rc = leaf_array(ex, n, root, 0, &a, "REDUCE"))
+    cnh_region wa, wb;
+    if (int rc = leaf_window(ex, n, root, 0, &a, &wa, "REDUCE"))
         return rc;
-    if (int rc = leaf_array(ex, n, root, 1, &b, "REDUCE"))
+    if (int rc = leaf_window(ex, n, root, 1, &b, &wb, "REDUCE"))
         return rc;
     CNH_CHECK(a->ndims == 1 && b->ndims == 1, -30, "REDUCE needs 1-D operands");
-    CNH_CHECK(a->shape[0] == b->shape[0], -30, "REDUCE: lengths %d and %d", a->shape[0], b->shape[0]);
+    const int64_t len = wa.stop[0] - wa.start[0];
+    CNH_CHECK(len == wb.stop[0] - wb.start[0], -30, "REDUCE: lengths %lld and %d", (long long)len,
+              wb.stop[0] - wb.start[0]);
     CNH_CHECK(a->dtype == b->dtype, -27, "REDUCE: operand dtypes %d and %d", a->dtype, b->dtype);
     XArray* out;
     if (int rc = new_scalar_array(ex, root.result_name, a->dtype, &out))
         return rc;
-    // make_array inserted into the map: re-find the operands (std::map keeps references valid).
+    // 1-D arrays are contiguous as a whole. The partial sums follow the first operand's tiles
+    // (the pieces of them its window covers); the second operand is cut at the same places.
+    const int esz = dtype_size(a->dtype);
+    std::vector<const void*> pa, pb;
+    std::vector<int64_t> cnt;
+    for (int64_t t = 0; t < a->ntiles; ++t) {
+        int32_t lo[3], ext[3];
+        a->tile_extent(t, lo, ext);
+        const int64_t first = std::max<int64_t>(lo[0], wa.start[0]);
+        const int64_t last = std::min<int64_t>(lo[0] + ext[0], wa.stop[0]);
+        if (last <= first)
+            continue;
+        pa.push_back(static_cast<const char*>(a->tiles[0]) + first * esz);
+        pb.push_back(static_cast<const char*>(b->tiles[0]) + (first - wa.start[0] + wb.start[0]) * esz);
+        cnt.push_back(last - first);
+    }
     ex->log("reduce " + std::to_string(a->name) + "." + std::to_string(b->name) + " tiles=" +
-            std::to_string(a->ntiles) + " out=" + std::to_string(out->name));
+            std::to_string(pa.size()) + " out=" + std::to_string(out->name));
     if (ex->dry)
         return 0;
-    // 1-D arrays are contiguous as a whole: b is cut where a's tiles end, whatever its own tiles are
-    std::vector<const void*> pa(a->tiles.begin(), a->tiles.end()), pb((size_t)a->ntiles);
-    for (int64_t t = 0; t < a->ntiles; ++t)
-        pb[(size_t)t] = static_cast<const char*>(b->tiles[0]) + a->tile_off[(size_t)t];
-    return cnh_dot_tiles(a->dtype, (int)a->ntiles, pa.data(), pb.data(), a->tile_elems.data(),
-                         out->tiles[0], ex->stream);
+    return cnh_dot_tiles(a->dtype, (int)pa.size(), pa.data(), pb.data(), cnt.data(), out->tiles[0],
+                         ex->stream);
 }
 
 int exec_reduce_ext(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
@@ -929,52 +972,68 @@ int exec_reduce_ext(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
     return rc;
 }
 
-// A 2-D array, or a 3-D array with exactly one extent-1 dimension, seen as a matrix
-// (the dimension-dropped operands of charmnumeric.py:510-519, src/executor_matmatmul.cpp:485-813).
+// A window of a 2-D array, or of a 3-D array where the window has an extent of 1 along one
+// dimension (the first such is dropped), seen as a matrix in the array's own coordinates
+// (the sliced and dimension-dropped operands of charmnumeric.py:510-519,536-578 upstream,
+// src/executor_matmatmul.cpp:485-813). The array's tile grid starts at element 0 (unphased()).
 struct MatView {
     const XArray* a = nullptr;
-    int rd = 0, cd = 1; // which array dimensions are rows and columns
+    int rd = 0, cd = 1, dd = -1; // row, column and dropped dimension of the array
+    int r0 = 0, c0 = 0, plane = 0; // where the window starts; index along the dropped dimension
     int rows = 0, cols = 0;
-    int tile_index(int tr, int tc) const {
+    // Pointer to array element (row ar, column ac) of the plane, the row stride of the tile that
+    // holds it, and that tile's bounds [rlo, rhi) x [clo, chi) in array coordinates.
+    const char* at(int ar, int ac, int64_t* ld, int* rlo, int* rhi, int* clo, int* chi) const {
         int idx[3] = {0, 0, 0};
-        idx[rd] = tr;
-        idx[cd] = tc;
+        idx[rd] = ar;
+        idx[cd] = ac;
+        if (dd >= 0)
+            idx[dd] = plane;
         int64_t t = 0;
         for (int d = 0; d < a->ndims; ++d)
-            t = t * a->grid[d] + idx[d];
-        return (int)t;
-    }
-    // extents of tile (tr, tc): rows, columns (= leading dimension: the dropped extent is 1)
-    void extent(int tr, int tc, int* lo_r, int* lo_c, int* er, int* ec) const {
+            t = t * a->grid[d] + idx[d] / a->tile;
         int32_t lo[3], ext[3];
-        a->tile_extent(tile_index(tr, tc), lo, ext);
-        *lo_r = lo[rd];
-        *lo_c = lo[cd];
-        *er = ext[rd];
-        *ec = ext[cd];
+        a->tile_extent(t, lo, ext);
+        int64_t stride[3] = {1, 1, 1}, off = 0;
+        for (int d = a->ndims - 2; d >= 0; --d)
+            stride[d] = stride[d + 1] * ext[d + 1];
+        for (int d = 0; d < a->ndims; ++d)
+            off += (int64_t)(idx[d] - lo[d]) * stride[d];
+        *ld = stride[rd];
+        *rlo = lo[rd];
+        *rhi = lo[rd] + ext[rd];
+        *clo = lo[cd];
+        *chi = lo[cd] + ext[cd];
+        return static_cast<const char*>(a->tiles[(size_t)t]) + off * dtype_size(a->dtype);
     }
 };
 
-int as_matrix(const XArray& a, MatView* m, const char* what) {
+int as_matrix(const XArray& a, const cnh_region& win, MatView* m, const char* what) {
     m->a = &a;
     if (a.ndims == 2) {
         m->rd = 0;
         m->cd = 1;
+        m->dd = -1;
     } else {
         CNH_CHECK(a.ndims == 3, -32, "%s needs 2-D operands (or 3-D with one extent of 1)", what);
-        int dropped = -1, ones = 0;
-        for (int d = 0; d < 3; ++d)
-            if (a.shape[d] == 1) {
-                ++ones;
-                if (dropped < 0)
-                    dropped = d;
-            }
-        CNH_CHECK(ones >= 1, -32, "%s: 3-D operand %d has no extent of 1", what, a.name);
+        int dropped = -1;
+        for (int d = 0; d < 3 && dropped < 0; ++d)
+            if (win.stop[d] - win.start[d] == 1)
+                dropped = d;
+        CNH_CHECK(dropped >= 0, -32, "%s: 3-D operand %d has no extent of 1", what, a.name);
+        m->dd = dropped;
         m->rd = dropped == 0 ? 1 : 0;
         m->cd = dropped == 2 ? 1 : 2;
+        m->plane = win.start[dropped];
+        // rows of the matrix must be contiguous in memory: nothing but extent 1 after the columns
+        CNH_CHECK(m->cd == 2 || a.shape[2] == 1, -29,
+                  "%s: the last dimension of array %d is dropped but has extent %d", what, a.name,
+                  a.shape[2]);
     }
-    m->rows = a.shape[m->rd];
-    m->cols = a.shape[m->cd];
+    m->r0 = win.start[m->rd];
+    m->c0 = win.start[m->cd];
+    m->rows = win.stop[m->rd] - m->r0;
+    m->cols = win.stop[m->cd] - m->c0;
     return 0;
 }
 
@@ -982,9 +1041,10 @@ int as_matrix(const XArray& a, MatView* m, const char* what) {
 // src/execute_node.cpp:116-273,489-583).
 int exec_matmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
     XArray *Aa, *x;
-    if (int rc = leaf_array(ex, n, root, 0, &Aa, "MATMUL"))
+    cnh_region wA, wx;
+    if (int rc = leaf_window(ex, n, root, 0, &Aa, &wA, "MATMUL"))
         return rc;
-    if (int rc = leaf_array(ex, n, root, 1, &x, "MATMUL"))
+    if (int rc = leaf_window(ex, n, root, 1, &x, &wx, "MATMUL"))
         return rc;
     bool a_copy = false;
     if (int rc = unphased(ex, Aa, &Aa, &a_copy))
@@ -992,10 +1052,11 @@ int exec_matmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
     // a 3-D matrix operand with one extent of 1 is the plane that remains
     // (charmnumeric.py:552-563, the K14 case of src/executor_matmul.cpp upstream)
     MatView A;
-    if (int rc = as_matrix(*Aa, &A, "MATMUL"))
+    if (int rc = as_matrix(*Aa, wA, &A, "MATMUL"))
         return rc;
     CNH_CHECK(x->ndims == 1, -31, "MATMUL needs a 1-D vector operand");
-    CNH_CHECK(A.cols == x->shape[0], -31, "MATMUL: %d columns, vector of %d", A.cols, x->shape[0]);
+    CNH_CHECK(A.cols == wx.stop[0] - wx.start[0], -31, "MATMUL: %d columns, vector of %d", A.cols,
+              wx.stop[0] - wx.start[0]);
     CNH_CHECK(Aa->dtype == x->dtype, -27, "MATMUL: operand dtypes %d and %d", Aa->dtype, x->dtype);
     int32_t shape[3] = {A.rows, 1, 1};
     XArray* y;
@@ -1005,27 +1066,38 @@ int exec_matmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
             std::to_string(x->name) + " out=" + std::to_string(y->name));
     int rc = 0;
     if (!ex->dry) {
-        const int gr = Aa->grid[A.rd], gc = Aa->grid[A.cd];
-        std::vector<const void*> pt((size_t)gr * gc);
-        for (int tr = 0; tr < gr; ++tr)
-            for (int tc = 0; tc < gc; ++tc)
-                pt[(size_t)tr * gc + tc] = Aa->tiles[(size_t)A.tile_index(tr, tc)];
-        // 1-D arrays are contiguous: tile 0 is the whole vector.
-        rc = cnh_gemv_tiles(Aa->dtype, A.rows, A.cols, Aa->tile, pt.data(), x->tiles[0], y->tiles[0],
-                            ex->stream);
+        // one panel per tile the window meets; panel rows are the array's tile rows
+        const int T = Aa->tile;
+        const int pr0 = A.r0 / T, pr1 = (A.r0 + A.rows - 1) / T;
+        const int pc0 = A.c0 / T, pc1 = (A.c0 + A.cols - 1) / T;
+        std::vector<cnh_gemv_panel> panels;
+        for (int pr = pr0; pr <= pr1; ++pr)
+            for (int pc = pc0; pc <= pc1; ++pc) {
+                const int ac = std::max(pc * T, A.c0);
+                int64_t ld;
+                int rlo, rhi, clo, chi;
+                const char* p = A.at(pr * T, ac, &ld, &rlo, &rhi, &clo, &chi);
+                const int cend = std::min(chi, A.c0 + A.cols);
+                panels.push_back(cnh_gemv_panel{p, ld, cend - ac, ac - A.c0});
+            }
+        // 1-D arrays are contiguous: the vector window is a pointer into tile 0.
+        const char* xp = static_cast<const char*>(x->tiles[0]) + (int64_t)wx.start[0] * dtype_size(x->dtype);
+        rc = cnh_gemv_panels(Aa->dtype, A.rows, pc1 - pc0 + 1, T, A.r0 - pr0 * T, (int64_t)panels.size(),
+                             panels.data(), xp, y->tiles[0], ex->stream);
     }
     if (a_copy)
         drop_array(ex, Aa->name);
     return rc;
 }
 
-// MATMATMUL: C (zeroed) += A_panel * B_panel for every k-overlapping pair of tiles, k ascending
+// MATMATMUL: C = sum of A_panel * B_panel over every k-overlapping pair of tiles, k ascending
 // (src/executor_matmatmul.cpp:105-484, src/executor_incremental.cpp:97-132).
 int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
     XArray *Aa, *Ba;
-    if (int rc = leaf_array(ex, n, root, 0, &Aa, "MATMATMUL"))
+    cnh_region wA, wB;
+    if (int rc = leaf_window(ex, n, root, 0, &Aa, &wA, "MATMATMUL"))
         return rc;
-    if (int rc = leaf_array(ex, n, root, 1, &Ba, "MATMATMUL"))
+    if (int rc = leaf_window(ex, n, root, 1, &Ba, &wB, "MATMATMUL"))
         return rc;
     bool a_copy = false, b_copy = false;
     if (int rc = unphased(ex, Aa, &Aa, &a_copy))
@@ -1033,9 +1105,9 @@ int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
     if (int rc = unphased(ex, Ba, &Ba, &b_copy))
         return rc;
     MatView A, B;
-    if (int rc = as_matrix(*Aa, &A, "MATMATMUL"))
+    if (int rc = as_matrix(*Aa, wA, &A, "MATMATMUL"))
         return rc;
-    if (int rc = as_matrix(*Ba, &B, "MATMATMUL"))
+    if (int rc = as_matrix(*Ba, wB, &B, "MATMATMUL"))
         return rc;
     CNH_CHECK(A.cols == B.rows, -32, "MATMATMUL: (%d,%d) @ (%d,%d)", A.rows, A.cols, B.rows, B.cols);
     CNH_CHECK(Aa->dtype == Ba->dtype, -27, "MATMATMUL: operand dtypes %d and %d", Aa->dtype, Ba->dtype);
@@ -1047,45 +1119,41 @@ int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
     if (int rc = make_array(ex, root.result_name, 2, Aa->dtype, shape, !f64, &Cc))
         return rc;
     const int esz = dtype_size(Aa->dtype);
-    const int TA = Aa->tile, TB = Ba->tile;
+    const int TA = Aa->tile, TB = Ba->tile, K = A.cols;
     int calls = 0;
     std::vector<cnh_gemm_job> jobs;   // all panel products of the node go out as one launch
     for (int ci = 0; ci < Cc->grid[0]; ++ci)
         for (int cj = 0; cj < Cc->grid[1]; ++cj) {
             int32_t clo[3], cext[3];
             Cc->tile_extent((int64_t)ci * Cc->grid[1] + cj, clo, cext);
-            // rows of this C tile fall into A row tiles, its columns into B column tiles
-            for (int ai = clo[0] / TA; ai <= (clo[0] + cext[0] - 1) / TA; ++ai)
-                for (int bj = clo[1] / TB; bj <= (clo[1] + cext[1] - 1) / TB; ++bj) {
-                    int r0 = std::max(clo[0], ai * TA);
-                    int r1 = std::min(clo[0] + cext[0], std::min((ai + 1) * TA, A.rows));
-                    int c0 = std::max(clo[1], bj * TB);
-                    int c1 = std::min(clo[1] + cext[1], std::min((bj + 1) * TB, B.cols));
+            // rows i of this C tile are rows A.r0 + i of A's array, its columns j are columns
+            // B.c0 + j of B's: cut both ranges where those arrays' tiles end
+            for (int r0 = clo[0]; r0 < clo[0] + cext[0];) {
+                const int r1 = std::min(clo[0] + cext[0], ((A.r0 + r0) / TA + 1) * TA - A.r0);
+                for (int c0 = clo[1]; c0 < clo[1] + cext[1];) {
+                    const int c1 = std::min(clo[1] + cext[1], ((B.c0 + c0) / TB + 1) * TB - B.c0);
                     // k pieces: common refinement of A's column tiles and B's row tiles
-                    int k0 = 0;
-                    const int K = A.cols;
-                    while (k0 < K) {
-                        int ak = k0 / TA, bk = k0 / TB;
-                        int k1 = std::min(K, std::min((ak + 1) * TA, (bk + 1) * TB));
-                        int alr, alc, aer, aec, blr, blc, ber, bec;
-                        A.extent(ai, ak, &alr, &alc, &aer, &aec);
-                        B.extent(bk, bj, &blr, &blc, &ber, &bec);
-                        const char* ap = static_cast<const char*>(Aa->tiles[(size_t)A.tile_index(ai, ak)]) +
-                                         ((int64_t)(r0 - alr) * aec + (k0 - alc)) * esz;
-                        const char* bp = static_cast<const char*>(Ba->tiles[(size_t)B.tile_index(bk, bj)]) +
-                                         ((int64_t)(k0 - blr) * bec + (c0 - blc)) * esz;
+                    for (int k0 = 0; k0 < K;) {
+                        const int k1 = std::min(K, std::min(((A.c0 + k0) / TA + 1) * TA - A.c0,
+                                                            ((B.r0 + k0) / TB + 1) * TB - B.r0));
+                        int64_t lda, ldb;
+                        int t0, t1, t2, t3;
+                        const char* ap = A.at(A.r0 + r0, A.c0 + k0, &lda, &t0, &t1, &t2, &t3);
+                        const char* bp = B.at(B.r0 + k0, B.c0 + c0, &ldb, &t0, &t1, &t2, &t3);
                         char* cp = static_cast<char*>(Cc->tiles[(size_t)ci * Cc->grid[1] + cj]) +
                                    ((int64_t)(r0 - clo[0]) * cext[1] + (c0 - clo[1])) * esz;
                         ++calls;
-                        jobs.push_back(cnh_gemm_job{r1 - r0, c1 - c0, k1 - k0, ap, aec, bp, bec, cp, cext[1]});
+                        jobs.push_back(cnh_gemm_job{r1 - r0, c1 - c0, k1 - k0, ap, lda, bp, ldb, cp, cext[1]});
                         k0 = k1;
                     }
+                    c0 = c1;
                 }
+                r0 = r1;
+            }
         }
-    if (!ex->dry) {
+    if (!ex->dry)
         if (int rc = cnh_gemm_batch(Aa->dtype, (int)jobs.size(), jobs.data(), f64 ? 1 : 0, ex->stream))
             return rc;
-    }
     ex->log("matmatmul A=" + std::to_string(Aa->name) + " B=" + std::to_string(Ba->name) + " out=" +
             std::to_string(Cc->name) + " panel_products=" + std::to_string(calls));
     if (a_copy)
@@ -1374,23 +1442,29 @@ void plan_message(Ex* ex, const std::vector<DagNode>& dag) {
         auto it = meta.find(op.result_name);
         return it == meta.end() ? nullptr : &it->second;
     };
-    // rows and columns of a 2-D array or of the plane a 3-D array with an extent of 1 leaves
-    auto matrix_dims = [](const DecompMeta& m, int* rows, int* cols) {
+    // rows and columns of operand i seen as a matrix: a 2-D array (or window of one), or the plane
+    // that a 3-D window with an extent of 1 leaves (src/dag_group_receive.cpp:251-323)
+    auto matrix_dims = [](const DecompMeta& m, const cnh_ast_node& root, int i, int* rows, int* cols) {
+        int ext[3] = {m.shape[0], m.shape[1], m.shape[2]};
+        if (root.has_operand_region[i] && !root.operand_regions[i].is_global &&
+            root.operand_regions[i].ndims == m.ndims)
+            for (int d = 0; d < m.ndims; ++d)
+                ext[d] = root.operand_regions[i].stop[d] - root.operand_regions[i].start[d];
         if (m.ndims == 2) {
-            *rows = m.shape[0];
-            *cols = m.shape[1];
+            *rows = ext[0];
+            *cols = ext[1];
             return true;
         }
         if (m.ndims != 3)
             return false;
         int dropped = -1;
         for (int d = 0; d < 3 && dropped < 0; ++d)
-            if (m.shape[d] == 1)
+            if (ext[d] == 1)
                 dropped = d;
         if (dropped < 0)
             return false;
-        *rows = m.shape[dropped == 0 ? 1 : 0];
-        *cols = m.shape[dropped == 2 ? 1 : 2];
+        *rows = ext[dropped == 0 ? 1 : 0];
+        *cols = ext[dropped == 2 ? 1 : 2];
         return true;
     };
     std::vector<int> fresh;
@@ -1431,7 +1505,7 @@ void plan_message(Ex* ex, const std::vector<DagNode>& dag) {
         case CNH_OP_MATMUL: {
             int rows, cols;
             const DecompMeta* A = known(n, root, 0);
-            if (A && matrix_dims(*A, &rows, &cols)) {
+            if (A && matrix_dims(*A, root, 0, &rows, &cols)) {
                 shape[0] = rows;
                 result(root.result_name, 1, shape);
             }
@@ -1440,7 +1514,7 @@ void plan_message(Ex* ex, const std::vector<DagNode>& dag) {
         case CNH_OP_MATMATMUL: {
             int ar, ac, br, bc;
             const DecompMeta *A = known(n, root, 0), *B = known(n, root, 1);
-            if (A && B && matrix_dims(*A, &ar, &ac) && matrix_dims(*B, &br, &bc)) {
+            if (A && B && matrix_dims(*A, root, 0, &ar, &ac) && matrix_dims(*B, root, 1, &br, &bc)) {
                 shape[0] = ar;
                 shape[1] = bc;
                 result(root.result_name, 2, shape);

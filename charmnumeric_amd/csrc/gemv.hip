@@ -61,11 +61,12 @@ __device__ __forceinline__ A wave_sum(A v) {
 constexpr int kWavesPerBlock = 4;
 constexpr int kUnroll = 8;
 
-// tiles[ti * ncol_tiles + tj]; row r belongs to tile row r / tile_rows.
+// tiles[ti * ncol_tiles + tj]; row r belongs to tile row (r + row_shift) / tile_rows: a window that
+// starts row_shift rows into its first tile row.
 template <typename T, bool VEC16>
 __global__ __launch_bounds__(kWavesPerBlock * 64) void gemv_rows(const ColTile* __restrict__ tiles,
                                                                  int ncol_tiles, int64_t tile_rows,
-                                                                 int64_t rows,
+                                                                 int64_t rows, int64_t row_shift,
                                                                  const T* __restrict__ x,
                                                                  T* __restrict__ y, int beta) {
     typedef typename Acc<T>::type A;
@@ -75,8 +76,8 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void gemv_rows(const ColTile* 
     const int64_t r = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
     if (r >= rows)
         return;
-    const int64_t ti = r / tile_rows;
-    const int64_t lr = r - ti * tile_rows;
+    const int64_t ti = (r + row_shift) / tile_rows;
+    const int64_t lr = r + row_shift - ti * tile_rows;
     A total = 0;
     for (int tj = 0; tj < ncol_tiles; ++tj) {
         const ColTile ct = tiles[ti * ncol_tiles + tj];
@@ -135,7 +136,7 @@ __global__ __launch_bounds__(256) void axpy1_kernel(int64_t n, const T* __restri
 
 template <typename T>
 int run_gemv(const std::vector<ColTile>& tiles, int ncol_tiles, int64_t tile_rows, int64_t rows,
-             const void* x, void* y, int beta, hipStream_t st) {
+             int64_t row_shift, const void* x, void* y, int beta, hipStream_t st) {
     bool vec = ((uintptr_t)x & 15) == 0;
     constexpr int VEC = 16 / sizeof(T);
     for (const ColTile& t : tiles) {
@@ -150,23 +151,23 @@ int run_gemv(const std::vector<ColTile>& tiles, int ncol_tiles, int64_t tile_row
               (long long)rows);
     if (vec)
         hipLaunchKernelGGL((gemv_rows<T, true>), dim3((unsigned)blocks), dim3(kWavesPerBlock * 64),
-                           0, st, (const ColTile*)dtiles, ncol_tiles, tile_rows, rows, (const T*)x,
-                           (T*)y, beta);
+                           0, st, (const ColTile*)dtiles, ncol_tiles, tile_rows, rows, row_shift,
+                           (const T*)x, (T*)y, beta);
     else
         hipLaunchKernelGGL((gemv_rows<T, false>), dim3((unsigned)blocks), dim3(kWavesPerBlock * 64),
-                           0, st, (const ColTile*)dtiles, ncol_tiles, tile_rows, rows, (const T*)x,
-                           (T*)y, beta);
+                           0, st, (const ColTile*)dtiles, ncol_tiles, tile_rows, rows, row_shift,
+                           (const T*)x, (T*)y, beta);
     CNH_HIP(hipGetLastError());
     return 0;
 }
 
 int dispatch_gemv(int dtype, const std::vector<ColTile>& tiles, int ncol_tiles, int64_t tile_rows,
-                  int64_t rows, const void* x, void* y, int beta, hipStream_t st) {
+                  int64_t rows, const void* x, void* y, int beta, hipStream_t st, int64_t row_shift = 0) {
     switch (dtype) {
-    case CNH_F32: return run_gemv<float>(tiles, ncol_tiles, tile_rows, rows, x, y, beta, st);
-    case CNH_F64: return run_gemv<double>(tiles, ncol_tiles, tile_rows, rows, x, y, beta, st);
-    case CNH_I32: return run_gemv<int32_t>(tiles, ncol_tiles, tile_rows, rows, x, y, beta, st);
-    case CNH_I64: return run_gemv<int64_t>(tiles, ncol_tiles, tile_rows, rows, x, y, beta, st);
+    case CNH_F32: return run_gemv<float>(tiles, ncol_tiles, tile_rows, rows, row_shift, x, y, beta, st);
+    case CNH_F64: return run_gemv<double>(tiles, ncol_tiles, tile_rows, rows, row_shift, x, y, beta, st);
+    case CNH_I32: return run_gemv<int32_t>(tiles, ncol_tiles, tile_rows, rows, row_shift, x, y, beta, st);
+    case CNH_I64: return run_gemv<int64_t>(tiles, ncol_tiles, tile_rows, rows, row_shift, x, y, beta, st);
     }
     return set_error(-2, "unknown dtype %d", dtype);
 }
@@ -208,6 +209,30 @@ int cnh_gemv_tiles(int dtype, int64_t rows, int64_t cols, int32_t tile, const vo
             tiles[(size_t)(i * gc + j)] = {p, nc, nc, j * tile};
         }
     return dispatch_gemv(dtype, tiles, (int)gc, tile, rows, x, y, 0, as_stream(s));
+}
+
+static_assert(sizeof(cnh_gemv_panel) == sizeof(ColTile), "cnh_gemv_panel is the kernel's descriptor");
+
+int cnh_gemv_panels(int dtype, int64_t rows, int32_t n_col_panels, int64_t tile_rows, int64_t row_shift,
+                    int64_t n_panels, const cnh_gemv_panel* panels, const void* x, void* y,
+                    cnh_stream s) {
+    if (int rc = ensure_init())
+        return rc;
+    CNH_CHECK(rows > 0 && n_col_panels > 0 && tile_rows > 0 && row_shift >= 0 && row_shift < tile_rows,
+              -2, "cnh_gemv_panels: bad shape");
+    CNH_CHECK(panels && x && y, -2, "cnh_gemv_panels: null pointer");
+    const int64_t panel_rows = (rows + row_shift + tile_rows - 1) / tile_rows;
+    CNH_CHECK(n_panels == panel_rows * n_col_panels, -2,
+              "cnh_gemv_panels: %lld panels given, %lld x %d needed", (long long)n_panels,
+              (long long)panel_rows, n_col_panels);
+    std::vector<ColTile> tiles((size_t)n_panels);
+    for (int64_t i = 0; i < n_panels; ++i) {
+        CNH_CHECK(panels[i].base != nullptr && panels[i].ncols > 0 && panels[i].ld >= panels[i].ncols &&
+                      panels[i].xoff >= 0,
+                  -2, "cnh_gemv_panels: bad panel %lld", (long long)i);
+        tiles[(size_t)i] = {panels[i].base, panels[i].ld, panels[i].ncols, panels[i].xoff};
+    }
+    return dispatch_gemv(dtype, tiles, n_col_panels, tile_rows, rows, x, y, 0, as_stream(s), row_shift);
 }
 
 int cnh_axpy1(int dtype, int64_t n, const void* partial, void* y, cnh_stream s) {

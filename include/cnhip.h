@@ -252,6 +252,22 @@ int cnh_axpy1(int dtype, int64_t n, const void* partial, void* y, cnh_stream s);
 int cnh_gemv_tiles(int dtype, int64_t rows, int64_t cols, int32_t tile, const void* const* tiles,
                    const void* x, void* y, cnh_stream s);
 
+/* The same over a window of a tiled matrix (a sliced or dimension-dropped operand,
+ * charmnumeric.py:536-578, src/executor_matmul.cpp:150-498): row r of the window lies in panel row
+ * p = (r + row_shift) / tile_rows at local row (r + row_shift) % tile_rows; panels[p * n_col_panels
+ * + j] describes the part of tile (p, j) the window covers: base = the element at that tile's
+ * local row 0 and the window's first column inside it, ld = the tile's row stride, ncols = columns
+ * covered, xoff = index in x of the first of them. y[r] = sum over j = 0,1,.. in that order. */
+typedef struct cnh_gemv_panel {
+    const void* base;
+    int64_t ld;
+    int64_t ncols;
+    int64_t xoff;
+} cnh_gemv_panel;
+int cnh_gemv_panels(int dtype, int64_t rows, int32_t n_col_panels, int64_t tile_rows, int64_t row_shift,
+                    int64_t n_panels, const cnh_gemv_panel* panels, const void* x, void* y,
+                    cnh_stream s);
+
 /* ---- MATMATMUL: C += A_panel * B_panel, row-major with row strides
  *      (src/backend_internal.hpp:113-133, src/executor_incremental.cpp:97-132) ---- */
 int cnh_gemm_acc(int dtype, int64_t M, int64_t N, int64_t K, const void* A, int64_t lda,

@@ -303,3 +303,52 @@ def test_jacobi_1d_with_a_temporary(itf, n, dtype):
     got = u.get(itf)
     assert got.dtype == dtype and np.array_equal(got, hu)
     assert got[1] == 0.625 and got[2] == 0.25 and got[3] == 0.125   # three sweeps from the ends
+
+
+# ---- products and dots read unit-step windows in place ----
+
+def _creates(itf):
+    return [ln for ln in itf.trace() if ln.startswith("create")]
+
+
+@pytest.mark.parametrize("r0,r1,c0,c1", [(0, 70, 0, 50), (3, 61, 5, 47), (16, 48, 16, 32), (17, 18, 1, 50)])
+def test_windows_of_matrices_and_vectors_in_place(itf, r0, r1, c0, c1):
+    rng = np.random.default_rng(r0 + c1)
+    hA, hB, hv = rng.standard_normal((70, 50)), rng.standard_normal((50, 70)), rng.standard_normal(90)
+    A, B, v = cnp.array(hA), cnp.array(hB), cnp.array(hv)
+    A.get(itf), B.get(itf), v.get(itf)
+    itf.set_trace()
+    k = c1 - c0
+    y = A[r0:r1, c0:c1] @ v[7:7 + k]
+    P = A[r0:r1, c0:c1] @ B[c0:c1, 2:60]
+    d = v[3:3 + k] @ v[11:11 + k]
+    got_y, got_P, got_d = y.get(itf), P.get(itf), d.get(itf)
+    assert len(_creates(itf)) == 3                      # the three results, no copies of operands
+    wa = hA[r0:r1, c0:c1]
+    assert np.abs(got_y - wa @ hv[7:7 + k]).max() <= 1e-12 * (np.abs(wa) @ np.abs(hv[7:7 + k])).max()
+    wb = hB[c0:c1, 2:60]
+    assert np.all(np.abs(got_P - wa @ wb) <= 1e-12 * (np.abs(wa) @ np.abs(wb)))
+    want_d = hv[3:3 + k] @ hv[11:11 + k]
+    assert abs(got_d.reshape(-1)[0] - want_d) <= 1e-12 * (np.abs(hv[3:3 + k]) @ np.abs(hv[11:11 + k]))
+
+
+def test_planes_of_a_rank3_array_in_place(itf):
+    rng = np.random.default_rng(77)
+    hX, hW, hv = rng.standard_normal((5, 40, 36)), rng.standard_normal((36, 20)), rng.standard_normal(36)
+    X, W, v = cnp.array(hX), cnp.array(hW), cnp.array(hv)
+    X.get(itf), W.get(itf), v.get(itf)
+    itf.set_trace()
+    got = [(X[2] @ W).get(itf), (X[3, 4:30, :] @ W).get(itf), (X[4] @ v).get(itf),
+           (X[:, 7, :] @ W).get(itf), (X[1:4, 9, 2:36] @ v[0:34]).get(itf)]
+    assert len(_creates(itf)) == 5
+    want = [hX[2] @ hW, hX[3, 4:30, :] @ hW, hX[4] @ hv, hX[:, 7, :] @ hW, hX[1:4, 9, 2:36] @ hv[0:34]]
+    for g, w in zip(got, want):
+        assert g.shape == w.shape and np.allclose(g, w, rtol=1e-12, atol=1e-12)
+    # dropping the last dimension leaves rows that are not contiguous: copied out first
+    g = (X[:, 0:36, 5] @ W).get(itf)
+    assert len(_creates(itf)) == 2
+    assert np.allclose(g, hX[:, 0:36, 5] @ hW, rtol=1e-12, atol=1e-12)
+    # strided windows are copied out too
+    g = (X[2, ::2, :] @ W).get(itf)
+    assert len(_creates(itf)) == 2
+    assert np.allclose(g, hX[2, ::2, :] @ hW, rtol=1e-12, atol=1e-12)

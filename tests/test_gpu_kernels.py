@@ -347,6 +347,41 @@ def test_gemm_batch_overwrites_without_reading(dev, M, N, K):
     dev.free_all()
 
 
+@pytest.mark.parametrize("dt,npdt", [(L.F64, np.float64), (L.I32, np.int32)])
+def test_gemv_over_a_window_of_tiles(dev, dt, npdt):
+    """A 100 x 90 matrix in 32 x 32 tiles; the window rows 5..77, columns 9..70 against x."""
+    rng = np.random.default_rng(31)
+    M, N, T = 100, 90, 32
+    A = (rng.standard_normal((M, N)) if npdt == np.float64 else rng.integers(-99, 99, (M, N))).astype(npdt)
+    x = (rng.standard_normal(80) if npdt == np.float64 else rng.integers(-99, 99, 80)).astype(npdt)
+    r0, r1, c0, c1 = 5, 77, 9, 70
+    tiles = {}
+    for ti in range((M + T - 1) // T):
+        for tj in range((N + T - 1) // T):
+            tiles[ti, tj] = dev.array(np.ascontiguousarray(A[ti * T:(ti + 1) * T, tj * T:(tj + 1) * T]))
+    pr0, pr1, pc0, pc1 = r0 // T, (r1 - 1) // T, c0 // T, (c1 - 1) // T
+    panels = (L.GemvPanel * ((pr1 - pr0 + 1) * (pc1 - pc0 + 1)))()
+    i = 0
+    for pr in range(pr0, pr1 + 1):
+        for pc in range(pc0, pc1 + 1):
+            width = min(T, N - pc * T)
+            first = max(pc * T, c0)
+            panels[i].base = tiles[pr, pc].ptr + (first - pc * T) * A.itemsize
+            panels[i].ld, panels[i].ncols, panels[i].xoff = width, min((pc + 1) * T, c1) - first, first - c0
+            i += 1
+    dx, dy = dev.array(x), dev.array(np.zeros(r1 - r0, npdt))
+    L.check(L.lib.cnh_gemv_panels(dt, r1 - r0, pc1 - pc0 + 1, T, r0 - pr0 * T, len(panels), panels,
+                                  dx.ptr + 3 * A.itemsize, dy.ptr, None))
+    want = A[r0:r1, c0:c1] @ x[3:3 + c1 - c0]
+    if npdt == np.float64:
+        assert np.abs(dy.get() - want).max() <= REL * (np.abs(A[r0:r1, c0:c1]) @ np.abs(x[3:3 + c1 - c0])).max()
+    else:
+        assert np.array_equal(dy.get(), want)
+    assert L.lib.cnh_gemv_panels(dt, r1 - r0, pc1 - pc0 + 1, T, T, len(panels), panels, dx.ptr, dy.ptr, None) != 0
+    assert L.lib.cnh_gemv_panels(dt, r1 - r0, pc1 - pc0 + 1, T, 0, len(panels) - 1, panels, dx.ptr, dy.ptr, None) != 0
+    dev.free_all()
+
+
 def test_descriptor_table_outlives_the_stream_it_was_uploaded_on(dev):
     """The same job list (hence the same descriptor table) on a stream, then on a second stream after
     the first was destroyed: the cached table must be usable without touching the dead stream."""
