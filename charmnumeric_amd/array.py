@@ -251,9 +251,10 @@ class _ArrayLike:
                 raise NotImplementedError("assignment across dtypes is not implemented")
             if tuple(value.shape) != tuple(shape):
                 # a lower-rank value fits a region whose extra dimensions have extent 1
-                # (IFOG[t] = M with M 2-D)
+                # (IFOG[t] = M with M 2-D), and a whole higher-rank one whose extra dimensions
+                # have extent 1 fits a lower-rank target (vec[:] = column)
                 squeeze = lambda sh: tuple(x for x in sh if x != 1)
-                if not (value.ndims < len(shape) and squeeze(value.shape) == squeeze(shape)
+                if not (value.ndims != len(shape) and squeeze(value.shape) == squeeze(shape)
                         and _is_whole(value._region(), value._base().shape)):
                     raise ValueError(
                         f"could not broadcast input from shape {value.shape} into shape {shape}")
@@ -513,12 +514,20 @@ def _matmul(lhs, rhs):
     if rhs.ndims == 1:
         return _matvec(lhs, rhs)
     if rhs.ndims == 2 and rhs.shape[1] == 1:
-        raise NotImplementedError("matmul with an (N, 1) column operand is not implemented")
+        return _matvec(lhs, _column_as_vector(rhs))
     lr, lc = _matrix_shape(lhs)
     rr, rc = _matrix_shape(rhs)
     if lc != rr:
         raise ValueError(f"Shape mismatch: ({lr},{lc}) @ ({rr},{rc})")
     return nonfusible(L.OP_MATMATMUL, [lhs, rhs], (lr, rc), _same_dtype(lhs, rhs, "matmul"))
+
+
+def _column_as_vector(col):
+    """An (N, 1) operand of a matvec becomes a 1-D temporary, and the result is 1-D
+    (charmnumeric.py:528-531,542-545 upstream)."""
+    temp = create_array((col.shape[0],), dtype=col.dtype)
+    temp[:] = _whole(col)
+    return temp
 
 
 def _matrix_shape(x):
@@ -539,7 +548,7 @@ def _matvec(mat, vec):
     if not isinstance(vec, _ArrayLike):
         raise ValueError("matvec requires an Array vector")
     if vec.ndims == 2 and vec.shape[1] == 1:
-        raise NotImplementedError("matvec with an (N, 1) column operand is not implemented")
+        vec = _column_as_vector(vec)
     if vec.ndims != 1:
         raise ValueError("matvec requires a 1D vector (N,) or 2D column vector (N, 1)")
     if mat.ndims == 2:

@@ -770,6 +770,33 @@ int exec_group(Ex* ex, const DagNode& n) {
             CNH_CHECK(j == a.ndims, -35, "node %d: operand %d does not fit the assigned region", n.id,
                       a.name);
             tin[i] = t;
+        } else if (in_arr[i]->ndims > target->ndims) {
+            // A higher-rank operand whose extra dimensions have extent 1 (vec[:] = column with
+            // column of shape (N, 1), charmnumeric.py:528-531 upstream): drop them. A row-major
+            // tile (e0, 1) is the same memory as (e0).
+            CNH_CHECK(!in_has_reg[i], -35, "node %d: operand %d has rank %d in a rank-%d group", n.id,
+                      in_arr[i]->name, in_arr[i]->ndims, target->ndims);
+            const XArray& a = *in_arr[i];
+            cnh_tiled t;
+            std::memset(&t, 0, sizeof t);
+            t.ndims = target->ndims;
+            t.tile = a.tile;
+            t.tiles = a.tiles.data();
+            int j = 0;
+            for (int d = 0; d < a.ndims; ++d) {
+                if (a.shape[d] == 1 && a.ndims - d > target->ndims - j)
+                    continue; // dropped
+                CNH_CHECK(j < target->ndims, -35, "node %d: operand %d of shape rank %d does not fit a "
+                          "rank-%d target", n.id, a.name, a.ndims, target->ndims);
+                t.shape[j] = a.shape[d];
+                t.grid[j] = a.grid[d];
+                t.offset[j] = a.offset[d];
+                t.grid_lo[j] = a.offset[d] / a.tile;
+                ++j;
+            }
+            CNH_CHECK(j == target->ndims, -35, "node %d: operand %d does not reduce to rank %d", n.id,
+                      a.name, target->ndims);
+            tin[i] = t;
         } else {
             CNH_CHECK(in_arr[i]->ndims == target->ndims, -35,
                       "node %d: operand %d has rank %d in a rank-%d group", n.id, in_arr[i]->name,

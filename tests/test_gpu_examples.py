@@ -352,3 +352,23 @@ def test_planes_of_a_rank3_array_in_place(itf):
     g = (X[2, ::2, :] @ W).get(itf)
     assert len(_creates(itf)) == 2
     assert np.allclose(g, hX[2, ::2, :] @ hW, rtol=1e-12, atol=1e-12)
+
+
+def test_column_operand_becomes_a_vector(itf):
+    """A @ c with c of shape (N, 1): upstream copies the column into a 1-D temporary and returns
+    the 1-D matvec result (charmnumeric.py:528-531 upstream)."""
+    rng = np.random.default_rng(12)
+    hA, hc = rng.standard_normal((70, 50)), rng.standard_normal((50, 1))
+    A, c = cnp.array(hA), cnp.array(hc)
+    got = (A @ c).get(itf)
+    want = hA @ hc[:, 0]
+    assert got.shape == (70,)
+    assert np.abs(got - want).max() <= 1e-12 * (np.abs(hA) @ np.abs(hc[:, 0])).max()
+    # a column cut out of a matrix
+    hM = rng.standard_normal((50, 9))
+    M = cnp.array(hM)
+    got = A.matvec(M[:, 4:5]).get(itf)
+    assert np.abs(got - hA @ hM[:, 4]).max() <= 1e-12 * (np.abs(hA) @ np.abs(hM[:, 4])).max()
+    v = cnp.zeros((50,))
+    v[:] = c                                  # the assignment itself, bit for bit
+    assert np.array_equal(v.get(itf), hc[:, 0])
