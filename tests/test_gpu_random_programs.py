@@ -166,6 +166,7 @@ def test_random_program(seed, rank, solver):
     for nd, t in MIN_TILE.items():
         itf.set_min_tile(nd, t)
     itf.set_solver(solver)
+    itf.set_pipeline(seed % 2 == 1)       # odd seeds: messages queue for the executor's own thread
     cnp.set_auto_flush(itf, int(np.random.default_rng(seed).choice([4, 16, 1000])))
     try:
         prog = Program(1000 * rank + seed, rank, np.float32 if seed % 5 == 4 else np.float64)
