@@ -82,6 +82,11 @@ struct DirectShape {
     // the other arrays it reads at the element's own position (source terms, weights)
     std::vector<int> other;
     std::vector<int> other_names; // array names in the order the indices above number them
+    // The array read through the window. Usually the assigned one (a sweep in place); when only
+    // another array is read at shifted positions (unew[interior] = f(u shifted)), that one: the
+    // launch then reads its tiles and writes the assigned elements of the target, nothing else.
+    int window_name = 0;
+    bool masked = false;
 };
 constexpr int kDirectMaxOther = 4;
 int direct_shape(const GroupProgram& p, const DirectConfig& cfg, DirectShape& sh, std::string& err);

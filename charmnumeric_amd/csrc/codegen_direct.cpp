@@ -42,14 +42,33 @@ int direct_shape(const GroupProgram& p, const DirectConfig& cfg, DirectShape& sh
     }
     sh.shifts.assign(p.load_leaf.size(), {0, 0, 0});
     sh.other.assign(p.load_leaf.size(), -1);
-    bool reads_target = false;
+    // The window array: the one array read at positions other than the element's own; the
+    // assigned array when there is none.
+    sh.window_name = p.out_target[0];
+    bool found_shifted = false;
     for (size_t l = 0; l < p.load_leaf.size(); ++l) {
         const LeafUse& u = p.leaves[p.load_leaf[l]];
         if (!u.has_region) {
             err = "operand without a region";
             return -18;
         }
-        if (u.name != p.out_target[0]) {
+        bool shifted = false;
+        for (int d = 0; d < nd; ++d)
+            shifted = shifted || u.region.start[d] != ro.start[d];
+        if (!shifted)
+            continue;
+        if (found_shifted && u.name != sh.window_name) {
+            err = "two arrays are read at shifted positions";
+            return -18;
+        }
+        found_shifted = true;
+        sh.window_name = u.name;
+    }
+    sh.masked = sh.window_name != p.out_target[0];
+    bool reads_target = false;
+    for (size_t l = 0; l < p.load_leaf.size(); ++l) {
+        const LeafUse& u = p.leaves[p.load_leaf[l]];
+        if (u.name != sh.window_name) {
             // another array (a source term, a weight): only at the element's own position
             for (int d = 0; d < nd; ++d)
                 if (u.region.step[d] != 1 || u.region.start[d] != ro.start[d] ||
@@ -83,7 +102,7 @@ int direct_shape(const GroupProgram& p, const DirectConfig& cfg, DirectShape& sh
         }
     }
     if (!reads_target) {
-        err = "the assigned array is not read";
+        err = "no array is read through a window";
         return -18;
     }
     for (int d = 0; d < 3; ++d)
@@ -132,7 +151,8 @@ std::string direct_source(const GroupProgram& p, const DirectConfig& cfg, std::s
     auto floordiv2 = [](int v) { return v >= 0 ? v / 2 : -((-v + 1) / 2); };
     for (int rz = 0; rz < sh.rz; ++rz)
         for (int ry = 0; ry < sh.ry; ++ry) {
-            at(rz + H0, ry + H1, HK) = 1; // the element itself (kept outside the assigned region)
+            if (!sh.masked)
+                at(rz + H0, ry + H1, HK) = 1; // the element itself (kept outside the assigned region)
             for (int e = 0; e < 2; ++e)
                 for (const auto& s : sh.shifts)
                     at(rz + H0 + s[0], ry + H1 + s[1], HK + floordiv2(e + s[2])) = 1;
@@ -149,6 +169,7 @@ std::string direct_source(const GroupProgram& p, const DirectConfig& cfg, std::s
           << sh.shifts[l][2] << "}";
     s << "};\n";
     const int NOTH = (int)sh.other_names.size();
+    s << "#define DR_MASKED " << (sh.masked ? 1 : 0) << "\n";
     s << "#define DR_NOTH " << NOTH << "\n#define DR_NOTHA " << (NOTH > 0 ? NOTH : 1) << "\n";
     s << "__device__ constexpr int DR_OTHER[NLA] = {";
     for (size_t l = 0; l < sh.other.size(); ++l)
@@ -197,6 +218,20 @@ typedef T P2 __attribute__((ext_vector_type(2)));
 typedef int I2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ int floordiv2(int v) { return v >= 0 ? v / 2 : -((-v + 1) / 2); }
+
+// One pair of results. A sweep in place of the window array writes every pair whole (elements
+// outside the assigned region carry their old values in `v`); a launch whose window array is
+// another one (DR_MASKED) writes assigned elements only and leaves the rest of the target alone.
+template <bool NTS>
+__device__ __forceinline__ void store_pair(P2* out, P2 v, bool in0, bool in1) {
+    if (!DR_MASKED || (in0 && in1)) {
+        if (NTS) __builtin_nontemporal_store(v, out); else *out = v;
+    } else {
+        T* one = reinterpret_cast<T*>(out);
+        if (in0) one[0] = v[0];
+        if (in1) one[1] = v[1];
+    }
+}
 
 // A build that runs the lanes of a wavefront as coroutines on a host (bounds checking of this
 // source) supplies its own lane exchange and readfirstlane.
@@ -361,6 +396,7 @@ __device__ __forceinline__ void direct_fast(const DirectArgs& a, const T* s) {
 #pragma unroll
         for (int ry = 0; ry < DR_RY; ++ry) {
             P2 res;
+            bool in_e[2];
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
                 T l[NLA], o[NOA];
@@ -374,10 +410,11 @@ __device__ __forceinline__ void direct_fast(const DirectArgs& a, const T* s) {
                 }
                 group_eval(l, s, o);
                 const int gx = p.tx0 + lx + e;
-                res[e] = (gx >= a.rs[2] && gx < a.re[2]) ? o[0] : win[rz + DR_H0][ry + DR_H1][DR_HK][e];
+                in_e[e] = gx >= a.rs[2] && gx < a.re[2];
+                res[e] = (DR_MASKED || in_e[e]) ? o[0] : win[rz + DR_H0][ry + DR_H1][DR_HK][e];
             }
             P2* out = reinterpret_cast<P2*>(out_tile + ((lz0 + rz) * PZ + (ly0 + ry) * PY + lx));
-            if (NTS) __builtin_nontemporal_store(res, out); else *out = res;
+            store_pair<NTS>(out, res, in_e[0], in_e[1]);
         }
 }
 
@@ -527,6 +564,7 @@ __device__ __forceinline__ void direct_rest(const DirectArgs& a, const T* s, int
                     const int gy = ty0 + ly;
                     const bool yin = zin && gy >= a.rs[1] && gy < a.re[1];
                     P2 res;
+                    bool in_e[2];
 #pragma unroll
                     for (int e = 0; e < 2; ++e) {
                         const int gx = tx0 + lx + e;
@@ -544,10 +582,11 @@ __device__ __forceinline__ void direct_rest(const DirectArgs& a, const T* s, int
                                             [DR_HK + floordiv2(xx)][xx & 1];
                         }
                         group_eval(l, s, o);
-                        res[e] = in_region ? o[0] : win[rz + DR_H0][ry + DR_H1][DR_HK][e];
+                        in_e[e] = in_region;
+                        res[e] = (DR_MASKED || in_region) ? o[0] : win[rz + DR_H0][ry + DR_H1][DR_HK][e];
                     }
                     P2* out = reinterpret_cast<P2*>(out_tile + (lz * OPZ + ly * OPY + lx));
-                    if (NTS) __builtin_nontemporal_store(res, out); else *out = res;
+                    store_pair<NTS>(out, res, in_e[0], in_e[1]);
                 }
             }
         }

@@ -720,6 +720,19 @@ int try_launch_direct(cnh_kernel* k, const std::vector<const cnh_tiled*>& arrays
     if (self < 0)
         return 0;
     const std::vector<const cnh_tiled*> own(1, arrays[(size_t)self]);
+    if (sh.masked) {
+        // The window array is not the assigned one: the launch reads that array's tiles and
+        // writes the target's assigned elements in place. Both must be cut alike.
+        const cnh_tiled* w = own[0];
+        if (cur == nullptr || dst->tiles[0] != cur->tiles[0] || w->ndims != dst->ndims ||
+            w->tile != dst->tile)
+            return 0;
+        for (int d = 0; d < w->ndims; ++d)
+            if (w->shape[d] != dst->shape[d] || w->grid[d] != dst->grid[d] || w->offset[d] != 0 ||
+                dst->offset[d] != 0 || w->pitch[d] != dst->pitch[d])
+                return 0;
+        return launch_direct(k, sh, own, others, (int)sh.other_names.size(), w, dst, scal, st, handled);
+    }
     return launch_direct(k, sh, own, others, (int)sh.other_names.size(), cur, dst, scal, st, handled);
 }
 
@@ -785,8 +798,10 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
             if (o->offset[d] != 0 || o->shape[d] != cur->shape[d] || o->grid[d] != cur->grid[d] ||
                 o->grid_lo[d] != cur->grid_lo[d])
                 return 0;
+        // (an operand at the element's own position may be the target itself when the window
+        // array is another one: a lane then reads the very elements it writes)
         for (int64_t t = 0; t < ntiles; ++t)
-            if (((uintptr_t)o->tiles[t] & 15) || o->tiles[t] == dst->tiles[t])
+            if (((uintptr_t)o->tiles[t] & 15) || (!sh.masked && o->tiles[t] == dst->tiles[t]))
                 return 0;
     }
     DirectArgsDev a;

@@ -28,3 +28,25 @@ def test_register_window_kernel_builds_for_other_element_types(dt):
     L.check(L.lib.cnh_kernel_build(k, b"direct"))
     k3 = H.compile_group(H.ast_jacobi3d(32, dtype=dt, coef=2.0), dt, 3)
     L.check(L.lib.cnh_kernel_build(k3, b"direct"))
+
+
+def test_register_window_kernel_for_a_sweep_from_one_array_into_another():
+    """out[1:-1,1:-1] = coef*(shifted reads of u): the window array is u, the launch writes the
+    assigned elements of out only."""
+    from charmnumeric_amd.astbuild import AstBuilder
+    n = 64
+    b = AstBuilder(L.F64, 2)
+    u, out = b.leaf(0), b.leaf(1)
+    mid = ((1, 1), (n - 1, n - 1), (1, 1))
+    t1 = b.binary(L.OP_ADD, 100, u, u, ((0, 1), (n - 2, n - 1), (1, 1)), ((2, 1), (n, n - 1), (1, 1)))
+    t2 = b.binary(L.OP_ADD, 101, t1, u, None, ((1, 0), (n - 1, n - 2), (1, 1)))
+    t3 = b.binary(L.OP_ADD, 102, t2, u, None, ((1, 2), (n - 1, n), (1, 1)))
+    t4 = b.binary(L.OP_MUL, 103, b.scalar(0.25), t3)
+    b.set_region(104, out, t4, mid)
+    k = H.compile_group(b.finish(), L.F64, 2)
+    L.check(L.lib.cnh_kernel_build(k, b"direct"))
+    src = H.kernel_source(k, "direct")
+    assert "#define DR_MASKED 1" in src and "#define DR_NOTH 0" in src
+    k2 = H.compile_group(H.ast_jacobi2d(64), L.F64, 2)
+    L.check(L.lib.cnh_kernel_build(k2, b"direct"))
+    assert "#define DR_MASKED 0" in H.kernel_source(k2, "direct")

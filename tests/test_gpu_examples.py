@@ -372,3 +372,60 @@ def test_column_operand_becomes_a_vector(itf):
     v = cnp.zeros((50,))
     v[:] = c                                  # the assignment itself, bit for bit
     assert np.array_equal(v.get(itf), hc[:, 0])
+
+
+# ---- stencils that read one array and assign another ----
+
+def _kernels(itf):
+    return [ln.rsplit("kernel=", 1)[1] for ln in itf.trace() if ln.startswith("group") and "kernel=" in ln]
+
+
+@pytest.mark.parametrize("nd,n,dtype", [(2, 96, np.float64), (2, 50, np.float32), (3, 40, np.float64)])
+def test_two_array_sweeps_take_the_register_window_kernel(itf, nd, n, dtype):
+    rng = np.random.default_rng(nd * n)
+    hu = rng.standard_normal((n,) * nd).astype(dtype)
+    hv = rng.standard_normal((n,) * nd).astype(dtype)
+    hf = rng.standard_normal((n,) * nd).astype(dtype)
+    u, v, f = cnp.array(hu), cnp.array(hv), cnp.array(hf)
+    u.get(itf), v.get(itf), f.get(itf)
+    inner = (slice(1, -1),) * nd
+
+    def neighbours(x):
+        out = None
+        for d in range(nd):
+            for s in (slice(0, -2), slice(2, None)):
+                key = list(inner)
+                key[d] = s
+                out = x[tuple(key)] if out is None else out + x[tuple(key)]
+        return out
+
+    itf.set_trace()
+    c = 1.0 / (2 * nd)
+    for _ in range(4):                                   # unew = sweep(u); swap
+        v[inner] = c * neighbours(u)
+        hv[inner] = c * neighbours(hu)
+        u, v, hu, hv = v, u, hv, hu
+    r = cnp.zeros((n,) * nd, dtype=dtype)
+    hr = np.zeros((n,) * nd, dtype=dtype)
+    r[inner] = f[inner] - (2.0 * nd * u[inner] - neighbours(u))        # residual: three arrays
+    hr[inner] = hf[inner] - (2.0 * nd * hu[inner] - neighbours(hu))
+    v[inner] = v[inner] + 0.125 * neighbours(u)                        # the target at its own position
+    hv[inner] = hv[inner] + 0.125 * neighbours(hu)
+    got_u, got_v, got_r = u.get(itf), v.get(itf), r.get(itf)
+    assert np.array_equal(got_u, hu) and np.array_equal(got_v, hv) and np.array_equal(got_r, hr)
+    kernels = _kernels(itf)
+    assert len(kernels) == 6 and all(k == "direct" for k in kernels), kernels
+
+
+def test_two_shifted_arrays_fall_back_to_the_gather(itf):
+    rng = np.random.default_rng(5)
+    hu, hw = rng.standard_normal((64, 64)), rng.standard_normal((64, 64))
+    u, w = cnp.array(hu), cnp.array(hw)
+    v = cnp.zeros((64, 64))
+    hv = np.zeros((64, 64))
+    u.get(itf), w.get(itf), v.get(itf)
+    itf.set_trace()
+    v[1:-1, 1:-1] = u[:-2, 1:-1] + w[2:, 1:-1]
+    hv[1:-1, 1:-1] = hu[:-2, 1:-1] + hw[2:, 1:-1]
+    assert np.array_equal(v.get(itf), hv)
+    assert _kernels(itf) == ["gather"]
