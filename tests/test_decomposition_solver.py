@@ -398,3 +398,61 @@ def test_cycle_with_conflicting_wishes_follows_the_heavier_one():
         out = solve({a: ((256,), (0,), 64, True), b: ((nb,), (0,), 64, True), t: ((100,), (0,), 0, False)},
                     message(w, w2), odf=64)
         assert out[t][0] == 64 and out[t][1][0] % 64 == want, (nb, out[t])
+
+
+# ---- robustness: random DAGs never crash the solver and always give usable tiles ----
+
+def test_random_dags_give_power_of_two_tiles_and_finite_offsets():
+    rng = np.random.default_rng(2024)
+    for case in range(300):
+        nd = int(rng.integers(1, 4))
+        names = list(range(1, 7))
+        arrays = {}
+        for name in names:
+            shape = tuple(int(rng.integers(1, 300)) for _ in range(nd))
+            final = bool(rng.integers(0, 2))
+            tile = int(rng.choice([0, 16, 64, 128])) if not final else int(rng.choice([16, 64, 128]))
+            offset = tuple(int(rng.integers(0, 200)) if final else 0 for _ in range(nd))
+            arrays[name] = (shape, offset, tile, final)
+        # one lower- or higher-rank array for assignments across ranks
+        other_nd = nd - 1 if nd > 1 else nd + 1
+        arrays[9] = (tuple(int(rng.integers(1, 100)) for _ in range(other_nd)), (0,) * other_nd, 0, False)
+
+        def region(shape):
+            start, stop, step = [], [], []
+            for n in shape:
+                st = int(rng.choice([1, 1, 2, 3]))
+                a = int(rng.integers(0, n))
+                b = int(rng.integers(a + 1, n + 1))
+                start.append(a), stop.append(b), step.append(st)
+            return reg(start, stop, step)
+
+        nodes = []
+        for _ in range(int(rng.integers(1, 6))):
+            w = lazy._NodeWriter()
+            kind = int(rng.integers(0, 4))
+            a, b, out = (int(x) for x in rng.choice(names, 3))
+            la, lb = w.leaf(Ref(a, nd)), w.leaf(Ref(b, nd))
+            ra = region(arrays[a][0]) if rng.integers(0, 2) else None
+            rb = region(arrays[b][0]) if rng.integers(0, 2) else None
+            if kind == 0:
+                w.op(out, L.OP_ADD, False, nd, L.F64, [la, lb], [ra, rb])
+            elif kind == 1:
+                t = w.op(100 + len(nodes), L.OP_MUL, True, nd, L.F64, [la, lb], [ra, rb])
+                w.op(200 + len(nodes), L.OP_SET_REGION, False, nd, L.F64, [w.leaf(Ref(out, nd)), t],
+                     [None, None], region=region(arrays[out][0]))
+            elif kind == 2:
+                w.op(300 + len(nodes), L.OP_SET_REGION, False, nd, L.F64,
+                     [w.leaf(Ref(out, nd)), w.leaf(Ref(9, other_nd))], [None, None],
+                     region=region(arrays[out][0]))
+            else:
+                w.op(out, L.OP_MATMATMUL if nd == 2 else L.OP_COPY, False, nd, L.F64,
+                     [la, lb] if nd == 2 else [la], [ra, rb] if nd == 2 else [ra])
+            nodes.append(w)
+        got = solve(arrays, message(*nodes), odf=int(rng.choice([1, 4, 64])), min_tile=(16, 16, 16))
+        for name, (tile, offset) in got.items():
+            shape, off0, tile0, final = arrays[name]
+            assert tile >= 16 and tile & (tile - 1) == 0, (case, name, tile)
+            assert all(abs(o) < (1 << 24) for o in offset), (case, name, offset)
+            if final:
+                assert (tile, offset) == (tile0, off0), (case, name)
