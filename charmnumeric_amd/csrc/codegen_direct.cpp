@@ -175,6 +175,23 @@ std::string direct_source(const GroupProgram& p, const DirectConfig& cfg, std::s
     for (size_t l = 0; l < sh.other.size(); ++l)
         s << (l ? ", " : "") << sh.other[l];
     s << "};\n";
+    // Rows of the window whose first or last lane needs the pair beyond the wavefront's 128
+    // columns. When they form a full block of at most 32 rows, one partial load per wavefront
+    // fetches all of them (lane 2r + side for row r) and lanes 0 and 63 pick theirs by readlane.
+    int bi0 = WZ, bi1 = -1, bj0 = WY, bj1 = -1, brows = 0;
+    for (int z = 0; z < WZ; ++z)
+        for (int y = 0; y < WY; ++y)
+            if (at(z, y, 0) || at(z, y, WK - 1)) {
+                bi0 = std::min(bi0, z);
+                bi1 = std::max(bi1, z);
+                bj0 = std::min(bj0, y);
+                bj1 = std::max(bj1, y);
+                ++brows;
+            }
+    const bool gather = brows > 0 && brows == (bi1 - bi0 + 1) * (bj1 - bj0 + 1) && brows <= 32 && HK == 1;
+    s << "#define DR_EDGE_GATHER " << (gather ? 1 : 0) << "\n#define DR_BI0 " << (gather ? bi0 : 0)
+      << "\n#define DR_BJ0 " << (gather ? bj0 : 0) << "\n#define DR_BNJ " << (gather ? bj1 - bj0 + 1 : 1)
+      << "\n#define DR_NB " << (gather ? brows : 0) << "\n";
     s << "__device__ constexpr bool DR_NEED[DR_WZ][DR_WY][DR_WK] = {";
     for (int z = 0; z < WZ; ++z) {
         s << (z ? ", " : "") << "{";
@@ -248,6 +265,18 @@ __device__ __forceinline__ V lane_shift(V v) {
     } else {
         const int a = __builtin_bit_cast(int, v);
         return __builtin_bit_cast(V, __builtin_amdgcn_update_dpp(a, a, CTRL, 0xf, 0xf, false));
+    }
+}
+// The value a given lane holds, as a wavefront-uniform value.
+template <typename V>
+__device__ __forceinline__ V from_lane(V v, int src) {
+    if constexpr (sizeof(V) == 8) {
+        I2 a = __builtin_bit_cast(I2, v), r;
+        r[0] = __builtin_amdgcn_readlane(a[0], src);
+        r[1] = __builtin_amdgcn_readlane(a[1], src);
+        return __builtin_bit_cast(V, r);
+    } else {
+        return __builtin_bit_cast(V, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), src));
     }
 }
 __device__ __forceinline__ T from_prev_lane(T v) { return lane_shift<0x138>(v); }
@@ -342,9 +371,10 @@ __device__ __forceinline__ void direct_fast(const DirectArgs& a, const T* s) {
     }
     const bool first = lane == 0, last = lane == 63;
 
-    // All loads first, none under a branch: the two end lanes of the wavefront fetch the pair
-    // beyond their end, every other lane re-reads its own centre pair (a cache hit), so each row
-    // costs one more full-wave load and the wavefront waits for memory once.
+    // All loads first. The pairs beyond the two ends of the wavefront are fetched by one load when
+    // the rows that need them form a block (the usual case); otherwise the two end lanes fetch
+    // theirs row by row while every other lane re-reads its own centre pair (a cache hit), one
+    // more full-wave load per row. Either way the wavefront waits for memory once.
     P2 win[DR_WZ][DR_WY][DR_WK];
     P2 beyond[DR_WZ][DR_WY];
 #pragma unroll
@@ -353,16 +383,27 @@ __device__ __forceinline__ void direct_fast(const DirectArgs& a, const T* s) {
         for (int j = 0; j < DR_WY; ++j)
             if (DR_NEED[i][j][0] || DR_NEED[i][j][DR_HK] || DR_NEED[i][j][DR_WK - 1])
                 win[i][j][DR_HK] = *reinterpret_cast<const P2*>(pc + i * PZ + j * PY);
+    P2 edge = (P2){(T)0, (T)0};
+    if (DR_EDGE_GATHER) {
+        // one load for all of them: lane 2r holds the pair left of row r, lane 2r + 1 the pair
+        // right of it (r counts the rows of the block in row-major order)
+        if (lane < 2 * DR_NB) {
+            const int r = lane >> 1, i = DR_BI0 + r / DR_BNJ, j = DR_BJ0 + r % DR_BNJ;
+            const T* src = (lane & 1) ? rp + i * rpz + j * rpy : lp + i * lpz + j * lpy;
+            edge = *reinterpret_cast<const P2*>(src);
+        }
+    } else {
 #pragma unroll
-    for (int i = 0; i < DR_WZ; ++i)
+        for (int i = 0; i < DR_WZ; ++i)
 #pragma unroll
-        for (int j = 0; j < DR_WY; ++j)
-            if (DR_NEED[i][j][0] || DR_NEED[i][j][DR_WK - 1]) {
-                const T* src = pc + i * PZ + j * PY;
-                src = first ? lp + i * lpz + j * lpy : src;
-                src = last ? rp + i * rpz + j * rpy : src;
-                beyond[i][j] = *reinterpret_cast<const P2*>(src);
-            }
+            for (int j = 0; j < DR_WY; ++j)
+                if (DR_NEED[i][j][0] || DR_NEED[i][j][DR_WK - 1]) {
+                    const T* src = pc + i * PZ + j * PY;
+                    src = first ? lp + i * lpz + j * lpy : src;
+                    src = last ? rp + i * rpz + j * rpy : src;
+                    beyond[i][j] = *reinterpret_cast<const P2*>(src);
+                }
+    }
     P2 ov[DR_NOTHA][DR_RZ][DR_RY];
 #pragma unroll
     for (int j = 0; j < DR_NOTH; ++j) {
@@ -377,17 +418,26 @@ __device__ __forceinline__ void direct_fast(const DirectArgs& a, const T* s) {
     for (int i = 0; i < DR_WZ; ++i)
 #pragma unroll
         for (int j = 0; j < DR_WY; ++j) {
+            const int r = (i - DR_BI0) * DR_BNJ + (j - DR_BJ0);   // row of the gathered block
             if (DR_NEED[i][j][0]) {
-                P2 sh;
+                P2 sh, far = beyond[i][j];
                 sh[0] = from_prev_lane(win[i][j][DR_HK][0]);
                 sh[1] = from_prev_lane(win[i][j][DR_HK][1]);
-                win[i][j][0] = first ? beyond[i][j] : sh;
+                if (DR_EDGE_GATHER) {
+                    far[0] = from_lane(edge[0], 2 * r);
+                    far[1] = from_lane(edge[1], 2 * r);
+                }
+                win[i][j][0] = first ? far : sh;
             }
             if (DR_NEED[i][j][DR_WK - 1]) {
-                P2 sh;
+                P2 sh, far = beyond[i][j];
                 sh[0] = from_next_lane(win[i][j][DR_HK][0]);
                 sh[1] = from_next_lane(win[i][j][DR_HK][1]);
-                win[i][j][DR_WK - 1] = last ? beyond[i][j] : sh;
+                if (DR_EDGE_GATHER) {
+                    far[0] = from_lane(edge[0], 2 * r + 1);
+                    far[1] = from_lane(edge[1], 2 * r + 1);
+                }
+                win[i][j][DR_WK - 1] = last ? far : sh;
             }
         }
     T* const out_tile = a.dst[p.t];

@@ -429,3 +429,40 @@ def test_two_shifted_arrays_fall_back_to_the_gather(itf):
     hv[1:-1, 1:-1] = hu[:-2, 1:-1] + hw[2:, 1:-1]
     assert np.array_equal(v.get(itf), hv)
     assert _kernels(itf) == ["gather"]
+
+
+# ---- both register-window kernels in both ranks ----
+
+@pytest.mark.parametrize("lean", [0, 1])
+@pytest.mark.parametrize("shape,tile", [((20, 40, 384), 128), ((300, 512), 128)])
+def test_stencil_kernels_with_and_without_lane_exchange(itf, shape, tile, lean):
+    """The wavefront-level kernel (neighbours in x by lane exchange, the pairs beyond the
+    wavefront's 128 columns gathered by one load) and the general one give the same bits; by
+    default rank 2 takes the first and rank 3 the second, here each rank runs both."""
+    from charmnumeric_amd import _lib as L
+    nd = len(shape)
+    itf.set_min_tile(nd, tile)
+    L.check(L.lib.cnh_set_option(b"direct_lean", lean))
+    try:
+        rng = np.random.default_rng(lean + nd)
+        hu, hf = rng.standard_normal(shape), rng.standard_normal(shape)
+        u, f = cnp.array(hu), cnp.array(hf)
+        inner = (slice(1, -1),) * nd
+
+        def neighbours(x):
+            out = None
+            for d in range(nd):
+                for s in (slice(0, -2), slice(2, None)):
+                    key = list(inner)
+                    key[d] = s
+                    out = x[tuple(key)] if out is None else out + x[tuple(key)]
+            return out
+
+        itf.set_trace()
+        for _ in range(3):
+            u[inner] = (1.0 / (2 * nd)) * (neighbours(u) + f[inner])
+            hu[inner] = (1.0 / (2 * nd)) * (neighbours(hu) + hf[inner])
+        assert np.array_equal(u.get(itf), hu)
+        assert _kernels(itf) == ["direct"] * 3
+    finally:
+        L.check(L.lib.cnh_set_option(b"direct_lean", -1))
