@@ -176,7 +176,7 @@ std::string direct_source(const GroupProgram& p, const DirectConfig& cfg, std::s
         s << (l ? ", " : "") << sh.other[l];
     s << "};\n";
     // Rows of the window whose first or last lane needs the pair beyond the wavefront's 128
-    // columns. When they form a full block of at most 32 rows, one partial load per wavefront
+    // columns. When they form a full block of 4 to 32 rows, one partial load per wavefront
     // fetches all of them (lane 2r + side for row r) and lanes 0 and 63 pick theirs by readlane.
     int bi0 = WZ, bi1 = -1, bj0 = WY, bj1 = -1, brows = 0;
     for (int z = 0; z < WZ; ++z)
@@ -188,7 +188,8 @@ std::string direct_source(const GroupProgram& p, const DirectConfig& cfg, std::s
                 bj1 = std::max(bj1, y);
                 ++brows;
             }
-    const bool gather = brows > 0 && brows == (bi1 - bi0 + 1) * (bj1 - bj0 + 1) && brows <= 32 && HK == 1;
+    // (with two rows, rank 2, the row-by-row form measured 0.7 % faster: 184.0 against 185.3 us)
+    const bool gather = brows >= 4 && brows == (bi1 - bi0 + 1) * (bj1 - bj0 + 1) && brows <= 32 && HK == 1;
     s << "#define DR_EDGE_GATHER " << (gather ? 1 : 0) << "\n#define DR_BI0 " << (gather ? bi0 : 0)
       << "\n#define DR_BJ0 " << (gather ? bj0 : 0) << "\n#define DR_BNJ " << (gather ? bj1 - bj0 + 1 : 1)
       << "\n#define DR_NB " << (gather ? brows : 0) << "\n";
