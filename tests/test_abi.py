@@ -34,6 +34,9 @@ def test_struct_layouts_match_header():
     assert L.AstNode.region.offset == 144
     assert C.sizeof(L.Memref) == 72
     assert C.sizeof(L.Tiled) == 88 and L.Tiled.pitch.offset == 64
+    assert C.sizeof(L.GemmJob) == 72 and L.GemmJob.C.offset == 56
+    assert C.sizeof(L.GemvPanel) == 32 and L.GemvPanel.xoff.offset == 24
+    assert C.sizeof(L.Decomp) == 40 and L.Decomp.tile.offset == 32
 
 
 def test_scalar_conversion():
