@@ -456,3 +456,39 @@ def test_random_dags_give_power_of_two_tiles_and_finite_offsets():
             assert all(abs(o) < (1 << 24) for o in offset), (case, name, offset)
             if final:
                 assert (tile, offset) == (tile0, off0), (case, name)
+
+
+def test_the_seven_known_answers_of_the_golden_file():
+    """The same seven cases, with inputs and expectations taken from the committed fixture."""
+    from tests import helpers as H
+    cases = {c["name"]: c for c in H.golden()["decomposition_offsets"]["cases"]}
+    assert len(cases) == 7
+
+    def as_tuple(v):
+        return tuple(v) if isinstance(v, list) else (v,)
+
+    for name in ("shifted_copy_uses_absolute_offset", "shifted_copy_from_nonzero_source_offset",
+                 "strided_copy_reduces_tile_and_sets_offset"):
+        c = cases[name]
+        src, (lo, hi, step) = c["source_array"], c["copy_region"]
+        count = (hi - lo + step - 1) // step
+        out = solve({1: ((src["size"],), (src["offset"],), src["tile"], True),
+                     2: ((count,), (0,), src["tile"] if step > 1 else 0, False)},
+                    message(copy_node(2, 1, reg([lo], [hi], [step]))))
+        assert out[2] == (c["expect"]["tile"], as_tuple(c["expect"]["offset"])), name
+        assert out[2][1][0] % out[2][0] == c["expect"]["phase"], name
+    c = cases["shifted_expression_temp_uses_absolute_representative"]
+    w = lazy._NodeWriter()
+    a = w.leaf(Ref(1, 1))
+    w.op(10, L.OP_ADD, True, 1, L.F64, [a, a], [reg([r[0]], [r[1]], [r[2]]) for r in c["operand_regions"]])
+    s0, s1, s2 = c["set_region"]
+    w.op(11, L.OP_SET_REGION, False, 1, L.F64, [a, w.leaf(Ref(10, 1))], [None, None], region=reg([s0], [s1], [s2]))
+    out = solve({1: ((512,), (0,), 64, True), 10: ((s1 - s0,), (0,), 0, False)}, message(w))
+    assert out[10] == (c["expect"]["tile"], (c["expect"]["offset"],))
+    assert out[1][1] == (c["expect"]["target_offset"],)
+    for nd, name in ((1, "jacobi1d_temp_offset"), (2, "jacobi2d_temp_offset"), (3, "jacobi3d_temp_offset")):
+        c = cases[name]
+        n = c["shape"][0]
+        arrays, msg, (ts, tw) = jacobi_like(nd, n, with_source=nd < 3)
+        out = solve(arrays, msg)
+        assert out[ts] == out[tw] == (c["expect"]["tile"], as_tuple(c["expect"]["offset"])), name
