@@ -878,8 +878,10 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
     // Two launches over the same grid: wavefronts that lie inside their tile in y and z take the
     // lean kernel, the other kernel does what is left (all of it when the lean one does not apply).
     // measured on MI355X: the lean kernel pays off for rank 2 (tiles much wider than a wavefront
-    // run); with 128-wide tiles of rank 3 every wavefront reads both x neighbours and it does not
-    const bool want_lean = g_direct_lean < 0 ? nd == 2 : g_direct_lean != 0;
+    // run: 8192^2 183 against 200 us); with the 128-wide tiles of rank 3 every wavefront reads both
+    // x neighbours, and it pays a little once those reads are one gathered load per wavefront
+    // (512^3: 424.0 against 430.7 us, six alternating runs)
+    const bool want_lean = g_direct_lean < 0 ? true : g_direct_lean != 0;
     const bool lean = want_lean && sh.tx % 64 == 0 && sh.halo[2] >= 1;
     int skip_fast = lean ? 1 : 0;
     hipFunction_t fn;

@@ -92,7 +92,7 @@ int cnh_version(void);
  *   "stencil_mode"   kernel cnh_launch_group_tiles uses for same-array unit-step stencils:
  *                    2 (default) register window, 1 LDS sliding window, 0 general gather
  *   "direct_tx/ry/rz"  register window: lanes along x per workgroup row, rows and planes per lane
- *   "direct_lean"    wavefront-level lean kernel with lane exchange: 1 on, 0 off, -1 (default) rank 2 only
+ *   "direct_lean"    wavefront-level lean kernel with lane exchange: 1 on, 0 off, -1 (default) on
  *   "direct_group"   workgroup order for rank 3: 0 (default) tile by tile, 1 groups of G^3 tiles,
  *                    2 rows of tiles along x
  *   "direct_stagger" concurrent groups start at different places of their tiles (default 0)

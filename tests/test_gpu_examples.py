@@ -437,8 +437,8 @@ def test_two_shifted_arrays_fall_back_to_the_gather(itf):
 @pytest.mark.parametrize("shape,tile", [((20, 40, 384), 128), ((300, 512), 128)])
 def test_stencil_kernels_with_and_without_lane_exchange(itf, shape, tile, lean):
     """The wavefront-level kernel (neighbours in x by lane exchange, the pairs beyond the
-    wavefront's 128 columns gathered by one load) and the general one give the same bits; by
-    default rank 2 takes the first and rank 3 the second, here each rank runs both."""
+    wavefront's 128 columns gathered by one load) and the general one give the same bits; the first
+    is the default, here each rank runs both."""
     from charmnumeric_amd import _lib as L
     nd = len(shape)
     itf.set_min_tile(nd, tile)
