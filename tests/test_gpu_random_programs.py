@@ -3,7 +3,7 @@ drawn from what the frontend offers (element-wise expressions over shifted and s
 assignments into slices from expressions, literals and other slices, copies, named temporaries,
 sums, dots and products on windows). NumPy runs the same statements in the same order. Element-wise
 results must agree bit for bit; reductions and products to 1e-12 of the sum of absolute terms
-(1e-5 in the fp32 programs).
+(1e-5 in the fp32 programs). Integer programs (wrap-around arithmetic) are element-wise only.
 Every program runs twice: with the tile rule alone and with the decomposition solver laying the
 arrays out (tiles that do not start at element 0)."""
 import numpy as np
@@ -43,7 +43,13 @@ class Program:
         self.rel = 1e-12 if dtype == np.float64 else 1e-5
         edge = {1: (150, 400), 2: (20, 70), 3: (9, 26)}[rank]
         self.shape = tuple(int(self.rng.integers(*edge)) for _ in range(rank))
-        self.host = [self.rng.standard_normal(self.shape).astype(dtype) for _ in range(3)]
+        self.integer = np.issubdtype(dtype, np.integer)
+        if self.integer:        # values near the top of the range: sums and products wrap around
+            info = np.iinfo(dtype)
+            self.host = [self.rng.integers(info.min // 2, info.max // 2, self.shape, dtype=dtype)
+                         for _ in range(3)]
+        else:
+            self.host = [self.rng.standard_normal(self.shape).astype(dtype) for _ in range(3)]
         self.dev = [cnp.array(h) for h in self.host]
         self.checks = []     # (device value, host value, kind)
 
@@ -67,8 +73,8 @@ class Program:
             terms.append((self.dev[i][k], self.host[i][k]))
         d, h = terms[0]
         for td, th in terms[1:]:
-            op = int(rng.integers(0, 4))
-            c = float(rng.choice([0.5, 2.0, -1.25, 3.0]))
+            op = int(rng.integers(0, 3 if self.integer else 4))
+            c = int(rng.choice([2, -3, 5])) if self.integer else float(rng.choice([0.5, 2.0, -1.25, 3.0]))
             if op == 0:
                 d, h = d + td, h + th
             elif op == 1:
@@ -84,6 +90,8 @@ class Program:
         kind = int(rng.integers(0, 8))
         key, other = self.key_pair()
         t = int(rng.integers(0, 3))
+        if self.integer and kind in (1, 3, 6, 7):       # integer programs: element-wise work only
+            kind = 0
         if kind == 0:                                   # slice = expression of slices
             d, h = self.expression([key, other])
             self.dev[t][key] = d
@@ -169,7 +177,8 @@ def test_random_program(seed, rank, solver):
     itf.set_pipeline(seed % 2 == 1)       # odd seeds: messages queue for the executor's own thread
     cnp.set_auto_flush(itf, int(np.random.default_rng(seed).choice([4, 16, 1000])))
     try:
-        prog = Program(1000 * rank + seed, rank, np.float32 if seed % 5 == 4 else np.float64)
+        dtype = {4: np.float32, 3: np.int64, 8: np.int32}.get(seed % 10, np.float64)
+        prog = Program(1000 * rank + seed, rank, dtype)
         for _ in range(18):
             prog.statement()
         prog.verify(itf)
