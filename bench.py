@@ -120,7 +120,10 @@ def cg_asts(L):
     return scalar_div(), axpy(L.OP_ADD), axpy(L.OP_SUB)
 
 
-def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True):
+def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True, trace_iters=0):
+    """`steps` timed CG iterations. With trace_iters > 0 an untimed pass over the same system runs
+    first and reads alpha, beta and r.r back after each of its iterations (and x at its end):
+    what the parity check against the CPU leg compares."""
     tile = tile_rule_tile or cg_tile(n)
     g = (n + tile - 1) // tile
     t0 = time.time()
@@ -143,13 +146,15 @@ def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True):
     mr = lambda b_, cnt=n: L.Memref.dense(b_.ptr, (cnt,))
     smr = lambda i: L.Memref.dense(S(i), (1,))
 
+    state = {}
+
     def reset():
+        # x = 0, r = p = b, r.r; the ping-pong roles go back to their starting assignment too
+        state.update({"x": x, "r": r, "p": p, "x2": x2, "r2": r2, "p2": p2, "rtr": 0, "rtr_new": 3})
         L.check(L.lib.cnh_memset0(x.ptr, n * 8, None))
         L.check(L.lib.cnh_d2d(r.ptr, bvec.ptr, n * 8, None))
         L.check(L.lib.cnh_d2d(p.ptr, bvec.ptr, n * 8, None))
         L.check(L.lib.cnh_dot_partial(L.F64, n, r.ptr, r.ptr, S(0), None))
-
-    state = {"x": x, "r": r, "p": p, "x2": x2, "r2": r2, "p2": p2, "rtr": 0, "rtr_new": 3}
 
     def iteration(ev=None, i=0):
         st = state
@@ -176,6 +181,18 @@ def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True):
     L.check(L.lib.cnh_device_sync())
     setup_s = time.time() - t0
 
+    trace = None
+    if trace_iters > 0:
+        reset()
+        trace = {"alpha": [], "beta": [], "rtr": []}
+        for _ in range(trace_iters):
+            iteration()
+            v = sc.get(np.float64)           # waits for the iteration
+            trace["alpha"].append(float(v[2]))
+            trace["beta"].append(float(v[4]))
+            trace["rtr"].append(float(v[state["rtr"]]))
+        trace["x"] = state["x"].get()
+
     reset()
     ev = Events(L, steps)
     e0, e1 = C.c_void_p(), C.c_void_p()
@@ -199,6 +216,7 @@ def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True):
         "setup_s": setup_s,
         "rtr_final": float(sc.get(np.float64)[state["rtr"]]),
         "x": state["x"].get() if check else None,
+        "trace": trace,
     }
     ev.free()
     for b_ in tiles + [bvec, x, r, p, Ap, x2, r2, p2, sc]:
@@ -226,8 +244,10 @@ def cpu_cg_setup(n, seed=2):
     return orc, tile, g, tiles, b
 
 
-def cpu_cg(setup, n, iters, threads):
-    """CG with the oracle's kernels in the reference's order of operations; returns (it/s, x, rtr)."""
+def cpu_cg(setup, n, iters, threads, keep_x_at=None):
+    """CG with the oracle's kernels in the reference's order of operations; returns
+    (it/s, x, rtr, trace) where trace holds alpha, beta and r.r of every iteration and, with
+    keep_x_at = k, a copy of x after k iterations."""
     from oracle import cn_oracle as O
 
     orc, tile, g, tiles, b = setup
@@ -238,8 +258,9 @@ def cpu_cg(setup, n, iters, threads):
     rtr = orc.dot(r, r)
     Ap = np.zeros(n)
     part = np.zeros(tile)
+    trace = {"alpha": [], "beta": [], "rtr": [], "x": None, "rtr0": rtr}
     t0 = time.perf_counter()
-    for _ in range(iters):
+    for it in range(iters):
         # tile GEMV + partial accumulate on the 1-D owner, column tiles in order
         for i in range(g):
             rows = tiles[i][0].shape[0]
@@ -261,8 +282,32 @@ def cpu_cg(setup, n, iters, threads):
         beta = rtr_new / rtr
         p = r + beta * p
         rtr = rtr_new
+        trace["alpha"].append(alpha)
+        trace["beta"].append(beta)
+        trace["rtr"].append(rtr)
+        if keep_x_at == it + 1:
+            trace["x"] = x.copy()
     dt = time.perf_counter() - t0
-    return iters / dt, x, rtr
+    return iters / dt, x, rtr, trace
+
+
+def cg_parity(gpu_trace, cpu_trace, rtr0, floor=1e-24):
+    """Agreement of the device's CG with the CPU leg on the same system: the solutions after the
+    same number of iterations, and alpha, beta, r.r of every iteration whose r.r is still above
+    `floor` times the initial one. Below that the recursion works on rounding noise (on this system
+    from the sixth iteration on) and two correct implementations differ by factors."""
+    n = min(len(gpu_trace["alpha"]), len(cpu_trace["alpha"]))
+    k = 0
+    while k < n and cpu_trace["rtr"][k] >= floor * rtr0:
+        k += 1
+    out = {"iterations_compared": n, "scalar_iterations": k}
+    for key in ("alpha", "beta", "rtr"):
+        g = np.array(gpu_trace[key][:k])
+        c = np.array(cpu_trace[key][:k])
+        out[f"{key}_max_rel_dev"] = float(np.max(np.abs(g - c) / np.abs(c))) if k else None
+    xc = cpu_trace["x"]
+    out["x_max_rel_diff"] = float(np.max(np.abs(gpu_trace["x"] - xc)) / np.max(np.abs(xc)))
+    return out
 
 
 # -------------------------------------------------------------------------------------------------
@@ -834,7 +879,8 @@ def main():
     name = C.create_string_buffer(256)
     L.check(L.lib.cnh_device_name(name, 256))
     n = args.n
-    cg = run_cg(L, n, args.steps, args.warmup)
+    parity_iters = 0 if args.no_cpu else min(args.steps, args.cpu_iters)
+    cg = run_cg(L, n, args.steps, args.warmup, trace_iters=parity_iters)
     gemv_bytes = 8.0 * n * n + 2 * 8.0 * n
     achieved = gemv_bytes / (cg["gemv_avg_us"] * 1e-6) / 1e9
     line = {
@@ -856,6 +902,8 @@ def main():
         "roofline": {"bound": "hbm", "kernel": "gemv_rows<double>", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": GEMV_N16384_TRAFFIC_BYTES if n == 16384 else None,
+                     "traffic_source": "rocprofv3 --pmc counters of an earlier run of this kernel "
+                                       "(profiles/bench_hbm_traffic_pmc.txt), not measured in this run",
                      "avg_us": round(cg["gemv_avg_us"], 2),
                      "bytes_per_launch": gemv_bytes},
         "gemv_roofline_iters_per_s": round(HBM_PEAK_GBS * 1e9 / gemv_bytes, 1),
@@ -888,8 +936,8 @@ def main():
         cores = os.cpu_count() or 1
         threads = min(cores, 16)
         setup = cpu_cg_setup(n)
-        ips1, xc, rtr_c = cpu_cg(setup, n, args.cpu_iters, 1)
-        ipsN, _, _ = cpu_cg(setup, n, args.cpu_iters, threads)
+        ips1, _, _, _ = cpu_cg(setup, n, args.cpu_iters, 1)
+        ipsN, _, _, cpu_trace = cpu_cg(setup, n, args.cpu_iters, threads, keep_x_at=parity_iters)
         line["cpu_baseline"] = {
             "value": round(ipsN, 3), "unit": "iterations/s", "cores": threads, "kind": "port",
             "sample": f"same system (n={n}, {cg['tile']}^2 tiles), {args.cpu_iters} CG iterations, "
@@ -902,9 +950,11 @@ def main():
                 line["also"]["c4_jacobi3d_512"]["cpu_port"] = cpu_jacobi(3, 512, 128, 2, threads)
             except Exception as exc:
                 line["also"]["cpu_port_error"] = str(exc)
-        if args.cpu_iters == args.steps and cg.get("x") is not None:
-            # same system, same number of iterations: the two solutions must agree
-            line["cg_parity_max_rel_diff"] = float(np.max(np.abs(cg["x"] - xc)) / np.max(np.abs(xc)))
+        # same system, same number of iterations (an untimed pass of the device path before the
+        # timed one): the two solutions and the per-iteration scalars must agree
+        par = cg_parity(cg["trace"], cpu_trace, cpu_trace["rtr0"])
+        line["cg_parity_max_rel_diff"] = par["x_max_rel_diff"]
+        line["cg_parity"] = par
     print(json.dumps(line))
 
 

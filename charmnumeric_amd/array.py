@@ -159,15 +159,24 @@ def region_shape(region):
 
 
 def compose(outer, inner):
-    """Region `inner` (relative to the view `outer`) expressed relative to outer's base array."""
+    """Region `inner` (relative to the view `outer`) expressed relative to outer's base array.
+    The stop is one past the last selected element, so a region taken through a strided view never
+    reaches beyond the view's own last element (`a[::4][:]` on 10 elements is [0:9:4], not
+    [0:12:4]); upstream keeps the outer region as it is when the inner one is the whole view
+    (charmnumeric.py:215-220 upstream), with the same effect."""
     if outer is None:
         return inner
     ostart, _, ostep = outer
     istart, istop, istep = inner
     nd = len(istart)
-    return (tuple(ostart[d] + istart[d] * ostep[d] for d in range(nd)),
-            tuple(ostart[d] + istop[d] * ostep[d] for d in range(nd)),
-            tuple(ostep[d] * istep[d] for d in range(nd)))
+    start, stop, step = [], [], []
+    for d in range(nd):
+        count = max(0, (istop[d] - istart[d] + istep[d] - 1) // istep[d])
+        first = ostart[d] + istart[d] * ostep[d]
+        start.append(first)
+        step.append(ostep[d] * istep[d])
+        stop.append(first + (count - 1) * step[-1] + 1 if count else first)
+    return tuple(start), tuple(stop), tuple(step)
 
 
 def _is_whole(region, shape):
@@ -567,136 +576,152 @@ def _matvec(mat, vec):
 
 # ---------------------------------------------------------------------------------------------
 # creation
+#
+# Every constructor ends in one of two recorded forms: CREATE alone (the executor zero-fills new
+# arrays), CREATE followed by either one fill (constant contents) or one bulk upload. Host values
+# pass through _HostValues, which settles rank, dtype and broadcasting once for all constructors.
+
+
+class _HostValues:
+    """Host-side contents for a device array: a NumPy array of a wire dtype, rank >= 1."""
+
+    __slots__ = ("data",)
+
+    def __init__(self, values, dtype=None, copy=False, ndmin=0, broadcast=None, what="input"):
+        want = _normalize_dtype(dtype, allow_none=True)
+        data = np.array(values, dtype=want, copy=True) if copy else np.asarray(values, dtype=want)
+        if data.ndim < ndmin:
+            data = data.reshape((1,) * (ndmin - data.ndim) + data.shape)
+        if broadcast is not None and data.ndim > 0:
+            try:
+                data = np.broadcast_to(data, broadcast)
+            except ValueError as exc:
+                label = "fill_value" if what == "fill_value" else "input"
+                raise ValueError(f"could not broadcast {label} from shape {data.shape} into shape "
+                                 f"{tuple(broadcast)}") from exc
+        self.data = data
+
+    @property
+    def is_scalar(self):
+        return self.data.ndim == 0
+
+    def constant(self):
+        """The single value all elements share, or None."""
+        flat = self.data.reshape(-1)
+        if flat.size and (flat.size == 1 or bool(np.all(flat == flat[0]))):
+            return flat[0]
+        return None
+
+    def upload(self):
+        """A new device array holding these values."""
+        if self.is_scalar:
+            raise NotImplementedError("0D charmnumeric arrays are not supported yet")
+        out = create_array(self.data.shape, dtype=_normalize_dtype(self.data.dtype))
+        return _assign_host_data(out, self.data)
 
 
 def create_array(shape, dtype=_DEFAULT_DTYPE):
-    shape = _normalize_shape(shape)
-    dtype = _normalize_dtype(dtype)
-    out = Array(shape, dtype)
-    lazy.record(lazy.Instr("create", name=out.name, shape=shape, dtype=out.wire_dtype()))
+    out = Array(_normalize_shape(shape), _normalize_dtype(dtype))
+    lazy.record(lazy.Instr("create", name=out.name, shape=out.shape, dtype=out.wire_dtype()))
     return out
 
 
-def empty(shape, dtype=_DEFAULT_DTYPE):
-    return create_array(shape, dtype=dtype)
-
-
-def zeros(shape, dtype=_DEFAULT_DTYPE):
-    return create_array(shape, dtype=dtype)       # new arrays are zero-filled by the executor
-
-
 def _assign_host_data(target, values):
-    """Whole-array load from host data. A constant array becomes one fill; anything else one bulk
-    upload (upstream assigns element by element here, charmnumeric.py:863-878)."""
-    host = np.ascontiguousarray(values, dtype=target.dtype)
-    if host.shape != tuple(target.shape):
-        raise ValueError(f"cannot assign data with shape {host.shape} into shape {target.shape}")
-    first = host.reshape(-1)[0]
-    if host.size == 1 or np.all(host == first):
-        target[...] = _coerce_scalar(first)
+    """Whole-array load from host data: one fill when all elements are equal, else one bulk upload
+    (upstream assigns element by element here, charmnumeric.py:863-878)."""
+    src = _HostValues(values, dtype=target.dtype)
+    if src.data.shape != tuple(target.shape):
+        raise ValueError(f"cannot assign data with shape {src.data.shape} into shape {target.shape}")
+    if src.data.size == 0:
         return target
-    lazy.record(lazy.Instr("call", name=target.name, opcode="put", shape=target.shape,
-                           dtype=target.wire_dtype(), payload=host.copy()))
+    same = src.constant()
+    if same is not None:
+        target[...] = _coerce_scalar(same)
+    else:
+        lazy.record(lazy.Instr("call", name=target.name, opcode="put", shape=target.shape,
+                               dtype=target.wire_dtype(), payload=np.ascontiguousarray(src.data).copy()))
     return target
 
 
-def _from_host(values, dtype=None, copy=True, ndmin=0):
-    host = np.array(values, dtype=_normalize_dtype(dtype, allow_none=True), copy=copy)
-    while host.ndim < ndmin:
-        host = host[None]
-    if host.ndim == 0:
-        raise NotImplementedError("0D charmnumeric arrays are not supported yet")
-    out = create_array(host.shape, dtype=_normalize_dtype(host.dtype))
-    return _assign_host_data(out, host)
-
-
 def _coerce_assignment_operand(rhs, shape, dtype):
+    """Right-hand side of an assignment: device objects and scalars pass, host data is uploaded."""
     if isinstance(rhs, _ArrayLike):
         return rhs
     if _is_scalar_like(rhs):
         return _coerce_scalar(rhs)
-    host = np.asarray(rhs, dtype=dtype)
-    if host.ndim == 0:
-        return _coerce_scalar(host.item())
-    try:
-        host = np.broadcast_to(host, shape)
-    except ValueError as exc:
-        raise ValueError(f"could not broadcast input from shape {host.shape} into shape {shape}") from exc
-    return _from_host(host, dtype=host.dtype)
+    src = _HostValues(rhs, dtype=dtype, broadcast=shape)
+    return _coerce_scalar(src.data.item()) if src.is_scalar else src.upload()
+
+
+def empty(shape, dtype=_DEFAULT_DTYPE):
+    return create_array(shape, dtype)
+
+
+zeros = empty          # new arrays are zero-filled by the executor
 
 
 def full(shape, fill_value, dtype=None):
     shape = _normalize_shape(shape)
-    if _is_scalar_like(fill_value):
-        dt = _normalize_dtype(dtype, allow_none=True)
-        if dt is None:
-            dt = _normalize_dtype(np.asarray(fill_value).dtype)
-        out = empty(shape, dtype=dt)
-        out[...] = _coerce_scalar(fill_value)
-        return out
-    host = np.asarray(fill_value, dtype=_normalize_dtype(dtype, allow_none=True))
-    try:
-        host = np.broadcast_to(host, shape)
-    except ValueError as exc:
-        raise ValueError(f"could not broadcast fill_value from shape {host.shape} into shape {shape}") from exc
-    return _from_host(host, dtype=host.dtype)
+    src = None if _is_scalar_like(fill_value) else _HostValues(fill_value, dtype=dtype, broadcast=shape,
+                                                                what="fill_value")
+    if src is not None and not src.is_scalar:
+        return src.upload()
+    value = fill_value if src is None else src.data.item()
+    dt = _normalize_dtype(dtype, allow_none=True) or _normalize_dtype(np.asarray(value).dtype)
+    out = create_array(shape, dt)
+    out[...] = _coerce_scalar(value)
+    return out
 
 
 def ones(shape, dtype=_DEFAULT_DTYPE):
     return full(shape, 1, dtype=dtype)
 
 
-def _like(a, dtype, shape):
-    if isinstance(a, _ArrayLike):
-        s, d = a.shape, a.dtype
-    else:
-        host = np.asarray(a)
-        if host.ndim == 0:
-            raise NotImplementedError("0D charmnumeric arrays are not supported yet")
-        s, d = host.shape, _normalize_dtype(host.dtype)
-    return (s if shape is None else _normalize_shape(shape)), (d if dtype is None else _normalize_dtype(dtype))
+def _like_constructor(make, doc):
+    """X_like(a, ..., dtype=None, shape=None): shape and dtype of `a` unless overridden."""
+    def ctor(a, *args, dtype=None, shape=None):
+        if isinstance(a, _ArrayLike):
+            s, d = a.shape, a.dtype
+        else:
+            host = np.asarray(a)
+            if host.ndim == 0:
+                raise NotImplementedError("0D charmnumeric arrays are not supported yet")
+            s, d = host.shape, _normalize_dtype(host.dtype)
+        return make(s if shape is None else _normalize_shape(shape), *args,
+                    dtype=d if dtype is None else _normalize_dtype(dtype))
+    ctor.__doc__ = doc
+    return ctor
 
 
-def empty_like(a, dtype=None, shape=None):
-    s, d = _like(a, dtype, shape)
-    return empty(s, dtype=d)
+empty_like = _like_constructor(empty, "empty_like(a, dtype=None, shape=None)")
+zeros_like = _like_constructor(zeros, "zeros_like(a, dtype=None, shape=None)")
+ones_like = _like_constructor(ones, "ones_like(a, dtype=None, shape=None)")
+full_like = _like_constructor(full, "full_like(a, fill_value, dtype=None, shape=None)")
 
 
-def zeros_like(a, dtype=None, shape=None):
-    s, d = _like(a, dtype, shape)
-    return zeros(s, dtype=d)
-
-
-def ones_like(a, dtype=None, shape=None):
-    s, d = _like(a, dtype, shape)
-    return ones(s, dtype=d)
-
-
-def full_like(a, fill_value, dtype=None, shape=None):
-    s, d = _like(a, dtype, shape)
-    return full(s, fill_value, dtype=d)
+def _existing(a, dtype):
+    """`a` when it is a device object of the requested dtype (None for host data)."""
+    if not isinstance(a, _ArrayLike):
+        return None
+    want = _normalize_dtype(dtype, allow_none=True)
+    if want is not None and want != a.dtype:
+        raise NotImplementedError(
+            "dtype conversion for existing charmnumeric arrays is not implemented yet")
+    return a
 
 
 def asarray(a, dtype=None):
-    want = _normalize_dtype(dtype, allow_none=True)
-    if isinstance(a, _ArrayLike):
-        if want is None or want == a.dtype:
-            return a
-        raise NotImplementedError(
-            "dtype conversion for existing charmnumeric arrays is not implemented yet")
-    return _from_host(a, dtype=want, copy=False)
+    have = _existing(a, dtype)
+    return have if have is not None else _HostValues(a, dtype=dtype).upload()
 
 
 def array(a, dtype=None, copy=True, ndmin=0):
-    want = _normalize_dtype(dtype, allow_none=True)
-    if isinstance(a, _ArrayLike):
-        if want is not None and want != a.dtype:
-            raise NotImplementedError(
-                "dtype conversion for existing charmnumeric arrays is not implemented yet")
-        if len(a.shape) < ndmin:
-            raise NotImplementedError("ndmin on an existing charmnumeric array is not implemented")
-        return a.copy() if copy else a
-    return _from_host(a, dtype=want, copy=copy, ndmin=ndmin)
+    have = _existing(a, dtype)
+    if have is None:
+        return _HostValues(a, dtype=dtype, copy=copy, ndmin=ndmin).upload()
+    if len(have.shape) < ndmin:
+        raise NotImplementedError("ndmin on an existing charmnumeric array is not implemented")
+    return have.copy() if copy else have
 
 
 def copy(a, order="K"):
@@ -711,14 +736,13 @@ def copyto(dst, src):
 
 
 def arange(start, stop=None, step=1, dtype=None):
-    host = np.arange(start, stop, step, dtype=_normalize_dtype(dtype, allow_none=True))
-    return _from_host(host, dtype=host.dtype, copy=False)
+    return _HostValues(np.arange(start, stop, step, dtype=_normalize_dtype(dtype, allow_none=True))).upload()
 
 
 def eye(N, M=None, k=0, dtype=_DEFAULT_DTYPE):
     rows = int(N)
     cols = rows if M is None else int(M)
-    return _from_host(np.eye(rows, cols, int(k), dtype=_normalize_dtype(dtype)))
+    return _HostValues(np.eye(rows, cols, int(k), dtype=_normalize_dtype(dtype))).upload()
 
 
 def identity(n, dtype=_DEFAULT_DTYPE):

@@ -9,6 +9,7 @@
 #include <string>
 
 #include "../../include/cnhip.h"
+#include "../../include/cnbench.h"
 
 namespace cnh {
 
@@ -44,6 +45,8 @@ inline hipStream_t as_stream(cnh_stream s) { return reinterpret_cast<hipStream_t
 
 // Lazily selects the device on first use of any entry point.
 int ensure_init();
+// The device cnh_init selected, -1 before the first call.
+int current_device();
 
 // Device scratch for reduction partials, one region per stream handle so that calls on
 // different streams never share slots. Returns a device pointer to `bytes` bytes.

@@ -30,24 +30,34 @@ namespace {
 std::mutex g_mu;
 bool g_inited = false;
 int g_device = 0;
+constexpr int kMaxDevices = 64;
 
 struct Workspace {
     void* ptr = nullptr;
     size_t bytes = 0;
+    std::vector<void*> retired; // outgrown blocks, possibly still read by kernels in flight
 };
-std::unordered_map<hipStream_t, Workspace> g_ws;
 
-// Descriptor slab: device memory + pinned host mirror, bump-allocated.
-const size_t kSlabBytes = 16u << 20;
-char* g_slab_dev = nullptr;
-char* g_slab_host = nullptr;
-size_t g_slab_used = 0;
 struct DescEntry {
     size_t off, bytes;
     hipStream_t stream; // where the copy was queued
     bool visible;       // known complete for every stream
 };
-std::unordered_map<uint64_t, std::vector<DescEntry>> g_desc;
+
+// Everything the library keeps in device memory belongs to one device.
+const size_t kSlabBytes = 16u << 20;
+struct DeviceState {
+    std::unordered_map<hipStream_t, Workspace> ws;
+    // Descriptor slab: device memory + pinned host mirror, bump-allocated.
+    char* slab_dev = nullptr;
+    char* slab_host = nullptr;
+    size_t slab_used = 0;
+    std::unordered_map<uint64_t, std::vector<DescEntry>> desc;
+    hipStream_t fill_stream = nullptr; // zero-fills of fresh allocations
+};
+DeviceState g_dev[kMaxDevices];
+
+DeviceState& dev_state() { return g_dev[g_device]; }
 
 uint64_t fnv1a(const void* p, size_t n) {
     const unsigned char* b = static_cast<const unsigned char*>(p);
@@ -58,6 +68,14 @@ uint64_t fnv1a(const void* p, size_t n) {
     }
     return h;
 }
+
+// Blocks a workspace outgrew are freed once the stream that used them has drained.
+int release_retired(Workspace& w) {
+    for (void* p : w.retired)
+        CNH_HIP(hipFree(p));
+    w.retired.clear();
+    return 0;
+}
 } // namespace
 
 int ensure_init() {
@@ -66,14 +84,19 @@ int ensure_init() {
     return cnh_init(0);
 }
 
+int current_device() { return g_inited ? g_device : -1; }
+
 int reduce_workspace(hipStream_t s, size_t bytes, void** out) {
     std::lock_guard<std::mutex> lk(g_mu);
-    Workspace& w = g_ws[s];
+    Workspace& w = dev_state().ws[s];
     if (w.bytes < bytes) {
-        // The old block may still be read by kernels in flight on `s`; it is parked, not freed.
         size_t want = bytes < (1u << 20) ? (1u << 20) : bytes;
         void* p = nullptr;
         CNH_HIP(hipMalloc(&p, want));
+        // The old block may still be read by kernels in flight on `s`: it waits in `retired` for
+        // the next synchronisation of that stream.
+        if (w.ptr)
+            w.retired.push_back(w.ptr);
         w.ptr = p;
         w.bytes = want;
     }
@@ -87,37 +110,38 @@ int reduce_workspace(hipStream_t s, size_t bytes, void** out) {
 // over the slab, and the slab is recycled only after the device has drained.
 int desc_upload(const void* host, size_t bytes, hipStream_t st, const void** dev_out) {
     std::lock_guard<std::mutex> lk(g_mu);
-    if (!g_slab_dev) {
-        CNH_HIP(hipMalloc((void**)&g_slab_dev, kSlabBytes));
-        CNH_HIP(hipHostMalloc((void**)&g_slab_host, kSlabBytes, hipHostMallocDefault));
+    DeviceState& D = dev_state();
+    if (!D.slab_dev) {
+        CNH_HIP(hipMalloc((void**)&D.slab_dev, kSlabBytes));
+        CNH_HIP(hipHostMalloc((void**)&D.slab_host, kSlabBytes, hipHostMallocDefault));
     }
     CNH_CHECK(bytes <= kSlabBytes / 4, -3, "descriptor table of %zu bytes is too large", bytes);
     uint64_t h = fnv1a(host, bytes);
-    auto it = g_desc.find(h);
-    if (it != g_desc.end())
+    auto it = D.desc.find(h);
+    if (it != D.desc.end())
         for (DescEntry& e : it->second)
-            if (e.bytes == bytes && std::memcmp(g_slab_host + e.off, host, bytes) == 0) {
+            if (e.bytes == bytes && std::memcmp(D.slab_host + e.off, host, bytes) == 0) {
                 if (!e.visible && e.stream != st) {
                     // uploaded on another stream: its copy must have landed before this one reads
                     CNH_HIP(hipStreamSynchronize(e.stream));
                     e.visible = true;
                 }
-                *dev_out = g_slab_dev + e.off;
+                *dev_out = D.slab_dev + e.off;
                 return 0;
             }
     size_t need = (bytes + 255) & ~size_t(255);
-    if (g_slab_used + need > kSlabBytes) {
+    if (D.slab_used + need > kSlabBytes) {
         // Tables handed out earlier may still be in use by queued kernels: drain, then recycle.
         CNH_HIP(hipDeviceSynchronize());
-        g_desc.clear();
-        g_slab_used = 0;
+        D.desc.clear();
+        D.slab_used = 0;
     }
-    size_t off = g_slab_used;
-    g_slab_used += need;
-    std::memcpy(g_slab_host + off, host, bytes);
-    CNH_HIP(hipMemcpyAsync(g_slab_dev + off, g_slab_host + off, bytes, hipMemcpyHostToDevice, st));
-    g_desc[h].push_back({off, bytes, st, false});
-    *dev_out = g_slab_dev + off;
+    size_t off = D.slab_used;
+    D.slab_used += need;
+    std::memcpy(D.slab_host + off, host, bytes);
+    CNH_HIP(hipMemcpyAsync(D.slab_dev + off, D.slab_host + off, bytes, hipMemcpyHostToDevice, st));
+    D.desc[h].push_back({off, bytes, st, false});
+    *dev_out = D.slab_dev + off;
     return 0;
 }
 
@@ -140,8 +164,11 @@ int cnh_init(int device) {
     if (e != hipSuccess || count <= 0)
         return set_error(-101, "no HIP device available (%s)",
                          e == hipSuccess ? "device count is 0" : hipGetErrorString(e));
-    CNH_CHECK(device >= 0 && device < count, -2, "device %d out of range (have %d)", device, count);
+    CNH_CHECK(device >= 0 && device < count && device < kMaxDevices, -2,
+              "device %d out of range (have %d)", device, count);
     CNH_HIP(hipSetDevice(device));
+    // Descriptor tables and reduction workspaces are kept per device, so a later call with
+    // another device finds its own (or none yet) and never one of this device.
     g_device = device;
     g_inited = true;
     return 0;
@@ -152,7 +179,9 @@ int cnh_device_name(char* buf, size_t cap) {
         return rc;
     hipDeviceProp_t prop;
     CNH_HIP(hipGetDeviceProperties(&prop, g_device));
-    snprintf(buf, cap, "%s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
+    // some driver stacks leave the marketing name empty
+    snprintf(buf, cap, "%s (%s, %d CUs)", prop.name[0] ? prop.name : "AMD GPU", prop.gcnArchName,
+             prop.multiProcessorCount);
     return 0;
 }
 
@@ -163,10 +192,19 @@ int cnh_alloc(size_t bytes, int zero, void** dptr) {
     void* p = nullptr;
     CNH_HIP(hipMalloc(&p, bytes ? bytes : 1));
     if (zero && bytes) {
-        // The fill runs on the null stream, which streams made by cnh_stream_create do not wait
-        // for: without the wait a first write queued on such a stream can be overtaken by it.
-        CNH_HIP(hipMemsetAsync(p, 0, bytes, nullptr));
-        CNH_HIP(hipStreamSynchronize(nullptr));
+        // The caller may first write the block on any stream, and no stream waits for another's
+        // fill by itself: the fill runs on a stream of the library's own and the host waits for
+        // that stream alone, so work queued elsewhere keeps running meanwhile.
+        hipStream_t fs;
+        {
+            std::lock_guard<std::mutex> lk(g_mu);
+            DeviceState& D = dev_state();
+            if (!D.fill_stream)
+                CNH_HIP(hipStreamCreateWithFlags(&D.fill_stream, hipStreamNonBlocking));
+            fs = D.fill_stream;
+        }
+        CNH_HIP(hipMemsetAsync(p, 0, bytes, fs));
+        CNH_HIP(hipStreamSynchronize(fs));
     }
     *dptr = p;
     return 0;
@@ -263,10 +301,20 @@ int cnh_stream_destroy(cnh_stream s) {
         // the copies land and mark them complete, so that no later call waits on a dead handle.
         std::lock_guard<std::mutex> lk(g_mu);
         CNH_HIP(hipStreamSynchronize(as_stream(s)));
-        for (auto& kv : g_desc)
+        DeviceState& D = dev_state();
+        for (auto& kv : D.desc)
             for (DescEntry& e : kv.second)
                 if (e.stream == as_stream(s))
                     e.visible = true;
+        // the stream's reduction workspace goes with it
+        auto it = D.ws.find(as_stream(s));
+        if (it != D.ws.end()) {
+            if (int rc = release_retired(it->second))
+                return rc;
+            if (it->second.ptr)
+                CNH_HIP(hipFree(it->second.ptr));
+            D.ws.erase(it);
+        }
     }
     CNH_HIP(hipStreamDestroy(as_stream(s)));
     return 0;
@@ -276,6 +324,10 @@ int cnh_stream_sync(cnh_stream s) {
     if (int rc = ensure_init())
         return rc;
     CNH_HIP(hipStreamSynchronize(as_stream(s)));
+    std::lock_guard<std::mutex> lk(g_mu);
+    auto it = dev_state().ws.find(as_stream(s));
+    if (it != dev_state().ws.end())
+        return release_retired(it->second);
     return 0;
 }
 
@@ -308,6 +360,10 @@ int cnh_device_sync(void) {
     if (int rc = ensure_init())
         return rc;
     CNH_HIP(hipDeviceSynchronize());
+    std::lock_guard<std::mutex> lk(g_mu);
+    for (auto& kv : dev_state().ws)
+        if (int rc = release_retired(kv.second))
+            return rc;
     return 0;
 }
 

@@ -106,8 +106,6 @@ int cnx_get(cnx_executor* ex, int ndims, int epoch, int name, int64_t size, int 
 int cnx_put(cnx_executor* ex, int name, int64_t size, int dtype, const void* host_in);
 /* array[i] = lo + (hi-lo)*u01(seed, stream_id, i), i = global row-major index; fp64 arrays. */
 int cnx_fill_uniform(cnx_executor* ex, int name, uint64_t seed, uint64_t stream_id, double lo, double hi);
-/* The dense CG test matrix (symmetric, diagonal 2.0) into the square fp64 array `name`. */
-int cnx_fill_cg_matrix(cnx_executor* ex, int name, uint64_t seed);
 /* Waits for everything queued so far. */
 int cnx_sync(cnx_executor* ex);
 

@@ -291,10 +291,6 @@ int cnh_gemm_acc_batch(int dtype, int njobs, const cnh_gemm_job* jobs, cnh_strea
  * neither read nor kept, so a freshly allocated result needs no zero-fill
  * (upstream zero-fills result_data and accumulates, src/executor_matmatmul.cpp:105-160). */
 int cnh_gemm_batch(int dtype, int njobs, const cnh_gemm_job* jobs, int overwrite, cnh_stream s);
-/* Measurement aid without a counterpart upstream: the rate at which this device issues the fp64
- * matrix instruction (v_mfma_f64_16x16x4) from registers, 8 wavefronts per CU with four
- * accumulators each, `iters` rounds; the ceiling the matmatmul figure is set beside. Synchronous. */
-int cnh_probe_mfma_f64(int iters, double* tflops);
 
 /* ---- synthetic inputs generated on the device (no upstream counterpart: upstream has no RNG,
  *      charmnumeric/random.py:4-5, and no bulk upload, charmnumeric.py:863-878) ---- */
@@ -306,9 +302,6 @@ int cnh_fill_uniform(double* out, int64_t n, uint64_t seed, uint64_t stream_id, 
 int cnh_fill_uniform_tile(double* out, int ndims, const int64_t* ext, const int64_t* origin,
                           const int64_t* global_shape, uint64_t seed, uint64_t stream_id, double lo,
                           double hi, cnh_stream s);
-/* Block of the dense CG test matrix of order n (symmetric, diagonal 2.0). */
-int cnh_fill_cg_matrix(double* out, int64_t n, int64_t row0, int64_t nrows, int64_t col0,
-                       int64_t ncols, int64_t ld, uint64_t seed, cnh_stream s);
 
 #ifdef __cplusplus
 }

@@ -20,6 +20,9 @@ def test_every_declared_symbol_is_exported():
     executor = open(os.path.join(ROOT, "include", "cnexec.h")).read()
     executor = re.sub(r"/\*.*?\*/", "", executor, flags=re.S)       # comments mention cnx_ names too
     declared |= set(re.findall(r"\b(cnx_[a-z0-9_]+)\s*\(", executor))
+    fixtures = open(os.path.join(ROOT, "include", "cnbench.h")).read()          # benchmark fixtures
+    fixtures = re.sub(r"/\*.*?\*/", "", fixtures, flags=re.S)
+    declared |= set(re.findall(r"\b(cn[hx]_[a-z0-9_]+)\s*\(", fixtures))
     assert declared, "no declarations found"
     for name in sorted(declared):
         assert hasattr(L.lib, name), f"{name} declared in a header but not exported"

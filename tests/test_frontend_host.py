@@ -60,6 +60,30 @@ def test_view_of_view_composes_like_numpy():
     assert np.array_equal(got, want)
 
 
+def test_region_through_a_strided_view_stays_inside_the_base_array(itf):
+    # extent 10 is not a multiple of the step: the composed stop must not pass the array's end
+    outer = parse_key(slice(None, None, 4), (10,))
+    assert compose(outer, parse_key(slice(None), region_shape(outer))) == ((0,), (9,), (4,))
+    assert compose(outer, parse_key(slice(0, 3), region_shape(outer))) == ((0,), (9,), (4,))
+    assert compose(outer, parse_key(slice(1, 1), region_shape(outer))) == ((4,), (4,), (4,))
+    for n, so, si in ((10, 4, 1), (17, 3, 2), (200, 7, 5), (11, 2, 3)):
+        base = np.arange(n)
+        o = parse_key(slice(1, None, so), base.shape)
+        i = parse_key(slice(None, None, si), region_shape(o))
+        r = compose(o, i)
+        assert r[1][0] <= n
+        assert np.array_equal(base[r[0][0]:r[1][0]:r[2][0]], base[1::so][::si])
+    # the executor accepts the assignments (dry mode: decisions only)
+    a = cnp.zeros(10)
+    a[::4][:] = 1.0
+    u = cnp.zeros(11)
+    u[::3].fill(2.0)
+    b = cnp.ones(3)
+    a[::4][0:3] = b + b
+    cnp.execute(itf)
+    assert not [ln for ln in itf.trace() if "error" in ln.lower()]
+
+
 def test_dtype_and_shape_rules(itf):
     a = cnp.zeros((8,), dtype=cnp.float32)
     assert (a + 1.5).dtype == np.float32          # scalars never promote (charmnumeric.py:369-373)

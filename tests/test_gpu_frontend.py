@@ -300,6 +300,28 @@ def test_view_of_view_assignment_and_inplace_update(small_tiles):
     assert np.array_equal(a.get(small_tiles), host)
 
 
+def test_assignment_through_a_strided_view_whose_extent_is_no_multiple_of_the_step(small_tiles):
+    ha = np.zeros(10)
+    a = cnp.zeros(10)
+    a[::4][:] = 1.0
+    ha[::4][:] = 1.0
+    hu = np.arange(11, dtype=np.float64)
+    u = cnp.array(hu)
+    u[::3].fill(2.0)
+    hu[::3].fill(2.0)
+    hb = np.arange(3, dtype=np.float64) + 1.0
+    b = cnp.array(hb)
+    a[::4][0:3] = b + b
+    ha[::4][0:3] = hb + hb
+    hm = np.arange(150, dtype=np.float64).reshape(10, 15)
+    m = cnp.array(hm)
+    m[1::4, ::7][:, 1:] = m[1::4, ::7][:, 1:] * 3.0
+    hm[1::4, ::7][:, 1:] = hm[1::4, ::7][:, 1:] * 3.0
+    assert np.array_equal(a.get(small_tiles), ha)
+    assert np.array_equal(u.get(small_tiles), hu)
+    assert np.array_equal(m.get(small_tiles), hm)
+
+
 # ---- the LSTM forward pass of upstream's example, statement for statement ----
 
 def _lstm_numpy(X, h0, W, n, b, d, word):

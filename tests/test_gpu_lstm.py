@@ -15,7 +15,7 @@ _exp = np.vectorize(math.exp, otypes=[np.float64])    # host libm, as the refere
 _tanh = np.vectorize(math.tanh, otypes=[np.float64])
 
 
-def _reference(steps, batch, nin, d, seed=5):
+def _reference(steps, batch, nin, d, seed=5, extended=True):
     X = H.np_uniform(steps * batch * nin, seed, 0, -1.0, 1.0).reshape(steps, batch, nin)
     Wih = H.np_uniform(4 * d * nin, seed, 1, -1 / 32, 1 / 32).reshape(4 * d, nin)
     Whh = H.np_uniform(4 * d * d, seed, 2, -1 / 32, 1 / 32).reshape(4 * d, d)
@@ -26,7 +26,10 @@ def _reference(steps, batch, nin, d, seed=5):
     for t in range(steps):
         prev = Hout[t - 1] if t > 0 else np.zeros((batch, d))
         hin = np.concatenate([X[t], prev], axis=1)
-        IFOG[t] = (hin.astype(np.longdouble) @ W.astype(np.longdouble)).astype(np.float64)
+        if extended:
+            IFOG[t] = (hin.astype(np.longdouble) @ W.astype(np.longdouble)).astype(np.float64)
+        else:
+            IFOG[t] = hin @ W          # BLAS, fp64: at the full shape extended precision takes minutes
         f3 = 1.0 / (1.0 + _exp(IFOG[t][:, :3 * d] * -1))
         g = _tanh(IFOG[t][:, 3 * d:])
         Cc[t] = f3[:, :d] * g
@@ -34,6 +37,27 @@ def _reference(steps, batch, nin, d, seed=5):
             Cc[t] = Cc[t] + f3[:, d:2 * d] * Cc[t - 1]
         Hout[t] = f3[:, 2 * d:3 * d] * _tanh(Cc[t])
     return Hout, Cc, IFOG, np.abs(X).max()
+
+
+def test_lstm_forward_full_shape_four_steps(dev):
+    """Batch 256, input 1024, hidden 1024 (the benchmark's shape), 4 steps: gate pre-activations
+    within 1e-12 * sum_k |a_ik| |w_kj|, cell and hidden states at rtol 1e-12."""
+    steps, batch, nin, d = 4, 256, 1024, 1024
+    got = bench.run_lstm(L, steps=steps, batch=batch, nin=nin, d=d, timed=False, keep=True)
+    Hout, Cc, IFOG, _ = _reference(steps, batch, nin, d, extended=False)
+    Wih = H.np_uniform(4 * d * nin, 5, 1, -1 / 32, 1 / 32).reshape(4 * d, nin)
+    Whh = H.np_uniform(4 * d * d, 5, 2, -1 / 32, 1 / 32).reshape(4 * d, d)
+    Wabs = np.abs(np.concatenate([Wih.T, Whh.T], axis=0))
+    X = H.np_uniform(steps * batch * nin, 5, 0, -1.0, 1.0).reshape(steps, batch, nin)
+    for t in range(steps):
+        prev = Hout[t - 1] if t > 0 else np.zeros((batch, d))
+        bound = np.abs(np.concatenate([X[t], prev], axis=1)) @ Wabs
+        # the device's own h feeds the next step's product: its deviation (<= 1e-12 relative) adds
+        # at most 1e-12 * sum |w| <= 1e-12 * d / 32 on top
+        assert np.all(np.abs(got["IFOG"][t] - IFOG[t]) <= 1e-12 * (bound + d / 32.0)), t
+    assert np.allclose(got["C"], Cc, rtol=1e-12, atol=1e-13)
+    assert np.allclose(got["Hout"], Hout, rtol=1e-12, atol=1e-13)
+    assert np.all(np.abs(got["Hout"]) <= 1.0)
 
 
 @pytest.mark.parametrize("steps,batch,nin,d", [(3, 8, 16, 16), (4, 64, 64, 32), (2, 70, 24, 40)])
