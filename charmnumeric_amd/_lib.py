@@ -218,6 +218,8 @@ _PROTOS = {
                                          C.c_int, C.POINTER(Tiled), C.POINTER(Tiled), C.c_void_p]),
     "cnh_dot_partial": (C.c_int, [C.c_int, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p,
                                   C.c_void_p]),
+    "cnh_dot_partial_noalloc": (C.c_int, [C.c_int, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p,
+                                          C.c_void_p]),
     "cnh_reduce_final": (C.c_int, [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
     "cnh_dot_tiles": (C.c_int, [C.c_int, C.c_int, _vpp, _vpp, _i64p, C.c_void_p, C.c_void_p]),
     "cnh_sum_tiles": (C.c_int, [C.c_int, C.c_int, _vpp, _i64p, C.c_void_p, C.c_void_p]),

@@ -47,6 +47,8 @@ inline hipStream_t as_stream(cnh_stream s) { return reinterpret_cast<hipStream_t
 int ensure_init();
 // The device cnh_init selected, -1 before the first call.
 int current_device();
+// Resolves the address of the no-allocation dot's scratch array on `device` (which is current).
+int reduce_scratch_init(int device);
 
 // Device scratch for reduction partials, one region per stream handle so that calls on
 // different streams never share slots. Returns a device pointer to `bytes` bytes.

@@ -160,6 +160,31 @@ __device__ __forceinline__ typename Acc<T>::type slice_reduce(const T* a, const 
     return combine<A, MODE>(acc0, acc1);
 }
 
+// Stage 1 of one workgroup: reduce slice `rel` of chunk `c` into its slot.
+template <typename T, int MODE>
+__device__ __forceinline__ void stage1_body(const Chunk& c, int rel, typename Acc<T>::type* lds,
+                                            typename Acc<T>::type* slot) {
+    typedef typename Acc<T>::type A;
+    const int64_t b0 = (int64_t)rel * c.per_block;
+    const int64_t b1 = b0 + c.per_block < c.n ? b0 + c.per_block : c.n;
+    A v = slice_reduce<T, MODE, kThreads>((const T*)c.a, (const T*)c.b, b0, b1);
+    v = block_reduce<A, MODE, kThreads>(v, lds);
+    if (threadIdx.x == 0)
+        *slot = v;
+}
+
+// Stage 2 for one chunk: a fixed tree over its `nb` slots (every lane returns the value lane 0 holds
+// only in lane 0).
+template <typename T, int MODE>
+__device__ __forceinline__ typename Acc<T>::type stage2_chunk(const typename Acc<T>::type* slots,
+                                                               int nb, typename Acc<T>::type* lds) {
+    typedef typename Acc<T>::type A;
+    A v = 0;
+    for (int i = threadIdx.x; i < nb; i += kThreads)
+        v = combine<A, MODE>(v, slots[i]);
+    return block_reduce<A, MODE, kThreads>(v, lds);
+}
+
 template <typename T, int MODE>
 __global__ __launch_bounds__(kThreads) void reduce_stage1(const Chunk* __restrict__ chunks,
                                                           int nchunk,
@@ -176,12 +201,7 @@ __global__ __launch_bounds__(kThreads) void reduce_stage1(const Chunk* __restric
             hi = mid - 1;
     }
     const Chunk c = chunks[lo];
-    const int64_t b0 = (int64_t)(blk - c.blk0) * c.per_block;
-    const int64_t b1 = b0 + c.per_block < c.n ? b0 + c.per_block : c.n;
-    A v = slice_reduce<T, MODE, kThreads>((const T*)c.a, (const T*)c.b, b0, b1);
-    v = block_reduce<A, MODE, kThreads>(v, lds);
-    if (threadIdx.x == 0)
-        partials[blk] = v;
+    stage1_body<T, MODE>(c, blk - c.blk0, lds, partials + blk);
 }
 
 // One workgroup: per chunk a fixed tree over its slots, then chunks added in index order.
@@ -194,16 +214,32 @@ __global__ __launch_bounds__(kThreads) void reduce_stage2(const Chunk* __restric
     __shared__ A lds[kThreads / 64];
     A total = 0;
     for (int c = 0; c < nchunk; ++c) {
-        const int b0 = chunks[c].blk0, nb = chunks[c].nblk;
-        A v = 0;
-        for (int i = threadIdx.x; i < nb; i += kThreads)
-            v = combine<A, MODE>(v, partials[b0 + i]);
-        v = block_reduce<A, MODE, kThreads>(v, lds);
+        A v = stage2_chunk<T, MODE>(partials + chunks[c].blk0, chunks[c].nblk, lds);
         if (threadIdx.x == 0)
             total = c == 0 ? v : combine<A, MODE>(total, v);
     }
     if (threadIdx.x == 0)
         *out = (T)total;
+}
+
+// The same two stages for a single chunk handed over by value: no descriptor table on the device.
+template <typename T, int MODE>
+__global__ __launch_bounds__(kThreads) void reduce_stage1_one(const Chunk c,
+                                                              typename Acc<T>::type* __restrict__ partials) {
+    typedef typename Acc<T>::type A;
+    __shared__ A lds[kThreads / 64];
+    stage1_body<T, MODE>(c, blockIdx.x, lds, partials + blockIdx.x);
+}
+
+template <typename T, int MODE>
+__global__ __launch_bounds__(kThreads) void reduce_stage2_one(int nblk,
+                                                              const typename Acc<T>::type* __restrict__ partials,
+                                                              T* __restrict__ out) {
+    typedef typename Acc<T>::type A;
+    __shared__ A lds[kThreads / 64];
+    A v = stage2_chunk<T, MODE>(partials, nblk, lds);
+    if (threadIdx.x == 0)
+        *out = (T)v;
 }
 
 // Short single tile: one workgroup of 1024 lanes does everything in one launch.
@@ -233,6 +269,29 @@ __global__ void reduce_final_seq(const T* __restrict__ partials, int n, T* __res
 
 constexpr int64_t kSingleMax = 1 << 16;
 
+// How one contiguous chunk is cut into stage-1 slices: about 8192 elements per workgroup, at most
+// kMaxBlocksPerChunk workgroups, slice lengths a multiple of 512. Depends on n only.
+Chunk plan_chunk(const void* a, const void* b, int64_t n, int blk0) {
+    Chunk c;
+    c.a = a;
+    c.b = b;
+    c.n = n;
+    int64_t nb = (n + 8191) / 8192;
+    if (nb < 1)
+        nb = 1;
+    if (nb > kMaxBlocksPerChunk)
+        nb = kMaxBlocksPerChunk;
+    int64_t per = (n + nb - 1) / nb;
+    per = (per + 511) / 512 * 512;
+    if (per < 512)
+        per = 512;
+    nb = n > 0 ? (n + per - 1) / per : 1;
+    c.per_block = per;
+    c.blk0 = blk0;
+    c.nblk = (int)nb;
+    return c;
+}
+
 template <typename T, int MODE>
 int run_tiles(int n_tiles, const void* const* a, const void* const* b, const int64_t* n, void* out,
               hipStream_t st) {
@@ -254,24 +313,8 @@ int run_tiles(int n_tiles, const void* const* a, const void* const* b, const int
     std::vector<Chunk> chunks(n_tiles);
     int blocks = 0;
     for (int t = 0; t < n_tiles; ++t) {
-        Chunk& c = chunks[t];
-        c.a = a[t];
-        c.b = two ? b[t] : a[t];
-        c.n = n[t];
-        int64_t nb = (n[t] + 8191) / 8192;
-        if (nb < 1)
-            nb = 1;
-        if (nb > kMaxBlocksPerChunk)
-            nb = kMaxBlocksPerChunk;
-        int64_t per = (n[t] + nb - 1) / nb;
-        per = (per + 511) / 512 * 512;
-        if (per < 512)
-            per = 512;
-        nb = n[t] > 0 ? (n[t] + per - 1) / per : 1;
-        c.per_block = per;
-        c.blk0 = blocks;
-        c.nblk = (int)nb;
-        blocks += (int)nb;
+        chunks[t] = plan_chunk(a[t], two ? b[t] : a[t], n[t], blocks);
+        blocks += chunks[t].nblk;
     }
     typedef typename Acc<T>::type A;
     void* ws = nullptr;
@@ -301,9 +344,76 @@ int dispatch_tiles(int dtype, int n_tiles, const void* const* a, const void* con
     return set_error(-2, "unknown dtype %d", dtype);
 }
 
+// ---- dot without any allocation ----
+// Slots for the stage-1 partials of cnh_dot_partial_noalloc: part of the code object, so every
+// device the library runs on holds its own copy from load until the process ends.
+constexpr int kScratchSlots = 32768;                      // 256 KiB
+constexpr int64_t kScratchMaxN = (int64_t)kScratchSlots * 8192;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned long long scratch[kScratchSlots];
+void* g_scratch_ptr[kMaxDevices] = {};
+
+template <typename T>
+int run_dot_noalloc(int64_t n, const void* a, const void* b, void* out, void* slots, hipStream_t st) {
+    typedef typename Acc<T>::type A;
+    if (n <= kSingleMax) {
+        hipLaunchKernelGGL((reduce_single<T, M_DOT>), dim3(1), dim3(1024), 0, st, (const T*)a,
+                           (const T*)b, n, (T*)out);
+        CNH_HIP(hipGetLastError());
+        return 0;
+    }
+    const Chunk c = plan_chunk(a, b, n, 0);
+    CNH_CHECK(c.nblk <= kScratchSlots, -3, "cnh_dot_partial_noalloc: %d partial slots needed, %d held",
+              c.nblk, kScratchSlots);
+    hipLaunchKernelGGL((reduce_stage1_one<T, M_DOT>), dim3(c.nblk), dim3(kThreads), 0, st, c, (A*)slots);
+    CNH_HIP(hipGetLastError());
+    hipLaunchKernelGGL((reduce_stage2_one<T, M_DOT>), dim3(1), dim3(kThreads), 0, st, c.nblk,
+                       (const A*)slots, (T*)out);
+    CNH_HIP(hipGetLastError());
+    return 0;
+}
+
 } // namespace
 
+namespace cnh {
+// Called by cnh_init with `device` current: resolves this device's copy of the scratch array.
+int reduce_scratch_init(int device) {
+    CNH_CHECK(device >= 0 && device < kMaxDevices, -2, "device %d beyond the %d the scratch table holds",
+              device, kMaxDevices);
+    if (g_scratch_ptr[device])
+        return 0;
+    void* p = nullptr;
+    CNH_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    CNH_CHECK(p != nullptr, -100, "hipGetSymbolAddress returned a null scratch address");
+    g_scratch_ptr[device] = p;
+    return 0;
+}
+} // namespace cnh
+
 extern "C" {
+
+int cnh_dot_partial_noalloc(int dtype, int64_t n, const void* a, const void* b, void* out,
+                            cnh_stream s) {
+    if (int rc = ensure_init())
+        return rc;
+    CNH_CHECK(out != nullptr && n >= 0, -2, "cnh_dot_partial_noalloc: bad arguments");
+    CNH_CHECK(n == 0 || (a != nullptr && b != nullptr), -2, "cnh_dot_partial_noalloc: null operand");
+    CNH_CHECK(n <= kScratchMaxN, -3,
+              "cnh_dot_partial_noalloc: %lld elements exceed the maximum of %lld",
+              (long long)n, (long long)kScratchMaxN);
+    const int dev = current_device();
+    void* slots = dev >= 0 && dev < kMaxDevices ? g_scratch_ptr[dev] : nullptr;
+    CNH_CHECK(slots != nullptr, -100, "cnh_dot_partial_noalloc: scratch of device %d not resolved", dev);
+    hipStream_t st = as_stream(s);
+    switch (dtype) {
+    case CNH_F32: return run_dot_noalloc<float>(n, a, b, out, slots, st);
+    case CNH_F64: return run_dot_noalloc<double>(n, a, b, out, slots, st);
+    case CNH_I32: return run_dot_noalloc<int32_t>(n, a, b, out, slots, st);
+    case CNH_I64: return run_dot_noalloc<int64_t>(n, a, b, out, slots, st);
+    }
+    return set_error(-2, "unknown dtype %d", dtype);
+}
+
 
 int cnh_dot_tiles(int dtype, int n_tiles, const void* const* a, const void* const* b,
                   const int64_t* n, void* out, cnh_stream s) {

@@ -167,8 +167,10 @@ int cnh_init(int device) {
     CNH_CHECK(device >= 0 && device < count && device < kMaxDevices, -2,
               "device %d out of range (have %d)", device, count);
     CNH_HIP(hipSetDevice(device));
-    // Descriptor tables and reduction workspaces are kept per device, so a later call with
-    // another device finds its own (or none yet) and never one of this device.
+    // Descriptor tables, reduction workspaces and the scratch array are kept per device, so a
+    // later call with another device finds its own (or none yet) and never one of this device.
+    if (int rc = reduce_scratch_init(device))
+        return rc;
     g_device = device;
     g_inited = true;
     return 0;

@@ -229,6 +229,16 @@ int cnh_reduce_final(int dtype, int n_partials, const void* partials, void* out,
 /* All tiles in one launch + the final pass: out = sum_t dot(a[t], b[t]), tiles in index order. */
 int cnh_dot_tiles(int dtype, int n_tiles, const void* const* a, const void* const* b,
                   const int64_t* n, void* out, cnh_stream s);
+/* cnh_dot_partial for callers that cannot allocate (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc). No counterpart upstream. Same kernels, same slicing and
+ * the same bits as cnh_dot_partial, but the stage-1 partials go to a 256 KiB array that is part of
+ * the library's code object on every device instead of a workspace the library allocates, and the
+ * call allocates and frees nothing. n is limited to 2^28 elements (-3 beyond that). All calls on
+ * one device share the array: calls that overlap in time on one device (different streams) race;
+ * calls on one stream are ordered. Nothing in the array needs clearing between calls: stage 1
+ * writes every slot stage 2 reads. */
+int cnh_dot_partial_noalloc(int dtype, int64_t n, const void* a, const void* b, void* out,
+                            cnh_stream s);
 /* Extensions with no upstream counterpart (upstream REDUCE is 1-D dot only,
  * src/executor_reduce.cpp:9-12): sum of elements, sum of squared differences, max |a-b|,
  * over lists of contiguous chunks. fp64 only for the last two. */
