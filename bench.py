@@ -413,35 +413,50 @@ class SubBuf:
 
 
 class TiledDev:
-    """n^nd fp64 array in row-major tiles of edge `tile`. The tiles are carved from one device
-    allocation the way the host executor does it; `skew` extra bytes between consecutive tiles
-    keep equally sized power-of-two tiles from starting at addresses that differ by a multiple of
-    their size."""
+    """n^nd fp64 array in tiles of edge `tile`, laid out the way the host executor lays arrays out:
+    rank 2 — every tile a row-major buffer of its own extents, carved back to back from one
+    allocation; rank 3 — one row-major block over the whole array with the tiles as views into it
+    (common row and plane pitches). CNH_BENCH_TILE_MAJOR=1 gives rank 3 separate tile buffers too,
+    `skew` extra bytes apart (equally sized power-of-two tiles back to back start at addresses
+    that differ by a multiple of their size: 462 us per 512^3 sweep against 424 us with 2 MiB +
+    256 B between them)."""
 
     def __init__(self, L, nd, n, tile, skew=None):
         self.L, self.nd, self.n, self.tile = L, nd, n, tile
         self.g = (n + tile - 1) // tile
+        self.flat = nd == 3 and not os.environ.get("CNH_BENCH_TILE_MAJOR")
         if skew is None:
-            # measured on MI355X: 64 tiles of 128^3 (16 MiB each) back to back 462 us per sweep,
-            # 2 MiB + 256 B apart 424 us; tiles of 2048^2 are best back to back
             skew = (2 << 20) + 256 if nd == 3 else 0
             if os.environ.get("CNH_BENCH_SKEW"):
                 skew = int(os.environ["CNH_BENCH_SKEW"])
-        exts = [[min(tile, n - i * tile) for i in idx] for idx in np.ndindex(*([self.g] * nd))]
+        idxs = list(np.ndindex(*([self.g] * nd)))
+        exts = [[min(tile, n - i * tile) for i in idx] for idx in idxs]
         offs, off = [], 0
-        for ext in exts:
-            offs.append(off)
-            off += (int(np.prod(ext)) * 8 + 255) // 256 * 256 + skew
+        if self.flat:
+            offs = [sum(i * tile * n ** (nd - 1 - d) for d, i in enumerate(idx)) * 8 for idx in idxs]
+            off = n ** nd * 8
+        else:
+            for ext in exts:
+                offs.append(off)
+                off += (int(np.prod(ext)) * 8 + 255) // 256 * 256 + skew
         self.slab = Buf(L, off, zero=True)
         self.bufs = [(idx, ext, SubBuf(L, self.slab.ptr + o, int(np.prod(ext)) * 8))
-                     for idx, ext, o in zip(np.ndindex(*([self.g] * nd)), exts, offs)]
+                     for idx, ext, o in zip(idxs, exts, offs)]
         self.ptrs = (C.c_void_p * len(self.bufs))(*[C.c_void_p(b.ptr) for _, _, b in self.bufs])
         d = L.Tiled()
         d.ndims, d.tile = nd, tile
         for i in range(nd):
             d.offset[i], d.shape[i], d.grid_lo[i], d.grid[i] = 0, n, 0, self.g
+            if self.flat:
+                d.pitch[i] = n ** (nd - 1 - i)
         d.tiles = C.cast(self.ptrs, C.POINTER(C.c_void_p))
         self.desc = d
+
+    def strides(self, ext):
+        """Elements between consecutive indices of each dimension inside a tile of extents ext."""
+        if self.flat:
+            return [self.n ** (self.nd - 1 - d) for d in range(self.nd)]
+        return [int(np.prod(ext[d + 1:])) for d in range(self.nd)]
 
     def free(self):
         self.slab.free()
@@ -464,6 +479,8 @@ def run_jacobi(L, nd, n, tile, sweeps, reduce_every=10, reps_note=""):
     res = Buf(L, 8, zero=True)
     ntile = len(a.bufs)
     lens = L.i64arr([int(np.prod(e)) for _, e, _ in a.bufs])
+    if a.flat:      # one block: the reductions read it as a single chunk
+        ntile, lens = 1, L.i64arr([n ** nd])
 
     def sweep(src, dst):
         descs = (L.Tiled * nleaf)(*([src.desc] * nleaf))
@@ -472,7 +489,10 @@ def run_jacobi(L, nd, n, tile, sweeps, reduce_every=10, reps_note=""):
 
     def residual(src, dst):
         fn = L.lib.cnh_sumsq_diff_tiles if nd == 2 else L.lib.cnh_maxabs_diff_tiles
-        L.check(fn(ntile, dst.ptrs, src.ptrs, lens, res.ptr, None))
+        if a.flat:
+            L.check(fn(1, L.vparr([dst.slab.ptr]), L.vparr([src.slab.ptr]), lens, res.ptr, None))
+        else:
+            L.check(fn(ntile, dst.ptrs, src.ptrs, lens, res.ptr, None))
 
     for _ in range(3):
         sweep(a, b)
@@ -509,7 +529,8 @@ def run_jacobi(L, nd, n, tile, sweeps, reduce_every=10, reps_note=""):
            "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
            "bytes_per_sweep": nbytes, "total_ms_with_reductions": round(ms.value, 3),
            "reduction_us": round(1e3 * float(np.median(tr)), 2),
-           "last_reduction": float(res.get(np.float64)[0]), "partitions": ntile, "tile": tile}
+           "last_reduction": float(res.get(np.float64)[0]), "partitions": len(a.bufs), "tile": tile,
+           "layout": "one block, partitions as views" if a.flat else "one buffer per partition"}
     ev.free()
     evr.free()
     a.free()
@@ -521,13 +542,16 @@ def run_jacobi(L, nd, n, tile, sweeps, reduce_every=10, reps_note=""):
 def _fill_3d(L, arr, n):
     """Interior uniform[0,1) (seed 1, element index = row-major flat index), faces 0."""
     t = arr.tile
-    for idx, ext, buf in arr.bufs:
-        L.check(L.lib.cnh_fill_uniform_tile(buf.ptr, 3, L.i64arr(ext), L.i64arr([i * t for i in idx]),
-                                            L.i64arr([n, n, n]), 1, 0, 0.0, 1.0, None))
+    if arr.flat:
+        L.check(L.lib.cnh_fill_uniform(arr.slab.ptr, n ** 3, 1, 0, 0, 0.0, 1.0, None))
+    else:
+        for idx, ext, buf in arr.bufs:
+            L.check(L.lib.cnh_fill_uniform_tile(buf.ptr, 3, L.i64arr(ext), L.i64arr([i * t for i in idx]),
+                                                L.i64arr([n, n, n]), 1, 0, 0.0, 1.0, None))
     # zero the six faces
     zero = np.zeros(1).view(np.uint8)
     for idx, ext, buf in arr.bufs:
-        st = L.i64arr([ext[1] * ext[2], ext[2], 1])
+        st = L.i64arr(arr.strides(ext))
         for d in range(3):
             for side in (0, 1):
                 if (side == 0 and idx[d] != 0) or (side == 1 and idx[d] != arr.g - 1):

@@ -494,9 +494,12 @@ std::string tiles_source(const GroupProgram& p) {
 // Gather over tiled arrays resident on this device: every element of every destination tile is
 // produced by one thread, which resolves each shifted/strided input coordinate to its owning
 // tile (tile edge is a power of two) and reads it there. Rank padded to 3.
+// py, pz: elements between rows and between planes inside every tile when the tiles are views
+// into one larger row-major block; py = 0: a tile is contiguous over its own extents.
 struct Tiled {
     int shift; int tile; int off[3]; int shape[3]; int glo[3]; int grid[3];
     const T* const* tiles;
+    int py, pz;
 };
 // cs, w: origin and extents of the tile; bs, bw: what of it this launch visits. A ping-pong
 // launch walks the whole tile (bs = 0, bw = w, in elements). An in-place launch (TilesArgs.lattice)
@@ -504,7 +507,7 @@ struct Tiled {
 // first such point along each dimension, bw = how many.
 // rsh: a workgroup covers 2^rsh consecutive rows with 256 >> rsh lanes each (short rows, e.g. the
 // 128-wide tiles of rank-3 arrays, would otherwise leave most lanes idle); 0 = one row.
-struct DTile { i64 blk0; int cs[3]; int w[3]; int nchunks; int rsh; int bs[3]; int bw[3]; T* dst; const T* cur; };
+struct DTile { i64 blk0; int cs[3]; int w[3]; int nchunks; int rsh; int bs[3]; int bw[3]; T* dst; const T* cur; int py, pz; };
 struct LeafReg { int arr; int start[3]; int step[3]; };
 struct TilesArgs {
     int out_off[3];
@@ -523,7 +526,8 @@ __device__ __forceinline__ T tiled_read(const Tiled& a, int g0, int g1, int g2) 
     const int w2 = min((t2 + 1) << a.shift, a.off[2] + a.shape[2]) - lo2;
     const int ti = ((t0 - a.glo[0]) * a.grid[1] + (t1 - a.glo[1])) * a.grid[2] + (t2 - a.glo[2]);
     const T* base = a.tiles[ti];
-    return base[((i64)(g0 - lo0) * w1 + (g1 - lo1)) * w2 + (g2 - lo2)];
+    const i64 s1 = a.py ? a.py : w2, s0 = a.py ? (i64)a.pz : (i64)w1 * w2;
+    return base[(g0 - lo0) * s0 + (g1 - lo1) * s1 + (g2 - lo2)];
 }
 
 template <bool ROWS>
@@ -565,7 +569,8 @@ __device__ __forceinline__ void tiles_run(const Tiled* arrs, const DTile* dts, i
         const int i2 = dt.bs[2] + j2;
         const int a2 = ta.lattice ? ta.rs[2] + i2 * ta.rst[2] : dt.cs[2] + i2 - ta.out_off[2];
         const int l2 = a2 + ta.out_off[2] - dt.cs[2];
-        const i64 di = ((i64)l0 * dt.w[1] + l1) * dt.w[2] + l2;
+        const i64 ds1 = dt.py ? dt.py : dt.w[2], ds0 = dt.py ? (i64)dt.pz : (i64)dt.w[1] * dt.w[2];
+        const i64 di = l0 * ds0 + l1 * ds1 + l2;
         const bool inside = in01 && (ta.lattice || (a2 >= ta.rs[2] && a2 < ta.re[2] &&
                                                     (a2 - ta.rs[2]) % ta.rst[2] == 0));
         if (inside) {

@@ -644,6 +644,172 @@ __device__ __forceinline__ void direct_rest(const DirectArgs& a, const T* s, int
     }
 }
 
+// ---- the whole array as one row-major block ----
+// When every tile of every array of the launch is a view into one block (an executor that keeps all
+// partitions of an array on one device may store it that way), tiles need no pointers and no
+// neighbour logic: a wavefront works on 128 columns of DR_RY rows in DR_RZ planes of the ARRAY,
+// window coordinates are clamped into the array (what a clamped entry holds is only ever used by
+// elements outside the assigned region, which keep their old value), and the only faces left are
+// the array's own. Workgroups are ordered in blocks of ob[] workgroups (x fastest inside a block,
+// then y, then z) and the 8 XCDs get contiguous runs of that order, so that the planes and rows a
+// block re-reads stay in one L2.
+struct FlatArgs {
+    const T* cur;          // current contents of the window array
+    T* dst;                // new contents of the assigned array
+    const T* oth[4];       // other arrays read at the element's own position
+    int shape[3];          // array extents (leading dims padded with 1)
+    int rs[3], re[3];      // assigned region
+    int py, pz;            // elements between rows and between planes
+    int nb[3];             // workgroups along z, y, x
+    int ob[3];             // ordering block, in workgroups along z, y, x
+    int nblocks8;          // launched workgroups / 8 when that is exact, else 0
+    FDiv per_block;        // workgroups per ordering block
+    FDiv gb1, gb2;         // ordering blocks along y and x
+    FDiv obx, oby;         // = ob[2], ob[1]
+};
+
+template <bool NTS>
+__device__ __forceinline__ void direct_flat(const FlatArgs& a, const T* s) {
+    int blk = (int)blockIdx.x;
+    if (a.nblocks8) blk = (blk & 7) * a.nblocks8 + (blk >> 3);
+    const int g = fdiv(blk, a.per_block), w = blk - g * (int)a.per_block.d;
+    const int gq = fdiv(g, a.gb2), g2 = g - gq * (int)a.gb2.d;
+    const int g0 = fdiv(gq, a.gb1), g1 = gq - g0 * (int)a.gb1.d;
+    const int wq = fdiv(w, a.obx), wx = w - wq * (int)a.obx.d;
+    const int wz = fdiv(wq, a.oby), wy = wq - wz * (int)a.oby.d;
+    const int bz = g0 * a.ob[0] + wz, by = g1 * a.ob[1] + wy, bx = g2 * a.ob[2] + wx;
+    if (bz >= a.nb[0] || by >= a.nb[1] || bx >= a.nb[2]) return;   // padding of a ragged block
+    const int tid = (int)threadIdx.x;
+    const int wv = wave_uniform(tid >> 6);
+    const int lane = tid & 63;
+    const int S0 = a.shape[0], S1 = a.shape[1], S2 = a.shape[2];
+    const int z0 = bz * DR_RZ, y0 = (by * 4 + wv) * DR_RY, x0 = bx * 128;
+    if (y0 >= S1) return;                                            // wavefront-uniform
+    const int PY = a.py, PZ = a.pz;
+    const int lx = x0 + 2 * lane;
+    const bool live = lx < S2;                  // S2 is even: a live lane owns a whole pair
+    const int cx = min(lx, S2 - 2);             // idle lanes re-read the last pair of the row
+    const bool first = lane == 0, last = lane == 63;
+    // clamped planes and rows of the window (wavefront-uniform)
+    int zo[DR_WZ], yo[DR_WY];
+#pragma unroll
+    for (int i = 0; i < DR_WZ; ++i) zo[i] = min(max(z0 - DR_H0 + i, 0), S0 - 1) * PZ;
+#pragma unroll
+    for (int j = 0; j < DR_WY; ++j) yo[j] = min(max(y0 - DR_H1 + j, 0), S1 - 1) * PY;
+    const T* const cur = a.cur;
+
+    // All loads first: the centre pairs, then the pairs beyond the two ends of the wavefront.
+    P2 win[DR_WZ][DR_WY][DR_WK];
+    P2 beyond[DR_WZ][DR_WY];
+#pragma unroll
+    for (int i = 0; i < DR_WZ; ++i)
+#pragma unroll
+        for (int j = 0; j < DR_WY; ++j)
+            if (DR_NEED[i][j][0] || DR_NEED[i][j][DR_HK] || DR_NEED[i][j][DR_WK - 1])
+                win[i][j][DR_HK] = *reinterpret_cast<const P2*>(cur + (zo[i] + yo[j] + cx));
+    const int xl = max(x0 - 2, 0), xr = min(x0 + 128, S2 - 2);   // columns of the two far pairs
+    P2 edge = (P2){(T)0, (T)0};
+    if (DR_HK == 1) {
+        if (DR_EDGE_GATHER) {
+            // one load for all of them: lane 2r holds the pair left of row r of the block of rows
+            // that need one, lane 2r + 1 the pair right of it
+            if (lane < 2 * DR_NB) {
+                const int r = lane >> 1, i = DR_BI0 + r / DR_BNJ, j = DR_BJ0 + r % DR_BNJ;
+                const int zz = min(max(z0 - DR_H0 + i, 0), S0 - 1), yy = min(max(y0 - DR_H1 + j, 0), S1 - 1);
+                edge = *reinterpret_cast<const P2*>(cur + (zz * PZ + yy * PY + ((lane & 1) ? xr : xl)));
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < DR_WZ; ++i)
+#pragma unroll
+                for (int j = 0; j < DR_WY; ++j)
+                    if (DR_NEED[i][j][0] || DR_NEED[i][j][DR_WK - 1]) {
+                        const int c = first ? xl : (last ? xr : cx);
+                        beyond[i][j] = *reinterpret_cast<const P2*>(cur + (zo[i] + yo[j] + c));
+                    }
+        }
+    }
+    P2 ov[DR_NOTHA][DR_RZ][DR_RY];
+#pragma unroll
+    for (int j = 0; j < DR_NOTH; ++j)
+#pragma unroll
+        for (int rz = 0; rz < DR_RZ; ++rz)
+#pragma unroll
+            for (int ry = 0; ry < DR_RY; ++ry)
+                ov[j][rz][ry] = *reinterpret_cast<const P2*>(
+                    a.oth[j] + (zo[rz + DR_H0] + yo[ry + DR_H1] + cx));
+    if (DR_HK == 1) {
+#pragma unroll
+        for (int i = 0; i < DR_WZ; ++i)
+#pragma unroll
+            for (int j = 0; j < DR_WY; ++j) {
+                const int r = (i - DR_BI0) * DR_BNJ + (j - DR_BJ0);   // row of the gathered block
+                if (DR_NEED[i][j][0]) {
+                    P2 sh, far = beyond[i][j];
+                    sh[0] = from_prev_lane(win[i][j][DR_HK][0]);
+                    sh[1] = from_prev_lane(win[i][j][DR_HK][1]);
+                    if (DR_EDGE_GATHER) {
+                        far[0] = from_lane(edge[0], 2 * r);
+                        far[1] = from_lane(edge[1], 2 * r);
+                    }
+                    win[i][j][0] = first ? far : sh;
+                }
+                if (DR_NEED[i][j][DR_WK - 1]) {
+                    P2 sh, far = beyond[i][j];
+                    sh[0] = from_next_lane(win[i][j][DR_HK][0]);
+                    sh[1] = from_next_lane(win[i][j][DR_HK][1]);
+                    if (DR_EDGE_GATHER) {
+                        far[0] = from_lane(edge[0], 2 * r + 1);
+                        far[1] = from_lane(edge[1], 2 * r + 1);
+                    }
+                    win[i][j][DR_WK - 1] = last ? far : sh;
+                }
+            }
+    }
+    T* const dst = a.dst;
+#pragma unroll
+    for (int rz = 0; rz < DR_RZ; ++rz) {
+        const int z = z0 + rz;
+        const bool zin = z >= a.rs[0] && z < a.re[0];
+#pragma unroll
+        for (int ry = 0; ry < DR_RY; ++ry) {
+            const int y = y0 + ry;
+            const bool yin = zin && y >= a.rs[1] && y < a.re[1];
+            P2 res;
+            bool in_e[2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                T l[NLA], o[NOA];
+#pragma unroll
+                for (int q = 0; q < NL; ++q) {
+                    const int xx = e + DR_SHIFT[q][2];
+                    l[q] = DR_OTHER[q] >= 0
+                               ? ov[DR_OTHER[q] >= 0 ? DR_OTHER[q] : 0][rz][ry][e]
+                               : win[rz + DR_H0 + DR_SHIFT[q][0]][ry + DR_H1 + DR_SHIFT[q][1]]
+                                    [DR_HK + floordiv2(xx)][xx & 1];
+                }
+                group_eval(l, s, o);
+                const int gx = lx + e;
+                in_e[e] = yin && gx >= a.rs[2] && gx < a.re[2];
+                res[e] = (DR_MASKED || in_e[e]) ? o[0] : win[rz + DR_H0][ry + DR_H1][DR_HK][e];
+            }
+            // rows and planes beyond the array (a ragged last workgroup) and idle lanes store nothing
+            if (live && z < S0 && y < S1) {
+                P2* out = reinterpret_cast<P2*>(dst + (z * PZ + y * PY + lx));
+                store_pair<NTS>(out, res, in_e[0], in_e[1]);
+            }
+        }
+    }
+}
+extern "C" __global__ __launch_bounds__(256) void grp_direct_flat(FlatArgs a, Scal sc) {
+    T s[NSA]; load_scalars(sc, s);
+    direct_flat<false>(a, s);
+}
+extern "C" __global__ __launch_bounds__(256) void grp_direct_flat_nts(FlatArgs a, Scal sc) {
+    T s[NSA]; load_scalars(sc, s);
+    direct_flat<true>(a, s);
+}
+
 // nts: the written stream is not read back soon, store it non-temporally.
 extern "C" __global__ __launch_bounds__(256) void grp_direct_fast(DirectArgs a, Scal sc) {
     T s[NSA]; load_scalars(sc, s);

@@ -461,8 +461,9 @@ namespace {
 struct TiledDev {
     int32_t shift, tile, off[3], shape[3], glo[3], grid[3];
     const void* tiles;
+    int32_t py, pz;
 };
-static_assert(sizeof(TiledDev) == 64, "TiledDev layout must match the generated struct");
+static_assert(sizeof(TiledDev) == 72, "TiledDev layout must match the generated struct");
 
 struct DTileDev {
     int64_t blk0;
@@ -470,8 +471,9 @@ struct DTileDev {
     int32_t bs[3], bw[3];
     void* dst;
     const void* cur;
+    int32_t py, pz;
 };
-static_assert(sizeof(DTileDev) == 80, "DTileDev layout must match the generated struct");
+static_assert(sizeof(DTileDev) == 88, "DTileDev layout must match the generated struct");
 
 int check_tiled(const cnh_tiled* t, int nd, const char* what) {
     CNH_CHECK(t != nullptr, -2, "%s: null descriptor", what);
@@ -498,6 +500,8 @@ int check_tiled(const cnh_tiled* t, int nd, const char* what) {
     }
     CNH_CHECK(!any || (all && t->pitch[nd - 1] == 1), -4,
               "%s: pitches must be all zero, or positive with 1 along the last dimension", what);
+    for (int d = 0; any && d < nd; ++d)
+        CNH_CHECK(t->pitch[d] < (1ll << 31), -4, "%s: pitch of dim %d does not fit 31 bits", what, d);
     for (int d = 0; any && d + 1 < nd; ++d)
         CNH_CHECK(t->pitch[d] >= t->pitch[d + 1] * std::min(t->tile, t->shape[d + 1]), -4,
                   "%s: pitch %lld of dim %d is shorter than a tile's extent below it", what,
@@ -537,6 +541,9 @@ int make_tiled_dev(const cnh_tiled* t, hipStream_t st, TiledDev& d) {
     if (int rc = desc_upload(t->tiles, (size_t)count * sizeof(void*), st, &table))
         return rc;
     d.tiles = table;
+    // rank 1 has nothing between rows; rank 2 has no planes
+    d.py = nd >= 2 ? (int32_t)t->pitch[nd - 2] : 0;
+    d.pz = nd >= 3 ? (int32_t)t->pitch[0] : 0;
     return 0;
 }
 
@@ -670,6 +677,18 @@ struct DirectArgsDev {
 static_assert(sizeof(DirectArgsDev) == 16 + 4 * 22 + 12 * 8 + 8 * kDirectMaxOther + 8,
               "DirectArgsDev layout must match the generated struct");
 
+struct FlatArgsDev {
+    const void* cur;
+    void* dst;
+    const void* oth[kDirectMaxOther];
+    int32_t shape[3], rs[3], re[3], py, pz, nb[3], ob[3], nblocks8;
+    FDivDev per_block, gb1, gb2, obx, oby;
+};
+static_assert(sizeof(FlatArgsDev) == 16 + 8 * kDirectMaxOther + 4 * 18 + 12 * 5 + 4,
+              "FlatArgsDev layout must match the generated struct");
+
+int g_direct_flat = 1;          // arrays stored as one block take the whole-array kernel
+int g_flat_ob[3] = {0, 0, 0};   // ordering block of that kernel in elements (z, y, x); 0 = default
 int g_stencil_mode = 2; // 0 = general gather, 1 = LDS sliding window, 2 = register window
 int g_direct_group = 0; // order workgroups by groups of neighbouring tiles (rank 3)
 int g_direct_lean = -1;   // wavefront-level lean kernel: 1 on, 0 off, -1 by rank
@@ -803,6 +822,84 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
         for (int64_t t = 0; t < ntiles; ++t)
             if (((uintptr_t)o->tiles[t] & 15) || (!sh.masked && o->tiles[t] == dst->tiles[t]))
                 return 0;
+    }
+    // Every array of the launch one row-major block behind its tile views: no tile logic at all.
+    if (pitched && g_direct_flat) {
+        const int esz = dtype_size(p.dtype);
+        auto one_block = [&](const cnh_tiled* t) {
+            // tile (i0, i1, i2) must start where element (i0, i1, i2) * tile of the block lies
+            const char* base = static_cast<const char*>(t->tiles[0]);
+            int64_t idx[3] = {0, 0, 0};
+            for (int64_t n = 0; n < ntiles; ++n) {
+                int64_t off = 0;
+                for (int d = 0; d < nd; ++d)
+                    off += idx[d] * t->tile * t->pitch[d];
+                if (static_cast<const char*>(t->tiles[n]) != base + off * esz)
+                    return false;
+                for (int d = nd - 1; d >= 0; --d) {
+                    if (++idx[d] < t->grid[d])
+                        break;
+                    idx[d] = 0;
+                }
+            }
+            return true;
+        };
+        bool flat = one_block(cur) && one_block(dst) && pitch[1] >= cur->shape[nd - 1] &&
+                    (nd < 3 || pitch[0] >= pitch[1] * cur->shape[1]) &&
+                    pitch[0] * (nd == 3 ? cur->shape[0] : 1) + pitch[1] * cur->shape[nd - 2] < (1ll << 31);
+        for (int j = 0; j < n_other && flat; ++j)
+            flat = one_block(others[j]);
+        if (flat) {
+            FlatArgsDev f;
+            std::memset(&f, 0, sizeof f);
+            f.cur = cur->tiles[0];
+            f.dst = dst->tiles[0];
+            for (int j = 0; j < n_other; ++j)
+                f.oth[j] = others[j]->tiles[0];
+            for (int d = 0; d < 3; ++d) {
+                f.shape[d] = 1;
+                f.rs[d] = 0;
+                f.re[d] = 1;
+            }
+            for (int d = 0; d < nd; ++d) {
+                f.shape[pad + d] = cur->shape[d];
+                f.rs[pad + d] = p.out_region[0].start[d];
+                f.re[pad + d] = p.out_region[0].stop[d];
+            }
+            f.py = (int32_t)pitch[1];
+            f.pz = (int32_t)pitch[0];
+            // a workgroup: 4 wavefronts stacked along y, each 128 columns x ry rows x rz planes
+            const int foot[3] = {sh.rz, 4 * sh.ry, 128};
+            // ordering block: 256^3 elements for rank 3 (measured on MI355X, 512^3: 382 us per
+            // sweep against 390 with 128^3 and 449 with whole planes); rank 2: bands of whole rows
+            const int dflt[3] = {256, nd == 3 ? 256 : 1 << 30, nd == 3 ? 256 : 1 << 30};
+            int64_t launched = 1, gb[3];
+            for (int d = 0; d < 3; ++d) {
+                f.nb[d] = (f.shape[d] + foot[d] - 1) / foot[d];
+                const int want = g_flat_ob[d] > 0 ? g_flat_ob[d] : dflt[d];
+                f.ob[d] = std::max(1, std::min(f.nb[d], want / foot[d]));
+                gb[d] = (f.nb[d] + f.ob[d] - 1) / f.ob[d];
+                launched *= gb[d] * f.ob[d];
+            }
+            CNH_CHECK(launched > 0 && launched < (1ll << 31), -3, "stencil launch of %lld workgroups",
+                      (long long)launched);
+            f.nblocks8 = launched % 8 == 0 ? (int32_t)(launched / 8) : 0;
+            f.per_block = fdiv_make((uint32_t)(f.ob[0] * f.ob[1] * f.ob[2]));
+            f.gb1 = fdiv_make((uint32_t)gb[1]);
+            f.gb2 = fdiv_make((uint32_t)gb[2]);
+            f.obx = fdiv_make((uint32_t)f.ob[2]);
+            f.oby = fdiv_make((uint32_t)f.ob[1]);
+            const bool nts = volume * 2 * esz >= (128ll << 20);
+            hipFunction_t fn;
+            if (int rc = get_function(k, g_direct_cfg.variant(),
+                                      nts ? "grp_direct_flat_nts" : "grp_direct_flat", &fn))
+                return rc;
+            void* params[] = {&f, const_cast<unsigned char*>(scal.data())};
+            if (int rc = launch(fn, launched, params, st))
+                return rc;
+            *handled = true;
+            return 0;
+        }
     }
     DirectArgsDev a;
     std::memset(&a, 0, sizeof a);
@@ -1009,6 +1106,16 @@ extern "C" int cnh_set_option(const char* name, int value) {
         g_slide_cfg.march2d = value != 0;
         return 0;
     }
+    if (std::strcmp(name, "direct_flat") == 0) {
+        g_direct_flat = value != 0;
+        return 0;
+    }
+    if (std::strcmp(name, "flat_obz") == 0 || std::strcmp(name, "flat_oby") == 0 ||
+        std::strcmp(name, "flat_obx") == 0) {
+        CNH_CHECK(value >= 0, -2, "ordering block extent must not be negative");
+        g_flat_ob[name[7] == 'z' ? 0 : (name[7] == 'y' ? 1 : 2)] = value;
+        return 0;
+    }
     if (std::strcmp(name, "slide_bx") == 0) {
         g_slide_cfg.bx = value;
         return 0;
@@ -1046,8 +1153,8 @@ extern "C" int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* 
             return rc;
         CNH_CHECK(cur->tile == dst->tile, -4, "cur and dst differ in tile edge");
         for (int d = 0; d < nd; ++d)
-            CNH_CHECK(cur->offset[d] == dst->offset[d] && cur->shape[d] == dst->shape[d], -4,
-                      "cur and dst differ in decomposition");
+            CNH_CHECK(cur->offset[d] == dst->offset[d] && cur->shape[d] == dst->shape[d] &&
+                          cur->pitch[d] == dst->pitch[d], -4, "cur and dst differ in decomposition");
     }
     for (int i = 0; i < n_in; ++i)
         if (int rc = check_tiled(&in[i], nd, "input"))
@@ -1131,14 +1238,14 @@ extern "C" int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* 
             return rc;
         if (handled)
             return 0;
-        // the other kernels address a tile through its own extents
+        // the sliding-window kernel addresses a tile through its own extents; the general gather
+        // below takes pitched views too
         bool pitched = is_pitched(dst) || (cur && is_pitched(cur));
         for (const cnh_tiled* a : arrays)
             pitched = pitched || is_pitched(a);
-        CNH_CHECK(!pitched, -4, "tiles given as pitched views are taken by the register-window stencil "
-                  "kernels only, and this group or its arrays do not qualify for them");
-        if (int rc = try_launch_slide(k, arrays, cur, dst, scal, st, &handled))
-            return rc;
+        if (!pitched)
+            if (int rc = try_launch_slide(k, arrays, cur, dst, scal, st, &handled))
+                return rc;
         if (handled)
             return 0;
     }
@@ -1177,6 +1284,8 @@ extern "C" int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* 
             continue;
         dt.dst = dst->tiles[t];
         dt.cur = cur ? cur->tiles[t] : nullptr;
+        dt.py = nd >= 2 ? (int32_t)dst->pitch[nd - 2] : 0;
+        dt.pz = nd >= 3 ? (int32_t)dst->pitch[0] : 0;
         // In place (or with nothing to copy from), elements outside the assigned region keep
         // their values without being touched: the launch walks the points of the region's index
         // lattice that fall into the tile (bs = index of the first one along each dimension,

@@ -23,6 +23,7 @@ class CharmNumericInterface:
         self._min_tiles = {}
         self._pipeline = False
         self._solver = os.environ.get("CHARMNUMERIC_SOLVER", "0") not in ("", "0")
+        self._flat3 = os.environ.get("CHARMNUMERIC_FLAT3", "1") not in ("", "0")
 
     # -- decomposition planning ----------------------------------------------------------------
     def set_solver(self, on=True):
@@ -34,6 +35,14 @@ class CharmNumericInterface:
         self._solver = bool(on)
         if self._ex is not None:
             L.check(L.lib.cnx_set_solver(self._ex, 1 if on else 0))
+
+    def set_layout(self, flat_rank3=True):
+        """How rank-3 arrays created from now on are stored: one row-major block with the
+        partitions as views into it (default; environment variable CHARMNUMERIC_FLAT3=0 turns it
+        off for every interface), or one contiguous buffer per partition."""
+        self._flat3 = bool(flat_rank3)
+        if self._ex is not None:
+            L.check(L.lib.cnx_set_layout(self._ex, 1 if flat_rank3 else 0))
 
     # -- pipelining --------------------------------------------------------------------------
     def set_pipeline(self, on=True):
@@ -60,6 +69,8 @@ class CharmNumericInterface:
             L.check(L.lib.cnx_set_min_tile(self._ex, nd, t))
         if self._solver:
             L.check(L.lib.cnx_set_solver(self._ex, 1))
+        if not self._flat3:
+            L.check(L.lib.cnx_set_layout(self._ex, 0))
         if self._pipeline:
             L.check(L.lib.cnx_set_async(self._ex, 1))
         return self

@@ -83,6 +83,11 @@ int cnx_set_min_tile(cnx_executor* ex, int ndims, int min_tile);
  * gather; a product or paired reduction whose operand's tile grid does not start at element 0
  * works on a copy that does. */
 int cnx_set_solver(cnx_executor* ex, int on);
+/* Storage of rank-3 arrays created from now on. flat_rank3 != 0 (default): one row-major block
+ * over the whole array, its partitions (src/backend.hpp:112-200 keeps one buffer per chare) being
+ * views into it with the array's row and plane pitches; stencil sweeps then run on the block as a
+ * whole. 0: one contiguous buffer per partition, as for the other ranks. Values never depend on it. */
+int cnx_set_layout(cnx_executor* ex, int flat_rank3);
 
 /* ArrayDAGGroup::receive_dag(int epoch, int size, char msg[size]) (src/backend.ci:15,
  * src/dag_group_receive.cpp:190-575) followed by the partitions' run(): executes every node of the

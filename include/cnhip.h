@@ -97,6 +97,10 @@ int cnh_version(void);
  *                    2 rows of tiles along x
  *   "direct_stagger" concurrent groups start at different places of their tiles (default 0)
  *   "direct_merge"   lean part and the rest in one launch (default 1) or two
+ *   "direct_flat"    arrays whose tiles are views into one row-major block take the whole-array
+ *                    register-window kernel (default 1)
+ *   "flat_obz/oby/obx"  extents in elements of the blocks that kernel's workgroups are ordered by
+ *                    (default 256^3 for rank 3, bands of whole rows for rank 2)
  *   "tiles_rows"     general gather: rows shorter than 1024 elements share a workgroup (default 1)
  *   "slide_bx/ry/zc/pd", "slide2d_march"  geometry of the sliding-window kernel */
 int cnh_set_option(const char* name, int value);

@@ -206,7 +206,7 @@ def test_jacobi2d_sweeps_match_numpy_bit_for_bit(small_tiles):
     assert st["compiled"] <= 4 and st["cache_hits"] >= 6
 
 
-def test_jacobi3d_sweeps_with_residual(small_tiles):
+def test_jacobi3d_sweeps_with_residual(small_tiles, rank3_layout):
     n = 20
     u = cnp.random.uniform((n, n, n), seed=1, stream=0, low=0.0, high=1.0)
     _faces(u, 0.0)
@@ -243,7 +243,7 @@ def test_c1_statement_and_reductions(itf):
     assert abs(zz - math.fsum(hz * hz)) <= 1e-12 * np.sum(hz * hz)
 
 
-def test_put_get_roundtrip_on_ragged_tiles(small_tiles):
+def test_put_get_roundtrip_on_ragged_tiles(small_tiles, rank3_layout):
     rng = np.random.default_rng(11)
     for shape, dt in [((200,), np.float64), ((37, 53), np.float32), ((9, 14, 21), np.int64),
                       ((70, 70), np.int32)]:
@@ -349,8 +349,15 @@ def _lstm_numpy(X, h0, W, n, b, d, word):
     return Hout, Cc, IFOG
 
 
+@pytest.fixture(params=[True, False], ids=["one-block", "buffer-per-partition"])
+def rank3_layout(request, itf):
+    """Both storage forms of rank-3 arrays."""
+    itf.set_layout(request.param)
+    return request.param
+
+
 @pytest.mark.parametrize("n,b,d,word,small", [(4, 32, 10, 10, False), (3, 48, 40, 24, True)])
-def test_lstm_forward_example(itf, n, b, d, word, small):
+def test_lstm_forward_example(itf, rank3_layout, n, b, d, word, small):
     """examples/lstm_forward.py upstream: 3-D state arrays, one time step per leading index, a
     dimension-dropped matmul per step, tile() for the first hidden state, in-place cell update."""
     if small:
@@ -418,7 +425,7 @@ def test_pipelined_executor_gives_the_same_results(small_tiles):
     assert np.array_equal(x.get(itf), hx)
 
 
-def test_tile_matches_numpy(small_tiles):
+def test_tile_matches_numpy(small_tiles, rank3_layout):
     host = np.arange(12, dtype=np.float64).reshape(3, 4)
     a = cnp.array(host)
     for reps in [(2, 3), (1, 1), 2, (2, 1, 2), (5, 1)]:

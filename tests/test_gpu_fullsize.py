@@ -11,9 +11,10 @@ from tests import helpers as H
 pytestmark = pytest.mark.gpu
 
 
-def _connect(odf):
+def _connect(odf, flat_rank3=True):
     cnp.reset()
     it = cnp.CharmNumericInterface(device=0)
+    it.set_layout(flat_rank3)
     it.connect(odf=odf)
     return it
 
@@ -39,9 +40,10 @@ def test_jacobi2d_8192_two_sweeps_match_numpy():
         itf.close()
 
 
-def test_jacobi3d_512_two_sweeps_match_numpy():
+@pytest.mark.parametrize("flat_rank3", [True, False], ids=["one-block", "buffer-per-partition"])
+def test_jacobi3d_512_two_sweeps_match_numpy(flat_rank3):
     n = 512
-    itf = _connect(64)
+    itf = _connect(64, flat_rank3)
     try:
         u = cnp.random.uniform((n, n, n), seed=1, stream=0, low=0.0, high=1.0)
         w = H.np_uniform(n * n * n, 1, 0, 0.0, 1.0).reshape(n, n, n)
@@ -63,13 +65,14 @@ def test_jacobi3d_512_two_sweeps_match_numpy():
         itf.close()
 
 
+@pytest.mark.parametrize("flat_rank3", [True, False], ids=["one-block", "buffer-per-partition"])
 @pytest.mark.parametrize("tx,ry,rz", [(16, 2, 4), (16, 1, 2), (32, 4, 1)])
-def test_small_workgroup_footprints_reach_the_interior_paths(tx, ry, rz):
+def test_small_workgroup_footprints_reach_the_interior_paths(tx, ry, rz, flat_rank3):
     """Narrow workgroups make interior workgroups, lane exchange at row ends inside a wavefront
     and ordering groups occur on small arrays too (256^3 in 8 tiles of 128^3, 700^2 in 4 tiles)."""
     for name, v in (("direct_tx", tx), ("direct_ry", ry), ("direct_rz", rz)):
         L.check(L.lib.cnh_set_option(name.encode(), v))
-    itf = _connect(8)
+    itf = _connect(8, flat_rank3)
     try:
         n = 256
         u = cnp.random.uniform((n, n, n), seed=7, stream=0, low=-1.0, high=1.0)

@@ -106,33 +106,44 @@ def test_source_term_at_a_shifted_position_takes_the_general_gather(dev):
     assert np.array_equal(got, want) and not took_direct
 
 
-def _pitched_views(dev, host, tile):
-    """One row-major block on the device and a descriptor whose tiles are views into it."""
+def _pitched_views(dev, host, tile, pad=(0, 0)):
+    """One row-major block on the device and a descriptor whose tiles are views into it. `pad`
+    = extra elements per row and extra rows per plane between the array's own."""
     import ctypes as C
-    nd, n = host.ndim, host.shape[0]
-    block = dev.array(host)
-    g = (n + tile - 1) // tile
-    ptrs = (C.c_void_p * (g ** nd))()
-    for i, idx in enumerate(np.ndindex(*([g] * nd))):
-        off = 0
-        for d in range(nd):
-            off = off * n + idx[d] * tile
-        ptrs[i] = block.ptr + off * 8
+    nd, shape = host.ndim, host.shape
+    padded = list(shape)
+    padded[-1] += pad[0]
+    if nd == 3:
+        padded[1] += pad[1]
+    store = np.full(padded, -777.0, dtype=host.dtype)
+    store[tuple(slice(0, s) for s in shape)] = host
+    block = dev.array(store)
+    pitch = [1] * nd
+    for k in range(nd - 2, -1, -1):
+        pitch[k] = pitch[k + 1] * padded[k + 1]
+    grid = [(s + tile - 1) // tile for s in shape]
+    ptrs = (C.c_void_p * int(np.prod(grid)))()
+    for i, idx in enumerate(np.ndindex(*grid)):
+        ptrs[i] = block.ptr + sum(idx[k] * tile * pitch[k] for k in range(nd)) * host.dtype.itemsize
     d = L.Tiled()
     d.ndims, d.tile = nd, tile
     for k in range(nd):
-        d.offset[k], d.shape[k], d.grid_lo[k], d.grid[k] = 0, n, 0, g
-        d.pitch[k] = n ** (nd - 1 - k)
+        d.offset[k], d.shape[k], d.grid_lo[k], d.grid[k] = 0, shape[k], 0, grid[k]
+        d.pitch[k] = pitch[k]
     d.tiles = C.cast(ptrs, C.POINTER(C.c_void_p))
+    block.view = lambda: block.get()[tuple(slice(0, s) for s in shape)]
+    block.padding_untouched = lambda: bool(np.all(block.get()[..., shape[-1]:] == -777.0))
     return block, ptrs, d
 
 
+@pytest.mark.parametrize("flat", [1, 0])
 @pytest.mark.parametrize("nd,n,tile,source", [(2, 70, 32, False), (2, 256, 128, True), (3, 36, 16, False),
                                                (3, 64, 32, True)])
-def test_tiles_as_pitched_views_into_one_block(dev, nd, n, tile, source):
-    """The register-window kernels take tiles that are views into one row-major block (common row
-    and plane pitches): an array stored whole, addressed through the same tile grid. Bit for bit
-    against NumPy; other kernels refuse such descriptors."""
+def test_tiles_as_pitched_views_into_one_block(dev, nd, n, tile, source, flat):
+    """Tiles that are views into one row-major block (common row and plane pitches): an array
+    stored whole, addressed through the same tile grid. With direct_flat the whole-array kernel
+    runs, without it the per-tile register-window kernels with pitches; the general gather takes
+    such views too. Bit for bit against NumPy."""
     import ctypes as C
     rng = np.random.default_rng(n + nd)
     u0, f0 = rng.standard_normal((n,) * nd), rng.standard_normal((n,) * nd)
@@ -141,28 +152,134 @@ def test_tiles_as_pitched_views_into_one_block(dev, nd, n, tile, source):
         ast = H.ast_poisson2d(n, coef=coef) if nd == 2 else H.ast_poisson3d(n, coef=coef)
     else:
         ast = H.ast_jacobi2d(n, coef=coef) if nd == 2 else H.ast_jacobi3d(n, coef=coef)
+    step = (lambda r: H.np_poisson(r, f0, coef)) if source else (
+        (lambda r: H.np_jacobi2d(r, coef)) if nd == 2 else (lambda r: H.np_jacobi3d(r, coef)))
     k = H.compile_group(ast, L.F64, nd)
     ba, _pa, da = _pitched_views(dev, u0, tile)
     bb, _pb, db = _pitched_views(dev, np.zeros_like(u0), tile)
     bf, _pf, df = _pitched_views(dev, f0, tile)
     nleaf = 2 * nd + (1 if source else 0)
     ref = u0.copy()
-    for _ in range(3):
+    L.check(L.lib.cnh_set_option(b"direct_flat", flat))
+    try:
+        for _ in range(3):
+            descs = (L.Tiled * nleaf)(*([da] * (2 * nd) + ([df] if source else [])))
+            L.check(L.lib.cnh_launch_group_tiles(k, nleaf, descs, 0, None, 0, C.byref(da), C.byref(db), None))
+            da, db, ba, bb = db, da, bb, ba
+            ref = step(ref)
+        dev.sync()
+        assert np.array_equal(ba.view(), ref)
+        assert L.lib.cnh_kernel_variants_loaded(k, b"direct") == 1
+        # one more sweep through the general gather
+        L.check(L.lib.cnh_set_option(b"stencil_mode", 0))
         descs = (L.Tiled * nleaf)(*([da] * (2 * nd) + ([df] if source else [])))
         L.check(L.lib.cnh_launch_group_tiles(k, nleaf, descs, 0, None, 0, C.byref(da), C.byref(db), None))
-        da, db, ba, bb = db, da, bb, ba
-        ref = H.np_poisson(ref, f0, coef) if source else (H.np_jacobi2d(ref, coef) if nd == 2 else H.np_jacobi3d(ref, coef))
-    dev.sync()
-    got = ba.get().reshape(u0.shape)
-    assert np.array_equal(got, ref)
-    assert L.lib.cnh_kernel_variants_loaded(k, b"direct") == 1
-    # the general gather addresses tiles through their own extents: pitched views are refused
-    L.check(L.lib.cnh_set_option(b"stencil_mode", 0))
-    try:
-        descs = (L.Tiled * nleaf)(*([da] * (2 * nd) + ([df] if source else [])))
-        assert L.lib.cnh_launch_group_tiles(k, nleaf, descs, 0, None, 0, C.byref(da), C.byref(db), None) != 0
+        dev.sync()
+        assert np.array_equal(bb.view(), step(ref))
+        assert L.lib.cnh_kernel_variants_loaded(k, b"tiles") == 1
     finally:
         L.check(L.lib.cnh_set_option(b"stencil_mode", 2))
+        L.check(L.lib.cnh_set_option(b"direct_flat", 1))
+    dev.free_all()
+
+
+def _ast_star(shape, dtype=L.F64, coef=0.125, source=False, target=0, window=0):
+    """target[1:-1,..] = coef * (sum of the 2*nd face neighbours of `window` [+ f[1:-1,..]]) on an
+    array of any extents (array names: window, target, f = 9)."""
+    nd = len(shape)
+    b = AstBuilder(dtype, nd)
+    w = b.leaf(window)
+    tgt = w if target == window else b.leaf(target)
+
+    def reg(shift):
+        return (tuple(shift), tuple(s + e - 2 for s, e in zip(shift, shape)), (1,) * nd)
+
+    shifts = []
+    for d in range(nd):
+        lo, hi = [1] * nd, [1] * nd
+        lo[d], hi[d] = 0, 2
+        shifts += [reg(lo), reg(hi)]
+    t = b.binary(L.OP_ADD, 100, w, w, shifts[0], shifts[1])
+    for i, r in enumerate(shifts[2:]):
+        t = b.binary(L.OP_ADD, 101 + i, t, w, None, r)
+    if source:
+        t = b.binary(L.OP_ADD, 119, t, b.leaf(9), None, reg([1] * nd))
+    t = b.binary(L.OP_MUL, 120, b.scalar(coef), t)
+    b.set_region(121, tgt, t, reg([1] * nd))
+    return b.finish()
+
+
+def _np_star(u, coef, f=None):
+    nd = u.ndim
+    mid = (slice(1, -1),) * nd
+    acc = None
+    for d in range(nd):
+        for sl in (slice(0, -2), slice(2, None)):
+            idx = tuple(sl if k == d else slice(1, -1) for k in range(nd))
+            acc = u[idx] if acc is None else acc + u[idx]
+    if f is not None:
+        acc = acc + f[mid]
+    return mid, coef * acc
+
+
+@pytest.mark.parametrize("shape,tile,pad,ob", [
+    ((9, 17, 130), 8, (0, 0), None), ((9, 17, 130), 16, (6, 1), (8, 16, 128)), ((33, 40, 258), 32, (2, 0), (16, 32, 256)),
+    ((50, 300), 64, (0, 0), None), ((37, 128), 32, (4, 0), (0, 16, 128)), ((5, 9, 2), 4, (0, 0), None),
+    ((130, 1026), 128, (0, 0), (0, 64, 512)), ((64, 72, 384), 64, (0, 0), None)])
+@pytest.mark.parametrize("source", [False, True])
+def test_whole_array_kernel_on_ragged_blocks(dev, shape, tile, pad, ob, source):
+    """The whole-array register-window kernel on extents that are no multiple of a wavefront's
+    128 columns, of a workgroup's rows and planes or of the ordering block, with padded rows and
+    planes: bit for bit against NumPy, and nothing written between the rows."""
+    import ctypes as C
+    nd = len(shape)
+    rng = np.random.default_rng(sum(shape))
+    u0, f0 = rng.standard_normal(shape), rng.standard_normal(shape)
+    k = H.compile_group(_ast_star(shape, source=source), L.F64, nd)
+    ba, _pa, da = _pitched_views(dev, u0, tile, pad)
+    bb, _pb, db = _pitched_views(dev, np.zeros_like(u0), tile, pad)
+    bf, _pf, df = _pitched_views(dev, f0, tile, pad)
+    nleaf = 2 * nd + (1 if source else 0)
+    for name, v in zip((b"flat_obz", b"flat_oby", b"flat_obx"), ob or (0, 0, 0)):
+        L.check(L.lib.cnh_set_option(name, v))
+    try:
+        ref = u0.copy()
+        for _ in range(2):
+            descs = (L.Tiled * nleaf)(*([da] * (2 * nd) + ([df] if source else [])))
+            L.check(L.lib.cnh_launch_group_tiles(k, nleaf, descs, 0, None, 0, C.byref(da), C.byref(db), None))
+            da, db, ba, bb = db, da, bb, ba
+            mid, val = _np_star(ref, 0.125, f0 if source else None)
+            ref = ref.copy()
+            ref[mid] = val
+        dev.sync()
+        assert np.array_equal(ba.view(), ref)
+        assert ba.padding_untouched() and bb.padding_untouched()
+        assert L.lib.cnh_kernel_variants_loaded(k, b"direct") == 1
+    finally:
+        for name in (b"flat_obz", b"flat_oby", b"flat_obx"):
+            L.check(L.lib.cnh_set_option(name, 0))
+    dev.free_all()
+
+
+def test_whole_array_kernel_from_one_array_into_another(dev):
+    """unew[interior] = f(u shifted): the window array is not the assigned one; only assigned
+    elements of the target are written."""
+    import ctypes as C
+    shape, tile = (20, 24, 260), 16
+    rng = np.random.default_rng(4)
+    u0, t0 = rng.standard_normal(shape), rng.standard_normal(shape)
+    k = H.compile_group(_ast_star(shape, target=1, window=0), L.F64, 3)
+    bu, _pu, du = _pitched_views(dev, u0, tile)
+    bt, _pt, dt = _pitched_views(dev, t0, tile)
+    descs = (L.Tiled * 6)(*([du] * 6))
+    L.check(L.lib.cnh_launch_group_tiles(k, 6, descs, 0, None, 0, C.byref(dt), C.byref(dt), None))
+    dev.sync()
+    mid, val = _np_star(u0, 0.125)
+    want = t0.copy()
+    want[mid] = val
+    assert np.array_equal(bt.view(), want)
+    assert np.array_equal(bu.view(), u0)
+    assert L.lib.cnh_kernel_variants_loaded(k, b"direct") == 1
     dev.free_all()
 
 
