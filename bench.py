@@ -424,7 +424,7 @@ class TiledDev:
     def __init__(self, L, nd, n, tile, skew=None):
         self.L, self.nd, self.n, self.tile = L, nd, n, tile
         self.g = (n + tile - 1) // tile
-        self.flat = nd == 3 and not os.environ.get("CNH_BENCH_TILE_MAJOR")
+        self.flat = (nd == 3 or bool(os.environ.get("CNH_BENCH_FLAT2"))) and not os.environ.get("CNH_BENCH_TILE_MAJOR")
         if skew is None:
             skew = (2 << 20) + 256 if nd == 3 else 0
             if os.environ.get("CNH_BENCH_SKEW"):
@@ -469,7 +469,7 @@ def run_jacobi(L, nd, n, tile, sweeps, reduce_every=10, reps_note=""):
         if nd == 2:
             if idx[0] == 0:
                 one = np.array([1.0]).view(np.uint8)
-                L.check(L.lib.cnh_fill_region(2, 8, buf.ptr, L.i64arr([ext[1], 1]), L.i64arr([0, 0]),
+                L.check(L.lib.cnh_fill_region(2, 8, buf.ptr, L.i64arr(a.strides(ext)), L.i64arr([0, 0]),
                                               L.i64arr([1, 1]), L.i64arr([1, ext[1]]),
                                               one.ctypes.data, None))
     if nd == 3:
@@ -487,6 +487,12 @@ def run_jacobi(L, nd, n, tile, sweeps, reduce_every=10, reps_note=""):
         L.check(L.lib.cnh_launch_group_tiles(k, nleaf, descs, 0, None, 0, C.byref(src.desc),
                                              C.byref(dst.desc), None))
 
+    def sweep_with_residual(src, dst):
+        # the sweep accumulates sum (new - old)^2 (2-D) or max |new - old| (3-D) on the way
+        descs = (L.Tiled * nleaf)(*([src.desc] * nleaf))
+        L.check(L.lib.cnh_launch_group_tiles_residual(k, nleaf, descs, 0, None, 0, C.byref(src.desc),
+                                                      C.byref(dst.desc), 0 if nd == 2 else 1, res.ptr, None))
+
     def residual(src, dst):
         fn = L.lib.cnh_sumsq_diff_tiles if nd == 2 else L.lib.cnh_maxabs_diff_tiles
         if a.flat:
@@ -496,40 +502,72 @@ def run_jacobi(L, nd, n, tile, sweeps, reduce_every=10, reps_note=""):
 
     for _ in range(3):
         sweep(a, b)
-        sweep(b, a)
+        sweep_with_residual(b, a)
     L.check(L.lib.cnh_device_sync())
     ev = Events(L, sweeps)
-    evr = Events(L, max(1, sweeps // reduce_every))
     e0, e1 = C.c_void_p(), C.c_void_p()
     L.check(L.lib.cnh_event_create(C.byref(e0)))
     L.check(L.lib.cnh_event_create(C.byref(e1)))
     L.check(L.lib.cnh_event_record(e0, None))
     cur, nxt = a, b
-    nres = 0
+    reducing = []
     for i in range(sweeps):
         L.check(L.lib.cnh_event_record(ev.a[i], None))
-        sweep(cur, nxt)
-        L.check(L.lib.cnh_event_record(ev.b[i], None))
         if (i + 1) % reduce_every == 0:
-            L.check(L.lib.cnh_event_record(evr.a[nres], None))
-            residual(cur, nxt)
-            L.check(L.lib.cnh_event_record(evr.b[nres], None))
-            nres += 1
+            sweep_with_residual(cur, nxt)
+            reducing.append(i)
+        else:
+            sweep(cur, nxt)
+        L.check(L.lib.cnh_event_record(ev.b[i], None))
         cur, nxt = nxt, cur
     L.check(L.lib.cnh_event_record(e1, None))
     L.check(L.lib.cnh_device_sync())
     ms = C.c_float()
     L.check(L.lib.cnh_event_elapsed_ms(e0, e1, C.byref(ms)))
     t = ev.times_ms(sweeps)
-    tr = evr.times_ms(nres) if nres else [0.0]
-    us = 1e3 * float(np.median(t))
+    last_fused = float(res.get(np.float64)[0])
+    # The whole run again between two events only (an event pair around every sweep costs a few
+    # microseconds per sweep itself): once with the residual every reduce_every sweeps, once without.
+    totals = {}
+    for label, with_res in (("with", True), ("without", False)):
+        L.check(L.lib.cnh_device_sync())
+        L.check(L.lib.cnh_event_record(e0, None))
+        cur, nxt = a, b
+        for i in range(sweeps):
+            if with_res and (i + 1) % reduce_every == 0:
+                sweep_with_residual(cur, nxt)
+            else:
+                sweep(cur, nxt)
+            cur, nxt = nxt, cur
+        L.check(L.lib.cnh_event_record(e1, None))
+        L.check(L.lib.cnh_device_sync())
+        L.check(L.lib.cnh_event_elapsed_ms(e0, e1, C.byref(ms)))
+        totals[label] = ms.value
+    # the same residual by a second pass over both buffers (what every tenth sweep cost before the
+    # sweep accumulated it on the way), for comparison and as a check
+    evr = Events(L, 5)
+    for i in range(5):
+        L.check(L.lib.cnh_event_record(evr.a[i], None))
+        residual(nxt, cur)              # cur holds the newest contents, nxt the ones before
+        L.check(L.lib.cnh_event_record(evr.b[i], None))
+    L.check(L.lib.cnh_device_sync())
+    tr = evr.times_ms(5)
+    last_separate = float(res.get(np.float64)[0])
+    plain = [t[i] for i in range(sweeps) if i not in reducing]
+    us = 1e3 * float(np.median(plain))
+    us_red = 1e3 * float(np.median([t[i] for i in reducing])) if reducing else None
     interior = (n - 2) ** nd
     nbytes = 8.0 * ((n ** nd - (4 if nd == 2 else 0)) + interior) if nd == 2 else 8.0 * (n ** 3 + interior)
     out = {"sweeps": sweeps, "us_per_sweep": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
            "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
-           "bytes_per_sweep": nbytes, "total_ms_with_reductions": round(ms.value, 3),
-           "reduction_us": round(1e3 * float(np.median(tr)), 2),
-           "last_reduction": float(res.get(np.float64)[0]), "partitions": len(a.bufs), "tile": tile,
+           "bytes_per_sweep": nbytes, "total_ms_with_reductions": round(totals["with"], 3),
+           "total_ms_without_reductions": round(totals["without"], 3),
+           "reductions_add_pct": round(100.0 * (totals["with"] / totals["without"] - 1.0), 2),
+           "sweeps_times_us_per_sweep_ms": round(sweeps * us / 1e3, 3),
+           "us_per_reducing_sweep": round(us_red, 2) if us_red else None,
+           "separate_reduction_pass_us": round(1e3 * float(np.median(tr)), 2),
+           "last_reduction": last_fused, "last_reduction_by_separate_pass": last_separate,
+           "partitions": len(a.bufs), "tile": tile,
            "layout": "one block, partitions as views" if a.flat else "one buffer per partition"}
     ev.free()
     evr.free()
@@ -600,7 +638,60 @@ def lstm_asts(L, d):
     return sigmoid(), tanh(), mul(), muladd()
 
 
-def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=False):
+def lstm_fused_ast(L, first):
+    """All gate statements of one step (examples/lstm_forward.py:40-49 upstream) as one group with
+    several output roots, each statement over its (batch x d) column window; later roots read
+    earlier ones from registers. Leaves: 1..4 = the i, f, o, g windows of IFOG[t], 5 = C[t-1].
+    Outputs: 11..14 = the windows of IFOGf[t], 15 = C[t], 16 = tanh(C[t]), 17 = Hout[t],
+    18 = the same values again, for the right half of Hin[t+1]."""
+    from charmnumeric_amd.astbuild import AstBuilder
+
+    b = AstBuilder(L.F64, 2)
+
+    def sigmoid(src, name, tmp):
+        t0 = b.binary(L.OP_MUL, tmp, b.leaf(src), b.scalar(-1))
+        t1 = b.unary(L.OP_EXP, tmp + 1, t0)
+        t2 = b.binary(L.OP_ADD, tmp + 2, b.scalar(1.0), t1)
+        return b.binary(L.OP_DIV, name, b.scalar(1.0), t2, is_temp=False)
+
+    gi = sigmoid(1, 11, 100)
+    gf = sigmoid(2, 12, 110)
+    go = sigmoid(3, 13, 120)
+    gg = b.unary(L.OP_TANH, 14, b.leaf(4), is_temp=False)
+    if first:
+        c = b.binary(L.OP_MUL, 15, gi, gg, is_temp=False)
+    else:
+        c0 = b.binary(L.OP_MUL, 130, gi, gg)
+        fc = b.binary(L.OP_MUL, 131, gf, b.leaf(5))
+        c = b.binary(L.OP_ADD, 15, c0, fc, is_temp=False)
+    ct = b.unary(L.OP_TANH, 16, c, is_temp=False)
+    h = b.binary(L.OP_MUL, 17, go, ct, is_temp=False)
+    idx = b._new(18, L.OP_COPY, is_temp=False)
+    node = b._nodes[idx]
+    node.n_operands = 1
+    b._attach(node, 0, h, None)
+    b._roots.append(idx)
+    return b.finish()
+
+
+def _launch_named(L, k, nd, ins, outs, stream=None):
+    """One partition; memrefs given by leaf name and by output name."""
+    n_in, n_sc, n_out = C.c_int(), C.c_int(), C.c_int()
+    L.check(L.lib.cnh_kernel_signature(k, C.byref(n_in), C.byref(n_sc), C.byref(n_out)))
+    name, has, tgt, sr = C.c_int(), C.c_int(), C.c_int(), C.c_int()
+    reg = L.Region()
+    ia = (L.Memref * max(1, n_in.value))()
+    oa = (L.Memref * max(1, n_out.value))()
+    for i in range(n_in.value):
+        L.check(L.lib.cnh_kernel_input(k, i, C.byref(name), C.byref(has), C.byref(reg)))
+        ia[i] = ins[name.value]
+    for i in range(n_out.value):
+        L.check(L.lib.cnh_kernel_output(k, i, C.byref(name), C.byref(tgt), C.byref(sr), C.byref(reg)))
+        oa[i] = outs[name.value]
+    L.check(L.lib.cnh_launch_group(k, nd, n_in.value, ia, 0, None, 1, n_out.value, oa, stream))
+
+
+def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=False, fused=True):
     k_in = nin + d
     X = Buf(L, steps * batch * nin * 8)
     W = Buf(L, k_in * 4 * d * 8)
@@ -630,6 +721,8 @@ def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=
     Hout = Buf(L, steps * batch * d * 8, zero=True)
     a_sig, a_tanh, a_mul, a_muladd = lstm_asts(L, d)
     k_sig, k_tanh, k_mul, k_muladd = (_compile(L, a, L.F64, 2) for a in (a_sig, a_tanh, a_mul, a_muladd))
+    k_first, k_later = (_compile(L, lstm_fused_ast(L, f), L.F64, 2) for f in (True, False))
+    spare = Buf(L, batch * d * 8)      # where the last step's copy of h goes (no Hin[steps])
 
     def view(buf, t, row_len, c0, ncols):
         base = buf.ptr + (t * batch * row_len + c0) * 8
@@ -654,7 +747,7 @@ def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=
         L.check(L.lib.cnh_copy_region(2, 8, Hin.ptr + t * batch * k_in * 8, i64([k_in, 1]), zero2, one,
                                       X.ptr + t * batch * nin * 8, i64([nin, 1]), zero2, one,
                                       i64([batch, nin]), None))
-        if t > 0:
+        if t > 0 and not fused:
             L.check(L.lib.cnh_copy_region(2, 8, Hin.ptr + (t * batch * k_in + nin) * 8, i64([k_in, 1]),
                                           zero2, one, Hout.ptr + (t - 1) * batch * d * 8, i64([d, 1]),
                                           zero2, one, i64([batch, d]), None))
@@ -663,17 +756,31 @@ def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=
         gate_product(t)
         if record:
             L.check(L.lib.cnh_event_record(ev.b[t], None))
-        _launch1(L, k_sig, 2, [view(IFOG, t, 4 * d, 0, 3 * d)], [], [view(IFOGf, t, 4 * d, 0, 3 * d)])
-        _launch1(L, k_tanh, 2, [view(IFOG, t, 4 * d, 3 * d, d)], [], [view(IFOGf, t, 4 * d, 3 * d, d)])
-        _launch1(L, k_mul, 2, [view(IFOGf, t, 4 * d, 0, d), view(IFOGf, t, 4 * d, 3 * d, d)], [],
-                 [view(Cc, t, d, 0, d)])
-        if t > 0:
-            # leaf uses are collected root by root: (f, C[t-1]) of the product, then C[t]
-            _launch1(L, k_muladd, 2, [view(IFOGf, t, 4 * d, d, d), view(Cc, t - 1, d, 0, d),
-                                      view(Cc, t, d, 0, d)], [], [view(Cc, t, d, 0, d)])
-        _launch1(L, k_tanh, 2, [view(Cc, t, d, 0, d)], [], [view(Ct, t, d, 0, d)])
-        _launch1(L, k_mul, 2, [view(IFOGf, t, 4 * d, 2 * d, d), view(Ct, t, d, 0, d)], [],
-                 [view(Hout, t, d, 0, d)])
+        if fused:
+            # every gate statement of the step in one launch; h goes to Hout[t] and, for the next
+            # step's product, to the right half of Hin[t+1]
+            ins = {1: view(IFOG, t, 4 * d, 0, d), 2: view(IFOG, t, 4 * d, d, d),
+                   3: view(IFOG, t, 4 * d, 2 * d, d), 4: view(IFOG, t, 4 * d, 3 * d, d)}
+            if t > 0:
+                ins[5] = view(Cc, t - 1, d, 0, d)
+            nxt = (view(Hin, t + 1, k_in, nin, d) if t + 1 < steps
+                   else L.Memref.strided(spare.ptr, (batch, d), (d, 1)))
+            outs = {11: view(IFOGf, t, 4 * d, 0, d), 12: view(IFOGf, t, 4 * d, d, d),
+                    13: view(IFOGf, t, 4 * d, 2 * d, d), 14: view(IFOGf, t, 4 * d, 3 * d, d),
+                    15: view(Cc, t, d, 0, d), 16: view(Ct, t, d, 0, d), 17: view(Hout, t, d, 0, d), 18: nxt}
+            _launch_named(L, k_first if t == 0 else k_later, 2, ins, outs)
+        else:
+            _launch1(L, k_sig, 2, [view(IFOG, t, 4 * d, 0, 3 * d)], [], [view(IFOGf, t, 4 * d, 0, 3 * d)])
+            _launch1(L, k_tanh, 2, [view(IFOG, t, 4 * d, 3 * d, d)], [], [view(IFOGf, t, 4 * d, 3 * d, d)])
+            _launch1(L, k_mul, 2, [view(IFOGf, t, 4 * d, 0, d), view(IFOGf, t, 4 * d, 3 * d, d)], [],
+                     [view(Cc, t, d, 0, d)])
+            if t > 0:
+                # leaf uses are collected root by root: (f, C[t-1]) of the product, then C[t]
+                _launch1(L, k_muladd, 2, [view(IFOGf, t, 4 * d, d, d), view(Cc, t - 1, d, 0, d),
+                                          view(Cc, t, d, 0, d)], [], [view(Cc, t, d, 0, d)])
+            _launch1(L, k_tanh, 2, [view(Cc, t, d, 0, d)], [], [view(Ct, t, d, 0, d)])
+            _launch1(L, k_mul, 2, [view(IFOGf, t, 4 * d, 2 * d, d), view(Ct, t, d, 0, d)], [],
+                     [view(Hout, t, d, 0, d)])
         if record:
             L.check(L.lib.cnh_event_record(evs.b[t], None))
 
@@ -702,7 +809,8 @@ def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=
         out["IFOG"] = IFOG.get().reshape(steps, batch, 4 * d)
     ev.free()
     evs.free()
-    for b_ in (X, W, Hin, IFOG, IFOGf, Cc, Ct, Hout):
+    out["gate_launches_per_step"] = 1 if fused else 6
+    for b_ in (X, W, Hin, IFOG, IFOGf, Cc, Ct, Hout, spare):
         b_.free()
     return out
 

@@ -216,6 +216,9 @@ _PROTOS = {
                                            C.POINTER(Memref), C.c_void_p]),
     "cnh_launch_group_tiles": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(Tiled), C.c_int, _vpp,
                                          C.c_int, C.POINTER(Tiled), C.POINTER(Tiled), C.c_void_p]),
+    "cnh_launch_group_tiles_residual": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(Tiled), C.c_int, _vpp,
+                                                  C.c_int, C.POINTER(Tiled), C.POINTER(Tiled), C.c_int,
+                                                  C.c_void_p, C.c_void_p]),
     "cnh_dot_partial": (C.c_int, [C.c_int, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p,
                                   C.c_void_p]),
     "cnh_dot_partial_noalloc": (C.c_int, [C.c_int, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p,

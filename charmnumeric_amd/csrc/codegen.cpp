@@ -441,8 +441,10 @@ struct Cell {
     const T* in[NLA]; i64 istr[NLA][3];
     T* out[NOA]; i64 ostr[NOA][3];
 };
-#define ND_PER_THREAD 4
-
+// PER elements per lane, 256 apart: 4 for large launches; 1 for small ones, which then spread over
+// four times as many wavefronts (a 256 x 1024 gate statement with exp and tanh in fp64: 19.6 us
+// with one wavefront per SIMD busy, latency-bound).
+template <int ND_PER_THREAD>
 __device__ __forceinline__ void nd_run(const Cell& c, i64 blk, const T* s) {
     const i64 outer = blk / c.nchunks;
     const i64 chunk = blk - outer * c.nchunks;
@@ -477,11 +479,20 @@ __device__ __forceinline__ void nd_run(const Cell& c, i64 blk, const T* s) {
 extern "C" __global__ __launch_bounds__(256) void grp_nd(const Cell* cells, int ncell, Scal sc) {
     T s[NSA]; load_scalars(sc, s);
     const int k = find_seg(cells, ncell, (i64)blockIdx.x);
-    nd_run(cells[k], (i64)blockIdx.x - cells[k].blk0, s);
+    nd_run<4>(cells[k], (i64)blockIdx.x - cells[k].blk0, s);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_nd1(Cell cell, Scal sc) {
     T s[NSA]; load_scalars(sc, s);
-    nd_run(cell, (i64)blockIdx.x, s);
+    nd_run<4>(cell, (i64)blockIdx.x, s);
+}
+extern "C" __global__ __launch_bounds__(256) void grp_nd_p1(const Cell* cells, int ncell, Scal sc) {
+    T s[NSA]; load_scalars(sc, s);
+    const int k = find_seg(cells, ncell, (i64)blockIdx.x);
+    nd_run<1>(cells[k], (i64)blockIdx.x - cells[k].blk0, s);
+}
+extern "C" __global__ __launch_bounds__(256) void grp_nd1_p1(Cell cell, Scal sc) {
+    T s[NSA]; load_scalars(sc, s);
+    nd_run<1>(cell, (i64)blockIdx.x, s);
 }
 )";
     return s.str();
@@ -614,7 +625,7 @@ std::string direct_source(const GroupProgram& p, const DirectConfig& cfg, std::s
 
 std::string DirectConfig::variant() const {
     char buf[64];
-    snprintf(buf, sizeof buf, "direct@%d,%d,%d", tx, ry, rz);
+    snprintf(buf, sizeof buf, "direct%s@%d,%d,%d", reduce ? "r" : "", tx, ry, rz);
     return buf;
 }
 
@@ -622,6 +633,14 @@ bool DirectConfig::parse(const std::string& variant, DirectConfig& out) {
     out = DirectConfig();
     if (variant == "direct")
         return true;
+    if (variant == "directr") {
+        out.reduce = true;
+        return true;
+    }
+    if (sscanf(variant.c_str(), "directr@%d,%d,%d", &out.tx, &out.ry, &out.rz) == 3) {
+        out.reduce = true;
+        return true;
+    }
     return sscanf(variant.c_str(), "direct@%d,%d,%d", &out.tx, &out.ry, &out.rz) == 3;
 }
 

@@ -71,7 +71,8 @@ int slide_shape(const GroupProgram& p, const SlideConfig& cfg, SlideShape& sh, s
 // Register-window stencil variant (no LDS): lane grid tx x (256/tx), ry rows and rz planes per lane.
 struct DirectConfig {
     int tx = 0, ry = 0, rz = 0;                       // 0 = built-in default
-    std::string variant() const;                      // "direct" or "direct@tx,ry,rz"
+    bool reduce = false;                              // the forms that also reduce what they change
+    std::string variant() const;                      // "direct@tx,ry,rz" or "directr@tx,ry,rz"
     static bool parse(const std::string& variant, DirectConfig& out);
 };
 struct DirectShape {

@@ -170,6 +170,7 @@ std::string direct_source(const GroupProgram& p, const DirectConfig& cfg, std::s
     s << "};\n";
     const int NOTH = (int)sh.other_names.size();
     s << "#define DR_MASKED " << (sh.masked ? 1 : 0) << "\n";
+    s << "#define DR_RED " << (cfg.reduce ? 1 : 0) << "\n";
     s << "#define DR_NOTH " << NOTH << "\n#define DR_NOTHA " << (NOTH > 0 ? NOTH : 1) << "\n";
     s << "__device__ constexpr int DR_OTHER[NLA] = {";
     for (size_t l = 0; l < sh.other.size(); ++l)
@@ -231,6 +232,7 @@ struct DirectArgs {
     int py, pz;            // elements between rows and between planes inside every tile when the
                            // tiles are views into one larger row-major block; 0: a tile is
                            // contiguous over its own extents
+    T* slots;              // reducing launches: one partial per launched wavefront
 };
 typedef T P2 __attribute__((ext_vector_type(2)));
 typedef int I2 __attribute__((ext_vector_type(2)));
@@ -285,6 +287,28 @@ __device__ __forceinline__ T from_next_lane(T v) { return lane_shift<0x130>(v); 
 __device__ __forceinline__ int wave_uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 #endif
 
+// Sum of a value over the 64 lanes of a wavefront in a fixed tree (all lanes active); lane 0
+// holds the result. MAXV: the maximum instead.
+template <bool MAXV, typename V>
+__device__ __forceinline__ V wave_combine(V v) {
+#ifndef DR_HOST_BUILD
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        V o;
+        if constexpr (sizeof(V) == 8) {
+            I2 a = __builtin_bit_cast(I2, v), r;
+            r[0] = __shfl_down(a[0], off, 64);
+            r[1] = __shfl_down(a[1], off, 64);
+            o = __builtin_bit_cast(V, r);
+        } else {
+            o = __builtin_bit_cast(V, __shfl_down(__builtin_bit_cast(int, v), off, 64));
+        }
+        v = MAXV ? (o > v ? o : v) : v + o;
+    }
+#endif
+    return v;
+}
+
 // Where a workgroup works: tile, tile extents, origin, and the patch inside the tile.
 struct Place {
     int t, t0, t1, t2;           // tile index and coordinates
@@ -334,8 +358,13 @@ __device__ __forceinline__ bool wave_is_fast(const DirectArgs& a, const Place& p
            p.tz0 + lz0 >= a.rs[0] && p.tz0 + lz0 + DR_RZ <= a.re[0];
 }
 
-template <bool NTS>
+// RED: 0 = plain sweep; 1 = also the sum over the assigned elements of (new - old)^2; 2 = also the
+// maximum of |new - old|. A reducing launch leaves one partial per launched wavefront in
+// a.slots[4 * workgroup + wavefront] (0 from wavefronts that have nothing to do), added up
+// afterwards in index order: the result never depends on scheduling.
+template <bool NTS, int RED>
 __device__ __forceinline__ void direct_fast(const DirectArgs& a, const T* s) {
+    T* const my_slot = RED ? a.slots + ((size_t)blockIdx.x * 4 + (threadIdx.x >> 6)) : nullptr;
     const Place p = locate(a, xcd_order(a, (int)blockIdx.x));
     const int tid = (int)threadIdx.x;
     const int wv = wave_uniform(tid >> 6);              // wavefront inside the workgroup
@@ -343,8 +372,11 @@ __device__ __forceinline__ void direct_fast(const DirectArgs& a, const T* s) {
     const int lz0 = p.bz * DR_RZ;
     const int ly0 = (p.by * DR_TY + (wv * 64) / DR_TX) * DR_RY;
     const int x0 = (p.bx * DR_TX + (wv * 64) % DR_TX) * 2;   // first column of the wavefront
-    if (lz0 >= p.w0 || ly0 >= p.w1 || x0 >= p.w2) return;
-    if (!wave_is_fast(a, p, lz0, ly0, x0)) return;
+    // (both exits are taken by whole wavefronts: DR_TX is a multiple of 64 on this path)
+    if (lz0 >= p.w0 || ly0 >= p.w1 || x0 >= p.w2 || !wave_is_fast(a, p, lz0, ly0, x0)) {
+        if (RED && lane == 0) *my_slot = (T)0;
+        return;
+    }
     const int w1 = p.w1, w2 = p.w2;
     const int lx = x0 + 2 * lane;
     const T* const own = a.cur[p.t];
@@ -442,6 +474,7 @@ __device__ __forceinline__ void direct_fast(const DirectArgs& a, const T* s) {
             }
         }
     T* const out_tile = a.dst[p.t];
+    T acc = (T)0;
 #pragma unroll
     for (int rz = 0; rz < DR_RZ; ++rz)
 #pragma unroll
@@ -463,19 +496,30 @@ __device__ __forceinline__ void direct_fast(const DirectArgs& a, const T* s) {
                 const int gx = p.tx0 + lx + e;
                 in_e[e] = gx >= a.rs[2] && gx < a.re[2];
                 res[e] = (DR_MASKED || in_e[e]) ? o[0] : win[rz + DR_H0][ry + DR_H1][DR_HK][e];
+                if (RED) {
+                    T d = o[0] - win[rz + DR_H0][ry + DR_H1][DR_HK][e];
+                    d = in_e[e] ? d : (T)0;
+                    if (RED == 1) acc = acc + d * d;
+                    else { d = d < (T)0 ? (T)0 - d : d; acc = d > acc ? d : acc; }
+                }
             }
             P2* out = reinterpret_cast<P2*>(out_tile + ((lz0 + rz) * PZ + (ly0 + ry) * PY + lx));
             store_pair<NTS>(out, res, in_e[0], in_e[1]);
         }
+    if (RED) {
+        acc = wave_combine<RED == 2, T>(acc);
+        if (lane == 0) *my_slot = acc;
+    }
 }
 
 // Everything the fast path leaves (or, with skip_fast = 0, everything): windows that touch
 // neighbour tiles in y or z, partial tiles, rows and planes outside the assigned region,
 // workgroups narrower than a wavefront. With a list, workgroup i does position list[i] of the
 // order (the host lists the workgroups on the y and z faces of the tiles); without, all of them.
-template <bool NTS>
+template <bool NTS, int RED>
 __device__ __forceinline__ void direct_rest(const DirectArgs& a, const T* s, int skip_fast,
                                             const int* list, int first_block) {
+    T* const my_slot = RED ? a.slots + ((size_t)blockIdx.x * 4 + (threadIdx.x >> 6)) : nullptr;
     const int me = (int)blockIdx.x - first_block;   // this workgroup's number among those doing the rest
     const Place p = locate(a, list ? list[me] : xcd_order(a, me));
     const int t = p.t, t0 = p.t0, t1 = p.t1, t2 = p.t2;
@@ -484,17 +528,28 @@ __device__ __forceinline__ void direct_rest(const DirectArgs& a, const T* s, int
     const int w0n = min(a.tile, a.shape[0] - tz0 - a.tile), w1n = min(a.tile, a.shape[1] - ty0 - a.tile),
               w2n = min(a.tile, a.shape[2] - tx0 - a.tile);
     const int lz0 = p.bz * DR_RZ;
-    if (lz0 >= w0) return;
     const int tid = (int)threadIdx.x;
+    if (lz0 >= w0) {                                   // the whole workgroup
+        if (RED && (tid & 63) == 0) *my_slot = (T)0;
+        return;
+    }
     if (skip_fast && DR_WAVE_ROWS) {
         const int wv = wave_uniform(tid >> 6);
         const int wy0 = (p.by * DR_TY + (wv * 64) / DR_TX) * DR_RY;
         const int wx0 = (p.bx * DR_TX + (wv * 64) % DR_TX) * 2;
-        if (wy0 < w1 && wx0 < w2 && wave_is_fast(a, p, lz0, wy0, wx0)) return;
+        if (wy0 < w1 && wx0 < w2 && wave_is_fast(a, p, lz0, wy0, wx0)) {   // the whole wavefront
+            if (RED && (tid & 63) == 0) *my_slot = (T)0;
+            return;
+        }
     }
-    const int lx = (p.bx * DR_TX + tid % DR_TX) * 2;
-    const int ly0 = (p.by * DR_TY + tid / DR_TX) * DR_RY;
-    if (lx >= w2 || ly0 >= w1) return;
+    int lx = (p.bx * DR_TX + tid % DR_TX) * 2;
+    int ly0 = (p.by * DR_TY + tid / DR_TX) * DR_RY;
+    // Lanes beyond the tile have nothing to do. A plain sweep lets them go; a reducing one keeps
+    // every lane of the wavefront to the end (the lane exchange of the final sum needs all 64):
+    // such a lane works on the tile's first pair instead, stores nothing and adds nothing.
+    const bool idle = lx >= w2 || ly0 >= w1;
+    if (!RED && idle) return;
+    if (idle) { lx = 0; ly0 = 0; }
 
     // ---- the 27 tile pointers around this tile (uniform); missing neighbours fall back to own ----
     const T* nb[3][3][3];
@@ -602,6 +657,7 @@ __device__ __forceinline__ void direct_rest(const DirectArgs& a, const T* s, int
     }
 
     // ---- evaluate and store ----
+    T acc = (T)0;
 #pragma unroll
     for (int rz = 0; rz < DR_RZ; ++rz) {
         const int lz = lz0 + rz;
@@ -635,12 +691,24 @@ __device__ __forceinline__ void direct_rest(const DirectArgs& a, const T* s, int
                         group_eval(l, s, o);
                         in_e[e] = in_region;
                         res[e] = (DR_MASKED || in_region) ? o[0] : win[rz + DR_H0][ry + DR_H1][DR_HK][e];
+                        if (RED) {
+                            T d = o[0] - win[rz + DR_H0][ry + DR_H1][DR_HK][e];
+                            d = (in_region && !idle) ? d : (T)0;
+                            if (RED == 1) acc = acc + d * d;
+                            else { d = d < (T)0 ? (T)0 - d : d; acc = d > acc ? d : acc; }
+                        }
                     }
-                    P2* out = reinterpret_cast<P2*>(out_tile + (lz * OPZ + ly * OPY + lx));
-                    store_pair<NTS>(out, res, in_e[0], in_e[1]);
+                    if (!RED || !idle) {
+                        P2* out = reinterpret_cast<P2*>(out_tile + (lz * OPZ + ly * OPY + lx));
+                        store_pair<NTS>(out, res, in_e[0], in_e[1]);
+                    }
                 }
             }
         }
+    }
+    if (RED) {
+        acc = wave_combine<RED == 2, T>(acc);
+        if ((tid & 63) == 0) *my_slot = acc;
     }
 }
 
@@ -666,10 +734,13 @@ struct FlatArgs {
     FDiv per_block;        // workgroups per ordering block
     FDiv gb1, gb2;         // ordering blocks along y and x
     FDiv obx, oby;         // = ob[2], ob[1]
+    T* slots;              // reducing launches: one partial per launched wavefront
 };
 
-template <bool NTS>
+// RED as above.
+template <bool NTS, int RED>
 __device__ __forceinline__ void direct_flat(const FlatArgs& a, const T* s) {
+    T* const my_slot = RED ? a.slots + ((size_t)blockIdx.x * 4 + (threadIdx.x >> 6)) : nullptr;
     int blk = (int)blockIdx.x;
     if (a.nblocks8) blk = (blk & 7) * a.nblocks8 + (blk >> 3);
     const int g = fdiv(blk, a.per_block), w = blk - g * (int)a.per_block.d;
@@ -678,13 +749,19 @@ __device__ __forceinline__ void direct_flat(const FlatArgs& a, const T* s) {
     const int wq = fdiv(w, a.obx), wx = w - wq * (int)a.obx.d;
     const int wz = fdiv(wq, a.oby), wy = wq - wz * (int)a.oby.d;
     const int bz = g0 * a.ob[0] + wz, by = g1 * a.ob[1] + wy, bx = g2 * a.ob[2] + wx;
-    if (bz >= a.nb[0] || by >= a.nb[1] || bx >= a.nb[2]) return;   // padding of a ragged block
+    if (bz >= a.nb[0] || by >= a.nb[1] || bx >= a.nb[2]) {          // padding of a ragged block
+        if (RED && (threadIdx.x & 63) == 0) *my_slot = (T)0;
+        return;
+    }
     const int tid = (int)threadIdx.x;
     const int wv = wave_uniform(tid >> 6);
     const int lane = tid & 63;
     const int S0 = a.shape[0], S1 = a.shape[1], S2 = a.shape[2];
     const int z0 = bz * DR_RZ, y0 = (by * 4 + wv) * DR_RY, x0 = bx * 128;
-    if (y0 >= S1) return;                                            // wavefront-uniform
+    if (y0 >= S1) {                                                  // wavefront-uniform
+        if (RED && lane == 0) *my_slot = (T)0;
+        return;
+    }
     const int PY = a.py, PZ = a.pz;
     const int lx = x0 + 2 * lane;
     const bool live = lx < S2;                  // S2 is even: a live lane owns a whole pair
@@ -767,6 +844,7 @@ __device__ __forceinline__ void direct_flat(const FlatArgs& a, const T* s) {
             }
     }
     T* const dst = a.dst;
+    T acc = (T)0;
 #pragma unroll
     for (int rz = 0; rz < DR_RZ; ++rz) {
         const int z = z0 + rz;
@@ -792,6 +870,14 @@ __device__ __forceinline__ void direct_flat(const FlatArgs& a, const T* s) {
                 const int gx = lx + e;
                 in_e[e] = yin && gx >= a.rs[2] && gx < a.re[2];
                 res[e] = (DR_MASKED || in_e[e]) ? o[0] : win[rz + DR_H0][ry + DR_H1][DR_HK][e];
+                if (RED) {
+                    // assigned elements of live lanes only (rows and planes beyond the array are
+                    // never assigned: the region lies inside it)
+                    T d = o[0] - win[rz + DR_H0][ry + DR_H1][DR_HK][e];
+                    d = (in_e[e] && live) ? d : (T)0;
+                    if (RED == 1) acc = acc + d * d;
+                    else { d = d < (T)0 ? (T)0 - d : d; acc = d > acc ? d : acc; }
+                }
             }
             // rows and planes beyond the array (a ragged last workgroup) and idle lanes store nothing
             if (live && z < S0 && y < S1) {
@@ -800,48 +886,76 @@ __device__ __forceinline__ void direct_flat(const FlatArgs& a, const T* s) {
             }
         }
     }
+    if (RED) {
+        acc = wave_combine<RED == 2, T>(acc);
+        if (lane == 0) *my_slot = acc;
+    }
 }
+#if DR_RED
+// The reducing forms only (built on demand under a variant name of their own).
+#define FLAT_RED_ENTRY(NAME, NTS, RED)                                                            \
+extern "C" __global__ __launch_bounds__(256) void NAME(FlatArgs a, Scal sc) {                     \
+    T s[NSA]; load_scalars(sc, s);                                                                \
+    direct_flat<NTS, RED>(a, s);                                                                  \
+}
+FLAT_RED_ENTRY(grp_direct_flat_red1, false, 1)
+FLAT_RED_ENTRY(grp_direct_flat_red1_nts, true, 1)
+FLAT_RED_ENTRY(grp_direct_flat_red2, false, 2)
+FLAT_RED_ENTRY(grp_direct_flat_red2_nts, true, 2)
+// Tiles with buffers of their own: the lean part and the listed face workgroups in one launch.
+#define BOTH_RED_ENTRY(NAME, NTS, RED)                                                            \
+extern "C" __global__ __launch_bounds__(256) void NAME(DirectArgs a, Scal sc, const int* list) {  \
+    T s[NSA]; load_scalars(sc, s);                                                                \
+    if ((int)blockIdx.x < a.nblocks) direct_fast<NTS, RED>(a, s);                                 \
+    else direct_rest<NTS, RED>(a, s, 1, list, a.nblocks);                                         \
+}
+BOTH_RED_ENTRY(grp_direct_both_red1, false, 1)
+BOTH_RED_ENTRY(grp_direct_both_red1_nts, true, 1)
+BOTH_RED_ENTRY(grp_direct_both_red2, false, 2)
+BOTH_RED_ENTRY(grp_direct_both_red2_nts, true, 2)
+#else
 extern "C" __global__ __launch_bounds__(256) void grp_direct_flat(FlatArgs a, Scal sc) {
     T s[NSA]; load_scalars(sc, s);
-    direct_flat<false>(a, s);
+    direct_flat<false, 0>(a, s);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_direct_flat_nts(FlatArgs a, Scal sc) {
     T s[NSA]; load_scalars(sc, s);
-    direct_flat<true>(a, s);
+    direct_flat<true, 0>(a, s);
 }
 
 // nts: the written stream is not read back soon, store it non-temporally.
 extern "C" __global__ __launch_bounds__(256) void grp_direct_fast(DirectArgs a, Scal sc) {
     T s[NSA]; load_scalars(sc, s);
-    direct_fast<false>(a, s);
+    direct_fast<false, 0>(a, s);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_direct_fast_nts(DirectArgs a, Scal sc) {
     T s[NSA]; load_scalars(sc, s);
-    direct_fast<true>(a, s);
+    direct_fast<true, 0>(a, s);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_direct_rest(DirectArgs a, Scal sc, int skip_fast,
                                                                   const int* list) {
     T s[NSA]; load_scalars(sc, s);
-    direct_rest<false>(a, s, skip_fast, list, 0);
+    direct_rest<false, 0>(a, s, skip_fast, list, 0);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_direct_rest_nts(DirectArgs a, Scal sc, int skip_fast,
                                                                       const int* list) {
     T s[NSA]; load_scalars(sc, s);
-    direct_rest<true>(a, s, skip_fast, list, 0);
+    direct_rest<true, 0>(a, s, skip_fast, list, 0);
 }
 // Both in one launch: the first a.nblocks workgroups do the lean part, the ones after them what
 // the lean part leaves (those on `list`, or all positions again when there is no list). One
 // launch and no gap between the two, and the second part fills the tail of the first.
 extern "C" __global__ __launch_bounds__(256) void grp_direct_both(DirectArgs a, Scal sc, const int* list) {
     T s[NSA]; load_scalars(sc, s);
-    if ((int)blockIdx.x < a.nblocks) direct_fast<false>(a, s);
-    else direct_rest<false>(a, s, 1, list, a.nblocks);
+    if ((int)blockIdx.x < a.nblocks) direct_fast<false, 0>(a, s);
+    else direct_rest<false, 0>(a, s, 1, list, a.nblocks);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_direct_both_nts(DirectArgs a, Scal sc, const int* list) {
     T s[NSA]; load_scalars(sc, s);
-    if ((int)blockIdx.x < a.nblocks) direct_fast<true>(a, s);
-    else direct_rest<true>(a, s, 1, list, a.nblocks);
+    if ((int)blockIdx.x < a.nblocks) direct_fast<true, 0>(a, s);
+    else direct_rest<true, 0>(a, s, 1, list, a.nblocks);
 }
+#endif
 )";
     return s.str();
 }

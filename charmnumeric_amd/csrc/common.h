@@ -54,6 +54,12 @@ int reduce_scratch_init(int device);
 // different streams never share slots. Returns a device pointer to `bytes` bytes.
 int reduce_workspace(hipStream_t s, size_t bytes, void** out);
 
+// Folds the per-wavefront partials a reducing stencil launch left behind (sum, or maximum of
+// non-negative values) into *out, in index order, on the same stream.
+// The buffer behind `slots` holds n + kFoldRuns doubles: the fold keeps its run sums behind them.
+constexpr int64_t kFoldRuns = 1024;
+int reduce_slots_f64(bool maximum, double* slots, int64_t n, double* out, hipStream_t st);
+
 // Descriptor tables (per-partition pointers/shapes) live on the device. Identical tables are
 // uploaded once and found again by content hash, so steady-state launches issue no copy.
 int desc_upload(const void* host, size_t bytes, hipStream_t s, const void** dev_out);

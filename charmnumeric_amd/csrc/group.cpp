@@ -396,6 +396,15 @@ int cnh_launch_group_batched(cnh_kernel* k, int ndims, int n_parts, int n_in, co
     std::vector<int64_t> cells(cell_words * live.size(), 0);
     int64_t blocks = 0;
     const int pad = CNH_MAX_ND - ndims;
+    // elements per lane: 4 for large launches, 1 when that still leaves few wavefronts per SIMD
+    int64_t all_elems = 0;
+    for (size_t j = 0; j < live.size(); ++j) {
+        int64_t n = 1;
+        for (int d = 0; d < ndims; ++d)
+            n *= out[(size_t)live[j] * n_out].sizes[d];
+        all_elems += n;
+    }
+    const int per_lane = all_elems <= (1ll << 21) ? 1 : 4;
     for (size_t j = 0; j < live.size(); ++j) {
         int q = live[j];
         const cnh_memref* pi = in + (size_t)q * n_in;
@@ -404,7 +413,7 @@ int cnh_launch_group_batched(cnh_kernel* k, int ndims, int n_parts, int n_in, co
         int64_t sz[3] = {1, 1, 1};
         for (int d = 0; d < ndims; ++d)
             sz[pad + d] = po[0].sizes[d];
-        int64_t nchunks = (sz[2] + 1023) / 1024;
+        int64_t nchunks = (sz[2] + 256 * per_lane - 1) / (256 * per_lane);
         c[0] = sz[0];
         c[1] = sz[1];
         c[2] = sz[2];
@@ -429,12 +438,12 @@ int cnh_launch_group_batched(cnh_kernel* k, int ndims, int n_parts, int n_in, co
     }
     hipFunction_t fn;
     if (live.size() == 1) {
-        if (int rc = get_function(k, "nd", "grp_nd1", &fn))
+        if (int rc = get_function(k, "nd", per_lane == 1 ? "grp_nd1_p1" : "grp_nd1", &fn))
             return rc;
         void* params[] = {cells.data(), scal.data()};
         return launch(fn, blocks, params, st);
     }
-    if (int rc = get_function(k, "nd", "grp_nd", &fn))
+    if (int rc = get_function(k, "nd", per_lane == 1 ? "grp_nd_p1" : "grp_nd", &fn))
         return rc;
     const void* dcells = nullptr;
     if (int rc = desc_upload(cells.data(), cells.size() * 8, st, &dcells))
@@ -673,8 +682,9 @@ struct DirectArgsDev {
     FDivDev per_group, ggrid1, ggrid2, grow, gcol, tbz, tby, tbx;
     const void* oth[kDirectMaxOther];
     int32_t py, pz;
+    void* slots;
 };
-static_assert(sizeof(DirectArgsDev) == 16 + 4 * 22 + 12 * 8 + 8 * kDirectMaxOther + 8,
+static_assert(sizeof(DirectArgsDev) == 16 + 4 * 22 + 12 * 8 + 8 * kDirectMaxOther + 8 + 8,
               "DirectArgsDev layout must match the generated struct");
 
 struct FlatArgsDev {
@@ -683,9 +693,18 @@ struct FlatArgsDev {
     const void* oth[kDirectMaxOther];
     int32_t shape[3], rs[3], re[3], py, pz, nb[3], ob[3], nblocks8;
     FDivDev per_block, gb1, gb2, obx, oby;
+    void* slots;
 };
-static_assert(sizeof(FlatArgsDev) == 16 + 8 * kDirectMaxOther + 4 * 18 + 12 * 5 + 4,
+static_assert(sizeof(FlatArgsDev) == 16 + 8 * kDirectMaxOther + 4 * 18 + 12 * 5 + 4 + 8,
               "FlatArgsDev layout must match the generated struct");
+
+// A launch that should also reduce what it changes: mode 1 = sum of (new - old)^2, 2 = max
+// |new - old|, result to *out (device). `done` is set by the kernel path that took it.
+struct RedReq {
+    int mode = 0;
+    void* out = nullptr;
+    bool done = false;
+};
 
 int g_direct_flat = 1;          // arrays stored as one block take the whole-array kernel
 int g_flat_ob[3] = {0, 0, 0};   // ordering block of that kernel in elements (z, y, x); 0 = default
@@ -702,11 +721,12 @@ DirectConfig g_direct_cfg;
 int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const cnh_tiled*>& arrays,
                   const cnh_tiled* const* others, int n_other, const cnh_tiled* cur,
                   const cnh_tiled* dst, const std::vector<unsigned char>& scal, hipStream_t st,
-                  bool* handled);
+                  bool* handled, RedReq* red);
 
 int try_launch_direct(cnh_kernel* k, const std::vector<const cnh_tiled*>& arrays,
                       const std::vector<int>& leaf_array, const cnh_tiled* cur, const cnh_tiled* dst,
-                      const std::vector<unsigned char>& scal, hipStream_t st, bool* handled) {
+                      const std::vector<unsigned char>& scal, hipStream_t st, bool* handled,
+                      RedReq* red) {
     *handled = false;
     const GroupProgram& p = k->prog;
     DirectShape sh;
@@ -750,15 +770,16 @@ int try_launch_direct(cnh_kernel* k, const std::vector<const cnh_tiled*>& arrays
             if (w->shape[d] != dst->shape[d] || w->grid[d] != dst->grid[d] || w->offset[d] != 0 ||
                 dst->offset[d] != 0 || w->pitch[d] != dst->pitch[d])
                 return 0;
-        return launch_direct(k, sh, own, others, (int)sh.other_names.size(), w, dst, scal, st, handled);
+        return launch_direct(k, sh, own, others, (int)sh.other_names.size(), w, dst, scal, st, handled,
+                             nullptr);   // the target's old values are not read: nothing to reduce here
     }
-    return launch_direct(k, sh, own, others, (int)sh.other_names.size(), cur, dst, scal, st, handled);
+    return launch_direct(k, sh, own, others, (int)sh.other_names.size(), cur, dst, scal, st, handled, red);
 }
 
 int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const cnh_tiled*>& arrays,
                   const cnh_tiled* const* others, int n_other, const cnh_tiled* cur,
                   const cnh_tiled* dst, const std::vector<unsigned char>& scal, hipStream_t st,
-                  bool* handled) {
+                  bool* handled, RedReq* red) {
     const GroupProgram& p = k->prog;
     // a lane's own rows and planes must not straddle tiles: the tile edge (a power of two) has
     // to be a multiple of what one lane owns
@@ -891,12 +912,31 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
             f.oby = fdiv_make((uint32_t)f.ob[1]);
             const bool nts = volume * 2 * esz >= (128ll << 20);
             hipFunction_t fn;
-            if (int rc = get_function(k, g_direct_cfg.variant(),
-                                      nts ? "grp_direct_flat_nts" : "grp_direct_flat", &fn))
+            const bool reducing = red != nullptr && red->mode != 0 && p.dtype == CNH_F64;
+            if (reducing) {
+                // one partial per launched wavefront, folded in index order by a second launch
+                void* slots = nullptr;
+                if (int rc = reduce_workspace(st, (size_t)(launched * 4 + kFoldRuns) * sizeof(double), &slots))
+                    return rc;
+                f.slots = slots;
+                DirectConfig rcfg = g_direct_cfg;
+                rcfg.reduce = true;
+                const char* name = red->mode == 1 ? (nts ? "grp_direct_flat_red1_nts" : "grp_direct_flat_red1")
+                                                  : (nts ? "grp_direct_flat_red2_nts" : "grp_direct_flat_red2");
+                if (int rc = get_function(k, rcfg.variant(), name, &fn))
+                    return rc;
+            } else if (int rc = get_function(k, g_direct_cfg.variant(),
+                                             nts ? "grp_direct_flat_nts" : "grp_direct_flat", &fn))
                 return rc;
             void* params[] = {&f, const_cast<unsigned char*>(scal.data())};
             if (int rc = launch(fn, launched, params, st))
                 return rc;
+            if (reducing) {
+                if (int rc = reduce_slots_f64(red->mode == 2, static_cast<double*>(f.slots),
+                                              launched * 4, static_cast<double*>(red->out), st))
+                    return rc;
+                red->done = true;
+            }
             *handled = true;
             return 0;
         }
@@ -1031,12 +1071,32 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
     }
     if (lean && g_direct_merge) {
         // lean part and the rest in one launch
-        if (int rc = get_function(k, g_direct_cfg.variant(),
-                                  nt_stores ? "grp_direct_both_nts" : "grp_direct_both", &fn))
+        const bool reducing = red != nullptr && red->mode != 0 && p.dtype == CNH_F64 && !sh.masked;
+        const int64_t launched = blocks + rest_blocks;
+        if (reducing) {
+            // one partial per launched wavefront, folded in index order by a second launch
+            void* slots = nullptr;
+            if (int rc = reduce_workspace(st, (size_t)(launched * 4 + kFoldRuns) * sizeof(double), &slots))
+                return rc;
+            a.slots = slots;
+            DirectConfig rcfg = g_direct_cfg;
+            rcfg.reduce = true;
+            const char* name = red->mode == 1 ? (nt_stores ? "grp_direct_both_red1_nts" : "grp_direct_both_red1")
+                                              : (nt_stores ? "grp_direct_both_red2_nts" : "grp_direct_both_red2");
+            if (int rc = get_function(k, rcfg.variant(), name, &fn))
+                return rc;
+        } else if (int rc = get_function(k, g_direct_cfg.variant(),
+                                         nt_stores ? "grp_direct_both_nts" : "grp_direct_both", &fn))
             return rc;
         void* params[] = {&a, const_cast<unsigned char*>(scal.data()), &dlist};
-        if (int rc = launch(fn, blocks + rest_blocks, params, st))
+        if (int rc = launch(fn, launched, params, st))
             return rc;
+        if (reducing) {
+            if (int rc = reduce_slots_f64(red->mode == 2, static_cast<double*>(a.slots), launched * 4,
+                                          static_cast<double*>(red->out), st))
+                return rc;
+            red->done = true;
+        }
         *handled = true;
         return 0;
     }
@@ -1135,9 +1195,79 @@ extern "C" int cnh_set_option(const char* name, int value) {
     return set_error(-2, "unknown option '%s'", name);
 }
 
+namespace {
+int launch_group_tiles_impl(cnh_kernel* k, int n_in, const cnh_tiled* in, int n_scalar,
+                            const void* const* scalars, int scalars_on_device, const cnh_tiled* cur,
+                            const cnh_tiled* dst, cnh_stream s, RedReq* red);
+}
+
 extern "C" int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* in, int n_scalar,
                                       const void* const* scalars, int scalars_on_device,
                                       const cnh_tiled* cur, const cnh_tiled* dst, cnh_stream s) {
+    return launch_group_tiles_impl(k, n_in, in, n_scalar, scalars, scalars_on_device, cur, dst, s, nullptr);
+}
+
+extern "C" int cnh_launch_group_tiles_residual(cnh_kernel* k, int n_in, const cnh_tiled* in, int n_scalar,
+                                               const void* const* scalars, int scalars_on_device,
+                                               const cnh_tiled* cur, const cnh_tiled* dst, int mode,
+                                               void* out, cnh_stream s) {
+    CNH_CHECK(mode == 0 || mode == 1, -2, "residual mode %d is neither 0 (sum of squares) nor 1 (maximum)",
+              mode);
+    CNH_CHECK(out != nullptr && cur != nullptr && dst != nullptr, -2, "null argument");
+    CNH_CHECK(k != nullptr && k->prog.dtype == CNH_F64, -2, "the residual forms need an fp64 group");
+    CNH_CHECK(cur->tiles != nullptr && dst->tiles != nullptr && cur->tiles[0] != dst->tiles[0], -4,
+              "a residual needs the old contents: cur and dst must be different buffers");
+    RedReq red;
+    red.mode = mode + 1;
+    red.out = out;
+    if (int rc = launch_group_tiles_impl(k, n_in, in, n_scalar, scalars, scalars_on_device, cur, dst, s, &red))
+        return rc;
+    if (red.done)
+        return 0;
+    // Not taken by a kernel that reduces on the way: a second pass over both buffers. Contiguous
+    // tiles are one chunk each; views into one block without gaps are one chunk together.
+    const int nd = dst->ndims;
+    int64_t ntiles = 1, total = 1;
+    for (int d = 0; d < nd; ++d) {
+        ntiles *= dst->grid[d];
+        total *= dst->shape[d];
+    }
+    std::vector<const void*> pa, pb;
+    std::vector<int64_t> cnt;
+    if (is_pitched(dst)) {
+        bool gapless = dst->pitch[nd - 1] == 1;
+        for (int d = nd - 2; d >= 0 && gapless; --d)
+            gapless = dst->pitch[d] == dst->pitch[d + 1] * dst->shape[d + 1];
+        for (int d = 0; d < nd && gapless; ++d)
+            gapless = dst->offset[d] == 0;
+        CNH_CHECK(gapless, -4, "residual over pitched views with gaps between rows or planes");
+        pa.push_back(dst->tiles[0]);
+        pb.push_back(cur->tiles[0]);
+        cnt.push_back(total);
+    } else {
+        for (int64_t t = 0; t < ntiles; ++t) {
+            int64_t rem = t, n = 1;
+            for (int d = nd - 1; d >= 0; --d) {
+                const int g = dst->grid_lo[d] + (int)(rem % dst->grid[d]);
+                rem /= dst->grid[d];
+                const int lo = std::max(g * dst->tile, dst->offset[d]);
+                const int hi = std::min((g + 1) * dst->tile, dst->offset[d] + dst->shape[d]);
+                n *= std::max(0, hi - lo);
+            }
+            pa.push_back(dst->tiles[t]);
+            pb.push_back(cur->tiles[t]);
+            cnt.push_back(n);
+        }
+    }
+    if (mode == 0)
+        return cnh_sumsq_diff_tiles((int)pa.size(), pa.data(), pb.data(), cnt.data(), out, s);
+    return cnh_maxabs_diff_tiles((int)pa.size(), pa.data(), pb.data(), cnt.data(), out, s);
+}
+
+namespace {
+int launch_group_tiles_impl(cnh_kernel* k, int n_in, const cnh_tiled* in, int n_scalar,
+                            const void* const* scalars, int scalars_on_device, const cnh_tiled* cur,
+                            const cnh_tiled* dst, cnh_stream s, RedReq* red) {
     if (int rc = ensure_init())
         return rc;
     CNH_CHECK(k != nullptr, -2, "null kernel");
@@ -1234,7 +1364,7 @@ extern "C" int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* 
     // Same-array unit-step stencil with ping-pong buffers: register-window or LDS sliding window.
     {
         bool handled = false;
-        if (int rc = try_launch_direct(k, arrays, leaf_array, cur, dst, scal, st, &handled))
+        if (int rc = try_launch_direct(k, arrays, leaf_array, cur, dst, scal, st, &handled, red))
             return rc;
         if (handled)
             return 0;
@@ -1351,3 +1481,4 @@ extern "C" int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* 
     void* params[] = {&d_arrs, &d_dts, &ndt, targs.data(), scal.data()};
     return launch(fn, blocks, params, st);
 }
+} // namespace

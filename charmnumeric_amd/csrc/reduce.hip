@@ -375,7 +375,68 @@ int run_dot_noalloc(int64_t n, const void* a, const void* b, void* out, void* sl
 
 } // namespace
 
+namespace {
+// Folding the partials a kernel that reduced on the way left behind (one per wavefront, in launch
+// order; sums, or maxima of non-negative values). Few of them: one workgroup, lane t takes slots
+// t, t + 1024, ... in that order, then the fixed tree. Many: first every workgroup of a grid folds
+// its own run of `per` consecutive slots the same way into one value, then one workgroup folds
+// those. The grouping depends on n only.
+template <bool MAXV>
+__global__ __launch_bounds__(1024) void fold_slots(const double* __restrict__ slots, int64_t n,
+                                                   double* __restrict__ out) {
+    __shared__ double lds[1024 / 64];
+    double v = 0.0;
+    for (int64_t i = threadIdx.x; i < n; i += 1024) {
+        const double o = slots[i];
+        v = MAXV ? (o > v ? o : v) : v + o;
+    }
+    v = block_reduce<double, MAXV ? M_MAXABS_DIFF : M_SUM, 1024>(v, lds);
+    if (threadIdx.x == 0)
+        *out = v;
+}
+template <bool MAXV>
+__global__ __launch_bounds__(kThreads) void fold_slots_runs(const double* __restrict__ slots, int64_t n,
+                                                            int64_t per, double* __restrict__ runs) {
+    __shared__ double lds[kThreads / 64];
+    const int64_t lo = (int64_t)blockIdx.x * per, hi = lo + per < n ? lo + per : n;
+    double v = 0.0;
+    for (int64_t i = lo + threadIdx.x; i < hi; i += kThreads) {
+        const double o = slots[i];
+        v = MAXV ? (o > v ? o : v) : v + o;
+    }
+    v = block_reduce<double, MAXV ? M_MAXABS_DIFF : M_SUM, kThreads>(v, lds);
+    if (threadIdx.x == 0)
+        runs[blockIdx.x] = v;
+}
+} // namespace
+
 namespace cnh {
+// `slots` must have room for kFoldRuns more doubles behind its n entries (the run sums).
+int reduce_slots_f64(bool maximum, double* slots, int64_t n, double* out, hipStream_t st) {
+    CNH_CHECK(slots != nullptr && out != nullptr && n >= 1, -2, "reduce_slots_f64: bad arguments");
+    const double* src = slots;
+    int64_t count = n;
+    if (n > 8192) {
+        int64_t per = (n + kFoldRuns - 1) / kFoldRuns;
+        per = (per + 1023) / 1024 * 1024;               // whole passes of a workgroup
+        const int64_t runs = (n + per - 1) / per;
+        double* tmp = slots + n;
+        if (maximum)
+            hipLaunchKernelGGL(fold_slots_runs<true>, dim3((unsigned)runs), dim3(kThreads), 0, st, slots, n, per, tmp);
+        else
+            hipLaunchKernelGGL(fold_slots_runs<false>, dim3((unsigned)runs), dim3(kThreads), 0, st, slots, n, per, tmp);
+        CNH_HIP(hipGetLastError());
+        src = tmp;
+        count = runs;
+    }
+    if (maximum)
+        hipLaunchKernelGGL(fold_slots<true>, dim3(1), dim3(1024), 0, st, src, count, out);
+    else
+        hipLaunchKernelGGL(fold_slots<false>, dim3(1), dim3(1024), 0, st, src, count, out);
+    CNH_HIP(hipGetLastError());
+    return 0;
+}
+
 // Called by cnh_init with `device` current: resolves this device's copy of the scratch array.
 int reduce_scratch_init(int device) {
     CNH_CHECK(device >= 0 && device < kMaxDevices, -2, "device %d beyond the %d the scratch table holds",

@@ -221,6 +221,19 @@ int cnh_launch_group_tiles(cnh_kernel* k, int n_in, const cnh_tiled* in, int n_s
                            const void* const* scalars, int scalars_on_device,
                            const cnh_tiled* cur, const cnh_tiled* dst, cnh_stream s);
 
+/* The same launch, which also reduces what it changes (no upstream counterpart: upstream has no
+ * reduction over 2-D or 3-D arrays, src/executor_reduce.cpp:9-12, and its examples fetch the array
+ * and use NumPy, examples/multigrid2d.py:659-666). *out (device, fp64) = sum over all elements of
+ * (new - old)^2 for mode 0, max |new - old| for mode 1; fp64 groups with cur != dst (the old
+ * contents must survive the launch). The whole-array register-window kernel accumulates per
+ * wavefront while it sweeps and a second small launch adds the partials in index order, so the
+ * residual costs no second pass over the data; every other kernel path is followed by
+ * cnh_sumsq_diff_tiles / cnh_maxabs_diff_tiles over (dst, cur). Results never depend on scheduling. */
+int cnh_launch_group_tiles_residual(cnh_kernel* k, int n_in, const cnh_tiled* in, int n_scalar,
+                                    const void* const* scalars, int scalars_on_device,
+                                    const cnh_tiled* cur, const cnh_tiled* dst, int mode, void* out,
+                                    cnh_stream s);
+
 /* ---- REDUCE: eigen_dot + contribute + reduce_dot_sum + reduce_result
  *      (src/backend_internal.hpp:88-93, src/executor_reduce.cpp:8-119,
  *       src/executor_reducer.cpp:11-57, src/partition_comm.cpp:69-111) ---- */

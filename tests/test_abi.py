@@ -50,11 +50,11 @@ def test_scalar_conversion():
     assert buf.view(np.float32)[0] == np.float32(0.1)
 
 
-@pytest.mark.parametrize("variant", ["flat", "nd", "tiles", "slide", "direct"])
+@pytest.mark.parametrize("variant", ["flat", "nd", "tiles", "slide", "direct", "directr"])
 def test_generated_source_builds_for_gfx950(variant):
     """hipRTC cross-compiles the generated source without a GPU."""
-    ast = H.ast_jacobi2d(64) if variant in ("tiles", "slide", "direct") else H.ast_c1(L.F64)
-    nd = 2 if variant in ("tiles", "slide", "direct") else 1
+    ast = H.ast_jacobi2d(64) if variant in ("tiles", "slide", "direct", "directr") else H.ast_c1(L.F64)
+    nd = 2 if variant in ("tiles", "slide", "direct", "directr") else 1
     k = H.compile_group(ast, L.F64, nd)
     src = H.kernel_source(k, variant)
     assert "group_eval" in src and "fma" not in src

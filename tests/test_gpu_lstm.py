@@ -60,9 +60,10 @@ def test_lstm_forward_full_shape_four_steps(dev):
     assert np.all(np.abs(got["Hout"]) <= 1.0)
 
 
+@pytest.mark.parametrize("fused", [True, False], ids=["one-gate-launch", "six-gate-launches"])
 @pytest.mark.parametrize("steps,batch,nin,d", [(3, 8, 16, 16), (4, 64, 64, 32), (2, 70, 24, 40)])
-def test_lstm_forward_small(dev, steps, batch, nin, d):
-    got = bench.run_lstm(L, steps=steps, batch=batch, nin=nin, d=d, timed=False, keep=True)
+def test_lstm_forward_small(dev, steps, batch, nin, d, fused):
+    got = bench.run_lstm(L, steps=steps, batch=batch, nin=nin, d=d, timed=False, keep=True, fused=fused)
     Hout, Cc, IFOG, _ = _reference(steps, batch, nin, d)
     # gate pre-activations: 1e-12 relative to sum |a||b| (here <= (nin + d) / 32)
     assert np.max(np.abs(got["IFOG"] - IFOG)) <= 1e-12 * (nin + d) / 32

@@ -410,3 +410,77 @@ def test_tiles_rejects_bad_descriptors(dev):
     with pytest.raises(L.CnhError):
         H.launch_tiles(k, [a] * 3, [], a, a)          # wrong number of inputs
     dev.free_all()
+
+
+# ---- sweeps that also reduce what they change ----
+
+def _residual_cases():
+    # (shape, tile, one block?) — ragged tiles, tiles narrower and wider than a wavefront's 128 columns
+    return [((70, 70), 32, False), ((256, 512), 128, False), ((36, 36, 36), 16, False),
+            ((24, 40, 256), 128, False), ((50, 300), 64, True), ((33, 40, 258), 32, True),
+            ((9, 17, 130), 8, True), ((128, 128, 128), 128, True)]
+
+
+@pytest.mark.parametrize("mode", [0, 1], ids=["sumsq", "maxabs"])
+@pytest.mark.parametrize("shape,tile,block", _residual_cases())
+def test_sweep_with_residual_matches_the_separate_pass(dev, shape, tile, block, mode):
+    """cnh_launch_group_tiles_residual: the new contents bit for bit, the maximum of |new - old|
+    exactly and the sum of (new - old)^2 within 1e-12 of what the separate reduction kernels give
+    over the same two buffers; the same bits on a second run."""
+    import ctypes as C
+    nd = len(shape)
+    rng = np.random.default_rng(sum(shape) + tile)
+    u0 = rng.standard_normal(shape)
+    k = H.compile_group(_ast_star(shape), L.F64, nd)
+    if block:
+        ba, _pa, da = _pitched_views(dev, u0, tile)
+        bb, _pb, db = _pitched_views(dev, np.zeros_like(u0), tile)
+        new = lambda: bb.view()
+        chunks = ([bb.ptr], [ba.ptr], [int(np.prod(shape))])
+    else:
+        ta, tb = H.TiledArray(dev, u0, tile), H.TiledArray(dev, np.zeros_like(u0), tile)
+        da, db = ta.desc(), tb.desc()
+        new = lambda: tb.gather()
+        chunks = ([b.ptr for b in tb.bufs], [b.ptr for b in ta.bufs], [int(np.prod(b.shape)) for b in ta.bufs])
+    out = dev.array(np.full(3, -1.0))
+    descs = (L.Tiled * (2 * nd))(*([da] * (2 * nd)))
+    for slot in (0, 1):
+        L.check(L.lib.cnh_launch_group_tiles_residual(k, 2 * nd, descs, 0, None, 0, C.byref(da), C.byref(db),
+                                                      mode, out.ptr + 8 * slot, None))
+    fn = L.lib.cnh_sumsq_diff_tiles if mode == 0 else L.lib.cnh_maxabs_diff_tiles
+    L.check(fn(len(chunks[2]), L.vparr(chunks[0]), L.vparr(chunks[1]), L.i64arr(chunks[2]), out.ptr + 16, None))
+    dev.sync()
+    mid, val = _np_star(u0, 0.125)
+    want = u0.copy()
+    want[mid] = val
+    assert np.array_equal(new(), want)
+    got = out.get()
+    assert got.view(np.int64)[0] == got.view(np.int64)[1]            # run to run
+    d = want - u0
+    if mode == 1:
+        assert got[0] == got[2] == np.max(np.abs(d))
+    else:
+        ref = float(np.sum(d.astype(np.longdouble) ** 2))
+        assert abs(got[0] - ref) <= 1e-12 * ref and abs(got[0] - got[2]) <= 1e-12 * ref
+    dev.free_all()
+
+
+def test_residual_refuses_what_it_cannot_do(dev):
+    import ctypes as C
+    shape, tile = (64, 64), 32
+    k = H.compile_group(_ast_star(shape), L.F64, 2)
+    ta = H.TiledArray(dev, np.zeros(shape), tile)
+    da = ta.desc()
+    out = dev.array(np.zeros(1))
+    descs = (L.Tiled * 4)(*([da] * 4))
+    # in place: the old contents would be gone
+    assert L.lib.cnh_launch_group_tiles_residual(k, 4, descs, 0, None, 0, C.byref(da), C.byref(da), 0,
+                                                 out.ptr, None) == -4
+    tb = H.TiledArray(dev, np.zeros(shape), tile)
+    db = tb.desc()
+    assert L.lib.cnh_launch_group_tiles_residual(k, 4, descs, 0, None, 0, C.byref(da), C.byref(db), 2,
+                                                 out.ptr, None) == -2
+    k32 = H.compile_group(_ast_star(shape, dtype=L.F32), L.F32, 2)
+    assert L.lib.cnh_launch_group_tiles_residual(k32, 4, descs, 0, None, 0, C.byref(da), C.byref(db), 0,
+                                                 out.ptr, None) == -2
+    dev.free_all()
