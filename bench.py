@@ -526,6 +526,16 @@ def run_jacobi(L, nd, n, tile, sweeps, reduce_every=10, reps_note=""):
     L.check(L.lib.cnh_event_elapsed_ms(e0, e1, C.byref(ms)))
     t = ev.times_ms(sweeps)
     last_fused = float(res.get(np.float64)[0])
+    # the same residual by a second pass over both buffers (what every tenth sweep cost before the
+    # sweep accumulated it on the way), for comparison and as a check
+    evr = Events(L, 5)
+    for i in range(5):
+        L.check(L.lib.cnh_event_record(evr.a[i], None))
+        residual(nxt, cur)              # cur holds the newest contents, nxt the ones before
+        L.check(L.lib.cnh_event_record(evr.b[i], None))
+    L.check(L.lib.cnh_device_sync())
+    tr = evr.times_ms(5)
+    last_separate = float(res.get(np.float64)[0])
     # The whole run again between two events only (an event pair around every sweep costs a few
     # microseconds per sweep itself): once with the residual every reduce_every sweeps, once without.
     totals = {}
@@ -543,16 +553,6 @@ def run_jacobi(L, nd, n, tile, sweeps, reduce_every=10, reps_note=""):
         L.check(L.lib.cnh_device_sync())
         L.check(L.lib.cnh_event_elapsed_ms(e0, e1, C.byref(ms)))
         totals[label] = ms.value
-    # the same residual by a second pass over both buffers (what every tenth sweep cost before the
-    # sweep accumulated it on the way), for comparison and as a check
-    evr = Events(L, 5)
-    for i in range(5):
-        L.check(L.lib.cnh_event_record(evr.a[i], None))
-        residual(nxt, cur)              # cur holds the newest contents, nxt the ones before
-        L.check(L.lib.cnh_event_record(evr.b[i], None))
-    L.check(L.lib.cnh_device_sync())
-    tr = evr.times_ms(5)
-    last_separate = float(res.get(np.float64)[0])
     plain = [t[i] for i in range(sweeps) if i not in reducing]
     us = 1e3 * float(np.median(plain))
     us_red = 1e3 * float(np.median([t[i] for i in reducing])) if reducing else None

@@ -269,6 +269,7 @@ _PROTOS.update({
     "cnx_set_trace": (C.c_int, [C.c_void_p, C.c_int]),
     "cnx_set_solver": (C.c_int, [C.c_void_p, C.c_int]),
     "cnx_set_layout": (C.c_int, [C.c_void_p, C.c_int]),
+    "cnx_set_fusion": (C.c_int, [C.c_void_p, C.c_int]),
     "cnx_trace": (C.c_int64, [C.c_void_p, C.c_char_p, C.c_size_t]),
 })
 

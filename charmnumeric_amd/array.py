@@ -40,6 +40,9 @@ class DType:
         return DType.from_numpy(np.result_type(DType.to_numpy(a), DType.to_numpy(b)))
 
 
+_PLAIN_NUMBERS = (int, float)
+
+
 class _CallableInt(int):
     """`a.size` that may also be called as `a.size()` (both spellings occur upstream)."""
 
@@ -68,12 +71,16 @@ def _normalize_shape(shape):
 
 
 def _is_scalar_like(v):
+    if type(v) in _PLAIN_NUMBERS:          # the common case, without the abstract-class checks
+        return True
     if isinstance(v, np.ndarray):
         return v.ndim == 0
     return isinstance(v, (bool, numbers.Real, np.generic))
 
 
 def _coerce_scalar(v):
+    if type(v) in _PLAIN_NUMBERS:
+        return v
     if isinstance(v, (np.ndarray, np.generic)):
         v = v.item()
     if isinstance(v, bool):
@@ -155,7 +162,18 @@ def parse_key(key, shape):
 
 def region_shape(region):
     start, stop, step = region
+    if step in _UNIT:
+        if len(start) == 3:
+            return (max(0, stop[0] - start[0]), max(0, stop[1] - start[1]), max(0, stop[2] - start[2]))
+        return tuple(max(0, stop[d] - start[d]) for d in range(len(start)))
     return tuple(max(0, (stop[d] - start[d] + step[d] - 1) // step[d]) for d in range(len(start)))
+
+
+_UNIT = {(1,), (1, 1), (1, 1, 1)}
+
+
+def _unit_steps(step):
+    return step in _UNIT
 
 
 def compose(outer, inner):
@@ -166,6 +184,15 @@ def compose(outer, inner):
     (charmnumeric.py:215-220 upstream), with the same effect."""
     if outer is None:
         return inner
+    if inner[2] == outer[2] and _unit_steps(inner[2]):
+        # unit steps on both sides: plain offsets
+        ostart = outer[0]
+        n = len(ostart)
+        if n == 3:
+            return ((ostart[0] + inner[0][0], ostart[1] + inner[0][1], ostart[2] + inner[0][2]),
+                    (ostart[0] + inner[1][0], ostart[1] + inner[1][1], ostart[2] + inner[1][2]), inner[2])
+        return (tuple(ostart[d] + inner[0][d] for d in range(n)),
+                tuple(ostart[d] + inner[1][d] for d in range(n)), inner[2])
     ostart, _, ostep = outer
     istart, istop, istep = inner
     nd = len(istart)
@@ -254,11 +281,14 @@ class _ArrayLike:
         region = compose(self._region(), inner)
         shape = region_shape(inner)
         base = self._base()
-        value = _coerce_assignment_operand(rhs, shape, self.dtype)
+        if isinstance(rhs, _ArrayLike):
+            value = rhs
+        else:
+            value = _coerce_assignment_operand(rhs, shape, self.dtype)
         if isinstance(value, _ArrayLike):
-            if value.dtype != self.dtype:
+            if value._wire != base._wire:
                 raise NotImplementedError("assignment across dtypes is not implemented")
-            if tuple(value.shape) != tuple(shape):
+            if value.shape != shape:
                 # a lower-rank value fits a region whose extra dimensions have extent 1
                 # (IFOG[t] = M with M 2-D), and a whole higher-rank one whose extra dimensions
                 # have extent 1 fits a lower-rank target (vec[:] = column)
@@ -270,9 +300,8 @@ class _ArrayLike:
             operand = value._ref()
         else:
             operand = value
-        whole = lazy.ArrayRef(base.name, None, base.shape, base.ndims, base.wire_dtype())
-        lazy.record(lazy.Instr("set", name=base.name, operands=[operand], shape=shape,
-                               dtype=base.wire_dtype(), region=region, payload=whole))
+        whole = lazy.ArrayRef(base.name, None, base.shape, base.ndims, base._wire)
+        lazy.record(lazy.Instr("set", base.name, None, [operand], shape, base._wire, region, whole))
 
     # -- arithmetic --
     def __add__(self, o):
@@ -342,6 +371,20 @@ class Array(_ArrayLike):
         self.name = lazy.new_name() if name is None else name
         self._gen = lazy.generation()
 
+    @classmethod
+    def _result_of(cls, like, shape):
+        """A new array of `shape` with the element type of the array-like `like` (shape already a
+        tuple of ints): the result of an operation, without re-deriving what the operand knows."""
+        out = cls.__new__(cls)
+        out.shape = shape
+        out.ndims = len(shape)
+        out.dtype = like.dtype
+        out._wire = like._wire
+        out._n = like._n if shape is like.shape else _size(shape)
+        out.name = lazy.new_name()
+        out._gen = lazy.generation()
+        return out
+
     def __del__(self):
         lazy.record_delete(self.name, self._gen)
 
@@ -369,12 +412,15 @@ class ArrayView(_ArrayLike):
     def __init__(self, base, region):
         self.base = base
         self.region = region
-        self.shape = region_shape(region)
+        self.shape = shape = region_shape(region)
         self.ndims = base.ndims
         self.dtype = base.dtype
         self._wire = base._wire
-        self._n = _size(self.shape)
-        if any(s == 0 for s in self.shape):
+        n = 1
+        for extent in shape:
+            n *= extent
+        self._n = n
+        if n == 0:
             raise NotImplementedError("zero-sized slices are not supported")
 
     @property
@@ -391,9 +437,9 @@ class ArrayView(_ArrayLike):
         return self.region
 
     def _ref(self, broadcast=False):
-        region = None if _is_whole(self.region, self.base.shape) else self.region
-        return lazy.ArrayRef(self.base.name, region, self.shape, self.base.ndims, self.wire_dtype(),
-                             broadcast)
+        base = self.base
+        region = None if self._n == base._n and _is_whole(self.region, base.shape) else self.region
+        return lazy.ArrayRef(base.name, region, self.shape, base.ndims, self._wire, broadcast)
 
     def get(self, interface):
         out = empty(self.shape, dtype=self.dtype)
@@ -417,41 +463,52 @@ def _as_operand(v):
 
 
 def _binary(opcode, lhs, rhs):
-    lhs, rhs = _as_operand(lhs), _as_operand(rhs)
-    arrays = [x for x in (lhs, rhs) if isinstance(x, _ArrayLike)]
-    dtype = arrays[0].dtype
-    for a in arrays[1:]:
-        if a.dtype != dtype:
-            raise NotImplementedError(
-                f"elementwise operations across dtypes ({dtype} and {a.dtype}) are not implemented")
-    big = [a.shape for a in arrays if a._n > 1]
-    shape = tuple(big[0]) if big else tuple(arrays[0].shape)
-    for other in big[1:]:
-        if tuple(other) != shape:
-            raise ValueError(f"operands could not be broadcast together with shapes "
-                             f"{arrays[0].shape} and {arrays[1].shape}")
-    operands = []
-    for x in (lhs, rhs):
-        if isinstance(x, _ArrayLike):
-            bc = x._n == 1 and bool(big)
+    la, ra = isinstance(lhs, _ArrayLike), isinstance(rhs, _ArrayLike)
+    if not la:
+        lhs = _as_operand(lhs)
+        la = isinstance(lhs, _ArrayLike)
+    if not ra:
+        rhs = _as_operand(rhs)
+        ra = isinstance(rhs, _ArrayLike)
+    if la and ra:
+        if lhs.dtype != rhs.dtype:
+            raise NotImplementedError(f"elementwise operations across dtypes ({lhs.dtype} and "
+                                      f"{rhs.dtype}) are not implemented")
+        # the result takes the shape of the operand with more than one element; a one-element
+        # whole array beside it is a run-time scalar
+        if lhs._n > 1 and rhs._n > 1:
+            if lhs.shape != rhs.shape:
+                raise ValueError(f"operands could not be broadcast together with shapes "
+                                 f"{lhs.shape} and {rhs.shape}")
+            like, lb, rb = lhs, False, False
+        elif lhs._n > 1:
+            like, lb, rb = lhs, False, True
+        elif rhs._n > 1:
+            like, lb, rb = rhs, True, False
+        else:
+            like, lb, rb = lhs, False, False
+        for x, bc in ((lhs, lb), (rhs, rb)):
             if bc and not _is_whole(x._region(), x._base().shape):
                 raise NotImplementedError("a one-element slice cannot be used as a scalar operand")
-            operands.append(x._ref(broadcast=bc))
-        else:
-            operands.append(x)
-    out = Array(shape, dtype)
-    lazy.record(lazy.Instr("op", name=out.name, opcode=opcode, operands=operands, shape=shape,
-                           dtype=out.wire_dtype()))
+        operands = [lhs._ref(lb), rhs._ref(rb)]
+    elif la:
+        like = lhs
+        operands = [lhs._ref(), rhs]
+    else:
+        like = rhs
+        operands = [lhs, rhs._ref()]
+    out = Array._result_of(like, like.shape)
+    lazy.record(lazy.Instr("op", out.name, opcode, operands, out.shape, out._wire))
     return out
 
 
 def unary(opcode, x):
-    x = asarray(x)
-    if x.dtype.kind != "f":
+    if not isinstance(x, _ArrayLike):
+        x = asarray(x)
+    if x._wire > L.F64:                    # the two integer types follow the floating-point ones
         raise TypeError("tanh/exp need a floating-point array")
-    out = Array(x.shape, x.dtype)
-    lazy.record(lazy.Instr("op", name=out.name, opcode=opcode, operands=[x._ref()], shape=x.shape,
-                           dtype=out.wire_dtype()))
+    out = Array._result_of(x, x.shape)
+    lazy.record(lazy.Instr("op", out.name, opcode, [x._ref()], out.shape, out._wire))
     return out
 
 

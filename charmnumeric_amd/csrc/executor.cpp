@@ -12,6 +12,7 @@
 #include <cstring>
 #include <deque>
 #include <map>
+#include <set>
 #include <memory>
 #include <mutex>
 #include <sstream>
@@ -144,6 +145,13 @@ struct cnx_executor {
     int num_pes = 1, odf = 4;
     int min_tile[4] = {0, 262144, 512, 64}; // CT_MIN_TILE_1D/2D/3D, src/backend.hpp:10-18
     bool flat3 = true;  // new rank-3 arrays are one row-major block with tiles as views into it
+    bool fuse_on = true; // runs of assignments of one extent go out as one launch
+    // A run of mergeable assignments that reaches the end of a message waits here for the next
+    // message (where it may go on) or for the next call that needs the executor's state: what gets
+    // merged then depends on the statements alone, not on where the frontend happened to cut its
+    // messages, and a time loop keeps meeting the same few merged kernels.
+    std::vector<DagNode> held;
+    bool final_pass = false;   // running held nodes to the end: nothing may be held again
     cnh_stream stream = nullptr;
     std::map<int, XArray> arrays;
     // compile_cache (src/dag_group_compile.cpp:43-56), bounded: a time loop over slabs makes a new
@@ -1045,6 +1053,124 @@ int exec_reduce_ext(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
     return rc;
 }
 
+// ---- boxes: unit-step regions that are one strided block of device memory ----
+struct BoxUse {
+    XArray* arr = nullptr;
+    cnh_region reg;        // explicit, unit steps, in the array's own rank
+    int map[3] = {-1, -1, -1};   // statement dimension -> array dimension (or -1: extent 1, no such dim)
+};
+struct Stmt {
+    const DagNode* n = nullptr;
+    int nd = 0, dtype = CNH_F64;
+    int32_t cnt[3] = {1, 1, 1};
+    BoxUse out;
+    struct Read { int root, slot; BoxUse use; };
+    std::vector<Read> reads;
+};
+
+constexpr int64_t kFuseMaxElems = 1ll << 22;   // larger statements are bandwidth bound anyway
+constexpr size_t kFuseMaxStmts = 8, kFuseMaxReads = 16;
+
+bool boxes_identical(const BoxUse& a, const BoxUse& b) {
+    return a.arr == b.arr && same_region(a.reg, b.reg);
+}
+bool boxes_disjoint(const BoxUse& a, const BoxUse& b) {
+    if (a.arr != b.arr)
+        return true;
+    for (int d = 0; d < a.arr->ndims; ++d)
+        if (a.reg.stop[d] <= b.reg.start[d] || b.reg.stop[d] <= a.reg.start[d])
+            return true;
+    return false;
+}
+
+// One strided block of device memory?
+bool box_is_one_block(const XArray& a, const cnh_region& r) {
+    if (a.flat || a.ntiles == 1 || a.ndims == 1)
+        return true;
+    if (a.phased())
+        return false;
+    for (int d = 0; d < a.ndims; ++d)
+        if (r.start[d] / a.tile != (r.stop[d] - 1) / a.tile)
+            return false;
+    return true;
+}
+
+// Fills `use` for array `a` read or written through `reg` (whole array when !has) by a statement
+// of extents cnt[0..nd): unit steps, inside the array, extents equal to cnt with extent-1
+// dimensions inserted or dropped in order, one block of memory.
+bool make_box(XArray* a, bool has, const cnh_region& reg, int nd, const int32_t* cnt, BoxUse& use) {
+    use.arr = a;
+    std::memset(&use.reg, 0, sizeof use.reg);
+    use.reg.ndims = a->ndims;
+    if (has && !reg.is_global && reg.ndims != a->ndims)
+        return false;
+    for (int d = 0; d < a->ndims; ++d) {
+        const bool whole = !has || reg.is_global;
+        use.reg.start[d] = whole ? 0 : reg.start[d];
+        use.reg.stop[d] = whole ? a->shape[d] : reg.stop[d];
+        use.reg.step[d] = 1;
+        if (!whole && reg.step[d] != 1)
+            return false;
+        if (use.reg.start[d] < 0 || use.reg.stop[d] > a->shape[d] || use.reg.stop[d] <= use.reg.start[d])
+            return false;
+    }
+    // match the box's extents with the statement's, skipping extent-1 dimensions on either side
+    int ad = 0;
+    for (int d = 0; d < nd; ++d) {
+        use.map[d] = -1;
+        while (ad < a->ndims && use.reg.stop[ad] - use.reg.start[ad] == 1 && cnt[d] != 1)
+            ++ad;
+        if (ad < a->ndims && use.reg.stop[ad] - use.reg.start[ad] == cnt[d]) {
+            // an extent of 1 on both sides pairs up only when enough array dimensions remain
+            if (cnt[d] == 1 && a->ndims - ad < nd - d)
+                continue;
+            use.map[d] = ad++;
+        } else if (cnt[d] != 1) {
+            return false;
+        }
+    }
+    for (; ad < a->ndims; ++ad)
+        if (use.reg.stop[ad] - use.reg.start[ad] != 1)
+            return false;
+    return box_is_one_block(*a, use.reg);
+}
+
+cnh_memref box_memref(const BoxUse& u, int nd, const int32_t* cnt) {
+    const XArray& a = *u.arr;
+    const int esz = dtype_size(a.dtype);
+    int64_t stride[3] = {1, 1, 1};
+    char* base = nullptr;
+    if (a.flat || a.ndims == 1) {
+        // the whole array is one row-major run
+        int64_t run = 1, off = 0;
+        for (int d = a.ndims - 1; d >= 0; --d) {
+            stride[d] = a.flat ? a.pitch[d] : run;
+            run *= a.shape[d];
+            off += u.reg.start[d] * stride[d];
+        }
+        base = static_cast<char*>(a.tiles[0]) + off * esz;
+    } else {
+        int64_t t = 0;
+        for (int d = 0; d < a.ndims; ++d)
+            t = t * a.grid[d] + (a.ntiles == 1 ? 0 : u.reg.start[d] / a.tile);
+        int32_t lo[3], ext[3];
+        a.tile_extent(t, lo, ext);
+        a.tile_strides(ext, stride);
+        int64_t off = 0;
+        for (int d = 0; d < a.ndims; ++d)
+            off += (int64_t)(u.reg.start[d] - lo[d]) * stride[d];
+        base = static_cast<char*>(a.tiles[(size_t)t]) + off * esz;
+    }
+    cnh_memref m;
+    std::memset(&m, 0, sizeof m);
+    m.allocated = m.aligned = base;
+    for (int d = 0; d < nd; ++d) {
+        m.sizes[d] = cnt[d];
+        m.strides[d] = u.map[d] >= 0 ? stride[u.map[d]] : 0;
+    }
+    return m;
+}
+
 // A window of a 2-D array, or of a 3-D array where the window has an extent of 1 along one
 // dimension (the first such is dropped), seen as a matrix in the array's own coordinates
 // (the sliced and dimension-dropped operands of charmnumeric.py:510-519,536-578 upstream,
@@ -1164,7 +1290,10 @@ int exec_matmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
 
 // MATMATMUL: C = sum of A_panel * B_panel over every k-overlapping pair of tiles, k ascending
 // (src/executor_matmatmul.cpp:105-484, src/executor_incremental.cpp:97-132).
-int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
+// `dest`: where the product goes instead of a new array (the box a following assignment names),
+// null for the ordinary form.
+int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root, const DagNode* dest_node = nullptr,
+                   bool* dest_taken = nullptr) {
     XArray *Aa, *Ba;
     cnh_region wA, wB;
     if (int rc = leaf_window(ex, n, root, 0, &Aa, &wA, "MATMATMUL"))
@@ -1187,17 +1316,49 @@ int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
     // fp64 products overwrite their result (every C element belongs to exactly one chain), so the
     // new array needs no zero-fill; the other types accumulate into zeros as upstream does
     const bool f64 = Aa->dtype == CNH_F64;
-    XArray* Cc;
-    if (int rc = make_array(ex, root.result_name, 2, Aa->dtype, shape, !f64, &Cc))
-        return rc;
+    // The product of `target[box] = A @ B` goes straight into the box when that is one strided
+    // block with unit stride along the columns: no temporary, no copy (fp64 only: the product
+    // overwrites, so what the box held does not matter).
+    XArray* Cc = nullptr;
+    char* dest_base = nullptr;
+    int64_t dest_ld = 0;
+    int dest_name = 0;
+    if (dest_node != nullptr && f64) {
+        const cnh_ast_node* dest_set = &dest_node->nodes[dest_node->roots.back()];
+        XArray* target = nullptr;
+        auto it = ex->arrays.find(dest_node->nodes[dest_set->operands[0]].result_name);
+        if (it != ex->arrays.end())
+            target = &it->second;
+        BoxUse use;
+        const int32_t cnt2[2] = {A.rows, B.cols};
+        if (target != nullptr && target->dtype == Aa->dtype && target != Aa && target != Ba &&
+            make_box(target, true, dest_set->region, 2, cnt2, use) && use.map[0] >= 0 &&
+            use.map[1] == target->ndims - 1) {
+            const cnh_memref m = box_memref(use, 2, cnt2);
+            if (m.strides[1] == 1) {
+                dest_base = static_cast<char*>(m.aligned);
+                dest_ld = m.strides[0];
+                dest_name = target->name;
+            }
+        }
+    }
+    if (dest_taken != nullptr)
+        *dest_taken = dest_base != nullptr;
+    if (dest_base == nullptr)
+        if (int rc = make_array(ex, root.result_name, 2, Aa->dtype, shape, !f64, &Cc))
+            return rc;
     const int esz = dtype_size(Aa->dtype);
     const int TA = Aa->tile, TB = Ba->tile, K = A.cols;
     int calls = 0;
     std::vector<cnh_gemm_job> jobs;   // all panel products of the node go out as one launch
-    for (int ci = 0; ci < Cc->grid[0]; ++ci)
-        for (int cj = 0; cj < Cc->grid[1]; ++cj) {
-            int32_t clo[3], cext[3];
-            Cc->tile_extent((int64_t)ci * Cc->grid[1] + cj, clo, cext);
+    const int cgrid0 = Cc ? Cc->grid[0] : 1, cgrid1 = Cc ? Cc->grid[1] : 1;
+    for (int ci = 0; ci < cgrid0; ++ci)
+        for (int cj = 0; cj < cgrid1; ++cj) {
+            int32_t clo[3] = {0, 0, 0}, cext[3] = {A.rows, B.cols, 1};
+            if (Cc)
+                Cc->tile_extent((int64_t)ci * Cc->grid[1] + cj, clo, cext);
+            char* const ctile = Cc ? static_cast<char*>(Cc->tiles[(size_t)ci * Cc->grid[1] + cj]) : dest_base;
+            const int64_t cld = Cc ? cext[1] : dest_ld;
             // rows i of this C tile are rows A.r0 + i of A's array, its columns j are columns
             // B.c0 + j of B's: cut both ranges where those arrays' tiles end
             for (int r0 = clo[0]; r0 < clo[0] + cext[0];) {
@@ -1212,10 +1373,9 @@ int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
                         int t0, t1, t2, t3;
                         const char* ap = A.at(A.r0 + r0, A.c0 + k0, &lda, &t0, &t1, &t2, &t3);
                         const char* bp = B.at(B.r0 + k0, B.c0 + c0, &ldb, &t0, &t1, &t2, &t3);
-                        char* cp = static_cast<char*>(Cc->tiles[(size_t)ci * Cc->grid[1] + cj]) +
-                                   ((int64_t)(r0 - clo[0]) * cext[1] + (c0 - clo[1])) * esz;
+                        char* cp = ctile + ((int64_t)(r0 - clo[0]) * cld + (c0 - clo[1])) * esz;
                         ++calls;
-                        jobs.push_back(cnh_gemm_job{r1 - r0, c1 - c0, k1 - k0, ap, lda, bp, ldb, cp, cext[1]});
+                        jobs.push_back(cnh_gemm_job{r1 - r0, c1 - c0, k1 - k0, ap, lda, bp, ldb, cp, cld});
                         k0 = k1;
                     }
                     c0 = c1;
@@ -1227,7 +1387,8 @@ int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
         if (int rc = cnh_gemm_batch(Aa->dtype, (int)jobs.size(), jobs.data(), f64 ? 1 : 0, ex->stream))
             return rc;
     ex->log("matmatmul A=" + std::to_string(Aa->name) + " B=" + std::to_string(Ba->name) + " out=" +
-            std::to_string(Cc->name) + " panel_products=" + std::to_string(calls));
+            std::to_string(Cc ? Cc->name : dest_name) + (Cc ? "" : " into_region") + " panel_products=" +
+            std::to_string(calls));
     if (a_copy)
         drop_array(ex, Aa->name);
     if (b_copy)
@@ -1432,6 +1593,295 @@ int exec_node(Ex* ex, const DagNode& n) {
         return set_error(-34, "DAG node %d: opcode %d is not supported by this executor", n.id,
                          root.opcode);
     }
+}
+
+// ---- several assignments of one extent as one launch ----
+// A run of statements `target[box] = f(operands[boxes])` whose boxes all have the same extents
+// (the gate statements of an LSTM step, the updates of several fields over one window) is launch
+// bound when run one by one. Where every box is a single strided block of device memory — the
+// array is one row-major block, or has one tile, or the box lies inside one tile — the run becomes
+// one group with one output root per statement, launched through the memref interface
+// (cnh_launch_group, the dispatch_kernel seam) with a memref per box. A statement that reads
+// exactly the box an earlier one of the run assigned takes the value from registers; results are
+// those of running the statements one after the other:
+//   - a box read by a later statement and a box assigned by an earlier one of the same array are
+//     either identical or share no element;
+//   - a box assigned by a later statement and any box an earlier one read or assigned in the same
+//     array are either identical or share no element (identical: the lane that reads or writes an
+//     element is the lane that overwrites it later; an earlier identical store is dropped).
+
+bool open_ended_allowed(const Ex* ex) { return !ex->final_pass; }
+
+// Is node `n` an assignment this pass can take? Fills `st`.
+bool analyse_statement(Ex* ex, const DagNode& n, Stmt& st) {
+    if (n.roots.empty())
+        return false;
+    const cnh_ast_node& root = n.nodes[n.roots.back()];
+    if (root.opcode != CNH_OP_SET_REGION || root.n_operands != 2 || root.region.is_global)
+        return false;
+    if (n.nodes[root.operands[1]].is_scalar)
+        return false;                                   // a fill
+    for (size_t i = 0; i + 1 < n.roots.size(); ++i)
+        if (!n.nodes[n.roots[i]].is_temp)
+            return false;
+    st.n = &n;
+    st.nd = root.region.ndims;
+    int64_t elems = 1;
+    for (int d = 0; d < st.nd; ++d) {
+        if (root.region.step[d] != 1)
+            return false;
+        st.cnt[d] = root.region.stop[d] - root.region.start[d];
+        if (st.cnt[d] <= 0)
+            return false;
+        elems *= st.cnt[d];
+    }
+    if (elems > kFuseMaxElems)
+        return false;
+    auto tgt = ex->arrays.find(n.nodes[root.operands[0]].result_name);
+    if (tgt == ex->arrays.end() || tgt->second.ndims != st.nd)
+        return false;
+    st.dtype = tgt->second.dtype;
+    if (!make_box(&tgt->second, true, root.region, st.nd, st.cnt, st.out))
+        return false;
+    std::set<int> internal;
+    for (int32_t r : n.roots)
+        internal.insert(n.nodes[r].result_name);
+    st.reads.clear();
+    for (size_t ri = 0; ri < n.roots.size(); ++ri) {
+        const cnh_ast_node& r = n.nodes[n.roots[ri]];
+        if (r.dtype != st.dtype)
+            return false;
+        for (int oi = 0; oi < r.n_operands; ++oi) {
+            if (r.opcode == CNH_OP_SET_REGION && oi == 0)
+                continue;
+            if (r.operands[oi] < 0 || r.operands[oi] >= (int)n.nodes.size())
+                return false;
+            const cnh_ast_node& op = n.nodes[r.operands[oi]];
+            if (op.is_scalar || internal.count(op.result_name))
+                continue;
+            auto it = ex->arrays.find(op.result_name);
+            if (it == ex->arrays.end() || it->second.dtype != st.dtype)
+                return false;
+            if (op.is_broadcast) {
+                if (it->second.elems != 1)
+                    return false;
+                continue;
+            }
+            Stmt::Read rd;
+            rd.root = (int)ri;
+            rd.slot = oi;
+            if (!make_box(&it->second, r.has_operand_region[oi] != 0, r.operand_regions[oi], st.nd, st.cnt,
+                          rd.use))
+                return false;
+            // reading the assigned array elsewhere than at the assigned box: ping-pong territory
+            if (rd.use.arr == st.out.arr && !boxes_identical(rd.use, st.out) && !boxes_disjoint(rd.use, st.out))
+                return false;
+            st.reads.push_back(rd);
+        }
+    }
+    // one array read at several overlapping boxes is a stencil: the register-window route reads
+    // each element once, this one would read it once per box
+    for (size_t a = 0; a < st.reads.size(); ++a)
+        for (size_t b = a + 1; b < st.reads.size(); ++b)
+            if (st.reads[a].use.arr == st.reads[b].use.arr &&
+                !boxes_identical(st.reads[a].use, st.reads[b].use) &&
+                !boxes_disjoint(st.reads[a].use, st.reads[b].use))
+                return false;
+    return st.reads.size() <= kFuseMaxReads;
+}
+
+bool can_join(const std::vector<Stmt>& run, const Stmt& b) {
+    const Stmt& first = run.front();
+    if (b.nd != first.nd || b.dtype != first.dtype)
+        return false;
+    for (int d = 0; d < b.nd; ++d)
+        if (b.cnt[d] != first.cnt[d])
+            return false;
+    size_t reads = b.reads.size();
+    for (const Stmt& s : run) {
+        reads += s.reads.size();
+        for (const auto& rd : b.reads)
+            if (!boxes_identical(rd.use, s.out) && !boxes_disjoint(rd.use, s.out))
+                return false;
+        if (!boxes_identical(b.out, s.out) && !boxes_disjoint(b.out, s.out))
+            return false;
+        for (const auto& rd : s.reads)
+            if (!boxes_identical(b.out, rd.use) && !boxes_disjoint(b.out, rd.use))
+                return false;
+    }
+    return run.size() < kFuseMaxStmts && reads <= kFuseMaxReads;
+}
+
+// The run as one multi-root group. Boxes are numbered; the group's regions carry the numbers, not
+// the coordinates (the launch hands over memrefs), so every step of a time loop finds the kernel
+// of the first one in the cache.
+int exec_statement_run(Ex* ex, const std::vector<Stmt>& run) {
+    DagNode merged;
+    merged.id = run.front().n->id;
+    merged.fusible = 1;
+    std::vector<BoxUse> boxes;                 // by number
+    auto number_of = [&](const BoxUse& u) {
+        for (size_t i = 0; i < boxes.size(); ++i)
+            if (boxes_identical(boxes[i], u) && std::memcmp(boxes[i].map, u.map, sizeof u.map) == 0)
+                return (int)i;
+        boxes.push_back(u);
+        return (int)boxes.size() - 1;
+    };
+    auto tag_region = [&](cnh_region& r, int number, int nd) {
+        std::memset(&r, 0, sizeof r);
+        r.ndims = nd;
+        for (int d = 0; d < nd; ++d) {
+            r.start[d] = number;
+            r.stop[d] = number + 1;
+            r.step[d] = 1;
+        }
+    };
+    struct Done { int value_node; int set_root; const Stmt* st; };
+    std::vector<Done> done;
+    int next_literal = -1;
+    for (const Stmt& st : run) {
+        const DagNode& n = *st.n;
+        const int base = (int)merged.nodes.size();
+        for (const cnh_ast_node& a : n.nodes) {
+            merged.nodes.push_back(a);
+            cnh_ast_node& c = merged.nodes.back();
+            for (int oi = 0; oi < c.n_operands; ++oi)
+                if (c.operands[oi] >= 0)
+                    c.operands[oi] += base;
+            // literals are named per DAG node (-1, -2, ...): keep them apart across statements
+            if (c.is_scalar)
+                c.result_name = next_literal--;
+        }
+        for (const auto& rd : st.reads) {
+            cnh_ast_node& r = merged.nodes[(size_t)base + n.roots[(size_t)rd.root]];
+            // the newest earlier statement that assigned exactly this box supplies the value
+            const Done* src = nullptr;
+            for (const Done& d : done)
+                if (boxes_identical(d.st->out, rd.use))
+                    src = &d;
+            if (src != nullptr) {
+                const cnh_ast_node& set = merged.nodes[(size_t)src->set_root];
+                r.operands[rd.slot] = set.operands[1];
+                r.has_operand_region[rd.slot] = set.has_operand_region[1];
+                r.operand_regions[rd.slot] = set.operand_regions[1];
+            } else {
+                r.has_operand_region[rd.slot] = 1;
+                tag_region(r.operand_regions[rd.slot], number_of(rd.use), st.nd);
+            }
+        }
+        for (int32_t r : n.roots)
+            merged.roots.push_back(base + r);
+        const int set_root = base + n.roots.back();
+        tag_region(merged.nodes[(size_t)set_root].region, number_of(st.out), st.nd);
+        // an earlier store into the very same box is dead
+        for (const Done& d : done)
+            if (boxes_identical(d.st->out, st.out))
+                merged.nodes[(size_t)d.set_root].is_temp = 1;
+        done.push_back({merged.nodes[(size_t)set_root].operands[1], set_root, &st});
+    }
+
+    Group g;
+    canonicalise(merged, g);
+    cnh_kernel* k = nullptr;
+    if (int rc = compile_cached(ex, g, &k))
+        return rc;
+    int n_in = 0, n_scalar = 0, n_out = 0;
+    if (int rc = cnh_kernel_signature(k, &n_in, &n_scalar, &n_out))
+        return rc;
+    const int nd = run.front().nd;
+    const int32_t* cnt = run.front().cnt;
+    std::vector<cnh_memref> ins((size_t)std::max(1, n_in)), outs((size_t)std::max(1, n_out));
+    for (int i = 0; i < n_in; ++i) {
+        int cname = 0, has = 0;
+        cnh_region reg;
+        if (int rc = cnh_kernel_input(k, i, &cname, &has, &reg))
+            return rc;
+        CNH_CHECK(has && reg.start[0] >= 0 && reg.start[0] < (int)boxes.size(), -26,
+                  "statement run: input %d carries no box number", i);
+        ins[(size_t)i] = box_memref(boxes[(size_t)reg.start[0]], nd, cnt);
+    }
+    for (int i = 0; i < n_out; ++i) {
+        int rname = 0, tname = 0, is_set = 0;
+        cnh_region reg;
+        if (int rc = cnh_kernel_output(k, i, &rname, &tname, &is_set, &reg))
+            return rc;
+        CNH_CHECK(is_set && reg.start[0] >= 0 && reg.start[0] < (int)boxes.size(), -26,
+                  "statement run: output %d carries no box number", i);
+        outs[(size_t)i] = box_memref(boxes[(size_t)reg.start[0]], nd, cnt);
+    }
+    std::vector<const void*> scalars((size_t)std::max(1, n_scalar), nullptr);
+    for (int i = 0; i < n_scalar; ++i) {
+        int cname = 0;
+        if (int rc = cnh_kernel_scalar(k, i, &cname))
+            return rc;
+        XArray* sarr;
+        if (int rc = find_array(ex, g.canon_to_actual[cname], &sarr, "broadcast scalar"))
+            return rc;
+        scalars[(size_t)i] = sarr->tiles[0];
+    }
+    ex->stats[5]++;
+    std::string names;
+    for (const Stmt& st : run)
+        names += (names.empty() ? "" : ",") + std::to_string(st.out.arr->name);
+    ex->log("group node=" + std::to_string(merged.id) + " path=statements count=" +
+            std::to_string(run.size()) + " inputs=" + std::to_string(n_in) + " outputs=" +
+            std::to_string(n_out) + " out=" + names);
+    if (ex->dry)
+        return 0;
+    return cnh_launch_group(k, nd, n_in, ins.data(), n_scalar, scalars.data(), 1, n_out, outs.data(),
+                            ex->stream);
+}
+
+// Nodes [i, ...) of the message: a run of two or more assignments this pass can merge, deletions
+// in between put off until the run has been launched. Returns the number of nodes consumed.
+int try_statement_run(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t* used, bool* open_ended) {
+    *used = 0;
+    *open_ended = false;
+    std::vector<Stmt> run;
+    std::vector<int> deletions;
+    size_t j = i, last_stmt_end = i;
+    std::vector<int> deletions_kept;
+    for (; j < dag.size(); ++j) {
+        const DagNode& n = dag[j];
+        if (n.roots.empty())
+            break;
+        const cnh_ast_node& root = n.nodes[n.roots.back()];
+        if (root.opcode == kOpDelete) {
+            if (run.empty())
+                break;
+            deletions.push_back(root.result_name);
+            continue;
+        }
+        Stmt st;
+        if (!analyse_statement(ex, n, st))
+            break;
+        // an array deleted earlier in the run must not be touched by a later statement
+        bool touches_deleted = false;
+        for (int name : deletions) {
+            touches_deleted = touches_deleted || st.out.arr->name == name;
+            for (const auto& rd : st.reads)
+                touches_deleted = touches_deleted || rd.use.arr->name == name;
+        }
+        if (touches_deleted || (!run.empty() && !can_join(run, st)))
+            break;
+        run.push_back(st);
+        last_stmt_end = j + 1;
+        deletions_kept = deletions;
+    }
+    // ran off the end of the message with room left: more of the run may follow
+    if (j == dag.size() && !run.empty() && run.size() < kFuseMaxStmts && open_ended_allowed(ex)) {
+        *open_ended = true;
+        return 0;
+    }
+    if (run.empty())
+        return 0;
+    if (int rc = exec_statement_run(ex, run))
+        return rc;
+    for (int name : deletions_kept)
+        drop_array(ex, name);
+    ex->stats[2] += (int64_t)(last_stmt_end - i);
+    *used = last_stmt_end - i;
+    return 0;
 }
 
 int parse_dag(const char* msg, int64_t size, std::vector<DagNode>& out) {
@@ -1679,17 +2129,89 @@ void plan_message(Ex* ex, const std::vector<DagNode>& dag) {
     }
 }
 
-int run_message(Ex* ex, const char* msg, int64_t size) {
-    std::vector<DagNode> dag;
-    if (int rc = parse_dag(msg, size, dag))
+// MATMATMUL -> tmp; target[box] = tmp; delete tmp: the product is written into the box directly.
+int try_product_into_region(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t* used, bool* open_ended) {
+    *used = 0;
+    *open_ended = false;
+    if (!dag[i].roots.empty() && dag[i].nodes[dag[i].roots.back()].opcode == CNH_OP_MATMATMUL &&
+        i + 2 >= dag.size() && open_ended_allowed(ex)) {
+        // the assignment that takes the product, or the deletion of the temporary, may be the
+        // first nodes of the next message
+        *open_ended = true;
+        return 0;
+    }
+    if (i + 2 >= dag.size() || dag[i].roots.empty() || dag[i + 1].roots.size() != 1 || dag[i + 2].roots.empty())
+        return 0;
+    const cnh_ast_node& mm = dag[i].nodes[dag[i].roots.back()];
+    const cnh_ast_node& set = dag[i + 1].nodes[dag[i + 1].roots.back()];
+    const cnh_ast_node& del = dag[i + 2].nodes[dag[i + 2].roots.back()];
+    if (mm.opcode != CNH_OP_MATMATMUL || set.opcode != CNH_OP_SET_REGION || del.opcode != kOpDelete ||
+        set.n_operands != 2 || set.region.is_global || del.result_name != mm.result_name)
+        return 0;
+    const cnh_ast_node& value = dag[i + 1].nodes[set.operands[1]];
+    if (value.is_scalar || value.opcode != CNH_OP_NOOP || value.result_name != mm.result_name ||
+        (set.has_operand_region[1] && !set.operand_regions[1].is_global))
+        return 0;
+    for (int d = 0; d < set.region.ndims; ++d)
+        if (set.region.step[d] != 1)
+            return 0;
+    bool taken = false;
+    if (int rc = exec_matmatmul(ex, dag[i], mm, &dag[i + 1], &taken))
         return rc;
+    if (taken) {
+        ex->stats[2] += 3;
+        *used = 3;
+    } else {
+        ex->stats[2] += 1;
+        *used = 1;               // the product went to a temporary as usual; the rest follows node by node
+    }
+    return 0;
+}
+
+int run_nodes(Ex* ex, std::vector<DagNode>& dag) {
     if (ex->solver_on)
         plan_message(ex, dag);
     int rc = 0;
-    for (const DagNode& n : dag)
-        if ((rc = exec_node(ex, n)) != 0)
-            break;
+    for (size_t i = 0; i < dag.size() && rc == 0;) {
+        size_t used = 0;
+        if (ex->fuse_on && !ex->solver_on) {
+            bool open_ended = false;
+            rc = try_product_into_region(ex, dag, i, &used, &open_ended);
+            if (rc == 0 && used == 0 && !open_ended)
+                rc = try_statement_run(ex, dag, i, &used, &open_ended);
+            if (rc == 0 && open_ended) {
+                ex->held.assign(dag.begin() + (std::ptrdiff_t)i, dag.end());
+                break;
+            }
+        }
+        if (rc == 0 && used == 0) {
+            rc = exec_node(ex, dag[i]);
+            used = 1;
+        }
+        i += used;
+    }
     ex->planned.clear();
+    return rc;
+}
+
+int run_message(Ex* ex, const char* msg, int64_t size) {
+    std::vector<DagNode> dag, fresh;
+    dag.swap(ex->held);                 // what the previous message left open comes first
+    if (int rc = parse_dag(msg, size, fresh))
+        return rc;
+    dag.insert(dag.end(), std::make_move_iterator(fresh.begin()), std::make_move_iterator(fresh.end()));
+    return run_nodes(ex, dag);
+}
+
+// Executes whatever waits in `held`, to the end.
+int flush_held(Ex* ex) {
+    if (ex->held.empty())
+        return 0;
+    std::vector<DagNode> dag;
+    dag.swap(ex->held);
+    ex->final_pass = true;
+    const int rc = run_nodes(ex, dag);
+    ex->final_pass = false;
     return rc;
 }
 
@@ -1725,18 +2247,21 @@ void worker_loop(Ex* ex) {
 
 // Waits for queued messages and hands over the error one of them may have left.
 int drain(Ex* ex) {
-    if (!ex->async_on)
-        return 0;
-    std::unique_lock<std::mutex> lk(ex->qmu);
-    ex->idle_cv.wait(lk, [&] { return ex->queue.empty() && !ex->busy; });
-    if (ex->deferred_rc == 0)
-        return 0;
-    const int rc = ex->deferred_rc;
-    const std::string text = std::move(ex->deferred_msg);
-    ex->deferred_rc = 0;
-    ex->deferred_msg.clear();
-    lk.unlock();
-    return set_error(rc, "%s", text.c_str());
+    if (ex->async_on) {
+        std::unique_lock<std::mutex> lk(ex->qmu);
+        ex->idle_cv.wait(lk, [&] { return ex->queue.empty() && !ex->busy; });
+        if (ex->deferred_rc != 0) {
+            const int rc = ex->deferred_rc;
+            const std::string text = std::move(ex->deferred_msg);
+            ex->deferred_rc = 0;
+            ex->deferred_msg.clear();
+            ex->held.clear();           // work behind a failed message is dropped
+            lk.unlock();
+            return set_error(rc, "%s", text.c_str());
+        }
+    }
+    // the worker is idle now (or there is none): the statements it left open run on this thread
+    return flush_held(ex);
 }
 
 void stop_worker(Ex* ex) {
@@ -1775,10 +2300,9 @@ int cnx_create(int device, int num_pes, int odf, cnx_executor** out) {
 int cnx_destroy(cnx_executor* ex) {
     if (!ex)
         return 0;
-    if (ex->async_on) {
-        (void)drain(ex);
+    (void)drain(ex);
+    if (ex->async_on)
         stop_worker(ex);
-    }
     if (!ex->dry) {
         cnh_stream_sync(ex->stream);
         for (auto& kv : ex->arrays) {
@@ -1820,6 +2344,14 @@ int cnx_set_layout(cnx_executor* ex, int flat_rank3) {
     if (int rc = drain(ex))
         return rc;
     ex->flat3 = flat_rank3 != 0;
+    return 0;
+}
+
+int cnx_set_fusion(cnx_executor* ex, int on) {
+    CNH_CHECK(ex != nullptr, -2, "null executor");
+    if (int rc = drain(ex))
+        return rc;
+    ex->fuse_on = on != 0;
     return 0;
 }
 

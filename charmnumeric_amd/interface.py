@@ -24,6 +24,7 @@ class CharmNumericInterface:
         self._pipeline = False
         self._solver = os.environ.get("CHARMNUMERIC_SOLVER", "0") not in ("", "0")
         self._flat3 = os.environ.get("CHARMNUMERIC_FLAT3", "1") not in ("", "0")
+        self._fusion = os.environ.get("CHARMNUMERIC_FUSE", "1") not in ("", "0")
 
     # -- decomposition planning ----------------------------------------------------------------
     def set_solver(self, on=True):
@@ -43,6 +44,14 @@ class CharmNumericInterface:
         self._flat3 = bool(flat_rank3)
         if self._ex is not None:
             L.check(L.lib.cnx_set_layout(self._ex, 1 if flat_rank3 else 0))
+
+    def set_fusion(self, on=True):
+        """Whether the executor merges runs of same-extent assignments into one launch and writes
+        matrix products straight into the slice they are assigned to (default on; environment
+        variable CHARMNUMERIC_FUSE=0 turns it off for every interface). Values never depend on it."""
+        self._fusion = bool(on)
+        if self._ex is not None:
+            L.check(L.lib.cnx_set_fusion(self._ex, 1 if on else 0))
 
     # -- pipelining --------------------------------------------------------------------------
     def set_pipeline(self, on=True):
@@ -71,6 +80,8 @@ class CharmNumericInterface:
             L.check(L.lib.cnx_set_solver(self._ex, 1))
         if not self._flat3:
             L.check(L.lib.cnx_set_layout(self._ex, 0))
+        if not self._fusion:
+            L.check(L.lib.cnx_set_fusion(self._ex, 0))
         if self._pipeline:
             L.check(L.lib.cnx_set_async(self._ex, 1))
         return self

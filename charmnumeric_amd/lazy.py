@@ -37,7 +37,7 @@ class ArrayRef:
     def __init__(self, name, region, shape, base_ndims, dtype, broadcast=False):
         self.name = name
         self.region = region          # (start, stop, step) tuples relative to the base array, or None
-        self.shape = tuple(shape)
+        self.shape = shape if type(shape) is tuple else tuple(shape)
         self.base_ndims = base_ndims
         self.dtype = dtype            # wire dtype
         self.broadcast = broadcast
@@ -51,8 +51,8 @@ class Instr:
         self.kind = kind              # create | op | set | nonfusible | delete | call
         self.name = name
         self.opcode = opcode
-        self.operands = list(operands)  # ArrayRef or python scalars
-        self.shape = tuple(shape)
+        self.operands = operands if type(operands) is list else list(operands)  # ArrayRef or scalars
+        self.shape = shape if type(shape) is tuple else tuple(shape)
         self.dtype = dtype
         self.region = region
         self.payload = payload

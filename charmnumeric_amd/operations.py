@@ -12,12 +12,16 @@ from .array import tile as _tile_array
 
 
 def tanh(x):
+    if isinstance(x, _ArrayLike):
+        return unary(L.OP_TANH, x)
     if _is_scalar_like(x):
         return np.tanh(_coerce_scalar(x))
     return unary(L.OP_TANH, x)
 
 
 def exp(x):
+    if isinstance(x, _ArrayLike):
+        return unary(L.OP_EXP, x)
     if _is_scalar_like(x):
         return np.exp(_coerce_scalar(x))
     return unary(L.OP_EXP, x)

@@ -88,6 +88,15 @@ int cnx_set_solver(cnx_executor* ex, int on);
  * views into it with the array's row and plane pitches; stencil sweeps then run on the block as a
  * whole. 0: one contiguous buffer per partition, as for the other ranks. Values never depend on it. */
 int cnx_set_layout(cnx_executor* ex, int flat_rank3);
+/* Launch fusion across the nodes of a DAG message, on by default. (1) A run of assignments
+ * `target[box] = f(operand boxes)` of one extent (at most 2^22 elements each), every box one
+ * strided block of device memory, goes out as ONE group with an output root per statement through
+ * the memref launch (cnh_launch_group); a statement that reads the very box an earlier one of the
+ * run assigned takes it from registers, and boxes of one array that are neither identical nor
+ * disjoint end the run, so results are those of the statements run one by one. (2) MATMATMUL into a
+ * temporary followed by `target[box] = temporary` and the temporary's deletion writes the fp64
+ * product straight into the box. Off: every node is executed on its own, as upstream does. */
+int cnx_set_fusion(cnx_executor* ex, int on);
 
 /* ArrayDAGGroup::receive_dag(int epoch, int size, char msg[size]) (src/backend.ci:15,
  * src/dag_group_receive.cpp:190-575) followed by the partitions' run(): executes every node of the

@@ -307,7 +307,9 @@ def test_in_place_when_read_and_written_lattices_miss_each_other(itf):
         stmt()
         cnp.execute(itf)
         (line,) = lines(itf, "group")
-        return line.split()[-1]
+        # a statement whose boxes are single blocks and do not meet goes out through the memref
+        # launch (in place by construction)
+        return "inplace" if "path=statements" in line else line.split()[-1]
 
     def assign(dst, src):
         def stmt():
@@ -359,6 +361,7 @@ def test_get_checks_rank_size_and_dtype(itf):
 
 
 def test_auto_flush_happens_between_statements(itf):
+    itf.set_fusion(False)      # one launch per statement, so that the flushes can be counted
     cnp.set_auto_flush(itf, 5)
     a = cnp.zeros((16,))
     for _ in range(6):
@@ -407,10 +410,51 @@ def test_auto_flush_keeps_a_named_intermediate_fused(itf):
     assert sum(ln.startswith("delete") for ln in itf.trace()) == 1
 
 
+def test_runs_of_same_extent_assignments_become_one_launch(itf):
+    """Assignments of one extent whose boxes are single blocks of memory merge; a box that overlaps
+    an earlier one of the same array without being identical ends the run; a matrix product
+    assigned to a slab is written there directly."""
+    n, b, d = 6, 8, 16
+    A = cnp.zeros((n, b, 2 * d))
+    C = cnp.zeros((n, b, d))
+    H = cnp.zeros((n, b, d))
+    W = cnp.zeros((d, 2 * d))
+    cnp.execute(itf)
+    itf.trace()
+    t = 2
+    A[t] = H[t - 1].dot(W)
+    C[t] = A[t, :, :d] * A[t, :, d:]
+    C[t] += A[t, :, :d] * C[t - 1]
+    H[t] = cnp.tanh(C[t])
+    cnp.execute(itf)
+    log = itf.trace()
+    assert any("matmatmul" in ln and "into_region" in ln for ln in log)
+    assert not any(ln.startswith("create") for ln in log)          # no temporary for the product
+    runs = [ln for ln in log if "path=statements" in ln]
+    # three statements, two of them assigning C[t]: the first store is dropped
+    assert len(runs) == 1 and "count=3" in runs[0] and "outputs=2" in runs[0]
+    # overlapping, not identical: u[1:5] is read, then u[2:6] assigned -> two launches
+    u, v = cnp.zeros(8), cnp.zeros(8)
+    cnp.execute(itf)
+    itf.trace()
+    v[0:4] = u[1:5] * 2.0
+    u[2:6] = v[2:6] + 1.0
+    cnp.execute(itf)
+    runs = [ln for ln in itf.trace() if "path=statements" in ln]
+    assert len(runs) == 2 and all("count=1" in ln for ln in runs)
+    # switched off: node by node
+    itf.set_fusion(False)
+    H[3] = C[3] * 2.0
+    C[4] = H[3] + 1.0
+    cnp.execute(itf)
+    assert not any("path=statements" in ln for ln in itf.trace())
+
+
 def test_kernel_cache_is_bounded_over_a_long_slab_loop(itf):
     """Each step assigns another slab: another group (same code, other regions). The executor keeps
     a bounded number of them and lets the oldest go."""
     n = 4500
+    itf.set_fusion(False)              # one group per statement: that is what fills the cache
     a = cnp.zeros((n, 8))
     for t in range(1, n):
         a[t] = a[t - 1] * 0.5

@@ -449,4 +449,56 @@ def test_disjoint_self_reference_updates_in_place(itf):
     got = Cs.get(itf)
     assert np.array_equal(got, host)
     groups = [ln for ln in itf.trace() if ln.startswith("group")]
-    assert len(groups) == n - 1 and all("inplace" in g for g in groups)
+    # merged into runs of statements (one launch, the chained slab handed on in registers) or run
+    # one by one in place; never through a second buffer
+    assert all("inplace" in g or "path=statements" in g for g in groups)
+    counted = sum(int(g.split("count=")[1].split()[0]) if "count=" in g else 1 for g in groups)
+    assert counted == n - 1
+
+
+@pytest.mark.parametrize("fusion", [True, False], ids=["merged", "one-by-one"])
+def test_statement_runs_give_what_the_statements_give_one_by_one(itf, fusion, rank3_layout):
+    """Runs of same-extent assignments (merged into one launch by default) against NumPy executing
+    the same statements in order: register forwarding through an assigned box, a store dropped
+    because a later statement assigns the same box, other slabs of the assigned array, lower-rank
+    values into slabs, and the hazards that must end a run."""
+    itf.set_fusion(fusion)
+    rng = np.random.default_rng(8)
+    n, b, d = 5, 12, 20
+    hA, hC, hH = rng.standard_normal((n, b, 2 * d)), rng.standard_normal((n, b, d)), rng.standard_normal((n, b, d))
+    hW = rng.standard_normal((d, 2 * d))
+    hM = rng.standard_normal((b, d))
+    A, C, H, W, M = (cnp.array(x) for x in (hA, hC, hH, hW, hM))
+    for t in range(1, n):
+        A[t] = H[t - 1].dot(W)
+        hA[t] = hH[t - 1] @ hW
+        C[t] = A[t, :, :d] * A[t, :, d:]
+        hC[t] = hA[t, :, :d] * hA[t, :, d:]
+        C[t] += A[t, :, :d] * C[t - 1]
+        hC[t] += hA[t, :, :d] * hC[t - 1]
+        H[t] = cnp.tanh(C[t]) * 0.25
+        hH[t] = np.tanh(hC[t]) * 0.25
+        H[t - 1] = M * 0.5                    # assigns a slab an earlier statement of the run read
+        hH[t - 1] = hM * 0.5
+    assert np.allclose(A.get(itf), hA, rtol=1e-12, atol=1e-12)
+    assert np.allclose(C.get(itf), hC, rtol=1e-12, atol=1e-12)
+    assert np.allclose(H.get(itf), hH, rtol=1e-12, atol=1e-12)
+    # chains through one array, bit for bit
+    hx = rng.standard_normal((40, 6))
+    x = cnp.array(hx)
+    for t in range(1, 40):
+        x[t] = x[t - 1] * 0.5 + x[t]
+        hx[t] = hx[t - 1] * 0.5 + hx[t]
+    assert np.array_equal(x.get(itf), hx)
+    # hazards: shifted read of what the previous statement assigned, and assigning over what it read
+    hu, hv = rng.standard_normal(64), rng.standard_normal(64)
+    u, v = cnp.array(hu), cnp.array(hv)
+    v[0:32] = u[1:33] * 2.0
+    hv[0:32] = hu[1:33] * 2.0
+    u[2:34] = v[2:34] + 1.0
+    hu[2:34] = hv[2:34] + 1.0
+    v[4:36] = u[3:35] - v[4:36]
+    hv[4:36] = hu[3:35] - hv[4:36]
+    u[4:36] = u[4:36] * v[4:36]
+    hu[4:36] = hu[4:36] * hv[4:36]
+    assert np.array_equal(u.get(itf), hu) and np.array_equal(v.get(itf), hv)
