@@ -975,11 +975,16 @@ def run_frontend(n, steps, warmup):
             cnp.execute(itl)
             itl.sync()
 
-        lstm_steps(0, 4)
+        # the whole sequence twice: the first pass also compiles every kernel the program needs
+        # (the merged statement runs of steps 0, 1 and of the later ones), the second is what a
+        # longer sequence costs per step
         t0 = time.perf_counter()
-        lstm_steps(4, n)
+        lstm_steps(0, n)
+        out["lstm_first_pass_us_per_step"] = round((time.perf_counter() - t0) / n * 1e6, 1)
+        t0 = time.perf_counter()
+        lstm_steps(0, n)
         dt = time.perf_counter() - t0
-        out["lstm_us_per_step"] = round(dt / (n - 4) * 1e6, 1)
+        out["lstm_us_per_step"] = round(dt / n * 1e6, 1)
         out["lstm_h_last_abs_mean"] = float(np.mean(np.abs(Hout[n - 1].get(itl))))
         del X, W, h0, Hin, Hout, IFOG, IFOGf, Cs, Ct
         cnp.execute(itl)

@@ -255,6 +255,10 @@ _PROTOS.update({
     "cnx_destroy": (C.c_int, [C.c_void_p]),
     "cnx_set_min_tile": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
     "cnx_receive_dag": (C.c_int, [C.c_void_p, C.c_int, C.c_int64, C.c_char_p]),
+    "cnx_receive_log": (C.c_int, [C.c_void_p, C.c_int64, C.c_char_p, C.c_int]),
+    "cnx_discard_log": (C.c_int, [C.c_void_p]),
+    "cnx_set_capture": (C.c_int, [C.c_void_p, C.c_int]),
+    "cnx_captured": (C.c_int64, [C.c_void_p, C.c_char_p, C.c_size_t]),
     "cnx_set_async": (C.c_int, [C.c_void_p, C.c_int]),
     "cnx_get": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int, C.c_void_p]),
     "cnx_put": (C.c_int, [C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_void_p]),

@@ -125,21 +125,34 @@ def _expand_key(key, ndims):
 def parse_key(key, shape):
     """Index expression -> (start, stop, step) per dimension, relative to an object of `shape`."""
     ndims = len(shape)
-    start, stop, step = [0] * ndims, [0] * ndims, [1] * ndims
-    if type(key) is tuple and len(key) == ndims:
-        # the common form, one plain slice or integer per dimension: no ellipsis to expand
-        for d in range(ndims):
-            item = key[d]
-            if type(item) is slice and (item.step is None or (type(item.step) is int and item.step > 0)):
+    if type(key) is not tuple:
+        key = (key,)
+    if len(key) <= ndims:
+        # the common form, plain slices and integers only (dimensions not named are taken whole):
+        # nothing to expand
+        start, stop, step = [0] * ndims, list(shape), [1] * ndims
+        d = 0
+        for item in key:
+            kind = type(item)
+            if kind is int:
+                extent = shape[d]
+                if item < 0:
+                    item += extent
+                if not 0 <= item < extent:
+                    break
+                start[d] = item
+                stop[d] = item + 1
+            elif kind is slice:
+                st = item.step
+                if st is not None and not (type(st) is int and st > 0):
+                    break
                 start[d], stop[d], step[d] = item.indices(shape[d])
-            elif type(item) is int and -shape[d] <= item < shape[d]:
-                i = item + shape[d] if item < 0 else item
-                start[d], stop[d] = i, i + 1
             else:
                 break
+            d += 1
         else:
             return tuple(start), tuple(stop), tuple(step)
-        start, stop, step = [0] * ndims, [0] * ndims, [1] * ndims
+    start, stop, step = [0] * ndims, [0] * ndims, [1] * ndims
     for d, item in enumerate(_expand_key(key, ndims)):
         if isinstance(item, slice):
             st = 1 if item.step is None else int(item.step)
@@ -249,8 +262,8 @@ class _ArrayLike:
         raise TypeError("charmnumeric arrays are lazy frontend objects. "
                         "Call .get(interface) before converting to numpy.")
 
-    # -- operand form --
-    def _ref(self, broadcast=False):
+    # -- operand form: the bytes that name this object in a record of the statement log --
+    def _refb(self, broadcast=False):
         raise NotImplementedError
 
     def _base(self):
@@ -297,11 +310,10 @@ class _ArrayLike:
                         and _is_whole(value._region(), value._base().shape)):
                     raise ValueError(
                         f"could not broadcast input from shape {value.shape} into shape {shape}")
-            operand = value._ref()
+            operand = value._refb()
         else:
-            operand = value
-        whole = lazy.ArrayRef(base.name, None, base.shape, base.ndims, base._wire)
-        lazy.record(lazy.Instr("set", base.name, None, [operand], shape, base._wire, region, whole))
+            operand = lazy.scalar_bytes(value)
+        lazy.record_set(base.name, base._wire, base.ndims, shape, region, operand)
 
     # -- arithmetic --
     def __add__(self, o):
@@ -345,8 +357,7 @@ class _ArrayLike:
         """A new array holding these values: one COPY node (upstream's opcode -5), which fuses like
         any element-wise operation, instead of a zero-filled array assigned afterwards."""
         out = Array(self.shape, self.dtype)
-        lazy.record(lazy.Instr("op", name=out.name, opcode=L.OP_COPY, operands=[self._ref()],
-                               shape=self.shape, dtype=out.wire_dtype()))
+        lazy.record_op(out.name, L.OP_COPY, out._wire, out.shape, self._refb())
         return out
 
     def fill(self, value):
@@ -370,6 +381,7 @@ class Array(_ArrayLike):
         self._n = _size(self.shape)
         self.name = lazy.new_name() if name is None else name
         self._gen = lazy.generation()
+        self._rb = None
 
     @classmethod
     def _result_of(cls, like, shape):
@@ -383,6 +395,7 @@ class Array(_ArrayLike):
         out._n = like._n if shape is like.shape else _size(shape)
         out.name = lazy.new_name()
         out._gen = lazy.generation()
+        out._rb = None
         return out
 
     def __del__(self):
@@ -397,8 +410,13 @@ class Array(_ArrayLike):
     def _region(self):
         return None
 
-    def _ref(self, broadcast=False):
-        return lazy.ArrayRef(self.name, None, self.shape, self.ndims, self._wire, broadcast)
+    def _refb(self, broadcast=False):
+        if broadcast:
+            return lazy.ref_bytes(self.name, self.ndims, self._wire, None, True)
+        rb = self._rb
+        if rb is None:
+            rb = self._rb = lazy.ref_bytes(self.name, self.ndims, self._wire, None)
+        return rb
 
     def get(self, interface):
         lazy.execute(interface)
@@ -420,6 +438,7 @@ class ArrayView(_ArrayLike):
         for extent in shape:
             n *= extent
         self._n = n
+        self._rb = None
         if n == 0:
             raise NotImplementedError("zero-sized slices are not supported")
 
@@ -436,10 +455,15 @@ class ArrayView(_ArrayLike):
     def _region(self):
         return self.region
 
-    def _ref(self, broadcast=False):
-        base = self.base
-        region = None if self._n == base._n and _is_whole(self.region, base.shape) else self.region
-        return lazy.ArrayRef(base.name, region, self.shape, base.ndims, self._wire, broadcast)
+    def _refb(self, broadcast=False):
+        rb = self._rb
+        if rb is None or broadcast:
+            base = self.base
+            region = None if self._n == base._n and _is_whole(self.region, base.shape) else self.region
+            rb = lazy.ref_bytes(base.name, base.ndims, self._wire, region, broadcast)
+            if not broadcast:
+                self._rb = rb
+        return rb
 
     def get(self, interface):
         out = empty(self.shape, dtype=self.dtype)
@@ -490,15 +514,15 @@ def _binary(opcode, lhs, rhs):
         for x, bc in ((lhs, lb), (rhs, rb)):
             if bc and not _is_whole(x._region(), x._base().shape):
                 raise NotImplementedError("a one-element slice cannot be used as a scalar operand")
-        operands = [lhs._ref(lb), rhs._ref(rb)]
+        a, b = lhs._refb(lb), rhs._refb(rb)
     elif la:
         like = lhs
-        operands = [lhs._ref(), rhs]
+        a, b = lhs._refb(), lazy.scalar_bytes(rhs)
     else:
         like = rhs
-        operands = [lhs, rhs._ref()]
+        a, b = lazy.scalar_bytes(lhs), rhs._refb()
     out = Array._result_of(like, like.shape)
-    lazy.record(lazy.Instr("op", out.name, opcode, operands, out.shape, out._wire))
+    lazy.record_op(out.name, opcode, out._wire, out.shape, a, b)
     return out
 
 
@@ -508,7 +532,7 @@ def unary(opcode, x):
     if x._wire > L.F64:                    # the two integer types follow the floating-point ones
         raise TypeError("tanh/exp need a floating-point array")
     out = Array._result_of(x, x.shape)
-    lazy.record(lazy.Instr("op", out.name, opcode, [x._ref()], out.shape, out._wire))
+    lazy.record_op(out.name, opcode, out._wire, out.shape, x._refb())
     return out
 
 
@@ -540,9 +564,8 @@ def nonfusible(opcode, operands, shape, dtype):
     operands = [_whole(o) if isinstance(o, _ArrayLike) and not (opcode in _WINDOWED and _window_ok(o))
                 else o for o in operands]
     out = Array(shape, dtype)
-    lazy.record(lazy.Instr("nonfusible", name=out.name, opcode=opcode,
-                           operands=[o._ref() if isinstance(o, _ArrayLike) else o for o in operands],
-                           shape=shape, dtype=out.wire_dtype()))
+    lazy.record_nonfusible(out.name, opcode, out._wire, out.shape,
+                           [o._refb() if isinstance(o, _ArrayLike) else lazy.scalar_bytes(o) for o in operands])
     return out
 
 
@@ -679,7 +702,7 @@ class _HostValues:
 
 def create_array(shape, dtype=_DEFAULT_DTYPE):
     out = Array(_normalize_shape(shape), _normalize_dtype(dtype))
-    lazy.record(lazy.Instr("create", name=out.name, shape=out.shape, dtype=out.wire_dtype()))
+    lazy.record_create(out.name, out._wire, out.shape)
     return out
 
 
@@ -695,8 +718,8 @@ def _assign_host_data(target, values):
     if same is not None:
         target[...] = _coerce_scalar(same)
     else:
-        lazy.record(lazy.Instr("call", name=target.name, opcode="put", shape=target.shape,
-                               dtype=target.wire_dtype(), payload=np.ascontiguousarray(src.data).copy()))
+        lazy.record_call(lazy.Call(target.name, "put", target.wire_dtype(),
+                                   np.ascontiguousarray(src.data).copy()))
     return target
 
 

@@ -5,6 +5,7 @@
 #include "../../include/cnexec.h"
 #include "common.h"
 #include "decomp.h"
+#include "stmtlog.h"
 
 #include <algorithm>
 #include <array>
@@ -183,7 +184,19 @@ struct cnx_executor {
     std::thread worker;
     std::mutex qmu;
     std::condition_variable qcv, idle_cv;
-    std::deque<std::vector<char>> queue;
+    struct Queued {
+        std::vector<char> bytes;
+        bool is_log = false;   // a statement log (to be planned first) rather than a DAG message
+        int window = -1;
+    };
+    std::deque<Queued> queue;
+    // Statement log: what an automatic flush held back waits here, as parsed records, for the
+    // next stretch of the log. Names above every array name for the SET_REGION roots the planner
+    // makes. With capture on, every planned message is also kept as bytes (tests compare them).
+    std::vector<stmtlog::Instr> plog;
+    int32_t next_set_name = 1 << 30;
+    bool capture_on = false;
+    std::vector<char> captured;
     int deferred_rc = 0;
     std::string deferred_msg;
 
@@ -2194,13 +2207,52 @@ int run_nodes(Ex* ex, std::vector<DagNode>& dag) {
     return rc;
 }
 
-int run_message(Ex* ex, const char* msg, int64_t size) {
-    std::vector<DagNode> dag, fresh;
-    dag.swap(ex->held);                 // what the previous message left open comes first
-    if (int rc = parse_dag(msg, size, fresh))
-        return rc;
+// Runs freshly arrived nodes behind what the previous message left open.
+int run_fresh(Ex* ex, std::vector<DagNode>& fresh) {
+    std::vector<DagNode> dag;
+    dag.swap(ex->held);
     dag.insert(dag.end(), std::make_move_iterator(fresh.begin()), std::make_move_iterator(fresh.end()));
     return run_nodes(ex, dag);
+}
+
+int run_message(Ex* ex, const char* msg, int64_t size) {
+    std::vector<DagNode> fresh;
+    if (int rc = parse_dag(msg, size, fresh))
+        return rc;
+    return run_fresh(ex, fresh);
+}
+
+// A stretch of the statement log: appended to what an earlier automatic flush held back, planned
+// up to the hold-back cut (window >= 0) or to the end (window < 0), and run.
+int run_log(Ex* ex, const char* log, int64_t size, int window) {
+    if (int rc = stmtlog::parse(log, size, ex->plog)) {
+        ex->plog.clear();
+        return rc;
+    }
+    if (ex->plog.empty())
+        return 0;
+    const size_t cut = window >= 0 ? stmtlog::hold_back_cut(ex->plog, window) : ex->plog.size();
+    std::set<int32_t> dead, fused_away;
+    if (cut < ex->plog.size())
+        dead = stmtlog::dead_later(ex->plog, cut);
+    std::vector<DagNode> fresh;
+    stmtlog::plan(ex->plog, cut, dead, &ex->next_set_name, fresh, &fused_away);
+    // what stays behind; deletions of results that never became arrays have nothing to delete
+    std::vector<stmtlog::Instr> tail;
+    for (size_t i = cut; i < ex->plog.size(); ++i)
+        if (!(ex->plog[i].kind == stmtlog::kDelete && fused_away.count(ex->plog[i].name)))
+            tail.push_back(ex->plog[i]);
+    ex->plog.swap(tail);
+    if (ex->capture_on) {
+        const std::vector<char> bytes = stmtlog::to_message(fresh);
+        const int64_t len = (int64_t)bytes.size();
+        const char* lp = reinterpret_cast<const char*>(&len);
+        ex->captured.insert(ex->captured.end(), lp, lp + 8);
+        ex->captured.insert(ex->captured.end(), bytes.begin(), bytes.end());
+    }
+    if (fresh.empty())
+        return 0;
+    return run_fresh(ex, fresh);
 }
 
 // Executes whatever waits in `held`, to the end.
@@ -2223,7 +2275,7 @@ void worker_loop(Ex* ex) {
         ex->qcv.wait(lk, [&] { return ex->stop || !ex->queue.empty(); });
         if (ex->queue.empty())
             return;   // stop requested and nothing left
-        std::vector<char> msg = std::move(ex->queue.front());
+        Ex::Queued msg = std::move(ex->queue.front());
         ex->queue.pop_front();
         if (ex->deferred_rc != 0) {   // work behind a failed message is dropped
             if (ex->queue.empty())
@@ -2232,7 +2284,8 @@ void worker_loop(Ex* ex) {
         }
         ex->busy = true;
         lk.unlock();
-        const int rc = run_message(ex, msg.data(), (int64_t)msg.size());
+        const int rc = msg.is_log ? run_log(ex, msg.bytes.data(), (int64_t)msg.bytes.size(), msg.window)
+                                  : run_message(ex, msg.bytes.data(), (int64_t)msg.bytes.size());
         std::string text = rc ? cnh_last_error() : "";
         lk.lock();
         ex->busy = false;
@@ -2256,6 +2309,7 @@ int drain(Ex* ex) {
             ex->deferred_rc = 0;
             ex->deferred_msg.clear();
             ex->held.clear();           // work behind a failed message is dropped
+            ex->plog.clear();
             lk.unlock();
             return set_error(rc, "%s", text.c_str());
         }
@@ -2383,12 +2437,61 @@ int cnx_receive_dag(cnx_executor* ex, int epoch, int64_t size, const char* msg) 
     {
         std::unique_lock<std::mutex> lk(ex->qmu);
         if (ex->deferred_rc == 0) {
-            ex->queue.emplace_back(msg, msg + size);
+            ex->queue.emplace_back();
+            ex->queue.back().bytes.assign(msg, msg + size);
             ex->qcv.notify_one();
             return 0;
         }
     }
     return drain(ex);   // an earlier message failed: report that instead of queueing more
+}
+
+int cnx_receive_log(cnx_executor* ex, int64_t size, const char* log, int hold_back_window) {
+    CNH_CHECK(ex != nullptr && size >= 0 && (log != nullptr || size == 0), -2, "bad statement log");
+    if (!ex->async_on)
+        return run_log(ex, log, size, hold_back_window);
+    {
+        std::unique_lock<std::mutex> lk(ex->qmu);
+        if (ex->deferred_rc == 0) {
+            ex->queue.emplace_back();
+            if (size > 0)
+                ex->queue.back().bytes.assign(log, log + size);
+            ex->queue.back().is_log = true;
+            ex->queue.back().window = hold_back_window;
+            ex->qcv.notify_one();
+            return 0;
+        }
+    }
+    return drain(ex);
+}
+
+int cnx_discard_log(cnx_executor* ex) {
+    CNH_CHECK(ex != nullptr, -2, "null executor");
+    const int rc = drain(ex);
+    ex->plog.clear();
+    return rc;
+}
+
+int cnx_set_capture(cnx_executor* ex, int on) {
+    CNH_CHECK(ex != nullptr, -2, "null executor");
+    const int rc = drain(ex);
+    ex->capture_on = on != 0;
+    ex->captured.clear();
+    return rc;
+}
+
+int64_t cnx_captured(cnx_executor* ex, char* buf, size_t cap) {
+    if (ex == nullptr)
+        return -2;
+    if (int rc = drain(ex))
+        return rc;
+    const size_t need = ex->captured.size();
+    if (buf != nullptr && cap >= need) {
+        if (need)
+            std::memcpy(buf, ex->captured.data(), need);
+        ex->captured.clear();
+    }
+    return (int64_t)need;
 }
 
 int cnx_set_async(cnx_executor* ex, int on) {

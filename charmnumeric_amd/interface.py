@@ -116,6 +116,35 @@ class CharmNumericInterface:
     def send_dag(self, epoch, message):
         L.check(L.lib.cnx_receive_dag(self._handle(), int(epoch), len(message), message))
 
+    def send_log(self, log, hold_back_window=-1):
+        """A stretch of the statement log (lazy.py records it; format: include/cnexec.h). The
+        executor plans it into DAG nodes and runs them; a window >= 0 marks an automatic flush, which
+        may leave the most recent statements unplanned until the next call."""
+        L.check(L.lib.cnx_receive_log(self._handle(), len(log), log, int(hold_back_window)))
+
+    def discard_log(self):
+        """Drops what automatic flushes left unplanned in the executor (the frontend was reset)."""
+        if self._ex is not None:
+            L.check(L.lib.cnx_discard_log(self._ex))
+
+    def set_capture(self, on=True):
+        """Test hook: keep the DAG messages planned from the log; captured() returns and clears them."""
+        L.check(L.lib.cnx_set_capture(self._handle(), 1 if on else 0))
+
+    def captured(self):
+        ex = self._handle()
+        need = L.lib.cnx_captured(ex, None, 0)
+        if need < 0:
+            L.check(int(need))
+        buf = C.create_string_buffer(max(1, int(need)))
+        L.lib.cnx_captured(ex, buf, int(need))
+        raw, out, pos = buf.raw[:int(need)], [], 0
+        while pos < len(raw):
+            size = int.from_bytes(raw[pos:pos + 8], "little")
+            out.append(raw[pos + 8:pos + 8 + size])
+            pos += 8 + size
+        return out
+
     def direct_call(self, instr):
         ex = self._handle()
         if instr.opcode == "put":

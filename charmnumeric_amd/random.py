@@ -16,8 +16,8 @@ def uniform(shape, seed, stream=0, low=0.0, high=1.0):
     """fp64 array with element i (row-major) = low + (high-low)*u01(seed, stream, i), from the
     counter-based SplitMix64 generator the tests restate in NumPy."""
     out = create_array(shape, dtype="float64")
-    lazy.record(lazy.Instr("call", name=out.name, opcode="fill_uniform", shape=out.shape,
-                           dtype=out.wire_dtype(), payload=(int(seed), int(stream), float(low), float(high))))
+    lazy.record_call(lazy.Call(out.name, "fill_uniform", out.wire_dtype(),
+                               (int(seed), int(stream), float(low), float(high))))
     return out
 
 
@@ -25,6 +25,5 @@ def cg_matrix(n, seed):
     """The dense symmetric test matrix of the CG workload: diagonal 2.0, off-diagonal
     (u01(seed,0,i*n+j) + u01(seed,0,j*n+i)) / (2n)."""
     out = create_array((int(n), int(n)), dtype="float64")
-    lazy.record(lazy.Instr("call", name=out.name, opcode="fill_cg_matrix", shape=out.shape,
-                           dtype=out.wire_dtype(), payload=(int(seed),)))
+    lazy.record_call(lazy.Call(out.name, "fill_cg_matrix", out.wire_dtype(), (int(seed),)))
     return out

@@ -110,6 +110,34 @@ int cnx_receive_dag(cnx_executor* ex, int epoch, int64_t size, const char* msg);
  * error code and text are returned by the next call on the executor, whichever it is. */
 int cnx_set_async(cnx_executor* ex, int on);
 
+/* The statement log: the frontend's recording, shipped raw. Upstream's frontend groups what it
+ * recorded into DAG nodes itself (charmtyles, outside the charmnumeric tree) and sends the result to
+ * receive_dag; with this entry point the grouping (which element-wise operations fuse, which
+ * results never become arrays, which deletions have nothing to delete) runs inside the executor, on
+ * its own thread in asynchronous mode, and the nodes it makes run exactly as if they had arrived
+ * through cnx_receive_dag. Records (little endian, int32 words unless noted):
+ *   delete      := 5, name
+ *   create      := head, shape                                   kind 1
+ *   op          := head, shape, operand * n_operands             kind 2, element-wise, <= 2 operands
+ *   set         := head, shape, region, operand                  kind 3, target[region] = operand
+ *   nonfusible  := head, shape, operand * n_operands             kind 4: reductions, products, ...
+ *   head        := kind, name, opcode, dtype, n_operands, aux    aux: rank of the target (set), else 0
+ *   shape       := ndims, extent[3]                              of the result / the assigned region
+ *   region      := ndims, start[3], stop[3], step[3]
+ *   operand     := 0, 0, float64 value
+ *                | 1, name, base_ndims, dtype, broadcast, has_region, start[3], stop[3], step[3]
+ * hold_back_window < 0: everything recorded so far is planned and run. >= 0 (an automatic flush in
+ * the middle of a program): statements from the one that produced a still-live result within the
+ * last `window` records onwards stay in the executor until the next call, so that a result whose
+ * handle is about to go away is not turned into an array just because the flush fell there. */
+int cnx_receive_log(cnx_executor* ex, int64_t size, const char* log, int hold_back_window);
+/* Forgets the part of the log an automatic flush held back (the frontend's reset()). */
+int cnx_discard_log(cnx_executor* ex);
+/* Test hook: with capture on, every DAG message planned from the log is also kept as bytes, each
+ * preceded by its int64 length; cnx_captured copies them out as cnx_trace does and clears them. */
+int cnx_set_capture(cnx_executor* ex, int on);
+int64_t cnx_captured(cnx_executor* ex, char* buf, size_t cap);
+
 /* receive_get_request(int ndims, int epoch, int name, int size, int dtype) + gather + reply
  * (src/backend.ci:16-17, src/partition_get.cpp:4-67, src/dag_group_runtime.cpp:55-118): copies
  * array `name` into host_out as one global row-major array of `size` elements. Blocks. */
