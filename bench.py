@@ -29,8 +29,8 @@ HBM_PEAK_GBS = 8000.0
 FP64_MFMA_PEAK_TFLOPS = 78.6
 # HBM bytes per launch of the tiled matvec at n = 16384, from rocprofv3 FETCH_SIZE (x 2.0, the
 # factor a plain streaming kernel of known size gives on gfx950) + WRITE_SIZE (x 1.0):
-# (2 098 220 + 128.3) KiB, see profiles/bench_hbm_traffic_pmc.txt.
-GEMV_N16384_TRAFFIC_BYTES = 2148708659
+# (2 098 218 + 128.3) KiB, see profiles/bench_hbm_traffic_pmc.txt.
+GEMV_N16384_TRAFFIC_BYTES = 2148706611
 
 
 def _dev():
