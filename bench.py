@@ -102,22 +102,55 @@ def _launch1(L, k, nd, ins, scalars, outs, stream=None):
 # C2: dense CG, n = 16384
 # -------------------------------------------------------------------------------------------------
 def cg_asts(L):
+    """The element-wise part of one CG iteration as two groups. The scalar statements
+    (alpha = r.r / p.Ap, beta = r.r_new / r.r) are formed in registers by the group that uses them,
+    from the two reduction results it reads as run-time scalars, so an iteration is five launches
+    (matvec, dot, x and r together, dot, p) instead of eight.
+    Group 1 (leaves 1 = p, 2 = x, 3 = Ap, 4 = r; scalars 5 = r.r, 6 = p.Ap):
+        7 = x + alpha p, 8 = r - alpha Ap.   Group 2 (leaves 1 = p, 2 = r_new; scalars 5 = r.r_new,
+    6 = r.r): 7 = r_new + beta p."""
     from charmnumeric_amd.astbuild import AstBuilder
 
-    def scalar_div():
+    def update_x_r():
         b = AstBuilder(L.F64, 1)
-        b.binary(L.OP_DIV, 3, b.broadcast(1), b.broadcast(2), is_temp=False)
+        alpha = b.binary(L.OP_DIV, 100, b.broadcast(5), b.broadcast(6))
+        t1 = b.binary(L.OP_MUL, 101, alpha, b.leaf(1))
+        b.binary(L.OP_ADD, 7, b.leaf(2), t1, is_temp=False)
+        t2 = b.binary(L.OP_MUL, 102, alpha, b.leaf(3))
+        b.binary(L.OP_SUB, 8, b.leaf(4), t2, is_temp=False)
         return b.finish()
 
-    def axpy(op):
-        # out = u (op) s * v; leaf uses are collected root by root, so the memref order is (v, u)
+    def update_p():
         b = AstBuilder(L.F64, 1)
-        u, v = b.leaf(1), b.leaf(2)
-        t = b.binary(L.OP_MUL, 100, b.broadcast(3), v)
-        b.binary(op, 4, u, t, is_temp=False)
+        beta = b.binary(L.OP_DIV, 100, b.broadcast(5), b.broadcast(6))
+        t = b.binary(L.OP_MUL, 101, beta, b.leaf(1))
+        b.binary(L.OP_ADD, 7, b.leaf(2), t, is_temp=False)
         return b.finish()
 
-    return scalar_div(), axpy(L.OP_ADD), axpy(L.OP_SUB)
+    return update_x_r(), update_p()
+
+
+def prepare_launch(L, k, nd, ins, scalars, outs, stream=None):
+    """A launch of group kernel `k` over one partition, put together once: memrefs by leaf name,
+    device addresses of run-time scalars by name, memrefs by output name. Returns what fires it."""
+    n_in, n_sc, n_out = C.c_int(), C.c_int(), C.c_int()
+    L.check(L.lib.cnh_kernel_signature(k, C.byref(n_in), C.byref(n_sc), C.byref(n_out)))
+    name, has, tgt, sr = C.c_int(), C.c_int(), C.c_int(), C.c_int()
+    reg = L.Region()
+    ia = (L.Memref * max(1, n_in.value))()
+    oa = (L.Memref * max(1, n_out.value))()
+    sp = (C.c_void_p * max(1, n_sc.value))()
+    for i in range(n_in.value):
+        L.check(L.lib.cnh_kernel_input(k, i, C.byref(name), C.byref(has), C.byref(reg)))
+        ia[i] = ins[name.value]
+    for i in range(n_sc.value):
+        L.check(L.lib.cnh_kernel_scalar(k, i, C.byref(name)))
+        sp[i] = scalars[name.value]
+    for i in range(n_out.value):
+        L.check(L.lib.cnh_kernel_output(k, i, C.byref(name), C.byref(tgt), C.byref(sr), C.byref(reg)))
+        oa[i] = outs[name.value]
+    n_i, n_s, n_o = n_in.value, n_sc.value, n_out.value
+    return lambda: L.check(L.lib.cnh_launch_group(k, nd, n_i, ia, n_s, sp, 1, n_o, oa, stream))
 
 
 def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True, trace_iters=0):
@@ -139,41 +172,48 @@ def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True, trace_i
     bvec, x, r, p, Ap = vec(), vec(), vec(), vec(), vec()
     x2, r2, p2 = vec(), vec(), vec()
     L.check(L.lib.cnh_fill_uniform(bvec.ptr, n, seed, 1, 0, -1.0, 1.0, None))
-    sc = Buf(L, 8 * 8, zero=True)  # rtr, pAp, alpha, rtr_new, beta
+    sc = Buf(L, 8 * 8, zero=True)  # slot 0 / 3: r.r of the current / next iterate (swapping), 1: p.Ap
     S = lambda i: sc.ptr + 8 * i
-    ast_div, ast_add, ast_sub = cg_asts(L)
-    k_div, k_add, k_sub = (_compile(L, a, L.F64, 1) for a in (ast_div, ast_add, ast_sub))
+    k_xr, k_p = (_compile(L, a, L.F64, 1) for a in cg_asts(L))
     mr = lambda b_, cnt=n: L.Memref.dense(b_.ptr, (cnt,))
-    smr = lambda i: L.Memref.dense(S(i), (1,))
 
-    state = {}
+    # Vectors ping-pong between two buffers and r.r between two slots: an iteration's launches exist
+    # in two prepared forms, for even and odd iterations.
+    bufs = [{"x": x, "r": r, "p": p, "rtr": 0}, {"x": x2, "r": r2, "p": p2, "rtr": 3}]
+    forms = []
+    for cur, nxt in ((bufs[0], bufs[1]), (bufs[1], bufs[0])):
+        forms.append({
+            "p": cur["p"], "x_new": nxt["x"], "rtr": cur["rtr"], "rtr_new": nxt["rtr"], "r_new": nxt["r"],
+            "update_x_r": prepare_launch(L, k_xr, 1, {1: mr(cur["p"]), 2: mr(cur["x"]), 3: mr(Ap), 4: mr(cur["r"])},
+                                         {5: S(cur["rtr"]), 6: S(1)}, {7: mr(nxt["x"]), 8: mr(nxt["r"])}),
+            "update_p": prepare_launch(L, k_p, 1, {1: mr(cur["p"]), 2: mr(nxt["r"])},
+                                       {5: S(nxt["rtr"]), 6: S(cur["rtr"])}, {7: mr(nxt["p"])}),
+        })
+    state = {"parity": 0}
 
     def reset():
         # x = 0, r = p = b, r.r; the ping-pong roles go back to their starting assignment too
-        state.update({"x": x, "r": r, "p": p, "x2": x2, "r2": r2, "p2": p2, "rtr": 0, "rtr_new": 3})
+        state["parity"] = 0
         L.check(L.lib.cnh_memset0(x.ptr, n * 8, None))
         L.check(L.lib.cnh_d2d(r.ptr, bvec.ptr, n * 8, None))
         L.check(L.lib.cnh_d2d(p.ptr, bvec.ptr, n * 8, None))
         L.check(L.lib.cnh_dot_partial(L.F64, n, r.ptr, r.ptr, S(0), None))
 
     def iteration(ev=None, i=0):
-        st = state
+        f = forms[state["parity"]]
         if ev is not None:
             L.check(L.lib.cnh_event_record(ev.a[i], None))
-        L.check(L.lib.cnh_gemv_tiles(L.F64, n, n, tile, tptr, st["p"].ptr, Ap.ptr, None))
+        L.check(L.lib.cnh_gemv_tiles(L.F64, n, n, tile, tptr, f["p"].ptr, Ap.ptr, None))
         if ev is not None:
             L.check(L.lib.cnh_event_record(ev.b[i], None))
-        L.check(L.lib.cnh_dot_partial(L.F64, n, st["p"].ptr, Ap.ptr, S(1), None))
-        _launch1(L, k_div, 1, [], [S(st["rtr"]), S(1)], [smr(2)])                       # alpha
-        _launch1(L, k_add, 1, [mr(st["p"]), mr(st["x"])], [S(2)], [mr(st["x2"])])      # x + alpha p
-        _launch1(L, k_sub, 1, [mr(Ap), mr(st["r"])], [S(2)], [mr(st["r2"])])           # r - alpha Ap
-        L.check(L.lib.cnh_dot_partial(L.F64, n, st["r2"].ptr, st["r2"].ptr, S(st["rtr_new"]), None))
-        _launch1(L, k_div, 1, [], [S(st["rtr_new"]), S(st["rtr"])], [smr(4)])           # beta
-        _launch1(L, k_add, 1, [mr(st["p"]), mr(st["r2"])], [S(4)], [mr(st["p2"])])     # r + beta p
-        st["x"], st["x2"] = st["x2"], st["x"]
-        st["r"], st["r2"] = st["r2"], st["r"]
-        st["p"], st["p2"] = st["p2"], st["p"]
-        st["rtr"], st["rtr_new"] = st["rtr_new"], st["rtr"]
+        L.check(L.lib.cnh_dot_partial(L.F64, n, f["p"].ptr, Ap.ptr, S(1), None))
+        f["update_x_r"]()                      # x + alpha p, r - alpha Ap
+        L.check(L.lib.cnh_dot_partial(L.F64, n, f["r_new"].ptr, f["r_new"].ptr, S(f["rtr_new"]), None))
+        f["update_p"]()                        # r_new + beta p
+        state["parity"] ^= 1
+
+    def current():
+        return bufs[state["parity"]]
 
     reset()
     for _ in range(warmup):
@@ -186,12 +226,16 @@ def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True, trace_i
         reset()
         trace = {"alpha": [], "beta": [], "rtr": []}
         for _ in range(trace_iters):
+            before = current()["rtr"]
             iteration()
             v = sc.get(np.float64)           # waits for the iteration
-            trace["alpha"].append(float(v[2]))
-            trace["beta"].append(float(v[4]))
-            trace["rtr"].append(float(v[state["rtr"]]))
-        trace["x"] = state["x"].get()
+            after = current()["rtr"]
+            # alpha and beta exist in registers only; the same two divisions on the host, from the
+            # reduction results the device used (IEEE division: the same bits)
+            trace["alpha"].append(float(v[before] / v[1]))
+            trace["beta"].append(float(v[after] / v[before]))
+            trace["rtr"].append(float(v[after]))
+        trace["x"] = current()["x"].get()
 
     reset()
     ev = Events(L, steps)
@@ -214,8 +258,8 @@ def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True, trace_i
         "ms_per_step": wall * 1e3 / steps, "iters_per_s": steps / wall,
         "gemv_avg_us": 1e3 * float(np.mean(gemv_ms)), "gemv_min_us": 1e3 * float(np.min(gemv_ms)),
         "setup_s": setup_s,
-        "rtr_final": float(sc.get(np.float64)[state["rtr"]]),
-        "x": state["x"].get() if check else None,
+        "rtr_final": float(sc.get(np.float64)[current()["rtr"]]),
+        "x": current()["x"].get() if check else None,
         "trace": trace,
     }
     ev.free()
@@ -674,23 +718,6 @@ def lstm_fused_ast(L, first):
     return b.finish()
 
 
-def _launch_named(L, k, nd, ins, outs, stream=None):
-    """One partition; memrefs given by leaf name and by output name."""
-    n_in, n_sc, n_out = C.c_int(), C.c_int(), C.c_int()
-    L.check(L.lib.cnh_kernel_signature(k, C.byref(n_in), C.byref(n_sc), C.byref(n_out)))
-    name, has, tgt, sr = C.c_int(), C.c_int(), C.c_int(), C.c_int()
-    reg = L.Region()
-    ia = (L.Memref * max(1, n_in.value))()
-    oa = (L.Memref * max(1, n_out.value))()
-    for i in range(n_in.value):
-        L.check(L.lib.cnh_kernel_input(k, i, C.byref(name), C.byref(has), C.byref(reg)))
-        ia[i] = ins[name.value]
-    for i in range(n_out.value):
-        L.check(L.lib.cnh_kernel_output(k, i, C.byref(name), C.byref(tgt), C.byref(sr), C.byref(reg)))
-        oa[i] = outs[name.value]
-    L.check(L.lib.cnh_launch_group(k, nd, n_in.value, ia, 0, None, 1, n_out.value, oa, stream))
-
-
 def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=False, fused=True):
     k_in = nin + d
     X = Buf(L, steps * batch * nin * 8)
@@ -729,33 +756,53 @@ def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=
         return L.Memref.strided(base, (batch, ncols), (row_len, 1))
 
     ev = Events(L, steps)
-    evs = Events(L, steps)
-    jobs = (L.GemmJob * 1)()
+    stream = C.c_void_p()
+    L.check(L.lib.cnh_stream_create(C.byref(stream)))
 
-    def gate_product(t):
+    # Everything a step launches is put together before the clock starts (descriptor tables,
+    # memrefs by leaf name): the timed loop only fires prepared launches, as a compiled caller would.
+    def prepared_group(k, nd, ins, outs):
+        n_in, n_sc, n_out = C.c_int(), C.c_int(), C.c_int()
+        L.check(L.lib.cnh_kernel_signature(k, C.byref(n_in), C.byref(n_sc), C.byref(n_out)))
+        name, has, tgt, sr = C.c_int(), C.c_int(), C.c_int(), C.c_int()
+        reg = L.Region()
+        ia = (L.Memref * max(1, n_in.value))()
+        oa = (L.Memref * max(1, n_out.value))()
+        for i in range(n_in.value):
+            L.check(L.lib.cnh_kernel_input(k, i, C.byref(name), C.byref(has), C.byref(reg)))
+            ia[i] = ins[name.value]
+        for i in range(n_out.value):
+            L.check(L.lib.cnh_kernel_output(k, i, C.byref(name), C.byref(tgt), C.byref(sr), C.byref(reg)))
+            oa[i] = outs[name.value]
+        return lambda: L.check(L.lib.cnh_launch_group(k, nd, n_in.value, ia, 0, None, 1, n_out.value, oa, stream))
+
+    def prepared1(k, nd, ins, outs):
+        ia = (L.Memref * max(1, len(ins)))(*ins)
+        oa = (L.Memref * max(1, len(outs)))(*outs)
+        return lambda: L.check(L.lib.cnh_launch_group(k, nd, len(ins), ia, 0, None, 1, len(outs), oa, stream))
+
+    def prepared_copy(dst, dst_strides, src, src_strides, extent):
+        args = (2, 8, dst, i64(dst_strides), zero2, one, src, i64(src_strides), zero2, one, i64(extent), stream)
+        return lambda: L.check(L.lib.cnh_copy_region(*args))
+
+    def prepared_product(t):
         # IFOG[t] = Hin[t] @ W, written without reading what IFOG[t] held
+        jobs = (L.GemmJob * 1)()
         jobs[0].M, jobs[0].N, jobs[0].K = batch, 4 * d, k_in
         jobs[0].A, jobs[0].lda = Hin.ptr + t * batch * k_in * 8, k_in
         jobs[0].B, jobs[0].ldb = W.ptr, 4 * d
         jobs[0].C, jobs[0].ldc = IFOG.ptr + t * batch * 4 * d * 8, 4 * d
-        L.check(L.lib.cnh_gemm_batch(L.F64, 1, jobs, 1, None))
+        return lambda: L.check(L.lib.cnh_gemm_batch(L.F64, 1, jobs, 1, stream))
 
-    def step(t, record):
-        if record:
-            L.check(L.lib.cnh_event_record(evs.a[t], None))
+    def prepare(t):
+        """(what runs before the product, the product, what runs after it) of step t."""
         # Hin[t, :, :nin] = X[t]; Hin[t, :, nin:] = Hout[t-1] (h0 = 0 at t = 0)
-        L.check(L.lib.cnh_copy_region(2, 8, Hin.ptr + t * batch * k_in * 8, i64([k_in, 1]), zero2, one,
-                                      X.ptr + t * batch * nin * 8, i64([nin, 1]), zero2, one,
-                                      i64([batch, nin]), None))
+        before = [prepared_copy(Hin.ptr + t * batch * k_in * 8, [k_in, 1], X.ptr + t * batch * nin * 8,
+                                [nin, 1], [batch, nin])]
         if t > 0 and not fused:
-            L.check(L.lib.cnh_copy_region(2, 8, Hin.ptr + (t * batch * k_in + nin) * 8, i64([k_in, 1]),
-                                          zero2, one, Hout.ptr + (t - 1) * batch * d * 8, i64([d, 1]),
-                                          zero2, one, i64([batch, d]), None))
-        if record:
-            L.check(L.lib.cnh_event_record(ev.a[t], None))
-        gate_product(t)
-        if record:
-            L.check(L.lib.cnh_event_record(ev.b[t], None))
+            before.append(prepared_copy(Hin.ptr + (t * batch * k_in + nin) * 8, [k_in, 1],
+                                        Hout.ptr + (t - 1) * batch * d * 8, [d, 1], [batch, d]))
+        after = []
         if fused:
             # every gate statement of the step in one launch; h goes to Hout[t] and, for the next
             # step's product, to the right half of Hin[t+1]
@@ -768,32 +815,59 @@ def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=
             outs = {11: view(IFOGf, t, 4 * d, 0, d), 12: view(IFOGf, t, 4 * d, d, d),
                     13: view(IFOGf, t, 4 * d, 2 * d, d), 14: view(IFOGf, t, 4 * d, 3 * d, d),
                     15: view(Cc, t, d, 0, d), 16: view(Ct, t, d, 0, d), 17: view(Hout, t, d, 0, d), 18: nxt}
-            _launch_named(L, k_first if t == 0 else k_later, 2, ins, outs)
+            after.append(prepared_group(k_first if t == 0 else k_later, 2, ins, outs))
         else:
-            _launch1(L, k_sig, 2, [view(IFOG, t, 4 * d, 0, 3 * d)], [], [view(IFOGf, t, 4 * d, 0, 3 * d)])
-            _launch1(L, k_tanh, 2, [view(IFOG, t, 4 * d, 3 * d, d)], [], [view(IFOGf, t, 4 * d, 3 * d, d)])
-            _launch1(L, k_mul, 2, [view(IFOGf, t, 4 * d, 0, d), view(IFOGf, t, 4 * d, 3 * d, d)], [],
-                     [view(Cc, t, d, 0, d)])
+            after.append(prepared1(k_sig, 2, [view(IFOG, t, 4 * d, 0, 3 * d)], [view(IFOGf, t, 4 * d, 0, 3 * d)]))
+            after.append(prepared1(k_tanh, 2, [view(IFOG, t, 4 * d, 3 * d, d)], [view(IFOGf, t, 4 * d, 3 * d, d)]))
+            after.append(prepared1(k_mul, 2, [view(IFOGf, t, 4 * d, 0, d), view(IFOGf, t, 4 * d, 3 * d, d)],
+                                   [view(Cc, t, d, 0, d)]))
             if t > 0:
                 # leaf uses are collected root by root: (f, C[t-1]) of the product, then C[t]
-                _launch1(L, k_muladd, 2, [view(IFOGf, t, 4 * d, d, d), view(Cc, t - 1, d, 0, d),
-                                          view(Cc, t, d, 0, d)], [], [view(Cc, t, d, 0, d)])
-            _launch1(L, k_tanh, 2, [view(Cc, t, d, 0, d)], [], [view(Ct, t, d, 0, d)])
-            _launch1(L, k_mul, 2, [view(IFOGf, t, 4 * d, 2 * d, d), view(Ct, t, d, 0, d)], [],
-                     [view(Hout, t, d, 0, d)])
-        if record:
-            L.check(L.lib.cnh_event_record(evs.b[t], None))
+                after.append(prepared1(k_muladd, 2, [view(IFOGf, t, 4 * d, d, d), view(Cc, t - 1, d, 0, d),
+                                                     view(Cc, t, d, 0, d)], [view(Cc, t, d, 0, d)]))
+            after.append(prepared1(k_tanh, 2, [view(Cc, t, d, 0, d)], [view(Ct, t, d, 0, d)]))
+            after.append(prepared1(k_mul, 2, [view(IFOGf, t, 4 * d, 2 * d, d), view(Ct, t, d, 0, d)],
+                                   [view(Hout, t, d, 0, d)]))
+        return before, prepared_product(t), after
+
+    plan = [prepare(t) for t in range(steps)]
+    L.check(L.lib.cnh_device_sync())         # the fills above ran on the default stream
+
+    def run_steps(count, product_events):
+        for t in range(count):
+            before, product, after = plan[t]
+            for fire in before:
+                fire()
+            if product_events:
+                L.check(L.lib.cnh_event_record(ev.a[t], stream))
+            product()
+            if product_events:
+                L.check(L.lib.cnh_event_record(ev.b[t], stream))
+            for fire in after:
+                fire()
 
     out = {}
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    L.check(L.lib.cnh_event_create(C.byref(e0)))
+    L.check(L.lib.cnh_event_create(C.byref(e1)))
+    total_ms, wall = C.c_float(0.0), 0.0
     if timed:
-        for t in range(min(steps, 3)):   # warm-up (builds the kernels)
-            step(t, False)
-        L.check(L.lib.cnh_device_sync())
-    for t in range(steps):
-        step(t, True)
-    L.check(L.lib.cnh_device_sync())
+        run_steps(min(steps, 3), False)      # warm-up (builds the kernels)
+        L.check(L.lib.cnh_stream_sync(stream))
+    # one pass with an event pair around every product (the product's own duration) ...
+    run_steps(steps, True)
+    L.check(L.lib.cnh_stream_sync(stream))
     g = ev.times_ms(steps)
-    st = evs.times_ms(steps)
+    if timed:
+        # ... then the pass that is timed as a whole: one event pair around all steps, nothing
+        # between the launches
+        w0 = time.perf_counter()
+        L.check(L.lib.cnh_event_record(e0, stream))
+        run_steps(steps, False)
+        L.check(L.lib.cnh_event_record(e1, stream))
+        L.check(L.lib.cnh_stream_sync(stream))
+        wall = time.perf_counter() - w0
+        L.check(L.lib.cnh_event_elapsed_ms(e0, e1, C.byref(total_ms)))
     flop = 2.0 * batch * k_in * 4 * d
     gus = 1e3 * float(np.median(g))
     ceiling = C.c_double()
@@ -802,13 +876,16 @@ def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=
            "mfma_frac": round(flop / gus / 1e6 / FP64_MFMA_PEAK_TFLOPS, 4),
            "mfma_measured_ceiling_tflops": round(ceiling.value, 1),
            "mfma_frac_of_measured_ceiling": round(flop / gus / 1e6 / ceiling.value, 4) if ceiling.value else None,
-           "step_us": round(1e3 * float(np.median(st)), 2), "flop_per_step": flop}
+           "step_us": round(1e3 * total_ms.value / steps, 2), "step_wall_us": round(1e6 * wall / steps, 2),
+           "flop_per_step": flop}
     if keep:
         out["Hout"] = Hout.get().reshape(steps, batch, d)
         out["C"] = Cc.get().reshape(steps, batch, d)
         out["IFOG"] = IFOG.get().reshape(steps, batch, 4 * d)
     ev.free()
-    evs.free()
+    for e in (e0, e1):
+        L.lib.cnh_event_destroy(e)
+    L.check(L.lib.cnh_stream_destroy(stream))
     out["gate_launches_per_step"] = 1 if fused else 6
     for b_ in (X, W, Hin, IFOG, IFOGf, Cc, Ct, Hout, spare):
         b_.free()
