@@ -16,6 +16,7 @@ F32, F64, I32, I64 = 0, 1, 2, 3
 OP_COPY, OP_SET_REGION, OP_GET_REGION, OP_CREATE, OP_NOOP = -5, -4, -3, -2, -1
 OP_ADD, OP_SUB, OP_MUL, OP_DIV, OP_MATMUL, OP_TANH, OP_EXP = 0, 1, 2, 3, 4, 5, 6
 OP_TILE, OP_REDUCE, OP_MATMATMUL, OP_DIAG = 7, 8, 9, 10
+OP_SUM_OF, OP_MAXABS_OF = 20, 21          # reducing roots of a fused group (extension)
 
 
 class CnhError(RuntimeError):

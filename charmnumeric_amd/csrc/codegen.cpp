@@ -227,10 +227,14 @@ int build_group_program(const cnh_ast* ast, int dtype, int ndims, GroupProgram& 
                 err = "SET_REGION without a usable right-hand side";
                 return -10;
             }
-        } else if (opc == CNH_OP_COPY) {
+        } else if (opc == CNH_OP_COPY || opc == CNH_OP_SUM_OF || opc == CNH_OP_MAXABS_OF) {
             res = lookup(root, 0);
             if (!res.valid || res.scalar) {
-                err = "COPY needs an array operand";
+                err = "COPY and the reducing roots need an array operand";
+                return -12;
+            }
+            if (opc != CNH_OP_COPY && (root.is_temp || dtype != CNH_F64)) {
+                err = "a reducing root is an fp64 output of its group";
                 return -12;
             }
         } else if (opc >= CNH_OP_ADD && opc <= CNH_OP_DIV) {
@@ -280,6 +284,7 @@ int build_group_program(const cnh_ast* ast, int dtype, int ndims, GroupProgram& 
         p.out_names.push_back(root.result_name);
         bool sr = root.opcode == CNH_OP_SET_REGION;
         p.out_is_set_region.push_back(sr ? 1 : 0);
+        p.out_reduce.push_back(root.opcode == CNH_OP_SUM_OF ? 1 : root.opcode == CNH_OP_MAXABS_OF ? 2 : 0);
         int target = root.result_name;
         if (sr && root.n_operands > 0 && root.operands[0] >= 0)
             target = ast->nodes[root.operands[0]].result_name;
@@ -348,16 +353,54 @@ std::string flat_source(const GroupProgram& p) {
     std::ostringstream s;
     s << prelude(p);
     s << "#define VECW " << vec << "\n";
+    // Outputs that are reduced instead of stored: a mask over the output list, and the statement
+    // that folds one element's values into the lane's running results.
+    unsigned mask = 0;
+    int nred = 0;
+    std::ostringstream fold, init;
+    for (size_t j = 0; j < p.out_reduce.size(); ++j) {
+        if (!p.out_reduce[j])
+            continue;
+        mask |= 1u << j;
+        if (p.out_reduce[j] == 1)
+            fold << " racc[" << nred << "] += o[" << j << "];";
+        else
+            fold << " { const T a_ = o[" << j << "] < 0 ? -o[" << j << "] : o[" << j << "]; racc[" << nred
+                 << "] = a_ > racc[" << nred << "] ? a_ : racc[" << nred << "]; }";
+        ++nred;
+    }
+    s << "#define RED_MASK " << mask << "u\n#define NR " << nred << "\n#define NRA " << (nred ? nred : 1) << "\n";
+    s << "#define RED_FOLD(o, racc) do {" << fold.str() << " } while (0)\n";
+    std::ostringstream comb;
+    {
+        int q = 0;
+        for (size_t j = 0; j < p.out_reduce.size(); ++j) {
+            if (!p.out_reduce[j])
+                continue;
+            if (p.out_reduce[j] == 1)
+                comb << " racc[" << q << "] += other[" << q << "];";
+            else
+                comb << " racc[" << q << "] = other[" << q << "] > racc[" << q << "] ? other[" << q
+                     << "] : racc[" << q << "];";
+            ++q;
+        }
+    }
+    s << "#define RED_COMBINE(racc, other) do {" << comb.str() << " } while (0)\n";
     s << R"(
 // Contiguous segments: every memref of a partition is dense and has the same element count.
 // One 128-bit vector per lane and a grid that covers the data once: on this part the plain form
 // streams faster than unrolled or persistent ones. NT selects non-temporal loads and stores for
 // launches whose traffic exceeds what the last-level cache could keep anyway.
+// Outputs in RED_MASK are not stored: every lane folds its elements' values into racc[], the
+// wavefront combines the lanes in a fixed order, and lane 0 writes one partial per reduction into
+// slots[q * slot_stride + 4 * blockIdx.x + wavefront] for the host to fold.
 struct Seg { i64 n; i64 blk0; const T* in[NLA]; T* out[NOA]; };
 typedef T TV __attribute__((ext_vector_type(VECW)));
+#define OUT_STORED(j) (((RED_MASK >> (j)) & 1u) == 0u)
 
 template <bool NT>
-__device__ __forceinline__ void flat_vec(const Seg& sg, i64 blk, const T* s) {
+__device__ __forceinline__ void flat_vec(const Seg& sg, i64 blk, const T* s, T* racc) {
+    (void)racc;
     const i64 i = (blk * 256 + threadIdx.x) * VECW;
     const i64 n = sg.n;
     if (i + VECW <= n) {
@@ -374,13 +417,16 @@ __device__ __forceinline__ void flat_vec(const Seg& sg, i64 blk, const T* s) {
 #pragma unroll
             for (int k = 0; k < NL; ++k) l[k] = lv[k][e];
             group_eval(l, s, o);
+            RED_FOLD(o, racc);
 #pragma unroll
             for (int j = 0; j < NO; ++j) ov[j][e] = o[j];
         }
 #pragma unroll
         for (int j = 0; j < NO; ++j) {
-            TV* dst = reinterpret_cast<TV*>(sg.out[j] + i);
-            if (NT) __builtin_nontemporal_store(ov[j], dst); else *dst = ov[j];
+            if (OUT_STORED(j)) {
+                TV* dst = reinterpret_cast<TV*>(sg.out[j] + i);
+                if (NT) __builtin_nontemporal_store(ov[j], dst); else *dst = ov[j];
+            }
         }
     } else {
         for (i64 x = i; x < n; ++x) {
@@ -388,14 +434,17 @@ __device__ __forceinline__ void flat_vec(const Seg& sg, i64 blk, const T* s) {
 #pragma unroll
             for (int k = 0; k < NL; ++k) l[k] = sg.in[k][x];
             group_eval(l, s, o);
+            RED_FOLD(o, racc);
 #pragma unroll
-            for (int j = 0; j < NO; ++j) sg.out[j][x] = o[j];
+            for (int j = 0; j < NO; ++j)
+                if (OUT_STORED(j)) sg.out[j][x] = o[j];
         }
     }
 }
 
 // Pointers that are not 16-byte aligned: one element per lane.
-__device__ __forceinline__ void flat_scalar(const Seg& sg, i64 blk, const T* s) {
+__device__ __forceinline__ void flat_scalar(const Seg& sg, i64 blk, const T* s, T* racc) {
+    (void)racc;
 #pragma unroll
     for (int u = 0; u < VECW; ++u) {
         const i64 i = (blk * VECW + u) * 256 + threadIdx.x;
@@ -404,29 +453,59 @@ __device__ __forceinline__ void flat_scalar(const Seg& sg, i64 blk, const T* s) 
 #pragma unroll
             for (int k = 0; k < NL; ++k) l[k] = sg.in[k][i];
             group_eval(l, s, o);
+            RED_FOLD(o, racc);
 #pragma unroll
-            for (int j = 0; j < NO; ++j) sg.out[j][i] = o[j];
+            for (int j = 0; j < NO; ++j)
+                if (OUT_STORED(j)) sg.out[j][i] = o[j];
         }
     }
 }
 
+#if NR > 0
+__device__ __forceinline__ void red_finish(T* racc, T* slots, i64 slot_stride) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+        T other[NRA];
+#pragma unroll
+        for (int q = 0; q < NR; ++q) other[q] = __shfl_xor(racc[q], m, 64);
+        RED_COMBINE(racc, other);
+    }
+    if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+        for (int q = 0; q < NR; ++q)
+            slots[q * slot_stride + 4 * (i64)blockIdx.x + (threadIdx.x >> 6)] = racc[q];
+    }
+}
+#define RED_PARAM , T* slots, i64 slot_stride
+#define RED_BEGIN T racc[NRA]; for (int q = 0; q < NRA; ++q) racc[q] = 0;
+#define RED_END red_finish(racc, slots, slot_stride);
+#else
+#define RED_PARAM
+#define RED_BEGIN T* racc = nullptr;
+#define RED_END
+#endif
+
 #define FLAT_ENTRY(NAME, CALL)                                                                   \
 extern "C" __global__ __launch_bounds__(256) void grp_flat_##NAME(const Seg* segs, int nseg,    \
-                                                                  Scal sc) {                     \
+                                                                  Scal sc RED_PARAM) {           \
     T s[NSA]; load_scalars(sc, s);                                                               \
+    RED_BEGIN                                                                                    \
     const int k = find_seg(segs, nseg, (i64)blockIdx.x);                                         \
     const Seg& sg = segs[k];                                                                     \
     const i64 blk = (i64)blockIdx.x - sg.blk0;                                                   \
     CALL;                                                                                        \
+    RED_END                                                                                      \
 }                                                                                                \
-extern "C" __global__ __launch_bounds__(256) void grp_flat1_##NAME(Seg sg, Scal sc) {           \
+extern "C" __global__ __launch_bounds__(256) void grp_flat1_##NAME(Seg sg, Scal sc RED_PARAM) { \
     T s[NSA]; load_scalars(sc, s);                                                               \
+    RED_BEGIN                                                                                    \
     const i64 blk = (i64)blockIdx.x;                                                             \
     CALL;                                                                                        \
+    RED_END                                                                                      \
 }
-FLAT_ENTRY(v, flat_vec<false>(sg, blk, s))
-FLAT_ENTRY(vn, flat_vec<true>(sg, blk, s))
-FLAT_ENTRY(s, flat_scalar(sg, blk, s))
+FLAT_ENTRY(v, flat_vec<false>(sg, blk, s, racc))
+FLAT_ENTRY(vn, flat_vec<true>(sg, blk, s, racc))
+FLAT_ENTRY(s, flat_scalar(sg, blk, s, racc))
 )";
     return s.str();
 }
@@ -671,6 +750,10 @@ int emit_variant_source(const GroupProgram& p, const std::string& variant, std::
     if (variant == "flat") {
         src = flat_source(p);
         return 0;
+    }
+    if (p.reductions() > 0) {
+        err = "a group with reducing roots runs over dense, equally laid out operands only";
+        return -17;
     }
     if (variant == "nd") {
         src = nd_source(p);

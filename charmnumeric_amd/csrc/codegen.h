@@ -32,11 +32,18 @@ struct GroupProgram {
     std::vector<int> out_names;   // result name of each output root
     std::vector<int> out_roots;   // root positions of the non-temp roots
     std::vector<int> out_is_set_region;
+    std::vector<int> out_reduce;  // 0: stored element by element; 1: summed, 2: largest |value|
     std::vector<int> out_target;  // SET_REGION target array name (or result name)
     std::vector<cnh_region> out_region; // SET_REGION region (is_global when absent)
     std::vector<std::string> out_expr;  // value expression of each output
     std::string body;             // statements computing t<k> from l<load>, s<bcast>
     bool uses_transcendental = false;
+    int reductions() const {
+        int n = 0;
+        for (int r : out_reduce)
+            n += r != 0;
+        return n;
+    }
 };
 
 // Returns 0 or a negative code with the reason in `err` for an AST the upstream JIT could not

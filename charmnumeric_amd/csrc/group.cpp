@@ -314,6 +314,20 @@ int cnh_launch_group_batched(cnh_kernel* k, int ndims, int n_parts, int n_in, co
     const int esz = dtype_size(p.dtype);
     const int vec = 16 / esz;
 
+    // Outputs that are reduced over the launch (CNH_OP_SUM_OF / CNH_OP_MAXABS_OF roots): their
+    // memref names the one element the result goes to (partition 0's counts); `e0` is the first
+    // output that is stored element by element, whose extents every other memref must match.
+    const int n_red = p.reductions();
+    int e0 = -1;
+    for (int o = 0; o < n_out; ++o)
+        if (!p.out_reduce[(size_t)o]) {
+            e0 = o;
+            break;
+        }
+    CNH_CHECK(e0 >= 0, -4, "a group needs an output that is stored element by element");
+    CNH_CHECK(n_red <= kFoldMaxVectors, -4, "%d reducing roots in one group (at most %d)", n_red,
+              kFoldMaxVectors);
+
     // Shapes must agree across all memrefs of a partition (identity indexing maps upstream).
     bool all_dense = true, all_aligned = true;
     std::vector<int> live;
@@ -322,8 +336,8 @@ int cnh_launch_group_batched(cnh_kernel* k, int ndims, int n_parts, int n_in, co
         const cnh_memref* po = out + (size_t)q * n_out;
         int64_t total = 1;
         for (int d = 0; d < ndims; ++d) {
-            CNH_CHECK(po[0].sizes[d] >= 0, -4, "negative extent");
-            total *= po[0].sizes[d];
+            CNH_CHECK(po[e0].sizes[d] >= 0, -4, "negative extent");
+            total *= po[e0].sizes[d];
         }
         if (total == 0)
             continue;
@@ -331,11 +345,13 @@ int cnh_launch_group_batched(cnh_kernel* k, int ndims, int n_parts, int n_in, co
         for (int i = 0; i < n_in + n_out; ++i) {
             const cnh_memref& m = i < n_in ? pi[i] : po[i - n_in];
             CNH_CHECK(m.aligned != nullptr, -4, "partition %d: memref %d has a null pointer", q, i);
+            if (i >= n_in && p.out_reduce[(size_t)(i - n_in)])
+                continue;
             for (int d = 0; d < ndims; ++d)
-                CNH_CHECK(m.sizes[d] == po[0].sizes[d], -4,
+                CNH_CHECK(m.sizes[d] == po[e0].sizes[d], -4,
                           "partition %d: memref %d extent %lld differs from the output's %lld in "
                           "dim %d",
-                          q, i, (long long)m.sizes[d], (long long)po[0].sizes[d], d);
+                          q, i, (long long)m.sizes[d], (long long)po[e0].sizes[d], d);
             if (!dense_memref(ndims, m))
                 all_dense = false;
             uintptr_t addr = (uintptr_t)m.aligned + (uintptr_t)(m.offset * esz);
@@ -361,7 +377,7 @@ int cnh_launch_group_batched(cnh_kernel* k, int ndims, int n_parts, int n_in, co
             const cnh_memref* po = out + (size_t)q * n_out;
             int64_t n = 1;
             for (int d = 0; d < ndims; ++d)
-                n *= po[0].sizes[d];
+                n *= po[e0].sizes[d];
             uint64_t* sg = &segs[j * seg_words];
             sg[0] = (uint64_t)n;
             sg[1] = (uint64_t)blocks;
@@ -379,17 +395,43 @@ int cnh_launch_group_batched(cnh_kernel* k, int ndims, int n_parts, int n_in, co
         hipFunction_t fn;
         if (int rc = get_function(k, "flat", name.c_str(), &fn))
             return rc;
-        if (live.size() == 1) {
-            void* params[] = {segs.data(), scal.data()};
-            return launch(fn, blocks, params, st);
+        // reducing roots: one partial per wavefront and reduction, folded after the launch
+        void* slots = nullptr;
+        const int64_t nslots = 4 * blocks;
+        int64_t slot_stride = nslots + kFoldRuns;     // the fold keeps its run sums behind each vector
+        if (n_red > 0) {
+            CNH_CHECK(p.dtype == CNH_F64, -27, "reducing roots need an fp64 group");
+            if (int rc = reduce_workspace(st, (size_t)(slot_stride * n_red) * sizeof(double), &slots))
+                return rc;
         }
-        const void* dsegs = nullptr;
-        if (int rc = desc_upload(segs.data(), segs.size() * 8, st, &dsegs))
-            return rc;
-        int nseg = (int)live.size();
-        void* params[] = {&dsegs, &nseg, scal.data()};
-        return launch(fn, blocks, params, st);
+        if (live.size() == 1) {
+            void* params[] = {segs.data(), scal.data(), &slots, &slot_stride};
+            if (int rc = launch(fn, blocks, params, st))
+                return rc;
+        } else {
+            const void* dsegs = nullptr;
+            if (int rc = desc_upload(segs.data(), segs.size() * 8, st, &dsegs))
+                return rc;
+            int nseg = (int)live.size();
+            void* params[] = {&dsegs, &nseg, scal.data(), &slots, &slot_stride};
+            if (int rc = launch(fn, blocks, params, st))
+                return rc;
+        }
+        if (n_red == 0)
+            return 0;
+        int maximum[kFoldMaxVectors] = {0, 0, 0, 0};
+        double* outs[kFoldMaxVectors] = {nullptr, nullptr, nullptr, nullptr};
+        int q = 0;
+        const cnh_memref* po = out + (size_t)live[0] * n_out;
+        for (int o = 0; o < n_out; ++o)
+            if (p.out_reduce[(size_t)o]) {
+                maximum[q] = p.out_reduce[(size_t)o] == 2;
+                outs[q] = reinterpret_cast<double*>((uintptr_t)base_ptr(po[o]));
+                ++q;
+            }
+        return reduce_slots_f64_many(n_red, maximum, static_cast<double*>(slots), nslots, slot_stride, outs, st);
     }
+    CNH_CHECK(n_red == 0, -28, "a group with reducing roots needs dense, equally laid out operands");
 
     // Strided cells.
     const size_t cell_words = 5 + NLA + 3 * NLA + NOA + 3 * NOA;

@@ -31,7 +31,12 @@ enum {
     CNH_OP_COPY = -5, CNH_OP_SET_REGION = -4, CNH_OP_GET_REGION = -3, CNH_OP_CREATE = -2,
     CNH_OP_NOOP = -1, CNH_OP_ADD = 0, CNH_OP_SUB = 1, CNH_OP_MUL = 2, CNH_OP_DIV = 3,
     CNH_OP_MATMUL = 4, CNH_OP_TANH = 5, CNH_OP_EXP = 6, CNH_OP_TILE = 7, CNH_OP_REDUCE = 8,
-    CNH_OP_MATMATMUL = 9, CNH_OP_DIAG = 10
+    CNH_OP_MATMATMUL = 9, CNH_OP_DIAG = 10,
+    /* Extension, no upstream counterpart: a group root that reduces its operand over every
+     * element of the launch instead of storing it (sum, or the largest absolute value). Upstream
+     * runs a reduction as a pass of its own over the stored array (src/executor_reduce.cpp:8-119);
+     * as a root of the group that produces the values it costs no second read. */
+    CNH_OP_SUM_OF = 20, CNH_OP_MAXABS_OF = 21
 };
 enum { CNH_F32 = 0, CNH_F64 = 1, CNH_I32 = 2, CNH_I64 = 3 };
 

@@ -1,0 +1,122 @@
+"""Reducing roots of a fused group (CNH_OP_SUM_OF / CNH_OP_MAXABS_OF): the values a group produces
+are summed (or their largest magnitude taken) by the launch that produces them. Checked against
+NumPy on the same inputs: the stored output bit for bit, maxima exactly, sums to rounding of the
+summation order (and exactly where every partial sum is an integer)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from charmnumeric_amd import _lib as L
+from charmnumeric_amd.astbuild import AstBuilder
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def ast_c1_reduced():
+    """z = 2.5x - 0.5y + xy stored (name 10); 20 = sum(z * w), 21 = sum(z * z), 22 = max|z - x|.
+    Leaves: x = 0, y = 1, w = 2."""
+    b = AstBuilder(L.F64, 1)
+    x, y, w = b.leaf(0), b.leaf(1), b.leaf(2)
+    t1 = b.binary(L.OP_MUL, 100, b.scalar(2.5), x)
+    t2 = b.binary(L.OP_MUL, 101, b.scalar(0.5), y)
+    t3 = b.binary(L.OP_SUB, 102, t1, t2)
+    t4 = b.binary(L.OP_MUL, 103, x, y)
+    z = b.binary(L.OP_ADD, 10, t3, t4, is_temp=False)
+    zw = b.binary(L.OP_MUL, 104, z, w)
+    b.unary(L.OP_SUM_OF, 20, zw, is_temp=False)
+    zz = b.binary(L.OP_MUL, 105, z, z)
+    b.unary(L.OP_SUM_OF, 21, zz, is_temp=False)
+    d = b.binary(L.OP_SUB, 106, z, x)
+    b.unary(L.OP_MAXABS_OF, 22, d, is_temp=False)
+    return b.finish()
+
+
+def bind(k, ins, outs):
+    """Memrefs in the kernel's argument order, from dictionaries by array name."""
+    n_in, n_sc, n_out = C.c_int(), C.c_int(), C.c_int()
+    L.check(L.lib.cnh_kernel_signature(k, C.byref(n_in), C.byref(n_sc), C.byref(n_out)))
+    name, has, tgt, sr = C.c_int(), C.c_int(), C.c_int(), C.c_int()
+    reg = L.Region()
+    a, b = [], []
+    for i in range(n_in.value):
+        L.check(L.lib.cnh_kernel_input(k, i, C.byref(name), C.byref(has), C.byref(reg)))
+        a.append(ins[name.value])
+    for i in range(n_out.value):
+        L.check(L.lib.cnh_kernel_output(k, i, C.byref(name), C.byref(tgt), C.byref(sr), C.byref(reg)))
+        b.append(outs[name.value])
+    return a, b
+
+
+@pytest.mark.parametrize("n,parts,shift", [(1, 1, 0), (77, 1, 0), (1000, 3, 0), (4099, 2, 1),
+                                           ((1 << 20) + 3, 1, 0), ((1 << 22) + 517, 4, 0)])
+def test_group_with_reducing_roots(dev, n, parts, shift):
+    rng = np.random.default_rng(n)
+    k = H.compile_group(ast_c1_reduced(), L.F64, 1)
+    hx, hy, hw = (rng.standard_normal(n + shift) for _ in range(3))
+    x, y, w = dev.array(hx), dev.array(hy), dev.array(hw)
+    z = dev.empty((n + shift,), np.float64)
+    res = dev.array(np.full(3, np.nan))
+    cuts = [shift + (n * q) // parts for q in range(parts + 1)]
+    pin, pout = [], []
+    for q in range(parts):
+        lo, cnt = cuts[q], cuts[q + 1] - cuts[q]
+        view = lambda buf: L.Memref.dense(buf.ptr + 8 * lo, (cnt,))
+        scalar = lambda i: L.Memref.dense(res.ptr + 8 * i, (1,))
+        a, b = bind(k, {0: view(x), 1: view(y), 2: view(w)},
+                    {10: view(z), 20: scalar(0), 21: scalar(1), 22: scalar(2)})
+        pin.append(a)
+        pout.append(b)
+    H.launch_batched(k, 1, pin, [], pout)
+    ex, ey, ew = hx[shift:], hy[shift:], hw[shift:]
+    ez = ((2.5 * ex) - (0.5 * ey)) + (ex * ey)
+    assert np.array_equal(z.get()[shift:], ez)
+    got = res.get()
+    for value, terms in ((got[0], ez * ew), (got[1], ez * ez)):
+        assert abs(value - np.sum(terms)) <= 1e-13 * np.sum(np.abs(terms)) + 1e-300
+    assert got[2] == np.max(np.abs(ez - ex))
+    dev.free_all()
+
+
+def test_sums_of_integers_are_exact(dev):
+    """Every partial sum is an integer below 2^53: whatever the order, the result is the closed form."""
+    n = (1 << 21) + 11
+    b = AstBuilder(L.F64, 1)
+    v = b.binary(L.OP_ADD, 10, b.leaf(0), b.scalar(1.0), is_temp=False)
+    b.unary(L.OP_SUM_OF, 20, v, is_temp=False)
+    sq = b.binary(L.OP_MUL, 100, v, v)
+    b.unary(L.OP_SUM_OF, 21, sq, is_temp=False)
+    k = H.compile_group(b.finish(), L.F64, 1)
+    x = dev.array(np.arange(n, dtype=np.float64) % 1000)
+    out = dev.empty((n,), np.float64)
+    res = dev.array(np.zeros(2))
+    a, o = bind(k, {0: x.memref()}, {10: out.memref(), 20: L.Memref.dense(res.ptr, (1,)),
+                                      21: L.Memref.dense(res.ptr + 8, (1,))})
+    for _ in range(2):                      # the partials of a launch do not leak into the next
+        H.launch_batched(k, 1, [a], [], [o])
+    v = (np.arange(n) % 1000 + 1).astype(np.int64)
+    got = res.get()
+    assert got[0] == float(v.sum()) and got[1] == float((v * v).sum())
+    dev.free_all()
+
+
+def test_reducing_roots_need_dense_operands(dev):
+    b = AstBuilder(L.F64, 2)
+    v = b.binary(L.OP_MUL, 10, b.leaf(0), b.scalar(2.0), is_temp=False)
+    b.unary(L.OP_SUM_OF, 20, v, is_temp=False)
+    k = H.compile_group(b.finish(), L.F64, 2)
+    x = dev.array(np.ones((8, 16)))
+    out = dev.empty((8, 16), np.float64)
+    res = dev.array(np.zeros(1))
+    strided = L.Memref.strided(x.ptr, (8, 8), (16, 1))          # every other half row
+    a, o = bind(k, {0: strided}, {10: L.Memref.strided(out.ptr, (8, 8), (16, 1)),
+                                  20: L.Memref.dense(res.ptr, (1,))})
+    with pytest.raises(L.CnhError, match="dense"):
+        H.launch_batched(k, 2, [a], [], [o])
+    # a reducing root is never a temporary, and there is no integer form
+    bad = AstBuilder(L.I32, 1)
+    bad.unary(L.OP_SUM_OF, 20, bad.binary(L.OP_ADD, 10, bad.leaf(0), bad.scalar(1), is_temp=False), is_temp=False)
+    with pytest.raises(L.CnhError):
+        H.compile_group(bad.finish(), L.I32, 1)
+    dev.free_all()
