@@ -357,7 +357,9 @@ def cg_parity(gpu_trace, cpu_trace, rtr0, floor=1e-24):
 # -------------------------------------------------------------------------------------------------
 # C1: fused elementwise 2^24 + sum + dot
 # -------------------------------------------------------------------------------------------------
-def c1_ast(L):
+def c1_ast(L, reduced=False):
+    """z = 2.5 x - 0.5 y + x y (name 10). With `reduced`, sum(z) (20) and z.z (21) as reducing
+    roots of the same group: the launch that stores z also sums it."""
     from charmnumeric_amd.astbuild import AstBuilder
 
     b = AstBuilder(L.F64, 1)
@@ -366,7 +368,11 @@ def c1_ast(L):
     t2 = b.binary(L.OP_MUL, 101, b.scalar(0.5), y)
     t3 = b.binary(L.OP_SUB, 102, t1, t2)
     t4 = b.binary(L.OP_MUL, 103, x, y)
-    b.binary(L.OP_ADD, 10, t3, t4, is_temp=False)
+    z = b.binary(L.OP_ADD, 10, t3, t4, is_temp=False)
+    if reduced:
+        b.unary(L.OP_SUM_OF, 20, z, is_temp=False)
+        zz = b.binary(L.OP_MUL, 104, z, z)
+        b.unary(L.OP_SUM_OF, 21, zz, is_temp=False)
     return b.finish()
 
 
@@ -399,8 +405,22 @@ def run_c1(L, n=1 << 24, parts=4, reps=20):
     def dt():
         L.check(L.lib.cnh_dot_tiles(L.F64, parts, zp, zp, lens, res.ptr + 8, None))
 
+    # the three as one group with reducing roots: one pass over x and y, z stored once and never
+    # read back (the results go to a second pair of slots, compared with the first below)
+    kr = _compile(L, c1_ast(L, reduced=True), L.F64, 1)
+    res2 = Buf(L, 16, zero=True)
+    outs_r = (L.Memref * (3 * parts))()
+    for q in range(parts):
+        outs_r[3 * q] = outs[q]
+        outs_r[3 * q + 1] = L.Memref.dense(res2.ptr, (1,))
+        outs_r[3 * q + 2] = L.Memref.dense(res2.ptr + 8, (1,))
+
+    def fused():
+        L.check(L.lib.cnh_launch_group_batched(kr, 1, parts, 4, ins, 0, None, 0, 3, outs_r, None))
+
     out = {}
-    for name, fn, nbytes in (("elementwise", ew, 24 * n), ("sum", sm, 8 * n), ("dot_zz", dt, 8 * n)):
+    for name, fn, nbytes in (("elementwise", ew, 24 * n), ("sum", sm, 8 * n), ("dot_zz", dt, 8 * n),
+                             ("elementwise_sum_dot_one_pass", fused, 24 * n)):
         for _ in range(3):
             fn()
         ev = Events(L, reps)
@@ -415,7 +435,10 @@ def run_c1(L, n=1 << 24, parts=4, reps=20):
         us = 1e3 * float(np.median(t))
         out[name] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
                      "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
-    for b_ in xs + ys + zs + [ones, res]:
+    separate, one_pass = res.get(np.float64), res2.get(np.float64)
+    out["one_pass_vs_separate_rel_diff"] = float(np.max(np.abs(separate - one_pass) / np.abs(separate)))
+    out["separate_passes_us"] = round(out["elementwise"]["us"] + out["sum"]["us"] + out["dot_zz"]["us"], 2)
+    for b_ in xs + ys + zs + [ones, res, res2]:
         b_.free()
     return out
 

@@ -1897,6 +1897,276 @@ int try_statement_run(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t*
     return 0;
 }
 
+// ---- reductions taken by the launch that produces what they reduce ----
+//
+// `z = f(x, y)` followed by `z @ w`, `sum(z)`, `sum((z - w)^2)` or `max|z - w|` (a CG residual
+// update and its r.r, a field and its norms) reads z again once per reduction when every node
+// runs on its own. Where the group's result is a new array laid out like its operands (the dense
+// path) and the reductions that follow take whole arrays of that layout, the reductions become
+// reducing roots of the group (CNH_OP_SUM_OF / CNH_OP_MAXABS_OF): one launch stores z and leaves
+// the partial results, one or two small launches fold them.
+
+// Will an array of `shape`, created now, have exactly the tiles of `a`?
+bool laid_out_like_new(const Ex* ex, const XArray& a, int nd, const int32_t* shape) {
+    if (a.ndims != nd || a.tile != tile_rule(ex, nd, shape) || a.flat != (nd == 3 && ex->flat3))
+        return false;
+    for (int d = 0; d < nd; ++d)
+        if (a.shape[d] != shape[d] || a.offset[d] % a.tile != 0)
+            return false;
+    return true;
+}
+
+int try_group_with_reductions(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t* used, bool* open_ended) {
+    *used = 0;
+    *open_ended = false;
+    const DagNode& n = dag[i];
+    if (n.roots.empty() || !n.fusible)
+        return 0;
+    const cnh_ast_node& root = n.nodes[n.roots.back()];
+    const bool elementwise = (root.opcode >= CNH_OP_ADD && root.opcode <= CNH_OP_DIV) || root.opcode == CNH_OP_TANH ||
+                             root.opcode == CNH_OP_EXP || root.opcode == CNH_OP_COPY;
+    if (!elementwise || root.is_temp || root.dtype != CNH_F64)
+        return 0;
+    for (size_t r = 0; r + 1 < n.roots.size(); ++r)
+        if (!n.nodes[n.roots[r]].is_temp)
+            return 0;
+    int32_t shape[3] = {1, 1, 1};
+    {
+        // every array the group reads: whole, fp64, laid out as the result will be
+        bool any = false;
+        for (const cnh_ast_node& a : n.nodes) {
+            if (a.opcode != CNH_OP_NOOP || a.is_scalar || a.is_broadcast)
+                continue;
+            auto it = ex->arrays.find(a.result_name);
+            if (it == ex->arrays.end() || it->second.dtype != CNH_F64)
+                return 0;
+            if (!any)
+                for (int d = 0; d < it->second.ndims; ++d)
+                    shape[d] = it->second.shape[d];
+            any = true;
+            if (it->second.ndims != root.ndims || !laid_out_like_new(ex, it->second, root.ndims, shape))
+                return 0;
+        }
+        if (!any)
+            return 0;
+        for (int32_t r : n.roots) {
+            const cnh_ast_node& a = n.nodes[r];
+            for (int oi = 0; oi < a.n_operands; ++oi)
+                if (a.has_operand_region[oi] && !a.operand_regions[oi].is_global) {
+                    const cnh_ast_node& op = n.nodes[a.operands[oi]];
+                    auto it = ex->arrays.find(op.result_name);
+                    if (it == ex->arrays.end() || !region_is_whole(a.operand_regions[oi], it->second))
+                        return 0;
+                }
+        }
+    }
+    const int result = root.result_name;
+
+    // the reductions that follow, deletions in between put off until after the launch
+    struct Red { const DagNode* node; int op; int other; };      // other: the second array (0: none, -1: the result itself)
+    std::vector<Red> reds;
+    std::vector<int> deletions, deletions_kept;
+    size_t j = i + 1, end = i + 1;
+    for (; j < dag.size() && reds.size() < (size_t)kFoldMaxVectors; ++j) {
+        const DagNode& m = dag[j];
+        if (m.roots.empty())
+            break;
+        const cnh_ast_node& r = m.nodes[m.roots.back()];
+        if (r.opcode == kOpDelete) {
+            if (r.result_name == result)
+                break;
+            deletions.push_back(r.result_name);
+            continue;
+        }
+        const bool paired = r.opcode == CNH_OP_REDUCE || r.opcode == kOpSumsqDiff || r.opcode == kOpMaxabsDiff;
+        if (!(paired || r.opcode == kOpSum) || m.roots.size() != 1 || r.n_operands != (paired ? 2 : 1) ||
+            r.dtype != CNH_F64)
+            break;
+        if (r.opcode == CNH_OP_REDUCE && root.ndims != 1)
+            break;
+        int names[2] = {0, 0};
+        bool ok = true;
+        for (int oi = 0; oi < r.n_operands && ok; ++oi) {
+            const cnh_ast_node& op = m.nodes[r.operands[oi]];
+            ok = op.opcode == CNH_OP_NOOP && !op.is_scalar && !op.is_broadcast &&
+                 (!r.has_operand_region[oi] || r.operand_regions[oi].is_global);
+            names[oi] = op.result_name;
+        }
+        if (!ok || (names[0] != result && !(paired && names[1] == result)))
+            break;
+        int other = 0;
+        if (paired) {
+            const int b = names[0] == result ? names[1] : names[0];
+            if (b == result) {
+                other = -1;
+            } else {
+                auto it = ex->arrays.find(b);
+                if (it == ex->arrays.end() || it->second.dtype != CNH_F64 ||
+                    !laid_out_like_new(ex, it->second, root.ndims, shape) ||
+                    std::find(deletions.begin(), deletions.end(), b) != deletions.end())
+                    break;
+                other = b;
+            }
+        }
+        reds.push_back({&m, r.opcode, other});
+        end = j + 1;
+        deletions_kept = deletions;
+    }
+    if (j == dag.size() && reds.size() < (size_t)kFoldMaxVectors && open_ended_allowed(ex)) {
+        *open_ended = true;           // the reductions may be in the next message
+        return 0;
+    }
+    if (reds.empty())
+        return 0;
+
+    // the group with the reductions as reducing roots
+    DagNode merged = n;
+    const int value = n.roots.back();
+    int next_tmp = 0x7f000000;
+    auto leaf_of = [&](int name) {
+        for (size_t q = 0; q < merged.nodes.size(); ++q)
+            if (merged.nodes[q].opcode == CNH_OP_NOOP && !merged.nodes[q].is_scalar &&
+                !merged.nodes[q].is_broadcast && merged.nodes[q].result_name == name)
+                return (int)q;
+        cnh_ast_node leaf;
+        std::memset(&leaf, 0, sizeof leaf);
+        leaf.result_name = name;
+        leaf.opcode = CNH_OP_NOOP;
+        leaf.ndims = root.ndims;
+        leaf.dtype = CNH_F64;
+        leaf.region.is_global = 1;
+        merged.nodes.push_back(leaf);
+        return (int)merged.nodes.size() - 1;
+    };
+    auto add_root = [&](int name, int opcode, bool is_temp, int a, int b) {
+        cnh_ast_node r;
+        std::memset(&r, 0, sizeof r);
+        r.result_name = name;
+        r.opcode = opcode;
+        r.is_temp = is_temp;
+        r.ndims = root.ndims;
+        r.dtype = CNH_F64;
+        r.n_operands = b >= 0 ? 2 : 1;
+        r.operands[0] = a;
+        r.operands[1] = b;
+        r.region.is_global = 1;
+        r.operand_regions[0].is_global = r.operand_regions[1].is_global = 1;
+        merged.nodes.push_back(r);
+        merged.roots.push_back((int)merged.nodes.size() - 1);
+        return (int)merged.nodes.size() - 1;
+    };
+    for (const Red& rd : reds) {
+        const int out_name = rd.node->nodes[rd.node->roots.back()].result_name;
+        const int b = rd.other == 0 ? -1 : rd.other == -1 ? value : leaf_of(rd.other);
+        if (rd.op == kOpSum) {
+            add_root(out_name, CNH_OP_SUM_OF, false, value, -1);
+        } else if (rd.op == CNH_OP_REDUCE) {
+            const int t = add_root(next_tmp++, CNH_OP_MUL, true, value, b);
+            add_root(out_name, CNH_OP_SUM_OF, false, t, -1);
+        } else {
+            const int d = add_root(next_tmp++, CNH_OP_SUB, true, value, b);
+            if (rd.op == kOpSumsqDiff) {
+                const int t = add_root(next_tmp++, CNH_OP_MUL, true, d, d);
+                add_root(out_name, CNH_OP_SUM_OF, false, t, -1);
+            } else {
+                add_root(out_name, CNH_OP_MAXABS_OF, false, d, -1);
+            }
+        }
+    }
+
+    Group g;
+    canonicalise(merged, g);
+    cnh_kernel* k = nullptr;
+    if (int rc = compile_cached(ex, g, &k))
+        return rc;
+    int n_in = 0, n_scalar = 0, n_out = 0;
+    if (int rc = cnh_kernel_signature(k, &n_in, &n_scalar, &n_out))
+        return rc;
+    CNH_CHECK(n_out == 1 + (int)reds.size(), -26, "node %d: %d outputs for %d reductions", n.id, n_out,
+              (int)reds.size());
+    std::vector<XArray*> in_arr((size_t)n_in);
+    for (int q = 0; q < n_in; ++q) {
+        int cname = 0, has = 0;
+        cnh_region reg;
+        if (int rc = cnh_kernel_input(k, q, &cname, &has, &reg))
+            return rc;
+        if (int rc = find_array(ex, g.canon_to_actual[cname], &in_arr[(size_t)q], "group input"))
+            return rc;
+    }
+    std::vector<const void*> scalars((size_t)std::max(1, n_scalar), nullptr);
+    for (int q = 0; q < n_scalar; ++q) {
+        int cname = 0;
+        if (int rc = cnh_kernel_scalar(k, q, &cname))
+            return rc;
+        XArray* sarr;
+        if (int rc = find_array(ex, g.canon_to_actual[cname], &sarr, "broadcast scalar"))
+            return rc;
+        CNH_CHECK(sarr->elems == 1 && sarr->dtype == CNH_F64, -27, "node %d: broadcast operand %d", n.id, sarr->name);
+        scalars[(size_t)q] = sarr->tiles[0];
+    }
+    // outputs by name: the group's result first created, then one element per reduction
+    std::vector<XArray*> out_arr((size_t)n_out);
+    XArray* target = nullptr;
+    for (int q = 0; q < n_out; ++q) {
+        int rname = 0, tname = 0, is_set = 0;
+        cnh_region reg;
+        if (int rc = cnh_kernel_output(k, q, &rname, &tname, &is_set, &reg))
+            return rc;
+        const int actual = g.canon_to_actual[rname];
+        if (actual == result) {
+            if (int rc = make_array(ex, result, root.ndims, CNH_F64, shape, false, &out_arr[(size_t)q]))
+                return rc;
+        } else if (int rc = new_scalar_array(ex, actual, CNH_F64, &out_arr[(size_t)q])) {
+            return rc;
+        }
+    }
+    // std::map keeps element addresses: the pointers taken above stay valid
+    if (int rc = find_array(ex, result, &target, "group result"))
+        return rc;
+    for (XArray* a : in_arr)
+        CNH_CHECK(same_decomposition(*a, *target), -26, "node %d: operand %d is laid out differently", n.id, a->name);
+    const int nd = target->ndims;
+    const int64_t parts = target->flat ? 1 : target->ntiles;
+    std::vector<cnh_memref> in(std::max<size_t>(1, (size_t)parts * n_in)), out((size_t)parts * n_out);
+    for (int64_t t = 0; t < parts; ++t) {
+        int32_t lo[3], ext[3];
+        target->tile_extent(t, lo, ext);
+        if (target->flat)
+            for (int d = 0; d < nd; ++d)
+                ext[d] = target->shape[d];
+        auto fill = [&](cnh_memref& m, void* ptr, bool one) {
+            std::memset(&m, 0, sizeof m);
+            m.allocated = m.aligned = ptr;
+            int64_t stride = 1;
+            for (int d = nd - 1; d >= 0; --d) {
+                m.sizes[d] = one ? 1 : ext[d];
+                m.strides[d] = stride;
+                stride *= m.sizes[d];
+            }
+        };
+        for (int q = 0; q < n_in; ++q)
+            fill(in[(size_t)t * n_in + q], in_arr[(size_t)q]->tiles[t], false);
+        for (int q = 0; q < n_out; ++q)
+            fill(out[(size_t)t * n_out + q], out_arr[(size_t)q] == target ? target->tiles[t] : out_arr[(size_t)q]->tiles[0],
+                 out_arr[(size_t)q] != target);
+    }
+    ex->stats[5]++;
+    ex->log("group node=" + std::to_string(n.id) + " path=dense+reduce parts=" + std::to_string(parts) +
+            " inputs=" + std::to_string(n_in) + " scalars=" + std::to_string(n_scalar) + " reductions=" +
+            std::to_string(reds.size()) + " out=" + std::to_string(target->name));
+    int rc = 0;
+    if (!ex->dry)
+        rc = cnh_launch_group_batched(k, nd, (int)parts, n_in, in.data(), n_scalar, scalars.data(), 1, n_out,
+                                      out.data(), ex->stream);
+    if (rc)
+        return rc;
+    for (int name : deletions_kept)
+        drop_array(ex, name);
+    ex->stats[2] += (int64_t)(end - i);
+    *used = end - i;
+    return 0;
+}
+
 int parse_dag(const char* msg, int64_t size, std::vector<DagNode>& out) {
     Reader r{msg, msg + size};
     int32_t magic = r.get<int32_t>(), version = r.get<int32_t>(), count = r.get<int32_t>();
@@ -2192,6 +2462,8 @@ int run_nodes(Ex* ex, std::vector<DagNode>& dag) {
             rc = try_product_into_region(ex, dag, i, &used, &open_ended);
             if (rc == 0 && used == 0 && !open_ended)
                 rc = try_statement_run(ex, dag, i, &used, &open_ended);
+            if (rc == 0 && used == 0 && !open_ended)
+                rc = try_group_with_reductions(ex, dag, i, &used, &open_ended);
             if (rc == 0 && open_ended) {
                 ex->held.assign(dag.begin() + (std::ptrdiff_t)i, dag.end());
                 break;

@@ -198,7 +198,9 @@ def test_cg_iteration_compiles_once_and_reuses_buffers(itf):
     assert st["reuses"] > 0 and st["live_arrays"] <= 12
     tr = itf.trace()
     assert sum(ln.startswith("matmul") for ln in tr) == 4
-    assert sum(ln.startswith("reduce") for ln in tr) == 1 + 2 * 4
+    # p.Ap follows a product and runs on its own; r.r rides on the launch that updates r
+    assert sum(ln.startswith("reduce") for ln in tr) == 1 + 4
+    assert sum("path=dense+reduce" in ln and "reductions=1" in ln for ln in tr) == 4
     scal = [ln for ln in tr if ln.startswith("group") and "scalars=1" in ln]
     assert len(scal) == 3 * 4                                 # x, r, p updates take alpha/beta from the device
 
@@ -448,6 +450,52 @@ def test_runs_of_same_extent_assignments_become_one_launch(itf):
     C[4] = H[3] + 1.0
     cnp.execute(itf)
     assert not any("path=statements" in ln for ln in itf.trace())
+
+
+def test_reductions_ride_on_the_group_that_produces_their_operand(itf):
+    """A new array and the reductions of it that follow go out as one launch with reducing roots;
+    slices, other layouts and results that are not fresh keep every node on its own."""
+    n = 4096
+    x, y, ones = cnp.zeros((n,)), cnp.zeros((n,)), cnp.ones((n,))
+    cnp.execute(itf)
+    itf.trace()
+    z = 2.5 * x - 0.5 * y + x * y
+    s1 = z @ ones
+    s2 = z @ z
+    s3 = cnp.sumsq_diff(z, x)
+    s4 = cnp.maxabs_diff(y, z)
+    s5 = cnp.sum(z)                 # the fifth: a launch carries four at most
+    cnp.execute(itf)
+    log = itf.trace()
+    fused = [ln for ln in log if "path=dense+reduce" in ln]
+    assert len(fused) == 1 and "reductions=4" in fused[0]
+    assert sum(ln.startswith("reduce") for ln in log) == 1
+    assert sum(ln.startswith("create") for ln in log) == 6       # z and five one-element results
+    # a 3-D field and its norms
+    u, f = cnp.zeros((12, 10, 8)), cnp.zeros((12, 10, 8))
+    cnp.execute(itf)
+    itf.trace()
+    r = f - 6.0 * u
+    nrm = cnp.sumsq_diff(r, f)
+    top = cnp.maxabs_diff(r, u)
+    cnp.execute(itf)
+    fused = [ln for ln in itf.trace() if "path=dense+reduce" in ln]
+    assert len(fused) == 1 and "reductions=2" in fused[0]
+    # not a fresh array (an assignment into a slice), or a reduction over a window: node by node
+    y[0:n // 2] = x[0:n // 2] * 2.0
+    w1 = y @ ones
+    t = x + y
+    w2 = t[0:n // 2] @ ones[0:n // 2]
+    cnp.execute(itf)
+    log = itf.trace()
+    assert not any("path=dense+reduce" in ln for ln in log)
+    assert sum(ln.startswith("reduce") for ln in log) == 2
+    # switched off
+    itf.set_fusion(False)
+    t2 = x * 3.0
+    w3 = t2 @ t2
+    cnp.execute(itf)
+    assert not any("path=dense+reduce" in ln for ln in itf.trace())
 
 
 def test_kernel_cache_is_bounded_over_a_long_slab_loop(itf):

@@ -502,3 +502,32 @@ def test_statement_runs_give_what_the_statements_give_one_by_one(itf, fusion, ra
     u[4:36] = u[4:36] * v[4:36]
     hu[4:36] = hu[4:36] * hv[4:36]
     assert np.array_equal(u.get(itf), hu) and np.array_equal(v.get(itf), hv)
+
+
+@pytest.mark.parametrize("fusion", [True, False], ids=["fused", "node-by-node"])
+@pytest.mark.parametrize("shape", [(100000,), (300, 70), (20, 30, 40)])
+def test_reductions_fused_into_their_producer(itf, small_tiles, fusion, shape):
+    """z = f(x, y) followed by reductions of z: one launch with reducing roots by default. The
+    stored array is the same bit for bit either way; sums agree with NumPy to summation order and
+    the maximum exactly."""
+    itf.set_fusion(fusion)
+    rng = np.random.default_rng(len(shape))
+    hx, hy = rng.standard_normal(shape), rng.standard_normal(shape)
+    x, y = cnp.array(hx), cnp.array(hy)
+    x.get(itf)
+    itf.set_trace()
+    z = 2.5 * x - 0.5 * y + x * y
+    hz = 2.5 * hx - 0.5 * hy + hx * hy
+    total = cnp.sum(z)
+    ssd = cnp.sumsq_diff(z, y)
+    top = cnp.maxabs_diff(x, z)
+    dot = z @ x if len(shape) == 1 else None
+    assert np.array_equal(z.get(itf), hz)
+    close = lambda got, terms: abs(got - terms.sum()) <= 1e-13 * np.abs(terms).sum()
+    assert close(total.get(itf).item(), hz)
+    assert close(ssd.get(itf).item(), (hz - hy) ** 2)
+    assert top.get(itf).item() == np.max(np.abs(hx - hz))
+    if dot is not None:
+        assert close(dot.get(itf).item(), hz * hx)
+    fused = [ln for ln in itf.trace() if "path=dense+reduce" in ln]
+    assert len(fused) == (1 if fusion else 0)
