@@ -200,6 +200,7 @@ _PROTOS = {
     "cnh_scalar_to_dtype": (C.c_int, [C.c_int, C.c_double, C.c_void_p]),
     "cnh_compile_group": (C.c_int, [C.POINTER(Ast), C.c_int, C.c_int, C.c_uint64, _vpp]),
     "cnh_kernel_release": (C.c_int, [C.c_void_p]),
+    "cnh_kernel_matches": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int]),
     "cnh_kernel_signature": (C.c_int, [C.c_void_p, C.POINTER(C.c_int), C.POINTER(C.c_int),
                                        C.POINTER(C.c_int)]),
     "cnh_kernel_input": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int),

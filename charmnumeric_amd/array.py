@@ -306,10 +306,11 @@ class _ArrayLike:
                 # (IFOG[t] = M with M 2-D), and a whole higher-rank one whose extra dimensions
                 # have extent 1 fits a lower-rank target (vec[:] = column)
                 squeeze = lambda sh: tuple(x for x in sh if x != 1)
-                if not (value.ndims != len(shape) and squeeze(value.shape) == squeeze(shape)
-                        and _is_whole(value._region(), value._base().shape)):
+                if not (value.ndims != len(shape) and squeeze(value.shape) == squeeze(shape)):
                     raise ValueError(
                         f"could not broadcast input from shape {value.shape} into shape {shape}")
+                if not _is_whole(value._region(), value._base().shape):
+                    value = value.copy()        # a slice of another rank: copied out first
             operand = value._refb()
         else:
             operand = lazy.scalar_bytes(value)

@@ -540,13 +540,19 @@ void canonicalise(const DagNode& n, Group& g) {
 }
 
 int compile_cached(Ex* ex, Group& g, cnh_kernel** out) {
-    auto it = ex->kernels.find(g.key);
-    if (it != ex->kernels.end()) {
-        ex->stats[1]++;
-        *out = it->second;
-        return 0;
-    }
     cnh_ast ast{(int32_t)g.nodes.size(), (int32_t)g.roots.size(), g.nodes.data(), g.roots.data()};
+    // the key is a hash: a hit counts only when the kernel was compiled from this very group;
+    // another group under the same key moves on to the next key of a fixed sequence
+    for (auto it = ex->kernels.find(g.key); it != ex->kernels.end(); it = ex->kernels.find(g.key)) {
+        if (cnh_kernel_matches(it->second, &ast, g.dtype, g.ndims)) {
+            ex->stats[1]++;
+            *out = it->second;
+            return 0;
+        }
+        g.key = g.key * 6364136223846793005ull + 1442695040888963407ull;
+        if (g.key == 0)
+            g.key = 1;
+    }
     cnh_kernel* k = nullptr;
     if (int rc = cnh_compile_group(&ast, g.dtype, g.ndims, g.key, &k))
         return rc;

@@ -21,6 +21,7 @@ using namespace cnh;
 struct CodeObject {
     std::string src;
     std::vector<char> code;
+    std::mutex mu;                 // guards mod and fns: code objects are shared between kernels
     hipModule_t mod = nullptr;
     std::map<std::string, hipFunction_t> fns;
 };
@@ -34,6 +35,8 @@ struct cnh_kernel {
     GroupProgram prog;
     uint64_t key = 0;
     int refs = 1;
+    std::string ident;             // the AST it was compiled from, field by field (see ast_ident)
+    std::mutex mu;                 // guards variants: a kernel found by key is shared between executors
     std::map<std::string, KernelVariant> variants;
 };
 
@@ -53,7 +56,34 @@ uint64_t text_hash(const std::string& t) {
     return h;
 }
 
+// Everything of an AST that decides the generated code, as bytes: what a cache key stands for.
+std::string ast_ident(const cnh_ast* ast, int dtype, int ndims) {
+    std::string out;
+    auto put = [&](const void* p, size_t n) { out.append(static_cast<const char*>(p), n); };
+    auto put_region = [&](const cnh_region& r) {
+        const int32_t v[11] = {r.is_global, r.ndims,   r.start[0], r.start[1], r.start[2], r.stop[0],
+                               r.stop[1],   r.stop[2], r.step[0],  r.step[1],  r.step[2]};
+        put(v, sizeof v);
+    };
+    const int32_t head[4] = {dtype, ndims, ast->n_nodes, ast->n_roots};
+    put(head, sizeof head);
+    for (int i = 0; i < ast->n_nodes; ++i) {
+        const cnh_ast_node& a = ast->nodes[i];
+        const int32_t f[12] = {a.result_name, a.opcode,      a.is_temp,     a.is_scalar,
+                               a.is_broadcast, a.ndims,      a.dtype,       a.n_operands,
+                               a.operands[0], a.operands[1], a.has_operand_region[0], a.has_operand_region[1]};
+        put(f, sizeof f);
+        put(&a.scalar, sizeof a.scalar);
+        put_region(a.operand_regions[0]);
+        put_region(a.operand_regions[1]);
+        put_region(a.region);
+    }
+    put(ast->roots, sizeof(int32_t) * (size_t)ast->n_roots);
+    return out;
+}
+
 int build_variant(cnh_kernel* k, const std::string& variant, KernelVariant** out) {
+    std::lock_guard<std::mutex> kernel_lock(k->mu);
     auto it = k->variants.find(variant);
     if (it != k->variants.end() && it->second.obj) {
         *out = &it->second;
@@ -116,6 +146,7 @@ int get_function(cnh_kernel* k, const std::string& variant, const char* name, hi
     if (int rc = build_variant(k, variant, &v))
         return rc;
     CodeObject* c = v->obj.get();
+    std::lock_guard<std::mutex> object_lock(c->mu);
     if (!c->mod)
         CNH_HIP(hipModuleLoadData(&c->mod, c->code.data()));
     auto it = c->fns.find(name);
@@ -173,16 +204,24 @@ extern "C" {
 
 int cnh_compile_group(const cnh_ast* ast, int dtype, int ndims, uint64_t key, cnh_kernel** out) {
     CNH_CHECK(out != nullptr, -2, "cnh_compile_group: null output");
+    CNH_CHECK(ast != nullptr && ast->nodes != nullptr && ast->roots != nullptr && ast->n_nodes > 0 &&
+                  ast->n_roots > 0,
+              -2, "cnh_compile_group: empty AST");
+    std::string ident = ast_ident(ast, dtype, ndims);
     std::lock_guard<std::mutex> lk(g_kmu);
     if (key != 0) {
         auto it = g_kernels.find(key);
         if (it != g_kernels.end()) {
-            it->second->refs++;
-            *out = it->second;
-            return 0;
+            if (it->second->ident == ident) {
+                it->second->refs++;
+                *out = it->second;
+                return 0;
+            }
+            key = 0;   // two different groups under one key: this one is compiled and kept apart
         }
     }
     cnh_kernel* k = new cnh_kernel;
+    k->ident = std::move(ident);
     std::string err;
     int rc = build_group_program(ast, dtype, ndims, k->prog, err);
     if (rc) {
@@ -194,6 +233,12 @@ int cnh_compile_group(const cnh_ast* ast, int dtype, int ndims, uint64_t key, cn
         g_kernels[key] = k; // found again by key while somebody holds it; gone with its last user
     *out = k;
     return 0;
+}
+
+int cnh_kernel_matches(const cnh_kernel* k, const cnh_ast* ast, int dtype, int ndims) {
+    if (k == nullptr || ast == nullptr || ast->nodes == nullptr || ast->roots == nullptr)
+        return 0;
+    return k->ident == ast_ident(ast, dtype, ndims) ? 1 : 0;
 }
 
 int cnh_kernel_release(cnh_kernel* k) {

@@ -164,6 +164,9 @@ int cnh_compile_group(const cnh_ast* ast, int dtype, int ndims, uint64_t key, cn
 /* Drops one reference; the kernel object goes with its last holder (a later compile with the same
  * key builds it again). Code objects are shared between kernels with identical generated text
  * and stay loaded. */
+/* 1 when `k` was compiled from exactly this AST, element type and rank (a cache keyed by a hash of
+ * the AST asks before it reuses a kernel), else 0. */
+int cnh_kernel_matches(const cnh_kernel* k, const cnh_ast* ast, int dtype, int ndims);
 int cnh_kernel_release(cnh_kernel* k);
 /* Argument counts in the upstream order: memref per leaf use, scalar per unique broadcast leaf,
  * memref per non-temp root (src/jit.cpp:78-87). */

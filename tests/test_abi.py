@@ -92,6 +92,25 @@ def test_compile_cache_by_key():
     L.check(L.lib.cnh_kernel_release(k2))
 
 
+def test_two_groups_under_one_key_stay_apart():
+    """The cache key is a hash of the AST: a kernel found by key is reused only when it was compiled
+    from that very AST; another group under the same key gets a kernel of its own."""
+    k1 = H.compile_group(H.ast_c1(L.F64), L.F64, 1, key=0x5150)
+    other = AstBuilder(L.F64, 1)
+    other.binary(L.OP_MUL, 10, other.leaf(0), other.scalar(3.0), is_temp=False)
+    ast2 = other.finish()
+    k2 = H.compile_group(ast2, L.F64, 1, key=0x5150)
+    assert k1.value != k2.value
+    same, c1 = H.ast_c1(L.F64), H.ast_c1(L.F64)
+    assert L.lib.cnh_kernel_matches(k1, C.byref(same), L.F64, 1) == 1
+    assert L.lib.cnh_kernel_matches(k2, C.byref(c1), L.F64, 1) == 0
+    assert L.lib.cnh_kernel_matches(k2, C.byref(ast2), L.F64, 1) == 1
+    assert L.lib.cnh_kernel_matches(k2, C.byref(ast2), L.F32, 1) == 0       # another element type
+    assert "0x1.8p+1" in H.kernel_source(k2, "prelude")          # times three, not the first group
+    L.check(L.lib.cnh_kernel_release(k1))
+    L.check(L.lib.cnh_kernel_release(k2))
+
+
 def test_uncompilable_groups_report_an_error():
     b = AstBuilder(L.I64, 1)
     b.unary(L.OP_EXP, 2, b.leaf(0), is_temp=False)

@@ -531,3 +531,20 @@ def test_reductions_fused_into_their_producer(itf, small_tiles, fusion, shape):
         assert close(dot.get(itf).item(), hz * hx)
     fused = [ln for ln in itf.trace() if "path=dense+reduce" in ln]
     assert len(fused) == (1 if fusion else 0)
+
+
+def test_slices_of_another_rank_are_assigned_through_a_copy(itf):
+    """`A[2] = u[0:16]` (a slice of a 1-D array into a row of a matrix) and a column slice into a
+    vector: the slice is copied out, then assigned like a whole array of that rank."""
+    rng = np.random.default_rng(12)
+    hA, hu, hB = rng.standard_normal((6, 16)), rng.standard_normal(40), rng.standard_normal((16, 5))
+    A, u, B = cnp.array(hA), cnp.array(hu), cnp.array(hB)
+    A[2] = u[3:19]
+    hA[2] = hu[3:19]
+    v = cnp.zeros(16)
+    hv = np.zeros(16)
+    v[:] = B[:, 1:2]
+    hv[:] = hB[:, 1]
+    A[4, 2:10] = u[30:38] * 2.0
+    hA[4, 2:10] = hu[30:38] * 2.0
+    assert np.array_equal(A.get(itf), hA) and np.array_equal(v.get(itf), hv)
