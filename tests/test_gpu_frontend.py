@@ -2,6 +2,8 @@
 and the HIP kernels, and compared with NumPy evaluating the same statements in the same order.
 The first block restates the cases of upstream's integration tests
 (tests/test_backend_integration.py upstream) and of its self-checking example scripts."""
+import os
+
 import numpy as np
 import pytest
 
@@ -530,7 +532,9 @@ def test_reductions_fused_into_their_producer(itf, small_tiles, fusion, shape):
     if dot is not None:
         assert close(dot.get(itf).item(), hz * hx)
     fused = [ln for ln in itf.trace() if "path=dense+reduce" in ln]
-    assert len(fused) == (1 if fusion else 0)
+    # with decomposition planning forced on (CHARMNUMERIC_SOLVER=1) nodes run one by one
+    planning = os.environ.get("CHARMNUMERIC_SOLVER", "0") not in ("", "0")
+    assert len(fused) == (1 if fusion and not planning else 0)
 
 
 def test_slices_of_another_rank_are_assigned_through_a_copy(itf):
