@@ -104,11 +104,13 @@ def _launch1(L, k, nd, ins, scalars, outs, stream=None):
 def cg_asts(L):
     """The element-wise part of one CG iteration as two groups. The scalar statements
     (alpha = r.r / p.Ap, beta = r.r_new / r.r) are formed in registers by the group that uses them,
-    from the two reduction results it reads as run-time scalars, so an iteration is five launches
-    (matvec, dot, x and r together, dot, p) instead of eight.
+    and r.r_new is taken by the launch that produces r_new: it leaves one partial sum per wavefront,
+    which the p update sums (every workgroup in the same order) and stores for the next iteration.
+    An iteration is four launches (matvec, dot, x and r, p) instead of eight.
     Group 1 (leaves 1 = p, 2 = x, 3 = Ap, 4 = r; scalars 5 = r.r, 6 = p.Ap):
-        7 = x + alpha p, 8 = r - alpha Ap.   Group 2 (leaves 1 = p, 2 = r_new; scalars 5 = r.r_new,
-    6 = r.r): 7 = r_new + beta p."""
+        7 = x + alpha p, 8 = r - alpha Ap, 9 = sum of (8)^2 as partial sums.
+    Group 2 (leaves 1 = p, 2 = r_new; scalars 5 = r.r_new given as those partial sums, 6 = r.r):
+        7 = r_new + beta p."""
     from charmnumeric_amd.astbuild import AstBuilder
 
     def update_x_r():
@@ -117,7 +119,8 @@ def cg_asts(L):
         t1 = b.binary(L.OP_MUL, 101, alpha, b.leaf(1))
         b.binary(L.OP_ADD, 7, b.leaf(2), t1, is_temp=False)
         t2 = b.binary(L.OP_MUL, 102, alpha, b.leaf(3))
-        b.binary(L.OP_SUB, 8, b.leaf(4), t2, is_temp=False)
+        r_new = b.binary(L.OP_SUB, 8, b.leaf(4), t2, is_temp=False)
+        b.unary(L.OP_SUM_OF, 9, b.binary(L.OP_MUL, 103, r_new, r_new), is_temp=False)
         return b.finish()
 
     def update_p():
@@ -132,25 +135,27 @@ def cg_asts(L):
 
 def prepare_launch(L, k, nd, ins, scalars, outs, stream=None):
     """A launch of group kernel `k` over one partition, put together once: memrefs by leaf name,
-    device addresses of run-time scalars by name, memrefs by output name. Returns what fires it."""
+    run-time scalars by name (a device address, or (address, count, where the sum goes) for one that
+    is given as partial sums), memrefs by output name. Returns what fires it."""
     n_in, n_sc, n_out = C.c_int(), C.c_int(), C.c_int()
     L.check(L.lib.cnh_kernel_signature(k, C.byref(n_in), C.byref(n_sc), C.byref(n_out)))
     name, has, tgt, sr = C.c_int(), C.c_int(), C.c_int(), C.c_int()
     reg = L.Region()
     ia = (L.Memref * max(1, n_in.value))()
     oa = (L.Memref * max(1, n_out.value))()
-    sp = (C.c_void_p * max(1, n_sc.value))()
+    sp = (L.ScalarSum * max(1, n_sc.value))()
     for i in range(n_in.value):
         L.check(L.lib.cnh_kernel_input(k, i, C.byref(name), C.byref(has), C.byref(reg)))
         ia[i] = ins[name.value]
     for i in range(n_sc.value):
         L.check(L.lib.cnh_kernel_scalar(k, i, C.byref(name)))
-        sp[i] = scalars[name.value]
+        what = scalars[name.value]
+        sp[i].ptr, sp[i].count, sp[i].folded = what if isinstance(what, tuple) else (what, 1, None)
     for i in range(n_out.value):
         L.check(L.lib.cnh_kernel_output(k, i, C.byref(name), C.byref(tgt), C.byref(sr), C.byref(reg)))
         oa[i] = outs[name.value]
     n_i, n_s, n_o = n_in.value, n_sc.value, n_out.value
-    return lambda: L.check(L.lib.cnh_launch_group(k, nd, n_i, ia, n_s, sp, 1, n_o, oa, stream))
+    return lambda: L.check(L.lib.cnh_launch_group_sums(k, nd, n_i, ia, n_s, sp, n_o, oa, stream))
 
 
 def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True, trace_iters=0):
@@ -173,6 +178,9 @@ def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True, trace_i
     x2, r2, p2 = vec(), vec(), vec()
     L.check(L.lib.cnh_fill_uniform(bvec.ptr, n, seed, 1, 0, -1.0, 1.0, None))
     sc = Buf(L, 8 * 8, zero=True)  # slot 0 / 3: r.r of the current / next iterate (swapping), 1: p.Ap
+    # partial sums of r_new . r_new, one per wavefront of the launch that updates r (rest stays 0)
+    n_partials = 4 * ((n + 511) // 512)
+    partials = Buf(L, n_partials * 8, zero=True)
     S = lambda i: sc.ptr + 8 * i
     k_xr, k_p = (_compile(L, a, L.F64, 1) for a in cg_asts(L))
     mr = lambda b_, cnt=n: L.Memref.dense(b_.ptr, (cnt,))
@@ -185,9 +193,12 @@ def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True, trace_i
         forms.append({
             "p": cur["p"], "x_new": nxt["x"], "rtr": cur["rtr"], "rtr_new": nxt["rtr"], "r_new": nxt["r"],
             "update_x_r": prepare_launch(L, k_xr, 1, {1: mr(cur["p"]), 2: mr(cur["x"]), 3: mr(Ap), 4: mr(cur["r"])},
-                                         {5: S(cur["rtr"]), 6: S(1)}, {7: mr(nxt["x"]), 8: mr(nxt["r"])}),
+                                         {5: S(cur["rtr"]), 6: S(1)},
+                                         {7: mr(nxt["x"]), 8: mr(nxt["r"]),
+                                          9: L.Memref.dense(partials.ptr, (n_partials,))}),
             "update_p": prepare_launch(L, k_p, 1, {1: mr(cur["p"]), 2: mr(nxt["r"])},
-                                       {5: S(nxt["rtr"]), 6: S(cur["rtr"])}, {7: mr(nxt["p"])}),
+                                       {5: (partials.ptr, n_partials, S(nxt["rtr"])), 6: S(cur["rtr"])},
+                                       {7: mr(nxt["p"])}),
         })
     state = {"parity": 0}
 
@@ -207,9 +218,8 @@ def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True, trace_i
         if ev is not None:
             L.check(L.lib.cnh_event_record(ev.b[i], None))
         L.check(L.lib.cnh_dot_partial(L.F64, n, f["p"].ptr, Ap.ptr, S(1), None))
-        f["update_x_r"]()                      # x + alpha p, r - alpha Ap
-        L.check(L.lib.cnh_dot_partial(L.F64, n, f["r_new"].ptr, f["r_new"].ptr, S(f["rtr_new"]), None))
-        f["update_p"]()                        # r_new + beta p
+        f["update_x_r"]()                      # x + alpha p, r - alpha Ap, partial sums of r_new . r_new
+        f["update_p"]()                        # r.r_new summed and stored, r_new + beta p
         state["parity"] ^= 1
 
     def current():
@@ -263,7 +273,7 @@ def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True, trace_i
         "trace": trace,
     }
     ev.free()
-    for b_ in tiles + [bvec, x, r, p, Ap, x2, r2, p2, sc]:
+    for b_ in tiles + [bvec, x, r, p, Ap, x2, r2, p2, sc, partials]:
         b_.free()
     return res
 
@@ -1134,7 +1144,9 @@ def main():
         "dtype": "f64",
         "data": "synthetic",
         "config": {"workload": f"dense CG, n={n}, A in {cg['tile']}^2 row-major tiles, one CG "
-                               "iteration per step (matvec, 2 dots, 2 scalar ops, 3 fused updates)",
+                               "iteration per step (matvec, 2 dots, 2 scalar ops, 3 updates) in four launches: "
+                               "matvec; p.Ap; x and r with alpha formed in registers and r.r taken on the way; "
+                               "p with beta formed in registers",
                    "device": name.value.decode()},
         "roofline": {"bound": "hbm", "kernel": "gemv_rows<double>", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),

@@ -84,6 +84,12 @@ class GemmJob(C.Structure):
                 ("B", C.c_void_p), ("ldb", C.c_int64), ("C", C.c_void_p), ("ldc", C.c_int64)]
 
 
+class ScalarSum(C.Structure):
+    """cnh_scalar_sum: a run-time scalar given as `count` partial sums at `ptr`."""
+
+    _fields_ = [("ptr", C.c_void_p), ("count", C.c_int64), ("folded", C.c_void_p)]
+
+
 class Memref(C.Structure):
     _fields_ = [
         ("allocated", C.c_void_p),
@@ -200,6 +206,8 @@ _PROTOS = {
     "cnh_scalar_to_dtype": (C.c_int, [C.c_int, C.c_double, C.c_void_p]),
     "cnh_compile_group": (C.c_int, [C.POINTER(Ast), C.c_int, C.c_int, C.c_uint64, _vpp]),
     "cnh_kernel_release": (C.c_int, [C.c_void_p]),
+    "cnh_launch_group_sums": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int,
+                                        C.c_void_p, C.c_void_p]),
     "cnh_kernel_matches": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int]),
     "cnh_kernel_signature": (C.c_int, [C.c_void_p, C.POINTER(C.c_int), C.POINTER(C.c_int),
                                        C.POINTER(C.c_int)]),

@@ -393,7 +393,7 @@ std::string flat_source(const GroupProgram& p) {
 // launches whose traffic exceeds what the last-level cache could keep anyway.
 // Outputs in RED_MASK are not stored: every lane folds its elements' values into racc[], the
 // wavefront combines the lanes in a fixed order, and lane 0 writes one partial per reduction into
-// slots[q * slot_stride + 4 * blockIdx.x + wavefront] for the host to fold.
+// ro.slots[q][4 * blockIdx.x + wavefront] for the host (or a later launch) to fold.
 struct Seg { i64 n; i64 blk0; const T* in[NLA]; T* out[NOA]; };
 typedef T TV __attribute__((ext_vector_type(VECW)));
 #define OUT_STORED(j) (((RED_MASK >> (j)) & 1u) == 0u)
@@ -462,7 +462,8 @@ __device__ __forceinline__ void flat_scalar(const Seg& sg, i64 blk, const T* s, 
 }
 
 #if NR > 0
-__device__ __forceinline__ void red_finish(T* racc, T* slots, i64 slot_stride) {
+struct RedOut { T* slots[NRA]; };
+__device__ __forceinline__ void red_finish(T* racc, const RedOut& ro) {
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) {
         T other[NRA];
@@ -473,17 +474,45 @@ __device__ __forceinline__ void red_finish(T* racc, T* slots, i64 slot_stride) {
     if ((threadIdx.x & 63) == 0) {
 #pragma unroll
         for (int q = 0; q < NR; ++q)
-            slots[q * slot_stride + 4 * (i64)blockIdx.x + (threadIdx.x >> 6)] = racc[q];
+            ro.slots[q][4 * (i64)blockIdx.x + (threadIdx.x >> 6)] = racc[q];
     }
 }
-#define RED_PARAM , T* slots, i64 slot_stride
+#define RED_PARAM , RedOut ro
 #define RED_BEGIN T racc[NRA]; for (int q = 0; q < NRA; ++q) racc[q] = 0;
-#define RED_END red_finish(racc, slots, slot_stride);
+#define RED_END red_finish(racc, ro);
 #else
 #define RED_PARAM
 #define RED_BEGIN T* racc = nullptr;
 #define RED_END
 #endif
+
+// Run-time scalars that are given as partial sums (what a reducing launch left behind): scalar i is
+// the sum of n[i] values at sc.p[i], taken by every workgroup in the same fixed order (lane-strided
+// running sums, butterfly over the wavefront, the four wavefronts left to right), so all workgroups
+// compute with the same bits; workgroup 0 also stores it at out[i] when that is not null.
+struct Fold { T* out[NSA]; int n[NSA]; };
+__device__ __forceinline__ void load_scalars_folding(const Scal& sc, const Fold& fd, T* s) {
+    __shared__ T fold_lds[4];
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+        if (sc.p[i] == nullptr) {
+            s[i] = sc.v[i];
+        } else if (fd.n[i] <= 1) {
+            s[i] = *sc.p[i];
+        } else {
+            T v = 0;
+            for (int j = threadIdx.x; j < fd.n[i]; j += 256) v += sc.p[i][j];
+#pragma unroll
+            for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+            if ((threadIdx.x & 63) == 0) fold_lds[threadIdx.x >> 6] = v;
+            __syncthreads();
+            v = ((fold_lds[0] + fold_lds[1]) + fold_lds[2]) + fold_lds[3];
+            __syncthreads();
+            s[i] = v;
+            if (fd.out[i] != nullptr && blockIdx.x == 0 && threadIdx.x == 0) *fd.out[i] = v;
+        }
+    }
+}
 
 #define FLAT_ENTRY(NAME, CALL)                                                                   \
 extern "C" __global__ __launch_bounds__(256) void grp_flat_##NAME(const Seg* segs, int nseg,    \
@@ -498,6 +527,14 @@ extern "C" __global__ __launch_bounds__(256) void grp_flat_##NAME(const Seg* seg
 }                                                                                                \
 extern "C" __global__ __launch_bounds__(256) void grp_flat1_##NAME(Seg sg, Scal sc RED_PARAM) { \
     T s[NSA]; load_scalars(sc, s);                                                               \
+    RED_BEGIN                                                                                    \
+    const i64 blk = (i64)blockIdx.x;                                                             \
+    CALL;                                                                                        \
+    RED_END                                                                                      \
+}                                                                                                \
+extern "C" __global__ __launch_bounds__(256) void grp_flat1f_##NAME(Seg sg, Scal sc, Fold fd    \
+                                                                    RED_PARAM) {                 \
+    T s[NSA]; load_scalars_folding(sc, fd, s);                                                   \
     RED_BEGIN                                                                                    \
     const i64 blk = (i64)blockIdx.x;                                                             \
     CALL;                                                                                        \

@@ -59,8 +59,8 @@ int reduce_workspace(hipStream_t s, size_t bytes, void** out);
 // The buffer behind `slots` holds n + kFoldRuns doubles: the fold keeps its run sums behind them.
 constexpr int64_t kFoldRuns = 1024;
 constexpr int kFoldMaxVectors = 4;
-int reduce_slots_f64_many(int nvec, const int* maximum, double* slots, int64_t n, int64_t stride,
-                          double* const* outs, hipStream_t st);
+int reduce_slots_f64_many(int nvec, const int* maximum, double* const* vecs, int64_t n, double* const* outs,
+                          hipStream_t st);
 int reduce_slots_f64(bool maximum, double* slots, int64_t n, double* out, hipStream_t st);
 
 // Descriptor tables (per-partition pointers/shapes) live on the device. Identical tables are

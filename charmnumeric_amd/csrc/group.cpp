@@ -334,9 +334,14 @@ int cnh_kernel_build(cnh_kernel* k, const char* variant) {
     return build_variant(k, variant, &v);
 }
 
-int cnh_launch_group_batched(cnh_kernel* k, int ndims, int n_parts, int n_in, const cnh_memref* in,
-                             int n_scalar, const void* const* scalars, int scalars_on_device,
-                             int n_out, const cnh_memref* out, cnh_stream s) {
+} // extern "C"
+
+namespace {
+// The memref launch. `sums` (or null): per run-time scalar, how many partial sums stand behind its
+// address and where the folded value is to be stored.
+int launch_group_impl(cnh_kernel* k, int ndims, int n_parts, int n_in, const cnh_memref* in,
+                      int n_scalar, const void* const* scalars, int scalars_on_device,
+                      const cnh_scalar_sum* sums, int n_out, const cnh_memref* out, cnh_stream s) {
     if (int rc = ensure_init())
         return rc;
     CNH_CHECK(k != nullptr, -2, "null kernel");
@@ -440,17 +445,72 @@ int cnh_launch_group_batched(cnh_kernel* k, int ndims, int n_parts, int n_in, co
         hipFunction_t fn;
         if (int rc = get_function(k, "flat", name.c_str(), &fn))
             return rc;
-        // reducing roots: one partial per wavefront and reduction, folded after the launch
-        void* slots = nullptr;
+        // Reducing roots: one partial per wavefront and reduction. A reduction whose output memref
+        // names more than one element keeps its partials there (the caller, or a later launch that
+        // takes them as a summed scalar, folds them; entries past the last wavefront are left as
+        // they are). The others go to the stream's workspace and are folded right after the launch.
         const int64_t nslots = 4 * blocks;
-        int64_t slot_stride = nslots + kFoldRuns;     // the fold keeps its run sums behind each vector
+        void* red_slots[kFoldMaxVectors] = {nullptr, nullptr, nullptr, nullptr};
+        int maximum[kFoldMaxVectors] = {0, 0, 0, 0}, n_fold = 0;
+        double* fold_vec[kFoldMaxVectors] = {nullptr, nullptr, nullptr, nullptr};
+        double* fold_out[kFoldMaxVectors] = {nullptr, nullptr, nullptr, nullptr};
         if (n_red > 0) {
             CNH_CHECK(p.dtype == CNH_F64, -27, "reducing roots need an fp64 group");
-            if (int rc = reduce_workspace(st, (size_t)(slot_stride * n_red) * sizeof(double), &slots))
-                return rc;
+            const cnh_memref* po = out + (size_t)live[0] * n_out;
+            int kept = 0, q = 0;
+            for (int o = 0; o < n_out; ++o)
+                if (p.out_reduce[(size_t)o]) {
+                    int64_t room = 1;
+                    for (int d = 0; d < ndims; ++d)
+                        room *= po[o].sizes[d];
+                    if (room > 1) {
+                        CNH_CHECK(room >= nslots, -4, "output %d has room for %lld partial results, the launch "
+                                  "leaves %lld", o, (long long)room, (long long)nslots);
+                        red_slots[q] = reinterpret_cast<void*>((uintptr_t)base_ptr(po[o]));
+                        ++kept;
+                    }
+                    ++q;
+                }
+            if (kept < n_red) {
+                const int64_t stride = nslots + kFoldRuns;   // the fold keeps its run sums behind each vector
+                void* ws = nullptr;
+                if (int rc = reduce_workspace(st, (size_t)(stride * (n_red - kept)) * sizeof(double), &ws))
+                    return rc;
+                q = 0;
+                for (int o = 0; o < n_out; ++o)
+                    if (p.out_reduce[(size_t)o]) {
+                        if (red_slots[q] == nullptr) {
+                            red_slots[q] = static_cast<double*>(ws) + stride * n_fold;
+                            maximum[n_fold] = p.out_reduce[(size_t)o] == 2;
+                            fold_vec[n_fold] = static_cast<double*>(red_slots[q]);
+                            fold_out[n_fold] = reinterpret_cast<double*>((uintptr_t)base_ptr(po[o]));
+                            ++n_fold;
+                        }
+                        ++q;
+                    }
+            }
         }
-        if (live.size() == 1) {
-            void* params[] = {segs.data(), scal.data(), &slots, &slot_stride};
+        if (sums != nullptr) {
+            CNH_CHECK(live.size() == 1, -28, "summed scalars go with launches over one partition");
+            const int NS = (int)p.bcast_nodes.size(), NSA = NS > 0 ? NS : 1;
+            // Fold { T* out[NSA]; int n[NSA]; } as the generated code lays it out
+            std::vector<unsigned char> fold(((size_t)NSA * 12 + 7) & ~size_t(7), 0);
+            for (int i = 0; i < NS; ++i) {
+                CNH_CHECK(sums[i].count >= 1 && sums[i].count <= (1 << 20), -4,
+                          "scalar %d: %lld partial sums", i, (long long)sums[i].count);
+                const void* fo = sums[i].folded;
+                const int32_t cnt = (int32_t)sums[i].count;
+                std::memcpy(&fold[(size_t)i * 8], &fo, 8);
+                std::memcpy(&fold[(size_t)NSA * 8 + (size_t)i * 4], &cnt, 4);
+            }
+            hipFunction_t ffn;
+            if (int rc = get_function(k, "flat", (std::string("grp_flat1f_") + suffix).c_str(), &ffn))
+                return rc;
+            void* params[] = {segs.data(), scal.data(), fold.data(), red_slots};
+            if (int rc = launch(ffn, blocks, params, st))
+                return rc;
+        } else if (live.size() == 1) {
+            void* params[] = {segs.data(), scal.data(), red_slots};
             if (int rc = launch(fn, blocks, params, st))
                 return rc;
         } else {
@@ -458,24 +518,15 @@ int cnh_launch_group_batched(cnh_kernel* k, int ndims, int n_parts, int n_in, co
             if (int rc = desc_upload(segs.data(), segs.size() * 8, st, &dsegs))
                 return rc;
             int nseg = (int)live.size();
-            void* params[] = {&dsegs, &nseg, scal.data(), &slots, &slot_stride};
+            void* params[] = {&dsegs, &nseg, scal.data(), red_slots};
             if (int rc = launch(fn, blocks, params, st))
                 return rc;
         }
-        if (n_red == 0)
+        if (n_fold == 0)
             return 0;
-        int maximum[kFoldMaxVectors] = {0, 0, 0, 0};
-        double* outs[kFoldMaxVectors] = {nullptr, nullptr, nullptr, nullptr};
-        int q = 0;
-        const cnh_memref* po = out + (size_t)live[0] * n_out;
-        for (int o = 0; o < n_out; ++o)
-            if (p.out_reduce[(size_t)o]) {
-                maximum[q] = p.out_reduce[(size_t)o] == 2;
-                outs[q] = reinterpret_cast<double*>((uintptr_t)base_ptr(po[o]));
-                ++q;
-            }
-        return reduce_slots_f64_many(n_red, maximum, static_cast<double*>(slots), nslots, slot_stride, outs, st);
+        return reduce_slots_f64_many(n_fold, maximum, fold_vec, nslots, fold_out, st);
     }
+    CNH_CHECK(sums == nullptr, -28, "summed scalars need dense, equally laid out operands");
     CNH_CHECK(n_red == 0, -28, "a group with reducing roots needs dense, equally laid out operands");
 
     // Strided cells.
@@ -538,6 +589,26 @@ int cnh_launch_group_batched(cnh_kernel* k, int ndims, int n_parts, int n_in, co
     int ncell = (int)live.size();
     void* params[] = {&dcells, &ncell, scal.data()};
     return launch(fn, blocks, params, st);
+}
+
+} // namespace
+
+extern "C" {
+
+int cnh_launch_group_batched(cnh_kernel* k, int ndims, int n_parts, int n_in, const cnh_memref* in,
+                             int n_scalar, const void* const* scalars, int scalars_on_device,
+                             int n_out, const cnh_memref* out, cnh_stream s) {
+    return launch_group_impl(k, ndims, n_parts, n_in, in, n_scalar, scalars, scalars_on_device, nullptr,
+                             n_out, out, s);
+}
+
+int cnh_launch_group_sums(cnh_kernel* k, int ndims, int n_in, const cnh_memref* in, int n_scalar,
+                          const cnh_scalar_sum* scalars, int n_out, const cnh_memref* out, cnh_stream s) {
+    CNH_CHECK(n_scalar == 0 || scalars != nullptr, -2, "null scalars");
+    std::vector<const void*> ptrs((size_t)std::max(1, n_scalar), nullptr);
+    for (int i = 0; i < n_scalar; ++i)
+        ptrs[(size_t)i] = scalars[i].ptr;
+    return launch_group_impl(k, ndims, 1, n_in, in, n_scalar, ptrs.data(), 1, scalars, n_out, out, s);
 }
 
 int cnh_launch_group(cnh_kernel* k, int ndims, int n_in, const cnh_memref* in, int n_scalar,

@@ -409,17 +409,17 @@ __global__ __launch_bounds__(kThreads) void fold_slots_runs(const double* __rest
         runs[blockIdx.x] = v;
 }
 
-// Several slot vectors at once (vector q at slots + q * stride, blockIdx.y = q), each a sum or a
-// maximum: the reductions a group kernel carried along are folded by the same one or two launches.
+// Several slot vectors at once (blockIdx.y picks the vector), each a sum or a maximum: the
+// reductions a group kernel carried along are folded by the same one or two launches.
 struct FoldMany {
+    double* vec[kFoldMaxVectors];
     double* out[kFoldMaxVectors];
     int maximum[kFoldMaxVectors];
 };
-__global__ __launch_bounds__(kThreads) void fold_many_runs(double* __restrict__ slots, int64_t n,
-                                                           int64_t stride, int64_t per, FoldMany f) {
+__global__ __launch_bounds__(kThreads) void fold_many_runs(int64_t n, int64_t per, FoldMany f) {
     __shared__ double lds[kThreads / 64];
     const int q = blockIdx.y;
-    const double* __restrict__ src = slots + (int64_t)q * stride;
+    const double* __restrict__ src = f.vec[q];
     const bool maxv = f.maximum[q] != 0;
     const int64_t lo = (int64_t)blockIdx.x * per, hi = lo + per < n ? lo + per : n;
     double v = 0.0;
@@ -429,13 +429,12 @@ __global__ __launch_bounds__(kThreads) void fold_many_runs(double* __restrict__ 
     }
     v = maxv ? block_reduce<double, M_MAXABS_DIFF, kThreads>(v, lds) : block_reduce<double, M_SUM, kThreads>(v, lds);
     if (threadIdx.x == 0)
-        slots[(int64_t)q * stride + n + blockIdx.x] = v;
+        f.vec[q][n + blockIdx.x] = v;
 }
-__global__ __launch_bounds__(1024) void fold_many(const double* __restrict__ slots, int64_t first,
-                                                  int64_t count, int64_t stride, FoldMany f) {
+__global__ __launch_bounds__(1024) void fold_many(int64_t first, int64_t count, FoldMany f) {
     __shared__ double lds[1024 / 64];
     const int q = blockIdx.y;
-    const double* __restrict__ src = slots + (int64_t)q * stride + first;
+    const double* __restrict__ src = f.vec[q] + first;
     const bool maxv = f.maximum[q] != 0;
     double v = 0.0;
     for (int64_t i = threadIdx.x; i < count; i += 1024) {
@@ -449,14 +448,14 @@ __global__ __launch_bounds__(1024) void fold_many(const double* __restrict__ slo
 } // namespace
 
 namespace cnh {
-// Vector q occupies slots[q * stride, q * stride + n); stride >= n + kFoldRuns.
-int reduce_slots_f64_many(int nvec, const int* maximum, double* slots, int64_t n, int64_t stride,
-                          double* const* outs, hipStream_t st) {
-    CNH_CHECK(slots != nullptr && outs != nullptr && n >= 1 && nvec >= 1 && nvec <= kFoldMaxVectors &&
-                  stride >= n + kFoldRuns,
-              -2, "reduce_slots_f64_many: bad arguments");
+// Every vector holds n entries with room for kFoldRuns more behind them.
+int reduce_slots_f64_many(int nvec, const int* maximum, double* const* vecs, int64_t n, double* const* outs,
+                          hipStream_t st) {
+    CNH_CHECK(vecs != nullptr && outs != nullptr && n >= 1 && nvec >= 1 && nvec <= kFoldMaxVectors, -2,
+              "reduce_slots_f64_many: bad arguments");
     FoldMany f;
     for (int q = 0; q < kFoldMaxVectors; ++q) {
+        f.vec[q] = q < nvec ? vecs[q] : nullptr;
         f.out[q] = q < nvec ? outs[q] : nullptr;
         f.maximum[q] = q < nvec ? maximum[q] : 0;
     }
@@ -465,13 +464,12 @@ int reduce_slots_f64_many(int nvec, const int* maximum, double* slots, int64_t n
         int64_t per = (n + kFoldRuns - 1) / kFoldRuns;
         per = (per + 1023) / 1024 * 1024;               // whole passes of a workgroup
         const int64_t runs = (n + per - 1) / per;
-        hipLaunchKernelGGL(fold_many_runs, dim3((unsigned)runs, (unsigned)nvec), dim3(kThreads), 0, st, slots, n,
-                           stride, per, f);
+        hipLaunchKernelGGL(fold_many_runs, dim3((unsigned)runs, (unsigned)nvec), dim3(kThreads), 0, st, n, per, f);
         CNH_HIP(hipGetLastError());
         first = n;
         count = runs;
     }
-    hipLaunchKernelGGL(fold_many, dim3(1, (unsigned)nvec), dim3(1024), 0, st, slots, first, count, stride, f);
+    hipLaunchKernelGGL(fold_many, dim3(1, (unsigned)nvec), dim3(1024), 0, st, first, count, f);
     CNH_HIP(hipGetLastError());
     return 0;
 }

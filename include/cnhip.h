@@ -196,6 +196,25 @@ int cnh_launch_group(cnh_kernel* k, int ndims, int n_in, const cnh_memref* in, i
 int cnh_launch_group_batched(cnh_kernel* k, int ndims, int n_parts, int n_in, const cnh_memref* in,
                              int n_scalar, const void* const* scalars, int scalars_on_device,
                              int n_out, const cnh_memref* out, cnh_stream s);
+/* Outputs that are CNH_OP_SUM_OF / CNH_OP_MAXABS_OF roots (fp64, dense operands): the memref of such
+ * an output names ONE element, which receives the result over all partitions of the launch, or more
+ * than one, in which case the launch leaves its partial results there (one per wavefront, 4 per 512
+ * elements of a partition, at most as many as the memref has room for) and folds nothing: a later
+ * launch takes them through cnh_launch_group_sums. Elements past the last partial are not written,
+ * so a buffer that starts out as zeros can be summed over its whole length.
+ *
+ * cnh_launch_group with run-time scalars that are sums of partial results (no upstream counterpart:
+ * upstream finishes every reduction in a pass and a contribute of its own,
+ * src/executor_reduce.cpp:60-110). Scalar i is the sum of `count` fp64 values at device address
+ * `ptr` (count 1: the value itself), formed by every workgroup in the same fixed order, and stored at
+ * `folded` too when that is not null. One partition, dense operands. */
+typedef struct cnh_scalar_sum {
+    const void* ptr;
+    int64_t count;
+    void* folded;
+} cnh_scalar_sum;
+int cnh_launch_group_sums(cnh_kernel* k, int ndims, int n_in, const cnh_memref* in, int n_scalar,
+                          const cnh_scalar_sum* scalars, int n_out, const cnh_memref* out, cnh_stream s);
 
 /* Shifted-slice groups over tiles that all live on this device: replaces send_remote_input +
  * receive_data + align_fragments + M kernel calls + the SET_REGION copy

@@ -120,3 +120,56 @@ def test_reducing_roots_need_dense_operands(dev):
     with pytest.raises(L.CnhError):
         H.compile_group(bad.finish(), L.I32, 1)
     dev.free_all()
+
+
+def test_partials_left_by_one_launch_are_summed_by_the_next(dev):
+    """A reducing output with room for many elements keeps the launch's partial results; a later
+    launch takes their sum as a run-time scalar, stores it, and computes with it."""
+    n, room = 5000, 256
+    rng = np.random.default_rng(3)
+    hx, hy = rng.standard_normal(n), rng.standard_normal(n)
+    p = AstBuilder(L.F64, 1)
+    z = p.binary(L.OP_MUL, 10, p.leaf(0), p.scalar(2.0), is_temp=False)
+    p.unary(L.OP_SUM_OF, 20, p.binary(L.OP_MUL, 100, z, z), is_temp=False)
+    kp = H.compile_group(p.finish(), L.F64, 1)
+    c = AstBuilder(L.F64, 1)
+    t = c.binary(L.OP_MUL, 100, c.leaf(0), c.broadcast(5))
+    c.binary(L.OP_ADD, 10, t, c.broadcast(6), is_temp=False)
+    kc = H.compile_group(c.finish(), L.F64, 1)
+
+    x, y = dev.array(hx), dev.array(hy)
+    zb, ob = dev.empty((n,), np.float64), dev.empty((n,), np.float64)
+    partials = dev.array(np.zeros(room))
+    sc = dev.array(np.array([np.nan, 0.75]))                   # [folded sum, a plain scalar]
+    a, o = bind(kp, {0: x.memref()}, {10: zb.memref(), 20: L.Memref.dense(partials.ptr, (room,))})
+    H.launch_batched(kp, 1, [a], [], [o])
+    hz = hx * 2.0
+    got = partials.get()
+    used = 4 * ((n + 511) // 512)
+    assert np.all(got[used:] == 0.0) and np.count_nonzero(got[:used]) > used // 2
+    assert abs(got.sum() - np.sum(hz * hz)) <= 1e-13 * np.sum(hz * hz)
+
+    # the consumer: out = y * sum(partials) + sc[1]
+    n_in, n_sc, n_out = C.c_int(), C.c_int(), C.c_int()
+    L.check(L.lib.cnh_kernel_signature(kc, C.byref(n_in), C.byref(n_sc), C.byref(n_out)))
+    assert (n_in.value, n_sc.value, n_out.value) == (1, 2, 1)
+    sums = (L.ScalarSum * 2)()
+    name = C.c_int()
+    for i in range(2):
+        L.check(L.lib.cnh_kernel_scalar(kc, i, C.byref(name)))
+        if name.value == 5:
+            sums[i].ptr, sums[i].count, sums[i].folded = partials.ptr, room, sc.ptr
+        else:
+            sums[i].ptr, sums[i].count, sums[i].folded = sc.ptr + 8, 1, None
+    ins = (L.Memref * 1)(y.memref())
+    outs = (L.Memref * 1)(ob.memref())
+    L.check(L.lib.cnh_launch_group_sums(kc, 1, 1, ins, 2, sums, 1, outs, None))
+    folded = sc.get()[0]
+    assert abs(folded - got.sum()) <= 4e-16 * got.sum() * 8
+    assert np.array_equal(ob.get(), hy * folded + 0.75)        # every workgroup used the same bits
+    # too little room for the partial results of a launch is refused
+    small = dev.array(np.zeros(8))
+    a, o = bind(kp, {0: x.memref()}, {10: zb.memref(), 20: L.Memref.dense(small.ptr, (8,))})
+    with pytest.raises(L.CnhError, match="room"):
+        H.launch_batched(kp, 1, [a], [], [o])
+    dev.free_all()
