@@ -1207,6 +1207,18 @@ struct MatView {
         idx[cd] = ac;
         if (dd >= 0)
             idx[dd] = plane;
+        if (a->flat) {
+            // one row-major block: nothing cuts a panel short, whatever the array's partitions are
+            int64_t off = 0;
+            for (int d = 0; d < a->ndims; ++d)
+                off += (int64_t)idx[d] * a->pitch[d];
+            *ld = a->pitch[rd];
+            *rlo = 0;
+            *rhi = a->shape[rd];
+            *clo = 0;
+            *chi = a->shape[cd];
+            return static_cast<const char*>(a->slab) + off * dtype_size(a->dtype);
+        }
         int64_t t = 0;
         for (int d = 0; d < a->ndims; ++d)
             t = t * a->grid[d] + idx[d] / a->tile;
@@ -1283,8 +1295,9 @@ int exec_matmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
             std::to_string(x->name) + " out=" + std::to_string(y->name));
     int rc = 0;
     if (!ex->dry) {
-        // one panel per tile the window meets; panel rows are the array's tile rows
-        const int T = Aa->tile;
+        // one panel per tile the window meets; panel rows are the array's tile rows (an array
+        // stored as one block is a single panel)
+        const int T = Aa->flat ? (1 << 30) : Aa->tile;
         const int pr0 = A.r0 / T, pr1 = (A.r0 + A.rows - 1) / T;
         const int pc0 = A.c0 / T, pc1 = (A.c0 + A.cols - 1) / T;
         std::vector<cnh_gemv_panel> panels;
@@ -1367,7 +1380,9 @@ int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root, const Dag
         if (int rc = make_array(ex, root.result_name, 2, Aa->dtype, shape, !f64, &Cc))
             return rc;
     const int esz = dtype_size(Aa->dtype);
-    const int TA = Aa->tile, TB = Ba->tile, K = A.cols;
+    // panels end where an operand's tiles end; an array stored as one block has no such ends
+    const int kNoCut = 1 << 30;
+    const int TA = Aa->flat ? kNoCut : Aa->tile, TB = Ba->flat ? kNoCut : Ba->tile, K = A.cols;
     int calls = 0;
     std::vector<cnh_gemm_job> jobs;   // all panel products of the node go out as one launch
     const int cgrid0 = Cc ? Cc->grid[0] : 1, cgrid1 = Cc ? Cc->grid[1] : 1;
