@@ -1156,7 +1156,7 @@ def main():
                                "matvec; p.Ap; x and r with alpha formed in registers and r.r taken on the way; "
                                "p with beta formed in registers",
                    "device": name.value.decode()},
-        "roofline": {"bound": "hbm", "kernel": "gemv_rows<double>", "achieved": round(achieved, 1),
+        "roofline": {"bound": "hbm", "kernel": "gemv_rows_xlds<double,8,8,4>", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": GEMV_N16384_TRAFFIC_BYTES if n == 16384 else None,
                      "traffic_source": "rocprofv3 --pmc counters of an earlier run of this kernel "

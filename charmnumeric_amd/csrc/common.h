@@ -61,6 +61,7 @@ constexpr int64_t kFoldRuns = 1024;
 constexpr int kFoldMaxVectors = 4;
 int reduce_slots_f64_many(int nvec, const int* maximum, double* const* vecs, int64_t n, double* const* outs,
                           hipStream_t st);
+void gemv_set_xlds(int on);
 int reduce_slots_f64(bool maximum, double* slots, int64_t n, double* out, hipStream_t st);
 
 // Descriptor tables (per-partition pointers/shapes) live on the device. Identical tables are

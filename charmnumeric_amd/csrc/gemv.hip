@@ -6,6 +6,7 @@
 // matrix is read from HBM exactly once and the per-row sum has a fixed order.
 #include "common.h"
 
+#include <type_traits>
 #include <vector>
 
 using namespace cnh;
@@ -63,7 +64,8 @@ constexpr int kWavesPerBlockDefault = 4;
 // tiles[ti * ncol_tiles + tj]; row r belongs to tile row (r + row_shift) / tile_rows: a window that
 // starts row_shift rows into its first tile row.
 // Measured on MI355X (n = 16384, fp64): 4 loads in flight per lane 326 us, 8: 330-336, 2: 345;
-// 1, 2 or 4 wavefronts per workgroup make no difference, 8 are slower.
+// 1, 2 or 4 wavefronts per workgroup make no difference, 8 are slower. Large products take
+// gemv_rows_xlds below instead.
 template <typename T, bool VEC16, int kWavesPerBlock = 4, int kUnroll = 4>
 __global__ __launch_bounds__(kWavesPerBlock * 64) void gemv_rows(const ColTile* __restrict__ tiles,
                                                                  int ncol_tiles, int64_t tile_rows,
@@ -126,6 +128,94 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void gemv_rows(const ColTile* 
         y[r] = beta ? (T)((A)y[r] + total) : (T)total;
 }
 
+// The same matvec with x staged in LDS. In gemv_rows every wavefront reads all of x for its one row
+// (from L2: as many bytes again as the matrix, and half of all load instructions); here a workgroup
+// of kWaves wavefronts owns kWaves * kRows rows, copies the x of one column tile into LDS (64 KB)
+// and every wavefront streams its rows' parts of that tile against it, column tiles in index
+// order. Per lane the same elements meet in the same order as in gemv_rows, so the results are the
+// same bits. Needs: 128-bit alignment, every column tile at most 64 KB of x wide, and the column
+// tiles cut alike in every tile row.
+constexpr int kXldsBytes = 65536;
+template <typename T, int kWaves, int kRows, int kUnroll>
+__global__ __launch_bounds__(kWaves * 64) void gemv_rows_xlds(const ColTile* __restrict__ tiles, int ncol_tiles,
+                                                              int64_t tile_rows, int64_t rows, int64_t row_shift,
+                                                              const T* __restrict__ x, T* __restrict__ y,
+                                                              int beta) {
+    typedef typename Acc<T>::type A;
+    constexpr int VEC = 16 / sizeof(T);
+    typedef T P __attribute__((ext_vector_type(VEC)));
+    __shared__ __attribute__((aligned(16))) T xs[kXldsBytes / sizeof(T)];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t r0 = ((int64_t)blockIdx.x * kWaves + wave) * kRows;
+    A total[kRows];
+#pragma unroll
+    for (int q = 0; q < kRows; ++q)
+        total[q] = 0;
+    for (int tj = 0; tj < ncol_tiles; ++tj) {
+        const int64_t ncols = tiles[tj].ncols, xoff = tiles[tj].xoff;
+        if (tj > 0)
+            __syncthreads();       // everybody is done with the previous tile's x
+        for (int64_t i = (int64_t)threadIdx.x * VEC; i + VEC <= ncols; i += (int64_t)kWaves * 64 * VEC)
+            *reinterpret_cast<P*>(xs + i) = *reinterpret_cast<const P*>(x + xoff + i);
+        for (int64_t i = ncols / VEC * VEC + threadIdx.x; i < ncols; i += kWaves * 64)
+            xs[i] = x[xoff + i];
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < kRows; ++q) {
+            const int64_t r = r0 + q;
+            if (r >= rows)
+                continue;
+            const int64_t ti = (r + row_shift) / tile_rows;
+            const int64_t lr = r + row_shift - ti * tile_rows;
+            const ColTile ct = tiles[ti * ncol_tiles + tj];
+            const T* row = (const T*)ct.base + lr * ct.ld;
+            A acc[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u)
+                acc[u] = 0;
+            int64_t c = 0;
+            const int64_t step = 64 * VEC;
+            for (; c + kUnroll * step <= ncols; c += kUnroll * step) {
+                P av[kUnroll], xv[kUnroll];
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u)
+                    av[u] = __builtin_nontemporal_load(reinterpret_cast<const P*>(row + c + u * step + lane * VEC));
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u)
+                    xv[u] = *reinterpret_cast<const P*>(xs + c + u * step + lane * VEC);
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e)
+                        acc[u] += (A)av[u][e] * (A)xv[u][e];
+            }
+            for (; c + step <= ncols; c += step) {
+                P av = *reinterpret_cast<const P*>(row + c + lane * VEC);
+                P xv = *reinterpret_cast<const P*>(xs + c + lane * VEC);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e)
+                    acc[0] += (A)av[e] * (A)xv[e];
+            }
+            for (int64_t j = c + lane; j < ncols; j += 64)
+                acc[1] += (A)row[j] * (A)xs[j];
+            A part = 0;
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u)
+                part += acc[u];
+            part = wave_sum<A>(part);
+            total[q] = tj == 0 ? part : total[q] + part; // column tiles added in index order
+        }
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int q = 0; q < kRows; ++q)
+            if (r0 + q < rows)
+                y[r0 + q] = beta ? (T)((A)y[r0 + q] + total[q]) : (T)total[q];
+    }
+}
+
+int g_gemv_xlds = 1;   // 0: always one wavefront per row reading x from cache; 1: the LDS form where it applies
+
 template <typename T>
 __global__ __launch_bounds__(256) void axpy1_kernel(int64_t n, const T* __restrict__ p,
                                                     T* __restrict__ y) {
@@ -147,6 +237,36 @@ int run_gemv(const std::vector<ColTile>& tiles, int ncol_tiles, int64_t tile_row
     const void* dtiles = nullptr;
     if (int rc = desc_upload(tiles.data(), tiles.size() * sizeof(ColTile), st, &dtiles))
         return rc;
+    // x staged in LDS: big aligned products whose column tiles are cut alike in every tile row
+    if (vec && g_gemv_xlds > 0 && rows >= 8192) {
+        bool ok = true;
+        const int64_t tile_rows_used = (int64_t)tiles.size() / ncol_tiles;
+        for (int tj = 0; tj < ncol_tiles && ok; ++tj) {
+            ok = tiles[(size_t)tj].ncols * (int64_t)sizeof(T) <= kXldsBytes;
+            for (int64_t ti = 1; ti < tile_rows_used && ok; ++ti)
+                ok = tiles[(size_t)(ti * ncol_tiles + tj)].ncols == tiles[(size_t)tj].ncols &&
+                     tiles[(size_t)(ti * ncol_tiles + tj)].xoff == tiles[(size_t)tj].xoff;
+        }
+        if (ok) {
+            // 8 wavefronts per workgroup; rows per wavefront so that every CU still gets a workgroup
+            // (n = 16384, fp64: 8 x 8 rows 311 us, 16 x 4 317, 8 x 4 318, 16 x 8 383, one row per
+            // wavefront without LDS 327-333)
+            constexpr int kW = 8;
+            if (rows >= 16384) {
+                const int64_t nb = (rows + kW * 8 - 1) / (kW * 8);
+                hipLaunchKernelGGL((gemv_rows_xlds<T, kW, 8, 4>), dim3((unsigned)nb), dim3(kW * 64), 0, st,
+                                   (const ColTile*)dtiles, ncol_tiles, tile_rows, rows, row_shift, (const T*)x,
+                                   (T*)y, beta);
+            } else {
+                const int64_t nb = (rows + kW * 4 - 1) / (kW * 4);
+                hipLaunchKernelGGL((gemv_rows_xlds<T, kW, 4, 4>), dim3((unsigned)nb), dim3(kW * 64), 0, st,
+                                   (const ColTile*)dtiles, ncol_tiles, tile_rows, rows, row_shift, (const T*)x,
+                                   (T*)y, beta);
+            }
+            CNH_HIP(hipGetLastError());
+            return 0;
+        }
+    }
     constexpr int kWavesPerBlock = kWavesPerBlockDefault;
     int64_t blocks = (rows + kWavesPerBlock - 1) / kWavesPerBlock;
     CNH_CHECK(blocks < (1ll << 31), -3, "matvec with %lld rows is too large for one launch",
@@ -175,6 +295,10 @@ int dispatch_gemv(int dtype, const std::vector<ColTile>& tiles, int ncol_tiles, 
 }
 
 } // namespace
+
+namespace cnh {
+void gemv_set_xlds(int on) { g_gemv_xlds = on; }
+} // namespace cnh
 
 extern "C" {
 

@@ -1288,6 +1288,11 @@ extern "C" int cnh_set_option(const char* name, int value) {
         g_slide_enabled = value == 1;
         return 0;
     }
+    if (std::strcmp(name, "gemv_xlds") == 0) {
+        CNH_CHECK(value == 0 || value == 1, -2, "gemv_xlds: 0 or 1");
+        gemv_set_xlds(value);
+        return 0;
+    }
     if (std::strcmp(name, "direct_lean") == 0) {
         g_direct_lean = value;
         return 0;

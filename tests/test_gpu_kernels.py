@@ -454,3 +454,44 @@ def test_stream_event_and_callback(dev):
     L.check(L.lib.cnh_event_destroy(e1))
     L.check(L.lib.cnh_stream_destroy(s))
     dev.free_all()
+
+
+@pytest.mark.parametrize("rows,widths,dt", [(16400, (2048, 1000), np.float64), (8200, (2048, 1024, 520), np.float64),
+                                             (16384, (3000,), np.float32)])
+def test_large_matvec_with_x_staged_in_lds(dev, orc, rows, widths, dt):
+    """Matvecs of 8192 rows or more keep the vector in LDS, 32 or 64 rows per workgroup. The result
+    has the bits of the one-wavefront-per-row kernel (same elements meet in the same order) and
+    agrees with a float64 NumPy product to the summation bound. Ragged column panels, a row count
+    that is no multiple of the rows per workgroup, two panel rows."""
+    rng = np.random.default_rng(rows)
+    cols = sum(widths)
+    tile_rows = 8192 if rows > 8192 else rows
+    hA = rng.standard_normal((rows, cols)).astype(dt)
+    hx = rng.standard_normal(cols).astype(dt)
+    panels, keep, xoff = [], [], 0
+    n_panel_rows = (rows + tile_rows - 1) // tile_rows
+    for pr in range(n_panel_rows):
+        r0, r1 = pr * tile_rows, min(rows, (pr + 1) * tile_rows)
+        xoff = 0
+        for w in widths:
+            b = dev.array(np.ascontiguousarray(hA[r0:r1, xoff:xoff + w]))
+            keep.append(b)
+            panels.append((b.ptr, w, w, xoff))
+            xoff += w
+    arr = (L.GemvPanel * len(panels))(*[L.GemvPanel(*p) for p in panels])
+    x = dev.array(hx)
+    out = {}
+    for mode in (1, 0):
+        y = dev.array(np.full(rows, -7.0, dtype=dt))
+        L.check(L.lib.cnh_set_option(b"gemv_xlds", mode))
+        try:
+            L.check(L.lib.cnh_gemv_panels(H.DT[np.dtype(dt)], rows, len(widths), tile_rows, 0, len(panels), arr,
+                                          x.ptr, y.ptr, None))
+        finally:
+            L.check(L.lib.cnh_set_option(b"gemv_xlds", 1))
+        out[mode] = y.get()
+    assert np.array_equal(out[0], out[1])
+    exact = hA.astype(np.float64) @ hx.astype(np.float64)
+    bound = (np.abs(hA).astype(np.float64) @ np.abs(hx).astype(np.float64)) * (1e-12 if dt == np.float64 else 2e-5)
+    assert np.all(np.abs(out[1] - exact) <= bound)
+    dev.free_all()
