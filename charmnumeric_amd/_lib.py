@@ -203,6 +203,8 @@ _PROTOS = {
                                   C.c_void_p, C.c_void_p]),
     "cnh_copy_region": (C.c_int, [C.c_int, C.c_int, C.c_void_p, _i64p, _i64p, _i64p, C.c_void_p,
                                   _i64p, _i64p, _i64p, _i64p, C.c_void_p]),
+    "cnh_convert_region": (C.c_int, [C.c_int, C.c_int, C.c_void_p, _i64p, _i64p, _i64p, C.c_int, C.c_void_p,
+                                     _i64p, _i64p, _i64p, _i64p, C.c_void_p]),
     "cnh_scalar_to_dtype": (C.c_int, [C.c_int, C.c_double, C.c_void_p]),
     "cnh_compile_group": (C.c_int, [C.POINTER(Ast), C.c_int, C.c_int, C.c_uint64, _vpp]),
     "cnh_kernel_release": (C.c_int, [C.c_void_p]),

@@ -300,7 +300,7 @@ class _ArrayLike:
             value = _coerce_assignment_operand(rhs, shape, self.dtype)
         if isinstance(value, _ArrayLike):
             if value._wire != base._wire:
-                raise NotImplementedError("assignment across dtypes is not implemented")
+                value = _converted(value, base.dtype)      # NumPy's rule: the target's type wins
             if value.shape != shape:
                 # a lower-rank value fits a region whose extra dimensions have extent 1
                 # (IFOG[t] = M with M 2-D), and a whole higher-rank one whose extra dimensions
@@ -365,9 +365,11 @@ class _ArrayLike:
         self[...] = value
 
     def astype(self, dtype, copy=True):
-        if _normalize_dtype(dtype) != self.dtype:
-            raise NotImplementedError(
-                "dtype conversion for existing charmnumeric arrays is not implemented yet")
+        """Upstream refuses a change of element type (charmnumeric.py:738-744, 842-848); here it is
+        one converting copy on the device (C conversion rules, as numpy.ndarray.astype)."""
+        want = _normalize_dtype(dtype)
+        if want != self.dtype:
+            return _converted(self, want)
         return self.copy() if copy else self
 
 
@@ -497,8 +499,7 @@ def _binary(opcode, lhs, rhs):
         ra = isinstance(rhs, _ArrayLike)
     if la and ra:
         if lhs.dtype != rhs.dtype:
-            raise NotImplementedError(f"elementwise operations across dtypes ({lhs.dtype} and "
-                                      f"{rhs.dtype}) are not implemented")
+            lhs, rhs = _promoted(lhs, rhs)
         # the result takes the shape of the operand with more than one element; a one-element
         # whole array beside it is a run-time scalar
         if lhs._n > 1 and rhs._n > 1:
@@ -585,10 +586,22 @@ def tile(x, reps):
     return nonfusible(L.OP_TILE, [x], tuple(s * r for s, r in zip(shape, reps)), x.dtype)
 
 
-def _same_dtype(a, b, what):
-    if a.dtype != b.dtype:
-        raise NotImplementedError(f"{what} across dtypes ({a.dtype} and {b.dtype}) is not implemented")
-    return a.dtype
+def _converted(x, dtype):
+    """x as a new array of element type `dtype`: one ASTYPE node (slices are copied out first)."""
+    dtype = np.dtype(dtype)
+    src = _whole(x)
+    out = Array(src.shape, dtype)
+    lazy.record_nonfusible(out.name, lazy.OP_ASTYPE, out._wire, out.shape, [src._refb()])
+    return out
+
+
+def _promoted(a, b):
+    """Both operands in np.result_type of their element types, the type upstream gives the result
+    (charmnumeric.py:369-373 upstream). Upstream's kernels then read every operand in that one type
+    whatever it holds (src/jit.cpp:47-69); here the operand of the other type is converted first."""
+    want = _normalize_dtype(np.result_type(a.dtype, b.dtype))
+    return (a if a.dtype == want else _converted(a, want),
+            b if b.dtype == want else _converted(b, want))
 
 
 def _matmul(lhs, rhs):
@@ -598,7 +611,9 @@ def _matmul(lhs, rhs):
     if lhs.ndims == 1 and rhs.ndims == 1:
         if lhs.shape[0] != rhs.shape[0]:
             raise ValueError(f"Shape mismatch for dot product: ({lhs.shape[0]},) @ ({rhs.shape[0]},)")
-        return nonfusible(L.OP_REDUCE, [lhs, rhs], (1,), _same_dtype(lhs, rhs, "dot"))
+        if lhs.dtype != rhs.dtype:
+            lhs, rhs = _promoted(lhs, rhs)
+        return nonfusible(L.OP_REDUCE, [lhs, rhs], (1,), lhs.dtype)
     if lhs.ndims not in (2, 3):
         raise ValueError(f"matmul requires a 2D matrix, got {lhs.ndims}D")
     if rhs.ndims == 1:
@@ -609,7 +624,9 @@ def _matmul(lhs, rhs):
     rr, rc = _matrix_shape(rhs)
     if lc != rr:
         raise ValueError(f"Shape mismatch: ({lr},{lc}) @ ({rr},{rc})")
-    return nonfusible(L.OP_MATMATMUL, [lhs, rhs], (lr, rc), _same_dtype(lhs, rhs, "matmul"))
+    if lhs.dtype != rhs.dtype:
+        lhs, rhs = _promoted(lhs, rhs)
+    return nonfusible(L.OP_MATMATMUL, [lhs, rhs], (lr, rc), lhs.dtype)
 
 
 def _column_as_vector(col):
@@ -652,7 +669,9 @@ def _matvec(mat, vec):
         raise ValueError(f"matvec requires a 2D or 3D matrix, got {mat.ndims}D")
     if cols != vec.shape[0]:
         raise ValueError(f"Shape mismatch: matrix cols {cols} != vector size {vec.shape[0]}")
-    return nonfusible(L.OP_MATMUL, [mat, vec], (rows,), _same_dtype(mat, vec, "matvec"))
+    if mat.dtype != vec.dtype:
+        mat, vec = _promoted(mat, vec)
+    return nonfusible(L.OP_MATMUL, [mat, vec], (rows,), mat.dtype)
 
 
 # ---------------------------------------------------------------------------------------------

@@ -27,7 +27,7 @@ using namespace cnh;
 namespace {
 
 constexpr int kOpDelete = CNX_OP_DELETE, kOpSum = CNX_OP_SUM, kOpSumsqDiff = CNX_OP_SUMSQ_DIFF,
-              kOpMaxabsDiff = CNX_OP_MAXABS_DIFF;
+              kOpMaxabsDiff = CNX_OP_MAXABS_DIFF, kOpAstype = CNX_OP_ASTYPE;
 
 struct Reader {
     const char* p;
@@ -1072,6 +1072,66 @@ int exec_reduce_ext(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
     return rc;
 }
 
+// ASTYPE: a new array of the operand's shape and the node's dtype. One converting strided copy per
+// pair of tiles that meet (the two arrays are cut by the same rule, so unless a plan placed them
+// differently that is one launch per tile, or one for a whole rank-3 block).
+int exec_astype(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
+    XArray* in;
+    if (int rc = leaf_array(ex, n, root, 0, &in, "ASTYPE"))
+        return rc;
+    CNH_CHECK(dtype_size(root.dtype) != 0, -27, "ASTYPE: unknown dtype %d", root.dtype);
+    const int nd = in->ndims;
+    int32_t shape[3] = {1, 1, 1};
+    for (int d = 0; d < nd; ++d)
+        shape[d] = in->shape[d];
+    XArray* out;
+    if (int rc = make_array(ex, root.result_name, nd, root.dtype, shape, false, &out))
+        return rc;
+    if (int rc = find_array(ex, n.nodes[root.operands[0]].result_name, &in, "ASTYPE"))   // the map may have moved it
+        return rc;
+    int launches = 0;
+    const bool blocks = in->flat && out->flat;
+    for (int64_t ot = 0; ot < (blocks ? 1 : out->ntiles); ++ot) {
+        int32_t olo[3] = {0, 0, 0}, oext[3] = {1, 1, 1};
+        if (blocks)
+            for (int d = 0; d < nd; ++d)
+                oext[d] = shape[d];
+        else
+            out->tile_extent(ot, olo, oext);
+        for (int64_t it = 0; it < (blocks ? 1 : in->ntiles); ++it) {
+            int32_t ilo[3] = {0, 0, 0}, iext[3] = {1, 1, 1};
+            if (blocks)
+                for (int d = 0; d < nd; ++d)
+                    iext[d] = shape[d];
+            else
+                in->tile_extent(it, ilo, iext);
+            int64_t dstr[3], sstr[3], dsta[3], ssta[3], one[3] = {1, 1, 1}, counts[3];
+            bool empty = false;
+            for (int d = 0; d < nd; ++d) {
+                const int lo = std::max(olo[d], ilo[d]), hi = std::min(olo[d] + oext[d], ilo[d] + iext[d]);
+                if (hi <= lo)
+                    empty = true;
+                dsta[d] = lo - olo[d];
+                ssta[d] = lo - ilo[d];
+                counts[d] = hi - lo;
+            }
+            if (empty)
+                continue;
+            out->tile_strides(oext, dstr);
+            in->tile_strides(iext, sstr);
+            ++launches;
+            if (!ex->dry)
+                if (int rc = cnh_convert_region(nd, out->dtype, blocks ? out->slab : out->tiles[ot], dstr, dsta, one,
+                                                in->dtype, blocks ? in->slab : in->tiles[it], sstr, ssta, one,
+                                                counts, ex->stream))
+                    return rc;
+        }
+    }
+    ex->log("astype in=" + std::to_string(in->name) + " out=" + std::to_string(out->name) + " dtype=" +
+            std::to_string(out->dtype) + " launches=" + std::to_string(launches));
+    return 0;
+}
+
 // ---- boxes: unit-step regions that are one strided block of device memory ----
 struct BoxUse {
     XArray* arr = nullptr;
@@ -1610,6 +1670,7 @@ int exec_node(Ex* ex, const DagNode& n) {
     case kOpSum:
     case kOpSumsqDiff:
     case kOpMaxabsDiff: return exec_reduce_ext(ex, n, root);
+    case kOpAstype: return exec_astype(ex, n, root);
     case CNH_OP_MATMUL: return exec_matmul(ex, n, root);
     case CNH_OP_MATMATMUL: return exec_matmatmul(ex, n, root);
     case CNH_OP_TILE: return exec_tile(ex, n, root);
@@ -2333,6 +2394,12 @@ void plan_message(Ex* ex, const std::vector<DagNode>& dag) {
         case kOpSum:
         case kOpSumsqDiff:
         case kOpMaxabsDiff: result(root.result_name, 1, shape); break;
+        case kOpAstype: {
+            const DecompMeta* in = known(n, root, 0);
+            if (in)
+                result(root.result_name, in->ndims, in->shape);
+            break;
+        }
         case CNH_OP_MATMUL: {
             int rows, cols;
             const DecompMeta* A = known(n, root, 0);

@@ -25,7 +25,7 @@ import numpy as np
 from . import _lib as L
 
 # Extension opcodes of include/cnexec.h
-OP_DELETE, OP_SUM, OP_SUMSQ_DIFF, OP_MAXABS_DIFF = 100, 101, 102, 103
+OP_DELETE, OP_SUM, OP_SUMSQ_DIFF, OP_MAXABS_DIFF, OP_ASTYPE = 100, 101, 102, 103, 104
 DAG_MAGIC = 0x47444E43
 
 _ELEMENTWISE = {L.OP_ADD, L.OP_SUB, L.OP_MUL, L.OP_DIV, L.OP_TANH, L.OP_EXP, L.OP_COPY}

@@ -56,12 +56,16 @@ extern "C" {
 /* Extension opcodes (no upstream counterpart; upstream has no N-D reduction, no random numbers and
  * no bulk upload: src/executor_reduce.cpp:9-12, charmnumeric/random.py:4-5, charmnumeric.py:863-878).
  * Operand layout: SUM(a); SUMSQ_DIFF(a, b); MAXABS_DIFF(a, b) -> size-1 fp64 array `result_name`,
- * over whole arrays of any rank; DELETE names the array in result_name. */
+ * over whole arrays of any rank; DELETE names the array in result_name; ASTYPE(a) -> a new array
+ * `result_name` of a's shape holding a's values converted to the node's dtype (C conversion rules;
+ * upstream's astype raises, charmnumeric/charmnumeric.py:738-744, and its mixed-dtype operations
+ * only label the result, :369-373). */
 enum {
     CNX_OP_DELETE = 100,
     CNX_OP_SUM = 101,
     CNX_OP_SUMSQ_DIFF = 102,
-    CNX_OP_MAXABS_DIFF = 103
+    CNX_OP_MAXABS_DIFF = 103,
+    CNX_OP_ASTYPE = 104
 };
 
 typedef struct cnx_executor cnx_executor;

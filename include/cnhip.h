@@ -153,6 +153,17 @@ int cnh_copy_region(int ndims, int esz, void* dst, const int64_t* dst_strides,
                     const int64_t* dst_start, const int64_t* dst_step, const void* src,
                     const int64_t* src_strides, const int64_t* src_start, const int64_t* src_step,
                     const int64_t* counts, cnh_stream s);
+/* The strided copy with a change of element type, dst = (dst type)src with C's conversion rules
+ * (to floating point: round to nearest even; to an integer type: truncation towards zero; a
+ * floating-point value outside the integer type's range, or NaN, gives an unspecified integer).
+ * What NumPy's astype computes. Upstream labels the result of an operation between arrays of two
+ * element types with np.result_type (charmnumeric/charmnumeric.py:369-373) but its kernels read
+ * every operand in one element type (src/jit.cpp:47-69) and astype raises
+ * (charmnumeric.py:738-744): this is the conversion those lines leave open. */
+int cnh_convert_region(int ndims, int dst_dtype, void* dst, const int64_t* dst_strides,
+                       const int64_t* dst_start, const int64_t* dst_step, int src_dtype, const void* src,
+                       const int64_t* src_strides, const int64_t* src_start, const int64_t* src_step,
+                       const int64_t* counts, cnh_stream s);
 /* Scalar -> dtype conversion used by the fill ((T)double, src/executor_ast_visitor.cpp:112-147). */
 int cnh_scalar_to_dtype(int dtype, double s, void* out8);
 

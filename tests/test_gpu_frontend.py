@@ -53,6 +53,40 @@ def test_add_on_every_rank(itf, shape):
     assert got.shape == shape and np.array_equal(got, np.full(shape, 2.0, np.float32))
 
 
+@pytest.mark.parametrize("shape", [(1000,), (40, 50), (10, 12, 20)])
+def test_mixed_element_types_promote_like_numpy(small_tiles, shape):
+    """Upstream labels such results with np.result_type (charmnumeric.py:369-373); NumPy evaluating
+    the same statements is the answer the label promises."""
+    itf = small_tiles
+    rng = np.random.default_rng(21)
+    hi32 = rng.integers(-1000, 1000, shape).astype(np.int32)
+    hi64 = rng.integers(-10**12, 10**12, shape).astype(np.int64)
+    hf32 = rng.uniform(-3, 3, shape).astype(np.float32)
+    hf64 = rng.uniform(-3, 3, shape)
+    i32, i64, f32, f64 = (cnp.array(h) for h in (hi32, hi64, hf32, hf64))
+    for got, want in (((i32 + f32) * 2, (hi32 + hf32) * 2), (i64 - i32, hi64 - hi32),
+                      (f64 * f32 + i32, hf64 * hf32 + hi32), (f32 / i64, hf32 / hi64),
+                      (i32.astype(np.float32) + f32, hi32.astype(np.float32) + hf32),
+                      (f64.astype(np.int64), hf64.astype(np.int64)),
+                      (i64.astype(np.float32), hi64.astype(np.float32))):
+        g = got.get(itf)
+        assert g.dtype == want.dtype and g.tobytes() == want.tobytes()
+    # a slice of one type into a region of another: the target's type wins, as in NumPy
+    sl = tuple(slice(1, s - 1) for s in shape)
+    tgt = cnp.array(hi32)
+    tgt[sl] = f64[sl] * 100.0
+    hw = hi32.copy()
+    hw[sl] = hf64[sl] * 100.0
+    assert np.array_equal(tgt.get(itf), hw)
+    if len(shape) == 1:
+        assert (i32 @ f64).get(itf)[0] == pytest.approx(float(hi32 @ hf64), rel=1e-12)
+    if len(shape) == 2:
+        v = cnp.array(rng.uniform(-1, 1, shape[1]))
+        np.testing.assert_allclose((i32 @ v).get(itf), hi32 @ v.get(itf), rtol=1e-12, atol=1e-9)
+        m = cnp.array(rng.integers(-5, 5, (shape[1], 7)).astype(np.int32))
+        np.testing.assert_allclose((f32 @ m).get(itf), hf32.astype(np.float64) @ m.get(itf), rtol=1e-12, atol=1e-9)
+
+
 def test_shifted_slices_of_arange(small_tiles):
     src = cnp.arange(512, dtype=np.float32)
     got = (src[100:300] + src[150:350]).get(small_tiles)

@@ -72,6 +72,54 @@ def test_fill_and_copy_region_bit_exact(dev, esz, npdt):
     dev.free_all()
 
 
+def test_convert_region_is_numpy_astype(dev):
+    """Every pair of element types, whole and strided: bit-exact against ndarray.astype (round to
+    nearest even into floating point, truncation into integers; values kept inside the range of
+    every integer type, beyond it C leaves the result open)."""
+    rng = np.random.default_rng(5)
+    types = ((L.F32, np.float32), (L.F64, np.float64), (L.I32, np.int32), (L.I64, np.int64))
+    n = 70001
+    for sdt, snp in types:
+        if np.issubdtype(snp, np.floating):
+            src = (rng.uniform(-2.0e9, 2.0e9, n) * rng.choice([1.0, 1e-3, 1e-9], n)).astype(snp)
+            src[:6] = np.array([0.5, -0.5, 1.5, 2.5, -0.0, 16777217.0]).astype(snp)
+        else:
+            hi = 2**31 - 1 if snp is np.int32 else 2**62
+            src = rng.integers(-hi, hi, n).astype(snp)
+            src[:4] = np.array([16777217, -16777217, 2**31 - 1, 0]).astype(snp)   # ties of float32
+        dsrc = dev.array(src)
+        for ddt, dnp in types:
+            if np.issubdtype(snp, np.floating) and dnp is np.int32:
+                use = np.clip(src, -2.0e9, 2.0e9).astype(snp)
+                dsrc.put(use)
+            elif snp is np.int64 and dnp is np.int32:
+                use = (src >> 33).astype(snp)
+                dsrc.put(use)
+            else:
+                use = src
+                dsrc.put(use)
+            out = dev.empty((n,), dnp)
+            L.check(L.lib.cnh_convert_region(1, ddt, out.ptr, H.L.i64arr([1]), H.L.i64arr([0]), H.L.i64arr([1]),
+                                             sdt, dsrc.ptr, H.L.i64arr([1]), H.L.i64arr([0]), H.L.i64arr([1]),
+                                             H.L.i64arr([n]), None))
+            with np.errstate(all="ignore"):
+                want = use.astype(dnp)
+            assert out.get().tobytes() == want.tobytes(), (snp, dnp)
+    # strided 2-D window into a window of another type
+    a = rng.integers(-1000, 1000, (40, 50)).astype(np.int32)
+    da = dev.array(a)
+    b = np.full((30, 64), -1.0)
+    db = dev.array(b)
+    L.check(L.lib.cnh_convert_region(2, L.F64, db.ptr, H.L.i64arr([64, 1]), H.L.i64arr([2, 5]), H.L.i64arr([1, 3]),
+                                     L.I32, da.ptr, H.L.i64arr([50, 1]), H.L.i64arr([1, 0]), H.L.i64arr([2, 1]),
+                                     H.L.i64arr([19, 17]), None))
+    b[2:21, 5:56:3] = a[1:39:2, 0:17]
+    assert np.array_equal(db.get(), b)
+    assert L.lib.cnh_convert_region(1, 7, db.ptr, H.L.i64arr([1]), H.L.i64arr([0]), H.L.i64arr([1]), L.I32, da.ptr,
+                                    H.L.i64arr([1]), H.L.i64arr([0]), H.L.i64arr([1]), H.L.i64arr([4]), None) == -2
+    dev.free_all()
+
+
 def test_d2h_region_gathers_tiles(dev):
     g = np.arange(40 * 56, dtype=np.float64).reshape(40, 56)
     out = np.zeros_like(g)
