@@ -441,10 +441,20 @@ def run_c1(L, n=1 << 24, parts=4, reps=20):
             L.check(L.lib.cnh_event_record(ev.b[i], None))
         L.check(L.lib.cnh_device_sync())
         t = ev.times_ms(reps)
+        # the same call issued `reps` times back to back between ONE pair of events: what it costs
+        # inside a stream of launches, without an event record before and after every call
+        L.check(L.lib.cnh_event_record(ev.a[0], None))
+        for i in range(reps):
+            fn()
+        L.check(L.lib.cnh_event_record(ev.b[0], None))
+        L.check(L.lib.cnh_device_sync())
+        stream_us = 1e3 * ev.times_ms(1)[0] / reps
         ev.free()
         us = 1e3 * float(np.median(t))
         out[name] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1),
-                     "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+                     "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                     "us_back_to_back": round(stream_us, 2),
+                     "hbm_frac_back_to_back": round(nbytes / stream_us / 1e3 / HBM_PEAK_GBS, 4)}
     separate, one_pass = res.get(np.float64), res2.get(np.float64)
     out["one_pass_vs_separate_rel_diff"] = float(np.max(np.abs(separate - one_pass) / np.abs(separate)))
     out["separate_passes_us"] = round(out["elementwise"]["us"] + out["sum"]["us"] + out["dot_zz"]["us"], 2)
