@@ -106,7 +106,8 @@ def cg_asts(L):
     (alpha = r.r / p.Ap, beta = r.r_new / r.r) are formed in registers by the group that uses them,
     and r.r_new is taken by the launch that produces r_new: it leaves one partial sum per wavefront,
     which the p update sums (every workgroup in the same order) and stores for the next iteration.
-    An iteration is four launches (matvec, dot, x and r, p) instead of eight.
+    An iteration is four launches (matvec, dot, x and r, p) instead of eight; with the fused matvec
+    (cnh_gemv_tiles_fused), which also forms p and leaves the partial sums of p.Ap, two.
     Group 1 (leaves 1 = p, 2 = x, 3 = Ap, 4 = r; scalars 5 = r.r, 6 = p.Ap):
         7 = x + alpha p, 8 = r - alpha Ap, 9 = sum of (8)^2 as partial sums.
     Group 2 (leaves 1 = p, 2 = r_new; scalars 5 = r.r_new given as those partial sums, 6 = r.r):
@@ -158,7 +159,7 @@ def prepare_launch(L, k, nd, ins, scalars, outs, stream=None):
     return lambda: L.check(L.lib.cnh_launch_group_sums(k, nd, n_i, ia, n_s, sp, n_o, oa, stream))
 
 
-def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True, trace_iters=0):
+def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True, trace_iters=0, fuse=True):
     """`steps` timed CG iterations. With trace_iters > 0 an untimed pass over the same system runs
     first and reads alpha, beta and r.r back after each of its iterations (and x at its end):
     what the parity check against the CPU leg compares."""
@@ -200,17 +201,59 @@ def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True, trace_i
                                        {5: (partials.ptr, n_partials, S(nxt["rtr"])), 6: S(cur["rtr"])},
                                        {7: mr(nxt["p"])}),
         })
-    state = {"parity": 0}
+    state = {"parity": 0, "first": True}
+
+    # Two launches per iteration where the fused matvec applies (16384 rows or more): the matvec
+    # forms p = r + beta p on the way (beta from the partial sums of r.r the previous launch left,
+    # which it also folds and stores) and leaves the partial sums of p.Ap, one per workgroup; the
+    # x and r update forms alpha from those. The p of the LAST iteration is formed by one closing
+    # launch of the p update, so that the timed iterations leave the full CG state behind.
+    n_pap = (n + 63) // 64
+    pap = Buf(L, n_pap * 8, zero=True)
+    fused = fuse and n >= 16384 and tile * 8 <= 65536 and tile % 2 == 0 and n % 2 == 0
+    fforms = []
+    if fused:
+        for cur, nxt in ((bufs[0], bufs[1]), (bufs[1], bufs[0])):
+            # iteration k of parity e: p_k -> cur["p"], formed from r_k = cur["r"] and p_{k-1} = nxt["p"];
+            # r.r_k -> slot cur["rtr"], r.r_{k-1} in slot nxt["rtr"]
+            fforms.append({
+                "form_p": L.GemvFusion(cur["r"].ptr, nxt["p"].ptr, partials.ptr, n_partials, S(nxt["rtr"]),
+                                       S(cur["rtr"]), cur["p"].ptr, pap.ptr, n_pap),
+                "plain": L.GemvFusion(None, None, None, 0, None, None, cur["p"].ptr, pap.ptr, n_pap),
+                "p": cur["p"],
+                "update_x_r": prepare_launch(L, k_xr, 1, {1: mr(cur["p"]), 2: mr(cur["x"]), 3: mr(Ap), 4: mr(cur["r"])},
+                                             {5: S(cur["rtr"]), 6: (pap.ptr, n_pap, S(1))},
+                                             {7: mr(nxt["x"]), 8: mr(nxt["r"]),
+                                              9: L.Memref.dense(partials.ptr, (n_partials,))}),
+                # closes a run of iterations: p_{k+1} = r_{k+1} + beta p_k, r.r_{k+1} folded and stored
+                "close": prepare_launch(L, k_p, 1, {1: mr(cur["p"]), 2: mr(nxt["r"])},
+                                        {5: (partials.ptr, n_partials, S(nxt["rtr"])), 6: S(cur["rtr"])},
+                                        {7: mr(nxt["p"])}),
+            })
 
     def reset():
         # x = 0, r = p = b, r.r; the ping-pong roles go back to their starting assignment too
         state["parity"] = 0
+        state["first"] = True
         L.check(L.lib.cnh_memset0(x.ptr, n * 8, None))
         L.check(L.lib.cnh_d2d(r.ptr, bvec.ptr, n * 8, None))
         L.check(L.lib.cnh_d2d(p.ptr, bvec.ptr, n * 8, None))
         L.check(L.lib.cnh_dot_partial(L.F64, n, r.ptr, r.ptr, S(0), None))
 
     def iteration(ev=None, i=0):
+        if fused:
+            f = fforms[state["parity"]]
+            if ev is not None:
+                L.check(L.lib.cnh_event_record(ev.a[i], None))
+            # the first iteration after a reset (or after a closing launch) finds p ready
+            fu = f["plain"] if state["first"] else f["form_p"]
+            L.check(L.lib.cnh_gemv_tiles_fused(n, n, tile, tptr, f["p"].ptr, Ap.ptr, C.byref(fu), None, None))
+            if ev is not None:
+                L.check(L.lib.cnh_event_record(ev.b[i], None))
+            f["update_x_r"]()                  # alpha from the partial sums of p.Ap; x, r, partial sums of r.r
+            state["first"] = False
+            state["parity"] ^= 1
+            return
         f = forms[state["parity"]]
         if ev is not None:
             L.check(L.lib.cnh_event_record(ev.a[i], None))
@@ -222,12 +265,19 @@ def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True, trace_i
         f["update_p"]()                        # r.r_new summed and stored, r_new + beta p
         state["parity"] ^= 1
 
+    def close():
+        """After a run of fused iterations: forms the p (and stores the r.r) the last one left open."""
+        if fused and not state["first"]:
+            fforms[state["parity"] ^ 1]["close"]()
+            state["first"] = True
+
     def current():
         return bufs[state["parity"]]
 
     reset()
     for _ in range(warmup):
         iteration()
+    close()
     L.check(L.lib.cnh_device_sync())
     setup_s = time.time() - t0
 
@@ -238,6 +288,7 @@ def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True, trace_i
         for _ in range(trace_iters):
             before = current()["rtr"]
             iteration()
+            close()                          # r.r of the new iterate is folded by the p update
             v = sc.get(np.float64)           # waits for the iteration
             after = current()["rtr"]
             # alpha and beta exist in registers only; the same two divisions on the host, from the
@@ -257,6 +308,7 @@ def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True, trace_i
     L.check(L.lib.cnh_event_record(e0, None))
     for i in range(steps):
         iteration(ev, i)
+    close()                                  # inside the timed region: the last iteration's p and r.r
     L.check(L.lib.cnh_event_record(e1, None))
     L.check(L.lib.cnh_device_sync())
     wall = time.perf_counter() - w0
@@ -267,13 +319,13 @@ def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True, trace_i
         "n": n, "tile": tile, "steps": steps, "wall_s": wall, "gpu_ms": ms.value,
         "ms_per_step": wall * 1e3 / steps, "iters_per_s": steps / wall,
         "gemv_avg_us": 1e3 * float(np.mean(gemv_ms)), "gemv_min_us": 1e3 * float(np.min(gemv_ms)),
-        "setup_s": setup_s,
+        "setup_s": setup_s, "launches_per_iteration": 2 if fused else 4,
         "rtr_final": float(sc.get(np.float64)[current()["rtr"]]),
         "x": current()["x"].get() if check else None,
         "trace": trace,
     }
     ev.free()
-    for b_ in tiles + [bvec, x, r, p, Ap, x2, r2, p2, sc, partials]:
+    for b_ in tiles + [bvec, x, r, p, Ap, x2, r2, p2, sc, partials, pap]:
         b_.free()
     return res
 
@@ -1132,6 +1184,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-also", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--cpu-iters", type=int, default=50)
+    ap.add_argument("--cg-separate", action="store_true",
+                    help="CG iteration as four launches (matvec, dot, x and r, p) instead of the fused two")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: every partition of the path lives on a single MI355X; "
@@ -1145,7 +1199,7 @@ def main():
     L.check(L.lib.cnh_device_name(name, 256))
     n = args.n
     parity_iters = 0 if args.no_cpu else min(args.steps, args.cpu_iters)
-    cg = run_cg(L, n, args.steps, args.warmup, trace_iters=parity_iters)
+    cg = run_cg(L, n, args.steps, args.warmup, trace_iters=parity_iters, fuse=not args.cg_separate)
     gemv_bytes = 8.0 * n * n + 2 * 8.0 * n
     achieved = gemv_bytes / (cg["gemv_avg_us"] * 1e-6) / 1e9
     line = {
@@ -1162,11 +1216,17 @@ def main():
         "dtype": "f64",
         "data": "synthetic",
         "config": {"workload": f"dense CG, n={n}, A in {cg['tile']}^2 row-major tiles, one CG "
-                               "iteration per step (matvec, 2 dots, 2 scalar ops, 3 updates) in four launches: "
-                               "matvec; p.Ap; x and r with alpha formed in registers and r.r taken on the way; "
-                               "p with beta formed in registers",
+                               "iteration per step (matvec, 2 dots, 2 scalar ops, 3 updates) in "
+                               + ("two launches: the matvec, which forms p = r + beta p on the way (beta from the "
+                                  "partial sums of r.r) and leaves the partial sums of p.Ap; x and r with alpha "
+                                  "formed in registers and the partial sums of r.r taken on the way"
+                                  if cg["launches_per_iteration"] == 2 else
+                                  "four launches: matvec; p.Ap; x and r with alpha formed in registers and r.r "
+                                  "taken on the way; p with beta formed in registers"),
                    "device": name.value.decode()},
-        "roofline": {"bound": "hbm", "kernel": "gemv_rows_xlds<double,8,8,4>", "achieved": round(achieved, 1),
+        "roofline": {"bound": "hbm",
+                     "kernel": "gemv_rows_xlds<double,8,8,4,true>" if cg["launches_per_iteration"] == 2
+                     else "gemv_rows_xlds<double,8,8,4>", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": GEMV_N16384_TRAFFIC_BYTES if n == 16384 else None,
                      "traffic_source": "rocprofv3 --pmc counters of an earlier run of this kernel "

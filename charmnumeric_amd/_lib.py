@@ -84,6 +84,13 @@ class GemmJob(C.Structure):
                 ("B", C.c_void_p), ("ldb", C.c_int64), ("C", C.c_void_p), ("ldc", C.c_int64)]
 
 
+class GemvFusion(C.Structure):
+    """cnh_gemv_fusion: the vector work a fused matvec takes along."""
+    _fields_ = [("xa", C.c_void_p), ("xb", C.c_void_p), ("num", C.c_void_p), ("num_count", C.c_int64),
+                ("den", C.c_void_p), ("num_folded", C.c_void_p), ("w", C.c_void_p),
+                ("dot_partials", C.c_void_p), ("dot_capacity", C.c_int64)]
+
+
 class ScalarSum(C.Structure):
     """cnh_scalar_sum: a run-time scalar given as `count` partial sums at `ptr`."""
 
@@ -245,6 +252,8 @@ _PROTOS = {
     "cnh_axpy1": (C.c_int, [C.c_int, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]),
     "cnh_gemv_tiles": (C.c_int, [C.c_int, C.c_int64, C.c_int64, C.c_int32, _vpp, C.c_void_p,
                                  C.c_void_p, C.c_void_p]),
+    "cnh_gemv_tiles_fused": (C.c_int, [C.c_int64, C.c_int64, C.c_int32, _vpp, C.c_void_p, C.c_void_p,
+                                       C.c_void_p, C.POINTER(C.c_int64), C.c_void_p]),
     "cnh_gemm_acc": (C.c_int, [C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_int64,
                                C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p]),
     "cnh_gemm_acc_batch": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmJob), C.c_void_p]),

@@ -136,29 +136,92 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void gemv_rows(const ColTile* 
 // same bits. Needs: 128-bit alignment, every column tile at most 64 KB of x wide, and the column
 // tiles cut alike in every tile row.
 constexpr int kXldsBytes = 65536;
-template <typename T, int kWaves, int kRows, int kUnroll>
+
+// What a fused launch does besides the product (fp64 only): the vector formed on the way as
+// xa + (S / den) * xb, S the sum of `num_count` values in a fixed order (x then receives the vector,
+// every element written by exactly one workgroup), and the partial sums of w . y per workgroup.
+struct GemvFuse {
+    const double* xa;
+    const double* xb;
+    const double* num;
+    int64_t num_count;
+    const double* den;
+    double* num_folded;
+    const double* w;
+    double* dot_partials;
+};
+
+template <typename T, int kWaves, int kRows, int kUnroll, bool FUSED = false>
 __global__ __launch_bounds__(kWaves * 64) void gemv_rows_xlds(const ColTile* __restrict__ tiles, int ncol_tiles,
                                                               int64_t tile_rows, int64_t rows, int64_t row_shift,
                                                               const T* __restrict__ x, T* __restrict__ y,
-                                                              int beta) {
+                                                              int beta, GemvFuse f = GemvFuse()) {
     typedef typename Acc<T>::type A;
     constexpr int VEC = 16 / sizeof(T);
     typedef T P __attribute__((ext_vector_type(VEC)));
     __shared__ __attribute__((aligned(16))) T xs[kXldsBytes / sizeof(T)];
+    __shared__ double fuse_lds[kWaves + 1];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t r0 = ((int64_t)blockIdx.x * kWaves + wave) * kRows;
     A total[kRows];
 #pragma unroll
     for (int q = 0; q < kRows; ++q)
         total[q] = 0;
+    double factor = 0.0;
+    if (FUSED && f.xa != nullptr) {
+        // S: lane l of the first wavefront adds num[l], num[l + 64], ... in that order, then the
+        // fixed lane tree; every workgroup forms the same bits
+        if (wave == 0) {
+            double sacc = 0.0;
+            for (int64_t i = lane; i < f.num_count; i += 64)
+                sacc += f.num[i];
+            sacc = wave_sum<double>(sacc);
+            if (lane == 0) {
+                fuse_lds[kWaves] = sacc;
+                if (blockIdx.x == 0 && f.num_folded != nullptr)
+                    *f.num_folded = sacc;
+            }
+        }
+        __syncthreads();
+        factor = fuse_lds[kWaves] / f.den[0];
+    }
+    // the elements of the vector this workgroup stores when it forms the vector itself
+    const int64_t own_per = FUSED ? (rows + gridDim.x - 1) / gridDim.x : 0;
+    const int64_t own_lo = own_per * blockIdx.x, own_hi = own_lo + own_per;
     for (int tj = 0; tj < ncol_tiles; ++tj) {
         const int64_t ncols = tiles[tj].ncols, xoff = tiles[tj].xoff;
         if (tj > 0)
             __syncthreads();       // everybody is done with the previous tile's x
+        if (FUSED && f.xa != nullptr) {
+            // x = xa + factor * xb, one rounding per operation (no contraction), kept in LDS and,
+            // for this workgroup's own share, stored
+#pragma clang fp contract(off)
+            for (int64_t i = (int64_t)threadIdx.x * 2; i + 2 <= ncols; i += (int64_t)kWaves * 64 * 2) {
+                const double2 a = *reinterpret_cast<const double2*>(f.xa + xoff + i);
+                const double2 b = *reinterpret_cast<const double2*>(f.xb + xoff + i);
+                double2 v;
+                v.x = a.x + factor * b.x;
+                v.y = a.y + factor * b.y;
+                *reinterpret_cast<double2*>(reinterpret_cast<double*>(xs) + i) = v;
+                const int64_t g = xoff + i;
+                if (g >= own_lo && g < own_hi)
+                    const_cast<T*>(x)[g] = (T)v.x;
+                if (g + 1 >= own_lo && g + 1 < own_hi)
+                    const_cast<T*>(x)[g + 1] = (T)v.y;
+            }
+            if ((ncols & 1) && threadIdx.x == 0) {
+                const int64_t i = ncols - 1, g = xoff + i;
+                const double v = f.xa[g] + factor * f.xb[g];
+                reinterpret_cast<double*>(xs)[i] = v;
+                if (g >= own_lo && g < own_hi)
+                    const_cast<T*>(x)[g] = (T)v;
+            }
+        } else {
         for (int64_t i = (int64_t)threadIdx.x * VEC; i + VEC <= ncols; i += (int64_t)kWaves * 64 * VEC)
             *reinterpret_cast<P*>(xs + i) = *reinterpret_cast<const P*>(x + xoff + i);
         for (int64_t i = ncols / VEC * VEC + threadIdx.x; i < ncols; i += kWaves * 64)
             xs[i] = x[xoff + i];
+        }
         __syncthreads();
 #pragma unroll
         for (int q = 0; q < kRows; ++q) {
@@ -211,6 +274,26 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_rows_xlds(const ColTile* __r
         for (int q = 0; q < kRows; ++q)
             if (r0 + q < rows)
                 y[r0 + q] = beta ? (T)((A)y[r0 + q] + total[q]) : (T)total[q];
+    }
+    if (FUSED && f.w != nullptr) {
+        // w . y over this workgroup's rows: a wavefront's rows in order, then the wavefronts in order
+        if (lane == 0) {
+#pragma clang fp contract(off)
+            double d = 0.0;
+#pragma unroll
+            for (int q = 0; q < kRows; ++q)
+                if (r0 + q < rows)
+                    d += f.w[r0 + q] * (double)total[q];
+            fuse_lds[wave] = d;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            double d = fuse_lds[0];
+#pragma unroll
+            for (int wv = 1; wv < kWaves; ++wv)
+                d += fuse_lds[wv];
+            f.dot_partials[blockIdx.x] = d;
+        }
     }
 }
 
@@ -335,6 +418,59 @@ int cnh_gemv_tiles(int dtype, int64_t rows, int64_t cols, int32_t tile, const vo
             tiles[(size_t)(i * gc + j)] = {p, nc, nc, j * tile};
         }
     return dispatch_gemv(dtype, tiles, (int)gc, tile, rows, x, y, 0, as_stream(s));
+}
+
+int cnh_gemv_tiles_fused(int64_t rows, int64_t cols, int32_t tile, const void* const* tptr, void* x, void* y,
+                         const cnh_gemv_fusion* fu, int64_t* n_partials, cnh_stream s) {
+    if (int rc = ensure_init())
+        return rc;
+    CNH_CHECK(rows > 0 && cols > 0 && tile > 0, -2, "cnh_gemv_tiles_fused: bad shape");
+    CNH_CHECK(tptr && x && y && fu, -2, "cnh_gemv_tiles_fused: null pointer");
+    CNH_CHECK(rows >= 16384 && (int64_t)tile * 8 <= kXldsBytes && tile % 2 == 0 && cols % 2 == 0, -3,
+              "cnh_gemv_tiles_fused: needs 16384 rows or more and even column tiles of at most %d columns",
+              kXldsBytes / 8);
+    const bool form_x = fu->xa != nullptr;
+    CNH_CHECK(!form_x || (fu->xb && fu->num && fu->num_count >= 1 && fu->den), -2,
+              "cnh_gemv_tiles_fused: the vector's parts are incomplete");
+    CNH_CHECK(!form_x || (rows == cols && x != fu->xa && x != fu->xb), -2,
+              "cnh_gemv_tiles_fused: a vector formed on the way needs a square matrix and a buffer of its own");
+    CNH_CHECK(fu->w == nullptr || fu->dot_partials != nullptr, -2, "cnh_gemv_tiles_fused: no room for the partial sums");
+    int64_t gr = (rows + tile - 1) / tile, gc = (cols + tile - 1) / tile;
+    std::vector<ColTile> tiles((size_t)(gr * gc));
+    bool aligned = (((uintptr_t)x | (uintptr_t)fu->xa | (uintptr_t)fu->xb) & 15) == 0;
+    for (int64_t i = 0; i < gr; ++i)
+        for (int64_t j = 0; j < gc; ++j) {
+            const void* p = tptr[i * gc + j];
+            CNH_CHECK(p != nullptr, -2, "cnh_gemv_tiles_fused: tile (%lld,%lld) is null", (long long)i, (long long)j);
+            int64_t nc = std::min<int64_t>(tile, cols - j * tile);
+            tiles[(size_t)(i * gc + j)] = {p, nc, nc, j * tile};
+            aligned = aligned && ((uintptr_t)p & 15) == 0 && nc % 2 == 0;
+        }
+    CNH_CHECK(aligned, -3, "cnh_gemv_tiles_fused: operands must be 16-byte aligned");
+    constexpr int kW = 8, kR = 8;
+    const int64_t nb = (rows + kW * kR - 1) / (kW * kR);
+    CNH_CHECK(fu->w == nullptr || fu->dot_capacity >= nb, -3,
+              "cnh_gemv_tiles_fused: %lld partial sums, room for %lld", (long long)nb, (long long)fu->dot_capacity);
+    if (n_partials)
+        *n_partials = nb;
+    hipStream_t st = as_stream(s);
+    const void* dtiles = nullptr;
+    if (int rc = desc_upload(tiles.data(), tiles.size() * sizeof(ColTile), st, &dtiles))
+        return rc;
+    GemvFuse f;
+    f.xa = (const double*)fu->xa;
+    f.xb = (const double*)fu->xb;
+    f.num = (const double*)fu->num;
+    f.num_count = fu->num_count;
+    f.den = (const double*)fu->den;
+    f.num_folded = (double*)fu->num_folded;
+    f.w = (const double*)fu->w;
+    f.dot_partials = (double*)fu->dot_partials;
+    hipLaunchKernelGGL((gemv_rows_xlds<double, kW, kR, 4, true>), dim3((unsigned)nb), dim3(kW * 64), 0, st,
+                       (const ColTile*)dtiles, (int)gc, (int64_t)tile, rows, (int64_t)0, (const double*)x,
+                       (double*)y, 0, f);
+    CNH_HIP(hipGetLastError());
+    return 0;
 }
 
 static_assert(sizeof(cnh_gemv_panel) == sizeof(ColTile), "cnh_gemv_panel is the kernel's descriptor");

@@ -320,6 +320,34 @@ int cnh_axpy1(int dtype, int64_t n, const void* partial, void* y, cnh_stream s);
 int cnh_gemv_tiles(int dtype, int64_t rows, int64_t cols, int32_t tile, const void* const* tiles,
                    const void* x, void* y, cnh_stream s);
 
+/* cnh_gemv_tiles (fp64) with the vector work around the product of a Krylov iteration taken along
+ * (no upstream counterpart: upstream runs MATMUL, REDUCE and the vector update as nodes of their
+ * own, examples/cg.py:40-52, src/execute_node.cpp:116-273, src/executor_reduce.cpp:8-119):
+ *  - xa != NULL: the vector is formed on the way, x[j] = xa[j] + (S / den[0]) * xb[j] (one rounding
+ *    per operation), S = the sum of the num_count values at num in a fixed order; x receives the
+ *    vector (a buffer of its own, every element stored once) and *num_folded receives S if not
+ *    null. CG: p = r + (r.r_new / r.r_old) p with r.r_new left as partial sums by the launch that
+ *    updated r. Needs a square matrix.
+ *  - w != NULL: dot_partials[b] = sum of w[r] * y[r] over the rows of workgroup b (64 rows each, in
+ *    row order), b < *n_partials <= dot_capacity; their sum in index order is w . y (CG: p . Ap),
+ *    which cnh_launch_group_sums hands to the next launch.
+ * Applies to products of 16384 rows or more with even column tiles of at most 8192 columns and
+ * 16-byte aligned operands (-3 otherwise: use cnh_gemv_tiles and the separate calls). y has the
+ * bits cnh_gemv_tiles gives for the same x. */
+typedef struct cnh_gemv_fusion {
+    const void* xa;
+    const void* xb;
+    const void* num;
+    int64_t num_count;
+    const void* den;
+    void* num_folded;
+    const void* w;
+    void* dot_partials;
+    int64_t dot_capacity;
+} cnh_gemv_fusion;
+int cnh_gemv_tiles_fused(int64_t rows, int64_t cols, int32_t tile, const void* const* tiles, void* x, void* y,
+                         const cnh_gemv_fusion* fusion, int64_t* n_partials, cnh_stream s);
+
 /* The same over a window of a tiled matrix (a sliced or dimension-dropped operand,
  * charmnumeric.py:536-578, src/executor_matmul.cpp:150-498): row r of the window lies in panel row
  * p = (r + row_shift) / tile_rows at local row (r + row_shift) % tile_rows; panels[p * n_col_panels

@@ -64,6 +64,67 @@ def test_gemv_tiles_n16384_matches_oracle_tile_matvec(dev, cpu_system):
     dev.free_all()
 
 
+def test_fused_matvec_forms_its_vector_and_leaves_the_dot(dev, cpu_system):
+    """cnh_gemv_tiles_fused against the separate steps: the vector xa + (S / den) xb bit for bit
+    (S summed in the kernel's stated order), y the bits cnh_gemv_tiles gives for that vector, the
+    per-workgroup partial sums of x . y bit for bit in their stated order."""
+    orc, tile, g, tiles, b = cpu_system
+    bufs = []
+    for i in range(g):
+        for j in range(g):
+            t = tiles[i][j]
+            buf = bench.Buf(L, t.nbytes)
+            L.check(L.lib.cnh_fill_cg_matrix(buf.ptr, N, i * tile, t.shape[0], j * tile, t.shape[1],
+                                             t.shape[1], 2, None))
+            bufs.append(buf)
+    tp = L.vparr([t.ptr for t in bufs])
+    xa = orc.uniform(N, 9, 1, -1.0, 1.0)
+    xb = orc.uniform(N, 9, 2, -1.0, 1.0)
+    num = orc.uniform(128, 9, 3, 0.0, 1.0)
+    den = np.array([3.25])
+    dxa, dxb, dnum, dden = dev.array(xa), dev.array(xb), dev.array(num), dev.array(den)
+    dx, dy, dy2 = dev.empty((N,), np.float64), dev.empty((N,), np.float64), dev.empty((N,), np.float64)
+    dfold, dpart = dev.empty((1,), np.float64), dev.empty((N // 64,), np.float64)
+    f = L.GemvFusion(dxa.ptr, dxb.ptr, dnum.ptr, 128, dden.ptr, dfold.ptr, dx.ptr, dpart.ptr, N // 64)
+    npart = C.c_int64()
+    L.check(L.lib.cnh_gemv_tiles_fused(N, N, tile, tp, dx.ptr, dy.ptr, C.byref(f), C.byref(npart), None))
+    assert npart.value == N // 64
+    # S: lane l adds num[l], num[l + 64], ... in order, then the halving tree over the 64 lanes
+    lanes = num[:64] + num[64:128]
+    for off in (32, 16, 8, 4, 2, 1):
+        lanes[:off] = lanes[:off] + lanes[off:2 * off]
+    S = lanes[0]
+    assert dfold.get()[0] == S
+    want_x = xa + (S / den[0]) * xb
+    got_x = dx.get()
+    assert got_x.tobytes() == want_x.tobytes()
+    L.check(L.lib.cnh_gemv_tiles(L.F64, N, N, tile, tp, dx.ptr, dy2.ptr, None))
+    y = dy.get()
+    assert y.tobytes() == dy2.get().tobytes()
+    # partial b: its 8 wavefronts' 8 rows each in order, then the wavefronts in order
+    prod = (got_x * y).reshape(N // 64, 8, 8)
+    wave = np.zeros((N // 64, 8))
+    for q in range(8):
+        wave = wave + prod[:, :, q]
+    part = wave[:, 0].copy()
+    for w in range(1, 8):
+        part = part + wave[:, w]
+    assert dpart.get().tobytes() == part.tobytes()
+    # the plain product with the dot alone (first CG iteration): x is read as given
+    f2 = L.GemvFusion(None, None, None, 0, None, None, dx.ptr, dpart.ptr, N // 64)
+    L.check(L.lib.cnh_memset0(dy.ptr, N * 8, None))
+    L.check(L.lib.cnh_gemv_tiles_fused(N, N, tile, tp, dx.ptr, dy.ptr, C.byref(f2), None, None))
+    assert dy.get().tobytes() == y.tobytes() and dpart.get().tobytes() == part.tobytes()
+    assert dx.get().tobytes() == want_x.tobytes()
+    # refused where it does not apply
+    assert L.lib.cnh_gemv_tiles_fused(4096, 4096, 2048, tp, dx.ptr, dy.ptr, C.byref(f2), None, None) == -3
+    f3 = L.GemvFusion(dx.ptr, dxb.ptr, dnum.ptr, 128, dden.ptr, None, None, None, 0)
+    assert L.lib.cnh_gemv_tiles_fused(N, N, tile, tp, dx.ptr, dy.ptr, C.byref(f3), None, None) == -2
+    for t in bufs:
+        t.free()
+    dev.free_all()
+
+
 def test_cg_50_iterations_n16384_match_oracle(cpu_system):
     iters = 50
     cg = bench.run_cg(L, N, iters, 0, trace_iters=iters)
