@@ -294,6 +294,7 @@ class _ArrayLike:
         region = compose(self._region(), inner)
         shape = region_shape(inner)
         base = self._base()
+        base._all_ones = False
         if isinstance(rhs, _ArrayLike):
             value = rhs
         else:
@@ -375,6 +376,11 @@ class _ArrayLike:
 
 class Array(_ArrayLike):
     """A whole distributed array, existing or about to be computed."""
+
+    # True while every element is known to be exactly 1 (set by ones()/full(.., 1), dropped by any
+    # assignment into the array): a dot with such an array is recorded as a sum, which reads one
+    # array instead of two and gives the same bits (a * 1 is a, the order of additions is the same).
+    _all_ones = False
 
     def __init__(self, shape, dtype, name=None):
         self.shape = tuple(shape)
@@ -613,6 +619,9 @@ def _matmul(lhs, rhs):
             raise ValueError(f"Shape mismatch for dot product: ({lhs.shape[0]},) @ ({rhs.shape[0]},)")
         if lhs.dtype != rhs.dtype:
             lhs, rhs = _promoted(lhs, rhs)
+        for a, b in ((lhs, rhs), (rhs, lhs)):
+            if isinstance(b, Array) and b._all_ones and (isinstance(a, Array) or _is_whole(a.region, a.base.shape)):
+                return nonfusible(lazy.OP_SUM, [a], (1,), a.dtype)
         return nonfusible(L.OP_REDUCE, [lhs, rhs], (1,), lhs.dtype)
     if lhs.ndims not in (2, 3):
         raise ValueError(f"matmul requires a 2D matrix, got {lhs.ndims}D")
@@ -770,6 +779,7 @@ def full(shape, fill_value, dtype=None):
     dt = _normalize_dtype(dtype, allow_none=True) or _normalize_dtype(np.asarray(value).dtype)
     out = create_array(shape, dt)
     out[...] = _coerce_scalar(value)
+    out._all_ones = value == 1
     return out
 
 

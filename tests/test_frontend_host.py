@@ -120,6 +120,28 @@ def test_dtype_and_shape_rules(itf):
     assert a[2:6].shape == (4,) and cnp.zeros((4, 6))[1].shape == (1, 6)
 
 
+def test_dot_with_an_array_of_ones_is_recorded_as_a_sum(itf):
+    z = cnp.zeros((4096,)) + 2.0
+    one = cnp.ones((4096,))
+    s1 = z @ one
+    s2 = one @ z
+    cnp.execute(itf)
+    log = itf.trace()
+    assert not [ln for ln in log if ln.startswith("reduce ")], log
+    # any assignment into the array ends it, also through a view; a dot with it is a dot again
+    one[5:9] = 3.0
+    s3 = z @ one
+    w = cnp.full((4096,), 1.0)
+    v = w[:]
+    v[0] = 2.0
+    s4 = z @ w
+    s5 = z[8:24] @ cnp.ones((16,))          # a slice is not summed whole: stays a dot
+    cnp.execute(itf)
+    log = itf.trace()
+    assert len([ln for ln in log if ln.startswith("reduce ")]) == 3, log
+    del s1, s2, s3, s4, s5
+
+
 # ---- grouping ----
 
 def test_statement_with_dead_temporaries_is_one_group(itf):

@@ -87,6 +87,26 @@ def test_mixed_element_types_promote_like_numpy(small_tiles, shape):
         np.testing.assert_allclose((f32 @ m).get(itf), hf32.astype(np.float64) @ m.get(itf), rtol=1e-12, atol=1e-9)
 
 
+def test_dot_with_ones_gives_the_bits_of_the_dot(small_tiles):
+    """`z @ ones` is recorded as a sum (one array read instead of two): the same bits as the dot
+    with an array that merely holds ones, for every element type."""
+    itf = small_tiles
+    rng = np.random.default_rng(8)
+    for dt in (np.float64, np.float32, np.int32, np.int64):
+        h = (rng.uniform(-3, 3, 70001) * 100).astype(dt)
+        z = cnp.array(h)
+        ones = cnp.ones((70001,), dtype=dt)
+        held = cnp.array(np.ones(70001, dt))          # uploaded: not known to be ones
+        a, b = (z @ ones).get(itf), (z @ held).get(itf)
+        assert a.dtype == dt and a.tobytes() == b.tobytes()
+        assert (ones @ z).get(itf).tobytes() == b.tobytes()
+        ones[3] = 2                                   # assigned into: a dot again
+        got = (z @ ones).get(itf)[0]
+        with np.errstate(over="ignore"):
+            want = b[0] + h[3]
+        assert got == want if np.issubdtype(dt, np.integer) else got == pytest.approx(want, rel=1e-5)
+
+
 def test_shifted_slices_of_arange(small_tiles):
     src = cnp.arange(512, dtype=np.float32)
     got = (src[100:300] + src[150:350]).get(small_tiles)
