@@ -29,8 +29,10 @@ HBM_PEAK_GBS = 8000.0
 FP64_MFMA_PEAK_TFLOPS = 78.6
 # HBM bytes per launch of the tiled matvec at n = 16384, from rocprofv3 FETCH_SIZE (x 2.0, the
 # factor a plain streaming kernel of known size gives on gfx950) + WRITE_SIZE (x 1.0):
-# (2 098 216 + 128.3) KiB, see profiles/bench_hbm_traffic_pmc.txt.
-GEMV_N16384_TRAFFIC_BYTES = 2148704563
+# (2 099 620 + 259.9) KiB for the fused form, (2 098 440 + 128.1) KiB for the plain one,
+# see profiles/bench_hbm_traffic_pmc.txt.
+GEMV_N16384_TRAFFIC_BYTES = 2150277018
+GEMV_N16384_TRAFFIC_BYTES_PLAIN = 2148933734
 
 
 def _dev():
@@ -1228,7 +1230,8 @@ def main():
                      "kernel": "gemv_rows_xlds<double,8,8,4,true>" if cg["launches_per_iteration"] == 2
                      else "gemv_rows_xlds<double,8,8,4>", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": GEMV_N16384_TRAFFIC_BYTES if n == 16384 else None,
+                     "traffic": (GEMV_N16384_TRAFFIC_BYTES if cg["launches_per_iteration"] == 2
+                                 else GEMV_N16384_TRAFFIC_BYTES_PLAIN) if n == 16384 else None,
                      "traffic_source": "rocprofv3 --pmc counters of an earlier run of this kernel "
                                        "(profiles/bench_hbm_traffic_pmc.txt), not measured in this run",
                      "avg_us": round(cg["gemv_avg_us"], 2),
