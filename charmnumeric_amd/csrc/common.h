@@ -62,6 +62,7 @@ constexpr int kFoldMaxVectors = 4;
 int reduce_slots_f64_many(int nvec, const int* maximum, double* const* vecs, int64_t n, double* const* outs,
                           hipStream_t st);
 void gemv_set_xlds(int on);
+void gemm_set_buffer_loads(int on);
 int reduce_slots_f64(bool maximum, double* slots, int64_t n, double* out, hipStream_t st);
 
 // Descriptor tables (per-partition pointers/shapes) live on the device. Identical tables are

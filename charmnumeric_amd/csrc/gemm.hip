@@ -51,7 +51,7 @@ static_assert(sizeof(GemmSeg) == 40 && sizeof(GemmChain) == 40, "descriptor tabl
 // buffer being filled while the other is read): one K step of matrix instructions is shorter than
 // a trip to memory. A workgroup keeps its accumulators across the segments of its chain, so the
 // panel products of one C block cost one pass over C however many K pieces they come in.
-template <int WM, int WN, int TM, int TN, int BKT, bool FULL>
+template <int WM, int WN, int TM, int TN, int BKT, bool FULL, bool BUF = false>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_f64_mfma(const GemmChain* __restrict__ chains,
                                                               int nchains,
                                                               const GemmSeg* __restrict__ segs,
@@ -102,7 +102,37 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_f64_mfma(const GemmChain* _
         if (si > 0)
             __syncthreads();   // the previous segment's last reads of LDS are done
 
+        // BUF: buffer loads. The descriptor (base of this workgroup's rows of A, of its columns of
+        // B, moved along K on the scalar unit) sits in scalar registers and a lane contributes one
+        // 32-bit offset that never changes: no 64-bit address arithmetic on the vector unit, which
+        // the fp64 matrix instructions compete with (3-6 % on the 256 x 2048 x 4096 product).
+        typedef int v4i __attribute__((ext_vector_type(4)));
+        const int a_off = BUF ? (int)((a_row * lda + a_k) * 8) : 0;
+        const int b_off = BUF ? (int)((b_k * ldb + b_n) * 8) : 0;
         auto fetch = [&](int k0, double (&ra)[APT], double (&rb)[BPT]) {
+            if (BUF) {
+                const __amdgpu_buffer_rsrc_t da = __builtin_amdgcn_make_buffer_rsrc(
+                    (void*)(A + (int64_t)m0 * lda + k0), 0, 0x7fffffff, 0x00020000);
+                const __amdgpu_buffer_rsrc_t db = __builtin_amdgcn_make_buffer_rsrc(
+                    (void*)(B + (int64_t)k0 * ldb + n0), 0, 0x7fffffff, 0x00020000);
+#pragma unroll
+                for (int j = 0; j < APT; j += 2) {
+                    const v4i v = __builtin_amdgcn_raw_buffer_load_b128(da, a_off + j * 8, 0, 0);
+                    v2d d;
+                    __builtin_memcpy(&d, &v, 16);
+                    ra[j] = d[0];
+                    ra[j + 1] = d[1];
+                }
+#pragma unroll
+                for (int j = 0; j < BPT; j += 2) {
+                    const v4i v = __builtin_amdgcn_raw_buffer_load_b128(db, b_off + j * 8, 0, 0);
+                    v2d d;
+                    __builtin_memcpy(&d, &v, 16);
+                    rb[j] = d[0];
+                    rb[j + 1] = d[1];
+                }
+                return;
+            }
             const int gr = m0 + a_row;
             const int gk = k0 + a_k;
             if (FULL) {
@@ -279,6 +309,8 @@ int check_job(const cnh_gemm_job& j) {
     return 0;
 }
 
+int g_gemm_buffer_loads = 1;   // option "gemm_buffer_loads"
+
 template <int WM, int WN, int TM, int TN, int BKT>
 int launch_chains(std::vector<GemmChain>& chains, const std::vector<GemmSeg>& segs, bool full,
                   int overwrite, hipStream_t st) {
@@ -306,7 +338,15 @@ int launch_chains(std::vector<GemmChain>& chains, const std::vector<GemmSeg>& se
                                                chains.size() * sizeof(GemmChain));
     }
     const int nch = (int)chains.size(), nb = (int)blocks;
-    if (full)
+    // buffer loads need a lane's offset inside its workgroup's block of A (BM rows) and K step of
+    // B (BKT rows) to fit 31 bits
+    bool buf = full && g_gemm_buffer_loads;
+    for (const GemmSeg& sg : segs)
+        buf = buf && (int64_t)BM * sg.lda * 8 < (1ll << 31) && (int64_t)BKT * sg.ldb * 8 < (1ll << 31);
+    if (buf)
+        hipLaunchKernelGGL((gemm_f64_mfma<WM, WN, TM, TN, BKT, true, true>), dim3((unsigned)blocks),
+                           dim3(WM * WN * 64), 0, st, dch, nch, dsg, nb, chains[0], segs[0], overwrite);
+    else if (full)
         hipLaunchKernelGGL((gemm_f64_mfma<WM, WN, TM, TN, BKT, true>), dim3((unsigned)blocks),
                            dim3(WM * WN * 64), 0, st, dch, nch, dsg, nb, chains[0], segs[0], overwrite);
     else
@@ -379,6 +419,10 @@ __global__ __launch_bounds__(512) void mfma_f64_probe(double* out, int iters, do
     out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
 }
 } // namespace
+
+namespace cnh {
+void gemm_set_buffer_loads(int on) { g_gemm_buffer_loads = on; }
+} // namespace cnh
 
 extern "C" int cnh_probe_mfma_f64(int iters, double* tflops) {
     CNH_CHECK(iters >= 1 && iters <= (1 << 20) && tflops != nullptr, -2, "cnh_probe_mfma_f64: bad argument");

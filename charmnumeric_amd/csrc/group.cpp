@@ -1293,6 +1293,11 @@ extern "C" int cnh_set_option(const char* name, int value) {
         gemv_set_xlds(value);
         return 0;
     }
+    if (std::strcmp(name, "gemm_buffer_loads") == 0) {
+        CNH_CHECK(value == 0 || value == 1, -2, "gemm_buffer_loads: 0 or 1");
+        gemm_set_buffer_loads(value);
+        return 0;
+    }
     if (std::strcmp(name, "direct_lean") == 0) {
         g_direct_lean = value;
         return 0;

@@ -110,6 +110,7 @@ int cnh_version(void);
  *   "gemv_xlds"      matvecs of 8192 rows or more whose column tiles are at most 64 KB of x wide
  *                    stage x in LDS, 32 or 64 rows per workgroup (default 1); 0: one wavefront per
  *                    row reading x through the caches. Same bits either way.
+ *   "gemm_buffer_loads"  aligned fp64 products fetch A and B with buffer loads (default 1). Same bits.
  *   "slide_bx/ry/zc/pd", "slide2d_march"  geometry of the sliding-window kernel */
 int cnh_set_option(const char* name, int value);
 
