@@ -185,3 +185,120 @@ def test_random_program(seed, rank, solver):
     finally:
         cnp.reset()
         itf.close()
+
+
+class MixedProgram:
+    """Four arrays of one shape, one per element type; statements meet arrays of two types.
+    Results must have np.result_type's element type and NumPy's bits (the operand of the other
+    type is converted first, exactly); assignments convert to the target's type (truncation into
+    integers; values stay far inside every integer range, beyond which C leaves the result open)."""
+    TYPES = (np.float64, np.float32, np.int32, np.int64)
+
+    def __init__(self, seed, rank):
+        self.rng = np.random.default_rng(seed)
+        self.rank = rank
+        edge = {1: (150, 400), 2: (20, 70), 3: (9, 26)}[rank]
+        self.shape = tuple(int(self.rng.integers(*edge)) for _ in range(rank))
+        self.host = []
+        for dt in self.TYPES:
+            if np.issubdtype(dt, np.integer):
+                self.host.append(self.rng.integers(-1000, 1000, self.shape).astype(dt))
+            else:
+                self.host.append((self.rng.standard_normal(self.shape) * 10).astype(dt))
+        self.dev = [cnp.array(h) for h in self.host]
+        self.checks = []
+
+    def keys(self):
+        key, other = [], []
+        for n in self.shape:
+            s, count = random_slice(self.rng, n)
+            o = same_count_slice(self.rng, n, count)
+            key.append(s)
+            other.append(o if o is not None else s)
+        return tuple(key), tuple(other)
+
+    def statement(self):
+        rng = self.rng
+        kind = int(rng.integers(0, 5))
+        key, other = self.keys()
+        i, j, t = (int(v) for v in rng.integers(0, 4, 3))
+        if kind == 0:                                   # expression of two types, kept
+            op = int(rng.integers(0, 3))
+            d, h = self.dev[i][key], self.host[i][key]
+            e, g = self.dev[j][other], self.host[j][other]
+            with np.errstate(over="ignore"):
+                d, h = ((d + e, h + g), (d - e, h - g), (d * e, h * g))[op]
+            self.checks.append((d, h.copy(), "exact"))
+        elif kind == 1:                                 # slice of one type = sum of slices of others
+            h = self.host[i][other] + self.host[j][other]
+            self.dev[t][key] = self.dev[i][other] + self.dev[j][other]
+            self.host[t][key] = h
+        elif kind == 2:                                 # slice = slice of another type
+            h = self.host[i][other].copy()
+            self.dev[t][key] = self.dev[i][other]
+            self.host[t][key] = h
+        elif kind == 3:                                 # astype of a whole array and of a slice
+            dt = self.TYPES[int(rng.integers(0, 4))]
+            self.checks.append((self.dev[i].astype(dt), self.host[i].astype(dt), "exact"))
+            self.checks.append((self.dev[j][key].astype(dt), self.host[j][key].astype(dt), "exact"))
+        elif self.rank == 1:                            # dot of windows of two types
+            n = self.shape[0]
+            s, count = random_slice(rng, n, 8)
+            s = slice(s.start, s.start + count)
+            o = same_count_slice(rng, n, count)
+            o = slice(o.start, o.start + count)
+            ha, hb = self.host[i][s], self.host[j][o]
+            rt = np.result_type(ha.dtype, hb.dtype)
+            with np.errstate(over="ignore"):
+                want = ha.astype(rt) @ hb.astype(rt)
+            bound = float(np.abs(ha.astype(np.float64)) @ np.abs(hb.astype(np.float64)))
+            self.checks.append((self.dev[i][s] @ self.dev[j][o], (want, bound, rt), "dot"))
+        else:                                           # matrix of one type times a vector of another
+            if self.rank != 2:
+                return
+            v = cnp.array(self.host[j][0].copy())
+            hv = self.host[j][0]
+            rt = np.result_type(self.host[i].dtype, hv.dtype)
+            want = self.host[i].astype(rt) @ hv.astype(rt)
+            bound = np.abs(self.host[i].astype(np.float64)) @ np.abs(hv.astype(np.float64))
+            self.checks.append((self.dev[i] @ v, (want, bound, rt), "matvec"))
+
+    def verify(self, itf):
+        for d, h in zip(self.dev, self.host):
+            got = d.get(itf)
+            assert got.dtype == h.dtype and np.array_equal(got, h), "array contents differ"
+        for d, h, kind in self.checks:
+            got = d.get(itf)
+            if kind == "exact":
+                assert got.dtype == h.dtype and got.shape == h.shape and got.tobytes() == h.tobytes()
+            else:
+                want, bound, rt = h
+                assert got.dtype == rt
+                if np.issubdtype(rt, np.integer):
+                    assert np.array_equal(got.reshape(np.shape(want) or (1,)), np.reshape(want, np.shape(want) or (1,)))
+                else:
+                    rel = 1e-12 if rt == np.float64 else 1e-5
+                    assert np.all(np.abs(got.reshape(np.shape(want) or (1,)).astype(np.float64)
+                                         - np.asarray(want, np.float64).reshape(np.shape(want) or (1,)))
+                                  <= rel * np.asarray(bound).reshape(np.shape(want) or (1,)) + 1e-300)
+
+
+@pytest.mark.parametrize("rank", [1, 2, 3])
+@pytest.mark.parametrize("seed", range(8))
+def test_random_program_of_mixed_element_types(seed, rank):
+    cnp.reset()
+    itf = cnp.CharmNumericInterface(device=0)
+    itf.connect(odf=4)
+    for nd, t in MIN_TILE.items():
+        itf.set_min_tile(nd, t)
+    itf.set_solver(seed % 4 == 3)
+    itf.set_pipeline(seed % 2 == 1)
+    cnp.set_auto_flush(itf, int(np.random.default_rng(seed).choice([4, 16, 1000])))
+    try:
+        prog = MixedProgram(5000 * rank + seed, rank)
+        for _ in range(14):
+            prog.statement()
+        prog.verify(itf)
+    finally:
+        cnp.reset()
+        itf.close()
