@@ -106,7 +106,7 @@ def _launch1(L, k, nd, ins, scalars, outs, stream=None):
 def cg_asts(L):
     """The element-wise part of one CG iteration as two groups. The scalar statements
     (alpha = r.r / p.Ap, beta = r.r_new / r.r) are formed in registers by the group that uses them,
-    and r.r_new is taken by the launch that produces r_new: it leaves one partial sum per wavefront,
+    and r.r_new is taken by the launch that produces r_new: it leaves one partial sum per workgroup,
     which the p update sums (every workgroup in the same order) and stores for the next iteration.
     An iteration is four launches (matvec, dot, x and r, p) instead of eight; with the fused matvec
     (cnh_gemv_tiles_fused), which also forms p and leaves the partial sums of p.Ap, two.
@@ -181,8 +181,8 @@ def run_cg(L, n, steps, warmup, tile_rule_tile=None, seed=2, check=True, trace_i
     x2, r2, p2 = vec(), vec(), vec()
     L.check(L.lib.cnh_fill_uniform(bvec.ptr, n, seed, 1, 0, -1.0, 1.0, None))
     sc = Buf(L, 8 * 8, zero=True)  # slot 0 / 3: r.r of the current / next iterate (swapping), 1: p.Ap
-    # partial sums of r_new . r_new, one per wavefront of the launch that updates r (rest stays 0)
-    n_partials = 4 * ((n + 511) // 512)
+    # partial sums of r_new . r_new, one per workgroup (512 elements) of the launch that updates r
+    n_partials = (n + 511) // 512
     partials = Buf(L, n_partials * 8, zero=True)
     S = lambda i: sc.ptr + 8 * i
     k_xr, k_p = (_compile(L, a, L.F64, 1) for a in cg_asts(L))

@@ -392,8 +392,8 @@ std::string flat_source(const GroupProgram& p) {
 // streams faster than unrolled or persistent ones. NT selects non-temporal loads and stores for
 // launches whose traffic exceeds what the last-level cache could keep anyway.
 // Outputs in RED_MASK are not stored: every lane folds its elements' values into racc[], the
-// wavefront combines the lanes in a fixed order, and lane 0 writes one partial per reduction into
-// ro.slots[q][4 * blockIdx.x + wavefront] for the host (or a later launch) to fold.
+// wavefront combines the lanes in a fixed order, the workgroup its four wavefronts in order, and
+// one partial per workgroup and reduction goes to ro.slots[q][blockIdx.x] for a later launch to fold.
 struct Seg { i64 n; i64 blk0; const T* in[NLA]; T* out[NOA]; };
 typedef T TV __attribute__((ext_vector_type(VECW)));
 #define OUT_STORED(j) (((RED_MASK >> (j)) & 1u) == 0u)
@@ -471,10 +471,24 @@ __device__ __forceinline__ void red_finish(T* racc, const RedOut& ro) {
         for (int q = 0; q < NR; ++q) other[q] = __shfl_xor(racc[q], m, 64);
         RED_COMBINE(racc, other);
     }
+    // the four wavefronts of the workgroup, in order, then one partial per workgroup and reduction
+    __shared__ T red_lds[4][NRA];
     if ((threadIdx.x & 63) == 0) {
 #pragma unroll
+        for (int q = 0; q < NR; ++q) red_lds[threadIdx.x >> 6][q] = racc[q];
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int w = 1; w < 4; ++w) {
+            T other[NRA];
+#pragma unroll
+            for (int q = 0; q < NR; ++q) other[q] = red_lds[w][q];
+            RED_COMBINE(racc, other);
+        }
+#pragma unroll
         for (int q = 0; q < NR; ++q)
-            ro.slots[q][4 * (i64)blockIdx.x + (threadIdx.x >> 6)] = racc[q];
+            ro.slots[q][(i64)blockIdx.x] = racc[q];
     }
 }
 #define RED_PARAM , RedOut ro

@@ -445,11 +445,11 @@ int launch_group_impl(cnh_kernel* k, int ndims, int n_parts, int n_in, const cnh
         hipFunction_t fn;
         if (int rc = get_function(k, "flat", name.c_str(), &fn))
             return rc;
-        // Reducing roots: one partial per wavefront and reduction. A reduction whose output memref
+        // Reducing roots: one partial per workgroup and reduction. A reduction whose output memref
         // names more than one element keeps its partials there (the caller, or a later launch that
-        // takes them as a summed scalar, folds them; entries past the last wavefront are left as
+        // takes them as a summed scalar, folds them; entries past the last workgroup are left as
         // they are). The others go to the stream's workspace and are folded right after the launch.
-        const int64_t nslots = 4 * blocks;
+        const int64_t nslots = blocks;
         void* red_slots[kFoldMaxVectors] = {nullptr, nullptr, nullptr, nullptr};
         int maximum[kFoldMaxVectors] = {0, 0, 0, 0}, n_fold = 0;
         double* fold_vec[kFoldMaxVectors] = {nullptr, nullptr, nullptr, nullptr};

@@ -407,6 +407,9 @@ __global__ __launch_bounds__(kThreads) void fold_slots_runs(const double* __rest
 
 // Several slot vectors at once (blockIdx.y picks the vector), each a sum or a maximum: the
 // reductions a group kernel carried along are folded by the same one or two launches.
+// Up to this many partials per vector one workgroup of 1024 lanes folds by itself (64 loads per
+// lane, all in flight together); beyond it a grid folds runs first.
+constexpr int64_t kFoldSingleMax = 8192;
 struct FoldMany {
     double* vec[kFoldMaxVectors];
     double* out[kFoldMaxVectors];
@@ -456,7 +459,7 @@ int reduce_slots_f64_many(int nvec, const int* maximum, double* const* vecs, int
         f.maximum[q] = q < nvec ? maximum[q] : 0;
     }
     int64_t first = 0, count = n;
-    if (n > 8192) {
+    if (n > kFoldSingleMax) {
         int64_t per = (n + kFoldRuns - 1) / kFoldRuns;
         per = (per + 1023) / 1024 * 1024;               // whole passes of a workgroup
         const int64_t runs = (n + per - 1) / per;

@@ -213,8 +213,8 @@ int cnh_launch_group_batched(cnh_kernel* k, int ndims, int n_parts, int n_in, co
                              int n_out, const cnh_memref* out, cnh_stream s);
 /* Outputs that are CNH_OP_SUM_OF / CNH_OP_MAXABS_OF roots (fp64, dense operands): the memref of such
  * an output names ONE element, which receives the result over all partitions of the launch, or more
- * than one, in which case the launch leaves its partial results there (one per wavefront, 4 per 512
- * elements of a partition, at most as many as the memref has room for) and folds nothing: a later
+ * than one, in which case the launch leaves its partial results there (one per workgroup of 256
+ * lanes, i.e. per 512 fp64 elements of a partition; it needs room for all of them) and folds nothing: a later
  * launch takes them through cnh_launch_group_sums. Elements past the last partial are not written,
  * so a buffer that starts out as zeros can be summed over its whole length.
  *
