@@ -386,6 +386,14 @@ def test_gemm_batch_overwrites_without_reading(dev, M, N, K):
         j.M, j.N, j.K, j.A, j.lda, j.B, j.ldb, j.C, j.ldc = M, N, k1 - k0, dA.ptr + 8 * k0, K, dB.ptr + 8 * k0 * N, N, dC.ptr, N
     L.check(L.lib.cnh_gemm_batch(L.F64, 2, arr, 1, None))
     got = dC.get()
+    # aligned products fetch through buffer descriptors by default; plain global loads give the same bits
+    L.check(L.lib.cnh_set_option(b"gemm_buffer_loads", 0))
+    try:
+        dC.put(C0)
+        L.check(L.lib.cnh_gemm_batch(L.F64, 2, arr, 1, None))
+        assert dC.get().tobytes() == got.tobytes()
+    finally:
+        L.check(L.lib.cnh_set_option(b"gemm_buffer_loads", 1))
     bound = REL * (np.abs(A) @ np.abs(B))
     assert np.all(np.abs(got - (A.astype(np.longdouble) @ B.astype(np.longdouble)).astype(np.float64)) <= bound)
     # accumulate on top of it
