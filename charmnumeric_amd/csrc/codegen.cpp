@@ -59,6 +59,40 @@ std::string literal(int dtype, double c) {
     return fmt("((T)(%a))", c);
 }
 
+// Small multiples of a quarter (0, +-1, 0.5, 2.5, -1 for a negation, ...) stay in the source, where
+// the compiler can fold them; any other literal (a time step, a coefficient computed on the host)
+// becomes a launch parameter, so that a loop whose literal changes every step keeps one code object
+// instead of compiling a kernel per value.
+bool literal_stays_in_source(int dtype, double c) {
+    if (!std::isfinite(c))
+        return true;
+    if (std::fabs(c) > 16.0)
+        return false;
+    const double q = c * 4.0;
+    return q == std::floor(q) || is_int(dtype);
+}
+
+} // namespace
+void literal_value(int dtype, double c, void* out) {
+    if (is_int(dtype)) {
+        long long v = 0;
+        if (std::isfinite(c) && c > -9.2233720368547758e18 && c < 9.2233720368547758e18)
+            v = (long long)c;
+        if (dtype == CNH_I32) {
+            const int32_t w = (int32_t)(uint32_t)(uint64_t)v;
+            std::memcpy(out, &w, 4);
+        } else {
+            std::memcpy(out, &v, 8);
+        }
+    } else if (dtype == CNH_F32) {
+        const float f = (float)c;
+        std::memcpy(out, &f, 4);
+    } else {
+        std::memcpy(out, &c, 8);
+    }
+}
+namespace {
+
 struct Value {
     std::string expr;
     bool scalar = false;
@@ -146,8 +180,16 @@ int build_group_program(const cnh_ast* ast, int dtype, int ndims, GroupProgram& 
             if (op.opcode != CNH_OP_NOOP && op.opcode != CNH_OP_CREATE)
                 continue;
             if (op.is_scalar) {
+                auto seen = values.find(op.result_name);
+                if (seen != values.end() && seen->second.scalar)
+                    continue;                  // the same literal node under another root
                 Value v;
-                v.expr = literal(dtype, op.scalar);
+                if (literal_stays_in_source(dtype, op.scalar)) {
+                    v.expr = literal(dtype, op.scalar);
+                } else {
+                    v.expr = fmt("s[NS + %d]", (int)p.lit_values.size());
+                    p.lit_values.push_back(op.scalar);
+                }
                 v.scalar = true;
                 v.valid = true;
                 values[op.result_name] = v;
@@ -310,9 +352,13 @@ std::string prelude(const GroupProgram& p) {
     s << "typedef unsigned " << (p.dtype == CNH_I64 ? "long long" : "int") << " UT;\n";
     s << "typedef long long i64;\n";
     s << "#define NL " << NL << "\n#define NS " << NS << "\n#define NO " << NO << "\n";
+    const int NLIT = (int)p.lit_values.size();
     s << "#define NLA " << (NL > 0 ? NL : 1) << "\n#define NSA " << (NS > 0 ? NS : 1)
       << "\n#define NOA " << (NO > 0 ? NO : 1) << "\n";
-    s << "struct Scal { const T* p[NSA]; T v[NSA]; };\n";
+    // literal scalars handed over with the launch: s[NS .. NS + NLIT) of the scalar values
+    s << "#define NLIT " << NLIT << "\n#define NLITA " << (NLIT > 0 ? NLIT : 1) << "\n#define NSV "
+      << (NS + NLIT > 0 ? NS + NLIT : 1) << "\n";
+    s << "struct Scal { const T* p[NSA]; T v[NSA]; T c[NLITA]; };\n";
     if (is_int(p.dtype)) {
         // Truncating signed division; x/0 -> 0 and MIN/-1 -> MIN are fixed here because the
         // upstream operation (arith.divsi) leaves both undefined.
@@ -335,7 +381,9 @@ std::string prelude(const GroupProgram& p) {
     }
     s << "__device__ __forceinline__ void load_scalars(const Scal& sc, T* s) {\n"
          "#pragma unroll\n"
-         "    for (int i = 0; i < NS; ++i) s[i] = sc.p[i] ? *sc.p[i] : sc.v[i];\n}\n";
+         "    for (int i = 0; i < NS; ++i) s[i] = sc.p[i] ? *sc.p[i] : sc.v[i];\n"
+         "#pragma unroll\n"
+         "    for (int i = 0; i < NLIT; ++i) s[NS + i] = sc.c[i];\n}\n";
     s << "__device__ __forceinline__ void group_eval(const T* l, const T* s, T* o) {\n"
       << "    (void)l; (void)s;\n"
       << p.body << "}\n";
@@ -508,6 +556,8 @@ struct Fold { T* out[NSA]; int n[NSA]; };
 __device__ __forceinline__ void load_scalars_folding(const Scal& sc, const Fold& fd, T* s) {
     __shared__ T fold_lds[4];
 #pragma unroll
+    for (int i = 0; i < NLIT; ++i) s[NS + i] = sc.c[i];
+#pragma unroll
     for (int i = 0; i < NS; ++i) {
         if (sc.p[i] == nullptr) {
             s[i] = sc.v[i];
@@ -531,7 +581,7 @@ __device__ __forceinline__ void load_scalars_folding(const Scal& sc, const Fold&
 #define FLAT_ENTRY(NAME, CALL)                                                                   \
 extern "C" __global__ __launch_bounds__(256) void grp_flat_##NAME(const Seg* segs, int nseg,    \
                                                                   Scal sc RED_PARAM) {           \
-    T s[NSA]; load_scalars(sc, s);                                                               \
+    T s[NSV]; load_scalars(sc, s);                                                               \
     RED_BEGIN                                                                                    \
     const int k = find_seg(segs, nseg, (i64)blockIdx.x);                                         \
     const Seg& sg = segs[k];                                                                     \
@@ -540,7 +590,7 @@ extern "C" __global__ __launch_bounds__(256) void grp_flat_##NAME(const Seg* seg
     RED_END                                                                                      \
 }                                                                                                \
 extern "C" __global__ __launch_bounds__(256) void grp_flat1_##NAME(Seg sg, Scal sc RED_PARAM) { \
-    T s[NSA]; load_scalars(sc, s);                                                               \
+    T s[NSV]; load_scalars(sc, s);                                                               \
     RED_BEGIN                                                                                    \
     const i64 blk = (i64)blockIdx.x;                                                             \
     CALL;                                                                                        \
@@ -548,7 +598,7 @@ extern "C" __global__ __launch_bounds__(256) void grp_flat1_##NAME(Seg sg, Scal 
 }                                                                                                \
 extern "C" __global__ __launch_bounds__(256) void grp_flat1f_##NAME(Seg sg, Scal sc, Fold fd    \
                                                                     RED_PARAM) {                 \
-    T s[NSA]; load_scalars_folding(sc, fd, s);                                                   \
+    T s[NSV]; load_scalars_folding(sc, fd, s);                                                   \
     RED_BEGIN                                                                                    \
     const i64 blk = (i64)blockIdx.x;                                                             \
     CALL;                                                                                        \
@@ -607,21 +657,21 @@ __device__ __forceinline__ void nd_run(const Cell& c, i64 blk, const T* s) {
 }
 
 extern "C" __global__ __launch_bounds__(256) void grp_nd(const Cell* cells, int ncell, Scal sc) {
-    T s[NSA]; load_scalars(sc, s);
+    T s[NSV]; load_scalars(sc, s);
     const int k = find_seg(cells, ncell, (i64)blockIdx.x);
     nd_run<4>(cells[k], (i64)blockIdx.x - cells[k].blk0, s);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_nd1(Cell cell, Scal sc) {
-    T s[NSA]; load_scalars(sc, s);
+    T s[NSV]; load_scalars(sc, s);
     nd_run<4>(cell, (i64)blockIdx.x, s);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_nd_p1(const Cell* cells, int ncell, Scal sc) {
-    T s[NSA]; load_scalars(sc, s);
+    T s[NSV]; load_scalars(sc, s);
     const int k = find_seg(cells, ncell, (i64)blockIdx.x);
     nd_run<1>(cells[k], (i64)blockIdx.x - cells[k].blk0, s);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_nd1_p1(Cell cell, Scal sc) {
-    T s[NSA]; load_scalars(sc, s);
+    T s[NSV]; load_scalars(sc, s);
     nd_run<1>(cell, (i64)blockIdx.x, s);
 }
 )";
@@ -735,12 +785,12 @@ __device__ __forceinline__ void tiles_run(const Tiled* arrs, const DTile* dts, i
 
 extern "C" __global__ __launch_bounds__(256) void grp_tiles(const Tiled* arrs, const DTile* dts,
                                                             int ndt, TilesArgs ta, Scal sc) {
-    T s[NSA]; load_scalars(sc, s);
+    T s[NSV]; load_scalars(sc, s);
     tiles_run<false>(arrs, dts, ndt, ta, s);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_tiles_rows(const Tiled* arrs, const DTile* dts,
                                                                  int ndt, TilesArgs ta, Scal sc) {
-    T s[NSA]; load_scalars(sc, s);
+    T s[NSV]; load_scalars(sc, s);
     tiles_run<true>(arrs, dts, ndt, ta, s);
 }
 )";

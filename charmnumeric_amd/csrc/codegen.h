@@ -29,6 +29,9 @@ struct GroupProgram {
     std::vector<int> load_leaf;   // distinct load -> the leaf use that supplies its memref
     std::vector<int> bcast_nodes; // one run-time scalar per unique broadcast leaf
     std::vector<int> bcast_names; // array name of each broadcast leaf
+    // Literal scalars that are passed with the launch instead of being written into the source
+    // (s[NS + i] in the body): the text, and with it the code object, does not depend on them.
+    std::vector<double> lit_values;
     std::vector<int> out_names;   // result name of each output root
     std::vector<int> out_roots;   // root positions of the non-temp roots
     std::vector<int> out_is_set_region;
@@ -50,6 +53,10 @@ struct GroupProgram {
 // compile either (tanh/exp on integers, a unary op on a scalar, unknown opcodes).
 int build_group_program(const cnh_ast* ast, int dtype, int ndims, GroupProgram& out,
                         std::string& err);
+// The value of literal scalar `c` in element type `dtype`, as the generated source would spell it
+// (integers cast through int64, floats through double; src/jit.cpp:108-116 upstream), written to
+// out (4 or 8 bytes).
+void literal_value(int dtype, double c, void* out);
 
 // Launch geometry of the sliding-window variant. Kernel dimensions are (march, row, column).
 // A rank-3 array maps to them one to one. A rank-2 array maps to (-, dim0, dim1) — one patch per

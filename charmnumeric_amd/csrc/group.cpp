@@ -159,16 +159,20 @@ int get_function(cnh_kernel* k, const std::string& variant, const char* name, hi
     return 0;
 }
 
-// Scal { const T* p[NSA]; T v[NSA]; } as the generated code lays it out.
+// Scal { const T* p[NSA]; T v[NSA]; T c[NLITA]; } as the generated code lays it out: broadcast
+// scalars by pointer or by value, then the literal scalars the source takes as parameters.
 int pack_scalars(const GroupProgram& p, int n_scalar, const void* const* scalars, int on_device,
                  std::vector<unsigned char>& buf) {
     int ns = (int)p.bcast_nodes.size();
     CNH_CHECK(n_scalar == ns, -4, "group expects %d broadcast scalars, got %d", ns, n_scalar);
     int nsa = ns > 0 ? ns : 1;
     int esz = dtype_size(p.dtype);
-    size_t bytes = (size_t)nsa * 8 + (size_t)nsa * esz;
+    const int nlit = (int)p.lit_values.size(), nlita = nlit > 0 ? nlit : 1;
+    size_t bytes = (size_t)nsa * 8 + (size_t)nsa * esz + (size_t)nlita * esz;
     bytes = (bytes + 7) & ~size_t(7);
     buf.assign(bytes, 0);
+    for (int i = 0; i < nlit; ++i)
+        literal_value(p.dtype, p.lit_values[(size_t)i], &buf[(size_t)nsa * 8 + (size_t)(nsa + i) * esz]);
     for (int i = 0; i < ns; ++i) {
         CNH_CHECK(scalars && scalars[i], -4, "broadcast scalar %d is null", i);
         if (on_device) {
@@ -1279,6 +1283,11 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
 }
 
 } // namespace
+
+extern "C" int64_t cnh_code_objects(void) {
+    std::lock_guard<std::mutex> lk(g_cmu);
+    return (int64_t)g_code.size();
+}
 
 extern "C" int cnh_set_option(const char* name, int value) {
     CNH_CHECK(name != nullptr, -2, "null option name");

@@ -201,6 +201,12 @@ int cnh_kernel_build(cnh_kernel* k, const char* variant);
 /* How many variants whose name starts with `prefix` ("flat", "nd", "tiles", "slide", "direct")
  * have a code object, i.e. were built or launched: tells a test which kernel a launch took. */
 int cnh_kernel_variants_loaded(const cnh_kernel* k, const char* prefix);
+/* How many distinct code objects this process has compiled so far. Kernels whose generated text is
+ * the same share one: groups that differ only in literal scalars other than small multiples of a
+ * quarter do (such literals travel with the launch), so a loop whose coefficient changes every
+ * step compiles once. Upstream writes every scalar leaf into the module as a constant
+ * (src/jit.cpp:108-116). */
+int64_t cnh_code_objects(void);
 /* One fragment / one tile. scalars[i] points at one element of the group dtype; with
  * scalars_on_device != 0 they are device pointers and are read by the kernel itself (no host
  * round trip for dot results feeding later groups). */

@@ -111,6 +111,31 @@ def test_two_groups_under_one_key_stay_apart():
     L.check(L.lib.cnh_kernel_release(k2))
 
 
+def test_literals_that_vary_share_one_code_object():
+    """A literal that is no small multiple of a quarter is a launch parameter: two groups that
+    differ only in it generate the same text and share the code object (built here for gfx950
+    without a GPU); small literals stay in the source."""
+    def scaled(c):
+        b = AstBuilder(L.F64, 1)
+        t = b.binary(L.OP_MUL, 100, b.leaf(0), b.scalar(c))
+        b.binary(L.OP_ADD, 10, t, b.scalar(0.5), is_temp=False)
+        return b.finish()
+
+    ks = [H.compile_group(scaled(c), L.F64, 1) for c in (0.1234, 0.777, 1e-3)]
+    assert len({k.value for k in ks}) == 3                   # three kernels (they carry their values) ...
+    before = L.lib.cnh_code_objects()
+    for k in ks:
+        L.check(L.lib.cnh_kernel_build(k, b"flat"))
+    assert L.lib.cnh_code_objects() == before + 1            # ... one code object
+    src = [H.kernel_source(k, "flat") for k in ks]
+    assert src[0] == src[1] == src[2] and "s[NS + 0]" in src[0] and "0x1p-1" in src[0]
+    assert "0x1.f9" not in src[0]                            # 0.1234 is not in the text
+    k4 = H.compile_group(scaled(2.5), L.F64, 1)              # a small multiple of a quarter stays
+    assert "0x1.4p+1" in H.kernel_source(k4, "flat")
+    for k in ks + [k4]:
+        L.check(L.lib.cnh_kernel_release(k))
+
+
 def test_uncompilable_groups_report_an_error():
     b = AstBuilder(L.I64, 1)
     b.unary(L.OP_EXP, 2, b.leaf(0), is_temp=False)

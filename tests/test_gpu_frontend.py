@@ -107,6 +107,27 @@ def test_dot_with_ones_gives_the_bits_of_the_dot(small_tiles):
         assert got == want if np.issubdtype(dt, np.integer) else got == pytest.approx(want, rel=1e-5)
 
 
+def test_a_coefficient_that_changes_every_step_compiles_once(small_tiles):
+    """u = u + c_k * v and a stencil with a changing weight, 12 steps with 12 different Python
+    floats: NumPy's bits, and after the first step no further code object is compiled."""
+    from charmnumeric_amd import _lib as L
+    itf = small_tiles
+    rng = np.random.default_rng(4)
+    hu, hv = rng.standard_normal((70, 90)), rng.standard_normal((70, 90))
+    u, v = cnp.array(hu), cnp.array(hv)
+    counts = []
+    for k in range(12):
+        c = 0.1 + 0.0137 * k
+        w = 1.0 / (3.5 + k)
+        u = u + c * v
+        hu = hu + c * hv
+        u[1:-1, 1:-1] = w * (u[:-2, 1:-1] + u[2:, 1:-1]) + (c * u[1:-1, :-2] - u[1:-1, 2:])
+        hu[1:-1, 1:-1] = w * (hu[:-2, 1:-1] + hu[2:, 1:-1]) + (c * hu[1:-1, :-2] - hu[1:-1, 2:])
+        assert np.array_equal(u.get(itf), hu)
+        counts.append(L.lib.cnh_code_objects())
+    assert counts[-1] == counts[0], counts
+
+
 def test_shifted_slices_of_arange(small_tiles):
     src = cnp.arange(512, dtype=np.float32)
     got = (src[100:300] + src[150:350]).get(small_tiles)
