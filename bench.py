@@ -695,7 +695,10 @@ def run_jacobi(L, nd, n, tile, sweeps, reduce_every=10, reps_note=""):
         L.check(L.lib.cnh_event_elapsed_ms(e0, e1, C.byref(ms)))
         totals[label] = ms.value
     plain = [t[i] for i in range(sweeps) if i not in reducing]
-    us = 1e3 * float(np.median(plain))
+    us_pair = 1e3 * float(np.median(plain))          # one sweep between its own pair of events
+    # a sweep's cost in the loop: all sweeps between ONE pair of events (what the kernel trace shows
+    # too; the event pair around every single sweep adds 2-4 us of its own)
+    us = 1e3 * totals["without"] / sweeps
     us_red = 1e3 * float(np.median([t[i] for i in reducing])) if reducing else None
     interior = (n - 2) ** nd
     nbytes = 8.0 * ((n ** nd - (4 if nd == 2 else 0)) + interior) if nd == 2 else 8.0 * (n ** 3 + interior)
@@ -704,7 +707,8 @@ def run_jacobi(L, nd, n, tile, sweeps, reduce_every=10, reps_note=""):
            "bytes_per_sweep": nbytes, "total_ms_with_reductions": round(totals["with"], 3),
            "total_ms_without_reductions": round(totals["without"], 3),
            "reductions_add_pct": round(100.0 * (totals["with"] / totals["without"] - 1.0), 2),
-           "sweeps_times_us_per_sweep_ms": round(sweeps * us / 1e3, 3),
+           "us_per_sweep_between_its_own_events": round(us_pair, 2),
+           "hbm_frac_between_its_own_events": round(nbytes / us_pair / 1e3 / HBM_PEAK_GBS, 4),
            "us_per_reducing_sweep": round(us_red, 2) if us_red else None,
            "separate_reduction_pass_us": round(1e3 * float(np.median(tr)), 2),
            "last_reduction": last_fused, "last_reduction_by_separate_pass": last_separate,
