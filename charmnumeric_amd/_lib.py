@@ -189,6 +189,7 @@ _PROTOS = {
     "cnh_version": (C.c_int, []),
     "cnh_set_option": (C.c_int, [C.c_char_p, C.c_int]),
     "cnh_code_objects": (C.c_int64, []),
+    "cnh_code_objects_from_disk": (C.c_int64, []),
     "cnh_alloc": (C.c_int, [C.c_size_t, C.c_int, _vpp]),
     "cnh_free": (C.c_int, [C.c_void_p]),
     "cnh_memset0": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p]),

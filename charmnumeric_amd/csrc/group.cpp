@@ -7,6 +7,10 @@
 
 #include <hip/hiprtc.h>
 
+#include <unistd.h>
+
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <memory>
@@ -82,6 +86,62 @@ std::string ast_ident(const cnh_ast* ast, int dtype, int ndims) {
     return out;
 }
 
+// Code objects on disk, across processes: off unless CHARMNUMERIC_KERNEL_CACHE names a directory.
+// One file per code object, named by the hash of the generated text and holding that text in
+// full (compared before the code is trusted) next to the compiler's version; written under a
+// temporary name and renamed, so a reader never sees half a file. Any failure here just means
+// compiling as usual.
+std::string disk_cache_path(uint64_t h) {
+    const char* dir = std::getenv("CHARMNUMERIC_KERNEL_CACHE");
+    if (dir == nullptr || dir[0] == '\0')
+        return std::string();
+    int major = 0, minor = 0;
+    hiprtcVersion(&major, &minor);
+    char name[96];
+    std::snprintf(name, sizeof name, "/cnh-gfx950-rtc%d.%d-%016llx.co", major, minor, (unsigned long long)h);
+    return std::string(dir) + name;
+}
+
+bool disk_cache_load(uint64_t h, const std::string& src, std::vector<char>& code) {
+    const std::string path = disk_cache_path(h);
+    if (path.empty())
+        return false;
+    FILE* f = std::fopen(path.c_str(), "rb");
+    if (f == nullptr)
+        return false;
+    bool ok = false;
+    uint64_t head[3] = {0, 0, 0};   // magic, text bytes, code bytes
+    if (std::fread(head, sizeof head, 1, f) == 1 && head[0] == 0x314f43484e43ull && head[1] == src.size() &&
+        head[2] > 0 && head[2] < (1ull << 30)) {
+        std::string text(head[1], '\0');
+        code.resize(head[2]);
+        ok = std::fread(&text[0], 1, text.size(), f) == text.size() && text == src &&
+             std::fread(code.data(), 1, code.size(), f) == code.size();
+    }
+    std::fclose(f);
+    return ok;
+}
+
+void disk_cache_store(uint64_t h, const std::string& src, const std::vector<char>& code) {
+    const std::string path = disk_cache_path(h);
+    if (path.empty())
+        return;
+    char tmp_tail[48];
+    std::snprintf(tmp_tail, sizeof tmp_tail, ".tmp%ld", (long)getpid());
+    const std::string tmp = path + tmp_tail;
+    FILE* f = std::fopen(tmp.c_str(), "wb");
+    if (f == nullptr)
+        return;
+    const uint64_t head[3] = {0x314f43484e43ull, src.size(), code.size()};
+    const bool ok = std::fwrite(head, sizeof head, 1, f) == 1 &&
+                    std::fwrite(src.data(), 1, src.size(), f) == src.size() &&
+                    std::fwrite(code.data(), 1, code.size(), f) == code.size();
+    if (std::fclose(f) != 0 || !ok || std::rename(tmp.c_str(), path.c_str()) != 0)
+        std::remove(tmp.c_str());
+}
+
+int64_t g_disk_hits = 0;
+
 int build_variant(cnh_kernel* k, const std::string& variant, KernelVariant** out) {
     std::lock_guard<std::mutex> kernel_lock(k->mu);
     auto it = k->variants.find(variant);
@@ -109,6 +169,17 @@ int build_variant(cnh_kernel* k, const std::string& variant, KernelVariant** out
                 return 0;
             }
     }
+    {
+        auto cached = std::make_shared<CodeObject>();
+        if (disk_cache_load(h, v.src, cached->code)) {
+            cached->src = v.src;
+            g_code.emplace(h, cached);
+            ++g_disk_hits;
+            v.obj = cached;
+            *out = &v;
+            return 0;
+        }
+    }
     hiprtcProgram prog;
     hiprtcResult r = hiprtcCreateProgram(&prog, v.src.c_str(), "cnh_group.hip", 0, nullptr, nullptr);
     if (r != HIPRTC_SUCCESS)
@@ -135,6 +206,7 @@ int build_variant(cnh_kernel* k, const std::string& variant, KernelVariant** out
     obj->code.resize(cs);
     hiprtcGetCode(prog, obj->code.data());
     hiprtcDestroyProgram(&prog);
+    disk_cache_store(h, obj->src, obj->code);
     g_code.emplace(h, obj);
     v.obj = obj;
     *out = &v;
@@ -1283,6 +1355,11 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
 }
 
 } // namespace
+
+extern "C" int64_t cnh_code_objects_from_disk(void) {
+    std::lock_guard<std::mutex> lk(g_cmu);
+    return g_disk_hits;
+}
 
 extern "C" int64_t cnh_code_objects(void) {
     std::lock_guard<std::mutex> lk(g_cmu);

@@ -207,6 +207,12 @@ int cnh_kernel_variants_loaded(const cnh_kernel* k, const char* prefix);
  * step compiles once. Upstream writes every scalar leaf into the module as a constant
  * (src/jit.cpp:108-116). */
 int64_t cnh_code_objects(void);
+/* With the environment variable CHARMNUMERIC_KERNEL_CACHE naming a directory, code objects are also
+ * kept there, one file each (named by the hash of the generated text, which the file repeats in
+ * full and which is compared before the code is used), and a later process loads them instead of
+ * compiling: how many of the code objects above came from there. Off when the variable is unset.
+ * Upstream compiles every group anew in every run (src/dag_group_compile.cpp:6-56). */
+int64_t cnh_code_objects_from_disk(void);
 /* One fragment / one tile. scalars[i] points at one element of the group dtype; with
  * scalars_on_device != 0 they are device pointers and are read by the kernel itself (no host
  * round trip for dot results feeding later groups). */

@@ -156,3 +156,30 @@ def test_slide_variant_builds_for_3d_and_is_refused_for_other_groups():
     assert "SL_SHIFT[NLA][3] = {{-1, 0, 0}, {1, 0, 0}, {0, -1, 0}, {0, 1, 0}, {0, 0, -1}, {0, 0, 1}}" in src
     k1 = H.compile_group(H.ast_c1(L.F64), L.F64, 1)
     assert L.lib.cnh_kernel_build(k1, b"slide") < 0
+
+
+def test_code_objects_kept_on_disk_are_loaded_by_the_next_process(tmp_path):
+    """CHARMNUMERIC_KERNEL_CACHE: the first process compiles and writes one file per code object,
+    the second loads it (no compile); a damaged file is ignored."""
+    import subprocess
+    import sys
+
+    prog = (
+        "import ctypes as C\n"
+        "from charmnumeric_amd import _lib as L\n"
+        "from tests import helpers as H\n"
+        "k = H.compile_group(H.ast_jacobi2d(64), L.F64, 2)\n"
+        "L.check(L.lib.cnh_kernel_build(k, b'tiles'))\n"
+        "print(L.lib.cnh_code_objects(), L.lib.cnh_code_objects_from_disk())\n"
+    )
+    env = dict(os.environ, CHARMNUMERIC_KERNEL_CACHE=str(tmp_path), PYTHONPATH=os.getcwd())
+    run = lambda: subprocess.run([sys.executable, "-c", prog], env=env, capture_output=True, text=True, check=True).stdout.split()
+    assert run() == ["1", "0"]
+    files = list(tmp_path.iterdir())
+    assert len(files) == 1 and files[0].name.startswith("cnh-gfx950-") and files[0].stat().st_size > 1000
+    assert run() == ["1", "1"]
+    data = bytearray(files[0].read_bytes())
+    data[40] ^= 0xFF                                   # inside the stored text: no longer this group's
+    files[0].write_bytes(bytes(data))
+    assert run() == ["1", "0"]
+    assert run() == ["1", "1"]                         # rewritten by the process that had to compile

@@ -627,3 +627,30 @@ def test_slices_of_another_rank_are_assigned_through_a_copy(itf):
     A[4, 2:10] = u[30:38] * 2.0
     hA[4, 2:10] = hu[30:38] * 2.0
     assert np.array_equal(A.get(itf), hA) and np.array_equal(v.get(itf), hv)
+
+
+def test_code_objects_from_the_disk_cache_run(tmp_path):
+    """A second process loads the code objects the first one compiled (CHARMNUMERIC_KERNEL_CACHE)
+    and computes the same bits with them."""
+    import subprocess
+    import sys
+
+    prog = (
+        "import numpy as np\n"
+        "import charmnumeric_amd as cnp\n"
+        "from charmnumeric_amd import _lib as L\n"
+        "itf = cnp.CharmNumericInterface(device=0); itf.connect(odf=4)\n"
+        "h = np.arange(4096.0).reshape(64, 64) / 7.0\n"
+        "u = cnp.array(h)\n"
+        "u[1:-1, 1:-1] = 0.3 * (u[:-2, 1:-1] + u[2:, 1:-1]) + cnp.tanh(u[1:-1, :-2] * 0.01)\n"
+        "s = (u @ cnp.ones((64,))).get(itf)\n"
+        "print(L.lib.cnh_code_objects(), L.lib.cnh_code_objects_from_disk(), s.tobytes().hex())\n"
+        "itf.close()\n"
+    )
+    env = dict(os.environ, CHARMNUMERIC_KERNEL_CACHE=str(tmp_path), PYTHONPATH=os.getcwd())
+    run = lambda: subprocess.run([sys.executable, "-c", prog], env=env, capture_output=True, text=True,
+                                 check=True, timeout=150).stdout.split()
+    first, second = run(), run()
+    assert int(first[0]) >= 1 and first[1] == "0"
+    assert second[0] == first[0] and second[1] == first[0]       # every code object came from disk
+    assert second[2] == first[2]
