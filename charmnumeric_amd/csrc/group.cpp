@@ -151,12 +151,17 @@ int build_variant(cnh_kernel* k, const std::string& variant, KernelVariant** out
     }
     KernelVariant& v = k->variants[variant];
     if (v.src.empty()) {
+        // "variant#entry": the variant's text built for that one entry point only
+        const size_t hash_at = variant.find('#');
+        const std::string base = variant.substr(0, hash_at);
         std::string err;
-        int rc = emit_variant_source(k->prog, variant, v.src, err);
+        int rc = emit_variant_source(k->prog, base, v.src, err);
         if (rc) {
             k->variants.erase(variant);
             return set_error(rc, "codegen(%s): %s", variant.c_str(), err.c_str());
         }
+        if (hash_at != std::string::npos)
+            v.src = "#define CNH_ONLY 1\n#define CNH_IS_" + variant.substr(hash_at + 1) + " 1\n" + v.src;
     }
     const uint64_t h = text_hash(v.src);
     std::lock_guard<std::mutex> code_lock(g_cmu);
@@ -215,7 +220,9 @@ int build_variant(cnh_kernel* k, const std::string& variant, KernelVariant** out
 
 int get_function(cnh_kernel* k, const std::string& variant, const char* name, hipFunction_t* fn) {
     KernelVariant* v = nullptr;
-    if (int rc = build_variant(k, variant, &v))
+    // groups that carry the exp/tanh text build the flat and strided-cell variants per entry point
+    const bool per_entry = k->prog.uses_transcendental && (variant == "flat" || variant == "nd");
+    if (int rc = build_variant(k, per_entry ? variant + "#" + name : variant, &v))
         return rc;
     CodeObject* c = v->obj.get();
     std::lock_guard<std::mutex> object_lock(c->mu);
