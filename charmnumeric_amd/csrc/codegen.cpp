@@ -379,14 +379,12 @@ std::string prelude(const GroupProgram& p) {
               << "__device__ __forceinline__ T cn_exp(T x) { return cn_exp_f32(x); }\n"
                  "__device__ __forceinline__ T cn_tanh(T x) { return cn_tanh_f32(x); }\n";
     }
-    // A code object may be built for ONE of the flat / strided-cell entry points (CNH_ONLY with
-    // CNH_IS_<entry> = 1 set ahead of this text): the others return at once and cost the compiler
-    // nothing, which matters for groups that carry the exp/tanh text (seconds per entry point).
-    s << "#ifdef CNH_ONLY\n#define CNH_SKIP(name) (CNH_IS_##name == 0)\n#else\n#define CNH_SKIP(name) false\n#endif\n";
-    for (const char* e : {"grp_flat_v", "grp_flat_vn", "grp_flat_s", "grp_flat1_v", "grp_flat1_vn", "grp_flat1_s",
-                          "grp_flat1f_v", "grp_flat1f_vn", "grp_flat1f_s", "grp_nd", "grp_nd1", "grp_nd_p1",
-                          "grp_nd1_p1"})
-        s << "#ifndef CNH_IS_" << e << "\n#define CNH_IS_" << e << " 0\n#endif\n";
+    // A code object may be built for ONE entry point (CNH_ONLY_NAME set ahead of this text): every
+    // other entry point returns at once and costs the compiler nothing. The comparison of two
+    // constant strings is folded at compile time.
+    s << "#ifdef CNH_ONLY_NAME\n"
+         "#define CNH_ENTRY_GUARD if (__builtin_strcmp(__func__, CNH_ONLY_NAME) != 0) return;\n"
+         "#else\n#define CNH_ENTRY_GUARD\n#endif\n";
     s << "__device__ __forceinline__ void load_scalars(const Scal& sc, T* s) {\n"
          "#pragma unroll\n"
          "    for (int i = 0; i < NS; ++i) s[i] = sc.p[i] ? *sc.p[i] : sc.v[i];\n"
@@ -589,8 +587,7 @@ __device__ __forceinline__ void load_scalars_folding(const Scal& sc, const Fold&
 #define FLAT_ENTRY(NAME, CALL)                                                                   \
 extern "C" __global__ __launch_bounds__(256) void grp_flat_##NAME(const Seg* segs, int nseg,    \
                                                                   Scal sc RED_PARAM) {           \
-    if (CNH_SKIP(grp_flat_##NAME)) return;                                                       \
-    T s[NSV]; load_scalars(sc, s);                                                               \
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);                                                               \
     RED_BEGIN                                                                                    \
     const int k = find_seg(segs, nseg, (i64)blockIdx.x);                                         \
     const Seg& sg = segs[k];                                                                     \
@@ -599,8 +596,7 @@ extern "C" __global__ __launch_bounds__(256) void grp_flat_##NAME(const Seg* seg
     RED_END                                                                                      \
 }                                                                                                \
 extern "C" __global__ __launch_bounds__(256) void grp_flat1_##NAME(Seg sg, Scal sc RED_PARAM) { \
-    if (CNH_SKIP(grp_flat1_##NAME)) return;                                                      \
-    T s[NSV]; load_scalars(sc, s);                                                               \
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);                                                               \
     RED_BEGIN                                                                                    \
     const i64 blk = (i64)blockIdx.x;                                                             \
     CALL;                                                                                        \
@@ -608,8 +604,7 @@ extern "C" __global__ __launch_bounds__(256) void grp_flat1_##NAME(Seg sg, Scal 
 }                                                                                                \
 extern "C" __global__ __launch_bounds__(256) void grp_flat1f_##NAME(Seg sg, Scal sc, Fold fd    \
                                                                     RED_PARAM) {                 \
-    if (CNH_SKIP(grp_flat1f_##NAME)) return;                                                     \
-    T s[NSV]; load_scalars_folding(sc, fd, s);                                                   \
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars_folding(sc, fd, s);                                                   \
     RED_BEGIN                                                                                    \
     const i64 blk = (i64)blockIdx.x;                                                             \
     CALL;                                                                                        \
@@ -668,25 +663,21 @@ __device__ __forceinline__ void nd_run(const Cell& c, i64 blk, const T* s) {
 }
 
 extern "C" __global__ __launch_bounds__(256) void grp_nd(const Cell* cells, int ncell, Scal sc) {
-    if (CNH_SKIP(grp_nd)) return;
-    T s[NSV]; load_scalars(sc, s);
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
     const int k = find_seg(cells, ncell, (i64)blockIdx.x);
     nd_run<4>(cells[k], (i64)blockIdx.x - cells[k].blk0, s);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_nd1(Cell cell, Scal sc) {
-    if (CNH_SKIP(grp_nd1)) return;
-    T s[NSV]; load_scalars(sc, s);
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
     nd_run<4>(cell, (i64)blockIdx.x, s);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_nd_p1(const Cell* cells, int ncell, Scal sc) {
-    if (CNH_SKIP(grp_nd_p1)) return;
-    T s[NSV]; load_scalars(sc, s);
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
     const int k = find_seg(cells, ncell, (i64)blockIdx.x);
     nd_run<1>(cells[k], (i64)blockIdx.x - cells[k].blk0, s);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_nd1_p1(Cell cell, Scal sc) {
-    if (CNH_SKIP(grp_nd1_p1)) return;
-    T s[NSV]; load_scalars(sc, s);
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
     nd_run<1>(cell, (i64)blockIdx.x, s);
 }
 )";
@@ -800,12 +791,12 @@ __device__ __forceinline__ void tiles_run(const Tiled* arrs, const DTile* dts, i
 
 extern "C" __global__ __launch_bounds__(256) void grp_tiles(const Tiled* arrs, const DTile* dts,
                                                             int ndt, TilesArgs ta, Scal sc) {
-    T s[NSV]; load_scalars(sc, s);
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
     tiles_run<false>(arrs, dts, ndt, ta, s);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_tiles_rows(const Tiled* arrs, const DTile* dts,
                                                                  int ndt, TilesArgs ta, Scal sc) {
-    T s[NSV]; load_scalars(sc, s);
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
     tiles_run<true>(arrs, dts, ndt, ta, s);
 }
 )";

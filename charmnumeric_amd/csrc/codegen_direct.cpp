@@ -895,7 +895,7 @@ __device__ __forceinline__ void direct_flat(const FlatArgs& a, const T* s) {
 // The reducing forms only (built on demand under a variant name of their own).
 #define FLAT_RED_ENTRY(NAME, NTS, RED)                                                            \
 extern "C" __global__ __launch_bounds__(256) void NAME(FlatArgs a, Scal sc) {                     \
-    T s[NSV]; load_scalars(sc, s);                                                                \
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);                                                                \
     direct_flat<NTS, RED>(a, s);                                                                  \
 }
 FLAT_RED_ENTRY(grp_direct_flat_red1, false, 1)
@@ -905,7 +905,7 @@ FLAT_RED_ENTRY(grp_direct_flat_red2_nts, true, 2)
 // Tiles with buffers of their own: the lean part and the listed face workgroups in one launch.
 #define BOTH_RED_ENTRY(NAME, NTS, RED)                                                            \
 extern "C" __global__ __launch_bounds__(256) void NAME(DirectArgs a, Scal sc, const int* list) {  \
-    T s[NSV]; load_scalars(sc, s);                                                                \
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);                                                                \
     if ((int)blockIdx.x < a.nblocks) direct_fast<NTS, RED>(a, s);                                 \
     else direct_rest<NTS, RED>(a, s, 1, list, a.nblocks);                                         \
 }
@@ -915,43 +915,43 @@ BOTH_RED_ENTRY(grp_direct_both_red2, false, 2)
 BOTH_RED_ENTRY(grp_direct_both_red2_nts, true, 2)
 #else
 extern "C" __global__ __launch_bounds__(256) void grp_direct_flat(FlatArgs a, Scal sc) {
-    T s[NSV]; load_scalars(sc, s);
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
     direct_flat<false, 0>(a, s);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_direct_flat_nts(FlatArgs a, Scal sc) {
-    T s[NSV]; load_scalars(sc, s);
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
     direct_flat<true, 0>(a, s);
 }
 
 // nts: the written stream is not read back soon, store it non-temporally.
 extern "C" __global__ __launch_bounds__(256) void grp_direct_fast(DirectArgs a, Scal sc) {
-    T s[NSV]; load_scalars(sc, s);
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
     direct_fast<false, 0>(a, s);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_direct_fast_nts(DirectArgs a, Scal sc) {
-    T s[NSV]; load_scalars(sc, s);
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
     direct_fast<true, 0>(a, s);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_direct_rest(DirectArgs a, Scal sc, int skip_fast,
                                                                   const int* list) {
-    T s[NSV]; load_scalars(sc, s);
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
     direct_rest<false, 0>(a, s, skip_fast, list, 0);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_direct_rest_nts(DirectArgs a, Scal sc, int skip_fast,
                                                                       const int* list) {
-    T s[NSV]; load_scalars(sc, s);
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
     direct_rest<true, 0>(a, s, skip_fast, list, 0);
 }
 // Both in one launch: the first a.nblocks workgroups do the lean part, the ones after them what
 // the lean part leaves (those on `list`, or all positions again when there is no list). One
 // launch and no gap between the two, and the second part fills the tail of the first.
 extern "C" __global__ __launch_bounds__(256) void grp_direct_both(DirectArgs a, Scal sc, const int* list) {
-    T s[NSV]; load_scalars(sc, s);
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
     if ((int)blockIdx.x < a.nblocks) direct_fast<false, 0>(a, s);
     else direct_rest<false, 0>(a, s, 1, list, a.nblocks);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_direct_both_nts(DirectArgs a, Scal sc, const int* list) {
-    T s[NSV]; load_scalars(sc, s);
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
     if ((int)blockIdx.x < a.nblocks) direct_fast<true, 0>(a, s);
     else direct_rest<true, 0>(a, s, 1, list, a.nblocks);
 }

@@ -340,15 +340,15 @@ __device__ __forceinline__ void slide_run(const SlideArgs& a, const T* s) {
 }
 
 extern "C" __global__ __launch_bounds__(256) void grp_slide_v(SlideArgs a, Scal sc) {
-    T s[NSV]; load_scalars(sc, s);
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
     slide_run<true, false>(a, s);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_slide_vn(SlideArgs a, Scal sc) {
-    T s[NSV]; load_scalars(sc, s);
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
     slide_run<true, true>(a, s);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_slide_s(SlideArgs a, Scal sc) {
-    T s[NSV]; load_scalars(sc, s);
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
     slide_run<false, false>(a, s);
 }
 )";
