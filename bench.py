@@ -819,7 +819,7 @@ def lstm_fused_ast(L, first):
     return b.finish()
 
 
-def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=False, fused=True):
+def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=False, fused=True, warm_passes=5):
     k_in = nin + d
     X = Buf(L, steps * batch * nin * 8)
     W = Buf(L, k_in * 4 * d * 8)
@@ -951,33 +951,47 @@ def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=
     e0, e1 = C.c_void_p(), C.c_void_p()
     L.check(L.lib.cnh_event_create(C.byref(e0)))
     L.check(L.lib.cnh_event_create(C.byref(e1)))
-    total_ms, wall = C.c_float(0.0), 0.0
-    if timed:
-        run_steps(min(steps, 3), False)      # warm-up (builds the kernels)
-        L.check(L.lib.cnh_stream_sync(stream))
-    # one pass with an event pair around every product (the product's own duration) ...
-    run_steps(steps, True)
-    L.check(L.lib.cnh_stream_sync(stream))
-    g = ev.times_ms(steps)
-    if timed:
-        # ... then the pass that is timed as a whole: one event pair around all steps, nothing
-        # between the launches
-        w0 = time.perf_counter()
-        L.check(L.lib.cnh_event_record(e0, stream))
-        run_steps(steps, False)
-        L.check(L.lib.cnh_event_record(e1, stream))
-        L.check(L.lib.cnh_stream_sync(stream))
-        wall = time.perf_counter() - w0
-        L.check(L.lib.cnh_event_elapsed_ms(e0, e1, C.byref(total_ms)))
     flop = 2.0 * batch * k_in * 4 * d
-    gus = 1e3 * float(np.median(g))
+    if timed:
+        run_steps(min(steps, 3), False)      # builds the kernels
+        L.check(L.lib.cnh_stream_sync(stream))
+
+    def measure(warm):
+        """(median product time, whole-pass time per step), each after `warm` untimed passes queued
+        right ahead of it: no pause, the device never idles between them and the measured pass."""
+        total_ms = C.c_float(0.0)
+        for _ in range(warm):
+            run_steps(steps, False)
+        run_steps(steps, True)               # an event pair around every product
+        L.check(L.lib.cnh_stream_sync(stream))
+        g = ev.times_ms(steps)
+        if timed:
+            for _ in range(warm):
+                run_steps(steps, False)
+            L.check(L.lib.cnh_event_record(e0, stream))
+            run_steps(steps, False)          # one event pair around all steps, nothing between the launches
+            L.check(L.lib.cnh_event_record(e1, stream))
+            L.check(L.lib.cnh_stream_sync(stream))
+            L.check(L.lib.cnh_event_elapsed_ms(e0, e1, C.byref(total_ms)))
+        return 1e3 * float(np.median(g)), 1e3 * total_ms.value / steps
+
+    # The matrix pipe's clock rises under sustained load: right after an idle device the product
+    # takes 81-87 us, after about 30 ms of uninterrupted steps 72-73 us (measured on MI355X; the
+    # HBM-bound workloads do not change). Both are reported; the sustained figure is the one a long
+    # sequence sees and the one the fraction of peak is computed from.
+    gus_idle, step_idle = measure(0)
+    gus, step_us = measure(warm_passes) if (timed and warm_passes > 0) else (gus_idle, step_idle)
     ceiling = C.c_double()
     L.check(L.lib.cnh_probe_mfma_f64(8192, C.byref(ceiling)))   # ~1 ms of back-to-back matrix instructions
     out = {"steps": steps, "gemm_us": round(gus, 2), "gemm_tflops": round(flop / gus / 1e6, 2),
            "mfma_frac": round(flop / gus / 1e6 / FP64_MFMA_PEAK_TFLOPS, 4),
            "mfma_measured_ceiling_tflops": round(ceiling.value, 1),
            "mfma_frac_of_measured_ceiling": round(flop / gus / 1e6 / ceiling.value, 4) if ceiling.value else None,
-           "step_us": round(1e3 * total_ms.value / steps, 2), "step_wall_us": round(1e6 * wall / steps, 2),
+           "step_us": round(step_us, 2),
+           "untimed_passes_queued_ahead": warm_passes if timed else 0,
+           "after_an_idle_device": {"gemm_us": round(gus_idle, 2),
+                                    "mfma_frac": round(flop / gus_idle / 1e6 / FP64_MFMA_PEAK_TFLOPS, 4),
+                                    "step_us": round(step_idle, 2)},
            "flop_per_step": flop}
     if keep:
         out["Hout"] = Hout.get().reshape(steps, batch, d)
@@ -1145,7 +1159,7 @@ def run_frontend(n, steps, warmup):
         Cs = cnp.zeros((n, b, d))
         Ct = cnp.zeros((n, b, d))
 
-        def lstm_steps(t0, t1):
+        def lstm_steps(t0, t1, wait=True):
             for t in range(t0, t1):
                 prev = cnp.tile(h0, (b, 1)) if t == 0 else Hout[t - 1]
                 Hin[t, :, :word] = X[t]
@@ -1159,7 +1173,8 @@ def run_frontend(n, steps, warmup):
                 Ct[t] = cnp.tanh(Cs[t])
                 Hout[t] = IFOGf[t, :, 2 * d: 3 * d] * Ct[t]
             cnp.execute(itl)
-            itl.sync()
+            if wait:
+                itl.sync()
 
         # the whole sequence twice: the first pass also compiles every kernel the program needs
         # (the merged statement runs of steps 0, 1 and of the later ones), the second is what a
@@ -1167,10 +1182,15 @@ def run_frontend(n, steps, warmup):
         t0 = time.perf_counter()
         lstm_steps(0, n)
         out["lstm_first_pass_us_per_step"] = round((time.perf_counter() - t0) / n * 1e6, 1)
+        # six passes without a pause between them (the executor's thread and the device run on while
+        # the next pass is recorded): what a long sequence costs per step, clock rise included
+        passes = 6
         t0 = time.perf_counter()
-        lstm_steps(0, n)
+        for q in range(passes):
+            lstm_steps(0, n, wait=q == passes - 1)
         dt = time.perf_counter() - t0
-        out["lstm_us_per_step"] = round(dt / n * 1e6, 1)
+        out["lstm_us_per_step"] = round(dt / (passes * n) * 1e6, 1)
+        out["lstm_passes_timed"] = passes
         out["lstm_h_last_abs_mean"] = float(np.mean(np.abs(Hout[n - 1].get(itl))))
         del X, W, h0, Hin, Hout, IFOG, IFOGf, Cs, Ct
         cnp.execute(itl)
