@@ -25,6 +25,11 @@ struct Chunk {
 };
 
 constexpr int kThreads = 256;
+// Stage 1 runs 512 lanes a workgroup and stage 2 one workgroup of 1024: over 2^24 doubles the pair took
+// 23.6 us with 256 and 256, 22.9 us with 256 and 1024, 22.45 us with 512 and 1024 (stage 2 then reads
+// its 2048 slots two to a lane instead of eight).
+constexpr int kStage1Threads = 512;
+constexpr int kStage2Threads = 1024;
 constexpr int kMaxBlocksPerChunk = 65536;
 
 template <typename T>
@@ -167,8 +172,8 @@ __device__ __forceinline__ void stage1_body(const Chunk& c, int rel, typename Ac
     typedef typename Acc<T>::type A;
     const int64_t b0 = (int64_t)rel * c.per_block;
     const int64_t b1 = b0 + c.per_block < c.n ? b0 + c.per_block : c.n;
-    A v = slice_reduce<T, MODE, kThreads>((const T*)c.a, (const T*)c.b, b0, b1);
-    v = block_reduce<A, MODE, kThreads>(v, lds);
+    A v = slice_reduce<T, MODE, kStage1Threads>((const T*)c.a, (const T*)c.b, b0, b1);
+    v = block_reduce<A, MODE, kStage1Threads>(v, lds);
     if (threadIdx.x == 0)
         *slot = v;
 }
@@ -180,17 +185,17 @@ __device__ __forceinline__ typename Acc<T>::type stage2_chunk(const typename Acc
                                                                int nb, typename Acc<T>::type* lds) {
     typedef typename Acc<T>::type A;
     A v = 0;
-    for (int i = threadIdx.x; i < nb; i += kThreads)
+    for (int i = threadIdx.x; i < nb; i += kStage2Threads)
         v = combine<A, MODE>(v, slots[i]);
-    return block_reduce<A, MODE, kThreads>(v, lds);
+    return block_reduce<A, MODE, kStage2Threads>(v, lds);
 }
 
 template <typename T, int MODE>
-__global__ __launch_bounds__(kThreads) void reduce_stage1(const Chunk* __restrict__ chunks,
-                                                          int nchunk,
-                                                          typename Acc<T>::type* __restrict__ partials) {
+__global__ __launch_bounds__(kStage1Threads) void reduce_stage1(const Chunk* __restrict__ chunks,
+                                                                int nchunk,
+                                                                typename Acc<T>::type* __restrict__ partials) {
     typedef typename Acc<T>::type A;
-    __shared__ A lds[kThreads / 64];
+    __shared__ A lds[kStage1Threads / 64];
     int lo = 0, hi = nchunk - 1;
     const int blk = blockIdx.x;
     while (lo < hi) {
@@ -208,11 +213,11 @@ __global__ __launch_bounds__(kThreads) void reduce_stage1(const Chunk* __restric
 // t, t + 256, ... in that order, then the fixed tree. One trip to memory for all slots instead of
 // one per chunk (a chunk at a time cost 4.6 us for the four partitions of 2^24 elements).
 template <typename T, int MODE>
-__global__ __launch_bounds__(kThreads) void reduce_stage2(int nslots,
-                                                          const typename Acc<T>::type* __restrict__ partials,
-                                                          T* __restrict__ out) {
+__global__ __launch_bounds__(kStage2Threads) void reduce_stage2(int nslots,
+                                                                const typename Acc<T>::type* __restrict__ partials,
+                                                                T* __restrict__ out) {
     typedef typename Acc<T>::type A;
-    __shared__ A lds[kThreads / 64];
+    __shared__ A lds[kStage2Threads / 64];
     A v = stage2_chunk<T, MODE>(partials, nslots, lds);
     if (threadIdx.x == 0)
         *out = (T)v;
@@ -220,19 +225,19 @@ __global__ __launch_bounds__(kThreads) void reduce_stage2(int nslots,
 
 // The same two stages for a single chunk handed over by value: no descriptor table on the device.
 template <typename T, int MODE>
-__global__ __launch_bounds__(kThreads) void reduce_stage1_one(const Chunk c,
-                                                              typename Acc<T>::type* __restrict__ partials) {
+__global__ __launch_bounds__(kStage1Threads) void reduce_stage1_one(const Chunk c,
+                                                                    typename Acc<T>::type* __restrict__ partials) {
     typedef typename Acc<T>::type A;
-    __shared__ A lds[kThreads / 64];
+    __shared__ A lds[kStage1Threads / 64];
     stage1_body<T, MODE>(c, blockIdx.x, lds, partials + blockIdx.x);
 }
 
 template <typename T, int MODE>
-__global__ __launch_bounds__(kThreads) void reduce_stage2_one(int nblk,
-                                                              const typename Acc<T>::type* __restrict__ partials,
-                                                              T* __restrict__ out) {
+__global__ __launch_bounds__(kStage2Threads) void reduce_stage2_one(int nblk,
+                                                                    const typename Acc<T>::type* __restrict__ partials,
+                                                                    T* __restrict__ out) {
     typedef typename Acc<T>::type A;
-    __shared__ A lds[kThreads / 64];
+    __shared__ A lds[kStage2Threads / 64];
     A v = stage2_chunk<T, MODE>(partials, nblk, lds);
     if (threadIdx.x == 0)
         *out = (T)v;
@@ -316,13 +321,15 @@ int run_tiles(int n_tiles, const void* const* a, const void* const* b, const int
     void* ws = nullptr;
     if (int rc = reduce_workspace(st, (size_t)blocks * sizeof(A), &ws))
         return rc;
+    // The chunk table stays in device memory: handed over by value (8 chunks, 320 bytes of kernel
+    // arguments) the same launch took 0.8 us longer.
     const void* dchunks = nullptr;
     if (int rc = desc_upload(chunks.data(), chunks.size() * sizeof(Chunk), st, &dchunks))
         return rc;
-    hipLaunchKernelGGL((reduce_stage1<T, MODE>), dim3(blocks), dim3(kThreads), 0, st,
+    hipLaunchKernelGGL((reduce_stage1<T, MODE>), dim3(blocks), dim3(kStage1Threads), 0, st,
                        (const Chunk*)dchunks, n_tiles, (A*)ws);
     CNH_HIP(hipGetLastError());
-    hipLaunchKernelGGL((reduce_stage2<T, MODE>), dim3(1), dim3(kThreads), 0, st, blocks, (const A*)ws,
+    hipLaunchKernelGGL((reduce_stage2<T, MODE>), dim3(1), dim3(kStage2Threads), 0, st, blocks, (const A*)ws,
                        (T*)out);
     CNH_HIP(hipGetLastError());
     return 0;
@@ -361,9 +368,10 @@ int run_dot_noalloc(int64_t n, const void* a, const void* b, void* out, void* sl
     const Chunk c = plan_chunk(a, b, n, 0);
     CNH_CHECK(c.nblk <= kScratchSlots, -3, "cnh_dot_partial_noalloc: %d partial slots needed, %d held",
               c.nblk, kScratchSlots);
-    hipLaunchKernelGGL((reduce_stage1_one<T, M_DOT>), dim3(c.nblk), dim3(kThreads), 0, st, c, (A*)slots);
+    hipLaunchKernelGGL((reduce_stage1_one<T, M_DOT>), dim3(c.nblk), dim3(kStage1Threads), 0, st, c,
+                       (A*)slots);
     CNH_HIP(hipGetLastError());
-    hipLaunchKernelGGL((reduce_stage2_one<T, M_DOT>), dim3(1), dim3(kThreads), 0, st, c.nblk,
+    hipLaunchKernelGGL((reduce_stage2_one<T, M_DOT>), dim3(1), dim3(kStage2Threads), 0, st, c.nblk,
                        (const A*)slots, (T*)out);
     CNH_HIP(hipGetLastError());
     return 0;
