@@ -218,6 +218,52 @@ def test_sumsq_and_maxabs_diff(dev, orc):
     dev.free_all()
 
 
+@pytest.mark.parametrize("dt,npdt", [(L.F64, np.float64), (L.F32, np.float32), (L.I64, np.int64), (L.I32, np.int32)])
+def test_reductions_count_every_element_once(dev, dt, npdt):
+    """Small integer values make sums and dots exact in any order of additions, so an element that a
+    slice boundary, a ragged end or a misaligned start drops or takes twice changes the result.
+    Tile lengths sit on and around the slice sizes (512, 8192 per workgroup, 65536 for the one-launch
+    form); every tile also runs from a start that is not 16-byte aligned."""
+    rng = np.random.default_rng(11)
+    esz = np.dtype(npdt).itemsize
+    lens = [1, 2, 3, 511, 512, 513, 1023, 1025, 8191, 8192, 8193, 12289, 65535, 65536, 65537,
+            65536 + 8192, 100003, 3 * 8192 + 7, 1 << 20, (1 << 20) + 1]
+    hi = 3 if npdt == np.float32 else 50          # float32 sums stay below 2^24
+    for shift in (0, 1):
+        host_a = [rng.integers(-hi, hi + 1, n + shift).astype(npdt) for n in lens]
+        host_b = [rng.integers(-hi, hi + 1, n + shift).astype(npdt) for n in lens]
+        da = [dev.array(x) for x in host_a]
+        db = [dev.array(x) for x in host_b]
+        out = dev.empty((1,), npdt)
+        for i, n in enumerate(lens):           # tiles one at a time
+            a, b = host_a[i][shift:], host_b[i][shift:]
+            pa, pb = da[i].ptr + shift * esz, db[i].ptr + shift * esz
+            L.check(L.lib.cnh_dot_partial(dt, n, pa, pb, out.ptr, None))
+            assert out.get()[0] == np.sum(a.astype(np.int64) * b.astype(np.int64)), (n, shift, "dot")
+            L.check(L.lib.cnh_sum_tiles(dt, 1, L.vparr([pa]), L.i64arr([n]), out.ptr, None))
+            assert out.get()[0] == np.sum(a.astype(np.int64)), (n, shift, "sum")
+        # all tiles in one call
+        pas = [d.ptr + shift * esz for d in da]
+        pbs = [d.ptr + shift * esz for d in db]
+        L.check(L.lib.cnh_dot_tiles(dt, len(lens), L.vparr(pas), L.vparr(pbs), L.i64arr(lens), out.ptr, None))
+        want = sum(int(np.sum(a[shift:].astype(np.int64) * b[shift:].astype(np.int64)))
+                   for a, b in zip(host_a, host_b))
+        assert out.get()[0] == want, (shift, "dot over all tiles")
+        L.check(L.lib.cnh_sum_tiles(dt, len(lens), L.vparr(pas), L.i64arr(lens), out.ptr, None))
+        assert out.get()[0] == sum(int(np.sum(a[shift:].astype(np.int64))) for a in host_a)
+        if npdt == np.float64:
+            o64 = dev.empty((1,), np.float64)
+            L.check(L.lib.cnh_sumsq_diff_tiles(len(lens), L.vparr(pas), L.vparr(pbs), L.i64arr(lens),
+                                               o64.ptr, None))
+            assert o64.get()[0] == sum(float(np.sum((a[shift:] - b[shift:]) ** 2))
+                                       for a, b in zip(host_a, host_b))
+            L.check(L.lib.cnh_maxabs_diff_tiles(len(lens), L.vparr(pas), L.vparr(pbs), L.i64arr(lens),
+                                                o64.ptr, None))
+            assert o64.get()[0] == max(float(np.max(np.abs(a[shift:] - b[shift:])))
+                                       for a, b in zip(host_a, host_b))
+        dev.free_all()
+
+
 def _check_matvec(got, A, x):
     ref = np.array([math.fsum((A[i] * x).tolist()) for i in range(A.shape[0])])
     denom = np.abs(A) @ np.abs(x)
