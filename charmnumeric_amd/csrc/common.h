@@ -63,6 +63,7 @@ int reduce_slots_f64_many(int nvec, const int* maximum, double* const* vecs, int
                           hipStream_t st);
 void gemv_set_xlds(int on);
 void gemm_set_buffer_loads(int on);
+void gemm_set_ksplit(int on);
 int reduce_slots_f64(bool maximum, double* slots, int64_t n, double* out, hipStream_t st);
 
 // Descriptor tables (per-partition pointers/shapes) live on the device. Identical tables are

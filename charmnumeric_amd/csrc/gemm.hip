@@ -51,13 +51,17 @@ static_assert(sizeof(GemmSeg) == 40 && sizeof(GemmChain) == 40, "descriptor tabl
 // buffer being filled while the other is read): one K step of matrix instructions is shorter than
 // a trip to memory. A workgroup keeps its accumulators across the segments of its chain, so the
 // panel products of one C block cost one pass over C however many K pieces they come in.
-template <int WM, int WN, int TM, int TN, int BKT, bool FULL, bool BUF = false>
-__global__ __launch_bounds__(WM * WN * 64) void gemm_f64_mfma(const GemmChain* __restrict__ chains,
-                                                              int nchains,
-                                                              const GemmSeg* __restrict__ segs,
-                                                              int nblocks, GemmChain only_chain,
-                                                              GemmSeg only_seg, int overwrite) {
-    constexpr int NT = WM * WN * 64;
+// KS = 2: the workgroup is two such sets of wavefronts; set g takes the K steps g, g + 2, ... of every
+// segment into accumulators of its own (staging buffers of its own too), and at the end the second
+// set hands its sums over through LDS and the first adds them, first + second, and stores. Twice
+// the wavefronts per SIMD for grids that give a CU one workgroup; K must be a multiple of 2 * BKT.
+template <int WM, int WN, int TM, int TN, int BKT, bool FULL, bool BUF = false, int KS = 1>
+__global__ __launch_bounds__(WM * WN * 64 * KS) void gemm_f64_mfma(const GemmChain* __restrict__ chains,
+                                                                   int nchains,
+                                                                   const GemmSeg* __restrict__ segs,
+                                                                   int nblocks, GemmChain only_chain,
+                                                                   GemmSeg only_seg, int overwrite) {
+    constexpr int NT = WM * WN * 64;   // lanes of one set
     constexpr int BM = WM * TM * 16, BN = WN * TN * 16;
     constexpr int APT = BM * BKT / NT, BPT = BN * BKT / NT;   // doubles staged per lane
     static_assert(APT >= 2 && BPT >= 2 && APT % 2 == 0 && BPT % 2 == 0, "staging uses 128-bit loads");
@@ -65,8 +69,12 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_f64_mfma(const GemmChain* _
     // A stays row-major in LDS with rows of BKT + 1 doubles: the operand read of 16 consecutive
     // rows at one k then touches 16 different bank pairs. B is k-major with rows of BN + 16.
     constexpr int AP = BKT + 1;
-    __shared__ double As[2][BM][AP];
-    __shared__ __attribute__((aligned(16))) double Bs[2][BKT][BN + PAD];
+    __shared__ double As_all[KS][2][BM][AP];
+    __shared__ __attribute__((aligned(16))) double Bs_all[KS][2][BKT][BN + PAD];
+    __shared__ double Cs[KS > 1 ? TM * TN * 4 : 1][KS > 1 ? NT : 1];
+    const int set = KS > 1 ? __builtin_amdgcn_readfirstlane((int)threadIdx.x / NT) : 0;   // the same for a whole wavefront
+    double (*As)[BM][AP] = As_all[set];
+    double (*Bs)[BKT][BN + PAD] = Bs_all[set];
     const int logical = xcd_remap(blockIdx.x, nblocks);
     // a lone product travels in the kernel arguments (chains == nullptr), lists in a table
     int ci = 0;
@@ -78,7 +86,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_f64_mfma(const GemmChain* _
     const int local = logical - ch.blk0;
     const int bn = local / ch.nbm, bm = local - bn * ch.nbm;
     const int m0 = bm * BM, n0 = bn * BN;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = KS > 1 ? (int)threadIdx.x % NT : (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
 
     // staging assignment: A tile BM rows x BKT k (APT along k), B tile BKT k x BN (BPT along n)
@@ -192,11 +200,12 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_f64_mfma(const GemmChain* _
         // Step t multiplies LDS buffer t&1, which holds K slice t. Register set t&1 receives
         // slice t+2 while that runs; the other set (slice t+1, requested a step earlier) goes to
         // LDS after it.
-        const int nk = (K + BKT - 1) / BKT;
+        const int nk = (K + BKT - 1) / BKT / KS;          // K steps of this set
+        auto kof = [&](int step) { return (step * KS + set) * BKT; };
         double ra0[APT], rb0[BPT], ra1[APT], rb1[BPT];
-        fetch(0, ra0, rb0);
+        fetch(kof(0), ra0, rb0);
         if (nk > 1)
-            fetch(BKT, ra1, rb1);
+            fetch(kof(1), ra1, rb1);
         stage(0, ra0, rb0);
         __syncthreads();
         // At the top of every round LDS buffer 0 holds slice t and register set 1 slice t + 1.
@@ -204,17 +213,17 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_f64_mfma(const GemmChain* _
         // the younger pair of loads in flight while the older pair is stored.
         int t = 0;
         for (; t + 3 < nk; t += 2) {
-            fetch((t + 2) * BKT, ra0, rb0);
+            fetch(kof(t + 2), ra0, rb0);
             multiply(0);
             stage(1, ra1, rb1);
             __syncthreads();
-            fetch((t + 3) * BKT, ra1, rb1);
+            fetch(kof(t + 3), ra1, rb1);
             multiply(1);
             stage(0, ra0, rb0);
             __syncthreads();
         }
         if (t + 2 < nk)
-            fetch((t + 2) * BKT, ra0, rb0);
+            fetch(kof(t + 2), ra0, rb0);
         multiply(0);
         if (t + 1 < nk) {
             stage(1, ra1, rb1);
@@ -226,6 +235,28 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_f64_mfma(const GemmChain* _
                 multiply(0);
             }
         }
+    }
+    if (KS > 1) {
+        // the second set's sums go through LDS, lane to lane; the first set adds them to its own
+        if (set == 1) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        Cs[(i * TN + j) * 4 + r][tid] = acc[i][j][r];
+        }
+        __syncthreads();
+        if (set == 1)
+            return;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    acc[i][j][r] += Cs[(i * TN + j) * 4 + r][tid];
     }
     // D layout of the 16x16x4 f64 instruction (measured on gfx950): register r of a lane holds
     // row 4*r + lane/16, column lane % 16.
@@ -309,9 +340,24 @@ int check_job(const cnh_gemm_job& j) {
     return 0;
 }
 
-int g_gemm_buffer_loads = 1;   // option "gemm_buffer_loads"
+int compute_units() {
+    static int cus[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+        return 0;
+    if (cus[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+            return 0;
+        cus[dev] = n;
+    }
+    return cus[dev];
+}
 
-template <int WM, int WN, int TM, int TN, int BKT>
+int g_gemm_buffer_loads = 1;   // option "gemm_buffer_loads"
+int g_gemm_ksplit = 1;         // option "gemm_ksplit": two sets of wavefronts per workgroup on small grids
+
+template <int WM, int WN, int TM, int TN, int BKT, bool KSPLIT = false>
 int launch_chains(std::vector<GemmChain>& chains, const std::vector<GemmSeg>& segs, bool full,
                   int overwrite, hipStream_t st) {
     constexpr int BM = WM * TM * 16, BN = WN * TN * 16;
@@ -343,7 +389,16 @@ int launch_chains(std::vector<GemmChain>& chains, const std::vector<GemmSeg>& se
     bool buf = full && g_gemm_buffer_loads;
     for (const GemmSeg& sg : segs)
         buf = buf && (int64_t)BM * sg.lda * 8 < (1ll << 31) && (int64_t)BKT * sg.ldb * 8 < (1ll << 31);
-    if (buf)
+    // two sets of wavefronts per workgroup where no CU gets more than one workgroup and every K
+    // divides (256 x 2048 @ 2048 x 4096 under sustained load: 72.0 -> 66.2 us; with 384 or 512
+    // workgroups on 256 CUs the split costs 4 %: its 106 KB of LDS keep a second workgroup off the CU)
+    bool split = buf && KSPLIT && g_gemm_ksplit && blocks <= compute_units();
+    for (const GemmSeg& sg : segs)
+        split = split && sg.K % (2 * BKT) == 0;
+    if (split)
+        hipLaunchKernelGGL((gemm_f64_mfma<WM, WN, TM, TN, BKT, true, true, KSPLIT ? 2 : 1>), dim3((unsigned)blocks),
+                           dim3(WM * WN * 64 * 2), 0, st, dch, nch, dsg, nb, chains[0], segs[0], overwrite);
+    else if (buf)
         hipLaunchKernelGGL((gemm_f64_mfma<WM, WN, TM, TN, BKT, true, true>), dim3((unsigned)blocks),
                            dim3(WM * WN * 64), 0, st, dch, nch, dsg, nb, chains[0], segs[0], overwrite);
     else if (full)
@@ -393,7 +448,7 @@ int run_f64_batch(int njobs, const cnh_gemm_job* jobs, int overwrite, hipStream_
     // x 32 columns per wavefront (256x2048 @ 2048x4096: 86 us against 92 for 32 x 16).
     if (blocks64 >= 1024)
         return launch_chains<2, 2, 2, 2, 16>(chains, segs, full, overwrite, st);
-    return launch_chains<4, 2, 1, 2, 16>(chains, segs, full, overwrite, st);
+    return launch_chains<4, 2, 1, 2, 16, true>(chains, segs, full, overwrite, st);
 }
 
 } // namespace
@@ -422,6 +477,7 @@ __global__ __launch_bounds__(512) void mfma_f64_probe(double* out, int iters, do
 
 namespace cnh {
 void gemm_set_buffer_loads(int on) { g_gemm_buffer_loads = on; }
+void gemm_set_ksplit(int on) { g_gemm_ksplit = on; }
 } // namespace cnh
 
 extern "C" int cnh_probe_mfma_f64(int iters, double* tflops) {

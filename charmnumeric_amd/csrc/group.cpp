@@ -1391,6 +1391,11 @@ extern "C" int cnh_set_option(const char* name, int value) {
         gemm_set_buffer_loads(value);
         return 0;
     }
+    if (std::strcmp(name, "gemm_ksplit") == 0) {
+        CNH_CHECK(value == 0 || value == 1, -2, "gemm_ksplit: 0 or 1");
+        gemm_set_ksplit(value);
+        return 0;
+    }
     if (std::strcmp(name, "direct_lean") == 0) {
         g_direct_lean = value;
         return 0;

@@ -111,6 +111,10 @@ int cnh_version(void);
  *                    stage x in LDS, 32 or 64 rows per workgroup (default 1); 0: one wavefront per
  *                    row reading x through the caches. Same bits either way.
  *   "gemm_buffer_loads"  aligned fp64 products fetch A and B with buffer loads (default 1). Same bits.
+ *   "gemm_ksplit"        fp64 products on grids of at most one workgroup per CU, every K a multiple of
+ *                        32: two sets of wavefronts per workgroup, each taking every other K step,
+ *                        their sums added first + second (default 1). One fixed order, another than
+ *                        with 0.
  *   "slide_bx/ry/zc/pd", "slide2d_march"  geometry of the sliding-window kernel */
 int cnh_set_option(const char* name, int value);
 

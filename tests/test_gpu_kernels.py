@@ -449,6 +449,53 @@ def test_gemm_batch_overwrites_without_reading(dev, M, N, K):
     dev.free_all()
 
 
+@pytest.mark.parametrize("M,N,Ks,overwrite", [(256, 1024, (512,), 1), (128, 512, (64, 96, 32), 0),
+                                              (64, 64, (32,), 1), (256, 4096, (2048,), 1)])
+def test_gemm_with_the_k_steps_split_over_two_sets_of_wavefronts(dev, M, N, Ks, overwrite):
+    """Grids of at most one workgroup per CU whose K pieces are multiples of 32 run with two sets of
+    wavefronts per workgroup, each taking every other K step (option gemm_ksplit, on by default).
+    Small integer values make every sum exact, so both forms and NumPy must give the same bits; with
+    real values both stay within the bound and the split form gives the same bits on every run."""
+    rng = np.random.default_rng(M + N + sum(Ks))
+    K = sum(Ks)
+    for integers in (True, False):
+        if integers:
+            A = rng.integers(-4, 5, (M, K)).astype(np.float64)
+            B = rng.integers(-4, 5, (K, N)).astype(np.float64)
+            C0 = rng.integers(-9, 10, (M, N)).astype(np.float64)
+        else:
+            A, B, C0 = rng.standard_normal((M, K)), rng.standard_normal((K, N)), rng.standard_normal((M, N))
+        dA, dB, dC = dev.array(A), dev.array(B), dev.array(C0)
+        arr = (L.GemmJob * len(Ks))()
+        k0 = 0
+        for j, kk in zip(arr, Ks):
+            j.M, j.N, j.K, j.A, j.lda, j.B, j.ldb, j.C, j.ldc = M, N, kk, dA.ptr + 8 * k0, K, dB.ptr + 8 * k0 * N, N, dC.ptr, N
+            k0 += kk
+        results = {}
+        try:
+            for split in (1, 0, 1):
+                L.check(L.lib.cnh_set_option(b"gemm_ksplit", split))
+                dC.put(C0)
+                L.check(L.lib.cnh_gemm_batch(L.F64, len(Ks), arr, overwrite, None))
+                got = dC.get()
+                if split in results:
+                    assert got.tobytes() == results[split].tobytes()       # run to run
+                results[split] = got
+        finally:
+            L.check(L.lib.cnh_set_option(b"gemm_ksplit", 1))
+        if integers or M * N * K > 10 ** 8:      # exact in fp64 / the bound is 1e4 roundings wide
+            want = A @ B + (0 if overwrite else C0)
+        else:
+            want = (A.astype(np.longdouble) @ B.astype(np.longdouble)).astype(np.float64) + (0 if overwrite else C0)
+        if integers:
+            assert results[1].tobytes() == want.tobytes() and results[0].tobytes() == want.tobytes()
+        else:
+            bound = REL * (np.abs(A) @ np.abs(B) + np.abs(C0))
+            assert np.all(np.abs(results[1] - want) <= bound) and np.all(np.abs(results[0] - want) <= bound)
+            assert results[1].tobytes() != results[0].tobytes() or K <= 32     # the split form did run
+        dev.free_all()
+
+
 @pytest.mark.parametrize("dt,npdt", [(L.F64, np.float64), (L.I32, np.int32)])
 def test_gemv_over_a_window_of_tiles(dev, dt, npdt):
     """A 100 x 90 matrix in 32 x 32 tiles; the window rows 5..77, columns 9..70 against x."""
