@@ -2,8 +2,10 @@
 // Upstream: Eigen `C.noalias() += A*B` / KokkosBlas::gemm on strided sub-block views, one call per
 // arriving panel pair (src/backend_internal.hpp:113-133, src/executor_incremental.cpp:97-132).
 // fp64 is the one dense contraction of the path, so it runs on the matrix cores
-// (v_mfma_f64_16x16x4_f64): 64x64 workgroup tiles, four wavefronts of 32x32, K in steps of 16
-// staged through double-buffered LDS. Other element types use a plain LDS-tiled kernel.
+// (v_mfma_f64_16x16x4_f64): 64x64 workgroup tiles, K in steps of 16 staged through double-buffered
+// LDS; four wavefronts of 32x32 on big grids, eight of 16x32 on smaller ones, and two such sets of
+// eight sharing the K steps where a CU gets a single workgroup. Other element types use a plain
+// LDS-tiled kernel.
 #include "common.h"
 
 #include <cstring>
