@@ -783,12 +783,14 @@ def lstm_asts(L, d):
     return sigmoid(), tanh(), mul(), muladd()
 
 
-def lstm_fused_ast(L, first):
+def lstm_fused_ast(L, first, with_x=False):
     """All gate statements of one step (examples/lstm_forward.py:40-49 upstream) as one group with
     several output roots, each statement over its (batch x d) column window; later roots read
     earlier ones from registers. Leaves: 1..4 = the i, f, o, g windows of IFOG[t], 5 = C[t-1].
     Outputs: 11..14 = the windows of IFOGf[t], 15 = C[t], 16 = tanh(C[t]), 17 = Hout[t],
-    18 = the same values again, for the right half of Hin[t+1]."""
+    18 = the same values again, for the right half of Hin[t+1]. with_x: leaf 6 = X[t+1] and output 19 =
+    its copy for the left half of Hin[t+1] (`Hin[t+1, :, :word] = X[t+1]`, same extents when the input
+    is as wide as the state)."""
     from charmnumeric_amd.astbuild import AstBuilder
 
     b = AstBuilder(L.F64, 2)
@@ -816,11 +818,19 @@ def lstm_fused_ast(L, first):
     node.n_operands = 1
     b._attach(node, 0, h, None)
     b._roots.append(idx)
+    if with_x:
+        idx = b._new(19, L.OP_COPY, is_temp=False)
+        node = b._nodes[idx]
+        node.n_operands = 1
+        b._attach(node, 0, b.leaf(6), None)
+        b._roots.append(idx)
     return b.finish()
 
 
-def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=False, fused=True, warm_passes=5):
+def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=False, fused=True, warm_passes=5,
+             merge_x=True):
     k_in = nin + d
+    merge_x = merge_x and fused and nin == d     # the copy of x_{t+1} rides on step t's gate launch
     X = Buf(L, steps * batch * nin * 8)
     W = Buf(L, k_in * 4 * d * 8)
     L.check(L.lib.cnh_fill_uniform(X.ptr, steps * batch * nin, seed, 0, 0, -1.0, 1.0, None))
@@ -849,7 +859,8 @@ def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=
     Hout = Buf(L, steps * batch * d * 8, zero=True)
     a_sig, a_tanh, a_mul, a_muladd = lstm_asts(L, d)
     k_sig, k_tanh, k_mul, k_muladd = (_compile(L, a, L.F64, 2) for a in (a_sig, a_tanh, a_mul, a_muladd))
-    k_first, k_later = (_compile(L, lstm_fused_ast(L, f), L.F64, 2) for f in (True, False))
+    k_first, k_later = (_compile(L, lstm_fused_ast(L, f, merge_x), L.F64, 2) for f in (True, False))
+    k_last = _compile(L, lstm_fused_ast(L, steps == 1), L.F64, 2) if merge_x else k_later
     spare = Buf(L, batch * d * 8)      # where the last step's copy of h goes (no Hin[steps])
 
     def view(buf, t, row_len, c0, ncols):
@@ -898,8 +909,10 @@ def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=
     def prepare(t):
         """(what runs before the product, the product, what runs after it) of step t."""
         # Hin[t, :, :nin] = X[t]; Hin[t, :, nin:] = Hout[t-1] (h0 = 0 at t = 0)
-        before = [prepared_copy(Hin.ptr + t * batch * k_in * 8, [k_in, 1], X.ptr + t * batch * nin * 8,
-                                [nin, 1], [batch, nin])]
+        before = []
+        if t == 0 or not merge_x:
+            before.append(prepared_copy(Hin.ptr + t * batch * k_in * 8, [k_in, 1], X.ptr + t * batch * nin * 8,
+                                        [nin, 1], [batch, nin]))
         if t > 0 and not fused:
             before.append(prepared_copy(Hin.ptr + (t * batch * k_in + nin) * 8, [k_in, 1],
                                         Hout.ptr + (t - 1) * batch * d * 8, [d, 1], [batch, d]))
@@ -916,7 +929,13 @@ def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=
             outs = {11: view(IFOGf, t, 4 * d, 0, d), 12: view(IFOGf, t, 4 * d, d, d),
                     13: view(IFOGf, t, 4 * d, 2 * d, d), 14: view(IFOGf, t, 4 * d, 3 * d, d),
                     15: view(Cc, t, d, 0, d), 16: view(Ct, t, d, 0, d), 17: view(Hout, t, d, 0, d), 18: nxt}
-            after.append(prepared_group(k_first if t == 0 else k_later, 2, ins, outs))
+            kern = k_first if t == 0 else k_later
+            if merge_x and t + 1 < steps:
+                ins[6] = view(X, t + 1, nin, 0, nin)
+                outs[19] = view(Hin, t + 1, k_in, 0, nin)
+            elif merge_x:
+                kern = k_last
+            after.append(prepared_group(kern, 2, ins, outs))
         else:
             after.append(prepared1(k_sig, 2, [view(IFOG, t, 4 * d, 0, 3 * d)], [view(IFOGf, t, 4 * d, 0, 3 * d)]))
             after.append(prepared1(k_tanh, 2, [view(IFOG, t, 4 * d, 3 * d, d)], [view(IFOGf, t, 4 * d, 3 * d, d)]))
@@ -1002,6 +1021,9 @@ def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=
         L.lib.cnh_event_destroy(e)
     L.check(L.lib.cnh_stream_destroy(stream))
     out["gate_launches_per_step"] = 1 if fused else 6
+    # the product, the gate launch (which also lays x_{t+1} into the next step's operand when the
+    # input is as wide as the state) and otherwise the copy of x_t
+    out["launches_per_step"] = (2 if merge_x else 3) if fused else 9
     for b_ in (X, W, Hin, IFOG, IFOGf, Cc, Ct, Hout, spare):
         b_.free()
     return out

@@ -1148,7 +1148,7 @@ struct Stmt {
 };
 
 constexpr int64_t kFuseMaxElems = 1ll << 22;   // larger statements are bandwidth bound anyway
-constexpr size_t kFuseMaxStmts = 8, kFuseMaxReads = 16;
+constexpr size_t kFuseMaxStmts = 12, kFuseMaxReads = 16;
 
 bool boxes_identical(const BoxUse& a, const BoxUse& b) {
     return a.arr == b.arr && same_region(a.reg, b.reg);
@@ -1807,6 +1807,47 @@ bool can_join(const std::vector<Stmt>& run, const Stmt& b) {
     return run.size() < kFuseMaxStmts && reads <= kFuseMaxReads;
 }
 
+// An assignment whose extent along one dimension is 2 to 4 times `want`'s there (the others equal)
+// as that many assignments side by side, each with `want`'s extents: elementwise work may be cut
+// anywhere, and the pieces can then join a run of statements of the smaller extent (an LSTM step's
+// sigmoid over three gates' columns next to the statements on one gate's columns).
+bool cut_statement(const Stmt& a, const int32_t* want, std::vector<Stmt>& pieces) {
+    int along = -1;
+    for (int d = 0; d < a.nd; ++d) {
+        if (a.cnt[d] == want[d])
+            continue;
+        if (along >= 0 || want[d] <= 0 || a.cnt[d] % want[d] != 0)
+            return false;
+        along = d;
+    }
+    if (along < 0)
+        return false;
+    const int m = a.cnt[along] / want[along];
+    if (m < 2 || m > 4)
+        return false;
+    auto narrowed = [&](const BoxUse& u, int k, BoxUse& out) {
+        out = u;
+        const int ad = u.map[along];
+        if (ad < 0)
+            return false;
+        out.reg.start[ad] = u.reg.start[ad] + k * want[along];
+        out.reg.stop[ad] = out.reg.start[ad] + want[along];
+        return true;
+    };
+    pieces.clear();
+    for (int k = 0; k < m; ++k) {
+        Stmt p = a;
+        p.cnt[along] = want[along];
+        if (!narrowed(a.out, k, p.out))
+            return false;
+        for (size_t r = 0; r < a.reads.size(); ++r)
+            if (!narrowed(a.reads[r].use, k, p.reads[r].use))
+                return false;
+        pieces.push_back(p);
+    }
+    return true;
+}
+
 // The run as one multi-root group. Boxes are numbered; the group's regions carry the numbers, not
 // the coordinates (the launch hands over memrefs), so every step of a time loop finds the kernel
 // of the first one in the cache.
@@ -1833,7 +1874,7 @@ int exec_statement_run(Ex* ex, const std::vector<Stmt>& run) {
     };
     struct Done { int value_node; int set_root; const Stmt* st; };
     std::vector<Done> done;
-    int next_literal = -1;
+    int next_literal = -1, next_temporary = 0x7e000000;
     for (const Stmt& st : run) {
         const DagNode& n = *st.n;
         const int base = (int)merged.nodes.size();
@@ -1847,6 +1888,18 @@ int exec_statement_run(Ex* ex, const std::vector<Stmt>& run) {
             if (c.is_scalar)
                 c.result_name = next_literal--;
         }
+        // the pieces of a cut statement are copies of one node: their temporaries and the
+        // assignment itself (a name nothing else refers to) need names of their own
+        std::map<int, int> renamed;
+        for (size_t ri = 0; ri + 1 < n.roots.size(); ++ri)
+            renamed[n.nodes[(size_t)n.roots[ri]].result_name] = next_temporary++;
+        for (size_t q = (size_t)base; q < merged.nodes.size(); ++q) {
+            cnh_ast_node& c = merged.nodes[q];
+            auto it = c.is_scalar ? renamed.end() : renamed.find(c.result_name);
+            if (it != renamed.end())
+                c.result_name = it->second;
+        }
+        merged.nodes[(size_t)base + n.roots.back()].result_name = next_temporary++;
         for (const auto& rd : st.reads) {
             cnh_ast_node& r = merged.nodes[(size_t)base + n.roots[(size_t)rd.root]];
             // the newest earlier statement that assigned exactly this box supplies the value
@@ -1957,9 +2010,39 @@ int try_statement_run(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t*
             for (const auto& rd : st.reads)
                 touches_deleted = touches_deleted || rd.use.arr->name == name;
         }
-        if (touches_deleted || (!run.empty() && !can_join(run, st)))
+        if (touches_deleted)
             break;
-        run.push_back(st);
+        if (!run.empty() && !can_join(run, st)) {
+            // extents that differ by a small factor along one dimension: the wider side in pieces
+            std::vector<Stmt> pieces, tried;
+            bool joined = false;
+            if (run.size() == 1 && cut_statement(run[0], st.cnt, pieces)) {
+                tried.assign(1, pieces[0]);
+                joined = true;
+                for (size_t q = 1; q < pieces.size() && joined; ++q) {
+                    joined = can_join(tried, pieces[q]);
+                    tried.push_back(pieces[q]);
+                }
+                joined = joined && can_join(tried, st);
+                if (joined) {
+                    tried.push_back(st);
+                    run.swap(tried);
+                }
+            } else if (cut_statement(st, run.front().cnt, pieces)) {
+                tried = run;
+                joined = true;
+                for (size_t q = 0; q < pieces.size() && joined; ++q) {
+                    joined = can_join(tried, pieces[q]);
+                    tried.push_back(pieces[q]);
+                }
+                if (joined)
+                    run.swap(tried);
+            }
+            if (!joined)
+                break;
+        } else {
+            run.push_back(st);
+        }
         last_stmt_end = j + 1;
         deletions_kept = deletions;
     }

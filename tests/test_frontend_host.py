@@ -657,3 +657,37 @@ def test_get_region_is_the_slice_of_the_same_bounds(itf):
 def test_randn_is_upstreams_placeholder(itf):
     r = cnp.random.randn(3, 5)
     assert r.shape == (3, 5) and r.dtype == np.float32
+
+
+def test_an_lstm_step_is_a_product_and_one_merged_launch(itf):
+    """examples/lstm_forward.py upstream, steps after the first two: the sigmoid over three gates'
+    columns is cut into three pieces that join the run of the statements on one gate's columns (and
+    the copies that prepare the next step's operand), so a step is the product plus one launch."""
+    n, b, word, d = 6, 32, 16, 16
+    X = cnp.zeros((n, b, word))
+    W = cnp.zeros((word + d, 4 * d))
+    h0 = cnp.zeros((1, d))
+    Hin, Hout = cnp.zeros((n, b, word + d)), cnp.zeros((n, b, d))
+    IFOG, IFOGf = cnp.zeros((n, b, 4 * d)), cnp.zeros((n, b, 4 * d))
+    Cs, Ct = cnp.zeros((n, b, d)), cnp.zeros((n, b, d))
+    for t in range(n):
+        prev = cnp.tile(h0, (b, 1)) if t == 0 else Hout[t - 1]
+        Hin[t, :, :word] = X[t]
+        Hin[t, :, word:] = prev
+        IFOG[t] = Hin[t].dot(W)
+        IFOGf[t, :, : 3 * d] = 1.0 / (1.0 + cnp.exp(-IFOG[t, :, : 3 * d]))
+        IFOGf[t, :, 3 * d:] = cnp.tanh(IFOG[t, :, 3 * d:])
+        Cs[t] = IFOGf[t, :, :d] * IFOGf[t, :, 3 * d:]
+        if t > 0:
+            Cs[t] += IFOGf[t, :, d: 2 * d] * Cs[t - 1]
+        Ct[t] = cnp.tanh(Cs[t])
+        Hout[t] = IFOGf[t, :, 2 * d: 3 * d] * Ct[t]
+    cnp.execute(itf)
+    work = [ln for ln in itf.trace() if ln.startswith("group") or ln.startswith("matmatmul")]
+    # from the second product on: product, merged launch, product, merged launch, ...
+    at = [i for i, ln in enumerate(work) if ln.startswith("matmatmul")]
+    assert len(at) == n
+    for a, b_ in zip(at[1:], at[2:] + [len(work)]):
+        assert b_ - a == 2 and "path=statements" in work[a + 1]
+    # three pieces + tanh + C + C += + Ct + Hout + the two copies for the next step
+    assert sum("count=10" in ln for ln in work) == n - 2

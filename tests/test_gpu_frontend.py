@@ -581,6 +581,39 @@ def test_statement_runs_give_what_the_statements_give_one_by_one(itf, fusion, ra
     assert np.array_equal(u.get(itf), hu) and np.array_equal(v.get(itf), hv)
 
 
+@pytest.mark.parametrize("fusion", [True, False], ids=["merged", "one-by-one"])
+def test_wider_assignments_are_cut_to_join_their_run(itf, fusion, rank3_layout):
+    """An assignment two to four times as wide as the statements next to it is cut into pieces that
+    join their run: the wide one first (an LSTM step's sigmoid over three gates' columns), the wide
+    one last, its pieces read from registers by later statements, and one that updates its own
+    box. Only + - * here, so NumPy running the statements in order gives the same bits."""
+    itf.set_fusion(fusion)
+    rng = np.random.default_rng(21)
+    n, b, d = 4, 12, 10
+    hI, hF = rng.standard_normal((n, b, 4 * d)), np.zeros((n, b, 4 * d))
+    hC, hH = rng.standard_normal((n, b, d)), np.zeros((n, b, d))
+    hP = rng.standard_normal((n, b, 2 * d))
+    I, F, C, H, P = (cnp.array(x) for x in (hI, hF, hC, hH, hP))
+    itf.set_trace()
+    for t in range(n):
+        F[t, :, : 3 * d] = I[t, :, : 3 * d] * 0.5 - 1.0             # three times as wide, first
+        hF[t, :, : 3 * d] = hI[t, :, : 3 * d] * 0.5 - 1.0
+        F[t, :, 3 * d:] = I[t, :, 3 * d:] * I[t, :, 3 * d:]
+        hF[t, :, 3 * d:] = hI[t, :, 3 * d:] * hI[t, :, 3 * d:]
+        C[t] = F[t, :, :d] * F[t, :, 3 * d:] + F[t, :, d: 2 * d] * C[t]
+        hC[t] = hF[t, :, :d] * hF[t, :, 3 * d:] + hF[t, :, d: 2 * d] * hC[t]
+        H[t] = F[t, :, 2 * d: 3 * d] * C[t]
+        hH[t] = hF[t, :, 2 * d: 3 * d] * hC[t]
+        P[t] = P[t] * 0.25 + F[t, :, d: 3 * d]                       # twice as wide, last, in place
+        hP[t] = hP[t] * 0.25 + hF[t, :, d: 3 * d]
+    for dev, host in ((F, hF), (C, hC), (H, hH), (P, hP)):
+        assert np.array_equal(dev.get(itf), host)
+    runs = [ln for ln in itf.trace() if ln.startswith("group") and "path=statements" in ln]
+    if fusion and runs:      # (layouts chosen by the decomposition solver may leave nothing to merge)
+        # per step one launch: 3 pieces + 3 statements + 2 pieces
+        assert any("count=8" in ln for ln in runs), runs
+
+
 @pytest.mark.parametrize("fusion", [True, False], ids=["fused", "node-by-node"])
 @pytest.mark.parametrize("shape", [(100000,), (300, 70), (20, 30, 40)])
 def test_reductions_fused_into_their_producer(itf, small_tiles, fusion, shape):
