@@ -452,10 +452,18 @@ struct Seg { i64 n; i64 blk0; const T* in[NLA]; T* out[NOA]; };
 typedef T TV __attribute__((ext_vector_type(VECW)));
 #define OUT_STORED(j) (((RED_MASK >> (j)) & 1u) == 0u)
 
-template <bool NT>
+// Workgroups of one wavefront where nothing is reduced (a plain triad over 2^24 doubles streams at
+// 0.86 of the HBM peak with 64 lanes a workgroup, 0.84 with 128, 0.82 with 256 to 1024); reducing
+// launches keep 256 lanes, whose four wavefronts share one partial.
+#if NR > 0
+#define FLAT_WG 256
+#else
+#define FLAT_WG 64
+#endif
+template <bool NT, int WG>
 __device__ __forceinline__ void flat_vec(const Seg& sg, i64 blk, const T* s, T* racc) {
     (void)racc;
-    const i64 i = (blk * 256 + threadIdx.x) * VECW;
+    const i64 i = (blk * WG + threadIdx.x) * VECW;
     const i64 n = sg.n;
     if (i + VECW <= n) {
         TV lv[NLA];
@@ -497,11 +505,12 @@ __device__ __forceinline__ void flat_vec(const Seg& sg, i64 blk, const T* s, T* 
 }
 
 // Pointers that are not 16-byte aligned: one element per lane.
+template <int WG>
 __device__ __forceinline__ void flat_scalar(const Seg& sg, i64 blk, const T* s, T* racc) {
     (void)racc;
 #pragma unroll
     for (int u = 0; u < VECW; ++u) {
-        const i64 i = (blk * VECW + u) * 256 + threadIdx.x;
+        const i64 i = (blk * VECW + u) * WG + threadIdx.x;
         if (i < sg.n) {
             T l[NLA], o[NOA];
 #pragma unroll
@@ -584,8 +593,8 @@ __device__ __forceinline__ void load_scalars_folding(const Scal& sc, const Fold&
     }
 }
 
-#define FLAT_ENTRY(NAME, CALL)                                                                   \
-extern "C" __global__ __launch_bounds__(256) void grp_flat_##NAME(const Seg* segs, int nseg,    \
+#define FLAT_ENTRY(NAME, CALL, CALL256)                                                          \
+extern "C" __global__ __launch_bounds__(FLAT_WG) void grp_flat_##NAME(const Seg* segs, int nseg, \
                                                                   Scal sc RED_PARAM) {           \
     CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);                                                               \
     RED_BEGIN                                                                                    \
@@ -595,7 +604,7 @@ extern "C" __global__ __launch_bounds__(256) void grp_flat_##NAME(const Seg* seg
     CALL;                                                                                        \
     RED_END                                                                                      \
 }                                                                                                \
-extern "C" __global__ __launch_bounds__(256) void grp_flat1_##NAME(Seg sg, Scal sc RED_PARAM) { \
+extern "C" __global__ __launch_bounds__(FLAT_WG) void grp_flat1_##NAME(Seg sg, Scal sc RED_PARAM) { \
     CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);                                                               \
     RED_BEGIN                                                                                    \
     const i64 blk = (i64)blockIdx.x;                                                             \
@@ -607,12 +616,12 @@ extern "C" __global__ __launch_bounds__(256) void grp_flat1f_##NAME(Seg sg, Scal
     CNH_ENTRY_GUARD T s[NSV]; load_scalars_folding(sc, fd, s);                                                   \
     RED_BEGIN                                                                                    \
     const i64 blk = (i64)blockIdx.x;                                                             \
-    CALL;                                                                                        \
+    CALL256;                                                                                     \
     RED_END                                                                                      \
 }
-FLAT_ENTRY(v, flat_vec<false>(sg, blk, s, racc))
-FLAT_ENTRY(vn, flat_vec<true>(sg, blk, s, racc))
-FLAT_ENTRY(s, flat_scalar(sg, blk, s, racc))
+FLAT_ENTRY(v, (flat_vec<false, FLAT_WG>(sg, blk, s, racc)), (flat_vec<false, 256>(sg, blk, s, racc)))
+FLAT_ENTRY(vn, (flat_vec<true, FLAT_WG>(sg, blk, s, racc)), (flat_vec<true, 256>(sg, blk, s, racc)))
+FLAT_ENTRY(s, (flat_scalar<FLAT_WG>(sg, blk, s, racc)), (flat_scalar<256>(sg, blk, s, racc)))
 )";
     return s.str();
 }
@@ -627,20 +636,20 @@ struct Cell {
     const T* in[NLA]; i64 istr[NLA][3];
     T* out[NOA]; i64 ostr[NOA][3];
 };
-// PER elements per lane, 256 apart: 4 for large launches; 1 for small ones, which then spread over
-// four times as many wavefronts (a 256 x 1024 gate statement with exp and tanh in fp64: 19.6 us
+// PER elements per lane, a workgroup's width apart: 4 for large launches (256 lanes a workgroup); 1
+// for small ones (one wavefront a workgroup), which then spread over four times as many wavefronts (a 256 x 1024 gate statement with exp and tanh in fp64: 19.6 us
 // with one wavefront per SIMD busy, latency-bound).
-template <int ND_PER_THREAD>
+template <int ND_PER_THREAD, int WG>
 __device__ __forceinline__ void nd_run(const Cell& c, i64 blk, const T* s) {
     const i64 outer = blk / c.nchunks;
     const i64 chunk = blk - outer * c.nchunks;
     const i64 i1 = outer % c.sizes[1];
     const i64 i0 = outer / c.sizes[1];
-    const i64 x0 = chunk * (256 * ND_PER_THREAD) + threadIdx.x;
+    const i64 x0 = chunk * (WG * ND_PER_THREAD) + threadIdx.x;
     T lv[NLA][ND_PER_THREAD];
 #pragma unroll
     for (int u = 0; u < ND_PER_THREAD; ++u) {
-        const i64 x = x0 + (i64)u * 256;
+        const i64 x = x0 + (i64)u * WG;
         if (x < c.sizes[2]) {
 #pragma unroll
             for (int k = 0; k < NL; ++k)
@@ -649,7 +658,7 @@ __device__ __forceinline__ void nd_run(const Cell& c, i64 blk, const T* s) {
     }
 #pragma unroll
     for (int u = 0; u < ND_PER_THREAD; ++u) {
-        const i64 x = x0 + (i64)u * 256;
+        const i64 x = x0 + (i64)u * WG;
         if (x < c.sizes[2]) {
             T l[NLA], o[NOA];
 #pragma unroll
@@ -665,20 +674,20 @@ __device__ __forceinline__ void nd_run(const Cell& c, i64 blk, const T* s) {
 extern "C" __global__ __launch_bounds__(256) void grp_nd(const Cell* cells, int ncell, Scal sc) {
     CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
     const int k = find_seg(cells, ncell, (i64)blockIdx.x);
-    nd_run<4>(cells[k], (i64)blockIdx.x - cells[k].blk0, s);
+    nd_run<4, 256>(cells[k], (i64)blockIdx.x - cells[k].blk0, s);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_nd1(Cell cell, Scal sc) {
     CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
-    nd_run<4>(cell, (i64)blockIdx.x, s);
+    nd_run<4, 256>(cell, (i64)blockIdx.x, s);
 }
-extern "C" __global__ __launch_bounds__(256) void grp_nd_p1(const Cell* cells, int ncell, Scal sc) {
+extern "C" __global__ __launch_bounds__(64) void grp_nd_p1(const Cell* cells, int ncell, Scal sc) {
     CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
     const int k = find_seg(cells, ncell, (i64)blockIdx.x);
-    nd_run<1>(cells[k], (i64)blockIdx.x - cells[k].blk0, s);
+    nd_run<1, 64>(cells[k], (i64)blockIdx.x - cells[k].blk0, s);
 }
-extern "C" __global__ __launch_bounds__(256) void grp_nd1_p1(Cell cell, Scal sc) {
+extern "C" __global__ __launch_bounds__(64) void grp_nd1_p1(Cell cell, Scal sc) {
     CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
-    nd_run<1>(cell, (i64)blockIdx.x, s);
+    nd_run<1, 64>(cell, (i64)blockIdx.x, s);
 }
 )";
     return s.str();

@@ -274,10 +274,10 @@ bool dense_memref(int nd, const cnh_memref& m) {
     return true;
 }
 
-int launch(hipFunction_t fn, int64_t blocks, void** params, hipStream_t st) {
+int launch(hipFunction_t fn, int64_t blocks, void** params, hipStream_t st, unsigned lanes = 256) {
     CNH_CHECK(blocks > 0 && blocks < (1ll << 31), -3, "launch of %lld workgroups is out of range",
               (long long)blocks);
-    CNH_HIP(hipModuleLaunchKernel(fn, (unsigned)blocks, 1, 1, 256, 1, 1, 0, st, params, nullptr));
+    CNH_HIP(hipModuleLaunchKernel(fn, (unsigned)blocks, 1, 1, lanes, 1, 1, 0, st, params, nullptr));
     return 0;
 }
 
@@ -500,7 +500,10 @@ int launch_group_impl(cnh_kernel* k, int ndims, int n_parts, int n_in, const cnh
     };
 
     if (all_dense) {
-        const int per_block = 256 * vec;
+        // the generated code's FLAT_WG: one wavefront per workgroup unless the launch reduces or
+        // sums partials on the way in (those kernels share values between four wavefronts)
+        const unsigned lanes = (n_red > 0 || sums != nullptr) ? 256 : 64;
+        const int per_block = (int)lanes * vec;
         const size_t seg_words = 2 + NLA + NOA;
         std::vector<uint64_t> segs(seg_words * live.size(), 0);
         int64_t blocks = 0, total = 0;
@@ -590,11 +593,11 @@ int launch_group_impl(cnh_kernel* k, int ndims, int n_parts, int n_in, const cnh
             if (int rc = get_function(k, "flat", (std::string("grp_flat1f_") + suffix).c_str(), &ffn))
                 return rc;
             void* params[] = {segs.data(), scal.data(), fold.data(), red_slots};
-            if (int rc = launch(ffn, blocks, params, st))
+            if (int rc = launch(ffn, blocks, params, st, 256))
                 return rc;
         } else if (live.size() == 1) {
             void* params[] = {segs.data(), scal.data(), red_slots};
-            if (int rc = launch(fn, blocks, params, st))
+            if (int rc = launch(fn, blocks, params, st, lanes))
                 return rc;
         } else {
             const void* dsegs = nullptr;
@@ -602,7 +605,7 @@ int launch_group_impl(cnh_kernel* k, int ndims, int n_parts, int n_in, const cnh
                 return rc;
             int nseg = (int)live.size();
             void* params[] = {&dsegs, &nseg, scal.data(), red_slots};
-            if (int rc = launch(fn, blocks, params, st))
+            if (int rc = launch(fn, blocks, params, st, lanes))
                 return rc;
         }
         if (n_fold == 0)
@@ -626,6 +629,7 @@ int launch_group_impl(cnh_kernel* k, int ndims, int n_parts, int n_in, const cnh
         all_elems += n;
     }
     const int per_lane = all_elems <= (1ll << 21) ? 1 : 4;
+    const unsigned nd_lanes = per_lane == 1 ? 64 : 256;      // as the generated entry points are built
     for (size_t j = 0; j < live.size(); ++j) {
         int q = live[j];
         const cnh_memref* pi = in + (size_t)q * n_in;
@@ -634,7 +638,7 @@ int launch_group_impl(cnh_kernel* k, int ndims, int n_parts, int n_in, const cnh
         int64_t sz[3] = {1, 1, 1};
         for (int d = 0; d < ndims; ++d)
             sz[pad + d] = po[0].sizes[d];
-        int64_t nchunks = (sz[2] + 256 * per_lane - 1) / (256 * per_lane);
+        int64_t nchunks = (sz[2] + nd_lanes * per_lane - 1) / (nd_lanes * per_lane);
         c[0] = sz[0];
         c[1] = sz[1];
         c[2] = sz[2];
@@ -662,7 +666,7 @@ int launch_group_impl(cnh_kernel* k, int ndims, int n_parts, int n_in, const cnh
         if (int rc = get_function(k, "nd", per_lane == 1 ? "grp_nd1_p1" : "grp_nd1", &fn))
             return rc;
         void* params[] = {cells.data(), scal.data()};
-        return launch(fn, blocks, params, st);
+        return launch(fn, blocks, params, st, nd_lanes);
     }
     if (int rc = get_function(k, "nd", per_lane == 1 ? "grp_nd_p1" : "grp_nd", &fn))
         return rc;
@@ -671,7 +675,7 @@ int launch_group_impl(cnh_kernel* k, int ndims, int n_parts, int n_in, const cnh
         return rc;
     int ncell = (int)live.size();
     void* params[] = {&dcells, &ncell, scal.data()};
-    return launch(fn, blocks, params, st);
+    return launch(fn, blocks, params, st, nd_lanes);
 }
 
 } // namespace
