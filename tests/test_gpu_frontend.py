@@ -614,6 +614,34 @@ def test_wider_assignments_are_cut_to_join_their_run(itf, fusion, rank3_layout):
         assert any("count=8" in ln for ln in runs), runs
 
 
+@pytest.mark.parametrize("m", [2, 3, 4, 5])
+@pytest.mark.parametrize("along", [0, 1])
+def test_cut_assignments_along_either_dimension(itf, m, along):
+    """A whole-window assignment m times as long as the statements that follow along rows or along
+    columns (m = 5 is beyond what is cut and runs on its own); the pieces are read back from
+    registers by the statements on the m blocks, one of which updates its block in place."""
+    rng = np.random.default_rng(10 * m + along)
+    b, d = 6, 8
+    shape = (m * b, d) if along == 0 else (b, m * d)
+    hS, hA = rng.standard_normal(shape), np.zeros(shape)
+    hR = [rng.standard_normal((b, d)) for _ in range(m)]
+    S, A = cnp.array(hS), cnp.array(hA)
+    R = [cnp.array(x) for x in hR]
+    block = (lambda k: (slice(k * b, (k + 1) * b), slice(None))) if along == 0 else \
+            (lambda k: (slice(None), slice(k * d, (k + 1) * d)))
+    for rounds in range(3):
+        A[:, :] = S * 0.5 - A                      # m blocks wide
+        hA[:, :] = hS * 0.5 - hA
+        for k in range(m):
+            R[k][:, :] = R[k] * 0.25 + A[block(k)]
+            hR[k][:, :] = hR[k] * 0.25 + hA[block(k)]
+        A[block(m - 1)] = A[block(m - 1)] * R[0]   # a block of the wide target, in place
+        hA[block(m - 1)] = hA[block(m - 1)] * hR[0]
+    assert np.array_equal(A.get(itf), hA)
+    for k in range(m):
+        assert np.array_equal(R[k].get(itf), hR[k])
+
+
 @pytest.mark.parametrize("fusion", [True, False], ids=["fused", "node-by-node"])
 @pytest.mark.parametrize("shape", [(100000,), (300, 70), (20, 30, 40)])
 def test_reductions_fused_into_their_producer(itf, small_tiles, fusion, shape):
