@@ -1145,6 +1145,9 @@ struct Stmt {
     BoxUse out;
     struct Read { int root, slot; BoxUse use; };
     std::vector<Read> reads;
+    // one-element arrays read as kernel scalars: the launch fetches them through a device pointer
+    // before any lane has stored, so no statement of the same launch may assign them
+    std::vector<const XArray*> scalars_read;
 };
 
 constexpr int64_t kFuseMaxElems = 1ll << 22;   // larger statements are bandwidth bound anyway
@@ -1742,6 +1745,7 @@ bool analyse_statement(Ex* ex, const DagNode& n, Stmt& st) {
     for (int32_t r : n.roots)
         internal.insert(n.nodes[r].result_name);
     st.reads.clear();
+    st.scalars_read.clear();
     for (size_t ri = 0; ri < n.roots.size(); ++ri) {
         const cnh_ast_node& r = n.nodes[n.roots[ri]];
         if (r.dtype != st.dtype)
@@ -1758,8 +1762,9 @@ bool analyse_statement(Ex* ex, const DagNode& n, Stmt& st) {
             if (it == ex->arrays.end() || it->second.dtype != st.dtype)
                 return false;
             if (op.is_broadcast) {
-                if (it->second.elems != 1)
+                if (it->second.elems != 1 || &it->second == st.out.arr)
                     return false;
+                st.scalars_read.push_back(&it->second);
                 continue;
             }
             Stmt::Read rd;
@@ -1802,6 +1807,14 @@ bool can_join(const std::vector<Stmt>& run, const Stmt& b) {
             return false;
         for (const auto& rd : s.reads)
             if (!boxes_identical(b.out, rd.use) && !boxes_disjoint(b.out, rd.use))
+                return false;
+        // a kernel scalar is read once, at the start of the launch, by every lane: a statement
+        // that assigns that array cannot share a launch with one that reads it as a scalar
+        for (const XArray* a : b.scalars_read)
+            if (a == s.out.arr)
+                return false;
+        for (const XArray* a : s.scalars_read)
+            if (a == b.out.arr)
                 return false;
     }
     return run.size() < kFuseMaxStmts && reads <= kFuseMaxReads;
@@ -2658,9 +2671,19 @@ int run_fresh(Ex* ex, std::vector<DagNode>& fresh) {
     return run_nodes(ex, dag);
 }
 
+int run_log(Ex* ex, const char* log, int64_t size, int window);
+
+// Statements an automatic flush held back are older than anything that arrives now: plan them to
+// the end and run them.
+int finish_log(Ex* ex) {
+    return ex->plog.empty() ? 0 : run_log(ex, nullptr, 0, -1);
+}
+
 int run_message(Ex* ex, const char* msg, int64_t size) {
     std::vector<DagNode> fresh;
     if (int rc = parse_dag(msg, size, fresh))
+        return rc;
+    if (int rc = finish_log(ex))
         return rc;
     return run_fresh(ex, fresh);
 }
@@ -2758,6 +2781,17 @@ int drain(Ex* ex) {
         }
     }
     // the worker is idle now (or there is none): the statements it left open run on this thread
+    return flush_held(ex);
+}
+
+// For calls that read or write array state (get, put, fills, sync, array_info): everything
+// received so far has run when this returns, the statements a hold-back flush left unplanned
+// included.
+int settle(Ex* ex) {
+    if (int rc = drain(ex))
+        return rc;
+    if (int rc = finish_log(ex))
+        return rc;
     return flush_held(ex);
 }
 
@@ -2953,7 +2987,7 @@ int cnx_set_async(cnx_executor* ex, int on) {
 int cnx_get(cnx_executor* ex, int ndims, int epoch, int name, int64_t size, int dtype, void* host_out) {
     (void)epoch;
     CNH_CHECK(ex != nullptr && host_out != nullptr, -2, "null argument");
-    if (int rc = drain(ex))
+    if (int rc = settle(ex))
         return rc;
     XArray* a;
     if (int rc = find_array(ex, name, &a, "get"))
@@ -2999,7 +3033,7 @@ int cnx_get(cnx_executor* ex, int ndims, int epoch, int name, int64_t size, int 
 
 int cnx_put(cnx_executor* ex, int name, int64_t size, int dtype, const void* host_in) {
     CNH_CHECK(ex != nullptr && host_in != nullptr, -2, "null argument");
-    if (int rc = drain(ex))
+    if (int rc = settle(ex))
         return rc;
     XArray* a;
     if (int rc = find_array(ex, name, &a, "put"))
@@ -3043,7 +3077,7 @@ int cnx_put(cnx_executor* ex, int name, int64_t size, int dtype, const void* hos
 
 int cnx_fill_uniform(cnx_executor* ex, int name, uint64_t seed, uint64_t stream_id, double lo, double hi) {
     CNH_CHECK(ex != nullptr, -2, "null executor");
-    if (int rc = drain(ex))
+    if (int rc = settle(ex))
         return rc;
     XArray* a;
     if (int rc = find_array(ex, name, &a, "fill_uniform"))
@@ -3075,7 +3109,7 @@ int cnx_fill_uniform(cnx_executor* ex, int name, uint64_t seed, uint64_t stream_
 
 int cnx_fill_cg_matrix(cnx_executor* ex, int name, uint64_t seed) {
     CNH_CHECK(ex != nullptr, -2, "null executor");
-    if (int rc = drain(ex))
+    if (int rc = settle(ex))
         return rc;
     XArray* a;
     if (int rc = find_array(ex, name, &a, "fill_cg_matrix"))
@@ -3097,7 +3131,7 @@ int cnx_fill_cg_matrix(cnx_executor* ex, int name, uint64_t seed) {
 
 int cnx_sync(cnx_executor* ex) {
     CNH_CHECK(ex != nullptr, -2, "null executor");
-    if (int rc = drain(ex))
+    if (int rc = settle(ex))
         return rc;
     if (ex->dry)
         return 0;
@@ -3107,7 +3141,7 @@ int cnx_sync(cnx_executor* ex) {
 int cnx_array_info(cnx_executor* ex, int name, int* ndims, int* dtype, int* tile, int32_t* shape3,
                    int32_t* offset3) {
     CNH_CHECK(ex != nullptr, -2, "null executor");
-    if (int rc = drain(ex))
+    if (int rc = settle(ex))
         return rc;
     XArray* a;
     if (int rc = find_array(ex, name, &a, "array_info"))

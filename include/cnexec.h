@@ -132,8 +132,11 @@ int cnx_set_async(cnx_executor* ex, int on);
  *                | 1, name, base_ndims, dtype, broadcast, has_region, start[3], stop[3], step[3]
  * hold_back_window < 0: everything recorded so far is planned and run. >= 0 (an automatic flush in
  * the middle of a program): statements from the one that produced a still-live result within the
- * last `window` records onwards stay in the executor until the next call, so that a result whose
- * handle is about to go away is not turned into an array just because the flush fell there. */
+ * last `window` records onwards stay unplanned in the executor, so that a result whose handle is
+ * about to go away is not turned into an array just because the flush fell there. They are planned
+ * with the next cnx_receive_log, and to their end by whatever needs the arrays' state first:
+ * cnx_get, cnx_put, cnx_fill_*, cnx_sync, cnx_array_info and cnx_receive_dag (a DAG message runs
+ * behind every statement logged before it). */
 int cnx_receive_log(cnx_executor* ex, int64_t size, const char* log, int hold_back_window);
 /* Forgets the part of the log an automatic flush held back (the frontend's reset()). */
 int cnx_discard_log(cnx_executor* ex);

@@ -444,6 +444,54 @@ def test_auto_flush_keeps_a_named_intermediate_fused(itf):
     assert sum(ln.startswith("delete") for ln in itf.trace()) == 1
 
 
+def test_state_queries_complete_what_a_hold_back_flush_left(itf):
+    """A flush with a hold-back window may leave its newest statements unplanned. Every call that
+    reads or writes array state (sync, get, array_info, put) and every DAG message that follows
+    sees them done, in order."""
+    n = 32
+    u, f = cnp.zeros((n, n)), cnp.ones((n, n))
+    cnp.execute(itf)
+    itf.trace()
+
+    def held_back_step():
+        f[0, :] = 2.0          # a flush that would hold everything back holds nothing back
+        upd = 0.25 * (u[:-2, 1:-1] + u[2:, 1:-1] + u[1:-1, :-2] + u[1:-1, 2:] + 0.1 * f[1:-1, 1:-1])
+        u[1:-1, 1:-1] = (1.0 / 3.0) * u[1:-1, 1:-1] + (2.0 / 3.0) * upd
+        log = b"".join(lazy._state.pending)
+        lazy._state.pending = []
+        itf.send_log(log, 16)
+        assert not any(ln.startswith("group") for ln in itf.trace())      # still unplanned
+        return upd
+
+    upd = held_back_step()
+    itf.sync()
+    assert sum(ln.startswith("group") for ln in itf.trace()) == 2
+    assert itf.array_info(upd.name)["shape"][:2] == (n - 2, n - 2)
+    del upd
+    cnp.execute(itf)
+    itf.trace()
+    # a DAG message behind a held-back log runs behind its statements
+    upd = held_back_step()
+    itf.send_dag(0, _message([_create(900, (8,), L.F64)]))
+    kinds = [ln.split()[0] for ln in itf.trace()]
+    assert kinds.index("create") < len(kinds) and kinds[-1] == "create" and kinds.count("group") == 2
+    del upd
+    # get
+    upd = held_back_step()
+    got = u.get(itf)
+    assert got.shape == (n, n) and sum(ln.startswith("group") for ln in itf.trace()) == 2
+
+
+def _message(nodes_bytes):
+    return struct.pack("<iii", lazy.DAG_MAGIC, 1, len(nodes_bytes)) + b"".join(nodes_bytes)
+
+
+def _create(name, shape, dtype, node_id=0):
+    w = lazy._NodeWriter()
+    w.op(name, L.OP_CREATE, False, len(shape), dtype, [], [], lazy._full_region(shape))
+    return w.to_bytes(node_id, False)
+
+
 def test_runs_of_same_extent_assignments_become_one_launch(itf):
     """Assignments of one extent whose boxes are single blocks of memory merge; a box that overlaps
     an earlier one of the same array without being identical ends the run; a matrix product
@@ -482,6 +530,35 @@ def test_runs_of_same_extent_assignments_become_one_launch(itf):
     C[4] = H[3] + 1.0
     cnp.execute(itf)
     assert not any("path=statements" in ln for ln in itf.trace())
+
+
+@pytest.mark.parametrize("shape,box", [((4,), (slice(0, 3),)), ((1, 4), (slice(0, 1), slice(0, 4))),
+                                       ((1, 1), (slice(0, 1), slice(0, 1)))])
+def test_a_run_never_assigns_an_array_it_reads_as_a_kernel_scalar(itf, shape, box):
+    """A one-element array used as a scalar is fetched once when the launch starts: the statement
+    that assigns it and the statement that reads it as a scalar stay separate launches, in either
+    order."""
+    c, a = cnp.zeros((1,)), cnp.zeros((1,))
+    x, y = cnp.zeros(shape), cnp.zeros(shape)
+    cnp.execute(itf)
+    itf.trace()
+    c[0:1] = a[0:1] + 1.0
+    y[box] = x[box] * c
+    cnp.execute(itf)
+    runs = [ln for ln in itf.trace() if "path=statements" in ln]
+    assert len(runs) == 2 and all("count=1" in ln for ln in runs)
+    # read as a scalar first, assigned afterwards
+    y[box] = x[box] * c
+    c[0:1] = a[0:1] + 2.0
+    cnp.execute(itf)
+    runs = [ln for ln in itf.trace() if "path=statements" in ln]
+    assert len(runs) == 2 and all("count=1" in ln for ln in runs)
+    # a scalar nobody assigns in the run does not keep statements apart
+    y[box] = x[box] * c
+    x[box] = y[box] + c
+    cnp.execute(itf)
+    runs = [ln for ln in itf.trace() if "path=statements" in ln]
+    assert len(runs) == 1 and "count=2" in runs[0]
 
 
 def test_reductions_ride_on_the_group_that_produces_their_operand(itf):
@@ -548,16 +625,6 @@ def test_kernel_cache_is_bounded_over_a_long_slab_loop(itf):
 
 
 # ---- error behaviour of the executor (messages built by hand where the frontend would refuse) ----
-
-def _message(nodes_bytes):
-    return struct.pack("<iii", lazy.DAG_MAGIC, 1, len(nodes_bytes)) + b"".join(nodes_bytes)
-
-
-def _create(name, shape, dtype, node_id=0):
-    w = lazy._NodeWriter()
-    w.op(name, L.OP_CREATE, False, len(shape), dtype, [], [], lazy._full_region(shape))
-    return w.to_bytes(node_id, False)
-
 
 def test_executor_refuses_what_it_cannot_do(itf):
     itf.send_dag(0, _message([_create(1, (8, 8), L.F64), _create(2, (8,), L.F64), _create(3, (8,), L.F32),
