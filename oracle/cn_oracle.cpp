@@ -2,6 +2,10 @@
 // TEST INFRASTRUCTURE ONLY: used by tests/, __graft_entry__.smoke() and bench.py's cpu_baseline
 // leg as the checker / the timed CPU baseline. The product never links or calls it.
 // Build: g++ -O3 -ffp-contract=off -fno-fast-math (see oracle/Makefile).
+// Every exported function is pinned by tests/test_oracle_*.py against upstream's own vectors, NumPy
+// in the same operand order, closed forms, exactly rounded sums or brute force. Left open at bit
+// level (only the 1e-12 bar applies): the summation order inside upstream's Eigen dot / GEMV / GEMM
+// and its reduction tree; integer x/0 and MIN/-1 (fixed values here, undefined upstream).
 #include "cn_oracle.h"
 
 #include <algorithm>

@@ -230,3 +230,118 @@ def test_cg_closed_form_system(orc):
         rtr = rtr_new
     want = (b - b.sum() / (2 * n)) / n
     assert np.allclose(x, want, rtol=1e-12, atol=1e-12)
+
+
+@pytest.mark.parametrize("dt,npdt", [(L.F32, np.float32), (L.F64, np.float64), (L.I32, np.int32),
+                                     (L.I64, np.int64)])
+def test_axpy1_is_one_ieee_or_wrapping_add_per_element(orc, dt, npdt):
+    """The 1-D accumulate of matvec partials: res[i] += partial[i], nothing else."""
+    rng = np.random.default_rng(11)
+    n = 4099
+    if np.issubdtype(npdt, np.integer):
+        info = np.iinfo(npdt)
+        res = rng.integers(info.min, info.max, n, dtype=npdt)
+        part = rng.integers(info.min, info.max, n, dtype=npdt)
+        res[:2], part[:2] = [info.max, info.min], [1, -1]          # wrap both ways
+        bits = info.bits
+        want = [((int(a) + int(b) + (1 << (bits - 1))) % (1 << bits)) - (1 << (bits - 1))
+                for a, b in zip(res, part)]                        # Python big integers
+        want = np.array(want, dtype=npdt)
+    else:
+        res = (rng.standard_normal(n) * 10.0 ** rng.integers(-8, 8, n)).astype(npdt)
+        part = (rng.standard_normal(n) * 10.0 ** rng.integers(-8, 8, n)).astype(npdt)
+        want = res + part
+    untouched = part.copy()
+    assert orc.lib.orc_axpy1(dt, n, O.ptr(part), O.ptr(res)) == 0
+    assert np.array_equal(res, want) and np.array_equal(part, untouched)
+    # n = 0 touches nothing
+    before = res.copy()
+    assert orc.lib.orc_axpy1(dt, 0, O.ptr(part), O.ptr(res)) == 0 and np.array_equal(res, before)
+    assert orc.lib.orc_axpy1(9, 1, O.ptr(part), O.ptr(res)) == -1
+
+
+def test_threaded_matvec_and_product_are_the_single_thread_bits(orc):
+    """Rows are split over threads, a row's sum is not: any thread count gives the same bits, and
+    those are within 1e-12 * sum|a||x| of the exactly rounded row dots."""
+    rng = np.random.default_rng(12)
+    rows, cols, ld = 301, 257, 300
+    M = rng.uniform(-1, 1, (rows + 7, ld))
+    x = rng.uniform(-1, 1, cols)
+    row_off, col_off = 5, 31
+
+    def run(threads):
+        y = np.full(rows, np.nan)
+        assert orc.lib.orc_gemv_sub_mt(L.F64, O.ptr(M), ld, row_off, col_off, rows, cols, O.ptr(x),
+                                       O.ptr(y), threads) == 0
+        return y
+
+    one = run(1)
+    for threads in (2, 5, 16, 1000):
+        assert np.array_equal(run(threads), one)
+    sub = M[row_off:row_off + rows, col_off:col_off + cols]
+    exact = np.array([math.fsum(sub[i] * x) for i in range(rows)])
+    assert np.all(np.abs(one - exact) <= 1e-12 * (np.abs(sub) @ np.abs(x)))
+    # left-to-right order, the one the single-thread pins fix
+    lr = np.zeros(rows)
+    for j in range(cols):
+        lr += sub[:, j] * x[j]
+    assert np.array_equal(one, lr)
+    # products: C += A.B with rows split over threads
+    A, B = rng.uniform(-1, 1, (37, 29)), rng.uniform(-1, 1, (29, 23))
+    C0 = rng.uniform(-1, 1, (37, 23))
+    ref = orc.gemm_acc(A, B, C0.copy(), threads=1)
+    for threads in (2, 5, 16):
+        assert np.array_equal(orc.gemm_acc(A, B, C0.copy(), threads=threads), ref)
+    exact = np.array([[math.fsum([C0[i, j]] + list(A[i] * B[:, j])) for j in range(23)] for i in range(37)])
+    assert np.all(np.abs(ref - exact) <= 1e-12 * (np.abs(C0) + np.abs(A) @ np.abs(B)))
+
+
+def test_sum_and_difference_reductions(orc):
+    """sum: one accumulator, index order (floats: Python's left-to-right sum of the same doubles;
+    integers wrap). sumsq_diff: sum of (a-b)*(a-b), same order. maxabs_diff: exact, any order."""
+    rng = np.random.default_rng(13)
+    n = 5003
+    a = rng.uniform(-1, 1, n) * 10.0 ** rng.integers(-3, 3, n)
+    b = rng.uniform(-1, 1, n)
+    out = np.zeros(1)
+    assert orc.lib.orc_sum(L.F64, n, O.ptr(a), O.ptr(out)) == 0
+    acc = 0.0
+    for v in a.tolist():
+        acc += v
+    assert out[0] == acc and abs(out[0] - math.fsum(a)) <= 1e-12 * np.abs(a).sum()
+    af = a.astype(np.float32)
+    outf = np.zeros(1, np.float32)
+    assert orc.lib.orc_sum(L.F32, n, O.ptr(af), O.ptr(outf)) == 0
+    accf = np.float32(0)
+    for v in af:
+        accf = np.float32(accf + v)
+    assert outf[0] == accf
+    for dt, npdt in ((L.I32, np.int32), (L.I64, np.int64)):
+        info = np.iinfo(npdt)
+        v = rng.integers(info.min, info.max, 777, dtype=npdt)
+        o = np.zeros(1, npdt)
+        assert orc.lib.orc_sum(dt, v.size, O.ptr(v), O.ptr(o)) == 0
+        total = sum(int(t) for t in v)
+        assert int(o[0]) == ((total + (1 << (info.bits - 1))) % (1 << info.bits)) - (1 << (info.bits - 1))
+    # closed forms: arange, ones (examples/reduction.py:3-6 upstream)
+    ar = np.arange(1.0, 1001.0)
+    assert orc.lib.orc_sum(L.F64, 1000, O.ptr(ar), O.ptr(out)) == 0 and out[0] == 500500.0
+    # sum of squared differences
+    assert orc.lib.orc_sumsq_diff(n, O.ptr(a), O.ptr(b), O.ptr(out)) == 0
+    acc = 0.0
+    for p, q in zip(a.tolist(), b.tolist()):
+        d = p - q
+        acc += d * d
+    assert out[0] == acc
+    assert abs(out[0] - math.fsum((a - b) ** 2)) <= 1e-12 * ((a - b) ** 2).sum()
+    assert orc.lib.orc_sumsq_diff(n, O.ptr(a), O.ptr(a), O.ptr(out)) == 0 and out[0] == 0.0
+    # a sign error (a + b) or a missing square would fail these
+    three, one = np.full(10, 3.0), np.ones(10)
+    assert orc.lib.orc_sumsq_diff(10, O.ptr(three), O.ptr(one), O.ptr(out)) == 0 and out[0] == 40.0
+    # largest absolute difference
+    assert orc.lib.orc_maxabs_diff(n, O.ptr(a), O.ptr(b), O.ptr(out)) == 0
+    assert out[0] == np.abs(a - b).max() == max(abs(p - q) for p, q in zip(a.tolist(), b.tolist()))
+    assert orc.lib.orc_maxabs_diff(n, O.ptr(b), O.ptr(a), O.ptr(out)) == 0 and out[0] == np.abs(a - b).max()
+    neg = -three
+    assert orc.lib.orc_maxabs_diff(10, O.ptr(neg), O.ptr(one), O.ptr(out)) == 0 and out[0] == 4.0
+    assert orc.lib.orc_maxabs_diff(0, O.ptr(a), O.ptr(b), O.ptr(out)) == 0 and out[0] == 0.0
