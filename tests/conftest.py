@@ -26,3 +26,12 @@ def dev():
     from tests.helpers import Device
 
     return Device()
+
+
+@pytest.fixture(scope="session")
+def cpu_cg_system():
+    """The dense CG configuration on the host (n = 16384, oracle generator, seed 2): matrix tiles
+    and right-hand side, built once per session (2 GiB)."""
+    import bench
+
+    return bench.cpu_cg_setup(16384)

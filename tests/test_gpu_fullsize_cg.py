@@ -19,9 +19,9 @@ THREADS = min(os.cpu_count() or 1, 16)
 
 
 @pytest.fixture(scope="module")
-def cpu_system():
+def cpu_system(cpu_cg_system):
     """Matrix tiles and right-hand side on the host (oracle generator, seed 2)."""
-    return bench.cpu_cg_setup(N)
+    return cpu_cg_system
 
 
 def test_gemv_tiles_n16384_matches_oracle_tile_matvec(dev, cpu_system):

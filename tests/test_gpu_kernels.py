@@ -140,8 +140,9 @@ def _tiles(dev, arr, parts):
     return bufs, [int(bounds[i + 1] - bounds[i]) for i in range(parts)]
 
 
-@pytest.mark.parametrize("n,parts", [(1 << 22, 4), (16384, 1), (100003, 3), (5, 1), (70000, 1)])
+@pytest.mark.parametrize("n,parts", [(1 << 24, 4), (1 << 22, 4), (16384, 1), (100003, 3), (5, 1), (70000, 1)])
 def test_dot_and_sum_fp64(dev, orc, n, parts):
+    """(2^24, 4) is the elementwise configuration's size: 4 partitions of 4 194 304."""
     a = orc.uniform(n, 0, 0, -1, 1)
     b = orc.uniform(n, 0, 1, -1, 1)
     ab, lens = _tiles(dev, a, parts)
@@ -163,6 +164,9 @@ def test_dot_and_sum_fp64(dev, orc, n, parts):
                                 out.ptr, None))
     got = out.get()[0]
     assert abs(got - math.fsum(a.tolist())) <= REL * math.fsum(np.abs(a).tolist())
+    osum = np.zeros(1)
+    assert orc.lib.orc_sum(L.F64, n, a.ctypes.data, osum.ctypes.data) == 0
+    assert abs(got - osum[0]) <= 2 * REL * math.fsum(np.abs(a).tolist())
     dev.free_all()
 
 
@@ -215,6 +219,12 @@ def test_sumsq_and_maxabs_diff(dev, orc):
     L.check(L.lib.cnh_maxabs_diff_tiles(3, L.vparr([x.ptr for x in ab]),
                                         L.vparr([x.ptr for x in bb]), L.i64arr(lens), out.ptr, None))
     assert out.get()[0] == np.max(np.abs(a - b))  # exact, order-independent
+    # and the oracle's own forms of the two
+    o = np.zeros(1)
+    assert orc.lib.orc_maxabs_diff(n, a.ctypes.data, b.ctypes.data, o.ctypes.data) == 0
+    assert out.get()[0] == o[0]
+    assert orc.lib.orc_sumsq_diff(n, a.ctypes.data, b.ctypes.data, o.ctypes.data) == 0
+    assert abs(o[0] - ref) <= REL * ref
     dev.free_all()
 
 
