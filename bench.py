@@ -1058,6 +1058,135 @@ def cpu_jacobi(nd, n, tile, sweeps, threads):
             "what": "oracle restatement of the reference's fragment path, one thread per chare"}
 
 
+def _physical_cores():
+    """(logical CPUs the process may use, physical cores of the box as /proc/cpuinfo lists them)."""
+    logical = os.cpu_count() or 1
+    try:
+        logical = len(os.sched_getaffinity(0))
+    except (AttributeError, OSError):
+        pass
+    cores = set()
+    try:
+        phys = core = None
+        with open("/proc/cpuinfo") as f:
+            for ln in f:
+                if ln.startswith("physical id"):
+                    phys = ln.split(":")[1].strip()
+                elif ln.startswith("core id"):
+                    core = ln.split(":")[1].strip()
+                elif not ln.strip():
+                    if core is not None:
+                        cores.add((phys, core))
+                    phys = core = None
+    except OSError:
+        pass
+    return logical, (len(cores) or None)
+
+
+def cpu_c1(threads, n=1 << 24, parts=4, passes=3):
+    """Configuration 1 on the host as the reference's fast path runs it
+    (src/execute_node.cpp:1263-1336 upstream): the fused statement chare by chare over the 4 tiles
+    (one interpreted kernel per chare, `threads` chares side by side, at most one thread per chare),
+    then z . ones and z . z tile by tile with the partials added in tile order
+    (src/executor_reduce.cpp:62-94 upstream). A bounded sample: `passes` passes at full size."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    from charmnumeric_amd import _lib as L
+    from oracle import cn_oracle as O
+
+    orc = O.Oracle()
+    per = n // parts
+    ast = c1_ast(L)
+    xs = [orc.uniform(per, 0, 0, -1.0, 1.0, first=q * per) for q in range(parts)]
+    ys = [orc.uniform(per, 0, 1, -1.0, 1.0, first=q * per) for q in range(parts)]
+    zs = [np.empty(per) for _ in range(parts)]
+    ones = np.ones(per)
+    workers = max(1, min(threads, parts))
+
+    def chare(q):
+        if orc.eval_group(ast, L.F64, 1, [xs[q], ys[q], xs[q], ys[q]], [], [zs[q]]):
+            raise RuntimeError("oracle group evaluation failed")
+
+    def dots(q):
+        return orc.dot(zs[q], ones), orc.dot(zs[q], zs[q])
+
+    t_elem = t_red = 0.0
+    s = nrm2 = 0.0
+    with ThreadPoolExecutor(workers) as pool:
+        list(pool.map(chare, range(parts)))       # untimed: the result tiles' pages are touched here
+        for _ in range(passes):
+            t0 = time.perf_counter()
+            list(pool.map(chare, range(parts)))
+            t1 = time.perf_counter()
+            partials = list(pool.map(dots, range(parts)))
+            s = nrm2 = 0.0
+            for a, b in partials:                 # tile order, as the reducer adds them
+                s += a
+                nrm2 += b
+            t2 = time.perf_counter()
+            t_elem += t1 - t0
+            t_red += t2 - t1
+    elem_us = t_elem / passes * 1e6
+    return {"elementwise_us": round(elem_us, 1), "elementwise_GBs": round(24.0 * n / (elem_us * 1e-6) / 1e9, 2),
+            "two_reductions_us": round(t_red / passes * 1e6, 1), "threads": workers, "passes": passes,
+            "sum": float(s), "norm": float(np.sqrt(nrm2)),
+            "what": "oracle restatement of the reference's fast path: one fused loop per chare over 4 chares, "
+                    "then tile dots added in tile order"}
+
+
+def cpu_lstm(threads, steps=2, batch=256, nin=1024, d=1024, seed=5):
+    """Configuration 5 on the host: per step the gate product as the reference's panel accumulate
+    (C zeroed, C += A.B, src/executor_incremental.cpp:120-132 upstream; rows split over `threads`)
+    and the gate statements of examples/lstm_forward.py:40-49 upstream as one interpreted group
+    each. A bounded sample: `steps` steps at the full shape."""
+    from charmnumeric_amd import _lib as L
+    from oracle import cn_oracle as O
+
+    orc = O.Oracle()
+    k_in = nin + d
+    X = orc.uniform(steps * batch * nin, seed, 0, -1.0, 1.0).reshape(steps, batch, nin)
+    Wih = orc.uniform(4 * d * nin, seed, 1, -1.0 / 32, 1.0 / 32).reshape(4 * d, nin)
+    Whh = orc.uniform(4 * d * d, seed, 2, -1.0 / 32, 1.0 / 32).reshape(4 * d, d)
+    W = np.ascontiguousarray(np.concatenate([Wih.T, Whh.T], axis=0))
+    Hin = np.zeros((steps, batch, k_in))
+    IFOG = np.zeros((steps, batch, 4 * d))
+    IFOGf = np.zeros((steps, batch, 4 * d))
+    Cc = np.zeros((steps, batch, d))
+    Ct = np.zeros((steps, batch, d))
+    Hout = np.zeros((steps, batch, d))
+    a_sig, a_tanh, a_mul, a_muladd = lstm_asts(L, d)
+
+    def group(ast, ins, outs):
+        if orc.eval_group(ast, L.F64, 2, ins, [], outs):
+            raise RuntimeError("oracle group evaluation failed")
+
+    t_gemm = t_gate = 0.0
+    for t in range(steps):
+        Hin[t, :, :nin] = X[t]
+        if t > 0:
+            Hin[t, :, nin:] = Hout[t - 1]
+        t0 = time.perf_counter()
+        IFOG[t] = 0.0
+        orc.gemm_acc(Hin[t], W, IFOG[t], threads=threads)
+        t1 = time.perf_counter()
+        group(a_sig, [IFOG[t, :, :3 * d]], [IFOGf[t, :, :3 * d]])
+        group(a_tanh, [IFOG[t, :, 3 * d:]], [IFOGf[t, :, 3 * d:]])
+        group(a_mul, [IFOGf[t, :, :d], IFOGf[t, :, 3 * d:]], [Cc[t]])
+        if t > 0:
+            group(a_muladd, [IFOGf[t, :, d:2 * d], Cc[t - 1], Cc[t]], [Cc[t]])
+        group(a_tanh, [Cc[t]], [Ct[t]])
+        group(a_mul, [IFOGf[t, :, 2 * d:3 * d], Ct[t]], [Hout[t]])
+        t2 = time.perf_counter()
+        t_gemm += t1 - t0
+        t_gate += t2 - t1
+    flop = 2.0 * batch * k_in * 4 * d
+    return {"gemm_us": round(t_gemm / steps * 1e6, 1), "gemm_GFLOPs": round(flop * steps / t_gemm / 1e9, 2),
+            "gates_us": round(t_gate / steps * 1e6, 1), "step_us": round((t_gemm + t_gate) / steps * 1e6, 1),
+            "threads": threads, "steps": steps, "h_last_abs_mean": float(np.mean(np.abs(Hout[steps - 1]))),
+            "what": "oracle restatement: panel accumulate C += A.B with rows over threads, then the six gate "
+                    "statements as interpreted groups on one thread"}
+
+
 def run_frontend(n, steps, warmup):
     """The same CG iteration and Jacobi sweeps written against the NumPy-like frontend: statements
     -> DAG message -> host executor -> the same kernels. Shows what the whole stack costs on top of
@@ -1312,13 +1441,14 @@ def main():
             also["frontend_error"] = str(exc)
         line["also"] = also
     if not args.no_cpu:
-        cores = os.cpu_count() or 1
-        threads = min(cores, 16)
+        logical, physical = _physical_cores()
+        threads = min(logical, 16)
         setup = cpu_cg_setup(n)
         ips1, _, _, _ = cpu_cg(setup, n, args.cpu_iters, 1)
         ipsN, _, _, cpu_trace = cpu_cg(setup, n, args.cpu_iters, threads, keep_x_at=parity_iters)
         line["cpu_baseline"] = {
             "value": round(ipsN, 3), "unit": "iterations/s", "cores": threads, "kind": "port",
+            "threads_used": threads, "host_logical_cpus": logical, "host_physical_cores": physical,
             "sample": f"same system (n={n}, {cg['tile']}^2 tiles), {args.cpu_iters} CG iterations, "
                       f"oracle kernels, tile matvec split over {threads} threads",
             "one_core": round(ips1, 3),
@@ -1327,6 +1457,16 @@ def main():
             try:
                 line["also"]["c3_jacobi2d_8192"]["cpu_port"] = cpu_jacobi(2, 8192, 2048, 3, threads)
                 line["also"]["c4_jacobi3d_512"]["cpu_port"] = cpu_jacobi(3, 512, 128, 2, threads)
+                line["also"]["c1_fused_elementwise_2p24"]["cpu_port"] = {
+                    "one_core": cpu_c1(1), "threads": cpu_c1(threads)}
+                line["also"]["c5_lstm_forward"]["cpu_port"] = {
+                    "one_core": cpu_lstm(1, steps=1), "threads": cpu_lstm(threads, steps=2)}
+                # the frontend's C1 results against the host's, relative to the sum of |terms|
+                # (sum: about 2^24 * 0.55; norm: relative to itself)
+                fe, cp = line["also"].get("through_frontend", {}), line["also"]["c1_fused_elementwise_2p24"]["cpu_port"]
+                if "c1_sum" in fe:
+                    fe["c1_sum_vs_cpu_rel_to_abs_terms"] = abs(fe["c1_sum"] - cp["threads"]["sum"]) / (0.55 * (1 << 24))
+                    fe["c1_norm_vs_cpu_rel"] = abs(fe["c1_norm"] - cp["threads"]["norm"]) / cp["threads"]["norm"]
             except Exception as exc:
                 line["also"]["cpu_port_error"] = str(exc)
         # same system, same number of iterations (an untimed pass of the device path before the
