@@ -17,6 +17,7 @@ OP_COPY, OP_SET_REGION, OP_GET_REGION, OP_CREATE, OP_NOOP = -5, -4, -3, -2, -1
 OP_ADD, OP_SUB, OP_MUL, OP_DIV, OP_MATMUL, OP_TANH, OP_EXP = 0, 1, 2, 3, 4, 5, 6
 OP_TILE, OP_REDUCE, OP_MATMATMUL, OP_DIAG = 7, 8, 9, 10
 OP_SUM_OF, OP_MAXABS_OF = 20, 21          # reducing roots of a fused group (extension)
+OP_SCALAR_OF = 22                         # an output formed from scalars alone, stored once (extension)
 
 
 class CnhError(RuntimeError):
@@ -88,7 +89,7 @@ class GemvFusion(C.Structure):
     """cnh_gemv_fusion: the vector work a fused matvec takes along."""
     _fields_ = [("xa", C.c_void_p), ("xb", C.c_void_p), ("num", C.c_void_p), ("num_count", C.c_int64),
                 ("den", C.c_void_p), ("num_folded", C.c_void_p), ("w", C.c_void_p),
-                ("dot_partials", C.c_void_p), ("dot_capacity", C.c_int64)]
+                ("dot_partials", C.c_void_p), ("dot_capacity", C.c_int64), ("quotient_out", C.c_void_p)]
 
 
 class ScalarSum(C.Structure):
@@ -219,6 +220,7 @@ _PROTOS = {
     "cnh_kernel_release": (C.c_int, [C.c_void_p]),
     "cnh_launch_group_sums": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int,
                                         C.c_void_p, C.c_void_p]),
+    "cnh_fold_sums": (C.c_int, [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]),
     "cnh_kernel_matches": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int]),
     "cnh_kernel_signature": (C.c_int, [C.c_void_p, C.POINTER(C.c_int), C.POINTER(C.c_int),
                                        C.POINTER(C.c_int)]),

@@ -269,6 +269,12 @@ int build_group_program(const cnh_ast* ast, int dtype, int ndims, GroupProgram& 
                 err = "SET_REGION without a usable right-hand side";
                 return -10;
             }
+        } else if (opc == CNH_OP_SCALAR_OF) {
+            res = lookup(root, 0);
+            if (!res.valid || !res.scalar || root.is_temp) {
+                err = "SCALAR_OF is an output that takes a value formed from scalars alone";
+                return -12;
+            }
         } else if (opc == CNH_OP_COPY || opc == CNH_OP_SUM_OF || opc == CNH_OP_MAXABS_OF) {
             res = lookup(root, 0);
             if (!res.valid || res.scalar) {
@@ -326,7 +332,8 @@ int build_group_program(const cnh_ast* ast, int dtype, int ndims, GroupProgram& 
         p.out_names.push_back(root.result_name);
         bool sr = root.opcode == CNH_OP_SET_REGION;
         p.out_is_set_region.push_back(sr ? 1 : 0);
-        p.out_reduce.push_back(root.opcode == CNH_OP_SUM_OF ? 1 : root.opcode == CNH_OP_MAXABS_OF ? 2 : 0);
+        p.out_reduce.push_back(root.opcode == CNH_OP_SUM_OF ? 1 : root.opcode == CNH_OP_MAXABS_OF ? 2
+                               : root.opcode == CNH_OP_SCALAR_OF ? 3 : 0);
         int target = root.result_name;
         if (sr && root.n_operands > 0 && root.operands[0] >= 0)
             target = ast->nodes[root.operands[0]].result_name;
@@ -409,13 +416,17 @@ std::string flat_source(const GroupProgram& p) {
     s << "#define VECW " << vec << "\n";
     // Outputs that are reduced instead of stored: a mask over the output list, and the statement
     // that folds one element's values into the lane's running results.
-    unsigned mask = 0;
+    unsigned mask = 0, once_mask = 0;
     int nred = 0;
     std::ostringstream fold, init;
     for (size_t j = 0; j < p.out_reduce.size(); ++j) {
         if (!p.out_reduce[j])
             continue;
         mask |= 1u << j;
+        if (p.out_reduce[j] == 3) {
+            once_mask |= 1u << j;
+            continue;
+        }
         if (p.out_reduce[j] == 1)
             fold << " racc[" << nred << "] += o[" << j << "];";
         else
@@ -423,13 +434,14 @@ std::string flat_source(const GroupProgram& p) {
                  << "] = a_ > racc[" << nred << "] ? a_ : racc[" << nred << "]; }";
         ++nred;
     }
-    s << "#define RED_MASK " << mask << "u\n#define NR " << nred << "\n#define NRA " << (nred ? nred : 1) << "\n";
+    s << "#define RED_MASK " << mask << "u\n#define ONCE_MASK " << once_mask << "u\n#define NR " << nred
+      << "\n#define NRA " << (nred ? nred : 1) << "\n";
     s << "#define RED_FOLD(o, racc) do {" << fold.str() << " } while (0)\n";
     std::ostringstream comb;
     {
         int q = 0;
         for (size_t j = 0; j < p.out_reduce.size(); ++j) {
-            if (!p.out_reduce[j])
+            if (!p.out_reduce[j] || p.out_reduce[j] == 3)
                 continue;
             if (p.out_reduce[j] == 1)
                 comb << " racc[" << q << "] += other[" << q << "];";
@@ -451,6 +463,20 @@ std::string flat_source(const GroupProgram& p) {
 struct Seg { i64 n; i64 blk0; const T* in[NLA]; T* out[NOA]; };
 typedef T TV __attribute__((ext_vector_type(VECW)));
 #define OUT_STORED(j) (((RED_MASK >> (j)) & 1u) == 0u)
+
+// Outputs in ONCE_MASK (CNH_OP_SCALAR_OF) hold a value formed from the launch's scalars alone: the
+// first lane of the launch stores it once, at element 0 of the first segment's output.
+__device__ __forceinline__ void store_once(T* const* out, const T* s) {
+    if (ONCE_MASK != 0u && blockIdx.x == 0 && threadIdx.x == 0) {
+        T l[NLA], o[NOA];
+#pragma unroll
+        for (int k = 0; k < NLA; ++k) l[k] = 0;
+        group_eval(l, s, o);
+#pragma unroll
+        for (int j = 0; j < NO; ++j)
+            if ((ONCE_MASK >> j) & 1u) out[j][0] = o[j];
+    }
+}
 
 // Workgroups of one wavefront where nothing is reduced (a plain triad over 2^24 doubles streams at
 // 0.86 of the HBM peak with 64 lanes a workgroup, 0.84 with 128, 0.82 with 256 to 1024); reducing
@@ -602,6 +628,7 @@ extern "C" __global__ __launch_bounds__(FLAT_WG) void grp_flat_##NAME(const Seg*
     const Seg& sg = segs[k];                                                                     \
     const i64 blk = (i64)blockIdx.x - sg.blk0;                                                   \
     CALL;                                                                                        \
+    store_once(segs[0].out, s);                                                                  \
     RED_END                                                                                      \
 }                                                                                                \
 extern "C" __global__ __launch_bounds__(FLAT_WG) void grp_flat1_##NAME(Seg sg, Scal sc RED_PARAM) { \
@@ -609,6 +636,7 @@ extern "C" __global__ __launch_bounds__(FLAT_WG) void grp_flat1_##NAME(Seg sg, S
     RED_BEGIN                                                                                    \
     const i64 blk = (i64)blockIdx.x;                                                             \
     CALL;                                                                                        \
+    store_once(sg.out, s);                                                                       \
     RED_END                                                                                      \
 }                                                                                                \
 extern "C" __global__ __launch_bounds__(256) void grp_flat1f_##NAME(Seg sg, Scal sc, Fold fd    \
@@ -617,6 +645,7 @@ extern "C" __global__ __launch_bounds__(256) void grp_flat1f_##NAME(Seg sg, Scal
     RED_BEGIN                                                                                    \
     const i64 blk = (i64)blockIdx.x;                                                             \
     CALL256;                                                                                     \
+    store_once(sg.out, s);                                                                       \
     RED_END                                                                                      \
 }
 FLAT_ENTRY(v, (flat_vec<false, FLAT_WG>(sg, blk, s, racc)), (flat_vec<false, 256>(sg, blk, s, racc)))

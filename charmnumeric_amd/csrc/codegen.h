@@ -35,16 +35,25 @@ struct GroupProgram {
     std::vector<int> out_names;   // result name of each output root
     std::vector<int> out_roots;   // root positions of the non-temp roots
     std::vector<int> out_is_set_region;
-    std::vector<int> out_reduce;  // 0: stored element by element; 1: summed, 2: largest |value|
+    std::vector<int> out_reduce;  // 0: stored element by element; 1: summed, 2: largest |value|,
+                                  // 3: a value without an index, stored once (CNH_OP_SCALAR_OF)
     std::vector<int> out_target;  // SET_REGION target array name (or result name)
     std::vector<cnh_region> out_region; // SET_REGION region (is_global when absent)
     std::vector<std::string> out_expr;  // value expression of each output
     std::string body;             // statements computing t<k> from l<load>, s<bcast>
     bool uses_transcendental = false;
+    // outputs that are not stored element by element (dense launches only)
     int reductions() const {
         int n = 0;
         for (int r : out_reduce)
             n += r != 0;
+        return n;
+    }
+    // those of them that are reduced over the launch and leave partial results
+    int folds() const {
+        int n = 0;
+        for (int r : out_reduce)
+            n += r == 1 || r == 2;
         return n;
     }
 };

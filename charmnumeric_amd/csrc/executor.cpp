@@ -199,6 +199,17 @@ struct cnx_executor {
     std::vector<char> captured;
     int deferred_rc = 0;
     std::string deferred_msg;
+    // One-element arrays whose value still stands as partial sums in a buffer of their own (what a
+    // launch with a reducing root, or a matvec that took the dot along, left behind). The next
+    // launch that reads such an array as a kernel scalar sums the partials itself and stores the
+    // value; anything else that needs it gets a fold launch first (resolve_pending). They exist
+    // only between the nodes of one run_nodes pass or while nodes are held.
+    struct PendingSum {
+        void* partials = nullptr;
+        size_t bytes = 0;
+        int64_t count = 0;
+    };
+    std::map<int, PendingSum> pending;
 
     void log(const std::string& s) {
         if (trace_on) {
@@ -368,6 +379,11 @@ void drop_array(Ex* ex, int name) {
     auto it = ex->arrays.find(name);
     if (it == ex->arrays.end())
         return;
+    auto pend = ex->pending.find(name);
+    if (pend != ex->pending.end()) {            // nobody asked for the value: no fold needed
+        slab_release(ex, pend->second.bytes, pend->second.partials);
+        ex->pending.erase(pend);
+    }
     slab_release(ex, it->second.bytes, it->second.slab);
     slab_release(ex, it->second.bytes, it->second.alt);
     ex->arrays.erase(it);
@@ -2345,6 +2361,773 @@ int try_group_with_reductions(Ex* ex, const std::vector<DagNode>& dag, size_t i,
     return 0;
 }
 
+// ---- partial sums that wait for their consumer ----
+//
+// A launch that reduces on the way leaves one partial sum per workgroup. Folding them takes a
+// launch of its own, and the value is usually wanted by exactly one thing: the next launch, as a
+// kernel scalar (alpha = r.r / p.Ap). Such a launch can sum a few hundred partials itself, every
+// workgroup in the same order, and store the value on the way. So the result array of a reduction
+// may stay "pending": its partials sit in a buffer of their own until a launch takes them
+// (pending_done) or something else needs the value (resolve_pending: one small fold launch in the
+// same order of additions).
+constexpr int64_t kDeferMaxPartials = 1024;
+
+int pending_buffer(Ex* ex, int64_t count, Ex::PendingSum* out) {
+    out->count = count;
+    out->bytes = (size_t)((count * 8 + 255) & ~(int64_t)255);
+    return slab_alloc(ex, out->bytes, false, &out->partials);
+}
+
+void pending_done(Ex* ex, int name) {
+    auto it = ex->pending.find(name);
+    if (it == ex->pending.end())
+        return;
+    slab_release(ex, it->second.bytes, it->second.partials);
+    ex->pending.erase(it);
+}
+
+int resolve_pending(Ex* ex, int name) {
+    auto it = ex->pending.find(name);
+    if (it == ex->pending.end())
+        return 0;
+    int rc = 0;
+    auto arr = ex->arrays.find(name);
+    if (arr != ex->arrays.end()) {
+        ex->log("fold " + std::to_string(name) + " partials=" + std::to_string(it->second.count));
+        if (!ex->dry)
+            rc = cnh_fold_sums(it->second.partials, it->second.count, arr->second.tiles[0], ex->stream);
+    }
+    pending_done(ex, name);
+    return rc;
+}
+
+int resolve_all(Ex* ex) {
+    while (!ex->pending.empty())
+        if (int rc = resolve_pending(ex, ex->pending.begin()->first))
+            return rc;
+    return 0;
+}
+
+// The first node at or after j that is not a deletion; the names deleted on the way go to `dels`.
+size_t skip_deletions(const std::vector<DagNode>& dag, size_t j, std::vector<int>& dels) {
+    for (; j < dag.size(); ++j) {
+        if (dag[j].roots.empty())
+            break;
+        const cnh_ast_node& r = dag[j].nodes[dag[j].roots.back()];
+        if (r.opcode != kOpDelete)
+            break;
+        dels.push_back(r.result_name);
+    }
+    return j;
+}
+
+bool operand_is_whole(const cnh_ast_node& r, int oi, const int32_t* shape, int nd) {
+    if (!r.has_operand_region[oi] || r.operand_regions[oi].is_global)
+        return true;
+    const cnh_region& g = r.operand_regions[oi];
+    if (g.ndims != nd)
+        return false;
+    for (int d = 0; d < nd; ++d)
+        if (g.start[d] != 0 || g.stop[d] != shape[d] || g.step[d] != 1)
+            return false;
+    return true;
+}
+
+cnh_memref dense_memref_of(void* ptr, int nd, const int32_t* shape) {
+    cnh_memref m;
+    std::memset(&m, 0, sizeof m);
+    m.allocated = m.aligned = ptr;
+    int64_t stride = 1;
+    for (int d = nd - 1; d >= 0; --d) {
+        m.sizes[d] = shape[d];
+        m.strides[d] = stride;
+        stride *= shape[d];
+    }
+    return m;
+}
+
+// ---- a matvec with the vector work of a Krylov iteration around it ----
+//
+//   [beta = a / b ; p = xa + beta * xb ;]  y = A @ p  [; d = p @ y]
+// (examples/cg.py:40-52 upstream: the p update of one iteration, the product and the dot of the
+// next) as ONE launch of the matvec that stages its vector in LDS: it forms the vector while it
+// stages it, stores it, beta and the numerator's sum on the way, and leaves the partial sums of the
+// dot. Deletions between these nodes wait until the launch is out. Applies to whole fp64 matrices
+// of 16384 rows or more cut into even tiles of at most 8192 columns; everything else runs node by
+// node as before.
+struct MatvecSite {
+    XArray* A = nullptr;
+    int x_name = 0, y_name = 0;
+    int64_t rows = 0, cols = 0;
+};
+
+bool fusable_matvec(Ex* ex, const DagNode& n, MatvecSite* site) {
+    if (n.roots.size() != 1)
+        return false;
+    const cnh_ast_node& root = n.nodes[n.roots.back()];
+    if (root.opcode != CNH_OP_MATMUL || root.n_operands != 2 || root.dtype != CNH_F64)
+        return false;
+    const cnh_ast_node& oa = n.nodes[root.operands[0]];
+    const cnh_ast_node& ox = n.nodes[root.operands[1]];
+    if (oa.opcode != CNH_OP_NOOP || oa.is_scalar || ox.opcode != CNH_OP_NOOP || ox.is_scalar)
+        return false;
+    auto it = ex->arrays.find(oa.result_name);
+    if (it == ex->arrays.end())
+        return false;
+    XArray& A = it->second;
+    if (A.ndims != 2 || A.dtype != CNH_F64 || A.flat || A.phased() || A.offset[0] != 0 || A.offset[1] != 0)
+        return false;
+    if (!operand_is_whole(root, 0, A.shape, 2))
+        return false;
+    const int32_t xshape[3] = {A.shape[1], 1, 1};
+    if (!operand_is_whole(root, 1, xshape, 1))
+        return false;
+    if (A.shape[0] < 16384 || (int64_t)A.tile * 8 > 65536 || A.tile % 2 != 0 || A.shape[1] % 2 != 0)
+        return false;
+    site->A = &A;
+    site->x_name = ox.result_name;
+    site->y_name = root.result_name;
+    site->rows = A.shape[0];
+    site->cols = A.shape[1];
+    return true;
+}
+
+bool vector_f64(const Ex* ex, int name, int64_t len, const XArray** out) {
+    auto it = ex->arrays.find(name);
+    if (it == ex->arrays.end() || it->second.ndims != 1 || it->second.dtype != CNH_F64 ||
+        it->second.shape[0] != len || it->second.offset[0] != 0)
+        return false;
+    *out = &it->second;
+    return true;
+}
+
+int try_fused_matvec(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t* used, bool* open_ended) {
+    *used = 0;
+    *open_ended = false;
+    if (dag[i].roots.empty())
+        return 0;
+    std::vector<int> dels, dels_kept;
+    size_t at = i;
+    // the prologue, if the run starts with one
+    bool form = false;
+    int beta_name = 0, num_name = 0, den_name = 0, xa_name = 0, xb_name = 0, p_name = 0;
+    {
+        const DagNode& s = dag[i];
+        const cnh_ast_node& r = s.nodes[s.roots.back()];
+        if (r.opcode == CNH_OP_DIV && s.roots.size() == 1 && s.fusible && !r.is_temp && r.dtype == CNH_F64 &&
+            r.n_operands == 2) {
+            const cnh_ast_node& a = s.nodes[r.operands[0]];
+            const cnh_ast_node& b = s.nodes[r.operands[1]];
+            auto one = [&](const cnh_ast_node& op) {
+                if (op.opcode != CNH_OP_NOOP || op.is_scalar)
+                    return false;
+                auto it = ex->arrays.find(op.result_name);
+                return it != ex->arrays.end() && it->second.elems == 1 && it->second.dtype == CNH_F64;
+            };
+            if (!one(a) || !one(b) || a.result_name == b.result_name)
+                return 0;
+            beta_name = r.result_name;
+            num_name = a.result_name;
+            den_name = b.result_name;
+            size_t j = skip_deletions(dag, i + 1, dels);
+            if (j == dag.size()) {
+                *open_ended = open_ended_allowed(ex);
+                return 0;
+            }
+            const DagNode& v = dag[j];
+            if (v.roots.size() != 2 || !v.fusible)
+                return 0;
+            const cnh_ast_node& t = v.nodes[v.roots[0]];
+            const cnh_ast_node& sum = v.nodes[v.roots[1]];
+            if (t.opcode != CNH_OP_MUL || !t.is_temp || t.n_operands != 2 || sum.opcode != CNH_OP_ADD || sum.is_temp ||
+                sum.n_operands != 2 || sum.dtype != CNH_F64)
+                return 0;
+            // t = beta * xb, either way round
+            int which_b = -1;
+            for (int oi = 0; oi < 2; ++oi) {
+                const cnh_ast_node& op = v.nodes[t.operands[oi]];
+                if (op.opcode == CNH_OP_NOOP && !op.is_scalar && op.is_broadcast && op.result_name == beta_name)
+                    which_b = oi;
+            }
+            if (which_b < 0)
+                return 0;
+            const cnh_ast_node& xb = v.nodes[t.operands[1 - which_b]];
+            if (xb.opcode != CNH_OP_NOOP || xb.is_scalar || xb.is_broadcast)
+                return 0;
+            // p = xa + t, either way round
+            int which_t = -1;
+            for (int oi = 0; oi < 2; ++oi) {
+                const cnh_ast_node& op = v.nodes[sum.operands[oi]];
+                if (sum.operands[oi] == v.roots[0] || (!op.is_scalar && op.result_name == t.result_name))
+                    which_t = oi;
+            }
+            if (which_t < 0)
+                return 0;
+            const cnh_ast_node& xa = v.nodes[sum.operands[1 - which_t]];
+            if (xa.opcode != CNH_OP_NOOP || xa.is_scalar || xa.is_broadcast)
+                return 0;
+            xa_name = xa.result_name;
+            xb_name = xb.result_name;
+            p_name = sum.result_name;
+            const XArray *pa = nullptr, *pb = nullptr;
+            auto ita = ex->arrays.find(xa_name);
+            if (ita == ex->arrays.end() || !vector_f64(ex, xa_name, ita->second.shape[0], &pa) ||
+                !vector_f64(ex, xb_name, pa->shape[0], &pb))
+                return 0;
+            const int32_t vshape[3] = {pa->shape[0], 1, 1};
+            if (!operand_is_whole(t, 1 - which_b, vshape, 1) || !operand_is_whole(sum, 1 - which_t, vshape, 1))
+                return 0;
+            at = skip_deletions(dag, j + 1, dels);
+            if (at == dag.size()) {
+                *open_ended = open_ended_allowed(ex);
+                return 0;
+            }
+            form = true;
+        }
+    }
+    MatvecSite mv;
+    if (!fusable_matvec(ex, dag[at], &mv))
+        return 0;
+    const XArray *xa = nullptr, *xb = nullptr, *xv = nullptr;
+    if (form) {
+        if (mv.x_name != p_name || mv.rows != mv.cols || !vector_f64(ex, xa_name, mv.cols, &xa) ||
+            !vector_f64(ex, xb_name, mv.cols, &xb))
+            return 0;
+    } else if (!vector_f64(ex, mv.x_name, mv.cols, &xv)) {
+        return 0;
+    }
+    dels_kept = dels;
+    size_t end = at + 1;
+    // the dot of the vector with the product
+    int dot_name = 0;
+    {
+        size_t k = skip_deletions(dag, at + 1, dels);
+        if (k == dag.size() && open_ended_allowed(ex)) {
+            *open_ended = true;
+            return 0;
+        }
+        if (k < dag.size() && dag[k].roots.size() == 1) {
+            const cnh_ast_node& r = dag[k].nodes[dag[k].roots.back()];
+            if (r.opcode == CNH_OP_REDUCE && r.n_operands == 2 && r.dtype == CNH_F64) {
+                const cnh_ast_node& a = dag[k].nodes[r.operands[0]];
+                const cnh_ast_node& b = dag[k].nodes[r.operands[1]];
+                const int32_t xs[3] = {(int32_t)mv.cols, 1, 1}, ys[3] = {(int32_t)mv.rows, 1, 1};
+                const bool xy = a.result_name == mv.x_name && b.result_name == mv.y_name &&
+                                operand_is_whole(r, 0, xs, 1) && operand_is_whole(r, 1, ys, 1);
+                const bool yx = a.result_name == mv.y_name && b.result_name == mv.x_name &&
+                                operand_is_whole(r, 0, ys, 1) && operand_is_whole(r, 1, xs, 1);
+                if (mv.rows == mv.cols && a.opcode == CNH_OP_NOOP && b.opcode == CNH_OP_NOOP && !a.is_scalar &&
+                    !b.is_scalar && (xy || yx)) {
+                    dot_name = r.result_name;
+                    end = k + 1;
+                    dels_kept = dels;
+                }
+            }
+        }
+    }
+    if (!form && dot_name == 0)
+        return 0;                      // nothing to take along: the plain node does the same
+
+    // from here on the nodes [i, end) are this launch
+    const int32_t yshape[3] = {(int32_t)mv.rows, 1, 1}, xshape[3] = {(int32_t)mv.cols, 1, 1};
+    XArray *y = nullptr, *p = nullptr, *beta = nullptr, *dot = nullptr;
+    cnh_gemv_fusion fu;
+    std::memset(&fu, 0, sizeof fu);
+    bool num_was_pending = false;
+    if (form) {
+        if (int rc = resolve_pending(ex, den_name))
+            return rc;
+        if (int rc = make_array(ex, p_name, 1, CNH_F64, xshape, false, &p))
+            return rc;
+        if (int rc = new_scalar_array(ex, beta_name, CNH_F64, &beta))
+            return rc;
+        XArray *num = nullptr, *den = nullptr;
+        if (int rc = find_array(ex, num_name, &num, "matvec numerator"))
+            return rc;
+        if (int rc = find_array(ex, den_name, &den, "matvec denominator"))
+            return rc;
+        fu.xa = xa->tiles[0];
+        fu.xb = xb->tiles[0];
+        auto pend = ex->pending.find(num_name);
+        if (pend != ex->pending.end()) {
+            fu.num = pend->second.partials;
+            fu.num_count = pend->second.count;
+            fu.num_folded = num->tiles[0];
+            num_was_pending = true;
+        } else {
+            fu.num = num->tiles[0];
+            fu.num_count = 1;
+        }
+        fu.den = den->tiles[0];
+        fu.quotient_out = beta->tiles[0];
+    }
+    if (int rc = make_array(ex, mv.y_name, 1, CNH_F64, yshape, false, &y))
+        return rc;
+    void* xptr = form ? p->tiles[0] : const_cast<XArray*>(xv)->tiles[0];
+    Ex::PendingSum dot_sums;
+    const int64_t nb = (mv.rows + 63) / 64;
+    if (dot_name != 0) {
+        if (int rc = new_scalar_array(ex, dot_name, CNH_F64, &dot))
+            return rc;
+        if (int rc = pending_buffer(ex, nb, &dot_sums))
+            return rc;
+        fu.w = xptr;
+        fu.dot_partials = dot_sums.partials;
+        fu.dot_capacity = nb;
+    }
+    ex->log("matmul A=" + std::to_string(mv.A->name) + " tiles=" + std::to_string(mv.A->ntiles) + " x=" +
+            std::to_string(mv.x_name) + " out=" + std::to_string(mv.y_name) + " fused" +
+            (form ? " vector=" + std::to_string(xa_name) + "+(" + std::to_string(num_name) + "/" +
+                        std::to_string(den_name) + ")*" + std::to_string(xb_name)
+                  : std::string()) +
+            (dot_name ? " dot=" + std::to_string(dot_name) : std::string()));
+    int rc = 0;
+    if (!ex->dry)
+        rc = cnh_gemv_tiles_fused(mv.rows, mv.cols, mv.A->tile, mv.A->tiles.data(), xptr, y->tiles[0], &fu, nullptr,
+                                  ex->stream);
+    if (rc)
+        return rc;
+    if (num_was_pending)
+        pending_done(ex, num_name);
+    if (dot_name != 0) {
+        ex->pending[dot_name] = dot_sums;
+        if (nb > kDeferMaxPartials)
+            if (int rc2 = resolve_pending(ex, dot_name))
+                return rc2;
+    }
+    for (int name : dels_kept)
+        drop_array(ex, name);
+    ex->stats[2] += (int64_t)(end - i);
+    ex->stats[5]++;
+    *used = end - i;
+    return 0;
+}
+
+// ---- dense statements, the scalars between them and the reductions behind them as one launch ----
+//
+//   alpha = rr / pAp ; x2 = x + alpha * p ; r2 = r - alpha * Ap ; rr2 = r2 @ r2
+// Statements that make new arrays of one shape from whole arrays laid out alike (the no-region fast
+// path, src/execute_node.cpp:1263-1336 upstream), statements on one-element arrays (which upstream
+// runs as kernels of their own, src/executor_core.cpp:390-605) and reductions of the new arrays
+// become ONE group with several roots: a scalar statement is formed in registers by every lane and
+// stored once (CNH_OP_SCALAR_OF), later statements read earlier results from registers, the
+// reductions leave partial sums that wait for their consumer. A run ends before the first statement
+// that needs the value of one of its own reductions. One partition only (a 1-D array up to the
+// minimum tile, an array with a single tile, a rank-3 block).
+constexpr size_t kRunMaxStatements = 8;
+
+int try_dense_run(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t* used, bool* open_ended) {
+    *used = 0;
+    *open_ended = false;
+    struct RunStmt { const DagNode* n; bool scalar; };
+    struct RunRed { const DagNode* n; int op; int a, b; };
+    std::vector<RunStmt> stmts;
+    std::vector<RunRed> reds;
+    std::set<int> vec_results, scal_results, red_results;
+    std::vector<int> deletions, deletions_kept;
+    int32_t shape[3] = {1, 1, 1};
+    int nd = 0;
+    bool reads_pending = false;
+    size_t n_vec = 0, end = i, j = i;
+
+    auto is_deleted = [&](int name) { return std::find(deletions.begin(), deletions.end(), name) != deletions.end(); };
+    // 0: not part of a run; 1: scalar statement; 2: vector statement
+    auto classify = [&](const DagNode& m) -> int {
+        if (!m.fusible || m.roots.empty())
+            return 0;
+        const cnh_ast_node& root = m.nodes[m.roots.back()];
+        const bool arith = root.opcode >= CNH_OP_ADD && root.opcode <= CNH_OP_DIV;
+        if (!(arith || root.opcode == CNH_OP_TANH || root.opcode == CNH_OP_EXP || root.opcode == CNH_OP_COPY) ||
+            root.is_temp || root.dtype != CNH_F64)
+            return 0;
+        std::set<int> own;
+        bool only_arith = true;
+        for (size_t r = 0; r < m.roots.size(); ++r) {
+            const cnh_ast_node& a = m.nodes[m.roots[r]];
+            if ((r + 1 < m.roots.size()) != (a.is_temp != 0) || a.dtype != CNH_F64)
+                return 0;
+            own.insert(a.result_name);
+            only_arith = only_arith && a.opcode >= CNH_OP_ADD && a.opcode <= CNH_OP_DIV;
+        }
+        bool any_vector = false, plain_scalar_operand = false;
+        int32_t shp[3] = {shape[0], shape[1], shape[2]};
+        int rank = nd;
+        for (int32_t ri : m.roots) {
+            const cnh_ast_node& a = m.nodes[ri];
+            for (int oi = 0; oi < a.n_operands; ++oi) {
+                if (a.operands[oi] < 0 || a.operands[oi] >= (int)m.nodes.size())
+                    return 0;
+                const cnh_ast_node& op = m.nodes[a.operands[oi]];
+                if (op.is_scalar)
+                    continue;
+                if (own.count(op.result_name))
+                    continue;                                  // another root of this statement
+                if (op.opcode != CNH_OP_NOOP)
+                    return 0;
+                const int name = op.result_name;
+                if (red_results.count(name) || is_deleted(name))
+                    return 0;
+                if (scal_results.count(name)) {
+                    plain_scalar_operand = plain_scalar_operand || !op.is_broadcast;
+                    continue;
+                }
+                if (vec_results.count(name)) {
+                    if (op.is_broadcast || !operand_is_whole(a, oi, shape, nd))
+                        return 0;
+                    any_vector = true;
+                    continue;
+                }
+                auto it = ex->arrays.find(name);
+                if (it == ex->arrays.end() || it->second.dtype != CNH_F64)
+                    return 0;
+                const XArray& arr = it->second;
+                if (arr.elems == 1) {
+                    plain_scalar_operand = plain_scalar_operand || !op.is_broadcast;
+                    continue;
+                }
+                if (op.is_broadcast)
+                    return 0;
+                if (rank == 0) {
+                    rank = arr.ndims;
+                    for (int d = 0; d < 3; ++d)
+                        shp[d] = d < arr.ndims ? arr.shape[d] : 1;
+                }
+                if (arr.ndims != rank || !laid_out_like_new(ex, arr, rank, shp) || !(arr.flat || arr.ntiles == 1) ||
+                    !operand_is_whole(a, oi, shp, rank))
+                    return 0;
+                any_vector = true;
+            }
+        }
+        if (!any_vector)
+            return only_arith ? 1 : 0;             // exp and tanh of a scalar have no generated form
+        if (plain_scalar_operand || root.ndims != rank)
+            return 0;
+        if (!root.region.is_global) {              // a result region, where given, spells the same shape
+            if (root.region.ndims != rank)
+                return 0;
+            for (int d = 0; d < rank; ++d)
+                if (region_count(root.region, d) != shp[d])
+                    return 0;
+        }
+        nd = rank;
+        for (int d = 0; d < 3; ++d)
+            shape[d] = shp[d];
+        return 2;
+    };
+
+    for (; j < dag.size(); ++j) {
+        const DagNode& m = dag[j];
+        if (m.roots.empty())
+            break;
+        const cnh_ast_node& root = m.nodes[m.roots.back()];
+        if (root.opcode == kOpDelete) {
+            const int name = root.result_name;
+            if (stmts.empty() || vec_results.count(name) || scal_results.count(name) || red_results.count(name))
+                break;
+            deletions.push_back(name);
+            continue;
+        }
+        const bool paired = root.opcode == CNH_OP_REDUCE || root.opcode == kOpSumsqDiff || root.opcode == kOpMaxabsDiff;
+        if (paired || root.opcode == kOpSum) {
+            if (n_vec == 0 || reds.size() >= (size_t)kFoldMaxVectors || m.roots.size() != 1 ||
+                root.n_operands != (paired ? 2 : 1) || root.dtype != CNH_F64 ||
+                (root.opcode == CNH_OP_REDUCE && nd != 1))
+                break;
+            int names[2] = {0, 0};
+            bool ok = true, from_run = false;
+            for (int oi = 0; oi < root.n_operands && ok; ++oi) {
+                const cnh_ast_node& op = m.nodes[root.operands[oi]];
+                ok = op.opcode == CNH_OP_NOOP && !op.is_scalar && !op.is_broadcast && operand_is_whole(root, oi, shape, nd) &&
+                     !is_deleted(op.result_name);
+                names[oi] = op.result_name;
+                if (!ok)
+                    break;
+                if (vec_results.count(op.result_name)) {
+                    from_run = true;
+                } else {
+                    auto it = ex->arrays.find(op.result_name);
+                    ok = it != ex->arrays.end() && it->second.dtype == CNH_F64 && it->second.ndims == nd &&
+                         laid_out_like_new(ex, it->second, nd, shape) && (it->second.flat || it->second.ntiles == 1);
+                }
+            }
+            if (!ok || !from_run)
+                break;
+            reds.push_back({&m, root.opcode, names[0], names[1]});
+            red_results.insert(root.result_name);
+        } else {
+            if (stmts.size() >= kRunMaxStatements)
+                break;
+            const int kind = classify(m);
+            if (kind == 0)
+                break;
+            stmts.push_back({&m, kind == 1});
+            (kind == 1 ? scal_results : vec_results).insert(root.result_name);
+            n_vec += kind == 2;
+            // does it read a value that still stands as partial sums?
+            for (const cnh_ast_node& a : m.nodes)
+                if (a.opcode == CNH_OP_NOOP && !a.is_scalar && ex->pending.count(a.result_name))
+                    reads_pending = true;
+        }
+        end = j + 1;
+        deletions_kept = deletions;
+    }
+    if (j == dag.size() && !stmts.empty() && stmts.size() < kRunMaxStatements && open_ended_allowed(ex)) {
+        *open_ended = true;            // the run may go on in the next message
+        return 0;
+    }
+    if (n_vec == 0 || !(stmts.size() >= 2 || reads_pending))
+        return 0;
+    // ---- the run as one group ----
+    DagNode merged;
+    merged.id = dag[i].id;
+    merged.fusible = 1;
+    std::map<int, int> produced;                 // result name -> node of `merged` that holds the value
+    int next_literal = -1, next_temporary = 0x7d000000;
+    auto whole = [](cnh_region& r) {
+        std::memset(&r, 0, sizeof r);
+        r.is_global = 1;
+    };
+    for (const RunStmt& st : stmts) {
+        const DagNode& n = *st.n;
+        const int base = (int)merged.nodes.size();
+        for (const cnh_ast_node& a : n.nodes) {
+            merged.nodes.push_back(a);
+            cnh_ast_node& c = merged.nodes.back();
+            for (int oi = 0; oi < c.n_operands; ++oi)
+                if (c.operands[oi] >= 0)
+                    c.operands[oi] += base;
+            if (c.is_scalar)
+                c.result_name = next_literal--;
+        }
+        std::map<int, int> renamed;
+        for (size_t ri = 0; ri + 1 < n.roots.size(); ++ri)
+            renamed[n.nodes[(size_t)n.roots[ri]].result_name] = next_temporary++;
+        for (size_t q = (size_t)base; q < merged.nodes.size(); ++q) {
+            cnh_ast_node& c = merged.nodes[q];
+            if (c.is_scalar)
+                continue;
+            auto it = renamed.find(c.result_name);
+            if (it != renamed.end())
+                c.result_name = it->second;
+        }
+        for (size_t q = (size_t)base; q < merged.nodes.size(); ++q) {
+            cnh_ast_node& c = merged.nodes[q];
+            if (c.is_scalar || c.opcode == CNH_OP_NOOP)
+                continue;
+            for (int oi = 0; oi < c.n_operands; ++oi) {
+                if (c.operands[oi] < 0)
+                    continue;
+                const cnh_ast_node& op = merged.nodes[(size_t)c.operands[oi]];
+                if (op.is_scalar || op.opcode != CNH_OP_NOOP)
+                    continue;
+                auto pr = produced.find(op.result_name);
+                if (pr != produced.end()) {      // made earlier in this launch: the value is in registers
+                    c.operands[oi] = pr->second;
+                    c.has_operand_region[oi] = 0;
+                    whole(c.operand_regions[oi]);
+                }
+            }
+        }
+        // one-element arrays are kernel scalars here
+        for (size_t q = (size_t)base; q < merged.nodes.size(); ++q) {
+            cnh_ast_node& c = merged.nodes[q];
+            if (c.opcode != CNH_OP_NOOP || c.is_scalar || c.is_broadcast)
+                continue;
+            auto it = ex->arrays.find(c.result_name);
+            if (it != ex->arrays.end() && it->second.elems == 1)
+                c.is_broadcast = 1;
+        }
+        for (int32_t r : n.roots)
+            merged.roots.push_back(base + r);
+        const int last = base + n.roots.back();
+        const int actual = merged.nodes[(size_t)last].result_name;
+        produced[actual] = last;
+        if (st.scalar) {
+            merged.nodes[(size_t)last].is_temp = 1;
+            merged.nodes[(size_t)last].result_name = next_temporary++;
+            cnh_ast_node once;
+            std::memset(&once, 0, sizeof once);
+            once.result_name = actual;
+            once.opcode = CNH_OP_SCALAR_OF;
+            once.ndims = nd;
+            once.dtype = CNH_F64;
+            once.n_operands = 1;
+            once.operands[0] = last;
+            once.operands[1] = -1;
+            whole(once.region);
+            whole(once.operand_regions[0]);
+            whole(once.operand_regions[1]);
+            merged.nodes.push_back(once);
+            merged.roots.push_back((int)merged.nodes.size() - 1);
+        }
+    }
+    auto value_of = [&](int name) {
+        auto pr = produced.find(name);
+        if (pr != produced.end())
+            return pr->second;
+        for (size_t q = 0; q < merged.nodes.size(); ++q)
+            if (merged.nodes[q].opcode == CNH_OP_NOOP && !merged.nodes[q].is_scalar && !merged.nodes[q].is_broadcast &&
+                merged.nodes[q].result_name == name)
+                return (int)q;
+        cnh_ast_node leaf;
+        std::memset(&leaf, 0, sizeof leaf);
+        leaf.result_name = name;
+        leaf.opcode = CNH_OP_NOOP;
+        leaf.ndims = nd;
+        leaf.dtype = CNH_F64;
+        whole(leaf.region);
+        whole(leaf.operand_regions[0]);
+        whole(leaf.operand_regions[1]);
+        merged.nodes.push_back(leaf);
+        return (int)merged.nodes.size() - 1;
+    };
+    auto add_root = [&](int name, int opcode, bool is_temp, int a, int b) {
+        cnh_ast_node r;
+        std::memset(&r, 0, sizeof r);
+        r.result_name = name;
+        r.opcode = opcode;
+        r.is_temp = is_temp;
+        r.ndims = nd;
+        r.dtype = CNH_F64;
+        r.n_operands = b >= 0 ? 2 : 1;
+        r.operands[0] = a;
+        r.operands[1] = b;
+        whole(r.region);
+        whole(r.operand_regions[0]);
+        whole(r.operand_regions[1]);
+        merged.nodes.push_back(r);
+        merged.roots.push_back((int)merged.nodes.size() - 1);
+        return (int)merged.nodes.size() - 1;
+    };
+    std::map<int, bool> red_is_sum;
+    for (const RunRed& rd : reds) {
+        const int out_name = rd.n->nodes[rd.n->roots.back()].result_name;
+        const int a = value_of(rd.a);
+        red_is_sum[out_name] = rd.op != kOpMaxabsDiff;
+        if (rd.op == kOpSum) {
+            add_root(out_name, CNH_OP_SUM_OF, false, a, -1);
+            continue;
+        }
+        const int b = value_of(rd.b);
+        if (rd.op == CNH_OP_REDUCE) {
+            const int t = add_root(next_temporary++, CNH_OP_MUL, true, a, b);
+            add_root(out_name, CNH_OP_SUM_OF, false, t, -1);
+        } else {
+            const int d = add_root(next_temporary++, CNH_OP_SUB, true, a, b);
+            if (rd.op == kOpSumsqDiff) {
+                const int t = add_root(next_temporary++, CNH_OP_MUL, true, d, d);
+                add_root(out_name, CNH_OP_SUM_OF, false, t, -1);
+            } else {
+                add_root(out_name, CNH_OP_MAXABS_OF, false, d, -1);
+            }
+        }
+    }
+    merged.nodes[(size_t)merged.roots.back()].ndims = nd;
+
+    Group g;
+    canonicalise(merged, g);
+    cnh_kernel* k = nullptr;
+    if (int rc = compile_cached(ex, g, &k))
+        return rc;
+    int n_in = 0, n_scalar = 0, n_out = 0;
+    if (int rc = cnh_kernel_signature(k, &n_in, &n_scalar, &n_out))
+        return rc;
+    int64_t elems = 1;
+    for (int d = 0; d < nd; ++d)
+        elems *= shape[d];
+    std::vector<cnh_memref> in((size_t)std::max(1, n_in)), out((size_t)std::max(1, n_out));
+    for (int q = 0; q < n_in; ++q) {
+        int cname = 0, has = 0;
+        cnh_region reg;
+        if (int rc = cnh_kernel_input(k, q, &cname, &has, &reg))
+            return rc;
+        XArray* a;
+        if (int rc = find_array(ex, g.canon_to_actual[cname], &a, "group input"))
+            return rc;
+        CNH_CHECK(a->elems == elems && (a->flat || a->ntiles == 1), -26, "node %d: operand %d is laid out differently",
+                  merged.id, a->name);
+        in[(size_t)q] = dense_memref_of(a->flat ? a->slab : a->tiles[0], nd, shape);
+    }
+    std::vector<cnh_scalar_sum> sums((size_t)std::max(1, n_scalar));
+    std::vector<const void*> scalar_ptrs((size_t)std::max(1, n_scalar), nullptr);
+    std::vector<int> taken;                    // pending sums this launch folds and stores
+    for (int q = 0; q < n_scalar; ++q) {
+        int cname = 0;
+        if (int rc = cnh_kernel_scalar(k, q, &cname))
+            return rc;
+        XArray* sarr;
+        if (int rc = find_array(ex, g.canon_to_actual[cname], &sarr, "kernel scalar"))
+            return rc;
+        CNH_CHECK(sarr->elems == 1 && sarr->dtype == CNH_F64, -27, "node %d: kernel scalar %d", merged.id, sarr->name);
+        auto pend = ex->pending.find(sarr->name);
+        if (pend != ex->pending.end()) {
+            sums[(size_t)q] = cnh_scalar_sum{pend->second.partials, pend->second.count, sarr->tiles[0]};
+            taken.push_back(sarr->name);
+        } else {
+            sums[(size_t)q] = cnh_scalar_sum{sarr->tiles[0], 1, nullptr};
+        }
+        scalar_ptrs[(size_t)q] = sarr->tiles[0];
+    }
+    // a launch that reduces, or that sums partials on the way in, runs 256 lanes a workgroup and
+    // leaves one partial per workgroup: per 512 elements
+    const int64_t nslots = (elems + 511) / 512;
+    std::map<int, Ex::PendingSum> left;
+    const int32_t one[3] = {1, 1, 1};
+    std::string out_names;
+    for (int q = 0; q < n_out; ++q) {
+        int rname = 0, tname = 0, is_set = 0;
+        cnh_region reg;
+        if (int rc = cnh_kernel_output(k, q, &rname, &tname, &is_set, &reg))
+            return rc;
+        const int actual = g.canon_to_actual[rname];
+        XArray* o = nullptr;
+        if (vec_results.count(actual)) {
+            if (int rc = make_array(ex, actual, nd, CNH_F64, shape, false, &o))
+                return rc;
+            CNH_CHECK(o->flat || o->ntiles == 1, -26, "node %d: result %d has several tiles", merged.id, actual);
+            out[(size_t)q] = dense_memref_of(o->flat ? o->slab : o->tiles[0], nd, shape);
+            out_names += (out_names.empty() ? "" : ",") + std::to_string(actual);
+            continue;
+        }
+        if (int rc = new_scalar_array(ex, actual, CNH_F64, &o))
+            return rc;
+        out[(size_t)q] = dense_memref_of(o->tiles[0], nd, one);
+        if (red_results.count(actual) && red_is_sum[actual] && nslots > 1 && nslots <= kDeferMaxPartials) {
+            Ex::PendingSum ps;
+            if (int rc = pending_buffer(ex, nslots, &ps))
+                return rc;
+            int32_t room[3] = {1, 1, 1};
+            room[nd - 1] = (int32_t)nslots;
+            out[(size_t)q] = dense_memref_of(ps.partials, nd, room);
+            left[actual] = ps;
+        }
+    }
+    ex->stats[5]++;
+    ex->log("group node=" + std::to_string(merged.id) + " path=run statements=" + std::to_string(stmts.size()) +
+            " scalars_formed=" + std::to_string(scal_results.size()) + " reductions=" + std::to_string(reds.size()) +
+            " inputs=" + std::to_string(n_in) + " scalars=" + std::to_string(n_scalar) + " sums_taken=" +
+            std::to_string(taken.size()) + " out=" + out_names);
+    int rc = 0;
+    if (!ex->dry) {
+        if (!taken.empty())
+            rc = cnh_launch_group_sums(k, nd, n_in, in.data(), n_scalar, sums.data(), n_out, out.data(), ex->stream);
+        else
+            rc = cnh_launch_group(k, nd, n_in, in.data(), n_scalar, scalar_ptrs.data(), 1, n_out, out.data(),
+                                  ex->stream);
+    }
+    if (rc)
+        return rc;
+    for (int name : taken)
+        pending_done(ex, name);
+    for (auto& kv : left)
+        ex->pending[kv.first] = kv.second;
+    for (int name : deletions_kept)
+        drop_array(ex, name);
+    ex->stats[2] += (int64_t)(end - i);
+    *used = end - i;
+    return 0;
+}
+
 int parse_dag(const char* msg, int64_t size, std::vector<DagNode>& out) {
     Reader r{msg, msg + size};
     int32_t magic = r.get<int32_t>(), version = r.get<int32_t>(), count = r.get<int32_t>();
@@ -2641,9 +3424,23 @@ int run_nodes(Ex* ex, std::vector<DagNode>& dag) {
     int rc = 0;
     for (size_t i = 0; i < dag.size() && rc == 0;) {
         size_t used = 0;
+        // a deletion needs no value: a pending sum nobody read goes with its array
+        if (!dag[i].roots.empty() && dag[i].nodes[dag[i].roots.back()].opcode == kOpDelete) {
+            rc = exec_node(ex, dag[i]);
+            ++i;
+            continue;
+        }
         if (ex->fuse_on && !ex->solver_on) {
             bool open_ended = false;
-            rc = try_product_into_region(ex, dag, i, &used, &open_ended);
+            // the two rewrites that know about pending sums go first ...
+            rc = try_fused_matvec(ex, dag, i, &used, &open_ended);
+            if (rc == 0 && used == 0 && !open_ended)
+                rc = try_dense_run(ex, dag, i, &used, &open_ended);
+            // ... everything else reads arrays as they are
+            if (rc == 0 && used == 0 && !open_ended)
+                rc = resolve_all(ex);
+            if (rc == 0 && used == 0 && !open_ended)
+                rc = try_product_into_region(ex, dag, i, &used, &open_ended);
             if (rc == 0 && used == 0 && !open_ended)
                 rc = try_statement_run(ex, dag, i, &used, &open_ended);
             if (rc == 0 && used == 0 && !open_ended)
@@ -2654,12 +3451,17 @@ int run_nodes(Ex* ex, std::vector<DagNode>& dag) {
             }
         }
         if (rc == 0 && used == 0) {
-            rc = exec_node(ex, dag[i]);
+            rc = resolve_all(ex);
+            if (rc == 0)
+                rc = exec_node(ex, dag[i]);
             used = 1;
         }
         i += used;
     }
     ex->planned.clear();
+    // sums may stay pending only while nodes are held: their consumer may be among what follows
+    if (rc == 0 && ex->held.empty())
+        rc = resolve_all(ex);
     return rc;
 }
 
@@ -2792,7 +3594,9 @@ int settle(Ex* ex) {
         return rc;
     if (int rc = finish_log(ex))
         return rc;
-    return flush_held(ex);
+    if (int rc = flush_held(ex))
+        return rc;
+    return resolve_all(ex);
 }
 
 void stop_worker(Ex* ex) {
@@ -2841,6 +3645,8 @@ int cnx_destroy(cnx_executor* ex) {
             if (kv.second.alt)
                 cnh_free(kv.second.alt);
         }
+        for (auto& kv : ex->pending)
+            cnh_free(kv.second.partials);
         for (auto& kv : ex->free_list)
             for (void* p : kv.second)
                 cnh_free(p);

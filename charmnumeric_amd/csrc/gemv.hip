@@ -149,12 +149,14 @@ struct GemvFuse {
     double* num_folded;
     const double* w;
     double* dot_partials;
+    double* x_out;          // where the formed vector is stored (the launch's x)
+    double* quotient_out;   // receives S / den when not null
 };
 
 template <typename T, int kWaves, int kRows, int kUnroll, bool FUSED = false>
 __global__ __launch_bounds__(kWaves * 64) void gemv_rows_xlds(const ColTile* __restrict__ tiles, int ncol_tiles,
                                                               int64_t tile_rows, int64_t rows, int64_t row_shift,
-                                                              const T* __restrict__ x, T* __restrict__ y,
+                                                              const T* x, T* __restrict__ y,
                                                               int beta, GemvFuse f = GemvFuse()) {
     typedef typename Acc<T>::type A;
     constexpr int VEC = 16 / sizeof(T);
@@ -184,10 +186,13 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_rows_xlds(const ColTile* __r
         }
         __syncthreads();
         factor = fuse_lds[kWaves] / f.den[0];
+        if (blockIdx.x == 0 && threadIdx.x == 0 && f.quotient_out != nullptr)
+            *f.quotient_out = factor;
     }
-    // the elements of the vector this workgroup stores when it forms the vector itself
-    const int64_t own_per = FUSED ? (rows + gridDim.x - 1) / gridDim.x : 0;
-    const int64_t own_lo = own_per * blockIdx.x, own_hi = own_lo + own_per;
+    // The elements of the vector this workgroup stores when it forms the vector itself: those with
+    // the indices of its own rows (the matrix is square), which are also the only elements of w it
+    // reads for the dot at the end, so w may be the vector being formed.
+    const int64_t own_lo = (int64_t)blockIdx.x * kWaves * kRows, own_hi = own_lo + kWaves * kRows;
     for (int tj = 0; tj < ncol_tiles; ++tj) {
         const int64_t ncols = tiles[tj].ncols, xoff = tiles[tj].xoff;
         if (tj > 0)
@@ -205,16 +210,16 @@ __global__ __launch_bounds__(kWaves * 64) void gemv_rows_xlds(const ColTile* __r
                 *reinterpret_cast<double2*>(reinterpret_cast<double*>(xs) + i) = v;
                 const int64_t g = xoff + i;
                 if (g >= own_lo && g < own_hi)
-                    const_cast<T*>(x)[g] = (T)v.x;
+                    f.x_out[g] = v.x;
                 if (g + 1 >= own_lo && g + 1 < own_hi)
-                    const_cast<T*>(x)[g + 1] = (T)v.y;
+                    f.x_out[g + 1] = v.y;
             }
             if ((ncols & 1) && threadIdx.x == 0) {
                 const int64_t i = ncols - 1, g = xoff + i;
                 const double v = f.xa[g] + factor * f.xb[g];
                 reinterpret_cast<double*>(xs)[i] = v;
                 if (g >= own_lo && g < own_hi)
-                    const_cast<T*>(x)[g] = (T)v;
+                    f.x_out[g] = v;
             }
         } else {
         for (int64_t i = (int64_t)threadIdx.x * VEC; i + VEC <= ncols; i += (int64_t)kWaves * 64 * VEC)
@@ -434,6 +439,15 @@ int cnh_gemv_tiles_fused(int64_t rows, int64_t cols, int32_t tile, const void* c
               "cnh_gemv_tiles_fused: the vector's parts are incomplete");
     CNH_CHECK(!form_x || (rows == cols && x != fu->xa && x != fu->xb), -2,
               "cnh_gemv_tiles_fused: a vector formed on the way needs a square matrix and a buffer of its own");
+    {
+        // y is written while x, xa, xb and w are still being read by other workgroups
+        auto overlaps = [&](const void* q, int64_t n) {
+            const char *a = static_cast<const char*>(y), *b = static_cast<const char*>(q);
+            return q != nullptr && a < b + n * 8 && b < a + rows * 8;
+        };
+        CNH_CHECK(!overlaps(x, cols) && !overlaps(fu->xa, cols) && !overlaps(fu->xb, cols) && !overlaps(fu->w, rows),
+                  -2, "cnh_gemv_tiles_fused: y overlaps one of the vectors the launch reads");
+    }
     CNH_CHECK(fu->w == nullptr || fu->dot_partials != nullptr, -2, "cnh_gemv_tiles_fused: no room for the partial sums");
     int64_t gr = (rows + tile - 1) / tile, gc = (cols + tile - 1) / tile;
     std::vector<ColTile> tiles((size_t)(gr * gc));
@@ -466,6 +480,8 @@ int cnh_gemv_tiles_fused(int64_t rows, int64_t cols, int32_t tile, const void* c
     f.num_folded = (double*)fu->num_folded;
     f.w = (const double*)fu->w;
     f.dot_partials = (double*)fu->dot_partials;
+    f.x_out = (double*)x;
+    f.quotient_out = form_x ? (double*)fu->quotient_out : nullptr;
     hipLaunchKernelGGL((gemv_rows_xlds<double, kW, kR, 4, true>), dim3((unsigned)nb), dim3(kW * 64), 0, st,
                        (const ColTile*)dtiles, (int)gc, (int64_t)tile, rows, (int64_t)0, (const double*)x,
                        (double*)y, 0, f);

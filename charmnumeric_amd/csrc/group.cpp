@@ -450,7 +450,8 @@ int launch_group_impl(cnh_kernel* k, int ndims, int n_parts, int n_in, const cnh
     // Outputs that are reduced over the launch (CNH_OP_SUM_OF / CNH_OP_MAXABS_OF roots): their
     // memref names the one element the result goes to (partition 0's counts); `e0` is the first
     // output that is stored element by element, whose extents every other memref must match.
-    const int n_red = p.reductions();
+    const int n_red = p.folds();
+    auto folds = [&](int o) { return p.out_reduce[(size_t)o] == 1 || p.out_reduce[(size_t)o] == 2; };
     int e0 = -1;
     for (int o = 0; o < n_out; ++o)
         if (!p.out_reduce[(size_t)o]) {
@@ -545,7 +546,7 @@ int launch_group_impl(cnh_kernel* k, int ndims, int n_parts, int n_in, const cnh
             const cnh_memref* po = out + (size_t)live[0] * n_out;
             int kept = 0, q = 0;
             for (int o = 0; o < n_out; ++o)
-                if (p.out_reduce[(size_t)o]) {
+                if (folds(o)) {
                     int64_t room = 1;
                     for (int d = 0; d < ndims; ++d)
                         room *= po[o].sizes[d];
@@ -564,7 +565,7 @@ int launch_group_impl(cnh_kernel* k, int ndims, int n_parts, int n_in, const cnh
                     return rc;
                 q = 0;
                 for (int o = 0; o < n_out; ++o)
-                    if (p.out_reduce[(size_t)o]) {
+                    if (folds(o)) {
                         if (red_slots[q] == nullptr) {
                             red_slots[q] = static_cast<double*>(ws) + stride * n_fold;
                             maximum[n_fold] = p.out_reduce[(size_t)o] == 2;
@@ -613,7 +614,7 @@ int launch_group_impl(cnh_kernel* k, int ndims, int n_parts, int n_in, const cnh
         return reduce_slots_f64_many(n_fold, maximum, fold_vec, nslots, fold_out, st);
     }
     CNH_CHECK(sums == nullptr, -28, "summed scalars need dense, equally laid out operands");
-    CNH_CHECK(n_red == 0, -28, "a group with reducing roots needs dense, equally laid out operands");
+    CNH_CHECK(p.reductions() == 0, -28, "a group with reducing or scalar roots needs dense, equally laid out operands");
 
     // Strided cells.
     const size_t cell_words = 5 + NLA + 3 * NLA + NOA + 3 * NOA;

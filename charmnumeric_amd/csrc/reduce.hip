@@ -452,6 +452,24 @@ __global__ __launch_bounds__(1024) void fold_many(int64_t first, int64_t count, 
     if (threadIdx.x == 0)
         *f.out[q] = v;
 }
+
+// The sum of n partial results in the order a group launch uses when it is handed them as a summed
+// scalar (cnh_launch_group_sums): 256 lanes take running sums a lane stride apart, a butterfly
+// combines the lanes of each wavefront, the four wavefronts are added left to right.
+__global__ __launch_bounds__(256) void fold_sums_f64(const double* __restrict__ p, int n, double* __restrict__ out) {
+    __shared__ double part[4];
+    double v = 0;
+    for (int j = threadIdx.x; j < n; j += 256)
+        v += p[j];
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1)
+        v += __shfl_xor(v, m, 64);
+    if ((threadIdx.x & 63) == 0)
+        part[threadIdx.x >> 6] = v;
+    __syncthreads();
+    if (threadIdx.x == 0)
+        *out = ((part[0] + part[1]) + part[2]) + part[3];
+}
 } // namespace
 
 namespace cnh {
@@ -585,6 +603,16 @@ int cnh_reduce_final(int dtype, int n_partials, const void* partials, void* out,
         break;
     default: return set_error(-2, "unknown dtype %d", dtype);
     }
+    CNH_HIP(hipGetLastError());
+    return 0;
+}
+
+int cnh_fold_sums(const void* partials, int64_t count, void* out, cnh_stream s) {
+    if (int rc = ensure_init())
+        return rc;
+    CNH_CHECK(partials && out && count >= 1 && count <= (1 << 20), -2, "cnh_fold_sums: bad arguments");
+    hipLaunchKernelGGL(fold_sums_f64, dim3(1), dim3(256), 0, as_stream(s), (const double*)partials, (int)count,
+                       (double*)out);
     CNH_HIP(hipGetLastError());
     return 0;
 }

@@ -36,7 +36,13 @@ enum {
      * element of the launch instead of storing it (sum, or the largest absolute value). Upstream
      * runs a reduction as a pass of its own over the stored array (src/executor_reduce.cpp:8-119);
      * as a root of the group that produces the values it costs no second read. */
-    CNH_OP_SUM_OF = 20, CNH_OP_MAXABS_OF = 21
+    CNH_OP_SUM_OF = 20, CNH_OP_MAXABS_OF = 21,
+    /* Extension, no upstream counterpart: an output root whose operand is formed from the launch's
+     * scalars alone (alpha = r.r / p.Ap next to the updates that use it). Upstream runs such a
+     * statement as a group of its own over one-element arrays (src/jit.cpp:329-333,
+     * src/executor_core.cpp:390-605); here the first lane of the launch stores the value once, at
+     * element 0 of the output's memref. Dense launches only. */
+    CNH_OP_SCALAR_OF = 22
 };
 enum { CNH_F32 = 0, CNH_F64 = 1, CNH_I32 = 2, CNH_I64 = 3 };
 
@@ -246,6 +252,10 @@ typedef struct cnh_scalar_sum {
 } cnh_scalar_sum;
 int cnh_launch_group_sums(cnh_kernel* k, int ndims, int n_in, const cnh_memref* in, int n_scalar,
                           const cnh_scalar_sum* scalars, int n_out, const cnh_memref* out, cnh_stream s);
+/* *out (device, fp64) = the sum of `count` partial results at `partials`, added in exactly the order a
+ * launch uses that takes them as a summed scalar: for the caller that needs the value with no such
+ * launch at hand. 1 <= count <= 2^20. */
+int cnh_fold_sums(const void* partials, int64_t count, void* out, cnh_stream s);
 
 /* Shifted-slice groups over tiles that all live on this device: replaces send_remote_input +
  * receive_data + align_fragments + M kernel calls + the SET_REGION copy
@@ -345,9 +355,13 @@ int cnh_gemv_tiles(int dtype, int64_t rows, int64_t cols, int32_t tile, const vo
  *    vector (a buffer of its own, every element stored once) and *num_folded receives S if not
  *    null. CG: p = r + (r.r_new / r.r_old) p with r.r_new left as partial sums by the launch that
  *    updated r. Needs a square matrix.
+ *    *quotient_out receives S / den if not null (CG: beta).
  *  - w != NULL: dot_partials[b] = sum of w[r] * y[r] over the rows of workgroup b (64 rows each, in
  *    row order), b < *n_partials <= dot_capacity; their sum in index order is w . y (CG: p . Ap),
- *    which cnh_launch_group_sums hands to the next launch.
+ *    which cnh_launch_group_sums hands to the next launch. w may be x, also when x is formed on the
+ *    way: a workgroup reads w at the indices of its own rows only, and those are the elements of x it
+ *    stores itself.
+ * y must not overlap x, xa, xb or w (-2).
  * Applies to products of 16384 rows or more with even column tiles of at most 8192 columns and
  * 16-byte aligned operands (-3 otherwise: use cnh_gemv_tiles and the separate calls). y has the
  * bits cnh_gemv_tiles gives for the same x. */
@@ -361,6 +375,7 @@ typedef struct cnh_gemv_fusion {
     const void* w;
     void* dot_partials;
     int64_t dot_capacity;
+    void* quotient_out;
 } cnh_gemv_fusion;
 int cnh_gemv_tiles_fused(int64_t rows, int64_t cols, int32_t tile, const void* const* tiles, void* x, void* y,
                          const cnh_gemv_fusion* fusion, int64_t* n_partials, cnh_stream s);

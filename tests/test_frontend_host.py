@@ -161,8 +161,14 @@ def test_live_intermediate_is_materialised_and_splits_the_group(itf):
     u = t * 2.0
     cnp.execute(itf)
     g = lines(itf, "group")
-    assert len(g) == 2
+    # two DAG nodes (t is an array of its own); the executor runs them as one launch that stores both
+    assert len(g) == 1 and "path=run statements=2" in g[0]
     assert itf.array_info(t.name)["shape"] == (64,) and itf.array_info(u.name)["shape"] == (64,)
+    itf.set_fusion(False)
+    v = a + 3.0
+    w = v * 2.0
+    cnp.execute(itf)
+    assert len(lines(itf, "group")) == 2
 
 
 def test_unused_results_are_dropped(itf):
@@ -230,11 +236,70 @@ def test_cg_iteration_compiles_once_and_reuses_buffers(itf):
     assert st["reuses"] > 0 and st["live_arrays"] <= 12
     tr = itf.trace()
     assert sum(ln.startswith("matmul") for ln in tr) == 4
-    # p.Ap follows a product and runs on its own; r.r rides on the launch that updates r
-    assert sum(ln.startswith("reduce") for ln in tr) == 1 + 4
-    assert sum("path=dense+reduce" in ln and "reductions=1" in ln for ln in tr) == 4
-    scal = [ln for ln in tr if ln.startswith("group") and "scalars=1" in ln]
-    assert len(scal) == 3 * 4                                 # x, r, p updates take alpha/beta from the device
+    # p.Ap follows a product and runs on its own (the matrix is too small for the fused matvec)
+    assert sum(ln.startswith("reduce") for ln in tr) == 4
+    # alpha, x, r and r.r are one launch, beta and p another (and the two copies of b with the
+    # first r.r ahead of the loop a third kind)
+    runs = [ln for ln in tr if "path=run" in ln]
+    assert len(runs) == 1 + 2 * 4 and "statements=2 scalars_formed=0 reductions=1" in runs[0]
+    assert sum("statements=3 scalars_formed=1 reductions=1" in ln for ln in runs) == 4
+    assert sum("statements=2 scalars_formed=1 reductions=0" in ln for ln in runs) == 4
+
+
+def test_a_cg_iteration_on_a_large_system_is_two_launches(itf):
+    """examples/cg.py:40-52 upstream at n = 16384: the matvec takes the p update before it and the
+    dot behind it along, the x and r updates form alpha in registers from the dot's partial sums and
+    leave those of r.r. Partial sums are folded by the launch that reads them; a value somebody
+    else asks for gets a fold of its own."""
+    n = 16384
+    A = cnp.zeros((n, n))
+    b = cnp.ones((n,))
+    x = cnp.zeros((n,))
+    r = b.copy()
+    p = b.copy()
+    rtr = r @ r
+    cnp.execute(itf)
+    itf.trace()
+    for k in range(3):
+        Ap = A @ p
+        pAp = p @ Ap
+        alpha = rtr / pAp
+        x = x + alpha * p
+        r = r - alpha * Ap
+        rtr_new = r @ r
+        beta = rtr_new / rtr
+        p = r + beta * p
+        rtr = rtr_new
+    cnp.execute(itf)
+    tr = [ln for ln in itf.trace() if not ln.startswith(("create", "delete"))]
+    assert len(tr) == 2 * 3 + 1, tr
+    assert tr[0].startswith("matmul") and "fused dot=" in tr[0] and "vector=" not in tr[0]
+    for k in (1, 2):
+        assert tr[2 * k].startswith("matmul") and "fused vector=" in tr[2 * k] and "dot=" in tr[2 * k]
+    for k in range(3):
+        assert "path=run statements=3 scalars_formed=1 reductions=1" in tr[2 * k + 1] and "sums_taken=1" in tr[2 * k + 1]
+    # the program ends: beta and p of the last iteration are a launch of their own
+    assert "path=run statements=2 scalars_formed=1 reductions=0" in tr[6] and "sums_taken=1" in tr[6]
+    assert not any(ln.startswith("fold") for ln in tr)
+    st = itf.stats()
+    assert st["live_arrays"] <= 12
+    # a value that is read back while it stands as partial sums is folded first
+    Ap = A @ p
+    pAp = p @ Ap
+    cnp.execute(itf)
+    info = itf.array_info(pAp.name)
+    assert info["shape"] == (1,)
+    tr = [ln for ln in itf.trace() if not ln.startswith(("create", "delete"))]
+    assert len(tr) == 2 and tr[0].startswith("matmul") and tr[1].startswith("fold") and "partials=256" in tr[1]
+    # switched off: node by node
+    itf.set_fusion(False)
+    Ap = A @ p
+    pAp = p @ Ap
+    alpha = rtr / pAp
+    x = x + alpha * p
+    cnp.execute(itf)
+    tr = [ln for ln in itf.trace() if not ln.startswith(("create", "delete"))]
+    assert [ln.split()[0] for ln in tr] == ["matmul", "reduce", "group", "group"] and "fused" not in tr[0]
 
 
 def test_tile_rule_and_minimum_tile_override(itf):

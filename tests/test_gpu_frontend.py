@@ -715,3 +715,118 @@ def test_code_objects_from_the_disk_cache_run(tmp_path):
     assert int(first[0]) >= 1 and first[1] == "0"
     assert second[0] == first[0] and second[1] == first[0]       # every code object came from disk
     assert second[2] == first[2]
+
+
+# ---- dense statements, scalar statements and reductions as one launch; partial sums that wait ----
+
+@pytest.mark.parametrize("fusion", [True, False], ids=["merged", "node-by-node"])
+@pytest.mark.parametrize("shape", [(300,), (2000,), (5000,), (40, 50), (12, 20, 30)])
+def test_vector_updates_with_the_scalars_between_them(itf, fusion, shape, rank3_layout):
+    """alpha = s / t; x2 = x + alpha p; r2 = r - alpha q; rr = sum-type reductions of r2; beta = rr / s;
+    p2 = r2 + beta p: element-wise results and the scalars formed from stored values are NumPy's bit
+    for bit whichever way the nodes are launched; values that depend on a reduction agree to the
+    order of summation."""
+    itf.set_fusion(fusion)
+    rng = np.random.default_rng(sum(shape))
+    hx, hp, hq, hr = (rng.standard_normal(shape) for _ in range(4))
+    x, p, q, r = cnp.array(hx), cnp.array(hp), cnp.array(hq), cnp.array(hr)
+    s, t = cnp.array(np.array([1.75])), cnp.array(np.array([-0.6]))
+    x.get(itf)
+    itf.set_trace()
+    alpha = s / t
+    x2 = x + alpha * p
+    r2 = r - alpha * q
+    rr = cnp.sum(r2 * r2) if len(shape) > 1 else r2 @ r2
+    top = cnp.maxabs_diff(r2, r)
+    beta = rr / s
+    p2 = r2 + beta * p
+    gamma = beta * alpha + 1.0
+    ha = np.float64(1.75) / np.float64(-0.6)
+    assert alpha.get(itf).item() == ha
+    assert np.array_equal(x2.get(itf), hx + ha * hp)
+    hr2 = hr - ha * hq
+    assert np.array_equal(r2.get(itf), hr2)
+    assert top.get(itf).item() == np.max(np.abs(hr2 - hr))
+    grr = rr.get(itf).item()
+    assert abs(grr - np.sum(hr2 * hr2)) <= 1e-13 * np.sum(hr2 * hr2)
+    gb = beta.get(itf).item()
+    assert gb == grr / 1.75                                   # from the stored sum: one IEEE division
+    assert np.array_equal(p2.get(itf), hr2 + gb * hp)
+    assert gamma.get(itf).item() == gb * ha + 1.0
+    runs = [ln for ln in itf.trace() if "path=run" in ln]
+    planning = os.environ.get("CHARMNUMERIC_SOLVER", "0") not in ("", "0")
+    if fusion and not planning:
+        assert len(runs) == 2 and "scalars_formed=1" in runs[0] and "scalars_formed=2" in runs[1]
+        if len(shape) == 1:
+            assert "statements=3 scalars_formed=1 reductions=2" in runs[0]
+            assert ("sums_taken=1" in runs[1]) == (int(np.prod(shape)) > 512)
+    if not fusion:
+        assert not runs
+
+
+def test_a_pending_sum_is_folded_for_whoever_else_reads_it(itf):
+    """r.r left as partial sums by the launch that made r: read back, used by a statement on a
+    slice, used as an operand of a product-free reduction. Same values as node by node."""
+    n = 3000
+    rng = np.random.default_rng(4)
+    hr, hq = rng.standard_normal(n), rng.standard_normal(n)
+
+    def program():
+        r, q = cnp.array(hr), cnp.array(hq)
+        r2 = r - 0.5 * q
+        w = r2 * 2.0
+        rr = r2 @ r2
+        y = cnp.zeros((8,))
+        y[0:3] = q[0:3] * rr                   # a statement run reads it as a kernel scalar
+        z = w + rr                             # a dense statement reads it: folded on the way in
+        return rr.get(itf).item(), y.get(itf), z.get(itf)
+
+    itf.set_fusion(True)
+    itf.set_trace()
+    a = program()
+    tr = itf.trace()
+    assert any("path=run" in ln and "reductions=1" in ln for ln in tr)
+    assert any(ln.startswith("fold") and "partials=6" in ln for ln in tr)
+    itf.set_fusion(False)
+    b = program()
+    hr2 = hr - 0.5 * hq
+    assert abs(a[0] - np.sum(hr2 * hr2)) <= 1e-13 * np.sum(hr2 * hr2)
+    assert abs(a[0] - b[0]) <= 1e-13 * abs(b[0])
+    for got in (a, b):
+        want_y = np.zeros(8)
+        want_y[0:3] = hq[0:3] * got[0]
+        assert np.array_equal(got[1], want_y)
+        assert np.array_equal(got[2], hr2 * 2.0 + got[0])
+
+
+def test_cg_on_a_small_system_with_merged_launches(small_tiles):
+    """The CG example with vectors longer than a workgroup's share (sums pending between launches):
+    converges to the closed-form solution as the node-by-node run does."""
+    itf = small_tiles
+    itf.set_min_tile(1, 4096)
+    n = 1200
+    A = cnp.ones((n, n), dtype=cnp.float64)
+    for i in range(n):
+        A[i, i] = n + 1.0
+    b = cnp.arange(1, n + 1, dtype=cnp.float64)
+    x = cnp.zeros((n,), dtype=cnp.float64)
+    r = b.copy()
+    p = b.copy()
+    rtr = r @ r
+    history = []
+    for k in range(3):
+        Ap = A @ p
+        pAp = p @ Ap
+        alpha = rtr / pAp
+        x = x + alpha * p
+        r = r - alpha * Ap
+        rtr_new = r @ r
+        beta = rtr_new / rtr
+        p = r + beta * p
+        rtr = rtr_new
+        if k == 1:
+            history.append(rtr.get(itf).item())
+    bn = np.arange(1, n + 1, dtype=np.float64)
+    want = (bn - bn.sum() / (2 * n)) / n
+    assert np.allclose(x.get(itf), want, rtol=1e-10, atol=0)
+    assert history[0] < 1e-12 * float(bn @ bn)

@@ -85,7 +85,8 @@ def test_fused_matvec_forms_its_vector_and_leaves_the_dot(dev, cpu_system):
     dxa, dxb, dnum, dden = dev.array(xa), dev.array(xb), dev.array(num), dev.array(den)
     dx, dy, dy2 = dev.empty((N,), np.float64), dev.empty((N,), np.float64), dev.empty((N,), np.float64)
     dfold, dpart = dev.empty((1,), np.float64), dev.empty((N // 64,), np.float64)
-    f = L.GemvFusion(dxa.ptr, dxb.ptr, dnum.ptr, 128, dden.ptr, dfold.ptr, dx.ptr, dpart.ptr, N // 64)
+    dquot = dev.array(np.array([np.nan, 5.0]))
+    f = L.GemvFusion(dxa.ptr, dxb.ptr, dnum.ptr, 128, dden.ptr, dfold.ptr, dx.ptr, dpart.ptr, N // 64, dquot.ptr)
     npart = C.c_int64()
     L.check(L.lib.cnh_gemv_tiles_fused(N, N, tile, tp, dx.ptr, dy.ptr, C.byref(f), C.byref(npart), None))
     assert npart.value == N // 64
@@ -96,6 +97,7 @@ def test_fused_matvec_forms_its_vector_and_leaves_the_dot(dev, cpu_system):
     S = lanes[0]
     assert dfold.get()[0] == S
     want_x = xa + (S / den[0]) * xb
+    assert dquot.get()[0] == S / den[0] and dquot.get()[1] == 5.0
     got_x = dx.get()
     assert got_x.tobytes() == want_x.tobytes()
     L.check(L.lib.cnh_gemv_tiles(L.F64, N, N, tile, tp, dx.ptr, dy2.ptr, None))
@@ -120,6 +122,9 @@ def test_fused_matvec_forms_its_vector_and_leaves_the_dot(dev, cpu_system):
     assert L.lib.cnh_gemv_tiles_fused(4096, 4096, 2048, tp, dx.ptr, dy.ptr, C.byref(f2), None, None) == -3
     f3 = L.GemvFusion(dx.ptr, dxb.ptr, dnum.ptr, 128, dden.ptr, None, None, None, 0)
     assert L.lib.cnh_gemv_tiles_fused(N, N, tile, tp, dx.ptr, dy.ptr, C.byref(f3), None, None) == -2
+    # y may not be one of the vectors other workgroups still read
+    for alias in (dx.ptr, dxa.ptr, dxb.ptr):
+        assert L.lib.cnh_gemv_tiles_fused(N, N, tile, tp, dx.ptr, alias, C.byref(f), None, None) == -2
     for t in bufs:
         t.free()
     dev.free_all()

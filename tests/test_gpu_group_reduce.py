@@ -173,3 +173,98 @@ def test_partials_left_by_one_launch_are_summed_by_the_next(dev):
     with pytest.raises(L.CnhError, match="room"):
         H.launch_batched(kp, 1, [a], [], [o])
     dev.free_all()
+
+
+def test_fold_sums_adds_in_the_order_a_consuming_launch_uses(dev):
+    """cnh_fold_sums is the value a launch would have formed from the same partial sums: the same
+    bits as the `folded` store of cnh_launch_group_sums, for counts on every side of the lane and
+    workgroup boundaries."""
+    rng = np.random.default_rng(17)
+    c = AstBuilder(L.F64, 1)
+    c.binary(L.OP_MUL, 10, c.leaf(0), c.broadcast(5), is_temp=False)
+    kc = H.compile_group(c.finish(), L.F64, 1)
+    y, ob = dev.array(np.ones(100)), dev.empty((100,), np.float64)
+    for count in (1, 2, 63, 64, 65, 255, 256, 257, 1000, 1024, 4097):
+        hp = rng.standard_normal(count) * 10.0 ** rng.integers(-3, 4, count)
+        partials = dev.array(hp)
+        out = dev.array(np.array([np.nan, np.nan]))
+        L.check(L.lib.cnh_fold_sums(partials.ptr, count, out.ptr, None))
+        sums = (L.ScalarSum * 1)()
+        sums[0].ptr, sums[0].count, sums[0].folded = partials.ptr, count, out.ptr + 8
+        ins, outs = (L.Memref * 1)(y.memref()), (L.Memref * 1)(ob.memref())
+        L.check(L.lib.cnh_launch_group_sums(kc, 1, 1, ins, 1, sums, 1, outs, None))
+        got = out.get()
+        if count > 1:
+            assert got[0].tobytes() == got[1].tobytes(), count
+        import math
+        assert abs(got[0] - math.fsum(hp)) <= 1e-12 * np.abs(hp).sum(), count
+        assert np.all(ob.get() == got[0])
+    assert L.lib.cnh_fold_sums(None, 4, y.ptr, None) == -2
+    assert L.lib.cnh_fold_sums(y.ptr, 0, y.ptr, None) == -2
+    dev.free_all()
+
+
+@pytest.mark.parametrize("n", [1, 5, 512, 513, 100003])
+def test_a_scalar_statement_rides_on_the_launch_that_uses_it(dev, n):
+    """CNH_OP_SCALAR_OF: alpha = s5 / s6 formed in registers by every lane, stored once; x2 = x + alpha p,
+    r2 = r - alpha q and the partial sums of r2 . r2 from the same launch. Checked against NumPy in
+    the same operand order, bit for bit (the sum to 1e-12)."""
+    rng = np.random.default_rng(n)
+    b = AstBuilder(L.F64, 1)
+    alpha = b.binary(L.OP_DIV, 100, b.broadcast(5), b.broadcast(6))
+    b.unary(L.OP_SCALAR_OF, 20, alpha, is_temp=False)
+    t1 = b.binary(L.OP_MUL, 101, alpha, b.leaf(1))
+    b.binary(L.OP_ADD, 7, b.leaf(2), t1, is_temp=False)
+    t2 = b.binary(L.OP_MUL, 102, alpha, b.leaf(3))
+    r_new = b.binary(L.OP_SUB, 8, b.leaf(4), t2, is_temp=False)
+    b.unary(L.OP_SUM_OF, 9, b.binary(L.OP_MUL, 103, r_new, r_new), is_temp=False)
+    k = H.compile_group(b.finish(), L.F64, 1)
+    hp, hx, hq, hr = (rng.standard_normal(n) for _ in range(4))
+    p, x, q, r = dev.array(hp), dev.array(hx), dev.array(hq), dev.array(hr)
+    x2, r2 = dev.empty((n,), np.float64), dev.empty((n,), np.float64)
+    # s5 as 37 partial sums, s6 a plain value
+    h5 = rng.uniform(0.5, 1.5, 37)
+    s5, s6 = dev.array(h5), dev.array(np.array([1.75]))
+    folded = dev.array(np.array([np.nan]))
+    alpha_out = dev.array(np.array([np.nan, 7.0, 7.0]))          # one element is written, no more
+    rr = dev.array(np.array([np.nan]))
+    ins, outs = bind(k, {1: p.memref(), 2: x.memref(), 3: q.memref(), 4: r.memref()},
+                     {20: L.Memref.dense(alpha_out.ptr, (1,)), 7: x2.memref(), 8: r2.memref(),
+                      9: L.Memref.dense(rr.ptr, (1,))})
+    sums = (L.ScalarSum * 2)()
+    name = C.c_int()
+    for i in range(2):
+        L.check(L.lib.cnh_kernel_scalar(k, i, C.byref(name)))
+        if name.value == 5:
+            sums[i].ptr, sums[i].count, sums[i].folded = s5.ptr, 37, folded.ptr
+        else:
+            sums[i].ptr, sums[i].count, sums[i].folded = s6.ptr, 1, None
+    ia, oa = (L.Memref * 4)(*ins), (L.Memref * 4)(*outs)
+    L.check(L.lib.cnh_launch_group_sums(k, 1, 4, ia, 2, sums, 4, oa, None))
+    S = folded.get()[0]
+    chk = dev.array(np.array([np.nan]))
+    L.check(L.lib.cnh_fold_sums(s5.ptr, 37, chk.ptr, None))
+    assert S.tobytes() == chk.get()[0].tobytes()
+    a = S / 1.75
+    got_alpha = alpha_out.get()
+    assert got_alpha[0] == a and got_alpha[1] == 7.0 and got_alpha[2] == 7.0
+    want_r = hr - a * hq
+    assert np.array_equal(x2.get(), hx + a * hp) and np.array_equal(r2.get(), want_r)
+    assert abs(rr.get()[0] - np.sum(want_r * want_r)) <= 1e-12 * np.sum(want_r * want_r)
+    # the plain launch (scalars by pointer) stores the same alpha
+    s5v = dev.array(np.array([S]))
+    alpha_out.put(np.array([np.nan, 7.0, 7.0]))
+    names = []
+    for i in range(2):
+        L.check(L.lib.cnh_kernel_scalar(k, i, C.byref(name)))
+        names.append(name.value)
+    ptrs = L.vparr([s5v.ptr if nm == 5 else s6.ptr for nm in names])
+    L.check(L.lib.cnh_launch_group(k, 1, 4, ia, 2, ptrs, 1, 4, oa, None))
+    assert alpha_out.get()[0] == a and np.array_equal(r2.get(), want_r)
+    # a value with an index cannot be a scalar output, and strided launches refuse such a group
+    bad = AstBuilder(L.F64, 1)
+    v = bad.binary(L.OP_MUL, 10, bad.leaf(0), bad.broadcast(5), is_temp=False)
+    bad.unary(L.OP_SCALAR_OF, 20, v, is_temp=False)
+    with pytest.raises(L.CnhError):
+        H.compile_group(bad.finish(), L.F64, 1)
+    dev.free_all()
