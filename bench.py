@@ -1187,28 +1187,36 @@ def cpu_lstm(threads, steps=2, batch=256, nin=1024, d=1024, seed=5):
                     "statements as interpreted groups on one thread"}
 
 
-def run_frontend(n, steps, warmup):
-    """The same CG iteration and Jacobi sweeps written against the NumPy-like frontend: statements
-    -> DAG message -> host executor -> the same kernels. Shows what the whole stack costs on top of
-    the direct C ABI calls timed above (wall clock, flush + sync included)."""
+def run_frontend_cg(n, steps, warmup, trace_iters=0):
+    """The headline: the CG iteration of examples/cg.py:40-52 upstream written with the frontend's
+    operators and run by the host executor (statement log -> planner -> DAG nodes -> kernels), the
+    route a user of the drop-in takes. One step = one CG iteration; the timed region is `steps`
+    iterations between two syncs, recording and flushing included. The matvec launches of the
+    timed stretch are bracketed by events on the executor's own stream. With trace_iters > 0 an
+    untimed pass over the same system first keeps alpha, beta and r.r of every iteration and x at
+    its end for the parity check against the CPU leg."""
     import charmnumeric_amd as cnp
     out = {}
     cnp.reset()
     itf = cnp.CharmNumericInterface(device=0)
     itf.connect(odf=4)
     itf.set_pipeline(True)               # the executor works on its own thread while Python records
-    out["pipelined"] = True
     try:
         cnp.set_auto_flush(itf, 48)      # keep the device busy while later statements are recorded
         A = cnp.random.cg_matrix(n, 2)
         b = cnp.random.uniform((n,), seed=2, stream=1, low=-1.0, high=1.0)
-        x = cnp.zeros((n,))
-        r = b.copy()
-        p = b.copy()
-        rtr = r @ r
+        cnp.execute(itf)
+        out["tile"] = itf.array_info(A.name)["tile"]
+        state = {}
 
-        def iterate(k):
-            nonlocal x, r, p, rtr
+        def start():
+            state["x"] = cnp.zeros((n,))
+            state["r"] = b.copy()
+            state["p"] = b.copy()
+            state["rtr"] = state["r"] @ state["r"]
+
+        def iterate(k, keep=None):
+            x, r, p, rtr = state["x"], state["r"], state["p"], state["rtr"]
             for _ in range(k):
                 Ap = A @ p
                 pAp = p @ Ap
@@ -1219,26 +1227,61 @@ def run_frontend(n, steps, warmup):
                 beta = rtr_new / rtr
                 p = r + beta * p
                 rtr = rtr_new
+                if keep is not None:
+                    keep.append((alpha, beta, rtr))
+            state.update(x=x, r=r, p=p, rtr=rtr)
             cnp.execute(itf)
             itf.sync()
 
+        start()
         iterate(warmup)
-        # start again from x = 0, as the direct loop does, so that the timed iterations are the same
-        # ones (and r.r at the end can be compared with the direct loop's)
-        x = cnp.zeros((n,))
-        r = b.copy()
-        p = b.copy()
-        rtr = r @ r
+        if trace_iters > 0:
+            start()
+            kept = []
+            iterate(trace_iters, kept)
+            out["trace"] = {"alpha": [a.get(itf).item() for a, _, _ in kept],
+                            "beta": [b_.get(itf).item() for _, b_, _ in kept],
+                            "rtr": [r_.get(itf).item() for _, _, r_ in kept],
+                            "x": state["x"].get(itf)}
+            del kept
+        # the timed iterations start again from x = 0
+        start()
         cnp.execute(itf)
         itf.sync()
+        itf.time_matvecs(True)
         t0 = time.perf_counter()
         iterate(steps)
         dt = time.perf_counter() - t0
-        out["cg_iterations_per_s"] = round(steps / dt, 1)
-        out["cg_us_per_iteration"] = round(dt / steps * 1e6, 1)
-        out["cg_rtr_final"] = rtr.get(itf).item()
-        del A, b, x, r, p, rtr
+        gemv_ms = itf.matvec_times_ms()
+        itf.time_matvecs(False)
+        out.update({"iters_per_s": steps / dt, "ms_per_step": dt * 1e3 / steps, "wall_s": dt,
+                    "gemv_avg_us": 1e3 * float(np.mean(gemv_ms)), "gemv_min_us": 1e3 * float(np.min(gemv_ms)),
+                    "gemv_launches_timed": len(gemv_ms),
+                    "rtr_final": state["rtr"].get(itf).item()})
+        st = itf.stats()
+        out["executor"] = {"group_launches": st["group_launches"], "compiled": st["compiled"],
+                           "live_arrays": st["live_arrays"]}
+        state.clear()
+        del A, b
+    finally:
+        cnp.reset()
+        itf.close()
+    return out
 
+
+def run_frontend():
+    """The other configurations written against the NumPy-like frontend: statements -> statement log
+    -> host executor -> the same kernels. Shows what the whole stack costs on top of the direct
+    C ABI calls timed above (wall clock, flush + sync included)."""
+    import charmnumeric_amd as cnp
+    out = {}
+    cnp.reset()
+    itf = cnp.CharmNumericInterface(device=0)
+    itf.connect(odf=4)
+    itf.set_pipeline(True)               # the executor works on its own thread while Python records
+    out["pipelined"] = True
+    try:
+        cnp.set_auto_flush(itf, 48)      # keep the device busy while later statements are recorded
         # configuration 1 as examples/simple.py upstream writes it: one fused statement, sum, norm
         m = 1 << 24
         xs = cnp.random.uniform((m,), seed=0, stream=0, low=-1.0, high=1.0)
@@ -1379,43 +1422,56 @@ def main():
     L.check(L.lib.cnh_device_name(name, 256))
     n = args.n
     parity_iters = 0 if args.no_cpu else min(args.steps, args.cpu_iters)
+    # The headline is the route a user of the drop-in takes: the frontend's operators through the
+    # host executor. The same iteration by direct C ABI calls is timed beside it.
+    cgf = run_frontend_cg(n, args.steps, args.warmup, trace_iters=parity_iters)
     cg = run_cg(L, n, args.steps, args.warmup, trace_iters=parity_iters, fuse=not args.cg_separate)
     gemv_bytes = 8.0 * n * n + 2 * 8.0 * n
-    achieved = gemv_bytes / (cg["gemv_avg_us"] * 1e-6) / 1e9
+    achieved = gemv_bytes / (cgf["gemv_avg_us"] * 1e-6) / 1e9
+    two = cgf["gemv_launches_timed"] == args.steps and n >= 16384
     line = {
         "metric": "cg_iterations_per_second_n16384_fp64",
-        "value": round(cg["iters_per_s"], 2),
+        "value": round(cgf["iters_per_s"], 2),
         "unit": "iterations/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(cg["ms_per_step"], 4),
+        "ms_per_step": round(cgf["ms_per_step"], 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f64",
         "data": "synthetic",
-        "config": {"workload": f"dense CG, n={n}, A in {cg['tile']}^2 row-major tiles, one CG "
-                               "iteration per step (matvec, 2 dots, 2 scalar ops, 3 updates) in "
-                               + ("two launches: the matvec, which forms p = r + beta p on the way (beta from the "
+        "config": {"workload": f"dense CG, n={n}, A in {cgf['tile']}^2 row-major tiles, one CG iteration per step "
+                               "(matvec, 2 dots, 2 scalar statements, 3 vector updates) written with the frontend's "
+                               "operators as examples/cg.py:40-52 upstream and run by the host executor, which "
+                               "launches it as "
+                               + ("two kernels: the matvec, which forms p = r + beta p on the way (beta from the "
                                   "partial sums of r.r) and leaves the partial sums of p.Ap; x and r with alpha "
-                                  "formed in registers and the partial sums of r.r taken on the way"
-                                  if cg["launches_per_iteration"] == 2 else
-                                  "four launches: matvec; p.Ap; x and r with alpha formed in registers and r.r "
-                                  "taken on the way; p with beta formed in registers"),
+                                  "formed in registers and the partial sums of r.r taken on the way" if two else
+                                  "a matvec, a dot and two merged launches of the vector and scalar statements"),
+                   "route": "charmnumeric_amd frontend -> statement log -> host executor -> HIP kernels",
                    "device": name.value.decode()},
         "roofline": {"bound": "hbm",
-                     "kernel": "gemv_rows_xlds<double,8,8,4,true>" if cg["launches_per_iteration"] == 2
-                     else "gemv_rows_xlds<double,8,8,4>", "achieved": round(achieved, 1),
+                     "kernel": "gemv_rows_xlds<double,8,8,4,true>" if two else "gemv_rows_xlds<double,8,8,4>",
+                     "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": (GEMV_N16384_TRAFFIC_BYTES if cg["launches_per_iteration"] == 2
-                                 else GEMV_N16384_TRAFFIC_BYTES_PLAIN) if n == 16384 else None,
+                     "traffic": (GEMV_N16384_TRAFFIC_BYTES if two else GEMV_N16384_TRAFFIC_BYTES_PLAIN)
+                     if n == 16384 else None,
                      "traffic_source": "rocprofv3 --pmc counters of an earlier run of this kernel "
                                        "(profiles/bench_hbm_traffic_pmc.txt), not measured in this run",
-                     "avg_us": round(cg["gemv_avg_us"], 2),
+                     "avg_us": round(cgf["gemv_avg_us"], 2),
+                     "timed_by": "HIP events around every matvec launch on the executor's stream, inside the timed "
+                                 "iterations",
                      "bytes_per_launch": gemv_bytes},
         "gemv_roofline_iters_per_s": round(HBM_PEAK_GBS * 1e9 / gemv_bytes, 1),
-        "rtr_final": cg["rtr_final"],
+        "rtr_final": cgf["rtr_final"],
+        "executor": cgf["executor"],
+        "direct_c_abi": {"what": "the same iterations as direct calls of the C ABI with prepared launches "
+                                 "(cnh_gemv_tiles_fused + cnh_launch_group_sums), no frontend and no executor",
+                         "iterations_per_s": round(cg["iters_per_s"], 2), "ms_per_step": round(cg["ms_per_step"], 4),
+                         "gemv_avg_us": round(cg["gemv_avg_us"], 2),
+                         "launches_per_iteration": cg["launches_per_iteration"], "rtr_final": cg["rtr_final"]},
     }
     if not args.no_also:
         also = {}
@@ -1436,7 +1492,7 @@ def main():
         except Exception as exc:
             also["c5_error"] = str(exc)
         try:
-            also["through_frontend"] = run_frontend(n, args.steps, args.warmup)
+            also["through_frontend"] = run_frontend()
         except Exception as exc:
             also["frontend_error"] = str(exc)
         line["also"] = also
@@ -1449,7 +1505,7 @@ def main():
         line["cpu_baseline"] = {
             "value": round(ipsN, 3), "unit": "iterations/s", "cores": threads, "kind": "port",
             "threads_used": threads, "host_logical_cpus": logical, "host_physical_cores": physical,
-            "sample": f"same system (n={n}, {cg['tile']}^2 tiles), {args.cpu_iters} CG iterations, "
+            "sample": f"same system (n={n}, {cgf['tile']}^2 tiles), {args.cpu_iters} CG iterations, "
                       f"oracle kernels, tile matvec split over {threads} threads",
             "one_core": round(ips1, 3),
         }
@@ -1471,9 +1527,10 @@ def main():
                 line["also"]["cpu_port_error"] = str(exc)
         # same system, same number of iterations (an untimed pass of the device path before the
         # timed one): the two solutions and the per-iteration scalars must agree
-        par = cg_parity(cg["trace"], cpu_trace, cpu_trace["rtr0"])
+        par = cg_parity(cgf["trace"], cpu_trace, cpu_trace["rtr0"])
         line["cg_parity_max_rel_diff"] = par["x_max_rel_diff"]
         line["cg_parity"] = par
+        line["direct_c_abi"]["cg_parity"] = cg_parity(cg["trace"], cpu_trace, cpu_trace["rtr0"])
     print(json.dumps(line))
 
 

@@ -293,6 +293,8 @@ _PROTOS.update({
     "cnx_array_info": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int),
                                  C.POINTER(C.c_int), _i32p, _i32p]),
     "cnx_stats": (C.c_int, [C.c_void_p, _i64p]),
+    "cnx_set_matvec_timing": (C.c_int, [C.c_void_p, C.c_int]),
+    "cnx_matvec_times": (C.c_int64, [C.c_void_p, C.POINTER(C.c_float), C.c_int64]),
     "cnx_solve_decompositions": (C.c_int, [C.c_int, C.c_int, _i32p, C.c_int, C.POINTER(Decomp),
                                            C.c_int64, C.c_char_p]),
     "cnx_set_trace": (C.c_int, [C.c_void_p, C.c_int]),

@@ -210,6 +210,9 @@ struct cnx_executor {
         int64_t count = 0;
     };
     std::map<int, PendingSum> pending;
+    // Measurement: with timing on, every matvec launch sits between two events on the stream.
+    bool time_matvec = false;
+    std::vector<std::pair<cnh_event, cnh_event>> matvec_events;
 
     void log(const std::string& s) {
         if (trace_on) {
@@ -995,6 +998,23 @@ int new_scalar_array(Ex* ex, int name, int dtype, XArray** out) {
     return make_array(ex, name, 1, dtype, one, false, out);
 }
 
+// The matvec launches of a timed stretch (cnx_set_matvec_timing) are bracketed by event pairs.
+cnh_event matvec_timer_start(Ex* ex) {
+    if (!ex->time_matvec || ex->dry)
+        return nullptr;
+    cnh_event e0 = nullptr;
+    if (cnh_event_create(&e0) != 0 || cnh_event_record(e0, ex->stream) != 0)
+        return nullptr;
+    return e0;
+}
+void matvec_timer_stop(Ex* ex, cnh_event e0) {
+    if (e0 == nullptr)
+        return;
+    cnh_event e1 = nullptr;
+    if (cnh_event_create(&e1) == 0 && cnh_event_record(e1, ex->stream) == 0)
+        ex->matvec_events.emplace_back(e0, e1);
+}
+
 // REDUCE: per-tile dots and their in-order sum, result = size-1 array
 // (src/executor_reduce.cpp:8-119, src/executor_reducer.cpp:11-57, src/partition_comm.cpp:69-111).
 int exec_reduce(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
@@ -1391,8 +1411,10 @@ int exec_matmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
             }
         // 1-D arrays are contiguous: the vector window is a pointer into tile 0.
         const char* xp = static_cast<const char*>(x->tiles[0]) + (int64_t)wx.start[0] * dtype_size(x->dtype);
+        cnh_event t0 = matvec_timer_start(ex);
         rc = cnh_gemv_panels(Aa->dtype, A.rows, pc1 - pc0 + 1, T, A.r0 - pr0 * T, (int64_t)panels.size(),
                              panels.data(), xp, y->tiles[0], ex->stream);
+        matvec_timer_stop(ex, t0);
     }
     if (a_copy)
         drop_array(ex, Aa->name);
@@ -2682,9 +2704,12 @@ int try_fused_matvec(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t* 
                   : std::string()) +
             (dot_name ? " dot=" + std::to_string(dot_name) : std::string()));
     int rc = 0;
-    if (!ex->dry)
+    if (!ex->dry) {
+        cnh_event t0 = matvec_timer_start(ex);
         rc = cnh_gemv_tiles_fused(mv.rows, mv.cols, mv.A->tile, mv.A->tiles.data(), xptr, y->tiles[0], &fu, nullptr,
                                   ex->stream);
+        matvec_timer_stop(ex, t0);
+    }
     if (rc)
         return rc;
     if (num_was_pending)
@@ -3647,6 +3672,10 @@ int cnx_destroy(cnx_executor* ex) {
         }
         for (auto& kv : ex->pending)
             cnh_free(kv.second.partials);
+        for (auto& pr : ex->matvec_events) {
+            cnh_event_destroy(pr.first);
+            cnh_event_destroy(pr.second);
+        }
         for (auto& kv : ex->free_list)
             for (void* p : kv.second)
                 cnh_free(p);
@@ -3965,6 +3994,40 @@ int cnx_array_info(cnx_executor* ex, int name, int* ndims, int* dtype, int* tile
             offset3[d] = a->offset[d];
     }
     return 0;
+}
+
+int cnx_set_matvec_timing(cnx_executor* ex, int on) {
+    CNH_CHECK(ex != nullptr, -2, "null executor");
+    if (int rc = settle(ex))
+        return rc;
+    ex->time_matvec = on != 0;
+    for (auto& pr : ex->matvec_events) {
+        cnh_event_destroy(pr.first);
+        cnh_event_destroy(pr.second);
+    }
+    ex->matvec_events.clear();
+    return 0;
+}
+
+int64_t cnx_matvec_times(cnx_executor* ex, float* ms, int64_t cap) {
+    CNH_CHECK(ex != nullptr && (ms != nullptr || cap == 0), -2, "bad arguments");
+    if (int rc = settle(ex))
+        return rc;
+    if (!ex->dry)
+        if (int rc = cnh_stream_sync(ex->stream))
+            return rc;
+    int64_t n = 0;
+    for (auto& pr : ex->matvec_events) {
+        if (n < cap) {
+            if (int rc = cnh_event_elapsed_ms(pr.first, pr.second, &ms[n]))
+                return rc;
+            ++n;
+        }
+        cnh_event_destroy(pr.first);
+        cnh_event_destroy(pr.second);
+    }
+    ex->matvec_events.clear();
+    return n;
 }
 
 int cnx_stats(cnx_executor* ex, int64_t out[8]) {

@@ -179,6 +179,18 @@ class CharmNumericInterface:
         return {"ndims": nd.value, "dtype": dt.value, "tile": tile.value,
                 "shape": tuple(shape[:nd.value]), "offset": tuple(off[:nd.value])}
 
+    def time_matvecs(self, on=True):
+        """Brackets every matvec launch with events from now on (measurement only)."""
+        L.check(L.lib.cnx_set_matvec_timing(self._handle(), 1 if on else 0))
+
+    def matvec_times_ms(self, at_most=4096):
+        """Elapsed milliseconds of the matvec launches timed since the last call, oldest first."""
+        buf = (C.c_float * at_most)()
+        n = L.lib.cnx_matvec_times(self._handle(), buf, at_most)
+        if n < 0:
+            L.check(int(n))
+        return [buf[i] for i in range(n)]
+
     def stats(self):
         out = (C.c_int64 * 8)()
         L.check(L.lib.cnx_stats(self._handle(), out))

@@ -162,6 +162,12 @@ int cnx_sync(cnx_executor* ex);
 /* ndims, dtype, tile edge, shape[3], offset[3] of array `name`; < 0 if unknown. */
 int cnx_array_info(cnx_executor* ex, int name, int* ndims, int* dtype, int* tile, int32_t* shape3,
                    int32_t* offset3);
+/* Measurement (no upstream counterpart). With timing on, every matvec launch of the executor is
+ * bracketed by a pair of events on its stream; cnx_matvec_times waits for the stream, writes the
+ * elapsed milliseconds of the launches timed so far (oldest first, at most `cap`) to `ms`, forgets
+ * them and returns how many it wrote. Switching timing on or off also forgets them. */
+int cnx_set_matvec_timing(cnx_executor* ex, int on);
+int64_t cnx_matvec_times(cnx_executor* ex, float* ms, int64_t cap);
 /* Counters since creation: [0] kernels compiled (upstream num_compile, src/backend.hpp:241),
  * [1] compile-cache hits, [2] DAG nodes executed, [3] device allocations, [4] free-list reuses,
  * [5] fused-group launches, [6] live arrays, [7] bytes held (live + free list). */
