@@ -1269,6 +1269,134 @@ def run_frontend_cg(n, steps, warmup, trace_iters=0):
     return out
 
 
+def run_strided(reps=10, only=None):
+    """Programs whose statements do not fit the aligned, unit-step, even-width mould of the five
+    configurations: the sweeps and grid transfers of examples/multigrid2d.py and
+    examples/gauss_seidel.py upstream (odd 2^k + 1 grids, step-2 lattices). Through the frontend,
+    wall clock between two syncs. Bytes are the elements each statement has to touch, 8 bytes each
+    (no allowance for the halves of cache lines a stride of two leaves unused)."""
+    import charmnumeric_amd as cnp
+    out = {}
+    cnp.reset()
+    itf = cnp.CharmNumericInterface(device=0)
+    itf.connect(odf=4)
+    itf.set_pipeline(True)
+    try:
+        cnp.set_auto_flush(itf, 48)
+
+        def timed(fn, n, warm=2):
+            for _ in range(warm):
+                fn()
+            cnp.execute(itf)
+            itf.sync()
+            t0 = time.perf_counter()
+            for _ in range(n):
+                fn()
+            cnp.execute(itf)
+            itf.sync()
+            return (time.perf_counter() - t0) / n * 1e6
+
+        def want(name):
+            return only is None or only == name
+
+        def entry(us, nbytes, **more):
+            d = {"us": round(us, 1), "algorithmic_bytes": int(nbytes), "GBs": round(nbytes / (us * 1e-6) / 1e9, 1),
+                 "frac_of_hbm_peak": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 3)}
+            d.update(more)
+            return d
+
+        # weighted Jacobi with a source term on a 2^12 + 1 grid (examples/multigrid2d.py smoother)
+        n = 4097
+        u = cnp.random.uniform((n, n), seed=7, stream=0, low=0.0, high=1.0)
+        f = cnp.random.uniform((n, n), seed=7, stream=1, low=-1.0, high=1.0)
+        h2, omega = (1.0 / (n - 1)) ** 2, 2.0 / 3.0
+
+        def smooth():
+            upd = 0.25 * (u[:-2, 1:-1] + u[2:, 1:-1] + u[1:-1, :-2] + u[1:-1, 2:] + h2 * f[1:-1, 1:-1])
+            u[1:-1, 1:-1] = (1.0 - omega) * u[1:-1, 1:-1] + omega * upd
+
+        if want("weighted_jacobi_4097"):
+            out["weighted_jacobi_4097"] = entry(timed(smooth, 2 * reps), 3 * 8.0 * n * n)
+
+        # residual into a third array, restriction to 2049^2 and prolongation back
+        r = cnp.zeros((n, n))
+
+        def residual():
+            r[1:-1, 1:-1] = f[1:-1, 1:-1] - (1.0 / h2) * (4.0 * u[1:-1, 1:-1] - u[:-2, 1:-1] - u[2:, 1:-1]
+                                                           - u[1:-1, :-2] - u[1:-1, 2:])
+
+        if want("residual_4097"):
+            out["residual_4097"] = entry(timed(residual, 2 * reps), 3 * 8.0 * n * n)
+        nc = (n - 1) // 2 + 1
+        coarse = cnp.zeros((nc, nc))
+        c_, lo, hi = slice(2, -2, 2), slice(1, -3, 2), slice(3, -1, 2)
+
+        def restrict():
+            coarse[1:-1, 1:-1] = (0.25 * r[c_, c_]
+                                  + 0.125 * (r[lo, c_] + r[hi, c_] + r[c_, lo] + r[c_, hi])
+                                  + 0.0625 * (r[lo, lo] + r[lo, hi] + r[hi, lo] + r[hi, hi]))
+
+        if want("restriction_4097_to_2049"):
+            out["restriction_4097_to_2049"] = entry(timed(restrict, 2 * reps), 8.0 * n * n + 8.0 * nc * nc)
+        e = cnp.zeros((n, n))
+
+        def prolong():
+            e[2:-2:2, 2:-2:2] = coarse[1:-1, 1:-1]
+            e[1:-1:2, 2:-2:2] = 0.5 * (coarse[:-1, 1:-1] + coarse[1:, 1:-1])
+            e[2:-2:2, 1:-1:2] = 0.5 * (coarse[1:-1, :-1] + coarse[1:-1, 1:])
+            e[1:-1:2, 1:-1:2] = 0.25 * (coarse[:-1, :-1] + coarse[1:, :-1] + coarse[:-1, 1:] + coarse[1:, 1:])
+
+        if want("prolongation_2049_to_4097"):
+            out["prolongation_2049_to_4097"] = entry(timed(prolong, 2 * reps), 8.0 * n * n + 4 * 8.0 * nc * nc,
+                                                     statements=4)
+        del u, f, r, coarse, e
+        cnp.execute(itf)
+
+        # red-black Gauss-Seidel on 8192^2 (examples/gauss_seidel.py): four statements a sweep
+        n = 8192
+        phi = cnp.zeros((n, n))
+        g = cnp.random.uniform((n, n), seed=8, stream=0, low=-1.0, high=1.0)
+        h2 = (1.0 / (n - 1)) ** 2
+
+        def red_black():
+            for r0, c0 in ((1, 1), (2, 2), (1, 2), (2, 1)):
+                rows, cols = slice(r0, -1, 2), slice(c0, -1, 2)
+                up, down = slice(r0 - 1, -2, 2), slice(r0 + 1, None, 2)
+                left, right = slice(c0 - 1, -2, 2), slice(c0 + 1, None, 2)
+                phi[rows, cols] = 0.25 * (phi[up, cols] + phi[down, cols] + phi[rows, left] + phi[rows, right]
+                                          - h2 * g[rows, cols])
+
+        if want("red_black_8192"):
+            out["red_black_8192"] = entry(timed(red_black, reps), 4 * 8.0 * n * n, statements=4)
+        del phi, g
+        cnp.execute(itf)
+
+        # 7-point Poisson sweep with a source term on 257^3
+        n = 257
+        itf.close()
+        itf = cnp.CharmNumericInterface(device=0)
+        itf.connect(odf=64)
+        itf.set_pipeline(True)
+        cnp.set_auto_flush(itf, 48)
+        v = cnp.random.uniform((n, n, n), seed=9, stream=0, low=0.0, high=1.0)
+        q = cnp.random.uniform((n, n, n), seed=9, stream=1, low=-1.0, high=1.0)
+        c6, h2 = 0.16666666666666666, (1.0 / (n - 1)) ** 2
+
+        def poisson():
+            v[1:-1, 1:-1, 1:-1] = c6 * (v[:-2, 1:-1, 1:-1] + v[2:, 1:-1, 1:-1] + v[1:-1, :-2, 1:-1]
+                                        + v[1:-1, 2:, 1:-1] + v[1:-1, 1:-1, :-2] + v[1:-1, 1:-1, 2:]
+                                        + h2 * q[1:-1, 1:-1, 1:-1])
+
+        if want("poisson_257_cubed"):
+            out["poisson_257_cubed"] = entry(timed(poisson, 4 * reps), 3 * 8.0 * n ** 3)
+        del v, q
+        cnp.execute(itf)
+    finally:
+        cnp.reset()
+        itf.close()
+    return out
+
+
 def run_frontend():
     """The other configurations written against the NumPy-like frontend: statements -> statement log
     -> host executor -> the same kernels. Shows what the whole stack costs on top of the direct
@@ -1407,6 +1535,10 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-also", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--cpu-iters", type=int, default=50)
+    ap.add_argument("--strided", action="store_true",
+                    help="only the strided and odd-sized programs (multigrid transfers, red-black sweeps); "
+                         "prints their figures as one JSON line of their own")
+    ap.add_argument("--only", default=None, help="with --strided: the one program to run (by its key in the output)")
     ap.add_argument("--cg-separate", action="store_true",
                     help="CG iteration as four launches (matvec, dot, x and r, p) instead of the fused two")
     args = ap.parse_args()
@@ -1416,6 +1548,10 @@ def main():
         sys.exit(2)
 
     L = _dev()
+    if args.strided:
+        print(json.dumps({"metric": "strided_programs_through_the_frontend", "unit": "us per operation",
+                          "n_gpus": 1, "data": "synthetic", "programs": run_strided(only=args.only)}))
+        return
     if os.environ.get("CNH_BENCH_MARCH2D"):
         L.check(L.lib.cnh_set_option(b"slide2d_march", 1))
     name = C.create_string_buffer(256)
@@ -1491,6 +1627,10 @@ def main():
             also["c5_lstm_forward"] = run_lstm(L)
         except Exception as exc:
             also["c5_error"] = str(exc)
+        try:
+            also["strided_programs"] = run_strided()
+        except Exception as exc:
+            also["strided_error"] = str(exc)
         try:
             also["through_frontend"] = run_frontend()
         except Exception as exc:

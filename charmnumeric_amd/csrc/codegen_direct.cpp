@@ -735,14 +735,53 @@ struct FlatArgs {
     FDiv gb1, gb2;         // ordering blocks along y and x
     FDiv obx, oby;         // = ob[2], ob[1]
     T* slots;              // reducing launches: one partial per launched wavefront
+    int sub8;              // ragged grids: workgroups per ordering block / 8, else 0
+    FDiv fsub;             // = sub8
 };
 
+// Rows of odd length, odd pitches or a block that does not start on a 16-byte boundary (UA): pairs
+// are then only element-aligned. They still move as one access each (the hardware takes 128-bit
+// accesses at any 4-byte boundary); the pair that holds the last element of an odd row is read one
+// element to the left and shifted, and written as a single element, so that nothing outside the row
+// is touched.
+typedef P2 P2A __attribute__((aligned(sizeof(T))));
+template <bool UA>
+__device__ __forceinline__ P2 load_pair(const T* row, int c, int S2) {
+    if (!UA) return *reinterpret_cast<const P2*>(row + c);
+    const bool whole = c + 1 < S2;
+    const P2 u = *reinterpret_cast<const P2A*>(row + (whole ? c : S2 - 2));
+    return whole ? u : (P2){u[1], u[1]};
+}
+template <bool NTS, bool UA>
+__device__ __forceinline__ void store_pair_flat(T* out, P2 v, bool in0, bool in1, bool has1) {
+    if (!UA) {
+        store_pair<NTS>(reinterpret_cast<P2*>(out), v, in0, in1);
+        return;
+    }
+    const bool w0 = !DR_MASKED || in0, w1 = has1 && (!DR_MASKED || in1);
+    if (w0 && w1) {
+        if (NTS) __builtin_nontemporal_store(v, reinterpret_cast<P2A*>(out)); else *reinterpret_cast<P2A*>(out) = v;
+    } else {
+        if (w0) out[0] = v[0];
+        if (w1) out[1] = v[1];
+    }
+}
+
 // RED as above.
-template <bool NTS, int RED>
+template <bool NTS, int RED, bool UA>
 __device__ __forceinline__ void direct_flat(const FlatArgs& a, const T* s) {
     T* const my_slot = RED ? a.slots + ((size_t)blockIdx.x * 4 + (threadIdx.x >> 6)) : nullptr;
     int blk = (int)blockIdx.x;
-    if (a.nblocks8) blk = (blk & 7) * a.nblocks8 + (blk >> 3);
+    if (a.sub8) {
+        // Ragged grids pad their last ordering blocks with workgroups that do nothing, so whole
+        // blocks per XCD would leave most of the work to a few XCDs: here every ordering block is
+        // cut into eight contiguous runs, one per XCD, and all XCDs walk the blocks together.
+        const int xcd = blk & 7, j = blk >> 3;
+        const int gq = fdiv(j, a.fsub);
+        blk = gq * (int)a.per_block.d + xcd * a.sub8 + (j - gq * a.sub8);
+    } else if (a.nblocks8) {
+        blk = (blk & 7) * a.nblocks8 + (blk >> 3);
+    }
     const int g = fdiv(blk, a.per_block), w = blk - g * (int)a.per_block.d;
     const int gq = fdiv(g, a.gb2), g2 = g - gq * (int)a.gb2.d;
     const int g0 = fdiv(gq, a.gb1), g1 = gq - g0 * (int)a.gb1.d;
@@ -764,8 +803,10 @@ __device__ __forceinline__ void direct_flat(const FlatArgs& a, const T* s) {
     }
     const int PY = a.py, PZ = a.pz;
     const int lx = x0 + 2 * lane;
-    const bool live = lx < S2;                  // S2 is even: a live lane owns a whole pair
-    const int cx = min(lx, S2 - 2);             // idle lanes re-read the last pair of the row
+    const bool live = lx < S2;                  // a live lane owns a pair, or the last element of an odd row
+    const bool live1 = lx + 1 < S2;
+    const int lastc = (S2 - 1) & ~1;            // column of the last pair (even S2) or last element (odd)
+    const int cx = min(lx, lastc);              // idle lanes re-read the end of the row
     const bool first = lane == 0, last = lane == 63;
     // clamped planes and rows of the window (wavefront-uniform)
     int zo[DR_WZ], yo[DR_WY];
@@ -783,8 +824,8 @@ __device__ __forceinline__ void direct_flat(const FlatArgs& a, const T* s) {
 #pragma unroll
         for (int j = 0; j < DR_WY; ++j)
             if (DR_NEED[i][j][0] || DR_NEED[i][j][DR_HK] || DR_NEED[i][j][DR_WK - 1])
-                win[i][j][DR_HK] = *reinterpret_cast<const P2*>(cur + (zo[i] + yo[j] + cx));
-    const int xl = max(x0 - 2, 0), xr = min(x0 + 128, S2 - 2);   // columns of the two far pairs
+                win[i][j][DR_HK] = load_pair<UA>(cur + (zo[i] + yo[j]), cx, S2);
+    const int xl = max(x0 - 2, 0), xr = min(x0 + 128, lastc);    // columns of the two far pairs
     P2 edge = (P2){(T)0, (T)0};
     if (DR_HK == 1) {
         if (DR_EDGE_GATHER) {
@@ -793,7 +834,7 @@ __device__ __forceinline__ void direct_flat(const FlatArgs& a, const T* s) {
             if (lane < 2 * DR_NB) {
                 const int r = lane >> 1, i = DR_BI0 + r / DR_BNJ, j = DR_BJ0 + r % DR_BNJ;
                 const int zz = min(max(z0 - DR_H0 + i, 0), S0 - 1), yy = min(max(y0 - DR_H1 + j, 0), S1 - 1);
-                edge = *reinterpret_cast<const P2*>(cur + (zz * PZ + yy * PY + ((lane & 1) ? xr : xl)));
+                edge = load_pair<UA>(cur + (zz * PZ + yy * PY), (lane & 1) ? xr : xl, S2);
             }
         } else {
 #pragma unroll
@@ -802,7 +843,7 @@ __device__ __forceinline__ void direct_flat(const FlatArgs& a, const T* s) {
                 for (int j = 0; j < DR_WY; ++j)
                     if (DR_NEED[i][j][0] || DR_NEED[i][j][DR_WK - 1]) {
                         const int c = first ? xl : (last ? xr : cx);
-                        beyond[i][j] = *reinterpret_cast<const P2*>(cur + (zo[i] + yo[j] + c));
+                        beyond[i][j] = load_pair<UA>(cur + (zo[i] + yo[j]), c, S2);
                     }
         }
     }
@@ -813,8 +854,7 @@ __device__ __forceinline__ void direct_flat(const FlatArgs& a, const T* s) {
         for (int rz = 0; rz < DR_RZ; ++rz)
 #pragma unroll
             for (int ry = 0; ry < DR_RY; ++ry)
-                ov[j][rz][ry] = *reinterpret_cast<const P2*>(
-                    a.oth[j] + (zo[rz + DR_H0] + yo[ry + DR_H1] + cx));
+                ov[j][rz][ry] = load_pair<UA>(a.oth[j] + (zo[rz + DR_H0] + yo[ry + DR_H1]), cx, S2);
     if (DR_HK == 1) {
 #pragma unroll
         for (int i = 0; i < DR_WZ; ++i)
@@ -880,10 +920,8 @@ __device__ __forceinline__ void direct_flat(const FlatArgs& a, const T* s) {
                 }
             }
             // rows and planes beyond the array (a ragged last workgroup) and idle lanes store nothing
-            if (live && z < S0 && y < S1) {
-                P2* out = reinterpret_cast<P2*>(dst + (z * PZ + y * PY + lx));
-                store_pair<NTS>(out, res, in_e[0], in_e[1]);
-            }
+            if (live && z < S0 && y < S1)
+                store_pair_flat<NTS, UA>(dst + (z * PZ + y * PY + lx), res, in_e[0], in_e[1], live1);
         }
     }
     if (RED) {
@@ -893,15 +931,19 @@ __device__ __forceinline__ void direct_flat(const FlatArgs& a, const T* s) {
 }
 #if DR_RED
 // The reducing forms only (built on demand under a variant name of their own).
-#define FLAT_RED_ENTRY(NAME, NTS, RED)                                                            \
+#define FLAT_RED_ENTRY(NAME, NTS, RED, UA)                                                        \
 extern "C" __global__ __launch_bounds__(256) void NAME(FlatArgs a, Scal sc) {                     \
     CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);                                                                \
-    direct_flat<NTS, RED>(a, s);                                                                  \
+    direct_flat<NTS, RED, UA>(a, s);                                                              \
 }
-FLAT_RED_ENTRY(grp_direct_flat_red1, false, 1)
-FLAT_RED_ENTRY(grp_direct_flat_red1_nts, true, 1)
-FLAT_RED_ENTRY(grp_direct_flat_red2, false, 2)
-FLAT_RED_ENTRY(grp_direct_flat_red2_nts, true, 2)
+FLAT_RED_ENTRY(grp_direct_flat_red1, false, 1, false)
+FLAT_RED_ENTRY(grp_direct_flat_red1_nts, true, 1, false)
+FLAT_RED_ENTRY(grp_direct_flat_red2, false, 2, false)
+FLAT_RED_ENTRY(grp_direct_flat_red2_nts, true, 2, false)
+FLAT_RED_ENTRY(grp_direct_flatu_red1, false, 1, true)
+FLAT_RED_ENTRY(grp_direct_flatu_red1_nts, true, 1, true)
+FLAT_RED_ENTRY(grp_direct_flatu_red2, false, 2, true)
+FLAT_RED_ENTRY(grp_direct_flatu_red2_nts, true, 2, true)
 // Tiles with buffers of their own: the lean part and the listed face workgroups in one launch.
 #define BOTH_RED_ENTRY(NAME, NTS, RED)                                                            \
 extern "C" __global__ __launch_bounds__(256) void NAME(DirectArgs a, Scal sc, const int* list) {  \
@@ -916,11 +958,20 @@ BOTH_RED_ENTRY(grp_direct_both_red2_nts, true, 2)
 #else
 extern "C" __global__ __launch_bounds__(256) void grp_direct_flat(FlatArgs a, Scal sc) {
     CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
-    direct_flat<false, 0>(a, s);
+    direct_flat<false, 0, false>(a, s);
 }
 extern "C" __global__ __launch_bounds__(256) void grp_direct_flat_nts(FlatArgs a, Scal sc) {
     CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
-    direct_flat<true, 0>(a, s);
+    direct_flat<true, 0, false>(a, s);
+}
+// the same for blocks whose pairs are only element-aligned (odd rows or pitches)
+extern "C" __global__ __launch_bounds__(256) void grp_direct_flatu(FlatArgs a, Scal sc) {
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
+    direct_flat<false, 0, true>(a, s);
+}
+extern "C" __global__ __launch_bounds__(256) void grp_direct_flatu_nts(FlatArgs a, Scal sc) {
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
+    direct_flat<true, 0, true>(a, s);
 }
 
 // nts: the written stream is not read back soon, store it non-temporally.

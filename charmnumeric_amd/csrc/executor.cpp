@@ -284,6 +284,27 @@ int tile_rule(const Ex* ex, int ndims, const int32_t* shape) {
     return (int)tile;
 }
 
+// Storage form of a new array. Rank 3: one row-major block whenever blocks are allowed (flat3).
+// Rank 2: a buffer per tile, except where tiles would not help the kernels anyway: rows of odd
+// length (128-bit accesses cannot stay inside tiles then) and ragged tile grids (a 4097 x 4097
+// array cut at 4096 has tiles of one row and one column). Those are one block too, and their
+// sweeps run the whole-array kernels.
+bool flat_rule(const Ex* ex, int nd, const int32_t* shape, int tile, const int32_t* offset) {
+    if (nd == 3)
+        return ex->flat3;
+    if (nd != 2 || !ex->flat3)
+        return false;
+    if (shape[1] % 2 != 0)
+        return true;
+    for (int d = 0; d < 2; ++d) {
+        const int off = offset ? offset[d] : 0;
+        const int glo = off / tile, ghi = (off + shape[d] + tile - 1) / tile;
+        if (ghi - glo > 1 && ((off + shape[d]) % tile != 0 || off % tile != 0))
+            return true;
+    }
+    return false;
+}
+
 int make_array(Ex* ex, int name, int ndims, int dtype, const int32_t* shape, bool zero, XArray** out) {
     CNH_CHECK(ndims >= 1 && ndims <= 3, -20, "array %d: unsupported rank %d", name, ndims);
     CNH_CHECK(dtype_size(dtype) != 0, -20, "array %d: unknown dtype %d", name, dtype);
@@ -321,8 +342,18 @@ int make_array(Ex* ex, int name, int ndims, int dtype, const int32_t* shape, boo
     }
     const int esz = dtype_size(dtype);
     int64_t off = 0;
-    a.flat = ndims == 3 && ex->flat3;
-    if (a.flat) {
+    a.flat = flat_rule(ex, ndims, a.shape, a.tile, a.offset);
+    if (a.flat && ndims == 2) {
+        a.pitch[1] = 1;
+        a.pitch[0] = a.shape[1];
+        for (int64_t t = 0; t < a.ntiles; ++t) {
+            int32_t lo[3], ext[3];
+            a.tile_extent(t, lo, ext);
+            a.tile_off.push_back((lo[0] * a.pitch[0] + lo[1]) * esz);
+            a.tile_elems.push_back((int64_t)ext[0] * ext[1]);
+        }
+        off = a.elems * esz;
+    } else if (a.flat) {
         a.pitch[2] = 1;
         a.pitch[1] = a.shape[2];
         a.pitch[0] = (int64_t)a.shape[1] * a.shape[2];
@@ -1493,7 +1524,10 @@ int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root, const Dag
             if (Cc)
                 Cc->tile_extent((int64_t)ci * Cc->grid[1] + cj, clo, cext);
             char* const ctile = Cc ? static_cast<char*>(Cc->tiles[(size_t)ci * Cc->grid[1] + cj]) : dest_base;
-            const int64_t cld = Cc ? cext[1] : dest_ld;
+            int64_t cstr[3] = {dest_ld, 1, 1};
+            if (Cc)
+                Cc->tile_strides(cext, cstr);   // a tile's own width, or the pitch of a block
+            const int64_t cld = cstr[0];
             // rows i of this C tile are rows A.r0 + i of A's array, its columns j are columns
             // B.c0 + j of B's: cut both ranges where those arrays' tiles end
             for (int r0 = clo[0]; r0 < clo[0] + cext[0];) {
@@ -1685,10 +1719,12 @@ int exec_diag(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
         ++copies;
         if (ex->dry)
             continue;
-        const int64_t first = (int64_t)(i0 + r_off - lo[0]) * ext[1] + (i0 + c_off - lo[1]);
+        int64_t tstr[3];
+        mat->tile_strides(ext, tstr);           // row stride: the tile's own width, or the block's pitch
+        const int64_t first = (int64_t)(i0 + r_off - lo[0]) * tstr[0] + (i0 + c_off - lo[1]);
         char* mp = static_cast<char*>(mat->tiles[(size_t)t]) + first * esz;
         char* vp = static_cast<char*>(vec->tiles[0]) + (int64_t)i0 * esz; // 1-D arrays are contiguous
-        const int64_t mstr[1] = {ext[1] + 1}, vstr[1] = {1}, zero[1] = {0}, one[1] = {1}, cnt[1] = {i1 - i0};
+        const int64_t mstr[1] = {tstr[0] + 1}, vstr[1] = {1}, zero[1] = {0}, one[1] = {1}, cnt[1] = {i1 - i0};
         const int rc = in->ndims == 1
                            ? cnh_copy_region(1, esz, mp, mstr, zero, one, vp, vstr, zero, one, cnt, ex->stream)
                            : cnh_copy_region(1, esz, vp, vstr, zero, one, mp, mstr, zero, one, cnt, ex->stream);
@@ -2124,7 +2160,7 @@ int try_statement_run(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t*
 
 // Will an array of `shape`, created now, have exactly the tiles of `a`?
 bool laid_out_like_new(const Ex* ex, const XArray& a, int nd, const int32_t* shape) {
-    if (a.ndims != nd || a.tile != tile_rule(ex, nd, shape) || a.flat != (nd == 3 && ex->flat3))
+    if (a.ndims != nd || a.tile != tile_rule(ex, nd, shape) || a.flat != flat_rule(ex, nd, shape, a.tile, nullptr))
         return false;
     for (int d = 0; d < nd; ++d)
         if (a.shape[d] != shape[d] || a.offset[d] % a.tile != 0)
@@ -3957,8 +3993,10 @@ int cnx_fill_cg_matrix(cnx_executor* ex, int name, uint64_t seed) {
     for (int64_t t = 0; t < a->ntiles; ++t) {
         int32_t lo[3], ext[3];
         a->tile_extent(t, lo, ext);
+        int64_t tstr[3];
+        a->tile_strides(ext, tstr);
         if (int rc = cnh_fill_cg_matrix(static_cast<double*>(a->tiles[t]), a->shape[0], lo[0], ext[0], lo[1],
-                                        ext[1], ext[1], seed, ex->stream))
+                                        ext[1], tstr[0], seed, ex->stream))
             return rc;
     }
     return 0;

@@ -940,8 +940,10 @@ struct FlatArgsDev {
     int32_t shape[3], rs[3], re[3], py, pz, nb[3], ob[3], nblocks8;
     FDivDev per_block, gb1, gb2, obx, oby;
     void* slots;
+    int32_t sub8;
+    FDivDev fsub;
 };
-static_assert(sizeof(FlatArgsDev) == 16 + 8 * kDirectMaxOther + 4 * 18 + 12 * 5 + 4 + 8,
+static_assert(sizeof(FlatArgsDev) == 16 + 8 * kDirectMaxOther + 4 * 18 + 12 * 5 + 4 + 8 + 16,
               "FlatArgsDev layout must match the generated struct");
 
 // A launch that should also reduce what it changes: mode 1 = sum of (new - old)^2, 2 = max
@@ -1043,16 +1045,11 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
     }
     if (arrays[0]->tile != cur->tile || arrays[0]->tiles[0] != cur->tiles[0] || vol >= (1ll << 31))
         return 0;
-    if (cur->shape[nd - 1] % 2 != 0)
-        return 0;
-    for (int64_t t = 0; t < ntiles; ++t) {
+    for (int64_t t = 0; t < ntiles; ++t)
         if (cur->tiles[t] == dst->tiles[t])
             return 0; // in place: a sweep would read values it has already written
-        if (((uintptr_t)cur->tiles[t] & 15) || ((uintptr_t)dst->tiles[t] & 15))
-            return 0;
-    }
     // Pitched tiles (views into one row-major block): every array of the launch has to use the
-    // same pitches, even along the rows, and a pitch of 1 along them.
+    // same pitches, with a pitch of 1 along the rows.
     int64_t pitch[3] = {0, 0, 0};
     bool pitched = false;
     for (int d = 0; d < nd; ++d)
@@ -1064,7 +1061,7 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
                 return 0;
             pitch[pad + d] = cur->pitch[d];
         }
-        if (pitch[2] != 1 || pitch[1] % 2 != 0 || (nd == 3 && pitch[0] % 2 != 0))
+        if (pitch[2] != 1)
             return 0;
     }
     auto same_pitch = [&](const cnh_tiled* t) {
@@ -1087,8 +1084,17 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
         // (an operand at the element's own position may be the target itself when the window
         // array is another one: a lane then reads the very elements it writes)
         for (int64_t t = 0; t < ntiles; ++t)
-            if (((uintptr_t)o->tiles[t] & 15) || (!sh.masked && o->tiles[t] == dst->tiles[t]))
+            if (!sh.masked && o->tiles[t] == dst->tiles[t])
                 return 0;
+    }
+    // Pairs of elements move as 128-bit accesses where every pair is 16-byte aligned: even rows
+    // and pitches, aligned tile starts. The whole-array kernel below also has a form for the rest
+    // (rows of odd length, the 2^k + 1 grids of multigrid); the per-tile kernels need the alignment.
+    bool aligned = cur->shape[nd - 1] % 2 == 0 && pitch[1] % 2 == 0 && pitch[0] % 2 == 0;
+    for (int64_t t = 0; t < ntiles && aligned; ++t) {
+        aligned = !(((uintptr_t)cur->tiles[t] | (uintptr_t)dst->tiles[t]) & 15);
+        for (int j = 0; j < n_other && aligned; ++j)
+            aligned = !((uintptr_t)others[j]->tiles[t] & 15);
     }
     // Every array of the launch one row-major block behind its tile views: no tile logic at all.
     if (pitched && g_direct_flat) {
@@ -1111,7 +1117,7 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
             }
             return true;
         };
-        bool flat = one_block(cur) && one_block(dst) && pitch[1] >= cur->shape[nd - 1] &&
+        bool flat = one_block(cur) && one_block(dst) && pitch[1] >= cur->shape[nd - 1] && cur->shape[nd - 1] >= 2 &&
                     (nd < 3 || pitch[0] >= pitch[1] * cur->shape[1]) &&
                     pitch[0] * (nd == 3 ? cur->shape[0] : 1) + pitch[1] * cur->shape[nd - 2] < (1ll << 31);
         for (int j = 0; j < n_other && flat; ++j)
@@ -1146,12 +1152,24 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
                 const int want = g_flat_ob[d] > 0 ? g_flat_ob[d] : dflt[d];
                 f.ob[d] = std::max(1, std::min(f.nb[d], want / foot[d]));
                 gb[d] = (f.nb[d] + f.ob[d] - 1) / f.ob[d];
+                // as many blocks as that, of equal size: a 257-wide array gets blocks of 129 + 128
+                // columns' worth of workgroups instead of 256 + 1
+                f.ob[d] = (int32_t)((f.nb[d] + gb[d] - 1) / gb[d]);
                 launched *= gb[d] * f.ob[d];
             }
             CNH_CHECK(launched > 0 && launched < (1ll << 31), -3, "stencil launch of %lld workgroups",
                       (long long)launched);
             f.nblocks8 = launched % 8 == 0 ? (int32_t)(launched / 8) : 0;
             f.per_block = fdiv_make((uint32_t)(f.ob[0] * f.ob[1] * f.ob[2]));
+            {
+                // a grid that does not fill its ordering blocks: spread every block over the XCDs
+                bool ragged = false;
+                for (int d = 0; d < 3; ++d)
+                    ragged = ragged || f.nb[d] % f.ob[d] != 0;
+                const int64_t per = (int64_t)f.ob[0] * f.ob[1] * f.ob[2];
+                f.sub8 = ragged && per % 8 == 0 && launched > per ? (int32_t)(per / 8) : 0;
+                f.fsub = fdiv_make((uint32_t)std::max(1, f.sub8));
+            }
             f.gb1 = fdiv_make((uint32_t)gb[1]);
             f.gb2 = fdiv_make((uint32_t)gb[2]);
             f.obx = fdiv_make((uint32_t)f.ob[2]);
@@ -1167,13 +1185,15 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
                 f.slots = slots;
                 DirectConfig rcfg = g_direct_cfg;
                 rcfg.reduce = true;
-                const char* name = red->mode == 1 ? (nts ? "grp_direct_flat_red1_nts" : "grp_direct_flat_red1")
-                                                  : (nts ? "grp_direct_flat_red2_nts" : "grp_direct_flat_red2");
-                if (int rc = get_function(k, rcfg.variant(), name, &fn))
+                const std::string name = std::string(aligned ? "grp_direct_flat_red" : "grp_direct_flatu_red") +
+                                         (red->mode == 1 ? "1" : "2") + (nts ? "_nts" : "");
+                if (int rc = get_function(k, rcfg.variant(), name.c_str(), &fn))
                     return rc;
-            } else if (int rc = get_function(k, g_direct_cfg.variant(),
-                                             nts ? "grp_direct_flat_nts" : "grp_direct_flat", &fn))
-                return rc;
+            } else {
+                const std::string name = std::string(aligned ? "grp_direct_flat" : "grp_direct_flatu") + (nts ? "_nts" : "");
+                if (int rc = get_function(k, g_direct_cfg.variant(), name.c_str(), &fn))
+                    return rc;
+            }
             void* params[] = {&f, const_cast<unsigned char*>(scal.data())};
             if (int rc = launch(fn, launched, params, st))
                 return rc;
@@ -1187,6 +1207,8 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
             return 0;
         }
     }
+    if (!aligned)
+        return 0;
     DirectArgsDev a;
     std::memset(&a, 0, sizeof a);
     a.tile = cur->tile;
