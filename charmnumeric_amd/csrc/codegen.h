@@ -102,6 +102,8 @@ struct DirectShape {
     int halo[3] = {0, 0, 0};
     int tx = 0, ty = 0, ry = 0, rz = 0;
     std::vector<std::array<int, 3>> shifts; // per distinct load, dims padded to (z, y, x)
+    std::vector<std::array<int, 3>> shifts2; // the same for the second root of a lattice pair (a load
+                                             // both roots use may sit at another offset from each lattice)
     // per distinct load: -1 = the assigned array itself (read through the window), else which of
     // the other arrays it reads at the element's own position (source terms, weights)
     std::vector<int> other;
@@ -111,6 +113,13 @@ struct DirectShape {
     // launch then reads its tiles and writes the assigned elements of the target, nothing else.
     int window_name = 0;
     bool masked = false;
+    // Lattices: every region of the group has the same step (1 or 2) per dimension, lat[d] = step - 1
+    // in kernel dimensions (z, y, x). One or two SET_REGION roots on the same array whose lattices
+    // share no point (the two halves of one colour of a red-black sweep). inplace_safe: no shifted
+    // read of the assigned array can meet an assigned point, so the sweep may run in place.
+    int lat[3] = {0, 0, 0};
+    int nroots = 1;
+    bool lattice = false, inplace_safe = false;
 };
 constexpr int kDirectMaxOther = 4;
 int direct_shape(const GroupProgram& p, const DirectConfig& cfg, DirectShape& sh, std::string& err);

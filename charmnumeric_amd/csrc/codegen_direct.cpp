@@ -23,39 +23,99 @@ int direct_shape(const GroupProgram& p, const DirectConfig& cfg, DirectShape& sh
         err = "register-window stencil needs rank 2 or 3";
         return -18;
     }
-    if (p.out_roots.size() != 1 || !p.out_is_set_region[0] || p.out_region[0].is_global) {
-        err = "register-window stencil needs a single SET_REGION root";
+    const int nroots = (int)p.out_roots.size();
+    if (nroots < 1 || nroots > 2) {
+        err = "register-window stencil needs one or two SET_REGION roots";
         return -18;
     }
+    for (int j = 0; j < nroots; ++j)
+        if (!p.out_is_set_region[(size_t)j] || p.out_region[(size_t)j].is_global || p.out_reduce[(size_t)j] ||
+            p.out_target[(size_t)j] != p.out_target[0]) {
+            err = "register-window stencil needs SET_REGION roots on one array";
+            return -18;
+        }
+    sh.nroots = nroots;
     // A lane works on pairs of elements: 16-byte accesses for 8-byte types, 8-byte accesses for
     // 4-byte types (half the width per access, still one coalesced run per wavefront).
     const cnh_region& ro = p.out_region[0];
     const int nd = p.ndims, pad = CNH_MAX_ND - nd;
-    for (int d = 0; d < nd; ++d)
-        if (ro.step[d] != 1) {
-            err = "assigned region is strided";
+    for (int d = 0; d < nd; ++d) {
+        if (ro.step[d] != 1 && ro.step[d] != 2) {
+            err = "assigned region has a step other than 1 or 2";
             return -18;
         }
+        sh.lat[pad + d] = ro.step[d] - 1;
+        sh.lattice = sh.lattice || ro.step[d] == 2;
+    }
+    sh.lattice = sh.lattice || nroots == 2;
+    for (int j = 1; j < nroots; ++j) {
+        const cnh_region& rj = p.out_region[(size_t)j];
+        bool apart = false;
+        for (int d = 0; d < nd; ++d) {
+            if (rj.step[d] != ro.step[d]) {
+                err = "the roots' regions differ in step";
+                return -18;
+            }
+            apart = apart || (ro.step[d] == 2 && ((rj.start[d] - ro.start[d]) & 1) != 0);
+        }
+        if (!apart) {
+            err = "the roots' lattices can meet";
+            return -18;
+        }
+    }
     if (p.load_leaf.empty()) {
         err = "no array operand";
         return -18;
     }
-    sh.shifts.assign(p.load_leaf.size(), {0, 0, 0});
-    sh.other.assign(p.load_leaf.size(), -1);
-    // The window array: the one array read at positions other than the element's own; the
-    // assigned array when there is none.
-    sh.window_name = p.out_target[0];
-    bool found_shifted = false;
-    for (size_t l = 0; l < p.load_leaf.size(); ++l) {
-        const LeafUse& u = p.leaves[p.load_leaf[l]];
+    // the SET_REGION root a leaf use works for: the first output at or after its root position
+    auto owner_of = [&](const LeafUse& u) {
+        for (int j = 0; j < nroots; ++j)
+            if (p.out_roots[(size_t)j] >= u.root)
+                return j;
+        return nroots - 1;
+    };
+    const size_t NLd = p.load_leaf.size();
+    sh.shifts.assign(NLd, {0, 0, 0});
+    sh.shifts2.assign(NLd, {0, 0, 0});
+    sh.other.assign(NLd, -1);
+    // every use of a load by one root must sit at the same offset from that root's lattice
+    std::vector<std::array<int, 3>> rel[2] = {std::vector<std::array<int, 3>>(NLd, {0, 0, 0}),
+                                               std::vector<std::array<int, 3>>(NLd, {0, 0, 0})};
+    std::vector<int> seen[2] = {std::vector<int>(NLd, 0), std::vector<int>(NLd, 0)};
+    for (const LeafUse& u : p.leaves) {
         if (!u.has_region) {
             err = "operand without a region";
             return -18;
         }
-        bool shifted = false;
-        for (int d = 0; d < nd; ++d)
-            shifted = shifted || u.region.start[d] != ro.start[d];
-        if (!shifted)
+        const int j = owner_of(u);
+        const cnh_region& rr = p.out_region[(size_t)j];
+        std::array<int, 3> off = {0, 0, 0};
+        for (int d = 0; d < nd; ++d) {
+            if (u.region.step[d] != rr.step[d] ||
+                (u.region.stop[d] - u.region.start[d] + rr.step[d] - 1) / rr.step[d] !=
+                    (rr.stop[d] - rr.start[d] + rr.step[d] - 1) / rr.step[d]) {
+                err = "operand region differs from the assigned one in step or extent";
+                return -18;
+            }
+            off[(size_t)(pad + d)] = u.region.start[d] - rr.start[d];
+        }
+        if (seen[j][(size_t)u.load] && rel[j][(size_t)u.load] != off) {
+            err = "one load is used at two offsets";
+            return -18;
+        }
+        seen[j][(size_t)u.load] = 1;
+        rel[j][(size_t)u.load] = off;
+    }
+    auto shifted_at = [&](int j, size_t l) {
+        return seen[j][l] && (rel[j][l][0] != 0 || rel[j][l][1] != 0 || rel[j][l][2] != 0);
+    };
+    // The window array: the one array read at positions other than the element's own; the
+    // assigned array when there is none.
+    sh.window_name = p.out_target[0];
+    bool found_shifted = false;
+    for (size_t l = 0; l < NLd; ++l) {
+        const LeafUse& u = p.leaves[p.load_leaf[l]];
+        if (!shifted_at(0, l) && !shifted_at(1, l))
             continue;
         if (found_shifted && u.name != sh.window_name) {
             err = "two arrays are read at shifted positions";
@@ -65,17 +125,20 @@ int direct_shape(const GroupProgram& p, const DirectConfig& cfg, DirectShape& sh
         sh.window_name = u.name;
     }
     sh.masked = sh.window_name != p.out_target[0];
+    if (sh.masked && sh.lattice) {
+        err = "a lattice sweep reads its own array through the window";
+        return -18;
+    }
     bool reads_target = false;
-    for (size_t l = 0; l < p.load_leaf.size(); ++l) {
+    sh.inplace_safe = sh.lattice;
+    for (size_t l = 0; l < NLd; ++l) {
         const LeafUse& u = p.leaves[p.load_leaf[l]];
         if (u.name != sh.window_name) {
             // another array (a source term, a weight): only at the element's own position
-            for (int d = 0; d < nd; ++d)
-                if (u.region.step[d] != 1 || u.region.start[d] != ro.start[d] ||
-                    u.region.stop[d] != ro.stop[d]) {
-                    err = "operand of another array is shifted";
-                    return -18;
-                }
+            if (shifted_at(0, l) || shifted_at(1, l)) {
+                err = "operand of another array is shifted";
+                return -18;
+            }
             size_t j = 0;
             while (j < sh.other_names.size() && sh.other_names[j] != u.name)
                 ++j;
@@ -90,15 +153,25 @@ int direct_shape(const GroupProgram& p, const DirectConfig& cfg, DirectShape& sh
             continue;
         }
         reads_target = true;
-        for (int d = 0; d < nd; ++d) {
-            if (u.region.step[d] != 1 ||
-                u.region.stop[d] - u.region.start[d] != ro.stop[d] - ro.start[d]) {
-                err = "operand region is strided or of a different extent";
-                return -18;
+        for (int j = 0; j < nroots; ++j) {
+            if (!seen[j][l])
+                continue;
+            for (int d = 0; d < 3; ++d) {
+                (j == 0 ? sh.shifts : sh.shifts2)[l][(size_t)d] = rel[j][l][(size_t)d];
+                sh.halo[d] = std::max(sh.halo[d], std::abs(rel[j][l][(size_t)d]));
             }
-            int s = u.region.start[d] - ro.start[d];
-            sh.shifts[l][pad + d] = s;
-            sh.halo[pad + d] = std::max(sh.halo[pad + d], std::abs(s));
+            // in place: a shifted read must miss every assigned lattice in some stepped dimension
+            if (sh.lattice && shifted_at(j, l)) {
+                const cnh_region& rr = p.out_region[(size_t)j];
+                for (int q = 0; q < nroots; ++q) {
+                    const cnh_region& rq = p.out_region[(size_t)q];
+                    bool misses = false;
+                    for (int d = 0; d < nd; ++d)
+                        misses = misses || (rq.step[d] == 2 &&
+                                            ((rr.start[d] + rel[j][l][(size_t)(pad + d)] - rq.start[d]) & 1) != 0);
+                    sh.inplace_safe = sh.inplace_safe && misses;
+                }
+            }
         }
     }
     if (!reads_target) {
@@ -153,9 +226,13 @@ std::string direct_source(const GroupProgram& p, const DirectConfig& cfg, std::s
         for (int ry = 0; ry < sh.ry; ++ry) {
             if (!sh.masked)
                 at(rz + H0, ry + H1, HK) = 1; // the element itself (kept outside the assigned region)
-            for (int e = 0; e < 2; ++e)
+            for (int e = 0; e < 2; ++e) {
                 for (const auto& s : sh.shifts)
                     at(rz + H0 + s[0], ry + H1 + s[1], HK + floordiv2(e + s[2])) = 1;
+                if (sh.nroots > 1)
+                    for (const auto& s : sh.shifts2)
+                        at(rz + H0 + s[0], ry + H1 + s[1], HK + floordiv2(e + s[2])) = 1;
+            }
         }
     std::ostringstream s;
     s << pre;
@@ -168,6 +245,11 @@ std::string direct_source(const GroupProgram& p, const DirectConfig& cfg, std::s
         s << (l ? ", " : "") << "{" << sh.shifts[l][0] << ", " << sh.shifts[l][1] << ", "
           << sh.shifts[l][2] << "}";
     s << "};\n";
+    s << "__device__ constexpr int DR_SHIFT2[NLA][3] = {";
+    for (size_t l = 0; l < sh.shifts2.size(); ++l)
+        s << (l ? ", " : "") << "{" << sh.shifts2[l][0] << ", " << sh.shifts2[l][1] << ", "
+          << sh.shifts2[l][2] << "}";
+    s << "};\n#define DR_NROOTS " << sh.nroots << "\n";
     const int NOTH = (int)sh.other_names.size();
     s << "#define DR_MASKED " << (sh.masked ? 1 : 0) << "\n";
     s << "#define DR_RED " << (cfg.reduce ? 1 : 0) << "\n";
@@ -737,6 +819,9 @@ struct FlatArgs {
     T* slots;              // reducing launches: one partial per launched wavefront
     int sub8;              // ragged grids: workgroups per ordering block / 8, else 0
     FDiv fsub;             // = sub8
+    int lat[3];            // step - 1 of every region per dimension (0: unit step, 1: every other point)
+    int nroots;            // 1, or 2: a second assigned lattice [rs2, re2) with the same steps
+    int rs2[3], re2[3];
 };
 
 // Rows of odd length, odd pitches or a block that does not start on a 16-byte boundary (UA): pairs
@@ -884,15 +969,20 @@ __device__ __forceinline__ void direct_flat(const FlatArgs& a, const T* s) {
             }
     }
     T* const dst = a.dst;
+    // A sweep in place (a lattice whose shifted reads never meet an assigned point) leaves rows
+    // without assigned points alone; one into a second buffer writes every element of it.
+    const bool inplace = a.cur == a.dst;
     T acc = (T)0;
 #pragma unroll
     for (int rz = 0; rz < DR_RZ; ++rz) {
         const int z = z0 + rz;
-        const bool zin = z >= a.rs[0] && z < a.re[0];
+        const bool zin = z >= a.rs[0] && z < a.re[0] && ((z - a.rs[0]) & a.lat[0]) == 0;
+        const bool zin2 = DR_NROOTS > 1 && a.nroots > 1 && z >= a.rs2[0] && z < a.re2[0] && ((z - a.rs2[0]) & a.lat[0]) == 0;
 #pragma unroll
         for (int ry = 0; ry < DR_RY; ++ry) {
             const int y = y0 + ry;
-            const bool yin = zin && y >= a.rs[1] && y < a.re[1];
+            const bool yin = zin && y >= a.rs[1] && y < a.re[1] && ((y - a.rs[1]) & a.lat[1]) == 0;
+            const bool yin2 = zin2 && y >= a.rs2[1] && y < a.re2[1] && ((y - a.rs2[1]) & a.lat[1]) == 0;
             P2 res;
             bool in_e[2];
 #pragma unroll
@@ -907,9 +997,28 @@ __device__ __forceinline__ void direct_flat(const FlatArgs& a, const T* s) {
                                     [DR_HK + floordiv2(xx)][xx & 1];
                 }
                 group_eval(l, s, o);
+                T second = o[0];
+                if (DR_NROOTS > 1) {
+                    // the second root reads its operands at its own offsets (a load both roots use
+                    // sits at another offset from each lattice)
+                    T l2[NLA], o2[NOA];
+#pragma unroll
+                    for (int q = 0; q < NL; ++q) {
+                        const int xx = e + DR_SHIFT2[q][2];
+                        l2[q] = DR_OTHER[q] >= 0
+                                    ? ov[DR_OTHER[q] >= 0 ? DR_OTHER[q] : 0][rz][ry][e]
+                                    : win[rz + DR_H0 + DR_SHIFT2[q][0]][ry + DR_H1 + DR_SHIFT2[q][1]]
+                                         [DR_HK + floordiv2(xx)][xx & 1];
+                    }
+                    group_eval(l2, s, o2);
+                    second = o2[NO > 1 ? 1 : 0];
+                }
                 const int gx = lx + e;
-                in_e[e] = yin && gx >= a.rs[2] && gx < a.re[2];
-                res[e] = (DR_MASKED || in_e[e]) ? o[0] : win[rz + DR_H0][ry + DR_H1][DR_HK][e];
+                const bool in1 = yin && gx >= a.rs[2] && gx < a.re[2] && ((gx - a.rs[2]) & a.lat[2]) == 0;
+                const bool in2 = yin2 && gx >= a.rs2[2] && gx < a.re2[2] && ((gx - a.rs2[2]) & a.lat[2]) == 0;
+                in_e[e] = in1 || in2;
+                const T mine = in2 ? second : o[0];
+                res[e] = (DR_MASKED || in_e[e]) ? mine : win[rz + DR_H0][ry + DR_H1][DR_HK][e];
                 if (RED) {
                     // assigned elements of live lanes only (rows and planes beyond the array are
                     // never assigned: the region lies inside it)
@@ -920,7 +1029,7 @@ __device__ __forceinline__ void direct_flat(const FlatArgs& a, const T* s) {
                 }
             }
             // rows and planes beyond the array (a ragged last workgroup) and idle lanes store nothing
-            if (live && z < S0 && y < S1)
+            if (live && z < S0 && y < S1 && (!inplace || yin || yin2))
                 store_pair_flat<NTS, UA>(dst + (z * PZ + y * PY + lx), res, in_e[0], in_e[1], live1);
         }
     }

@@ -3189,6 +3189,204 @@ int try_dense_run(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t* use
     return 0;
 }
 
+// ---- two lattices of one colour as one sweep ----
+//
+// A red-black sweep (examples/gauss_seidel.py upstream) updates each colour with two statements,
+//   phi[1:-1:2, 1:-1:2] = f(neighbours, g[1:-1:2, 1:-1:2]);  phi[2:-1:2, 2:-1:2] = f(...)
+// which read only points of the other colour: neither reads what the other assigns. Run one by one
+// each is a pass of its own over all of phi's cache lines. Together they are one pass: a group with
+// two SET_REGION roots, launched as a register-window sweep that evaluates both at every point and
+// stores whichever lattice the point belongs to, in place. That sweep works on arrays stored as one
+// row-major block, so arrays still cut into tiles with buffers of their own are laid out anew
+// first (once: they stay that way).
+
+// Stores `a` as one row-major block (tiles become views into it).
+int make_block(Ex* ex, XArray& a) {
+    if (a.flat)
+        return 0;
+    CNH_CHECK(!a.phased(), -26, "array %d: tiles that do not start at element 0", a.name);
+    const int esz = dtype_size(a.dtype), nd = a.ndims;
+    const size_t bytes = (size_t)std::max<int64_t>(((int64_t)a.elems * esz + 255) & ~(int64_t)255, 256);
+    void* block = nullptr;
+    if (int rc = slab_alloc(ex, bytes, false, &block))
+        return rc;
+    int64_t pitch[3] = {0, 0, 0};
+    {
+        int64_t run = 1;
+        for (int d = nd - 1; d >= 0; --d) {
+            pitch[d] = run;
+            run *= a.shape[d];
+        }
+    }
+    std::vector<int64_t> offs;
+    for (int64_t t = 0; t < a.ntiles; ++t) {
+        int32_t lo[3], ext[3];
+        a.tile_extent(t, lo, ext);
+        int64_t sstr[3], zero[3] = {0, 0, 0}, one[3] = {1, 1, 1}, counts[3] = {1, 1, 1}, off = 0;
+        a.tile_strides(ext, sstr);
+        for (int d = 0; d < nd; ++d) {
+            counts[d] = ext[d];
+            off += lo[d] * pitch[d];
+        }
+        offs.push_back(off * esz);
+        if (!ex->dry)
+            if (int rc = cnh_copy_region(nd, esz, static_cast<char*>(block) + off * esz, pitch, zero, one, a.tiles[(size_t)t],
+                                         sstr, zero, one, counts, ex->stream))
+                return rc;
+    }
+    slab_release(ex, a.bytes, a.slab);
+    slab_release(ex, a.bytes, a.alt);
+    a.slab = block;
+    a.alt = nullptr;
+    a.alt_tiles.clear();
+    a.bytes = bytes;
+    a.flat = true;
+    for (int d = 0; d < 3; ++d)
+        a.pitch[d] = d < nd ? pitch[d] : 0;
+    a.tile_off = offs;
+    for (int64_t t = 0; t < a.ntiles; ++t)
+        a.tiles[(size_t)t] = static_cast<char*>(block) + offs[(size_t)t];
+    ex->log("block " + std::to_string(a.name) + " tiles=" + std::to_string(a.ntiles));
+    return 0;
+}
+
+// `target[lattice] = f(...)` with steps of 1 or 2, at least one of them 2, on an array of rank 2 or 3.
+bool lattice_statement(Ex* ex, const DagNode& n, XArray** target, const cnh_ast_node** set) {
+    if (!n.fusible || n.roots.empty())
+        return false;
+    const cnh_ast_node& root = n.nodes[n.roots.back()];
+    if (root.opcode != CNH_OP_SET_REGION || root.n_operands != 2 || root.region.is_global ||
+        n.nodes[root.operands[1]].is_scalar)
+        return false;
+    for (size_t r = 0; r + 1 < n.roots.size(); ++r)
+        if (!n.nodes[n.roots[r]].is_temp)
+            return false;
+    auto it = ex->arrays.find(n.nodes[root.operands[0]].result_name);
+    if (it == ex->arrays.end() || it->second.ndims < 2 || it->second.ndims != root.region.ndims)
+        return false;
+    bool stepped = false;
+    for (int d = 0; d < root.region.ndims; ++d) {
+        if (root.region.step[d] != 1 && root.region.step[d] != 2)
+            return false;
+        stepped = stepped || root.region.step[d] == 2;
+    }
+    *target = &it->second;
+    *set = &root;
+    return stepped;
+}
+
+int try_lattice_pair(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t* used, bool* open_ended) {
+    *used = 0;
+    *open_ended = false;
+    XArray *ta = nullptr, *tb = nullptr;
+    const cnh_ast_node *sa = nullptr, *sb = nullptr;
+    if (!lattice_statement(ex, dag[i], &ta, &sa))
+        return 0;
+    std::vector<int> dels;
+    const size_t j = skip_deletions(dag, i + 1, dels);
+    if (j == dag.size()) {
+        *open_ended = open_ended_allowed(ex);
+        return 0;
+    }
+    if (!lattice_statement(ex, dag[j], &tb, &sb) || tb != ta)
+        return 0;
+    for (int d = 0; d < sa->region.ndims; ++d)
+        if (sa->region.step[d] != sb->region.step[d])
+            return 0;
+    for (int name : dels)
+        if (name == ta->name)
+            return 0;
+    // one group: the first statement's roots, then the second's
+    DagNode merged;
+    merged.id = dag[i].id;
+    merged.fusible = 1;
+    int next_literal = -1, next_temporary = 0x7c000000;
+    for (const DagNode* n : {&dag[i], &dag[j]}) {
+        const int base = (int)merged.nodes.size();
+        for (const cnh_ast_node& a : n->nodes) {
+            merged.nodes.push_back(a);
+            cnh_ast_node& c = merged.nodes.back();
+            for (int oi = 0; oi < c.n_operands; ++oi)
+                if (c.operands[oi] >= 0)
+                    c.operands[oi] += base;
+            if (c.is_scalar)
+                c.result_name = next_literal--;
+        }
+        std::map<int, int> renamed;
+        for (size_t ri = 0; ri + 1 < n->roots.size(); ++ri)
+            renamed[n->nodes[(size_t)n->roots[ri]].result_name] = next_temporary++;
+        for (size_t q = (size_t)base; q < merged.nodes.size(); ++q) {
+            cnh_ast_node& c = merged.nodes[q];
+            auto it = c.is_scalar ? renamed.end() : renamed.find(c.result_name);
+            if (it != renamed.end())
+                c.result_name = it->second;
+        }
+        merged.nodes[(size_t)base + (size_t)n->roots.back()].result_name = next_temporary++;
+        for (int32_t r : n->roots)
+            merged.roots.push_back(base + r);
+    }
+    Group g;
+    canonicalise(merged, g);
+    cnh_kernel* k = nullptr;
+    if (int rc = compile_cached(ex, g, &k))
+        return rc;
+    if (cnh_kernel_lattice(k) != 2)
+        return 0;                               // not two lattices that can be swept in place
+    int n_in = 0, n_scalar = 0, n_out = 0;
+    if (int rc = cnh_kernel_signature(k, &n_in, &n_scalar, &n_out))
+        return rc;
+    std::vector<XArray*> in_arr((size_t)n_in);
+    for (int q = 0; q < n_in; ++q) {
+        int cname = 0, has = 0;
+        cnh_region reg;
+        if (int rc = cnh_kernel_input(k, q, &cname, &has, &reg))
+            return rc;
+        auto it = ex->arrays.find(g.canon_to_actual[cname]);
+        if (it == ex->arrays.end() || it->second.dtype != ta->dtype || it->second.ndims != ta->ndims ||
+            it->second.tile != ta->tile || it->second.phased())
+            return 0;
+        for (int d = 0; d < ta->ndims; ++d)
+            if (it->second.shape[d] != ta->shape[d])
+                return 0;
+        in_arr[(size_t)q] = &it->second;
+    }
+    if (ta->phased() || ta->elems >= (1ll << 31))
+        return 0;
+    std::vector<const void*> scalars((size_t)std::max(1, n_scalar), nullptr);
+    for (int q = 0; q < n_scalar; ++q) {
+        int cname = 0;
+        if (int rc = cnh_kernel_scalar(k, q, &cname))
+            return rc;
+        XArray* sarr;
+        if (int rc = find_array(ex, g.canon_to_actual[cname], &sarr, "broadcast scalar"))
+            return rc;
+        if (sarr->elems != 1 || sarr->dtype != ta->dtype)
+            return 0;
+        scalars[(size_t)q] = sarr->tiles[0];
+    }
+    // from here on the two statements are this launch
+    if (int rc = make_block(ex, *ta))
+        return rc;
+    for (XArray* a : in_arr)
+        if (int rc = make_block(ex, *a))
+            return rc;
+    std::vector<cnh_tiled> tin((size_t)std::max(1, n_in));
+    for (int q = 0; q < n_in; ++q)
+        tin[(size_t)q] = in_arr[(size_t)q]->tiled();
+    const cnh_tiled cur = ta->tiled();
+    ex->stats[5]++;
+    ex->log("group node=" + std::to_string(merged.id) + " path=lattices roots=2 inputs=" + std::to_string(n_in) +
+            " scalars=" + std::to_string(n_scalar) + " out=" + std::to_string(ta->name) + " inplace");
+    if (!ex->dry)
+        if (int rc = cnh_launch_group_tiles(k, n_in, tin.data(), n_scalar, scalars.data(), 1, &cur, &cur, ex->stream))
+            return rc;
+    for (int name : dels)
+        drop_array(ex, name);
+    ex->stats[2] += (int64_t)(j + 1 - i);
+    *used = j + 1 - i;
+    return 0;
+}
+
 int parse_dag(const char* msg, int64_t size, std::vector<DagNode>& out) {
     Reader r{msg, msg + size};
     int32_t magic = r.get<int32_t>(), version = r.get<int32_t>(), count = r.get<int32_t>();
@@ -3500,6 +3698,8 @@ int run_nodes(Ex* ex, std::vector<DagNode>& dag) {
             // ... everything else reads arrays as they are
             if (rc == 0 && used == 0 && !open_ended)
                 rc = resolve_all(ex);
+            if (rc == 0 && used == 0 && !open_ended)
+                rc = try_lattice_pair(ex, dag, i, &used, &open_ended);
             if (rc == 0 && used == 0 && !open_ended)
                 rc = try_product_into_region(ex, dag, i, &used, &open_ended);
             if (rc == 0 && used == 0 && !open_ended)

@@ -411,6 +411,16 @@ int cnh_kernel_variants_loaded(const cnh_kernel* k, const char* prefix) {
     return n;
 }
 
+int cnh_kernel_lattice(const cnh_kernel* k) {
+    if (k == nullptr)
+        return 0;
+    DirectShape sh;
+    std::string why;
+    if (direct_shape(k->prog, DirectConfig(), sh, why) != 0 || !sh.lattice)
+        return 0;
+    return sh.inplace_safe ? 2 : 1;
+}
+
 int cnh_kernel_build(cnh_kernel* k, const char* variant) {
     CNH_CHECK(k != nullptr && variant != nullptr, -2, "null argument");
     KernelVariant* v = nullptr;
@@ -942,8 +952,9 @@ struct FlatArgsDev {
     void* slots;
     int32_t sub8;
     FDivDev fsub;
+    int32_t lat[3], nroots, rs2[3], re2[3];
 };
-static_assert(sizeof(FlatArgsDev) == 16 + 8 * kDirectMaxOther + 4 * 18 + 12 * 5 + 4 + 8 + 16,
+static_assert(sizeof(FlatArgsDev) == 16 + 8 * kDirectMaxOther + 4 * 18 + 12 * 5 + 4 + 8 + 16 + 40,
               "FlatArgsDev layout must match the generated struct");
 
 // A launch that should also reduce what it changes: mode 1 = sum of (new - old)^2, 2 = max
@@ -1045,9 +1056,15 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
     }
     if (arrays[0]->tile != cur->tile || arrays[0]->tiles[0] != cur->tiles[0] || vol >= (1ll << 31))
         return 0;
+    // In place: a sweep would read values it has already written, unless it assigns a lattice that
+    // none of its shifted reads can meet (the colours of a red-black sweep).
+    bool inplace = false;
     for (int64_t t = 0; t < ntiles; ++t)
-        if (cur->tiles[t] == dst->tiles[t])
-            return 0; // in place: a sweep would read values it has already written
+        inplace = inplace || cur->tiles[t] == dst->tiles[t];
+    if (inplace && !(sh.lattice && sh.inplace_safe))
+        return 0;
+    if (inplace && red != nullptr && red->mode != 0)
+        return 0;                         // the old values do not survive: nothing to compare with
     // Pitched tiles (views into one row-major block): every array of the launch has to use the
     // same pitches, with a pitch of 1 along the rows.
     int64_t pitch[3] = {0, 0, 0};
@@ -1141,6 +1158,20 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
             }
             f.py = (int32_t)pitch[1];
             f.pz = (int32_t)pitch[0];
+            f.nroots = sh.nroots;
+            for (int d = 0; d < 3; ++d) {
+                f.lat[d] = sh.lat[d];
+                f.rs2[d] = 0;
+                f.re2[d] = 0;
+            }
+            if (sh.nroots > 1)
+                for (int d = 0; d < nd; ++d) {
+                    f.rs2[pad + d] = p.out_region[1].start[d];
+                    f.re2[pad + d] = p.out_region[1].stop[d];
+                }
+            if (sh.nroots > 1)
+                for (int d = 0; d < pad; ++d)
+                    f.re2[d] = 1;
             // a workgroup: 4 wavefronts stacked along y, each 128 columns x ry rows x rz planes
             const int foot[3] = {sh.rz, 4 * sh.ry, 128};
             // ordering block: 256^3 elements for rank 3 (measured on MI355X, 512^3: 382 us per
@@ -1176,7 +1207,7 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
             f.oby = fdiv_make((uint32_t)f.ob[1]);
             const bool nts = volume * 2 * esz >= (128ll << 20);
             hipFunction_t fn;
-            const bool reducing = red != nullptr && red->mode != 0 && p.dtype == CNH_F64;
+            const bool reducing = red != nullptr && red->mode != 0 && p.dtype == CNH_F64 && !sh.lattice;
             if (reducing) {
                 // one partial per launched wavefront, folded in index order by a second launch
                 void* slots = nullptr;
@@ -1207,8 +1238,8 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
             return 0;
         }
     }
-    if (!aligned)
-        return 0;
+    if (!aligned || sh.lattice)
+        return 0;                         // the per-tile kernels take aligned unit-step sweeps only
     DirectArgsDev a;
     std::memset(&a, 0, sizeof a);
     a.tile = cur->tile;
@@ -1566,7 +1597,12 @@ int launch_group_tiles_impl(cnh_kernel* k, int n_in, const cnh_tiled* in, int n_
     CNH_CHECK(k != nullptr, -2, "null kernel");
     const GroupProgram& p = k->prog;
     const int nd = p.ndims;
-    CNH_CHECK(p.out_roots.size() == 1, -17, "the tiled launch needs exactly one output root");
+    // two roots: the two lattices of one colour of a red-black sweep, for the lattice sweep below
+    const bool two_roots = p.out_roots.size() == 2 && p.out_is_set_region[0] && p.out_is_set_region[1] &&
+                           p.out_target[0] == p.out_target[1] && !p.out_region[0].is_global &&
+                           !p.out_region[1].is_global;
+    CNH_CHECK(p.out_roots.size() == 1 || two_roots, -17,
+              "the tiled launch needs one output root (or two SET_REGION roots on one array)");
     CNH_CHECK(n_in == (int)p.leaves.size(), -4, "group expects %d tiled inputs, got %d",
               (int)p.leaves.size(), n_in);
     if (int rc = check_tiled(dst, nd, "dst"))
@@ -1643,6 +1679,13 @@ int launch_group_tiles_impl(cnh_kernel* k, int n_in, const cnh_tiled* in, int n_
             CNH_CHECK(step >= 1, -4, "input %d: step %d in dim %d", l, step, d);
             int count = (stop - start + step - 1) / step;
             int ocount = (re[pad + d] - rs[pad + d] + rst[pad + d] - 1) / rst[pad + d];
+            if (two_roots && p.out_roots[0] < u.root) {   // a leaf of the second root
+                const cnh_region& r2 = p.out_region[1];
+                CNH_CHECK(r2.step[d] >= 1 && r2.start[d] >= 0 && r2.stop[d] <= dst->shape[d], -4,
+                          "second assigned region [%d:%d:%d] does not fit the target extent %d in dim %d",
+                          r2.start[d], r2.stop[d], r2.step[d], dst->shape[d], d);
+                ocount = (r2.stop[d] - r2.start[d] + r2.step[d] - 1) / r2.step[d];
+            }
             CNH_CHECK(count == ocount, -4,
                       "input %d has %d elements in dim %d, the assigned region has %d", l, count, d,
                       ocount);
@@ -1666,6 +1709,8 @@ int launch_group_tiles_impl(cnh_kernel* k, int n_in, const cnh_tiled* in, int n_
         bool pitched = is_pitched(dst) || (cur && is_pitched(cur));
         for (const cnh_tiled* a : arrays)
             pitched = pitched || is_pitched(a);
+        CNH_CHECK(!two_roots, -17, "a group with two SET_REGION roots runs as a lattice sweep over arrays "
+                  "stored as one block, and this one does not fit it");
         if (!pitched)
             if (int rc = try_launch_slide(k, arrays, cur, dst, scal, st, &handled))
                 return rc;

@@ -208,6 +208,13 @@ int cnh_kernel_output(const cnh_kernel* k, int i, int* result_name, int* target_
 int64_t cnh_kernel_source(cnh_kernel* k, const char* variant, char* buf, size_t cap);
 /* Builds the code object of one variant for gfx950 without loading it (works without a GPU). */
 int cnh_kernel_build(cnh_kernel* k, const char* variant);
+/* Can the group run as a register-window sweep over a lattice (cnh_launch_group_tiles on arrays
+ * stored as one block)? Every region of it then has the same step, 1 or 2, per dimension, its one or
+ * two SET_REGION roots assign lattices of one array that share no point (two: the halves of one
+ * colour of a red-black sweep, examples/gauss_seidel.py upstream), and operands are read at constant
+ * offsets from their root's lattice. 0: no; 1: yes, into a second buffer (dst != cur); 2: yes, also
+ * in place (no shifted read of the assigned array can meet an assigned point). */
+int cnh_kernel_lattice(const cnh_kernel* k);
 /* How many variants whose name starts with `prefix` ("flat", "nd", "tiles", "slide", "direct")
  * have a code object, i.e. were built or launched: tells a test which kernel a launch took. */
 int cnh_kernel_variants_loaded(const cnh_kernel* k, const char* prefix);

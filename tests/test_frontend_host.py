@@ -433,6 +433,33 @@ def test_in_place_when_read_and_written_lattices_miss_each_other(itf):
     assert how(jacobi) == "pingpong"
 
 
+def test_the_two_lattices_of_a_colour_are_one_sweep(itf):
+    """examples/gauss_seidel.py upstream: four statements a sweep, two launches; the arrays become
+    one block the first time."""
+    n = 8192
+    phi, f = cnp.zeros((n, n)), cnp.zeros((n, n))
+    cnp.execute(itf)
+    assert itf.array_info(phi.name)["tile"] == 4096
+    itf.trace()
+    for _ in range(2):
+        for r0, c0 in ((1, 1), (2, 2), (1, 2), (2, 1)):
+            rows, cols = slice(r0, -1, 2), slice(c0, -1, 2)
+            up, down = slice(r0 - 1, -2, 2), slice(r0 + 1, None, 2)
+            left, right = slice(c0 - 1, -2, 2), slice(c0 + 1, None, 2)
+            phi[rows, cols] = 0.25 * (phi[up, cols] + phi[down, cols] + phi[rows, left] + phi[rows, right]
+                                      - 0.5 * f[rows, cols])
+    cnp.execute(itf)
+    tr = [ln for ln in itf.trace() if ln.startswith(("group", "block"))]
+    assert [ln.split()[0] for ln in tr] == ["block", "block", "group", "group", "group", "group"]
+    assert all("path=lattices roots=2" in ln and "inplace" in ln for ln in tr[2:])
+    assert itf.stats()["compiled"] <= 3
+    # a statement that reads what the one before it assigns stays on its own
+    phi[1:-1:2, 1:-1:2] = phi[0:-2:2, 1:-1:2] * 2.0
+    phi[2:-1:2, 1:-1:2] = phi[1:-2:2, 1:-1:2] * 2.0
+    cnp.execute(itf)
+    assert not any("path=lattices" in ln for ln in itf.trace())
+
+
 def test_malformed_messages_are_refused(itf):
     with pytest.raises(RuntimeError, match="bad magic"):
         itf.send_dag(0, struct.pack("<iii", 1, 1, 0))

@@ -6,6 +6,8 @@ whole V-cycle of the 2-D multigrid solver (examples/multigrid2d.py, with its wei
 and residual), numpy.diag both ways (examples/diag.py) and the Jacobi iteration x += D^-1 (b - A x)
 built from diag and matvec (examples/jacobi_iteration.py). Element-wise statements must match NumPy
 bit for bit; products are held to 1e-12 of the sum of absolute products."""
+import os
+
 import numpy as np
 import pytest
 
@@ -51,6 +53,50 @@ def test_red_black_gauss_seidel(itf, n):
     got = phi.get(itf)
     assert np.array_equal(got, phi_host)
     assert np.abs(got).max() > 0
+
+
+@pytest.mark.parametrize("fusion", [True, False], ids=["paired", "one-by-one"])
+@pytest.mark.parametrize("shape", [(33, 33), (64, 64), (70, 131), (129, 258), (200, 64), (18, 20, 22), (17, 19, 33)])
+def test_red_black_sweeps_on_lattices(itf, shape, fusion):
+    """The two lattices of a colour go out as one sweep in place (arrays laid out as one block on
+    the way); one by one, or paired, the result is NumPy's bit for bit. Rank 3: the colours of a
+    red-black sweep are four lattices each, paired two by two."""
+    itf.set_fusion(fusion)
+    itf.set_trace()
+    rng = np.random.default_rng(sum(shape))
+    f_host = rng.standard_normal(shape)
+    phi_host = rng.standard_normal(shape)
+    phi, f = cnp.array(phi_host), cnp.array(f_host)
+    h2 = 0.37
+
+    def sweep2(p, g):
+        _red_black_sweep(p, g, h2)
+
+    def sweep3(p, g):
+        starts = [(a, b, c) for a in (1, 2) for b in (1, 2) for c in (1, 2)]
+        for colour in (0, 1):
+            for s in [t for t in starts if sum(t) % 2 == (1 + colour) % 2]:
+                me = tuple(slice(q, -1, 2) for q in s)
+                def sh(d, delta):
+                    k = list(me)
+                    k[d] = slice(s[d] + delta, -2 if delta < 0 else None, 2)
+                    return tuple(k)
+                p[me] = (1.0 / 6.0) * (p[sh(0, -1)] + p[sh(0, 1)] + p[sh(1, -1)] + p[sh(1, 1)]
+                                       + p[sh(2, -1)] + p[sh(2, 1)] - h2 * g[me])
+
+    sweep = sweep2 if len(shape) == 2 else sweep3
+    for _ in range(3):
+        sweep(phi, f)
+        sweep(phi_host, f_host)
+    got = phi.get(itf)
+    assert np.array_equal(got, phi_host)
+    tr = itf.trace()
+    paired = [ln for ln in tr if "path=lattices" in ln]
+    planning = os.environ.get("CHARMNUMERIC_SOLVER", "0") not in ("", "0")
+    if fusion and not planning:
+        assert len(paired) == 3 * (2 if len(shape) == 2 else 4), tr
+    else:
+        assert not paired
 
 
 # ---- products on slices ----
