@@ -827,6 +827,80 @@ __device__ __forceinline__ void tiles_run(const Tiled* arrs, const DTile* dts, i
     }
 }
 
+// ---- the same gather over arrays that are one row-major block each ----
+// No tile table, no tile arithmetic: element (g0, g1, g2) of an array is base[g0 * pz + g1 * py + g2],
+// so the part of an operand's address that belongs to a row is formed once per row and lane, and an
+// element costs one multiply-add per operand. Every strided or shifted statement on arrays of rank
+// 3, on rank-2 arrays with odd rows or ragged tile grids, and on single-tile arrays runs here.
+struct BlockLeaf { const T* base; int py, pz; int start[3]; int step[3]; };
+struct BlockArgs {
+    T* dst; const T* cur;       // cur != dst: a sweep into a second buffer copies what it does not assign
+    int shape[3]; int dpy, dpz; // the target (extents, elements between rows and planes)
+    int rs[3], re[3], rst[3];   // assigned region
+    int cnt[3];                 // points of its lattice per dimension
+    int lattice;                // 1: in place, walk the lattice's points only
+    int nchunks, rsh;           // chunks per row; 2^rsh rows share a workgroup
+    BlockLeaf leaf[NLA];
+};
+template <bool ROWS>
+__device__ __forceinline__ void block_run(const BlockArgs& a, const T* s) {
+    const int W0 = a.lattice ? a.cnt[0] : a.shape[0], W1 = a.lattice ? a.cnt[1] : a.shape[1];
+    const int W2 = a.lattice ? a.cnt[2] : a.shape[2];
+    const unsigned blk = blockIdx.x;
+    const unsigned group = blk / (unsigned)a.nchunks;
+    const int chunk = (int)(blk - group * (unsigned)a.nchunks);
+    int lanes = 256, lx = (int)threadIdx.x;
+    unsigned row = group;
+    if (ROWS) {
+        lanes = 256 >> a.rsh;
+        lx = (int)threadIdx.x & (lanes - 1);
+        row = (group << a.rsh) + ((unsigned)threadIdx.x >> (8 - a.rsh));
+        if (row >= (unsigned)W0 * (unsigned)W1) return;
+    }
+    const int i0 = (int)(row / (unsigned)W1), i1 = (int)(row - (unsigned)i0 * (unsigned)W1);
+    const int a0 = a.lattice ? a.rs[0] + i0 * a.rst[0] : i0;
+    const int a1 = a.lattice ? a.rs[1] + i1 * a.rst[1] : i1;
+    const bool in01 = a.lattice ||
+                      (a0 >= a.rs[0] && a0 < a.re[0] && (a0 - a.rs[0]) % a.rst[0] == 0 &&
+                       a1 >= a.rs[1] && a1 < a.re[1] && (a1 - a.rs[1]) % a.rst[1] == 0);
+    const int k0 = a.lattice ? i0 : (in01 ? (a0 - a.rs[0]) / a.rst[0] : 0);
+    const int k1 = a.lattice ? i1 : (in01 ? (a1 - a.rs[1]) / a.rst[1] : 0);
+    i64 rowoff[NLA];
+#pragma unroll
+    for (int q = 0; q < NL; ++q) {
+        const BlockLeaf& lf = a.leaf[q];
+        rowoff[q] = (i64)(lf.start[0] + k0 * lf.step[0]) * lf.pz + (i64)(lf.start[1] + k1 * lf.step[1]) * lf.py +
+                    lf.start[2];
+    }
+    const i64 drow = (i64)a0 * a.dpz + (i64)a1 * a.dpy;
+#pragma unroll
+    for (int u = 0; u < TL_PER_THREAD; ++u) {
+        const int j2 = chunk * (lanes * TL_PER_THREAD) + u * lanes + lx;
+        if (j2 >= W2) continue;
+        const int a2 = a.lattice ? a.rs[2] + j2 * a.rst[2] : j2;
+        const bool inside = in01 && (a.lattice || (a2 >= a.rs[2] && a2 < a.re[2] && (a2 - a.rs[2]) % a.rst[2] == 0));
+        if (inside) {
+            const int k2 = a.lattice ? j2 : (a2 - a.rs[2]) / a.rst[2];
+            T l[NLA], o[NOA];
+#pragma unroll
+            for (int q = 0; q < NL; ++q)
+                l[q] = a.leaf[q].base[rowoff[q] + (i64)k2 * a.leaf[q].step[2]];
+            group_eval(l, s, o);
+            a.dst[drow + a2] = o[0];
+        } else if (a.cur != nullptr && a.cur != a.dst) {
+            a.dst[drow + a2] = a.cur[drow + a2];
+        }
+    }
+}
+extern "C" __global__ __launch_bounds__(256) void grp_block(BlockArgs a, Scal sc) {
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
+    block_run<false>(a, s);
+}
+extern "C" __global__ __launch_bounds__(256) void grp_block_rows(BlockArgs a, Scal sc) {
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
+    block_run<true>(a, s);
+}
+
 extern "C" __global__ __launch_bounds__(256) void grp_tiles(const Tiled* arrs, const DTile* dts,
                                                             int ndt, TilesArgs ta, Scal sc) {
     CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);

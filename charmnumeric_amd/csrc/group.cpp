@@ -774,6 +774,67 @@ int check_tiled(const cnh_tiled* t, int nd, const char* what) {
     return 0;
 }
 
+// Is the array one row-major block starting at element 0 (tiles that are views into it, or a single
+// tile)? pitch[0], pitch[1] receive the elements between planes and between rows of the
+// rank-padded (z, y, x) view.
+bool one_block_of(const cnh_tiled* t, int esz, int64_t* pitch) {
+    const int nd = t->ndims;
+    int64_t ntiles = 1;
+    for (int d = 0; d < nd; ++d) {
+        if (t->offset[d] != 0)
+            return false;
+        ntiles *= t->grid[d];
+    }
+    int64_t p[3] = {0, 0, 0};
+    bool pitched = false;
+    for (int d = 0; d < nd; ++d)
+        pitched = pitched || t->pitch[d] != 0;
+    if (pitched) {
+        for (int d = 0; d < nd; ++d)
+            p[d] = t->pitch[d];
+        if (p[nd - 1] != 1)
+            return false;
+    } else {
+        if (ntiles != 1)
+            return false;
+        int64_t run = 1;
+        for (int d = nd - 1; d >= 0; --d) {
+            p[d] = run;
+            run *= t->shape[d];
+        }
+    }
+    // every tile starts where its first element lies in the block
+    const char* base = static_cast<const char*>(t->tiles[0]);
+    int64_t idx[3] = {0, 0, 0};
+    for (int64_t n = 0; n < ntiles; ++n) {
+        int64_t off = 0;
+        for (int d = 0; d < nd; ++d)
+            off += idx[d] * t->tile * p[d];
+        if (static_cast<const char*>(t->tiles[n]) != base + off * esz)
+            return false;
+        for (int d = nd - 1; d >= 0; --d) {
+            if (++idx[d] < t->grid[d])
+                break;
+            idx[d] = 0;
+        }
+    }
+    pitch[0] = nd >= 3 ? p[0] : 0;
+    pitch[1] = nd >= 2 ? p[nd - 2] : 0;
+    pitch[2] = 1;
+    return true;
+}
+
+struct BlockLeafDev {
+    const void* base;
+    int32_t py, pz, start[3], step[3];
+};
+struct BlockHeadDev {
+    void* dst;
+    const void* cur;
+    int32_t shape[3], dpy, dpz, rs[3], re[3], rst[3], cnt[3], lattice, nchunks, rsh;
+};
+static_assert(sizeof(BlockLeafDev) == 40 && sizeof(BlockHeadDev) == 96, "BlockArgs layout must match the generated struct");
+
 bool is_pitched(const cnh_tiled* t) {
     for (int d = 0; d < t->ndims; ++d)
         if (t->pitch[d] != 0)
@@ -971,6 +1032,7 @@ int g_stencil_mode = 2; // 0 = general gather, 1 = LDS sliding window, 2 = regis
 int g_direct_group = 0; // order workgroups by groups of neighbouring tiles (rank 3)
 int g_direct_lean = -1;   // wavefront-level lean kernel: 1 on, 0 off, -1 by rank
 int g_tiles_rows = 1;     // general gather: short rows share a workgroup
+int g_tiles_block = 1;    // general gather: arrays that are one block each skip the tile logic
 int g_direct_stagger = 0; // concurrent groups start at different offsets of their tiles
 int g_direct_merge = 1;   // lean part and the rest in one launch instead of two
 DirectConfig g_direct_cfg;
@@ -1116,24 +1178,8 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
     // Every array of the launch one row-major block behind its tile views: no tile logic at all.
     if (pitched && g_direct_flat) {
         const int esz = dtype_size(p.dtype);
-        auto one_block = [&](const cnh_tiled* t) {
-            // tile (i0, i1, i2) must start where element (i0, i1, i2) * tile of the block lies
-            const char* base = static_cast<const char*>(t->tiles[0]);
-            int64_t idx[3] = {0, 0, 0};
-            for (int64_t n = 0; n < ntiles; ++n) {
-                int64_t off = 0;
-                for (int d = 0; d < nd; ++d)
-                    off += idx[d] * t->tile * t->pitch[d];
-                if (static_cast<const char*>(t->tiles[n]) != base + off * esz)
-                    return false;
-                for (int d = nd - 1; d >= 0; --d) {
-                    if (++idx[d] < t->grid[d])
-                        break;
-                    idx[d] = 0;
-                }
-            }
-            return true;
-        };
+        int64_t unused_pitch[3];
+        auto one_block = [&](const cnh_tiled* t) { return one_block_of(t, esz, unused_pitch); };
         bool flat = one_block(cur) && one_block(dst) && pitch[1] >= cur->shape[nd - 1] && cur->shape[nd - 1] >= 2 &&
                     (nd < 3 || pitch[0] >= pitch[1] * cur->shape[1]) &&
                     pitch[0] * (nd == 3 ? cur->shape[0] : 1) + pitch[1] * cur->shape[nd - 2] < (1ll << 31);
@@ -1433,6 +1479,10 @@ extern "C" int64_t cnh_code_objects(void) {
 
 extern "C" int cnh_set_option(const char* name, int value) {
     CNH_CHECK(name != nullptr, -2, "null option name");
+    if (std::strcmp(name, "tiles_block") == 0) {
+        g_tiles_block = value != 0;
+        return 0;
+    }
     if (std::strcmp(name, "stencil_mode") == 0) {
         CNH_CHECK(value >= 0 && value <= 2, -2, "stencil_mode must be 0, 1 or 2");
         g_stencil_mode = value;
@@ -1716,6 +1766,71 @@ int launch_group_tiles_impl(cnh_kernel* k, int n_in, const cnh_tiled* in, int n_
                 return rc;
         if (handled)
             return 0;
+    }
+
+    // Every array of the launch one row-major block (or a single tile): the gather without tiles.
+    if (g_tiles_block) {
+        const int esz = dtype_size(p.dtype);
+        int64_t dpitch[3] = {0, 0, 1}, cpitch[3] = {0, 0, 1};
+        bool block = one_block_of(dst, esz, dpitch) &&
+                     (cur == nullptr || (one_block_of(cur, esz, cpitch) && cpitch[0] == dpitch[0] && cpitch[1] == dpitch[1]));
+        std::vector<std::array<int64_t, 3>> apitch(arrays.size(), std::array<int64_t, 3>{0, 0, 1});
+        for (size_t a = 0; a < arrays.size() && block; ++a)
+            block = one_block_of(arrays[a], esz, apitch[a].data()) && apitch[a][0] < (1ll << 31) && apitch[a][1] < (1ll << 31);
+        block = block && dpitch[0] < (1ll << 31) && dpitch[1] < (1ll << 31);
+        if (block) {
+            BlockHeadDev h;
+            std::memset(&h, 0, sizeof h);
+            h.dst = dst->tiles[0];
+            h.cur = cur ? cur->tiles[0] : nullptr;
+            const bool in_place = h.cur == nullptr || h.cur == h.dst;
+            for (int d = 0; d < 3; ++d) {
+                h.shape[d] = d >= pad ? dst->shape[d - pad] : 1;
+                h.rs[d] = rs[d];
+                h.re[d] = re[d];
+                h.rst[d] = rst[d];
+                h.cnt[d] = std::max(0, (re[d] - rs[d] + rst[d] - 1) / rst[d]);
+            }
+            h.dpy = (int32_t)dpitch[1];
+            h.dpz = (int32_t)dpitch[0];
+            h.lattice = in_place ? 1 : 0;
+            const int64_t W2 = in_place ? h.cnt[2] : h.shape[2];
+            const int64_t rows = in_place ? (int64_t)h.cnt[0] * h.cnt[1] : (int64_t)h.shape[0] * h.shape[1];
+            if (rows <= 0 || W2 <= 0)
+                return 0;
+            int lanes = 16;
+            while (lanes < 256 && lanes * 4 < W2)
+                lanes *= 2;
+            int rsh = 0;
+            while (g_tiles_rows && (256 >> rsh) > lanes && (1 << rsh) < rows)
+                rsh++;
+            lanes = 256 >> rsh;
+            const int64_t nchunks = (W2 + lanes * 4 - 1) / (lanes * 4);
+            const int64_t nblocks = ((rows + (1 << rsh) - 1) >> rsh) * nchunks;
+            if (nblocks < (1ll << 31) && rows < (1ll << 31)) {
+                h.nchunks = (int32_t)nchunks;
+                h.rsh = rsh;
+                std::vector<unsigned char> args(sizeof h + (size_t)NLA * sizeof(BlockLeafDev), 0);
+                std::memcpy(args.data(), &h, sizeof h);
+                for (int l = 0; l < NL; ++l) {
+                    const int32_t* lr = &targs[13 + 7 * l];
+                    BlockLeafDev lf;
+                    lf.base = arrays[(size_t)lr[0]]->tiles[0];
+                    lf.py = (int32_t)apitch[(size_t)lr[0]][1];
+                    lf.pz = (int32_t)apitch[(size_t)lr[0]][0];
+                    for (int d = 0; d < 3; ++d) {
+                        lf.start[d] = lr[1 + d];
+                        lf.step[d] = lr[4 + d];
+                    }
+                    std::memcpy(args.data() + sizeof h + (size_t)l * sizeof lf, &lf, sizeof lf);
+                }
+                hipFunction_t fn;
+                if (int rc = get_function(k, "tiles", rsh > 0 ? "grp_block_rows" : "grp_block", &fn))
+                    return rc;
+                void* params[] = {args.data(), scal.data()};
+                return launch(fn, nblocks, params, st);
+            }
+        }
     }
 
     // Destination tiles.

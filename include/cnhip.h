@@ -113,6 +113,8 @@ int cnh_version(void);
  *   "flat_obz/oby/obx"  extents in elements of the blocks that kernel's workgroups are ordered by
  *                    (default 256^3 for rank 3, bands of whole rows for rank 2)
  *   "tiles_rows"     general gather: rows shorter than 1024 elements share a workgroup (default 1)
+ *   "tiles_block"    general gather: a launch whose arrays are one row-major block each (or single
+ *                    tiles) addresses them without tile tables (default 1)
  *   "gemv_xlds"      matvecs of 8192 rows or more whose column tiles are at most 64 KB of x wide
  *                    stage x in LDS, 32 or 64 rows per workgroup (default 1); 0: one wavefront per
  *                    row reading x through the caches. Same bits either way.
