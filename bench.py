@@ -1539,6 +1539,9 @@ def main():
                     help="only the strided and odd-sized programs (multigrid transfers, red-black sweeps); "
                          "prints their figures as one JSON line of their own")
     ap.add_argument("--only", default=None, help="with --strided: the one program to run (by its key in the output)")
+    ap.add_argument("--config", default=None, choices=["c1", "c3", "c4", "c5"],
+                    help="only that configuration by direct C ABI calls (for profiling one kernel family); "
+                         "prints its figures as one JSON line of their own")
     ap.add_argument("--cg-separate", action="store_true",
                     help="CG iteration as four launches (matvec, dot, x and r, p) instead of the fused two")
     args = ap.parse_args()
@@ -1551,6 +1554,11 @@ def main():
     if args.strided:
         print(json.dumps({"metric": "strided_programs_through_the_frontend", "unit": "us per operation",
                           "n_gpus": 1, "data": "synthetic", "programs": run_strided(only=args.only)}))
+        return
+    if args.config:
+        one = {"c1": lambda: run_c1(L), "c3": lambda: run_jacobi(L, 2, 8192, 2048, 200),
+               "c4": lambda: run_jacobi(L, 3, 512, 128, 100), "c5": lambda: run_lstm(L)}[args.config]()
+        print(json.dumps({"metric": "configuration_" + args.config, "n_gpus": 1, "data": "synthetic", "figures": one}))
         return
     if os.environ.get("CNH_BENCH_MARCH2D"):
         L.check(L.lib.cnh_set_option(b"slide2d_march", 1))

@@ -1102,10 +1102,6 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
                   const cnh_tiled* dst, const std::vector<unsigned char>& scal, hipStream_t st,
                   bool* handled, RedReq* red) {
     const GroupProgram& p = k->prog;
-    // a lane's own rows and planes must not straddle tiles: the tile edge (a power of two) has
-    // to be a multiple of what one lane owns
-    if (cur->tile % sh.ry != 0 || cur->tile % sh.rz != 0)
-        return 0;
     const int nd = p.ndims, pad = CNH_MAX_ND - nd;
     int64_t ntiles = 1, vol = 1, volume = 1;
     for (int d = 0; d < nd; ++d) {
@@ -1286,6 +1282,10 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
     }
     if (!aligned || sh.lattice)
         return 0;                         // the per-tile kernels take aligned unit-step sweeps only
+    // a lane's own rows and planes must not straddle tiles: the tile edge (a power of two) has
+    // to be a multiple of what one lane owns
+    if (cur->tile % sh.ry != 0 || cur->tile % sh.rz != 0)
+        return 0;
     DirectArgsDev a;
     std::memset(&a, 0, sizeof a);
     a.tile = cur->tile;
