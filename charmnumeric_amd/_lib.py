@@ -221,6 +221,8 @@ _PROTOS = {
     "cnh_launch_group_sums": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int,
                                         C.c_void_p, C.c_void_p]),
     "cnh_fold_sums": (C.c_int, [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]),
+    "cnh_alloc_on": (C.c_int, [C.c_size_t, C.c_int, C.c_void_p, _vpp]),
+    "cnh_allocation_count": (C.c_int64, []),
     "cnh_kernel_lattice": (C.c_int, [C.c_void_p]),
     "cnh_kernel_matches": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int]),
     "cnh_kernel_signature": (C.c_int, [C.c_void_p, C.POINTER(C.c_int), C.POINTER(C.c_int),

@@ -543,8 +543,9 @@ extern "C" {
 
 int cnh_dot_partial_noalloc(int dtype, int64_t n, const void* a, const void* b, void* out,
                             cnh_stream s) {
-    if (int rc = ensure_init())
-        return rc;
+    // no lazy initialisation here: selecting a device and resolving the scratch symbol are not
+    // things to do under a caller's graph capture
+    CNH_CHECK(current_device() >= 0, -100, "cnh_dot_partial_noalloc: call cnh_init first");
     CNH_CHECK(out != nullptr && n >= 0, -2, "cnh_dot_partial_noalloc: bad arguments");
     CNH_CHECK(n == 0 || (a != nullptr && b != nullptr), -2, "cnh_dot_partial_noalloc: null operand");
     CNH_CHECK(n <= kScratchMaxN, -3,

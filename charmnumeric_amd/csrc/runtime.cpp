@@ -5,6 +5,7 @@
 
 #include <cstdlib>
 #include <cstring>
+#include <atomic>
 #include <mutex>
 #include <unordered_map>
 #include <vector>
@@ -78,6 +79,10 @@ int release_retired(Workspace& w) {
 }
 } // namespace
 
+// Device and pinned-host allocations and descriptor-table copies the library has made: what a
+// caller that must not allocate (a stream under graph capture) can watch.
+std::atomic<int64_t> g_allocations{0};
+
 int ensure_init() {
     if (g_inited)
         return 0;
@@ -93,6 +98,7 @@ int reduce_workspace(hipStream_t s, size_t bytes, void** out) {
         size_t want = bytes < (1u << 20) ? (1u << 20) : bytes;
         void* p = nullptr;
         CNH_HIP(hipMalloc(&p, want));
+        g_allocations++;
         // The old block may still be read by kernels in flight on `s`: it waits in `retired` for
         // the next synchronisation of that stream.
         if (w.ptr)
@@ -114,6 +120,7 @@ int desc_upload(const void* host, size_t bytes, hipStream_t st, const void** dev
     if (!D.slab_dev) {
         CNH_HIP(hipMalloc((void**)&D.slab_dev, kSlabBytes));
         CNH_HIP(hipHostMalloc((void**)&D.slab_host, kSlabBytes, hipHostMallocDefault));
+        g_allocations += 2;
     }
     CNH_CHECK(bytes <= kSlabBytes / 4, -3, "descriptor table of %zu bytes is too large", bytes);
     uint64_t h = fnv1a(host, bytes);
@@ -140,6 +147,7 @@ int desc_upload(const void* host, size_t bytes, hipStream_t st, const void** dev
     D.slab_used += need;
     std::memcpy(D.slab_host + off, host, bytes);
     CNH_HIP(hipMemcpyAsync(D.slab_dev + off, D.slab_host + off, bytes, hipMemcpyHostToDevice, st));
+    g_allocations++;
     D.desc[h].push_back({off, bytes, st, false});
     *dev_out = D.slab_dev + off;
     return 0;
@@ -193,6 +201,7 @@ int cnh_alloc(size_t bytes, int zero, void** dptr) {
     CNH_CHECK(dptr != nullptr, -2, "cnh_alloc: null output pointer");
     void* p = nullptr;
     CNH_HIP(hipMalloc(&p, bytes ? bytes : 1));
+    g_allocations++;
     if (zero && bytes) {
         // The caller may first write the block on any stream, and no stream waits for another's
         // fill by itself: the fill runs on a stream of the library's own and the host waits for
@@ -211,6 +220,22 @@ int cnh_alloc(size_t bytes, int zero, void** dptr) {
     *dptr = p;
     return 0;
 }
+
+int cnh_alloc_on(size_t bytes, int zero, cnh_stream s, void** dptr) {
+    if (int rc = ensure_init())
+        return rc;
+    CNH_CHECK(dptr != nullptr, -2, "cnh_alloc_on: null output pointer");
+    void* p = nullptr;
+    CNH_HIP(hipMalloc(&p, bytes ? bytes : 1));
+    g_allocations++;
+    // the fill is ordered with whatever the caller queues on `s` next; the host does not wait
+    if (zero && bytes)
+        CNH_HIP(hipMemsetAsync(p, 0, bytes, as_stream(s)));
+    *dptr = p;
+    return 0;
+}
+
+int64_t cnh_allocation_count(void) { return g_allocations.load(); }
 
 int cnh_free(void* dptr) {
     if (!dptr)

@@ -26,9 +26,13 @@ class Array : public CTArrayBase<N> {
     }
 
   public:
-    // Owning tile of `region_` (src/backend.hpp:122-144): zero-filled on the device; the host
-    // waits for the fill, so the first kernel on any stream sees zeros.
-    Array(ArrayRegion<N> region_, std::array<int, N> global_shape_, int name_, ArrayDecomp<N> decomp_) {
+    // Owning tile of `region_` (src/backend.hpp:122-144): zero-filled on the device. The fill is
+    // queued on the partition's compute stream (the stream every kernel on this tile is launched
+    // on, src/backend.hpp:549-554), so the entry method that creates the array returns without
+    // waiting for it; a caller with no such stream passes nullptr and cnh_alloc's blocking form
+    // applies instead.
+    Array(ArrayRegion<N> region_, std::array<int, N> global_shape_, int name_, ArrayDecomp<N> decomp_,
+          cnh_stream compute_stream = nullptr) {
         describe(name_, dtype_of<T>());
         this->region = region_;
         this->global_shape = global_shape_;
@@ -37,7 +41,11 @@ class Array : public CTArrayBase<N> {
         this->global_size = 1;
         for (int extent : global_shape_)
             this->global_size *= extent;
-        CNH_OR_ABORT(cnh_alloc(sizeof(T) * (size_t)this->region.size(), /*zero=*/1, (void**)&dev_));
+        const size_t bytes = sizeof(T) * (size_t)this->region.size();
+        if (compute_stream != nullptr)
+            CNH_OR_ABORT(cnh_alloc_on(bytes, /*zero=*/1, compute_stream, (void**)&dev_));
+        else
+            CNH_OR_ABORT(cnh_alloc(bytes, /*zero=*/1, (void**)&dev_));
     }
 
     // Wrapper around a device buffer somebody else owns (src/backend.hpp:147-160 zeroes it too).

@@ -128,8 +128,16 @@ int cnh_set_option(const char* name, int value);
 
 /* ---- storage: Array<N,T> ctor zero-fill / data_ptr / copyToHost / copyToDevice / dtor
  *      (src/backend.hpp:112-200) ---- */
-int cnh_alloc(size_t bytes, int zero, void** dptr);
+int cnh_alloc(size_t bytes, int zero, void** dptr);   /* zero: returns after the fill has landed */
+/* The same with the zero-fill queued on `s`: ordered with what the caller queues there next, and the
+ * host does not wait (an Array constructor on the scheduler thread of a PE should not block it;
+ * work on other streams must order itself with `s` before it touches the block). */
+int cnh_alloc_on(size_t bytes, int zero, cnh_stream s, void** dptr);
 int cnh_free(void* dptr);
+/* How many device or pinned-host allocations and descriptor-table copies the library has made so
+ * far in this process: a caller that must not allocate (cnh_dot_partial_noalloc) can check that a
+ * call left it unchanged. */
+int64_t cnh_allocation_count(void);
 int cnh_memset0(void* dptr, size_t bytes, cnh_stream s);
 int cnh_h2d(void* dst_dev, const void* src_host, size_t bytes, cnh_stream s); /* returns after the copy */
 int cnh_d2h(void* dst_host, const void* src_dev, size_t bytes, cnh_stream s); /* returns after the copy */

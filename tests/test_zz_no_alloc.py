@@ -74,6 +74,37 @@ def test_same_operand_twice_and_own_stream(dev):
     dev.free_all()
 
 
+def test_the_call_allocates_and_uploads_nothing(dev):
+    """The property the entry point exists for: no device or pinned allocation, no descriptor copy,
+    no workspace growth across the call, for a size that makes the ordinary entry point do all
+    three on a fresh stream."""
+    rng = np.random.default_rng(9)
+    n = 5_000_011
+    a, b = rng.uniform(-1, 1, n), rng.uniform(-1, 1, n)
+    da, db = dev.array(a), dev.array(b)
+    out = dev.array(np.zeros(2))
+    st = C.c_void_p()
+    L.check(L.lib.cnh_stream_create(C.byref(st)))
+    before = L.lib.cnh_allocation_count()
+    L.check(L.lib.cnh_dot_partial_noalloc(L.F64, n, da.ptr, db.ptr, out.ptr, st))
+    L.check(L.lib.cnh_dot_partial_noalloc(L.F64, n // 3, da.ptr, db.ptr, out.ptr + 8, st))
+    assert L.lib.cnh_allocation_count() == before
+    L.check(L.lib.cnh_dot_partial(L.F64, n, da.ptr, db.ptr, out.ptr + 8, st))     # a workspace for this stream
+    assert L.lib.cnh_allocation_count() > before
+    L.check(L.lib.cnh_stream_sync(st))
+    got = out.get()
+    assert got.view(np.int64)[0] == got.view(np.int64)[1]
+    # the zero-fill of an allocation queued on the caller's stream
+    p = C.c_void_p()
+    L.check(L.lib.cnh_alloc_on(1 << 20, 1, st, C.byref(p)))
+    host = np.ones(1 << 17)
+    L.check(L.lib.cnh_d2h(host.ctypes.data_as(C.c_void_p), p, 1 << 20, st))
+    assert not host.any()
+    L.check(L.lib.cnh_free(p))
+    L.check(L.lib.cnh_stream_destroy(st))
+    dev.free_all()
+
+
 def test_sizes_beyond_the_array_are_refused(dev):
     out = dev.array(np.zeros(1))
     rc = L.lib.cnh_dot_partial_noalloc(L.F64, (1 << 28) + 1, out.ptr, out.ptr, out.ptr, None)
