@@ -7,9 +7,12 @@
 #include "decomp.h"
 #include "stmtlog.h"
 
+#include <dlfcn.h>
+
 #include <algorithm>
 #include <array>
 #include <condition_variable>
+#include <cstdlib>
 #include <cstring>
 #include <deque>
 #include <map>
@@ -3677,12 +3680,74 @@ int try_product_into_region(Ex* ex, const std::vector<DagNode>& dag, size_t i, s
     return 0;
 }
 
+// Named ranges around the work of every DAG node, for profilers that trace roctx markers
+// (rocprofv3 --marker-trace): kernels then group by what the program asked for instead of by
+// grid size. Off unless CHARMNUMERIC_ROCTX is set to something other than 0; the marker library is
+// looked up at run time, so nothing links against it.
+struct Markers {
+    int (*push)(const char*) = nullptr;
+    int (*pop)() = nullptr;
+    Markers() {
+        const char* on = std::getenv("CHARMNUMERIC_ROCTX");
+        if (on == nullptr || on[0] == '\0' || (on[0] == '0' && on[1] == '\0'))
+            return;
+        for (const char* lib : {"librocprofiler-sdk-roctx.so", "libroctx64.so"}) {
+            void* h = dlopen(lib, RTLD_NOW | RTLD_GLOBAL);
+            if (h == nullptr)
+                continue;
+            push = reinterpret_cast<int (*)(const char*)>(dlsym(h, "roctxRangePushA"));
+            pop = reinterpret_cast<int (*)()>(dlsym(h, "roctxRangePop"));
+            if (push != nullptr && pop != nullptr)
+                return;
+            push = nullptr;
+            pop = nullptr;
+        }
+    }
+};
+const Markers& markers() {
+    static const Markers m;
+    return m;
+}
+const char* node_kind(const DagNode& n) {
+    if (n.roots.empty())
+        return "cnx:empty";
+    switch (n.nodes[n.roots.back()].opcode) {
+    case CNH_OP_CREATE: return "cnx:create";
+    case kOpDelete: return "cnx:delete";
+    case CNH_OP_REDUCE: return "cnx:reduce";
+    case kOpSum: return "cnx:sum";
+    case kOpSumsqDiff: return "cnx:sumsq_diff";
+    case kOpMaxabsDiff: return "cnx:maxabs_diff";
+    case kOpAstype: return "cnx:astype";
+    case CNH_OP_MATMUL: return "cnx:matmul";
+    case CNH_OP_MATMATMUL: return "cnx:matmatmul";
+    case CNH_OP_TILE: return "cnx:tile";
+    case CNH_OP_DIAG: return "cnx:diag";
+    case CNH_OP_SET_REGION: return "cnx:assign";
+    default: return "cnx:elementwise";
+    }
+}
+struct Range {
+    bool open = false;
+    explicit Range(const char* name) {
+        if (markers().push != nullptr) {
+            markers().push(name);
+            open = true;
+        }
+    }
+    ~Range() {
+        if (open)
+            markers().pop();
+    }
+};
+
 int run_nodes(Ex* ex, std::vector<DagNode>& dag) {
     if (ex->solver_on)
         plan_message(ex, dag);
     int rc = 0;
     for (size_t i = 0; i < dag.size() && rc == 0;) {
         size_t used = 0;
+        const Range range(node_kind(dag[i]));   // covers the nodes a rewrite takes along with this one
         // a deletion needs no value: a pending sum nobody read goes with its array
         if (!dag[i].roots.empty() && dag[i].nodes[dag[i].roots.back()].opcode == kOpDelete) {
             rc = exec_node(ex, dag[i]);
