@@ -46,9 +46,15 @@ class CharmNumericInterface:
             L.check(L.lib.cnx_set_layout(self._ex, 1 if flat_rank3 else 0))
 
     def set_fusion(self, on=True):
-        """Whether the executor merges runs of same-extent assignments into one launch and writes
-        matrix products straight into the slice they are assigned to (default on; environment
-        variable CHARMNUMERIC_FUSE=0 turns it off for every interface). Values never depend on it."""
+        """Whether the executor merges nodes into fewer launches: runs of same-extent assignments,
+        products written straight into the slice they are assigned to, dense statements with the
+        scalar statements between them and the reductions behind them, a matvec with the vector
+        update before it and the dot behind it, the two lattices of a red-black colour (default on;
+        environment variable CHARMNUMERIC_FUSE=0 turns it off for every interface). Stored arrays
+        of element-wise statements are the same bit for bit either way. Reductions (and what is
+        computed from them) agree to the order of summation only: a reduction taken by the launch
+        that produces its operand adds other partial sums than one that reads the array again, and
+        which form runs can also depend on where a flush falls."""
         self._fusion = bool(on)
         if self._ex is not None:
             L.check(L.lib.cnx_set_fusion(self._ex, 1 if on else 0))

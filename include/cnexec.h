@@ -99,7 +99,21 @@ int cnx_set_layout(cnx_executor* ex, int flat_rank3);
  * run assigned takes it from registers, and boxes of one array that are neither identical nor
  * disjoint end the run, so results are those of the statements run one by one. (2) MATMATMUL into a
  * temporary followed by `target[box] = temporary` and the temporary's deletion writes the fp64
- * product straight into the box. Off: every node is executed on its own, as upstream does. */
+ * product straight into the box. (3) Statements that make new arrays of one shape from whole arrays
+ * laid out alike, the statements on one-element arrays between them (alpha = rr / pAp) and the
+ * reductions of the new arrays go out as one group: scalar statements are formed in registers and
+ * stored once (CNH_OP_SCALAR_OF), reductions leave partial sums that the next launch to read them
+ * as a kernel scalar adds up itself (cnh_launch_group_sums) — anything else that needs the value
+ * gets a fold first (cnh_fold_sums). (4) `beta = a / b; p = xa + beta * xb; y = A @ p; d = p @ y` on a
+ * matrix of 16384 rows or more is one launch of cnh_gemv_tiles_fused. (5) Two SET_REGION statements
+ * on lattices of step 2 of one array that neither read what the other assigns (the two halves of a
+ * red-black colour) are one sweep in place; arrays cut into tiles are stored as one block first.
+ * Off: every node is executed on its own, as upstream does.
+ * Stored results of element-wise statements are the same bits either way. Reductions, and values
+ * computed from them, agree to the order of summation: fused and unfused forms add different partial
+ * sums, and (for a statement held back at the end of a message) which form runs can depend on where
+ * the caller's flushes fall. fp64 products: see "gemm_ksplit" in cnhip.h for the one other place
+ * where the order of additions depends on the launch's shape. */
 int cnx_set_fusion(cnx_executor* ex, int on);
 
 /* ArrayDAGGroup::receive_dag(int epoch, int size, char msg[size]) (src/backend.ci:15,
