@@ -1007,7 +1007,8 @@ def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=
     out = {"steps": steps, "gemm_us": round(gus_idle, 2), "gemm_tflops": round(flop / gus_idle / 1e6, 2),
            "mfma_frac": round(flop / gus_idle / 1e6 / FP64_MFMA_PEAK_TFLOPS, 4),
            "step_us": round(step_idle, 2),
-           "step_frac_of_mfma_roofline": round(flop / FP64_MFMA_PEAK_TFLOPS / 1e6 / step_idle, 4),
+           "step_frac_of_mfma_roofline": round(flop / FP64_MFMA_PEAK_TFLOPS / 1e6 / step_idle, 4)
+           if step_idle else None,
            "measured_from": "an idle device (one pass of 64 steps)",
            "mfma_measured_ceiling_tflops": round(ceiling.value, 1),
            "sustained": {"gemm_us": round(gus, 2), "gemm_tflops": round(flop / gus / 1e6, 2),
@@ -1015,7 +1016,8 @@ def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=
                          "mfma_frac_of_measured_ceiling": round(flop / gus / 1e6 / ceiling.value, 4)
                          if ceiling.value else None,
                          "step_us": round(step_us, 2),
-                         "step_frac_of_mfma_roofline": round(flop / FP64_MFMA_PEAK_TFLOPS / 1e6 / step_us, 4),
+                         "step_frac_of_mfma_roofline":
+                             round(flop / FP64_MFMA_PEAK_TFLOPS / 1e6 / step_us, 4) if step_us else None,
                          "untimed_passes_queued_ahead": warm_passes if timed else 0},
            "flop_per_step": flop}
     if keep:

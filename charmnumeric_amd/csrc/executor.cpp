@@ -862,6 +862,7 @@ int exec_group(Ex* ex, const DagNode& n) {
             t.tile = a.tile;
             t.tiles = a.tiles.data();
             int j = 0;
+            int from[3] = {-1, -1, -1};          // the operand's dimension behind each of the group's
             for (int d = 0; d < target->ndims; ++d) {
                 const int cnt = region_count(root.region, d);
                 const int left_t = target->ndims - d, left_a = a.ndims - j;
@@ -870,6 +871,7 @@ int exec_group(Ex* ex, const DagNode& n) {
                     t.grid[d] = a.grid[j];
                     t.offset[d] = a.offset[j];
                     t.grid_lo[d] = a.offset[j] / a.tile;
+                    from[d] = j;
                     ++j;
                 } else {
                     CNH_CHECK(cnt == 1, -35, "node %d: operand %d of shape rank %d does not fit the "
@@ -880,8 +882,13 @@ int exec_group(Ex* ex, const DagNode& n) {
             }
             CNH_CHECK(j == a.ndims, -35, "node %d: operand %d does not fit the assigned region", n.id,
                       a.name);
-            CNH_CHECK(!a.flat, -35, "node %d: operand %d of rank %d in a rank-%d group", n.id, a.name,
-                      a.ndims, target->ndims);
+            if (a.flat)
+                // one block: an inserted dimension has one index, so any pitch that keeps the
+                // pitches ordered serves; it takes the extent of what lies below it
+                for (int d = target->ndims - 1; d >= 0; --d)
+                    t.pitch[d] = from[d] >= 0                ? a.pitch[from[d]]
+                                 : d == target->ndims - 1 ? 1
+                                                          : t.pitch[d + 1] * t.shape[d + 1];
             tin[i] = t;
         } else if (in_arr[i]->ndims > target->ndims) {
             // A higher-rank operand whose extra dimensions have extent 1 (vec[:] = column with

@@ -850,3 +850,31 @@ def test_an_lstm_step_is_a_product_and_one_merged_launch(itf):
         assert b_ - a == 2 and "path=statements" in work[a + 1]
     # three pieces + tanh + C + C += + Ct + Hout + the two copies for the next step
     assert sum("count=10" in ln for ln in work) == n - 2
+
+
+def test_a_one_block_matrix_is_assigned_into_a_slab_of_a_rank3_array():
+    """IFOG[t] = M and Hin[t, :, w:] = prev with M, prev rank-2 arrays stored as one block (their
+    tile grid is ragged): presented to the rank-3 group with an extent-1 dimension in front."""
+    cnp.reset()
+    it = cnp.CharmNumericInterface(device=-1)
+    it.connect(odf=4)
+    it.set_trace()
+    it.set_solver(True)
+    it.set_layout(True)
+    it.set_min_tile(2, 16)
+    it.set_min_tile(3, 8)
+    try:
+        n, b, d, word = 2, 48, 40, 24
+        h0 = cnp.zeros((1, d))
+        Hin = cnp.zeros((n, b, word + d))
+        prev = cnp.tile(h0, (b, 1))
+        Hin[0, :, word:] = prev
+        Hin[1, :, word:] = prev * 2.0
+        cnp.execute(it)
+        tr = it.trace()
+        made = [ln for ln in tr if ln.startswith("create") and "shape=(48,40)" in ln]
+        assert made and all("tile=32" in ln for ln in made)        # 40 columns in tiles of 32: ragged
+        assert len([ln for ln in tr if ln.startswith("group") and "path=tiles" in ln]) == 2
+    finally:
+        cnp.reset()
+        it.close()
