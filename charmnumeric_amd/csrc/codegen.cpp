@@ -832,7 +832,11 @@ __device__ __forceinline__ void tiles_run(const Tiled* arrs, const DTile* dts, i
 // so the part of an operand's address that belongs to a row is formed once per row and lane, and an
 // element costs one multiply-add per operand. Every strided or shifted statement on arrays of rank
 // 3, on rank-2 arrays with odd rows or ragged tile grids, and on single-tile arrays runs here.
-struct BlockLeaf { const T* base; int py, pz; int start[3]; int step[3]; };
+struct BlockLeaf {
+    const T* base; int py, pz; int start[3]; int step[3];
+    int lim[3];                 // last index of the leaf's own region per dimension (scatter launches)
+    int unused;
+};
 struct BlockArgs {
     T* dst; const T* cur;       // cur != dst: a sweep into a second buffer copies what it does not assign
     int shape[3]; int dpy, dpz; // the target (extents, elements between rows and planes)
@@ -840,6 +844,8 @@ struct BlockArgs {
     int cnt[3];                 // points of its lattice per dimension
     int lattice;                // 1: in place, walk the lattice's points only
     int nchunks, rsh;           // chunks per row; 2^rsh rows share a workgroup
+    int nroots, unused;         // scatter launches: the assigned lattices (same steps rst), else 0
+    int rrs[4][3], rcnt[4][3];  // first point and number of points of each of them
     BlockLeaf leaf[NLA];
 };
 template <bool ROWS>
@@ -892,6 +898,66 @@ __device__ __forceinline__ void block_run(const BlockArgs& a, const T* s) {
         }
     }
 }
+#if NO > 1 && NO <= 4
+// Several statements that assign interleaved lattices of one array from other arrays (the four
+// statements of a prolongation, examples/multigrid2d.py upstream) as one launch, in place: a lane
+// takes one index (k0, k1, k2) of the lattices, evaluates every statement there and stores each
+// result at its own lattice's point, rs_r + k * step. The lattices may differ in their number of
+// points (cnt holds the largest per dimension): an index beyond a statement's own region reads that
+// statement's operands at their last index instead, and stores nothing for it.
+template <bool ROWS>
+__device__ __forceinline__ void block_scatter(const BlockArgs& a, const T* s) {
+    const int W0 = a.cnt[0], W1 = a.cnt[1], W2 = a.cnt[2];
+    const unsigned blk = blockIdx.x;
+    const unsigned group = blk / (unsigned)a.nchunks;
+    const int chunk = (int)(blk - group * (unsigned)a.nchunks);
+    int lanes = 256, lx = (int)threadIdx.x;
+    unsigned row = group;
+    if (ROWS) {
+        lanes = 256 >> a.rsh;
+        lx = (int)threadIdx.x & (lanes - 1);
+        row = (group << a.rsh) + ((unsigned)threadIdx.x >> (8 - a.rsh));
+        if (row >= (unsigned)W0 * (unsigned)W1) return;
+    }
+    const int k0 = (int)(row / (unsigned)W1), k1 = (int)(row - (unsigned)k0 * (unsigned)W1);
+    i64 rowoff[NLA];
+#pragma unroll
+    for (int q = 0; q < NL; ++q) {
+        const BlockLeaf& lf = a.leaf[q];
+        rowoff[q] = (i64)(lf.start[0] + min(k0, lf.lim[0]) * lf.step[0]) * lf.pz +
+                    (i64)(lf.start[1] + min(k1, lf.lim[1]) * lf.step[1]) * lf.py + lf.start[2];
+    }
+    i64 drow[NO];
+    bool rin[NO];
+#pragma unroll
+    for (int r = 0; r < NO; ++r) {
+        rin[r] = k0 < a.rcnt[r][0] && k1 < a.rcnt[r][1];
+        drow[r] = (i64)(a.rrs[r][0] + k0 * a.rst[0]) * a.dpz + (i64)(a.rrs[r][1] + k1 * a.rst[1]) * a.dpy + a.rrs[r][2];
+    }
+#pragma unroll
+    for (int u = 0; u < TL_PER_THREAD; ++u) {
+        const int k2 = chunk * (lanes * TL_PER_THREAD) + u * lanes + lx;
+        if (k2 >= W2) continue;
+        T l[NLA], o[NOA];
+#pragma unroll
+        for (int q = 0; q < NL; ++q)
+            l[q] = a.leaf[q].base[rowoff[q] + (i64)min(k2, a.leaf[q].lim[2]) * a.leaf[q].step[2]];
+        group_eval(l, s, o);
+#pragma unroll
+        for (int r = 0; r < NO; ++r)
+            if (rin[r] && k2 < a.rcnt[r][2])
+                a.dst[drow[r] + (i64)k2 * a.rst[2]] = o[r];
+    }
+}
+extern "C" __global__ __launch_bounds__(256) void grp_scatter(BlockArgs a, Scal sc) {
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
+    block_scatter<false>(a, s);
+}
+extern "C" __global__ __launch_bounds__(256) void grp_scatter_rows(BlockArgs a, Scal sc) {
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
+    block_scatter<true>(a, s);
+}
+#endif
 extern "C" __global__ __launch_bounds__(256) void grp_block(BlockArgs a, Scal sc) {
     CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
     block_run<false>(a, s);
@@ -979,8 +1045,10 @@ int emit_variant_source(const GroupProgram& p, const std::string& variant, std::
         return 0;
     }
     if (variant == "tiles") {
-        if (p.out_roots.size() != 1) {
-            err = "the tiled variant needs exactly one output root";
+        // one output root, or up to four SET_REGION roots (the scatter kernels of this variant;
+        // its other kernels store the first root only, and the launch never picks them then)
+        if (p.out_roots.size() > 4) {
+            err = "the tiled variant takes one to four output roots";
             return -17;
         }
         src = tiles_source(p);

@@ -812,7 +812,7 @@ struct FlatArgs {
     int py, pz;            // elements between rows and between planes
     int nb[3];             // workgroups along z, y, x
     int ob[3];             // ordering block, in workgroups along z, y, x
-    int nblocks8;          // launched workgroups / 8 when that is exact, else 0
+    int nblocks8;          // launched workgroups / 8 (the launch is padded to a multiple of 8)
     FDiv per_block;        // workgroups per ordering block
     FDiv gb1, gb2;         // ordering blocks along y and x
     FDiv obx, oby;         // = ob[2], ob[1]

@@ -3285,33 +3285,14 @@ bool lattice_statement(Ex* ex, const DagNode& n, XArray** target, const cnh_ast_
     return stepped;
 }
 
-int try_lattice_pair(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t* used, bool* open_ended) {
-    *used = 0;
-    *open_ended = false;
-    XArray *ta = nullptr, *tb = nullptr;
-    const cnh_ast_node *sa = nullptr, *sb = nullptr;
-    if (!lattice_statement(ex, dag[i], &ta, &sa))
-        return 0;
-    std::vector<int> dels;
-    const size_t j = skip_deletions(dag, i + 1, dels);
-    if (j == dag.size()) {
-        *open_ended = open_ended_allowed(ex);
-        return 0;
-    }
-    if (!lattice_statement(ex, dag[j], &tb, &sb) || tb != ta)
-        return 0;
-    for (int d = 0; d < sa->region.ndims; ++d)
-        if (sa->region.step[d] != sb->region.step[d])
-            return 0;
-    for (int name : dels)
-        if (name == ta->name)
-            return 0;
-    // one group: the first statement's roots, then the second's
-    DagNode merged;
-    merged.id = dag[i].id;
+// One group out of several statements: the roots of the first, then those of the next, and so on.
+// Literals and temporaries get names of their own per statement; every statement's SET_REGION
+// root becomes an output.
+void merge_statements(const std::vector<const DagNode*>& parts, DagNode& merged) {
+    merged.id = parts.front()->id;
     merged.fusible = 1;
     int next_literal = -1, next_temporary = 0x7c000000;
-    for (const DagNode* n : {&dag[i], &dag[j]}) {
+    for (const DagNode* n : parts) {
         const int base = (int)merged.nodes.size();
         for (const cnh_ast_node& a : n->nodes) {
             merged.nodes.push_back(a);
@@ -3335,6 +3316,164 @@ int try_lattice_pair(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t* 
         for (int32_t r : n->roots)
             merged.roots.push_back(base + r);
     }
+}
+
+// Does a statement read array `name` (other than as the array it assigns into)?
+bool statement_reads(const DagNode& n, int name) {
+    for (int32_t ri : n.roots) {
+        const cnh_ast_node& r = n.nodes[(size_t)ri];
+        for (int oi = 0; oi < r.n_operands; ++oi) {
+            if (r.opcode == CNH_OP_SET_REGION && oi == 0)
+                continue;
+            if (r.operands[oi] < 0 || r.operands[oi] >= (int)n.nodes.size())
+                return true;
+            const cnh_ast_node& op = n.nodes[(size_t)r.operands[oi]];
+            if (!op.is_scalar && op.result_name == name)
+                return true;
+        }
+    }
+    return false;
+}
+
+// ---- interleaved lattices of one array assigned from other arrays, as one launch ----
+//
+// The prolongation of examples/multigrid2d.py upstream fills a fine grid with four statements,
+//   e[2:-2:2, 2:-2:2] = c[1:-1, 1:-1];  e[1:-1:2, 2:-2:2] = 0.5 * (c[:-1, 1:-1] + c[1:, 1:-1]);  ...
+// each a pass over all of e's cache lines that writes a quarter of every line. None of them reads
+// e and their lattices share no point, so up to four of them run as one launch that reads the
+// coarse array once and stores all four lattices, in place, over arrays stored as one block each.
+int try_scatter_run(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t* used, bool* open_ended) {
+    *used = 0;
+    *open_ended = false;
+    XArray* ta = nullptr;
+    const cnh_ast_node* sa = nullptr;
+    if (!lattice_statement(ex, dag[i], &ta, &sa) || statement_reads(dag[i], ta->name))
+        return 0;
+    std::vector<const DagNode*> parts{&dag[i]};
+    std::vector<const cnh_ast_node*> sets{sa};
+    std::vector<int> dels;
+    size_t end = i + 1;
+    bool ran_out = false;
+    while (parts.size() < 4) {
+        std::vector<int> d2;
+        const size_t j = skip_deletions(dag, end, d2);
+        if (j == dag.size()) {
+            ran_out = true;
+            break;
+        }
+        XArray* tb = nullptr;
+        const cnh_ast_node* sb = nullptr;
+        if (!lattice_statement(ex, dag[j], &tb, &sb) || tb != ta || statement_reads(dag[j], ta->name))
+            break;
+        bool fits = true;
+        for (int d = 0; d < sa->region.ndims; ++d)
+            fits = fits && sb->region.step[d] == sa->region.step[d];
+        for (const cnh_ast_node* other : sets) {
+            bool apart = false;
+            for (int d = 0; d < sa->region.ndims; ++d)
+                apart = apart || progressions_disjoint(other->region.start[d], other->region.stop[d], other->region.step[d],
+                                                       sb->region.start[d], sb->region.stop[d], sb->region.step[d]);
+            fits = fits && apart;
+        }
+        for (int name : d2)
+            fits = fits && name != ta->name;
+        if (!fits)
+            break;
+        parts.push_back(&dag[j]);
+        sets.push_back(sb);
+        dels.insert(dels.end(), d2.begin(), d2.end());
+        end = j + 1;
+    }
+    if (ran_out && open_ended_allowed(ex)) {
+        *open_ended = true;                     // more statements of the run may follow
+        return 0;
+    }
+    if (parts.size() < 2)
+        return 0;
+    DagNode merged;
+    merge_statements(parts, merged);
+    Group g;
+    canonicalise(merged, g);
+    cnh_kernel* k = nullptr;
+    if (int rc = compile_cached(ex, g, &k))
+        return rc;
+    int n_in = 0, n_scalar = 0, n_out = 0;
+    if (int rc = cnh_kernel_signature(k, &n_in, &n_scalar, &n_out))
+        return rc;
+    if (n_out != (int)parts.size() || ta->phased() || ta->elems >= (1ll << 31))
+        return 0;
+    std::vector<XArray*> in_arr((size_t)n_in);
+    for (int q = 0; q < n_in; ++q) {
+        int cname = 0, has = 0;
+        cnh_region reg;
+        if (int rc = cnh_kernel_input(k, q, &cname, &has, &reg))
+            return rc;
+        auto it = ex->arrays.find(g.canon_to_actual[cname]);
+        if (it == ex->arrays.end() || it->second.dtype != ta->dtype || it->second.ndims != ta->ndims ||
+            it->second.phased() || &it->second == ta || it->second.elems >= (1ll << 31))
+            return 0;
+        in_arr[(size_t)q] = &it->second;
+    }
+    std::vector<const void*> scalars((size_t)std::max(1, n_scalar), nullptr);
+    for (int q = 0; q < n_scalar; ++q) {
+        int cname = 0;
+        if (int rc = cnh_kernel_scalar(k, q, &cname))
+            return rc;
+        XArray* sarr;
+        if (int rc = find_array(ex, g.canon_to_actual[cname], &sarr, "broadcast scalar"))
+            return rc;
+        if (sarr->elems != 1 || sarr->dtype != ta->dtype || sarr == ta)
+            return 0;
+        scalars[(size_t)q] = sarr->tiles[0];
+    }
+    // from here on the statements are this launch
+    if (int rc = make_block(ex, *ta))
+        return rc;
+    for (XArray* a : in_arr)
+        if (int rc = make_block(ex, *a))
+            return rc;
+    std::vector<cnh_tiled> tin((size_t)std::max(1, n_in));
+    for (int q = 0; q < n_in; ++q)
+        tin[(size_t)q] = in_arr[(size_t)q]->tiled();
+    const cnh_tiled cur = ta->tiled();
+    if (!ex->dry)
+        if (int rc = cnh_launch_group_tiles(k, n_in, tin.data(), n_scalar, scalars.data(), 1, &cur, &cur, ex->stream))
+            return rc == -17 ? 0 : rc;          // not a shape the scatter takes: statement by statement
+    ex->stats[5]++;
+    ex->log("group node=" + std::to_string(merged.id) + " path=scatter roots=" + std::to_string(parts.size()) +
+            " inputs=" + std::to_string(n_in) + " scalars=" + std::to_string(n_scalar) + " out=" +
+            std::to_string(ta->name) + " inplace");
+    for (int name : dels)
+        drop_array(ex, name);
+    ex->stats[2] += (int64_t)(end - i);
+    *used = end - i;
+    return 0;
+}
+
+int try_lattice_pair(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t* used, bool* open_ended) {
+    *used = 0;
+    *open_ended = false;
+    XArray *ta = nullptr, *tb = nullptr;
+    const cnh_ast_node *sa = nullptr, *sb = nullptr;
+    if (!lattice_statement(ex, dag[i], &ta, &sa))
+        return 0;
+    std::vector<int> dels;
+    const size_t j = skip_deletions(dag, i + 1, dels);
+    if (j == dag.size()) {
+        *open_ended = open_ended_allowed(ex);
+        return 0;
+    }
+    if (!lattice_statement(ex, dag[j], &tb, &sb) || tb != ta)
+        return 0;
+    for (int d = 0; d < sa->region.ndims; ++d)
+        if (sa->region.step[d] != sb->region.step[d])
+            return 0;
+    for (int name : dels)
+        if (name == ta->name)
+            return 0;
+    // one group: the first statement's roots, then the second's
+    DagNode merged;
+    merge_statements({&dag[i], &dag[j]}, merged);
     Group g;
     canonicalise(merged, g);
     cnh_kernel* k = nullptr;
@@ -3770,6 +3909,8 @@ int run_nodes(Ex* ex, std::vector<DagNode>& dag) {
             // ... everything else reads arrays as they are
             if (rc == 0 && used == 0 && !open_ended)
                 rc = resolve_all(ex);
+            if (rc == 0 && used == 0 && !open_ended)
+                rc = try_scatter_run(ex, dag, i, &used, &open_ended);
             if (rc == 0 && used == 0 && !open_ended)
                 rc = try_lattice_pair(ex, dag, i, &used, &open_ended);
             if (rc == 0 && used == 0 && !open_ended)

@@ -293,6 +293,46 @@ def test_bilinear_prolongation(itf, n):
     assert np.array_equal(u.get(itf), u_host)
 
 
+def _interpolate(fine, coarse):
+    """Linear interpolation onto a grid of 2 c - 1 points per dimension, one statement per parity
+    pattern of the fine index (4 statements in 2-D, 8 in 3-D), boundary points left alone."""
+    nd = coarse.ndim
+    for bits in np.ndindex(*([2] * nd)):
+        target = tuple(slice(1, -1, 2) if b else slice(2, -2, 2) for b in bits)
+        total, terms = None, 0
+        for side in np.ndindex(*[2 if b else 1 for b in bits]):
+            src = tuple((slice(None, -1) if s == 0 else slice(1, None)) if b else slice(1, -1)
+                        for b, s in zip(bits, side))
+            total = coarse[src] if total is None else total + coarse[src]
+            terms += 1
+        fine[target] = total if terms == 1 else (1.0 / terms) * total
+
+
+@pytest.mark.parametrize("fusion", [True, False], ids=["one-launch", "one-by-one"])
+@pytest.mark.parametrize("cshape", [(3, 3), (17, 33), (65, 64), (130, 257), (5, 9, 33), (12, 10, 70)])
+def test_interleaved_lattices_are_assigned_by_one_scatter(itf, cshape, fusion):
+    """The statements of a prolongation assign interleaved lattices of the fine array and read only
+    the coarse one: up to four of them are one launch. Same bits as NumPy and as one by one."""
+    rng = np.random.default_rng(sum(cshape))
+    fshape = tuple(2 * c - 1 for c in cshape)
+    c_host, f_host = rng.standard_normal(cshape), rng.standard_normal(fshape)
+    itf.set_fusion(fusion)
+    itf.set_trace()
+    c, f = cnp.array(c_host), cnp.array(f_host)
+    for _ in range(2):
+        _interpolate(f, c)
+        _interpolate(f_host, c_host)
+        c[...] = c * 0.5 + 1.0
+        c_host[...] = c_host * 0.5 + 1.0
+    assert np.array_equal(f.get(itf), f_host)
+    launches = [ln for ln in itf.trace() if "path=scatter" in ln]
+    planning = os.environ.get("CHARMNUMERIC_SOLVER", "0") not in ("", "0")
+    if fusion and not planning and min(cshape) > 3:
+        assert len(launches) == 2 * (1 << len(cshape)) // 4 and all("roots=4" in ln for ln in launches)
+    if not fusion:
+        assert not launches
+
+
 def test_weighted_jacobi_and_residual(itf):
     n = 65
     h2 = (1.0 / (n - 1)) ** 2
