@@ -1292,17 +1292,22 @@ def run_strided(reps=10, only=None):
     try:
         cnp.set_auto_flush(itf, 48)
 
-        def timed(fn, n, warm=2):
+        def timed(fn, n, warm=2, batches=3):
+            """Median over `batches` batches of n operations each (a batch is a millisecond or
+            two, so one late wake-up of a host thread would otherwise decide the figure)."""
             for _ in range(warm):
                 fn()
             cnp.execute(itf)
             itf.sync()
-            t0 = time.perf_counter()
-            for _ in range(n):
-                fn()
-            cnp.execute(itf)
-            itf.sync()
-            return (time.perf_counter() - t0) / n * 1e6
+            per = []
+            for _ in range(batches):
+                t0 = time.perf_counter()
+                for _ in range(n):
+                    fn()
+                cnp.execute(itf)
+                itf.sync()
+                per.append((time.perf_counter() - t0) / n * 1e6)
+            return float(np.median(per))
 
         def want(name):
             return only is None or only == name

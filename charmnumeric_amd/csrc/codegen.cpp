@@ -844,15 +844,23 @@ struct BlockArgs {
     int cnt[3];                 // points of its lattice per dimension
     int lattice;                // 1: in place, walk the lattice's points only
     int nchunks, rsh;           // chunks per row; 2^rsh rows share a workgroup
-    int nroots, unused;         // scatter launches: the assigned lattices (same steps rst), else 0
+    int nroots;                 // scatter launches: the assigned lattices (same steps rst), else 0
+    int nblk8;                  // launched workgroups / 8 (the launch is padded to a multiple of 8)
     int rrs[4][3], rcnt[4][3];  // first point and number of points of each of them
     BlockLeaf leaf[NLA];
 };
+// Consecutive workgroup ids go round the 8 XCDs: every XCD takes one contiguous eighth of the rows
+// instead, so that the rows neighbouring workgroups both read (a stencil's, a restriction's, the
+// coarse rows of a prolongation) are fetched into one L2 and not into two.
+__device__ __forceinline__ unsigned block_order(const BlockArgs& a) {
+    const unsigned b = blockIdx.x;
+    return a.nblk8 ? (b & 7u) * (unsigned)a.nblk8 + (b >> 3) : b;
+}
 template <bool ROWS>
 __device__ __forceinline__ void block_run(const BlockArgs& a, const T* s) {
     const int W0 = a.lattice ? a.cnt[0] : a.shape[0], W1 = a.lattice ? a.cnt[1] : a.shape[1];
     const int W2 = a.lattice ? a.cnt[2] : a.shape[2];
-    const unsigned blk = blockIdx.x;
+    const unsigned blk = block_order(a);
     const unsigned group = blk / (unsigned)a.nchunks;
     const int chunk = (int)(blk - group * (unsigned)a.nchunks);
     int lanes = 256, lx = (int)threadIdx.x;
@@ -861,8 +869,8 @@ __device__ __forceinline__ void block_run(const BlockArgs& a, const T* s) {
         lanes = 256 >> a.rsh;
         lx = (int)threadIdx.x & (lanes - 1);
         row = (group << a.rsh) + ((unsigned)threadIdx.x >> (8 - a.rsh));
-        if (row >= (unsigned)W0 * (unsigned)W1) return;
     }
+    if (row >= (unsigned)W0 * (unsigned)W1) return;       // a ragged last group, or padding of the launch
     const int i0 = (int)(row / (unsigned)W1), i1 = (int)(row - (unsigned)i0 * (unsigned)W1);
     const int a0 = a.lattice ? a.rs[0] + i0 * a.rst[0] : i0;
     const int a1 = a.lattice ? a.rs[1] + i1 * a.rst[1] : i1;
@@ -908,7 +916,7 @@ __device__ __forceinline__ void block_run(const BlockArgs& a, const T* s) {
 template <bool ROWS>
 __device__ __forceinline__ void block_scatter(const BlockArgs& a, const T* s) {
     const int W0 = a.cnt[0], W1 = a.cnt[1], W2 = a.cnt[2];
-    const unsigned blk = blockIdx.x;
+    const unsigned blk = block_order(a);
     const unsigned group = blk / (unsigned)a.nchunks;
     const int chunk = (int)(blk - group * (unsigned)a.nchunks);
     int lanes = 256, lx = (int)threadIdx.x;
@@ -917,8 +925,8 @@ __device__ __forceinline__ void block_scatter(const BlockArgs& a, const T* s) {
         lanes = 256 >> a.rsh;
         lx = (int)threadIdx.x & (lanes - 1);
         row = (group << a.rsh) + ((unsigned)threadIdx.x >> (8 - a.rsh));
-        if (row >= (unsigned)W0 * (unsigned)W1) return;
     }
+    if (row >= (unsigned)W0 * (unsigned)W1) return;       // a ragged last group, or padding of the launch
     const int k0 = (int)(row / (unsigned)W1), k1 = (int)(row - (unsigned)k0 * (unsigned)W1);
     i64 rowoff[NLA];
 #pragma unroll

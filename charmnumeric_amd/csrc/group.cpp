@@ -832,7 +832,7 @@ struct BlockHeadDev {
     void* dst;
     const void* cur;
     int32_t shape[3], dpy, dpz, rs[3], re[3], rst[3], cnt[3], lattice, nchunks, rsh;
-    int32_t nroots, unused, rrs[4][3], rcnt[4][3];
+    int32_t nroots, nblk8, rrs[4][3], rcnt[4][3];
 };
 static_assert(sizeof(BlockLeafDev) == 56 && sizeof(BlockHeadDev) == 200, "BlockArgs layout must match the generated struct");
 
@@ -1852,10 +1852,12 @@ int launch_group_tiles_impl(cnh_kernel* k, int n_in, const cnh_tiled* in, int n_
                 rsh++;
             lanes = 256 >> rsh;
             const int64_t nchunks = (W2 + lanes * 4 - 1) / (lanes * 4);
-            const int64_t nblocks = ((rows + (1 << rsh) - 1) >> rsh) * nchunks;
+            // padded to a multiple of 8: every XCD takes a contiguous eighth of the workgroups
+            const int64_t nblocks = (((rows + (1 << rsh) - 1) >> rsh) * nchunks + 7) / 8 * 8;
             if (nblocks < (1ll << 31) && rows < (1ll << 31)) {
                 h.nchunks = (int32_t)nchunks;
                 h.rsh = rsh;
+                h.nblk8 = (int32_t)(nblocks / 8);
                 std::vector<unsigned char> args(sizeof h + (size_t)NLA * sizeof(BlockLeafDev), 0);
                 std::memcpy(args.data(), &h, sizeof h);
                 for (int l = 0; l < NL; ++l) {
