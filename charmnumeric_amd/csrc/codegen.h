@@ -120,6 +120,11 @@ struct DirectShape {
     int lat[3] = {0, 0, 0};
     int nroots = 1;
     bool lattice = false, inplace_safe = false;
+    // Every output row of a lane holds the pair to the right of the wavefront's 128 columns (some
+    // load reads the window array at (0, 0, +1) or (0, 0, +2)): the last lane of a row's last
+    // wavefront can then copy one or two columns beyond it that no statement assigns, which saves
+    // the workgroups a 128 k + 1 (or + 2) wide array would otherwise launch for them.
+    bool tail_ok = false;
 };
 constexpr int kDirectMaxOther = 4;
 int direct_shape(const GroupProgram& p, const DirectConfig& cfg, DirectShape& sh, std::string& err);

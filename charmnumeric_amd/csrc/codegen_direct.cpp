@@ -199,6 +199,11 @@ int direct_shape(const GroupProgram& p, const DirectConfig& cfg, DirectShape& sh
         return -18;
     }
     sh.ty = 256 / sh.tx;
+    sh.tail_ok = false;
+    if (!sh.masked && !sh.lattice && sh.nroots == 1 && sh.halo[2] >= 1)
+        for (size_t l = 0; l < NLd; ++l)
+            if (sh.other[l] < 0 && sh.shifts[l][0] == 0 && sh.shifts[l][1] == 0 && sh.shifts[l][2] >= 1)
+                sh.tail_ok = true;
     const int hk = (sh.halo[2] + 1) / 2; // column pairs to each side
     const int window = (sh.rz + 2 * sh.halo[0]) * (sh.ry + 2 * sh.halo[1]) * (2 * hk + 1);
     if (window > 96) {
@@ -252,6 +257,7 @@ std::string direct_source(const GroupProgram& p, const DirectConfig& cfg, std::s
     s << "};\n#define DR_NROOTS " << sh.nroots << "\n";
     const int NOTH = (int)sh.other_names.size();
     s << "#define DR_MASKED " << (sh.masked ? 1 : 0) << "\n";
+    s << "#define DR_TAIL_OK " << (sh.tail_ok ? 1 : 0) << "\n";
     s << "#define DR_RED " << (cfg.reduce ? 1 : 0) << "\n";
     s << "#define DR_NOTH " << NOTH << "\n#define DR_NOTHA " << (NOTH > 0 ? NOTH : 1) << "\n";
     s << "__device__ constexpr int DR_OTHER[NLA] = {";
@@ -822,6 +828,8 @@ struct FlatArgs {
     int lat[3];            // step - 1 of every region per dimension (0: unit step, 1: every other point)
     int nroots;            // 1, or 2: a second assigned lattice [rs2, re2) with the same steps
     int rs2[3], re2[3];
+    int tail;              // 1 or 2: columns beyond the last wavefront of a row, copied by its last lane
+    int unused;
 };
 
 // Rows of odd length, odd pitches or a block that does not start on a 16-byte boundary (UA): pairs
@@ -1031,6 +1039,15 @@ __device__ __forceinline__ void direct_flat(const FlatArgs& a, const T* s) {
             // rows and planes beyond the array (a ragged last workgroup) and idle lanes store nothing
             if (live && z < S0 && y < S1 && (!inplace || yin || yin2))
                 store_pair_flat<NTS, UA>(dst + (z * PZ + y * PY + lx), res, in_e[0], in_e[1], live1);
+            // An array of 128 k + 1 or 128 k + 2 columns whose last columns no statement assigns
+            // (the boundary of a 2^k + 1 grid) launches k wavefronts per row: the last lane of the
+            // last one holds those columns as its right-hand neighbours and copies them over.
+            if (DR_TAIL_OK && a.tail && last && bx == a.nb[2] - 1 && !inplace && z < S0 && y < S1) {
+                const P2 far = win[rz + DR_H0][ry + DR_H1][DR_WK - 1];
+                T* const beyond_row = dst + (z * PZ + y * PY + x0 + 128);
+                beyond_row[0] = far[0];
+                if (a.tail > 1) beyond_row[1] = far[1];
+            }
         }
     }
     if (RED) {

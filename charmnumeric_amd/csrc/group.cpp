@@ -1014,9 +1014,9 @@ struct FlatArgsDev {
     void* slots;
     int32_t sub8;
     FDivDev fsub;
-    int32_t lat[3], nroots, rs2[3], re2[3];
+    int32_t lat[3], nroots, rs2[3], re2[3], tail, unused;
 };
-static_assert(sizeof(FlatArgsDev) == 16 + 8 * kDirectMaxOther + 4 * 18 + 12 * 5 + 4 + 8 + 16 + 40,
+static_assert(sizeof(FlatArgsDev) == 16 + 8 * kDirectMaxOther + 4 * 18 + 12 * 5 + 4 + 8 + 16 + 40 + 8,
               "FlatArgsDev layout must match the generated struct");
 
 // A launch that should also reduce what it changes: mode 1 = sum of (new - old)^2, 2 = max
@@ -1028,6 +1028,7 @@ struct RedReq {
 };
 
 int g_direct_flat = 1;          // arrays stored as one block take the whole-array kernel
+int g_flat_tail = 1;            // ... and fold one or two unassigned last columns into the wavefront before them
 int g_flat_ob[3] = {0, 0, 0};   // ordering block of that kernel in elements (z, y, x); 0 = default
 int g_stencil_mode = 2; // 0 = general gather, 1 = LDS sliding window, 2 = register window
 int g_direct_group = 0; // order workgroups by groups of neighbouring tiles (rank 3)
@@ -1221,8 +1222,20 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
             // sweep against 390 with 128^3 and 449 with whole planes); rank 2: bands of whole rows
             const int dflt[3] = {256, nd == 3 ? 256 : 1 << 30, nd == 3 ? 256 : 1 << 30};
             int64_t launched = 1, gb[3];
-            for (int d = 0; d < 3; ++d) {
+            for (int d = 0; d < 3; ++d)
                 f.nb[d] = (f.shape[d] + foot[d] - 1) / foot[d];
+            // One or two unassigned columns beyond a multiple of 128 (the right-hand boundary of a
+            // 2^k + 1 grid) get no workgroups of their own: the last lane of the row's last
+            // wavefront copies them. Only into a second buffer; a sweep in place leaves them alone.
+            {
+                const int beyond = f.shape[2] - 128 * (f.nb[2] - 1);
+                if (sh.tail_ok && f.nb[2] >= 2 && beyond <= 2 && f.re[2] <= 128 * (f.nb[2] - 1) &&
+                    f.cur != f.dst && g_flat_tail) {
+                    f.tail = beyond;
+                    f.nb[2] -= 1;
+                }
+            }
+            for (int d = 0; d < 3; ++d) {
                 const int want = g_flat_ob[d] > 0 ? g_flat_ob[d] : dflt[d];
                 f.ob[d] = std::max(1, std::min(f.nb[d], want / foot[d]));
                 gb[d] = (f.nb[d] + f.ob[d] - 1) / f.ob[d];
@@ -1549,6 +1562,10 @@ extern "C" int cnh_set_option(const char* name, int value) {
     }
     if (std::strcmp(name, "direct_flat") == 0) {
         g_direct_flat = value != 0;
+        return 0;
+    }
+    if (std::strcmp(name, "flat_tail") == 0) {
+        g_flat_tail = value != 0;
         return 0;
     }
     if (std::strcmp(name, "flat_obz") == 0 || std::strcmp(name, "flat_oby") == 0 ||

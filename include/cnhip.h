@@ -110,6 +110,8 @@ int cnh_version(void);
  *   "direct_merge"   lean part and the rest in one launch (default 1) or two
  *   "direct_flat"    arrays whose tiles are views into one row-major block take the whole-array
  *                    register-window kernel (default 1)
+ *   "flat_tail"      that kernel gives one or two unassigned columns beyond a multiple of 128 (the
+ *                    boundary of a 2^k + 1 grid) to the wavefront before them (default 1)
  *   "flat_obz/oby/obx"  extents in elements of the blocks that kernel's workgroups are ordered by
  *                    (default 256^3 for rank 3, bands of whole rows for rank 2)
  *   "tiles_rows"     general gather: rows shorter than 1024 elements share a workgroup (default 1)

@@ -552,3 +552,46 @@ def test_stencil_kernels_with_and_without_lane_exchange(itf, shape, tile, lean):
         assert _kernels(itf) == ["direct"] * 3
     finally:
         L.check(L.lib.cnh_set_option(b"direct_lean", -1))
+
+
+# ---- 2^k + 1 grids wider than a wavefront's 128 columns ----
+
+@pytest.mark.parametrize("tail", [1, 0], ids=["folded", "own-workgroups"])
+@pytest.mark.parametrize("shape", [(37, 257), (21, 129), (20, 385), (70, 258), (9, 10, 257), (6, 9, 129), (40, 130)])
+def test_last_column_of_a_2k_plus_1_grid(itf, shape, tail):
+    """A row of 128 k + 1 elements: the boundary column beyond the k-th wavefront is copied by that
+    wavefront's last lane instead of by workgroups of its own. Same bits either way and as NumPy;
+    a two-wide stencil (whose last two columns are boundary) covers 128 k + 2."""
+    from charmnumeric_amd import _lib as L
+    nd = len(shape)
+    L.check(L.lib.cnh_set_option(b"flat_tail", tail))
+    try:
+        rng = np.random.default_rng(shape[-1] + nd)
+        hu, hf = rng.standard_normal(shape), rng.standard_normal(shape)
+        u, f = cnp.array(hu), cnp.array(hf)
+        wide = shape[-1] % 128 == 2
+        h = 2 if wide else 1
+        inner = (slice(h, -h),) * nd
+
+        def neighbours(x):
+            out = None
+            for d in range(nd):
+                for s in (slice(0, -2 * h), slice(2 * h, None)):
+                    key = list(inner)
+                    key[d] = s
+                    out = x[tuple(key)] if out is None else out + x[tuple(key)]
+            return out
+
+        itf.set_trace()
+        for _ in range(3):
+            u[inner] = (1.0 / (2 * nd)) * (neighbours(u) + f[inner])
+            hu[inner] = (1.0 / (2 * nd)) * (neighbours(hu) + hf[inner])
+        r = cnp.zeros(shape)
+        hr = np.zeros(shape)
+        r[inner] = f[inner] - neighbours(u)              # into another array: its boundary stays 0
+        hr[inner] = hf[inner] - neighbours(hu)
+        assert np.array_equal(u.get(itf), hu)
+        assert np.array_equal(r.get(itf), hr)
+        assert _kernels(itf) == ["direct"] * 4
+    finally:
+        L.check(L.lib.cnh_set_option(b"flat_tail", 1))
