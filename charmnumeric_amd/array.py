@@ -15,6 +15,23 @@ import numpy as np
 from . import _lib as L
 from . import lazy
 
+# The recording hot path in C (csrc/recorder.c): the base type of the classes below, which then
+# take indexing, the binary operators, slice assignment and deletion records from it and keep the
+# methods here (`_py_*`, `_binary`) as the route for every form the C code does not handle.
+# CHARMNUMERIC_PYREC=1 runs on the Python methods alone.
+import os as _os
+
+if _os.environ.get("CHARMNUMERIC_PYREC", "0") not in ("", "0"):
+    _cnrec = None
+else:
+    try:
+        from . import _cnrec
+    except ImportError as exc:  # pragma: no cover
+        raise ImportError("charmnumeric_amd/_cnrec has not been built: run "
+                          "python -c 'import __graft_entry__ as g; g.build()' "
+                          "(or set CHARMNUMERIC_PYREC=1 to record in Python)") from exc
+_HandleBase = object if _cnrec is None else _cnrec.Handle
+
 _DEFAULT_DTYPE = np.dtype("float64")
 _SUPPORTED = (np.dtype("float32"), np.dtype("float64"), np.dtype("int32"), np.dtype("int64"))
 
@@ -228,7 +245,7 @@ def _is_whole(region, shape):
 # the objects
 
 
-class _ArrayLike:
+class _ArrayLike(_HandleBase):
     __array_priority__ = 1000
 
     # -- basic properties --
@@ -270,7 +287,7 @@ class _ArrayLike:
         raise NotImplementedError
 
     # -- slicing --
-    def __getitem__(self, key):
+    def _py_getitem(self, key):
         inner = parse_key(key, self.shape)
         return ArrayView(self._base(), compose(self._region(), inner))
 
@@ -289,7 +306,7 @@ class _ArrayLike:
                                  f"{self.shape[d]} in dimension {d}")
         return ArrayView(self._base(), compose(self._region(), (start, stop, step)))
 
-    def __setitem__(self, key, rhs):
+    def _py_setitem(self, key, rhs):
         inner = parse_key(key, self.shape)
         region = compose(self._region(), inner)
         shape = region_shape(inner)
@@ -317,34 +334,38 @@ class _ArrayLike:
             operand = lazy.scalar_bytes(value)
         lazy.record_set(base.name, base._wire, base.ndims, shape, region, operand)
 
-    # -- arithmetic --
-    def __add__(self, o):
-        return _binary(L.OP_ADD, self, o)
+    # -- arithmetic, indexing, assignment: from the C base type when it is there --
+    if _cnrec is None:
+        __getitem__ = _py_getitem
+        __setitem__ = _py_setitem
 
-    def __radd__(self, o):
-        return _binary(L.OP_ADD, o, self)
+        def __add__(self, o):
+            return _binary(L.OP_ADD, self, o)
 
-    def __sub__(self, o):
-        return _binary(L.OP_SUB, self, o)
+        def __radd__(self, o):
+            return _binary(L.OP_ADD, o, self)
 
-    def __rsub__(self, o):
-        return _binary(L.OP_SUB, o, self)
+        def __sub__(self, o):
+            return _binary(L.OP_SUB, self, o)
 
-    def __mul__(self, o):
-        return _binary(L.OP_MUL, self, o)
+        def __rsub__(self, o):
+            return _binary(L.OP_SUB, o, self)
 
-    def __rmul__(self, o):
-        return _binary(L.OP_MUL, o, self)
+        def __mul__(self, o):
+            return _binary(L.OP_MUL, self, o)
 
-    def __truediv__(self, o):
-        return _binary(L.OP_DIV, self, o)
+        def __rmul__(self, o):
+            return _binary(L.OP_MUL, o, self)
 
-    def __rtruediv__(self, o):
-        return _binary(L.OP_DIV, o, self)
+        def __truediv__(self, o):
+            return _binary(L.OP_DIV, self, o)
 
-    def __neg__(self):
-        # upstream spells negation as multiplication by -1 (charmnumeric.py:427-434)
-        return _binary(L.OP_MUL, self, -1)
+        def __rtruediv__(self, o):
+            return _binary(L.OP_DIV, o, self)
+
+        def __neg__(self):
+            # upstream spells negation as multiplication by -1 (charmnumeric.py:427-434)
+            return _binary(L.OP_MUL, self, -1)
 
     def __matmul__(self, o):
         return _matmul(self, o)
@@ -380,7 +401,8 @@ class Array(_ArrayLike):
     # True while every element is known to be exactly 1 (set by ones()/full(.., 1), dropped by any
     # assignment into the array): a dot with such an array is recorded as a sum, which reads one
     # array instead of two and gives the same bits (a * 1 is a, the order of additions is the same).
-    _all_ones = False
+    if _cnrec is None:
+        _all_ones = False
 
     def __init__(self, shape, dtype, name=None):
         self.shape = tuple(shape)
@@ -407,8 +429,9 @@ class Array(_ArrayLike):
         out._rb = None
         return out
 
-    def __del__(self):
-        lazy.record_delete(self.name, self._gen)
+    if _cnrec is None:
+        def __del__(self):
+            lazy.record_delete(self.name, self._gen)
 
     def __repr__(self):
         return f"Array(shape={self.shape}, dtype={self.dtype.name}, name={self.name})"
@@ -857,3 +880,15 @@ def eye(N, M=None, k=0, dtype=_DEFAULT_DTYPE):
 
 def identity(n, dtype=_DEFAULT_DTYPE):
     return eye(n, dtype=dtype)
+
+
+if _cnrec is not None:
+    _cnrec.setup(lazy._state, Array, ArrayView, _ArrayLike._py_getitem, _ArrayLike._py_setitem, _binary,
+                 lazy._flush_if_due, (L.OP_ADD, L.OP_SUB, L.OP_MUL, L.OP_DIV))
+
+
+def set_fast_recording(on=True):
+    """Switches the C fast paths of indexing, operators and assignment on or off (off: every call
+    takes the Python methods; the statement log is the same bytes either way). Returns the previous
+    setting; without the C module it is always off."""
+    return bool(_cnrec.set_fast(bool(on))) if _cnrec is not None else False

@@ -1,6 +1,7 @@
 """Host logic of the frontend and the executor, exercised without a GPU: the executor's dry mode
 takes every decision (shapes, tiles, kernel compilation and cache, launch path) and logs it."""
 import struct
+import sys
 
 import numpy as np
 import pytest
@@ -878,3 +879,109 @@ def test_a_one_block_matrix_is_assigned_into_a_slab_of_a_rank3_array():
     finally:
         cnp.reset()
         it.close()
+
+
+# ---- the recording fast paths in C against the Python methods they stand in for ----
+
+def _recorded(program, fast):
+    """The statement log `program` leaves (records as bytes; direct calls by name and opcode)."""
+    A = sys.modules["charmnumeric_amd.array"]
+    cnp.reset()
+    before = A.set_fast_recording(fast)
+    try:
+        program()
+        out = [item if type(item) is bytes else ("call", item.name, item.opcode) for item in lazy._state.pending]
+    finally:
+        A.set_fast_recording(before)
+        cnp.reset()
+    return out
+
+
+def _program_stencils():
+    u, f = cnp.zeros((33, 65)), cnp.ones((33, 65))
+    for _ in range(2):
+        upd = 0.25 * (u[:-2, 1:-1] + u[2:, 1:-1] + u[1:-1, :-2] + u[1:-1, 2:] + 0.001 * f[1:-1, 1:-1])
+        u[1:-1, 1:-1] = (1.0 - 2.0 / 3.0) * u[1:-1, 1:-1] + (2.0 / 3.0) * upd
+    u[0, :] = 1.0
+    u[-1] = 2
+    u[3:9:2, ::4] = f[3:9:2, ::4] * 3 - 1
+    u[5, 2:7] = u[6][:, 3:8] / 2.0
+    v = u[::2][1:5]                       # a view of a view, strided outside, unit inside
+    w = v[:, ::3][1:, 2:]
+    u[20:23, 0:7] = -w[0:3, 0:7] + 1
+    del upd, v, w
+
+
+def _program_ranks_and_types():
+    a, b = cnp.zeros(100), cnp.ones(100)
+    c = 2 * a - b / 4 + (a - 1) * (3 - b)
+    a[10:20] = c[30:40]
+    a[::7] = -b[::7]
+    a[5] = 1.5
+    s = a @ b                             # one-element results as run-time scalars: Python's route
+    a[:] = a * s + b
+    i = cnp.zeros((8, 9), dtype=cnp.int32)
+    i[1:3] = i[2:4] + 7
+    j = i / 2 + i * 3
+    x = cnp.zeros((4, 5, 6))
+    x[1] = x[2] + x[3, :, :] * 0.5
+    x[:, 1:4, ::2] = x[:, 0:3, 1::2] - 2
+    x[..., 0] = 1.0                       # an ellipsis: Python's route
+    y = cnp.zeros((4, 5, 6), dtype=cnp.float32)
+    z = x + y                             # two element types: converted first, Python's route
+    k = cnp.zeros((5, 6))
+    x[2] = k                              # a matrix into a slab: Python's route
+    del c, s, j, z
+
+
+@pytest.mark.parametrize("program", [_program_stencils, _program_ranks_and_types])
+def test_recording_in_c_leaves_the_same_log_as_the_python_methods(program):
+    A = sys.modules["charmnumeric_amd.array"]
+    if A._cnrec is None:
+        pytest.skip("recording in Python only (CHARMNUMERIC_PYREC)")
+    fast, slow = _recorded(program, True), _recorded(program, False)
+    assert len(fast) == len(slow) and len(fast) > 20
+    for n, (x, y) in enumerate(zip(fast, slow)):
+        assert x == y, f"record {n} differs"
+
+
+def test_errors_raised_through_the_c_paths_are_the_python_ones():
+    cnp.reset()
+    a, b = cnp.zeros((4, 6)), cnp.zeros((4, 7))
+    with pytest.raises(IndexError):
+        a[4]
+    with pytest.raises(IndexError):
+        a[0, 0, 0]
+    with pytest.raises(NotImplementedError):
+        a[::-1]
+    with pytest.raises(NotImplementedError):
+        a[2:2]
+    with pytest.raises(ValueError):
+        a + b
+    with pytest.raises(ValueError):
+        a[0:2] = b[0:2]
+    with pytest.raises(TypeError):
+        a["x"]
+    with pytest.raises((TypeError, AttributeError)):
+        del a[0]
+    with pytest.raises(ValueError):
+        a + "x"
+    assert (1 - a).shape == (4, 6) and (-a).shape == (4, 6) and (np.float64(2.0) * a).shape == (4, 6)
+    assert (a[1:3] / 2).shape == (2, 6) and a[1:3, 2].shape == (2, 1) and a[-1].shape == (1, 6)
+    v = a[1:4][1:, ::2]
+    assert v.region == ((2, 0), (4, 5), (1, 2)) and v.base is a and v.shape == (2, 3) and v.name == a.name
+    cnp.reset()
+
+
+def test_a_dying_array_leaves_one_deletion_record_and_an_old_generation_none():
+    cnp.reset()
+    a = cnp.zeros(10)
+    t = a + 1
+    name = t.name
+    n = len(lazy._state.pending)
+    del t
+    assert lazy._state.pending[n:] == [struct.pack("<2i", 5, name)]
+    old = a * 2
+    cnp.reset()                                   # names restart: the handle names nothing any more
+    del old, a
+    assert lazy._state.pending == []
