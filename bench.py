@@ -1293,8 +1293,9 @@ def run_strided(reps=10, only=None):
         cnp.set_auto_flush(itf, 48)
 
         def timed(fn, n, warm=2, batches=3):
-            """Median over `batches` batches of n operations each (a batch is a millisecond or
-            two, so one late wake-up of a host thread would otherwise decide the figure)."""
+            """Median over `batches` batches of n operations each, every batch between two syncs
+            (steady-state rate: a batch is several milliseconds, so the one flush and wait that end
+            it weigh little, and the median keeps one late wake-up of a host thread out)."""
             for _ in range(warm):
                 fn()
             cnp.execute(itf)
@@ -1329,7 +1330,7 @@ def run_strided(reps=10, only=None):
             u[1:-1, 1:-1] = (1.0 - omega) * u[1:-1, 1:-1] + omega * upd
 
         if want("weighted_jacobi_4097"):
-            out["weighted_jacobi_4097"] = entry(timed(smooth, 2 * reps), 3 * 8.0 * n * n)
+            out["weighted_jacobi_4097"] = entry(timed(smooth, 10 * reps), 3 * 8.0 * n * n)
 
         # residual into a third array, restriction to 2049^2 and prolongation back
         r = cnp.zeros((n, n))
@@ -1339,7 +1340,7 @@ def run_strided(reps=10, only=None):
                                                            - u[1:-1, :-2] - u[1:-1, 2:])
 
         if want("residual_4097"):
-            out["residual_4097"] = entry(timed(residual, 2 * reps), 3 * 8.0 * n * n)
+            out["residual_4097"] = entry(timed(residual, 10 * reps), 3 * 8.0 * n * n)
         nc = (n - 1) // 2 + 1
         coarse = cnp.zeros((nc, nc))
         c_, lo, hi = slice(2, -2, 2), slice(1, -3, 2), slice(3, -1, 2)
@@ -1350,7 +1351,7 @@ def run_strided(reps=10, only=None):
                                   + 0.0625 * (r[lo, lo] + r[lo, hi] + r[hi, lo] + r[hi, hi]))
 
         if want("restriction_4097_to_2049"):
-            out["restriction_4097_to_2049"] = entry(timed(restrict, 2 * reps), 8.0 * n * n + 8.0 * nc * nc)
+            out["restriction_4097_to_2049"] = entry(timed(restrict, 10 * reps), 8.0 * n * n + 8.0 * nc * nc)
         e = cnp.zeros((n, n))
 
         def prolong():
@@ -1360,8 +1361,14 @@ def run_strided(reps=10, only=None):
             e[1:-1:2, 1:-1:2] = 0.25 * (coarse[:-1, :-1] + coarse[1:, :-1] + coarse[:-1, 1:] + coarse[1:, 1:])
 
         if want("prolongation_2049_to_4097"):
-            out["prolongation_2049_to_4097"] = entry(timed(prolong, 2 * reps), 8.0 * n * n + 4 * 8.0 * nc * nc,
+            out["prolongation_2049_to_4097"] = entry(timed(prolong, 10 * reps), 8.0 * n * n + 4 * 8.0 * nc * nc,
                                                      statements=4)
+            # the four statements run as one launch that reads the coarse array once: the same time
+            # against the bytes of that single pass
+            once = 8.0 * n * n + 8.0 * nc * nc
+            us = out["prolongation_2049_to_4097"]["us"]
+            out["prolongation_2049_to_4097"].update(
+                bytes_read_once=int(once), frac_of_hbm_peak_read_once=round(once / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 3))
         del u, f, r, coarse, e
         cnp.execute(itf)
 
@@ -1380,7 +1387,7 @@ def run_strided(reps=10, only=None):
                                           - h2 * g[rows, cols])
 
         if want("red_black_8192"):
-            out["red_black_8192"] = entry(timed(red_black, reps), 4 * 8.0 * n * n, statements=4)
+            out["red_black_8192"] = entry(timed(red_black, 2 * reps), 4 * 8.0 * n * n, statements=4)
         del phi, g
         cnp.execute(itf)
 
@@ -1401,7 +1408,7 @@ def run_strided(reps=10, only=None):
                                         + h2 * q[1:-1, 1:-1, 1:-1])
 
         if want("poisson_257_cubed"):
-            out["poisson_257_cubed"] = entry(timed(poisson, 4 * reps), 3 * 8.0 * n ** 3)
+            out["poisson_257_cubed"] = entry(timed(poisson, 10 * reps), 3 * 8.0 * n ** 3)
         del v, q
         cnp.execute(itf)
     finally:
