@@ -124,7 +124,9 @@ int cnh_version(void);
  *   "gemm_ksplit"        fp64 products on grids of at most one workgroup per CU, every K a multiple of
  *                        32: two sets of wavefronts per workgroup, each taking every other K step,
  *                        their sums added first + second (default 1). One fixed order, another than
- *                        with 0.
+ *                        with 0; whether a product qualifies depends on the device's CU count, so two
+ *                        devices with different CU counts may differ in the last bits of a product
+ *                        (0 gives the single-set order everywhere).
  *   "slide_bx/ry/zc/pd", "slide2d_march"  geometry of the sliding-window kernel */
 int cnh_set_option(const char* name, int value);
 
