@@ -1227,10 +1227,15 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
             // One or two unassigned columns beyond a multiple of 128 (the right-hand boundary of a
             // 2^k + 1 grid) get no workgroups of their own: the last lane of the row's last
             // wavefront copies them. Only into a second buffer; a sweep in place leaves them alone.
-            {
+            // A launch that stores assigned elements only (a sweep from another array, a sweep in
+            // place) needs no workgroups at all for columns beyond the assigned region.
+            if (g_flat_tail && f.nb[2] >= 2 && f.re[2] <= 128 * (f.nb[2] - 1)) {
                 const int beyond = f.shape[2] - 128 * (f.nb[2] - 1);
-                if (sh.tail_ok && f.nb[2] >= 2 && beyond <= 2 && f.re[2] <= 128 * (f.nb[2] - 1) &&
-                    f.cur != f.dst && g_flat_tail) {
+                const bool writes_everything = f.cur != f.dst && !sh.masked;
+                if (!writes_everything) {
+                    while (f.nb[2] >= 2 && f.re[2] <= 128 * (f.nb[2] - 1))
+                        f.nb[2] -= 1;
+                } else if (sh.tail_ok && beyond <= 2) {
                     f.tail = beyond;
                     f.nb[2] -= 1;
                 }
