@@ -429,6 +429,15 @@ int cnh_kernel_build(cnh_kernel* k, const char* variant) {
 
 } // extern "C"
 
+// A launch streams past the caches (non-temporal loads and stores) when the arrays it touches
+// exceed what the 256 MiB last-level cache can hold from one launch to the next; below that the
+// next statement of a loop finds its operands there. Measured on MI355X with the arrays of a loop
+// adding up to 144 .. 384 MiB: cached 3-7 % faster up to 288 MiB, non-temporal 10 % faster at 384.
+int g_flat_nt_mib = 272;
+// The same for sweeps, where it matters more: a Jacobi sweep between two 134 MB buffers (4097^2)
+// takes 42 us with cached stores and 61.5 us with non-temporal ones; with a third array (402 MB in
+// all) 79.9 against 69.7 us; at 303 MB and above non-temporal wins by 3-8 %.
+int g_stencil_nt_mib = 272;
 namespace {
 // The memref launch. `sums` (or null): per run-time scalar, how many partial sums stand behind its
 // address and where the folded value is to be stored.
@@ -536,7 +545,7 @@ int launch_group_impl(cnh_kernel* k, int ndims, int n_parts, int n_in, const cnh
             total += n;
         }
         // Streams larger than the last-level cache bypass it; small operands (CG vectors) stay.
-        const bool nontemporal = total * (int64_t)(NL + n_out) * esz >= (128ll << 20);
+        const bool nontemporal = total * (int64_t)(NL + n_out) * esz >= ((int64_t)g_flat_nt_mib << 20);
         const char* suffix = !all_aligned ? "s" : nontemporal ? "vn" : "v";
         std::string name = std::string(live.size() == 1 ? "grp_flat1_" : "grp_flat_") + suffix;
         hipFunction_t fn;
@@ -966,7 +975,7 @@ int try_launch_slide(cnh_kernel* k, const std::vector<const cnh_tiled*>& arrays,
     int64_t volume = 1;
     for (int d = 0; d < nd; ++d)
         volume *= cur->shape[d];
-    const bool nontemporal = volume * 16 >= (128ll << 20); // read + write stream past the cache
+    const bool nontemporal = volume * 16 >= ((int64_t)g_stencil_nt_mib << 20); // read + write stream past the cache
     if (int rc = get_function(k, g_slide_cfg.variant(),
                               !vec ? "grp_slide_s" : nontemporal ? "grp_slide_vn" : "grp_slide_v", &fn))
         return rc;
@@ -1272,7 +1281,7 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
             f.gb2 = fdiv_make((uint32_t)gb[2]);
             f.obx = fdiv_make((uint32_t)f.ob[2]);
             f.oby = fdiv_make((uint32_t)f.ob[1]);
-            const bool nts = volume * 2 * esz >= (128ll << 20);
+            const bool nts = volume * (2 + n_other) * esz >= ((int64_t)g_stencil_nt_mib << 20);
             hipFunction_t fn;
             const bool reducing = red != nullptr && red->mode != 0 && p.dtype == CNH_F64 && !sh.lattice;
             if (reducing) {
@@ -1381,7 +1390,7 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
             return rc;
     a.py = (int32_t)pitch[1];
     a.pz = (int32_t)pitch[0];
-    const bool nt_stores = volume * 2 * dtype_size(p.dtype) >= (128ll << 20); // the written stream is not read back soon
+    const bool nt_stores = volume * (2 + n_other) * dtype_size(p.dtype) >= ((int64_t)g_stencil_nt_mib << 20); // the written stream is not read back soon
     // Two launches over the same grid: wavefronts that lie inside their tile in y and z take the
     // lean kernel, the other kernel does what is left (all of it when the lean one does not apply).
     // measured on MI355X: the lean kernel pays off for rank 2 (tiles much wider than a wavefront
@@ -1567,6 +1576,16 @@ extern "C" int cnh_set_option(const char* name, int value) {
     }
     if (std::strcmp(name, "direct_flat") == 0) {
         g_direct_flat = value != 0;
+        return 0;
+    }
+    if (std::strcmp(name, "flat_nt_mib") == 0) {
+        CNH_CHECK(value >= 0, -2, "threshold must not be negative");
+        g_flat_nt_mib = value;
+        return 0;
+    }
+    if (std::strcmp(name, "stencil_nt_mib") == 0) {
+        CNH_CHECK(value >= 0, -2, "threshold must not be negative");
+        g_stencil_nt_mib = value;
         return 0;
     }
     if (std::strcmp(name, "flat_tail") == 0) {

@@ -110,6 +110,9 @@ int cnh_version(void);
  *   "direct_merge"   lean part and the rest in one launch (default 1) or two
  *   "direct_flat"    arrays whose tiles are views into one row-major block take the whole-array
  *                    register-window kernel (default 1)
+ *   "flat_nt_mib", "stencil_nt_mib"  a dense launch / a sweep whose arrays add up to this many MiB or
+ *                    more streams past the caches with non-temporal accesses (default 272: what the
+ *                    256 MiB last-level cache keeps from one launch of a loop to the next)
  *   "flat_tail"      that kernel gives one or two unassigned columns beyond a multiple of 128 (the
  *                    boundary of a 2^k + 1 grid) to the wavefront before them (default 1)
  *   "flat_obz/oby/obx"  extents in elements of the blocks that kernel's workgroups are ordered by
