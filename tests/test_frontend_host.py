@@ -985,3 +985,38 @@ def test_a_dying_array_leaves_one_deletion_record_and_an_old_generation_none():
     cnp.reset()                                   # names restart: the handle names nothing any more
     del old, a
     assert lazy._state.pending == []
+
+
+@pytest.mark.parametrize("rank", [1, 2, 3])
+@pytest.mark.parametrize("seed", range(6))
+def test_random_programs_record_the_same_log_through_c_and_python(seed, rank):
+    """The random programs of the GPU suite (expressions over shifted and strided slices,
+    assignments, copies, named temporaries, sums, dots and products on windows, two element types
+    meeting), recorded twice: the two logs must be the same bytes, uploads included."""
+    A = sys.modules["charmnumeric_amd.array"]
+    if A._cnrec is None:
+        pytest.skip("recording in Python only (CHARMNUMERIC_PYREC)")
+    from tests.test_gpu_random_programs import MixedProgram, Program
+
+    def record(fast):
+        cnp.reset()
+        before = A.set_fast_recording(fast)
+        try:
+            dtype = {4: np.float32, 3: np.int64, 5: np.int32}.get(seed, np.float64)
+            prog = Program(1000 * rank + seed, rank, dtype)
+            for _ in range(18):
+                prog.statement()
+            mixed = MixedProgram(77 * rank + seed, rank)
+            for _ in range(8):
+                mixed.statement()
+            del prog, mixed
+            return [item if type(item) is bytes else ("call", item.name, item.opcode, item.dtype,
+                                                      item.payload.tobytes())
+                    for item in lazy._state.pending]
+        finally:
+            A.set_fast_recording(before)
+            cnp.reset()
+
+    fast, slow = record(True), record(False)
+    assert len(fast) == len(slow) and len(fast) > 50
+    assert fast == slow
