@@ -595,3 +595,34 @@ def test_last_column_of_a_2k_plus_1_grid(itf, shape, tail):
         assert _kernels(itf) == ["direct"] * 4
     finally:
         L.check(L.lib.cnh_set_option(b"flat_tail", 1))
+
+
+def test_large_tiled_arrays_of_a_gather_statement_are_laid_out_as_one_block(itf):
+    """A strided statement on large rank-2 arrays that have a buffer per tile runs through the
+    gather over tile tables once; the arrays are then one block each and its next occurrences (and
+    every other kind of statement on them) give NumPy's bits as before."""
+    n = 2048
+    rng = np.random.default_rng(12)
+    hr, hw = rng.standard_normal((n, n)), rng.standard_normal((n, n))
+    hc, hv = np.zeros((n // 2, n // 2)), np.zeros((n, n))
+    itf.set_min_tile(2, 512)
+    r, w = cnp.array(hr), cnp.array(hw)
+    c, v = cnp.zeros((n // 2, n // 2)), cnp.zeros((n, n))
+    mid, lo, hi = slice(2, -2, 2), slice(1, -3, 2), slice(3, -1, 2)
+    itf.set_trace()
+    for _ in range(3):
+        c[1:-1, 1:-1] = 0.25 * r[mid, mid] + 0.125 * (r[lo, mid] + r[hi, mid] + r[mid, lo] + r[mid, hi])
+        hc[1:-1, 1:-1] = 0.25 * hr[mid, mid] + 0.125 * (hr[lo, mid] + hr[hi, mid] + hr[mid, lo] + hr[mid, hi])
+        v[1:-1, 1:-1] = r[:-2, 1:-1] * w[2:, 1:-1] + r[1:-1, 2:] * w[1:-1, :-2]          # two shifted arrays
+        hv[1:-1, 1:-1] = hr[:-2, 1:-1] * hw[2:, 1:-1] + hr[1:-1, 2:] * hw[1:-1, :-2]
+        r[1:-1, 1:-1] = 0.25 * (r[:-2, 1:-1] + r[2:, 1:-1] + r[1:-1, :-2] + r[1:-1, 2:])  # an aligned sweep
+        hr[1:-1, 1:-1] = 0.25 * (hr[:-2, 1:-1] + hr[2:, 1:-1] + hr[1:-1, :-2] + hr[1:-1, 2:])
+        cnp.execute(itf)
+    y = r @ w[:, 0:1]                                          # a product on the arrays laid out anew
+    assert np.array_equal(c.get(itf), hc) and np.array_equal(v.get(itf), hv) and np.array_equal(r.get(itf), hr)
+    want = hr @ hw[:, 0]
+    assert np.all(np.abs(y.get(itf) - want) <= 1e-12 * (np.abs(hr) @ np.abs(hw[:, 0])))
+    planning = os.environ.get("CHARMNUMERIC_SOLVER", "0") not in ("", "0")
+    if not planning:
+        blocks = [ln for ln in itf.trace() if ln.startswith("block ")]
+        assert len(blocks) == 4 and all("tiles=16" in ln or "tiles=4" in ln for ln in blocks), blocks
