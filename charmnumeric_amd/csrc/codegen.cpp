@@ -906,6 +906,68 @@ __device__ __forceinline__ void block_run(const BlockArgs& a, const T* s) {
         }
     }
 }
+// The gather in place over unit steps along the rows (operands and target alike: shifted reads
+// of several arrays, halos wider than the register-window kernels take): a lane moves pairs of
+// neighbouring elements, as one 128-bit access each wherever that pair is (element-aligned), which
+// halves the memory instructions per element. A row of odd length ends in a single element.
+typedef T BP2 __attribute__((ext_vector_type(2)));
+typedef BP2 BP2A __attribute__((aligned(sizeof(T))));
+template <bool ROWS>
+__device__ __forceinline__ void block_pairs(const BlockArgs& a, const T* s) {
+    const int W0 = a.cnt[0], W1 = a.cnt[1], W2 = a.cnt[2];
+    const unsigned blk = block_order(a);
+    const unsigned group = blk / (unsigned)a.nchunks;
+    const int chunk = (int)(blk - group * (unsigned)a.nchunks);
+    int lanes = 256, lx = (int)threadIdx.x;
+    unsigned row = group;
+    if (ROWS) {
+        lanes = 256 >> a.rsh;
+        lx = (int)threadIdx.x & (lanes - 1);
+        row = (group << a.rsh) + ((unsigned)threadIdx.x >> (8 - a.rsh));
+    }
+    if (row >= (unsigned)W0 * (unsigned)W1) return;
+    const int k0 = (int)(row / (unsigned)W1), k1 = (int)(row - (unsigned)k0 * (unsigned)W1);
+    const T* rowp[NLA];
+#pragma unroll
+    for (int q = 0; q < NL; ++q) {
+        const BlockLeaf& lf = a.leaf[q];
+        rowp[q] = lf.base + ((i64)(lf.start[0] + k0 * lf.step[0]) * lf.pz + (i64)(lf.start[1] + k1 * lf.step[1]) * lf.py +
+                             lf.start[2]);
+    }
+    T* const drow = a.dst + ((i64)(a.rs[0] + k0 * a.rst[0]) * a.dpz + (i64)(a.rs[1] + k1 * a.rst[1]) * a.dpy + a.rs[2]);
+#pragma unroll
+    for (int u = 0; u < TL_PER_THREAD / 2; ++u) {
+        const int k2 = 2 * (chunk * (lanes * (TL_PER_THREAD / 2)) + u * lanes + lx);
+        if (k2 >= W2) continue;
+        const bool two = k2 + 1 < W2;
+        T l0[NLA], l1[NLA], o0[NOA], o1[NOA];
+#pragma unroll
+        for (int q = 0; q < NL; ++q) {
+            if (two) {
+                const BP2 v = *reinterpret_cast<const BP2A*>(rowp[q] + k2);
+                l0[q] = v[0];
+                l1[q] = v[1];
+            } else {
+                l0[q] = rowp[q][k2];
+                l1[q] = l0[q];
+            }
+        }
+        group_eval(l0, s, o0);
+        group_eval(l1, s, o1);
+        if (two)
+            *reinterpret_cast<BP2A*>(drow + k2) = (BP2){o0[0], o1[0]};
+        else
+            drow[k2] = o0[0];
+    }
+}
+extern "C" __global__ __launch_bounds__(256) void grp_block_pairs(BlockArgs a, Scal sc) {
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
+    block_pairs<false>(a, s);
+}
+extern "C" __global__ __launch_bounds__(256) void grp_block_pairs_rows(BlockArgs a, Scal sc) {
+    CNH_ENTRY_GUARD T s[NSV]; load_scalars(sc, s);
+    block_pairs<true>(a, s);
+}
 #if NO > 1 && NO <= 4
 // Several statements that assign interleaved lattices of one array from other arrays (the four
 // statements of a prolongation, examples/multigrid2d.py upstream) as one launch, in place: a lane

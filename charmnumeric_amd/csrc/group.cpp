@@ -1044,6 +1044,7 @@ int g_direct_group = 0; // order workgroups by groups of neighbouring tiles (ran
 int g_direct_lean = -1;   // wavefront-level lean kernel: 1 on, 0 off, -1 by rank
 int g_tiles_rows = 1;     // general gather: short rows share a workgroup
 int g_tiles_block = 1;    // general gather: arrays that are one block each skip the tile logic
+int g_block_pairs = 1;    // ... and unit-step statements among them move pairs of elements
 int g_direct_stagger = 0; // concurrent groups start at different offsets of their tiles
 int g_direct_merge = 1;   // lean part and the rest in one launch instead of two
 DirectConfig g_direct_cfg;
@@ -1578,6 +1579,10 @@ extern "C" int cnh_set_option(const char* name, int value) {
         g_direct_flat = value != 0;
         return 0;
     }
+    if (std::strcmp(name, "block_pairs") == 0) {
+        g_block_pairs = value != 0;
+        return 0;
+    }
     if (std::strcmp(name, "flat_nt_mib") == 0) {
         CNH_CHECK(value >= 0, -2, "threshold must not be negative");
         g_flat_nt_mib = value;
@@ -1881,18 +1886,25 @@ int launch_group_tiles_impl(cnh_kernel* k, int n_in, const cnh_tiled* in, int n_
                         h.cnt[d] = r == 0 ? h.rcnt[r][d] : std::max(h.cnt[d], h.rcnt[r][d]);
                     }
             }
-            const int64_t W2 = in_place ? h.cnt[2] : h.shape[2];
+            // unit steps along the rows everywhere, in place, one root: pairs of elements per access
+            bool pairs = in_place && !multi && g_block_pairs && rst[2] == 1 && NL > 0;
+            for (int l = 0; l < NL && pairs; ++l)
+                pairs = targs[13 + 7 * l + 4 + 2] == 1;
+            int64_t W2 = in_place ? h.cnt[2] : h.shape[2];
             const int64_t rows = in_place ? (int64_t)h.cnt[0] * h.cnt[1] : (int64_t)h.shape[0] * h.shape[1];
             if (rows <= 0 || W2 <= 0)
                 return 0;
+            if (pairs)
+                W2 = (W2 + 1) / 2;              // geometry in pairs: a lane takes two of them
+            const int per_lane = pairs ? 2 : 4;
             int lanes = 16;
-            while (lanes < 256 && lanes * 4 < W2)
+            while (lanes < 256 && lanes * per_lane < W2)
                 lanes *= 2;
             int rsh = 0;
             while (g_tiles_rows && (256 >> rsh) > lanes && (1 << rsh) < rows)
                 rsh++;
             lanes = 256 >> rsh;
-            const int64_t nchunks = (W2 + lanes * 4 - 1) / (lanes * 4);
+            const int64_t nchunks = (W2 + lanes * per_lane - 1) / (lanes * per_lane);
             // padded to a multiple of 8: every XCD takes a contiguous eighth of the workgroups
             const int64_t nblocks = (((rows + (1 << rsh) - 1) >> rsh) * nchunks + 7) / 8 * 8;
             if (nblocks < (1ll << 31) && rows < (1ll << 31)) {
@@ -1916,8 +1928,9 @@ int launch_group_tiles_impl(cnh_kernel* k, int n_in, const cnh_tiled* in, int n_
                     std::memcpy(args.data() + sizeof h + (size_t)l * sizeof lf, &lf, sizeof lf);
                 }
                 hipFunction_t fn;
-                const char* name = multi ? (rsh > 0 ? "grp_scatter_rows" : "grp_scatter")
-                                         : (rsh > 0 ? "grp_block_rows" : "grp_block");
+                const char* name = multi   ? (rsh > 0 ? "grp_scatter_rows" : "grp_scatter")
+                                   : pairs ? (rsh > 0 ? "grp_block_pairs_rows" : "grp_block_pairs")
+                                           : (rsh > 0 ? "grp_block_rows" : "grp_block");
                 if (int rc = get_function(k, "tiles", name, &fn))
                     return rc;
                 void* params[] = {args.data(), scal.data()};

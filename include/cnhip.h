@@ -120,6 +120,8 @@ int cnh_version(void);
  *   "tiles_rows"     general gather: rows shorter than 1024 elements share a workgroup (default 1)
  *   "tiles_block"    general gather: a launch whose arrays are one row-major block each (or single
  *                    tiles) addresses them without tile tables (default 1)
+ *   "block_pairs"    ... and statements with unit steps along the rows move pairs of elements as one
+ *                    access each (default 1). Same bits.
  *   "gemv_xlds"      matvecs of 8192 rows or more whose column tiles are at most 64 KB of x wide
  *                    stage x in LDS, 32 or 64 rows per workgroup (default 1); 0: one wavefront per
  *                    row reading x through the caches. Same bits either way.

@@ -626,3 +626,33 @@ def test_large_tiled_arrays_of_a_gather_statement_are_laid_out_as_one_block(itf)
     if not planning:
         blocks = [ln for ln in itf.trace() if ln.startswith("block ")]
         assert len(blocks) == 4 and all("tiles=16" in ln or "tiles=4" in ln for ln in blocks), blocks
+
+
+@pytest.mark.parametrize("pairs", [1, 0], ids=["pairs", "single-elements"])
+@pytest.mark.parametrize("shape", [(37, 129), (40, 131), (6, 200), (17, 19, 33), (9, 10, 130)])
+def test_shifted_reads_of_two_arrays_over_one_block_arrays(itf, shape, pairs):
+    """out[interior] = f(u shifted one way, w shifted another): no register-window kernel takes two
+    shifted arrays, so this runs as the gather over one-block arrays, by pairs of neighbouring
+    elements or one by one; rows of odd and even length, rows sharing a workgroup. NumPy's bits."""
+    from charmnumeric_amd import _lib as L
+    nd = len(shape)
+    L.check(L.lib.cnh_set_option(b"block_pairs", pairs))
+    try:
+        rng = np.random.default_rng(sum(shape))
+        hu, hw = rng.standard_normal(shape), rng.standard_normal(shape)
+        hv = np.zeros(shape)
+        u, w, v = cnp.array(hu), cnp.array(hw), cnp.zeros(shape)
+        inner = (slice(1, -1),) * nd
+        up = (slice(0, -2),) + inner[1:]
+        right = inner[:-1] + (slice(2, None),)
+        left = inner[:-1] + (slice(0, -2),)
+        itf.set_trace()
+        for _ in range(2):
+            v[inner] = u[up] * w[right] + u[right] * w[left] - 0.5 * v[inner]
+            hv[inner] = hu[up] * hw[right] + hu[right] * hw[left] - 0.5 * hv[inner]
+            u[inner] = u[inner] + 0.25 * v[left]                 # in place, reading another array shifted
+            hu[inner] = hu[inner] + 0.25 * hv[left]
+        assert np.array_equal(v.get(itf), hv) and np.array_equal(u.get(itf), hu)
+        assert _kernels(itf)[0] == "gather"
+    finally:
+        L.check(L.lib.cnh_set_option(b"block_pairs", 1))
