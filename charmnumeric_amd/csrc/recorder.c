@@ -516,6 +516,7 @@ static PyObject* binary(int which, PyObject* a, PyObject* b) {
     out->gen = (int)gen;
     PyObject* rec = PyBytes_FromStringAndSize(NULL, HEAD_BYTES + SHAPE_BYTES + na + nb);
     if (rec == NULL) {
+        out->name = 0;                      /* never recorded: nothing to delete */
         Py_DECREF(out);
         return NULL;
     }
