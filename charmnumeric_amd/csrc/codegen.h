@@ -125,6 +125,10 @@ struct DirectShape {
     // wavefront can then copy one or two columns beyond it that no statement assigns, which saves
     // the workgroups a 128 k + 1 (or + 2) wide array would otherwise launch for them.
     bool tail_ok = false;
+    // Some array other than the window array is read at shifted positions too (two arrays of a
+    // staggered or variable-coefficient stencil): the whole-array kernel then keeps a window per
+    // array; the per-tile kernels do not take such groups.
+    bool other_shifted = false;
 };
 constexpr int kDirectMaxOther = 4;
 int direct_shape(const GroupProgram& p, const DirectConfig& cfg, DirectShape& sh, std::string& err);

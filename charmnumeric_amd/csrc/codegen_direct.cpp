@@ -109,21 +109,23 @@ int direct_shape(const GroupProgram& p, const DirectConfig& cfg, DirectShape& sh
     auto shifted_at = [&](int j, size_t l) {
         return seen[j][l] && (rel[j][l][0] != 0 || rel[j][l][1] != 0 || rel[j][l][2] != 0);
     };
-    // The window array: the one array read at positions other than the element's own; the
-    // assigned array when there is none.
+    // The window array: an array read at positions other than the element's own -- the assigned
+    // one if it is among them (its sweep then goes into a second buffer), else the first such
+    // array; the assigned array when there is none. Further arrays read at shifted positions get
+    // windows of their own in the whole-array kernel (other_shifted).
     sh.window_name = p.out_target[0];
-    bool found_shifted = false;
+    bool found_shifted = false, target_shifted = false;
     for (size_t l = 0; l < NLd; ++l) {
         const LeafUse& u = p.leaves[p.load_leaf[l]];
         if (!shifted_at(0, l) && !shifted_at(1, l))
             continue;
-        if (found_shifted && u.name != sh.window_name) {
-            err = "two arrays are read at shifted positions";
-            return -18;
-        }
+        target_shifted = target_shifted || u.name == p.out_target[0];
+        if (!found_shifted)
+            sh.window_name = u.name;
         found_shifted = true;
-        sh.window_name = u.name;
     }
+    if (target_shifted)
+        sh.window_name = p.out_target[0];
     sh.masked = sh.window_name != p.out_target[0];
     if (sh.masked && sh.lattice) {
         err = "a lattice sweep reads its own array through the window";
@@ -134,10 +136,18 @@ int direct_shape(const GroupProgram& p, const DirectConfig& cfg, DirectShape& sh
     for (size_t l = 0; l < NLd; ++l) {
         const LeafUse& u = p.leaves[p.load_leaf[l]];
         if (u.name != sh.window_name) {
-            // another array (a source term, a weight): only at the element's own position
+            // another array (a source term, a weight): at the element's own position, or shifted
+            // (a window of its own, whole-array kernel, one root, unit steps)
             if (shifted_at(0, l) || shifted_at(1, l)) {
-                err = "operand of another array is shifted";
-                return -18;
+                if (sh.lattice || nroots != 1) {
+                    err = "a lattice sweep reads other arrays at the element's own position only";
+                    return -18;
+                }
+                sh.other_shifted = true;
+                for (int d = 0; d < 3; ++d) {
+                    sh.shifts[l][(size_t)d] = rel[0][l][(size_t)d];
+                    sh.halo[d] = std::max(sh.halo[d], std::abs(rel[0][l][(size_t)d]));
+                }
             }
             size_t j = 0;
             while (j < sh.other_names.size() && sh.other_names[j] != u.name)
@@ -232,13 +242,30 @@ std::string direct_source(const GroupProgram& p, const DirectConfig& cfg, std::s
             if (!sh.masked)
                 at(rz + H0, ry + H1, HK) = 1; // the element itself (kept outside the assigned region)
             for (int e = 0; e < 2; ++e) {
-                for (const auto& s : sh.shifts)
+                for (size_t l = 0; l < sh.shifts.size(); ++l) {
+                    if (sh.other_shifted && sh.other[l] >= 0)
+                        continue;                 // read through its own array's window, below
+                    const auto& s = sh.shifts[l];
                     at(rz + H0 + s[0], ry + H1 + s[1], HK + floordiv2(e + s[2])) = 1;
+                }
                 if (sh.nroots > 1)
                     for (const auto& s : sh.shifts2)
                         at(rz + H0 + s[0], ry + H1 + s[1], HK + floordiv2(e + s[2])) = 1;
             }
         }
+    // the same per other array, when some of them are read at shifted positions
+    const int NOTH0 = (int)sh.other_names.size();
+    std::vector<int> oneed((size_t)std::max(1, NOTH0) * WZ * WY * WK, 0);
+    auto oat = [&](int j, int z, int y, int k) -> int& { return oneed[(((size_t)j * WZ + z) * WY + y) * WK + k]; };
+    if (sh.other_shifted)
+        for (int rz = 0; rz < sh.rz; ++rz)
+            for (int ry = 0; ry < sh.ry; ++ry)
+                for (int e = 0; e < 2; ++e)
+                    for (size_t l = 0; l < sh.shifts.size(); ++l)
+                        if (sh.other[l] >= 0) {
+                            const auto& sft = sh.shifts[l];
+                            oat(sh.other[l], rz + H0 + sft[0], ry + H1 + sft[1], HK + floordiv2(e + sft[2])) = 1;
+                        }
     std::ostringstream s;
     s << pre;
     s << "#define DR_TX " << sh.tx << "\n#define DR_TY " << sh.ty << "\n#define DR_RY " << sh.ry
@@ -258,6 +285,7 @@ std::string direct_source(const GroupProgram& p, const DirectConfig& cfg, std::s
     const int NOTH = (int)sh.other_names.size();
     s << "#define DR_MASKED " << (sh.masked ? 1 : 0) << "\n";
     s << "#define DR_TAIL_OK " << (sh.tail_ok ? 1 : 0) << "\n";
+    s << "#define DR_OSH " << (sh.other_shifted ? 1 : 0) << "\n";
     s << "#define DR_RED " << (cfg.reduce ? 1 : 0) << "\n";
     s << "#define DR_NOTH " << NOTH << "\n#define DR_NOTHA " << (NOTH > 0 ? NOTH : 1) << "\n";
     s << "__device__ constexpr int DR_OTHER[NLA] = {";
@@ -289,6 +317,22 @@ std::string direct_source(const GroupProgram& p, const DirectConfig& cfg, std::s
             s << (y ? ", " : "") << "{";
             for (int k = 0; k < WK; ++k)
                 s << (k ? ", " : "") << (at(z, y, k) ? "true" : "false");
+            s << "}";
+        }
+        s << "}";
+    }
+    s << "};\n";
+    s << "__device__ constexpr bool DR_ONEED[DR_NOTHA][DR_WZ][DR_WY][DR_WK] = {";
+    for (int j = 0; j < std::max(1, NOTH0); ++j) {
+        s << (j ? ", " : "") << "{";
+        for (int z = 0; z < WZ; ++z) {
+            s << (z ? ", " : "") << "{";
+            for (int y = 0; y < WY; ++y) {
+                s << (y ? ", " : "") << "{";
+                for (int k = 0; k < WK; ++k)
+                    s << (k ? ", " : "") << (oat(j, z, y, k) ? "true" : "false");
+                s << "}";
+            }
             s << "}";
         }
         s << "}";
@@ -941,13 +985,49 @@ __device__ __forceinline__ void direct_flat(const FlatArgs& a, const T* s) {
         }
     }
     P2 ov[DR_NOTHA][DR_RZ][DR_RY];
+    if (!DR_OSH) {
 #pragma unroll
-    for (int j = 0; j < DR_NOTH; ++j)
+        for (int j = 0; j < DR_NOTH; ++j)
 #pragma unroll
-        for (int rz = 0; rz < DR_RZ; ++rz)
+            for (int rz = 0; rz < DR_RZ; ++rz)
 #pragma unroll
-            for (int ry = 0; ry < DR_RY; ++ry)
-                ov[j][rz][ry] = load_pair<UA>(a.oth[j] + (zo[rz + DR_H0] + yo[ry + DR_H1]), cx, S2);
+                for (int ry = 0; ry < DR_RY; ++ry)
+                    ov[j][rz][ry] = load_pair<UA>(a.oth[j] + (zo[rz + DR_H0] + yo[ry + DR_H1]), cx, S2);
+    }
+    // Other arrays read at shifted positions: a window per array, the same clamped rows and planes,
+    // the left and right pairs by lane exchange, the pairs beyond the wavefront's ends by one more
+    // load per row in which the first and the last lane fetch theirs.
+    P2 wo[DR_NOTHA][DR_WZ][DR_WY][DR_WK];      // unused (and gone from the code) unless DR_OSH
+    if (DR_OSH) {
+#pragma unroll
+        for (int j = 0; j < DR_NOTH; ++j)
+#pragma unroll
+            for (int i = 0; i < DR_WZ; ++i)
+#pragma unroll
+                for (int jj = 0; jj < DR_WY; ++jj) {
+                    const bool side0 = DR_HK == 1 && DR_ONEED[j][i][jj][0];
+                    const bool side1 = DR_HK == 1 && DR_ONEED[j][i][jj][DR_WK - 1];
+                    if (DR_ONEED[j][i][jj][DR_HK] || side0 || side1)
+                        wo[j][i][jj][DR_HK] =
+                            load_pair<UA>(a.oth[j] + (zo[i] + yo[jj]), cx, S2);
+                    if (side0 || side1) {
+                        const P2 mid = wo[j][i][jj][DR_HK];
+                        const P2 far = load_pair<UA>(a.oth[j] + (zo[i] + yo[jj]), first ? xl : (last ? xr : cx), S2);
+                        if (side0) {
+                            P2 sh;
+                            sh[0] = from_prev_lane(mid[0]);
+                            sh[1] = from_prev_lane(mid[1]);
+                            wo[j][i][jj][0] = first ? far : sh;
+                        }
+                        if (side1) {
+                            P2 sh;
+                            sh[0] = from_next_lane(mid[0]);
+                            sh[1] = from_next_lane(mid[1]);
+                            wo[j][i][jj][DR_WK - 1] = last ? far : sh;
+                        }
+                    }
+                }
+    }
     if (DR_HK == 1) {
 #pragma unroll
         for (int i = 0; i < DR_WZ; ++i)
@@ -999,8 +1079,11 @@ __device__ __forceinline__ void direct_flat(const FlatArgs& a, const T* s) {
 #pragma unroll
                 for (int q = 0; q < NL; ++q) {
                     const int xx = e + DR_SHIFT[q][2];
+                    const int oj = DR_OTHER[q] >= 0 ? DR_OTHER[q] : 0;
                     l[q] = DR_OTHER[q] >= 0
-                               ? ov[DR_OTHER[q] >= 0 ? DR_OTHER[q] : 0][rz][ry][e]
+                               ? (DR_OSH ? wo[oj][rz + DR_H0 + DR_SHIFT[q][0]][ry + DR_H1 + DR_SHIFT[q][1]]
+                                             [DR_HK + floordiv2(xx)][xx & 1]
+                                         : ov[oj][rz][ry][e])
                                : win[rz + DR_H0 + DR_SHIFT[q][0]][ry + DR_H1 + DR_SHIFT[q][1]]
                                     [DR_HK + floordiv2(xx)][xx & 1];
                 }

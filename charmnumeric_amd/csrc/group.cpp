@@ -1315,8 +1315,8 @@ int launch_direct(cnh_kernel* k, const DirectShape& sh, const std::vector<const 
             return 0;
         }
     }
-    if (!aligned || sh.lattice)
-        return 0;                         // the per-tile kernels take aligned unit-step sweeps only
+    if (!aligned || sh.lattice || sh.other_shifted)
+        return 0;                         // the per-tile kernels take aligned unit-step sweeps of one window only
     // a lane's own rows and planes must not straddle tiles: the tile edge (a power of two) has
     // to be a multiple of what one lane owns
     if (cur->tile % sh.ry != 0 || cur->tile % sh.rz != 0)

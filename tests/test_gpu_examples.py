@@ -628,15 +628,18 @@ def test_large_tiled_arrays_of_a_gather_statement_are_laid_out_as_one_block(itf)
         assert len(blocks) == 4 and all("tiles=16" in ln or "tiles=4" in ln for ln in blocks), blocks
 
 
-@pytest.mark.parametrize("pairs", [1, 0], ids=["pairs", "single-elements"])
-@pytest.mark.parametrize("shape", [(37, 129), (40, 131), (6, 200), (17, 19, 33), (9, 10, 130)])
-def test_shifted_reads_of_two_arrays_over_one_block_arrays(itf, shape, pairs):
-    """out[interior] = f(u shifted one way, w shifted another): no register-window kernel takes two
-    shifted arrays, so this runs as the gather over one-block arrays, by pairs of neighbouring
-    elements or one by one; rows of odd and even length, rows sharing a workgroup. NumPy's bits."""
+@pytest.mark.parametrize("route", ["windows", "gather-pairs", "gather-single-elements"])
+@pytest.mark.parametrize("shape", [(37, 129), (40, 131), (6, 200), (150, 258), (17, 19, 33), (9, 10, 130), (12, 9, 257)])
+def test_shifted_reads_of_two_arrays_over_one_block_arrays(itf, shape, route):
+    """out[interior] = f(u shifted one way, w shifted another) on arrays stored as one block: the
+    whole-array register-window kernel keeps a window per array; with the stencil kernels switched
+    off the same statements run as the gather, by pairs of neighbouring elements or one by one.
+    Rows of odd and even length, rows sharing a workgroup, more than one wavefront per row. NumPy's
+    bits on every route."""
     from charmnumeric_amd import _lib as L
     nd = len(shape)
-    L.check(L.lib.cnh_set_option(b"block_pairs", pairs))
+    L.check(L.lib.cnh_set_option(b"stencil_mode", 2 if route == "windows" else 0))
+    L.check(L.lib.cnh_set_option(b"block_pairs", 0 if route == "gather-single-elements" else 1))
     try:
         rng = np.random.default_rng(sum(shape))
         hu, hw = rng.standard_normal(shape), rng.standard_normal(shape)
@@ -644,6 +647,7 @@ def test_shifted_reads_of_two_arrays_over_one_block_arrays(itf, shape, pairs):
         u, w, v = cnp.array(hu), cnp.array(hw), cnp.zeros(shape)
         inner = (slice(1, -1),) * nd
         up = (slice(0, -2),) + inner[1:]
+        down = (slice(2, None),) + inner[1:]
         right = inner[:-1] + (slice(2, None),)
         left = inner[:-1] + (slice(0, -2),)
         itf.set_trace()
@@ -652,7 +656,12 @@ def test_shifted_reads_of_two_arrays_over_one_block_arrays(itf, shape, pairs):
             hv[inner] = hu[up] * hw[right] + hu[right] * hw[left] - 0.5 * hv[inner]
             u[inner] = u[inner] + 0.25 * v[left]                 # in place, reading another array shifted
             hu[inner] = hu[inner] + 0.25 * hv[left]
-        assert np.array_equal(v.get(itf), hv) and np.array_equal(u.get(itf), hu)
-        assert _kernels(itf)[0] == "gather"
+            w[inner] = 0.5 * (w[down] + w[left]) * u[up] + v[right]   # the target and two others, all shifted
+            hw[inner] = 0.5 * (hw[down] + hw[left]) * hu[up] + hv[right]
+        assert np.array_equal(v.get(itf), hv) and np.array_equal(u.get(itf), hu) and np.array_equal(w.get(itf), hw)
+        planning = os.environ.get("CHARMNUMERIC_SOLVER", "0") not in ("", "0")
+        if not planning:
+            assert set(_kernels(itf)) == {"direct" if route == "windows" else "gather"}
     finally:
+        L.check(L.lib.cnh_set_option(b"stencil_mode", 2))
         L.check(L.lib.cnh_set_option(b"block_pairs", 1))
