@@ -1,5 +1,6 @@
 // Register-window source for same-array unit-step stencils (the Jacobi-style SET_REGION groups),
-// optionally with operands of other arrays read at the element's own position (source terms).
+// optionally with operands of other arrays read at the element's own position (source terms) or,
+// in the whole-array kernel, at shifted positions too (a window per array).
 //
 // Every lane owns RZ x RY output rows of one 16-byte column pair inside ONE tile. It first issues
 // all the 128-bit loads of its window (the rows and planes its shifted operands touch, aligned
