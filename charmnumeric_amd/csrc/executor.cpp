@@ -334,7 +334,7 @@ int make_array(Ex* ex, int name, int ndims, int dtype, const int32_t* shape, boo
             for (int d = 0; d < ndims; ++d)
                 a.offset[d] = p.offset[d];
         } else {
-            ex->log("plan for " + std::to_string(name) + " does not fit the array; tile rule used");
+            if (ex->trace_on) ex->log("plan for " + std::to_string(name) + " does not fit the array; tile rule used");
         }
         ex->planned.erase(plan);
     }
@@ -389,7 +389,7 @@ int make_array(Ex* ex, int name, int ndims, int dtype, const int32_t* shape, boo
         return rc;
     for (int64_t t = 0; t < a.ntiles; ++t)
         a.tiles.push_back(static_cast<char*>(a.slab) + a.tile_off[t]);
-    ex->log("create " + std::to_string(name) + " shape=" + shape_str(a.shape, ndims) + " dtype=" +
+    if (ex->trace_on) ex->log("create " + std::to_string(name) + " shape=" + shape_str(a.shape, ndims) + " dtype=" +
             std::to_string(dtype) + " tile=" + std::to_string(a.tile) + " tiles=" +
             std::to_string(a.ntiles) + (a.phased() || a.offset[0] || a.offset[1] || a.offset[2]
                                             ? " offset=" + shape_str(a.offset, ndims)
@@ -427,7 +427,7 @@ void drop_array(Ex* ex, int name) {
     slab_release(ex, it->second.bytes, it->second.alt);
     ex->arrays.erase(it);
     ex->stats[6] = (int64_t)ex->arrays.size();
-    ex->log("delete " + std::to_string(name));
+    if (ex->trace_on) ex->log("delete " + std::to_string(name));
 }
 
 int find_array(Ex* ex, int name, XArray** out, const char* what) {
@@ -476,6 +476,22 @@ uint64_t fnv(const void* data, size_t n, uint64_t h = 1469598103934665603ull) {
     for (size_t i = 0; i < n; ++i) {
         h ^= p[i];
         h *= 1099511628211ull;
+    }
+    return h;
+}
+// The compile cache's key: 8 bytes per step (multiply, fold the high half back), the rest byte by
+// byte. A key that collides only costs a comparison of the groups themselves (compile_cached).
+uint64_t mix_words(const void* data, size_t n, uint64_t h = 0x9E3779B97F4A7C15ull) {
+    const unsigned char* p = static_cast<const unsigned char*>(data);
+    for (; n >= 8; n -= 8, p += 8) {
+        uint64_t w;
+        std::memcpy(&w, p, 8);
+        h = (h ^ w) * 0xD6E8FEB86659FD93ull;
+        h ^= h >> 32;
+    }
+    for (; n > 0; --n, ++p) {
+        h = (h ^ *p) * 0x100000001B3ull;
+        h ^= h >> 29;
     }
     return h;
 }
@@ -541,14 +557,14 @@ int exec_fill(Ex* ex, XArray& a, const cnh_region& reg, double value) {
                                          ex->stream))
                 return rc;
     }
-    ex->log("fill " + std::to_string(a.name) + " tiles_touched=" + std::to_string(launches));
+    if (ex->trace_on) ex->log("fill " + std::to_string(a.name) + " tiles_touched=" + std::to_string(launches));
     return 0;
 }
 
 struct Group {
     std::vector<cnh_ast_node> nodes; // canonical names
     std::vector<int32_t> roots;
-    std::map<int, int> canon_to_actual;
+    std::vector<int> canon_to_actual;   // indexed by canonical name (1, 2, ...)
     int dtype = CNH_F64;
     int ndims = 1;
     uint64_t key = 0;
@@ -559,15 +575,22 @@ struct Group {
 void canonicalise(const DagNode& n, Group& g) {
     g.nodes = n.nodes;
     g.roots = n.roots;
-    std::map<int, int> to_canon;
-    int next = 1;
+    // a group has a few dozen names at most: a flat list searched from the back (the operand
+    // just produced is the likeliest match) beats a tree of allocated nodes
+    g.canon_to_actual.assign(1, 0);
+    g.canon_to_actual.reserve(g.nodes.size() + 1);
     for (auto& a : g.nodes) {
-        auto it = to_canon.find(a.result_name);
-        if (it == to_canon.end()) {
-            it = to_canon.emplace(a.result_name, next++).first;
-            g.canon_to_actual[it->second] = a.result_name;
+        int canon = 0;
+        for (int c = (int)g.canon_to_actual.size() - 1; c >= 1; --c)
+            if (g.canon_to_actual[(size_t)c] == a.result_name) {
+                canon = c;
+                break;
+            }
+        if (canon == 0) {
+            canon = (int)g.canon_to_actual.size();
+            g.canon_to_actual.push_back(a.result_name);
         }
-        a.result_name = a.is_scalar ? -it->second : it->second;
+        a.result_name = a.is_scalar ? -canon : canon;
     }
     // Element type of the kernel: the first root that is not F32 decides (src/jit.cpp:50-69).
     g.dtype = CNH_F32;
@@ -577,20 +600,20 @@ void canonicalise(const DagNode& n, Group& g) {
             break;
         }
     g.ndims = g.nodes[g.roots.back()].ndims;
-    uint64_t h = fnv(&g.dtype, sizeof g.dtype);
-    h = fnv(&g.ndims, sizeof g.ndims, h);
+    uint64_t h = mix_words(&g.dtype, sizeof g.dtype);
+    h = mix_words(&g.ndims, sizeof g.ndims, h);
     for (auto& a : g.nodes) {
         // hash field by field: the struct has padding
         int32_t head[10] = {a.result_name, a.opcode, a.is_temp, a.is_scalar, a.is_broadcast,
                             a.ndims, a.dtype, a.n_operands, a.operands[0], a.operands[1]};
-        h = fnv(head, sizeof head, h);
-        h = fnv(&a.scalar, sizeof a.scalar, h);
-        h = fnv(a.has_operand_region, sizeof a.has_operand_region, h);
-        h = fnv(&a.operand_regions[0], sizeof(cnh_region), h);
-        h = fnv(&a.operand_regions[1], sizeof(cnh_region), h);
-        h = fnv(&a.region, sizeof(cnh_region), h);
+        h = mix_words(head, sizeof head, h);
+        h = mix_words(&a.scalar, sizeof a.scalar, h);
+        h = mix_words(a.has_operand_region, sizeof a.has_operand_region, h);
+        h = mix_words(&a.operand_regions[0], sizeof(cnh_region), h);
+        h = mix_words(&a.operand_regions[1], sizeof(cnh_region), h);
+        h = mix_words(&a.region, sizeof(cnh_region), h);
     }
-    h = fnv(g.roots.data(), g.roots.size() * sizeof(int32_t), h);
+    h = mix_words(g.roots.data(), g.roots.size() * sizeof(int32_t), h);
     g.key = h;
 }
 
@@ -807,7 +830,7 @@ int exec_group(Ex* ex, const DagNode& n) {
                 fill(in[(size_t)t * n_in + i], in_arr[i]->tiles[t]);
             fill(out[(size_t)t], target->tiles[t]);
         }
-        ex->log("group node=" + std::to_string(n.id) + " path=dense parts=" + std::to_string(parts) +
+        if (ex->trace_on) ex->log("group node=" + std::to_string(n.id) + " path=dense parts=" + std::to_string(parts) +
                 " inputs=" + std::to_string(n_in) + " scalars=" + std::to_string(n_scalar) +
                 " out=" + std::to_string(target->name));
         if (ex->dry)
@@ -941,7 +964,7 @@ int exec_group(Ex* ex, const DagNode& n) {
     const char* used = ex->dry ? "" : cnh_kernel_variants_loaded(k, "direct") > 0 ? " kernel=direct"
                                   : cnh_kernel_variants_loaded(k, "slide") > 0  ? " kernel=slide"
                                                                                 : " kernel=gather";
-    ex->log("group node=" + std::to_string(n.id) + " path=tiles inputs=" + std::to_string(n_in) +
+    if (ex->trace_on) ex->log("group node=" + std::to_string(n.id) + " path=tiles inputs=" + std::to_string(n_in) +
             " scalars=" + std::to_string(n_scalar) + " out=" + std::to_string(target->name) +
             (aliased ? " pingpong" : " inplace") + used);
     if (aliased) {
@@ -1034,7 +1057,7 @@ int relayout(Ex* ex, XArray* src, int tile, const int32_t* offset, XArray** out)
     dn.nodes[1].opcode = CNH_OP_COPY;
     dn.nodes[1].n_operands = 1;
     dn.roots = {1};
-    ex->log("relayout " + std::to_string(src->name) + " tile=" + std::to_string(tile) + " offset=" +
+    if (ex->trace_on) ex->log("relayout " + std::to_string(src->name) + " tile=" + std::to_string(tile) + " offset=" +
             shape_str(p.offset, src->ndims));
     if (int rc = exec_group(ex, dn))
         return rc;
@@ -1103,7 +1126,7 @@ int exec_reduce(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
         pb.push_back(static_cast<const char*>(b->tiles[0]) + (first - wa.start[0] + wb.start[0]) * esz);
         cnt.push_back(last - first);
     }
-    ex->log("reduce " + std::to_string(a->name) + "." + std::to_string(b->name) + " tiles=" +
+    if (ex->trace_on) ex->log("reduce " + std::to_string(a->name) + "." + std::to_string(b->name) + " tiles=" +
             std::to_string(pa.size()) + " out=" + std::to_string(out->name));
     if (ex->dry)
         return 0;
@@ -1133,7 +1156,7 @@ int exec_reduce_ext(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
     XArray* out;
     if (int rc = new_scalar_array(ex, root.result_name, a->dtype, &out))
         return rc;
-    ex->log("reduce_ext op=" + std::to_string(root.opcode) + " tiles=" + std::to_string(a->ntiles) +
+    if (ex->trace_on) ex->log("reduce_ext op=" + std::to_string(root.opcode) + " tiles=" + std::to_string(a->ntiles) +
             " out=" + std::to_string(out->name));
     int rc = 0;
     if (!ex->dry) {
@@ -1218,7 +1241,7 @@ int exec_astype(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
                     return rc;
         }
     }
-    ex->log("astype in=" + std::to_string(in->name) + " out=" + std::to_string(out->name) + " dtype=" +
+    if (ex->trace_on) ex->log("astype in=" + std::to_string(in->name) + " out=" + std::to_string(out->name) + " dtype=" +
             std::to_string(out->dtype) + " launches=" + std::to_string(launches));
     return 0;
 }
@@ -1445,7 +1468,7 @@ int exec_matmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
     XArray* y;
     if (int rc = make_array(ex, root.result_name, 1, Aa->dtype, shape, false, &y))
         return rc;
-    ex->log("matmul A=" + std::to_string(Aa->name) + " tiles=" + std::to_string(Aa->ntiles) + " x=" +
+    if (ex->trace_on) ex->log("matmul A=" + std::to_string(Aa->name) + " tiles=" + std::to_string(Aa->ntiles) + " x=" +
             std::to_string(x->name) + " out=" + std::to_string(y->name));
     int rc = 0;
     if (!ex->dry) {
@@ -1579,7 +1602,7 @@ int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root, const Dag
     if (!ex->dry)
         if (int rc = cnh_gemm_batch(Aa->dtype, (int)jobs.size(), jobs.data(), f64 ? 1 : 0, ex->stream))
             return rc;
-    ex->log("matmatmul A=" + std::to_string(Aa->name) + " B=" + std::to_string(Ba->name) + " out=" +
+    if (ex->trace_on) ex->log("matmatmul A=" + std::to_string(Aa->name) + " B=" + std::to_string(Ba->name) + " out=" +
             std::to_string(Cc ? Cc->name : dest_name) + (Cc ? "" : " into_region") + " panel_products=" +
             std::to_string(calls));
     if (a_copy)
@@ -1689,7 +1712,7 @@ int exec_tile(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
                     }
         }
     }
-    ex->log("tile in=" + std::to_string(in->name) + " out=" + std::to_string(out->name) + " shape=" +
+    if (ex->trace_on) ex->log("tile in=" + std::to_string(in->name) + " out=" + std::to_string(out->name) + " shape=" +
             shape_str(out->shape, nd) + " copies=" + std::to_string(copies));
     return 0;
 }
@@ -1755,7 +1778,7 @@ int exec_diag(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
         if (rc)
             return rc;
     }
-    ex->log("diag in=" + std::to_string(in->name) + " out=" + std::to_string(out->name) + " k=" +
+    if (ex->trace_on) ex->log("diag in=" + std::to_string(in->name) + " out=" + std::to_string(out->name) + " k=" +
             std::to_string(k) + " copies=" + std::to_string(copies));
     return 0;
 }
@@ -2082,7 +2105,7 @@ int exec_statement_run(Ex* ex, const std::vector<Stmt>& run) {
     std::string names;
     for (const Stmt& st : run)
         names += (names.empty() ? "" : ",") + std::to_string(st.out.arr->name);
-    ex->log("group node=" + std::to_string(merged.id) + " path=statements count=" +
+    if (ex->trace_on) ex->log("group node=" + std::to_string(merged.id) + " path=statements count=" +
             std::to_string(run.size()) + " inputs=" + std::to_string(n_in) + " outputs=" +
             std::to_string(n_out) + " out=" + names);
     if (ex->dry)
@@ -2427,7 +2450,7 @@ int try_group_with_reductions(Ex* ex, const std::vector<DagNode>& dag, size_t i,
                  out_arr[(size_t)q] != target);
     }
     ex->stats[5]++;
-    ex->log("group node=" + std::to_string(n.id) + " path=dense+reduce parts=" + std::to_string(parts) +
+    if (ex->trace_on) ex->log("group node=" + std::to_string(n.id) + " path=dense+reduce parts=" + std::to_string(parts) +
             " inputs=" + std::to_string(n_in) + " scalars=" + std::to_string(n_scalar) + " reductions=" +
             std::to_string(reds.size()) + " out=" + std::to_string(target->name));
     int rc = 0;
@@ -2475,7 +2498,7 @@ int resolve_pending(Ex* ex, int name) {
     int rc = 0;
     auto arr = ex->arrays.find(name);
     if (arr != ex->arrays.end()) {
-        ex->log("fold " + std::to_string(name) + " partials=" + std::to_string(it->second.count));
+        if (ex->trace_on) ex->log("fold " + std::to_string(name) + " partials=" + std::to_string(it->second.count));
         if (!ex->dry)
             rc = cnh_fold_sums(it->second.partials, it->second.count, arr->second.tiles[0], ex->stream);
     }
@@ -2757,7 +2780,7 @@ int try_fused_matvec(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t* 
         fu.dot_partials = dot_sums.partials;
         fu.dot_capacity = nb;
     }
-    ex->log("matmul A=" + std::to_string(mv.A->name) + " tiles=" + std::to_string(mv.A->ntiles) + " x=" +
+    if (ex->trace_on) ex->log("matmul A=" + std::to_string(mv.A->name) + " tiles=" + std::to_string(mv.A->ntiles) + " x=" +
             std::to_string(mv.x_name) + " out=" + std::to_string(mv.y_name) + " fused" +
             (form ? " vector=" + std::to_string(xa_name) + "+(" + std::to_string(num_name) + "/" +
                         std::to_string(den_name) + ")*" + std::to_string(xb_name)
@@ -3188,7 +3211,7 @@ int try_dense_run(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t* use
         }
     }
     ex->stats[5]++;
-    ex->log("group node=" + std::to_string(merged.id) + " path=run statements=" + std::to_string(stmts.size()) +
+    if (ex->trace_on) ex->log("group node=" + std::to_string(merged.id) + " path=run statements=" + std::to_string(stmts.size()) +
             " scalars_formed=" + std::to_string(scal_results.size()) + " reductions=" + std::to_string(reds.size()) +
             " inputs=" + std::to_string(n_in) + " scalars=" + std::to_string(n_scalar) + " sums_taken=" +
             std::to_string(taken.size()) + " out=" + out_names);
@@ -3270,7 +3293,7 @@ int make_block(Ex* ex, XArray& a) {
     a.tile_off = offs;
     for (int64_t t = 0; t < a.ntiles; ++t)
         a.tiles[(size_t)t] = static_cast<char*>(block) + offs[(size_t)t];
-    ex->log("block " + std::to_string(a.name) + " tiles=" + std::to_string(a.ntiles));
+    if (ex->trace_on) ex->log("block " + std::to_string(a.name) + " tiles=" + std::to_string(a.ntiles));
     return 0;
 }
 
@@ -3454,7 +3477,7 @@ int try_scatter_run(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t* u
         if (int rc = cnh_launch_group_tiles(k, n_in, tin.data(), n_scalar, scalars.data(), 1, &cur, &cur, ex->stream))
             return rc == -17 ? 0 : rc;          // not a shape the scatter takes: statement by statement
     ex->stats[5]++;
-    ex->log("group node=" + std::to_string(merged.id) + " path=scatter roots=" + std::to_string(parts.size()) +
+    if (ex->trace_on) ex->log("group node=" + std::to_string(merged.id) + " path=scatter roots=" + std::to_string(parts.size()) +
             " inputs=" + std::to_string(n_in) + " scalars=" + std::to_string(n_scalar) + " out=" +
             std::to_string(ta->name) + " inplace");
     for (int name : dels)
@@ -3538,7 +3561,7 @@ int try_lattice_pair(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t* 
         tin[(size_t)q] = in_arr[(size_t)q]->tiled();
     const cnh_tiled cur = ta->tiled();
     ex->stats[5]++;
-    ex->log("group node=" + std::to_string(merged.id) + " path=lattices roots=2 inputs=" + std::to_string(n_in) +
+    if (ex->trace_on) ex->log("group node=" + std::to_string(merged.id) + " path=lattices roots=2 inputs=" + std::to_string(n_in) +
             " scalars=" + std::to_string(n_scalar) + " out=" + std::to_string(ta->name) + " inplace");
     if (!ex->dry)
         if (int rc = cnh_launch_group_tiles(k, n_in, tin.data(), n_scalar, scalars.data(), 1, &cur, &cur, ex->stream))
@@ -3796,7 +3819,7 @@ void plan_message(Ex* ex, const std::vector<DagNode>& dag) {
             p.offset[d] = m.offset[d];
         }
         ex->planned[name] = p;
-        ex->log("plan " + std::to_string(name) + " tile=" + std::to_string(p.tile) + " offset=" +
+        if (ex->trace_on) ex->log("plan " + std::to_string(name) + " tile=" + std::to_string(p.tile) + " offset=" +
                 shape_str(p.offset, p.ndims));
     }
 }
@@ -4293,7 +4316,7 @@ int cnx_get(cnx_executor* ex, int ndims, int epoch, int name, int64_t size, int 
     CNH_CHECK(a->ndims == ndims && a->dtype == dtype && a->elems == size, -50,
               "get of array %d: asked for rank %d dtype %d size %lld, array has rank %d dtype %d size %lld",
               name, ndims, dtype, (long long)size, a->ndims, a->dtype, (long long)a->elems);
-    ex->log("get " + std::to_string(name) + " tiles=" + std::to_string(a->ntiles));
+    if (ex->trace_on) ex->log("get " + std::to_string(name) + " tiles=" + std::to_string(a->ntiles));
     if (ex->dry) {
         std::memset(host_out, 0, (size_t)size * dtype_size(dtype));
         return 0;
@@ -4339,7 +4362,7 @@ int cnx_put(cnx_executor* ex, int name, int64_t size, int dtype, const void* hos
     CNH_CHECK(a->dtype == dtype && a->elems == size, -50,
               "put into array %d: %lld elements of dtype %d offered, array has %lld of dtype %d", name,
               (long long)size, dtype, (long long)a->elems, a->dtype);
-    ex->log("put " + std::to_string(name));
+    if (ex->trace_on) ex->log("put " + std::to_string(name));
     if (ex->dry)
         return 0;
     const int esz = dtype_size(dtype);
@@ -4381,7 +4404,7 @@ int cnx_fill_uniform(cnx_executor* ex, int name, uint64_t seed, uint64_t stream_
     if (int rc = find_array(ex, name, &a, "fill_uniform"))
         return rc;
     CNH_CHECK(a->dtype == CNH_F64, -27, "fill_uniform needs an fp64 array");
-    ex->log("fill_uniform " + std::to_string(name));
+    if (ex->trace_on) ex->log("fill_uniform " + std::to_string(name));
     if (ex->dry)
         return 0;
     int64_t gshape[3];
@@ -4414,7 +4437,7 @@ int cnx_fill_cg_matrix(cnx_executor* ex, int name, uint64_t seed) {
         return rc;
     CNH_CHECK(a->dtype == CNH_F64 && a->ndims == 2 && a->shape[0] == a->shape[1], -27,
               "fill_cg_matrix needs a square fp64 array");
-    ex->log("fill_cg_matrix " + std::to_string(name));
+    if (ex->trace_on) ex->log("fill_cg_matrix " + std::to_string(name));
     if (ex->dry)
         return 0;
     for (int64_t t = 0; t < a->ntiles; ++t) {

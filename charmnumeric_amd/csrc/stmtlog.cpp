@@ -17,14 +17,64 @@
 #include "common.h"
 
 #include <cstring>
-#include <map>
-#include <unordered_map>
-#include <unordered_set>
 
 namespace cnh {
 namespace stmtlog {
 
 namespace {
+
+// int32 -> int32 table for array names (open addressing, sized for the batch at hand): the planner
+// looks names up a few times per record, and tree or node-based tables spend more time in the
+// allocator than in the plan.
+class NameTable {
+public:
+    explicit NameTable(size_t expected) {
+        size_t cap = 16;
+        while (cap < expected * 2 + 2)
+            cap *= 2;
+        keys_.assign(cap, kEmpty);
+        vals_.assign(cap, 0);
+    }
+    int32_t* find(int32_t key) {
+        const size_t i = slot(key);
+        return keys_[i] == key ? &vals_[i] : nullptr;
+    }
+    const int32_t* find(int32_t key) const { return const_cast<NameTable*>(this)->find(key); }
+    bool has(int32_t key) const { return find(key) != nullptr; }
+    // the value for `key`, inserted as `fresh` when new
+    int32_t& at(int32_t key, int32_t fresh = 0) {
+        if ((count_ + 1) * 2 > keys_.size())
+            grow();
+        const size_t i = slot(key);
+        if (keys_[i] != key) {
+            keys_[i] = key;
+            vals_[i] = fresh;
+            ++count_;
+        }
+        return vals_[i];
+    }
+    void insert(int32_t key) { (void)at(key, 1); }
+
+private:
+    static constexpr int32_t kEmpty = INT32_MIN;     // no record carries this name
+    size_t slot(int32_t key) const {
+        size_t i = ((uint32_t)key * 2654435761u) & (keys_.size() - 1);
+        while (keys_[i] != kEmpty && keys_[i] != key)
+            i = (i + 1) & (keys_.size() - 1);
+        return i;
+    }
+    void grow() {
+        std::vector<int32_t> k(keys_.size() * 2, kEmpty), v(keys_.size() * 2, 0);
+        k.swap(keys_);
+        v.swap(vals_);
+        count_ = 0;
+        for (size_t i = 0; i < k.size(); ++i)
+            if (k[i] != kEmpty)
+                at(k[i]) = v[i];
+    }
+    std::vector<int32_t> keys_, vals_;
+    size_t count_ = 0;
+};
 
 struct Words {
     const char* p;
@@ -98,7 +148,8 @@ bool same_shape(const Instr& a, const int32_t* shape, int nd) {
 // The AST nodes of one DAG node while it is put together.
 struct NodeWriter {
     DagNode node;
-    std::map<std::pair<int32_t, int32_t>, int32_t> leaf_of;   // (name, broadcast) -> index
+    struct Leaf { int32_t name, broadcast, index; };
+    std::vector<Leaf> leaves;          // a node has a handful of leaves: a list beats a tree
     int32_t next_scalar = -1;
 
     int32_t add(int32_t name, int32_t opcode, bool is_temp, bool is_scalar, bool is_bc, int32_t ndims,
@@ -118,12 +169,11 @@ struct NodeWriter {
         return (int32_t)node.nodes.size() - 1;
     }
     int32_t leaf(int32_t name, bool broadcast, int32_t base_ndims, int32_t dtype) {
-        auto key = std::make_pair(name, (int32_t)broadcast);
-        auto it = leaf_of.find(key);
-        if (it != leaf_of.end())
-            return it->second;
+        for (const Leaf& l : leaves)
+            if (l.name == name && l.broadcast == (int32_t)broadcast)
+                return l.index;
         const int32_t idx = add(name, CNH_OP_NOOP, false, false, broadcast, base_ndims, dtype, 0.0);
-        leaf_of.emplace(key, idx);
+        leaves.push_back({name, (int32_t)broadcast, idx});
         return idx;
     }
     int32_t leaf(const Ref& r) { return leaf(r.name, r.broadcast != 0, r.base_ndims, r.dtype); }
@@ -153,7 +203,6 @@ struct Group {
     int32_t shape[3] = {0, 0, 0};
     int nd = 0;
     int32_t dtype = 0;
-    std::unordered_set<int32_t> names;
 };
 
 enum ItemKind { kItemGroup, kItemInstr, kItemDelete };
@@ -234,13 +283,13 @@ int parse(const char* log, int64_t size, std::vector<Instr>& out) {
 
 size_t hold_back_cut(const std::vector<Instr>& batch, int window) {
     const size_t n = batch.size();
-    std::unordered_set<int32_t> deleted;
+    NameTable deleted(n);
     for (const Instr& in : batch)
         if (in.kind == kDelete)
             deleted.insert(in.name);
     size_t first_live = n;
     for (size_t i = n > (size_t)std::max(0, window) ? n - (size_t)window : 0; i < n; ++i)
-        if (batch[i].kind == kOp && !deleted.count(batch[i].name)) {
+        if (batch[i].kind == kOp && !deleted.has(batch[i].name)) {
             first_live = i;
             break;
         }
@@ -261,7 +310,7 @@ size_t hold_back_cut(const std::vector<Instr>& batch, int window) {
 }
 
 std::set<int32_t> dead_later(const std::vector<Instr>& batch, size_t cut) {
-    std::unordered_set<int32_t> touched, produced;
+    NameTable touched(batch.size()), produced(batch.size());
     for (size_t i = cut; i < batch.size(); ++i) {
         const Instr& in = batch[i];
         if (in.kind == kDelete)
@@ -277,7 +326,7 @@ std::set<int32_t> dead_later(const std::vector<Instr>& batch, size_t cut) {
             produced.insert(batch[i].name);
     std::set<int32_t> out;
     for (size_t i = cut; i < batch.size(); ++i)
-        if (batch[i].kind == kDelete && produced.count(batch[i].name) && !touched.count(batch[i].name))
+        if (batch[i].kind == kDelete && produced.has(batch[i].name) && !touched.has(batch[i].name))
             out.insert(batch[i].name);
     return out;
 }
@@ -285,34 +334,63 @@ std::set<int32_t> dead_later(const std::vector<Instr>& batch, size_t cut) {
 void plan(const std::vector<Instr>& batch, size_t count, const std::set<int32_t>& dead,
           int32_t* next_set_name, std::vector<DagNode>& out, std::set<int32_t>* fused_away) {
     const int n = (int)count;
-    std::unordered_map<int32_t, int> producer;       // result name -> index of the operation
-    std::unordered_set<int32_t> deleted(dead.begin(), dead.end());
+    NameTable producer((size_t)n);                    // result name -> index of the operation
+    NameTable deleted((size_t)n + dead.size());
+    for (int32_t name : dead)
+        deleted.insert(name);
     for (int i = 0; i < n; ++i) {
         if (batch[(size_t)i].kind == kOp)
-            producer[batch[(size_t)i].name] = i;
+            producer.at(batch[(size_t)i].name) = i;
         else if (batch[(size_t)i].kind == kDelete)
             deleted.insert(batch[(size_t)i].name);
     }
     std::vector<char> dropped((size_t)n, 0);          // dead code: operations never emitted
-    std::unordered_set<int32_t> forced;               // results that must exist as arrays
+    NameTable forced((size_t)n);                      // results that must exist as arrays
+
+    // Who reads the result of operation p (as instruction indices; -(i+1) marks instruction i
+    // assigning into it, which always counts as a use from outside any group): built once, as
+    // one list with an offset per operation; readers dropped later are skipped when it is read.
+    std::vector<int> use_first((size_t)n + 1, 0), use_list;
+    {
+        auto reader_of = [&](int32_t name) -> int {
+            const int32_t* p = producer.find(name);
+            return p != nullptr ? *p : -1;
+        };
+        for (int pass = 0; pass < 2; ++pass) {
+            std::vector<int> fill;
+            if (pass == 1) {
+                for (int i = 0; i < n; ++i)
+                    use_first[(size_t)i + 1] += use_first[(size_t)i];
+                use_list.assign((size_t)use_first[(size_t)n], 0);
+                fill.assign(use_first.begin(), use_first.end() - 1);
+            }
+            for (int i = 0; i < n; ++i) {
+                const Instr& in = batch[(size_t)i];
+                if (in.kind == kDelete || in.kind == kCreate)
+                    continue;
+                for (int j = 0; j < in.n_operands; ++j)
+                    if (in.operands[j].is_array) {
+                        const int p = reader_of(in.operands[j].name);
+                        if (p >= 0) {
+                            if (pass == 0) use_first[(size_t)p + 1]++;
+                            else use_list[(size_t)fill[(size_t)p]++] = i;
+                        }
+                    }
+                if (in.kind == kSet) {
+                    const int p = reader_of(in.name);
+                    if (p >= 0) {
+                        if (pass == 0) use_first[(size_t)p + 1]++;
+                        else use_list[(size_t)fill[(size_t)p]++] = -(i + 1);
+                    }
+                }
+            }
+        }
+    }
 
     std::vector<Item> items;
     std::vector<Group> groups;
     std::vector<int> group_of;
     for (;;) {
-        // name -> the instructions that read it; -(i+1) marks instruction i assigning into it,
-        // which always counts as a use from outside any group
-        std::unordered_map<int32_t, std::vector<int>> uses;
-        for (int i = 0; i < n; ++i) {
-            const Instr& in = batch[(size_t)i];
-            if (dropped[(size_t)i] || in.kind == kDelete || in.kind == kCreate)
-                continue;
-            for (int j = 0; j < in.n_operands; ++j)
-                if (in.operands[j].is_array)
-                    uses[in.operands[j].name].push_back(i);
-            if (in.kind == kSet)
-                uses[in.name].push_back(-(i + 1));
-        }
         items.clear();
         groups.clear();
         group_of.assign((size_t)n, -1);
@@ -335,8 +413,12 @@ void plan(const std::vector<Instr>& batch, size_t count, const std::set<int32_t>
                 if (cur >= 0)
                     for (int j = 0; j < in.n_operands; ++j) {
                         const Ref& o = in.operands[j];
-                        reads_slice_of_own = reads_slice_of_own ||
-                                             (o.is_array && o.has_region && groups[(size_t)cur].names.count(o.name));
+                        if (o.is_array && o.has_region) {
+                            // a slice of a result of the group that is open right now
+                            const int32_t* p = producer.find(o.name);
+                            reads_slice_of_own = reads_slice_of_own ||
+                                                 (p != nullptr && !dropped[(size_t)*p] && group_of[(size_t)*p] == cur);
+                        }
                     }
                 if (cur < 0 || !same_shape(in, groups[(size_t)cur].shape, groups[(size_t)cur].nd) ||
                     groups[(size_t)cur].dtype != in.dtype || reads_slice_of_own) {
@@ -349,13 +431,12 @@ void plan(const std::vector<Instr>& batch, size_t count, const std::set<int32_t>
                     g.dtype = in.dtype;
                 }
                 groups[(size_t)cur].ops.push_back(i);
-                groups[(size_t)cur].names.insert(in.name);
                 group_of[(size_t)i] = cur;
-                if (forced.count(in.name))
+                if (forced.has(in.name))
                     close();
             } else if (in.kind == kDelete) {
-                auto p = producer.find(in.name);
-                if (p != producer.end() && dropped[(size_t)p->second])
+                const int32_t* p = producer.find(in.name);
+                if (p != nullptr && dropped[(size_t)*p])
                     continue;
                 deferred.push_back(in.name);
                 if (cur < 0)
@@ -364,7 +445,7 @@ void plan(const std::vector<Instr>& batch, size_t count, const std::set<int32_t>
                 const Ref& v = in.operands[0];
                 const bool fuse = cur >= 0 && v.is_array && !v.has_region &&
                                   batch[(size_t)groups[(size_t)cur].ops.back()].name == v.name &&
-                                  !forced.count(v.name) && !v.broadcast &&
+                                  !forced.has(v.name) && !v.broadcast &&
                                   groups[(size_t)cur].nd == in.target_ndims && groups[(size_t)cur].dtype == in.dtype;
                 if (fuse) {
                     groups[(size_t)cur].set_idx = i;
@@ -388,20 +469,28 @@ void plan(const std::vector<Instr>& batch, size_t count, const std::set<int32_t>
                 continue;
             const int gi = group_of[(size_t)i];
             const Group& g = groups[(size_t)gi];
-            auto u = uses.find(in.name);
-            const bool is_dead = deleted.count(in.name) != 0;
-            if (is_dead && (u == uses.end() || u->second.empty())) {
+            // the readers of this result that are still part of the program (a result computed
+            // twice under one name does not occur: names are handed out once)
+            const int32_t* own = producer.find(in.name);
+            const int first = own != nullptr && *own == i ? use_first[(size_t)i] : 0;
+            const int past = own != nullptr && *own == i ? use_first[(size_t)i + 1] : 0;
+            bool any_reader = false, inside = true;
+            for (int q = first; q < past; ++q) {
+                const int x = use_list[(size_t)q];
+                if (x >= 0 && dropped[(size_t)x])
+                    continue;
+                any_reader = true;
+                inside = inside && x >= 0 && group_of[(size_t)x] == gi;
+            }
+            const bool is_dead = deleted.has(in.name);
+            if (is_dead && !any_reader) {
                 dropped[(size_t)i] = 1;       // computed, never read, handle gone
                 changed = true;
                 continue;
             }
-            bool inside = true;
-            if (u != uses.end())
-                for (int x : u->second)
-                    inside = inside && x >= 0 && group_of[(size_t)x] == gi;
             const bool is_last = g.ops.back() == i;
             const bool temp_ok = is_dead && inside && (!is_last || g.set_idx >= 0);
-            if (!temp_ok && !forced.count(in.name)) {
+            if (!temp_ok && !forced.has(in.name)) {
                 // must exist as an array: its group has to end here
                 if (!(is_last && g.set_idx < 0)) {
                     forced.insert(in.name);
@@ -414,11 +503,11 @@ void plan(const std::vector<Instr>& batch, size_t count, const std::set<int32_t>
     }
 
     // ---- emission ----
-    std::unordered_set<int32_t> materialised;
+    NameTable materialised((size_t)n);
     int node_id = 0;
     for (const Item& item : items) {
         if (item.kind == kItemDelete) {
-            if (producer.count(item.what) && !materialised.count(item.what))
+            if (producer.has(item.what) && !materialised.has(item.what))
                 continue;               // a temporary: it never became an array
             NodeWriter w;
             w.node.id = node_id++;
@@ -432,7 +521,7 @@ void plan(const std::vector<Instr>& batch, size_t count, const std::set<int32_t>
         w.node.id = node_id++;
         if (item.kind == kItemGroup) {
             const Group& g = groups[(size_t)item.what];
-            std::unordered_map<int32_t, int32_t> index_of;    // result name -> AST node of this group
+            NameTable index_of(g.ops.size());                 // result name -> AST node of this group
             const int last = g.ops.back();
             for (int i : g.ops) {
                 const Instr& in = batch[(size_t)i];
@@ -441,9 +530,9 @@ void plan(const std::vector<Instr>& batch, size_t count, const std::set<int32_t>
                 for (int j = 0; j < in.n_operands; ++j) {
                     const Ref& o = in.operands[j];
                     if (o.is_array) {
-                        auto it = index_of.find(o.name);
-                        if (it != index_of.end() && !o.has_region) {
-                            opnds[j] = it->second;
+                        const int32_t* it = index_of.find(o.name);
+                        if (it != nullptr && !o.has_region) {
+                            opnds[j] = *it;
                         } else {
                             opnds[j] = w.leaf(o);
                             oregs[j] = o.has_region ? &o.region : nullptr;
@@ -453,13 +542,13 @@ void plan(const std::vector<Instr>& batch, size_t count, const std::set<int32_t>
                     }
                 }
                 const bool is_root_result = i == last && g.set_idx < 0;
-                index_of[in.name] = w.op(in.name, in.opcode, !is_root_result, g.nd, in.dtype, in.n_operands, opnds,
-                                         oregs, is_root_result ? full_region(in.shape, in.ndims) : global_region());
+                index_of.at(in.name) = w.op(in.name, in.opcode, !is_root_result, g.nd, in.dtype, in.n_operands, opnds,
+                                            oregs, is_root_result ? full_region(in.shape, in.ndims) : global_region());
             }
             if (g.set_idx >= 0) {
                 const Instr& s = batch[(size_t)g.set_idx];
                 const int32_t opnds[2] = {w.leaf(s.name, false, s.target_ndims, s.dtype),
-                                          index_of[batch[(size_t)last].name]};
+                                          index_of.at(batch[(size_t)last].name)};
                 const cnh_region* oregs[2] = {nullptr, nullptr};
                 w.op((*next_set_name)++, CNH_OP_SET_REGION, false, s.target_ndims, s.dtype, 2, opnds, oregs, s.region);
             } else {
@@ -507,7 +596,7 @@ void plan(const std::vector<Instr>& batch, size_t count, const std::set<int32_t>
     }
     if (fused_away != nullptr)
         for (int32_t name : dead)
-            if (producer.count(name) && !materialised.count(name))
+            if (producer.has(name) && !materialised.has(name))
                 fused_away->insert(name);
 }
 
