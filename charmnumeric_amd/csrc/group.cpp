@@ -42,6 +42,11 @@ struct cnh_kernel {
     std::string ident;             // the AST it was compiled from, field by field (see ast_ident)
     std::mutex mu;                 // guards variants: a kernel found by key is shared between executors
     std::map<std::string, KernelVariant> variants;
+    // whether and how the group fits the register-window kernels, worked out once per geometry
+    // (every launch asks; the answer depends on the program and the three numbers only)
+    bool shape_known = false;
+    int shape_cfg[3] = {0, 0, 0}, shape_rc = 0;
+    DirectShape shape;
 };
 
 namespace {
@@ -1062,10 +1067,23 @@ int try_launch_direct(cnh_kernel* k, const std::vector<const cnh_tiled*>& arrays
                       RedReq* red) {
     *handled = false;
     const GroupProgram& p = k->prog;
-    DirectShape sh;
-    std::string why;
-    if (g_stencil_mode != 2 || direct_shape(p, g_direct_cfg, sh, why) != 0)
+    if (g_stencil_mode != 2)
         return 0;
+    {
+        std::lock_guard<std::mutex> lock(k->mu);
+        if (!k->shape_known || k->shape_cfg[0] != g_direct_cfg.tx || k->shape_cfg[1] != g_direct_cfg.ry ||
+            k->shape_cfg[2] != g_direct_cfg.rz) {
+            std::string why;
+            k->shape_rc = direct_shape(p, g_direct_cfg, k->shape, why);
+            k->shape_cfg[0] = g_direct_cfg.tx;
+            k->shape_cfg[1] = g_direct_cfg.ry;
+            k->shape_cfg[2] = g_direct_cfg.rz;
+            k->shape_known = true;
+        }
+    }
+    if (k->shape_rc != 0)
+        return 0;
+    const DirectShape& sh = k->shape;
     if (!cur || arrays.empty() || cur->tile < 2 || (cur->tile % 2) != 0)
         return 0;
     // Which operand array is the assigned one (read through the window), which are the others:
