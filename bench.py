@@ -828,7 +828,10 @@ def lstm_fused_ast(L, first, with_x=False):
 
 
 def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=False, fused=True, warm_passes=5,
-             merge_x=True):
+             merge_x=True, epilogue=True):
+    """epilogue: the gate launch of a step rides on the step's product (cnh_launch_product_group) where
+    the shape is one the product kernel takes that way; the events "around the product" then cover
+    the whole step's launch."""
     k_in = nin + d
     merge_x = merge_x and fused and nin == d     # the copy of x_{t+1} rides on step t's gate launch
     X = Buf(L, steps * batch * nin * 8)
@@ -897,14 +900,57 @@ def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=
         args = (2, 8, dst, i64(dst_strides), zero2, one, src, i64(src_strides), zero2, one, i64(extent), stream)
         return lambda: L.check(L.lib.cnh_copy_region(*args))
 
-    def prepared_product(t):
+    def product_job(t):
         # IFOG[t] = Hin[t] @ W, written without reading what IFOG[t] held
         jobs = (L.GemmJob * 1)()
         jobs[0].M, jobs[0].N, jobs[0].K = batch, 4 * d, k_in
         jobs[0].A, jobs[0].lda = Hin.ptr + t * batch * k_in * 8, k_in
         jobs[0].B, jobs[0].ldb = W.ptr, 4 * d
         jobs[0].C, jobs[0].ldc = IFOG.ptr + t * batch * 4 * d * 8, 4 * d
+        return jobs
+
+    def prepared_product(t):
+        jobs = product_job(t)
         return lambda: L.check(L.lib.cnh_gemm_batch(L.F64, 1, jobs, 1, stream))
+
+    one_launch = []      # per step: did the product take the gate statements along?
+
+    def prepared_product_group(t, k, ins, outs):
+        """The product of step t and the gate group in one launch, the group's leaves 1..4 being the
+        product's four column blocks; falls back to two launches where the kernel does not take the shape."""
+        jobs = product_job(t)
+        n_in, n_sc, n_out = C.c_int(), C.c_int(), C.c_int()
+        L.check(L.lib.cnh_kernel_signature(k, C.byref(n_in), C.byref(n_sc), C.byref(n_out)))
+        name, has, tgt, sr = C.c_int(), C.c_int(), C.c_int(), C.c_int()
+        reg = L.Region()
+        ia = (L.Memref * max(1, n_in.value))()
+        oa = (L.Memref * max(1, n_out.value))()
+        blocks = (C.c_int32 * max(1, n_in.value))()
+        for i in range(n_in.value):
+            L.check(L.lib.cnh_kernel_input(k, i, C.byref(name), C.byref(has), C.byref(reg)))
+            ia[i] = ins[name.value]
+            blocks[i] = name.value - 1 if 1 <= name.value <= 4 else -1
+        for i in range(n_out.value):
+            L.check(L.lib.cnh_kernel_output(k, i, C.byref(name), C.byref(tgt), C.byref(sr), C.byref(reg)))
+            oa[i] = outs[name.value]
+        two = [lambda: L.check(L.lib.cnh_gemm_batch(L.F64, 1, jobs, 1, stream)),
+               lambda: L.check(L.lib.cnh_launch_group(k, 2, n_in.value, ia, 0, None, 1, n_out.value, oa, stream))]
+        state = {"fused": None}
+
+        def fire():
+            if state["fused"] is not False:
+                rc = L.lib.cnh_launch_product_group(k, jobs, 4, 2, n_in.value, ia, blocks, 0, None, 1, n_out.value,
+                                                    oa, stream)
+                if rc == -17 and state["fused"] is None:
+                    state["fused"] = False
+                else:
+                    L.check(rc)
+                    state["fused"] = True
+                    return
+            for f in two:
+                f()
+        one_launch.append(state)
+        return fire
 
     def prepare(t):
         """(what runs before the product, the product, what runs after it) of step t."""
@@ -935,6 +981,8 @@ def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=
                 outs[19] = view(Hin, t + 1, k_in, 0, nin)
             elif merge_x:
                 kern = k_last
+            if epilogue:
+                return before, prepared_product_group(t, kern, ins, outs), []
             after.append(prepared_group(kern, 2, ins, outs))
         else:
             after.append(prepared1(k_sig, 2, [view(IFOG, t, 4 * d, 0, 3 * d)], [view(IFOGf, t, 4 * d, 0, 3 * d)]))
@@ -1024,6 +1072,9 @@ def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=
         out["Hout"] = Hout.get().reshape(steps, batch, d)
         out["C"] = Cc.get().reshape(steps, batch, d)
         out["IFOG"] = IFOG.get().reshape(steps, batch, 4 * d)
+        out["IFOGf"] = IFOGf.get().reshape(steps, batch, 4 * d)
+        out["Ct"] = Ct.get().reshape(steps, batch, d)
+        out["Hin"] = Hin.get().reshape(steps, batch, k_in)
     ev.free()
     for e in (e0, e1):
         L.lib.cnh_event_destroy(e)
@@ -1032,6 +1083,10 @@ def run_lstm(L, steps=64, batch=256, nin=1024, d=1024, seed=5, timed=True, keep=
     # the product, the gate launch (which also lays x_{t+1} into the next step's operand when the
     # input is as wide as the state) and otherwise the copy of x_t
     out["launches_per_step"] = (2 if merge_x else 3) if fused else 9
+    if one_launch and all(st["fused"] for st in one_launch):
+        # the gate statements ran in the product's epilogue: "gemm_us" above is that whole launch
+        out["launches_per_step"] -= 1
+        out["gate_launches_per_step"] = 0
     for b_ in (X, W, Hin, IFOG, IFOGf, Cc, Ct, Hout, spare):
         b_.free()
     return out

@@ -267,6 +267,9 @@ _PROTOS = {
     "cnh_gemv_panels": (C.c_int, [C.c_int, C.c_int64, C.c_int32, C.c_int64, C.c_int64, C.c_int64,
                                   C.POINTER(GemvPanel), C.c_void_p, C.c_void_p, C.c_void_p]),
     "cnh_gemm_batch": (C.c_int, [C.c_int, C.c_int, C.POINTER(GemmJob), C.c_int, C.c_void_p]),
+    "cnh_launch_product_group": (C.c_int, [C.c_void_p, C.POINTER(GemmJob), C.c_int, C.c_int, C.c_int,
+                                           C.POINTER(Memref), C.POINTER(C.c_int32), C.c_int, _vpp, C.c_int,
+                                           C.c_int, C.POINTER(Memref), C.c_void_p]),
     "cnh_probe_mfma_f64": (C.c_int, [C.c_int, C.POINTER(C.c_double)]),
     "cnh_fill_uniform": (C.c_int, [C.c_void_p, C.c_int64, C.c_uint64, C.c_uint64, C.c_uint64,
                                    C.c_double, C.c_double, C.c_void_p]),

@@ -722,6 +722,100 @@ extern "C" __global__ __launch_bounds__(64) void grp_nd1_p1(Cell cell, Scal sc) 
     return s.str();
 }
 
+// The product kernel with the group's statements in its epilogue: the text of gemm_kernel.inc in its
+// shape for grids of one workgroup per CU (2 sets of 4 x 2 wavefronts, 64 x 64 tiles, buffer loads),
+// with a workgroup's 64 columns taken as 64 / q from each of q column blocks of the product. When the
+// sums are complete they go to global memory and to an LDS tile; then every lane of the workgroup
+// takes elements (row, block column) of the tile's rows: loads that name a column block of the
+// product come from the tile, the others from their memrefs, and the statements are those of the
+// strided-cell kernel.
+std::string product_source(const GroupProgram& p, int q) {
+    std::ostringstream s;
+    s << prelude(p);
+    s << "typedef long long cn_i64;\ntypedef int cn_i32;\n";
+    s << "#define CN_EPILOGUE 1\n#define CN_EPI_Q " << q << "\n";
+    s << R"(
+struct Cell {
+    i64 sizes[3]; i64 blk0; i64 nchunks;
+    const T* in[NLA]; i64 istr[NLA][3];
+    T* out[NOA]; i64 ostr[NOA][3];
+};
+// src[k]: which column block of the product load k is (-1: an array of its own, read through
+// cell.in[k]); nblock: width of a column block
+struct EpiArgs { Cell cell; Scal sc; int src[NLA]; int nblock; int unused; };
+constexpr int WM = 4, WN = 2, TM = 1, TN = 2, BKT = 16, KS = 2;
+constexpr bool FULL = true, BUF = true;
+
+// Elements (row, block column) of the workgroup's tile a lane takes: e = lane, lane + LANES, ...
+// The loads that do not come from the product are issued before the first K step when a lane has a
+// single element (four column blocks): their latency then hides behind the whole product.
+template <int BM, int CPB, int LANES>
+struct CnEpi {
+    static constexpr int EPL = BM * CPB / LANES;
+    static_assert(EPL * LANES == BM * CPB, "the lanes divide the tile's elements evenly");
+    static constexpr bool EARLY = EPL == 1;
+    T pre[EARLY ? NLA : 1];
+    __device__ __forceinline__ T load(const EpiArgs& epi, int k, int e, int m0, int n0) const {
+        const Cell& c = epi.cell;
+        const i64 i1 = m0 + e / CPB, x = n0 + e % CPB;
+        return c.in[k][i1 * c.istr[k][1] + x * c.istr[k][2]];
+    }
+    __device__ __forceinline__ void prefetch(const EpiArgs& epi, int m0, int n0) {
+        if (EARLY) {
+#pragma unroll
+            for (int k = 0; k < NL; ++k)
+                if (epi.src[k] < 0)
+                    pre[k] = load(epi, k, (int)threadIdx.x, m0, n0);
+        }
+    }
+    // ct[g]: the tile of sums of wavefront set g. The product's value is set 0's sum plus set 1's.
+    __device__ __forceinline__ void run(const EpiArgs& epi, double (*ct)[BM][WN * TN * 16 + 1], double* C, i64 ldc,
+                                        int m0, int n0) const {
+        T s[NSV]; load_scalars(epi.sc, s);
+        const Cell& c = epi.cell;
+#pragma unroll
+        for (int u = 0; u < EPL; ++u) {
+            const int e = (int)threadIdx.x + u * LANES;
+            const int row = e / CPB, hc = e % CPB;
+            const i64 i1 = m0 + row, x = n0 + hc;
+            T v[CN_EPI_Q], l[NLA], o[NOA];
+#pragma unroll
+            for (int b = 0; b < CN_EPI_Q; ++b) {
+                v[b] = ct[0][row][b * CPB + hc];
+                if (KS > 1)
+                    v[b] += ct[1][row][b * CPB + hc];
+            }
+#pragma unroll
+            for (int k = 0; k < NL; ++k) {
+                const int b = epi.src[k];
+                if (b < 0) {
+                    l[k] = EARLY ? pre[k] : load(epi, k, e, m0, n0);
+                } else {
+                    l[k] = v[0];
+#pragma unroll
+                    for (int w = 1; w < CN_EPI_Q; ++w)
+                        l[k] = b == w ? v[w] : l[k];
+                }
+            }
+            group_eval(l, s, o);
+            // every store behind the arithmetic: a wait for a table lookup of exp in the middle of it
+            // would otherwise also wait for the stores issued before it
+#pragma unroll
+            for (int b = 0; b < CN_EPI_Q; ++b)
+                C[i1 * ldc + (i64)b * epi.nblock + x] = v[b];
+#pragma unroll
+            for (int j = 0; j < NO; ++j)
+                c.out[j][i1 * c.ostr[j][1] + x * c.ostr[j][2]] = o[j];
+        }
+    }
+};
+#define CN_GEMM_HEAD(...) extern "C" __global__ __launch_bounds__(WM * WN * 64 * KS) void grp_product(__VA_ARGS__)
+#define CN_GEMM_MORE_ARGS , EpiArgs epi
+)";
+    s << gemm_kernel_text();
+    return s.str();
+}
+
 std::string tiles_source(const GroupProgram& p) {
     std::ostringstream s;
     s << prelude(p);
@@ -1112,6 +1206,19 @@ int emit_variant_source(const GroupProgram& p, const std::string& variant, std::
     }
     if (variant == "nd") {
         src = nd_source(p);
+        return 0;
+    }
+    if (variant.compare(0, 7, "product") == 0) {
+        const int q = variant.size() == 8 ? variant[7] - '0' : 0;
+        if (q != 1 && q != 2 && q != 4) {
+            err = "the product variant is product1, product2 or product4 (column blocks per product)";
+            return -2;
+        }
+        if (p.dtype != CNH_F64) {
+            err = "statements in a product's epilogue are fp64 only";
+            return -17;
+        }
+        src = product_source(p, q);
         return 0;
     }
     if (variant == "tiles") {

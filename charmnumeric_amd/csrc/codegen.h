@@ -139,6 +139,10 @@ int emit_variant_source(const GroupProgram& p, const std::string& variant, std::
 
 const char* dtype_ctype(int dtype);
 
+// Text of the fp64 matrix-core product kernel (gemm_kernel.inc), for the variant that appends a
+// group's statements to it (codegen_product.cpp).
+std::string gemm_kernel_text();
+
 // fp64 exp/tanh restated to agree bit for bit with the host C library (codegen_libm.cpp).
 std::string libm_f64_text();
 std::string libm_f32_text();

@@ -64,7 +64,15 @@ int reduce_slots_f64_many(int nvec, const int* maximum, double* const* vecs, int
 void gemv_set_xlds(int on);
 void gemm_set_buffer_loads(int on);
 void gemm_set_ksplit(int on);
+// Would a single overwriting fp64 product of this shape take the kernel of two sets of eight
+// wavefronts per workgroup (64 x 64 tiles, one workgroup per CU, K steps shared between the sets)?
+// The product kernel with a group's statements in its epilogue exists in that form only, and adds
+// its sums in that form's order.
+bool gemm_split_form(int64_t M, int64_t N, int64_t K, const void* A, int64_t lda, const void* B, int64_t ldb);
 int reduce_slots_f64(bool maximum, double* slots, int64_t n, double* out, hipStream_t st);
+
+// Option "product_statements": may a product's launch evaluate the statements that follow it?
+bool product_statements_on();
 
 // Descriptor tables (per-partition pointers/shapes) live on the device. Identical tables are
 // uploaded once and found again by content hash, so steady-state launches issue no copy.

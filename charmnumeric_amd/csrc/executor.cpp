@@ -1503,14 +1503,30 @@ int exec_matmul(Ex* ex, const DagNode& n, const cnh_ast_node& root) {
 // (src/executor_matmatmul.cpp:105-484, src/executor_incremental.cpp:97-132).
 // `dest`: where the product goes instead of a new array (the box a following assignment names),
 // null for the ordinary form.
+// `plan_only`: nothing is launched, created or copied; when the product would go into the box as a
+// list of panel products of operands that need no copy, the list is left there (else it stays empty),
+// with the operands' arrays and windows in `operands`.
+struct ProductOperands {
+    XArray *A = nullptr, *B = nullptr;
+    cnh_region wA, wB;
+    int M = 0, N = 0, K = 0;
+};
 int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root, const DagNode* dest_node = nullptr,
-                   bool* dest_taken = nullptr) {
+                   bool* dest_taken = nullptr, std::vector<cnh_gemm_job>* plan_only = nullptr,
+                   ProductOperands* operands = nullptr) {
     XArray *Aa, *Ba;
     cnh_region wA, wB;
     if (int rc = leaf_window(ex, n, root, 0, &Aa, &wA, "MATMATMUL"))
         return rc;
     if (int rc = leaf_window(ex, n, root, 1, &Ba, &wB, "MATMATMUL"))
         return rc;
+    if (plan_only != nullptr) {
+        plan_only->clear();
+        if (Aa->phased() || Ba->phased())
+            return 0;
+        if (operands != nullptr)
+            *operands = ProductOperands{Aa, Ba, wA, wB, 0, 0, 0};
+    }
     bool a_copy = false, b_copy = false;
     if (int rc = unphased(ex, Aa, &Aa, &a_copy))
         return rc;
@@ -1523,6 +1539,11 @@ int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root, const Dag
         return rc;
     CNH_CHECK(A.cols == B.rows, -32, "MATMATMUL: (%d,%d) @ (%d,%d)", A.rows, A.cols, B.rows, B.cols);
     CNH_CHECK(Aa->dtype == Ba->dtype, -27, "MATMATMUL: operand dtypes %d and %d", Aa->dtype, Ba->dtype);
+    if (plan_only != nullptr && operands != nullptr) {
+        operands->M = A.rows;
+        operands->N = B.cols;
+        operands->K = A.cols;
+    }
     int32_t shape[3] = {A.rows, B.cols, 1};
     // fp64 products overwrite their result (every C element belongs to exactly one chain), so the
     // new array needs no zero-fill; the other types accumulate into zeros as upstream does
@@ -1555,6 +1576,8 @@ int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root, const Dag
     }
     if (dest_taken != nullptr)
         *dest_taken = dest_base != nullptr;
+    if (plan_only != nullptr && dest_base == nullptr)
+        return 0;
     if (dest_base == nullptr)
         if (int rc = make_array(ex, root.result_name, 2, Aa->dtype, shape, !f64, &Cc))
             return rc;
@@ -1599,6 +1622,10 @@ int exec_matmatmul(Ex* ex, const DagNode& n, const cnh_ast_node& root, const Dag
                 r0 = r1;
             }
         }
+    if (plan_only != nullptr) {
+        plan_only->swap(jobs);
+        return 0;
+    }
     if (!ex->dry)
         if (int rc = cnh_gemm_batch(Aa->dtype, (int)jobs.size(), jobs.data(), f64 ? 1 : 0, ex->stream))
             return rc;
@@ -1985,7 +2012,33 @@ bool cut_statement(const Stmt& a, const int32_t* want, std::vector<Stmt>& pieces
 // The run as one multi-root group. Boxes are numbered; the group's regions carry the numbers, not
 // the coordinates (the launch hands over memrefs), so every step of a time loop finds the kernel
 // of the first one in the cache.
-int exec_statement_run(Ex* ex, const std::vector<Stmt>& run) {
+// `site`: a product the run rides on. Reads of the product's box, column block by column block, take
+// their values from the product's launch (cnh_launch_product_group); `fused` tells whether that launch
+// took the shape, else the product and the run went out as two launches.
+struct ProductSite {
+    cnh_gemm_job job;
+    XArray* target = nullptr;
+    cnh_region region;         // the product's box in the target's coordinates
+    int blocks = 1;            // column blocks the run reads it in
+    std::string what;          // trace text of the product
+    bool fused = false;
+};
+// Which column block of the site's box is `u` (-1: none)?
+int product_block(const ProductSite& site, const BoxUse& u) {
+    if (u.arr != site.target)
+        return -1;
+    const int last = site.target->ndims - 1;
+    for (int d = 0; d < last; ++d)
+        if (u.reg.start[d] != site.region.start[d] || u.reg.stop[d] != site.region.stop[d])
+            return -1;
+    const int width = (site.region.stop[last] - site.region.start[last]) / site.blocks;
+    const int off = u.reg.start[last] - site.region.start[last];
+    if (off < 0 || off % width != 0 || u.reg.stop[last] - u.reg.start[last] != width || off / width >= site.blocks)
+        return -1;
+    return off / width;
+}
+
+int exec_statement_run(Ex* ex, const std::vector<Stmt>& run, ProductSite* site = nullptr) {
     DagNode merged;
     merged.id = run.front().n->id;
     merged.fusible = 1;
@@ -2073,6 +2126,7 @@ int exec_statement_run(Ex* ex, const std::vector<Stmt>& run) {
     const int nd = run.front().nd;
     const int32_t* cnt = run.front().cnt;
     std::vector<cnh_memref> ins((size_t)std::max(1, n_in)), outs((size_t)std::max(1, n_out));
+    std::vector<int32_t> in_block((size_t)std::max(1, n_in), -1);
     for (int i = 0; i < n_in; ++i) {
         int cname = 0, has = 0;
         cnh_region reg;
@@ -2081,6 +2135,8 @@ int exec_statement_run(Ex* ex, const std::vector<Stmt>& run) {
         CNH_CHECK(has && reg.start[0] >= 0 && reg.start[0] < (int)boxes.size(), -26,
                   "statement run: input %d carries no box number", i);
         ins[(size_t)i] = box_memref(boxes[(size_t)reg.start[0]], nd, cnt);
+        if (site != nullptr)
+            in_block[(size_t)i] = product_block(*site, boxes[(size_t)reg.start[0]]);
     }
     for (int i = 0; i < n_out; ++i) {
         int rname = 0, tname = 0, is_set = 0;
@@ -2105,10 +2161,24 @@ int exec_statement_run(Ex* ex, const std::vector<Stmt>& run) {
     std::string names;
     for (const Stmt& st : run)
         names += (names.empty() ? "" : ",") + std::to_string(st.out.arr->name);
+    if (site != nullptr && !ex->dry) {
+        // the product's launch evaluates the run on its tile of sums; shapes it does not take (-17)
+        // go out as the two launches below
+        const int rc = cnh_launch_product_group(k, &site->job, site->blocks, nd, n_in, ins.data(), in_block.data(),
+                                                n_scalar, scalars.data(), 1, n_out, outs.data(), ex->stream);
+        if (rc != 0 && rc != -17)
+            return rc;
+        site->fused = rc == 0;
+        if (!site->fused)
+            if (int rc2 = cnh_gemm_batch(CNH_F64, 1, &site->job, 1, ex->stream))
+                return rc2;
+    }
+    if (site != nullptr && ex->trace_on)
+        ex->log(site->what + (site->fused ? " with_statements" : ""));
     if (ex->trace_on) ex->log("group node=" + std::to_string(merged.id) + " path=statements count=" +
             std::to_string(run.size()) + " inputs=" + std::to_string(n_in) + " outputs=" +
-            std::to_string(n_out) + " out=" + names);
-    if (ex->dry)
+            std::to_string(n_out) + " out=" + names + (site != nullptr && site->fused ? " in_product" : ""));
+    if (ex->dry || (site != nullptr && site->fused))
         return 0;
     return cnh_launch_group(k, nd, n_in, ins.data(), n_scalar, scalars.data(), 1, n_out, outs.data(),
                             ex->stream);
@@ -2116,13 +2186,19 @@ int exec_statement_run(Ex* ex, const std::vector<Stmt>& run) {
 
 // Nodes [i, ...) of the message: a run of two or more assignments this pass can merge, deletions
 // in between put off until the run has been launched. Returns the number of nodes consumed.
-int try_statement_run(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t* used, bool* open_ended) {
-    *used = 0;
-    *open_ended = false;
+struct StatementRun {
     std::vector<Stmt> run;
+    std::vector<int> deletions_kept;   // deletions between the statements taken
+    size_t last_stmt_end = 0;          // index behind the last statement taken
+    bool ran_off_end = false;          // the message ended while the run could still grow
+};
+void collect_statement_run(Ex* ex, const std::vector<DagNode>& dag, size_t i, StatementRun& out) {
+    std::vector<Stmt>& run = out.run;
     std::vector<int> deletions;
-    size_t j = i, last_stmt_end = i;
-    std::vector<int> deletions_kept;
+    size_t j = i;
+    size_t& last_stmt_end = out.last_stmt_end;
+    last_stmt_end = i;
+    std::vector<int>& deletions_kept = out.deletions_kept;
     for (; j < dag.size(); ++j) {
         const DagNode& n = dag[j];
         if (n.roots.empty())
@@ -2181,18 +2257,26 @@ int try_statement_run(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t*
         deletions_kept = deletions;
     }
     // ran off the end of the message with room left: more of the run may follow
-    if (j == dag.size() && !run.empty() && run.size() < kFuseMaxStmts && open_ended_allowed(ex)) {
+    out.ran_off_end = j == dag.size() && !run.empty() && run.size() < kFuseMaxStmts && open_ended_allowed(ex);
+}
+
+int try_statement_run(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t* used, bool* open_ended) {
+    *used = 0;
+    *open_ended = false;
+    StatementRun sr;
+    collect_statement_run(ex, dag, i, sr);
+    if (sr.ran_off_end) {
         *open_ended = true;
         return 0;
     }
-    if (run.empty())
+    if (sr.run.empty())
         return 0;
-    if (int rc = exec_statement_run(ex, run))
+    if (int rc = exec_statement_run(ex, sr.run))
         return rc;
-    for (int name : deletions_kept)
+    for (int name : sr.deletions_kept)
         drop_array(ex, name);
-    ex->stats[2] += (int64_t)(last_stmt_end - i);
-    *used = last_stmt_end - i;
+    ex->stats[2] += (int64_t)(sr.last_stmt_end - i);
+    *used = sr.last_stmt_end - i;
     return 0;
 }
 
@@ -3863,6 +3947,144 @@ int try_product_into_region(Ex* ex, const std::vector<DagNode>& dag, size_t i, s
     return 0;
 }
 
+// ---- a product and the statements on its result as one launch ----
+//
+// `target[box] = A @ B` followed by a run of statements that read the box column block by column
+// block (the gate statements of an LSTM step read the four gates' columns of IFOG[t],
+// examples/lstm_forward.py:40-49 upstream): the product's launch evaluates the run on each
+// workgroup's tile of sums (cnh_launch_product_group), so the step is one launch and nothing waits
+// for a second one to start. Taken when
+//   - the product is a single fp64 panel product into the box, of the shape that gives every CU at
+//     most one workgroup (the fused kernel exists in that form only);
+//   - the run's extents are (rows of the product) x (its columns / q), q = 1, 2 or 4, and every read
+//     of the target that meets the box is exactly one of its q column blocks;
+//   - no statement assigns into the box or into a window the product reads (workgroups finish at
+//     different times: a statement's stores must not reach what another workgroup still multiplies).
+// The statements of one element depend on that element's values only (what a statement run is), so
+// evaluating them tile by tile as the tiles complete gives what the two launches give.
+bool unit_regions_disjoint(const cnh_region& a, const cnh_region& b, int nd) {
+    for (int d = 0; d < nd; ++d)
+        if (a.stop[d] <= b.start[d] || b.stop[d] <= a.start[d])
+            return true;
+    return false;
+}
+
+int try_product_with_statements(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t* used, bool* open_ended) {
+    *used = 0;
+    *open_ended = false;
+    if (!product_statements_on() || i + 3 >= dag.size() || dag[i].roots.empty() || dag[i + 1].roots.size() != 1 ||
+        dag[i + 2].roots.empty())
+        return 0;
+    const cnh_ast_node& mm = dag[i].nodes[dag[i].roots.back()];
+    const cnh_ast_node& set = dag[i + 1].nodes[dag[i + 1].roots.back()];
+    const cnh_ast_node& del = dag[i + 2].nodes[dag[i + 2].roots.back()];
+    if (mm.opcode != CNH_OP_MATMATMUL || set.opcode != CNH_OP_SET_REGION || del.opcode != kOpDelete ||
+        set.n_operands != 2 || set.region.is_global || del.result_name != mm.result_name)
+        return 0;
+    const cnh_ast_node& value = dag[i + 1].nodes[set.operands[1]];
+    if (value.is_scalar || value.opcode != CNH_OP_NOOP || value.result_name != mm.result_name ||
+        (set.has_operand_region[1] && !set.operand_regions[1].is_global))
+        return 0;
+    for (int d = 0; d < set.region.ndims; ++d)
+        if (set.region.step[d] != 1)
+            return 0;
+    // why a product that has statements behind it keeps a launch of its own, for the trace
+    auto no = [&](const char* why) {
+        if (ex->trace_on) ex->log(std::string("product node=") + std::to_string(dag[i].id) + " statements_not_taken: " + why);
+        return 0;
+    };
+    // the product as it would be launched, without launching it
+    std::vector<cnh_gemm_job> jobs;
+    ProductOperands ops;
+    bool taken = false;
+    if (int rc = exec_matmatmul(ex, dag[i], mm, &dag[i + 1], &taken, &jobs, &ops))
+        return rc;
+    if (!taken || jobs.empty())
+        return no("the product does not go into the box as panel products");
+    if (!gemm_split_form(ops.M, ops.N, ops.K, nullptr, ops.K, nullptr, ops.N))
+        return no("not of the one-workgroup-per-CU shape");
+    ProductSite site;
+    auto tgt = ex->arrays.find(dag[i + 1].nodes[set.operands[0]].result_name);
+    if (tgt == ex->arrays.end() || set.region.ndims != tgt->second.ndims)
+        return no("target unknown");
+    site.target = &tgt->second;
+    site.region = set.region;
+    const int tnd = site.target->ndims, last = tnd - 1;
+    if (site.region.stop[last] - site.region.start[last] != ops.N)
+        return no("the box's columns are not the target's last dimension");
+    StatementRun sr;
+    collect_statement_run(ex, dag, i + 3, sr);
+    if (sr.run.empty())
+        return no("no statement run follows");
+    // the run's extents: (1, ..., M, N / q)
+    const Stmt& first = sr.run.front();
+    if (first.nd < 2 || first.dtype != CNH_F64 || first.cnt[first.nd - 2] != ops.M ||
+        first.cnt[first.nd - 1] <= 0 || ops.N % first.cnt[first.nd - 1] != 0)
+        return no("the run's extents are not the product's rows by a fraction of its columns");
+    for (int d = 0; d + 2 < first.nd; ++d)
+        if (first.cnt[d] != 1)
+            return no("the run's extents are not the product's rows by a fraction of its columns");
+    site.blocks = (int)(ops.N / first.cnt[first.nd - 1]);
+    if (site.blocks != 1 && site.blocks != 2 && site.blocks != 4)
+        return no("column blocks other than 1, 2 or 4");
+    bool reads_product = false;
+    for (const Stmt& st : sr.run) {
+        if (!st.scalars_read.empty())
+            return no("a statement reads a one-element array");
+        // nothing is assigned where the product writes or reads
+        if (st.out.arr == site.target && !unit_regions_disjoint(st.out.reg, site.region, tnd))
+            return no("a statement assigns into the product's box");
+        if (st.out.arr == ops.A && !unit_regions_disjoint(st.out.reg, ops.wA, ops.A->ndims))
+            return no("a statement assigns into the left operand's window");
+        if (st.out.arr == ops.B && !unit_regions_disjoint(st.out.reg, ops.wB, ops.B->ndims))
+            return no("a statement assigns into the right operand's window");
+        for (const auto& rd : st.reads) {
+            if (rd.use.arr != site.target || unit_regions_disjoint(rd.use.reg, site.region, tnd))
+                continue;
+            if (product_block(site, rd.use) < 0)
+                return no("a statement reads the box other than by column blocks");
+            reads_product = true;
+        }
+    }
+    if (!reads_product)
+        return no("the run does not read the product");
+    if (jobs.size() != 1) {
+        // operands cut into tiles (a weight matrix of rank 2 is, by default) give one panel product
+        // per tile: laid out as one block each, once, they give a single one from now on
+        for (XArray* a : {ops.A, ops.B})
+            if (!ex->dry && ex->flat3 && a->ndims == 2 && !a->flat && a->ntiles > 1 && !a->phased())
+                if (int rc = make_block(ex, *a))
+                    return rc;
+        if (int rc = exec_matmatmul(ex, dag[i], mm, &dag[i + 1], &taken, &jobs, &ops))
+            return rc;
+        if (!taken || jobs.size() != 1)
+            return no("not a single panel product into the box");
+    }
+    if (!gemm_split_form(jobs[0].M, jobs[0].N, jobs[0].K, jobs[0].A, jobs[0].lda, jobs[0].B, jobs[0].ldb))
+        return no("not of the one-workgroup-per-CU shape");
+    site.job = jobs[0];
+    // the run may go on in the next message: the product waits with it
+    if (sr.ran_off_end) {
+        *open_ended = true;
+        return 0;
+    }
+    site.what = "matmatmul A=" + std::to_string(ops.A->name) + " B=" + std::to_string(ops.B->name) + " out=" +
+                std::to_string(site.target->name) + " into_region panel_products=1";
+    if (ex->dry) {
+        // a planning pass launches nothing: the product and the run are noted as they would go out
+        if (ex->trace_on) ex->log(site.what);
+        if (int rc = exec_statement_run(ex, sr.run))
+            return rc;
+    } else if (int rc = exec_statement_run(ex, sr.run, &site)) {
+        return rc;
+    }
+    for (int name : sr.deletions_kept)
+        drop_array(ex, name);
+    ex->stats[2] += (int64_t)(sr.last_stmt_end - i);
+    *used = sr.last_stmt_end - i;
+    return 0;
+}
+
 // Named ranges around the work of every DAG node, for profilers that trace roctx markers
 // (rocprofv3 --marker-trace): kernels then group by what the program asked for instead of by
 // grid size. Off unless CHARMNUMERIC_ROCTX is set to something other than 0; the marker library is
@@ -3950,6 +4172,8 @@ int run_nodes(Ex* ex, std::vector<DagNode>& dag) {
                 rc = try_scatter_run(ex, dag, i, &used, &open_ended);
             if (rc == 0 && used == 0 && !open_ended)
                 rc = try_lattice_pair(ex, dag, i, &used, &open_ended);
+            if (rc == 0 && used == 0 && !open_ended)
+                rc = try_product_with_statements(ex, dag, i, &used, &open_ended);
             if (rc == 0 && used == 0 && !open_ended)
                 rc = try_product_into_region(ex, dag, i, &used, &open_ended);
             if (rc == 0 && used == 0 && !open_ended)

@@ -15,268 +15,13 @@ using namespace cnh;
 
 namespace {
 
-typedef double v4d __attribute__((ext_vector_type(4)));
-typedef double v2d __attribute__((ext_vector_type(2)));
-
-constexpr int PAD = 16;
-
-// Workgroup ids are dealt round-robin to the 8 XCDs; give every XCD a contiguous run of logical
-// tiles so that the workgroups sharing a B column panel also share one L2.
-__device__ __forceinline__ int xcd_remap(int b, int nblocks) {
-    if (nblocks % 8 != 0)
-        return b;
-    return (b % 8) * (nblocks / 8) + b / 8;
-}
-
-// One C block and the panel products that accumulate into it, in order; a launch covers a list
-// of such chains (a single product is a chain of one segment).
-struct GemmSeg {
-    const double* A;
-    int64_t lda;
-    const double* B;
-    int64_t ldb;
-    int32_t K, pad;
-};
-struct GemmChain {
-    double* C;
-    int64_t ldc;
-    int32_t M, N;
-    int32_t seg0, nseg; // segments [seg0, seg0 + nseg)
-    int32_t blk0, nbm;  // first workgroup of the chain, tiles along M
-};
-static_assert(sizeof(GemmSeg) == 40 && sizeof(GemmChain) == 40, "descriptor tables are uploaded as bytes");
-
-// WM x WN wavefronts per workgroup, each owning TM x TN tiles of 16x16; K advances BKT at a time.
-// The fp64 matrix pipe needs two or more wavefronts per SIMD to stay busy (one wavefront issues at
-// ~70% of the rate eight reach), hence the 8-wavefront shape for grids that give each CU a single
-// workgroup. Global loads run two K steps ahead of the arithmetic (two register sets, one LDS
-// buffer being filled while the other is read): one K step of matrix instructions is shorter than
-// a trip to memory. A workgroup keeps its accumulators across the segments of its chain, so the
-// panel products of one C block cost one pass over C however many K pieces they come in.
-// KS = 2: the workgroup is two such sets of wavefronts; set g takes the K steps g, g + 2, ... of every
-// segment into accumulators of its own (staging buffers of its own too), and at the end the second
-// set hands its sums over through LDS and the first adds them, first + second, and stores. Twice
-// the wavefronts per SIMD for grids that give a CU one workgroup; K must be a multiple of 2 * BKT.
-template <int WM, int WN, int TM, int TN, int BKT, bool FULL, bool BUF = false, int KS = 1>
-__global__ __launch_bounds__(WM * WN * 64 * KS) void gemm_f64_mfma(const GemmChain* __restrict__ chains,
-                                                                   int nchains,
-                                                                   const GemmSeg* __restrict__ segs,
-                                                                   int nblocks, GemmChain only_chain,
-                                                                   GemmSeg only_seg, int overwrite) {
-    constexpr int NT = WM * WN * 64;   // lanes of one set
-    constexpr int BM = WM * TM * 16, BN = WN * TN * 16;
-    constexpr int APT = BM * BKT / NT, BPT = BN * BKT / NT;   // doubles staged per lane
-    static_assert(APT >= 2 && BPT >= 2 && APT % 2 == 0 && BPT % 2 == 0, "staging uses 128-bit loads");
-    static_assert(BKT % APT == 0 && BN % BPT == 0, "a lane's run stays inside one row");
-    // A stays row-major in LDS with rows of BKT + 1 doubles: the operand read of 16 consecutive
-    // rows at one k then touches 16 different bank pairs. B is k-major with rows of BN + 16.
-    constexpr int AP = BKT + 1;
-    __shared__ double As_all[KS][2][BM][AP];
-    __shared__ __attribute__((aligned(16))) double Bs_all[KS][2][BKT][BN + PAD];
-    __shared__ double Cs[KS > 1 ? TM * TN * 4 : 1][KS > 1 ? NT : 1];
-    const int set = KS > 1 ? __builtin_amdgcn_readfirstlane((int)threadIdx.x / NT) : 0;   // the same for a whole wavefront
-    double (*As)[BM][AP] = As_all[set];
-    double (*Bs)[BKT][BN + PAD] = Bs_all[set];
-    const int logical = xcd_remap(blockIdx.x, nblocks);
-    // a lone product travels in the kernel arguments (chains == nullptr), lists in a table
-    int ci = 0;
-    if (chains != nullptr)
-        while (ci + 1 < nchains && chains[ci + 1].blk0 <= logical)
-            ++ci;
-    const GemmChain ch = chains != nullptr ? chains[ci] : only_chain;
-    const int M = ch.M, N = ch.N;
-    const int local = logical - ch.blk0;
-    const int bn = local / ch.nbm, bm = local - bn * ch.nbm;
-    const int m0 = bm * BM, n0 = bn * BN;
-    const int tid = KS > 1 ? (int)threadIdx.x % NT : (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WN, wn = wave % WN;
-
-    // staging assignment: A tile BM rows x BKT k (APT along k), B tile BKT k x BN (BPT along n)
-    const int a_row = tid / (BKT / APT), a_k = (tid % (BKT / APT)) * APT;
-    const int b_k = tid / (BN / BPT), b_n = (tid % (BN / BPT)) * BPT;
-    const int lr = lane & 15, lk = lane >> 4;
-
-    v4d acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-            acc[i][j] = (v4d){0.0, 0.0, 0.0, 0.0};
-
-    for (int si = 0; si < ch.nseg; ++si) {
-        const GemmSeg sg = chains != nullptr ? segs[ch.seg0 + si] : only_seg;
-        const double* __restrict__ A = sg.A;
-        const double* __restrict__ B = sg.B;
-        const int64_t lda = sg.lda, ldb = sg.ldb;
-        const int K = sg.K;
-        if (si > 0)
-            __syncthreads();   // the previous segment's last reads of LDS are done
-
-        // BUF: buffer loads. The descriptor (base of this workgroup's rows of A, of its columns of
-        // B, moved along K on the scalar unit) sits in scalar registers and a lane contributes one
-        // 32-bit offset that never changes: no 64-bit address arithmetic on the vector unit, which
-        // the fp64 matrix instructions compete with (3-6 % on the 256 x 2048 x 4096 product).
-        typedef int v4i __attribute__((ext_vector_type(4)));
-        const int a_off = BUF ? (int)((a_row * lda + a_k) * 8) : 0;
-        const int b_off = BUF ? (int)((b_k * ldb + b_n) * 8) : 0;
-        auto fetch = [&](int k0, double (&ra)[APT], double (&rb)[BPT]) {
-            if (BUF) {
-                const __amdgpu_buffer_rsrc_t da = __builtin_amdgcn_make_buffer_rsrc(
-                    (void*)(A + (int64_t)m0 * lda + k0), 0, 0x7fffffff, 0x00020000);
-                const __amdgpu_buffer_rsrc_t db = __builtin_amdgcn_make_buffer_rsrc(
-                    (void*)(B + (int64_t)k0 * ldb + n0), 0, 0x7fffffff, 0x00020000);
-#pragma unroll
-                for (int j = 0; j < APT; j += 2) {
-                    const v4i v = __builtin_amdgcn_raw_buffer_load_b128(da, a_off + j * 8, 0, 0);
-                    v2d d;
-                    __builtin_memcpy(&d, &v, 16);
-                    ra[j] = d[0];
-                    ra[j + 1] = d[1];
-                }
-#pragma unroll
-                for (int j = 0; j < BPT; j += 2) {
-                    const v4i v = __builtin_amdgcn_raw_buffer_load_b128(db, b_off + j * 8, 0, 0);
-                    v2d d;
-                    __builtin_memcpy(&d, &v, 16);
-                    rb[j] = d[0];
-                    rb[j + 1] = d[1];
-                }
-                return;
-            }
-            const int gr = m0 + a_row;
-            const int gk = k0 + a_k;
-            if (FULL) {
-#pragma unroll
-                for (int j = 0; j < APT; j += 2) {
-                    const v2d v = *reinterpret_cast<const v2d*>(A + (int64_t)gr * lda + gk + j);
-                    ra[j] = v[0];
-                    ra[j + 1] = v[1];
-                }
-            } else {
-#pragma unroll
-                for (int j = 0; j < APT; ++j)
-                    ra[j] = (gr < M && gk + j < K) ? A[(int64_t)gr * lda + gk + j] : 0.0;
-            }
-            const int bk = k0 + b_k;
-            const int gn = n0 + b_n;
-            if (FULL) {
-#pragma unroll
-                for (int j = 0; j < BPT; j += 2) {
-                    const v2d v = *reinterpret_cast<const v2d*>(B + (int64_t)bk * ldb + gn + j);
-                    rb[j] = v[0];
-                    rb[j + 1] = v[1];
-                }
-            } else {
-#pragma unroll
-                for (int j = 0; j < BPT; ++j)
-                    rb[j] = (bk < K && gn + j < N) ? B[(int64_t)bk * ldb + gn + j] : 0.0;
-            }
-        };
-        auto stage = [&](int buf, const double (&ra)[APT], const double (&rb)[BPT]) {
-#pragma unroll
-            for (int j = 0; j < APT; ++j)
-                As[buf][a_row][a_k + j] = ra[j];
-#pragma unroll
-            for (int j = 0; j < BPT; j += 2)
-                *reinterpret_cast<v2d*>(&Bs[buf][b_k][b_n + j]) = (v2d){rb[j], rb[j + 1]};
-        };
-        auto multiply = [&](int buf) {
-#pragma unroll
-            for (int ks = 0; ks < BKT / 4; ++ks) {
-                const int kk = ks * 4 + lk;
-                double a[TM], b[TN];
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-                    a[i] = As[buf][(wm * TM + i) * 16 + lr][kk];
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    b[j] = Bs[buf][kk][(wn * TN + j) * 16 + lr];
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[i], b[j], acc[i][j], 0, 0, 0);
-            }
-        };
-
-        // Step t multiplies LDS buffer t&1, which holds K slice t. Register set t&1 receives
-        // slice t+2 while that runs; the other set (slice t+1, requested a step earlier) goes to
-        // LDS after it.
-        const int nk = (K + BKT - 1) / BKT / KS;          // K steps of this set
-        auto kof = [&](int step) { return (step * KS + set) * BKT; };
-        double ra0[APT], rb0[BPT], ra1[APT], rb1[BPT];
-        fetch(kof(0), ra0, rb0);
-        if (nk > 1)
-            fetch(kof(1), ra1, rb1);
-        stage(0, ra0, rb0);
-        __syncthreads();
-        // At the top of every round LDS buffer 0 holds slice t and register set 1 slice t + 1.
-        // The steady-state rounds carry no conditions, so that the compiler's wait counts leave
-        // the younger pair of loads in flight while the older pair is stored.
-        int t = 0;
-        for (; t + 3 < nk; t += 2) {
-            fetch(kof(t + 2), ra0, rb0);
-            multiply(0);
-            stage(1, ra1, rb1);
-            __syncthreads();
-            fetch(kof(t + 3), ra1, rb1);
-            multiply(1);
-            stage(0, ra0, rb0);
-            __syncthreads();
-        }
-        if (t + 2 < nk)
-            fetch(kof(t + 2), ra0, rb0);
-        multiply(0);
-        if (t + 1 < nk) {
-            stage(1, ra1, rb1);
-            __syncthreads();
-            multiply(1);
-            if (t + 2 < nk) {
-                stage(0, ra0, rb0);
-                __syncthreads();
-                multiply(0);
-            }
-        }
-    }
-    if (KS > 1) {
-        // the second set's sums go through LDS, lane to lane; the first set adds them to its own
-        if (set == 1) {
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        Cs[(i * TN + j) * 4 + r][tid] = acc[i][j][r];
-        }
-        __syncthreads();
-        if (set == 1)
-            return;
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    acc[i][j][r] += Cs[(i * TN + j) * 4 + r][tid];
-    }
-    // D layout of the 16x16x4 f64 instruction (measured on gfx950): register r of a lane holds
-    // row 4*r + lane/16, column lane % 16.
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int col = n0 + (wn * TN + j) * 16 + lr;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int row = m0 + (wm * TM + i) * 16 + r * 4 + lk;
-                if (FULL || (row < M && col < N)) {
-                    double* c = ch.C + (int64_t)row * ch.ldc + col;
-                    *c = overwrite ? acc[i][j][r] : *c + acc[i][j][r];
-                }
-            }
-        }
-}
+typedef int64_t cn_i64;
+typedef int32_t cn_i32;
+#define CN_GEMM_HEAD(...)                                                                             \
+    template <int WM, int WN, int TM, int TN, int BKT, bool FULL, bool BUF = false, int KS = 1>       \
+    __global__ __launch_bounds__(WM * WN * 64 * KS) void gemm_f64_mfma(__VA_ARGS__)
+#define CN_GEMM_MORE_ARGS
+#include "gemm_kernel.inc"
 
 template <typename T>
 struct Acc {
@@ -480,6 +225,13 @@ __global__ __launch_bounds__(512) void mfma_f64_probe(double* out, int iters, do
 namespace cnh {
 void gemm_set_buffer_loads(int on) { g_gemm_buffer_loads = on; }
 void gemm_set_ksplit(int on) { g_gemm_ksplit = on; }
+bool gemm_split_form(int64_t M, int64_t N, int64_t K, const void* A, int64_t lda, const void* B, int64_t ldb) {
+    const bool full = M % 64 == 0 && N % 64 == 0 && K % 32 == 0 && lda % 2 == 0 && ldb % 2 == 0 &&
+                      ((uintptr_t)A & 15) == 0 && ((uintptr_t)B & 15) == 0;
+    const int64_t blocks = (M / 64) * (N / 64);
+    return full && M > 0 && N > 0 && K > 0 && g_gemm_buffer_loads && g_gemm_ksplit && blocks < 1024 &&
+           blocks <= compute_units() && 64 * lda * 8 < (1ll << 31) && 16 * ldb * 8 < (1ll << 31);
+}
 } // namespace cnh
 
 extern "C" int cnh_probe_mfma_f64(int iters, double* tflops) {

@@ -733,6 +733,124 @@ int cnh_launch_group(cnh_kernel* k, int ndims, int n_in, const cnh_memref* in, i
 } // extern "C"
 
 // ---------------------------------------------------------------------------------------------
+// A product with the statements of a group in its epilogue.
+// ---------------------------------------------------------------------------------------------
+namespace {
+struct GemmSegDev {
+    const double* A;
+    int64_t lda;
+    const double* B;
+    int64_t ldb;
+    int32_t K, pad;
+};
+struct GemmChainDev {
+    double* C;
+    int64_t ldc;
+    int32_t M, N, seg0, nseg, blk0, nbm;
+};
+static_assert(sizeof(GemmSegDev) == 40 && sizeof(GemmChainDev) == 40, "as gemm_kernel.inc lays them out");
+} // namespace
+
+namespace cnh {
+int g_product_statements = 1;   // option "product_statements"
+bool product_statements_on() { return g_product_statements != 0; }
+} // namespace cnh
+
+extern "C" int cnh_launch_product_group(cnh_kernel* k, const cnh_gemm_job* job, int n_blocks, int ndims, int n_in,
+                                        const cnh_memref* in, const int32_t* in_block, int n_scalar,
+                                        const void* const* scalars, int scalars_on_device, int n_out,
+                                        const cnh_memref* out, cnh_stream s) {
+    if (int rc = ensure_init())
+        return rc;
+    CNH_CHECK(k != nullptr && job != nullptr, -2, "null argument");
+    const GroupProgram& p = k->prog;
+    CNH_CHECK(ndims == p.ndims, -4, "kernel was compiled for rank %d, launched with %d", p.ndims, ndims);
+    CNH_CHECK(n_in == (int)p.leaves.size(), -4, "group expects %d input memrefs, got %d", (int)p.leaves.size(),
+              n_in);
+    CNH_CHECK(n_out == (int)p.out_roots.size(), -4, "group expects %d output memrefs, got %d",
+              (int)p.out_roots.size(), n_out);
+    CNH_CHECK(n_out >= 1 && out != nullptr, -2, "a group needs at least one output memref");
+    CNH_CHECK(n_in == 0 || (in != nullptr && in_block != nullptr), -2, "null input memrefs");
+    CNH_CHECK(job->M >= 0 && job->N >= 0 && job->K >= 0 && job->A && job->B && job->C, -2,
+              "product: bad extent or null pointer");
+    CNH_CHECK(job->lda >= job->K && job->ldb >= job->N && job->ldc >= job->N, -2,
+              "product: row stride shorter than the row");
+    // what the fused kernel does not take is left to the caller's two launches
+    CNH_CHECK(g_product_statements, -17, "statements in a product's epilogue are switched off");
+    CNH_CHECK(p.dtype == CNH_F64 && p.reductions() == 0 && ndims >= 2, -17,
+              "statements in a product's epilogue: fp64, rank 2 or 3, no reducing roots");
+    CNH_CHECK(n_blocks == 1 || n_blocks == 2 || n_blocks == 4, -17, "%d column blocks (1, 2 or 4)", n_blocks);
+    CNH_CHECK(gemm_split_form(job->M, job->N, job->K, job->A, job->lda, job->B, job->ldb) &&
+                  job->N % n_blocks == 0, -17,
+              "product of %lld x %lld x %lld is not of the one-workgroup-per-CU form", (long long)job->M,
+              (long long)job->N, (long long)job->K);
+    const int64_t nblock = job->N / n_blocks;
+    const int NL = (int)p.load_leaf.size();
+    const int NLA = NL > 0 ? NL : 1, NOA = n_out;
+    const int pad = CNH_MAX_ND - ndims;
+    // every memref of the group has the extents (1, ..., rows of the product, width of a column block)
+    for (int i = 0; i < n_in + n_out; ++i) {
+        const cnh_memref& m = i < n_in ? in[i] : out[i - n_in];
+        if (i < n_in && in_block[i] >= 0) {
+            CNH_CHECK(in_block[i] < n_blocks, -4, "input %d names column block %d of %d", i, in_block[i], n_blocks);
+            continue;                       // taken from the tile of sums: its memref is not read
+        }
+        CNH_CHECK(m.aligned != nullptr, -4, "memref %d has a null pointer", i);
+        for (int d = 0; d < ndims; ++d) {
+            const int64_t want = d == ndims - 1 ? nblock : d == ndims - 2 ? job->M : 1;
+            CNH_CHECK(m.sizes[d] == want, -17, "memref %d has extent %lld in dim %d, the product's blocks have %lld",
+                      i, (long long)m.sizes[d], d, (long long)want);
+        }
+    }
+    std::vector<unsigned char> scal;
+    if (int rc = pack_scalars(p, n_scalar, scalars, scalars_on_device, scal))
+        return rc;
+    const int esz = 8;
+    auto base_ptr = [&](const cnh_memref& m) -> int64_t {
+        return (int64_t)((uintptr_t)m.aligned + (uintptr_t)(m.offset * esz));
+    };
+    // EpiArgs { Cell cell; Scal sc; int src[NLA]; int nblock; int unused; } as the generated text lays it out
+    const size_t cell_words = 5 + NLA + 3 * NLA + NOA + 3 * NOA;
+    const size_t tail_bytes = ((size_t)(NLA + 2) * 4 + 7) & ~size_t(7);
+    std::vector<unsigned char> epi(cell_words * 8 + scal.size() + tail_bytes, 0);
+    int64_t* c = reinterpret_cast<int64_t*>(epi.data());
+    c[0] = 1;
+    c[1] = job->M;
+    c[2] = nblock;
+    int64_t* cin = c + 5;
+    int64_t* cistr = cin + NLA;
+    int64_t* cout = cistr + 3 * NLA;
+    int64_t* costr = cout + NOA;
+    int32_t* src = reinterpret_cast<int32_t*>(epi.data() + cell_words * 8 + scal.size());
+    for (int l = 0; l < NL; ++l) {
+        const int leaf = p.load_leaf[l];
+        src[l] = in_block[leaf] >= 0 ? in_block[leaf] : -1;
+        if (src[l] >= 0)
+            continue;
+        cin[l] = base_ptr(in[leaf]);
+        for (int d = 0; d < ndims; ++d)
+            cistr[l * 3 + pad + d] = in[leaf].strides[d];
+    }
+    for (int o = 0; o < n_out; ++o) {
+        cout[o] = base_ptr(out[o]);
+        for (int d = 0; d < ndims; ++d)
+            costr[o * 3 + pad + d] = out[o].strides[d];
+    }
+    std::memcpy(epi.data() + cell_words * 8, scal.data(), scal.size());
+    src[NLA] = (int32_t)nblock;
+    hipFunction_t fn;
+    const std::string variant = "product" + std::to_string(n_blocks);
+    if (int rc = get_function(k, variant, "grp_product", &fn))
+        return rc;
+    GemmChainDev ch{(double*)job->C, job->ldc, (int32_t)job->M, (int32_t)job->N, 0, 1, 0, (int32_t)(job->M / 64)};
+    GemmSegDev sg{(const double*)job->A, job->lda, (const double*)job->B, job->ldb, (int32_t)job->K, 0};
+    const void* no_table = nullptr;
+    int nchains = 1, nblocks = (int)((job->M / 64) * (job->N / 64)), overwrite = 1;
+    void* params[] = {&no_table, &nchains, &no_table, &nblocks, &ch, &sg, &overwrite, epi.data()};
+    return launch(fn, nblocks, params, as_stream(s), 1024);
+}
+
+// ---------------------------------------------------------------------------------------------
 // Tiled launch: all tiles of the target in one launch, neighbour tiles read in place.
 // ---------------------------------------------------------------------------------------------
 namespace {
@@ -1550,6 +1668,11 @@ extern "C" int cnh_set_option(const char* name, int value) {
     if (std::strcmp(name, "gemm_buffer_loads") == 0) {
         CNH_CHECK(value == 0 || value == 1, -2, "gemm_buffer_loads: 0 or 1");
         gemm_set_buffer_loads(value);
+        return 0;
+    }
+    if (std::strcmp(name, "product_statements") == 0) {
+        CNH_CHECK(value == 0 || value == 1, -2, "product_statements: 0 or 1");
+        g_product_statements = value;
         return 0;
     }
     if (std::strcmp(name, "gemm_ksplit") == 0) {

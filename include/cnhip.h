@@ -132,6 +132,9 @@ int cnh_version(void);
  *                        with 0; whether a product qualifies depends on the device's CU count, so two
  *                        devices with different CU counts may differ in the last bits of a product
  *                        (0 gives the single-set order everywhere).
+ *   "product_statements"  cnh_launch_product_group takes the shapes it can (default 1); 0: it answers
+ *                        -17 for every shape, so callers issue the product and the group separately.
+ *                        Same bits.
  *   "slide_bx/ry/zc/pd", "slide2d_march"  geometry of the sliding-window kernel */
 int cnh_set_option(const char* name, int value);
 
@@ -445,6 +448,28 @@ int cnh_gemm_acc_batch(int dtype, int njobs, const cnh_gemm_job* jobs, cnh_strea
  * neither read nor kept, so a freshly allocated result needs no zero-fill
  * (upstream zero-fills result_data and accumulates, src/executor_matmatmul.cpp:105-160). */
 int cnh_gemm_batch(int dtype, int njobs, const cnh_gemm_job* jobs, int overwrite, cnh_stream s);
+
+/* One overwriting fp64 product C = A @ B and, in the same launch, the statements of a compiled
+ * group evaluated on its result (no upstream counterpart: upstream runs the panel products,
+ * src/executor_incremental.cpp:97-132, and the groups that read their result,
+ * src/dispatch.hpp:137-265, as separate tasks; examples/lstm_forward.py:40-49 is the
+ * program this is for: the gate statements of a step behind its product). The product's N columns
+ * are n_blocks (1, 2 or 4) column blocks of equal width; the group's memrefs all have the extents
+ * (1, ..., M, N / n_blocks), and input i with in_block[i] >= 0 is column block in_block[i] of the
+ * product (its memref is not read: the values come from the workgroup's tile of sums), the others
+ * are read through their memrefs. C receives the product as cnh_gemm_batch(overwrite = 1) would
+ * leave it, bit for bit, and the outputs what cnh_launch_group would store when launched behind
+ * it. The statements of an element run as soon as its workgroup's sums are complete, while other
+ * workgroups still multiply: no output may overlap A, B or C, and no input other than the
+ * product's blocks may overlap C or an output at a different element.
+ * Returns -17 without launching anything for shapes the fused kernel does not take (it exists for
+ * products of at most one 64 x 64 tile per compute unit with K a multiple of 32, the form
+ * cnh_gemm_batch runs with two sets of wavefronts per workgroup): the caller then issues
+ * cnh_gemm_batch and cnh_launch_group. */
+int cnh_launch_product_group(cnh_kernel* k, const cnh_gemm_job* job, int n_blocks, int ndims, int n_in,
+                             const cnh_memref* in, const int32_t* in_block, int n_scalar,
+                             const void* const* scalars, int scalars_on_device, int n_out,
+                             const cnh_memref* out, cnh_stream s);
 
 /* ---- synthetic inputs generated on the device (no upstream counterpart: upstream has no RNG,
  *      charmnumeric/random.py:4-5, and no bulk upload, charmnumeric.py:863-878) ---- */

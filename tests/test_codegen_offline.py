@@ -114,3 +114,19 @@ def test_the_boundary_column_rule_of_the_whole_array_kernel():
     k3 = H.compile_group(H.ast_jacobi3d(32), L.F64, 3)
     L.check(L.lib.cnh_kernel_build(k3, b"direct"))
     assert "#define DR_TAIL_OK 1" in H.kernel_source(k3, "direct")
+
+
+@pytest.mark.parametrize("blocks", [1, 2, 4])
+def test_product_kernel_with_a_groups_statements_builds(blocks):
+    """The matrix-core product kernel with the gate statements of an LSTM step appended (one launch
+    per step): its text is the ahead-of-time kernel's, compiled at run time with the group."""
+    import bench
+    k = H.compile_group(bench.lstm_fused_ast(L, False, True), L.F64, 2)
+    variant = b"product%d" % blocks
+    L.check(L.lib.cnh_kernel_build(k, variant))
+    src = H.kernel_source(k, variant.decode())
+    assert "#define CN_EPI_Q %d" % blocks in src and "grp_product" in src and "cn_tanh_f64" in src
+    assert L.lib.cnh_kernel_build(k, b"product3") != 0
+    # other element types keep their two launches
+    k32 = H.compile_group(H.ast_jacobi2d(64, dtype=L.F32, coef=2.0), L.F32, 2)
+    assert L.lib.cnh_kernel_build(k32, b"product4") != 0

@@ -159,3 +159,59 @@ def test_lstm_forward_full_shape_through_the_frontend(flat_rank3):
     finally:
         cnp.reset()
         itf.close()
+
+
+def _lstm_arrays(itf, steps, b, word, d):
+    """The program of examples/lstm_forward.py upstream; returns every array it leaves, on the host."""
+    hX = H.np_uniform(steps * b * word, 5, 0, -1.0, 1.0).reshape(steps, b, word)
+    hW = H.np_uniform((word + d) * 4 * d, 5, 1, -1 / 32, 1 / 32).reshape(word + d, 4 * d)
+    X, W = cnp.array(hX), cnp.array(hW)
+    h0 = cnp.zeros((1, d))
+    Hin = cnp.zeros((steps, b, word + d))
+    Hout = cnp.zeros((steps, b, d))
+    IFOG = cnp.zeros((steps, b, 4 * d))
+    IFOGf = cnp.zeros((steps, b, 4 * d))
+    Cs = cnp.zeros((steps, b, d))
+    Ct = cnp.zeros((steps, b, d))
+    for t in range(steps):
+        prev = cnp.tile(h0, (b, 1)) if t == 0 else Hout[t - 1]
+        Hin[t, :, :word] = X[t]
+        Hin[t, :, word:] = prev
+        IFOG[t] = Hin[t].dot(W)
+        IFOGf[t, :, : 3 * d] = 1.0 / (1.0 + cnp.exp(-IFOG[t, :, : 3 * d]))
+        IFOGf[t, :, 3 * d:] = cnp.tanh(IFOG[t, :, 3 * d:])
+        Cs[t] = IFOGf[t, :, :d] * IFOGf[t, :, 3 * d:]
+        if t > 0:
+            Cs[t] += IFOGf[t, :, d: 2 * d] * Cs[t - 1]
+        Ct[t] = cnp.tanh(Cs[t])
+        Hout[t] = IFOGf[t, :, 2 * d: 3 * d] * Ct[t]
+    got = {name: a.get(itf) for name, a in (("Hin", Hin), ("IFOG", IFOG), ("IFOGf", IFOGf), ("C", Cs),
+                                            ("Ct", Ct), ("Hout", Hout))}
+    del X, W, h0, Hin, Hout, IFOG, IFOGf, Cs, Ct, prev
+    return got
+
+
+@pytest.mark.parametrize("steps,b,word,d", [(4, 256, 1024, 1024), (3, 128, 256, 256), (3, 64, 192, 64)])
+def test_an_lstm_step_is_one_launch_and_the_same_bits_as_two(steps, b, word, d):
+    """The gate statements of a step ride on the step's product (the product's launch evaluates them
+    on its tiles of sums); with that switched off the product and the merged statements are two
+    launches. Every array of the program agrees bit for bit."""
+    from charmnumeric_amd import _lib as L
+    runs = {}
+    for on in (1, 0):
+        itf = _connect(4, True, True)
+        try:
+            L.check(L.lib.cnh_set_option(b"product_statements", on))
+            itf.set_trace()
+            runs[on] = _lstm_arrays(itf, steps, b, word, d)
+            trace = itf.trace()
+            if os.environ.get("CHARMNUMERIC_SOLVER", "0") in ("", "0"):
+                assert sum(" with_statements" in ln for ln in trace) == (steps if on else 0)
+                assert sum(" in_product" in ln for ln in trace) == (steps if on else 0)
+        finally:
+            L.check(L.lib.cnh_set_option(b"product_statements", 1))
+            cnp.reset()
+            itf.close()
+    for name in runs[1]:
+        assert np.array_equal(runs[1][name], runs[0][name]), name
+    assert np.any(runs[1]["Hout"][-1] != 0.0)

@@ -90,3 +90,25 @@ def test_gemm_full_lstm_shape_properties(dev):
     L.check(L.lib.cnh_gemm_acc(L.F64, M, N, K, A.ptr, K, B.ptr, N, Cz.ptr, N, None))
     assert np.array_equal(Cz.get(), a1 @ b1)               # exact in fp64, any summation order
     dev.free_all()
+
+
+@pytest.mark.parametrize("steps,batch,nin,d", [(3, 256, 1024, 1024), (4, 128, 512, 512), (3, 64, 256, 256),
+                                               (2, 192, 64, 64)])
+def test_gate_statements_in_the_products_epilogue_change_no_bit(dev, steps, batch, nin, d):
+    """One launch per step (the gate statements evaluated on the product's tile of sums before its
+    workgroup ends, a workgroup's 64 columns being 16 of each gate) against the product and the gate
+    launch one after the other: every array of the program, bit for bit."""
+    one = bench.run_lstm(L, steps=steps, batch=batch, nin=nin, d=d, timed=False, keep=True, epilogue=True)
+    two = bench.run_lstm(L, steps=steps, batch=batch, nin=nin, d=d, timed=False, keep=True, epilogue=False)
+    assert one["launches_per_step"] == 1 and two["launches_per_step"] == 2
+    for name in ("IFOG", "IFOGf", "C", "Ct", "Hout", "Hin"):
+        assert np.array_equal(one[name], two[name]), name
+    assert np.any(one["Hout"][-1] != 0.0)
+
+
+def test_shapes_the_fused_product_does_not_take_fall_back_to_two_launches(dev):
+    """70 rows are no multiple of the 64-row tile: cnh_launch_product_group answers -17 and launches nothing."""
+    got = bench.run_lstm(L, steps=2, batch=70, nin=24, d=24, timed=False, keep=True, epilogue=True)
+    assert got["launches_per_step"] == 2
+    Hout, Cc, IFOG, _ = _reference(2, 70, 24, 24)
+    assert np.allclose(got["Hout"], Hout, rtol=1e-12, atol=1e-13)
