@@ -722,14 +722,15 @@ extern "C" __global__ __launch_bounds__(64) void grp_nd1_p1(Cell cell, Scal sc) 
     return s.str();
 }
 
-// The product kernel with the group's statements in its epilogue: the text of gemm_kernel.inc in its
-// shape for grids of one workgroup per CU (2 sets of 4 x 2 wavefronts, 64 x 64 tiles, buffer loads),
+// The product kernel with the group's statements in its epilogue: the text of gemm_kernel.inc in one of
+// its three forms (1: two sets of 4 x 2 wavefronts sharing the K steps, for grids of one workgroup per
+// CU; 2: one such set; 3: 2 x 2 wavefronts of 32 x 32; 64 x 64 tiles and buffer loads in all of them),
 // with a workgroup's 64 columns taken as 64 / q from each of q column blocks of the product. When the
 // sums are complete they go to global memory and to an LDS tile; then every lane of the workgroup
 // takes elements (row, block column) of the tile's rows: loads that name a column block of the
 // product come from the tile, the others from their memrefs, and the statements are those of the
 // strided-cell kernel.
-std::string product_source(const GroupProgram& p, int q) {
+std::string product_source(const GroupProgram& p, int q, int form) {
     std::ostringstream s;
     s << prelude(p);
     s << "typedef long long cn_i64;\ntypedef int cn_i32;\n";
@@ -743,8 +744,13 @@ struct Cell {
 // src[k]: which column block of the product load k is (-1: an array of its own, read through
 // cell.in[k]); nblock: width of a column block
 struct EpiArgs { Cell cell; Scal sc; int src[NLA]; int nblock; int unused; };
-constexpr int WM = 4, WN = 2, TM = 1, TN = 2, BKT = 16, KS = 2;
+constexpr int BKT = 16;
 constexpr bool FULL = true, BUF = true;
+)";
+    s << (form == 3 ? "constexpr int WM = 2, WN = 2, TM = 2, TN = 2, KS = 1;\n"
+                    : form == 2 ? "constexpr int WM = 4, WN = 2, TM = 1, TN = 2, KS = 1;\n"
+                                : "constexpr int WM = 4, WN = 2, TM = 1, TN = 2, KS = 2;\n");
+    s << R"(
 
 // Elements (row, block column) of the workgroup's tile a lane takes: e = lane, lane + LANES, ...
 // The loads that do not come from the product are issued before the first K step when a lane has a
@@ -1209,16 +1215,19 @@ int emit_variant_source(const GroupProgram& p, const std::string& variant, std::
         return 0;
     }
     if (variant.compare(0, 7, "product") == 0) {
-        const int q = variant.size() == 8 ? variant[7] - '0' : 0;
-        if (q != 1 && q != 2 && q != 4) {
-            err = "the product variant is product1, product2 or product4 (column blocks per product)";
+        // "product<q>" + form: "" two sets of eight wavefronts, "e" eight wavefronts, "f" four
+        const int q = variant.size() >= 8 ? variant[7] - '0' : 0;
+        const int form = variant.size() == 8 ? 1 : variant.size() == 9 && variant[8] == 'e' ? 2
+                         : variant.size() == 9 && variant[8] == 'f' ? 3 : 0;
+        if ((q != 1 && q != 2 && q != 4) || form == 0) {
+            err = "the product variant is product<1|2|4>[e|f] (column blocks per product, form of the kernel)";
             return -2;
         }
         if (p.dtype != CNH_F64) {
             err = "statements in a product's epilogue are fp64 only";
             return -17;
         }
-        src = product_source(p, q);
+        src = product_source(p, q, form);
         return 0;
     }
     if (variant == "tiles") {

@@ -64,11 +64,13 @@ int reduce_slots_f64_many(int nvec, const int* maximum, double* const* vecs, int
 void gemv_set_xlds(int on);
 void gemm_set_buffer_loads(int on);
 void gemm_set_ksplit(int on);
-// Would a single overwriting fp64 product of this shape take the kernel of two sets of eight
-// wavefronts per workgroup (64 x 64 tiles, one workgroup per CU, K steps shared between the sets)?
-// The product kernel with a group's statements in its epilogue exists in that form only, and adds
-// its sums in that form's order.
-bool gemm_split_form(int64_t M, int64_t N, int64_t K, const void* A, int64_t lda, const void* B, int64_t ldb);
+// Which form of the matrix-core kernel a single overwriting fp64 product of this shape takes with
+// buffer loads (0: none of them — extents no multiples of the 64 x 64 x 16 tile, unaligned or too
+// widely strided operands): 1 = two sets of eight wavefronts per workgroup sharing the K steps (at
+// most one workgroup per CU, K a multiple of 32), 2 = eight wavefronts of 16 x 32, 3 = four of
+// 32 x 32 (1024 tiles and more). The kernel with a group's statements in its epilogue is built in
+// the same form, so it adds its sums in the same order.
+int gemm_form(int64_t M, int64_t N, int64_t K, const void* A, int64_t lda, const void* B, int64_t ldb);
 int reduce_slots_f64(bool maximum, double* slots, int64_t n, double* out, hipStream_t st);
 
 // Option "product_statements": may a product's launch evaluate the statements that follow it?

@@ -3954,8 +3954,8 @@ int try_product_into_region(Ex* ex, const std::vector<DagNode>& dag, size_t i, s
 // examples/lstm_forward.py:40-49 upstream): the product's launch evaluates the run on each
 // workgroup's tile of sums (cnh_launch_product_group), so the step is one launch and nothing waits
 // for a second one to start. Taken when
-//   - the product is a single fp64 panel product into the box, of the shape that gives every CU at
-//     most one workgroup (the fused kernel exists in that form only);
+//   - the product is a single fp64 panel product into the box, in whole 64 x 64 x 16 tiles of
+//     aligned operands (what the fused kernel is built for);
 //   - the run's extents are (rows of the product) x (its columns / q), q = 1, 2 or 4, and every read
 //     of the target that meets the box is exactly one of its q column blocks;
 //   - no statement assigns into the box or into a window the product reads (workgroups finish at
@@ -4001,8 +4001,8 @@ int try_product_with_statements(Ex* ex, const std::vector<DagNode>& dag, size_t 
         return rc;
     if (!taken || jobs.empty())
         return no("the product does not go into the box as panel products");
-    if (!gemm_split_form(ops.M, ops.N, ops.K, nullptr, ops.K, nullptr, ops.N))
-        return no("not of the one-workgroup-per-CU shape");
+    if (!gemm_form(ops.M, ops.N, ops.K, nullptr, ops.K, nullptr, ops.N))
+        return no("extents no multiples of the 64 x 64 x 16 tile");
     ProductSite site;
     auto tgt = ex->arrays.find(dag[i + 1].nodes[set.operands[0]].result_name);
     if (tgt == ex->arrays.end() || set.region.ndims != tgt->second.ndims)
@@ -4060,8 +4060,8 @@ int try_product_with_statements(Ex* ex, const std::vector<DagNode>& dag, size_t 
         if (!taken || jobs.size() != 1)
             return no("not a single panel product into the box");
     }
-    if (!gemm_split_form(jobs[0].M, jobs[0].N, jobs[0].K, jobs[0].A, jobs[0].lda, jobs[0].B, jobs[0].ldb))
-        return no("not of the one-workgroup-per-CU shape");
+    if (!gemm_form(jobs[0].M, jobs[0].N, jobs[0].K, jobs[0].A, jobs[0].lda, jobs[0].B, jobs[0].ldb))
+        return no("operands the buffer loads do not take");
     site.job = jobs[0];
     // the run may go on in the next message: the product waits with it
     if (sr.ran_off_end) {

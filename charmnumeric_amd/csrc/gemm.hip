@@ -225,12 +225,16 @@ __global__ __launch_bounds__(512) void mfma_f64_probe(double* out, int iters, do
 namespace cnh {
 void gemm_set_buffer_loads(int on) { g_gemm_buffer_loads = on; }
 void gemm_set_ksplit(int on) { g_gemm_ksplit = on; }
-bool gemm_split_form(int64_t M, int64_t N, int64_t K, const void* A, int64_t lda, const void* B, int64_t ldb) {
-    const bool full = M % 64 == 0 && N % 64 == 0 && K % 32 == 0 && lda % 2 == 0 && ldb % 2 == 0 &&
-                      ((uintptr_t)A & 15) == 0 && ((uintptr_t)B & 15) == 0;
+int gemm_form(int64_t M, int64_t N, int64_t K, const void* A, int64_t lda, const void* B, int64_t ldb) {
+    const bool full = M > 0 && N > 0 && K > 0 && M % 64 == 0 && N % 64 == 0 && K % 16 == 0 && lda % 2 == 0 &&
+                      ldb % 2 == 0 && ((uintptr_t)A & 15) == 0 && ((uintptr_t)B & 15) == 0;
+    const bool buf = full && g_gemm_buffer_loads && 64 * lda * 8 < (1ll << 31) && 16 * ldb * 8 < (1ll << 31);
+    if (!buf)
+        return 0;
     const int64_t blocks = (M / 64) * (N / 64);
-    return full && M > 0 && N > 0 && K > 0 && g_gemm_buffer_loads && g_gemm_ksplit && blocks < 1024 &&
-           blocks <= compute_units() && 64 * lda * 8 < (1ll << 31) && 16 * ldb * 8 < (1ll << 31);
+    if (blocks >= 1024)
+        return blocks < (1ll << 31) ? 3 : 0;
+    return g_gemm_ksplit && blocks <= compute_units() && K % 32 == 0 ? 1 : 2;
 }
 } // namespace cnh
 

@@ -780,10 +780,10 @@ extern "C" int cnh_launch_product_group(cnh_kernel* k, const cnh_gemm_job* job, 
     CNH_CHECK(p.dtype == CNH_F64 && p.reductions() == 0 && ndims >= 2, -17,
               "statements in a product's epilogue: fp64, rank 2 or 3, no reducing roots");
     CNH_CHECK(n_blocks == 1 || n_blocks == 2 || n_blocks == 4, -17, "%d column blocks (1, 2 or 4)", n_blocks);
-    CNH_CHECK(gemm_split_form(job->M, job->N, job->K, job->A, job->lda, job->B, job->ldb) &&
-                  job->N % n_blocks == 0, -17,
-              "product of %lld x %lld x %lld is not of the one-workgroup-per-CU form", (long long)job->M,
-              (long long)job->N, (long long)job->K);
+    const int form = gemm_form(job->M, job->N, job->K, job->A, job->lda, job->B, job->ldb);
+    CNH_CHECK(form != 0 && job->N % n_blocks == 0, -17,
+              "product of %lld x %lld x %lld: extents no multiples of the 64 x 64 x 16 tile, or operands the "
+              "buffer loads do not take", (long long)job->M, (long long)job->N, (long long)job->K);
     const int64_t nblock = job->N / n_blocks;
     const int NL = (int)p.load_leaf.size();
     const int NLA = NL > 0 ? NL : 1, NOA = n_out;
@@ -839,7 +839,7 @@ extern "C" int cnh_launch_product_group(cnh_kernel* k, const cnh_gemm_job* job, 
     std::memcpy(epi.data() + cell_words * 8, scal.data(), scal.size());
     src[NLA] = (int32_t)nblock;
     hipFunction_t fn;
-    const std::string variant = "product" + std::to_string(n_blocks);
+    const std::string variant = "product" + std::to_string(n_blocks) + (form == 2 ? "e" : form == 3 ? "f" : "");
     if (int rc = get_function(k, variant, "grp_product", &fn))
         return rc;
     GemmChainDev ch{(double*)job->C, job->ldc, (int32_t)job->M, (int32_t)job->N, 0, 1, 0, (int32_t)(job->M / 64)};
@@ -847,7 +847,7 @@ extern "C" int cnh_launch_product_group(cnh_kernel* k, const cnh_gemm_job* job, 
     const void* no_table = nullptr;
     int nchains = 1, nblocks = (int)((job->M / 64) * (job->N / 64)), overwrite = 1;
     void* params[] = {&no_table, &nchains, &no_table, &nblocks, &ch, &sg, &overwrite, epi.data()};
-    return launch(fn, nblocks, params, as_stream(s), 1024);
+    return launch(fn, nblocks, params, as_stream(s), form == 1 ? 1024 : form == 2 ? 512 : 256);
 }
 
 // ---------------------------------------------------------------------------------------------

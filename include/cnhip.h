@@ -462,9 +462,9 @@ int cnh_gemm_batch(int dtype, int njobs, const cnh_gemm_job* jobs, int overwrite
  * it. The statements of an element run as soon as its workgroup's sums are complete, while other
  * workgroups still multiply: no output may overlap A, B or C, and no input other than the
  * product's blocks may overlap C or an output at a different element.
- * Returns -17 without launching anything for shapes the fused kernel does not take (it exists for
- * products of at most one 64 x 64 tile per compute unit with K a multiple of 32, the form
- * cnh_gemm_batch runs with two sets of wavefronts per workgroup): the caller then issues
+ * Returns -17 without launching anything for shapes the fused kernel does not take: it is built
+ * in the three forms cnh_gemm_batch runs aligned products in (by tile count and K), so M and N must
+ * be multiples of 64, K of 16, lda and ldb even and A and B 16-byte aligned; the caller then issues
  * cnh_gemm_batch and cnh_launch_group. */
 int cnh_launch_product_group(cnh_kernel* k, const cnh_gemm_job* job, int n_blocks, int ndims, int n_in,
                              const cnh_memref* in, const int32_t* in_block, int n_scalar,

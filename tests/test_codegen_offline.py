@@ -127,6 +127,10 @@ def test_product_kernel_with_a_groups_statements_builds(blocks):
     src = H.kernel_source(k, variant.decode())
     assert "#define CN_EPI_Q %d" % blocks in src and "grp_product" in src and "cn_tanh_f64" in src
     assert L.lib.cnh_kernel_build(k, b"product3") != 0
+    # the other two forms of the product kernel (grids of more than one tile per CU)
+    for form in (b"e", b"f"):
+        L.check(L.lib.cnh_kernel_build(k, variant + form))
+    assert L.lib.cnh_kernel_build(k, variant + b"x") != 0
     # other element types keep their two launches
     k32 = H.compile_group(H.ast_jacobi2d(64, dtype=L.F32, coef=2.0), L.F32, 2)
     assert L.lib.cnh_kernel_build(k32, b"product4") != 0

@@ -93,7 +93,11 @@ def test_gemm_full_lstm_shape_properties(dev):
 
 
 @pytest.mark.parametrize("steps,batch,nin,d", [(3, 256, 1024, 1024), (4, 128, 512, 512), (3, 64, 256, 256),
-                                               (2, 192, 64, 64)])
+                                               (2, 192, 64, 64),
+                                               # more tiles than CUs: one set of eight wavefronts per workgroup
+                                               (2, 512, 1024, 1024), (2, 576, 256, 256),
+                                               # 1024 tiles and more: four wavefronts of 32 x 32
+                                               (2, 1024, 1024, 1024)])
 def test_gate_statements_in_the_products_epilogue_change_no_bit(dev, steps, batch, nin, d):
     """One launch per step (the gate statements evaluated on the product's tile of sums before its
     workgroup ends, a workgroup's 64 columns being 16 of each gate) against the product and the gate
