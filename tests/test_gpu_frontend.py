@@ -832,3 +832,57 @@ def test_cg_on_a_small_system_with_merged_launches(small_tiles):
     want = (bn - bn.sum() / (2 * n)) / n
     assert np.allclose(x.get(itf), want, rtol=1e-10, atol=0)
     assert history[0] < 1e-12 * float(bn @ bn)
+
+
+# ---- a product and the statements that read it ----
+
+def _product_program(xp, A, B, C, out1, out2, blocks, variant):
+    """C[...] = A @ B and statements on C's column blocks; `variant` picks what makes the executor
+    keep the product and the statements apart (or nothing)."""
+    n = C.shape[1] // blocks
+    C[:, :] = A @ B
+    if variant == "blocks":
+        out1[:, :] = C[:, :n] * 2.0 + out2[:, :]
+        if blocks > 1:
+            out2[:, :] = C[:, (blocks - 1) * n:] - C[:, :n]
+    elif variant == "assigns-left-operand":
+        out1[:, :] = C[:, :n] * 2.0
+        A[:, :n] = C[:, :n] * 0.5
+    elif variant == "off-block-read":
+        out1[:, :] = C[:, 8:8 + n] * 2.0
+        out2[:, :] = C[:, :n] + 1.0
+    elif variant == "assigns-into-product":
+        out1[:, :] = C[:, :n] * 2.0
+        C[:, :n] = out1[:, :] + 1.0
+
+
+@pytest.mark.parametrize("blocks", [1, 2, 4])
+@pytest.mark.parametrize("variant", ["blocks", "assigns-left-operand", "off-block-read", "assigns-into-product"])
+def test_statements_behind_a_product(itf, blocks, variant):
+    """Statements that read a product's box block by block ride on the product's launch; a statement
+    that assigns where the product reads or writes, or reads the box across blocks, keeps it a launch
+    of its own (the trace says why). NumPy runs the same statements; products agree to 1e-12 of
+    sum |a||b|, everything else follows from them."""
+    if variant == "off-block-read" and blocks == 1:
+        pytest.skip("a single block has no other offset of its width")
+    M, K, N = 128, 256, 256
+    n = N // blocks
+    rng = np.random.default_rng(50 + blocks)
+    hA, hB = rng.uniform(-1, 1, (M, K)), rng.uniform(-1, 1, (K, N))
+    h1, h2 = np.zeros((M, n)), rng.uniform(-1, 1, (M, n))
+    hC = np.zeros((M, N))
+    itf.set_trace()
+    A, B, C, o1, o2 = cnp.array(hA), cnp.array(hB), cnp.zeros((M, N)), cnp.zeros((M, n)), cnp.array(h2)
+    _product_program(cnp, A, B, C, o1, o2, blocks, variant)
+    _product_program(np, hA, hB, hC, h1, h2, blocks, variant)
+    tol = 1e-12 * K
+    for name, dev, host in (("C", C, hC), ("out1", o1, h1), ("out2", o2, h2), ("A", A, hA)):
+        assert np.allclose(dev.get(itf), host, rtol=0, atol=4 * tol), name
+    if os.environ.get("CHARMNUMERIC_SOLVER", "0") in ("", "0"):
+        trace = itf.trace()
+        taken = sum(" with_statements" in ln for ln in trace)
+        refused = [ln for ln in trace if "statements_not_taken" in ln]
+        if variant == "blocks":
+            assert taken == 1 and not refused, trace
+        else:
+            assert taken == 0 and len(refused) == 1, trace
