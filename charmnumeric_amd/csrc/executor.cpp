@@ -3972,7 +3972,7 @@ bool unit_regions_disjoint(const cnh_region& a, const cnh_region& b, int nd) {
 int try_product_with_statements(Ex* ex, const std::vector<DagNode>& dag, size_t i, size_t* used, bool* open_ended) {
     *used = 0;
     *open_ended = false;
-    if (!product_statements_on() || i + 3 >= dag.size() || dag[i].roots.empty() || dag[i + 1].roots.size() != 1 ||
+    if (!product_statements_on() || i + 2 >= dag.size() || dag[i].roots.empty() || dag[i + 1].roots.size() != 1 ||
         dag[i + 2].roots.empty())
         return 0;
     const cnh_ast_node& mm = dag[i].nodes[dag[i].roots.back()];
@@ -4003,6 +4003,11 @@ int try_product_with_statements(Ex* ex, const std::vector<DagNode>& dag, size_t 
         return no("the product does not go into the box as panel products");
     if (!gemm_form(ops.M, ops.N, ops.K, nullptr, ops.K, nullptr, ops.N))
         return no("extents no multiples of the 64 x 64 x 16 tile");
+    if (i + 3 >= dag.size()) {
+        // the statements that read it may be the first nodes of the next message
+        *open_ended = open_ended_allowed(ex);
+        return 0;
+    }
     ProductSite site;
     auto tgt = ex->arrays.find(dag[i + 1].nodes[set.operands[0]].result_name);
     if (tgt == ex->arrays.end() || set.region.ndims != tgt->second.ndims)
@@ -4016,6 +4021,12 @@ int try_product_with_statements(Ex* ex, const std::vector<DagNode>& dag, size_t 
     collect_statement_run(ex, dag, i + 3, sr);
     if (sr.run.empty())
         return no("no statement run follows");
+    // the run may go on in the next message (and its extents settle only when it is complete: a
+    // wider first statement is cut to fit the ones that follow): the product waits with it
+    if (sr.ran_off_end) {
+        *open_ended = true;
+        return 0;
+    }
     // the run's extents: (1, ..., M, N / q)
     const Stmt& first = sr.run.front();
     if (first.nd < 2 || first.dtype != CNH_F64 || first.cnt[first.nd - 2] != ops.M ||
@@ -4063,11 +4074,6 @@ int try_product_with_statements(Ex* ex, const std::vector<DagNode>& dag, size_t 
     if (!gemm_form(jobs[0].M, jobs[0].N, jobs[0].K, jobs[0].A, jobs[0].lda, jobs[0].B, jobs[0].ldb))
         return no("operands the buffer loads do not take");
     site.job = jobs[0];
-    // the run may go on in the next message: the product waits with it
-    if (sr.ran_off_end) {
-        *open_ended = true;
-        return 0;
-    }
     site.what = "matmatmul A=" + std::to_string(ops.A->name) + " B=" + std::to_string(ops.B->name) + " out=" +
                 std::to_string(site.target->name) + " into_region panel_products=1";
     if (ex->dry) {

@@ -215,3 +215,26 @@ def test_an_lstm_step_is_one_launch_and_the_same_bits_as_two(steps, b, word, d):
     for name in runs[1]:
         assert np.array_equal(runs[1][name], runs[0][name]), name
     assert np.any(runs[1]["Hout"][-1] != 0.0)
+
+
+@pytest.mark.parametrize("flush_at", [3, 5, 7, 11, 16])
+def test_where_the_frontend_cuts_its_messages_does_not_change_what_is_merged(flush_at):
+    """Automatic flushes every few statements cut the recording anywhere — right behind a product,
+    in the middle of the gate statements: the product waits for the statements that read it, so
+    every step is still one launch, and the arrays are the same bits as with one message."""
+    from charmnumeric_amd import _lib as L
+    steps, b, word, d = 3, 128, 256, 256
+    runs = {}
+    for cut in (flush_at, 100000):
+        itf = _connect(4, True, True)
+        try:
+            cnp.set_auto_flush(itf, cut)
+            itf.set_trace()
+            runs[cut] = _lstm_arrays(itf, steps, b, word, d)
+            if os.environ.get("CHARMNUMERIC_SOLVER", "0") in ("", "0"):
+                assert sum(" with_statements" in ln for ln in itf.trace()) == steps
+        finally:
+            cnp.reset()
+            itf.close()
+    for name in runs[flush_at]:
+        assert np.array_equal(runs[flush_at][name], runs[100000][name]), name
