@@ -947,6 +947,8 @@ struct BlockArgs {
     int nroots;                 // scatter launches: the assigned lattices (same steps rst), else 0
     int nblk8;                  // launched workgroups / 8 (the launch is padded to a multiple of 8)
     int rrs[4][3], rcnt[4][3];  // first point and number of points of each of them
+    int rmate[4];               // the lattice one element to the right on the same rows, stored with this
+                                // one as a pair (-1: none; -2: this lattice is such a mate itself)
     BlockLeaf leaf[NLA];
 };
 // Consecutive workgroup ids go round the 8 XCDs: every XCD takes one contiguous eighth of the rows
@@ -1074,7 +1076,8 @@ extern "C" __global__ __launch_bounds__(256) void grp_block_pairs_rows(BlockArgs
 // takes one index (k0, k1, k2) of the lattices, evaluates every statement there and stores each
 // result at its own lattice's point, rs_r + k * step. The lattices may differ in their number of
 // points (cnt holds the largest per dimension): an index beyond a statement's own region reads that
-// statement's operands at their last index instead, and stores nothing for it.
+// statement's operands at their last index instead, and stores nothing for it. Two lattices with a
+// step of 2 along the rows whose points lie side by side on the same rows are stored as pairs.
 template <bool ROWS>
 __device__ __forceinline__ void block_scatter(const BlockArgs& a, const T* s) {
     const int W0 = a.cnt[0], W1 = a.cnt[1], W2 = a.cnt[2];
@@ -1114,9 +1117,34 @@ __device__ __forceinline__ void block_scatter(const BlockArgs& a, const T* s) {
             l[q] = a.leaf[q].base[rowoff[q] + (i64)min(k2, a.leaf[q].lim[2]) * a.leaf[q].step[2]];
         group_eval(l, s, o);
 #pragma unroll
-        for (int r = 0; r < NO; ++r)
-            if (rin[r] && k2 < a.rcnt[r][2])
-                a.dst[drow[r] + (i64)k2 * a.rst[2]] = o[r];
+        for (int r = 0; r < NO; ++r) {
+            const int m = a.rmate[r];
+            if (!rin[r] || m == -2)
+                continue;
+            T* at = a.dst + drow[r] + (i64)k2 * a.rst[2];
+            const bool own = k2 < a.rcnt[r][2];
+            if (m < 0) {
+                if (own)
+                    at[0] = o[r];
+                continue;
+            }
+            // two lattices side by side (the even and the odd columns of a prolongation's rows):
+            // both values of a lane as one 128-bit store, wherever the pair lies
+            T right = o[0];
+            int rcount = a.rcnt[0][2];
+#pragma unroll
+            for (int w = 1; w < NO; ++w) {
+                right = m == w ? o[w] : right;
+                rcount = m == w ? a.rcnt[w][2] : rcount;
+            }
+            const bool other = k2 < rcount;
+            if (own && other)
+                *reinterpret_cast<BP2A*>(at) = (BP2){o[r], right};
+            else if (own)
+                at[0] = o[r];
+            else if (other)
+                at[1] = right;
+        }
     }
 }
 extern "C" __global__ __launch_bounds__(256) void grp_scatter(BlockArgs a, Scal sc) {

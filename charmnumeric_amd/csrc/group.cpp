@@ -964,9 +964,9 @@ struct BlockHeadDev {
     void* dst;
     const void* cur;
     int32_t shape[3], dpy, dpz, rs[3], re[3], rst[3], cnt[3], lattice, nchunks, rsh;
-    int32_t nroots, nblk8, rrs[4][3], rcnt[4][3];
+    int32_t nroots, nblk8, rrs[4][3], rcnt[4][3], rmate[4];
 };
-static_assert(sizeof(BlockLeafDev) == 56 && sizeof(BlockHeadDev) == 200, "BlockArgs layout must match the generated struct");
+static_assert(sizeof(BlockLeafDev) == 56 && sizeof(BlockHeadDev) == 216, "BlockArgs layout must match the generated struct");
 
 bool is_pitched(const cnh_tiled* t) {
     for (int d = 0; d < t->ndims; ++d)
@@ -2026,6 +2026,18 @@ int launch_group_tiles_impl(cnh_kernel* k, int n_in, const cnh_tiled* in, int n_
                                   "assigned region %d leaves the target in dim %d", r, d - pad);
                         h.cnt[d] = r == 0 ? h.rcnt[r][d] : std::max(h.cnt[d], h.rcnt[r][d]);
                     }
+                // lattices side by side along the rows (step 2, the same rows, first columns one
+                // apart) are stored as pairs of elements
+                for (int r = 0; r < 4; ++r)
+                    h.rmate[r] = -1;
+                for (int r = 0; r < nroots && g_block_pairs && h.rst[2] == 2; ++r)
+                    for (int m = 0; m < nroots && h.rmate[r] == -1; ++m)
+                        if (m != r && h.rmate[m] == -1 && h.rrs[m][2] == h.rrs[r][2] + 1 &&
+                            h.rrs[m][0] == h.rrs[r][0] && h.rrs[m][1] == h.rrs[r][1] &&
+                            h.rcnt[m][0] == h.rcnt[r][0] && h.rcnt[m][1] == h.rcnt[r][1]) {
+                            h.rmate[r] = m;
+                            h.rmate[m] = -2;
+                        }
             }
             // unit steps along the rows everywhere, in place, one root: pairs of elements per access
             bool pairs = in_place && !multi && g_block_pairs && rst[2] == 1 && NL > 0;
