@@ -471,14 +471,6 @@ bool same_region(const cnh_region& a, const cnh_region& b) {
     return true;
 }
 
-uint64_t fnv(const void* data, size_t n, uint64_t h = 1469598103934665603ull) {
-    const unsigned char* p = static_cast<const unsigned char*>(data);
-    for (size_t i = 0; i < n; ++i) {
-        h ^= p[i];
-        h *= 1099511628211ull;
-    }
-    return h;
-}
 // The compile cache's key: 8 bytes per step (multiply, fold the high half back), the rest byte by
 // byte. A key that collides only costs a comparison of the groups themselves (compile_cached).
 uint64_t mix_words(const void* data, size_t n, uint64_t h = 0x9E3779B97F4A7C15ull) {
