@@ -333,6 +333,32 @@ def test_interleaved_lattices_are_assigned_by_one_scatter(itf, cshape, fusion):
         assert not launches
 
 
+@pytest.mark.parametrize("width", [40, 41, 130, 131])
+@pytest.mark.parametrize("longer", ["left", "right", "equal"])
+def test_lattices_side_by_side_are_stored_as_pairs_whichever_is_longer(itf, width, longer):
+    """Two statements that assign the odd and the even columns of the same rows (step 2) from other
+    arrays are one scatter launch whose lanes store both values as one pair; where one lattice has a
+    point more than the other at the end of a row, that point is stored alone. Rows of even and
+    odd length (pairs aligned and not)."""
+    rows = 9
+    rng = np.random.default_rng(width)
+    # left lattice: columns 1, 3, ...; right lattice: columns 2, 4, ... of the rows 1, 3, 5, 7
+    stop_left, stop_right = {"left": (width, width - 2), "right": (width - 3, width),
+                             "equal": (width - 2, width - 1)}[longer]
+    left, right = slice(1, stop_left, 2), slice(2, stop_right, 2)
+    nl, nr = len(range(width)[left]), len(range(width)[right])
+    a_host, b_host = rng.standard_normal((4, nl)), rng.standard_normal((4, nr))
+    e_host = rng.standard_normal((rows, width))
+    itf.set_trace()
+    a, b, e = cnp.array(a_host), cnp.array(b_host), cnp.array(e_host)
+    for xp_e, xp_a, xp_b in ((e, a, b), (e_host, a_host, b_host)):
+        xp_e[1:-1:2, left] = xp_a * 2.0
+        xp_e[1:-1:2, right] = xp_b + 1.0
+    assert np.array_equal(e.get(itf), e_host)
+    if os.environ.get("CHARMNUMERIC_SOLVER", "0") in ("", "0"):
+        assert sum("path=scatter roots=2" in ln for ln in itf.trace()) == 1
+
+
 def test_weighted_jacobi_and_residual(itf):
     n = 65
     h2 = (1.0 / (n - 1)) ** 2
