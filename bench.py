@@ -1471,6 +1471,57 @@ def run_strided(reps=10, only=None):
             out["poisson_257_cubed"] = entry(timed(poisson, 10 * reps), 3 * 8.0 * n ** 3)
         del v, q
         cnp.execute(itf)
+
+        # a whole V-cycle of examples/multigrid2d.py upstream on 4097^2 down to 5^2: two smoothing
+        # sweeps before and after, residual, full-weighting restriction, bilinear prolongation and
+        # correction, temporaries created and dropped at every level (about a hundred launches, most
+        # of them on the small grids, where the host sets the pace)
+        if want("multigrid_v_cycle_4097"):
+            itf.close()
+            itf = cnp.CharmNumericInterface(device=0)
+            itf.connect(odf=4)
+            itf.set_pipeline(True)
+            cnp.set_auto_flush(itf, 48)
+            omega = 2.0 / 3.0
+
+            def smooth_on(ug, fg, hh2, sweeps):
+                for _ in range(sweeps):
+                    upd = 0.25 * (ug[:-2, 1:-1] + ug[2:, 1:-1] + ug[1:-1, :-2] + ug[1:-1, 2:] + hh2 * fg[1:-1, 1:-1])
+                    ug[1:-1, 1:-1] = (1.0 - omega) * ug[1:-1, 1:-1] + omega * upd
+
+            def v_cycle(ug, fg, h):
+                m, hh2 = ug.shape[0], h * h
+                if m <= 5:
+                    smooth_on(ug, fg, hh2, 40)
+                    return
+                smooth_on(ug, fg, hh2, 2)
+                rg = cnp.zeros((m, m))
+                rg[1:-1, 1:-1] = fg[1:-1, 1:-1] - (1.0 / hh2) * (4.0 * ug[1:-1, 1:-1] - ug[:-2, 1:-1] - ug[2:, 1:-1]
+                                                                  - ug[1:-1, :-2] - ug[1:-1, 2:])
+                mc = (m - 1) // 2 + 1
+                rc, ec = cnp.zeros((mc, mc)), cnp.zeros((mc, mc))
+                cc, lo_, hi_ = slice(2, -2, 2), slice(1, -3, 2), slice(3, -1, 2)
+                rc[1:-1, 1:-1] = (0.25 * rg[cc, cc] + 0.125 * (rg[lo_, cc] + rg[hi_, cc] + rg[cc, lo_] + rg[cc, hi_])
+                                  + 0.0625 * (rg[lo_, lo_] + rg[lo_, hi_] + rg[hi_, lo_] + rg[hi_, hi_]))
+                v_cycle(ec, rc, 2.0 * h)
+                eg = cnp.zeros((m, m))
+                eg[2:-2:2, 2:-2:2] = ec[1:-1, 1:-1]
+                eg[1:-1:2, 2:-2:2] = 0.5 * (ec[:-1, 1:-1] + ec[1:, 1:-1])
+                eg[2:-2:2, 1:-1:2] = 0.5 * (ec[1:-1, :-1] + ec[1:-1, 1:])
+                eg[1:-1:2, 1:-1:2] = 0.25 * (ec[:-1, :-1] + ec[1:, :-1] + ec[:-1, 1:] + ec[1:, 1:])
+                ug[1:-1, 1:-1] = ug[1:-1, 1:-1] + eg[1:-1, 1:-1]
+                smooth_on(ug, fg, hh2, 2)
+
+            n = 4097
+            xs_ = np.linspace(0.0, 1.0, n)
+            fv = cnp.array(2.0 * np.pi ** 2 * np.outer(np.sin(np.pi * xs_), np.sin(np.pi * xs_)))
+            uv = cnp.zeros((n, n))
+            us = timed(lambda: v_cycle(uv, fv, 1.0 / (n - 1)), reps, warm=2)
+            exact = np.outer(np.sin(np.pi * xs_), np.sin(np.pi * xs_))
+            out["multigrid_v_cycle_4097"] = {"us": round(us, 1), "levels": 11,
+                                             "max_error_after_the_cycles": float(np.max(np.abs(uv.get(itf) - exact)))}
+            del uv, fv
+            cnp.execute(itf)
     finally:
         cnp.reset()
         itf.close()
